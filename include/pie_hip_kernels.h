@@ -1,0 +1,76 @@
+/*
+ * pie_hip_kernels.h — C ABI of the gfx950 (MI355X) kernel library behind the
+ * Pie driver forward pass.
+ *
+ * Every entry point takes plain device pointers, shapes and a HIP stream
+ * (passed as `void*`, i.e. a `hipStream_t`; NULL = the default stream), does no
+ * allocation, keeps no global state, never throws, and returns a status code.
+ * The functions replace, one for one, the `launch_*` C++ launchers of the
+ * reference CUDA driver (the .hpp files under driver/cuda/src/kernels and driver/cuda/src/ops);
+ * each declaration cites the launcher whose contract it follows.
+ *
+ * Conventions
+ *   - bf16 tensors are raw 16-bit words (`uint16_t`), row-major.
+ *   - "act x W" products follow the reference: act[M,K] · W[N,K]^T -> y[M,N]
+ *     (driver/cuda/src/ops/gemm.hpp:152-160).
+ *   - `beta` is 0 (overwrite y) or 1 (y += result, the residual fuse of
+ *     driver/cuda/src/model/llama_like.cpp:626-628).
+ */
+#ifndef PIE_HIP_KERNELS_H
+#define PIE_HIP_KERNELS_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PIE_HIP_OK 0
+#define PIE_HIP_ERR_INVALID 1     /* null pointer, non-positive size, bad enum   */
+#define PIE_HIP_ERR_UNSUPPORTED 2 /* shape the kernels do not cover              */
+#define PIE_HIP_ERR_LAUNCH 3      /* HIP reported an error at launch             */
+
+/* Library/ABI version: bumped on any signature change. */
+int pie_hip_abi_version(void);
+
+/* ---- W4A16 ("int4b8", symmetric, group-quantised) ------------------------- */
+
+/*
+ * Integer unpack test hook: q[n, k] = ((packed[n, k/8] >> (4*(k%8))) & 0xF) - 8
+ * as int8.  Bit-exact statement of the nibble order used everywhere else.
+ * Reference: driver/cuda/src/kernels/dequant_wna16.cu:31-36.
+ */
+int pie_hip_unpack_w4(const uint32_t* packed, int8_t* q, int out_dim, int in_dim,
+                      void* stream);
+
+/*
+ * w[n, k] = bf16( float(nibble - 8) * float(scale[n, k / group_size]) ).
+ * packed: [out_dim, in_dim/8] u32, scale: [out_dim, in_dim/group_size] bf16,
+ * out: [out_dim, in_dim] bf16.
+ * Reference: launch_dequant_wna16_int4b8_to_bf16,
+ * driver/cuda/src/kernels/dequant_wna16.hpp:16-23, dequant_wna16.cu:11-38.
+ */
+int pie_hip_dequant_w4a16(const uint32_t* packed, const uint16_t* scale_bf16,
+                          uint16_t* out_bf16, int out_dim, int in_dim, int group_size,
+                          void* stream);
+
+/*
+ * Weight-only int4 GEMV/skinny GEMM for decode:
+ *   y[m, n] = bf16( beta*y[m, n] + sum_k act[m, k] * (nibble(n, k) - 8) * scale[n, k/G] )
+ * with fp32 accumulation; the group scale is applied to each group's partial
+ * sum (same value as the reference's per-element `x * (q * s)` up to fp32
+ * rounding, driver/cuda/src/kernels/dequant_wna16.cu:96-110).
+ * Requires K % 32 == 0, G % 32 == 0, K % G == 0, 1 <= M <= 32.
+ * Replaces the Marlin call `marlin_w4a16_gemm` for small M
+ * (driver/cuda/third_party/marlin/marlin_wrapper.hpp:39-51) and the
+ * dequant-then-GEMM fallback of gemm_act_x_w (driver/cuda/src/ops/gemm.cpp:1414-1583).
+ */
+int pie_hip_gemv_w4a16(const uint16_t* act_bf16, const uint32_t* packed,
+                       const uint16_t* scale_bf16, uint16_t* y_bf16, int M, int N, int K,
+                       int group_size, int beta, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PIE_HIP_KERNELS_H */

@@ -1,0 +1,132 @@
+"""CPU oracle for the Pie driver forward-pass kernels — TEST INFRASTRUCTURE ONLY.
+
+A ctypes front end over `oracle/src/*.c` (a plain-C restatement of the
+reference's arithmetic; each C function cites the reference lines it follows).
+Only `tests/`, `__graft_entry__.smoke()` and `bench.py`'s `cpu_baseline` leg may
+import this package, and only as the checker / reported CPU baseline.  The
+product (`pie_amd/`) must never import it.
+
+bf16 tensors travel as `numpy.uint16` arrays of raw bits.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from pathlib import Path
+
+import numpy as np
+
+_HERE = Path(__file__).resolve().parent
+_LIB_PATH = _HERE / "libpie_oracle.so"
+_lib = None
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        if not _LIB_PATH.exists():
+            from . import build as _build
+
+            _build.build()
+        _lib = C.CDLL(str(_LIB_PATH))
+    return _lib
+
+
+# ---------------------------------------------------------------- bf16 helpers
+def f32_to_bf16(x) -> np.ndarray:
+    """Round-to-nearest-even float32 -> bf16 bits (uint16)."""
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+    nan = (u & 0x7FFFFFFF) > 0x7F800000
+    r = ((u.astype(np.uint64) + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+    r[nan] = ((u[nan] >> 16) | 0x40).astype(np.uint16)
+    return r
+
+
+def bf16_to_f32(b) -> np.ndarray:
+    return (np.ascontiguousarray(b, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def _p(a: np.ndarray | None):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+def _c(a, dtype) -> np.ndarray:
+    a = np.ascontiguousarray(a, dtype=dtype)
+    return a
+
+
+# ---------------------------------------------------------------- W4A16
+def unpack_w4(packed: np.ndarray, out_dim: int, in_dim: int) -> np.ndarray:
+    packed = _c(packed, np.uint32)
+    q = np.empty((out_dim, in_dim), np.int8)
+    lib().orc_unpack_w4(_p(packed), _p(q), C.c_int(out_dim), C.c_int(in_dim))
+    return q
+
+
+def pack_w4(q: np.ndarray) -> np.ndarray:
+    q = _c(q, np.int8)
+    out_dim, in_dim = q.shape
+    packed = np.empty((out_dim, in_dim // 8), np.uint32)
+    lib().orc_pack_w4(_p(q), _p(packed), C.c_int(out_dim), C.c_int(in_dim))
+    return packed
+
+
+def dequant_w4a16(packed, scale_bf16, out_dim: int, in_dim: int, group: int) -> np.ndarray:
+    packed = _c(packed, np.uint32)
+    scale_bf16 = _c(scale_bf16, np.uint16)
+    out = np.empty((out_dim, in_dim), np.uint16)
+    lib().orc_dequant_w4a16(_p(packed), _p(scale_bf16), _p(out), C.c_int(out_dim),
+                            C.c_int(in_dim), C.c_int(group))
+    return out
+
+
+def gemm_w4a16(act_bf16, packed, scale_bf16, group: int, mode: int = 0, y_in=None,
+               want_abs: bool = False):
+    """Returns (y_f32[M,N], y_bf16[M,N]) (+ abs_sum[M,N] float64 if want_abs)."""
+    act = _c(act_bf16, np.uint16)
+    M, K = act.shape
+    packed = _c(packed, np.uint32)
+    N = packed.shape[0]
+    scale = _c(scale_bf16, np.uint16)
+    y32 = np.empty((M, N), np.float32)
+    y16 = np.empty((M, N), np.uint16)
+    ab = np.empty((M, N), np.float64) if want_abs else None
+    yin = None if y_in is None else _c(y_in, np.uint16)
+    lib().orc_gemm_w4a16(_p(act), _p(packed), _p(scale), _p(yin), _p(y32), _p(y16), _p(ab),
+                         C.c_int(M), C.c_int(N), C.c_int(K), C.c_int(group),
+                         C.c_int(0 if y_in is None else 1), C.c_int(mode))
+    return (y32, y16, ab) if want_abs else (y32, y16)
+
+
+# ---------------------------------------------------------------- int8 per channel
+def quant_int8_per_channel(w_bf16):
+    w = _c(w_bf16, np.uint16)
+    rows, cols = w.shape
+    q = np.empty((rows, cols), np.int8)
+    s = np.empty((rows,), np.float32)
+    lib().orc_quant_int8_per_channel(_p(w), _p(q), _p(s), C.c_int(rows), C.c_int(cols))
+    return q, s
+
+
+def dequant_int8_per_channel(q, scale_inv):
+    q = _c(q, np.int8)
+    s = _c(scale_inv, np.float32)
+    rows, cols = q.shape
+    out = np.empty((rows, cols), np.uint16)
+    lib().orc_dequant_int8_per_channel(_p(q), _p(s), _p(out), C.c_int(rows), C.c_int(cols))
+    return out
+
+
+def gemm_w8a16(act_bf16, q, scale_inv, mode: int = 0, y_in=None, want_abs: bool = False):
+    act = _c(act_bf16, np.uint16)
+    M, K = act.shape
+    q = _c(q, np.int8)
+    N = q.shape[0]
+    s = _c(scale_inv, np.float32)
+    y32 = np.empty((M, N), np.float32)
+    y16 = np.empty((M, N), np.uint16)
+    ab = np.empty((M, N), np.float64) if want_abs else None
+    yin = None if y_in is None else _c(y_in, np.uint16)
+    lib().orc_gemm_w8a16(_p(act), _p(q), _p(s), _p(yin), _p(y32), _p(y16), _p(ab), C.c_int(M),
+                         C.c_int(N), C.c_int(K), C.c_int(0 if y_in is None else 1),
+                         C.c_int(mode))
+    return (y32, y16, ab) if want_abs else (y32, y16)
