@@ -70,6 +70,37 @@ int pie_hip_gemv_w4a16(const uint16_t* act_bf16, const uint32_t* packed,
                        const uint16_t* scale_bf16, uint16_t* y_bf16, int M, int N, int K,
                        int group_size, int beta, void* stream);
 
+/* ---- paged-KV decode attention -------------------------------------------- */
+
+/*
+ * One query token per request over a paged KV pool:
+ *   o[r, h, :] = softmax_j( q[r,h,:]·K[j, kvh, :] * sm_scale ) · V[j, kvh, :],  kvh = h / (hq/hk)
+ * for j over the request's context, kv_len = (pages-1)*page_size + last_page_len
+ * (0 when the request lists no page; then o = 0 and lse = -inf).
+ *   q, o          [R, hq, d] bf16
+ *   k_pages/v_pages [num_pages, page_size, hk, d] bf16 (driver/cuda/src/kv_cache.hpp:3-8)
+ *   kv_page_indices / kv_page_indptr[R+1] / kv_last_page_lens[R]: the wire arrays of
+ *     the forward request, as the runtime sends them; requests may list the same
+ *     physical pages (forked prefixes) — they are read in place.
+ *   lse           optional [R, hq] f32, natural-log sum-exp of the scaled scores
+ *   sm_scale      <= 0 selects 1/sqrt(d)
+ *   max_kv_len    host-side upper bound on any request's kv_len (sizes the split grid)
+ *   workspace     device scratch of pie_hip_attn_decode_workspace_bytes(...) bytes
+ * fp32 maths, one bf16 rounding at the output.  d in {64,128}, hq/hk in {1,2,4,8},
+ * page_size % 16 == 0.
+ * Reference: launch_attention_naive_paged_decode,
+ * driver/cuda/src/ops/attention_naive_paged.hpp:57-69, kernel attention_naive_paged.cu:319-447;
+ * split-KV planning role of driver/cuda/src/ops/attention_flashinfer.hpp:17-24.
+ */
+size_t pie_hip_attn_decode_workspace_bytes(int num_requests, int num_q_heads, int num_kv_heads,
+                                           int head_dim, int max_kv_len);
+int pie_hip_attn_decode_paged(const uint16_t* q, const uint16_t* k_pages, const uint16_t* v_pages,
+                              uint16_t* o, float* lse, const uint32_t* kv_page_indices,
+                              const uint32_t* kv_page_indptr, const uint32_t* kv_last_page_lens,
+                              int num_requests, int num_q_heads, int num_kv_heads, int head_dim,
+                              int page_size, float sm_scale, int max_kv_len, void* workspace,
+                              size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -130,3 +130,48 @@ def gemm_w8a16(act_bf16, q, scale_inv, mode: int = 0, y_in=None, want_abs: bool 
                          C.c_int(N), C.c_int(K), C.c_int(0 if y_in is None else 1),
                          C.c_int(mode))
     return (y32, y16, ab) if want_abs else (y32, y16)
+
+
+# ---------------------------------------------------------------- paged attention
+def attn_paged(q_bf16, k_pages, v_pages, qo_indptr, page_indices, page_indptr, last_lens,
+               hq: int, hk: int, d: int, ps: int, sm_scale: float = -1.0, mode: int = 0):
+    """General paged attention (decode = one query row per request).
+    Returns (o_f32[T,hq,d], o_bf16[T,hq,d], lse[T,hq])."""
+    q = _c(q_bf16, np.uint16)
+    T = q.shape[0]
+    kp = _c(k_pages, np.uint16)
+    vp = _c(v_pages, np.uint16)
+    qo = _c(qo_indptr, np.uint32)
+    pi = _c(page_indices, np.uint32)
+    pp = _c(page_indptr, np.uint32)
+    ll = _c(last_lens, np.uint32)
+    R = len(ll)
+    o32 = np.zeros((T, hq, d), np.float32)
+    o16 = np.zeros((T, hq, d), np.uint16)
+    lse = np.zeros((T, hq), np.float32)
+    lib().orc_attn_paged(_p(q), _p(kp), _p(vp), _p(o32), _p(o16), _p(lse), _p(qo), _p(pi), _p(pp),
+                         _p(ll), C.c_int(R), C.c_int(hq), C.c_int(hk), C.c_int(d), C.c_int(ps),
+                         C.c_float(sm_scale), C.c_int(mode))
+    return o32, o16, lse
+
+
+def attn_decode_paged(q_bf16, k_pages, v_pages, page_indices, page_indptr, last_lens, hq, hk, d,
+                      ps, sm_scale: float = -1.0, mode: int = 0):
+    R = len(last_lens)
+    return attn_paged(q_bf16, k_pages, v_pages, np.arange(R + 1, dtype=np.uint32), page_indices,
+                      page_indptr, last_lens, hq, hk, d, ps, sm_scale, mode)
+
+
+def kv_write(k_curr, v_curr, k_pages, v_pages, qo_indptr, page_indices, page_indptr, last_lens,
+             hk: int, d: int, ps: int):
+    """In-place scatter of this step's K/V rows into the (uint16) page pools."""
+    kc = _c(k_curr, np.uint16)
+    vc = _c(v_curr, np.uint16)
+    assert k_pages.dtype == np.uint16 and k_pages.flags.c_contiguous
+    assert v_pages.dtype == np.uint16 and v_pages.flags.c_contiguous
+    qo = _c(qo_indptr, np.uint32)
+    pi = _c(page_indices, np.uint32)
+    pp = _c(page_indptr, np.uint32)
+    ll = _c(last_lens, np.uint32)
+    lib().orc_kv_write(_p(kc), _p(vc), _p(k_pages), _p(v_pages), _p(qo), _p(pi), _p(pp), _p(ll),
+                       C.c_int(len(ll)), C.c_int(hk), C.c_int(d), C.c_int(ps))

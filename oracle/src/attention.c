@@ -1,0 +1,135 @@
+/*
+ * Oracle: paged-KV attention and KV page writes.  TEST INFRASTRUCTURE ONLY
+ * (see oracle_common.h).
+ *
+ * Follows the reference's hand-written paged kernels:
+ *   decode (one query per request)  driver/cuda/src/ops/attention_naive_paged.cu:319-447
+ *   prefill / mixed, causal limit   driver/cuda/src/ops/attention_naive_paged.cu:148-317
+ *   KV page write                   driver/cuda/src/kernels/kv_paged.cu:28-80
+ * KV pool layout [num_pages, page_size, num_kv_heads, head_dim] bf16
+ * (driver/cuda/src/kv_cache.hpp:3-8); element address
+ * ((page*page_size + slot)*hk + h)*d + j, the same address the portable driver's
+ * per-slot rows give (driver/portable/src/kv_cache.hpp:5-17).
+ *
+ * Pinned by tests/test_oracle_attention.py: dense numpy fp64 softmax attention over
+ * the gathered rows, page-permutation invariance, forked-prefix equality, the LSE
+ * definition, the zero-length case and the causal limit on small brute-force cases.
+ */
+#include <stdlib.h>
+
+#include "oracle_common.h"
+
+static int orc_kv_len(const uint32_t* indptr, const uint32_t* last_lens, int r, int ps) {
+    const int pages = (int)(indptr[r + 1] - indptr[r]);
+    /* attention_naive_paged.cu:349-352, with the empty page list made explicit */
+    return pages > 0 ? (pages - 1) * ps + (int)last_lens[r] : 0;
+}
+
+/*
+ * General paged attention: request r owns query rows qo_indptr[r]..qo_indptr[r+1];
+ * query i of n_q sees kv positions j < kv_len - n_q + i + 1 (attention_naive_paged.cu:194-198).
+ * Decode is the n_q = 1 case (qo_indptr = 0,1,2,...).
+ * mode 0: fp32 two-pass softmax in the reference's order; mode 2: fp64.
+ * o_f32 [T,hq,d] unrounded, o_bf16 optional, lse optional [T,hq] (natural log).
+ */
+void orc_attn_paged(const uint16_t* q, const uint16_t* k_pages, const uint16_t* v_pages,
+                    float* o_f32, uint16_t* o_bf16, float* lse, const uint32_t* qo_indptr,
+                    const uint32_t* page_indices, const uint32_t* page_indptr,
+                    const uint32_t* last_lens, int R, int hq, int hk, int d, int ps,
+                    float sm_scale, int mode) {
+    const int gqa = hq / hk;
+    const float scale = sm_scale > 0.f ? sm_scale : 1.0f / sqrtf((float)d);
+#pragma omp parallel for schedule(dynamic)
+    for (int r = 0; r < R; ++r) {
+        const int kv_total = orc_kv_len(page_indptr, last_lens, r, ps);
+        const int q_lo = (int)qo_indptr[r], n_q = (int)qo_indptr[r + 1] - q_lo;
+        const uint32_t pg_lo = page_indptr[r];
+        double* w = (double*)malloc(sizeof(double) * (size_t)(kv_total > 0 ? kv_total : 1));
+        for (int qi = 0; qi < n_q; ++qi) {
+            int lim = kv_total - n_q + qi + 1;
+            if (lim > kv_total) lim = kv_total;
+            if (lim < 0) lim = 0;
+            for (int h = 0; h < hq; ++h) {
+                const int kvh = h / gqa;
+                const size_t qoff = ((size_t)(q_lo + qi) * hq + h) * d;
+                double row_max = -INFINITY;
+                for (int j = 0; j < lim; ++j) {
+                    const uint32_t pid = page_indices[pg_lo + j / ps];
+                    const size_t koff = (((size_t)pid * ps + j % ps) * hk + kvh) * d;
+                    double dot;
+                    if (mode == 0) {
+                        float f = 0.f;
+                        for (int e = 0; e < d; ++e)
+                            f += orc_bf16_to_f32(q[qoff + e]) * orc_bf16_to_f32(k_pages[koff + e]);
+                        dot = (double)(f * scale);
+                    } else {
+                        double f = 0.0;
+                        for (int e = 0; e < d; ++e)
+                            f += (double)orc_bf16_to_f32(q[qoff + e]) *
+                                 (double)orc_bf16_to_f32(k_pages[koff + e]);
+                        dot = f * (double)scale;
+                    }
+                    w[j] = dot;
+                    if (dot > row_max) row_max = dot;
+                }
+                double z = 0.0;
+                float zf = 0.f;
+                for (int j = 0; j < lim; ++j) {
+                    if (mode == 0) {
+                        const float e = expf((float)w[j] - (float)row_max);
+                        w[j] = (double)e;
+                        zf += e;
+                    } else {
+                        w[j] = exp(w[j] - row_max);
+                        z += w[j];
+                    }
+                }
+                if (mode == 0) z = (double)zf;
+                for (int e = 0; e < d; ++e) {
+                    double acc = 0.0;
+                    float accf = 0.f;
+                    for (int j = 0; j < lim; ++j) {
+                        const uint32_t pid = page_indices[pg_lo + j / ps];
+                        const size_t voff = (((size_t)pid * ps + j % ps) * hk + kvh) * d;
+                        const float v = orc_bf16_to_f32(v_pages[voff + e]);
+                        if (mode == 0) accf = fmaf(v, (float)w[j], accf);
+                        else acc += (double)v * w[j];
+                    }
+                    if (mode == 0) acc = (double)accf;
+                    float out;
+                    if (mode == 0) out = z > 0.0 ? (float)acc * (1.0f / (float)z) : 0.f;
+                    else out = z > 0.0 ? (float)(acc / z) : 0.f;
+                    o_f32[qoff + e] = out;
+                    if (o_bf16) o_bf16[qoff + e] = orc_f32_to_bf16(out);
+                }
+                if (lse)
+                    lse[(size_t)(q_lo + qi) * hq + h] =
+                        z > 0.0 ? (float)(log(z) + row_max) : -INFINITY;
+            }
+        }
+        free(w);
+    }
+}
+
+/*
+ * Scatter this step's K/V rows [T, hk, d] into the pages.  The slot of token t of request
+ * r comes from the page table alone: pre_kv_len = kv_len - n_new, abs = pre_kv_len + offset
+ * (kv_paged.cu:49-59).
+ */
+void orc_kv_write(const uint16_t* k_curr, const uint16_t* v_curr, uint16_t* k_pages,
+                  uint16_t* v_pages, const uint32_t* qo_indptr, const uint32_t* page_indices,
+                  const uint32_t* page_indptr, const uint32_t* last_lens, int R, int hk, int d,
+                  int ps) {
+    const size_t row = (size_t)hk * d;
+    for (int r = 0; r < R; ++r) {
+        const int q_lo = (int)qo_indptr[r], n_new = (int)qo_indptr[r + 1] - q_lo;
+        const int kv_total = orc_kv_len(page_indptr, last_lens, r, ps);
+        for (int i = 0; i < n_new; ++i) {
+            const int abs_pos = kv_total - n_new + i;
+            const uint32_t pid = page_indices[page_indptr[r] + abs_pos / ps];
+            const size_t dst = ((size_t)pid * ps + abs_pos % ps) * row;
+            memcpy(k_pages + dst, k_curr + (size_t)(q_lo + i) * row, row * 2);
+            memcpy(v_pages + dst, v_curr + (size_t)(q_lo + i) * row, row * 2);
+        }
+    }
+}

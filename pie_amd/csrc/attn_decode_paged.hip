@@ -1,0 +1,405 @@
+// Paged-KV decode attention (one query token per request) for gfx950.
+//
+// Semantics: driver/cuda/src/ops/attention_naive_paged.cu:319-447 of the
+// reference (softmax(q·K^T * scale)·V over the request's pages, fp32 maths,
+// bf16 output, optional log-sum-exp), with the KV pool laid out
+// [num_pages, page_size, num_kv_heads, head_dim] bf16
+// (driver/cuda/src/kv_cache.hpp:3-8).  Prefix-shared (forked) pages need no
+// special handling: several requests simply list the same physical page ids.
+//
+// HBM-bound design (every K and V byte of the context is read once):
+//   * split-K over pages: grid = (splits, kv_head, request); a block of four waves
+//     owns a run of 16-token units of one (request, kv head) and each wave walks
+//     every fourth unit, so ragged contexts turn into many equal-sized blocks that
+//     the dispatcher load-balances; blocks past a request's length exit at once;
+//   * one wave load instruction covers whole 256-byte K (or V) rows: lane l reads
+//     the 16 B piece (l % LPR) of token (l / LPR), LPR = head_dim/8, so every access
+//     is a full, contiguous row and the GQA group's q heads share each K/V byte;
+//   * q·k runs on v_dot2_f32_bf16; the LPR lanes of a token finish the dot product
+//     with DPP row operations (no LDS, no ds_bpermute in the loop);
+//   * each group of LPR lanes keeps its own online-softmax state (max, sum, 8
+//     output dims per q head), so nothing crosses lane groups until the unit loop
+//     ends; groups, then waves (through LDS), are merged once per block;
+//   * the next unit's K and V rows are requested before the current unit is
+//     reduced, so 2 x (K+V) = 16 KiB per wave is in flight;
+//   * a second, tiny kernel merges the splits (skipped when there is one split).
+#include "common.hip.h"
+
+namespace pie_hip {
+namespace {
+
+constexpr int kAttnBlock = 256;
+constexpr int kAttnWaves = kAttnBlock / kWave;
+constexpr int kUnitTokens = 16;
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+    const int t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true);
+    return v + __int_as_float(t);
+}
+// Sum over the LPR (8 or 16) adjacent lanes that share a token; every lane gets the sum.
+template <int LPR>
+__device__ __forceinline__ float token_lanes_sum(float v) {
+    v = dpp_add<0xB1>(v);   // quad_perm [1,0,3,2]
+    v = dpp_add<0x4E>(v);   // quad_perm [2,3,0,1]
+    v = dpp_add<0x141>(v);  // row_half_mirror
+    if (LPR == 16) v = dpp_add<0x140>(v);  // row_mirror
+    return v;
+}
+
+template <int D, int GQA>
+struct UnitRegs {
+    static constexpr int LPR = D / 8;
+    static constexpr int TPI = kWave / LPR;          // tokens per load instruction
+    static constexpr int IPU = kUnitTokens / TPI;    // load instructions per unit
+    u32x4_t k[IPU];
+    u32x4_t v[IPU];
+};
+
+// part_o  [R, hq, nsplit, D] f32 (unnormalised), part_ml [R, hq, nsplit, 2] f32 (max, sum),
+// both in units where scores were multiplied by scale*log2(e).
+template <int D, int GQA>
+__global__ __launch_bounds__(kAttnBlock) void attn_decode_split_kernel(
+    const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_pages,
+    const uint16_t* __restrict__ v_pages, const uint32_t* __restrict__ page_indices,
+    const uint32_t* __restrict__ page_indptr, const uint32_t* __restrict__ last_lens,
+    float* __restrict__ part_o, float* __restrict__ part_ml, uint16_t* __restrict__ o_direct,
+    float* __restrict__ lse, int hq, int hk, int ps, int units_per_split, int nsplit,
+    float scale_log2e) {
+    using U = UnitRegs<D, GQA>;
+    constexpr int LPR = U::LPR, TPI = U::TPI, IPU = U::IPU;
+    const int split = blockIdx.x, kvh = blockIdx.y, r = blockIdx.z;
+    const int tid = threadIdx.x, lane = tid & (kWave - 1);
+    const int wv = __builtin_amdgcn_readfirstlane(tid / kWave);  // wave-uniform -> SGPR
+    const int grp = lane / LPR, dl = lane % LPR;
+
+    const uint32_t pg_lo = page_indptr[r];
+    const int npages = static_cast<int>(page_indptr[r + 1] - pg_lo);
+    const int kv_len = npages > 0 ? (npages - 1) * ps + static_cast<int>(last_lens[r]) : 0;
+    const int nunits = (kv_len + kUnitTokens - 1) / kUnitTokens;
+    const int u_begin = split * units_per_split;
+    if (u_begin >= nunits) return;
+    const int u_end = min(u_begin + units_per_split, nunits);
+
+    // q for the GQA heads of this kv head: 8 dims per lane per head, as bf16 pairs.
+    u32x4_t qv[GQA];
+#pragma unroll
+    for (int h = 0; h < GQA; ++h)
+        qv[h] = *reinterpret_cast<const u32x4_t*>(
+            q + (static_cast<size_t>(r) * hq + kvh * GQA + h) * D + dl * 8);
+
+    const size_t row_stride = static_cast<size_t>(hk) * D;  // elements between tokens
+    auto issue = [&](U& u, int unit) {
+        const int tok0 = unit * kUnitTokens;
+        const int page = tok0 / ps;
+        const uint32_t pid = page_indices[pg_lo + page];
+        const size_t base =
+            ((static_cast<size_t>(pid) * ps + (tok0 - page * ps)) * hk + kvh) * D + dl * 8;
+#pragma unroll
+        for (int i = 0; i < IPU; ++i) {
+            const size_t off = base + static_cast<size_t>(i * TPI + grp) * row_stride;
+            u.k[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(k_pages + off));
+            u.v[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(v_pages + off));
+        }
+    };
+
+    float m[GQA], l[GQA], o[GQA][8];
+#pragma unroll
+    for (int h = 0; h < GQA; ++h) {
+        m[h] = -INFINITY;
+        l[h] = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[h][e] = 0.f;
+    }
+
+    auto compute = [&](U& u, int unit) {
+        const int tok0 = unit * kUnitTokens;
+        float s[IPU][GQA];
+#pragma unroll
+        for (int i = 0; i < IPU; ++i) {
+#pragma unroll
+            for (int h = 0; h < GQA; ++h) {
+                float p = 0.f;
+                p = dot2_bf16(u.k[i].x, qv[h].x, p);
+                p = dot2_bf16(u.k[i].y, qv[h].y, p);
+                p = dot2_bf16(u.k[i].z, qv[h].z, p);
+                p = dot2_bf16(u.k[i].w, qv[h].w, p);
+                s[i][h] = token_lanes_sum<LPR>(p) * scale_log2e;
+            }
+        }
+        if (tok0 + kUnitTokens > kv_len) {  // tail unit: drop slots past the context
+#pragma unroll
+            for (int i = 0; i < IPU; ++i) {
+                if (tok0 + i * TPI + grp >= kv_len) {
+#pragma unroll
+                    for (int h = 0; h < GQA; ++h) s[i][h] = -INFINITY;
+                    u.v[i] = u32x4_t{0u, 0u, 0u, 0u};
+                }
+            }
+        }
+        float alpha[GQA];
+        bool grew = false;
+#pragma unroll
+        for (int h = 0; h < GQA; ++h) {
+            float mx = m[h];
+#pragma unroll
+            for (int i = 0; i < IPU; ++i) mx = fmaxf(mx, s[i][h]);
+            const float safe = (mx == -INFINITY) ? 0.f : mx;
+            alpha[h] = exp2f(m[h] - safe);
+            grew |= (mx != m[h]);
+            m[h] = mx;
+            float sum = 0.f;
+#pragma unroll
+            for (int i = 0; i < IPU; ++i) {
+                s[i][h] = exp2f(s[i][h] - safe);
+                sum += s[i][h];
+            }
+            l[h] = l[h] * alpha[h] + sum;
+        }
+        if (__any(grew)) {
+#pragma unroll
+            for (int h = 0; h < GQA; ++h)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) o[h][e] *= alpha[h];
+        }
+#pragma unroll
+        for (int i = 0; i < IPU; ++i) {
+            float vf[8];
+            vf[0] = bf16_lo(u.v[i].x); vf[1] = bf16_hi(u.v[i].x);
+            vf[2] = bf16_lo(u.v[i].y); vf[3] = bf16_hi(u.v[i].y);
+            vf[4] = bf16_lo(u.v[i].z); vf[5] = bf16_hi(u.v[i].z);
+            vf[6] = bf16_lo(u.v[i].w); vf[7] = bf16_hi(u.v[i].w);
+#pragma unroll
+            for (int h = 0; h < GQA; ++h)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) o[h][e] = fmaf(s[i][h], vf[e], o[h][e]);
+        }
+    };
+
+    // Two-deep pipeline over this wave's units (every fourth unit of the block's run).
+    U ua, ub;
+    const int first = u_begin + wv;
+    const int last_valid = u_end - 1;
+    if (first < u_end) {
+        issue(ua, first);
+        for (int u = first; u < u_end; u += 2 * kAttnWaves) {
+            issue(ub, min(u + kAttnWaves, last_valid));
+            compute(ua, u);
+            issue(ua, min(u + 2 * kAttnWaves, last_valid));
+            if (u + kAttnWaves < u_end) compute(ub, u + kAttnWaves);
+        }
+    }
+
+    // Merge the lane groups of the wave (lanes with equal dl).
+#pragma unroll
+    for (int h = 0; h < GQA; ++h) {
+        float mx = m[h];
+#pragma unroll
+        for (int off = LPR; off < kWave; off <<= 1) mx = fmaxf(mx, __shfl_xor(mx, off, kWave));
+        const float safe = (mx == -INFINITY) ? 0.f : mx;
+        const float a = exp2f(m[h] - safe);
+        float ls = l[h] * a;
+#pragma unroll
+        for (int off = LPR; off < kWave; off <<= 1) ls += __shfl_xor(ls, off, kWave);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            float ov = o[h][e] * a;
+#pragma unroll
+            for (int off = LPR; off < kWave; off <<= 1) ov += __shfl_xor(ov, off, kWave);
+            o[h][e] = ov;
+        }
+        m[h] = mx;
+        l[h] = ls;
+    }
+
+    // Merge the four waves through LDS.
+    __shared__ float sm_o[kAttnWaves][GQA][D];
+    __shared__ float sm_m[kAttnWaves][GQA];
+    __shared__ float sm_l[kAttnWaves][GQA];
+    if (grp == 0) {
+#pragma unroll
+        for (int h = 0; h < GQA; ++h) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) sm_o[wv][h][dl * 8 + e] = o[h][e];
+            if (dl == 0) {
+                sm_m[wv][h] = m[h];
+                sm_l[wv][h] = l[h];
+            }
+        }
+    }
+    __syncthreads();
+    for (int idx = tid; idx < GQA * D; idx += kAttnBlock) {
+        const int h = idx / D, dd = idx - h * D;
+        float mx = sm_m[0][h];
+#pragma unroll
+        for (int w = 1; w < kAttnWaves; ++w) mx = fmaxf(mx, sm_m[w][h]);
+        const float safe = (mx == -INFINITY) ? 0.f : mx;
+        float ov = 0.f, ls = 0.f;
+#pragma unroll
+        for (int w = 0; w < kAttnWaves; ++w) {
+            const float a = exp2f(sm_m[w][h] - safe);
+            ov += sm_o[w][h][dd] * a;
+            ls += sm_l[w][h] * a;
+        }
+        const int head = kvh * GQA + h;
+        const size_t rh = static_cast<size_t>(r) * hq + head;
+        if (o_direct) {
+            o_direct[rh * D + dd] = f32_to_bf16_bits(ls > 0.f ? ov / ls : 0.f);
+            if (lse && dd == 0)
+                lse[rh] = ls > 0.f ? (logf(ls) + mx * 0.6931471805599453f) : -INFINITY;
+        } else {
+            part_o[(rh * nsplit + split) * D + dd] = ov;
+            if (dd == 0) {
+                part_ml[(rh * nsplit + split) * 2 + 0] = mx;
+                part_ml[(rh * nsplit + split) * 2 + 1] = ls;
+            }
+        }
+    }
+}
+
+// One block per (request, q head): combine the splits that exist for this request.
+template <int D>
+__global__ void attn_decode_merge_kernel(const float* __restrict__ part_o,
+                                         const float* __restrict__ part_ml,
+                                         const uint32_t* __restrict__ page_indptr,
+                                         const uint32_t* __restrict__ last_lens,
+                                         uint16_t* __restrict__ o, float* __restrict__ lse, int hq,
+                                         int ps, int units_per_split, int nsplit) {
+    const int rh = blockIdx.x;
+    const int r = rh / hq;
+    const int dd = threadIdx.x;
+    const int npages = static_cast<int>(page_indptr[r + 1] - page_indptr[r]);
+    const int kv_len = npages > 0 ? (npages - 1) * ps + static_cast<int>(last_lens[r]) : 0;
+    const int nunits = (kv_len + kUnitTokens - 1) / kUnitTokens;
+    const int ns = min(nsplit, (nunits + units_per_split - 1) / units_per_split);
+    float mx = -INFINITY;
+    for (int s = 0; s < ns; ++s) mx = fmaxf(mx, part_ml[(static_cast<size_t>(rh) * nsplit + s) * 2]);
+    const float safe = (mx == -INFINITY) ? 0.f : mx;
+    float ov = 0.f, ls = 0.f;
+    for (int s = 0; s < ns; ++s) {
+        const size_t ps_i = static_cast<size_t>(rh) * nsplit + s;
+        const float a = exp2f(part_ml[ps_i * 2] - safe);
+        ov += part_o[ps_i * D + dd] * a;
+        ls += part_ml[ps_i * 2 + 1] * a;
+    }
+    o[static_cast<size_t>(rh) * D + dd] = f32_to_bf16_bits(ls > 0.f ? ov / ls : 0.f);
+    if (lse && dd == 0) lse[rh] = ls > 0.f ? (logf(ls) + mx * 0.6931471805599453f) : -INFINITY;
+}
+
+// Zero-length contexts never enter the split kernel; the single-split fast path needs their
+// rows cleared (the merge kernel does it itself on the multi-split path).
+template <int D>
+__global__ void attn_decode_clear_empty_kernel(const uint32_t* __restrict__ page_indptr,
+                                               const uint32_t* __restrict__ last_lens,
+                                               uint16_t* __restrict__ o, float* __restrict__ lse,
+                                               int hq, int ps) {
+    const int rh = blockIdx.x;
+    const int r = rh / hq;
+    const int npages = static_cast<int>(page_indptr[r + 1] - page_indptr[r]);
+    const int kv_len = npages > 0 ? (npages - 1) * ps + static_cast<int>(last_lens[r]) : 0;
+    if (kv_len > 0) return;
+    o[static_cast<size_t>(rh) * D + threadIdx.x] = 0;
+    if (lse && threadIdx.x == 0) lse[rh] = -INFINITY;
+}
+
+struct SplitPlan {
+    int units_per_split;
+    int nsplit;
+};
+
+// Same rule for the workspace query and the launch: aim for >= ~8 blocks per CU over the
+// whole batch, never less than one unit per wave and per block.
+SplitPlan plan_splits(int R, int hk, int max_kv_len) {
+    const int max_units = (max_kv_len + kUnitTokens - 1) / kUnitTokens;
+    if (max_units <= 0) return {1, 1};
+    const long long rows = static_cast<long long>(R) * hk;
+    const long long want_blocks = 2048;
+    long long want_split = (want_blocks + rows - 1) / rows;
+    if (want_split < 1) want_split = 1;
+    long long ups = (max_units + want_split - 1) / want_split;
+    if (ups < 2 * kAttnWaves) ups = 2 * kAttnWaves;  // >= 2 units per wave amortises the merge
+    if (ups > max_units) ups = max_units;
+    const int nsplit = static_cast<int>((max_units + ups - 1) / ups);
+    return {static_cast<int>(ups), nsplit};
+}
+
+template <int D, int GQA>
+int launch_decode(const uint16_t* q, const uint16_t* k_pages, const uint16_t* v_pages, uint16_t* o,
+                  float* lse, const uint32_t* page_indices, const uint32_t* page_indptr,
+                  const uint32_t* last_lens, int R, int hq, int hk, int ps, float sm_scale,
+                  int max_kv_len, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+    const SplitPlan plan = plan_splits(R, hk, max_kv_len);
+    const float scale_log2e = sm_scale * 1.4426950408889634f;
+    if (plan.nsplit == 1) {
+        hipLaunchKernelGGL((attn_decode_clear_empty_kernel<D>), dim3(R * hq), dim3(D), 0, stream,
+                           page_indptr, last_lens, o, lse, hq, ps);
+        hipLaunchKernelGGL((attn_decode_split_kernel<D, GQA>), dim3(1, hk, R), dim3(kAttnBlock), 0,
+                           stream, q, k_pages, v_pages, page_indices, page_indptr, last_lens,
+                           nullptr, nullptr, o, lse, hq, hk, ps, plan.units_per_split, 1,
+                           scale_log2e);
+        return launch_status();
+    }
+    const size_t n_part = static_cast<size_t>(R) * hq * plan.nsplit;
+    const size_t need = n_part * (D + 2) * sizeof(float);
+    if (!workspace || workspace_bytes < need) return PIE_HIP_ERR_INVALID;
+    float* part_o = static_cast<float*>(workspace);
+    float* part_ml = part_o + n_part * D;
+    hipLaunchKernelGGL((attn_decode_split_kernel<D, GQA>), dim3(plan.nsplit, hk, R),
+                       dim3(kAttnBlock), 0, stream, q, k_pages, v_pages, page_indices, page_indptr,
+                       last_lens, part_o, part_ml, nullptr, nullptr, hq, hk, ps,
+                       plan.units_per_split, plan.nsplit, scale_log2e);
+    hipLaunchKernelGGL((attn_decode_merge_kernel<D>), dim3(R * hq), dim3(D), 0, stream, part_o,
+                       part_ml, page_indptr, last_lens, o, lse, hq, ps, plan.units_per_split,
+                       plan.nsplit);
+    return launch_status();
+}
+
+}  // namespace
+}  // namespace pie_hip
+
+extern "C" size_t pie_hip_attn_decode_workspace_bytes(int num_requests, int num_q_heads,
+                                                      int num_kv_heads, int head_dim,
+                                                      int max_kv_len) {
+    if (num_requests <= 0 || num_q_heads <= 0 || num_kv_heads <= 0 || head_dim <= 0) return 0;
+    const pie_hip::SplitPlan plan = pie_hip::plan_splits(num_requests, num_kv_heads, max_kv_len);
+    if (plan.nsplit == 1) return 0;
+    return static_cast<size_t>(num_requests) * num_q_heads * plan.nsplit * (head_dim + 2) *
+           sizeof(float);
+}
+
+extern "C" int pie_hip_attn_decode_paged(const uint16_t* q, const uint16_t* k_pages,
+                                         const uint16_t* v_pages, uint16_t* o, float* lse,
+                                         const uint32_t* kv_page_indices,
+                                         const uint32_t* kv_page_indptr,
+                                         const uint32_t* kv_last_page_lens, int num_requests,
+                                         int num_q_heads, int num_kv_heads, int head_dim,
+                                         int page_size, float sm_scale, int max_kv_len,
+                                         void* workspace, size_t workspace_bytes, void* stream) {
+    using namespace pie_hip;
+    if (!q || !k_pages || !v_pages || !o || !kv_page_indices || !kv_page_indptr ||
+        !kv_last_page_lens || num_requests <= 0 || num_q_heads <= 0 || num_kv_heads <= 0 ||
+        page_size <= 0 || max_kv_len < 0)
+        return PIE_HIP_ERR_INVALID;
+    if (num_q_heads % num_kv_heads != 0 || page_size % kUnitTokens != 0)
+        return PIE_HIP_ERR_UNSUPPORTED;
+    if (num_requests > 65535 || num_kv_heads > 65535) return PIE_HIP_ERR_UNSUPPORTED;
+    const float scale = sm_scale > 0.f ? sm_scale : 1.0f / sqrtf(static_cast<float>(head_dim));
+    const int gqa = num_q_heads / num_kv_heads;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+#define PIE_ATTN_CASE(DD, GG)                                                                  \
+    if (head_dim == DD && gqa == GG)                                                           \
+        return launch_decode<DD, GG>(q, k_pages, v_pages, o, lse, kv_page_indices,             \
+                                     kv_page_indptr, kv_last_page_lens, num_requests,          \
+                                     num_q_heads, num_kv_heads, page_size, scale, max_kv_len,  \
+                                     workspace, workspace_bytes, st);
+    PIE_ATTN_CASE(128, 1)
+    PIE_ATTN_CASE(128, 2)
+    PIE_ATTN_CASE(128, 4)
+    PIE_ATTN_CASE(128, 8)
+    PIE_ATTN_CASE(64, 1)
+    PIE_ATTN_CASE(64, 2)
+    PIE_ATTN_CASE(64, 4)
+    PIE_ATTN_CASE(64, 8)
+#undef PIE_ATTN_CASE
+    return PIE_HIP_ERR_UNSUPPORTED;
+}

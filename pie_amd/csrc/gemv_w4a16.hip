@@ -53,7 +53,7 @@ __global__ __launch_bounds__(kBlock) void gemv_w4a16_kernel(
     extern __shared__ __align__(16) unsigned char smem[];
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
-    const int wv = tid / kWave;
+    const int wv = __builtin_amdgcn_readfirstlane(tid / kWave);  // wave-uniform -> SGPR
     const int nchunks = (K + kChunkK - 1) / kChunkK;
     const int nwords = K / 8;
     const int padded_words = nchunks * 256;

@@ -124,3 +124,48 @@ def gemv_w4a16(act: torch.Tensor, w: WeightView, y: Optional[torch.Tensor] = Non
                                     w.group_size, beta, _stream())
     _check(st, "pie_hip_gemv_w4a16")
     return y
+
+
+# ---------------------------------------------------------------- paged decode attention
+def attn_decode_workspace_bytes(R: int, hq: int, hk: int, d: int, max_kv_len: int) -> int:
+    lib = kernels()
+    lib.pie_hip_attn_decode_workspace_bytes.restype = C.c_size_t
+    return int(lib.pie_hip_attn_decode_workspace_bytes(R, hq, hk, d, max_kv_len))
+
+
+def attention_paged_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
+                           kv_page_indices: torch.Tensor, kv_page_indptr: torch.Tensor,
+                           kv_last_page_lens: torch.Tensor, max_kv_len: int,
+                           sm_scale: float = -1.0, o: Optional[torch.Tensor] = None,
+                           lse: Optional[torch.Tensor] = None,
+                           workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """o[R,hq,d] for one query token per request (launch_attention_naive_paged_decode,
+    driver/cuda/src/ops/attention_naive_paged.hpp:57-69).  Page-table tensors are int32
+    device tensors holding the wire u32 values."""
+    _dev(q, torch.bfloat16, "q")
+    _dev(k_pages, torch.bfloat16, "k_pages")
+    _dev(v_pages, torch.bfloat16, "v_pages")
+    for name, t in (("kv_page_indices", kv_page_indices), ("kv_page_indptr", kv_page_indptr),
+                    ("kv_last_page_lens", kv_last_page_lens)):
+        _dev(t, torch.int32, name)
+    R, hq, d = q.shape
+    num_pages, ps, hk, d2 = k_pages.shape
+    if d2 != d or v_pages.shape != k_pages.shape:
+        raise KernelError("k_pages/v_pages must be [pages, page_size, hk, d] with q's d")
+    if kv_page_indptr.numel() != R + 1 or kv_last_page_lens.numel() != R:
+        raise KernelError("page table arrays do not match the request count")
+    if o is None:
+        o = torch.empty_like(q)
+    _dev(o, torch.bfloat16, "o")
+    if lse is not None:
+        _dev(lse, torch.float32, "lse")
+    need = attn_decode_workspace_bytes(R, hq, hk, d, max_kv_len)
+    if workspace is None and need:
+        workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
+    wbytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    st = kernels().pie_hip_attn_decode_paged(
+        _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(o), _ptr(lse), _ptr(kv_page_indices),
+        _ptr(kv_page_indptr), _ptr(kv_last_page_lens), R, hq, hk, d, ps, C.c_float(sm_scale),
+        max_kv_len, _ptr(workspace), C.c_size_t(wbytes), _stream())
+    _check(st, "pie_hip_attn_decode_paged")
+    return o

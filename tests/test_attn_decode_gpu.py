@@ -1,0 +1,139 @@
+"""GPU parity: paged-KV decode attention through the C ABI vs the CPU oracle."""
+import numpy as np
+import pytest
+
+from paged_cases import make_paged_batch
+
+pytestmark = pytest.mark.gpu
+
+
+def run_gpu(gpu, q, b, hq, hk, d, ps, max_kv_len, sm_scale=-1.0, want_lse=True):
+    import torch
+
+    from pie_amd import ops
+
+    def dev(a, dt=None):
+        t = torch.from_numpy(np.ascontiguousarray(a)).to(gpu)
+        return t.view(dt) if dt is not None else t
+
+    R = q.shape[0]
+    lse = torch.empty((R, hq), dtype=torch.float32, device=gpu) if want_lse else None
+    o = ops.attention_paged_decode(
+        dev(q, torch.bfloat16), dev(b["k_pages"], torch.bfloat16), dev(b["v_pages"], torch.bfloat16),
+        dev(b["page_indices"].view(np.int32)), dev(b["page_indptr"].view(np.int32)),
+        dev(b["last_lens"].view(np.int32)), max_kv_len, sm_scale=sm_scale, lse=lse)
+    torch.cuda.synchronize()
+    return o.view(torch.uint16).cpu().numpy(), (lse.cpu().numpy() if want_lse else None)
+
+
+def check(oracle, o_bits, lse, q, b, hq, hk, d, ps, sm_scale=-1.0):
+    truth, _, lse64 = oracle.attn_decode_paged(q, b["k_pages"], b["v_pages"], b["page_indices"],
+                                               b["page_indptr"], b["last_lens"], hq, hk, d, ps,
+                                               sm_scale=sm_scale, mode=2)
+    got = oracle.bf16_to_f32(o_bits).astype(np.float64)
+    # one bf16 rounding of the output + fp32 softmax/accumulation error (V ~ N(0,1))
+    tol = 2.0 ** -8 * np.maximum(np.abs(truth), np.abs(got)) + 1e-4
+    err = np.abs(got - truth)
+    assert np.all(err <= tol), f"worst {np.max(err / tol):.2f}x tol at {np.argmax(err / tol)}"
+    if lse is not None:
+        fin = np.isfinite(lse64)
+        assert np.array_equal(np.isneginf(lse), np.isneginf(lse64))
+        assert np.allclose(lse[fin], lse64[fin], rtol=0, atol=1e-4)
+    # and within 1 bf16 ulp of the reference-order fp32 evaluation almost everywhere
+    _, o0, _ = oracle.attn_decode_paged(q, b["k_pages"], b["v_pages"], b["page_indices"],
+                                        b["page_indptr"], b["last_lens"], hq, hk, d, ps,
+                                        sm_scale=sm_scale, mode=0)
+    dd = np.abs(o_bits.astype(np.int32) - o0.astype(np.int32))
+    assert (dd <= 1).mean() > 0.99
+
+
+@pytest.mark.parametrize("hq,hk,d,ps", [
+    (32, 8, 128, 16), (8, 8, 128, 16), (16, 8, 128, 32), (32, 4, 128, 16),
+    (32, 8, 64, 16), (8, 4, 64, 32), (4, 4, 64, 16), (16, 2, 64, 16),
+])
+def test_decode_matches_oracle_ragged(gpu, oracle, hq, hk, d, ps):
+    rng = np.random.default_rng(hq * 1000 + hk * 100 + d + ps)
+    ctx = [1, 15, 16, 17, 31, 33, 64, 100, 257, 0, 1000, 5]
+    b = make_paged_batch(rng, ctx, hk, d, ps, f32_to_bf16=oracle.f32_to_bf16)
+    q = oracle.f32_to_bf16(rng.standard_normal((len(ctx), hq, d)).astype(np.float32))
+    o, lse = run_gpu(gpu, q, b, hq, hk, d, ps, max(ctx))
+    check(oracle, o, lse, q, b, hq, hk, d, ps)
+
+
+@pytest.mark.parametrize("max_kv_len", [64, 1024, 4096, 8192, 100000])
+def test_split_plans_agree(gpu, oracle, max_kv_len):
+    """Different max_kv_len bounds pick different split grids; the result must not depend on it
+    beyond fp32 merge rounding."""
+    rng = np.random.default_rng(31)
+    hq, hk, d, ps = 32, 8, 128, 16
+    ctx = [64, 1, 40, 17]
+    b = make_paged_batch(rng, ctx, hk, d, ps, f32_to_bf16=oracle.f32_to_bf16)
+    q = oracle.f32_to_bf16(rng.standard_normal((len(ctx), hq, d)).astype(np.float32))
+    o, lse = run_gpu(gpu, q, b, hq, hk, d, ps, max_kv_len)
+    check(oracle, o, lse, q, b, hq, hk, d, ps)
+
+
+def test_single_request_long_context_and_scale(gpu, oracle):
+    rng = np.random.default_rng(32)
+    hq, hk, d, ps = 32, 8, 128, 16
+    ctx = [2048 + 7]
+    b = make_paged_batch(rng, ctx, hk, d, ps, f32_to_bf16=oracle.f32_to_bf16)
+    q = oracle.f32_to_bf16(rng.standard_normal((1, hq, d)).astype(np.float32))
+    for scale in (-1.0, 0.05, 0.25):
+        o, lse = run_gpu(gpu, q, b, hq, hk, d, ps, ctx[0], sm_scale=scale)
+        check(oracle, o, lse, q, b, hq, hk, d, ps, sm_scale=scale)
+
+
+def test_forked_prefix_equals_private_copies(gpu, oracle):
+    rng = np.random.default_rng(33)
+    hq, hk, d, ps = 32, 8, 128, 16
+    ctx = [1024 + 300, 1024 + 5, 1024, 700, 1500, 1024 + 64, 90, 2000]
+    b = make_paged_batch(rng, ctx, hk, d, ps, shared_prefix_tokens=1024, shared_fraction=0.5,
+                         f32_to_bf16=oracle.f32_to_bf16)
+    assert len(b["sharers"]) == 4
+    q = oracle.f32_to_bf16(rng.standard_normal((len(ctx), hq, d)).astype(np.float32))
+    o, lse = run_gpu(gpu, q, b, hq, hk, d, ps, max(ctx))
+    check(oracle, o, lse, q, b, hq, hk, d, ps)
+    # private copies at other physical pages: bit-identical output
+    total = int(b["page_indptr"][-1])
+    perm = rng.permutation(total + 5).astype(np.uint32)[:total]
+    b2 = dict(b)
+    b2["k_pages"] = np.zeros((total + 5, ps, hk, d), np.uint16)
+    b2["v_pages"] = np.zeros_like(b2["k_pages"])
+    b2["k_pages"][perm] = b["k_pages"][b["page_indices"]]
+    b2["v_pages"][perm] = b["v_pages"][b["page_indices"]]
+    b2["page_indices"] = perm
+    o2, _ = run_gpu(gpu, q, b2, hq, hk, d, ps, max(ctx))
+    assert np.array_equal(o, o2)
+
+
+def test_garbage_in_unused_slots_is_ignored(gpu, oracle):
+    """Slots past kv_len in the last page may hold NaN/Inf bit patterns."""
+    rng = np.random.default_rng(34)
+    hq, hk, d, ps = 8, 2, 128, 16
+    ctx = [21, 3]
+    b = make_paged_batch(rng, ctx, hk, d, ps, f32_to_bf16=oracle.f32_to_bf16)
+    q = oracle.f32_to_bf16(rng.standard_normal((2, hq, d)).astype(np.float32))
+    o_clean, _ = run_gpu(gpu, q, b, hq, hk, d, ps, 32)
+    for r, c in enumerate(ctx):
+        last_page = b["page_indices"][b["page_indptr"][r + 1] - 1]
+        b["k_pages"][last_page, c % ps:] = 0x7FC0  # NaN
+        b["v_pages"][last_page, c % ps:] = 0x7F80  # +Inf
+    o, lse = run_gpu(gpu, q, b, hq, hk, d, ps, 32)
+    assert np.array_equal(o, o_clean)
+    assert np.all(np.isfinite(lse))
+
+
+def test_baseline_shape_batch64(gpu, oracle):
+    """BASELINE attention config: 32q/8kv d128 page 16, batch 64, ctx U[512,8192], 25% of the
+    sequences share a forked 1024-token prefix.  Oracle on a sample of requests (fp64), plus
+    the forked-prefix and LSE invariants on all."""
+    rng = np.random.default_rng(35)
+    hq, hk, d, ps = 32, 8, 128, 16
+    ctx = rng.integers(512, 8193, size=64)
+    ctx[:16] = np.maximum(ctx[:16], 1024)
+    b = make_paged_batch(rng, ctx, hk, d, ps, shared_prefix_tokens=1024, shared_fraction=0.25,
+                         f32_to_bf16=oracle.f32_to_bf16)
+    q = oracle.f32_to_bf16(rng.standard_normal((64, hq, d)).astype(np.float32))
+    o, lse = run_gpu(gpu, q, b, hq, hk, d, ps, int(ctx.max()))
+    check(oracle, o, lse, q, b, hq, hk, d, ps)
