@@ -69,6 +69,41 @@ int pie_hip_dequant_w4a16(const uint32_t* packed, const uint16_t* scale_bf16,
 int pie_hip_gemv_w4a16(const uint16_t* act_bf16, const uint32_t* packed,
                        const uint16_t* scale_bf16, uint16_t* y_bf16, int M, int N, int K,
                        int group_size, int beta, void* stream);
+/* Same contract with explicit tiling (rows walked per wave step, resident waves per SIMD;
+ * 0 = library default).  For tuning sweeps; no reference counterpart. */
+int pie_hip_gemv_w4a16_tuned(const uint16_t* act_bf16, const uint32_t* packed,
+                             const uint16_t* scale_bf16, uint16_t* y_bf16, int M, int N, int K,
+                             int group_size, int beta, int rows_per_wave, int waves_per_simd,
+                             void* stream);
+
+/*
+ * Weight-only int8 GEMV (W8A16), per-output-channel scale:
+ *   y[m, n] = bf16( beta*y[m, n] + (sum_k f32(act[m,k]) * f32(q[n,k])) * scale_inv[n] )
+ * fp32 sum, scale applied once after it — the evaluation order of the reference's own
+ * weight-only int8 GEMV (driver/cuda/src/kernels/argmax.cu:846-854).  q: int8 [N,K];
+ * scale_inv (= absmax/127, driver/cuda/src/kernels/quant_bf16_to_fp8.cu:311-313) is given
+ * as f32 [N] or as bf16 [N]: pass exactly one of the two pointers.  K % 16 == 0, M <= 32.
+ */
+int pie_hip_gemv_w8a16(const uint16_t* act_bf16, const int8_t* w_int8,
+                       const float* scale_inv_f32, const uint16_t* scale_inv_bf16,
+                       uint16_t* y_bf16, int M, int N, int K, int beta, void* stream);
+
+/*
+ * Weight-only fp8 (OCP e4m3fn bytes) GEMV with per-output-channel scale, same shape rules
+ * and scale arguments as the int8 entry point.  Format:
+ * driver/cuda/src/kernels/dequant_fp8.cu:25-39 (w = fp8 * scale_inv[row]).
+ */
+int pie_hip_gemv_fp8(const uint16_t* act_bf16, const uint8_t* w_e4m3,
+                     const float* scale_inv_f32, const uint16_t* scale_inv_bf16,
+                     uint16_t* y_bf16, int M, int N, int K, int beta, void* stream);
+
+/*
+ * bf16 GEMV: y[m, n] = bf16( beta*y + sum_k act[m,k]*W[n,k] ), fp32 accumulation
+ * (gemm_act_x_w bf16 path, driver/cuda/src/ops/gemm.hpp:152-160; the lm_head and router
+ * projections stay unquantised in the reference).  K % 8 == 0, M <= 32.
+ */
+int pie_hip_gemv_bf16(const uint16_t* act_bf16, const uint16_t* w_bf16, uint16_t* y_bf16, int M,
+                      int N, int K, int beta, void* stream);
 
 /* ---- paged-KV decode attention -------------------------------------------- */
 
@@ -100,6 +135,64 @@ int pie_hip_attn_decode_paged(const uint16_t* q, const uint16_t* k_pages, const 
                               int num_requests, int num_q_heads, int num_kv_heads, int head_dim,
                               int page_size, float sm_scale, int max_kv_len, void* workspace,
                               size_t workspace_bytes, void* stream);
+
+/* ---- per-layer kernels of the llama-like decoder ---------------------------- */
+
+/* y[n,:] = table[token_ids[n],:]; ids >= vocab read row 0.
+ * Reference: launch_embed_bf16, driver/cuda/src/kernels/embed.cu:8-23. */
+int pie_hip_embed(const uint32_t* token_ids, const uint16_t* table_bf16, uint16_t* y_bf16,
+                  int num_tokens, int hidden, int vocab, void* stream);
+
+/* y = bf16( x * rsqrt(mean(x^2) + eps) * w ), fp32 inside.  hidden % 8 == 0.
+ * Reference: rmsnorm_bf16_kernel, driver/cuda/src/kernels/rmsnorm.cu:14-54. */
+int pie_hip_rmsnorm(const uint16_t* x_bf16, const uint16_t* weight_bf16, uint16_t* y_bf16,
+                    int rows, int hidden, float eps, void* stream);
+
+/* hidden = bf16(hidden + residual) (stored), norm_out = rmsnorm(hidden) of the rounded sum.
+ * Reference: residual_add_rmsnorm_bf16_kernel, driver/cuda/src/kernels/rmsnorm.cu:56-98. */
+int pie_hip_residual_rmsnorm(uint16_t* hidden_bf16, const uint16_t* residual_bf16,
+                             const uint16_t* weight_bf16, uint16_t* norm_out_bf16, int rows,
+                             int hidden, float eps, void* stream);
+
+/* table[n, i] = cos(positions[n] * inv_freq[i]); table[n, i + d/2] = sin(same), i < d/2,
+ * angle and sincos in fp32.  inv_freq[d/2] is a host table (theta^(-2i/d), optionally with
+ * llama3 band scaling, driver/portable/src/model.cpp:1414-1448).
+ * Reference: rope_standard_table_kernel, driver/cuda/src/kernels/rope.cu:35-53. */
+int pie_hip_rope_table(const int32_t* positions, const float* inv_freq, float* table,
+                       int num_tokens, int head_dim, void* stream);
+
+/*
+ * Split a packed QKV row [N, (hq + 2*hk)*d], apply optional per-head RMSNorm (both norm
+ * weights or neither) and RoPE to q and k, write q to q_out[N, hq, d], and write k (rotated)
+ * and v (copied) into the KV pool [pages, page_size, hk, d] at physical slot
+ * kv_slots[n] = page*page_size + offset (negative = token has no slot).  One bf16 rounding at
+ * the store.  interleaved: 0 pairs (i, i+d/2), 1 pairs (2i, 2i+1).
+ * Reference: launch_qkv_decode_qk_norm_rope_write_kv_bf16,
+ * driver/cuda/src/kernels/split_packed.hpp:34-57, split_packed.cu:62-178; slot arithmetic of
+ * driver/portable/src/plan.hpp:36-45 is done by the caller.
+ */
+int pie_hip_qkv_rope_kvwrite(const uint16_t* packed_qkv, uint16_t* q_out, uint16_t* k_pages,
+                             uint16_t* v_pages, const uint16_t* q_norm_weight,
+                             const uint16_t* k_norm_weight, const float* rope_table,
+                             const int64_t* kv_slots, int num_tokens, int num_q_heads,
+                             int num_kv_heads, int head_dim, int interleaved, float eps,
+                             void* stream);
+
+/* y[n, i] = bf16( g/(1+exp(-g)) * u ), g = gate_up[n, i], u = gate_up[n, I + i].
+ * Reference: swiglu_bf16_kernel, driver/cuda/src/kernels/swiglu.cu:9-22 (fused-row form
+ * swiglu.hpp:82). */
+int pie_hip_swiglu(const uint16_t* gate_up_bf16, uint16_t* y_bf16, int num_tokens,
+                   int intermediate, void* stream);
+
+/* out_idx[r] = argmax_i logits[r, i]; ties -> lowest index; NaN never wins.  vocab % 8 == 0.
+ * Reference: argmax_bf16_kernel, driver/cuda/src/kernels/argmax.cu:36-80. */
+int pie_hip_argmax(const uint16_t* logits_bf16, uint32_t* out_idx, int rows, int vocab,
+                   void* stream);
+
+/* pool page dst_pages[i] <- page src_pages[i] (device arrays), page_bytes each, in one pool.
+ * Reference: Copy D2D handling, driver/portable/src/service/inproc_service.cpp:149-172. */
+int pie_hip_copy_kv_pages(void* pool, const uint32_t* src_pages, const uint32_t* dst_pages,
+                          int num_copies, size_t page_bytes, void* stream);
 
 #ifdef __cplusplus
 }

@@ -175,3 +175,121 @@ def kv_write(k_curr, v_curr, k_pages, v_pages, qo_indptr, page_indices, page_ind
     ll = _c(last_lens, np.uint32)
     lib().orc_kv_write(_p(kc), _p(vc), _p(k_pages), _p(v_pages), _p(qo), _p(pi), _p(pp), _p(ll),
                        C.c_int(len(ll)), C.c_int(hk), C.c_int(d), C.c_int(ps))
+
+
+# ---------------------------------------------------------------- per-layer ops
+def embed(tokens, table_bf16, vocab=None):
+    t = _c(tokens, np.uint32)
+    tab = _c(table_bf16, np.uint16)
+    V, H = tab.shape
+    y = np.empty((len(t), H), np.uint16)
+    lib().orc_embed(_p(t), _p(tab), _p(y), C.c_int(len(t)), C.c_int(H), C.c_int(vocab or V))
+    return y
+
+
+def rmsnorm(x_bf16, w_bf16, eps, residual=None):
+    """Returns y (and the updated x when a residual is given)."""
+    x = np.array(x_bf16, dtype=np.uint16, order="C", copy=True)
+    rows, H = x.shape
+    w = _c(w_bf16, np.uint16)
+    r = None if residual is None else _c(residual, np.uint16)
+    y = np.empty_like(x)
+    lib().orc_rmsnorm(_p(x), _p(r), _p(w), _p(y), C.c_int(rows), C.c_int(H), C.c_float(eps))
+    return y if residual is None else (y, x)
+
+
+def rope_inv_freq(d, theta, factor=0.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                  original_max_pos=8192):
+    out = np.empty((d // 2,), np.float32)
+    lib().orc_rope_inv_freq(_p(out), C.c_int(d), C.c_float(theta), C.c_float(factor),
+                            C.c_float(low_freq_factor), C.c_float(high_freq_factor),
+                            C.c_int(original_max_pos))
+    return out
+
+
+def rope_table(positions, inv_freq, d):
+    pos = _c(positions, np.int32)
+    f = _c(inv_freq, np.float32)
+    tab = np.empty((len(pos), d), np.float32)
+    lib().orc_rope_table(_p(pos), _p(f), _p(tab), C.c_int(len(pos)), C.c_int(d))
+    return tab
+
+
+def qkv_rope_kvwrite(packed, k_pages, v_pages, table, kv_slots, hq, hk, d, interleaved,
+                     q_norm_w=None, k_norm_w=None, eps=1e-6):
+    """Returns q_out; k_pages / v_pages (uint16, C-contiguous) are updated in place."""
+    pk = _c(packed, np.uint16)
+    N = pk.shape[0]
+    q_out = np.zeros((N, hq, d), np.uint16)
+    tab = _c(table, np.float32)
+    sl = _c(kv_slots, np.int64)
+    assert k_pages.dtype == np.uint16 and k_pages.flags.c_contiguous
+    assert v_pages.dtype == np.uint16 and v_pages.flags.c_contiguous
+    qn = None if q_norm_w is None else _c(q_norm_w, np.uint16)
+    kn = None if k_norm_w is None else _c(k_norm_w, np.uint16)
+    lib().orc_qkv_rope_kvwrite(_p(pk), _p(q_out), _p(k_pages), _p(v_pages), _p(qn), _p(kn), _p(tab),
+                               _p(sl), C.c_int(N), C.c_int(hq), C.c_int(hk), C.c_int(d),
+                               C.c_int(interleaved), C.c_float(eps))
+    return q_out
+
+
+def swiglu(gate_up_bf16):
+    gu = _c(gate_up_bf16, np.uint16)
+    N, two_i = gu.shape
+    y = np.empty((N, two_i // 2), np.uint16)
+    lib().orc_swiglu(_p(gu), _p(y), C.c_int(N), C.c_int(two_i // 2))
+    return y
+
+
+def argmax_bf16(logits_bf16):
+    lg = _c(logits_bf16, np.uint16)
+    rows, V = lg.shape
+    out = np.empty((rows,), np.uint32)
+    lib().orc_argmax_bf16(_p(lg), _p(out), C.c_int(rows), C.c_int(V))
+    return out
+
+
+def gemm_bf16(act_bf16, w_bf16, mode: int = 0, y_in=None, want_abs: bool = False):
+    act = _c(act_bf16, np.uint16)
+    M, K = act.shape
+    w = _c(w_bf16, np.uint16)
+    N = w.shape[0]
+    y32 = np.empty((M, N), np.float32)
+    y16 = np.empty((M, N), np.uint16)
+    ab = np.empty((M, N), np.float64) if want_abs else None
+    yin = None if y_in is None else _c(y_in, np.uint16)
+    lib().orc_gemm_bf16(_p(act), _p(w), _p(yin), _p(y32), _p(y16), _p(ab), C.c_int(M), C.c_int(N),
+                        C.c_int(K), C.c_int(0 if y_in is None else 1), C.c_int(mode))
+    return (y32, y16, ab) if want_abs else (y32, y16)
+
+
+# ---------------------------------------------------------------- fp8 e4m3fn per channel
+def fp8_decode(b) -> np.ndarray:
+    b = _c(b, np.uint8)
+    out = np.empty(b.shape, np.float32)
+    lib().orc_fp8_decode(_p(b), _p(out), C.c_size_t(b.size))
+    return out
+
+
+def quant_fp8_per_channel(w_bf16):
+    w = _c(w_bf16, np.uint16)
+    rows, cols = w.shape
+    q = np.empty((rows, cols), np.uint8)
+    s = np.empty((rows,), np.float32)
+    lib().orc_quant_fp8_per_channel(_p(w), _p(q), _p(s), C.c_int(rows), C.c_int(cols))
+    return q, s
+
+
+def gemm_fp8(act_bf16, q, scale_inv, mode: int = 0, y_in=None, want_abs: bool = False):
+    act = _c(act_bf16, np.uint16)
+    M, K = act.shape
+    q = _c(q, np.uint8)
+    N = q.shape[0]
+    s = _c(scale_inv, np.float32)
+    y32 = np.empty((M, N), np.float32)
+    y16 = np.empty((M, N), np.uint16)
+    ab = np.empty((M, N), np.float64) if want_abs else None
+    yin = None if y_in is None else _c(y_in, np.uint16)
+    lib().orc_gemm_fp8(_p(act), _p(q), _p(s), _p(yin), _p(y32), _p(y16), _p(ab), C.c_int(M),
+                       C.c_int(N), C.c_int(K), C.c_int(0 if y_in is None else 1), C.c_int(mode))
+    return (y32, y16, ab) if want_abs else (y32, y16)

@@ -162,3 +162,94 @@ void orc_gemm_w8a16(const uint16_t* act, const int8_t* q, const float* scale_inv
         }
     }
 }
+
+/*
+ * OCP fp8 e4m3fn byte -> f32: sign, 4-bit exponent (bias 7), 3-bit mantissa, subnormals at
+ * exponent 0, no infinities, 0x7F/0xFF = NaN (the hardware conversion; the reference's host
+ * table at driver/portable/src/rust_loader.cpp:783-793 maps the NaN code to 0 instead — a
+ * code no satfinite quantiser emits).
+ */
+float orc_fp8_e4m3_to_f32(uint8_t v) {
+    const float sign = (v & 0x80) ? -1.0f : 1.0f;
+    const int exp = (v >> 3) & 0x0f, mant = v & 0x07;
+    if (exp == 0) return sign * ldexpf((float)mant / 8.0f, -6);
+    if (exp == 0x0f && mant == 0x07) return NAN;
+    return sign * ldexpf(1.0f + (float)mant / 8.0f, exp - 7);
+}
+
+void orc_fp8_decode(const uint8_t* src, float* dst, size_t n) {
+    for (size_t i = 0; i < n; ++i) dst[i] = orc_fp8_e4m3_to_f32(src[i]);
+}
+
+/* f32 -> e4m3fn, round to nearest even, saturating to +-448 (__NV_SATFINITE). */
+uint8_t orc_f32_to_fp8_e4m3(float f) {
+    if (f != f) return 0x7F;
+    const uint8_t sign = signbit(f) ? 0x80 : 0x00;
+    const float a = fabsf(f);
+    if (a >= 448.0f) return sign | 0x7E;
+    uint8_t best = 0;
+    float best_err = INFINITY;
+    for (int c = 0; c <= 0x7E; ++c) {
+        const float err = fabsf(orc_fp8_e4m3_to_f32((uint8_t)c) - a);
+        if (err < best_err || (err == best_err && (c & 1) == 0)) {
+            best_err = err;
+            best = (uint8_t)c;
+        }
+    }
+    return sign | best;
+}
+
+/* Per-row fp8 quantiser: scale_inv = absmax/448 (1 if the row is zero),
+ * q = e4m3_satfinite(w * 448/absmax).  quant_bf16_to_fp8.cu:181-226. */
+void orc_quant_fp8_per_channel(const uint16_t* w_bf16, uint8_t* q, float* scale_inv, int rows,
+                               int cols) {
+#pragma omp parallel for schedule(static)
+    for (int r = 0; r < rows; ++r) {
+        float absmax = 0.f;
+        for (int c = 0; c < cols; ++c) {
+            const float v = fabsf(orc_bf16_to_f32(w_bf16[(size_t)r * cols + c]));
+            if (v > absmax) absmax = v;
+        }
+        const float inv = absmax > 0.f ? 448.0f / absmax : 1.f;
+        scale_inv[r] = absmax > 0.f ? absmax / 448.0f : 1.f;
+        for (int c = 0; c < cols; ++c)
+            q[(size_t)r * cols + c] =
+                orc_f32_to_fp8_e4m3(orc_bf16_to_f32(w_bf16[(size_t)r * cols + c]) * inv);
+    }
+}
+
+/*
+ * fp8 weight-only linear, per-row scale:
+ *   mode 0  fused: (sum_k x * f32(fp8)) * scale_inv[n], fp32 sum
+ *   mode 1  dequant-then-GEMM: w = bf16(f32(fp8) * s) (dequant_fp8.cu:25-39), fp32 accumulation
+ *   mode 2  fp64 ground truth
+ */
+void orc_gemm_fp8(const uint16_t* act, const uint8_t* q, const float* scale_inv,
+                  const uint16_t* y_in, float* y_f32, uint16_t* y_bf16, double* abs_sum, int M,
+                  int N, int K, int beta, int mode) {
+#pragma omp parallel for schedule(static)
+    for (int n = 0; n < N; ++n) {
+        for (int m = 0; m < M; ++m) {
+            float accf = 0.f;
+            double accd = 0.0, absd = 0.0;
+            const float s = scale_inv[n];
+            for (int k = 0; k < K; ++k) {
+                const float x = orc_bf16_to_f32(act[(size_t)m * K + k]);
+                const float w = orc_fp8_e4m3_to_f32(q[(size_t)n * K + k]);
+                if (mode == 0) accf += x * w;
+                else if (mode == 1) accf += x * orc_round_bf16(w * s);
+                else accd += (double)x * (double)w;
+                absd += fabs((double)x * (double)w * (double)s);
+            }
+            double v;
+            if (mode == 0) v = (double)(accf * s);
+            else if (mode == 1) v = (double)accf;
+            else v = accd * (double)s;
+            const size_t o = (size_t)m * N + n;
+            if (beta) v += (double)orc_bf16_to_f32(y_in[o]);
+            y_f32[o] = (float)v;
+            if (y_bf16) y_bf16[o] = orc_f32_to_bf16((float)v);
+            if (abs_sum) abs_sum[o] = absd;
+        }
+    }
+}

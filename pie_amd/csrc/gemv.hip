@@ -1,0 +1,456 @@
+// Weight-streaming GEMV / skinny GEMM for decode on gfx950, one kernel template
+// for every weight storage format of the forward pass:
+//
+//   int4b8  W4A16, group scales    driver/cuda/src/kernels/dequant_wna16.cu:11-38, :96-110
+//   int8    W8A16, per-row scale   driver/cuda/src/kernels/argmax.cu:846-854 (fused order:
+//                                  scale applied once after the fp32 sum)
+//   fp8     e4m3fn, per-row scale  driver/cuda/src/kernels/dequant_fp8.cu:25-39
+//   bf16    plain                  gemm_act_x_w bf16 path, driver/cuda/src/ops/gemm.hpp:152-160
+//
+// y[m, n] = bf16( beta*y[m, n] + sum_k act[m, k] * w(n, k) ), fp32 accumulation.
+//
+// HBM-bound design (the N*K weight bytes dominate):
+//   * the grid is sized to the machine, not to the problem: `waves_per_simd`
+//     resident waves on each of the 1024 SIMDs, every wave owning one contiguous,
+//     balanced slice of the output rows, so all CUs start and finish together;
+//   * a wave walks its slice R rows at a time; every lane streams 16-byte pieces of
+//     each row, so one wave instruction covers 1 KiB of a row, fully coalesced.
+//     Loads are branch-free and issued one work unit (R rows x one 1 KiB chunk)
+//     ahead of the arithmetic, so 2R independent 16 B loads per lane are in flight
+//     while the previous unit is being reduced;
+//   * the first unit is requested before the activation row is staged, so the
+//     HBM latency of the weights overlaps the LDS staging;
+//   * activations are staged once per block into LDS in exactly the order the
+//     format's in-register decode produces weights, laid out so a lane's 16 B LDS
+//     reads are conflict free;
+//   * int4: nibbles become bf16 by OR-ing the exponent of 128.0 onto them,
+//     ((w >> 4j) & 0x000F000F) | 0x43004300 = (128+n_j, 128+n_{j+4}), and the dot
+//     product runs on v_dot2_f32_bf16 from an accumulator preset to -136*sum(x),
+//     which makes the result sum x*(n-8) exactly as the format defines; the bf16
+//     group scale multiplies each lane's 32-weight partial sum;
+//   * int8: bytes are flipped to offset binary (w ^ 0x80808080) so the byte->f32
+//     conversion instruction decodes them, with -128*sum(x) preset the same way;
+//   * fp8: the packed e4m3 -> f32 conversion instruction decodes two weights each;
+//   * bf16: weights feed v_dot2_f32_bf16 directly;
+//   * a wave64 butterfly finishes the row; the lane that stores an output has
+//     prefetched the residual / row scale it needs with the unit's loads.
+#include "common.hip.h"
+
+namespace pie_hip {
+namespace {
+
+constexpr int kBlock = 256;  // 4 waves: one per SIMD of a CU
+constexpr int kWavesPerBlock = kBlock / kWave;
+constexpr int kNumCU = 256;
+
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+
+// ---- weight formats ---------------------------------------------------------
+// WPP: weights in one 16-byte piece.  XV: 16-byte LDS vectors of staged activations
+// a lane reads per piece.  stage(): the XV vectors for the piece starting at k0, from
+// the bf16 activation row.  dot(): p += sum over the piece of x*w(raw).  sum_x():
+// the sum of the staged activations of a piece (only when kBias != 0).
+
+struct FmtInt4 {
+    static constexpr int WPP = 32, XV = 4;
+    static constexpr bool kGroupScale = true, kRowScale = false;
+    static constexpr float kBias = -136.f;
+    // vector i holds word i's 8 activations as pairs (0,4)(1,5)(2,6)(3,7)
+    static __device__ __forceinline__ u32x4_t stage(const uint16_t* row, int k0, int i) {
+        const u32x4_t v = *reinterpret_cast<const u32x4_t*>(row + k0 + 8 * i);
+        u32x4_t p;
+        p.x = (v.x & 0xFFFFu) | (v.z << 16);
+        p.y = (v.x >> 16) | (v.z & 0xFFFF0000u);
+        p.z = (v.y & 0xFFFFu) | (v.w << 16);
+        p.w = (v.y >> 16) | (v.w & 0xFFFF0000u);
+        return p;
+    }
+    static __device__ __forceinline__ float sum_x(const u32x4_t* xs) {
+        float s = 0.f;
+#pragma unroll
+        for (int i = 0; i < XV; ++i)
+            s += bf16_lo(xs[i].x) + bf16_hi(xs[i].x) + bf16_lo(xs[i].y) + bf16_hi(xs[i].y) +
+                 bf16_lo(xs[i].z) + bf16_hi(xs[i].z) + bf16_lo(xs[i].w) + bf16_hi(xs[i].w);
+        return s;
+    }
+    static __device__ __forceinline__ float dot(const u32x4_t w, const u32x4_t* xs, float p) {
+        constexpr uint32_t kMask = 0x000F000Fu, k128 = 0x43004300u;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t v = w[i];
+            p = dot2_bf16(xs[i].x, (v & kMask) | k128, p);
+            p = dot2_bf16(xs[i].y, ((v >> 4) & kMask) | k128, p);
+            p = dot2_bf16(xs[i].z, ((v >> 8) & kMask) | k128, p);
+            p = dot2_bf16(xs[i].w, ((v >> 12) & kMask) | k128, p);
+        }
+        return p;
+    }
+};
+
+struct FmtBf16 {
+    static constexpr int WPP = 8, XV = 1;
+    static constexpr bool kGroupScale = false, kRowScale = false;
+    static constexpr float kBias = 0.f;
+    static __device__ __forceinline__ u32x4_t stage(const uint16_t* row, int k0, int) {
+        return *reinterpret_cast<const u32x4_t*>(row + k0);
+    }
+    static __device__ __forceinline__ float sum_x(const u32x4_t*) { return 0.f; }
+    static __device__ __forceinline__ float dot(const u32x4_t w, const u32x4_t* xs, float p) {
+        p = dot2_bf16(xs[0].x, w.x, p);
+        p = dot2_bf16(xs[0].y, w.y, p);
+        p = dot2_bf16(xs[0].z, w.z, p);
+        p = dot2_bf16(xs[0].w, w.w, p);
+        return p;
+    }
+};
+
+// 16 weights per piece, activations staged as f32 in natural order.
+struct FmtF32Act {
+    static constexpr int WPP = 16, XV = 4;
+    static __device__ __forceinline__ u32x4_t stage(const uint16_t* row, int k0, int i) {
+        const u32x2_t v = *reinterpret_cast<const u32x2_t*>(row + k0 + 4 * i);
+        return u32x4_t{v.x << 16, v.x & 0xFFFF0000u, v.y << 16, v.y & 0xFFFF0000u};
+    }
+    static __device__ __forceinline__ float sum_x(const u32x4_t* xs) {
+        float s = 0.f;
+#pragma unroll
+        for (int i = 0; i < XV; ++i)
+            s += __uint_as_float(xs[i].x) + __uint_as_float(xs[i].y) + __uint_as_float(xs[i].z) +
+                 __uint_as_float(xs[i].w);
+        return s;
+    }
+};
+
+// Row scale stored as f32 (SB = false) or bf16 (SB = true).
+template <bool SB>
+struct RowScale {
+    static __device__ __forceinline__ float load(const void* p, int row) {
+        if (SB) return bf16_bits_to_f32(static_cast<const uint16_t*>(p)[row]);
+        return static_cast<const float*>(p)[row];
+    }
+};
+
+template <bool SB>
+struct FmtInt8 : FmtF32Act, RowScale<SB> {
+    static constexpr bool kGroupScale = false, kRowScale = true;
+    static constexpr float kBias = -128.f;
+    static __device__ __forceinline__ float dot(const u32x4_t w, const u32x4_t* xs, float p) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t u = w[i] ^ 0x80808080u;  // int8 -> offset binary
+            p = fmaf(__uint_as_float(xs[i].x), static_cast<float>(u & 0xFFu), p);
+            p = fmaf(__uint_as_float(xs[i].y), static_cast<float>((u >> 8) & 0xFFu), p);
+            p = fmaf(__uint_as_float(xs[i].z), static_cast<float>((u >> 16) & 0xFFu), p);
+            p = fmaf(__uint_as_float(xs[i].w), static_cast<float>(u >> 24), p);
+        }
+        return p;
+    }
+};
+
+template <bool SB>
+struct FmtFp8 : FmtF32Act, RowScale<SB> {
+    static constexpr bool kGroupScale = false, kRowScale = true;
+    static constexpr float kBias = 0.f;
+    static __device__ __forceinline__ float dot(const u32x4_t w, const u32x4_t* xs, float p) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const f32x2_t lo = __builtin_amdgcn_cvt_pk_f32_fp8(w[i], false);
+            const f32x2_t hi = __builtin_amdgcn_cvt_pk_f32_fp8(w[i], true);
+            p = fmaf(__uint_as_float(xs[i].x), lo.x, p);
+            p = fmaf(__uint_as_float(xs[i].y), lo.y, p);
+            p = fmaf(__uint_as_float(xs[i].z), hi.x, p);
+            p = fmaf(__uint_as_float(xs[i].w), hi.y, p);
+        }
+        return p;
+    }
+};
+
+template <int R>
+struct Unit {
+    u32x4_t w[R];
+    uint16_t gs[R];  // group scale (int4)
+    uint16_t prev;   // y element this lane may add to (lane = r*M + m), for beta = 1
+    float rs;        // row scale for that lane's row (int8 / fp8)
+};
+
+struct GemvArgs {
+    const uint16_t* act;
+    const u32x4_t* w;
+    const uint16_t* gscale;  // bf16 [N, K/G]        (int4)
+    const void* rscale;      // f32 or bf16 [N]      (int8 / fp8)
+    uint16_t* y;
+    int N, K, G, beta;
+};
+
+template <class F, int R, int M>
+__global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
+    constexpr int WPP = F::WPP, XV = F::XV;
+    constexpr int kChunkK = kWave * WPP;  // weights covered by one wave-wide 16 B load
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wv = __builtin_amdgcn_readfirstlane(tid / kWave);  // wave-uniform -> SGPR
+    const int N = a.N, K = a.K;
+    const int nchunks = (K + kChunkK - 1) / kChunkK;
+    const int vec_per_m = nchunks * XV * kWave;
+    const int row_stride_v4 = K / WPP;
+    const int groups_per_row = F::kGroupScale ? K / a.G : 0;
+
+    u32x4_t* lds_x = reinterpret_cast<u32x4_t*>(smem);               // [M][nchunks][XV][64]
+    float* lds_sx = reinterpret_cast<float*>(lds_x + M * vec_per_m);  // [M][nchunks][64]
+
+    // Balanced contiguous row slice of this wave.
+    const long long total_waves = static_cast<long long>(gridDim.x) * kWavesPerBlock;
+    const long long wg = static_cast<long long>(blockIdx.x) * kWavesPerBlock + wv;
+    const int row_begin = static_cast<int>(wg * N / total_waves);
+    const int row_end = static_cast<int>((wg + 1) * N / total_waves);
+    const int ngroups = (row_end - row_begin + R - 1) / R;
+    const int nunits = ngroups * nchunks;
+
+    // Branch-free loads: lanes past K re-read lane 0's piece and are masked out in compute;
+    // rows past the slice re-read its last row and are dropped at the store.
+    auto issue = [&](Unit<R>& u, int g, int c) {
+        const int kbase = c * kChunkK + lane * WPP;
+        const bool valid = kbase < K;
+        const int piece = valid ? c * kWave + lane : 0;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int row = min(row_begin + g * R + r, row_end - 1);
+            u.w[r] = __builtin_nontemporal_load(a.w + static_cast<size_t>(row) * row_stride_v4 +
+                                                piece);
+            if constexpr (F::kGroupScale)
+                u.gs[r] = a.gscale[static_cast<size_t>(row) * groups_per_row +
+                                   (valid ? kbase / a.G : 0)];
+        }
+        // Every unit prefetches what the lane that finishes an output needs, so the
+        // epilogue never stalls the pipeline (only the last chunk's values are used).
+        const int lr = lane < R * M ? lane / M : 0;
+        const int lm = lane < R * M ? lane % M : 0;
+        const int lrow = min(row_begin + g * R + lr, row_end - 1);
+        u.prev = a.y[static_cast<size_t>(lm) * N + lrow];
+        if constexpr (F::kRowScale) u.rs = F::load(a.rscale, lrow);
+    };
+
+    Unit<R> ua, ub;
+    if (nunits > 0) issue(ua, 0, 0);
+
+    // Stage activations in the format's decode order.
+    for (int v = tid; v < M * vec_per_m; v += kBlock) {
+        const int m = v / vec_per_m;
+        const int rem = v - m * vec_per_m;
+        const int c = rem / (XV * kWave);
+        const int i = (rem / kWave) % XV;
+        const int l = rem % kWave;
+        const int k0 = c * kChunkK + l * WPP;
+        u32x4_t p = {0u, 0u, 0u, 0u};
+        if (k0 < K) p = F::stage(a.act + static_cast<size_t>(m) * K, k0, i);
+        lds_x[v] = p;
+    }
+    __syncthreads();
+    if (F::kBias != 0.f) {
+        // Per-(chunk, lane) sum of the activations the lane will multiply.
+        for (int j = tid; j < M * nchunks * kWave; j += kBlock) {
+            const int m = j / (nchunks * kWave);
+            const int cl = j - m * (nchunks * kWave);
+            const int c = cl / kWave;
+            const int l = cl - c * kWave;
+            u32x4_t xs[XV];
+#pragma unroll
+            for (int i = 0; i < XV; ++i) xs[i] = lds_x[m * vec_per_m + (c * XV + i) * kWave + l];
+            lds_sx[j] = F::sum_x(xs);
+        }
+        __syncthreads();
+    }
+
+    float acc[R][M];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int m = 0; m < M; ++m) acc[r][m] = 0.f;
+
+    auto compute = [&](const Unit<R>& u, int g, int c) {
+        const bool valid = c * kChunkK + lane * WPP < K;
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+            u32x4_t xs[XV];
+#pragma unroll
+            for (int i = 0; i < XV; ++i) xs[i] = lds_x[m * vec_per_m + (c * XV + i) * kWave + lane];
+            const float p0 =
+                F::kBias != 0.f ? F::kBias * lds_sx[(m * nchunks + c) * kWave + lane] : 0.f;
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const float p = F::dot(u.w[r], xs, p0);
+                if constexpr (F::kGroupScale) {
+                    const float s = valid ? bf16_bits_to_f32(u.gs[r]) : 0.f;
+                    acc[r][m] = fmaf(s, p, acc[r][m]);
+                } else {
+                    acc[r][m] += valid ? p : 0.f;
+                }
+            }
+        }
+        if (c == nchunks - 1) {
+            float mine = 0.f;
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+#pragma unroll
+                for (int m = 0; m < M; ++m) {
+                    const float v = wave_sum(acc[r][m]);
+                    acc[r][m] = 0.f;
+                    if (lane == r * M + m) mine = v;
+                }
+            }
+            const int row = row_begin + g * R + lane / M;
+            if (lane < R * M && row < row_end) {
+                if constexpr (F::kRowScale) mine *= u.rs;
+                const float prev = a.beta ? bf16_bits_to_f32(u.prev) : 0.f;
+                a.y[static_cast<size_t>(lane % M) * N + row] = f32_to_bf16_bits(mine + prev);
+            }
+        }
+    };
+
+    // Two-deep software pipeline over (row group, chunk) units.  Loads are issued
+    // unconditionally (past the end they re-request the last unit) so the wait
+    // before each compute only covers the unit it consumes.
+    const int last_g = ngroups - 1, last_c = nchunks - 1;
+    auto advance = [&](int& gg, int& cc) {
+        if (gg == last_g && cc == last_c) return;
+        if (++cc == nchunks) { cc = 0; ++gg; }
+    };
+    int g = 0, c = 0;  // coordinates of the unit held in `ua`
+    for (int u = 0; u < nunits; u += 2) {
+        int g1 = g, c1 = c;
+        advance(g1, c1);
+        int g2 = g1, c2 = c1;
+        advance(g2, c2);
+        issue(ub, g1, c1);
+        compute(ua, g, c);
+        issue(ua, g2, c2);
+        if (u + 1 < nunits) compute(ub, g1, c1);
+        g = g2;
+        c = c2;
+    }
+}
+
+template <class F, int R, int M>
+int launch(const GemvArgs& a, int waves_per_simd, hipStream_t stream) {
+    constexpr int kChunkK = kWave * F::WPP;
+    const int nchunks = (a.K + kChunkK - 1) / kChunkK;
+    const size_t smem = static_cast<size_t>(M) * nchunks * kWave * (F::XV * 16 + 4);
+    if (smem > 64 * 1024) return PIE_HIP_ERR_UNSUPPORTED;
+    int grid = kNumCU * waves_per_simd;
+    const int max_grid = (a.N + kWavesPerBlock - 1) / kWavesPerBlock;  // >= 1 row per wave
+    if (grid > max_grid) grid = max_grid;
+    hipLaunchKernelGGL((gemv_kernel<F, R, M>), dim3(grid), dim3(kBlock), smem, stream, a);
+    return launch_status();
+}
+
+template <class F, int R>
+int launch_m(int M, const GemvArgs& a, int wps, hipStream_t stream) {
+    switch (M) {
+        case 1: return launch<F, R, 1>(a, wps, stream);
+        case 2: return launch<F, R, 2>(a, wps, stream);
+        case 3: return launch<F, R, 3>(a, wps, stream);
+        case 4: return launch<F, R, 4>(a, wps, stream);
+        default: return PIE_HIP_ERR_UNSUPPORTED;
+    }
+}
+
+// rows_per_wave (R) in {1,2,3,4}; waves_per_simd in 1..8.  0 = pick.
+template <class F>
+int dispatch(GemvArgs a, int M, int rows_per_wave, int waves_per_simd, hipStream_t stream) {
+    if (!a.act || !a.w || !a.y || M <= 0 || a.N <= 0 || a.K <= 0) return PIE_HIP_ERR_INVALID;
+    if (a.K % F::WPP != 0) return PIE_HIP_ERR_UNSUPPORTED;
+    // Measured on MI355X: two resident waves per SIMD, each walking its slice four rows
+    // at a time (fewer when the slice is shorter), is within a few percent of the best
+    // (rows, waves) pair for every decode shape of an 8B-class model.
+    if (waves_per_simd <= 0) waves_per_simd = 2;
+    if (waves_per_simd > 8) return PIE_HIP_ERR_INVALID;
+    if (rows_per_wave <= 0) {
+        const long long per_wave =
+            a.N / (static_cast<long long>(kNumCU) * kWavesPerBlock * waves_per_simd);
+        rows_per_wave = per_wave >= 4 ? 4 : (per_wave >= 3 ? 3 : (per_wave >= 2 ? 2 : 1));
+    }
+    // Up to four activation rows share one pass over the weights (fewer when their staged
+    // copies would not fit in 64 KiB of LDS); larger M re-reads the weights per group.
+    constexpr int kChunkK = kWave * F::WPP;
+    const size_t per_m = static_cast<size_t>((a.K + kChunkK - 1) / kChunkK) * kWave * (F::XV * 16 + 4);
+    if (per_m > 64 * 1024) return PIE_HIP_ERR_UNSUPPORTED;
+    int mcap = static_cast<int>(64 * 1024 / per_m);
+    if (mcap > 4) mcap = 4;
+    const uint16_t* act = a.act;
+    uint16_t* y = a.y;
+    for (int m0 = 0; m0 < M; m0 += mcap) {
+        const int mm = (M - m0) < mcap ? (M - m0) : mcap;
+        a.act = act + static_cast<size_t>(m0) * a.K;
+        a.y = y + static_cast<size_t>(m0) * a.N;
+        int st;
+        switch (rows_per_wave) {
+            case 1: st = launch_m<F, 1>(mm, a, waves_per_simd, stream); break;
+            case 2: st = launch_m<F, 2>(mm, a, waves_per_simd, stream); break;
+            case 3: st = launch_m<F, 3>(mm, a, waves_per_simd, stream); break;
+            case 4: st = launch_m<F, 4>(mm, a, waves_per_simd, stream); break;
+            default: return PIE_HIP_ERR_INVALID;
+        }
+        if (st != PIE_HIP_OK) return st;
+    }
+    return PIE_HIP_OK;
+}
+
+}  // namespace
+}  // namespace pie_hip
+
+using pie_hip::GemvArgs;
+
+extern "C" int pie_hip_gemv_w4a16_tuned(const uint16_t* act_bf16, const uint32_t* packed,
+                                        const uint16_t* scale_bf16, uint16_t* y_bf16, int M,
+                                        int N, int K, int group_size, int beta,
+                                        int rows_per_wave, int waves_per_simd, void* stream) {
+    if (!scale_bf16 || group_size <= 0) return PIE_HIP_ERR_INVALID;
+    if (group_size % 32 != 0 || K % group_size != 0) return PIE_HIP_ERR_UNSUPPORTED;
+    GemvArgs a{act_bf16, reinterpret_cast<const pie_hip::u32x4_t*>(packed), scale_bf16, nullptr,
+               y_bf16, N, K, group_size, beta};
+    return pie_hip::dispatch<pie_hip::FmtInt4>(a, M, rows_per_wave, waves_per_simd,
+                                               static_cast<hipStream_t>(stream));
+}
+
+extern "C" int pie_hip_gemv_w4a16(const uint16_t* act_bf16, const uint32_t* packed,
+                                  const uint16_t* scale_bf16, uint16_t* y_bf16, int M, int N,
+                                  int K, int group_size, int beta, void* stream) {
+    if (M > 32) return PIE_HIP_ERR_UNSUPPORTED;
+    return pie_hip_gemv_w4a16_tuned(act_bf16, packed, scale_bf16, y_bf16, M, N, K, group_size,
+                                    beta, 0, 0, stream);
+}
+
+extern "C" int pie_hip_gemv_w8a16(const uint16_t* act_bf16, const int8_t* w_int8,
+                                  const float* scale_inv_f32, const uint16_t* scale_inv_bf16,
+                                  uint16_t* y_bf16, int M, int N, int K, int beta, void* stream) {
+    if (M > 32) return PIE_HIP_ERR_UNSUPPORTED;
+    if (!scale_inv_f32 == !scale_inv_bf16) return PIE_HIP_ERR_INVALID;  // exactly one
+    GemvArgs a{act_bf16, reinterpret_cast<const pie_hip::u32x4_t*>(w_int8), nullptr,
+               scale_inv_f32 ? static_cast<const void*>(scale_inv_f32) : scale_inv_bf16, y_bf16,
+               N, K, 0, beta};
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    return scale_inv_f32 ? pie_hip::dispatch<pie_hip::FmtInt8<false>>(a, M, 0, 0, st)
+                         : pie_hip::dispatch<pie_hip::FmtInt8<true>>(a, M, 0, 0, st);
+}
+
+extern "C" int pie_hip_gemv_fp8(const uint16_t* act_bf16, const uint8_t* w_e4m3,
+                                const float* scale_inv_f32, const uint16_t* scale_inv_bf16,
+                                uint16_t* y_bf16, int M, int N, int K, int beta, void* stream) {
+    if (M > 32) return PIE_HIP_ERR_UNSUPPORTED;
+    if (!scale_inv_f32 == !scale_inv_bf16) return PIE_HIP_ERR_INVALID;
+    GemvArgs a{act_bf16, reinterpret_cast<const pie_hip::u32x4_t*>(w_e4m3), nullptr,
+               scale_inv_f32 ? static_cast<const void*>(scale_inv_f32) : scale_inv_bf16, y_bf16,
+               N, K, 0, beta};
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    return scale_inv_f32 ? pie_hip::dispatch<pie_hip::FmtFp8<false>>(a, M, 0, 0, st)
+                         : pie_hip::dispatch<pie_hip::FmtFp8<true>>(a, M, 0, 0, st);
+}
+
+extern "C" int pie_hip_gemv_bf16(const uint16_t* act_bf16, const uint16_t* w_bf16,
+                                 uint16_t* y_bf16, int M, int N, int K, int beta, void* stream) {
+    if (M > 32) return PIE_HIP_ERR_UNSUPPORTED;
+    GemvArgs a{act_bf16, reinterpret_cast<const pie_hip::u32x4_t*>(w_bf16), nullptr, nullptr,
+               y_bf16, N, K, 0, beta};
+    return pie_hip::dispatch<pie_hip::FmtBf16>(a, M, 0, 0, static_cast<hipStream_t>(stream));
+}

@@ -169,3 +169,163 @@ def attention_paged_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torc
         max_kv_len, _ptr(workspace), C.c_size_t(wbytes), _stream())
     _check(st, "pie_hip_attn_decode_paged")
     return o
+
+
+# ---------------------------------------------------------------- other weight formats
+def _row_scale_args(scale: torch.Tensor):
+    if scale.dtype == torch.float32:
+        return _ptr(scale), _ptr(None)
+    if scale.dtype == torch.bfloat16:
+        return _ptr(None), _ptr(scale)
+    raise KernelError("row scale must be float32 or bfloat16")
+
+
+def _gemv_out(act, N, y, beta):
+    M = act.shape[0]
+    if y is None:
+        if beta:
+            raise KernelError("beta=1 needs an existing y")
+        y = torch.empty((M, N), dtype=torch.bfloat16, device=act.device)
+    _dev(y, torch.bfloat16, "y")
+    if tuple(y.shape) != (M, N):
+        raise KernelError("y shape mismatch")
+    return y
+
+
+def gemv_w8a16(act, q_int8, scale_inv, y=None, beta=0):
+    """y = (act · q^T) * scale_inv[n]; q int8 [N,K], scale_inv f32 or bf16 [N]."""
+    _dev(act, torch.bfloat16, "act")
+    _dev(q_int8, torch.int8, "q_int8")
+    N, K = q_int8.shape
+    if act.shape[1] != K or scale_inv.numel() != N or not scale_inv.is_contiguous():
+        raise KernelError("shape mismatch")
+    y = _gemv_out(act, N, y, beta)
+    sf, sb = _row_scale_args(scale_inv)
+    _check(kernels().pie_hip_gemv_w8a16(_ptr(act), _ptr(q_int8), sf, sb, _ptr(y), act.shape[0], N,
+                                        K, beta, _stream()), "pie_hip_gemv_w8a16")
+    return y
+
+
+def gemv_fp8(act, w_e4m3, scale_inv, y=None, beta=0):
+    """y = (act · fp8(w)^T) * scale_inv[n]; w uint8 holding OCP e4m3fn bytes [N,K]."""
+    _dev(act, torch.bfloat16, "act")
+    _dev(w_e4m3, torch.uint8, "w_e4m3")
+    N, K = w_e4m3.shape
+    if act.shape[1] != K or scale_inv.numel() != N or not scale_inv.is_contiguous():
+        raise KernelError("shape mismatch")
+    y = _gemv_out(act, N, y, beta)
+    sf, sb = _row_scale_args(scale_inv)
+    _check(kernels().pie_hip_gemv_fp8(_ptr(act), _ptr(w_e4m3), sf, sb, _ptr(y), act.shape[0], N, K,
+                                      beta, _stream()), "pie_hip_gemv_fp8")
+    return y
+
+
+def gemv_bf16(act, w, y=None, beta=0):
+    _dev(act, torch.bfloat16, "act")
+    _dev(w, torch.bfloat16, "w")
+    N, K = w.shape
+    if act.shape[1] != K:
+        raise KernelError("shape mismatch")
+    y = _gemv_out(act, N, y, beta)
+    _check(kernels().pie_hip_gemv_bf16(_ptr(act), _ptr(w), _ptr(y), act.shape[0], N, K, beta,
+                                       _stream()), "pie_hip_gemv_bf16")
+    return y
+
+
+# ---------------------------------------------------------------- per-layer kernels
+def embed_bf16(token_ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
+    _dev(token_ids, torch.int32, "token_ids")
+    _dev(table, torch.bfloat16, "table")
+    V, H = table.shape
+    y = torch.empty((token_ids.numel(), H), dtype=torch.bfloat16, device=table.device)
+    _check(kernels().pie_hip_embed(_ptr(token_ids), _ptr(table), _ptr(y), token_ids.numel(), H, V,
+                                   _stream()), "pie_hip_embed")
+    return y
+
+
+def rmsnorm_bf16(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    _dev(x, torch.bfloat16, "x")
+    _dev(weight, torch.bfloat16, "weight")
+    rows, H = x.shape
+    y = torch.empty_like(x)
+    _check(kernels().pie_hip_rmsnorm(_ptr(x), _ptr(weight), _ptr(y), rows, H, C.c_float(eps),
+                                     _stream()), "pie_hip_rmsnorm")
+    return y
+
+
+def residual_add_rmsnorm_bf16(hidden: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor,
+                              eps: float) -> torch.Tensor:
+    """hidden += residual (in place, rounded to bf16); returns rmsnorm(hidden)."""
+    for n, t in (("hidden", hidden), ("residual", residual), ("weight", weight)):
+        _dev(t, torch.bfloat16, n)
+    rows, H = hidden.shape
+    y = torch.empty_like(hidden)
+    _check(kernels().pie_hip_residual_rmsnorm(_ptr(hidden), _ptr(residual), _ptr(weight), _ptr(y),
+                                              rows, H, C.c_float(eps), _stream()),
+           "pie_hip_residual_rmsnorm")
+    return y
+
+
+def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, head_dim: int) -> torch.Tensor:
+    _dev(positions, torch.int32, "positions")
+    _dev(inv_freq, torch.float32, "inv_freq")
+    if inv_freq.numel() != head_dim // 2:
+        raise KernelError("inv_freq must have head_dim/2 entries")
+    tab = torch.empty((positions.numel(), head_dim), dtype=torch.float32, device=positions.device)
+    _check(kernels().pie_hip_rope_table(_ptr(positions), _ptr(inv_freq), _ptr(tab),
+                                        positions.numel(), head_dim, _stream()),
+           "pie_hip_rope_table")
+    return tab
+
+
+def qkv_rope_kvwrite(packed, k_pages, v_pages, table, kv_slots, hq, hk, d, interleaved,
+                     q_norm_w=None, k_norm_w=None, eps=1e-6):
+    _dev(packed, torch.bfloat16, "packed")
+    _dev(k_pages, torch.bfloat16, "k_pages")
+    _dev(v_pages, torch.bfloat16, "v_pages")
+    _dev(table, torch.float32, "rope_table")
+    _dev(kv_slots, torch.int64, "kv_slots")
+    N = packed.shape[0]
+    if packed.shape[1] != (hq + 2 * hk) * d or tuple(table.shape) != (N, d) or kv_slots.numel() != N:
+        raise KernelError("shape mismatch")
+    total_slots = k_pages.numel() // (hk * d)
+    if N and int(kv_slots.max()) >= total_slots:
+        raise KernelError("kv slot out of range")
+    q_out = torch.empty((N, hq, d), dtype=torch.bfloat16, device=packed.device)
+    _check(kernels().pie_hip_qkv_rope_kvwrite(
+        _ptr(packed), _ptr(q_out), _ptr(k_pages), _ptr(v_pages), _ptr(q_norm_w), _ptr(k_norm_w),
+        _ptr(table), _ptr(kv_slots), N, hq, hk, d, int(interleaved), C.c_float(eps), _stream()),
+        "pie_hip_qkv_rope_kvwrite")
+    return q_out
+
+
+def swiglu_bf16(gate_up: torch.Tensor) -> torch.Tensor:
+    _dev(gate_up, torch.bfloat16, "gate_up")
+    N, two_i = gate_up.shape
+    y = torch.empty((N, two_i // 2), dtype=torch.bfloat16, device=gate_up.device)
+    _check(kernels().pie_hip_swiglu(_ptr(gate_up), _ptr(y), N, two_i // 2, _stream()),
+           "pie_hip_swiglu")
+    return y
+
+
+def argmax_bf16(logits: torch.Tensor) -> torch.Tensor:
+    _dev(logits, torch.bfloat16, "logits")
+    rows, V = logits.shape
+    out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    _check(kernels().pie_hip_argmax(_ptr(logits), _ptr(out), rows, V, _stream()), "pie_hip_argmax")
+    return out
+
+
+def copy_kv_pages(pool: torch.Tensor, srcs: torch.Tensor, dsts: torch.Tensor) -> None:
+    """pool[dsts[i]] <- pool[srcs[i]] over the leading (page) dimension."""
+    _dev(srcs, torch.int32, "srcs")
+    _dev(dsts, torch.int32, "dsts")
+    if not pool.is_contiguous() or srcs.numel() != dsts.numel():
+        raise KernelError("bad copy arguments")
+    n_pages = pool.shape[0]
+    if srcs.numel() and (int(srcs.max()) >= n_pages or int(dsts.max()) >= n_pages):
+        raise KernelError("page id out of range")
+    page_bytes = pool[0].numel() * pool.element_size()
+    _check(kernels().pie_hip_copy_kv_pages(_ptr(pool), _ptr(srcs), _ptr(dsts), srcs.numel(),
+                                           C.c_size_t(page_bytes), _stream()),
+           "pie_hip_copy_kv_pages")

@@ -181,3 +181,56 @@ def test_bf16_rounding_helpers(oracle):
     b = oracle.f32_to_bf16(x)
     assert b.tolist() == [0x3F80, 0x3F82, 0x3F81, 0x8000, 0x7F80]
     assert np.isnan(oracle.bf16_to_f32(oracle.f32_to_bf16(np.array([np.nan], np.float32))))[0]
+
+
+def test_fp8_e4m3_decode_table(oracle):
+    b = np.arange(256, dtype=np.uint8)
+    f = oracle.fp8_decode(b)
+    # literal anchors of the OCP e4m3fn format
+    assert f[0x00] == 0 and f[0x01] == 2.0 ** -9 and f[0x07] == 7 * 2.0 ** -9
+    assert f[0x08] == 2.0 ** -6 and f[0x38] == 1.0 and f[0x3C] == 1.5 and f[0x40] == 2.0
+    assert f[0x7E] == 448.0 and np.isnan(f[0x7F]) and np.isnan(f[0xFF]) and f[0xFE] == -448.0
+    fin = np.delete(f[:128], 0x7F)
+    assert np.all(np.diff(fin) > 0)  # codes are monotonic
+    assert np.array_equal(f[128:255], -f[:127])
+    # torch's float8_e4m3fn agrees on every finite code
+    import torch
+    t = torch.from_numpy(b.copy()).view(torch.float8_e4m3fn).float().numpy()
+    ok = ~np.isnan(f)
+    assert np.array_equal(t[ok], f[ok])
+
+
+def test_fp8_quant_round_trip_and_rounding(oracle):
+    import torch
+    rng = np.random.default_rng(8)
+    w = rand_bf16(rng, (6, 256), std=0.02)
+    q, s = oracle.quant_fp8_per_channel(w)
+    wf = oracle.bf16_to_f32(w)
+    assert np.allclose(s, np.abs(wf).max(axis=1) / 448.0, rtol=1e-6)
+    assert np.all(np.abs(oracle.fp8_decode(q)).max(axis=1) == 448.0)
+    # the quantiser's rounding is round-to-nearest-even saturating: same bytes as torch's cast
+    scaled = (wf * (np.float32(448.0) / np.abs(wf).max(axis=1, keepdims=True))).astype(np.float32)
+    tq = torch.from_numpy(scaled).clamp(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    assert np.array_equal(q, tq)
+    # exactly representable values survive
+    codes = np.delete(np.arange(255, dtype=np.uint8), [0x7F, 0x80])
+    vals = oracle.fp8_decode(codes)
+    row = oracle.f32_to_bf16(np.concatenate([vals, [448.0]]).astype(np.float32)[None, :] / 8)
+    q2, s2 = oracle.quant_fp8_per_channel(row)
+    assert s2[0] == np.float32(56.0) / np.float32(448.0)
+    assert np.array_equal(oracle.fp8_decode(q2[0, :-1]), vals)
+
+
+def test_gemm_fp8_against_fp64(oracle):
+    rng = np.random.default_rng(9)
+    w = rand_bf16(rng, (9, 128), std=0.02)
+    q, s = oracle.quant_fp8_per_channel(w)
+    act = rand_bf16(rng, (2, 128))
+    x = oracle.bf16_to_f32(act).astype(np.float64)
+    wd = oracle.fp8_decode(q).astype(np.float64)
+    truth = (x @ wd.T) * s[None, :]
+    y2, _ = oracle.gemm_fp8(act, q, s, mode=2)
+    y0, y0b = oracle.gemm_fp8(act, q, s, mode=0)
+    assert np.allclose(y2, truth, rtol=1e-6, atol=1e-8)
+    assert np.allclose(y0, truth, rtol=0, atol=1e-5 * np.abs(truth).max())
+    assert np.array_equal(y0b, oracle.f32_to_bf16(y0))
