@@ -61,7 +61,8 @@ int pie_hip_dequant_w4a16(const uint32_t* packed, const uint16_t* scale_bf16,
  * with fp32 accumulation; the group scale is applied to each group's partial
  * sum (same value as the reference's per-element `x * (q * s)` up to fp32
  * rounding, driver/cuda/src/kernels/dequant_wna16.cu:96-110).
- * Requires K % 32 == 0, G % 32 == 0, K % G == 0, 1 <= M <= 32.
+ * Requires K % 32 == 0, G % 32 == 0, K % G == 0.  Tuned for decode (small M): up to four
+ * activation rows share one pass over the weights, larger M re-streams them per group of four.
  * Replaces the Marlin call `marlin_w4a16_gemm` for small M
  * (driver/cuda/third_party/marlin/marlin_wrapper.hpp:39-51) and the
  * dequant-then-GEMM fallback of gemm_act_x_w (driver/cuda/src/ops/gemm.cpp:1414-1583).
@@ -82,7 +83,7 @@ int pie_hip_gemv_w4a16_tuned(const uint16_t* act_bf16, const uint32_t* packed,
  * fp32 sum, scale applied once after it — the evaluation order of the reference's own
  * weight-only int8 GEMV (driver/cuda/src/kernels/argmax.cu:846-854).  q: int8 [N,K];
  * scale_inv (= absmax/127, driver/cuda/src/kernels/quant_bf16_to_fp8.cu:311-313) is given
- * as f32 [N] or as bf16 [N]: pass exactly one of the two pointers.  K % 16 == 0, M <= 32.
+ * as f32 [N] or as bf16 [N]: pass exactly one of the two pointers.  K % 16 == 0.
  */
 int pie_hip_gemv_w8a16(const uint16_t* act_bf16, const int8_t* w_int8,
                        const float* scale_inv_f32, const uint16_t* scale_inv_bf16,
@@ -100,7 +101,7 @@ int pie_hip_gemv_fp8(const uint16_t* act_bf16, const uint8_t* w_e4m3,
 /*
  * bf16 GEMV: y[m, n] = bf16( beta*y + sum_k act[m,k]*W[n,k] ), fp32 accumulation
  * (gemm_act_x_w bf16 path, driver/cuda/src/ops/gemm.hpp:152-160; the lm_head and router
- * projections stay unquantised in the reference).  K % 8 == 0, M <= 32.
+ * projections stay unquantised in the reference).  K % 8 == 0.
  */
 int pie_hip_gemv_bf16(const uint16_t* act_bf16, const uint16_t* w_bf16, uint16_t* y_bf16, int M,
                       int N, int K, int beta, void* stream);
@@ -135,6 +136,22 @@ int pie_hip_attn_decode_paged(const uint16_t* q, const uint16_t* k_pages, const 
                               int num_requests, int num_q_heads, int num_kv_heads, int head_dim,
                               int page_size, float sm_scale, int max_kv_len, void* workspace,
                               size_t workspace_bytes, void* stream);
+
+/*
+ * Same attention over explicit per-row extents: query row r reads the page-list entries
+ * starting at kv_page_indices[row_page_begin[r]] and sees its first row_kv_len[r] keys.  A
+ * planner derives the pairs from the page table and the token positions
+ * (visible keys = min(seq_len, position + 1), driver/portable/src/plan.cpp:54-94), so a
+ * prefill or mixed batch runs as one row per query token, causal by construction, and a
+ * decode batch as one row per request.  Workspace: pie_hip_attn_decode_workspace_bytes with
+ * num_requests = num_rows.
+ */
+int pie_hip_attn_rows_paged(const uint16_t* q, const uint16_t* k_pages, const uint16_t* v_pages,
+                            uint16_t* o, float* lse, const uint32_t* kv_page_indices,
+                            const uint32_t* row_page_begin, const int32_t* row_kv_len,
+                            int num_rows, int num_q_heads, int num_kv_heads, int head_dim,
+                            int page_size, float sm_scale, int max_kv_len, void* workspace,
+                            size_t workspace_bytes, void* stream);
 
 /* ---- per-layer kernels of the llama-like decoder ---------------------------- */
 
@@ -193,6 +210,23 @@ int pie_hip_argmax(const uint16_t* logits_bf16, uint32_t* out_idx, int rows, int
  * Reference: Copy D2D handling, driver/portable/src/service/inproc_service.cpp:149-172. */
 int pie_hip_copy_kv_pages(void* pool, const uint32_t* src_pages, const uint32_t* dst_pages,
                           int num_copies, size_t page_bytes, void* stream);
+
+/* ---- load-time quantisers (bf16 weights -> storage formats) ---------------------- */
+
+/* Per-output-channel int8: scale_inv[r] = absmax/127 (1 for a zero row),
+ * q = clamp(rintf(w * 127/absmax), -128, 127), round half to even.
+ * Reference: quantize_bf16_to_int8_per_channel, driver/cuda/src/kernels/quant_bf16_to_fp8.cu:273-333. */
+int pie_hip_quant_int8_per_channel(const uint16_t* w_bf16, int8_t* q, float* scale_inv, int rows,
+                                   int cols, void* stream);
+/* Per-output-channel fp8 e4m3fn: scale_inv[r] = absmax/448, q = e4m3_satfinite(w * 448/absmax).
+ * Reference: quant_per_channel_kernel, driver/cuda/src/kernels/quant_bf16_to_fp8.cu:181-226. */
+int pie_hip_quant_fp8_per_channel(const uint16_t* w_bf16, uint8_t* q_e4m3, float* scale_inv,
+                                  int rows, int cols, void* stream);
+/* Symmetric group-wise int4 into the int4b8 layout: scale = bf16(absmax/7) per (row, group)
+ * (1 for a zero group), nibble = clamp(rintf(w/scale), -8, 7) + 8.  The reference defines the
+ * layout (driver/cuda/src/kernels/dequant_wna16.cu:11-38) but ships no quantiser for it. */
+int pie_hip_quant_int4b8_group(const uint16_t* w_bf16, uint32_t* packed, uint16_t* scale_bf16,
+                               int rows, int cols, int group_size, void* stream);
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,148 @@
+"""Oracle: llama-like decoder forward over a paged KV cache (ctypes front end of
+oracle/src/model.c) plus a greedy generation loop shaped like the reference's offline
+harness (driver/portable/src/executor/executor.cpp:1439-1597).  TEST INFRASTRUCTURE ONLY."""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+
+from . import bf16_to_f32, lib
+from .planner import plan_forward
+
+QUANT_CODE = {"int4b8": 0, "int8": 1, "fp8": 2, "bf16": 3}
+
+
+class _Linear(C.Structure):
+    _fields_ = [("data", C.c_void_p), ("scale", C.c_void_p)]
+
+
+class _Model(C.Structure):
+    _fields_ = [("hidden", C.c_int), ("layers", C.c_int), ("q_heads", C.c_int),
+                ("kv_heads", C.c_int), ("head_dim", C.c_int), ("intermediate", C.c_int),
+                ("vocab", C.c_int), ("rms_eps", C.c_float), ("rope_interleaved", C.c_int),
+                ("has_qk_norm", C.c_int), ("quant", C.c_int), ("group", C.c_int),
+                ("embed", C.c_void_p), ("lm_head", C.c_void_p), ("final_norm", C.c_void_p),
+                ("inv_freq", C.c_void_p),
+                ("attn_norm", C.POINTER(C.c_void_p)), ("ffn_norm", C.POINTER(C.c_void_p)),
+                ("q_norm", C.POINTER(C.c_void_p)), ("k_norm", C.POINTER(C.c_void_p)),
+                ("wqkv", C.POINTER(_Linear)), ("wo", C.POINTER(_Linear)),
+                ("wgu", C.POINTER(_Linear)), ("wdown", C.POINTER(_Linear))]
+
+
+class OracleModel:
+    """`cfg`: dict with hidden, layers, q_heads, kv_heads, head_dim, intermediate, vocab,
+    rms_eps, rope_interleaved, qk_norm, quant, group_size, page_size, total_pages.
+    `tensors`: name -> numpy array, names as the driver exports them; row scales of int8/fp8
+    may be bf16 bits (uint16) and are widened to f32 here."""
+
+    def __init__(self, cfg: dict, tensors: dict):
+        self.cfg = dict(cfg)
+        L = cfg["layers"]
+        self._keep = []
+
+        def ptr(a):
+            a = np.ascontiguousarray(a)
+            self._keep.append(a)
+            return a.ctypes.data
+
+        def lin(prefix):
+            data = tensors[prefix + ".data"]
+            sc = tensors.get(prefix + ".scale")
+            if sc is not None and cfg["quant"] in ("int8", "fp8") and sc.dtype == np.uint16:
+                sc = bf16_to_f32(sc)
+            return _Linear(ptr(data), ptr(sc) if sc is not None else None)
+
+        m = _Model()
+        for k in ("hidden", "layers", "q_heads", "kv_heads", "head_dim", "intermediate", "vocab"):
+            setattr(m, k, int(cfg[k]))
+        m.rms_eps = float(cfg["rms_eps"])
+        m.rope_interleaved = int(cfg["rope_interleaved"])
+        m.has_qk_norm = int(bool(cfg.get("qk_norm", False)))
+        m.quant = QUANT_CODE[cfg["quant"]]
+        m.group = int(cfg.get("group_size", 128))
+        m.embed = ptr(tensors["embed"])
+        m.lm_head = ptr(tensors["lm_head"])
+        m.final_norm = ptr(tensors["final_norm"])
+        m.inv_freq = ptr(np.asarray(tensors["inv_freq"], np.float32))
+
+        def parr(names):
+            arr = (C.c_void_p * L)(*[ptr(tensors[n]) if n in tensors else None for n in names])
+            self._keep.append(arr)
+            return C.cast(arr, C.POINTER(C.c_void_p))
+
+        def larr(suffix):
+            arr = (_Linear * L)(*[lin(f"layers.{l}.{suffix}") for l in range(L)])
+            self._keep.append(arr)
+            return C.cast(arr, C.POINTER(_Linear))
+
+        m.attn_norm = parr([f"layers.{l}.attn_norm" for l in range(L)])
+        m.ffn_norm = parr([f"layers.{l}.ffn_norm" for l in range(L)])
+        m.q_norm = parr([f"layers.{l}.q_norm" for l in range(L)])
+        m.k_norm = parr([f"layers.{l}.k_norm" for l in range(L)])
+        m.wqkv, m.wo, m.wgu, m.wdown = larr("wqkv"), larr("wo"), larr("wgu"), larr("wdown")
+        self._m = m
+        ps, tp = cfg["page_size"], cfg["total_pages"]
+        shape = (tp, ps, cfg["kv_heads"], cfg["head_dim"])
+        self.k_pages = [np.zeros(shape, np.uint16) for _ in range(L)]
+        self.v_pages = [np.zeros(shape, np.uint16) for _ in range(L)]
+        self._kp = (C.c_void_p * L)(*[a.ctypes.data for a in self.k_pages])
+        self._vp = (C.c_void_p * L)(*[a.ctypes.data for a in self.v_pages])
+
+    def forward(self, token_ids, position_ids, kv_page_indices, kv_page_indptr, kv_last_page_lens,
+                qo_indptr, sampling_indices=None, sampling_indptr=None, want_logits=False):
+        """One forward pass; returns (tokens per sampled row, logits bf16 bits or None, plan)."""
+        R = len(qo_indptr) - 1
+        if sampling_indices is None:
+            qo = np.asarray(qo_indptr, np.int64)
+            sampling_indices = qo[1:] - qo[:-1] - 1
+            sampling_indptr = np.arange(R + 1)
+        p = plan_forward(token_ids, position_ids, kv_page_indices, kv_page_indptr,
+                         kv_last_page_lens, qo_indptr, sampling_indices, sampling_indptr,
+                         self.cfg["page_size"], self.cfg["total_pages"])
+        N, S = p["N"], len(p["sample_rows"])
+        tok = np.ascontiguousarray(np.asarray(token_ids, np.uint32))
+        pos = np.ascontiguousarray(np.asarray(p["positions"], np.int32))
+        slots = np.ascontiguousarray(np.asarray(p["kv_slots"], np.int64))
+        rb = np.ascontiguousarray(np.asarray(p["row_page_begin"], np.uint32))
+        rl = np.ascontiguousarray(np.asarray(p["row_kv_len"], np.int32))
+        pages = np.ascontiguousarray(np.asarray(kv_page_indices, np.uint32))
+        sr = np.ascontiguousarray(np.asarray(p["sample_rows"], np.uint32))
+        out = np.zeros(max(S, 1), np.uint32)
+        logits = np.zeros((max(S, 1), self.cfg["vocab"]), np.uint16) if want_logits else None
+        vp = lambda a: C.c_void_p(a.ctypes.data)
+        lib().orc_llama_forward(C.byref(self._m), self._kp, self._vp, vp(tok), vp(pos), vp(slots),
+                                vp(rb), vp(rl), vp(pages), C.c_int(N), vp(sr), C.c_int(S),
+                                C.c_int(self.cfg["page_size"]), vp(out),
+                                vp(logits) if want_logits else None)
+        return out[:S], (logits[:S] if want_logits else None), p
+
+    def generate(self, prompt, max_new: int, replicate: int = 1, want_logits=False):
+        """Greedy generation over contiguous page ranges, one prefill per context and one
+        multi-request decode forward per step.  Returns tokens [replicate, max_new] (and the
+        per-step logits of context 0 when asked)."""
+        ps = self.cfg["page_size"]
+        n_prompt = len(prompt)
+        ppc = (n_prompt + max_new + ps - 1) // ps
+        toks = np.zeros((replicate, max_new), np.uint32)
+        logit_trace = []
+        for c in range(replicate):
+            npg = (n_prompt + ps - 1) // ps
+            t, lg, _ = self.forward(prompt, np.arange(n_prompt), np.arange(npg) + c * ppc, [0, npg],
+                                    [n_prompt - (npg - 1) * ps], [0, n_prompt],
+                                    want_logits=want_logits and c == 0)
+            toks[c, 0] = t[0]
+            if want_logits and c == 0:
+                logit_trace.append(lg[0])
+        for s in range(1, max_new):
+            pos = n_prompt + s - 1
+            npg = (pos + 1 + ps - 1) // ps
+            pages = np.concatenate([np.arange(npg) + c * ppc for c in range(replicate)])
+            t, lg, _ = self.forward(toks[:, s - 1], [pos] * replicate, pages,
+                                    np.arange(replicate + 1) * npg,
+                                    [pos + 1 - (npg - 1) * ps] * replicate,
+                                    np.arange(replicate + 1), want_logits=want_logits)
+            toks[:, s] = t
+            if want_logits:
+                logit_trace.append(lg[0])
+        return (toks, logit_trace) if want_logits else toks

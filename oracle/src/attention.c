@@ -26,10 +26,76 @@ static int orc_kv_len(const uint32_t* indptr, const uint32_t* last_lens, int r, 
 }
 
 /*
+ * One query row (all hq heads) over the first `lim` keys of the page list starting at
+ * page_indices[pg_lo].  mode 0: fp32 two-pass softmax in the reference's order
+ * (attention_naive_paged.cu:362-447); mode 2: fp64.
+ */
+static void orc_attn_row(const uint16_t* q_row, const uint16_t* k_pages, const uint16_t* v_pages,
+                         float* o_f32, uint16_t* o_bf16, float* lse, const uint32_t* page_indices,
+                         uint32_t pg_lo, int lim, int hq, int hk, int d, int ps, float scale,
+                         int mode, double* w) {
+    const int gqa = hq / hk;
+    for (int h = 0; h < hq; ++h) {
+        const int kvh = h / gqa;
+        const size_t qoff = (size_t)h * d;
+        double row_max = -INFINITY;
+        for (int j = 0; j < lim; ++j) {
+            const uint32_t pid = page_indices[pg_lo + j / ps];
+            const size_t koff = (((size_t)pid * ps + j % ps) * hk + kvh) * d;
+            double dot;
+            if (mode == 0) {
+                float f = 0.f;
+                for (int e = 0; e < d; ++e)
+                    f += orc_bf16_to_f32(q_row[qoff + e]) * orc_bf16_to_f32(k_pages[koff + e]);
+                dot = (double)(f * scale);
+            } else {
+                double f = 0.0;
+                for (int e = 0; e < d; ++e)
+                    f += (double)orc_bf16_to_f32(q_row[qoff + e]) *
+                         (double)orc_bf16_to_f32(k_pages[koff + e]);
+                dot = f * (double)scale;
+            }
+            w[j] = dot;
+            if (dot > row_max) row_max = dot;
+        }
+        double z = 0.0;
+        float zf = 0.f;
+        for (int j = 0; j < lim; ++j) {
+            if (mode == 0) {
+                const float e = expf((float)w[j] - (float)row_max);
+                w[j] = (double)e;
+                zf += e;
+            } else {
+                w[j] = exp(w[j] - row_max);
+                z += w[j];
+            }
+        }
+        if (mode == 0) z = (double)zf;
+        for (int e = 0; e < d; ++e) {
+            double acc = 0.0;
+            float accf = 0.f;
+            for (int j = 0; j < lim; ++j) {
+                const uint32_t pid = page_indices[pg_lo + j / ps];
+                const size_t voff = (((size_t)pid * ps + j % ps) * hk + kvh) * d;
+                const float v = orc_bf16_to_f32(v_pages[voff + e]);
+                if (mode == 0) accf = fmaf(v, (float)w[j], accf);
+                else acc += (double)v * w[j];
+            }
+            if (mode == 0) acc = (double)accf;
+            float out;
+            if (mode == 0) out = z > 0.0 ? (float)acc * (1.0f / (float)z) : 0.f;
+            else out = z > 0.0 ? (float)(acc / z) : 0.f;
+            o_f32[qoff + e] = out;
+            if (o_bf16) o_bf16[qoff + e] = orc_f32_to_bf16(out);
+        }
+        if (lse) lse[h] = z > 0.0 ? (float)(log(z) + row_max) : -INFINITY;
+    }
+}
+
+/*
  * General paged attention: request r owns query rows qo_indptr[r]..qo_indptr[r+1];
  * query i of n_q sees kv positions j < kv_len - n_q + i + 1 (attention_naive_paged.cu:194-198).
  * Decode is the n_q = 1 case (qo_indptr = 0,1,2,...).
- * mode 0: fp32 two-pass softmax in the reference's order; mode 2: fp64.
  * o_f32 [T,hq,d] unrounded, o_bf16 optional, lse optional [T,hq] (natural log).
  */
 void orc_attn_paged(const uint16_t* q, const uint16_t* k_pages, const uint16_t* v_pages,
@@ -37,76 +103,43 @@ void orc_attn_paged(const uint16_t* q, const uint16_t* k_pages, const uint16_t* 
                     const uint32_t* page_indices, const uint32_t* page_indptr,
                     const uint32_t* last_lens, int R, int hq, int hk, int d, int ps,
                     float sm_scale, int mode) {
-    const int gqa = hq / hk;
     const float scale = sm_scale > 0.f ? sm_scale : 1.0f / sqrtf((float)d);
 #pragma omp parallel for schedule(dynamic)
     for (int r = 0; r < R; ++r) {
         const int kv_total = orc_kv_len(page_indptr, last_lens, r, ps);
         const int q_lo = (int)qo_indptr[r], n_q = (int)qo_indptr[r + 1] - q_lo;
-        const uint32_t pg_lo = page_indptr[r];
         double* w = (double*)malloc(sizeof(double) * (size_t)(kv_total > 0 ? kv_total : 1));
         for (int qi = 0; qi < n_q; ++qi) {
             int lim = kv_total - n_q + qi + 1;
             if (lim > kv_total) lim = kv_total;
             if (lim < 0) lim = 0;
-            for (int h = 0; h < hq; ++h) {
-                const int kvh = h / gqa;
-                const size_t qoff = ((size_t)(q_lo + qi) * hq + h) * d;
-                double row_max = -INFINITY;
-                for (int j = 0; j < lim; ++j) {
-                    const uint32_t pid = page_indices[pg_lo + j / ps];
-                    const size_t koff = (((size_t)pid * ps + j % ps) * hk + kvh) * d;
-                    double dot;
-                    if (mode == 0) {
-                        float f = 0.f;
-                        for (int e = 0; e < d; ++e)
-                            f += orc_bf16_to_f32(q[qoff + e]) * orc_bf16_to_f32(k_pages[koff + e]);
-                        dot = (double)(f * scale);
-                    } else {
-                        double f = 0.0;
-                        for (int e = 0; e < d; ++e)
-                            f += (double)orc_bf16_to_f32(q[qoff + e]) *
-                                 (double)orc_bf16_to_f32(k_pages[koff + e]);
-                        dot = f * (double)scale;
-                    }
-                    w[j] = dot;
-                    if (dot > row_max) row_max = dot;
-                }
-                double z = 0.0;
-                float zf = 0.f;
-                for (int j = 0; j < lim; ++j) {
-                    if (mode == 0) {
-                        const float e = expf((float)w[j] - (float)row_max);
-                        w[j] = (double)e;
-                        zf += e;
-                    } else {
-                        w[j] = exp(w[j] - row_max);
-                        z += w[j];
-                    }
-                }
-                if (mode == 0) z = (double)zf;
-                for (int e = 0; e < d; ++e) {
-                    double acc = 0.0;
-                    float accf = 0.f;
-                    for (int j = 0; j < lim; ++j) {
-                        const uint32_t pid = page_indices[pg_lo + j / ps];
-                        const size_t voff = (((size_t)pid * ps + j % ps) * hk + kvh) * d;
-                        const float v = orc_bf16_to_f32(v_pages[voff + e]);
-                        if (mode == 0) accf = fmaf(v, (float)w[j], accf);
-                        else acc += (double)v * w[j];
-                    }
-                    if (mode == 0) acc = (double)accf;
-                    float out;
-                    if (mode == 0) out = z > 0.0 ? (float)acc * (1.0f / (float)z) : 0.f;
-                    else out = z > 0.0 ? (float)(acc / z) : 0.f;
-                    o_f32[qoff + e] = out;
-                    if (o_bf16) o_bf16[qoff + e] = orc_f32_to_bf16(out);
-                }
-                if (lse)
-                    lse[(size_t)(q_lo + qi) * hq + h] =
-                        z > 0.0 ? (float)(log(z) + row_max) : -INFINITY;
-            }
+            const size_t row = (size_t)(q_lo + qi) * hq;
+            orc_attn_row(q + row * d, k_pages, v_pages, o_f32 + row * d,
+                         o_bf16 ? o_bf16 + row * d : NULL, lse ? lse + row : NULL, page_indices,
+                         page_indptr[r], lim, hq, hk, d, ps, scale, mode, w);
         }
+        free(w);
+    }
+}
+
+/*
+ * Attention over explicit per-row extents: row r reads the page list from
+ * page_indices[row_begin[r]] and sees its first row_len[r] keys
+ * (visible keys = min(seq_len, position+1), driver/portable/src/plan.cpp:54-94).
+ */
+void orc_attn_rows(const uint16_t* q, const uint16_t* k_pages, const uint16_t* v_pages,
+                   float* o_f32, uint16_t* o_bf16, float* lse, const uint32_t* page_indices,
+                   const uint32_t* row_begin, const int32_t* row_len, int rows, int hq, int hk,
+                   int d, int ps, float sm_scale, int mode) {
+    const float scale = sm_scale > 0.f ? sm_scale : 1.0f / sqrtf((float)d);
+#pragma omp parallel for schedule(dynamic)
+    for (int r = 0; r < rows; ++r) {
+        const int lim = row_len[r] > 0 ? row_len[r] : 0;
+        double* w = (double*)malloc(sizeof(double) * (size_t)(lim > 0 ? lim : 1));
+        const size_t row = (size_t)r * hq;
+        orc_attn_row(q + row * d, k_pages, v_pages, o_f32 + row * d,
+                     o_bf16 ? o_bf16 + row * d : NULL, lse ? lse + row : NULL, page_indices,
+                     row_begin[r], lim, hq, hk, d, ps, scale, mode, w);
         free(w);
     }
 }

@@ -1,0 +1,124 @@
+/*
+ * Oracle: one forward pass of the llama-like decoder over a paged KV cache — the control
+ * flow and op sequence of the reference.  TEST INFRASTRUCTURE ONLY (see oracle_common.h).
+ *
+ * Graph: driver/portable/src/graph_qwen3.cpp:225-896 (norm -> QKV -> [qk-norm] -> RoPE ->
+ * KV write at the token's slot -> attention over the request's pages -> o_proj + residual ->
+ * norm -> SwiGLU FFN + residual; tail: final norm, lm_head on the sampled rows only, argmax).
+ * Rounding points: those of the reference's kernel-by-kernel CUDA forward
+ * (driver/cuda/src/model/llama_like.cpp:364-762): every inter-op activation is bf16, fp32
+ * inside an op, residual add fused into the projection with one rounding (:626-628,:703-705).
+ * Quantised linears use the fused evaluation order (scale applied to fp32 partial sums).
+ *
+ * The composition is pinned by tests/test_oracle_model.py: every op is one of the separately
+ * pinned oracle functions, and the whole pass is compared with an independent numpy fp64
+ * transformer on a tiny model (cosine of the logits, the tolerance precedent of
+ * driver/cuda/tests/parity_qwen3.py:160-181).
+ */
+#include <stdlib.h>
+
+#include "oracle_api.h"
+
+typedef struct {
+    const void* data;
+    const void* scale; /* int4: bf16 [N, K/G]; int8/fp8: f32 [N]; bf16: NULL */
+} OrcLinear;
+
+typedef struct {
+    int hidden, layers, q_heads, kv_heads, head_dim, intermediate, vocab;
+    float rms_eps;
+    int rope_interleaved, has_qk_norm;
+    int quant; /* 0 int4b8, 1 int8, 2 fp8, 3 bf16 */
+    int group;
+    const uint16_t* embed;
+    const uint16_t* lm_head;
+    const uint16_t* final_norm;
+    const float* inv_freq;
+    const uint16_t* const* attn_norm; /* [L] */
+    const uint16_t* const* ffn_norm;
+    const uint16_t* const* q_norm;
+    const uint16_t* const* k_norm;
+    const OrcLinear* wqkv; /* [L] */
+    const OrcLinear* wo;
+    const OrcLinear* wgu;
+    const OrcLinear* wdown;
+} OrcModel;
+
+static void orc_linear(const OrcModel* m, const OrcLinear* w, const uint16_t* act, uint16_t* y,
+                       int M, int N, int K, int beta) {
+    float* tmp = (float*)malloc(sizeof(float) * (size_t)M * N);
+    switch (m->quant) {
+        case 0:
+            orc_gemm_w4a16(act, (const uint32_t*)w->data, (const uint16_t*)w->scale, y, tmp, y, NULL,
+                           M, N, K, m->group, beta, 0);
+            break;
+        case 1:
+            orc_gemm_w8a16(act, (const int8_t*)w->data, (const float*)w->scale, y, tmp, y, NULL, M, N,
+                           K, beta, 0);
+            break;
+        case 2:
+            orc_gemm_fp8(act, (const uint8_t*)w->data, (const float*)w->scale, y, tmp, y, NULL, M, N, K,
+                         beta, 0);
+            break;
+        default:
+            orc_gemm_bf16(act, (const uint16_t*)w->data, y, tmp, y, NULL, M, N, K, beta, 0);
+            break;
+    }
+    free(tmp);
+}
+
+/*
+ * tokens/positions/kv_slots/row_begin/row_len: [N] as produced by the planner; k_pages/v_pages:
+ * [L] pools [pages, ps, hk, d], updated in place; sample_rows [S] -> out_tokens [S] and, when
+ * non-NULL, logits_bf16 [S, V].
+ */
+void orc_llama_forward(const OrcModel* m, uint16_t* const* k_pages, uint16_t* const* v_pages,
+                       const uint32_t* tokens, const int32_t* positions, const int64_t* kv_slots,
+                       const uint32_t* row_begin, const int32_t* row_len,
+                       const uint32_t* page_indices, int N, const uint32_t* sample_rows, int S,
+                       int page_size, uint32_t* out_tokens, uint16_t* logits_bf16) {
+    const int H = m->hidden, d = m->head_dim, hq = m->q_heads, hk = m->kv_heads;
+    const int I = m->intermediate, V = m->vocab;
+    const int qkv_dim = (hq + 2 * hk) * d;
+    uint16_t* x = (uint16_t*)malloc((size_t)N * H * 2);
+    uint16_t* xn = (uint16_t*)malloc((size_t)N * H * 2);
+    uint16_t* qkv = (uint16_t*)malloc((size_t)N * qkv_dim * 2);
+    uint16_t* q = (uint16_t*)malloc((size_t)N * hq * d * 2);
+    uint16_t* attn = (uint16_t*)malloc((size_t)N * hq * d * 2);
+    float* attn_f = (float*)malloc((size_t)N * hq * d * 4);
+    uint16_t* gu = (uint16_t*)malloc((size_t)N * 2 * I * 2);
+    uint16_t* act = (uint16_t*)malloc((size_t)N * I * 2);
+    float* tab = (float*)malloc((size_t)N * d * 4);
+
+    orc_embed(tokens, m->embed, x, N, H, V);
+    orc_rope_table(positions, m->inv_freq, tab, N, d);
+    for (int l = 0; l < m->layers; ++l) {
+        orc_rmsnorm(x, NULL, m->attn_norm[l], xn, N, H, m->rms_eps);
+        orc_linear(m, &m->wqkv[l], xn, qkv, N, qkv_dim, H, 0);
+        orc_qkv_rope_kvwrite(qkv, q, k_pages[l], v_pages[l], m->has_qk_norm ? m->q_norm[l] : NULL,
+                             m->has_qk_norm ? m->k_norm[l] : NULL, tab, kv_slots, N, hq, hk, d,
+                             m->rope_interleaved, m->rms_eps);
+        orc_attn_rows(q, k_pages[l], v_pages[l], attn_f, attn, NULL, page_indices, row_begin, row_len,
+                      N, hq, hk, d, page_size, -1.f, 0);
+        orc_linear(m, &m->wo[l], attn, x, N, H, hq * d, 1);
+        orc_rmsnorm(x, NULL, m->ffn_norm[l], xn, N, H, m->rms_eps);
+        orc_linear(m, &m->wgu[l], xn, gu, N, 2 * I, H, 0);
+        orc_swiglu(gu, act, N, I);
+        orc_linear(m, &m->wdown[l], act, x, N, H, I, 1);
+    }
+    if (S > 0) {
+        uint16_t* xs = (uint16_t*)malloc((size_t)S * H * 2);
+        uint16_t* xsn = (uint16_t*)malloc((size_t)S * H * 2);
+        uint16_t* lg = logits_bf16 ? logits_bf16 : (uint16_t*)malloc((size_t)S * V * 2);
+        float* lgf = (float*)malloc((size_t)S * V * 4);
+        orc_embed(sample_rows, x, xs, S, H, N); /* row gather */
+        orc_rmsnorm(xs, NULL, m->final_norm, xsn, S, H, m->rms_eps);
+        orc_gemm_bf16(xsn, m->lm_head, NULL, lgf, lg, NULL, S, V, H, 0, 0);
+        orc_argmax_bf16(lg, out_tokens, S, V);
+        free(xs);
+        free(xsn);
+        free(lgf);
+        if (!logits_bf16) free(lg);
+    }
+    free(x); free(xn); free(qkv); free(q); free(attn); free(attn_f); free(gu); free(act); free(tab);
+}

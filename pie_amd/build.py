@@ -17,6 +17,8 @@ CSRC = ROOT / "pie_amd" / "csrc"
 INCLUDE = ROOT / "include"
 OBJ_DIR = ROOT / "build" / "obj"
 KERNEL_LIB = ROOT / "pie_amd" / "libpie_hip_kernels.so"
+DRIVER_SRC = CSRC / "driver"
+DRIVER_LIB = ROOT / "pie_amd" / "libpie_driver_hip.so"
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 HIP_FLAGS = [
@@ -76,10 +78,34 @@ def build_kernels(force: bool = False, jobs: int | None = None) -> Path:
     return KERNEL_LIB
 
 
+def build_driver(force: bool = False, jobs: int | None = None) -> Path:
+    """The C++ host driver (`pie_driver_hip_run_inproc` and friends), linked against the
+    kernel library next to it."""
+    obj_dir = OBJ_DIR / "driver"
+    obj_dir.mkdir(parents=True, exist_ok=True)
+    headers = sorted(DRIVER_SRC.glob("*.hpp")) + sorted(INCLUDE.glob("*.h"))
+    todo, objs = [], []
+    for src in sorted(DRIVER_SRC.glob("*.hip")):
+        obj = obj_dir / (src.stem + ".o")
+        objs.append(obj)
+        if force or not _newer(obj, [src] + headers):
+            todo.append([HIPCC, *HIP_FLAGS, f"-I{DRIVER_SRC}", "-c", str(src), "-o", str(obj)])
+    jobs = jobs or min(8, os.cpu_count() or 1)
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        list(pool.map(_run, todo))
+    if force or todo or not DRIVER_LIB.exists() or not _newer(DRIVER_LIB, [KERNEL_LIB]):
+        _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(DRIVER_LIB),
+              *map(str, objs), f"-L{KERNEL_LIB.parent}", "-lpie_hip_kernels",
+              "-Wl,-rpath,$ORIGIN", "-lpthread"])
+    return DRIVER_LIB
+
+
 def build_all(force: bool = False) -> None:
     build_kernels(force=force)
+    build_driver(force=force)
 
 
 if __name__ == "__main__":
     build_all(force="--force" in sys.argv)
     print(KERNEL_LIB)
+    print(DRIVER_LIB)

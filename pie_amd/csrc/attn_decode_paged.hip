@@ -47,6 +47,24 @@ __device__ __forceinline__ float token_lanes_sum(float v) {
     return v;
 }
 
+// A query row's KV extent comes either from the wire arrays of a decode batch
+// (kv_page_indptr / kv_last_page_lens) or, when `row_len` is given, from explicit per-row
+// (first page-list entry, visible key count) pairs that a planner derived.
+struct RowExtent {
+    uint32_t pg_lo;
+    int kv_len;
+};
+__device__ __forceinline__ RowExtent row_extent(const uint32_t* __restrict__ page_indptr,
+                                                const uint32_t* __restrict__ last_lens,
+                                                const uint32_t* __restrict__ row_begin,
+                                                const int32_t* __restrict__ row_len, int r,
+                                                int ps) {
+    if (row_len) return {row_begin[r], row_len[r]};
+    const uint32_t lo = page_indptr[r];
+    const int npages = static_cast<int>(page_indptr[r + 1] - lo);
+    return {lo, npages > 0 ? (npages - 1) * ps + static_cast<int>(last_lens[r]) : 0};
+}
+
 template <int D, int GQA>
 struct UnitRegs {
     static constexpr int LPR = D / 8;
@@ -63,6 +81,7 @@ __global__ __launch_bounds__(kAttnBlock) void attn_decode_split_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_pages,
     const uint16_t* __restrict__ v_pages, const uint32_t* __restrict__ page_indices,
     const uint32_t* __restrict__ page_indptr, const uint32_t* __restrict__ last_lens,
+    const uint32_t* __restrict__ row_begin, const int32_t* __restrict__ row_len,
     float* __restrict__ part_o, float* __restrict__ part_ml, uint16_t* __restrict__ o_direct,
     float* __restrict__ lse, int hq, int hk, int ps, int units_per_split, int nsplit,
     float scale_log2e) {
@@ -73,9 +92,9 @@ __global__ __launch_bounds__(kAttnBlock) void attn_decode_split_kernel(
     const int wv = __builtin_amdgcn_readfirstlane(tid / kWave);  // wave-uniform -> SGPR
     const int grp = lane / LPR, dl = lane % LPR;
 
-    const uint32_t pg_lo = page_indptr[r];
-    const int npages = static_cast<int>(page_indptr[r + 1] - pg_lo);
-    const int kv_len = npages > 0 ? (npages - 1) * ps + static_cast<int>(last_lens[r]) : 0;
+    const RowExtent ext = row_extent(page_indptr, last_lens, row_begin, row_len, r, ps);
+    const uint32_t pg_lo = ext.pg_lo;
+    const int kv_len = ext.kv_len;
     const int nunits = (kv_len + kUnitTokens - 1) / kUnitTokens;
     const int u_begin = split * units_per_split;
     if (u_begin >= nunits) return;
@@ -263,13 +282,14 @@ __global__ void attn_decode_merge_kernel(const float* __restrict__ part_o,
                                          const float* __restrict__ part_ml,
                                          const uint32_t* __restrict__ page_indptr,
                                          const uint32_t* __restrict__ last_lens,
+                                         const uint32_t* __restrict__ row_begin,
+                                         const int32_t* __restrict__ row_len,
                                          uint16_t* __restrict__ o, float* __restrict__ lse, int hq,
                                          int ps, int units_per_split, int nsplit) {
     const int rh = blockIdx.x;
     const int r = rh / hq;
     const int dd = threadIdx.x;
-    const int npages = static_cast<int>(page_indptr[r + 1] - page_indptr[r]);
-    const int kv_len = npages > 0 ? (npages - 1) * ps + static_cast<int>(last_lens[r]) : 0;
+    const int kv_len = row_extent(page_indptr, last_lens, row_begin, row_len, r, ps).kv_len;
     const int nunits = (kv_len + kUnitTokens - 1) / kUnitTokens;
     const int ns = min(nsplit, (nunits + units_per_split - 1) / units_per_split);
     float mx = -INFINITY;
@@ -291,12 +311,13 @@ __global__ void attn_decode_merge_kernel(const float* __restrict__ part_o,
 template <int D>
 __global__ void attn_decode_clear_empty_kernel(const uint32_t* __restrict__ page_indptr,
                                                const uint32_t* __restrict__ last_lens,
+                                               const uint32_t* __restrict__ row_begin,
+                                               const int32_t* __restrict__ row_len,
                                                uint16_t* __restrict__ o, float* __restrict__ lse,
                                                int hq, int ps) {
     const int rh = blockIdx.x;
     const int r = rh / hq;
-    const int npages = static_cast<int>(page_indptr[r + 1] - page_indptr[r]);
-    const int kv_len = npages > 0 ? (npages - 1) * ps + static_cast<int>(last_lens[r]) : 0;
+    const int kv_len = row_extent(page_indptr, last_lens, row_begin, row_len, r, ps).kv_len;
     if (kv_len > 0) return;
     o[static_cast<size_t>(rh) * D + threadIdx.x] = 0;
     if (lse && threadIdx.x == 0) lse[rh] = -INFINITY;
@@ -326,16 +347,18 @@ SplitPlan plan_splits(int R, int hk, int max_kv_len) {
 template <int D, int GQA>
 int launch_decode(const uint16_t* q, const uint16_t* k_pages, const uint16_t* v_pages, uint16_t* o,
                   float* lse, const uint32_t* page_indices, const uint32_t* page_indptr,
-                  const uint32_t* last_lens, int R, int hq, int hk, int ps, float sm_scale,
+                  const uint32_t* last_lens, const uint32_t* row_begin, const int32_t* row_len,
+                  int R, int hq, int hk, int ps, float sm_scale,
                   int max_kv_len, void* workspace, size_t workspace_bytes, hipStream_t stream) {
     const SplitPlan plan = plan_splits(R, hk, max_kv_len);
     const float scale_log2e = sm_scale * 1.4426950408889634f;
     if (plan.nsplit == 1) {
         hipLaunchKernelGGL((attn_decode_clear_empty_kernel<D>), dim3(R * hq), dim3(D), 0, stream,
-                           page_indptr, last_lens, o, lse, hq, ps);
+                           page_indptr, last_lens, row_begin, row_len, o, lse, hq, ps);
         hipLaunchKernelGGL((attn_decode_split_kernel<D, GQA>), dim3(1, hk, R), dim3(kAttnBlock), 0,
                            stream, q, k_pages, v_pages, page_indices, page_indptr, last_lens,
-                           nullptr, nullptr, o, lse, hq, hk, ps, plan.units_per_split, 1,
+                           row_begin, row_len, nullptr, nullptr, o, lse, hq, hk, ps,
+                           plan.units_per_split, 1,
                            scale_log2e);
         return launch_status();
     }
@@ -346,10 +369,11 @@ int launch_decode(const uint16_t* q, const uint16_t* k_pages, const uint16_t* v_
     float* part_ml = part_o + n_part * D;
     hipLaunchKernelGGL((attn_decode_split_kernel<D, GQA>), dim3(plan.nsplit, hk, R),
                        dim3(kAttnBlock), 0, stream, q, k_pages, v_pages, page_indices, page_indptr,
-                       last_lens, part_o, part_ml, nullptr, nullptr, hq, hk, ps,
+                       last_lens, row_begin, row_len, part_o, part_ml, nullptr, nullptr, hq, hk, ps,
                        plan.units_per_split, plan.nsplit, scale_log2e);
     hipLaunchKernelGGL((attn_decode_merge_kernel<D>), dim3(R * hq), dim3(D), 0, stream, part_o,
-                       part_ml, page_indptr, last_lens, o, lse, hq, ps, plan.units_per_split,
+                       part_ml, page_indptr, last_lens, row_begin, row_len, o, lse, hq, ps,
+                       plan.units_per_split,
                        plan.nsplit);
     return launch_status();
 }
@@ -367,31 +391,29 @@ extern "C" size_t pie_hip_attn_decode_workspace_bytes(int num_requests, int num_
            sizeof(float);
 }
 
-extern "C" int pie_hip_attn_decode_paged(const uint16_t* q, const uint16_t* k_pages,
-                                         const uint16_t* v_pages, uint16_t* o, float* lse,
-                                         const uint32_t* kv_page_indices,
-                                         const uint32_t* kv_page_indptr,
-                                         const uint32_t* kv_last_page_lens, int num_requests,
-                                         int num_q_heads, int num_kv_heads, int head_dim,
-                                         int page_size, float sm_scale, int max_kv_len,
-                                         void* workspace, size_t workspace_bytes, void* stream) {
-    using namespace pie_hip;
-    if (!q || !k_pages || !v_pages || !o || !kv_page_indices || !kv_page_indptr ||
-        !kv_last_page_lens || num_requests <= 0 || num_q_heads <= 0 || num_kv_heads <= 0 ||
-        page_size <= 0 || max_kv_len < 0)
+namespace pie_hip {
+namespace {
+int attn_dispatch(const uint16_t* q, const uint16_t* k_pages, const uint16_t* v_pages, uint16_t* o,
+                  float* lse, const uint32_t* kv_page_indices, const uint32_t* kv_page_indptr,
+                  const uint32_t* kv_last_page_lens, const uint32_t* row_begin,
+                  const int32_t* row_len, int num_rows, int num_q_heads, int num_kv_heads,
+                  int head_dim, int page_size, float sm_scale, int max_kv_len, void* workspace,
+                  size_t workspace_bytes, void* stream) {
+    if (!q || !k_pages || !v_pages || !o || !kv_page_indices || num_rows <= 0 ||
+        num_q_heads <= 0 || num_kv_heads <= 0 || page_size <= 0 || max_kv_len < 0)
         return PIE_HIP_ERR_INVALID;
     if (num_q_heads % num_kv_heads != 0 || page_size % kUnitTokens != 0)
         return PIE_HIP_ERR_UNSUPPORTED;
-    if (num_requests > 65535 || num_kv_heads > 65535) return PIE_HIP_ERR_UNSUPPORTED;
+    if (num_rows > 65535 || num_kv_heads > 65535) return PIE_HIP_ERR_UNSUPPORTED;
     const float scale = sm_scale > 0.f ? sm_scale : 1.0f / sqrtf(static_cast<float>(head_dim));
     const int gqa = num_q_heads / num_kv_heads;
     hipStream_t st = static_cast<hipStream_t>(stream);
 #define PIE_ATTN_CASE(DD, GG)                                                                  \
     if (head_dim == DD && gqa == GG)                                                           \
         return launch_decode<DD, GG>(q, k_pages, v_pages, o, lse, kv_page_indices,             \
-                                     kv_page_indptr, kv_last_page_lens, num_requests,          \
-                                     num_q_heads, num_kv_heads, page_size, scale, max_kv_len,  \
-                                     workspace, workspace_bytes, st);
+                                     kv_page_indptr, kv_last_page_lens, row_begin, row_len,    \
+                                     num_rows, num_q_heads, num_kv_heads, page_size, scale,    \
+                                     max_kv_len, workspace, workspace_bytes, st);
     PIE_ATTN_CASE(128, 1)
     PIE_ATTN_CASE(128, 2)
     PIE_ATTN_CASE(128, 4)
@@ -402,4 +424,36 @@ extern "C" int pie_hip_attn_decode_paged(const uint16_t* q, const uint16_t* k_pa
     PIE_ATTN_CASE(64, 8)
 #undef PIE_ATTN_CASE
     return PIE_HIP_ERR_UNSUPPORTED;
+}
+}  // namespace
+}  // namespace pie_hip
+
+extern "C" int pie_hip_attn_decode_paged(const uint16_t* q, const uint16_t* k_pages,
+                                         const uint16_t* v_pages, uint16_t* o, float* lse,
+                                         const uint32_t* kv_page_indices,
+                                         const uint32_t* kv_page_indptr,
+                                         const uint32_t* kv_last_page_lens, int num_requests,
+                                         int num_q_heads, int num_kv_heads, int head_dim,
+                                         int page_size, float sm_scale, int max_kv_len,
+                                         void* workspace, size_t workspace_bytes, void* stream) {
+    if (!kv_page_indptr || !kv_last_page_lens) return PIE_HIP_ERR_INVALID;
+    return pie_hip::attn_dispatch(q, k_pages, v_pages, o, lse, kv_page_indices, kv_page_indptr,
+                                  kv_last_page_lens, nullptr, nullptr, num_requests, num_q_heads,
+                                  num_kv_heads, head_dim, page_size, sm_scale, max_kv_len,
+                                  workspace, workspace_bytes, stream);
+}
+
+extern "C" int pie_hip_attn_rows_paged(const uint16_t* q, const uint16_t* k_pages,
+                                       const uint16_t* v_pages, uint16_t* o, float* lse,
+                                       const uint32_t* kv_page_indices,
+                                       const uint32_t* row_page_begin, const int32_t* row_kv_len,
+                                       int num_rows, int num_q_heads, int num_kv_heads,
+                                       int head_dim, int page_size, float sm_scale,
+                                       int max_kv_len, void* workspace, size_t workspace_bytes,
+                                       void* stream) {
+    if (!row_page_begin || !row_kv_len) return PIE_HIP_ERR_INVALID;
+    return pie_hip::attn_dispatch(q, k_pages, v_pages, o, lse, kv_page_indices, nullptr, nullptr,
+                                  row_page_begin, row_kv_len, num_rows, num_q_heads, num_kv_heads,
+                                  head_dim, page_size, sm_scale, max_kv_len, workspace,
+                                  workspace_bytes, stream);
 }

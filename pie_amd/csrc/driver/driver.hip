@@ -1,0 +1,540 @@
+// The `hip` driver flavour: request dispatch, response packing, the serve loop and the
+// exported entry points.
+//
+//   serve loop / handler contract  driver/bridge/include/pie_bridge/inproc_server.hpp:35-96
+//   method dispatch + status codes driver/portable/src/service/inproc_service.cpp:54-320
+//   response CSR shape             driver/bridge/include/pie_bridge/response_builder.hpp:52-271
+//   entry points                   driver/portable/src/entry.cpp:483-505, server/src/driver_ffi.rs:18-46
+//   offline generation harness     driver/portable/src/executor/executor.cpp:1439-1597
+#include <atomic>
+#include <chrono>
+#include <csignal>
+#include <cstdio>
+#include <cstring>
+#include <memory>
+#include <mutex>
+#include <sstream>
+#include <string>
+#include <vector>
+
+#include "config.hpp"
+#include "executor.hpp"
+#include "model.hpp"
+#include "pie_driver_abi.h"
+#include "planner.hpp"
+
+using namespace pie_hip_driver;
+
+namespace {
+
+std::atomic<bool> g_stop{false};
+
+using clk = std::chrono::steady_clock;
+uint32_t us_since(clk::time_point t0) {
+    return static_cast<uint32_t>(
+        std::chrono::duration_cast<std::chrono::microseconds>(clk::now() - t0).count());
+}
+
+uint32_t method_of(const PieFrameDesc& f) {
+    const PieRequestPayloadDesc& p = f.payload;
+    switch (p.kind) {
+        case PIE_REQ_FORWARD: return PIE_METHOD_FORWARD;
+        case PIE_REQ_COPY:
+            if (p.copy.dir > PIE_COPY_H2H) return PIE_METHOD_UNKNOWN;
+            if (p.copy.resource == PIE_RESOURCE_KV) return PIE_METHOD_COPY_KV_D2H + p.copy.dir;
+            if (p.copy.resource == PIE_RESOURCE_RS) return PIE_METHOD_COPY_RS_D2H + p.copy.dir;
+            return PIE_METHOD_UNKNOWN;
+        case PIE_REQ_ADAPTER:
+            if (p.adapter.op == PIE_ADAPTER_GENERATE_AUDIO) return PIE_METHOD_GENERATE_AUDIO;
+            if (p.adapter.op <= PIE_ADAPTER_ZO_UPDATE) return PIE_METHOD_ADAPTER_LOAD + p.adapter.op;
+            return PIE_METHOD_UNKNOWN;
+        case PIE_REQ_HEALTH: return PIE_METHOD_HEALTH;
+        default: return PIE_METHOD_UNKNOWN;
+    }
+}
+
+// Driver-owned storage behind a PieForwardResponseDesc; reused across calls.
+struct ResponseStore {
+    std::vector<uint32_t> tokens_indptr, tokens, dists_req_indptr, dists_kv_indptr,
+        logits_req_indptr, logits_byte_indptr, logprobs_req_indptr, logprobs_val_indptr,
+        entropies_indptr, spec_indptr;
+
+    // R requests, every list empty except tokens (per-request CSR from sample_indptr).
+    void build(int R, const std::vector<int32_t>& sample_indptr, const std::vector<uint32_t>& toks,
+               PieForwardResponseDesc& out) {
+        std::memset(&out, 0, sizeof(out));
+        const size_t n1 = static_cast<size_t>(R) + 1;
+        tokens_indptr.assign(n1, 0);
+        for (int r = 0; r <= R && r < static_cast<int>(sample_indptr.size()); ++r)
+            tokens_indptr[r] = static_cast<uint32_t>(sample_indptr[r]);
+        tokens = toks;
+        dists_req_indptr.assign(n1, 0);
+        logits_req_indptr.assign(n1, 0);
+        logprobs_req_indptr.assign(n1, 0);
+        entropies_indptr.assign(n1, 0);
+        spec_indptr.assign(n1, 0);
+        dists_kv_indptr.assign(1, 0);      // second-level indptrs start with a leading 0
+        logits_byte_indptr.assign(1, 0);
+        logprobs_val_indptr.assign(1, 0);
+        out.num_requests = static_cast<uint32_t>(R);
+        out.tokens_indptr = {tokens_indptr.data(), tokens_indptr.size()};
+        out.tokens = {tokens.data(), tokens.size()};
+        out.dists_req_indptr = {dists_req_indptr.data(), dists_req_indptr.size()};
+        out.dists_kv_indptr = {dists_kv_indptr.data(), dists_kv_indptr.size()};
+        out.logits_req_indptr = {logits_req_indptr.data(), logits_req_indptr.size()};
+        out.logits_byte_indptr = {logits_byte_indptr.data(), logits_byte_indptr.size()};
+        out.logprobs_req_indptr = {logprobs_req_indptr.data(), logprobs_req_indptr.size()};
+        out.logprobs_val_indptr = {logprobs_val_indptr.data(), logprobs_val_indptr.size()};
+        out.entropies_indptr = {entropies_indptr.data(), entropies_indptr.size()};
+        out.spec_indptr = {spec_indptr.data(), spec_indptr.size()};
+    }
+    // Failure shape: num_requests = 0, nothing else (driver/portable/src/executor/executor.cpp:1325-1341).
+    static void build_failed(PieForwardResponseDesc& out) { std::memset(&out, 0, sizeof(out)); }
+};
+
+std::string json_escape(const std::string& s) {
+    std::string o;
+    for (char c : s) {
+        if (c == '"' || c == '\\') { o.push_back('\\'); o.push_back(c); }
+        else if (static_cast<unsigned char>(c) < 0x20) { char b[8]; std::snprintf(b, sizeof b, "\\u%04x", c); o += b; }
+        else o.push_back(c);
+    }
+    return o;
+}
+
+}  // namespace
+
+struct PieHipDriver {
+    DriverConfig cfg;
+    Model model;
+    std::unique_ptr<Executor> exec;
+    std::string caps;
+    ResponseStore store;
+    std::vector<uint32_t> toks;
+    std::string last_error;
+
+    explicit PieHipDriver(const DriverConfig& c) : cfg(c) {
+        int ndev = 0;
+        if (hipGetDeviceCount(&ndev) != hipSuccess || ndev <= 0)
+            throw std::runtime_error("no HIP device is visible: this driver has no CPU path");
+        hipStream_t s = nullptr;
+        if (hipStreamCreateWithFlags(&s, hipStreamNonBlocking) != hipSuccess)
+            throw std::runtime_error("cannot create a HIP stream");
+        try {
+            model.init_synthetic(cfg.model, s);
+        } catch (...) {
+            (void)hipStreamDestroy(s);
+            throw;
+        }
+        (void)hipStreamDestroy(s);
+        exec = std::make_unique<Executor>(cfg, model);
+        build_caps();
+    }
+
+    // Capabilities handshake (driver/bridge/src/capabilities.rs:18-78; values as
+    // driver/portable/src/entry.cpp:432-452).
+    void build_caps() {
+        const auto& m = cfg.model;
+        const long long total_pages = exec->total_pages();
+        const long long ps = exec->page_size();
+        const unsigned long long umax = 4294967295ull;
+        std::ostringstream j;
+        j << "{\"total_pages\":" << total_pages << ",\"kv_page_size\":" << ps
+          << ",\"swap_pool_size\":" << cfg.batching.cpu_pages
+          << ",\"rs_cache_required\":false,\"rs_cache_slots\":0,\"rs_cache_slot_bytes\":0"
+          << ",\"max_forward_tokens\":" << cfg.batching.max_forward_tokens
+          << ",\"max_forward_requests\":" << cfg.batching.max_forward_requests
+          << ",\"max_page_refs\":" << total_pages << ",\"max_logit_rows\":" << umax
+          << ",\"max_prob_rows\":" << umax << ",\"max_custom_mask_bytes\":" << umax
+          << ",\"max_sampler_rows\":" << umax << ",\"max_logprob_labels\":" << umax
+          << ",\"arch_name\":\"" << json_escape(m.arch) << "\",\"vocab_size\":" << m.vocab
+          << ",\"max_model_len\":" << total_pages * ps << ",\"activation_dtype\":\"bfloat16\""
+          << ",\"snapshot_dir\":\"" << json_escape(cfg.runtime.snapshot_dir) << "\"}";
+        caps = j.str();
+    }
+
+    void forward(const PieForwardRequestDesc& f, PieForwardResponseDesc& out) {
+        const auto t_start = clk::now();
+        // Empty batch: R empty per-request outputs (driver/portable/src/executor/executor.cpp:1310-1322).
+        const int R = f.qo_indptr.len > 0 ? static_cast<int>(f.qo_indptr.len) - 1 : 0;
+        if (f.token_ids.len == 0 || R <= 0) {
+            store.build(R > 0 ? R : 0, std::vector<int32_t>(static_cast<size_t>(R > 0 ? R : 0) + 1, 0), {}, out);
+            return;
+        }
+        try {
+            auto t0 = clk::now();
+            const BatchPlan plan = plan_forward(f, exec->page_size(), exec->total_pages());
+            if (plan.has_user_masks)
+                throw std::runtime_error("forward: custom attention masks are not supported by this driver yet");
+            if (!plan.all_greedy && !plan.sample_rows.empty())
+                throw std::runtime_error("forward: only greedy (temperature 0) token samplers are supported yet");
+            if (R > cfg.batching.max_forward_requests)
+                throw std::runtime_error("forward: batch exceeds max_forward_requests");
+            const uint32_t plan_us = us_since(t0);
+            ForwardTimings ft;
+            exec->forward(plan, toks, &ft);
+            t0 = clk::now();
+            store.build(plan.R, plan.sample_indptr, toks, out);
+            out.probe_wire_parse_us = 0;
+            out.probe_plan_us = plan_us;
+            out.probe_h2d_us = ft.h2d_us;
+            out.probe_kernel_launch_us = ft.launch_us;
+            out.probe_sync_us = ft.sync_us;
+            out.probe_response_build_us = us_since(t0);
+            (void)t_start;
+        } catch (const std::exception& e) {
+            last_error = e.what();
+            if (cfg.runtime.verbose) std::fprintf(stderr, "[pie-driver-hip] forward failed: %s\n", e.what());
+            ResponseStore::build_failed(out);
+        }
+    }
+
+    int copy(const PieCopyRequestDesc& c, uint32_t method) {
+        if (c.srcs.len != c.dsts.len) return PIE_STATUS_FAILED;
+        if (method >= PIE_METHOD_COPY_RS_D2H) return PIE_STATUS_UNSUPPORTED;  // no recurrent state
+        const uint32_t total = static_cast<uint32_t>(exec->total_pages());
+        switch (method) {
+            case PIE_METHOD_COPY_KV_D2D:
+                for (size_t i = 0; i < c.srcs.len; ++i)
+                    if (c.srcs.ptr[i] >= total || c.dsts.ptr[i] >= total) return PIE_STATUS_OUT_OF_RANGE;
+                exec->copy_pages_d2d(c.srcs.ptr, c.dsts.ptr, c.srcs.len);
+                return PIE_STATUS_OK;
+            default:
+                return PIE_STATUS_UNSUPPORTED;  // no host swap pool (cpu_pages = 0)
+        }
+    }
+
+    void handle(const PieFrameDesc& frame, PieResponseFrameDesc& out) {
+        std::memset(&out, 0, sizeof(out));
+        out.driver_id = frame.driver_id;
+        const uint32_t method = method_of(frame);
+        if (method == PIE_METHOD_FORWARD) {
+            out.payload.kind = PIE_RESP_FORWARD;
+            forward(frame.payload.forward, out.payload.forward);
+            return;
+        }
+        out.payload.kind = PIE_RESP_STATUS;
+        int status;
+        try {
+            switch (method) {
+                case PIE_METHOD_COPY_KV_D2H: case PIE_METHOD_COPY_KV_H2D: case PIE_METHOD_COPY_KV_D2D:
+                case PIE_METHOD_COPY_KV_H2H: case PIE_METHOD_COPY_RS_D2H: case PIE_METHOD_COPY_RS_H2D:
+                case PIE_METHOD_COPY_RS_D2D: case PIE_METHOD_COPY_RS_H2H:
+                    status = copy(frame.payload.copy, method);
+                    break;
+                case PIE_METHOD_HEALTH: status = PIE_STATUS_OK; break;
+                case PIE_METHOD_ADAPTER_LOAD: case PIE_METHOD_ADAPTER_SAVE:
+                case PIE_METHOD_ADAPTER_ZO_INIT: case PIE_METHOD_ADAPTER_ZO_UPDATE:
+                case PIE_METHOD_GENERATE_AUDIO:
+                    status = PIE_STATUS_UNSUPPORTED;
+                    break;
+                default: status = PIE_STATUS_UNKNOWN_METHOD; break;
+            }
+        } catch (const std::exception& e) {
+            last_error = e.what();
+            status = PIE_STATUS_EXCEPTION;
+        }
+        out.payload.status.status = status;
+    }
+};
+
+namespace {
+
+void set_err(char* err, size_t cap, const std::string& msg) {
+    if (err && cap) {
+        std::snprintf(err, cap, "%s", msg.c_str());
+    }
+}
+
+// Fills a forward frame over borrowed vectors (the harness plays the runtime's role).
+struct FrameBuilder {
+    std::vector<uint32_t> tokens, positions, pages, page_indptr, last_lens, qo_indptr, samp_idx,
+        samp_indptr, sampler_indptr;
+    std::vector<PieSamplerDesc> samplers;
+    std::vector<uint64_t> ctx_ids;
+    PieFrameDesc frame;
+    void finish() {
+        std::memset(&frame, 0, sizeof(frame));
+        frame.payload.kind = PIE_REQ_FORWARD;
+        PieForwardRequestDesc& f = frame.payload.forward;
+        f.token_ids = {tokens.data(), tokens.size()};
+        f.position_ids = {positions.data(), positions.size()};
+        f.kv_page_indices = {pages.data(), pages.size()};
+        f.kv_page_indptr = {page_indptr.data(), page_indptr.size()};
+        f.kv_last_page_lens = {last_lens.data(), last_lens.size()};
+        f.qo_indptr = {qo_indptr.data(), qo_indptr.size()};
+        f.sampling_indices = {samp_idx.data(), samp_idx.size()};
+        f.sampling_indptr = {samp_indptr.data(), samp_indptr.size()};
+        f.samplers = {samplers.data(), samplers.size()};
+        f.sampler_indptr = {sampler_indptr.data(), sampler_indptr.size()};
+        f.context_ids = {ctx_ids.data(), ctx_ids.size()};
+        f.single_token_mode = 1;
+    }
+};
+
+PieSamplerDesc greedy_sampler() {
+    // greedy arrives on the wire as TopP{temperature 0, p 1} (sdk/rust/inferlet/src/sample.rs:77-79)
+    PieSamplerDesc s;
+    std::memset(&s, 0, sizeof(s));
+    s.kind = PIE_SAMPLER_KIND_TOP_P;
+    s.temperature = 0.f;
+    s.p = 1.f;
+    return s;
+}
+
+}  // namespace
+
+extern "C" PieHipDriver* pie_hip_driver_create(const char* config_toml, char* err, size_t err_cap) {
+    try {
+        if (!config_toml) throw std::runtime_error("null config");
+        return new PieHipDriver(load_config(config_toml));
+    } catch (const std::exception& e) {
+        set_err(err, err_cap, e.what());
+        return nullptr;
+    } catch (...) {
+        set_err(err, err_cap, "unknown error");
+        return nullptr;
+    }
+}
+
+extern "C" void pie_hip_driver_destroy(PieHipDriver* d) { delete d; }
+
+extern "C" const char* pie_hip_driver_capabilities(const PieHipDriver* d) {
+    return d ? d->caps.c_str() : nullptr;
+}
+
+extern "C" int pie_hip_driver_handle(PieHipDriver* d, const PieFrameDesc* frame,
+                                     PieResponseFrameDesc* out) {
+    if (!d || !frame || !out) return -1;
+    try {
+        d->handle(*frame, *out);
+    } catch (...) {  // handler exception -> status -1 (inproc_server.hpp:66-74)
+        std::memset(out, 0, sizeof(*out));
+        out->payload.kind = PIE_RESP_STATUS;
+        out->payload.status.status = PIE_STATUS_EXCEPTION;
+    }
+    return 0;
+}
+
+extern "C" size_t pie_hip_driver_export_tensor(PieHipDriver* d, const char* name, void* dst,
+                                               size_t cap) {
+    if (!d || !name) return 0;
+    if (std::string(name) == "debug.logits") {
+        const size_t bytes = static_cast<size_t>(d->exec->last_logit_rows()) * d->cfg.model.vocab * 2;
+        if (dst && bytes) {
+            const size_t n = bytes < cap ? bytes : cap;
+            if (hipMemcpy(dst, d->exec->last_logits(), n, hipMemcpyDeviceToHost) != hipSuccess) return 0;
+        }
+        return bytes;
+    }
+    const auto& t = d->model.tensors();
+    const auto it = t.find(name);
+    if (it == t.end()) return 0;
+    if (dst) {
+        const size_t n = it->second.bytes < cap ? it->second.bytes : cap;
+        if (hipMemcpy(dst, it->second.ptr, n, hipMemcpyDeviceToHost) != hipSuccess) return 0;
+    }
+    return it->second.bytes;
+}
+
+extern "C" int pie_hip_driver_generate(PieHipDriver* d, const uint32_t* prompt, int n_prompt,
+                                       int max_new, int replicate, uint32_t* out_tokens,
+                                       double* timings_us, char* err, size_t err_cap) {
+    if (!d || !prompt || n_prompt <= 0 || max_new <= 0 || replicate <= 0 || !out_tokens) {
+        set_err(err, err_cap, "bad arguments");
+        return -1;
+    }
+    try {
+        const int ps = d->exec->page_size();
+        const int pages_per_ctx = (n_prompt + max_new + ps - 1) / ps;
+        if (static_cast<long long>(pages_per_ctx) * replicate > d->exec->total_pages())
+            throw std::runtime_error("generate: needs " + std::to_string(pages_per_ctx * replicate) +
+                                     " pages, pool has " + std::to_string(d->exec->total_pages()));
+        if (replicate > d->cfg.batching.max_forward_requests)
+            throw std::runtime_error("generate: replicate exceeds max_forward_requests");
+        PieResponseFrameDesc resp;
+        std::vector<uint32_t> last(replicate);
+        const int chunk_cap = d->cfg.batching.max_forward_tokens;
+        const auto t_prefill = clk::now();
+        // Prefill: one plan per context (contiguous page range), chunked to the token cap;
+        // only the final chunk samples.
+        for (int c = 0; c < replicate; ++c) {
+            for (int t0 = 0; t0 < n_prompt; t0 += chunk_cap) {
+                const int n = std::min(chunk_cap, n_prompt - t0);
+                const int upto = t0 + n;  // tokens in the context after this chunk
+                FrameBuilder fb;
+                fb.tokens.assign(prompt + t0, prompt + upto);
+                for (int i = t0; i < upto; ++i) fb.positions.push_back(static_cast<uint32_t>(i));
+                const int np = (upto + ps - 1) / ps;
+                for (int p = 0; p < np; ++p) fb.pages.push_back(static_cast<uint32_t>(c * pages_per_ctx + p));
+                fb.page_indptr = {0u, static_cast<uint32_t>(np)};
+                fb.last_lens = {static_cast<uint32_t>(upto - (np - 1) * ps)};
+                fb.qo_indptr = {0u, static_cast<uint32_t>(n)};
+                fb.ctx_ids = {static_cast<uint64_t>(c)};
+                const bool final_chunk = upto == n_prompt;
+                if (final_chunk) {
+                    fb.samp_idx = {static_cast<uint32_t>(n - 1)};
+                    fb.samp_indptr = {0u, 1u};
+                    fb.samplers = {greedy_sampler()};
+                    fb.sampler_indptr = {0u, 1u};
+                } else {
+                    fb.samp_indptr = {0u, 0u};
+                    fb.sampler_indptr = {0u, 0u};
+                }
+                fb.finish();
+                fb.frame.payload.forward.single_token_mode = 0;
+                d->handle(fb.frame, resp);
+                const PieForwardResponseDesc& fr = resp.payload.forward;
+                if (fr.num_requests != 1) throw std::runtime_error("generate: prefill failed: " + d->last_error);
+                if (final_chunk) {
+                    if (fr.tokens.len != 1) throw std::runtime_error("generate: prefill returned no token");
+                    last[c] = fr.tokens.ptr[0];
+                    out_tokens[static_cast<size_t>(c) * max_new] = last[c];
+                }
+            }
+        }
+        const double prefill_us = us_since(t_prefill);
+        // Decode: one multi-request single-token plan per step.
+        hipEvent_t e0 = nullptr, e1 = nullptr;
+        (void)hipEventCreate(&e0);
+        (void)hipEventCreate(&e1);
+        const auto t_decode = clk::now();
+        (void)hipEventRecord(e0, d->exec->stream());
+        for (int s = 1; s < max_new; ++s) {
+            const int pos = n_prompt + s - 1;  // position of the token fed in this step
+            const int np = (pos + 1 + ps - 1) / ps;
+            FrameBuilder fb;
+            for (int c = 0; c < replicate; ++c) {
+                fb.tokens.push_back(last[c]);
+                fb.positions.push_back(static_cast<uint32_t>(pos));
+                for (int p = 0; p < np; ++p) fb.pages.push_back(static_cast<uint32_t>(c * pages_per_ctx + p));
+                fb.last_lens.push_back(static_cast<uint32_t>(pos + 1 - (np - 1) * ps));
+                fb.samp_idx.push_back(0u);
+                fb.samplers.push_back(greedy_sampler());
+                fb.ctx_ids.push_back(static_cast<uint64_t>(c));
+            }
+            for (int c = 0; c <= replicate; ++c) {
+                fb.page_indptr.push_back(static_cast<uint32_t>(c * np));
+                fb.qo_indptr.push_back(static_cast<uint32_t>(c));
+                fb.samp_indptr.push_back(static_cast<uint32_t>(c));
+                fb.sampler_indptr.push_back(static_cast<uint32_t>(c));
+            }
+            fb.finish();
+            d->handle(fb.frame, resp);
+            const PieForwardResponseDesc& fr = resp.payload.forward;
+            if (fr.num_requests != static_cast<uint32_t>(replicate) || fr.tokens.len != static_cast<size_t>(replicate))
+                throw std::runtime_error("generate: decode step failed: " + d->last_error);
+            for (int c = 0; c < replicate; ++c) {
+                last[c] = fr.tokens.ptr[c];
+                out_tokens[static_cast<size_t>(c) * max_new + s] = last[c];
+            }
+        }
+        (void)hipEventRecord(e1, d->exec->stream());
+        (void)hipEventSynchronize(e1);
+        float dev_ms = 0.f;
+        (void)hipEventElapsedTime(&dev_ms, e0, e1);
+        (void)hipEventDestroy(e0);
+        (void)hipEventDestroy(e1);
+        if (timings_us) {
+            timings_us[0] = prefill_us;
+            timings_us[1] = us_since(t_decode);
+            timings_us[2] = static_cast<double>(dev_ms) * 1e3;
+            timings_us[3] = static_cast<double>(max_new - 1);
+        }
+        return 0;
+    } catch (const std::exception& e) {
+        set_err(err, err_cap, e.what());
+        return -2;
+    } catch (...) {
+        set_err(err, err_cap, "unknown error");
+        return -3;
+    }
+}
+
+extern "C" void pie_driver_hip_request_stop(void) { g_stop.store(true, std::memory_order_release); }
+
+extern "C" int pie_driver_hip_run_inproc(int argc, char** argv, int install_signal_handlers,
+                                         void (*ready_cb)(const char* caps_json, void* ctx),
+                                         void* ready_ctx, PieInProcVTable vtable) {
+    try {
+        std::string config_path;
+        for (int i = 1; i < argc; ++i) {
+            const std::string a = argv[i] ? argv[i] : "";
+            if ((a == "--config" || a == "-c") && i + 1 < argc) config_path = argv[++i];
+            else if (a.rfind("--config=", 0) == 0) config_path = a.substr(9);
+        }
+        if (config_path.empty()) {
+            std::fprintf(stderr, "[pie-driver-hip] missing --config <file.toml>\n");
+            return -1;
+        }
+        if (!vtable.recv || !vtable.send_response) {
+            std::fprintf(stderr, "[pie-driver-hip] incomplete vtable\n");
+            return -1;
+        }
+        if (install_signal_handlers) {
+            std::signal(SIGINT, [](int) { g_stop.store(true); });
+            std::signal(SIGTERM, [](int) { g_stop.store(true); });
+        }
+        g_stop.store(false, std::memory_order_release);
+        PieHipDriver driver(load_config(config_path));
+        if (ready_cb) ready_cb(driver.caps.c_str(), ready_ctx);
+        if (driver.cfg.runtime.verbose) std::fprintf(stderr, "[pie-driver-hip] serving on in-process channel\n");
+        PieResponseFrameDesc resp;
+        while (!g_stop.load(std::memory_order_acquire)) {
+            const PieFrameDesc* req = nullptr;
+            uint32_t req_id = 0;
+            const int32_t rc = vtable.recv(vtable.ctx, &req, &req_id);
+            if (rc != 0) break;  // -1 clean shutdown, anything else an error: stop either way
+            if (!req) continue;
+            try {
+                driver.handle(*req, resp);
+            } catch (...) {
+                std::memset(&resp, 0, sizeof(resp));
+                resp.driver_id = req->driver_id;
+                resp.payload.kind = PIE_RESP_STATUS;
+                resp.payload.status.status = PIE_STATUS_EXCEPTION;
+            }
+            vtable.send_response(vtable.ctx, req_id, &resp);
+        }
+        return 0;
+    } catch (const std::exception& e) {
+        std::fprintf(stderr, "[pie-driver-hip] fatal: %s\n", e.what());
+        return -1;
+    } catch (...) {
+        std::fprintf(stderr, "[pie-driver-hip] fatal: unknown error\n");
+        return -1;
+    }
+}
+
+// Host-only planner hook: runs the planner on a forward request and copies the integer
+// plan out, so that the page-table arithmetic can be checked bit-exactly without a GPU.
+// out_i64 receives kv_slots[N]; out_i32 receives, back to back: positions[N],
+// row_page_begin[N], row_kv_len[N], seq_len[R], sample_rows[S], sample_indptr[R+1], then
+// {R, N, S, max_kv_len, pure_decode, all_greedy, has_user_masks}.  Returns the number of
+// int32 values written, or -1 with the planner's message in err.
+extern "C" long long pie_hip_driver_plan(const PieForwardRequestDesc* f, int page_size,
+                                         int total_pages, long long* out_i64, int* out_i32,
+                                         size_t out_i32_cap, char* err, size_t err_cap) {
+    try {
+        if (!f) throw std::runtime_error("null request");
+        const BatchPlan p = plan_forward(*f, page_size, total_pages);
+        const size_t S = p.sample_rows.size();
+        const size_t need = 3 * static_cast<size_t>(p.N) + p.R + S + (p.R + 1) + 7;
+        if (need > out_i32_cap) throw std::runtime_error("output buffer too small");
+        size_t o = 0;
+        for (int i = 0; i < p.N; ++i) out_i64[i] = p.kv_slots[i];
+        for (int i = 0; i < p.N; ++i) out_i32[o++] = p.positions[i];
+        for (int i = 0; i < p.N; ++i) out_i32[o++] = static_cast<int>(p.row_page_begin[i]);
+        for (int i = 0; i < p.N; ++i) out_i32[o++] = p.row_kv_len[i];
+        for (int r = 0; r < p.R; ++r) out_i32[o++] = p.seq_len[r];
+        for (size_t i = 0; i < S; ++i) out_i32[o++] = p.sample_rows[i];
+        for (int r = 0; r <= p.R; ++r) out_i32[o++] = p.sample_indptr[r];
+        const int tail[7] = {p.R, p.N, static_cast<int>(S), p.max_kv_len, p.pure_decode ? 1 : 0,
+                             p.all_greedy ? 1 : 0, p.has_user_masks ? 1 : 0};
+        for (int v : tail) out_i32[o++] = v;
+        return static_cast<long long>(o);
+    } catch (const std::exception& e) {
+        set_err(err, err_cap, e.what());
+        return -1;
+    }
+}

@@ -1,0 +1,95 @@
+// Forward-pass executor: owns the paged KV pool, the activation workspaces and the
+// per-shape HIP graphs, and turns a BatchPlan into kernel launches.
+//
+// Op sequence per layer (bf16 activations, fp32 inside each op, one rounding per op —
+// the rounding points of driver/cuda/src/model/llama_like.cpp:364-762; op order of
+// driver/portable/src/graph_qwen3.cpp:225-829):
+//   xn   = rmsnorm(x, attn_norm)
+//   qkv  = xn · Wqkv^T                                  (weight-streaming GEMV)
+//   q,K,V: optional qk-norm, RoPE, K/V written into their page slots
+//   a    = paged attention(q, pages)                    (split-K over pages)
+//   x    = x + a · Wo^T                                 (residual fused, one rounding)
+//   xn   = rmsnorm(x, ffn_norm)
+//   gu   = xn · Wgu^T ; h = silu(gate) * up ; x = x + h · Wdown^T
+// tail: gather sampled rows -> final norm -> lm_head -> argmax (first index wins).
+//
+// Split into a host `prepare` (plan upload, outside any capture) and a device-only `body`
+// that is captured into a HIP graph per (rows, sampled rows, context bucket) for pure decode,
+// the prepare/body split of driver/cuda/src/executor/executor.hpp:42-75.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <map>
+#include <tuple>
+#include <vector>
+
+#include "config.hpp"
+#include "model.hpp"
+#include "planner.hpp"
+
+namespace pie_hip_driver {
+
+struct ForwardTimings {
+    uint32_t h2d_us = 0, launch_us = 0, sync_us = 0;
+};
+
+class Executor {
+  public:
+    Executor(const DriverConfig& cfg, Model& model);
+    ~Executor();
+    Executor(const Executor&) = delete;
+    Executor& operator=(const Executor&) = delete;
+
+    // Runs one forward pass; greedy tokens for plan.sample_rows land in tokens_out.
+    void forward(const BatchPlan& plan, std::vector<uint32_t>& tokens_out, ForwardTimings* t);
+
+    // KV page copies inside the device pool (every layer, K and V).
+    void copy_pages_d2d(const uint32_t* srcs, const uint32_t* dsts, size_t n);
+
+    int total_pages() const { return total_pages_; }
+    int page_size() const { return page_size_; }
+    size_t page_bytes() const;
+    hipStream_t stream() const { return stream_; }
+    int graphs_cached() const { return static_cast<int>(graphs_.size()); }
+    // Logits [rows, vocab] bf16 of the last forward's (last chunk of) sampled rows; debug/test hook.
+    const uint16_t* last_logits() const { return logits_; }
+    int last_logit_rows() const { return last_logit_rows_; }
+
+  private:
+    void body(int N, int S, int max_kv_len);
+    void alloc_kv();
+
+    DriverConfig cfg_;
+    Model& model_;
+    hipStream_t stream_ = nullptr;
+    int total_pages_ = 0, page_size_ = 0, max_tokens_ = 0, max_page_refs_ = 0;
+
+    std::vector<uint16_t*> k_pool_, v_pool_;  // per layer [pages, ps, hk, d]
+    // activations
+    uint16_t *x_ = nullptr, *xn_ = nullptr, *qkv_ = nullptr, *q_ = nullptr, *attn_ = nullptr;
+    uint16_t *gu_ = nullptr, *act_ = nullptr, *xs_ = nullptr, *logits_ = nullptr;
+    float* rope_tab_ = nullptr;
+    uint32_t* out_tokens_ = nullptr;
+    void* attn_ws_ = nullptr;
+    size_t attn_ws_bytes_ = 0;
+    uint32_t* copy_ids_ = nullptr;  // staging for page-copy id lists
+    size_t copy_ids_cap_ = 0;
+
+    // staged inputs: one pinned host block mirrored by one device block
+    struct Inputs {
+        size_t off_tokens, off_positions, off_slots, off_row_begin, off_row_len, off_sample_rows,
+            off_pages, total;
+    };
+    static Inputs input_layout(int N, int S);
+    Inputs in_{};  // layout at capacity: sizes the staging buffers
+    unsigned char* in_host_ = nullptr;
+    unsigned char* in_dev_ = nullptr;
+    uint32_t* out_host_ = nullptr;  // pinned
+
+    std::map<std::tuple<int, int, int>, hipGraphExec_t> graphs_;
+    int last_logit_rows_ = 0;
+};
+
+}  // namespace pie_hip_driver

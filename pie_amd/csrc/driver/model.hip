@@ -1,0 +1,223 @@
+#include "model.hpp"
+
+#include <cmath>
+#include <stdexcept>
+
+#include "pie_hip_kernels.h"
+
+namespace pie_hip_driver {
+
+#define PIE_HIP_CHECK(expr)                                                              \
+    do {                                                                                 \
+        hipError_t e_ = (expr);                                                          \
+        if (e_ != hipSuccess)                                                            \
+            throw std::runtime_error(std::string(#expr) + ": " + hipGetErrorString(e_)); \
+    } while (0)
+
+namespace {
+
+__device__ __forceinline__ uint64_t splitmix64(uint64_t x) {
+    x += 0x9E3779B97F4A7C15ull;
+    x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+    x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
+    return x ^ (x >> 31);
+}
+
+// out[i] = bf16(mean + std * z_i): z_i is the centred sum of four 16-bit uniforms drawn from
+// a counter hash of (seed, i) — integer arithmetic plus one exact int->float conversion and
+// two IEEE operations, so the stream is a pure function of (seed, i).
+__global__ void fill_normal_bf16_kernel(uint16_t* __restrict__ out, size_t n, uint64_t seed,
+                                        float mean, float std) {
+    const size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x;
+    if (i >= n) return;
+    const uint64_t h = splitmix64(seed ^ (i * 0xD1342543DE82EF95ull));
+    const int sum = static_cast<int>(h & 0xFFFF) + static_cast<int>((h >> 16) & 0xFFFF) +
+                    static_cast<int>((h >> 32) & 0xFFFF) + static_cast<int>(h >> 48);
+    const float z = static_cast<float>(sum - 131070) * (1.0f / 37837.227f);
+    const float v = mean + std * z;
+    const __bf16 b = static_cast<__bf16>(v);
+    out[i] = __builtin_bit_cast(uint16_t, b);
+}
+
+void fill_normal(uint16_t* dst, size_t n, uint64_t seed, float mean, float std,
+                 hipStream_t stream) {
+    if (n == 0) return;
+    hipLaunchKernelGGL(fill_normal_bf16_kernel, dim3(static_cast<unsigned>((n + 255) / 256)),
+                       dim3(256), 0, stream, dst, n, seed, mean, std);
+    PIE_HIP_CHECK(hipGetLastError());
+}
+
+Quant parse_quant(const std::string& q) {
+    if (q == "int4b8") return Quant::Int4b8;
+    if (q == "int8") return Quant::Int8;
+    if (q == "fp8") return Quant::Fp8;
+    return Quant::Bf16;
+}
+
+__global__ void f32_to_bf16_kernel(const float* __restrict__ in, uint16_t* __restrict__ out,
+                                   int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const __bf16 b = static_cast<__bf16>(in[i]);
+    out[i] = __builtin_bit_cast(uint16_t, b);
+}
+
+}  // namespace
+
+std::vector<float> rope_inv_freq(const ModelConfig& cfg) {
+    const int d = cfg.head_dim, half = d / 2;
+    std::vector<float> out(half);
+    const double pi = 3.14159265358979323846;
+    for (int i = 0; i < half; ++i) {
+        const double base = std::pow(static_cast<double>(cfg.rope_theta), -2.0 * i / d);
+        double f = base;
+        if (cfg.rope_factor > 0.f && cfg.rope_original_max_pos > 0) {
+            const double low_wl = cfg.rope_original_max_pos / static_cast<double>(cfg.rope_low_freq_factor);
+            const double high_wl = cfg.rope_original_max_pos / static_cast<double>(cfg.rope_high_freq_factor);
+            const double wl = 2.0 * pi / base;
+            if (wl < high_wl) {
+                f = base;
+            } else if (wl > low_wl) {
+                f = base / cfg.rope_factor;
+            } else {
+                const double smooth = (cfg.rope_original_max_pos / wl - cfg.rope_low_freq_factor) /
+                                      (cfg.rope_high_freq_factor - cfg.rope_low_freq_factor);
+                f = (1.0 - smooth) * base / cfg.rope_factor + smooth * base;
+            }
+        }
+        out[i] = static_cast<float>(f);
+    }
+    return out;
+}
+
+Model::~Model() {
+    for (void* p : allocs_) (void)hipFree(p);
+}
+
+void* Model::alloc(size_t bytes, const std::string& name) {
+    void* p = nullptr;
+    PIE_HIP_CHECK(hipMalloc(&p, bytes ? bytes : 16));
+    allocs_.push_back(p);
+    if (!name.empty()) names_[name] = TensorRef{p, bytes};
+    return p;
+}
+
+void Model::make_linear(Linear& lin, int N, int K, const std::string& name, std::uint64_t seed,
+                        hipStream_t stream) {
+    lin.kind = quant_;
+    lin.N = N;
+    lin.K = K;
+    lin.group = cfg_.group_size;
+    lin.scale_bf16 = cfg_.scale_dtype == "bf16";
+    const size_t nk = static_cast<size_t>(N) * K;
+    if (quant_ == Quant::Int4b8 && (K % lin.group != 0 || lin.group % 32 != 0))
+        throw std::runtime_error("model: int4b8 needs K % group == 0 and group % 32 == 0 (" + name + ")");
+    lin.data = alloc(lin.data_bytes(), name + ".data");
+    if (lin.scale_bytes()) lin.scale = alloc(lin.scale_bytes(), name + ".scale");
+    decode_bytes_ += lin.data_bytes() + lin.scale_bytes();
+    if (quant_ == Quant::Bf16) {
+        fill_normal(static_cast<uint16_t*>(lin.data), nk, seed, 0.f, cfg_.init_std, stream);
+        return;
+    }
+    if (nk > tmp_elems_) throw std::runtime_error("model: scratch too small for " + name);
+    fill_normal(tmp_bf16_, nk, seed, 0.f, cfg_.init_std, stream);
+    int st = 0;
+    if (quant_ == Quant::Int4b8) {
+        st = pie_hip_quant_int4b8_group(tmp_bf16_, static_cast<uint32_t*>(lin.data),
+                                        static_cast<uint16_t*>(lin.scale), N, K, lin.group, stream);
+    } else {
+        // row-scale formats quantise into an f32 scale first; bf16 scales are its rounding
+        float* s32 = lin.scale_bf16 ? static_cast<float*>(alloc(static_cast<size_t>(N) * 4, ""))
+                                    : static_cast<float*>(lin.scale);
+        if (quant_ == Quant::Int8)
+            st = pie_hip_quant_int8_per_channel(tmp_bf16_, static_cast<int8_t*>(lin.data), s32, N, K, stream);
+        else
+            st = pie_hip_quant_fp8_per_channel(tmp_bf16_, static_cast<uint8_t*>(lin.data), s32, N, K, stream);
+        if (st == 0 && lin.scale_bf16) {
+            hipLaunchKernelGGL(f32_to_bf16_kernel, dim3((N + 255) / 256), dim3(256), 0, stream, s32,
+                               static_cast<uint16_t*>(lin.scale), N);
+            PIE_HIP_CHECK(hipGetLastError());
+        }
+    }
+    if (st != 0) throw std::runtime_error("model: quantiser failed for " + name);
+}
+
+void Model::init_synthetic(const ModelConfig& cfg, hipStream_t stream) {
+    cfg_ = cfg;
+    quant_ = parse_quant(cfg.quant);
+    const int H = cfg.hidden, d = cfg.head_dim, hq = cfg.q_heads, hk = cfg.kv_heads;
+    const int V = cfg.vocab, L = cfg.layers;
+    const bool moe = is_moe();
+    const int I = moe ? cfg.expert_intermediate : cfg.intermediate;
+    if (H % 32 != 0 || d % 8 != 0 || I % 32 != 0 || V % 8 != 0)
+        throw std::runtime_error("model: hidden/intermediate must be multiples of 32, head_dim and vocab of 8");
+
+    size_t biggest = static_cast<size_t>((hq + 2 * hk) * d) * H;
+    biggest = std::max(biggest, static_cast<size_t>(2 * I) * H);
+    biggest = std::max(biggest, static_cast<size_t>(H) * hq * d);
+    tmp_elems_ = biggest;
+    PIE_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&tmp_bf16_), biggest * 2));
+
+    std::uint64_t seed = cfg.seed;
+    auto next_seed = [&]() { return seed += 0xA0761D6478BD642Full; };
+
+    embed = static_cast<uint16_t*>(alloc(static_cast<size_t>(V) * H * 2, "embed"));
+    fill_normal(embed, static_cast<size_t>(V) * H, next_seed(), 0.f, cfg.init_std, stream);
+    if (cfg.tie_embeddings) {
+        lm_head = embed;
+        names_["lm_head"] = names_["embed"];
+    } else {
+        lm_head = static_cast<uint16_t*>(alloc(static_cast<size_t>(V) * H * 2, "lm_head"));
+        fill_normal(lm_head, static_cast<size_t>(V) * H, next_seed(), 0.f, cfg.init_std, stream);
+    }
+    decode_bytes_ += static_cast<size_t>(V) * H * 2;
+    final_norm = static_cast<uint16_t*>(alloc(static_cast<size_t>(H) * 2, "final_norm"));
+    fill_normal(final_norm, H, next_seed(), 1.f, 0.1f, stream);
+
+    const std::vector<float> f = rope_inv_freq(cfg);
+    inv_freq = static_cast<float*>(alloc(f.size() * 4, "inv_freq"));
+    PIE_HIP_CHECK(hipMemcpyAsync(inv_freq, f.data(), f.size() * 4, hipMemcpyHostToDevice, stream));
+    PIE_HIP_CHECK(hipStreamSynchronize(stream));
+
+    layers.resize(L);
+    for (int l = 0; l < L; ++l) {
+        LayerWeights& w = layers[l];
+        const std::string p = "layers." + std::to_string(l) + ".";
+        w.attn_norm = static_cast<uint16_t*>(alloc(static_cast<size_t>(H) * 2, p + "attn_norm"));
+        fill_normal(w.attn_norm, H, next_seed(), 1.f, 0.1f, stream);
+        w.ffn_norm = static_cast<uint16_t*>(alloc(static_cast<size_t>(H) * 2, p + "ffn_norm"));
+        fill_normal(w.ffn_norm, H, next_seed(), 1.f, 0.1f, stream);
+        if (has_qk_norm()) {
+            w.q_norm = static_cast<uint16_t*>(alloc(static_cast<size_t>(d) * 2, p + "q_norm"));
+            fill_normal(w.q_norm, d, next_seed(), 1.f, 0.1f, stream);
+            w.k_norm = static_cast<uint16_t*>(alloc(static_cast<size_t>(d) * 2, p + "k_norm"));
+            fill_normal(w.k_norm, d, next_seed(), 1.f, 0.1f, stream);
+        }
+        make_linear(w.wqkv, (hq + 2 * hk) * d, H, p + "wqkv", next_seed(), stream);
+        make_linear(w.wo, H, hq * d, p + "wo", next_seed(), stream);
+        if (!moe) {
+            make_linear(w.wgu, 2 * I, H, p + "wgu", next_seed(), stream);
+            make_linear(w.wdown, H, I, p + "wdown", next_seed(), stream);
+        } else {
+            const int E = cfg.num_experts;
+            w.router = static_cast<uint16_t*>(alloc(static_cast<size_t>(E) * H * 2, p + "router"));
+            fill_normal(w.router, static_cast<size_t>(E) * H, next_seed(), 0.f, cfg.init_std, stream);
+            const size_t before = decode_bytes_;
+            w.e_wgu.resize(E);
+            w.e_wdown.resize(E);
+            for (int e = 0; e < E; ++e) {
+                const std::string pe = p + "experts." + std::to_string(e) + ".";
+                make_linear(w.e_wgu[e], 2 * I, H, pe + "wgu", next_seed(), stream);
+                make_linear(w.e_wdown[e], H, I, pe + "wdown", next_seed(), stream);
+            }
+            // a batch-1 decode step touches top_k of the E experts
+            const size_t all = decode_bytes_ - before;
+            decode_bytes_ = before + all / E * cfg.top_k + static_cast<size_t>(E) * H * 2;
+        }
+    }
+    PIE_HIP_CHECK(hipStreamSynchronize(stream));
+    (void)hipFree(tmp_bf16_);
+    tmp_bf16_ = nullptr;
+}
+
+}  // namespace pie_hip_driver

@@ -1,0 +1,108 @@
+// Model weights resident in HBM, in the storage formats the kernels stream.
+//
+// Layout per decoder layer (llama-like; op sequence of
+// driver/portable/src/graph_qwen3.cpp:225-829 and driver/cuda/src/model/llama_like.cpp:364-762):
+//   attn_norm [H] bf16, wqkv [(hq+2hk)d, H] (q rows, then k rows, then v rows — per-row /
+//   per-group scales make the fusion exact), optional q_norm/k_norm [d], wo [H, hq*d],
+//   ffn_norm [H], then either wgu [2I, H] (gate rows then up rows) + wdown [H, I], or the
+//   MoE block: router [E, H] bf16, per-expert wgu [E][2Ie, H] and wdown [E][H, Ie].
+// embed [V, H] bf16, final_norm [H], lm_head [V, H] bf16 (aliases embed when tied); those
+// three stay unquantised like the reference (driver/cuda/src/config.hpp:20-30).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <map>
+#include <string>
+#include <vector>
+
+#include "config.hpp"
+
+namespace pie_hip_driver {
+
+enum class Quant { Int4b8, Int8, Fp8, Bf16 };
+
+struct Linear {
+    Quant kind = Quant::Bf16;
+    void* data = nullptr;   // packed weights, [N, K] in the format's element size
+    void* scale = nullptr;  // int4: bf16 [N, K/G]; int8/fp8: f32 or bf16 [N]; bf16: null
+    bool scale_bf16 = true;
+    int N = 0, K = 0, group = 0;
+    size_t data_bytes() const {
+        const size_t nk = static_cast<size_t>(N) * K;
+        switch (kind) {
+            case Quant::Int4b8: return nk / 2;
+            case Quant::Bf16: return nk * 2;
+            default: return nk;
+        }
+    }
+    size_t scale_bytes() const {
+        switch (kind) {
+            case Quant::Int4b8: return static_cast<size_t>(N) * (K / group) * 2;
+            case Quant::Bf16: return 0;
+            default: return static_cast<size_t>(N) * (scale_bf16 ? 2 : 4);
+        }
+    }
+};
+
+struct LayerWeights {
+    uint16_t* attn_norm = nullptr;
+    uint16_t* ffn_norm = nullptr;
+    uint16_t* q_norm = nullptr;
+    uint16_t* k_norm = nullptr;
+    Linear wqkv, wo, wgu, wdown;
+    // MoE
+    uint16_t* router = nullptr;     // [E, H] bf16
+    std::vector<Linear> e_wgu, e_wdown;
+};
+
+struct TensorRef {
+    void* ptr;
+    size_t bytes;
+};
+
+class Model {
+  public:
+    Model() = default;
+    ~Model();
+    Model(const Model&) = delete;
+    Model& operator=(const Model&) = delete;
+
+    // Allocates every tensor and fills it with seeded synthetic weights on the device:
+    // N(0, init_std) rounded to bf16, then quantised by the library's quantiser kernels.
+    void init_synthetic(const ModelConfig& cfg, hipStream_t stream);
+
+    const ModelConfig& cfg() const { return cfg_; }
+    bool is_moe() const { return cfg_.arch == "qwen3_moe"; }
+    bool has_qk_norm() const { return cfg_.arch != "llama3"; }
+    Quant quant() const { return quant_; }
+
+    uint16_t* embed = nullptr;
+    uint16_t* lm_head = nullptr;
+    uint16_t* final_norm = nullptr;
+    float* inv_freq = nullptr;  // [d/2] device
+    std::vector<LayerWeights> layers;
+
+    // bytes streamed from HBM by one decode step at batch 1 (every weight once)
+    size_t decode_weight_bytes() const { return decode_bytes_; }
+    const std::map<std::string, TensorRef>& tensors() const { return names_; }
+
+  private:
+    void* alloc(size_t bytes, const std::string& name);
+    void make_linear(Linear& lin, int N, int K, const std::string& name, std::uint64_t seed,
+                     hipStream_t stream);
+    ModelConfig cfg_;
+    Quant quant_ = Quant::Bf16;
+    std::vector<void*> allocs_;
+    std::map<std::string, TensorRef> names_;
+    uint16_t* tmp_bf16_ = nullptr;  // scratch for the largest bf16 tensor being quantised
+    size_t tmp_elems_ = 0;
+    size_t decode_bytes_ = 0;
+};
+
+// Host-side inv_freq table (theta^(-2i/d) with optional llama3 band scaling,
+// driver/portable/src/model.cpp:1414-1448: the stored factor divides the base frequency).
+std::vector<float> rope_inv_freq(const ModelConfig& cfg);
+
+}  // namespace pie_hip_driver

@@ -416,7 +416,6 @@ extern "C" int pie_hip_gemv_w4a16_tuned(const uint16_t* act_bf16, const uint32_t
 extern "C" int pie_hip_gemv_w4a16(const uint16_t* act_bf16, const uint32_t* packed,
                                   const uint16_t* scale_bf16, uint16_t* y_bf16, int M, int N,
                                   int K, int group_size, int beta, void* stream) {
-    if (M > 32) return PIE_HIP_ERR_UNSUPPORTED;
     return pie_hip_gemv_w4a16_tuned(act_bf16, packed, scale_bf16, y_bf16, M, N, K, group_size,
                                     beta, 0, 0, stream);
 }
@@ -424,7 +423,6 @@ extern "C" int pie_hip_gemv_w4a16(const uint16_t* act_bf16, const uint32_t* pack
 extern "C" int pie_hip_gemv_w8a16(const uint16_t* act_bf16, const int8_t* w_int8,
                                   const float* scale_inv_f32, const uint16_t* scale_inv_bf16,
                                   uint16_t* y_bf16, int M, int N, int K, int beta, void* stream) {
-    if (M > 32) return PIE_HIP_ERR_UNSUPPORTED;
     if (!scale_inv_f32 == !scale_inv_bf16) return PIE_HIP_ERR_INVALID;  // exactly one
     GemvArgs a{act_bf16, reinterpret_cast<const pie_hip::u32x4_t*>(w_int8), nullptr,
                scale_inv_f32 ? static_cast<const void*>(scale_inv_f32) : scale_inv_bf16, y_bf16,
@@ -437,7 +435,6 @@ extern "C" int pie_hip_gemv_w8a16(const uint16_t* act_bf16, const int8_t* w_int8
 extern "C" int pie_hip_gemv_fp8(const uint16_t* act_bf16, const uint8_t* w_e4m3,
                                 const float* scale_inv_f32, const uint16_t* scale_inv_bf16,
                                 uint16_t* y_bf16, int M, int N, int K, int beta, void* stream) {
-    if (M > 32) return PIE_HIP_ERR_UNSUPPORTED;
     if (!scale_inv_f32 == !scale_inv_bf16) return PIE_HIP_ERR_INVALID;
     GemvArgs a{act_bf16, reinterpret_cast<const pie_hip::u32x4_t*>(w_e4m3), nullptr,
                scale_inv_f32 ? static_cast<const void*>(scale_inv_f32) : scale_inv_bf16, y_bf16,
@@ -449,7 +446,6 @@ extern "C" int pie_hip_gemv_fp8(const uint16_t* act_bf16, const uint8_t* w_e4m3,
 
 extern "C" int pie_hip_gemv_bf16(const uint16_t* act_bf16, const uint16_t* w_bf16,
                                  uint16_t* y_bf16, int M, int N, int K, int beta, void* stream) {
-    if (M > 32) return PIE_HIP_ERR_UNSUPPORTED;
     GemvArgs a{act_bf16, reinterpret_cast<const pie_hip::u32x4_t*>(w_bf16), nullptr, nullptr,
                y_bf16, N, K, 0, beta};
     return pie_hip::dispatch<pie_hip::FmtBf16>(a, M, 0, 0, static_cast<hipStream_t>(stream));

@@ -1,0 +1,86 @@
+"""Helpers for driver-level tests: TOML configs for tiny models, and an oracle model built
+from the tensors the driver exports (so both sides hold bit-identical weights)."""
+import numpy as np
+
+
+def toml_config(arch="llama3", hidden=512, layers=2, q_heads=8, kv_heads=2, head_dim=64,
+                intermediate=1024, vocab=2048, quant="int4b8", group_size=128, scale_dtype="bf16",
+                page_size=16, total_pages=64, max_forward_tokens=256, max_forward_requests=16,
+                rope_theta=500000.0, rope_factor=0.0, tie=False, seed=1234, use_graphs=True,
+                rms_eps=1e-5):
+    return f"""
+[model]
+arch = "{arch}"
+hidden = {hidden}
+layers = {layers}
+q_heads = {q_heads}
+kv_heads = {kv_heads}
+head_dim = {head_dim}
+intermediate = {intermediate}
+vocab = {vocab}
+quant = "{quant}"
+group_size = {group_size}
+scale_dtype = "{scale_dtype}"
+rope_theta = {rope_theta}
+rope_factor = {rope_factor}
+rms_eps = {rms_eps}
+tie_embeddings = {"true" if tie else "false"}
+seed = {seed}
+
+[batching]
+kv_page_size = {page_size}
+total_pages = {total_pages}
+max_forward_tokens = {max_forward_tokens}
+max_forward_requests = {max_forward_requests}
+
+[runtime]
+use_graphs = {"true" if use_graphs else "false"}
+verbose = true
+"""
+
+
+DATA_DTYPE = {"int4b8": np.uint32, "int8": np.int8, "fp8": np.uint8, "bf16": np.uint16}
+
+
+def oracle_model_from_driver(drv, cfg: dict):
+    """cfg: the keyword arguments given to toml_config (defaults filled in)."""
+    from oracle.model import OracleModel
+
+    L, quant = cfg["layers"], cfg["quant"]
+    t = {}
+    for name in ("embed", "lm_head", "final_norm"):
+        t[name] = drv.export_tensor(name, np.uint16)
+    t["inv_freq"] = drv.export_tensor("inv_freq", np.float32)
+    scale_dt = np.uint16 if (quant == "int4b8" or cfg["scale_dtype"] == "bf16") else np.float32
+    for l in range(L):
+        p = f"layers.{l}."
+        for n in ("attn_norm", "ffn_norm", "q_norm", "k_norm"):
+            a = drv.export_tensor(p + n, np.uint16)
+            if a is not None:
+                t[p + n] = a
+        for w in ("wqkv", "wo", "wgu", "wdown"):
+            t[p + w + ".data"] = drv.export_tensor(p + w + ".data", DATA_DTYPE[quant])
+            sc = drv.export_tensor(p + w + ".scale", scale_dt)
+            if sc is not None:
+                t[p + w + ".scale"] = sc
+    ocfg = dict(hidden=cfg["hidden"], layers=L, q_heads=cfg["q_heads"], kv_heads=cfg["kv_heads"],
+                head_dim=cfg["head_dim"], intermediate=cfg["intermediate"], vocab=cfg["vocab"],
+                rms_eps=cfg["rms_eps"], rope_interleaved=1 if cfg["arch"] == "llama3" else 0,
+                qk_norm=cfg["arch"] != "llama3", quant=quant, group_size=cfg["group_size"],
+                page_size=cfg["page_size"], total_pages=cfg["total_pages"])
+    return OracleModel(ocfg, t), t
+
+
+def full_cfg(**kw):
+    import inspect
+
+    sig = inspect.signature(toml_config)
+    cfg = {k: v.default for k, v in sig.parameters.items()}
+    cfg.update(kw)
+    return cfg
+
+
+def cosine(a, b):
+    a = a.astype(np.float64)
+    b = b.astype(np.float64)
+    return float(a @ b / (np.linalg.norm(a) * np.linalg.norm(b) + 1e-30))
