@@ -1,0 +1,326 @@
+#!/usr/bin/env python3
+"""Decode benchmark of the MI355X Pie driver on its headline workload.
+
+Workload (BASELINE.json configs[3], the configuration the metric's target is quoted on and
+the largest single-GPU one): Llama-3-8B-shaped decoder, random-init N(0, 0.02) weights
+quantised to W4A16 (int4b8, group 128), bf16 embeddings / lm_head, page size 16; prefill a
+2048-token random prompt, then greedy decode at batch 1.  A "step" is one decode forward pass
+through the driver boundary (frame -> planner -> kernels -> argmax -> response), so
+`value` is whole-job decode tokens/s with weights and KV resident in HBM.
+
+Also reported on the same JSON line:
+  roofline     the dominant kernel (the weight-streaming W4A16 GEMV) over every decoder
+               linear of the model: algorithmic bytes / kernel duration, each launch bracketed
+               by HIP events on its own stream, against the 8 TB/s HBM peak;
+  cpu_baseline the CPU oracle (a port of the reference's forward pass) timed on this box's
+               host cores on a bounded sample of the same decode steps, and its tokens
+               compared with the GPU's;
+  extra        per-shape GEMV figures, the paged decode-attention kernel on BASELINE's
+               attention config (batch 64, contexts U[512, 8192], 25% forked prefix), and the
+               lm_head GEMV.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+import numpy as np
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBPS = 8000.0
+
+MODEL = dict(arch="llama3", hidden=4096, layers=32, q_heads=32, kv_heads=8, head_dim=128,
+             intermediate=14336, vocab=128256, rope_theta=500000.0, quant="int4b8", group_size=128)
+
+
+def toml(model: dict, page_size: int, total_pages: int, max_tokens: int, max_requests: int) -> str:
+    lines = ["[model]"]
+    for k, v in model.items():
+        lines.append(f'{k} = "{v}"' if isinstance(v, str) else f"{k} = {v}")
+    lines += ["[batching]", f"kv_page_size = {page_size}", f"total_pages = {total_pages}",
+              f"max_forward_tokens = {max_tokens}", f"max_forward_requests = {max_requests}",
+              "[runtime]", "use_graphs = true"]
+    return "\n".join(lines) + "\n"
+
+
+class Hip:
+    """The few HIP runtime calls the measurement needs (events bracketing single kernels)."""
+
+    def __init__(self):
+        self.lib = C.CDLL("libamdhip64.so")
+        self.lib.hipEventCreate.argtypes = [C.POINTER(C.c_void_p)]
+        self.lib.hipEventElapsedTime.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p]
+        self.lib.hipEventDestroy.argtypes = [C.c_void_p]
+        self.lib.hipDeviceSynchronize.argtypes = []
+
+    def event(self) -> C.c_void_p:
+        e = C.c_void_p()
+        if self.lib.hipEventCreate(C.byref(e)) != 0:
+            raise RuntimeError("hipEventCreate failed")
+        return e
+
+    def elapsed_ms(self, a, b) -> float:
+        ms = C.c_float()
+        if self.lib.hipEventElapsedTime(C.byref(ms), a, b) != 0:
+            raise RuntimeError("hipEventElapsedTime failed")
+        return float(ms.value)
+
+    def sync(self):
+        if self.lib.hipDeviceSynchronize() != 0:
+            raise RuntimeError("hipDeviceSynchronize failed")
+
+
+def gemv_roofline(drv, hip, model, reps: int):
+    """Every int4 decoder linear of the model, M = 1, each kernel bracketed by its own events.
+    Walking all layers streams 3.6 GB per pass, far beyond the last-level cache, so every launch
+    reads its weights from HBM as it does inside a decode step."""
+    import torch
+
+    from pie_amd._lib import kernels
+
+    k = kernels()
+    H, d, hq, hk, I, G = (model[x] for x in ("hidden", "head_dim", "q_heads", "kv_heads",
+                                             "intermediate", "group_size"))
+    shapes = {"wqkv": ((hq + 2 * hk) * d, H), "wo": (H, hq * d), "wgu": (2 * I, H), "wdown": (H, I)}
+    dev = torch.device("cuda:0")
+    acts = {K: torch.randn(1, K, device=dev).bfloat16() for K in {s[1] for s in shapes.values()}}
+    outs = {N: torch.zeros(1, N, device=dev, dtype=torch.bfloat16) for N in {s[0] for s in shapes.values()}}
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    per_shape = {n: [0.0, 0] for n in shapes}
+    events = []
+    for rep in range(reps + 1):  # first pass warms code objects and is dropped
+        for l in range(model["layers"]):
+            for name, (N, K) in shapes.items():
+                e0, e1 = hip.event(), hip.event()
+                k.pie_hip_gemv_time_next(e0, e1)
+                st = k.pie_hip_gemv_w4a16(C.c_void_p(acts[K].data_ptr()),
+                                          C.c_void_p(drv.tensor_ptr(f"layers.{l}.{name}.data")),
+                                          C.c_void_p(drv.tensor_ptr(f"layers.{l}.{name}.scale")),
+                                          C.c_void_p(outs[N].data_ptr()), 1, N, K, G, 0, stream)
+                if st != 0:
+                    raise RuntimeError(f"pie_hip_gemv_w4a16 status {st}")
+                if rep > 0:
+                    events.append((name, e0, e1))
+    hip.sync()
+    for name, e0, e1 in events:
+        per_shape[name][0] += hip.elapsed_ms(e0, e1) * 1e-3
+        per_shape[name][1] += 1
+    def alg_bytes(N, K):
+        return N * K // 2 + N * (K // G) * 2 + K * 2 + N * 2
+    tot_t = sum(v[0] for v in per_shape.values())
+    tot_b = sum(alg_bytes(*shapes[n]) * v[1] for n, v in per_shape.items())
+    launches = sum(v[1] for v in per_shape.values())
+    detail = {n: dict(N=shapes[n][0], K=shapes[n][1], us=round(v[0] / v[1] * 1e6, 2),
+                      gbps=round(alg_bytes(*shapes[n]) / (v[0] / v[1]) / 1e9, 1))
+              for n, v in per_shape.items()}
+    return dict(achieved=tot_b / tot_t / 1e9, avg_us=tot_t / launches * 1e6,
+                bytes_per_launch=tot_b / launches, launches=launches, detail=detail)
+
+
+def time_graph(fn, n_launch: int, reps: int = 5) -> float:
+    """Average seconds per launch of fn() replayed from a HIP graph on torch's stream."""
+    import torch
+
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        for _ in range(2):
+            fn()
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for _ in range(n_launch):
+            fn()
+    g.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        g.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e-3 / (reps * n_launch)
+
+
+def attention_extra():
+    """Paged decode attention on BASELINE's attention config, timed from a HIP graph."""
+    import torch
+
+    from pie_amd import ops
+
+    dev = torch.device("cuda:0")
+    hq, hk, d, ps, R = 32, 8, 128, 16, 64
+    rng = np.random.default_rng(3)
+    ctx = rng.integers(512, 8193, size=R)
+    ctx[:16] = np.maximum(ctx[:16], 1024)
+    npg = (ctx + ps - 1) // ps
+    shared = 1024 // ps
+    total = int(npg.sum() - 15 * shared) + 8
+    perm = rng.permutation(total).astype(np.int32)
+    idx, indptr, last = [], [0], []
+    nxt, prefix = shared, perm[:shared]
+    for r in range(R):
+        n = int(npg[r])
+        if r < 16:
+            pages = np.concatenate([prefix, perm[nxt:nxt + n - shared]])
+            nxt += n - shared
+        else:
+            pages = perm[nxt:nxt + n]
+            nxt += n
+        idx.append(pages)
+        indptr.append(indptr[-1] + n)
+        last.append(int(ctx[r]) - (n - 1) * ps)
+    kp = torch.randn(total, ps, hk, d, device=dev).bfloat16()
+    vp = torch.randn(total, ps, hk, d, device=dev).bfloat16()
+    q = torch.randn(R, hq, d, device=dev).bfloat16()
+    pi = torch.from_numpy(np.concatenate(idx)).to(dev)
+    pp = torch.tensor(indptr, dtype=torch.int32, device=dev)
+    ll = torch.tensor(last, dtype=torch.int32, device=dev)
+    maxlen = int(ctx.max())
+    need = ops.attn_decode_workspace_bytes(R, hq, hk, d, maxlen)
+    ws = torch.empty(max(need, 16), dtype=torch.uint8, device=dev)
+    o = torch.empty_like(q)
+    t = time_graph(lambda: ops.attention_paged_decode(q, kp, vp, pi, pp, ll, maxlen, o=o, workspace=ws), 10)
+    alg = int(ctx.sum()) * 2 * hk * d * 2 + R * hq * d * 2 * 2
+    dedup = alg - 15 * 1024 * 2 * hk * d * 2
+    return dict(workload="decode attention 32q/8kv d128 page16 batch64 ctx U[512,8192] 25% forked 1024 prefix",
+                us=round(t * 1e6, 1), algorithmic_bytes=alg, gbps=round(alg / t / 1e9, 1),
+                frac_of_hbm_peak=round(alg / t / 1e9 / HBM_PEAK_GBPS, 4),
+                dedup_bytes=dedup, note="split kernel + merge kernel per call")
+
+
+def lm_head_extra(drv, model):
+    import torch
+
+    from pie_amd._lib import kernels
+
+    k = kernels()
+    dev = torch.device("cuda:0")
+    V, H = model["vocab"], model["hidden"]
+    x = torch.randn(1, H, device=dev).bfloat16()
+    y = torch.empty(1, V, device=dev, dtype=torch.bfloat16)
+    w = drv.tensor_ptr("lm_head")
+    fn = lambda: k.pie_hip_gemv_bf16(C.c_void_p(x.data_ptr()), C.c_void_p(w), C.c_void_p(y.data_ptr()),
+                                     1, V, H, 0, C.c_void_p(torch.cuda.current_stream().cuda_stream))
+    t = time_graph(fn, 4)
+    b = V * H * 2 + H * 2 + V * 2
+    return dict(workload="bf16 lm_head GEMV [128256 x 4096]", us=round(t * 1e6, 1),
+                gbps=round(b / t / 1e9, 1), frac_of_hbm_peak=round(b / t / 1e9 / HBM_PEAK_GBPS, 4),
+                note="1 GB per call: larger than L2, smaller than the 256 MB last-level cache x4")
+
+
+def cpu_baseline(drv, model, page_size, total_pages, n_prompt, gpu_tokens, budget_s: float):
+    """The CPU oracle on the same decode steps: weights and the prefilled KV pools are copied
+    from the GPU, then the oracle decodes from the first post-prompt position."""
+    from oracle.model import model_from_driver
+
+    cfg = dict(model, page_size=page_size, total_pages=total_pages, scale_dtype="bf16", rms_eps=1e-5)
+    om, _ = model_from_driver(drv, cfg)
+    for l in range(model["layers"]):
+        om.k_pages[l][...] = drv.export_tensor(f"kv.k.{l}", np.uint16).reshape(om.k_pages[l].shape)
+        om.v_pages[l][...] = drv.export_tensor(f"kv.v.{l}", np.uint16).reshape(om.v_pages[l].shape)
+    steps, matched, t_total = 0, 0, 0.0
+    tok = int(gpu_tokens[0])
+    while steps < len(gpu_tokens) - 1 and (steps < 2 or t_total < budget_s):
+        pos = n_prompt + steps
+        npg = (pos + 1 + page_size - 1) // page_size
+        t0 = time.perf_counter()
+        out, _, _ = om.forward([tok], [pos], np.arange(npg), [0, npg],
+                               [pos + 1 - (npg - 1) * page_size], [0, 1])
+        t_total += time.perf_counter() - t0
+        steps += 1
+        matched += int(int(out[0]) == int(gpu_tokens[steps]))
+        tok = int(gpu_tokens[steps])  # teacher-forced: every step is compared on the same context
+    cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    return dict(value=steps / t_total, unit="tokens/s", cores=cores, kind="port",
+                sample=f"{steps} batch-1 decode steps of the same model at context {n_prompt}+, "
+                       "oracle (C restatement of the reference forward pass, OpenMP over rows) "
+                       "fed the GPU's weights and prefilled KV pages",
+                greedy_tokens_matched=matched, greedy_tokens_compared=steps)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--prompt", type=int, default=2048)
+    ap.add_argument("--batch", type=int, default=1)
+    ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-extra", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this driver path is built and measured on one GPU; "
+              f"--gpus {args.gpus} is not supported (run with --gpus 1).", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    from pie_amd import driver as drvmod
+
+    page_size = 16
+    max_new = args.warmup + args.steps + 1
+    pages_per_ctx = (args.prompt + max_new + page_size - 1) // page_size
+    total_pages = pages_per_ctx * args.batch + 8
+    cfg_text = toml(MODEL, page_size, total_pages, 512, max(16, args.batch))
+    hip = Hip()
+    rng = np.random.default_rng(2048)
+    prompt = rng.integers(0, MODEL["vocab"], args.prompt)
+
+    t0 = time.perf_counter()
+    drv = drvmod.Driver(cfg_text)
+    t_init = time.perf_counter() - t0
+
+    torch.cuda.synchronize()
+    tokens, tm = drv.generate(prompt, max_new, replicate=args.batch, warmup=args.warmup)
+    steps = tm["decode_steps"]
+    assert steps == args.steps, (steps, args.steps)
+    wall_s = tm["decode_wall_us"] * 1e-6
+    value = args.batch * steps / wall_s
+
+    roof = gemv_roofline(drv, hip, MODEL, reps=2)
+    extra = {"gemv_w4a16_shapes": roof["detail"], "init_s": round(t_init, 2),
+             "prefill_s": round(tm["prefill_us"] * 1e-6, 3),
+             "decode_device_ms_per_step": round(tm["decode_device_us"] * 1e-3 / steps, 4)}
+    if not args.no_extra:
+        extra["decode_attention"] = attention_extra()
+        extra["lm_head"] = lm_head_extra(drv, MODEL)
+    cpu = None
+    if not args.no_cpu:
+        cpu = cpu_baseline(drv, MODEL, page_size, total_pages, args.prompt, tokens[0], args.cpu_seconds)
+    drv.close()
+
+    out = {
+        "metric": "decode tokens/sec @1 GPU + quant-GEMV/attention HBM GB/s as % of 8 TB/s",
+        "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": steps,
+        "warmup": args.warmup, "ms_per_step": round(wall_s / steps * 1e3, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "Llama-3-8B-shaped W4A16 (int4b8 group 128) greedy decode, "
+                               f"batch {args.batch}, after a {args.prompt}-token prefill, page size 16",
+                   "batch": args.batch, "prompt_tokens": args.prompt, "page_size": page_size,
+                   "weights": "int4b8 group 128, bf16 scales; bf16 embed/lm_head; fp32 accumulation"},
+        "roofline": {"bound": "hbm", "kernel": "gemv_kernel<FmtInt4> (W4A16 weight-streaming GEMV, M=1)",
+                     "achieved": round(roof["achieved"], 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(roof["achieved"] / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "avg_launch_us": round(roof["avg_us"], 2),
+                     "algorithmic_bytes_per_launch": int(roof["bytes_per_launch"]),
+                     "launches_timed": roof["launches"]},
+        "cpu_baseline": cpu,
+        "extra": extra,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

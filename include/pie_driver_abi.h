@@ -245,16 +245,22 @@ int pie_hip_driver_handle(PieHipDriver* d, const PieFrameDesc* frame, PieRespons
 /*
  * Greedy generation harness: `replicate` independent contexts, each prefilled with the same
  * prompt on contiguous page ranges, then `max_new` single-token decode steps over all of
- * them in one forward per step.  out_tokens: [replicate, max_new].  timings_us (optional,
- * 4 entries): prefill wall, decode wall, decode device time (HIP events), steps timed.
+ * them in one forward per step.  out_tokens: [replicate, max_new].  The first `warmup`
+ * decode steps are excluded from the decode timings.  timings_us (optional, 4 entries):
+ * prefill wall, timed decode wall, timed decode device time (HIP events), steps timed.
  * Returns 0 or a negative error (message in err).
  */
 int pie_hip_driver_generate(PieHipDriver* d, const uint32_t* prompt, int n_prompt, int max_new,
-                            int replicate, uint32_t* out_tokens, double* timings_us, char* err,
-                            size_t err_cap);
-/* Copy a named model tensor to host memory (test/bench hook).  Returns the byte size, 0 if
- * the tensor does not exist; copies min(size, cap) bytes when dst is non-null. */
+                            int replicate, int warmup, uint32_t* out_tokens, double* timings_us,
+                            char* err, size_t err_cap);
+/* Copy a named tensor to host memory (test/bench hook): model weights by name, "kv.k.<l>" /
+ * "kv.v.<l>" (layer l's page pool) and "debug.logits" (last forward's sampled-row logits).
+ * Returns the byte size, 0 if the tensor does not exist; copies min(size, cap) bytes when dst
+ * is non-null. */
 size_t pie_hip_driver_export_tensor(PieHipDriver* d, const char* name, void* dst, size_t cap);
+/* Device address of a named model tensor (measurement hook: lets a harness launch single
+ * kernels of the kernel library on the resident weights).  NULL if unknown. */
+void* pie_hip_driver_tensor_ptr(PieHipDriver* d, const char* name);
 
 /*
  * Host-only planner hook (no GPU work): runs the forward-request planner and copies the

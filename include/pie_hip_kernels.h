@@ -77,6 +77,11 @@ int pie_hip_gemv_w4a16_tuned(const uint16_t* act_bf16, const uint32_t* packed,
                              int group_size, int beta, int rows_per_wave, int waves_per_simd,
                              void* stream);
 
+/* Measurement hook: the next GEMV kernel this thread launches (any format, M <= 4) is
+ * bracketed by the two HIP events (hipEvent_t), so hipEventElapsedTime(start, stop) is that
+ * kernel's own duration.  No reference counterpart. */
+int pie_hip_gemv_time_next(void* start_event, void* stop_event);
+
 /*
  * Weight-only int8 GEMV (W8A16), per-output-channel scale:
  *   y[m, n] = bf16( beta*y[m, n] + (sum_k f32(act[m,k]) * f32(q[n,k])) * scale_inv[n] )

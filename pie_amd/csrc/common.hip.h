@@ -40,6 +40,33 @@ __device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float acc) {
                                            __builtin_bit_cast(bf16x2_t, b), acc, false);
 }
 
+// (a & mask) | bits in one VALU op.  On gfx9-family encodings a three-source VALU op may
+// read one scalar operand and no literal, so the mask rides in an SGPR and `bits` in a VGPR;
+// written as asm because the compiler otherwise splits it into v_and + v_or.
+__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask_sgpr, uint32_t bits_vgpr) {
+    uint32_t d;
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "s"(mask_sgpr), "v"(bits_vgpr));
+    return d;
+}
+
+template <int CTRL, int ROW_MASK = 0xF, int BANK_MASK = 0xF>
+__device__ __forceinline__ float dpp_add_f32(float v) {
+    const int t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, BANK_MASK, true);
+    return v + __int_as_float(t);
+}
+
+// Wave64 sum on the DPP network (no LDS traffic): butterflies inside each row of 16 lanes,
+// then the two row-broadcast steps; lane 63 holds the total, which readlane makes uniform.
+__device__ __forceinline__ float wave_sum_dpp(float v) {
+    v = dpp_add_f32<0xB1>(v);             // quad_perm [1,0,3,2]
+    v = dpp_add_f32<0x4E>(v);             // quad_perm [2,3,0,1]
+    v = dpp_add_f32<0x141>(v);            // row_half_mirror
+    v = dpp_add_f32<0x140>(v);            // row_mirror: every lane holds its row's sum
+    v = dpp_add_f32<0x142, 0xA, 0xF>(v);  // row_bcast:15 into rows 1 and 3
+    v = dpp_add_f32<0x143, 0xC, 0xF>(v);  // row_bcast:31 into rows 2 and 3
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);

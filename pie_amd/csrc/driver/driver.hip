@@ -327,6 +327,18 @@ extern "C" size_t pie_hip_driver_export_tensor(PieHipDriver* d, const char* name
         }
         return bytes;
     }
+    const std::string nm(name);
+    if (nm.rfind("kv.k.", 0) == 0 || nm.rfind("kv.v.", 0) == 0) {
+        const int l = std::atoi(nm.c_str() + 5);
+        const uint16_t* pool = d->exec->kv_pool(nm[3] == 'k', l);
+        if (!pool) return 0;
+        const size_t bytes = d->exec->page_bytes() * static_cast<size_t>(d->exec->total_pages());
+        if (dst) {
+            const size_t n = bytes < cap ? bytes : cap;
+            if (hipMemcpy(dst, pool, n, hipMemcpyDeviceToHost) != hipSuccess) return 0;
+        }
+        return bytes;
+    }
     const auto& t = d->model.tensors();
     const auto it = t.find(name);
     if (it == t.end()) return 0;
@@ -337,10 +349,19 @@ extern "C" size_t pie_hip_driver_export_tensor(PieHipDriver* d, const char* name
     return it->second.bytes;
 }
 
+extern "C" void* pie_hip_driver_tensor_ptr(PieHipDriver* d, const char* name) {
+    if (!d || !name) return nullptr;
+    const auto& t = d->model.tensors();
+    const auto it = t.find(name);
+    return it == t.end() ? nullptr : it->second.ptr;
+}
+
 extern "C" int pie_hip_driver_generate(PieHipDriver* d, const uint32_t* prompt, int n_prompt,
-                                       int max_new, int replicate, uint32_t* out_tokens,
-                                       double* timings_us, char* err, size_t err_cap) {
-    if (!d || !prompt || n_prompt <= 0 || max_new <= 0 || replicate <= 0 || !out_tokens) {
+                                       int max_new, int replicate, int warmup,
+                                       uint32_t* out_tokens, double* timings_us, char* err,
+                                       size_t err_cap) {
+    if (!d || !prompt || n_prompt <= 0 || max_new <= 0 || replicate <= 0 || !out_tokens ||
+        warmup < 0) {
         set_err(err, err_cap, "bad arguments");
         return -1;
     }
@@ -398,9 +419,17 @@ extern "C" int pie_hip_driver_generate(PieHipDriver* d, const uint32_t* prompt, 
         hipEvent_t e0 = nullptr, e1 = nullptr;
         (void)hipEventCreate(&e0);
         (void)hipEventCreate(&e1);
-        const auto t_decode = clk::now();
+        auto t_decode = clk::now();
         (void)hipEventRecord(e0, d->exec->stream());
+        int timed_steps = 0;
         for (int s = 1; s < max_new; ++s) {
+            if (s == warmup + 1 && warmup > 0) {  // restart the clocks after the warm-up steps
+                (void)hipStreamSynchronize(d->exec->stream());
+                t_decode = clk::now();
+                (void)hipEventRecord(e0, d->exec->stream());
+                timed_steps = 0;
+            }
+            ++timed_steps;
             const int pos = n_prompt + s - 1;  // position of the token fed in this step
             const int np = (pos + 1 + ps - 1) / ps;
             FrameBuilder fb;
@@ -439,7 +468,7 @@ extern "C" int pie_hip_driver_generate(PieHipDriver* d, const uint32_t* prompt, 
             timings_us[0] = prefill_us;
             timings_us[1] = us_since(t_decode);
             timings_us[2] = static_cast<double>(dev_ms) * 1e3;
-            timings_us[3] = static_cast<double>(max_new - 1);
+            timings_us[3] = static_cast<double>(timed_steps);
         }
         return 0;
     } catch (const std::exception& e) {

@@ -56,6 +56,10 @@ class Executor {
     // Logits [rows, vocab] bf16 of the last forward's (last chunk of) sampled rows; debug/test hook.
     const uint16_t* last_logits() const { return logits_; }
     int last_logit_rows() const { return last_logit_rows_; }
+    const uint16_t* kv_pool(bool k, int layer) const {
+        if (layer < 0 || layer >= static_cast<int>(k_pool_.size())) return nullptr;
+        return k ? k_pool_[layer] : v_pool_[layer];
+    }
 
   private:
     void body(int N, int S, int max_kv_len);

@@ -34,6 +34,8 @@
 //   * bf16: weights feed v_dot2_f32_bf16 directly;
 //   * a wave64 butterfly finishes the row; the lane that stores an output has
 //     prefetched the residual / row scale it needs with the unit's loads.
+#include <hip/hip_ext.h>
+
 #include "common.hip.h"
 
 namespace pie_hip {
@@ -74,14 +76,16 @@ struct FmtInt4 {
         return s;
     }
     static __device__ __forceinline__ float dot(const u32x4_t w, const u32x4_t* xs, float p) {
-        constexpr uint32_t kMask = 0x000F000Fu, k128 = 0x43004300u;
+        const uint32_t kMask = 0x000F000Fu;
+        uint32_t k128 = 0x43004300u;  // (128.0bf16, 128.0bf16), kept in a VGPR for and_or
+        asm volatile("" : "+v"(k128));
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const uint32_t v = w[i];
-            p = dot2_bf16(xs[i].x, (v & kMask) | k128, p);
-            p = dot2_bf16(xs[i].y, ((v >> 4) & kMask) | k128, p);
-            p = dot2_bf16(xs[i].z, ((v >> 8) & kMask) | k128, p);
-            p = dot2_bf16(xs[i].w, ((v >> 12) & kMask) | k128, p);
+            p = dot2_bf16(xs[i].x, and_or(v, kMask, k128), p);
+            p = dot2_bf16(xs[i].y, and_or(v >> 4, kMask, k128), p);
+            p = dot2_bf16(xs[i].z, and_or(v >> 8, kMask, k128), p);
+            p = dot2_bf16(xs[i].w, and_or(v >> 12, kMask, k128), p);
         }
         return p;
     }
@@ -294,7 +298,7 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
             for (int r = 0; r < R; ++r) {
 #pragma unroll
                 for (int m = 0; m < M; ++m) {
-                    const float v = wave_sum(acc[r][m]);
+                    const float v = wave_sum_dpp(acc[r][m]);
                     acc[r][m] = 0.f;
                     if (lane == r * M + m) mine = v;
                 }
@@ -331,6 +335,11 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
     }
 }
 
+// Optional per-thread event pair that brackets exactly the next GEMV kernel (set by
+// pie_hip_gemv_time_next); consumed by one launch.
+thread_local hipEvent_t t_start_event = nullptr;
+thread_local hipEvent_t t_stop_event = nullptr;
+
 template <class F, int R, int M>
 int launch(const GemvArgs& a, int waves_per_simd, hipStream_t stream) {
     constexpr int kChunkK = kWave * F::WPP;
@@ -340,7 +349,14 @@ int launch(const GemvArgs& a, int waves_per_simd, hipStream_t stream) {
     int grid = kNumCU * waves_per_simd;
     const int max_grid = (a.N + kWavesPerBlock - 1) / kWavesPerBlock;  // >= 1 row per wave
     if (grid > max_grid) grid = max_grid;
-    hipLaunchKernelGGL((gemv_kernel<F, R, M>), dim3(grid), dim3(kBlock), smem, stream, a);
+    if (t_start_event && t_stop_event) {
+        hipExtLaunchKernelGGL((gemv_kernel<F, R, M>), dim3(grid), dim3(kBlock),
+                              static_cast<uint32_t>(smem), stream, t_start_event, t_stop_event, 0,
+                              a);
+        t_start_event = t_stop_event = nullptr;
+    } else {
+        hipLaunchKernelGGL((gemv_kernel<F, R, M>), dim3(grid), dim3(kBlock), smem, stream, a);
+    }
     return launch_status();
 }
 
@@ -400,6 +416,12 @@ int dispatch(GemvArgs a, int M, int rows_per_wave, int waves_per_simd, hipStream
 }  // namespace pie_hip
 
 using pie_hip::GemvArgs;
+
+extern "C" int pie_hip_gemv_time_next(void* start_event, void* stop_event) {
+    pie_hip::t_start_event = static_cast<hipEvent_t>(start_event);
+    pie_hip::t_stop_event = static_cast<hipEvent_t>(stop_event);
+    return PIE_HIP_OK;
+}
 
 extern "C" int pie_hip_gemv_w4a16_tuned(const uint16_t* act_bf16, const uint32_t* packed,
                                         const uint16_t* scale_bf16, uint16_t* y_bf16, int M,

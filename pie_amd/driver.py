@@ -146,9 +146,11 @@ def lib() -> C.CDLL:
         l.pie_hip_driver_capabilities.argtypes = [C.c_void_p]
         l.pie_hip_driver_handle.argtypes = [C.c_void_p, C.POINTER(FrameDesc), C.POINTER(ResponseFrameDesc)]
         l.pie_hip_driver_generate.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int,
-                                              C.c_void_p, C.c_void_p, C.c_char_p, C.c_size_t]
+                                              C.c_int, C.c_void_p, C.c_void_p, C.c_char_p, C.c_size_t]
         l.pie_hip_driver_export_tensor.restype = C.c_size_t
         l.pie_hip_driver_export_tensor.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t]
+        l.pie_hip_driver_tensor_ptr.restype = C.c_void_p
+        l.pie_hip_driver_tensor_ptr.argtypes = [C.c_void_p, C.c_char_p]
         l.pie_hip_driver_plan.restype = C.c_longlong
         l.pie_hip_driver_plan.argtypes = [C.POINTER(ForwardRequestDesc), C.c_int, C.c_int, C.c_void_p,
                                           C.c_void_p, C.c_size_t, C.c_char_p, C.c_size_t]
@@ -298,18 +300,25 @@ class Driver:
     def forward(self, frame: ForwardFrame) -> ForwardResult:
         return ForwardResult(self.handle(frame))
 
-    def generate(self, prompt: Sequence[int], max_new: int, replicate: int = 1):
-        """Greedy generation harness; returns (tokens[replicate, max_new], timings dict)."""
+    def generate(self, prompt: Sequence[int], max_new: int, replicate: int = 1, warmup: int = 0):
+        """Greedy generation harness; returns (tokens[replicate, max_new], timings dict).
+        The first `warmup` decode steps are left out of the decode timings."""
         p = np.ascontiguousarray(np.asarray(prompt, dtype=np.uint32))
         out = np.zeros((replicate, max_new), np.uint32)
         tm = np.zeros(4, np.float64)
         err = C.create_string_buffer(1024)
         rc = lib().pie_hip_driver_generate(self._h, p.ctypes.data, len(p), max_new, replicate,
-                                           out.ctypes.data, tm.ctypes.data, err, len(err))
+                                           warmup, out.ctypes.data, tm.ctypes.data, err, len(err))
         if rc != 0:
             raise RuntimeError(f"pie_hip_driver_generate: {err.value.decode()}")
         return out, dict(prefill_us=tm[0], decode_wall_us=tm[1], decode_device_us=tm[2],
                          decode_steps=int(tm[3]))
+
+    def tensor_ptr(self, name: str) -> int:
+        p = lib().pie_hip_driver_tensor_ptr(self._h, name.encode())
+        if not p:
+            raise KeyError(name)
+        return int(p)
 
     def export_tensor(self, name: str, dtype) -> Optional[np.ndarray]:
         n = lib().pie_hip_driver_export_tensor(self._h, name.encode(), None, 0)

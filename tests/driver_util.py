@@ -39,36 +39,11 @@ verbose = true
 """
 
 
-DATA_DTYPE = {"int4b8": np.uint32, "int8": np.int8, "fp8": np.uint8, "bf16": np.uint16}
-
-
 def oracle_model_from_driver(drv, cfg: dict):
     """cfg: the keyword arguments given to toml_config (defaults filled in)."""
-    from oracle.model import OracleModel
+    from oracle.model import model_from_driver
 
-    L, quant = cfg["layers"], cfg["quant"]
-    t = {}
-    for name in ("embed", "lm_head", "final_norm"):
-        t[name] = drv.export_tensor(name, np.uint16)
-    t["inv_freq"] = drv.export_tensor("inv_freq", np.float32)
-    scale_dt = np.uint16 if (quant == "int4b8" or cfg["scale_dtype"] == "bf16") else np.float32
-    for l in range(L):
-        p = f"layers.{l}."
-        for n in ("attn_norm", "ffn_norm", "q_norm", "k_norm"):
-            a = drv.export_tensor(p + n, np.uint16)
-            if a is not None:
-                t[p + n] = a
-        for w in ("wqkv", "wo", "wgu", "wdown"):
-            t[p + w + ".data"] = drv.export_tensor(p + w + ".data", DATA_DTYPE[quant])
-            sc = drv.export_tensor(p + w + ".scale", scale_dt)
-            if sc is not None:
-                t[p + w + ".scale"] = sc
-    ocfg = dict(hidden=cfg["hidden"], layers=L, q_heads=cfg["q_heads"], kv_heads=cfg["kv_heads"],
-                head_dim=cfg["head_dim"], intermediate=cfg["intermediate"], vocab=cfg["vocab"],
-                rms_eps=cfg["rms_eps"], rope_interleaved=1 if cfg["arch"] == "llama3" else 0,
-                qk_norm=cfg["arch"] != "llama3", quant=quant, group_size=cfg["group_size"],
-                page_size=cfg["page_size"], total_pages=cfg["total_pages"])
-    return OracleModel(ocfg, t), t
+    return model_from_driver(drv, cfg)
 
 
 def full_cfg(**kw):
