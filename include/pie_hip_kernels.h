@@ -77,6 +77,64 @@ int pie_hip_gemv_w4a16_tuned(const uint16_t* act_bf16, const uint32_t* packed,
                              int group_size, int beta, int rows_per_wave, int waves_per_simd,
                              void* stream);
 
+/*
+ * The decoder layer's fused projection: y = epilogue( rmsnorm?(act) · W^T ) in one kernel.
+ *   norm_weight_bf16 != NULL: act is replaced, while it is staged, by
+ *     bf16(act * rsqrt(mean(act^2) + eps) * norm_weight) — value and rounding of the separate
+ *     RMSNorm kernel (driver/cuda/src/kernels/rmsnorm.cu:14-54), so results do not change;
+ *   swiglu != 0: W's rows are interleaved (gate_0, up_0, gate_1, up_1, ...) and
+ *     y[m, i] = bf16( silu(bf16(g_i)) * bf16(u_i) ), y is [M, N/2] — the values of the unfused
+ *     projection followed by swiglu_bf16_kernel (driver/cuda/src/kernels/swiglu.cu:9-22);
+ *     not combinable with beta.
+ * format: PIE_HIP_FMT_*; scale: int4b8 bf16 [N, K/G]; int8/fp8 row scale [N] (f32, or bf16
+ * when scale_is_bf16); bf16: NULL.  Other arguments as the per-format GEMV entry points.
+ * Replaces the rmsnorm -> gemm_act_x_w (-> swiglu) sequences of
+ * driver/cuda/src/model/llama_like.cpp:370-705.
+ */
+#define PIE_HIP_FMT_INT4B8 0
+#define PIE_HIP_FMT_INT8 1
+#define PIE_HIP_FMT_FP8 2
+#define PIE_HIP_FMT_BF16 3
+int pie_hip_linear_fused(int format, const uint16_t* act_bf16, const uint16_t* norm_weight_bf16,
+                         float eps, const void* weight, const void* scale, int scale_is_bf16,
+                         int group_size, uint16_t* y_bf16, int M, int N, int K, int beta,
+                         int swiglu, void* stream);
+
+/*
+ * Weight-only GEMM for a handful to a few hundred activation rows on the matrix cores:
+ *   y[m, n] = epilogue( sum_k act[m,k] * w(n,k) ), same formats, scales, beta and swiglu
+ * contracts as pie_hip_linear_fused (no fused norm); the weights are streamed once per 64
+ * activation rows instead of once per 4.  bf16 products, fp32 accumulation; int4/int8 weights
+ * enter the MFMA offset-binary (128+nibble / 128+byte, exact in bf16) and the offset is removed
+ * per group / per row in fp32, so the result differs from the GEMV only by fp32 summation order.
+ * Requirements: K % 128 (int4b8; group_size a multiple of 128 dividing K), K % 64 (int8, fp8),
+ * K % 32 (bf16).
+ * Replaces Marlin W4A16 for small/medium M (driver/cuda/third_party/marlin/marlin_wrapper.hpp:39-51)
+ * and the cuBLASLt small-M path of gemm_act_x_w (driver/cuda/src/ops/gemm.cpp:1414-1583).
+ */
+int pie_hip_gemm_skinny(int format, const uint16_t* act_bf16, const void* weight,
+                        const void* scale, int scale_is_bf16, int group_size, uint16_t* y_bf16,
+                        int M, int N, int K, int beta, int swiglu, void* stream);
+
+/*
+ * MoE grouped weight-only GEMM: one skinny problem per expert in a single launch.
+ *   rows [expert_offsets[e], expert_offsets[e+1]) of y (routes sorted by expert) are
+ *   act[route_act_rows[r]] (or act[r] when route_act_rows is NULL) times expert e's [N,K]
+ *   weights at weights + e*weight_stride_bytes (scales at scales + e*scale_stride_bytes).
+ * Experts without routes cost nothing and their weights are never read; an expert's weights
+ * are read once however many routes hit it.  max_rows_per_expert bounds the per-expert row
+ * count (host-known upper bound, e.g. the number of tokens).  With swiglu the weight rows are
+ * interleaved (gate_0, up_0, ...) and y is [routes, N/2].
+ * Replaces the per-route MoE decode GEMVs (driver/cuda/src/kernels/dequant_wna16.cu:59-169)
+ * and the grouped GEMM of driver/cuda/src/ops/gemm.hpp:189-198.
+ */
+int pie_hip_moe_grouped_gemm(int format, const uint16_t* act_bf16, const int32_t* route_act_rows,
+                             const int32_t* expert_offsets, int num_experts,
+                             int max_rows_per_expert, const void* weights,
+                             size_t weight_stride_bytes, const void* scales,
+                             size_t scale_stride_bytes, int scale_is_bf16, int group_size,
+                             uint16_t* y_bf16, int N, int K, int swiglu, void* stream);
+
 /* Measurement hook: the next GEMV kernel this thread launches (any format, M <= 4) is
  * bracketed by the two HIP events (hipEvent_t), so hipEventElapsedTime(start, stop) is that
  * kernel's own duration.  No reference counterpart. */

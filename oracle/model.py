@@ -169,8 +169,18 @@ def model_from_driver(drv, cfg: dict):
             if a is not None:
                 t[p + n] = a
         for w in ("wqkv", "wo", "wgu", "wdown"):
-            t[p + w + ".data"] = drv.export_tensor(p + w + ".data", _DATA_DTYPE[quant])
+            data = drv.export_tensor(p + w + ".data", _DATA_DTYPE[quant])
             sc = drv.export_tensor(p + w + ".scale", scale_dt)
+            if w == "wgu":
+                # the driver stores gate/up rows interleaved (gate_0, up_0, ...); the oracle uses
+                # the canonical order (all gate rows, then all up rows)
+                n = 2 * cfg["intermediate"]
+                data = data.reshape(n, -1)
+                data = np.concatenate([data[0::2], data[1::2]]).reshape(-1)
+                if sc is not None:
+                    sc = sc.reshape(n, -1)
+                    sc = np.concatenate([sc[0::2], sc[1::2]]).reshape(-1)
+            t[p + w + ".data"] = data
             if sc is not None:
                 t[p + w + ".scale"] = sc
     ocfg = dict(hidden=cfg["hidden"], layers=L, q_heads=cfg["q_heads"], kv_heads=cfg["kv_heads"],

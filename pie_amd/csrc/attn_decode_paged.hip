@@ -276,32 +276,63 @@ __global__ __launch_bounds__(kAttnBlock) void attn_decode_split_kernel(
     }
 }
 
-// One block per (request, q head): combine the splits that exist for this request.
+// One block per (request, q head): combine the splits that exist for this request.  Two
+// parallel phases instead of a serial walk over splits: (1) the (max, sum) pairs of all splits
+// are loaded at once and reduced to per-split weights in LDS, (2) each thread sums its output
+// dimension over splits with independent, unrolled loads.
+constexpr int kMaxSplits = 1024;
+
 template <int D>
-__global__ void attn_decode_merge_kernel(const float* __restrict__ part_o,
-                                         const float* __restrict__ part_ml,
-                                         const uint32_t* __restrict__ page_indptr,
-                                         const uint32_t* __restrict__ last_lens,
-                                         const uint32_t* __restrict__ row_begin,
-                                         const int32_t* __restrict__ row_len,
-                                         uint16_t* __restrict__ o, float* __restrict__ lse, int hq,
-                                         int ps, int units_per_split, int nsplit) {
+__global__ __launch_bounds__(D) void attn_decode_merge_kernel(
+    const float* __restrict__ part_o, const float* __restrict__ part_ml,
+    const uint32_t* __restrict__ page_indptr, const uint32_t* __restrict__ last_lens,
+    const uint32_t* __restrict__ row_begin, const int32_t* __restrict__ row_len,
+    uint16_t* __restrict__ o, float* __restrict__ lse, int hq, int ps, int units_per_split,
+    int nsplit) {
+    __shared__ float s_w[kMaxSplits];
+    __shared__ float s_red[2 * (D / kWave)];
     const int rh = blockIdx.x;
     const int r = rh / hq;
     const int dd = threadIdx.x;
+    const int lane = dd & (kWave - 1), wv = dd / kWave;
     const int kv_len = row_extent(page_indptr, last_lens, row_begin, row_len, r, ps).kv_len;
     const int nunits = (kv_len + kUnitTokens - 1) / kUnitTokens;
     const int ns = min(nsplit, (nunits + units_per_split - 1) / units_per_split);
-    float mx = -INFINITY;
-    for (int s = 0; s < ns; ++s) mx = fmaxf(mx, part_ml[(static_cast<size_t>(rh) * nsplit + s) * 2]);
+    const float* ml = part_ml + static_cast<size_t>(rh) * nsplit * 2;
+
+    float mloc = -INFINITY;
+    for (int s = dd; s < ns; s += D) mloc = fmaxf(mloc, ml[2 * s]);
+    mloc = wave_max(mloc);
+    if (lane == 0) s_red[wv] = mloc;
+    __syncthreads();
+    float mx = s_red[0];
+#pragma unroll
+    for (int w = 1; w < D / kWave; ++w) mx = fmaxf(mx, s_red[w]);
     const float safe = (mx == -INFINITY) ? 0.f : mx;
-    float ov = 0.f, ls = 0.f;
-    for (int s = 0; s < ns; ++s) {
-        const size_t ps_i = static_cast<size_t>(rh) * nsplit + s;
-        const float a = exp2f(part_ml[ps_i * 2] - safe);
-        ov += part_o[ps_i * D + dd] * a;
-        ls += part_ml[ps_i * 2 + 1] * a;
+    float lloc = 0.f;
+    for (int s = dd; s < ns; s += D) {
+        const float a = exp2f(ml[2 * s] - safe);
+        s_w[s] = a;
+        lloc += ml[2 * s + 1] * a;
     }
+    lloc = wave_sum(lloc);
+    if (lane == 0) s_red[D / kWave + wv] = lloc;
+    __syncthreads();
+    float ls = 0.f;
+#pragma unroll
+    for (int w = 0; w < D / kWave; ++w) ls += s_red[D / kWave + w];
+
+    const float* po = part_o + static_cast<size_t>(rh) * nsplit * D + dd;
+    float acc0 = 0.f, acc1 = 0.f, acc2 = 0.f, acc3 = 0.f;
+    int s = 0;
+    for (; s + 4 <= ns; s += 4) {
+        acc0 = fmaf(po[static_cast<size_t>(s) * D], s_w[s], acc0);
+        acc1 = fmaf(po[static_cast<size_t>(s + 1) * D], s_w[s + 1], acc1);
+        acc2 = fmaf(po[static_cast<size_t>(s + 2) * D], s_w[s + 2], acc2);
+        acc3 = fmaf(po[static_cast<size_t>(s + 3) * D], s_w[s + 3], acc3);
+    }
+    for (; s < ns; ++s) acc0 = fmaf(po[static_cast<size_t>(s) * D], s_w[s], acc0);
+    const float ov = (acc0 + acc1) + (acc2 + acc3);
     o[static_cast<size_t>(rh) * D + dd] = f32_to_bf16_bits(ls > 0.f ? ov / ls : 0.f);
     if (lse && dd == 0) lse[rh] = ls > 0.f ? (logf(ls) + mx * 0.6931471805599453f) : -INFINITY;
 }
@@ -340,6 +371,7 @@ SplitPlan plan_splits(int R, int hk, int max_kv_len) {
     long long ups = (max_units + want_split - 1) / want_split;
     if (ups < 2 * kAttnWaves) ups = 2 * kAttnWaves;  // >= 2 units per wave amortises the merge
     if (ups > max_units) ups = max_units;
+    if ((max_units + ups - 1) / ups > kMaxSplits) ups = (max_units + kMaxSplits - 1) / kMaxSplits;
     const int nsplit = static_cast<int>((max_units + ups - 1) / ups);
     return {static_cast<int>(ups), nsplit};
 }

@@ -42,6 +42,23 @@ T* dmalloc(size_t elems) {
 
 size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
+int fmt_code(Quant q) {
+    switch (q) {
+        case Quant::Int4b8: return PIE_HIP_FMT_INT4B8;
+        case Quant::Int8: return PIE_HIP_FMT_INT8;
+        case Quant::Fp8: return PIE_HIP_FMT_FP8;
+        default: return PIE_HIP_FMT_BF16;
+    }
+}
+
+// y = epilogue(rmsnorm?(act) · W^T): the norm that precedes a projection rides in its
+// activation staging, SwiGLU in the gate/up projection's epilogue.
+void linear_fused(const Linear& w, const uint16_t* act, const uint16_t* norm_w, float eps,
+                  uint16_t* y, int M, int beta, int swiglu, hipStream_t s) {
+    PIE_KERNEL(pie_hip_linear_fused(fmt_code(w.kind), act, norm_w, eps, w.data, w.scale,
+                                    w.scale_bf16 ? 1 : 0, w.group, y, M, w.N, w.K, beta, swiglu, s));
+}
+
 // y[M, N] = act[M, K] · W[N, K]^T (+ y when beta), by the weight's storage format — the
 // dispatcher role of gemm_act_x_w (driver/cuda/src/ops/gemm.cpp:1414-1583).
 void linear(const Linear& w, const uint16_t* act, uint16_t* y, int M, int beta, hipStream_t s) {
@@ -183,7 +200,6 @@ void Executor::body(int N, int S, int max_kv_len) {
     const Inputs in_ = input_layout(N, S);
     const ModelConfig& m = model_.cfg();
     const int H = m.hidden, d = m.head_dim, hq = m.q_heads, hk = m.kv_heads;
-    const int I = m.intermediate;
     hipStream_t s = stream_;
     const auto* tokens = reinterpret_cast<const uint32_t*>(in_dev_ + in_.off_tokens);
     const auto* positions = reinterpret_cast<const int32_t*>(in_dev_ + in_.off_positions);
@@ -199,8 +215,7 @@ void Executor::body(int N, int S, int max_kv_len) {
     PIE_KERNEL(pie_hip_rope_table(positions, model_.inv_freq, rope_tab_, N, d, s));
     for (int l = 0; l < m.layers; ++l) {
         const LayerWeights& w = model_.layers[l];
-        PIE_KERNEL(pie_hip_rmsnorm(x_, w.attn_norm, xn_, N, H, m.rms_eps, s));
-        linear(w.wqkv, xn_, qkv_, N, 0, s);
+        linear_fused(w.wqkv, x_, w.attn_norm, m.rms_eps, qkv_, N, 0, 0, s);
         PIE_KERNEL(pie_hip_qkv_rope_kvwrite(qkv_, q_, k_pool_[l], v_pool_[l], w.q_norm, w.k_norm,
                                             rope_tab_, slots, N, hq, hk, d, m.rope_interleaved,
                                             m.rms_eps, s));
@@ -208,9 +223,7 @@ void Executor::body(int N, int S, int max_kv_len) {
                                            row_begin, row_len, N, hq, hk, d, page_size_, -1.f,
                                            max_kv_len, attn_ws_, attn_ws_bytes_, s));
         linear(w.wo, attn_, x_, N, 1, s);
-        PIE_KERNEL(pie_hip_rmsnorm(x_, w.ffn_norm, xn_, N, H, m.rms_eps, s));
-        linear(w.wgu, xn_, gu_, N, 0, s);
-        PIE_KERNEL(pie_hip_swiglu(gu_, act_, N, I, s));
+        linear_fused(w.wgu, x_, w.ffn_norm, m.rms_eps, act_, N, 0, 1, s);
         linear(w.wdown, act_, x_, N, 1, s);
     }
     // lm_head only on the sampled rows (driver/portable/src/graph_qwen3.cpp:867-896)
@@ -218,8 +231,8 @@ void Executor::body(int N, int S, int max_kv_len) {
     for (int s0 = 0; s0 < S; s0 += cap) {
         const int n = std::min(cap, S - s0);
         PIE_KERNEL(pie_hip_embed(sample_rows + s0, x_, xs_, n, H, N, s));  // row gather
-        PIE_KERNEL(pie_hip_rmsnorm(xs_, model_.final_norm, xn_, n, H, m.rms_eps, s));
-        PIE_KERNEL(pie_hip_gemv_bf16(xn_, model_.lm_head, logits_, n, m.vocab, H, 0, s));
+        PIE_KERNEL(pie_hip_linear_fused(PIE_HIP_FMT_BF16, xs_, model_.final_norm, m.rms_eps,
+                                        model_.lm_head, nullptr, 0, 0, logits_, n, m.vocab, H, 0, 0, s));
         PIE_KERNEL(pie_hip_argmax(logits_, out_tokens_ + s0, n, m.vocab, s));
     }
 }

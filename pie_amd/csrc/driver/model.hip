@@ -47,6 +47,21 @@ void fill_normal(uint16_t* dst, size_t n, uint64_t seed, float mean, float std,
     PIE_HIP_CHECK(hipGetLastError());
 }
 
+// dst row 2i = src row i (gate_i), dst row 2i+1 = src row half + i (up_i); rows of
+// row_bytes bytes (always even), moved two bytes at a time — a load-time kernel.
+__global__ void interleave_rows_kernel(const unsigned char* __restrict__ src,
+                                       unsigned char* __restrict__ dst, size_t half,
+                                       size_t row_bytes) {
+    const size_t total = 2 * half * row_bytes;
+    for (size_t b = (blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x) * 2; b < total;
+         b += static_cast<size_t>(gridDim.x) * blockDim.x * 2) {
+        const size_t drow = b / row_bytes, off = b - drow * row_bytes;
+        const size_t srow = (drow & 1) ? half + (drow >> 1) : (drow >> 1);
+        *reinterpret_cast<uint16_t*>(dst + b) =
+            *reinterpret_cast<const uint16_t*>(src + srow * row_bytes + off);
+    }
+}
+
 Quant parse_quant(const std::string& q) {
     if (q == "int4b8") return Quant::Int4b8;
     if (q == "int8") return Quant::Int8;
@@ -142,6 +157,29 @@ void Model::make_linear(Linear& lin, int N, int K, const std::string& name, std:
     if (st != 0) throw std::runtime_error("model: quantiser failed for " + name);
 }
 
+// Re-orders the rows of a fused gate/up projection from (all gate rows, all up rows) to
+// (gate_0, up_0, gate_1, up_1, ...), the row order the SwiGLU epilogue of the fused projection
+// kernel pairs up.  A pure row permutation of the canonical [N, K] layout: data and scales move
+// together, no value changes.
+void Model::interleave_gate_up(Linear& lin, hipStream_t stream) {
+    const size_t half = static_cast<size_t>(lin.N) / 2;
+    auto permute = [&](void* buf, size_t bytes) {
+        if (!buf || bytes == 0) return;
+        const size_t row_bytes = bytes / lin.N;
+        void* tmp = nullptr;
+        PIE_HIP_CHECK(hipMalloc(&tmp, bytes));
+        hipLaunchKernelGGL(interleave_rows_kernel, dim3(2048), dim3(256), 0, stream,
+                           static_cast<const unsigned char*>(buf), static_cast<unsigned char*>(tmp),
+                           half, row_bytes);
+        PIE_HIP_CHECK(hipGetLastError());
+        PIE_HIP_CHECK(hipMemcpyAsync(buf, tmp, bytes, hipMemcpyDeviceToDevice, stream));
+        PIE_HIP_CHECK(hipStreamSynchronize(stream));
+        (void)hipFree(tmp);
+    };
+    permute(lin.data, lin.data_bytes());
+    permute(lin.scale, lin.scale_bytes());
+}
+
 void Model::init_synthetic(const ModelConfig& cfg, hipStream_t stream) {
     cfg_ = cfg;
     quant_ = parse_quant(cfg.quant);
@@ -197,6 +235,7 @@ void Model::init_synthetic(const ModelConfig& cfg, hipStream_t stream) {
         make_linear(w.wo, H, hq * d, p + "wo", next_seed(), stream);
         if (!moe) {
             make_linear(w.wgu, 2 * I, H, p + "wgu", next_seed(), stream);
+            interleave_gate_up(w.wgu, stream);
             make_linear(w.wdown, H, I, p + "wdown", next_seed(), stream);
         } else {
             const int E = cfg.num_experts;

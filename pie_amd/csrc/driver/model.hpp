@@ -4,7 +4,8 @@
 // driver/portable/src/graph_qwen3.cpp:225-829 and driver/cuda/src/model/llama_like.cpp:364-762):
 //   attn_norm [H] bf16, wqkv [(hq+2hk)d, H] (q rows, then k rows, then v rows — per-row /
 //   per-group scales make the fusion exact), optional q_norm/k_norm [d], wo [H, hq*d],
-//   ffn_norm [H], then either wgu [2I, H] (gate rows then up rows) + wdown [H, I], or the
+//   ffn_norm [H], then either wgu [2I, H] (rows interleaved gate_0, up_0, gate_1, ... for the
+//   fused SwiGLU epilogue) + wdown [H, I], or the
 //   MoE block: router [E, H] bf16, per-expert wgu [E][2Ie, H] and wdown [E][H, Ie].
 // embed [V, H] bf16, final_norm [H], lm_head [V, H] bf16 (aliases embed when tied); those
 // three stay unquantised like the reference (driver/cuda/src/config.hpp:20-30).
@@ -92,6 +93,7 @@ class Model {
     void* alloc(size_t bytes, const std::string& name);
     void make_linear(Linear& lin, int N, int K, const std::string& name, std::uint64_t seed,
                      hipStream_t stream);
+    void interleave_gate_up(Linear& lin, hipStream_t stream);
     ModelConfig cfg_;
     Quant quant_ = Quant::Bf16;
     std::vector<void*> allocs_;

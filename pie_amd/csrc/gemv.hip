@@ -53,13 +53,42 @@ typedef float f32x2_t __attribute__((ext_vector_type(2)));
 // the bf16 activation row.  dot(): p += sum over the piece of x*w(raw).  sum_x():
 // the sum of the staged activations of a piece (only when kBias != 0).
 
+// Reads activations for staging; with `norm_w` set it applies the RMSNorm that precedes the
+// projection on the fly: bf16(x * inv_rms * w), the value and the single rounding of
+// rmsnorm_bf16_kernel (driver/cuda/src/kernels/rmsnorm.cu:47-52), so fusing the norm into the
+// GEMV leaves every bit of the result unchanged.
+struct ActLoader {
+    const uint16_t* row;
+    const uint16_t* norm_w;
+    float inv_rms;
+    __device__ __forceinline__ uint32_t norm2(uint32_t x, uint32_t w) const {
+        return pack_bf16x2(bf16_lo(x) * inv_rms * bf16_lo(w), bf16_hi(x) * inv_rms * bf16_hi(w));
+    }
+    __device__ __forceinline__ u32x4_t load8(int k) const {
+        u32x4_t v = *reinterpret_cast<const u32x4_t*>(row + k);
+        if (norm_w) {
+            const u32x4_t w = *reinterpret_cast<const u32x4_t*>(norm_w + k);
+            v = u32x4_t{norm2(v.x, w.x), norm2(v.y, w.y), norm2(v.z, w.z), norm2(v.w, w.w)};
+        }
+        return v;
+    }
+    __device__ __forceinline__ u32x2_t load4(int k) const {
+        u32x2_t v = *reinterpret_cast<const u32x2_t*>(row + k);
+        if (norm_w) {
+            const u32x2_t w = *reinterpret_cast<const u32x2_t*>(norm_w + k);
+            v = u32x2_t{norm2(v.x, w.x), norm2(v.y, w.y)};
+        }
+        return v;
+    }
+};
+
 struct FmtInt4 {
     static constexpr int WPP = 32, XV = 4;
     static constexpr bool kGroupScale = true, kRowScale = false;
     static constexpr float kBias = -136.f;
     // vector i holds word i's 8 activations as pairs (0,4)(1,5)(2,6)(3,7)
-    static __device__ __forceinline__ u32x4_t stage(const uint16_t* row, int k0, int i) {
-        const u32x4_t v = *reinterpret_cast<const u32x4_t*>(row + k0 + 8 * i);
+    static __device__ __forceinline__ u32x4_t stage(const ActLoader& ld, int k0, int i) {
+        const u32x4_t v = ld.load8(k0 + 8 * i);
         u32x4_t p;
         p.x = (v.x & 0xFFFFu) | (v.z << 16);
         p.y = (v.x >> 16) | (v.z & 0xFFFF0000u);
@@ -95,8 +124,8 @@ struct FmtBf16 {
     static constexpr int WPP = 8, XV = 1;
     static constexpr bool kGroupScale = false, kRowScale = false;
     static constexpr float kBias = 0.f;
-    static __device__ __forceinline__ u32x4_t stage(const uint16_t* row, int k0, int) {
-        return *reinterpret_cast<const u32x4_t*>(row + k0);
+    static __device__ __forceinline__ u32x4_t stage(const ActLoader& ld, int k0, int) {
+        return ld.load8(k0);
     }
     static __device__ __forceinline__ float sum_x(const u32x4_t*) { return 0.f; }
     static __device__ __forceinline__ float dot(const u32x4_t w, const u32x4_t* xs, float p) {
@@ -111,8 +140,8 @@ struct FmtBf16 {
 // 16 weights per piece, activations staged as f32 in natural order.
 struct FmtF32Act {
     static constexpr int WPP = 16, XV = 4;
-    static __device__ __forceinline__ u32x4_t stage(const uint16_t* row, int k0, int i) {
-        const u32x2_t v = *reinterpret_cast<const u32x2_t*>(row + k0 + 4 * i);
+    static __device__ __forceinline__ u32x4_t stage(const ActLoader& ld, int k0, int i) {
+        const u32x2_t v = ld.load4(k0 + 4 * i);
         return u32x4_t{v.x << 16, v.x & 0xFFFF0000u, v.y << 16, v.y & 0xFFFF0000u};
     }
     static __device__ __forceinline__ float sum_x(const u32x4_t* xs) {
@@ -175,6 +204,7 @@ struct Unit {
     uint16_t gs[R];  // group scale (int4)
     uint16_t prev;   // y element this lane may add to (lane = r*M + m), for beta = 1
     float rs;        // row scale for that lane's row (int8 / fp8)
+    float rs2;       // swiglu epilogue: row scale of the pair's second (up) row
 };
 
 struct GemvArgs {
@@ -184,6 +214,9 @@ struct GemvArgs {
     const void* rscale;      // f32 or bf16 [N]      (int8 / fp8)
     uint16_t* y;
     int N, K, G, beta;
+    const uint16_t* norm_w;  // bf16 [K] or null: RMSNorm applied to act while staging
+    float eps;
+    int swiglu;  // 1: rows are (gate_i, up_i) pairs; y[m, i] = silu(bf16 g) * bf16 u, y is [M, N/2]
 };
 
 template <class F, int R, int M>
@@ -206,8 +239,10 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
     // Balanced contiguous row slice of this wave.
     const long long total_waves = static_cast<long long>(gridDim.x) * kWavesPerBlock;
     const long long wg = static_cast<long long>(blockIdx.x) * kWavesPerBlock + wv;
-    const int row_begin = static_cast<int>(wg * N / total_waves);
-    const int row_end = static_cast<int>((wg + 1) * N / total_waves);
+    // (slices fall on even rows for the swiglu epilogue, which pairs rows 2i and 2i+1)
+    const int gran = a.swiglu ? 2 : 1;
+    const int row_begin = static_cast<int>(wg * (N / gran) / total_waves) * gran;
+    const int row_end = static_cast<int>((wg + 1) * (N / gran) / total_waves) * gran;
     const int ngroups = (row_end - row_begin + R - 1) / R;
     const int nunits = ngroups * nchunks;
 
@@ -228,15 +263,54 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
         }
         // Every unit prefetches what the lane that finishes an output needs, so the
         // epilogue never stalls the pipeline (only the last chunk's values are used).
-        const int lr = lane < R * M ? lane / M : 0;
-        const int lm = lane < R * M ? lane % M : 0;
-        const int lrow = min(row_begin + g * R + lr, row_end - 1);
-        u.prev = a.y[static_cast<size_t>(lm) * N + lrow];
-        if constexpr (F::kRowScale) u.rs = F::load(a.rscale, lrow);
+        // (branch-free on purpose: a branch around loads would merge the outstanding-load state
+        // of both arms and force the next wait to drain the whole pipeline)
+        const int per = a.swiglu ? (R / 2) * M : R * M;
+        const int li = lane < per ? lane / M : 0;
+        const int lm = lane < per ? lane % M : 0;
+        const int lrow = a.swiglu ? min(row_begin + g * R + 2 * li, row_end - 2)
+                                  : min(row_begin + g * R + li, row_end - 1);
+        u.prev = a.y[a.swiglu ? 0 : static_cast<size_t>(lm) * N + lrow];
+        if constexpr (F::kRowScale) {
+            u.rs = F::load(a.rscale, lrow);
+            u.rs2 = F::load(a.rscale, min(lrow + 1, N - 1));
+        }
     };
 
     Unit<R> ua, ub;
     if (nunits > 0) issue(ua, 0, 0);
+
+    // Optional fused RMSNorm: sum of squares of each activation row (fp32), block-reduced.
+    float inv_rms[M];
+#pragma unroll
+    for (int m = 0; m < M; ++m) inv_rms[m] = 1.f;
+    if (a.norm_w) {
+        float* red = lds_sx;  // free until the sum_x pass below
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+            float local = 0.f;
+            for (int v = tid; v < K / 8; v += kBlock) {
+                const u32x4_t t =
+                    *reinterpret_cast<const u32x4_t*>(a.act + static_cast<size_t>(m) * K + v * 8);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float lo = bf16_lo(t[i]), hi = bf16_hi(t[i]);
+                    local += lo * lo + hi * hi;
+                }
+            }
+            local = wave_sum_dpp(local);
+            if (lane == 0) red[m * kWavesPerBlock + wv] = local;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+            float t = 0.f;
+#pragma unroll
+            for (int w = 0; w < kWavesPerBlock; ++w) t += red[m * kWavesPerBlock + w];
+            inv_rms[m] = rsqrtf(t / static_cast<float>(K) + a.eps);
+        }
+        __syncthreads();
+    }
 
     // Stage activations in the format's decode order.
     for (int v = tid; v < M * vec_per_m; v += kBlock) {
@@ -247,7 +321,12 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
         const int l = rem % kWave;
         const int k0 = c * kChunkK + l * WPP;
         u32x4_t p = {0u, 0u, 0u, 0u};
-        if (k0 < K) p = F::stage(a.act + static_cast<size_t>(m) * K, k0, i);
+        if (k0 < K) {
+            float ir = inv_rms[0];
+#pragma unroll
+            for (int mm = 1; mm < M; ++mm) ir = (m == mm) ? inv_rms[mm] : ir;
+            p = F::stage(ActLoader{a.act + static_cast<size_t>(m) * K, a.norm_w, ir}, k0, i);
+        }
         lds_x[v] = p;
     }
     __syncthreads();
@@ -293,21 +372,58 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
             }
         }
         if (c == nchunks - 1) {
-            float mine = 0.f;
+            float tot[R][M];
 #pragma unroll
             for (int r = 0; r < R; ++r) {
 #pragma unroll
                 for (int m = 0; m < M; ++m) {
-                    const float v = wave_sum_dpp(acc[r][m]);
+                    tot[r][m] = wave_sum_dpp(acc[r][m]);
                     acc[r][m] = 0.f;
-                    if (lane == r * M + m) mine = v;
                 }
             }
-            const int row = row_begin + g * R + lane / M;
-            if (lane < R * M && row < row_end) {
-                if constexpr (F::kRowScale) mine *= u.rs;
-                const float prev = a.beta ? bf16_bits_to_f32(u.prev) : 0.f;
-                a.y[static_cast<size_t>(lane % M) * N + row] = f32_to_bf16_bits(mine + prev);
+            if (a.swiglu) {
+                if constexpr (R % 2 == 0) {
+                    // lane p*M + m finishes pair p: g and u are rounded to bf16 first, as the
+                    // unfused projection would store them (swiglu.cu:18-21 reads bf16 inputs)
+                    float gv = 0.f, uv = 0.f;
+#pragma unroll
+                    for (int pr = 0; pr < R / 2; ++pr) {
+#pragma unroll
+                        for (int m = 0; m < M; ++m) {
+                            if (lane == pr * M + m) {
+                                gv = tot[2 * pr][m];
+                                uv = tot[2 * pr + 1][m];
+                            }
+                        }
+                    }
+                    const int row = row_begin + g * R + 2 * (lane / M);
+                    if (lane < (R / 2) * M && row < row_end) {
+                        if constexpr (F::kRowScale) {
+                            gv *= u.rs;
+                            uv *= u.rs2;
+                        }
+                        const float gb = bf16_bits_to_f32(f32_to_bf16_bits(gv));
+                        const float ub = bf16_bits_to_f32(f32_to_bf16_bits(uv));
+                        const float silu = gb / (1.f + expf(-gb));
+                        a.y[static_cast<size_t>(lane % M) * (N / 2) + row / 2] =
+                            f32_to_bf16_bits(silu * ub);
+                    }
+                }
+            } else {
+                float mine = 0.f;
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+#pragma unroll
+                    for (int m = 0; m < M; ++m) {
+                        if (lane == r * M + m) mine = tot[r][m];
+                    }
+                }
+                const int row = row_begin + g * R + lane / M;
+                if (lane < R * M && row < row_end) {
+                    if constexpr (F::kRowScale) mine *= u.rs;
+                    const float prev = a.beta ? bf16_bits_to_f32(u.prev) : 0.f;
+                    a.y[static_cast<size_t>(lane % M) * N + row] = f32_to_bf16_bits(mine + prev);
+                }
             }
         }
     };
@@ -347,7 +463,8 @@ int launch(const GemvArgs& a, int waves_per_simd, hipStream_t stream) {
     const size_t smem = static_cast<size_t>(M) * nchunks * kWave * (F::XV * 16 + 4);
     if (smem > 64 * 1024) return PIE_HIP_ERR_UNSUPPORTED;
     int grid = kNumCU * waves_per_simd;
-    const int max_grid = (a.N + kWavesPerBlock - 1) / kWavesPerBlock;  // >= 1 row per wave
+    // >= 1 row (or row pair) per wave
+    const int max_grid = (a.N / (a.swiglu ? 2 : 1) + kWavesPerBlock - 1) / kWavesPerBlock;
     if (grid > max_grid) grid = max_grid;
     if (t_start_event && t_stop_event) {
         hipExtLaunchKernelGGL((gemv_kernel<F, R, M>), dim3(grid), dim3(kBlock),
@@ -376,6 +493,8 @@ template <class F>
 int dispatch(GemvArgs a, int M, int rows_per_wave, int waves_per_simd, hipStream_t stream) {
     if (!a.act || !a.w || !a.y || M <= 0 || a.N <= 0 || a.K <= 0) return PIE_HIP_ERR_INVALID;
     if (a.K % F::WPP != 0) return PIE_HIP_ERR_UNSUPPORTED;
+    if (a.norm_w && a.K % 8 != 0) return PIE_HIP_ERR_UNSUPPORTED;
+    if (a.swiglu && (a.N % 2 != 0 || a.beta)) return PIE_HIP_ERR_INVALID;
     // Measured on MI355X: two resident waves per SIMD, each walking its slice four rows
     // at a time (fewer when the slice is shorter), is within a few percent of the best
     // (rows, waves) pair for every decode shape of an 8B-class model.
@@ -386,6 +505,7 @@ int dispatch(GemvArgs a, int M, int rows_per_wave, int waves_per_simd, hipStream
             a.N / (static_cast<long long>(kNumCU) * kWavesPerBlock * waves_per_simd);
         rows_per_wave = per_wave >= 4 ? 4 : (per_wave >= 3 ? 3 : (per_wave >= 2 ? 2 : 1));
     }
+    if (a.swiglu && rows_per_wave % 2 != 0) rows_per_wave = rows_per_wave == 3 ? 4 : 2;
     // Up to four activation rows share one pass over the weights (fewer when their staged
     // copies would not fit in 64 KiB of LDS); larger M re-reads the weights per group.
     constexpr int kChunkK = kWave * F::WPP;
@@ -398,7 +518,7 @@ int dispatch(GemvArgs a, int M, int rows_per_wave, int waves_per_simd, hipStream
     for (int m0 = 0; m0 < M; m0 += mcap) {
         const int mm = (M - m0) < mcap ? (M - m0) : mcap;
         a.act = act + static_cast<size_t>(m0) * a.K;
-        a.y = y + static_cast<size_t>(m0) * a.N;
+        a.y = y + static_cast<size_t>(m0) * (a.swiglu ? a.N / 2 : a.N);
         int st;
         switch (rows_per_wave) {
             case 1: st = launch_m<F, 1>(mm, a, waves_per_simd, stream); break;
@@ -471,4 +591,38 @@ extern "C" int pie_hip_gemv_bf16(const uint16_t* act_bf16, const uint16_t* w_bf1
     GemvArgs a{act_bf16, reinterpret_cast<const pie_hip::u32x4_t*>(w_bf16), nullptr, nullptr,
                y_bf16, N, K, 0, beta};
     return pie_hip::dispatch<pie_hip::FmtBf16>(a, M, 0, 0, static_cast<hipStream_t>(stream));
+}
+
+// One entry point for the fused forms the decoder layer uses: optional RMSNorm of the
+// activations while they are staged, optional SwiGLU over (gate, up) row pairs in the epilogue.
+extern "C" int pie_hip_linear_fused(int format, const uint16_t* act_bf16,
+                                    const uint16_t* norm_weight_bf16, float eps,
+                                    const void* weight, const void* scale, int scale_is_bf16,
+                                    int group_size, uint16_t* y_bf16, int M, int N, int K,
+                                    int beta, int swiglu, void* stream) {
+    using namespace pie_hip;
+    GemvArgs a{act_bf16, static_cast<const u32x4_t*>(weight), nullptr, nullptr, y_bf16, N, K,
+               group_size, beta, norm_weight_bf16, eps, swiglu ? 1 : 0};
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (format) {
+        case PIE_HIP_FMT_INT4B8:
+            if (!scale || group_size <= 0) return PIE_HIP_ERR_INVALID;
+            if (group_size % 32 != 0 || K % group_size != 0) return PIE_HIP_ERR_UNSUPPORTED;
+            a.gscale = static_cast<const uint16_t*>(scale);
+            return dispatch<FmtInt4>(a, M, 0, 0, st);
+        case PIE_HIP_FMT_INT8:
+            if (!scale) return PIE_HIP_ERR_INVALID;
+            a.rscale = scale;
+            return scale_is_bf16 ? dispatch<FmtInt8<true>>(a, M, 0, 0, st)
+                                 : dispatch<FmtInt8<false>>(a, M, 0, 0, st);
+        case PIE_HIP_FMT_FP8:
+            if (!scale) return PIE_HIP_ERR_INVALID;
+            a.rscale = scale;
+            return scale_is_bf16 ? dispatch<FmtFp8<true>>(a, M, 0, 0, st)
+                                 : dispatch<FmtFp8<false>>(a, M, 0, 0, st);
+        case PIE_HIP_FMT_BF16:
+            return dispatch<FmtBf16>(a, M, 0, 0, st);
+        default:
+            return PIE_HIP_ERR_INVALID;
+    }
 }

@@ -329,3 +329,100 @@ def copy_kv_pages(pool: torch.Tensor, srcs: torch.Tensor, dsts: torch.Tensor) ->
     _check(kernels().pie_hip_copy_kv_pages(_ptr(pool), _ptr(srcs), _ptr(dsts), srcs.numel(),
                                            C.c_size_t(page_bytes), _stream()),
            "pie_hip_copy_kv_pages")
+
+
+FMT = {"int4b8": 0, "int8": 1, "fp8": 2, "bf16": 3}
+
+
+def linear_fused(act: torch.Tensor, w: WeightView, norm_weight: Optional[torch.Tensor] = None,
+                 eps: float = 1e-5, y: Optional[torch.Tensor] = None, beta: int = 0,
+                 swiglu: bool = False) -> torch.Tensor:
+    """y = epilogue(rmsnorm?(act) · W^T): optional RMSNorm fused into the activation staging,
+    optional SwiGLU over interleaved (gate_i, up_i) weight rows (then y is [M, N/2])."""
+    _dev(act, torch.bfloat16, "act")
+    M, K = act.shape
+    if K != w.K:
+        raise KernelError("act K != weight K")
+    if norm_weight is not None:
+        _dev(norm_weight, torch.bfloat16, "norm_weight")
+        if norm_weight.numel() != K:
+            raise KernelError("norm weight must have K entries")
+    n_out = w.N // 2 if swiglu else w.N
+    if y is None:
+        if beta:
+            raise KernelError("beta=1 needs an existing y")
+        y = torch.empty((M, n_out), dtype=torch.bfloat16, device=act.device)
+    _dev(y, torch.bfloat16, "y")
+    if tuple(y.shape) != (M, n_out):
+        raise KernelError("y shape mismatch")
+    scale_is_bf16 = int(w.scale is not None and w.scale.dtype == torch.bfloat16)
+    st = kernels().pie_hip_linear_fused(FMT[w.kind], _ptr(act), _ptr(norm_weight), C.c_float(eps),
+                                        _ptr(w.data), _ptr(w.scale), scale_is_bf16, w.group_size,
+                                        _ptr(y), M, w.N, K, beta, int(swiglu), _stream())
+    _check(st, "pie_hip_linear_fused")
+    return y
+
+
+def gemm_skinny(act: torch.Tensor, w: WeightView, y: Optional[torch.Tensor] = None, beta: int = 0,
+                swiglu: bool = False) -> torch.Tensor:
+    """Matrix-core weight-only GEMM for a handful to a few dozen activation rows (same contract as
+    `linear_fused` without the norm)."""
+    _dev(act, torch.bfloat16, "act")
+    M, K = act.shape
+    if K != w.K:
+        raise KernelError("act K != weight K")
+    n_out = w.N // 2 if swiglu else w.N
+    if y is None:
+        if beta:
+            raise KernelError("beta=1 needs an existing y")
+        y = torch.empty((M, n_out), dtype=torch.bfloat16, device=act.device)
+    _dev(y, torch.bfloat16, "y")
+    if tuple(y.shape) != (M, n_out):
+        raise KernelError("y shape mismatch")
+    scale_is_bf16 = int(w.scale is not None and w.scale.dtype == torch.bfloat16)
+    st = kernels().pie_hip_gemm_skinny(FMT[w.kind], _ptr(act), _ptr(w.data), _ptr(w.scale),
+                                       scale_is_bf16, w.group_size, _ptr(y), M, w.N, K, beta,
+                                       int(swiglu), _stream())
+    _check(st, "pie_hip_gemm_skinny")
+    return y
+
+
+def moe_grouped_gemm(act: torch.Tensor, route_act_rows: Optional[torch.Tensor],
+                     expert_offsets: torch.Tensor, kind: str, weights: torch.Tensor,
+                     scales: Optional[torch.Tensor], N: int, K: int, rows_hint: int,
+                     group_size: int = 0, swiglu: bool = False,
+                     y: Optional[torch.Tensor] = None, num_routes: Optional[int] = None) -> torch.Tensor:
+    """One skinny GEMM per expert in a single launch.  `weights` is [E, N, K] in the format's
+    element type (int4b8: [E, N, K/8] words), `scales` [E, N] (int4b8: [E, N, K/G]);
+    `expert_offsets` int32 [E+1] are the first route row of each expert (routes sorted by expert);
+    `route_act_rows` int32 [routes] names each route's activation row (None: route r reads
+    act[r])."""
+    _dev(act, torch.bfloat16, "act")
+    _dev(expert_offsets, torch.int32, "expert_offsets")
+    E = expert_offsets.numel() - 1
+    if weights.shape[0] != E:
+        raise KernelError("weights must have one [N, K] block per expert")
+    if route_act_rows is not None:
+        _dev(route_act_rows, torch.int32, "route_act_rows")
+        routes = route_act_rows.numel()
+    else:
+        routes = act.shape[0] if num_routes is None else num_routes
+    if act.shape[1] != K:
+        raise KernelError("act K mismatch")
+    if not weights.is_contiguous() or (scales is not None and not scales.is_contiguous()):
+        raise KernelError("weights/scales must be contiguous")
+    n_out = N // 2 if swiglu else N
+    if y is None:
+        y = torch.empty((routes, n_out), dtype=torch.bfloat16, device=act.device)
+    _dev(y, torch.bfloat16, "y")
+    if tuple(y.shape) != (routes, n_out):
+        raise KernelError("y shape mismatch")
+    wstride = weights[0].numel() * weights.element_size()
+    sstride = 0 if scales is None else scales[0].numel() * scales.element_size()
+    scale_is_bf16 = int(scales is not None and scales.dtype == torch.bfloat16)
+    st = kernels().pie_hip_moe_grouped_gemm(
+        FMT[kind], _ptr(act), _ptr(route_act_rows), _ptr(expert_offsets), E, int(rows_hint),
+        _ptr(weights), C.c_size_t(wstride), _ptr(scales), C.c_size_t(sstride), scale_is_bf16,
+        group_size, _ptr(y), N, K, int(swiglu), _stream())
+    _check(st, "pie_hip_moe_grouped_gemm")
+    return y

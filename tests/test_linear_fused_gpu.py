@@ -1,0 +1,128 @@
+"""GPU parity: the fused projection (RMSNorm in the staging, SwiGLU in the epilogue) against the
+composition of the separately pinned oracle ops — the fusion must not change values."""
+import numpy as np
+import pytest
+
+from gpu_util import bits, dev, ulp_diff
+
+pytestmark = pytest.mark.gpu
+
+
+def make_weight(oracle, rng, kind, N, K, G=128):
+    import torch
+    from pie_amd import ops
+
+    w = oracle.f32_to_bf16(rng.standard_normal((N, K)).astype(np.float32) * 0.02)
+    if kind == "int4b8":
+        packed = rng.integers(0, 2 ** 32, size=(N, K // 8), dtype=np.uint32)
+        scale = oracle.f32_to_bf16(rng.uniform(0.002, 0.008, size=(N, K // G)).astype(np.float32))
+        return dict(kind=kind, data=packed, scale=scale, G=G), \
+            lambda gpu: ops.WeightView("int4b8", dev(packed, gpu), dev(scale, gpu, torch.bfloat16), G, N, K)
+    if kind == "int8":
+        q, s = oracle.quant_int8_per_channel(w)
+        return dict(kind=kind, data=q, scale=s), \
+            lambda gpu: ops.WeightView("int8", dev(q, gpu), dev(s, gpu), 0, N, K)
+    if kind == "fp8":
+        q, s = oracle.quant_fp8_per_channel(w)
+        sb = oracle.f32_to_bf16(s)
+        return dict(kind=kind, data=q, scale=oracle.bf16_to_f32(sb)), \
+            lambda gpu: ops.WeightView("fp8", dev(q, gpu), dev(sb, gpu, torch.bfloat16), 0, N, K)
+    return dict(kind=kind, data=w), lambda gpu: ops.WeightView("bf16", dev(w, gpu, torch.bfloat16), None, 0, N, K)
+
+
+def close_to_oracle(oracle, got_bits, ref_bits, rel=2.0 ** -7, floor=2e-3):
+    """bf16 outputs of a long dot product: relative to the value, with a floor relative to the
+    largest output for elements that are sums of cancelling terms."""
+    g = oracle.bf16_to_f32(got_bits).astype(np.float64)
+    r = oracle.bf16_to_f32(ref_bits).astype(np.float64)
+    tol = rel * np.abs(r) + floor * np.abs(r).max()
+    return bool(np.all(np.abs(g - r) <= tol))
+
+
+def oracle_linear(oracle, wd, act, y_in=None):
+    if wd["kind"] == "int4b8":
+        return oracle.gemm_w4a16(act, wd["data"], wd["scale"], wd["G"], mode=0, y_in=y_in)[1]
+    if wd["kind"] == "int8":
+        return oracle.gemm_w8a16(act, wd["data"], wd["scale"], mode=0, y_in=y_in)[1]
+    if wd["kind"] == "fp8":
+        return oracle.gemm_fp8(act, wd["data"], wd["scale"], mode=0, y_in=y_in)[1]
+    return oracle.gemm_bf16(act, wd["data"], mode=0, y_in=y_in)[1]
+
+
+@pytest.mark.parametrize("kind", ["int4b8", "int8", "fp8", "bf16"])
+@pytest.mark.parametrize("M,N,K", [(1, 256, 2048), (3, 96, 4096), (6, 64, 1024)])
+def test_norm_fused_equals_norm_then_linear(gpu, oracle, kind, M, N, K):
+    import torch
+    from pie_amd import ops
+
+    rng = np.random.default_rng(110 + M + N)
+    wd, mk = make_weight(oracle, rng, kind, N, K)
+    x = oracle.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32) * 3)
+    nw = oracle.f32_to_bf16(rng.uniform(0.5, 1.5, K).astype(np.float32))
+    w = mk(gpu)
+    xg, nwg = dev(x, gpu, torch.bfloat16), dev(nw, gpu, torch.bfloat16)
+    fused = bits(ops.linear_fused(xg, w, norm_weight=nwg, eps=1e-5))
+    # same kernels, unfused: must be bit-identical (the staged activations are the same bf16 values
+    # up to the block-vs-kernel reduction order of the sum of squares)
+    xn = ops.rmsnorm_bf16(xg, nwg, 1e-5)
+    unfused = bits(ops.linear_fused(xn, w))
+    d = ulp_diff(fused, unfused)
+    assert d.max() <= 1 and (d == 0).mean() > 0.97
+    ref = oracle_linear(oracle, wd, oracle.rmsnorm(x, nw, 1e-5))
+    assert close_to_oracle(oracle, fused, ref)
+    assert (ulp_diff(fused, ref) <= 1).mean() > 0.98
+
+
+@pytest.mark.parametrize("kind", ["int4b8", "int8", "fp8", "bf16"])
+@pytest.mark.parametrize("M,I,K", [(1, 256, 2048), (2, 1024, 512), (4, 152, 1024), (5, 64, 4096)])
+def test_swiglu_epilogue_equals_linear_then_swiglu(gpu, oracle, kind, M, I, K):
+    import torch
+    from pie_amd import ops
+
+    rng = np.random.default_rng(120 + M + I)
+    wd, mk = make_weight(oracle, rng, kind, 2 * I, K)   # canonical rows: gate then up
+    x = oracle.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32))
+    # interleave rows (gate_0, up_0, gate_1, ...) for the fused kernel
+    perm = np.empty(2 * I, np.int64)
+    perm[0::2], perm[1::2] = np.arange(I), np.arange(I) + I
+    wi = dict(wd)
+    wi["data"] = wd["data"][perm]
+    if "scale" in wd:
+        wi["scale"] = wd["scale"][perm]
+    _, mk_i = None, None
+    w_can = mk(gpu)
+    w_int = ops.WeightView(w_can.kind, w_can.data[torch.from_numpy(perm).to(gpu)].contiguous(),
+                           None if w_can.scale is None else w_can.scale[torch.from_numpy(perm).to(gpu)].contiguous(),
+                           w_can.group_size, w_can.N, w_can.K)
+    xg = dev(x, gpu, torch.bfloat16)
+    fused = bits(ops.linear_fused(xg, w_int, swiglu=True))
+    assert fused.shape == (M, I)
+    unfused = bits(ops.swiglu_bf16(ops.linear_fused(xg, w_can)))
+    assert np.array_equal(fused, unfused)   # same sums, same rounding points: bit-identical
+    ref = oracle.swiglu(oracle_linear(oracle, wd, x))
+    assert close_to_oracle(oracle, fused, ref, rel=2.0 ** -6)
+    assert (ulp_diff(fused, ref) <= 1).mean() > 0.97
+
+
+def test_norm_and_swiglu_together_with_residual_variant(gpu, oracle):
+    import torch
+    from pie_amd import ops
+
+    rng = np.random.default_rng(130)
+    K, I, M = 2048, 512, 2
+    wd, mk = make_weight(oracle, rng, "int4b8", 2 * I, K)
+    perm = np.empty(2 * I, np.int64)
+    perm[0::2], perm[1::2] = np.arange(I), np.arange(I) + I
+    w_can = mk(gpu)
+    idx = torch.from_numpy(perm).to(gpu)
+    w_int = ops.WeightView("int4b8", w_can.data[idx].contiguous(), w_can.scale[idx].contiguous(), 128, 2 * I, K)
+    x = oracle.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32) * 2)
+    nw = oracle.f32_to_bf16(rng.uniform(0.5, 1.5, K).astype(np.float32))
+    xg, nwg = dev(x, gpu, torch.bfloat16), dev(nw, gpu, torch.bfloat16)
+    both = bits(ops.linear_fused(xg, w_int, norm_weight=nwg, swiglu=True))
+    steps = bits(ops.swiglu_bf16(ops.linear_fused(ops.rmsnorm_bf16(xg, nwg, 1e-5), w_can)))
+    d = ulp_diff(both, steps)
+    assert (d == 0).mean() > 0.9 and (d <= 2).mean() > 0.995
+    # beta with swiglu is rejected, beta without is fine
+    with pytest.raises(ops.KernelError):
+        ops.linear_fused(xg, w_int, y=torch.zeros(M, I, device=gpu, dtype=torch.bfloat16), beta=1, swiglu=True)
