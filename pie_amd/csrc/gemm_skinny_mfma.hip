@@ -1,0 +1,466 @@
+// Skinny / grouped weight-only GEMM on the matrix cores (v_mfma_f32_16x16x32_bf16) for
+// gfx950: y[m, n] = sum_k act[m, k] * w(n, k) for a handful to a few dozen activation rows,
+// and the MoE grouped form (one small-M problem per expert, rows gathered by route).
+//
+// Same contracts as the weight-streaming GEMV (formats, fused evaluation order, fp32
+// accumulation); it replaces re-streaming the weights once per four activation rows with one
+// pass over the weights per 16 rows.  Reference roles: Marlin W4A16 for small/medium M
+// (driver/cuda/third_party/marlin/marlin_wrapper.hpp:39-51), the per-route MoE decode GEMVs
+// (driver/cuda/src/kernels/dequant_wna16.cu:59-169, grid = routes x rows, which re-read an
+// expert's weights once per route) and the grouped GEMM (driver/cuda/src/ops/gemm.hpp:189-198).
+//
+// Design — still HBM-bound, the weights are the traffic:
+//   * weights never touch LDS.  Each lane loads 16 bytes of ONE weight row straight into the
+//     MFMA B-operand layout (column n = lane % 16, k-block = lane / 16) and decodes them in
+//     registers (int4 -> bf16 by OR-ing the exponent of 128.0 onto nibble pairs; int8/fp8 ->
+//     bf16 exactly through the conversion instructions); one 16-byte load feeds 4 / 2 / 1 MFMA
+//     steps.  Weight loads run a ring of PW blocks ahead of the MFMAs and nothing else uses the
+//     vector-memory counter inside the stream, so the waits stay partial;
+//   * activations are the A operand (row m = lane % 16): a tile of 16 rows x CK k-values sits in
+//     LDS (rows padded by one 16-byte vector so the 16 rows a read touches hit different banks),
+//     already in the element order the weight decode produces, staged once per K chunk and
+//     reused by all NG tiles of 16 weight rows the block owns;
+//   * with activations as A and weights as B, the accumulator lane holding outputs of column n
+//     is the lane that loaded row n's weights: int4 group scales and int8/fp8 row scales are
+//     per-lane scalars.  The offset-binary bias (-136 / -128 times the sum of the activations)
+//     needs sum_k x[m, k] in the accumulator layout — one more MFMA against a tile of ones,
+//     done once per K block and reused for every weight tile;
+//   * the KP waves of a block split K (wave w takes 16-byte blocks b = KP*g + w, so together they
+//     read KP*64 contiguous bytes of each weight row per step); partial sums meet in LDS once;
+//   * epilogue: row scale, residual add, or SwiGLU over adjacent (gate, up) columns exchanged
+//     with one DPP move.
+#include "common.hip.h"
+
+namespace pie_hip {
+namespace {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t pack_hi16(float lo, float hi) {
+    // bf16 pair by truncation (exact for values with <= 8 significant bits)
+    return __builtin_amdgcn_perm(__float_as_uint(hi), __float_as_uint(lo), 0x07060302u);
+}
+
+// ---- formats: K per 16-byte load (per lane), MFMA steps per load, decode of step s --------
+struct SkInt4 {
+    static constexpr int kPerLane = 32, kSteps = 4, kBytesPer2K = 1;
+    static constexpr float kBias = -136.f;
+    static constexpr bool kGroupScale = true;
+    static __device__ __forceinline__ u32x4_t decode(const u32x4_t w, int s) {
+        uint32_t k128 = 0x43004300u;
+        asm volatile("" : "+v"(k128));
+        const uint32_t v = w[s];
+        return u32x4_t{and_or(v, 0x000F000Fu, k128), and_or(v >> 4, 0x000F000Fu, k128),
+                       and_or(v >> 8, 0x000F000Fu, k128), and_or(v >> 12, 0x000F000Fu, k128)};
+    }
+    // activations of one 8-block in the order decode() yields weights: (0,4)(1,5)(2,6)(3,7)
+    static __device__ __forceinline__ u32x4_t order(const u32x4_t v) {
+        return u32x4_t{__builtin_amdgcn_perm(v.z, v.x, 0x05040100u),
+                       __builtin_amdgcn_perm(v.z, v.x, 0x07060302u),
+                       __builtin_amdgcn_perm(v.w, v.y, 0x05040100u),
+                       __builtin_amdgcn_perm(v.w, v.y, 0x07060302u)};
+    }
+};
+struct SkFp8 {
+    static constexpr int kPerLane = 16, kSteps = 2, kBytesPer2K = 2;
+    static constexpr float kBias = 0.f;
+    static constexpr bool kGroupScale = false;
+    static __device__ __forceinline__ u32x4_t decode(const u32x4_t w, int s) {
+        const uint32_t a = w[2 * s], b = w[2 * s + 1];
+        const f32x2_t a0 = __builtin_amdgcn_cvt_pk_f32_fp8(a, false);
+        const f32x2_t a1 = __builtin_amdgcn_cvt_pk_f32_fp8(a, true);
+        const f32x2_t b0 = __builtin_amdgcn_cvt_pk_f32_fp8(b, false);
+        const f32x2_t b1 = __builtin_amdgcn_cvt_pk_f32_fp8(b, true);
+        return u32x4_t{pack_hi16(a0.x, a0.y), pack_hi16(a1.x, a1.y), pack_hi16(b0.x, b0.y),
+                       pack_hi16(b1.x, b1.y)};
+    }
+    static __device__ __forceinline__ u32x4_t order(const u32x4_t v) { return v; }
+};
+struct SkInt8 {
+    static constexpr int kPerLane = 16, kSteps = 2, kBytesPer2K = 2;
+    static constexpr float kBias = -128.f;
+    static constexpr bool kGroupScale = false;
+    static __device__ __forceinline__ uint32_t two(uint32_t u, int lo_shift) {
+        return pack_hi16(static_cast<float>((u >> lo_shift) & 0xFFu),
+                         static_cast<float>((u >> (lo_shift + 8)) & 0xFFu));
+    }
+    static __device__ __forceinline__ u32x4_t decode(const u32x4_t w, int s) {
+        const uint32_t a = w[2 * s] ^ 0x80808080u, b = w[2 * s + 1] ^ 0x80808080u;
+        return u32x4_t{two(a, 0), two(a, 16), two(b, 0), two(b, 16)};
+    }
+    static __device__ __forceinline__ u32x4_t order(const u32x4_t v) { return v; }
+};
+struct SkBf16 {
+    static constexpr int kPerLane = 8, kSteps = 1, kBytesPer2K = 4;
+    static constexpr float kBias = 0.f;
+    static constexpr bool kGroupScale = false;
+    static __device__ __forceinline__ u32x4_t decode(const u32x4_t w, int) { return w; }
+    static __device__ __forceinline__ u32x4_t order(const u32x4_t v) { return v; }
+};
+
+struct SkinnyArgs {
+    const uint16_t* act;        // bf16 [*, K]
+    const int32_t* act_rows;    // gather: activation row of each problem row, or null
+    const unsigned char* w;     // weights of problem 0, row-major [N, K] in the format
+    const unsigned char* scale; // int4: bf16 [N, K/G]; int8/fp8: row scale [N]; bf16: null
+    uint16_t* y;                // [rows, N] (or [rows, N/2] with swiglu)
+    const int32_t* offsets;     // grouped: [P+1] first row of each problem; null: one problem
+    int M;                      // rows when offsets == null
+    int N, K, G, g_shift, beta, swiglu, scale_is_bf16;
+    size_t w_stride, scale_stride;  // bytes between problems
+};
+
+constexpr int gcd_c(int a, int b) { return b == 0 ? a : gcd_c(b, a % b); }
+
+template <int WL>
+struct WSlot {
+    u32x4_t w[WL];
+    uint16_t gs[WL];
+};
+
+// KP waves split K; CK k-values of activations per LDS chunk; NG tiles of 16 weight rows per
+// block; PW ring slots of WL adjacent 16-byte weight blocks in flight per lane (WL = 2: a
+// wave's two loads of a step cover whole 128-byte lines of each of its 16 rows).
+template <class F, int KP, int CK, int NG, int PW, int WL>
+__global__ __launch_bounds__(KP* kWave) void skinny_kernel(const SkinnyArgs a) {
+    constexpr int KPL = F::kPerLane, S = F::kSteps;
+    constexpr int LK = 4 * KPL;               // k covered by one wave-wide 16-byte load
+    constexpr int GC = CK / (KP * LK * WL);   // steps per wave per full chunk
+    constexpr int STRIDE = CK / 8 + 1;        // 16-byte vectors per staged activation row
+    constexpr int NT = KP * kWave;
+    constexpr bool kBiased = F::kBias != 0.f;
+    constexpr bool kRowBias = kBiased && !F::kGroupScale;
+    static_assert(GC >= 1 && (GC < PW || GC % PW == 0), "ring must tile a chunk");
+    static_assert(!F::kGroupScale || GC <= PW, "per-block activation sums are kept per step of a tile");
+    extern __shared__ __align__(16) unsigned char smem[];
+    u32x4_t* lds_a = reinterpret_cast<u32x4_t*>(smem);
+    float* red = reinterpret_cast<float*>(smem);
+    const int tid = threadIdx.x, lane = tid & (kWave - 1);
+    const int wv = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const int j = lane & 15, q = lane >> 4;
+    const int N = a.N, K = a.K;
+    const int p = blockIdx.y;
+    const int r0 = a.offsets ? a.offsets[p] : 0;
+    const int r1 = a.offsets ? a.offsets[p + 1] : a.M;
+    if (r1 <= r0) return;
+
+    const int T = (N + 15) / 16;
+    const int tile0 = blockIdx.x * NG;
+    const size_t row_bytes = static_cast<size_t>(K) * F::kBytesPer2K / 2;
+    const unsigned char* wbase = a.w + static_cast<size_t>(p) * a.w_stride;
+    const unsigned char* sbase = a.scale ? a.scale + static_cast<size_t>(p) * a.scale_stride : nullptr;
+    const uint16_t* gsbase = reinterpret_cast<const uint16_t*>(sbase);
+    const int groups = F::kGroupScale ? K >> a.g_shift : 0;
+    const int blk_shift = a.g_shift - (F::kGroupScale ? 7 : 0);   // 16-byte blocks per scale group, log2
+    const unsigned char* wptr[NG];
+    int nrow[NG];
+    float row_scale[NG];
+#pragma unroll
+    for (int i = 0; i < NG; ++i) {
+        const int n = min(min(tile0 + i, T - 1) * 16 + j, N - 1);
+        nrow[i] = n;
+        wptr[i] = wbase + static_cast<size_t>(n) * row_bytes + static_cast<size_t>(q) * KPL * F::kBytesPer2K / 2;
+        row_scale[i] = 1.f;
+        if (!F::kGroupScale && sbase)
+            row_scale[i] = a.scale_is_bf16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(sbase)[n])
+                                           : reinterpret_cast<const float*>(sbase)[n];
+    }
+    const int nb = K / LK;                      // 16-byte blocks along K per lane quad
+    const int nchunks = (K + CK - 1) / CK;
+    const bf16x8_t ones = __builtin_bit_cast(bf16x8_t, u32x4_t{0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u});
+    const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
+
+    auto load_w = [&](int c, const unsigned char* wp, int n, int g) {
+        WSlot<WL> sl;
+        const int b0 = c * (CK / LK) + (KP * g + wv) * WL;
+#pragma unroll
+        for (int h = 0; h < WL; ++h) {
+            const int b = min(b0 + h, nb - 1);
+            sl.w[h] = *reinterpret_cast<const u32x4_t*>(wp + static_cast<size_t>(b) * LK * F::kBytesPer2K / 2);
+            sl.gs[h] = F::kGroupScale ? gsbase[static_cast<size_t>(n) * groups + (b >> blk_shift)] : uint16_t(0);
+        }
+        return sl;
+    };
+
+    // staging: TPR threads per activation row, SV 16-byte vectors per thread per chunk, held in
+    // registers from one chunk's compute to the next chunk's LDS write
+    constexpr int TPR = NT / 16, SV = (CK / 8) / TPR;
+    const int sm = tid / TPR, sv = tid % TPR;
+
+    for (int mt0 = r0; mt0 < r1; mt0 += 16) {
+        // rows past the problem repeat its last row and are never stored
+        const int srow = min(mt0 + sm, r1 - 1);
+        const uint16_t* arow = a.act + static_cast<size_t>(a.act_rows ? a.act_rows[srow] : srow) * K;
+        u32x4_t stg[SV];
+        auto stage_load = [&](int c) {
+            const int cc = min(c, nchunks - 1);
+            const int nvec = min(CK, K - cc * CK) / 8;
+#pragma unroll
+            for (int u = 0; u < SV; ++u)
+                stg[u] = *reinterpret_cast<const u32x4_t*>(arow + cc * CK + min(u * TPR + sv, nvec - 1) * 8);
+        };
+        auto stage_store = [&](int c) {
+            const int nvec = min(CK, K - min(c, nchunks - 1) * CK) / 8;
+#pragma unroll
+            for (int u = 0; u < SV; ++u)
+                if (u * TPR + sv < nvec) lds_a[sm * STRIDE + u * TPR + sv] = F::order(stg[u]);
+        };
+
+        constexpr int NSX = F::kGroupScale ? GC * WL : 1;
+        f32x4_t acc[NG], sxs[NSX], sxt = zero4;
+#pragma unroll
+        for (int i = 0; i < NG; ++i) acc[i] = zero4;
+#pragma unroll
+        for (int i = 0; i < NSX; ++i) sxs[i] = zero4;
+
+        // the ring holds the next PW steps of the sequence (chunk, tile, g), g fastest
+        WSlot<WL> ring[PW];
+#pragma unroll
+        for (int l = 0; l < PW; ++l) {
+            const int t = l / GC;
+            ring[l] = load_w(t / NG, wptr[t % NG], nrow[t % NG], l % GC);
+        }
+        stage_load(0);
+        __syncthreads();  // the previous pass's reduction is consumed
+        stage_store(0);
+
+        auto step = [&](const WSlot<WL>& cur, int ng, int g) {
+#pragma unroll
+            for (int h = 0; h < WL; ++h) {
+                const int vbase = ((KP * g + wv) * WL + h) * (LK / 8) + q * S;
+                const int sxi = F::kGroupScale ? g * WL + h : 0;
+                bf16x8_t ax[S];
+#pragma unroll
+                for (int s = 0; s < S; ++s) ax[s] = __builtin_bit_cast(bf16x8_t, lds_a[j * STRIDE + vbase + s]);
+                f32x4_t part = zero4;
+#pragma unroll
+                for (int s = 0; s < S; ++s) {
+                    const bf16x8_t bw = __builtin_bit_cast(bf16x8_t, F::decode(cur.w[h], s));
+                    if (kBiased && ng == 0) {
+                        if (F::kGroupScale)
+                            sxs[sxi] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax[s], ones, s == 0 ? zero4 : sxs[sxi], 0, 0, 0);
+                        else
+                            sxt = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax[s], ones, sxt, 0, 0, 0);
+                    }
+                    if (F::kGroupScale)
+                        part = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax[s], bw, part, 0, 0, 0);
+                    else
+                        acc[ng] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax[s], bw, acc[ng], 0, 0, 0);
+                }
+                if (F::kGroupScale) {
+                    // a 16-byte block per lane quad = 128 k inside one scale group; the block's
+                    // activation sums are kept already multiplied by the offset-binary bias
+                    if (ng == 0) sxs[sxi] = sxs[sxi] * F::kBias;
+                    const float sc = bf16_bits_to_f32(cur.gs[h]);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) acc[ng][r] = fmaf(sc, part[r] + sxs[sxi][r], acc[ng][r]);
+                }
+            }
+        };
+
+        // CU chunks per trip of the chunk loop keep ring slots compile-time constants; the
+        // chunk count is padded up to a multiple (a padded chunk has no steps, its loads are
+        // clamped repeats)
+        constexpr int CU = (GC >= PW) ? 1 : PW / gcd_c(PW, NG * GC);
+        for (int c0 = 0; c0 < nchunks; c0 += CU) {
+#pragma unroll
+            for (int cu = 0; cu < CU; ++cu) {
+                const int c = c0 + cu;
+                __syncthreads();      // chunk c is staged
+                stage_load(c + 1);    // next chunk's activations travel while this one is consumed
+                const int gc_here = max(0, min(GC, (nb - c * (CK / LK)) / (KP * WL)));
+
+#pragma unroll
+                for (int ng = 0; ng < NG; ++ng) {
+                    if constexpr (GC >= PW) {
+                        for (int g0 = 0; g0 < GC; g0 += PW) {
+#pragma unroll
+                            for (int i = 0; i < PW; ++i) {
+                                const int g = g0 + i;
+                                const WSlot<WL> cur = ring[i];
+                                // refill with the step PW ahead: same tile, or the next on wrap
+                                int gn = g + PW;
+                                const bool wrap = gn >= GC;
+                                gn = wrap ? gn - GC : gn;
+                                const int ngn = (ng + 1 < NG) ? ng + 1 : 0;
+                                const unsigned char* wpn = wrap ? wptr[ngn] : wptr[ng];
+                                const int nn = wrap ? nrow[ngn] : nrow[ng];
+                                const int cn = (wrap && ng + 1 == NG) ? c + 1 : c;
+                                ring[i] = load_w(cn, wpn, nn, gn);
+                                if (g < gc_here) step(cur, ng, F::kGroupScale ? i : g);
+                            }
+                        }
+                    } else {
+#pragma unroll
+                        for (int g = 0; g < GC; ++g) {
+                            const int lin = (cu * NG + ng) * GC + g;
+                            const int slot = lin % PW;
+                            const WSlot<WL> cur = ring[slot];
+                            const int tn = (lin + PW) / GC;
+                            ring[slot] = load_w(c0 + tn / NG, wptr[tn % NG], nrow[tn % NG], (lin + PW) % GC);
+                            if (g < gc_here) step(cur, ng, g);
+                        }
+                    }
+                }
+                __syncthreads();      // every wave is done with chunk c
+                stage_store(c + 1);   // (after the last chunk: a harmless rewrite)
+            }
+        }
+
+        // ---- meet the KP waves' partial sums; wave w finishes accumulator row r = w % 4 ----
+        __syncthreads();  // every wave is done with the staged activations
+        constexpr int kItems = NG + (kRowBias ? 1 : 0);
+        float* mine = red + static_cast<size_t>(wv) * kItems * 4 * kWave;
+#pragma unroll
+        for (int i = 0; i < NG; ++i)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) mine[(i * 4 + r) * kWave + lane] = acc[i][r];
+        if (kRowBias) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) mine[(NG * 4 + r) * kWave + lane] = sxt[r];
+        }
+        __syncthreads();
+        const int rr = wv & 3;
+        auto total = [&](int item) {
+            float v = 0.f;
+#pragma unroll
+            for (int w = 0; w < KP; ++w)
+                v += red[((static_cast<size_t>(w) * kItems + item) * 4 + rr) * kWave + lane];
+            return v;
+        };
+        const int nout = a.swiglu ? N / 2 : N;
+        const int m = mt0 + 4 * q + rr;
+        const float bias = kRowBias ? F::kBias * total(NG) : 0.f;
+#pragma unroll
+        for (int i = 0; i < NG; ++i) {
+            if (KP > 4 && (i & 1) != (wv >> 2) && NG > 1) continue;   // 8 waves: split the tiles
+            if (KP > 4 && NG == 1 && wv >= 4) continue;
+            const int n = (tile0 + i) * 16 + j;
+            const bool ok = m < r1 && n < N;
+            float v = (total(i) + bias) * row_scale[i];
+            if (a.swiglu) {
+                // columns (2i, 2i+1) = (gate_i, up_i) sit in adjacent lanes
+                const float gb = bf16_bits_to_f32(f32_to_bf16_bits(v));
+                const float other = __int_as_float(__builtin_amdgcn_update_dpp(
+                    0, __float_as_int(gb), 0xB1, 0xF, 0xF, true));  // quad_perm [1,0,3,2]
+                if ((j & 1) == 0 && ok) {
+                    const float silu = gb / (1.f + expf(-gb));
+                    a.y[static_cast<size_t>(m) * nout + n / 2] = f32_to_bf16_bits(silu * other);
+                }
+            } else if (ok) {
+                const size_t o = static_cast<size_t>(m) * nout + n;
+                if (a.beta) v += bf16_bits_to_f32(a.y[o]);
+                a.y[o] = f32_to_bf16_bits(v);
+            }
+        }
+    }
+}
+
+template <class F, int KP, int CK, int NG, int PW, int WL>
+int launch_cfg(const SkinnyArgs& a, int problems, hipStream_t stream) {
+    constexpr bool kRowBias = F::kBias != 0.f && !F::kGroupScale;
+    constexpr size_t kStage = static_cast<size_t>(16) * (CK / 8 + 1) * 16;
+    constexpr size_t kRed = static_cast<size_t>(KP) * (NG + (kRowBias ? 1 : 0)) * 4 * kWave * sizeof(float);
+    constexpr size_t smem = kStage > kRed ? kStage : kRed;
+    static const hipError_t attr = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(&skinny_kernel<F, KP, CK, NG, PW, WL>),
+        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
+    if (attr != hipSuccess) return PIE_HIP_ERR_LAUNCH;
+    const int tiles = (a.N + 15) / 16;
+    const dim3 grid((tiles + NG - 1) / NG, problems);
+    hipLaunchKernelGGL((skinny_kernel<F, KP, CK, NG, PW, WL>), grid, dim3(KP * kWave), smem, stream, a);
+    return launch_status();
+}
+
+template <class F>
+int launch_skinny(SkinnyArgs a, int problems, hipStream_t stream) {
+    constexpr int LK = 4 * F::kPerLane;
+    constexpr int CK = 1024;
+    if (a.K <= 0 || a.N <= 0 || a.K % (4 * LK) != 0) return PIE_HIP_ERR_UNSUPPORTED;
+    if (F::kGroupScale) {
+        // group = 128 * 2^i k-values: a 16-byte block per lane quad never straddles two groups
+        if (a.G < LK || (a.G & (a.G - 1)) != 0 || a.K % a.G != 0) return PIE_HIP_ERR_UNSUPPORTED;
+        a.g_shift = __builtin_ctz(static_cast<unsigned>(a.G));
+    }
+    if (a.swiglu && (a.N % 2 != 0 || a.beta)) return PIE_HIP_ERR_INVALID;
+    if (problems > 65535) return PIE_HIP_ERR_UNSUPPORTED;
+    // tiles of 16 weight rows per block: as many as still leave two blocks per CU; with few
+    // tiles, eight waves split K instead of four.  Paired loads (whole 128-byte lines per row
+    // and wave) when K allows.
+    const long tiles = static_cast<long>((a.N + 15) / 16) * problems;
+    constexpr int W8 = (CK / (8 * LK) >= 2) ? 2 : 1;   // loads per step with eight waves
+    if (a.K % (8 * LK) == 0) {
+        if (tiles / 8 >= 448) return launch_cfg<F, 4, CK, 8, 4, 2>(a, problems, stream);
+        if (tiles / 4 >= 448) return launch_cfg<F, 4, CK, 4, 4, 2>(a, problems, stream);
+        if (tiles / 2 >= 448) return launch_cfg<F, 4, CK, 2, 4, 2>(a, problems, stream);
+        if (a.K % (8 * LK * W8) == 0) return launch_cfg<F, 8, CK, 1, 4, W8>(a, problems, stream);
+    }
+    if (tiles / 4 >= 448) return launch_cfg<F, 4, CK, 4, 4, 1>(a, problems, stream);
+    return launch_cfg<F, 4, CK, 1, 4, 1>(a, problems, stream);
+}
+
+int dispatch_skinny(int format, const SkinnyArgs& a, int problems, hipStream_t st) {
+    switch (format) {
+        case PIE_HIP_FMT_INT4B8: return launch_skinny<SkInt4>(a, problems, st);
+        case PIE_HIP_FMT_INT8: return launch_skinny<SkInt8>(a, problems, st);
+        case PIE_HIP_FMT_FP8: return launch_skinny<SkFp8>(a, problems, st);
+        case PIE_HIP_FMT_BF16: return launch_skinny<SkBf16>(a, problems, st);
+        default: return PIE_HIP_ERR_INVALID;
+    }
+}
+
+}  // namespace
+}  // namespace pie_hip
+
+extern "C" int pie_hip_gemm_skinny(int format, const uint16_t* act_bf16, const void* weight,
+                                   const void* scale, int scale_is_bf16, int group_size,
+                                   uint16_t* y_bf16, int M, int N, int K, int beta, int swiglu,
+                                   void* stream) {
+    using namespace pie_hip;
+    if (!act_bf16 || !weight || !y_bf16 || M <= 0) return PIE_HIP_ERR_INVALID;
+    if (format != PIE_HIP_FMT_BF16 && !scale) return PIE_HIP_ERR_INVALID;
+    SkinnyArgs a{};
+    a.act = act_bf16;
+    a.w = static_cast<const unsigned char*>(weight);
+    a.scale = static_cast<const unsigned char*>(scale);
+    a.y = y_bf16;
+    a.M = M;
+    a.N = N;
+    a.K = K;
+    a.G = group_size;
+    a.beta = beta;
+    a.swiglu = swiglu ? 1 : 0;
+    a.scale_is_bf16 = scale_is_bf16;
+    return dispatch_skinny(format, a, 1, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int pie_hip_moe_grouped_gemm(int format, const uint16_t* act_bf16,
+                                        const int32_t* route_act_rows,
+                                        const int32_t* expert_offsets, int num_experts,
+                                        int max_rows_per_expert, const void* weights,
+                                        size_t weight_stride_bytes, const void* scales,
+                                        size_t scale_stride_bytes, int scale_is_bf16,
+                                        int group_size, uint16_t* y_bf16, int N, int K, int swiglu,
+                                        void* stream) {
+    using namespace pie_hip;
+    if (!act_bf16 || !expert_offsets || !weights || !y_bf16 || num_experts <= 0 ||
+        max_rows_per_expert <= 0)
+        return PIE_HIP_ERR_INVALID;
+    if (format != PIE_HIP_FMT_BF16 && !scales) return PIE_HIP_ERR_INVALID;
+    SkinnyArgs a{};
+    a.act = act_bf16;
+    a.act_rows = route_act_rows;
+    a.w = static_cast<const unsigned char*>(weights);
+    a.scale = static_cast<const unsigned char*>(scales);
+    a.y = y_bf16;
+    a.offsets = expert_offsets;
+    a.N = N;
+    a.K = K;
+    a.G = group_size;
+    a.swiglu = swiglu ? 1 : 0;
+    a.scale_is_bf16 = scale_is_bf16;
+    a.w_stride = weight_stride_bytes;
+    a.scale_stride = scale_stride_bytes;
+    return dispatch_skinny(format, a, num_experts, static_cast<hipStream_t>(stream));
+}

@@ -1,0 +1,148 @@
+"""GPU parity: the matrix-core skinny GEMM (5 <= M <= a few dozen rows) and the MoE grouped GEMM
+against the CPU oracle's fused-order quantised GEMM (fp32 sums differ only in order), plus exact
+structural checks (one-hot activations recover the dequantised rows bit-exactly)."""
+import numpy as np
+import pytest
+
+from gpu_util import bits, dev, ulp_diff
+from test_linear_fused_gpu import close_to_oracle, make_weight, oracle_linear
+
+pytestmark = pytest.mark.gpu
+
+KINDS = ["int4b8", "int8", "fp8", "bf16"]
+
+
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("M,N,K", [(5, 64, 512), (8, 200, 1024), (16, 256, 4096), (17, 96, 2048),
+                                   (32, 1040, 1536), (45, 48, 512),
+                                   # enough 16-row tiles for two and four tiles per block
+                                   (8, 12304, 512), (20, 24592, 512)])
+def test_skinny_matches_oracle(gpu, oracle, kind, M, N, K):
+    import torch
+    from pie_amd import ops
+
+    rng = np.random.default_rng(300 + M + N)
+    wd, mk = make_weight(oracle, rng, kind, N, K)
+    x = oracle.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32))
+    w = mk(gpu)
+    got = bits(ops.gemm_skinny(dev(x, gpu, torch.bfloat16), w))
+    ref = oracle_linear(oracle, wd, x)
+    assert got.shape == ref.shape
+    assert close_to_oracle(oracle, got, ref)
+    assert (ulp_diff(got, ref) <= 1).mean() > 0.98
+
+
+@pytest.mark.parametrize("kind", KINDS)
+def test_skinny_equals_gemv_path_rowwise(gpu, oracle, kind):
+    """Same contract as the GEMV: every activation row gives the value the GEMV gives for it
+    (sum order differs, so within one bf16 step on almost all elements)."""
+    import torch
+    from pie_amd import ops
+
+    rng = np.random.default_rng(311)
+    M, N, K = 24, 512, 2048
+    wd, mk = make_weight(oracle, rng, kind, N, K)
+    x = oracle.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32))
+    w = mk(gpu)
+    xg = dev(x, gpu, torch.bfloat16)
+    a = bits(ops.gemm_skinny(xg, w))
+    b = bits(ops.linear_fused(xg, w))
+    d = ulp_diff(a, b)
+    assert (d <= 1).mean() > 0.99 and close_to_oracle(oracle, a, b)
+
+
+@pytest.mark.parametrize("kind", KINDS)
+def test_skinny_one_hot_rows_are_exact(gpu, oracle, kind):
+    """act = one-hot rows: y[m, n] must be bf16(dequantised w[n, k_m]) exactly — pins the
+    lane/k layout of both MFMA operands and the offset-binary bias removal."""
+    import torch
+    from pie_amd import ops
+
+    rng = np.random.default_rng(312)
+    M, N, K = 16, 80, 1024
+    wd, mk = make_weight(oracle, rng, kind, N, K)
+    ks = rng.choice(K, size=M, replace=False)
+    x = np.zeros((M, K), np.float32)
+    x[np.arange(M), ks] = 1.0
+    xb = oracle.f32_to_bf16(x)
+    got = bits(ops.gemm_skinny(dev(xb, gpu, torch.bfloat16), mk(gpu)))
+    ref = oracle_linear(oracle, wd, xb)
+    assert np.array_equal(got, ref)
+
+
+@pytest.mark.parametrize("kind", ["int4b8", "fp8"])
+def test_skinny_beta_and_swiglu(gpu, oracle, kind):
+    import torch
+    from pie_amd import ops
+
+    rng = np.random.default_rng(313)
+    M, I, K = 12, 192, 1024
+    wd, mk = make_weight(oracle, rng, kind, 2 * I, K)
+    x = oracle.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32))
+    xg = dev(x, gpu, torch.bfloat16)
+    w = mk(gpu)
+    # residual accumulate
+    y0 = oracle.f32_to_bf16(rng.standard_normal((M, 2 * I)).astype(np.float32))
+    got = bits(ops.gemm_skinny(xg, w, y=dev(y0, gpu, torch.bfloat16).clone(), beta=1))
+    ref = oracle_linear(oracle, wd, x, y_in=y0)
+    assert close_to_oracle(oracle, got, ref) and (ulp_diff(got, ref) <= 1).mean() > 0.98
+    # swiglu epilogue over interleaved rows
+    perm = np.empty(2 * I, np.int64)
+    perm[0::2], perm[1::2] = np.arange(I), np.arange(I) + I
+    idx = torch.from_numpy(perm).to(gpu)
+    wi = ops.WeightView(w.kind, w.data[idx].contiguous(), w.scale[idx].contiguous(), w.group_size,
+                        w.N, w.K)
+    fused = bits(ops.gemm_skinny(xg, wi, swiglu=True))
+    assert fused.shape == (M, I)
+    unfused = bits(ops.swiglu_bf16(ops.gemm_skinny(xg, w)))
+    assert np.array_equal(fused, unfused)
+    with pytest.raises(ops.KernelError):
+        ops.gemm_skinny(xg, wi, y=torch.zeros(M, I, device=gpu, dtype=torch.bfloat16), beta=1,
+                        swiglu=True)
+
+
+def test_skinny_rejects_unsupported_k(gpu, oracle):
+    import torch
+    from pie_amd import ops
+
+    rng = np.random.default_rng(314)
+    wd, mk = make_weight(oracle, rng, "int4b8", 32, 640)   # K not a multiple of 512
+    x = torch.zeros(8, 640, device=gpu, dtype=torch.bfloat16)
+    with pytest.raises(ops.KernelError):
+        ops.gemm_skinny(x, mk(gpu))
+
+
+@pytest.mark.parametrize("kind", ["fp8", "int4b8", "bf16"])
+@pytest.mark.parametrize("swiglu", [False, True])
+def test_moe_grouped_gemm_matches_per_expert_oracle(gpu, oracle, kind, swiglu):
+    """Routes sorted by expert, gathered activation rows, empty experts, an expert with more
+    rows than one tile."""
+    import torch
+    from pie_amd import ops
+
+    rng = np.random.default_rng(320)
+    E, N, K, T = 6, 96, 512, 20
+    counts = np.array([3, 0, 21, 1, 0, 7])
+    offs = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    R = int(offs[-1])
+    rows = rng.integers(0, T, size=R).astype(np.int32)
+    x = oracle.f32_to_bf16(rng.standard_normal((T, K)).astype(np.float32))
+    experts = [make_weight(oracle, rng, kind, N, K) for _ in range(E)]
+    views = [mk(gpu) for _, mk in experts]
+    wstack = torch.stack([v.data for v in views]).contiguous()
+    sstack = None if views[0].scale is None else torch.stack([v.scale for v in views]).contiguous()
+    got = bits(ops.moe_grouped_gemm(dev(x, gpu, torch.bfloat16), dev(rows, gpu), dev(offs, gpu),
+                                    kind, wstack, sstack, N, K, rows_hint=16,
+                                    group_size=views[0].group_size, swiglu=swiglu))
+    ref = np.zeros((R, N), np.uint16)
+    for e in range(E):
+        lo, hi = offs[e], offs[e + 1]
+        if hi > lo:
+            ref[lo:hi] = oracle_linear(oracle, experts[e][0], x[rows[lo:hi]])
+    if swiglu:
+        # kernel pairs adjacent rows (gate_i, up_i) = canonical rows (2i, 2i+1)
+        canon = np.concatenate([ref[:, 0::2], ref[:, 1::2]], axis=1)
+        ref = oracle.swiglu(canon)
+    assert got.shape == ref.shape
+    assert close_to_oracle(oracle, got, ref, rel=2.0 ** -6)
+    assert (ulp_diff(got, ref) <= 1).mean() > 0.97
