@@ -51,40 +51,31 @@ int fmt_code(Quant q) {
     }
 }
 
-// y = epilogue(rmsnorm?(act) · W^T): the norm that precedes a projection rides in its
-// activation staging, SwiGLU in the gate/up projection's epilogue.
+// y = epilogue(rmsnorm?(act) · W^T) by the weight's storage format — the dispatcher role of
+// gemm_act_x_w (driver/cuda/src/ops/gemm.cpp:1414-1583).  Up to four rows: the weight-streaming
+// GEMV with the norm riding in its activation staging and SwiGLU in its epilogue.  More rows:
+// the matrix-core skinny GEMM (norm as its own kernel into `norm_tmp`), which streams the
+// weights once per 16 rows; shapes it does not take fall back to the GEMV path.
 void linear_fused(const Linear& w, const uint16_t* act, const uint16_t* norm_w, float eps,
-                  uint16_t* y, int M, int beta, int swiglu, hipStream_t s) {
-    PIE_KERNEL(pie_hip_linear_fused(fmt_code(w.kind), act, norm_w, eps, w.data, w.scale,
-                                    w.scale_bf16 ? 1 : 0, w.group, y, M, w.N, w.K, beta, swiglu, s));
-}
-
-// y[M, N] = act[M, K] · W[N, K]^T (+ y when beta), by the weight's storage format — the
-// dispatcher role of gemm_act_x_w (driver/cuda/src/ops/gemm.cpp:1414-1583).
-void linear(const Linear& w, const uint16_t* act, uint16_t* y, int M, int beta, hipStream_t s) {
-    switch (w.kind) {
-        case Quant::Int4b8:
-            PIE_KERNEL(pie_hip_gemv_w4a16(act, static_cast<const uint32_t*>(w.data),
-                                          static_cast<const uint16_t*>(w.scale), y, M, w.N, w.K,
-                                          w.group, beta, s));
-            break;
-        case Quant::Int8:
-            PIE_KERNEL(pie_hip_gemv_w8a16(act, static_cast<const int8_t*>(w.data),
-                                          w.scale_bf16 ? nullptr : static_cast<const float*>(w.scale),
-                                          w.scale_bf16 ? static_cast<const uint16_t*>(w.scale) : nullptr,
-                                          y, M, w.N, w.K, beta, s));
-            break;
-        case Quant::Fp8:
-            PIE_KERNEL(pie_hip_gemv_fp8(act, static_cast<const uint8_t*>(w.data),
-                                        w.scale_bf16 ? nullptr : static_cast<const float*>(w.scale),
-                                        w.scale_bf16 ? static_cast<const uint16_t*>(w.scale) : nullptr,
-                                        y, M, w.N, w.K, beta, s));
-            break;
-        case Quant::Bf16:
-            PIE_KERNEL(pie_hip_gemv_bf16(act, static_cast<const uint16_t*>(w.data), y, M, w.N, w.K,
-                                         beta, s));
-            break;
+                  uint16_t* y, int M, int beta, int swiglu, uint16_t* norm_tmp, hipStream_t s) {
+    const int fmt = fmt_code(w.kind);
+    const int sbf = w.scale_bf16 ? 1 : 0;
+    if (M > 4) {
+        const uint16_t* a = act;
+        if (norm_w) {
+            PIE_KERNEL(pie_hip_rmsnorm(act, norm_w, norm_tmp, M, w.K, eps, s));
+            a = norm_tmp;
+        }
+        const int st = pie_hip_gemm_skinny(fmt, a, w.data, w.scale, sbf, w.group, y, M, w.N, w.K,
+                                           beta, swiglu, s);
+        if (st == PIE_HIP_OK) return;
+        if (st != PIE_HIP_ERR_UNSUPPORTED) PIE_KERNEL(st);
+        PIE_KERNEL(pie_hip_linear_fused(fmt, a, nullptr, eps, w.data, w.scale, sbf, w.group, y, M,
+                                        w.N, w.K, beta, swiglu, s));
+        return;
     }
+    PIE_KERNEL(pie_hip_linear_fused(fmt, act, norm_w, eps, w.data, w.scale, sbf, w.group, y, M,
+                                    w.N, w.K, beta, swiglu, s));
 }
 
 }  // namespace
@@ -215,24 +206,28 @@ void Executor::body(int N, int S, int max_kv_len) {
     PIE_KERNEL(pie_hip_rope_table(positions, model_.inv_freq, rope_tab_, N, d, s));
     for (int l = 0; l < m.layers; ++l) {
         const LayerWeights& w = model_.layers[l];
-        linear_fused(w.wqkv, x_, w.attn_norm, m.rms_eps, qkv_, N, 0, 0, s);
+        linear_fused(w.wqkv, x_, w.attn_norm, m.rms_eps, qkv_, N, 0, 0, xn_, s);
         PIE_KERNEL(pie_hip_qkv_rope_kvwrite(qkv_, q_, k_pool_[l], v_pool_[l], w.q_norm, w.k_norm,
                                             rope_tab_, slots, N, hq, hk, d, m.rope_interleaved,
                                             m.rms_eps, s));
         PIE_KERNEL(pie_hip_attn_rows_paged(q_, k_pool_[l], v_pool_[l], attn_, nullptr, pages,
                                            row_begin, row_len, N, hq, hk, d, page_size_, -1.f,
                                            max_kv_len, attn_ws_, attn_ws_bytes_, s));
-        linear(w.wo, attn_, x_, N, 1, s);
-        linear_fused(w.wgu, x_, w.ffn_norm, m.rms_eps, act_, N, 0, 1, s);
-        linear(w.wdown, act_, x_, N, 1, s);
+        linear_fused(w.wo, attn_, nullptr, m.rms_eps, x_, N, 1, 0, xn_, s);
+        linear_fused(w.wgu, x_, w.ffn_norm, m.rms_eps, act_, N, 0, 1, xn_, s);
+        linear_fused(w.wdown, act_, nullptr, m.rms_eps, x_, N, 1, 0, xn_, s);
     }
     // lm_head only on the sampled rows (driver/portable/src/graph_qwen3.cpp:867-896)
     const int cap = static_cast<int>(std::min<size_t>(max_tokens_, 2 * static_cast<size_t>(cfg_.batching.max_forward_requests)));
     for (int s0 = 0; s0 < S; s0 += cap) {
         const int n = std::min(cap, S - s0);
         PIE_KERNEL(pie_hip_embed(sample_rows + s0, x_, xs_, n, H, N, s));  // row gather
-        PIE_KERNEL(pie_hip_linear_fused(PIE_HIP_FMT_BF16, xs_, model_.final_norm, m.rms_eps,
-                                        model_.lm_head, nullptr, 0, 0, logits_, n, m.vocab, H, 0, 0, s));
+        Linear head;
+        head.kind = Quant::Bf16;
+        head.data = model_.lm_head;
+        head.N = m.vocab;
+        head.K = H;
+        linear_fused(head, xs_, model_.final_norm, m.rms_eps, logits_, n, 0, 0, xn_, s);
         PIE_KERNEL(pie_hip_argmax(logits_, out_tokens_ + s0, n, m.vocab, s));
     }
 }
