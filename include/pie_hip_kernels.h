@@ -101,14 +101,14 @@ int pie_hip_linear_fused(int format, const uint16_t* act_bf16, const uint16_t* n
                          int swiglu, void* stream);
 
 /*
- * Weight-only GEMM for a handful to a few hundred activation rows on the matrix cores:
+ * Weight-only GEMM for a handful to a few dozen activation rows on the matrix cores:
  *   y[m, n] = epilogue( sum_k act[m,k] * w(n,k) ), same formats, scales, beta and swiglu
- * contracts as pie_hip_linear_fused (no fused norm); the weights are streamed once per 64
+ * contracts as pie_hip_linear_fused (no fused norm); the weights are streamed once per 16
  * activation rows instead of once per 4.  bf16 products, fp32 accumulation; int4/int8 weights
  * enter the MFMA offset-binary (128+nibble / 128+byte, exact in bf16) and the offset is removed
  * per group / per row in fp32, so the result differs from the GEMV only by fp32 summation order.
- * Requirements: K % 128 (int4b8; group_size a multiple of 128 dividing K), K % 64 (int8, fp8),
- * K % 32 (bf16).
+ * Requirements (else PIE_HIP_ERR_UNSUPPORTED): K % 512 == 0 and group_size = 128 * 2^i dividing
+ * K (int4b8); K % 256 == 0 (int8, fp8); K % 128 == 0 (bf16).
  * Replaces Marlin W4A16 for small/medium M (driver/cuda/third_party/marlin/marlin_wrapper.hpp:39-51)
  * and the cuBLASLt small-M path of gemm_act_x_w (driver/cuda/src/ops/gemm.cpp:1414-1583).
  */
@@ -122,9 +122,9 @@ int pie_hip_gemm_skinny(int format, const uint16_t* act_bf16, const void* weight
  *   act[route_act_rows[r]] (or act[r] when route_act_rows is NULL) times expert e's [N,K]
  *   weights at weights + e*weight_stride_bytes (scales at scales + e*scale_stride_bytes).
  * Experts without routes cost nothing and their weights are never read; an expert's weights
- * are read once however many routes hit it.  max_rows_per_expert bounds the per-expert row
- * count (host-known upper bound, e.g. the number of tokens).  With swiglu the weight rows are
- * interleaved (gate_0, up_0, ...) and y is [routes, N/2].
+ * are read once per 16 routes that hit it.  max_rows_per_expert is a hint (> 0) of the largest
+ * per-expert row count.  With swiglu the weight rows are interleaved (gate_0, up_0, ...) and y
+ * is [routes, N/2].  Same K requirements as pie_hip_gemm_skinny.
  * Replaces the per-route MoE decode GEMVs (driver/cuda/src/kernels/dequant_wna16.cu:59-169)
  * and the grouped GEMM of driver/cuda/src/ops/gemm.hpp:189-198.
  */
@@ -134,6 +134,32 @@ int pie_hip_moe_grouped_gemm(int format, const uint16_t* act_bf16, const int32_t
                              size_t weight_stride_bytes, const void* scales,
                              size_t scale_stride_bytes, int scale_is_bf16, int group_size,
                              uint16_t* y_bf16, int N, int K, int swiglu, void* stream);
+
+/*
+ * MoE routing: per token softmax over router_logits[t, 0..E) (bf16 in, fp32 inside), top_k by
+ * repeated argmax with exclusion (ties to the lowest expert index), weights renormalised to
+ * sum 1 — topk_softmax_bf16_kernel, driver/cuda/src/kernels/topk_softmax.cu:19-86 (graph form:
+ * driver/portable/src/graph_common.cpp:262-283).  The same launch builds the grouped layout of
+ * pie_hip_moe_grouped_gemm: routes (t, k) counting-sorted by expert.
+ *   topk_idx [T, top_k] int32, topk_weight [T, top_k] f32 (bit-exact integer outputs given the
+ *   probabilities; the order of routes inside one expert is unspecified),
+ *   expert_offsets [E+1], route_token [T*top_k] (token of each sorted route),
+ *   route_pos [T*top_k] (sorted position of route (t, k)).
+ * num_experts <= 512, top_k <= 16 (the reference's bounds).
+ */
+int pie_hip_moe_route(const uint16_t* router_logits_bf16, int32_t* topk_idx, float* topk_weight,
+                      int32_t* expert_offsets, int32_t* route_token, int32_t* route_pos,
+                      int num_tokens, int num_experts, int top_k, void* stream);
+
+/*
+ * MoE combine: out[t, :] = bf16( (add ? out[t, :] : 0) + sum_k topk_weight[t, k] *
+ * y_routes[route_pos[t, k], :] ), fp32 sum in top-k order, one rounding —
+ * token_batched_weighted_sum[_add]_bf16_kernel, driver/cuda/src/kernels/moe_dispatch.cu:152-196.
+ * hidden % 8 == 0.
+ */
+int pie_hip_moe_combine(const uint16_t* y_routes_bf16, const int32_t* route_pos,
+                        const float* topk_weight, uint16_t* out_bf16, int num_tokens, int top_k,
+                        int hidden, int add, void* stream);
 
 /* Measurement hook: the next GEMV kernel this thread launches (any format, M <= 4) is
  * bracketed by the two HIP events (hipEvent_t), so hipEventElapsedTime(start, stop) is that

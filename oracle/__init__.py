@@ -293,3 +293,27 @@ def gemm_fp8(act_bf16, q, scale_inv, mode: int = 0, y_in=None, want_abs: bool = 
     lib().orc_gemm_fp8(_p(act), _p(q), _p(s), _p(yin), _p(y32), _p(y16), _p(ab), C.c_int(M),
                        C.c_int(N), C.c_int(K), C.c_int(0 if y_in is None else 1), C.c_int(mode))
     return (y32, y16, ab) if want_abs else (y32, y16)
+
+
+def topk_softmax(logits_bf16, top_k: int):
+    """(idx int32 [N, k], weights f32 [N, k]) — driver/cuda/src/kernels/topk_softmax.cu:19-86."""
+    lg = _c(logits_bf16, np.uint16)
+    N, E = lg.shape
+    idx = np.empty((N, top_k), np.int32)
+    w = np.empty((N, top_k), np.float32)
+    lib().orc_topk_softmax(_p(lg), _p(idx), _p(w), C.c_int(N), C.c_int(E), C.c_int(top_k))
+    return idx, w
+
+
+def moe_combine(y_routes_bf16, topk_w, out_bf16=None):
+    """out[t] (+)= sum_k w[t,k] * y_routes[t*k + k] (driver/cuda/src/kernels/moe_dispatch.cu:152-196).
+    y_routes: [N*k, H] in (token, k) order; `out_bf16` given = accumulate onto it."""
+    w = _c(topk_w, np.float32)
+    N, K = w.shape
+    yr = _c(y_routes_bf16, np.uint16)
+    H = yr.shape[1]
+    add = out_bf16 is not None
+    out = np.array(out_bf16, np.uint16, copy=True) if add else np.zeros((N, H), np.uint16)
+    out = np.ascontiguousarray(out)
+    lib().orc_moe_combine(_p(yr), _p(w), _p(out), C.c_int(N), C.c_int(K), C.c_int(H), C.c_int(int(add)))
+    return out

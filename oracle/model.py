@@ -27,12 +27,17 @@ class _Model(C.Structure):
                 ("attn_norm", C.POINTER(C.c_void_p)), ("ffn_norm", C.POINTER(C.c_void_p)),
                 ("q_norm", C.POINTER(C.c_void_p)), ("k_norm", C.POINTER(C.c_void_p)),
                 ("wqkv", C.POINTER(_Linear)), ("wo", C.POINTER(_Linear)),
-                ("wgu", C.POINTER(_Linear)), ("wdown", C.POINTER(_Linear))]
+                ("wgu", C.POINTER(_Linear)), ("wdown", C.POINTER(_Linear)),
+                ("num_experts", C.c_int), ("top_k", C.c_int), ("expert_intermediate", C.c_int),
+                ("router", C.POINTER(C.c_void_p))]
 
 
 class OracleModel:
     """`cfg`: dict with hidden, layers, q_heads, kv_heads, head_dim, intermediate, vocab,
-    rms_eps, rope_interleaved, qk_norm, quant, group_size, page_size, total_pages.
+    rms_eps, rope_interleaved, qk_norm, quant, group_size, page_size, total_pages; for MoE also
+    num_experts, top_k, expert_intermediate (then `layers.l.wgu` / `.wdown` hold the experts
+    stacked along the rows, gate rows before up rows inside each expert, and `layers.l.router`
+    is bf16 [E, H]).
     `tensors`: name -> numpy array, names as the driver exports them; row scales of int8/fp8
     may be bf16 bits (uint16) and are widened to f32 here."""
 
@@ -81,6 +86,11 @@ class OracleModel:
         m.q_norm = parr([f"layers.{l}.q_norm" for l in range(L)])
         m.k_norm = parr([f"layers.{l}.k_norm" for l in range(L)])
         m.wqkv, m.wo, m.wgu, m.wdown = larr("wqkv"), larr("wo"), larr("wgu"), larr("wdown")
+        m.num_experts = int(cfg.get("num_experts", 0))
+        m.top_k = int(cfg.get("top_k", 0))
+        m.expert_intermediate = int(cfg.get("expert_intermediate", 0))
+        if m.num_experts:
+            m.router = parr([f"layers.{l}.router" for l in range(L)])
         self._m = m
         ps, tp = cfg["page_size"], cfg["total_pages"]
         shape = (tp, ps, cfg["kv_heads"], cfg["head_dim"])
@@ -168,18 +178,24 @@ def model_from_driver(drv, cfg: dict):
             a = drv.export_tensor(p + n, np.uint16)
             if a is not None:
                 t[p + n] = a
+        E = int(cfg.get("num_experts", 0)) if cfg["arch"] == "qwen3_moe" else 0
+        if E:
+            t[p + "router"] = drv.export_tensor(p + "router", np.uint16)
         for w in ("wqkv", "wo", "wgu", "wdown"):
             data = drv.export_tensor(p + w + ".data", _DATA_DTYPE[quant])
             sc = drv.export_tensor(p + w + ".scale", scale_dt)
             if w == "wgu":
-                # the driver stores gate/up rows interleaved (gate_0, up_0, ...); the oracle uses
-                # the canonical order (all gate rows, then all up rows)
-                n = 2 * cfg["intermediate"]
-                data = data.reshape(n, -1)
-                data = np.concatenate([data[0::2], data[1::2]]).reshape(-1)
+                # the driver stores gate/up rows interleaved (gate_0, up_0, ...) — per expert for
+                # MoE; the oracle uses the canonical order (all gate rows, then all up rows)
+                n = 2 * (cfg["expert_intermediate"] if E else cfg["intermediate"])
+                blocks = max(E, 1)
+
+                def canon(a):
+                    a = a.reshape(blocks, n, -1)
+                    return np.concatenate([a[:, 0::2], a[:, 1::2]], axis=1).reshape(-1)
+                data = canon(data)
                 if sc is not None:
-                    sc = sc.reshape(n, -1)
-                    sc = np.concatenate([sc[0::2], sc[1::2]]).reshape(-1)
+                    sc = canon(sc)
             t[p + w + ".data"] = data
             if sc is not None:
                 t[p + w + ".scale"] = sc
@@ -188,4 +204,7 @@ def model_from_driver(drv, cfg: dict):
                 rms_eps=cfg.get("rms_eps", 1e-5), rope_interleaved=1 if cfg["arch"] == "llama3" else 0,
                 qk_norm=cfg["arch"] != "llama3", quant=quant, group_size=cfg.get("group_size", 128),
                 page_size=cfg["page_size"], total_pages=cfg["total_pages"])
+    if cfg["arch"] == "qwen3_moe":
+        ocfg.update(num_experts=cfg["num_experts"], top_k=cfg["top_k"],
+                    expert_intermediate=cfg["expert_intermediate"], intermediate=0)
     return OracleModel(ocfg, t), t

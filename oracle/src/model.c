@@ -9,6 +9,10 @@
  * (driver/cuda/src/model/llama_like.cpp:364-762): every inter-op activation is bf16, fp32
  * inside an op, residual add fused into the projection with one rounding (:626-628,:703-705).
  * Quantised linears use the fused evaluation order (scale applied to fp32 partial sums).
+ * MoE layers (qwen3_moe): router GEMM -> top-k softmax -> per-route gate/up -> SwiGLU (bf16) ->
+ * per-route down, rounded to bf16 per route -> weighted sum onto the residual — the composition
+ * of driver/cuda/src/model/kimi_forward.cpp:662-714 (graph form
+ * driver/portable/src/graph_common.cpp:237-345).
  *
  * The composition is pinned by tests/test_oracle_model.py: every op is one of the separately
  * pinned oracle functions, and the whole pass is compared with an independent numpy fp64
@@ -42,6 +46,10 @@ typedef struct {
     const OrcLinear* wo;
     const OrcLinear* wgu;
     const OrcLinear* wdown;
+    /* MoE (num_experts > 0): wgu / wdown hold the experts stacked along the rows,
+     * [E * 2*Ie, H] (per expert: gate rows then up rows) and [E * H, Ie]. */
+    int num_experts, top_k, expert_intermediate;
+    const uint16_t* const* router; /* [L] bf16 [E, H] */
 } OrcModel;
 
 static void orc_linear(const OrcModel* m, const OrcLinear* w, const uint16_t* act, uint16_t* y,
@@ -65,6 +73,55 @@ static void orc_linear(const OrcModel* m, const OrcLinear* w, const uint16_t* ac
             break;
     }
     free(tmp);
+}
+
+/* Expert e's [N, K] slice of a stacked linear. */
+static OrcLinear orc_expert_slice(const OrcModel* m, const OrcLinear* w, int e, int N, int K) {
+    OrcLinear s;
+    const size_t nk = (size_t)e * N * K;
+    switch (m->quant) {
+        case 0:
+            s.data = (const unsigned char*)w->data + nk / 2;
+            s.scale = (const unsigned char*)w->scale + (size_t)e * N * (K / m->group) * 2;
+            break;
+        case 1:
+        case 2:
+            s.data = (const unsigned char*)w->data + nk;
+            s.scale = (const unsigned char*)w->scale + (size_t)e * N * 4;
+            break;
+        default:
+            s.data = (const unsigned char*)w->data + nk * 2;
+            s.scale = NULL;
+            break;
+    }
+    return s;
+}
+
+/* x[t] += sum_k w[t,k] * down_e(swiglu(gateup_e(xn[t]))) over the token's top-k experts. */
+static void orc_moe_ffn(const OrcModel* m, int l, const uint16_t* xn, uint16_t* x, int N) {
+    const int H = m->hidden, E = m->num_experts, K = m->top_k, Ie = m->expert_intermediate;
+    uint16_t* logits = (uint16_t*)malloc((size_t)N * E * 2);
+    float* lf = (float*)malloc((size_t)N * E * 4);
+    int32_t* idx = (int32_t*)malloc((size_t)N * K * 4);
+    float* wts = (float*)malloc((size_t)N * K * 4);
+    uint16_t* yr = (uint16_t*)malloc((size_t)N * K * H * 2);
+    orc_gemm_bf16(xn, m->router[l], NULL, lf, logits, NULL, N, E, H, 0, 0);
+    orc_topk_softmax(logits, idx, wts, N, E, K);
+#pragma omp parallel for schedule(dynamic)
+    for (int r = 0; r < N * K; ++r) {
+        const int t = r / K, e = idx[r];
+        uint16_t* gu = (uint16_t*)malloc((size_t)2 * Ie * 2);
+        uint16_t* act = (uint16_t*)malloc((size_t)Ie * 2);
+        const OrcLinear wg = orc_expert_slice(m, &m->wgu[l], e, 2 * Ie, H);
+        const OrcLinear wd = orc_expert_slice(m, &m->wdown[l], e, H, Ie);
+        orc_linear(m, &wg, xn + (size_t)t * H, gu, 1, 2 * Ie, H, 0);
+        orc_swiglu(gu, act, 1, Ie);
+        orc_linear(m, &wd, act, yr + (size_t)r * H, 1, H, Ie, 0);
+        free(gu);
+        free(act);
+    }
+    orc_moe_combine(yr, wts, x, N, K, H, 1);
+    free(logits); free(lf); free(idx); free(wts); free(yr);
 }
 
 /*
@@ -102,9 +159,13 @@ void orc_llama_forward(const OrcModel* m, uint16_t* const* k_pages, uint16_t* co
                       N, hq, hk, d, page_size, -1.f, 0);
         orc_linear(m, &m->wo[l], attn, x, N, H, hq * d, 1);
         orc_rmsnorm(x, NULL, m->ffn_norm[l], xn, N, H, m->rms_eps);
-        orc_linear(m, &m->wgu[l], xn, gu, N, 2 * I, H, 0);
-        orc_swiglu(gu, act, N, I);
-        orc_linear(m, &m->wdown[l], act, x, N, H, I, 1);
+        if (m->num_experts > 0) {
+            orc_moe_ffn(m, l, xn, x, N);
+        } else {
+            orc_linear(m, &m->wgu[l], xn, gu, N, 2 * I, H, 0);
+            orc_swiglu(gu, act, N, I);
+            orc_linear(m, &m->wdown[l], act, x, N, H, I, 1);
+        }
     }
     if (S > 0) {
         uint16_t* xs = (uint16_t*)malloc((size_t)S * H * 2);

@@ -37,6 +37,7 @@ struct ModelConfig {
     // synthetic random-init weights: N(0, init_std) in bf16, then quantised
     std::uint64_t seed = 0x9E3779B97F4A7C15ull;
     float init_std = 0.02f;
+    float router_std = 0.f;  // MoE router rows; 0 = init_std
 };
 
 struct BatchingConfig {
@@ -167,6 +168,7 @@ inline DriverConfig parse_config_text(const std::string& text) {
                 else if (k == "norm_topk") m.norm_topk = to_bool(v, key);
                 else if (k == "seed") m.seed = (std::uint64_t)to_int(v, key);
                 else if (k == "init_std") m.init_std = (float)to_float(v, key);
+                else if (k == "router_std") m.router_std = (float)to_float(v, key);
                 // other [model] keys (paths, dtype hints) belong to loaders this driver lacks
             } else if (sec == "batching") {
                 auto& b = c.batching;

@@ -115,7 +115,21 @@ Executor::Executor(const DriverConfig& cfg, Model& model) : cfg_(cfg), model_(mo
     q_ = dmalloc<uint16_t>(T * hq * d);
     attn_ = dmalloc<uint16_t>(T * hq * d);
     gu_ = dmalloc<uint16_t>(T * 2 * I);
-    act_ = dmalloc<uint16_t>(T * I);
+    if (model.is_moe()) {
+        // one row per route (token, k): expert activations and per-route outputs, the router
+        // logits, and the grouped layout the routing kernel builds
+        const size_t R = T * m.top_k;
+        act_ = dmalloc<uint16_t>(R * I);
+        moe_y_ = dmalloc<uint16_t>(R * H);
+        moe_logits_ = dmalloc<uint16_t>(T * m.num_experts);
+        moe_idx_ = dmalloc<int32_t>(R);
+        moe_w_ = dmalloc<float>(R);
+        moe_offsets_ = dmalloc<int32_t>(m.num_experts + 1);
+        moe_route_token_ = dmalloc<int32_t>(R);
+        moe_route_pos_ = dmalloc<int32_t>(R);
+    } else {
+        act_ = dmalloc<uint16_t>(T * I);
+    }
     rope_tab_ = dmalloc<float>(T * d);
     const size_t srows = std::min<size_t>(T, 2 * static_cast<size_t>(cfg.batching.max_forward_requests));
     xs_ = dmalloc<uint16_t>(srows * H);
@@ -142,7 +156,11 @@ Executor::~Executor() {
                     static_cast<void*>(q_), static_cast<void*>(attn_), static_cast<void*>(gu_),
                     static_cast<void*>(act_), static_cast<void*>(xs_), static_cast<void*>(logits_),
                     static_cast<void*>(rope_tab_), static_cast<void*>(out_tokens_), attn_ws_,
-                    static_cast<void*>(in_dev_), static_cast<void*>(copy_ids_)})
+                    static_cast<void*>(in_dev_), static_cast<void*>(copy_ids_),
+                    static_cast<void*>(moe_y_), static_cast<void*>(moe_logits_),
+                    static_cast<void*>(moe_idx_), static_cast<void*>(moe_w_),
+                    static_cast<void*>(moe_offsets_), static_cast<void*>(moe_route_token_),
+                    static_cast<void*>(moe_route_pos_)})
         if (p) (void)hipFree(p);
     if (in_host_) (void)hipHostFree(in_host_);
     if (out_host_) (void)hipHostFree(out_host_);
@@ -187,6 +205,30 @@ void Executor::alloc_kv() {
     }
 }
 
+// x += sum_k w_k * down_e(swiglu(gate_up_e(norm(x)))) over each token's top-k experts
+// (driver/portable/src/graph_common.cpp:237-345; kernel-by-kernel form
+// driver/cuda/src/model/kimi_forward.cpp:662-714): norm, router GEMM, one routing kernel, two
+// grouped expert GEMMs that read every touched expert once, one combine onto the residual.
+void Executor::moe_block(const LayerWeights& w, int N, hipStream_t s) {
+    const ModelConfig& m = model_.cfg();
+    const int H = m.hidden, E = m.num_experts, K = m.top_k, Ie = m.expert_intermediate;
+    const int fmt = fmt_code(w.wgu.kind);
+    const int sbf = w.wgu.scale_bf16 ? 1 : 0;
+    PIE_KERNEL(pie_hip_rmsnorm(x_, w.ffn_norm, xn_, N, H, m.rms_eps, s));
+    linear_fused(w.router, xn_, nullptr, m.rms_eps, moe_logits_, N, 0, 0, nullptr, s);
+    PIE_KERNEL(pie_hip_moe_route(moe_logits_, moe_idx_, moe_w_, moe_offsets_, moe_route_token_,
+                                 moe_route_pos_, N, E, K, s));
+    const int hint = std::max(1, std::min(N, 2 * ((N * K + E - 1) / E)));
+    PIE_KERNEL(pie_hip_moe_grouped_gemm(fmt, xn_, moe_route_token_, moe_offsets_, E, hint, w.wgu.data,
+                                        w.wgu.data_bytes() / E, w.wgu.scale, w.wgu.scale_bytes() / E,
+                                        sbf, w.wgu.group, act_, 2 * Ie, H, 1, s));
+    PIE_KERNEL(pie_hip_moe_grouped_gemm(fmt, act_, nullptr, moe_offsets_, E, hint, w.wdown.data,
+                                        w.wdown.data_bytes() / E, w.wdown.scale,
+                                        w.wdown.scale_bytes() / E, sbf, w.wdown.group, moe_y_, H, Ie,
+                                        0, s));
+    PIE_KERNEL(pie_hip_moe_combine(moe_y_, moe_route_pos_, moe_w_, x_, N, K, H, 1, s));
+}
+
 void Executor::body(int N, int S, int max_kv_len) {
     const Inputs in_ = input_layout(N, S);
     const ModelConfig& m = model_.cfg();
@@ -200,8 +242,6 @@ void Executor::body(int N, int S, int max_kv_len) {
     const auto* sample_rows = reinterpret_cast<const uint32_t*>(in_dev_ + in_.off_sample_rows);
     const auto* pages = reinterpret_cast<const uint32_t*>(in_dev_ + in_.off_pages);
 
-    if (model_.is_moe()) throw std::runtime_error("executor: the MoE block is not wired into the forward body yet");
-
     PIE_KERNEL(pie_hip_embed(tokens, model_.embed, x_, N, H, m.vocab, s));
     PIE_KERNEL(pie_hip_rope_table(positions, model_.inv_freq, rope_tab_, N, d, s));
     for (int l = 0; l < m.layers; ++l) {
@@ -214,6 +254,10 @@ void Executor::body(int N, int S, int max_kv_len) {
                                            row_begin, row_len, N, hq, hk, d, page_size_, -1.f,
                                            max_kv_len, attn_ws_, attn_ws_bytes_, s));
         linear_fused(w.wo, attn_, nullptr, m.rms_eps, x_, N, 1, 0, xn_, s);
+        if (model_.is_moe()) {
+            moe_block(w, N, s);
+            continue;
+        }
         linear_fused(w.wgu, x_, w.ffn_norm, m.rms_eps, act_, N, 0, 1, xn_, s);
         linear_fused(w.wdown, act_, nullptr, m.rms_eps, x_, N, 1, 0, xn_, s);
     }

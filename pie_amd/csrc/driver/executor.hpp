@@ -63,6 +63,7 @@ class Executor {
 
   private:
     void body(int N, int S, int max_kv_len);
+    void moe_block(const LayerWeights& w, int N, hipStream_t s);
     void alloc_kv();
 
     DriverConfig cfg_;
@@ -74,6 +75,11 @@ class Executor {
     // activations
     uint16_t *x_ = nullptr, *xn_ = nullptr, *qkv_ = nullptr, *q_ = nullptr, *attn_ = nullptr;
     uint16_t *gu_ = nullptr, *act_ = nullptr, *xs_ = nullptr, *logits_ = nullptr;
+    // MoE: per-route outputs, router logits, routing tables (see moe_block)
+    uint16_t *moe_y_ = nullptr, *moe_logits_ = nullptr;
+    int32_t *moe_idx_ = nullptr, *moe_offsets_ = nullptr, *moe_route_token_ = nullptr,
+            *moe_route_pos_ = nullptr;
+    float* moe_w_ = nullptr;
     float* rope_tab_ = nullptr;
     uint32_t* out_tokens_ = nullptr;
     void* attn_ws_ = nullptr;

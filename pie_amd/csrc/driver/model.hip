@@ -47,16 +47,18 @@ void fill_normal(uint16_t* dst, size_t n, uint64_t seed, float mean, float std,
     PIE_HIP_CHECK(hipGetLastError());
 }
 
-// dst row 2i = src row i (gate_i), dst row 2i+1 = src row half + i (up_i); rows of
-// row_bytes bytes (always even), moved two bytes at a time — a load-time kernel.
+// Inside every block of 2*half rows: dst row 2i = src row i (gate_i), dst row 2i+1 = src row
+// half + i (up_i); rows of row_bytes bytes (always even), moved two bytes at a time — a
+// load-time kernel.  One block for a dense FFN, one block per expert for stacked MoE experts.
 __global__ void interleave_rows_kernel(const unsigned char* __restrict__ src,
                                        unsigned char* __restrict__ dst, size_t half,
-                                       size_t row_bytes) {
-    const size_t total = 2 * half * row_bytes;
+                                       size_t row_bytes, size_t rows_total) {
+    const size_t total = rows_total * row_bytes;
     for (size_t b = (blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x) * 2; b < total;
          b += static_cast<size_t>(gridDim.x) * blockDim.x * 2) {
-        const size_t drow = b / row_bytes, off = b - drow * row_bytes;
-        const size_t srow = (drow & 1) ? half + (drow >> 1) : (drow >> 1);
+        const size_t grow = b / row_bytes, off = b - grow * row_bytes;
+        const size_t blk = grow / (2 * half), drow = grow - blk * 2 * half;
+        const size_t srow = blk * 2 * half + ((drow & 1) ? half + (drow >> 1) : (drow >> 1));
         *reinterpret_cast<uint16_t*>(dst + b) =
             *reinterpret_cast<const uint16_t*>(src + srow * row_bytes + off);
     }
@@ -161,8 +163,8 @@ void Model::make_linear(Linear& lin, int N, int K, const std::string& name, std:
 // (gate_0, up_0, gate_1, up_1, ...), the row order the SwiGLU epilogue of the fused projection
 // kernel pairs up.  A pure row permutation of the canonical [N, K] layout: data and scales move
 // together, no value changes.
-void Model::interleave_gate_up(Linear& lin, hipStream_t stream) {
-    const size_t half = static_cast<size_t>(lin.N) / 2;
+void Model::interleave_gate_up(Linear& lin, int blocks, hipStream_t stream) {
+    const size_t half = static_cast<size_t>(lin.N) / blocks / 2;
     auto permute = [&](void* buf, size_t bytes) {
         if (!buf || bytes == 0) return;
         const size_t row_bytes = bytes / lin.N;
@@ -170,7 +172,7 @@ void Model::interleave_gate_up(Linear& lin, hipStream_t stream) {
         PIE_HIP_CHECK(hipMalloc(&tmp, bytes));
         hipLaunchKernelGGL(interleave_rows_kernel, dim3(2048), dim3(256), 0, stream,
                            static_cast<const unsigned char*>(buf), static_cast<unsigned char*>(tmp),
-                           half, row_bytes);
+                           half, row_bytes, static_cast<size_t>(lin.N));
         PIE_HIP_CHECK(hipGetLastError());
         PIE_HIP_CHECK(hipMemcpyAsync(buf, tmp, bytes, hipMemcpyDeviceToDevice, stream));
         PIE_HIP_CHECK(hipStreamSynchronize(stream));
@@ -191,7 +193,7 @@ void Model::init_synthetic(const ModelConfig& cfg, hipStream_t stream) {
         throw std::runtime_error("model: hidden/intermediate must be multiples of 32, head_dim and vocab of 8");
 
     size_t biggest = static_cast<size_t>((hq + 2 * hk) * d) * H;
-    biggest = std::max(biggest, static_cast<size_t>(2 * I) * H);
+    biggest = std::max(biggest, static_cast<size_t>(2 * I) * H * (moe ? cfg.num_experts : 1));
     biggest = std::max(biggest, static_cast<size_t>(H) * hq * d);
     tmp_elems_ = biggest;
     PIE_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&tmp_bf16_), biggest * 2));
@@ -235,20 +237,22 @@ void Model::init_synthetic(const ModelConfig& cfg, hipStream_t stream) {
         make_linear(w.wo, H, hq * d, p + "wo", next_seed(), stream);
         if (!moe) {
             make_linear(w.wgu, 2 * I, H, p + "wgu", next_seed(), stream);
-            interleave_gate_up(w.wgu, stream);
+            interleave_gate_up(w.wgu, 1, stream);
             make_linear(w.wdown, H, I, p + "wdown", next_seed(), stream);
         } else {
+            // experts stacked along the rows: wgu [E * 2I, H] (gate/up interleaved inside each
+            // expert), wdown [E * H, I]; row / group scales make the stacking exact
             const int E = cfg.num_experts;
-            w.router = static_cast<uint16_t*>(alloc(static_cast<size_t>(E) * H * 2, p + "router"));
-            fill_normal(w.router, static_cast<size_t>(E) * H, next_seed(), 0.f, cfg.init_std, stream);
+            w.router.kind = Quant::Bf16;
+            w.router.N = E;
+            w.router.K = H;
+            w.router.data = alloc(static_cast<size_t>(E) * H * 2, p + "router");
+            fill_normal(static_cast<uint16_t*>(w.router.data), static_cast<size_t>(E) * H, next_seed(), 0.f,
+                        cfg.router_std > 0.f ? cfg.router_std : cfg.init_std, stream);
             const size_t before = decode_bytes_;
-            w.e_wgu.resize(E);
-            w.e_wdown.resize(E);
-            for (int e = 0; e < E; ++e) {
-                const std::string pe = p + "experts." + std::to_string(e) + ".";
-                make_linear(w.e_wgu[e], 2 * I, H, pe + "wgu", next_seed(), stream);
-                make_linear(w.e_wdown[e], H, I, pe + "wdown", next_seed(), stream);
-            }
+            make_linear(w.wgu, E * 2 * I, H, p + "wgu", next_seed(), stream);
+            interleave_gate_up(w.wgu, E, stream);
+            make_linear(w.wdown, E * H, I, p + "wdown", next_seed(), stream);
             // a batch-1 decode step touches top_k of the E experts
             const size_t all = decode_bytes_ - before;
             decode_bytes_ = before + all / E * cfg.top_k + static_cast<size_t>(E) * H * 2;

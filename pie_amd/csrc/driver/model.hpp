@@ -6,7 +6,8 @@
 //   per-group scales make the fusion exact), optional q_norm/k_norm [d], wo [H, hq*d],
 //   ffn_norm [H], then either wgu [2I, H] (rows interleaved gate_0, up_0, gate_1, ... for the
 //   fused SwiGLU epilogue) + wdown [H, I], or the
-//   MoE block: router [E, H] bf16, per-expert wgu [E][2Ie, H] and wdown [E][H, Ie].
+//   MoE block: router [E, H] bf16, experts stacked along the rows — wgu [E * 2Ie, H] (gate/up
+//   interleaved inside each expert) and wdown [E * H, Ie].
 // embed [V, H] bf16, final_norm [H], lm_head [V, H] bf16 (aliases embed when tied); those
 // three stay unquantised like the reference (driver/cuda/src/config.hpp:20-30).
 #pragma once
@@ -52,10 +53,8 @@ struct LayerWeights {
     uint16_t* ffn_norm = nullptr;
     uint16_t* q_norm = nullptr;
     uint16_t* k_norm = nullptr;
-    Linear wqkv, wo, wgu, wdown;
-    // MoE
-    uint16_t* router = nullptr;     // [E, H] bf16
-    std::vector<Linear> e_wgu, e_wdown;
+    Linear wqkv, wo, wgu, wdown;  // MoE: wgu / wdown hold the experts stacked along the rows
+    Linear router;                // MoE: [E, H] bf16
 };
 
 struct TensorRef {
@@ -93,7 +92,7 @@ class Model {
     void* alloc(size_t bytes, const std::string& name);
     void make_linear(Linear& lin, int N, int K, const std::string& name, std::uint64_t seed,
                      hipStream_t stream);
-    void interleave_gate_up(Linear& lin, hipStream_t stream);
+    void interleave_gate_up(Linear& lin, int blocks, hipStream_t stream);
     ModelConfig cfg_;
     Quant quant_ = Quant::Bf16;
     std::vector<void*> allocs_;

@@ -1,0 +1,203 @@
+// MoE routing and combine for gfx950.
+//
+//   pie_hip_moe_route: per token softmax over the router logits, top-k by repeated argmax with
+//   exclusion (lowest expert index wins ties), renormalised weights — the arithmetic of
+//   topk_softmax_bf16_kernel (driver/cuda/src/kernels/topk_softmax.cu:19-86; graph form
+//   driver/portable/src/graph_common.cpp:262-283) — and, in the same launch, the grouped layout
+//   the expert GEMM consumes: routes counting-sorted by expert (offsets per expert, the token of
+//   each sorted route, the sorted position of each (token, k) route).  The reference instead
+//   launches one GEMV per route (driver/cuda/src/model/kimi_forward.cpp:662-714).
+//
+//   pie_hip_moe_combine: out[t] (+)= sum_k w[t, k] * y_route[pos[t, k]] in top-k order, fp32,
+//   one rounding (token_batched_weighted_sum[_add]_bf16_kernel,
+//   driver/cuda/src/kernels/moe_dispatch.cu:152-196).
+#include "common.hip.h"
+
+namespace pie_hip {
+namespace {
+
+constexpr int kRouteThreads = 1024;
+constexpr int kMaxExperts = 512;   // the reference's MAX_EXPERTS (topk_softmax.cu:14)
+constexpr int kMaxTopK = 16;       // the reference's combine unroll bound (moe_dispatch.cu:128)
+constexpr int kPerLane = kMaxExperts / kWave;
+
+// (value, index) max with ties to the lower index, across the wave.
+__device__ __forceinline__ void wave_argmax(float& v, int& i) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(v, off, kWave);
+        const int oi = __shfl_xor(i, off, kWave);
+        if (ov > v || (ov == v && oi < i)) {
+            v = ov;
+            i = oi;
+        }
+    }
+}
+
+__global__ __launch_bounds__(kRouteThreads) void moe_route_kernel(
+    const uint16_t* __restrict__ logits, int32_t* __restrict__ topk_idx,
+    float* __restrict__ topk_w, int32_t* __restrict__ expert_offsets,
+    int32_t* __restrict__ route_token, int32_t* __restrict__ route_pos, int N, int E, int K) {
+    __shared__ int cnt[kMaxExperts];
+    __shared__ int base[kMaxExperts + 1];
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wv = tid / kWave;
+    for (int e = tid; e < E; e += kRouteThreads) cnt[e] = 0;
+
+    // ---- phase 1: one wave per token: softmax, top-k, renormalise ----
+    for (int t = wv; t < N; t += kRouteThreads / kWave) {
+        const uint16_t* row = logits + static_cast<size_t>(t) * E;
+        float p[kPerLane];
+        float mx = -3.4e38f;
+#pragma unroll
+        for (int j = 0; j < kPerLane; ++j) {
+            const int e = lane + kWave * j;
+            p[j] = e < E ? bf16_bits_to_f32(row[e]) : -3.4e38f;
+            mx = fmaxf(mx, p[j]);
+        }
+        mx = wave_max(mx);
+        float sum = 0.f;
+#pragma unroll
+        for (int j = 0; j < kPerLane; ++j) {
+            const int e = lane + kWave * j;
+            p[j] = e < E ? expf(p[j] - mx) : 0.f;
+            sum += p[j];
+        }
+        sum = wave_sum(sum);
+        const float inv_z = 1.f / sum;
+#pragma unroll
+        for (int j = 0; j < kPerLane; ++j) p[j] = (lane + kWave * j < E) ? p[j] * inv_z : -2.f;
+        float w_sum = 0.f, my_w = 0.f;   // lane k keeps the k-th weight
+        int my_e = 0;
+        for (int k = 0; k < K; ++k) {
+            float bv = -1.f;
+            int bi = kMaxExperts;
+#pragma unroll
+            for (int j = 0; j < kPerLane; ++j)
+                if (p[j] > bv) {
+                    bv = p[j];
+                    bi = lane + kWave * j;
+                }
+            wave_argmax(bv, bi);
+            bi = min(bi, E - 1);   // only reachable with NaN logits; keeps every index in range
+#pragma unroll
+            for (int j = 0; j < kPerLane; ++j)
+                if (bi == lane + kWave * j) p[j] = -1.f;   // exclude on the next pass
+            w_sum += bv;
+            if (lane == k) {
+                my_w = bv;
+                my_e = bi;
+            }
+        }
+        const float inv_w = 1.f / w_sum;
+        if (lane < K) {
+            topk_idx[static_cast<size_t>(t) * K + lane] = my_e;
+            topk_w[static_cast<size_t>(t) * K + lane] = my_w * inv_w;
+        }
+    }
+    __syncthreads();
+
+    // ---- phase 2: rank of every route inside its expert, expert offsets ----
+    const int R = N * K;
+    for (int r = tid; r < R; r += kRouteThreads) route_pos[r] = atomicAdd(&cnt[topk_idx[r]], 1);
+    __syncthreads();
+    if (wv == 0) {
+        // exclusive scan of cnt[0..E): each lane owns a run of consecutive experts
+        const int per = (E + kWave - 1) / kWave;
+        int run = 0;
+        for (int i = 0; i < per; ++i) {
+            const int e = lane * per + i;
+            if (e < E) run += cnt[e];
+        }
+        int incl = run;
+#pragma unroll
+        for (int off = 1; off < kWave; off <<= 1) {
+            const int o = __shfl_up(incl, off, kWave);
+            if (lane >= off) incl += o;
+        }
+        int acc = incl - run;
+        for (int i = 0; i < per; ++i) {
+            const int e = lane * per + i;
+            if (e < E) {
+                base[e] = acc;
+                acc += cnt[e];
+            }
+        }
+        if (lane == kWave - 1) base[E] = incl;
+    }
+    __syncthreads();
+    for (int e = tid; e <= E; e += kRouteThreads) expert_offsets[e] = base[e];
+    for (int r = tid; r < R; r += kRouteThreads) {
+        const int pos = base[topk_idx[r]] + route_pos[r];
+        route_pos[r] = pos;
+        route_token[pos] = r / K;
+    }
+}
+
+__global__ __launch_bounds__(256) void moe_combine_kernel(
+    const uint16_t* __restrict__ y_routes, const int32_t* __restrict__ route_pos,
+    const float* __restrict__ topk_w, uint16_t* __restrict__ out, int K, int H, int add) {
+    const int t = blockIdx.y;
+    const int h = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
+    if (h >= H) return;
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int k = 0; k < K; ++k) {
+        const int pos = route_pos[static_cast<size_t>(t) * K + k];
+        const float w = topk_w[static_cast<size_t>(t) * K + k];
+        const u32x4_t v = *reinterpret_cast<const u32x4_t*>(y_routes + static_cast<size_t>(pos) * H + h);
+        acc[0] = fmaf(w, bf16_lo(v.x), acc[0]);
+        acc[1] = fmaf(w, bf16_hi(v.x), acc[1]);
+        acc[2] = fmaf(w, bf16_lo(v.y), acc[2]);
+        acc[3] = fmaf(w, bf16_hi(v.y), acc[3]);
+        acc[4] = fmaf(w, bf16_lo(v.z), acc[4]);
+        acc[5] = fmaf(w, bf16_hi(v.z), acc[5]);
+        acc[6] = fmaf(w, bf16_lo(v.w), acc[6]);
+        acc[7] = fmaf(w, bf16_hi(v.w), acc[7]);
+    }
+    u32x4_t* o = reinterpret_cast<u32x4_t*>(out + static_cast<size_t>(t) * H + h);
+    if (add) {
+        const u32x4_t p = *o;
+        acc[0] += bf16_lo(p.x);
+        acc[1] += bf16_hi(p.x);
+        acc[2] += bf16_lo(p.y);
+        acc[3] += bf16_hi(p.y);
+        acc[4] += bf16_lo(p.z);
+        acc[5] += bf16_hi(p.z);
+        acc[6] += bf16_lo(p.w);
+        acc[7] += bf16_hi(p.w);
+    }
+    *o = u32x4_t{pack_bf16x2(acc[0], acc[1]), pack_bf16x2(acc[2], acc[3]),
+                 pack_bf16x2(acc[4], acc[5]), pack_bf16x2(acc[6], acc[7])};
+}
+
+}  // namespace
+}  // namespace pie_hip
+
+extern "C" int pie_hip_moe_route(const uint16_t* router_logits_bf16, int32_t* topk_idx,
+                                 float* topk_weight, int32_t* expert_offsets,
+                                 int32_t* route_token, int32_t* route_pos, int num_tokens,
+                                 int num_experts, int top_k, void* stream) {
+    using namespace pie_hip;
+    if (!router_logits_bf16 || !topk_idx || !topk_weight || !expert_offsets || !route_token ||
+        !route_pos || num_tokens <= 0)
+        return PIE_HIP_ERR_INVALID;
+    if (num_experts <= 0 || num_experts > kMaxExperts || top_k <= 0 || top_k > kMaxTopK ||
+        top_k > num_experts)
+        return PIE_HIP_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(kRouteThreads), 0,
+                       static_cast<hipStream_t>(stream), router_logits_bf16, topk_idx, topk_weight,
+                       expert_offsets, route_token, route_pos, num_tokens, num_experts, top_k);
+    return launch_status();
+}
+
+extern "C" int pie_hip_moe_combine(const uint16_t* y_routes_bf16, const int32_t* route_pos,
+                                   const float* topk_weight, uint16_t* out_bf16, int num_tokens,
+                                   int top_k, int hidden, int add, void* stream) {
+    using namespace pie_hip;
+    if (!y_routes_bf16 || !route_pos || !topk_weight || !out_bf16 || num_tokens <= 0)
+        return PIE_HIP_ERR_INVALID;
+    if (hidden <= 0 || hidden % 8 != 0 || top_k <= 0 || top_k > kMaxTopK) return PIE_HIP_ERR_UNSUPPORTED;
+    const dim3 grid((hidden / 8 + 255) / 256, num_tokens);
+    hipLaunchKernelGGL(moe_combine_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream),
+                       y_routes_bf16, route_pos, topk_weight, out_bf16, top_k, hidden, add ? 1 : 0);
+    return launch_status();
+}

@@ -426,3 +426,37 @@ def moe_grouped_gemm(act: torch.Tensor, route_act_rows: Optional[torch.Tensor],
         group_size, _ptr(y), N, K, int(swiglu), _stream())
     _check(st, "pie_hip_moe_grouped_gemm")
     return y
+
+
+def moe_route(router_logits: torch.Tensor, top_k: int):
+    """Softmax -> top-k -> renormalise per token, plus the expert-sorted route layout.
+    Returns (topk_idx [T,k] int32, topk_w [T,k] f32, expert_offsets [E+1] int32,
+    route_token [T*k] int32, route_pos [T*k] int32)."""
+    _dev(router_logits, torch.bfloat16, "router_logits")
+    T, E = router_logits.shape
+    d = router_logits.device
+    idx = torch.empty((T, top_k), dtype=torch.int32, device=d)
+    w = torch.empty((T, top_k), dtype=torch.float32, device=d)
+    offs = torch.empty(E + 1, dtype=torch.int32, device=d)
+    rtok = torch.empty(T * top_k, dtype=torch.int32, device=d)
+    rpos = torch.empty(T * top_k, dtype=torch.int32, device=d)
+    _check(kernels().pie_hip_moe_route(_ptr(router_logits), _ptr(idx), _ptr(w), _ptr(offs), _ptr(rtok),
+                                       _ptr(rpos), T, E, top_k, _stream()), "pie_hip_moe_route")
+    return idx, w, offs, rtok, rpos
+
+
+def moe_combine(y_routes: torch.Tensor, route_pos: torch.Tensor, topk_w: torch.Tensor,
+                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[t] (+)= sum_k w[t,k] * y_routes[route_pos[t,k]]; `out` given = accumulate onto it."""
+    _dev(y_routes, torch.bfloat16, "y_routes")
+    _dev(route_pos, torch.int32, "route_pos")
+    _dev(topk_w, torch.float32, "topk_w")
+    T, K = topk_w.shape
+    H = y_routes.shape[1]
+    add = out is not None
+    if out is None:
+        out = torch.empty((T, H), dtype=torch.bfloat16, device=y_routes.device)
+    _dev(out, torch.bfloat16, "out")
+    _check(kernels().pie_hip_moe_combine(_ptr(y_routes), _ptr(route_pos), _ptr(topk_w), _ptr(out), T, K,
+                                         H, int(add), _stream()), "pie_hip_moe_combine")
+    return out

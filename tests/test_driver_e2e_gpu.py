@@ -69,6 +69,12 @@ def check_step(oracle, gpu_logit_bits, orc_logit_bits, gpu_tok, orc_tok):
     dict(arch="qwen3", quant="int4b8", head_dim=128, q_heads=4, kv_heads=1, rope_theta=1e6),
     dict(quant="int4b8", head_dim=128, q_heads=8, kv_heads=2, hidden=1024, rope_factor=8.0),
     dict(quant="int4b8", page_size=32, use_graphs=False),
+    dict(arch="qwen3_moe", quant="fp8", head_dim=128, q_heads=4, kv_heads=1, num_experts=8, top_k=2,
+         expert_intermediate=256, router_std=0.2, intermediate=0),
+    dict(arch="qwen3_moe", quant="int4b8", head_dim=128, q_heads=4, kv_heads=1, num_experts=16,
+         top_k=4, expert_intermediate=512, router_std=0.2, intermediate=0),
+    dict(arch="qwen3_moe", quant="bf16", head_dim=64, q_heads=8, kv_heads=2, num_experts=6, top_k=3,
+         expert_intermediate=128, router_std=0.2, intermediate=0, use_graphs=False),
 ], ids=lambda k: "-".join(f"{a}={b}" for a, b in k.items()))
 def test_greedy_generation_matches_oracle(gpu, oracle, kw):
     from pie_amd import driver as drvmod

@@ -21,8 +21,13 @@ def make_tensors(oracle, rng, cfg):
         if cfg["qk_norm"]:
             t[p + "q_norm"] = bf(rng.uniform(0.8, 1.2, d))
             t[p + "k_norm"] = bf(rng.uniform(0.8, 1.2, d))
-        for name, (n, k) in dict(wqkv=((hq + 2 * hk) * d, H), wo=(H, hq * d), wgu=(2 * I, H),
-                                 wdown=(H, I)).items():
+        E, Ie = cfg.get("num_experts", 0), cfg.get("expert_intermediate", 0)
+        shapes = dict(wqkv=((hq + 2 * hk) * d, H), wo=(H, hq * d), wgu=(2 * I, H), wdown=(H, I))
+        if E:
+            # experts stacked along the rows: per expert gate rows then up rows / down rows
+            t[p + "router"] = bf(rng.standard_normal((E, H)) * (4.0 / np.sqrt(H)))
+            shapes.update(wgu=(E * 2 * Ie, H), wdown=(E * H, Ie))
+        for name, (n, k) in shapes.items():
             w = bf(rng.standard_normal((n, k)) * (0.7 / np.sqrt(k)))
             if cfg["quant"] == "bf16":
                 t[p + name + ".data"] = w
@@ -101,10 +106,34 @@ class DenseRef:
                 out[h] = (w / w.sum()) @ V[:, kv]
             x = x + dequant(self.o, cfg, self.t, p + "wo", H, hq * d) @ out.reshape(-1)
             xn = self.norm(x, self.f(p + "ffn_norm"))
+            E = cfg.get("num_experts", 0)
+            if E:
+                x = x + self.moe(p, xn)
+                continue
             gu = dequant(self.o, cfg, self.t, p + "wgu", 2 * I, H) @ xn
             g, u = gu[:I], gu[I:]
             x = x + dequant(self.o, cfg, self.t, p + "wdown", H, I) @ (g / (1 + np.exp(-g)) * u)
         return self.f("lm_head") @ self.norm(x, self.f("final_norm"))
+
+    def moe(self, p, xn):
+        """softmax router -> top-k (ties to the lowest index) -> renormalise -> weighted sum of
+        the selected experts' SwiGLU FFNs (driver/portable/src/graph_common.cpp:237-345)."""
+        cfg = self.cfg
+        H, E, K, Ie = cfg["hidden"], cfg["num_experts"], cfg["top_k"], cfg["expert_intermediate"]
+        logits = self.f(p + "router") @ xn
+        pr = np.exp(logits - logits.max())
+        pr /= pr.sum()
+        sel = np.argsort(-pr, kind="stable")[:K]
+        self.min_gap = min(getattr(self, "min_gap", 1.0), float(pr[sel[-1]] - np.sort(pr)[-K - 1]))
+        w = pr[sel] / pr[sel].sum()
+        wgu = dequant(self.o, cfg, self.t, p + "wgu", E * 2 * Ie, H).reshape(E, 2 * Ie, H)
+        wdn = dequant(self.o, cfg, self.t, p + "wdown", E * H, Ie).reshape(E, H, Ie)
+        out = np.zeros(H)
+        for e, we in zip(sel, w):
+            gu = wgu[e] @ xn
+            g, u = gu[:Ie], gu[Ie:]
+            out += we * (wdn[e] @ (g / (1 + np.exp(-g)) * u))
+        return out
 
 
 @pytest.mark.parametrize("quant,qk_norm,interleaved", [("bf16", False, 1), ("int8", False, 1),
