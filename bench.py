@@ -39,11 +39,29 @@ HBM_PEAK_GBPS = 8000.0
 MODEL = dict(arch="llama3", hidden=4096, layers=32, q_heads=32, kv_heads=8, head_dim=128,
              intermediate=14336, vocab=128256, rope_theta=500000.0, quant="int4b8", group_size=128)
 
+# Other BASELINE configurations, selectable with --model (no roofline / CPU leg on these lines):
+# configs[0] Llama-3.2-1B-shaped int8 per-channel, configs[4] Qwen3-30B-A3B-shaped fp8 MoE.
+OTHER_MODELS = {
+    "llama1b-int8": (dict(arch="llama3", hidden=2048, layers=16, q_heads=32, kv_heads=8, head_dim=64,
+                          intermediate=8192, vocab=128256, rope_theta=500000.0, quant="int8",
+                          scale_dtype="bf16", tie_embeddings=True),
+                     "Llama-3.2-1B-shaped W8A16 (int8 per-channel, bf16 scales) greedy decode"),
+    "qwen3-30b-a3b-fp8": (dict(arch="qwen3_moe", hidden=2048, layers=48, q_heads=32, kv_heads=4,
+                               head_dim=128, intermediate=0, vocab=151936, rope_theta=1000000.0,
+                               quant="fp8", scale_dtype="bf16", num_experts=128, top_k=8,
+                               expert_intermediate=768, router_std=0.0221),
+                          "Qwen3-30B-A3B-shaped MoE (128 experts, top-8, fp8 e4m3 experts with bf16 "
+                          "row scales) greedy decode"),
+}
+
 
 def toml(model: dict, page_size: int, total_pages: int, max_tokens: int, max_requests: int) -> str:
     lines = ["[model]"]
     for k, v in model.items():
-        lines.append(f'{k} = "{v}"' if isinstance(v, str) else f"{k} = {v}")
+        if isinstance(v, bool):
+            lines.append(f"{k} = {'true' if v else 'false'}")
+        else:
+            lines.append(f'{k} = "{v}"' if isinstance(v, str) else f"{k} = {v}")
     lines += ["[batching]", f"kv_page_size = {page_size}", f"total_pages = {total_pages}",
               f"max_forward_tokens = {max_tokens}", f"max_forward_requests = {max_requests}",
               "[runtime]", "use_graphs = true"]
@@ -255,6 +273,7 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-extra", action="store_true")
+    ap.add_argument("--model", default="llama8b-w4a16", choices=["llama8b-w4a16", *OTHER_MODELS])
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this driver path is built and measured on one GPU; "
@@ -272,10 +291,11 @@ def main():
     max_new = args.warmup + args.steps + 1
     pages_per_ctx = (args.prompt + max_new + page_size - 1) // page_size
     total_pages = pages_per_ctx * args.batch + 8
-    cfg_text = toml(MODEL, page_size, total_pages, 512, max(16, args.batch))
+    model, label = (MODEL, None) if args.model == "llama8b-w4a16" else OTHER_MODELS[args.model]
+    cfg_text = toml(model, page_size, total_pages, 512, max(16, args.batch))
     hip = Hip()
     rng = np.random.default_rng(2048)
-    prompt = rng.integers(0, MODEL["vocab"], args.prompt)
+    prompt = rng.integers(0, model["vocab"], args.prompt)
 
     t0 = time.perf_counter()
     drv = drvmod.Driver(cfg_text)
@@ -287,6 +307,21 @@ def main():
     assert steps == args.steps, (steps, args.steps)
     wall_s = tm["decode_wall_us"] * 1e-6
     value = args.batch * steps / wall_s
+    if label is not None:
+        drv.close()
+        print(json.dumps({
+            "metric": "decode tokens/sec @1 GPU + quant-GEMV/attention HBM GB/s as % of 8 TB/s",
+            "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": steps,
+            "warmup": args.warmup, "ms_per_step": round(wall_s / steps * 1e3, 4),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+            "data": "synthetic",
+            "config": {"workload": f"{label}, batch {args.batch}, after a {args.prompt}-token "
+                                   "prefill, page size 16", "batch": args.batch,
+                       "prompt_tokens": args.prompt, "page_size": page_size},
+            "roofline": None, "cpu_baseline": None,
+            "extra": {"init_s": round(t_init, 2), "prefill_s": round(tm["prefill_us"] * 1e-6, 3),
+                      "decode_device_ms_per_step": round(tm["decode_device_us"] * 1e-3 / steps, 4)}}))
+        return
 
     roof = gemv_roofline(drv, hip, MODEL, reps=2)
     extra = {"gemv_w4a16_shapes": roof["detail"], "init_s": round(t_init, 2),

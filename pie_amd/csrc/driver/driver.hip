@@ -377,9 +377,10 @@ extern "C" int pie_hip_driver_generate(PieHipDriver* d, const uint32_t* prompt, 
         std::vector<uint32_t> last(replicate);
         const int chunk_cap = d->cfg.batching.max_forward_tokens;
         const auto t_prefill = clk::now();
-        // Prefill: one plan per context (contiguous page range), chunked to the token cap;
-        // only the final chunk samples.
-        for (int c = 0; c < replicate; ++c) {
+        // Prefill: context 0 runs the prompt (contiguous page range), chunked to the token cap,
+        // only the final chunk samples; the other contexts hold the same prompt, so their pages
+        // are device-to-device copies of context 0's (the fork-by-copy path of Copy{D2D}).
+        for (int c = 0; c < 1; ++c) {
             for (int t0 = 0; t0 < n_prompt; t0 += chunk_cap) {
                 const int n = std::min(chunk_cap, n_prompt - t0);
                 const int upto = t0 + n;  // tokens in the context after this chunk
@@ -412,6 +413,20 @@ extern "C" int pie_hip_driver_generate(PieHipDriver* d, const uint32_t* prompt, 
                     last[c] = fr.tokens.ptr[0];
                     out_tokens[static_cast<size_t>(c) * max_new] = last[c];
                 }
+            }
+        }
+        if (replicate > 1) {
+            const int np = (n_prompt + ps - 1) / ps;
+            std::vector<uint32_t> srcs, dsts;
+            for (int c = 1; c < replicate; ++c)
+                for (int p = 0; p < np; ++p) {
+                    srcs.push_back(static_cast<uint32_t>(p));
+                    dsts.push_back(static_cast<uint32_t>(c * pages_per_ctx + p));
+                }
+            d->exec->copy_pages_d2d(srcs.data(), dsts.data(), srcs.size());
+            for (int c = 1; c < replicate; ++c) {
+                last[c] = last[0];
+                out_tokens[static_cast<size_t>(c) * max_new] = last[0];
             }
         }
         const double prefill_us = us_since(t_prefill);
