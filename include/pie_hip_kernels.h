@@ -117,6 +117,21 @@ int pie_hip_gemm_skinny(int format, const uint16_t* act_bf16, const void* weight
                         int M, int N, int K, int beta, int swiglu, void* stream);
 
 /*
+ * Tiled weight-only GEMM on the matrix cores for prefill and large batches (compute-bound M):
+ *   y[M, N] = epilogue( act[M, K] · W[N, K]^T ), formats / scales / beta / swiglu as above.
+ * Evaluation order of the reference's large-M paths: the weights become bf16 first — int4b8 as
+ * bf16((nibble-8) * group_scale), the value of launch_dequant_wna16_int4b8_to_bf16
+ * (driver/cuda/src/kernels/dequant_wna16.cu:11-38) followed by a bf16 GEMM
+ * (driver/cuda/src/ops/gemm.cpp:1213-1236); int8 / fp8 values are exact in bf16 and their row
+ * scale multiplies the fp32 sum — then bf16 x bf16 products, fp32 accumulation, one rounding.
+ * 128 x 128 x 64 tiles, v_mfma_f32_16x16x32_bf16.  Requirements: K % 64 == 0; int4b8
+ * group_size a power of two >= 32 dividing K.
+ */
+int pie_hip_gemm_mfma(int format, const uint16_t* act_bf16, const void* weight, const void* scale,
+                      int scale_is_bf16, int group_size, uint16_t* y_bf16, int M, int N, int K,
+                      int beta, int swiglu, void* stream);
+
+/*
  * MoE grouped weight-only GEMM: one skinny problem per expert in a single launch.
  *   rows [expert_offsets[e], expert_offsets[e+1]) of y (routes sorted by expert) are
  *   act[route_act_rows[r]] (or act[r] when route_act_rows is NULL) times expert e's [N,K]

@@ -460,3 +460,26 @@ def moe_combine(y_routes: torch.Tensor, route_pos: torch.Tensor, topk_w: torch.T
     _check(kernels().pie_hip_moe_combine(_ptr(y_routes), _ptr(route_pos), _ptr(topk_w), _ptr(out), T, K,
                                          H, int(add), _stream()), "pie_hip_moe_combine")
     return out
+
+
+def gemm_mfma(act: torch.Tensor, w: WeightView, y: Optional[torch.Tensor] = None, beta: int = 0,
+              swiglu: bool = False) -> torch.Tensor:
+    """Tiled matrix-core GEMM for large M (weights dequantised to bf16 while staged)."""
+    _dev(act, torch.bfloat16, "act")
+    M, K = act.shape
+    if K != w.K:
+        raise KernelError("act K != weight K")
+    n_out = w.N // 2 if swiglu else w.N
+    if y is None:
+        if beta:
+            raise KernelError("beta=1 needs an existing y")
+        y = torch.empty((M, n_out), dtype=torch.bfloat16, device=act.device)
+    _dev(y, torch.bfloat16, "y")
+    if tuple(y.shape) != (M, n_out):
+        raise KernelError("y shape mismatch")
+    scale_is_bf16 = int(w.scale is not None and w.scale.dtype == torch.bfloat16)
+    st = kernels().pie_hip_gemm_mfma(FMT[w.kind], _ptr(act), _ptr(w.data), _ptr(w.scale),
+                                     scale_is_bf16, w.group_size, _ptr(y), M, w.N, K, beta,
+                                     int(swiglu), _stream())
+    _check(st, "pie_hip_gemm_mfma")
+    return y

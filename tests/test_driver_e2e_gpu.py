@@ -98,6 +98,30 @@ def test_greedy_generation_matches_oracle(gpu, oracle, kw):
         assert np.array_equal(gtoks[0], gtoks[1])
 
 
+@pytest.mark.parametrize("quant", ["int4b8", "fp8"])
+def test_long_prefill_through_the_tiled_gemm(gpu, oracle, quant):
+    """A 150-token prompt (two chunks under max_forward_tokens=128: 128 rows through the tiled
+    matrix-core GEMM, 22 through the skinny one), then decode; logits and tokens against the
+    oracle."""
+    from pie_amd import driver as drvmod
+
+    kw = dict(quant=quant, max_forward_tokens=128, total_pages=32)
+    cfg = full_cfg(**kw)
+    rng = np.random.default_rng(93)
+    prompt = rng.integers(0, cfg["vocab"], 150)
+    with drvmod.Driver(toml_config(**kw)) as d:
+        om, _ = oracle_model_from_driver(d, cfg)
+        otoks, otrace = om.generate(prompt, 4, 1, want_logits=True)
+        gtoks, _ = d.generate(prompt, 4, replicate=1)
+        lg = d.export_tensor("debug.logits", np.uint16).reshape(-1, cfg["vocab"])[0]
+        check_step(oracle, lg, otrace[3], gtoks[0, 3], otoks[0, 3]) if np.array_equal(gtoks[0, :3], otoks[0, :3]) else None
+        # the first token comes straight out of the prefill
+        o0 = oracle.bf16_to_f32(otrace[0])
+        top2 = np.sort(o0)[-2:]
+        if top2[1] - top2[0] > 2.0 ** -6 * abs(top2[1]) + 1e-6:
+            assert int(gtoks[0, 0]) == int(otoks[0, 0])
+
+
 def test_mixed_batch_prefill_plus_decode_and_kv_copy(gpu, oracle):
     """A decode request and a chunked prefill in one forward, then a forked context whose
     partially filled tail page is duplicated with Copy D2D."""
