@@ -154,7 +154,7 @@ int pie_hip_moe_grouped_gemm(int format, const uint16_t* act_bf16, const int32_t
  * MoE routing: per token softmax over router_logits[t, 0..E) (bf16 in, fp32 inside), top_k by
  * repeated argmax with exclusion (ties to the lowest expert index), weights renormalised to
  * sum 1 — topk_softmax_bf16_kernel, driver/cuda/src/kernels/topk_softmax.cu:19-86 (graph form:
- * driver/portable/src/graph_common.cpp:262-283).  The same launch builds the grouped layout of
+ * driver/portable/src/graph_common.cpp:262-283).  A second small kernel builds the grouped layout of
  * pie_hip_moe_grouped_gemm: routes (t, k) counting-sorted by expert.
  *   topk_idx [T, top_k] int32, topk_weight [T, top_k] f32 (bit-exact integer outputs given the
  *   probabilities; the order of routes inside one expert is unspecified),

@@ -55,7 +55,7 @@ int fmt_code(Quant q) {
 // gemm_act_x_w (driver/cuda/src/ops/gemm.cpp:1414-1583).  Up to four rows: the weight-streaming
 // GEMV with the norm riding in its activation staging and SwiGLU in its epilogue.  More rows
 // (norm as its own kernel into `norm_tmp`): the matrix-core skinny GEMM, which streams the
-// weights once per 16 rows, and from 49 rows on the tiled matrix-core GEMM; shapes those do
+// weights once per 16 rows, and from 193 rows on the tiled matrix-core GEMM; shapes those do
 // not take fall back to the GEMV path.
 void linear_fused(const Linear& w, const uint16_t* act, const uint16_t* norm_w, float eps,
                   uint16_t* y, int M, int beta, int swiglu, uint16_t* norm_tmp, hipStream_t s) {
@@ -67,8 +67,9 @@ void linear_fused(const Linear& w, const uint16_t* act, const uint16_t* norm_w, 
             PIE_KERNEL(pie_hip_rmsnorm(act, norm_w, norm_tmp, M, w.K, eps, s));
             a = norm_tmp;
         }
-        if (M > 48) {
-            // compute-bound: the tiled GEMM (weights dequantised to bf16 while staged)
+        if (M > 192) {
+            // compute-bound: the tiled GEMM (weights dequantised to bf16 while staged); below
+            // that the 16-row passes of the skinny kernel are still faster
             const int sg = pie_hip_gemm_mfma(fmt, a, w.data, w.scale, sbf, w.group, y, M, w.N, w.K,
                                              beta, swiglu, s);
             if (sg == PIE_HIP_OK) return;

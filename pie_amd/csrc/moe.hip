@@ -3,7 +3,7 @@
 //   pie_hip_moe_route: per token softmax over the router logits, top-k by repeated argmax with
 //   exclusion (lowest expert index wins ties), renormalised weights — the arithmetic of
 //   topk_softmax_bf16_kernel (driver/cuda/src/kernels/topk_softmax.cu:19-86; graph form
-//   driver/portable/src/graph_common.cpp:262-283) — and, in the same launch, the grouped layout
+//   driver/portable/src/graph_common.cpp:262-283) — followed by a one-block kernel that builds the grouped layout
 //   the expert GEMM consumes: routes counting-sorted by expert (offsets per expert, the token of
 //   each sorted route, the sorted position of each (token, k) route).  The reference instead
 //   launches one GEMV per route (driver/cuda/src/model/kimi_forward.cpp:662-714).
@@ -34,69 +34,72 @@ __device__ __forceinline__ void wave_argmax(float& v, int& i) {
     }
 }
 
-__global__ __launch_bounds__(kRouteThreads) void moe_route_kernel(
-    const uint16_t* __restrict__ logits, int32_t* __restrict__ topk_idx,
-    float* __restrict__ topk_w, int32_t* __restrict__ expert_offsets,
+// One wave per token: softmax over the experts, top-k with exclusion, renormalise.
+__global__ __launch_bounds__(256) void moe_topk_kernel(const uint16_t* __restrict__ logits,
+                                                       int32_t* __restrict__ topk_idx,
+                                                       float* __restrict__ topk_w, int N, int E, int K) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int t = blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+    if (t >= N) return;
+    const uint16_t* row = logits + static_cast<size_t>(t) * E;
+    float p[kPerLane];
+    float mx = -3.4e38f;
+#pragma unroll
+    for (int j = 0; j < kPerLane; ++j) {
+        const int e = lane + kWave * j;
+        p[j] = e < E ? bf16_bits_to_f32(row[e]) : -3.4e38f;
+        mx = fmaxf(mx, p[j]);
+    }
+    mx = wave_max(mx);
+    float sum = 0.f;
+#pragma unroll
+    for (int j = 0; j < kPerLane; ++j) {
+        const int e = lane + kWave * j;
+        p[j] = e < E ? expf(p[j] - mx) : 0.f;
+        sum += p[j];
+    }
+    sum = wave_sum(sum);
+    const float inv_z = 1.f / sum;
+#pragma unroll
+    for (int j = 0; j < kPerLane; ++j) p[j] = (lane + kWave * j < E) ? p[j] * inv_z : -2.f;
+    float w_sum = 0.f, my_w = 0.f;   // lane k keeps the k-th weight
+    int my_e = 0;
+    for (int k = 0; k < K; ++k) {
+        float bv = -1.f;
+        int bi = kMaxExperts;
+#pragma unroll
+        for (int j = 0; j < kPerLane; ++j)
+            if (p[j] > bv) {
+                bv = p[j];
+                bi = lane + kWave * j;
+            }
+        wave_argmax(bv, bi);
+        bi = min(bi, E - 1);   // only reachable with NaN logits; keeps every index in range
+#pragma unroll
+        for (int j = 0; j < kPerLane; ++j)
+            if (bi == lane + kWave * j) p[j] = -1.f;   // exclude on the next pass
+        w_sum += bv;
+        if (lane == k) {
+            my_w = bv;
+            my_e = bi;
+        }
+    }
+    const float inv_w = 1.f / w_sum;
+    if (lane < K) {
+        topk_idx[static_cast<size_t>(t) * K + lane] = my_e;
+        topk_w[static_cast<size_t>(t) * K + lane] = my_w * inv_w;
+    }
+}
+
+// One block: rank of every route inside its expert, expert offsets, sorted positions.
+__global__ __launch_bounds__(kRouteThreads) void moe_sort_kernel(
+    const int32_t* __restrict__ topk_idx, int32_t* __restrict__ expert_offsets,
     int32_t* __restrict__ route_token, int32_t* __restrict__ route_pos, int N, int E, int K) {
     __shared__ int cnt[kMaxExperts];
     __shared__ int base[kMaxExperts + 1];
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wv = tid / kWave;
     for (int e = tid; e < E; e += kRouteThreads) cnt[e] = 0;
-
-    // ---- phase 1: one wave per token: softmax, top-k, renormalise ----
-    for (int t = wv; t < N; t += kRouteThreads / kWave) {
-        const uint16_t* row = logits + static_cast<size_t>(t) * E;
-        float p[kPerLane];
-        float mx = -3.4e38f;
-#pragma unroll
-        for (int j = 0; j < kPerLane; ++j) {
-            const int e = lane + kWave * j;
-            p[j] = e < E ? bf16_bits_to_f32(row[e]) : -3.4e38f;
-            mx = fmaxf(mx, p[j]);
-        }
-        mx = wave_max(mx);
-        float sum = 0.f;
-#pragma unroll
-        for (int j = 0; j < kPerLane; ++j) {
-            const int e = lane + kWave * j;
-            p[j] = e < E ? expf(p[j] - mx) : 0.f;
-            sum += p[j];
-        }
-        sum = wave_sum(sum);
-        const float inv_z = 1.f / sum;
-#pragma unroll
-        for (int j = 0; j < kPerLane; ++j) p[j] = (lane + kWave * j < E) ? p[j] * inv_z : -2.f;
-        float w_sum = 0.f, my_w = 0.f;   // lane k keeps the k-th weight
-        int my_e = 0;
-        for (int k = 0; k < K; ++k) {
-            float bv = -1.f;
-            int bi = kMaxExperts;
-#pragma unroll
-            for (int j = 0; j < kPerLane; ++j)
-                if (p[j] > bv) {
-                    bv = p[j];
-                    bi = lane + kWave * j;
-                }
-            wave_argmax(bv, bi);
-            bi = min(bi, E - 1);   // only reachable with NaN logits; keeps every index in range
-#pragma unroll
-            for (int j = 0; j < kPerLane; ++j)
-                if (bi == lane + kWave * j) p[j] = -1.f;   // exclude on the next pass
-            w_sum += bv;
-            if (lane == k) {
-                my_w = bv;
-                my_e = bi;
-            }
-        }
-        const float inv_w = 1.f / w_sum;
-        if (lane < K) {
-            topk_idx[static_cast<size_t>(t) * K + lane] = my_e;
-            topk_w[static_cast<size_t>(t) * K + lane] = my_w * inv_w;
-        }
-    }
     __syncthreads();
-
-    // ---- phase 2: rank of every route inside its expert, expert offsets ----
     const int R = N * K;
     for (int r = tid; r < R; r += kRouteThreads) route_pos[r] = atomicAdd(&cnt[topk_idx[r]], 1);
     __syncthreads();
@@ -183,9 +186,11 @@ extern "C" int pie_hip_moe_route(const uint16_t* router_logits_bf16, int32_t* to
     if (num_experts <= 0 || num_experts > kMaxExperts || top_k <= 0 || top_k > kMaxTopK ||
         top_k > num_experts)
         return PIE_HIP_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(kRouteThreads), 0,
-                       static_cast<hipStream_t>(stream), router_logits_bf16, topk_idx, topk_weight,
-                       expert_offsets, route_token, route_pos, num_tokens, num_experts, top_k);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    hipLaunchKernelGGL(moe_topk_kernel, dim3((num_tokens + 3) / 4), dim3(256), 0, st,
+                       router_logits_bf16, topk_idx, topk_weight, num_tokens, num_experts, top_k);
+    hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(kRouteThreads), 0, st, topk_idx, expert_offsets,
+                       route_token, route_pos, num_tokens, num_experts, top_k);
     return launch_status();
 }
 

@@ -100,15 +100,15 @@ def test_greedy_generation_matches_oracle(gpu, oracle, kw):
 
 @pytest.mark.parametrize("quant", ["int4b8", "fp8"])
 def test_long_prefill_through_the_tiled_gemm(gpu, oracle, quant):
-    """A 150-token prompt (two chunks under max_forward_tokens=128: 128 rows through the tiled
+    """A 230-token prompt (two chunks under max_forward_tokens=208: 208 rows through the tiled
     matrix-core GEMM, 22 through the skinny one), then decode; logits and tokens against the
     oracle."""
     from pie_amd import driver as drvmod
 
-    kw = dict(quant=quant, max_forward_tokens=128, total_pages=32)
+    kw = dict(quant=quant, max_forward_tokens=208, total_pages=32)
     cfg = full_cfg(**kw)
     rng = np.random.default_rng(93)
-    prompt = rng.integers(0, cfg["vocab"], 150)
+    prompt = rng.integers(0, cfg["vocab"], 230)
     with drvmod.Driver(toml_config(**kw)) as d:
         om, _ = oracle_model_from_driver(d, cfg)
         otoks, otrace = om.generate(prompt, 4, 1, want_logits=True)
