@@ -263,6 +263,40 @@ def cpu_baseline(drv, model, page_size, total_pages, n_prompt, gpu_tokens, budge
                 greedy_tokens_matched=matched, greedy_tokens_compared=steps)
 
 
+# HBM bytes per GEMV launch, averaged over the model's four int4 linears at M = 1, from two
+# `rocprofv3 --pmc` runs of `bench.py --pmc-workload` (FETCH_SIZE, then WRITE_SIZE, KiB per
+# dispatch), each scaled by what the same counter reads for the 256 MiB copy in that run
+# (FETCH_SIZE reads 131 085 for 262 144 KiB: factor 2.0; WRITE_SIZE reads 262 144: factor 1.0).
+# GEMV: FETCH_SIZE 14 018.8 -> 28.71 MB, WRITE_SIZE 30.0 -> 0.03 MB; algorithmic 28.15 MB.
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = 28_742_000
+
+
+def pmc_workload():
+    import torch
+
+    from pie_amd import ops
+
+    dev = torch.device("cuda:0")
+    src = torch.empty(256 * 1024 * 1024 // 4, dtype=torch.float32, device=dev).normal_()
+    dst = torch.empty_like(src)
+    for _ in range(4):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    H, I, G = MODEL["hidden"], MODEL["intermediate"], MODEL["group_size"]
+    qkv = (MODEL["q_heads"] + 2 * MODEL["kv_heads"]) * MODEL["head_dim"]
+    for (N, K) in [(qkv, H), (H, H), (2 * I, H), (H, I)]:
+        ws = [ops.int4b8_view(torch.randint(-2 ** 31, 2 ** 31 - 1, (N, K // 8), dtype=torch.int32, device=dev),
+                              (torch.rand(N, K // G, device=dev) * 0.015 + 0.005).bfloat16(), G)
+              for _ in range(6)]
+        act = torch.randn(1, K, device=dev).bfloat16()
+        y = torch.empty(1, N, device=dev, dtype=torch.bfloat16)
+        for i in range(12):
+            ops.linear_fused(act, ws[i % 6], y=y)
+        torch.cuda.synchronize()
+        del ws
+    print(json.dumps({"pmc_workload": "4 x 256 MiB copy, 12 launches of each int4 GEMV shape at M=1"}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -274,6 +308,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-extra", action="store_true")
     ap.add_argument("--model", default="llama8b-w4a16", choices=["llama8b-w4a16", *OTHER_MODELS])
+    ap.add_argument("--pmc-workload", action="store_true",
+                    help="only launch what a `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE` run needs: a "
+                         "256 MiB device copy (the counter's scale) and the four int4 GEMV shapes")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this driver path is built and measured on one GPU; "
@@ -287,6 +324,9 @@ def main():
         sys.exit(1)
     from pie_amd import driver as drvmod
 
+    if args.pmc_workload:
+        pmc_workload()
+        return
     page_size = 16
     max_new = args.warmup + args.steps + 1
     pages_per_ctx = (args.prompt + max_new + page_size - 1) // page_size
@@ -347,7 +387,8 @@ def main():
                    "weights": "int4b8 group 128, bf16 scales; bf16 embed/lm_head; fp32 accumulation"},
         "roofline": {"bound": "hbm", "kernel": "gemv_kernel<FmtInt4> (W4A16 weight-streaming GEMV, M=1)",
                      "achieved": round(roof["achieved"], 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(roof["achieved"] / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "frac": round(roof["achieved"] / HBM_PEAK_GBPS, 4),
+                     "traffic": GEMV_TRAFFIC_BYTES_PER_LAUNCH,
                      "avg_launch_us": round(roof["avg_us"], 2),
                      "algorithmic_bytes_per_launch": int(roof["bytes_per_launch"]),
                      "launches_timed": roof["launches"]},
