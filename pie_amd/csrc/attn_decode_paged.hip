@@ -87,7 +87,7 @@ __global__ __launch_bounds__(kAttnBlock) void attn_decode_split_kernel(
     float scale_log2e) {
     using U = UnitRegs<D, GQA>;
     constexpr int LPR = U::LPR, TPI = U::TPI, IPU = U::IPU;
-    const int split = blockIdx.x, kvh = blockIdx.y, r = blockIdx.z;
+    const int kvh = blockIdx.x, split = blockIdx.y, r = blockIdx.z;  // kv heads of the same tokens are dispatched together
     const int tid = threadIdx.x, lane = tid & (kWave - 1);
     const int wv = __builtin_amdgcn_readfirstlane(tid / kWave);  // wave-uniform -> SGPR
     const int grp = lane / LPR, dl = lane % LPR;
@@ -365,11 +365,13 @@ SplitPlan plan_splits(int R, int hk, int max_kv_len) {
     const int max_units = (max_kv_len + kUnitTokens - 1) / kUnitTokens;
     if (max_units <= 0) return {1, 1};
     const long long rows = static_cast<long long>(R) * hk;
-    const long long want_blocks = 2048;
+    // ~12 blocks per CU measured best on batch 64 x U[512, 8192] contexts (5.0 TB/s vs 4.4 at 8)
+    const long long want_blocks = 3072;
+    const long long min_ups = 2 * kAttnWaves;
     long long want_split = (want_blocks + rows - 1) / rows;
     if (want_split < 1) want_split = 1;
     long long ups = (max_units + want_split - 1) / want_split;
-    if (ups < 2 * kAttnWaves) ups = 2 * kAttnWaves;  // >= 2 units per wave amortises the merge
+    if (ups < min_ups) ups = min_ups;  // >= 2 units per wave amortises the merge
     if (ups > max_units) ups = max_units;
     if ((max_units + ups - 1) / ups > kMaxSplits) ups = (max_units + kMaxSplits - 1) / kMaxSplits;
     const int nsplit = static_cast<int>((max_units + ups - 1) / ups);
@@ -387,7 +389,7 @@ int launch_decode(const uint16_t* q, const uint16_t* k_pages, const uint16_t* v_
     if (plan.nsplit == 1) {
         hipLaunchKernelGGL((attn_decode_clear_empty_kernel<D>), dim3(R * hq), dim3(D), 0, stream,
                            page_indptr, last_lens, row_begin, row_len, o, lse, hq, ps);
-        hipLaunchKernelGGL((attn_decode_split_kernel<D, GQA>), dim3(1, hk, R), dim3(kAttnBlock), 0,
+        hipLaunchKernelGGL((attn_decode_split_kernel<D, GQA>), dim3(hk, 1, R), dim3(kAttnBlock), 0,
                            stream, q, k_pages, v_pages, page_indices, page_indptr, last_lens,
                            row_begin, row_len, nullptr, nullptr, o, lse, hq, hk, ps,
                            plan.units_per_split, 1,
@@ -399,7 +401,7 @@ int launch_decode(const uint16_t* q, const uint16_t* k_pages, const uint16_t* v_
     if (!workspace || workspace_bytes < need) return PIE_HIP_ERR_INVALID;
     float* part_o = static_cast<float*>(workspace);
     float* part_ml = part_o + n_part * D;
-    hipLaunchKernelGGL((attn_decode_split_kernel<D, GQA>), dim3(plan.nsplit, hk, R),
+    hipLaunchKernelGGL((attn_decode_split_kernel<D, GQA>), dim3(hk, plan.nsplit, R),
                        dim3(kAttnBlock), 0, stream, q, k_pages, v_pages, page_indices, page_indptr,
                        last_lens, row_begin, row_len, part_o, part_ml, nullptr, nullptr, hq, hk, ps,
                        plan.units_per_split, plan.nsplit, scale_log2e);

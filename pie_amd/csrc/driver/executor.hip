@@ -145,8 +145,8 @@ Executor::Executor(const DriverConfig& cfg, Model& model) : cfg_(cfg), model_(mo
     logits_ = dmalloc<uint16_t>(srows * m.vocab);
     out_tokens_ = dmalloc<uint32_t>(T);
     // Bound of the split-K partial buffers over every (rows, context) the planner can pick:
-    // rows * splits <= 2048/hk + rows.
-    attn_ws_bytes_ = (2048 / static_cast<size_t>(hk) + 1 + T) * hq * (d + 2) * sizeof(float);
+    // rows * splits <= 3072/hk + rows.
+    attn_ws_bytes_ = (3072 / static_cast<size_t>(hk) + 1 + T) * hq * (d + 2) * sizeof(float);
     PIE_HIP_CHECK(hipMalloc(&attn_ws_, attn_ws_bytes_));
 
     in_ = input_layout(max_tokens_, max_tokens_);
