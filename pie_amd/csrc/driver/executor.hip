@@ -51,11 +51,22 @@ int fmt_code(Quant q) {
     }
 }
 
+// Measured cost models (MI355X, microseconds): the skinny GEMM streams the weights once per 16
+// rows at ~2.4 TB/s plus ~4 us per pass; the tiled GEMM walks K in 64-wide steps of ~1 us
+// while its 128 x 128 tiles fit the machine (512 resident blocks), longer in proportion beyond.
+bool tiled_gemm_is_faster(const Linear& w, int M) {
+    if (w.K % 64 != 0 || M < 48) return false;
+    const double skinny = ((M + 15) / 16) * (4.0 + static_cast<double>(w.data_bytes()) / 2.4e6);
+    const double tiles = static_cast<double>((w.N + 127) / 128) * ((M + 127) / 128);
+    const double gemm = (w.K / 64) * 0.97 * std::max(1.0, tiles / 512.0);
+    return gemm < skinny;
+}
+
 // y = epilogue(rmsnorm?(act) · W^T) by the weight's storage format — the dispatcher role of
 // gemm_act_x_w (driver/cuda/src/ops/gemm.cpp:1414-1583).  Up to four rows: the weight-streaming
 // GEMV with the norm riding in its activation staging and SwiGLU in its epilogue.  More rows
 // (norm as its own kernel into `norm_tmp`): the matrix-core skinny GEMM, which streams the
-// weights once per 16 rows, and from 193 rows on the tiled matrix-core GEMM; shapes those do
+// weights once per 16 rows, or the tiled matrix-core GEMM where its cost model wins; shapes those do
 // not take fall back to the GEMV path.
 void linear_fused(const Linear& w, const uint16_t* act, const uint16_t* norm_w, float eps,
                   uint16_t* y, int M, int beta, int swiglu, uint16_t* norm_tmp, hipStream_t s) {
@@ -67,9 +78,8 @@ void linear_fused(const Linear& w, const uint16_t* act, const uint16_t* norm_w, 
             PIE_KERNEL(pie_hip_rmsnorm(act, norm_w, norm_tmp, M, w.K, eps, s));
             a = norm_tmp;
         }
-        if (M > 192) {
-            // compute-bound: the tiled GEMM (weights dequantised to bf16 while staged); below
-            // that the 16-row passes of the skinny kernel are still faster
+        if (tiled_gemm_is_faster(w, M)) {
+            // compute-bound: the tiled GEMM (weights dequantised to bf16 while staged)
             const int sg = pie_hip_gemm_mfma(fmt, a, w.data, w.scale, sbf, w.group, y, M, w.N, w.K,
                                              beta, swiglu, s);
             if (sg == PIE_HIP_OK) return;

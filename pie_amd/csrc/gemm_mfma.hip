@@ -11,12 +11,19 @@
 // bf16 x bf16 products, fp32 accumulation, one rounding at the end.
 //
 // Tiling: a 128 x 128 output tile per block of four waves, each wave a 64 x 64 quadrant held as
-// 4 x 4 accumulators of v_mfma_f32_16x16x32_bf16; K advances 64 at a time through two LDS
-// buffers (global loads of tile t+1 are in flight while tile t is multiplied; one barrier per
-// step).  LDS rows are padded to 144 bytes so the 16 rows an operand read touches fall in
-// distinct banks.  Activations are the MFMA A operand, weights the B operand: an accumulator
-// lane holds one weight row n (column of y) for four consecutive activation rows, so row scales
-// are per-lane scalars and the SwiGLU partner (gate_i, up_i interleaved) is the neighbouring lane.
+// 4 x 4 accumulators of v_mfma_f32_16x16x32_bf16; K advances 64 at a time.
+//   * activations (and bf16 weights) travel global -> LDS directly (global_load_lds_dwordx4,
+//     no registers) into a ring of three stages, issued two K steps ahead; every wave waits
+//     for its own transfers with an explicit vmcnt and the block meets at one barrier per step;
+//   * quantised weights travel through registers, three K steps ahead (a tile row is only
+//     16-32 bytes per thread), are decoded to bf16 and written to a double-buffered LDS tile one
+//     step before use;
+//   * LDS tiles are unpadded and XOR-swizzled in 16-byte granules (granule g of row r sits at
+//     g ^ ((r >> 1) & 7)) so that the 16 rows an MFMA operand read touches fall in distinct
+//     banks while a direct-to-LDS transfer still writes 1 KiB contiguous per wave;
+//   * activations are the MFMA A operand, weights the B operand: an accumulator lane holds one
+//     weight row n (column of y) for four consecutive activation rows, so row scales are
+//     per-lane scalars and the SwiGLU partner (gate_i, up_i interleaved) is the neighbour lane.
 #include "common.hip.h"
 
 namespace pie_hip {
@@ -27,9 +34,10 @@ typedef float f32x2_t __attribute__((ext_vector_type(2)));
 
 constexpr int BM = 128, BN = 128, BK = 64;
 constexpr int kThreads = 256;
-constexpr int kVecPerRow = BK / 8;           // 16-byte vectors per tile row
-constexpr int kRowStride = kVecPerRow + 1;   // padded
-constexpr int kTileVecs = BM * kRowStride;   // per operand per buffer
+constexpr int kTileVecs = BM * (BK / 8);   // 16-byte vectors per bf16 tile (16 KiB)
+constexpr int kStages = 3;
+
+#define PIE_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
 
 struct GemmArgs {
     const uint16_t* act;
@@ -43,29 +51,37 @@ __device__ __forceinline__ uint32_t pack_trunc(float lo, float hi) {
     return __builtin_amdgcn_perm(__float_as_uint(hi), __float_as_uint(lo), 0x07060302u);
 }
 
-// ---- weight staging: global -> registers (raw) -> bf16 vectors in LDS --------------------
-// Every format hands each thread the raw bytes of 32 (int4/int8/fp8) or 32 (bf16: 4 x 8)
-// weights of one tile row per K step.
+// position of granule g of tile row r (in 16-byte vectors)
+__device__ __forceinline__ int swz(int r, int g) { return r * 8 + (g ^ ((r >> 1) & 7)); }
+
+// ---- quantised weight staging: global -> registers (raw) -> bf16 vectors in LDS ------------
+// Thread t holds the 32 k-values (t % 2) of tile row t / 2 of one K step.
 struct GInt4 {
-    static constexpr int kRawVecs = 1;   // 16 bytes = 32 nibbles of row t/2, k half t%2
-    static constexpr bool kRowScale = false;
-    static __device__ __forceinline__ void load(const GemmArgs& a, int n, int k0, int tid, u32x4_t* raw,
-                                                float& gs) {
+    static constexpr int kRawVecs = 1;
+    static constexpr int kLoads = 2;   // vector-memory operations per thread per K step
+    static constexpr bool kRowScale = false, kDirect = false;
+    struct Raw {
+        u32x4_t v[1];
+        uint16_t gs;
+    };
+    static __device__ __forceinline__ Raw load(const GemmArgs& a, int n, int k0, int tid) {
+        Raw r;
         const int half = tid & 1;
-        const unsigned char* p = a.w + (static_cast<size_t>(n) * a.K + k0 + half * 32) / 2;
-        raw[0] = *reinterpret_cast<const u32x4_t*>(p);
-        const uint16_t* sc = reinterpret_cast<const uint16_t*>(a.scale);
-        gs = bf16_bits_to_f32(sc[static_cast<size_t>(n) * (a.K >> a.g_shift) + ((k0 + half * 32) >> a.g_shift)]);
+        r.v[0] = *reinterpret_cast<const u32x4_t*>(a.w + (static_cast<size_t>(n) * a.K + k0 + half * 32) / 2);
+        r.gs = reinterpret_cast<const uint16_t*>(a.scale)[static_cast<size_t>(n) * (a.K >> a.g_shift) +
+                                                          ((k0 + half * 32) >> a.g_shift)];
+        return r;
     }
-    static __device__ __forceinline__ void store(u32x4_t* row, int tid, const u32x4_t* raw, float gs) {
+    static __device__ __forceinline__ void store(u32x4_t* tile, int row, int tid, const Raw& r) {
         const int half = tid & 1;
+        const float gs = bf16_bits_to_f32(r.gs);
         const float off = -136.f * gs;
         uint32_t k128 = 0x43004300u;
         asm volatile("" : "+v"(k128));
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
-            const uint32_t v = raw[0][s];
-            uint32_t pr[4];   // pr[j] = (128 + nib_j, 128 + nib_{j+4}) as bf16 pair
+            const uint32_t v = r.v[0][s];
+            uint32_t pr[4];   // pr[j] = (128 + nib_j, 128 + nib_{j+4}) as a bf16 pair
 #pragma unroll
             for (int j = 0; j < 4; ++j) pr[j] = and_or(v >> (4 * j), 0x000F000Fu, k128);
             float f[8];
@@ -74,41 +90,45 @@ struct GInt4 {
                 f[j] = fmaf(bf16_lo(pr[j]), gs, off);       // exact: (nib - 8) * scale
                 f[j + 4] = fmaf(bf16_hi(pr[j]), gs, off);
             }
-            row[half * 4 + s] = u32x4_t{pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]),
-                                        pack_bf16x2(f[4], f[5]), pack_bf16x2(f[6], f[7])};
+            tile[swz(row, half * 4 + s)] = u32x4_t{pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]),
+                                                   pack_bf16x2(f[4], f[5]), pack_bf16x2(f[6], f[7])};
         }
     }
 };
 struct GFp8 {
-    static constexpr int kRawVecs = 2;   // 32 bytes of row t/2, k half t%2
-    static constexpr bool kRowScale = true;
-    static __device__ __forceinline__ void load(const GemmArgs& a, int n, int k0, int tid, u32x4_t* raw,
-                                                float&) {
+    static constexpr int kLoads = 2;
+    static constexpr bool kRowScale = true, kDirect = false;
+    struct Raw {
+        u32x4_t v[2];
+    };
+    static __device__ __forceinline__ Raw load(const GemmArgs& a, int n, int k0, int tid) {
+        Raw r;
         const unsigned char* p = a.w + static_cast<size_t>(n) * a.K + k0 + (tid & 1) * 32;
-        raw[0] = *reinterpret_cast<const u32x4_t*>(p);
-        raw[1] = *reinterpret_cast<const u32x4_t*>(p + 16);
+        r.v[0] = *reinterpret_cast<const u32x4_t*>(p);
+        r.v[1] = *reinterpret_cast<const u32x4_t*>(p + 16);
+        return r;
     }
     static __device__ __forceinline__ uint32_t cv(uint32_t w, bool hi) {
         const f32x2_t f = hi ? __builtin_amdgcn_cvt_pk_f32_fp8(w, true) : __builtin_amdgcn_cvt_pk_f32_fp8(w, false);
         return pack_trunc(f.x, f.y);
     }
-    static __device__ __forceinline__ void store(u32x4_t* row, int tid, const u32x4_t* raw, float) {
+    static __device__ __forceinline__ void store(u32x4_t* tile, int row, int tid, const Raw& r) {
         const int half = tid & 1;
 #pragma unroll
         for (int v = 0; v < 2; ++v)
 #pragma unroll
             for (int s = 0; s < 2; ++s) {
-                const uint32_t a = raw[v][2 * s], b = raw[v][2 * s + 1];
-                row[half * 4 + v * 2 + s] = u32x4_t{cv(a, false), cv(a, true), cv(b, false), cv(b, true)};
+                const uint32_t a = r.v[v][2 * s], b = r.v[v][2 * s + 1];
+                tile[swz(row, half * 4 + v * 2 + s)] = u32x4_t{cv(a, false), cv(a, true), cv(b, false), cv(b, true)};
             }
     }
 };
 struct GInt8 {
-    static constexpr int kRawVecs = 2;
-    static constexpr bool kRowScale = true;
-    static __device__ __forceinline__ void load(const GemmArgs& a, int n, int k0, int tid, u32x4_t* raw,
-                                                float& gs) {
-        GFp8::load(a, n, k0, tid, raw, gs);
+    static constexpr int kLoads = 2;
+    static constexpr bool kRowScale = true, kDirect = false;
+    using Raw = GFp8::Raw;
+    static __device__ __forceinline__ Raw load(const GemmArgs& a, int n, int k0, int tid) {
+        return GFp8::load(a, n, k0, tid);
     }
     static __device__ __forceinline__ uint32_t two(uint32_t u, int sh) {
         // signed bytes -> exact bf16 pair: (byte ^ 0x80) - 128
@@ -116,53 +136,67 @@ struct GInt8 {
         const float hi = static_cast<float>((u >> (sh + 8)) & 0xFFu) - 128.f;
         return pack_trunc(lo, hi);
     }
-    static __device__ __forceinline__ void store(u32x4_t* row, int tid, const u32x4_t* raw, float) {
+    static __device__ __forceinline__ void store(u32x4_t* tile, int row, int tid, const Raw& r) {
         const int half = tid & 1;
 #pragma unroll
         for (int v = 0; v < 2; ++v)
 #pragma unroll
             for (int s = 0; s < 2; ++s) {
-                const uint32_t a = raw[v][2 * s] ^ 0x80808080u, b = raw[v][2 * s + 1] ^ 0x80808080u;
-                row[half * 4 + v * 2 + s] = u32x4_t{two(a, 0), two(a, 16), two(b, 0), two(b, 16)};
+                const uint32_t a = r.v[v][2 * s] ^ 0x80808080u, b = r.v[v][2 * s + 1] ^ 0x80808080u;
+                tile[swz(row, half * 4 + v * 2 + s)] = u32x4_t{two(a, 0), two(a, 16), two(b, 0), two(b, 16)};
             }
     }
 };
 struct GBf16 {
-    static constexpr int kRawVecs = 4;   // 64 bytes of row t/2, k half t%2
-    static constexpr bool kRowScale = false;
-    static __device__ __forceinline__ void load(const GemmArgs& a, int n, int k0, int tid, u32x4_t* raw,
-                                                float&) {
-        const uint16_t* p = reinterpret_cast<const uint16_t*>(a.w) + static_cast<size_t>(n) * a.K + k0 + (tid & 1) * 32;
-#pragma unroll
-        for (int v = 0; v < 4; ++v) raw[v] = *reinterpret_cast<const u32x4_t*>(p + 8 * v);
-    }
-    static __device__ __forceinline__ void store(u32x4_t* row, int tid, const u32x4_t* raw, float) {
-        const int half = tid & 1;
-#pragma unroll
-        for (int v = 0; v < 4; ++v) row[half * 4 + v] = raw[v];
-    }
+    static constexpr int kLoads = 4;   // direct-to-LDS transfers per wave per K step
+    static constexpr bool kRowScale = false, kDirect = true;
+    struct Raw {};
+    static __device__ __forceinline__ Raw load(const GemmArgs&, int, int, int) { return {}; }
+    static __device__ __forceinline__ void store(u32x4_t*, int, int, const Raw&) {}
 };
+
+// s_waitcnt with vmcnt(n) (n < 16) and lgkmcnt(0), expcnt untouched (gfx9 encoding)
+#define PIE_WAIT_VM_LGKM0(n) __builtin_amdgcn_s_waitcnt(0x0070 | (n))
 
 template <class F>
 __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(const GemmArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
-    u32x4_t* lds = reinterpret_cast<u32x4_t*>(smem);   // [2 buffers][A tile | B tile]
+    u32x4_t* lds_a = reinterpret_cast<u32x4_t*>(smem);            // [kStages][tile]
+    u32x4_t* lds_b = lds_a + kStages * kTileVecs;                 // direct: [kStages][tile]; else [2][tile]
     const int tid = threadIdx.x, lane = tid & (kWave - 1);
     const int wv = __builtin_amdgcn_readfirstlane(tid / kWave);
     const int j = lane & 15, q = lane >> 4;
     const int wm = wv >> 1, wn = wv & 1;
     const int M = a.M, N = a.N, K = a.K;
     const int n0 = blockIdx.x * BN, m0 = blockIdx.y * BM;
+    const int nk = K / BK;
 
-    // staging roles: activations — 4 vectors per thread (row tid/8 + 32u, vector tid%8);
-    // weights — the 32 k-values (tid%2) of tile row tid/2
-    const int arow = tid >> 3, avec = tid & 7;
+    // direct transfers: wave w moves the 1 KiB chunks ci = 4u + w (8 tile rows each); lane p
+    // lands at chunk position p = (row ci*8 + p/8, slot p%8), which holds granule slot ^ key(row)
     const uint16_t* aptr[4];
+    const uint16_t* bptr[4];
 #pragma unroll
-    for (int u = 0; u < 4; ++u)
-        aptr[u] = a.act + static_cast<size_t>(min(m0 + arow + 32 * u, M - 1)) * K + avec * 8;
+    for (int u = 0; u < 4; ++u) {
+        const int r = (u * 4 + wv) * 8 + (lane >> 3);
+        const int g = (lane & 7) ^ ((r >> 1) & 7);
+        aptr[u] = a.act + static_cast<size_t>(min(m0 + r, M - 1)) * K + g * 8;
+        bptr[u] = reinterpret_cast<const uint16_t*>(a.w) + static_cast<size_t>(min(n0 + r, N - 1)) * K + g * 8;
+    }
+    auto issue_direct = [&](int kt) {
+        const int k0 = min(kt, nk - 1) * BK;
+        const int st = kt % kStages;
+        if (F::kDirect) {
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                __builtin_amdgcn_global_load_lds(bptr[u] + k0, PIE_LDS_PTR(lds_b + st * kTileVecs + (u * 4 + wv) * 64), 16, 0, 0);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            __builtin_amdgcn_global_load_lds(aptr[u] + k0, PIE_LDS_PTR(lds_a + st * kTileVecs + (u * 4 + wv) * 64), 16, 0, 0);
+    };
     const int wrow = tid >> 1;
     const int wn_glob = min(n0 + wrow, N - 1);
+    auto load_w = [&](int kt) { return F::load(a, wn_glob, min(kt, nk - 1) * BK, tid); };
 
     f32x4_t acc[4][4];
 #pragma unroll
@@ -170,46 +204,59 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(const GemmArgs a) {
 #pragma unroll
         for (int nt = 0; nt < 4; ++nt) acc[mt][nt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-    u32x4_t areg[4], wreg[F::kRawVecs];
-    float gs = 1.f;
-    auto gload = [&](int k0) {
+    // prologue: activations of steps 0 and 1 in flight, weights of steps 0..2 in registers,
+    // the bf16 tile of step 0 written
+    typename F::Raw rr[kStages];
+    issue_direct(0);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int u = 0; u < 4; ++u) areg[u] = *reinterpret_cast<const u32x4_t*>(aptr[u] + k0);
-        F::load(a, wn_glob, k0, tid, wreg, gs);
-    };
-    auto lstore = [&](int buf) {
-        u32x4_t* A = lds + buf * 2 * kTileVecs;
-        u32x4_t* B = A + kTileVecs;
-#pragma unroll
-        for (int u = 0; u < 4; ++u) A[(arow + 32 * u) * kRowStride + avec] = areg[u];
-        F::store(B + wrow * kRowStride, tid, wreg, gs);
-    };
+    for (int i = 0; i < kStages; ++i) rr[i] = load_w(i);
+    __builtin_amdgcn_sched_barrier(0);
+    issue_direct(1);
+    __builtin_amdgcn_sched_barrier(0);
+    if (!F::kDirect) F::store(lds_b, wrow, tid, rr[0]);
 
-    const int nk = K / BK;
-    gload(0);
-    lstore(0);
-    __syncthreads();
-    for (int kt = 0; kt < nk; ++kt) {
-        const int buf = kt & 1;
-        gload(min(kt + 1, nk - 1) * BK);   // next tile travels while this one is multiplied
-        const u32x4_t* A = lds + buf * 2 * kTileVecs + (wm * 64 + j) * kRowStride + q;
-        const u32x4_t* B = lds + buf * 2 * kTileVecs + kTileVecs + (wn * 64 + j) * kRowStride + q;
+    // The loop body is unrolled three times so that ring slots (LDS stage, register set) are
+    // compile-time constants: a register rotation would have to wait for the newest load.
+    for (int kt0 = 0; kt0 < nk; kt0 += kStages) {
 #pragma unroll
-        for (int ks = 0; ks < BK / 32; ++ks) {
-            bf16x8_t af[4], bfr[4];
+        for (int i = 0; i < kStages; ++i) {
+            const int kt = kt0 + i;
+            // Transfers of step kt are complete when at most the operations issued after them
+            // are outstanding: the previous iteration's weight loads and its 4 (8) transfers.
+            __builtin_amdgcn_sched_barrier(0);
+            if (F::kDirect) PIE_WAIT_VM_LGKM0(8);
+            else PIE_WAIT_VM_LGKM0(4 + F::kLoads);
+            __builtin_amdgcn_s_barrier();
+            __builtin_amdgcn_sched_barrier(0);
+            rr[i] = load_w(kt + kStages);   // slot i held step kt, already written to LDS
+            __builtin_amdgcn_sched_barrier(0);
+            issue_direct(kt + 2);           // into the stage step kt - 1 was read from
+            __builtin_amdgcn_sched_barrier(0);
+
+            if (kt < nk) {
+                const u32x4_t* A = lds_a + i * kTileVecs + (wm * 64 + j) * 8;
+                const u32x4_t* B = lds_b + (F::kDirect ? i : (kt & 1)) * kTileVecs + (wn * 64 + j) * 8;
+                const int key = j >> 1;   // swizzle key of rows base16 + j
 #pragma unroll
-            for (int t = 0; t < 4; ++t) {
-                af[t] = __builtin_bit_cast(bf16x8_t, A[t * 16 * kRowStride + ks * 4]);
-                bfr[t] = __builtin_bit_cast(bf16x8_t, B[t * 16 * kRowStride + ks * 4]);
+                for (int ks = 0; ks < BK / 32; ++ks) {
+                    bf16x8_t af[4], bfr[4];
+                    const int slot = (ks * 4 + q) ^ key;
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        af[t] = __builtin_bit_cast(bf16x8_t, A[t * 16 * 8 + slot]);
+                        bfr[t] = __builtin_bit_cast(bf16x8_t, B[t * 16 * 8 + slot]);
+                    }
+#pragma unroll
+                    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+                        for (int nt = 0; nt < 4; ++nt)
+                            acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[mt], bfr[nt], acc[mt][nt], 0, 0, 0);
+                }
             }
-#pragma unroll
-            for (int mt = 0; mt < 4; ++mt)
-#pragma unroll
-                for (int nt = 0; nt < 4; ++nt)
-                    acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[mt], bfr[nt], acc[mt][nt], 0, 0, 0);
+            // next step's weights -> bf16 tile (the other buffer; its readers passed the barrier)
+            if (!F::kDirect) F::store(lds_b + ((kt + 1) & 1) * kTileVecs, wrow, tid, rr[(i + 1) % kStages]);
         }
-        lstore(buf ^ 1);   // the other buffer was released by the barrier of the previous step
-        __syncthreads();
     }
 
     // ---- epilogue: lane holds column n for rows 4q + r of each 16 x 16 tile ----
@@ -249,7 +296,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(const GemmArgs a) {
 
 template <class F>
 int launch_gemm(const GemmArgs& a, hipStream_t stream) {
-    constexpr size_t smem = static_cast<size_t>(2) * 2 * kTileVecs * sizeof(u32x4_t);
+    constexpr size_t smem = static_cast<size_t>(kStages + (F::kDirect ? kStages : 2)) * kTileVecs * sizeof(u32x4_t);
     static const hipError_t attr =
         hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_mfma_kernel<F>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
