@@ -101,6 +101,25 @@ int pie_hip_linear_fused(int format, const uint16_t* act_bf16, const uint16_t* n
                          int swiglu, void* stream);
 
 /*
+ * The fused q|k|v projection of a decode step with RoPE and the KV-cache write in its epilogue:
+ * rows of W are the q, k and v heads ([(hq + 2 hk) * d, K]); adjacent output pairs (2i, 2i+1)
+ * of every q and k head are rotated by rope_table[m] (interleaved pairing,
+ * driver/cuda/src/kernels/rope.cu:14-33), q goes to q_out [M, hq*d], k and v to slot
+ * kv_slots[m] of the paged pools (NHD addressing, driver/cuda/src/kernels/split_packed.cu:116-138).
+ * Values are those of pie_hip_linear_fused followed by pie_hip_qkv_rope_kvwrite with
+ * interleaved = 1 and no q/k norm (every intermediate rounded to bf16 at the same points).
+ * Replaces the qkv gemm + qkv_decode_qk_norm_rope_write_kv_kernel pair of
+ * driver/cuda/src/model/llama_like.cpp:370-470 for llama-type decode.  head_dim a power of two,
+ * M <= 4 per weight pass like the GEMV.
+ */
+int pie_hip_qkv_rope_fused(int format, const uint16_t* act_bf16, const uint16_t* norm_weight_bf16,
+                           float eps, const void* weight, const void* scale, int scale_is_bf16,
+                           int group_size, int M, int K, const float* rope_table,
+                           const int64_t* kv_slots, uint16_t* q_out, uint16_t* k_pages,
+                           uint16_t* v_pages, int num_q_heads, int num_kv_heads, int head_dim,
+                           void* stream);
+
+/*
  * Weight-only GEMM for a handful to a few dozen activation rows on the matrix cores:
  *   y[m, n] = epilogue( sum_k act[m,k] * w(n,k) ), same formats, scales, beta and swiglu
  * contracts as pie_hip_linear_fused (no fused norm); the weights are streamed once per 16

@@ -265,10 +265,18 @@ void Executor::body(int N, int S, int max_kv_len) {
     PIE_KERNEL(pie_hip_rope_table(positions, model_.inv_freq, rope_tab_, N, d, s));
     for (int l = 0; l < m.layers; ++l) {
         const LayerWeights& w = model_.layers[l];
-        linear_fused(w.wqkv, x_, w.attn_norm, m.rms_eps, qkv_, N, 0, 0, xn_, s);
-        PIE_KERNEL(pie_hip_qkv_rope_kvwrite(qkv_, q_, k_pool_[l], v_pool_[l], w.q_norm, w.k_norm,
-                                            rope_tab_, slots, N, hq, hk, d, m.rope_interleaved,
-                                            m.rms_eps, s));
+        if (N <= 4 && m.rope_interleaved && !w.q_norm && (d & (d - 1)) == 0) {
+            // decode rows of llama-type layers: rotation and KV write ride in the projection
+            PIE_KERNEL(pie_hip_qkv_rope_fused(fmt_code(w.wqkv.kind), x_, w.attn_norm, m.rms_eps,
+                                              w.wqkv.data, w.wqkv.scale, w.wqkv.scale_bf16 ? 1 : 0,
+                                              w.wqkv.group, N, H, rope_tab_, slots, q_, k_pool_[l],
+                                              v_pool_[l], hq, hk, d, s));
+        } else {
+            linear_fused(w.wqkv, x_, w.attn_norm, m.rms_eps, qkv_, N, 0, 0, xn_, s);
+            PIE_KERNEL(pie_hip_qkv_rope_kvwrite(qkv_, q_, k_pool_[l], v_pool_[l], w.q_norm, w.k_norm,
+                                                rope_tab_, slots, N, hq, hk, d, m.rope_interleaved,
+                                                m.rms_eps, s));
+        }
         PIE_KERNEL(pie_hip_attn_rows_paged(q_, k_pool_[l], v_pool_[l], attn_, nullptr, pages,
                                            row_begin, row_len, N, hq, hk, d, page_size_, -1.f,
                                            max_kv_len, attn_ws_, attn_ws_bytes_, s));

@@ -205,6 +205,8 @@ struct Unit {
     uint16_t prev;   // y element this lane may add to (lane = r*M + m), for beta = 1
     float rs;        // row scale for that lane's row (int8 / fp8)
     float rs2;       // swiglu epilogue: row scale of the pair's second (up) row
+    float rc, rsn;   // qkv epilogue: cos / sin of this lane's (token, pair)
+    int slot;        // qkv epilogue: KV slot of this lane's token (< 0: none)
 };
 
 struct GemvArgs {
@@ -217,9 +219,19 @@ struct GemvArgs {
     const uint16_t* norm_w;  // bf16 [K] or null: RMSNorm applied to act while staging
     float eps;
     int swiglu;  // 1: rows are (gate_i, up_i) pairs; y[m, i] = silu(bf16 g) * bf16 u, y is [M, N/2]
+    // qkv epilogue (rope_table != null): rows are the fused q | k | v projection; pairs
+    // (2i, 2i+1) of a q / k head are rotated (interleaved RoPE), q goes to y = q_out
+    // [M, hq*d], k and v to the token's slot of the paged pools
+    const float* rope_table;  // f32 [M, d]: cos at [i], sin at [d/2 + i]
+    const int64_t* kv_slots;  // [M], < 0: no KV slot
+    uint16_t* k_pages;
+    uint16_t* v_pages;
+    int hq, hk, d;
 };
 
-template <class F, int R, int M>
+// ROPE: the q|k|v epilogue (rotation + KV write); its per-lane cos / sin / slot ride with every
+// unit's loads like the residual does, so the epilogue itself issues no loads.
+template <class F, int R, int M, bool ROPE>
 __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
     constexpr int WPP = F::WPP, XV = F::XV;
     constexpr int kChunkK = kWave * WPP;  // weights covered by one wave-wide 16 B load
@@ -240,7 +252,8 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
     const long long total_waves = static_cast<long long>(gridDim.x) * kWavesPerBlock;
     const long long wg = static_cast<long long>(blockIdx.x) * kWavesPerBlock + wv;
     // (slices fall on even rows for the swiglu epilogue, which pairs rows 2i and 2i+1)
-    const int gran = a.swiglu ? 2 : 1;
+    const bool pairs = a.swiglu || ROPE;
+    const int gran = pairs ? 2 : 1;
     const int row_begin = static_cast<int>(wg * (N / gran) / total_waves) * gran;
     const int row_end = static_cast<int>((wg + 1) * (N / gran) / total_waves) * gran;
     const int ngroups = (row_end - row_begin + R - 1) / R;
@@ -265,15 +278,22 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
         // epilogue never stalls the pipeline (only the last chunk's values are used).
         // (branch-free on purpose: a branch around loads would merge the outstanding-load state
         // of both arms and force the next wait to drain the whole pipeline)
-        const int per = a.swiglu ? (R / 2) * M : R * M;
+        const int per = pairs ? (R / 2) * M : R * M;
         const int li = lane < per ? lane / M : 0;
         const int lm = lane < per ? lane % M : 0;
-        const int lrow = a.swiglu ? min(row_begin + g * R + 2 * li, row_end - 2)
-                                  : min(row_begin + g * R + li, row_end - 1);
-        u.prev = a.y[a.swiglu ? 0 : static_cast<size_t>(lm) * N + lrow];
+        const int lrow = pairs ? min(row_begin + g * R + 2 * li, row_end - 2)
+                               : min(row_begin + g * R + li, row_end - 1);
+        u.prev = a.y[pairs ? 0 : static_cast<size_t>(lm) * N + lrow];
         if constexpr (F::kRowScale) {
             u.rs = F::load(a.rscale, lrow);
             u.rs2 = F::load(a.rscale, min(lrow + 1, N - 1));
+        }
+        if constexpr (ROPE) {
+            const int dd = lrow & (a.d - 1);   // head_dim is a power of two here
+            const float* tab = a.rope_table + static_cast<size_t>(lm) * a.d + (dd >> 1);
+            u.rc = tab[0];
+            u.rsn = tab[a.d >> 1];
+            u.slot = static_cast<int>(a.kv_slots[lm]);
         }
     };
 
@@ -381,7 +401,7 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
                     acc[r][m] = 0.f;
                 }
             }
-            if (a.swiglu) {
+            if (pairs) {
                 if constexpr (R % 2 == 0) {
                     // lane p*M + m finishes pair p: g and u are rounded to bf16 first, as the
                     // unfused projection would store them (swiglu.cu:18-21 reads bf16 inputs)
@@ -404,9 +424,27 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
                         }
                         const float gb = bf16_bits_to_f32(f32_to_bf16_bits(gv));
                         const float ub = bf16_bits_to_f32(f32_to_bf16_bits(uv));
-                        const float silu = gb / (1.f + expf(-gb));
-                        a.y[static_cast<size_t>(lane % M) * (N / 2) + row / 2] =
-                            f32_to_bf16_bits(silu * ub);
+                        const int m = lane % M;
+                        if (!ROPE) {
+                            const float silu = gb / (1.f + expf(-gb));
+                            a.y[static_cast<size_t>(m) * (N / 2) + row / 2] = f32_to_bf16_bits(silu * ub);
+                        } else {
+                            // the projection's bf16 values, then the rotation of
+                            // qkv_rope_kvwrite_kernel with the same operations and rounding
+                            const int head = row / a.d, dd = row - head * a.d;
+                            const int slot = u.slot;
+                            if (head < a.hq + a.hk) {
+                                const float c = u.rc, sn = u.rsn;
+                                const uint32_t out = pack_bf16x2(gb * c - ub * sn, ub * c + gb * sn);
+                                if (head < a.hq)
+                                    *reinterpret_cast<uint32_t*>(a.y + (static_cast<size_t>(m) * a.hq + head) * a.d + dd) = out;
+                                else if (slot >= 0)
+                                    *reinterpret_cast<uint32_t*>(a.k_pages + (static_cast<size_t>(slot) * a.hk + (head - a.hq)) * a.d + dd) = out;
+                            } else if (slot >= 0) {
+                                *reinterpret_cast<uint32_t*>(a.v_pages + (static_cast<size_t>(slot) * a.hk + (head - a.hq - a.hk)) * a.d + dd) =
+                                    pack_bf16x2(gb, ub);
+                            }
+                        }
                     }
                 }
             } else {
@@ -464,15 +502,20 @@ int launch(const GemvArgs& a, int waves_per_simd, hipStream_t stream) {
     if (smem > 64 * 1024) return PIE_HIP_ERR_UNSUPPORTED;
     int grid = kNumCU * waves_per_simd;
     // >= 1 row (or row pair) per wave
-    const int max_grid = (a.N / (a.swiglu ? 2 : 1) + kWavesPerBlock - 1) / kWavesPerBlock;
+    const int max_grid = (a.N / ((a.swiglu || a.rope_table) ? 2 : 1) + kWavesPerBlock - 1) / kWavesPerBlock;
     if (grid > max_grid) grid = max_grid;
-    if (t_start_event && t_stop_event) {
-        hipExtLaunchKernelGGL((gemv_kernel<F, R, M>), dim3(grid), dim3(kBlock),
+    if (a.rope_table) {
+        if constexpr (R % 2 == 0)
+            hipLaunchKernelGGL((gemv_kernel<F, R, M, true>), dim3(grid), dim3(kBlock), smem, stream, a);
+        else
+            return PIE_HIP_ERR_INVALID;
+    } else if (t_start_event && t_stop_event) {
+        hipExtLaunchKernelGGL((gemv_kernel<F, R, M, false>), dim3(grid), dim3(kBlock),
                               static_cast<uint32_t>(smem), stream, t_start_event, t_stop_event, 0,
                               a);
         t_start_event = t_stop_event = nullptr;
     } else {
-        hipLaunchKernelGGL((gemv_kernel<F, R, M>), dim3(grid), dim3(kBlock), smem, stream, a);
+        hipLaunchKernelGGL((gemv_kernel<F, R, M, false>), dim3(grid), dim3(kBlock), smem, stream, a);
     }
     return launch_status();
 }
@@ -505,7 +548,7 @@ int dispatch(GemvArgs a, int M, int rows_per_wave, int waves_per_simd, hipStream
             a.N / (static_cast<long long>(kNumCU) * kWavesPerBlock * waves_per_simd);
         rows_per_wave = per_wave >= 4 ? 4 : (per_wave >= 3 ? 3 : (per_wave >= 2 ? 2 : 1));
     }
-    if (a.swiglu && rows_per_wave % 2 != 0) rows_per_wave = rows_per_wave == 3 ? 4 : 2;
+    if ((a.swiglu || a.rope_table) && rows_per_wave % 2 != 0) rows_per_wave = rows_per_wave == 3 ? 4 : 2;
     // Up to four activation rows share one pass over the weights (fewer when their staged
     // copies would not fit in 64 KiB of LDS); larger M re-reads the weights per group.
     constexpr int kChunkK = kWave * F::WPP;
@@ -515,10 +558,16 @@ int dispatch(GemvArgs a, int M, int rows_per_wave, int waves_per_simd, hipStream
     if (mcap > 4) mcap = 4;
     const uint16_t* act = a.act;
     uint16_t* y = a.y;
+    const float* rope_table = a.rope_table;
+    const int64_t* kv_slots = a.kv_slots;
     for (int m0 = 0; m0 < M; m0 += mcap) {
         const int mm = (M - m0) < mcap ? (M - m0) : mcap;
         a.act = act + static_cast<size_t>(m0) * a.K;
-        a.y = y + static_cast<size_t>(m0) * (a.swiglu ? a.N / 2 : a.N);
+        a.y = y + static_cast<size_t>(m0) * (a.rope_table ? a.hq * a.d : (a.swiglu ? a.N / 2 : a.N));
+        if (rope_table) {
+            a.rope_table = rope_table + static_cast<size_t>(m0) * a.d;
+            a.kv_slots = kv_slots + m0;
+        }
         int st;
         switch (rows_per_wave) {
             case 1: st = launch_m<F, 1>(mm, a, waves_per_simd, stream); break;
@@ -603,6 +652,49 @@ extern "C" int pie_hip_linear_fused(int format, const uint16_t* act_bf16,
     using namespace pie_hip;
     GemvArgs a{act_bf16, static_cast<const u32x4_t*>(weight), nullptr, nullptr, y_bf16, N, K,
                group_size, beta, norm_weight_bf16, eps, swiglu ? 1 : 0};
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (format) {
+        case PIE_HIP_FMT_INT4B8:
+            if (!scale || group_size <= 0) return PIE_HIP_ERR_INVALID;
+            if (group_size % 32 != 0 || K % group_size != 0) return PIE_HIP_ERR_UNSUPPORTED;
+            a.gscale = static_cast<const uint16_t*>(scale);
+            return dispatch<FmtInt4>(a, M, 0, 0, st);
+        case PIE_HIP_FMT_INT8:
+            if (!scale) return PIE_HIP_ERR_INVALID;
+            a.rscale = scale;
+            return scale_is_bf16 ? dispatch<FmtInt8<true>>(a, M, 0, 0, st)
+                                 : dispatch<FmtInt8<false>>(a, M, 0, 0, st);
+        case PIE_HIP_FMT_FP8:
+            if (!scale) return PIE_HIP_ERR_INVALID;
+            a.rscale = scale;
+            return scale_is_bf16 ? dispatch<FmtFp8<true>>(a, M, 0, 0, st)
+                                 : dispatch<FmtFp8<false>>(a, M, 0, 0, st);
+        case PIE_HIP_FMT_BF16:
+            return dispatch<FmtBf16>(a, M, 0, 0, st);
+        default:
+            return PIE_HIP_ERR_INVALID;
+    }
+}
+
+// The fused q|k|v projection of a decode step with the rotation and the KV-cache write in its
+// epilogue (interleaved RoPE, no per-head q/k norm): replaces the projection followed by
+// qkv_rope_kvwrite_kernel with identical values.
+extern "C" int pie_hip_qkv_rope_fused(int format, const uint16_t* act_bf16,
+                                      const uint16_t* norm_weight_bf16, float eps,
+                                      const void* weight, const void* scale, int scale_is_bf16,
+                                      int group_size, int M, int K, const float* rope_table,
+                                      const int64_t* kv_slots, uint16_t* q_out, uint16_t* k_pages,
+                                      uint16_t* v_pages, int num_q_heads, int num_kv_heads,
+                                      int head_dim, void* stream) {
+    using namespace pie_hip;
+    if (!rope_table || !kv_slots || !q_out || !k_pages || !v_pages || num_q_heads <= 0 ||
+        num_kv_heads <= 0 || head_dim <= 0)
+        return PIE_HIP_ERR_INVALID;
+    if (head_dim < 2 || (head_dim & (head_dim - 1)) != 0) return PIE_HIP_ERR_UNSUPPORTED;
+    const int N = (num_q_heads + 2 * num_kv_heads) * head_dim;
+    GemvArgs a{act_bf16, static_cast<const u32x4_t*>(weight), nullptr, nullptr, q_out, N, K,
+               group_size, 0, norm_weight_bf16, eps, 0, rope_table, kv_slots, k_pages, v_pages,
+               num_q_heads, num_kv_heads, head_dim};
     hipStream_t st = static_cast<hipStream_t>(stream);
     switch (format) {
         case PIE_HIP_FMT_INT4B8:

@@ -483,3 +483,27 @@ def gemm_mfma(act: torch.Tensor, w: WeightView, y: Optional[torch.Tensor] = None
                                      int(swiglu), _stream())
     _check(st, "pie_hip_gemm_mfma")
     return y
+
+
+def qkv_rope_fused(act: torch.Tensor, w: WeightView, table: torch.Tensor, kv_slots: torch.Tensor,
+                   k_pages: torch.Tensor, v_pages: torch.Tensor, hq: int, hk: int, d: int,
+                   norm_weight: Optional[torch.Tensor] = None, eps: float = 1e-5) -> torch.Tensor:
+    """Fused q|k|v projection + interleaved RoPE + KV-cache write (decode rows).  Returns q
+    [M, hq, d]; k / v land in their slots of the pools."""
+    _dev(act, torch.bfloat16, "act")
+    _dev(table, torch.float32, "rope_table")
+    _dev(kv_slots, torch.int64, "kv_slots")
+    _dev(k_pages, torch.bfloat16, "k_pages")
+    _dev(v_pages, torch.bfloat16, "v_pages")
+    M, K = act.shape
+    if K != w.K or w.N != (hq + 2 * hk) * d or tuple(table.shape) != (M, d) or kv_slots.numel() != M:
+        raise KernelError("shape mismatch")
+    if M and int(kv_slots.max()) >= k_pages.numel() // (hk * d):
+        raise KernelError("kv slot out of range")
+    q_out = torch.empty((M, hq, d), dtype=torch.bfloat16, device=act.device)
+    scale_is_bf16 = int(w.scale is not None and w.scale.dtype == torch.bfloat16)
+    _check(kernels().pie_hip_qkv_rope_fused(
+        FMT[w.kind], _ptr(act), _ptr(norm_weight), C.c_float(eps), _ptr(w.data), _ptr(w.scale),
+        scale_is_bf16, w.group_size, M, K, _ptr(table), _ptr(kv_slots), _ptr(q_out), _ptr(k_pages),
+        _ptr(v_pages), hq, hk, d, _stream()), "pie_hip_qkv_rope_fused")
+    return q_out

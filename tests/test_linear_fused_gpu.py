@@ -126,3 +126,42 @@ def test_norm_and_swiglu_together_with_residual_variant(gpu, oracle):
     # beta with swiglu is rejected, beta without is fine
     with pytest.raises(ops.KernelError):
         ops.linear_fused(xg, w_int, y=torch.zeros(M, I, device=gpu, dtype=torch.bfloat16), beta=1, swiglu=True)
+
+
+@pytest.mark.parametrize("kind", ["int4b8", "int8", "fp8", "bf16"])
+@pytest.mark.parametrize("M,hq,hk,d,K", [(1, 8, 2, 64, 512), (3, 4, 4, 128, 1024), (4, 32, 8, 128, 4096)])
+def test_qkv_rope_epilogue_equals_projection_then_rope_kernel(gpu, oracle, kind, M, hq, hk, d, K):
+    """The fused q|k|v projection with RoPE and the KV write in its epilogue must give exactly
+    the bytes of the projection followed by the (separately pinned) rope + KV-write kernel:
+    q, and the touched K / V slots (one token without a slot)."""
+    import torch
+    from pie_amd import ops
+
+    rng = np.random.default_rng(140 + M + hq)
+    N = (hq + 2 * hk) * d
+    wd, mk = make_weight(oracle, rng, kind, N, K)
+    w = mk(gpu)
+    x = oracle.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32))
+    nw = oracle.f32_to_bf16(rng.uniform(0.5, 1.5, K).astype(np.float32))
+    xg, nwg = dev(x, gpu, torch.bfloat16), dev(nw, gpu, torch.bfloat16)
+    pos = rng.integers(0, 500, M).astype(np.int32)
+    inv = oracle.rope_inv_freq(d, 10000.0)
+    tab = ops.rope_table(dev(pos, gpu), dev(inv, gpu), d)
+    slots = rng.permutation(40)[:M].astype(np.int64)
+    if M > 1:
+        slots[1] = -1
+    sg = dev(slots, gpu)
+    pools = [torch.full((40, hk, d), 0.5, device=gpu, dtype=torch.bfloat16) for _ in range(4)]
+    q1 = ops.qkv_rope_fused(xg, w, tab, sg, pools[0], pools[1], hq, hk, d, norm_weight=nwg)
+    packed = ops.linear_fused(xg, w, norm_weight=nwg)
+    q2 = ops.qkv_rope_kvwrite(packed, pools[2], pools[3], tab, sg, hq, hk, d, True)
+    assert np.array_equal(bits(q1), bits(q2))
+    assert np.array_equal(bits(pools[0]), bits(pools[2]))
+    assert np.array_equal(bits(pools[1]), bits(pools[3]))
+    # and against the oracle's projection + rope
+    ref_packed = oracle_linear(oracle, wd, oracle.rmsnorm(x, nw, 1e-5))
+    kp = np.full((40, hk, d), oracle.f32_to_bf16(np.float32(0.5)), np.uint16)
+    vp = kp.copy()
+    tab_np = tab.cpu().numpy()
+    qo = oracle.qkv_rope_kvwrite(ref_packed, kp, vp, tab_np, slots, hq, hk, d, 1)
+    assert (ulp_diff(bits(q1).reshape(M, -1), np.asarray(qo).reshape(M, -1)) <= 2).mean() > 0.97
