@@ -367,7 +367,10 @@ SplitPlan plan_splits(int R, int hk, int max_kv_len) {
     const long long rows = static_cast<long long>(R) * hk;
     // ~12 blocks per CU measured best on batch 64 x U[512, 8192] contexts (5.0 TB/s vs 4.4 at 8)
     const long long want_blocks = 3072;
-    const long long min_ups = 2 * kAttnWaves;
+    // a block should walk >= 512 tokens when that still leaves two blocks per CU (measured:
+    // batch 64 x 1024..2048 tokens runs 8-25 % faster than with 128-token blocks); with few
+    // rows, down to 128 tokens so the machine fills
+    const long long min_ups = rows * ((max_units + 31) / 32) >= 512 ? 32 : 2 * kAttnWaves;
     long long want_split = (want_blocks + rows - 1) / rows;
     if (want_split < 1) want_split = 1;
     long long ups = (max_units + want_split - 1) / want_split;
