@@ -108,6 +108,7 @@ struct SkinnyArgs {
     const int32_t* offsets;     // grouped: [P+1] first row of each problem; null: one problem
     int M;                      // rows when offsets == null
     int N, K, G, g_shift, beta, swiglu, scale_is_bf16;
+    int m_split;                // dense only: blockIdx.y = 16-row pass
     size_t w_stride, scale_stride;  // bytes between problems
 };
 
@@ -140,9 +141,11 @@ __global__ __launch_bounds__(KP* kWave) void skinny_kernel(const SkinnyArgs a) {
     const int wv = __builtin_amdgcn_readfirstlane(tid / kWave);
     const int j = lane & 15, q = lane >> 4;
     const int N = a.N, K = a.K;
-    const int p = blockIdx.y;
-    const int r0 = a.offsets ? a.offsets[p] : 0;
-    const int r1 = a.offsets ? a.offsets[p + 1] : a.M;
+    // blockIdx.y: the problem (expert) of a grouped launch, or — dense launches of small
+    // matrices — the 16-row pass, so that the passes run side by side instead of in a loop
+    const int p = a.offsets ? blockIdx.y : 0;
+    const int r0 = a.offsets ? a.offsets[p] : (a.m_split ? blockIdx.y * 16 : 0);
+    const int r1 = a.offsets ? a.offsets[p + 1] : (a.m_split ? min(a.M, r0 + 16) : a.M);
     if (r1 <= r0) return;
 
     const int T = (N + 15) / 16;
@@ -368,7 +371,7 @@ int launch_cfg(const SkinnyArgs& a, int problems, hipStream_t stream) {
         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
     if (attr != hipSuccess) return PIE_HIP_ERR_LAUNCH;
     const int tiles = (a.N + 15) / 16;
-    const dim3 grid((tiles + NG - 1) / NG, problems);
+    const dim3 grid((tiles + NG - 1) / NG, a.m_split ? (a.M + 15) / 16 : problems);
     hipLaunchKernelGGL((skinny_kernel<F, KP, CK, NG, PW, WL>), grid, dim3(KP * kWave), smem, stream, a);
     return launch_status();
 }
@@ -385,10 +388,15 @@ int launch_skinny(SkinnyArgs a, int problems, hipStream_t stream) {
     }
     if (a.swiglu && (a.N % 2 != 0 || a.beta)) return PIE_HIP_ERR_INVALID;
     if (problems > 65535) return PIE_HIP_ERR_UNSUPPORTED;
+    // Dense matrices small enough to stay in L2 / MALL across passes (<= 16 MB) with more than
+    // one 16-row pass: one block per (tile group, pass) instead of a pass loop inside the block.
+    if (!a.offsets && a.M > 16 && a.M <= 16 * 65535 &&
+        static_cast<size_t>(a.N) * a.K * F::kBytesPer2K / 2 <= (16u << 20))
+        a.m_split = 1;
     // tiles of 16 weight rows per block: as many as still leave two blocks per CU; with few
     // tiles, eight waves split K instead of four.  Paired loads (whole 128-byte lines per row
     // and wave) when K allows.
-    const long tiles = static_cast<long>((a.N + 15) / 16) * problems;
+    const long tiles = static_cast<long>((a.N + 15) / 16) * (a.m_split ? (a.M + 15) / 16 : problems);
     constexpr int W8 = (CK / (8 * LK) >= 2) ? 2 : 1;   // loads per step with eight waves
     if (a.K % (8 * LK) == 0) {
         if (tiles / 8 >= 448) return launch_cfg<F, 4, CK, 8, 4, 2>(a, problems, stream);
