@@ -388,10 +388,12 @@ int launch_skinny(SkinnyArgs a, int problems, hipStream_t stream) {
     }
     if (a.swiglu && (a.N % 2 != 0 || a.beta)) return PIE_HIP_ERR_INVALID;
     if (problems > 65535) return PIE_HIP_ERR_UNSUPPORTED;
-    // Dense matrices small enough to stay in L2 / MALL across passes (<= 16 MB) with more than
-    // one 16-row pass: one block per (tile group, pass) instead of a pass loop inside the block.
+    // Dense matrices with more than one 16-row pass: one block per (tile group, pass) instead
+    // of a pass loop inside the block.  The passes then read the same weights at about the same
+    // time, so all but one of them hit L2 / the 256 MB MALL (measured: batch-64 decode 9.9 ->
+    // 9.0 ms per step); beyond the MALL size the loop form keeps HBM traffic at one pass.
     if (!a.offsets && a.M > 16 && a.M <= 16 * 65535 &&
-        static_cast<size_t>(a.N) * a.K * F::kBytesPer2K / 2 <= (16u << 20))
+        static_cast<size_t>(a.N) * a.K * F::kBytesPer2K / 2 <= (size_t(256) << 20))
         a.m_split = 1;
     // tiles of 16 weight rows per block: as many as still leave two blocks per CU; with few
     // tiles, eight waves split K instead of four.  Paired loads (whole 128-byte lines per row
