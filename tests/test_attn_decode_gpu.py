@@ -137,3 +137,33 @@ def test_baseline_shape_batch64(gpu, oracle):
     q = oracle.f32_to_bf16(rng.standard_normal((64, hq, d)).astype(np.float32))
     o, lse = run_gpu(gpu, q, b, hq, hk, d, ps, int(ctx.max()))
     check(oracle, o, lse, q, b, hq, hk, d, ps)
+
+
+def test_back_to_back_calls_share_workspace(gpu, oracle):
+    """Calls queued in a row over one workspace, with different inputs and different split
+    grids, must each give their own result (no partial of an earlier call is picked up)."""
+    import torch
+
+    from pie_amd import ops
+
+    hq, hk, d, ps = 32, 8, 128, 16
+    cases = []
+    for seed, ctx in [(41, [700, 33, 1500, 0, 260]), (42, [2048]), (43, [90, 900, 64, 1024, 17, 300])]:
+        rng = np.random.default_rng(seed)
+        b = make_paged_batch(rng, ctx, hk, d, ps, f32_to_bf16=oracle.f32_to_bf16)
+        q = oracle.f32_to_bf16(rng.standard_normal((len(ctx), hq, d)).astype(np.float32))
+        ref, _ = run_gpu(gpu, q, b, hq, hk, d, ps, max(ctx), want_lse=False)
+        check(oracle, ref, None, q, b, hq, hk, d, ps)
+        dev = lambda a, dt=None: (lambda t: t.view(dt) if dt is not None else t)(
+            torch.from_numpy(np.ascontiguousarray(a)).to(gpu))
+        cases.append((ref, max(ctx), dev(q, torch.bfloat16), dev(b["k_pages"], torch.bfloat16),
+                      dev(b["v_pages"], torch.bfloat16), dev(b["page_indices"].view(np.int32)),
+                      dev(b["page_indptr"].view(np.int32)), dev(b["last_lens"].view(np.int32))))
+    ws = torch.empty(64 << 20, dtype=torch.uint8, device=gpu)
+    outs = []
+    for it in range(30):   # queued back to back, no host synchronisation in between
+        ref, mx, q, k, v, pi, pp, ll = cases[it % 3]
+        outs.append((it, ops.attention_paged_decode(q, k, v, pi, pp, ll, mx, workspace=ws)))
+    torch.cuda.synchronize()
+    for it, o in outs:
+        assert np.array_equal(o.view(torch.uint16).cpu().numpy(), cases[it % 3][0]), it
