@@ -213,6 +213,45 @@ def attention_extra():
                 dedup_bytes=dedup, note="split kernel + merge kernel per call")
 
 
+def w4a16_sweep_extra():
+    """The W4A16 GEMM sweep of BASELINE's second config: (K, N) x M, int4b8 group 128.  Each
+    (shape, M) is timed from a HIP graph that walks a ring of weight copies larger than the
+    256 MB last-level cache, so every launch streams its weights from HBM.  M <= 4 runs the GEMV,
+    above that the faster of the skinny and the tiled matrix-core GEMM (both reported)."""
+    import torch
+
+    from pie_amd import ops
+
+    dev = torch.device("cuda:0")
+    G = 128
+    out = {}
+    for K, N in ((4096, 4096), (4096, 14336), (14336, 4096)):
+        wbytes = N * K // 2 + N * (K // G) * 2
+        ncopy = max(2, -(-600_000_000 // wbytes))
+        ring = [ops.int4b8_view(torch.randint(-2**31, 2**31 - 1, (N, K // 8), dtype=torch.int32, device=dev),
+                                (torch.rand(N, K // G, device=dev) * 0.015 + 0.005).bfloat16(), G)
+                for _ in range(ncopy)]
+        for M in (1, 8, 32, 128, 2048):
+            act = torch.randn(M, K, device=dev).bfloat16()
+            y = torch.empty(M, N, device=dev, dtype=torch.bfloat16)
+            it = iter(range(10**9))
+            alg = wbytes + M * K * 2 + M * N * 2
+            kernels = {"gemv": ops.linear_fused} if M <= 4 else {}
+            if 4 < M <= 128:
+                kernels["skinny"] = ops.gemm_skinny
+            if M >= 48:
+                kernels["tiled"] = ops.gemm_mfma
+            res = {}
+            for name, fn in kernels.items():
+                t = time_graph(lambda: fn(act, ring[next(it) % ncopy], y=y), ncopy, reps=3)
+                res[name] = dict(us=round(t * 1e6, 1), gbps=round(alg / t / 1e9, 1),
+                                 tflops=round(2.0 * M * N * K / t / 1e12, 1))
+            out[f"K{K}_N{N}_M{M}"] = res
+        del ring
+        torch.cuda.empty_cache()
+    return out
+
+
 def lm_head_extra(drv, model):
     import torch
 
@@ -370,6 +409,7 @@ def main():
     if not args.no_extra:
         extra["decode_attention"] = attention_extra()
         extra["lm_head"] = lm_head_extra(drv, MODEL)
+        extra["w4a16_gemm_sweep"] = w4a16_sweep_extra()
     cpu = None
     if not args.no_cpu:
         cpu = cpu_baseline(drv, MODEL, page_size, total_pages, args.prompt, tokens[0], args.cpu_seconds)
