@@ -317,3 +317,78 @@ def moe_combine(y_routes_bf16, topk_w, out_bf16=None):
     out = np.ascontiguousarray(out)
     lib().orc_moe_combine(_p(yr), _p(w), _p(out), C.c_int(N), C.c_int(K), C.c_int(H), C.c_int(int(add)))
     return out
+
+
+# ---------------------------------------------------------------- samplers
+SAMPLER_KINDS = {"multinomial": 0, "top_k": 1, "top_p": 2, "min_p": 3, "top_k_top_p": 4,
+                 "dist": 6, "raw_logits": 7, "logprob": 8, "logprobs": 9, "entropy": 10}
+
+
+def pcg32_sequence(seed: int, stream: int, n: int) -> np.ndarray:
+    """n outputs of PCG32 seeded like Pcg32(seed, stream) (driver/portable/src/sampler.cpp:31-57)."""
+    out = np.empty(n, np.uint32)
+    lib().orc_pcg32_sequence(C.c_uint64(seed), C.c_uint64(stream), _p(out), C.c_int(n))
+    return out
+
+
+def pcg32_first_uniform(seed: int) -> float:
+    """The uniform a slot with wire seed `seed` draws: first output of the default stream."""
+    f = lib().orc_pcg32_first_uniform
+    f.restype = C.c_float
+    return float(f(C.c_uint64(seed)))
+
+
+def apply_brle_logit_mask(logits_f32, runs) -> np.ndarray:
+    lg = np.array(logits_f32, np.float32, copy=True)
+    r = _c(np.asarray(runs, np.uint32), np.uint32)
+    lib().orc_apply_brle_logit_mask(_p(lg), C.c_int(lg.shape[-1]), _p(r), C.c_size_t(r.size))
+    return lg
+
+
+def softmax_temperature(logits_f32, temperature: float) -> np.ndarray:
+    lg = _c(logits_f32, np.float32)
+    out = np.empty_like(lg)
+    lib().orc_softmax_temperature(_p(lg), C.c_int(lg.size), C.c_float(temperature), _p(out))
+    return out
+
+
+def sample_token(logits_f32, kind, temperature=1.0, top_k=0, top_p=1.0, min_p=0.0, u=None, seed=0):
+    """(token, margin) of one slot (sample_token, driver/portable/src/sampler.cpp:345-409).
+    `u` overrides the uniform the seed would draw."""
+    lg = _c(logits_f32, np.float32)
+    k = SAMPLER_KINDS[kind] if isinstance(kind, str) else int(kind)
+    if u is None:
+        u = pcg32_first_uniform(seed)
+    tok = C.c_uint32(0)
+    mg = C.c_float(0)
+    rc = lib().orc_sample_token(_p(lg), C.c_int(lg.size), C.c_int(k), C.c_float(temperature),
+                                C.c_uint32(top_k), C.c_float(top_p), C.c_float(min_p), C.c_float(u),
+                                C.byref(tok), C.byref(mg))
+    if rc != 0:
+        raise ValueError("sampler kind produces no token")
+    return int(tok.value), float(mg.value)
+
+
+def distribution(logits_f32, temperature: float, k: int):
+    lg = _c(logits_f32, np.float32)
+    ids = np.empty(lg.size, np.uint32)
+    vals = np.empty(lg.size, np.float32)
+    n = lib().orc_distribution(_p(lg), C.c_int(lg.size), C.c_float(temperature), C.c_uint32(k),
+                               _p(ids), _p(vals))
+    return ids[:n].copy(), vals[:n].copy()
+
+
+def logprobs_at(logits_f32, labels) -> np.ndarray:
+    lg = _c(logits_f32, np.float32)
+    lb = _c(np.asarray(labels, np.uint32), np.uint32)
+    out = np.empty(lb.size, np.float32)
+    if lib().orc_logprobs_at(_p(lg), C.c_int(lg.size), _p(lb), C.c_int(lb.size), _p(out)) != 0:
+        raise ValueError("label outside the vocabulary")
+    return out
+
+
+def entropy(logits_f32) -> float:
+    lg = _c(logits_f32, np.float32)
+    f = lib().orc_entropy
+    f.restype = C.c_float
+    return float(f(_p(lg), C.c_int(lg.size)))

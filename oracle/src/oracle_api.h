@@ -34,4 +34,14 @@ void orc_attn_rows(const uint16_t* q, const uint16_t* k_pages, const uint16_t* v
 void orc_topk_softmax(const uint16_t* logits, int32_t* topk_idx, float* topk_w, int N, int E, int K);
 void orc_moe_combine(const uint16_t* y_routes, const float* topk_w, uint16_t* out, int N, int K,
                      int H, int add);
+void orc_pcg32_sequence(uint64_t seed, uint64_t stream, uint32_t* out, int n);
+float orc_pcg32_first_uniform(uint64_t seed);
+void orc_apply_brle_logit_mask(float* logits, int V, const uint32_t* runs, size_t n_runs);
+void orc_softmax_temperature(const float* logits, int V, float temperature, float* probs);
+int orc_sample_token(const float* logits, int V, int kind, float temperature, uint32_t top_k,
+                     float top_p, float min_p, float u, uint32_t* token, float* margin);
+int orc_distribution(const float* logits, int V, float temperature, uint32_t k, uint32_t* ids,
+                     float* vals);
+int orc_logprobs_at(const float* logits, int V, const uint32_t* labels, int n, float* out);
+float orc_entropy(const float* logits, int V);
 #endif
