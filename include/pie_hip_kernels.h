@@ -195,6 +195,46 @@ int pie_hip_moe_combine(const uint16_t* y_routes_bf16, const int32_t* route_pos,
                         const float* topk_weight, uint16_t* out_bf16, int num_tokens, int top_k,
                         int hidden, int add, void* stream);
 
+/*
+ * Sampling beyond greedy argmax, one slot = one sampled logits row.
+ *
+ * pie_hip_sample_gather_logits: out[s, :] = f32(logits[rows[s], :]) (rows == NULL: row s), with
+ * slot s's BRLE logit mask applied: mask_bounds[mask_bounds_indptr[s] .. [s+1]) are the
+ * cumulative ends of the slot's runs; run j (0-based) allows its tokens when j is odd, tokens
+ * past the last run are masked (-inf), a slot with no runs is unconstrained
+ * (apply_brle_logit_mask, driver/portable/src/sampler.cpp:169-198).
+ *
+ * pie_hip_sample: per slot, by `kind` (the wire order of the Sampler variants,
+ * driver/bridge/include/pie_bridge/view.hpp:346-358):
+ *   MULTINOMIAL / TOP_K / TOP_P / MIN_P / TOP_K_TOP_P -> tokens[s]
+ *       (sample_token, driver/portable/src/sampler.cpp:345-409; uniform[s] is the draw the
+ *       reference takes from its per-slot PCG32, made by the caller)
+ *   DIST      -> ids / values [out_indptr[s], out_indptr[s+1]): the most probable tokens of
+ *                softmax(logits / T), descending (run_distribution, :224-251); the range length
+ *                is the caller's k (the whole vocabulary for k = 0)
+ *   LOGPROB / LOGPROBS -> values[i] = log_softmax(logits)[labels[i]] over the slot's range
+ *                (run_logprob / run_logprobs_many, :262-292); labels must be < vocab
+ *   ENTROPY   -> values[out_indptr[s]] (run_entropy, :294-306)
+ *   RAW_LOGITS -> nothing: the f32 row of pie_hip_sample_gather_logits is the payload
+ * Equal probabilities are ordered by ascending token id.  Running sums are taken in double and
+ * compared after rounding to float.  workspace: pie_hip_sample_workspace_bytes(S, vocab).
+ */
+enum {
+    PIE_HIP_SAMPLER_MULTINOMIAL = 0, PIE_HIP_SAMPLER_TOP_K = 1, PIE_HIP_SAMPLER_TOP_P = 2,
+    PIE_HIP_SAMPLER_MIN_P = 3, PIE_HIP_SAMPLER_TOP_K_TOP_P = 4, PIE_HIP_SAMPLER_DIST = 6,
+    PIE_HIP_SAMPLER_RAW_LOGITS = 7, PIE_HIP_SAMPLER_LOGPROB = 8, PIE_HIP_SAMPLER_LOGPROBS = 9,
+    PIE_HIP_SAMPLER_ENTROPY = 10
+};
+size_t pie_hip_sample_workspace_bytes(int num_slots, int vocab);
+int pie_hip_sample_gather_logits(const uint16_t* logits_bf16, const int32_t* rows, float* out_f32,
+                                 const uint32_t* mask_bounds, const int32_t* mask_bounds_indptr,
+                                 int num_slots, int vocab, void* stream);
+int pie_hip_sample(const float* logits_f32, const int32_t* kind, const float* temperature,
+                   const uint32_t* top_k, const float* top_p, const float* min_p,
+                   const float* uniform, const int32_t* out_indptr, const uint32_t* labels,
+                   uint32_t* tokens, float* values, uint32_t* ids, void* workspace,
+                   size_t workspace_bytes, int num_slots, int vocab, void* stream);
+
 /* Measurement hook: the next GEMV kernel this thread launches (any format, M <= 4) is
  * bracketed by the two HIP events (hipEvent_t), so hipEventElapsedTime(start, stop) is that
  * kernel's own duration.  No reference counterpart. */

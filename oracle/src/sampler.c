@@ -19,8 +19,9 @@
  * The reference sorts with std::sort / std::partial_sort, which leave the order of equal
  * probabilities unspecified; here equal probabilities are ordered by ascending token id.
  *
- * orc_sample_token also reports `margin`: the smallest distance (in probability mass) between
- * any comparison that decided the outcome and its flipping point, so a caller comparing against
+ * orc_sample_token also reports `margin`: the smallest distance (in probability mass; relative
+ * for the min-p threshold test) between any comparison that decided the outcome and its
+ * flipping point, so a caller comparing against
  * an implementation with different float summation order can set near-boundary draws aside.
  *
  * Pinned by tests/test_oracle_sampler.py: the published PCG32 demo sequence (seed 42, stream
@@ -204,8 +205,10 @@ int orc_sample_token(const float* logits, int V, int kind, float temperature, ui
         for (; cut < keep; ++cut)
             if (c[cut].p < thr) break;
         if (cut > 0) {
-            note(&mg, (double)c[cut - 1].p - thr);
-            if (cut < keep) note(&mg, (double)thr - c[cut].p);
+            /* p and thr are single float products on both sides: what matters is their
+             * relative distance against a last-bit difference in p */
+            note(&mg, ((double)c[cut - 1].p - thr) / c[cut - 1].p);
+            if (cut < keep) note(&mg, ((double)thr - c[cut].p) / thr);
             keep = cut;
         }
     }

@@ -507,3 +507,84 @@ def qkv_rope_fused(act: torch.Tensor, w: WeightView, table: torch.Tensor, kv_slo
         scale_is_bf16, w.group_size, M, K, _ptr(table), _ptr(kv_slots), _ptr(q_out), _ptr(k_pages),
         _ptr(v_pages), hq, hk, d, _stream()), "pie_hip_qkv_rope_fused")
     return q_out
+
+
+# ---------------------------------------------------------------- sampling
+SAMPLER_KINDS = {"multinomial": 0, "top_k": 1, "top_p": 2, "min_p": 3, "top_k_top_p": 4,
+                 "dist": 6, "raw_logits": 7, "logprob": 8, "logprobs": 9, "entropy": 10}
+
+
+def brle_bounds(runs_per_slot, device) -> tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
+    """Cumulative run ends (u32, saturating) + per-slot offsets for `sample_gather_logits`."""
+    if runs_per_slot is None or not any(len(r) for r in runs_per_slot):
+        return None, None
+    bounds, indptr = [], [0]
+    for runs in runs_per_slot:
+        acc = 0
+        for r in runs:
+            acc = min(acc + int(r), 0xFFFFFFFF)
+            bounds.append(acc)
+        indptr.append(len(bounds))
+    import numpy as np
+    b = torch.from_numpy(np.asarray(bounds, np.uint32).view(np.int32)).to(device)
+    return b, torch.tensor(indptr, dtype=torch.int32, device=device)
+
+
+def sample_gather_logits(logits: torch.Tensor, rows: Optional[torch.Tensor] = None,
+                         mask_runs=None) -> torch.Tensor:
+    """f32 copies of the sampled logits rows with per-slot BRLE logit masks applied
+    (apply_brle_logit_mask, driver/portable/src/sampler.cpp:169-198)."""
+    _dev(logits, torch.bfloat16, "logits")
+    V = logits.shape[1]
+    S = logits.shape[0] if rows is None else rows.numel()
+    if rows is not None:
+        _dev(rows, torch.int32, "rows")
+    bounds, indptr = brle_bounds(mask_runs, logits.device)
+    if mask_runs is not None and len(mask_runs) != S:
+        raise KernelError("one run list per slot expected")
+    out = torch.empty((S, V), dtype=torch.float32, device=logits.device)
+    _check(kernels().pie_hip_sample_gather_logits(_ptr(logits), _ptr(rows), _ptr(out), _ptr(bounds),
+                                                  _ptr(indptr), S, V, _stream()),
+           "pie_hip_sample_gather_logits")
+    return out
+
+
+def sample(logits_f32: torch.Tensor, kinds, temperature, top_k, top_p, min_p, uniform,
+           out_counts=None, labels=None):
+    """Runs every slot's sampler (sample_slot, driver/portable/src/sampler.cpp:308-343).
+    Per-slot python lists in; returns (tokens u32 [S], values f32, ids u32, out_indptr) where
+    slot s's dist / logprob / entropy payload is values[out_indptr[s]:out_indptr[s+1]]."""
+    import numpy as np
+
+    _dev(logits_f32, torch.float32, "logits_f32")
+    S, V = logits_f32.shape
+    dev = logits_f32.device
+    kinds = [SAMPLER_KINDS[k] if isinstance(k, str) else int(k) for k in kinds]
+    counts = list(out_counts) if out_counts is not None else [0] * S
+    indptr = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    total = int(indptr[-1])
+    lab = np.zeros(max(total, 1), np.uint32)
+    if labels is not None:
+        for s in range(S):
+            if labels[s] is not None and len(labels[s]):
+                if max(labels[s]) >= V:
+                    raise KernelError("label outside the vocabulary")
+                lab[indptr[s]:indptr[s + 1]] = labels[s]
+    t = lambda a, dt: torch.from_numpy(np.ascontiguousarray(np.asarray(a, dt))).to(dev)
+    kind_t, temp_t = t(kinds, np.int32), t(temperature, np.float32)
+    topk_t = t(np.asarray(top_k, np.uint32).view(np.int32), np.int32)
+    topp_t, minp_t, u_t = t(top_p, np.float32), t(min_p, np.float32), t(uniform, np.float32)
+    indptr_t = t(indptr, np.int32)
+    lab_t = t(lab.view(np.int32), np.int32)
+    tokens = torch.zeros(S, dtype=torch.int32, device=dev)
+    values = torch.zeros(max(total, 1), dtype=torch.float32, device=dev)
+    ids = torch.zeros(max(total, 1), dtype=torch.int32, device=dev)
+    k = kernels()
+    k.pie_hip_sample_workspace_bytes.restype = C.c_size_t
+    need = int(k.pie_hip_sample_workspace_bytes(S, V))
+    ws = torch.empty(need, dtype=torch.uint8, device=dev)
+    _check(k.pie_hip_sample(_ptr(logits_f32), _ptr(kind_t), _ptr(temp_t), _ptr(topk_t), _ptr(topp_t),
+                            _ptr(minp_t), _ptr(u_t), _ptr(indptr_t), _ptr(lab_t), _ptr(tokens),
+                            _ptr(values), _ptr(ids), _ptr(ws), C.c_size_t(need), S, V, _stream()),
+           "pie_hip_sample")
+    return tokens, values, ids, indptr
