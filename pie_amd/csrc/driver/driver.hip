@@ -57,7 +57,110 @@ uint32_t method_of(const PieFrameDesc& f) {
 struct ResponseStore {
     std::vector<uint32_t> tokens_indptr, tokens, dists_req_indptr, dists_kv_indptr,
         logits_req_indptr, logits_byte_indptr, logprobs_req_indptr, logprobs_val_indptr,
-        entropies_indptr, spec_indptr;
+        entropies_indptr, spec_indptr, dists_ids;
+    std::vector<float> dists_probs, logprobs_values, entropies;
+    std::vector<uint8_t> logits_bytes;
+
+    // Accepted tokens of one request from its slots' tokens: without drafts every slot's token;
+    // with drafts the verifier walk — slot k predicts the token after draft k-1, the matching
+    // prefix is accepted plus one bonus token (resolve_request_output,
+    // driver/portable/src/executor/executor.cpp:204-248).
+    static void resolve_tokens(const uint32_t* slot_tokens, int n_slots,
+                               const std::vector<uint32_t>& drafts, std::vector<uint32_t>& out) {
+        const int n_drafts = static_cast<int>(drafts.size());
+        if (n_drafts == 0 || n_slots < n_drafts + 1) {
+            out.insert(out.end(), slot_tokens, slot_tokens + n_slots);
+            return;
+        }
+        for (int k = 0; k < n_drafts; ++k) {
+            if (slot_tokens[k] != drafts[k]) {
+                out.push_back(slot_tokens[k]);   // the model's own token replaces the rejected draft
+                return;
+            }
+            out.push_back(drafts[k]);
+        }
+        out.push_back(slot_tokens[n_drafts]);
+    }
+
+    // Full response: per request, token slots -> tokens, Distribution -> dists, RawLogits ->
+    // logits bytes (native f32), Logprob(s) -> logprobs, Entropy -> entropies, in slot order
+    // (driver/portable/src/executor/executor.cpp:1343-1394; CSR shape of
+    // driver/bridge/include/pie_bridge/response_builder.hpp:61-165).  `samples` == nullptr:
+    // every slot is a greedy token slot.
+    void build_full(const BatchPlan& plan, const std::vector<uint32_t>& slot_tokens,
+                    const SampleOutputs* samples, int vocab, PieForwardResponseDesc& out) {
+        const int R = plan.R;
+        std::memset(&out, 0, sizeof(out));
+        tokens_indptr.clear(); tokens.clear(); dists_req_indptr.clear(); dists_ids.clear();
+        dists_probs.clear(); logits_req_indptr.clear(); logits_bytes.clear();
+        logprobs_req_indptr.clear(); logprobs_values.clear(); entropies_indptr.clear();
+        entropies.clear();
+        dists_kv_indptr.assign(1, 0);
+        logits_byte_indptr.assign(1, 0);
+        logprobs_val_indptr.assign(1, 0);
+        spec_indptr.assign(static_cast<size_t>(R) + 1, 0);
+        size_t raw_at = 0;
+        for (int r = 0; r < R; ++r) {
+            tokens_indptr.push_back(static_cast<uint32_t>(tokens.size()));
+            dists_req_indptr.push_back(static_cast<uint32_t>(dists_kv_indptr.size() - 1));
+            logits_req_indptr.push_back(static_cast<uint32_t>(logits_byte_indptr.size() - 1));
+            logprobs_req_indptr.push_back(static_cast<uint32_t>(logprobs_val_indptr.size() - 1));
+            entropies_indptr.push_back(static_cast<uint32_t>(entropies.size()));
+            const int s0 = plan.sample_indptr[r], s1 = plan.sample_indptr[r + 1];
+            bool any_special = false;
+            if (samples)
+                for (int s = s0; s < s1; ++s) any_special |= !sampler_is_token_kind(plan.slot_samplers[s].kind);
+            if (!any_special) {
+                resolve_tokens(slot_tokens.data() + s0, s1 - s0, plan.draft_tokens[r], tokens);
+                continue;
+            }
+            for (int s = s0; s < s1; ++s) {
+                const int o0 = samples->out_indptr[s], o1 = samples->out_indptr[s + 1];
+                switch (plan.slot_samplers[s].kind) {
+                    case PIE_SAMPLER_KIND_DIST:
+                        dists_ids.insert(dists_ids.end(), samples->ids.begin() + o0, samples->ids.begin() + o1);
+                        dists_probs.insert(dists_probs.end(), samples->values.begin() + o0, samples->values.begin() + o1);
+                        dists_kv_indptr.push_back(static_cast<uint32_t>(dists_ids.size()));
+                        break;
+                    case PIE_SAMPLER_KIND_RAW_LOGITS: {
+                        const auto* b = reinterpret_cast<const uint8_t*>(samples->raw_logits.data() + raw_at);
+                        logits_bytes.insert(logits_bytes.end(), b, b + static_cast<size_t>(vocab) * sizeof(float));
+                        logits_byte_indptr.push_back(static_cast<uint32_t>(logits_bytes.size()));
+                        break;
+                    }
+                    case PIE_SAMPLER_KIND_LOGPROB: case PIE_SAMPLER_KIND_LOGPROBS:
+                        logprobs_values.insert(logprobs_values.end(), samples->values.begin() + o0, samples->values.begin() + o1);
+                        logprobs_val_indptr.push_back(static_cast<uint32_t>(logprobs_values.size()));
+                        break;
+                    case PIE_SAMPLER_KIND_ENTROPY: entropies.push_back(samples->values[o0]); break;
+                    default: tokens.push_back(slot_tokens[s]); break;
+                }
+                if (plan.slot_samplers[s].kind == PIE_SAMPLER_KIND_RAW_LOGITS) raw_at += vocab;
+            }
+            // raw rows of requests without specials never exist: raw is itself a special kind
+        }
+        tokens_indptr.push_back(static_cast<uint32_t>(tokens.size()));
+        dists_req_indptr.push_back(static_cast<uint32_t>(dists_kv_indptr.size() - 1));
+        logits_req_indptr.push_back(static_cast<uint32_t>(logits_byte_indptr.size() - 1));
+        logprobs_req_indptr.push_back(static_cast<uint32_t>(logprobs_val_indptr.size() - 1));
+        entropies_indptr.push_back(static_cast<uint32_t>(entropies.size()));
+        out.num_requests = static_cast<uint32_t>(R);
+        out.tokens_indptr = {tokens_indptr.data(), tokens_indptr.size()};
+        out.tokens = {tokens.data(), tokens.size()};
+        out.dists_req_indptr = {dists_req_indptr.data(), dists_req_indptr.size()};
+        out.dists_kv_indptr = {dists_kv_indptr.data(), dists_kv_indptr.size()};
+        out.dists_ids = {dists_ids.data(), dists_ids.size()};
+        out.dists_probs = {dists_probs.data(), dists_probs.size()};
+        out.logits_req_indptr = {logits_req_indptr.data(), logits_req_indptr.size()};
+        out.logits_byte_indptr = {logits_byte_indptr.data(), logits_byte_indptr.size()};
+        out.logits_bytes = {logits_bytes.data(), logits_bytes.size()};
+        out.logprobs_req_indptr = {logprobs_req_indptr.data(), logprobs_req_indptr.size()};
+        out.logprobs_val_indptr = {logprobs_val_indptr.data(), logprobs_val_indptr.size()};
+        out.logprobs_values = {logprobs_values.data(), logprobs_values.size()};
+        out.entropies_indptr = {entropies_indptr.data(), entropies_indptr.size()};
+        out.entropies = {entropies.data(), entropies.size()};
+        out.spec_indptr = {spec_indptr.data(), spec_indptr.size()};
+    }
 
     // R requests, every list empty except tokens (per-request CSR from sample_indptr).
     void build(int R, const std::vector<int32_t>& sample_indptr, const std::vector<uint32_t>& toks,
@@ -111,6 +214,7 @@ struct PieHipDriver {
     std::string caps;
     ResponseStore store;
     std::vector<uint32_t> toks;
+    SampleOutputs samples;
     std::string last_error;
 
     explicit PieHipDriver(const DriverConfig& c) : cfg(c) {
@@ -166,15 +270,14 @@ struct PieHipDriver {
             const BatchPlan plan = plan_forward(f, exec->page_size(), exec->total_pages());
             if (plan.has_user_masks)
                 throw std::runtime_error("forward: custom attention masks are not supported by this driver yet");
-            if (!plan.all_greedy && !plan.sample_rows.empty())
-                throw std::runtime_error("forward: only greedy (temperature 0) token samplers are supported yet");
             if (R > cfg.batching.max_forward_requests)
                 throw std::runtime_error("forward: batch exceeds max_forward_requests");
             const uint32_t plan_us = us_since(t0);
             ForwardTimings ft;
-            exec->forward(plan, toks, &ft);
+            const bool sampling = !plan.all_greedy && !plan.sample_rows.empty();
+            exec->forward(plan, toks, &ft, sampling ? &samples : nullptr);
             t0 = clk::now();
-            store.build(plan.R, plan.sample_indptr, toks, out);
+            store.build_full(plan, toks, sampling ? &samples : nullptr, cfg.model.vocab, out);
             out.probe_wire_parse_us = 0;
             out.probe_plan_us = plan_us;
             out.probe_h2d_us = ft.h2d_us;

@@ -181,6 +181,8 @@ Executor::~Executor() {
                     static_cast<void*>(moe_offsets_), static_cast<void*>(moe_route_token_),
                     static_cast<void*>(moe_route_pos_)})
         if (p) (void)hipFree(p);
+    for (Growable* g : {&samp_f32_, &samp_ws_, &samp_in_dev_, &samp_in_host_, &samp_out_dev_, &samp_out_host_})
+        g->release();
     if (in_host_) (void)hipHostFree(in_host_);
     if (out_host_) (void)hipHostFree(out_host_);
     if (stream_) (void)hipStreamDestroy(stream_);
@@ -300,11 +302,203 @@ void Executor::body(int N, int S, int max_kv_len) {
         head.K = H;
         linear_fused(head, xs_, model_.final_norm, m.rms_eps, logits_, n, 0, 0, xn_, s);
         PIE_KERNEL(pie_hip_argmax(logits_, out_tokens_ + s0, n, m.vocab, s));
+        if (samp_gather_in_body_) {   // more sampled rows than one chunk: keep each chunk's f32 rows
+            const auto* in = static_cast<const unsigned char*>(samp_in_dev_.ptr);
+            PIE_KERNEL(pie_hip_sample_gather_logits(
+                logits_, nullptr, static_cast<float*>(samp_f32_.ptr) + static_cast<size_t>(s0) * m.vocab,
+                samp_.n_bounds ? reinterpret_cast<const uint32_t*>(in + samp_.bounds) : nullptr,
+                samp_.n_bounds ? reinterpret_cast<const int32_t*>(in + samp_.bounds_indptr) + s0 : nullptr,
+                n, m.vocab, s));
+        }
     }
 }
 
+void Executor::Growable::ensure(size_t bytes) {
+    if (bytes <= cap) return;
+    release();
+    const size_t want = std::max<size_t>(bytes, 256);
+    if (pinned) PIE_HIP_CHECK(hipHostMalloc(&ptr, want, hipHostMallocDefault));
+    else PIE_HIP_CHECK(hipMalloc(&ptr, want));
+    cap = want;
+}
+
+void Executor::Growable::release() {
+    if (ptr) (void)(pinned ? hipHostFree(ptr) : hipFree(ptr));
+    ptr = nullptr;
+    cap = 0;
+}
+
+namespace {
+
+// The reference's per-slot generator (Pcg32, driver/portable/src/sampler.cpp:31-57): PCG-XSH-RR
+// 64/32, seeded in the canonical two steps on the default stream; a slot draws one uniform,
+// the top 24 bits of the first output.
+float pcg32_first_uniform(uint64_t seed) {
+    const uint64_t inc = (0xda3e39cb94b95bdbULL << 1u) | 1u;
+    uint64_t state = 0;
+    state = state * 6364136223846793005ULL + inc;
+    state += seed;
+    state = state * 6364136223846793005ULL + inc;
+    const uint64_t old = state;
+    const uint32_t xorshifted = static_cast<uint32_t>(((old >> 18u) ^ old) >> 27u);
+    const uint32_t rot = static_cast<uint32_t>(old >> 59u);
+    const uint32_t r = (xorshifted >> rot) | (xorshifted << ((32u - rot) & 31u));
+    return static_cast<float>(r >> 8) * (1.0f / 16777216.0f);
+}
+
+}  // namespace
+
+// Host half of the sampler stage: per-slot parameter arrays, uniforms, payload ranges, BRLE
+// bounds — staged in pinned memory and sent to the device ahead of the forward body.
+void Executor::prepare_samplers(const BatchPlan& plan) {
+    const int S = static_cast<int>(plan.sample_rows.size());
+    const int V = cfg_.model.vocab;
+    if (static_cast<int>(plan.slot_samplers.size()) != S)
+        throw std::runtime_error("executor: one sampler per sampling slot expected");
+    std::vector<int32_t> out_indptr(static_cast<size_t>(S) + 1, 0), bounds_indptr(static_cast<size_t>(S) + 1, 0);
+    std::vector<uint32_t> bounds;
+    for (int r = 0, s = 0; r < plan.R; ++r) {
+        const auto& runs = plan.logit_mask_runs[r];
+        for (; s < plan.sample_indptr[r + 1]; ++s) {
+            uint64_t acc = 0;
+            for (uint32_t len : runs) {
+                acc = std::min<uint64_t>(acc + len, 0xFFFFFFFFull);
+                bounds.push_back(static_cast<uint32_t>(acc));
+            }
+            bounds_indptr[s + 1] = static_cast<int32_t>(bounds.size());
+        }
+    }
+    for (int s = 0; s < S; ++s) {
+        const SlotSampler& sp = plan.slot_samplers[s];
+        int n = 0;
+        switch (sp.kind) {
+            case PIE_SAMPLER_KIND_MULTINOMIAL: case PIE_SAMPLER_KIND_TOP_K: case PIE_SAMPLER_KIND_TOP_P:
+            case PIE_SAMPLER_KIND_MIN_P: case PIE_SAMPLER_KIND_TOP_K_TOP_P: case PIE_SAMPLER_KIND_RAW_LOGITS:
+                break;
+            case PIE_SAMPLER_KIND_DIST:
+                n = sp.top_k > 0 ? static_cast<int>(std::min<uint32_t>(sp.top_k, static_cast<uint32_t>(V))) : V;
+                break;
+            case PIE_SAMPLER_KIND_LOGPROB: case PIE_SAMPLER_KIND_LOGPROBS:
+                n = static_cast<int>(sp.labels_end - sp.labels_begin);
+                if (n == 0) throw std::runtime_error("sampler: Logprob slot has no labels");
+                for (uint32_t i = sp.labels_begin; i < sp.labels_end; ++i)
+                    if (plan.label_ids[i] >= static_cast<uint32_t>(V))
+                        throw std::runtime_error("sampler: Logprob label id out of vocab");
+                break;
+            case PIE_SAMPLER_KIND_ENTROPY: n = 1; break;
+            default:
+                throw std::runtime_error("sampler: unknown type " + std::to_string(static_cast<int>(sp.kind)));
+        }
+        out_indptr[s + 1] = out_indptr[s] + n;
+    }
+    const int payload = out_indptr[S];
+    SampLayout L{};
+    L.slots = S;
+    L.payload = payload;
+    L.n_bounds = static_cast<int>(bounds.size());
+    size_t o = 0;
+    auto take = [&](size_t bytes) { const size_t at = o; o = align_up(o + bytes, 16); return at; };
+    L.kind = take(4ull * S);
+    L.temperature = take(4ull * S);
+    L.top_k = take(4ull * S);
+    L.top_p = take(4ull * S);
+    L.min_p = take(4ull * S);
+    L.uniform = take(4ull * S);
+    L.out_indptr = take(4ull * (S + 1));
+    L.labels = take(4ull * std::max(payload, 1));
+    L.bounds_indptr = take(4ull * (S + 1));
+    L.bounds = take(4ull * std::max<size_t>(bounds.size(), 1));
+    L.total = o;
+    o = 0;
+    L.o_tokens = take(4ull * S);
+    L.o_values = take(4ull * std::max(payload, 1));
+    L.o_ids = take(4ull * std::max(payload, 1));
+    L.o_total = o;
+    samp_ = L;
+
+    samp_in_host_.pinned = true;
+    samp_out_host_.pinned = true;
+    samp_in_host_.ensure(L.total);
+    samp_in_dev_.ensure(L.total);
+    samp_out_dev_.ensure(L.o_total);
+    samp_out_host_.ensure(L.o_total);
+    samp_f32_.ensure(static_cast<size_t>(S) * V * sizeof(float));
+    samp_ws_.ensure(pie_hip_sample_workspace_bytes(S, V));
+
+    auto* h = static_cast<unsigned char*>(samp_in_host_.ptr);
+    std::memset(h, 0, L.total);
+    auto* kind = reinterpret_cast<int32_t*>(h + L.kind);
+    auto* temp = reinterpret_cast<float*>(h + L.temperature);
+    auto* top_k = reinterpret_cast<uint32_t*>(h + L.top_k);
+    auto* top_p = reinterpret_cast<float*>(h + L.top_p);
+    auto* min_p = reinterpret_cast<float*>(h + L.min_p);
+    auto* uni = reinterpret_cast<float*>(h + L.uniform);
+    auto* labels = reinterpret_cast<uint32_t*>(h + L.labels);
+    for (int s = 0; s < S; ++s) {
+        const SlotSampler& sp = plan.slot_samplers[s];
+        kind[s] = sp.kind;
+        temp[s] = sp.temperature;
+        top_k[s] = sp.top_k;
+        top_p[s] = sp.top_p;
+        min_p[s] = sp.min_p;
+        // no caller seed: a process-wide counter, as the reference's default_rng_seed (:62-65)
+        const uint64_t seed = sp.seed != 0 ? sp.seed : (0x9E3779B97F4A7C15ULL ^ unseeded_draws_++);
+        uni[s] = pcg32_first_uniform(seed);
+        for (uint32_t i = sp.labels_begin; i < sp.labels_end; ++i)
+            labels[out_indptr[s] + (i - sp.labels_begin)] = plan.label_ids[i];
+    }
+    std::memcpy(h + L.out_indptr, out_indptr.data(), 4ull * (S + 1));
+    std::memcpy(h + L.bounds_indptr, bounds_indptr.data(), 4ull * (S + 1));
+    if (!bounds.empty()) std::memcpy(h + L.bounds, bounds.data(), 4ull * bounds.size());
+    PIE_HIP_CHECK(hipMemcpyAsync(samp_in_dev_.ptr, h, L.total, hipMemcpyHostToDevice, stream_));
+}
+
+// Device half: f32 rows (+ masks) unless the body gathered them chunk by chunk, one sampler
+// block per slot, results back through pinned memory.  Ends with the stream drained.
+void Executor::run_samplers(const BatchPlan& plan, SampleOutputs& out) {
+    const int S = samp_.slots, V = cfg_.model.vocab;
+    const auto* in = static_cast<const unsigned char*>(samp_in_dev_.ptr);
+    auto* od = static_cast<unsigned char*>(samp_out_dev_.ptr);
+    float* f32 = static_cast<float*>(samp_f32_.ptr);
+    if (!samp_gather_in_body_) {
+        PIE_KERNEL(pie_hip_sample_gather_logits(
+            logits_, nullptr, f32, samp_.n_bounds ? reinterpret_cast<const uint32_t*>(in + samp_.bounds) : nullptr,
+            samp_.n_bounds ? reinterpret_cast<const int32_t*>(in + samp_.bounds_indptr) : nullptr, S, V, stream_));
+    }
+    PIE_HIP_CHECK(hipMemsetAsync(od, 0, samp_.o_total, stream_));   // eager stage, never captured
+    PIE_KERNEL(pie_hip_sample(
+        f32, reinterpret_cast<const int32_t*>(in + samp_.kind), reinterpret_cast<const float*>(in + samp_.temperature),
+        reinterpret_cast<const uint32_t*>(in + samp_.top_k), reinterpret_cast<const float*>(in + samp_.top_p),
+        reinterpret_cast<const float*>(in + samp_.min_p), reinterpret_cast<const float*>(in + samp_.uniform),
+        reinterpret_cast<const int32_t*>(in + samp_.out_indptr), reinterpret_cast<const uint32_t*>(in + samp_.labels),
+        reinterpret_cast<uint32_t*>(od + samp_.o_tokens), reinterpret_cast<float*>(od + samp_.o_values),
+        reinterpret_cast<uint32_t*>(od + samp_.o_ids), samp_ws_.ptr, samp_ws_.cap, S, V, stream_));
+    auto* oh = static_cast<unsigned char*>(samp_out_host_.ptr);
+    PIE_HIP_CHECK(hipMemcpyAsync(oh, od, samp_.o_total, hipMemcpyDeviceToHost, stream_));
+    out.raw_logits.clear();
+    size_t n_raw = 0;
+    for (const SlotSampler& sp : plan.slot_samplers) n_raw += sp.kind == PIE_SAMPLER_KIND_RAW_LOGITS;
+    out.raw_logits.resize(n_raw * static_cast<size_t>(V));
+    PIE_HIP_CHECK(hipStreamSynchronize(stream_));
+    size_t at = 0;
+    for (int s = 0; s < S; ++s)
+        if (plan.slot_samplers[s].kind == PIE_SAMPLER_KIND_RAW_LOGITS) {
+            PIE_HIP_CHECK(hipMemcpy(out.raw_logits.data() + at, f32 + static_cast<size_t>(s) * V,
+                                    static_cast<size_t>(V) * sizeof(float), hipMemcpyDeviceToHost));
+            at += V;
+        }
+    const auto* tok = reinterpret_cast<const uint32_t*>(oh + samp_.o_tokens);
+    out.tokens.assign(tok, tok + S);
+    const auto* val = reinterpret_cast<const float*>(oh + samp_.o_values);
+    out.values.assign(val, val + samp_.payload);
+    const auto* ids = reinterpret_cast<const uint32_t*>(oh + samp_.o_ids);
+    out.ids.assign(ids, ids + samp_.payload);
+    const auto* ip = reinterpret_cast<const int32_t*>(static_cast<const unsigned char*>(samp_in_host_.ptr) + samp_.out_indptr);
+    out.out_indptr.assign(ip, ip + S + 1);
+}
+
 void Executor::forward(const BatchPlan& plan, std::vector<uint32_t>& tokens_out,
-                       ForwardTimings* t) {
+                       ForwardTimings* t, SampleOutputs* samples) {
     const int N = plan.N, S = static_cast<int>(plan.sample_rows.size());
     if (N <= 0) throw std::runtime_error("executor: empty plan");
     if (N > max_tokens_) throw std::runtime_error("executor: batch exceeds max_forward_tokens");
@@ -323,10 +517,18 @@ void Executor::forward(const BatchPlan& plan, std::vector<uint32_t>& tokens_out,
     if (S) std::memcpy(in_host_ + in.off_sample_rows, plan.sample_rows.data(), static_cast<size_t>(S) * 4);
     std::memcpy(in_host_ + in.off_pages, plan.page_indices.data(), plan.page_indices.size() * 4);
     PIE_HIP_CHECK(hipMemcpyAsync(in_dev_, in_host_, used, hipMemcpyHostToDevice, stream_));
+    const bool sampling = !plan.all_greedy && S > 0;
+    const int chunk = static_cast<int>(std::min<size_t>(max_tokens_, 2 * static_cast<size_t>(cfg_.batching.max_forward_requests)));
+    samp_gather_in_body_ = false;
+    if (sampling) {
+        if (!samples) throw std::runtime_error("executor: a sampling plan needs a SampleOutputs");
+        prepare_samplers(plan);
+        samp_gather_in_body_ = S > chunk;   // logits_ keeps one chunk of rows only
+    }
     if (t) t->h2d_us = us_since(t0);
 
     t0 = clk::now();
-    const bool use_graph = cfg_.runtime.use_graphs && plan.pure_decode;
+    const bool use_graph = cfg_.runtime.use_graphs && plan.pure_decode && !samp_gather_in_body_;
     if (use_graph) {
         // The split grid depends on the context bound only through 512-token buckets.
         const int bucket = (plan.max_kv_len + 511) / 512 * 512;
@@ -360,6 +562,11 @@ void Executor::forward(const BatchPlan& plan, std::vector<uint32_t>& tokens_out,
     PIE_HIP_CHECK(hipStreamSynchronize(stream_));
     if (t) t->sync_us = us_since(t0);
     tokens_out.assign(out_host_, out_host_ + S);
+    if (sampling) {
+        run_samplers(plan, *samples);
+        tokens_out = samples->tokens;
+        if (t) t->sync_us = us_since(t0);
+    }
     const int cap = static_cast<int>(std::min<size_t>(max_tokens_, 2 * static_cast<size_t>(cfg_.batching.max_forward_requests)));
     last_logit_rows_ = S == 0 ? 0 : ((S - 1) % cap) + 1;
 }

@@ -35,6 +35,18 @@ struct ForwardTimings {
     uint32_t h2d_us = 0, launch_us = 0, sync_us = 0;
 };
 
+// What the non-greedy samplers of one forward pass produced, per sampling slot (slot order =
+// BatchPlan::sample_rows).  Slot s's Distribution / Logprob(s) / Entropy payload is
+// values / ids [out_indptr[s], out_indptr[s+1]); RawLogits slots own `vocab` floats each in
+// raw_logits, in slot order.
+struct SampleOutputs {
+    std::vector<uint32_t> tokens;
+    std::vector<float> values;
+    std::vector<uint32_t> ids;
+    std::vector<int32_t> out_indptr;
+    std::vector<float> raw_logits;
+};
+
 class Executor {
   public:
     Executor(const DriverConfig& cfg, Model& model);
@@ -42,8 +54,11 @@ class Executor {
     Executor(const Executor&) = delete;
     Executor& operator=(const Executor&) = delete;
 
-    // Runs one forward pass; greedy tokens for plan.sample_rows land in tokens_out.
-    void forward(const BatchPlan& plan, std::vector<uint32_t>& tokens_out, ForwardTimings* t);
+    // Runs one forward pass; greedy tokens for plan.sample_rows land in tokens_out.  A plan that
+    // is not all-greedy also runs every slot's sampler on the device and fills `samples`
+    // (required then); tokens_out then holds the samplers' tokens.
+    void forward(const BatchPlan& plan, std::vector<uint32_t>& tokens_out, ForwardTimings* t,
+                 SampleOutputs* samples = nullptr);
 
     // KV page copies inside the device pool (every layer, K and V).
     void copy_pages_d2d(const uint32_t* srcs, const uint32_t* dsts, size_t n);
@@ -63,6 +78,8 @@ class Executor {
 
   private:
     void body(int N, int S, int max_kv_len);
+    void prepare_samplers(const BatchPlan& plan);
+    void run_samplers(const BatchPlan& plan, SampleOutputs& out);
     void moe_block(const LayerWeights& w, int N, hipStream_t s);
     void alloc_kv();
 
@@ -97,6 +114,25 @@ class Executor {
     unsigned char* in_host_ = nullptr;
     unsigned char* in_dev_ = nullptr;
     uint32_t* out_host_ = nullptr;  // pinned
+
+    // Sampler stage (allocated on first use, grown on demand; never touched by captured graphs
+    // except the per-chunk logits gather of batches with more sampled rows than one chunk).
+    struct Growable {
+        void* ptr = nullptr;
+        size_t cap = 0;
+        bool pinned = false;
+        void ensure(size_t bytes);
+        void release();
+    };
+    Growable samp_f32_, samp_ws_, samp_in_dev_, samp_in_host_, samp_out_dev_, samp_out_host_;
+    struct SampLayout {
+        size_t kind, temperature, top_k, top_p, min_p, uniform, out_indptr, labels, bounds_indptr,
+            bounds, total;
+        size_t o_tokens, o_values, o_ids, o_total;
+        int slots = 0, payload = 0, n_bounds = 0;
+    } samp_{};
+    bool samp_gather_in_body_ = false;
+    uint64_t unseeded_draws_ = 0;
 
     std::map<std::tuple<int, int, int>, hipGraphExec_t> graphs_;
     int last_logit_rows_ = 0;

@@ -8,6 +8,9 @@
 //   physical slot           driver/portable/src/plan.hpp:36-45
 //   synthesised causal mask driver/portable/src/plan.cpp:139-173
 //   pure-decode / all-greedy driver/portable/src/executor/executor.cpp:537-543, :568-586
+//   per-slot sampler params  driver/portable/src/plan.cpp:408-453 with the AoS -> SoA field
+//                           mapping of driver/bridge/include/pie_bridge/view.hpp:441-496
+//   logit masks, drafts     driver/portable/src/plan.cpp:379-406, :455-466
 // The request count comes from qo_indptr (as the CUDA driver does,
 // driver/cuda/src/executor/executor.cpp:2240); a non-empty context_ids must agree with it.
 #pragma once
@@ -21,6 +24,18 @@
 
 namespace pie_hip_driver {
 
+// One sampling slot's sampler, fields as the reference's SamplerParams
+// (driver/portable/src/sampler.hpp:41-51) but with the wire kind.
+struct SlotSampler {
+    uint8_t kind = PIE_SAMPLER_KIND_TOP_P;
+    float temperature = 0.f;
+    uint32_t top_k = 0;       // TopK / TopKTopP: k; Dist: number of entries (0 = whole vocabulary)
+    float top_p = 1.f;
+    float min_p = 0.f;
+    uint32_t seed = 0;        // 0 = no caller seed
+    uint32_t labels_begin = 0, labels_end = 0;   // range in BatchPlan::label_ids
+};
+
 struct BatchPlan {
     int R = 0;  // requests
     int N = 0;  // token rows
@@ -33,6 +48,10 @@ struct BatchPlan {
     std::vector<uint32_t> page_indices;    // copy of the wire list (uploaded as is)
     std::vector<int32_t> sample_rows;      // global token rows to sample, request-major
     std::vector<int32_t> sample_indptr;    // [R+1]
+    std::vector<SlotSampler> slot_samplers;  // one per sample row
+    std::vector<uint32_t> label_ids;         // Logprob / Logprobs labels of all slots
+    std::vector<std::vector<uint32_t>> logit_mask_runs;  // [R] BRLE runs (empty = no constraint)
+    std::vector<std::vector<uint32_t>> draft_tokens;     // [R] speculative drafts to verify
     int max_kv_len = 0;
     bool pure_decode = false;  // every request has exactly one token row, no user masks
     bool all_greedy = false;   // every sampling slot is a token sampler with temperature ~ 0
@@ -60,6 +79,28 @@ inline bool masks_are_synthesised_causal(const PieForwardRequestDesc& f) {
 
 // Token-producing sampler kinds on the wire (Multinomial, TopK, TopP, MinP, TopKTopP).
 inline bool sampler_is_token_kind(uint8_t kind) { return kind <= PIE_SAMPLER_KIND_TOP_K_TOP_P; }
+
+// Wire sampler -> per-slot parameters; fields a variant does not carry take the neutral value.
+inline SlotSampler slot_sampler_of(const PieSamplerDesc& s, std::vector<uint32_t>& label_ids) {
+    SlotSampler o;
+    o.kind = s.kind;
+    o.temperature = s.temperature;
+    o.seed = s.seed;
+    switch (s.kind) {
+        case PIE_SAMPLER_KIND_TOP_K: o.top_k = s.k; break;
+        case PIE_SAMPLER_KIND_TOP_P: o.top_p = s.p; break;
+        case PIE_SAMPLER_KIND_MIN_P: o.min_p = s.p; break;
+        case PIE_SAMPLER_KIND_TOP_K_TOP_P: o.top_k = s.k; o.top_p = s.p; break;
+        case PIE_SAMPLER_KIND_DIST: o.top_k = s.num_tokens; break;
+        default: break;
+    }
+    o.labels_begin = static_cast<uint32_t>(label_ids.size());
+    if (s.kind == PIE_SAMPLER_KIND_LOGPROB) label_ids.push_back(s.token_id);
+    else if (s.kind == PIE_SAMPLER_KIND_LOGPROBS)
+        label_ids.insert(label_ids.end(), s.token_ids.ptr, s.token_ids.ptr + s.token_ids.len);
+    o.labels_end = static_cast<uint32_t>(label_ids.size());
+    return o;
+}
 
 inline BatchPlan plan_forward(const PieForwardRequestDesc& f, int page_size, int total_pages) {
     BatchPlan p;
@@ -102,6 +143,15 @@ inline BatchPlan plan_forward(const PieForwardRequestDesc& f, int page_size, int
     p.seq_len.resize(R);
     p.page_indices.assign(f.kv_page_indices.ptr, f.kv_page_indices.ptr + f.kv_page_indices.len);
     p.sample_indptr.assign(1, 0);
+    p.logit_mask_runs.resize(R);
+    p.draft_tokens.resize(R);
+    const bool has_logit_masks = f.logit_mask_indptr.len == n_plus_1;
+    const bool has_drafts = f.spec_indptr.len == n_plus_1;
+    if (has_logit_masks && f.logit_mask_indptr.ptr[R] > f.logit_masks.len)
+        throw std::runtime_error("plan: logit_mask_indptr exceeds logit_masks");
+    if (has_drafts && (f.spec_indptr.ptr[R] > f.spec_token_ids.len ||
+                       f.spec_indptr.ptr[R] > f.spec_position_ids.len))
+        throw std::runtime_error("plan: spec_indptr exceeds the draft arrays");
     p.has_user_masks = !masks_are_synthesised_causal(f);
     p.pure_decode = !p.has_user_masks;
     p.all_greedy = true;
@@ -157,10 +207,40 @@ inline BatchPlan plan_forward(const PieForwardRequestDesc& f, int page_size, int
             const size_t si = f.sampler_indptr.ptr[r] + (n_samplers == n_slots ? static_cast<size_t>(k - s_start) : 0);
             const PieSamplerDesc& s = f.samplers.ptr[si];
             if (!sampler_is_token_kind(s.kind) || !(s.temperature <= 1e-5f)) p.all_greedy = false;
+            p.slot_samplers.push_back(slot_sampler_of(s, p.label_ids));
+        }
+        if (has_drafts && !prefill_only) {
+            // each draft is verified at the row holding its position; the extra slots reuse the
+            // request's first sampler
+            const uint32_t d0 = f.spec_indptr.ptr[r], d1 = f.spec_indptr.ptr[r + 1];
+            for (uint32_t k = d0; k < d1; ++k) {
+                const int draft_pos = static_cast<int>(f.spec_position_ids.ptr[k]);
+                int idx = -1;
+                for (int i = qo_start; i < qo_end; ++i)
+                    if (static_cast<int>(f.position_ids.ptr[i]) == draft_pos) {
+                        idx = i;
+                        break;
+                    }
+                if (idx < 0)
+                    throw std::runtime_error("plan: spec draft at position " + std::to_string(draft_pos) +
+                                             " not found in request " + std::to_string(r) + "'s qo range");
+                p.draft_tokens[r].push_back(f.spec_token_ids.ptr[k]);
+                p.sample_rows.push_back(idx);
+                const PieSamplerDesc& s = f.samplers.ptr[f.sampler_indptr.ptr[r]];
+                if (!sampler_is_token_kind(s.kind) || !(s.temperature <= 1e-5f)) p.all_greedy = false;
+                p.slot_samplers.push_back(slot_sampler_of(s, p.label_ids));
+            }
+        }
+        if (has_logit_masks && !prefill_only) {
+            for (uint32_t i = f.logit_mask_indptr.ptr[r]; i < f.logit_mask_indptr.ptr[r + 1]; ++i) {
+                const PieBrleDesc& b = f.logit_masks.ptr[i];
+                p.logit_mask_runs[r].insert(p.logit_mask_runs[r].end(), b.buffer.ptr,
+                                            b.buffer.ptr + b.buffer.len);
+            }
+            if (!p.logit_mask_runs[r].empty()) p.all_greedy = false;
         }
         p.sample_indptr.push_back(static_cast<int32_t>(p.sample_rows.size()));
     }
-    if (f.logit_masks.len != 0) p.all_greedy = false;
     return p;
 }
 

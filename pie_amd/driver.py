@@ -170,7 +170,9 @@ class ForwardFrame:
                  kv_last_page_lens, qo_indptr, sampling_indices=None, sampling_indptr=None,
                  samplers: Optional[Sequence[dict]] = None, sampler_indptr=None,
                  context_ids=None, masks: Optional[Sequence[Sequence[int]]] = None,
-                 driver_id: int = 0):
+                 driver_id: int = 0, logit_masks: Optional[Sequence[Sequence[int]]] = None,
+                 logit_mask_indptr=None, spec_token_ids=None, spec_position_ids=None,
+                 spec_indptr=None):
         R = len(qo_indptr) - 1
         self._keep = []
 
@@ -206,6 +208,10 @@ class ForwardFrame:
             arr[i].seed = s.get("seed", 0)
             arr[i].k = s.get("k", 0)
             arr[i].p = s.get("p", 1.0)
+            arr[i].num_tokens = s.get("num_tokens", 0)
+            arr[i].token_id = s.get("token_id", 0)
+            if s.get("token_ids") is not None:
+                arr[i].token_ids = u32(s["token_ids"])
         self._keep.append(arr)
         f.samplers = SamplerSlice(C.cast(arr, C.POINTER(SamplerDesc)), len(samplers))
         f.sampler_indptr = u32(sampler_indptr)
@@ -221,6 +227,18 @@ class ForwardFrame:
                 marr[i].total_size = int(np.sum(runs))
             self._keep.append(marr)
             f.masks = BrleSlice(C.cast(marr, C.POINTER(BrleDesc)), len(masks))
+        if logit_masks is not None:   # one BRLE per entry; logit_mask_indptr partitions them per request
+            larr = (BrleDesc * max(len(logit_masks), 1))()
+            for i, runs in enumerate(logit_masks):
+                larr[i].buffer = u32(runs)
+                larr[i].total_size = int(np.sum(runs))
+            self._keep.append(larr)
+            f.logit_masks = BrleSlice(C.cast(larr, C.POINTER(BrleDesc)), len(logit_masks))
+            f.logit_mask_indptr = u32(logit_mask_indptr)
+        if spec_indptr is not None:
+            f.spec_token_ids = u32(spec_token_ids)
+            f.spec_position_ids = u32(spec_position_ids)
+            f.spec_indptr = u32(spec_indptr)
         f.single_token_mode = 1 if len(token_ids) == R else 0
 
 
@@ -256,12 +274,50 @@ class ForwardResult:
             "logprobs_val_indptr": fr.logprobs_val_indptr.len,
             "entropies_indptr": fr.entropies_indptr.len, "spec_indptr": fr.spec_indptr.len,
         }
+        f32 = lambda sl: np.ctypeslib.as_array(sl.ptr, shape=(sl.len,)).copy() if sl.len else np.zeros(0, np.float32)
+        self.dists_req_indptr = _u32_list(fr.dists_req_indptr)
+        self.dists_kv_indptr = _u32_list(fr.dists_kv_indptr)
+        self.dists_ids = _u32_list(fr.dists_ids)
+        self.dists_probs = f32(fr.dists_probs)
+        self.logits_req_indptr = _u32_list(fr.logits_req_indptr)
+        self.logits_byte_indptr = _u32_list(fr.logits_byte_indptr)
+        self.logits_bytes = C.string_at(fr.logits_bytes.ptr, fr.logits_bytes.len) if fr.logits_bytes.len else b""
+        self.logprobs_req_indptr = _u32_list(fr.logprobs_req_indptr)
+        self.logprobs_val_indptr = _u32_list(fr.logprobs_val_indptr)
+        self.logprobs_values = f32(fr.logprobs_values)
+        self.entropies_indptr = _u32_list(fr.entropies_indptr)
+        self.entropies = f32(fr.entropies)
         self.probes = dict(plan=fr.probe_plan_us, h2d=fr.probe_h2d_us,
                            launch=fr.probe_kernel_launch_us, sync=fr.probe_sync_us,
                            build=fr.probe_response_build_us)
 
     def tokens_of(self, r: int) -> list:
         return self.tokens[self.tokens_indptr[r]:self.tokens_indptr[r + 1]]
+
+    def dists_of(self, r: int) -> list:
+        """[(ids, probs), ...] of request r, one pair per Distribution slot."""
+        out = []
+        for i in range(self.dists_req_indptr[r], self.dists_req_indptr[r + 1]):
+            a, b = self.dists_kv_indptr[i], self.dists_kv_indptr[i + 1]
+            out.append((np.asarray(self.dists_ids[a:b], np.uint32), self.dists_probs[a:b]))
+        return out
+
+    def logits_of(self, r: int) -> list:
+        """f32 logits rows of request r's RawLogits slots."""
+        out = []
+        for i in range(self.logits_req_indptr[r], self.logits_req_indptr[r + 1]):
+            a, b = self.logits_byte_indptr[i], self.logits_byte_indptr[i + 1]
+            out.append(np.frombuffer(self.logits_bytes[a:b], np.float32))
+        return out
+
+    def logprobs_of(self, r: int) -> list:
+        out = []
+        for i in range(self.logprobs_req_indptr[r], self.logprobs_req_indptr[r + 1]):
+            out.append(self.logprobs_values[self.logprobs_val_indptr[i]:self.logprobs_val_indptr[i + 1]])
+        return out
+
+    def entropies_of(self, r: int) -> list:
+        return list(self.entropies[self.entropies_indptr[r]:self.entropies_indptr[r + 1]])
 
 
 class Driver:

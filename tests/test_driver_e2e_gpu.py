@@ -188,9 +188,10 @@ def test_forward_failures_return_empty_response(gpu):
     with drvmod.Driver(toml_config()) as d:
         ok = dict(token_ids=[1], position_ids=[0], kv_page_indices=[0], kv_page_indptr=[0, 1],
                   kv_last_page_lens=[1], qo_indptr=[0, 1])
-        # out-of-range page id, position past the context, non-greedy sampler, user mask
+        # out-of-range page id, position past the context, a sampler kind without an
+        # implementation (Embedding), user mask
         for bad in (dict(kv_page_indices=[9999]), dict(position_ids=[5]),
-                    dict(samplers=[dict(temperature=0.8)], sampling_indices=[0],
+                    dict(samplers=[dict(kind=5, temperature=0.8)], sampling_indices=[0],
                          sampling_indptr=[0, 1], sampler_indptr=[0, 1]),
                     dict(masks=[[1, 0]])):
             args = dict(ok)
