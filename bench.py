@@ -347,6 +347,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-extra", action="store_true")
     ap.add_argument("--model", default="llama8b-w4a16", choices=["llama8b-w4a16", *OTHER_MODELS])
+    ap.add_argument("--sampler", default="greedy", choices=["greedy", "top_p", "top_k", "min_p", "multinomial"],
+                    help="decode-step sampler (default greedy = the headline workload); the others run "
+                         "the device samplers at temperature 0.8 (top_p 0.95 / top_k 50 / min_p 0.05)")
     ap.add_argument("--pmc-workload", action="store_true",
                     help="only launch what a `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE` run needs: a "
                          "256 MiB device copy (the counter's scale) and the four int4 GEMV shapes")
@@ -380,6 +383,11 @@ def main():
     drv = drvmod.Driver(cfg_text)
     t_init = time.perf_counter() - t0
 
+    if args.sampler != "greedy":
+        kind, k, p = {"multinomial": (0, 0, 1.0), "top_k": (1, 50, 1.0), "top_p": (2, 0, 0.95),
+                      "min_p": (3, 0, 0.05)}[args.sampler]
+        drv.set_generate_sampler(kind, 0.8, k, p, seed=12345)
+        label = (label or "Llama-3-8B-shaped W4A16 (int4b8 group 128) decode") + f", {args.sampler} sampling at T=0.8"
     torch.cuda.synchronize()
     tokens, tm = drv.generate(prompt, max_new, replicate=args.batch, warmup=args.warmup)
     steps = tm["decode_steps"]

@@ -216,6 +216,8 @@ struct PieHipDriver {
     std::vector<uint32_t> toks;
     SampleOutputs samples;
     std::string last_error;
+    PieSamplerDesc gen_sampler{};   // decode-step sampler of the generation harness (kind 2, T 0 = greedy)
+    bool gen_sampler_set = false;
 
     explicit PieHipDriver(const DriverConfig& c) : cfg(c) {
         int ndev = 0;
@@ -459,6 +461,21 @@ extern "C" void* pie_hip_driver_tensor_ptr(PieHipDriver* d, const char* name) {
     return it == t.end() ? nullptr : it->second.ptr;
 }
 
+// Sampler the generation harness attaches to its decode steps (wire kind and fields; the seed
+// is advanced per step and context).  Default: greedy.
+extern "C" int pie_hip_driver_set_generate_sampler(PieHipDriver* d, int kind, float temperature,
+                                                   uint32_t k, float p, uint32_t seed) {
+    if (!d || kind < 0 || kind > PIE_SAMPLER_KIND_TOP_K_TOP_P) return -1;
+    std::memset(&d->gen_sampler, 0, sizeof(d->gen_sampler));
+    d->gen_sampler.kind = static_cast<uint8_t>(kind);
+    d->gen_sampler.temperature = temperature;
+    d->gen_sampler.k = k;
+    d->gen_sampler.p = p;
+    d->gen_sampler.seed = seed;
+    d->gen_sampler_set = true;
+    return 0;
+}
+
 extern "C" int pie_hip_driver_generate(PieHipDriver* d, const uint32_t* prompt, int n_prompt,
                                        int max_new, int replicate, int warmup,
                                        uint32_t* out_tokens, double* timings_us, char* err,
@@ -557,7 +574,9 @@ extern "C" int pie_hip_driver_generate(PieHipDriver* d, const uint32_t* prompt, 
                 for (int p = 0; p < np; ++p) fb.pages.push_back(static_cast<uint32_t>(c * pages_per_ctx + p));
                 fb.last_lens.push_back(static_cast<uint32_t>(pos + 1 - (np - 1) * ps));
                 fb.samp_idx.push_back(0u);
-                fb.samplers.push_back(greedy_sampler());
+                PieSamplerDesc sd = d->gen_sampler_set ? d->gen_sampler : greedy_sampler();
+                if (sd.seed != 0) sd.seed += static_cast<uint32_t>(s * replicate + c);   // a fresh draw per slot
+                fb.samplers.push_back(sd);
                 fb.ctx_ids.push_back(static_cast<uint64_t>(c));
             }
             for (int c = 0; c <= replicate; ++c) {

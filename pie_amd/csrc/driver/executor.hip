@@ -453,9 +453,9 @@ void Executor::prepare_samplers(const BatchPlan& plan) {
     PIE_HIP_CHECK(hipMemcpyAsync(samp_in_dev_.ptr, h, L.total, hipMemcpyHostToDevice, stream_));
 }
 
-// Device half: f32 rows (+ masks) unless the body gathered them chunk by chunk, one sampler
-// block per slot, results back through pinned memory.  Ends with the stream drained.
-void Executor::run_samplers(const BatchPlan& plan, SampleOutputs& out) {
+// Device half, queued behind the forward body: f32 rows (+ masks) unless the body gathered them
+// chunk by chunk, one sampler block per slot, results into pinned memory.
+void Executor::enqueue_samplers() {
     const int S = samp_.slots, V = cfg_.model.vocab;
     const auto* in = static_cast<const unsigned char*>(samp_in_dev_.ptr);
     auto* od = static_cast<unsigned char*>(samp_out_dev_.ptr);
@@ -473,13 +473,18 @@ void Executor::run_samplers(const BatchPlan& plan, SampleOutputs& out) {
         reinterpret_cast<const int32_t*>(in + samp_.out_indptr), reinterpret_cast<const uint32_t*>(in + samp_.labels),
         reinterpret_cast<uint32_t*>(od + samp_.o_tokens), reinterpret_cast<float*>(od + samp_.o_values),
         reinterpret_cast<uint32_t*>(od + samp_.o_ids), samp_ws_.ptr, samp_ws_.cap, S, V, stream_));
-    auto* oh = static_cast<unsigned char*>(samp_out_host_.ptr);
-    PIE_HIP_CHECK(hipMemcpyAsync(oh, od, samp_.o_total, hipMemcpyDeviceToHost, stream_));
+    PIE_HIP_CHECK(hipMemcpyAsync(samp_out_host_.ptr, od, samp_.o_total, hipMemcpyDeviceToHost, stream_));
+}
+
+// After the stream has drained: results out of pinned memory, RawLogits rows copied back.
+void Executor::collect_samplers(const BatchPlan& plan, SampleOutputs& out) {
+    const int S = samp_.slots, V = cfg_.model.vocab;
+    const float* f32 = static_cast<const float*>(samp_f32_.ptr);
+    const auto* oh = static_cast<const unsigned char*>(samp_out_host_.ptr);
     out.raw_logits.clear();
     size_t n_raw = 0;
     for (const SlotSampler& sp : plan.slot_samplers) n_raw += sp.kind == PIE_SAMPLER_KIND_RAW_LOGITS;
     out.raw_logits.resize(n_raw * static_cast<size_t>(V));
-    PIE_HIP_CHECK(hipStreamSynchronize(stream_));
     size_t at = 0;
     for (int s = 0; s < S; ++s)
         if (plan.slot_samplers[s].kind == PIE_SAMPLER_KIND_RAW_LOGITS) {
@@ -556,6 +561,7 @@ void Executor::forward(const BatchPlan& plan, std::vector<uint32_t>& tokens_out,
     }
     if (S) PIE_HIP_CHECK(hipMemcpyAsync(out_host_, out_tokens_, static_cast<size_t>(S) * 4,
                                         hipMemcpyDeviceToHost, stream_));
+    if (sampling) enqueue_samplers();
     if (t) t->launch_us = us_since(t0);
 
     t0 = clk::now();
@@ -563,9 +569,8 @@ void Executor::forward(const BatchPlan& plan, std::vector<uint32_t>& tokens_out,
     if (t) t->sync_us = us_since(t0);
     tokens_out.assign(out_host_, out_host_ + S);
     if (sampling) {
-        run_samplers(plan, *samples);
+        collect_samplers(plan, *samples);
         tokens_out = samples->tokens;
-        if (t) t->sync_us = us_since(t0);
     }
     const int cap = static_cast<int>(std::min<size_t>(max_tokens_, 2 * static_cast<size_t>(cfg_.batching.max_forward_requests)));
     last_logit_rows_ = S == 0 ? 0 : ((S - 1) % cap) + 1;

@@ -79,7 +79,8 @@ class Executor {
   private:
     void body(int N, int S, int max_kv_len);
     void prepare_samplers(const BatchPlan& plan);
-    void run_samplers(const BatchPlan& plan, SampleOutputs& out);
+    void enqueue_samplers();
+    void collect_samplers(const BatchPlan& plan, SampleOutputs& out);
     void moe_block(const LayerWeights& w, int N, hipStream_t s);
     void alloc_kv();
 

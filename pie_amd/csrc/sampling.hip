@@ -33,6 +33,9 @@ namespace {
 constexpr int kSampBlock = 1024;
 constexpr int kSampWaves = kSampBlock / kWave;   // 16
 constexpr int kDigits = 256;
+// A single block walks a whole vocabulary row: every pass requests kLoads values per thread
+// before it uses the first, or it would pay one memory latency per element.
+constexpr int kLoads = 32;
 
 struct SampleArgs {
     const float* logits;        // [S, V]
@@ -54,7 +57,15 @@ struct SampleArgs {
     int V;
 };
 
+// Candidate thresholds t_j = p_max * 2^(-3j), j = 1..kLevels: how many entries, and how much
+// probability mass, lie at or above each (mass in float: a guide for picking a level, not a
+// result).
+constexpr int kLevels = 8;
+constexpr uint32_t kLevelStep = 3u << 23;   // three binades in the float bit pattern
+
 struct BlockShared {
+    uint32_t lcnt[kSampWaves][kLevels];
+    float lmass[kSampWaves][kLevels];
     uint32_t cnt[kSampWaves][kDigits];
     double f64[kSampWaves];
     float f32[kSampWaves];
@@ -112,11 +123,20 @@ __device__ void block_argmax(const float* row, int V, BlockShared& sh, int tid, 
                              float& mx_out, int& idx_out) {
     float bv = -INFINITY;
     int bi = 0x7FFFFFFF;
-    for (int v = tid; v < V; v += kSampBlock) {
-        const float x = row[v];
-        if (x > bv || (bi == 0x7FFFFFFF && x == bv)) {
-            bv = x;
-            bi = v;
+    for (int v0 = tid; v0 < V; v0 += kSampBlock * kLoads) {
+        float x[kLoads];
+#pragma unroll
+        for (int j = 0; j < kLoads; ++j) {
+            const int v = v0 + j * kSampBlock;
+            x[j] = v < V ? row[v] : -INFINITY;
+        }
+#pragma unroll
+        for (int j = 0; j < kLoads; ++j) {
+            const int v = v0 + j * kSampBlock;
+            if (v < V && (x[j] > bv || (bi == 0x7FFFFFFF && x[j] == bv))) {
+                bv = x[j];
+                bi = v;
+            }
         }
     }
 #pragma unroll
@@ -169,13 +189,21 @@ __device__ void radix_pass(const uint32_t* __restrict__ kin, const uint32_t* __r
     __syncthreads();
     const int seg = ((n + kSampBlock - 1) / kSampBlock) * kWave;   // per wave, a multiple of 64
     const int lo = wv * seg, hi = min(n, lo + seg);
-    for (int i0 = lo; i0 < hi; i0 += kWave) {
-        const int i = i0 + lane;
-        const bool valid = i < hi;
-        const uint32_t key = valid ? kin[i] : 0u;
-        const uint32_t d = 255u - ((key >> shift) & 255u);
-        const uint64_t m = match_digit(d, valid);
-        if (valid && lane == __ffsll(static_cast<long long>(m)) - 1) sh.cnt[wv][d] += __popcll(m);
+    constexpr int kSteps = 16;   // 64-key steps whose loads are requested together
+    for (int i0 = lo; i0 < hi; i0 += kWave * kSteps) {
+        uint32_t keys[kSteps];
+#pragma unroll
+        for (int j = 0; j < kSteps; ++j) {
+            const int i = i0 + j * kWave + lane;
+            keys[j] = i < hi ? kin[i] : 0u;
+        }
+#pragma unroll
+        for (int j = 0; j < kSteps; ++j) {
+            const bool valid = i0 + j * kWave + lane < hi;
+            const uint32_t d = 255u - ((keys[j] >> shift) & 255u);
+            const uint64_t m = match_digit(d, valid);
+            if (valid && lane == __ffsll(static_cast<long long>(m)) - 1) sh.cnt[wv][d] += __popcll(m);
+        }
     }
     __syncthreads();
     {   // exclusive offsets in (digit, wave) order: thread t owns digit t/4, waves 4*(t%4)..+3
@@ -189,28 +217,36 @@ __device__ void radix_pass(const uint32_t* __restrict__ kin, const uint32_t* __r
         sh.cnt[w0 + 3][d] = ex + c0 + c1 + c2;
     }
     __syncthreads();
-    for (int i0 = lo; i0 < hi; i0 += kWave) {
-        const int i = i0 + lane;
-        const bool valid = i < hi;
-        const uint32_t key = valid ? kin[i] : 0u;
-        const uint32_t id = valid ? (iin ? iin[i] : static_cast<uint32_t>(i)) : 0u;
-        const uint32_t d = 255u - ((key >> shift) & 255u);
-        const uint64_t m = match_digit(d, valid);
-        const uint32_t base = valid ? sh.cnt[wv][d] : 0u;
-        const uint32_t rank = __popcll(m & ((1ull << lane) - 1ull));
-        if (valid) {
-            kout[base + rank] = key;
-            iout[base + rank] = id;
-            if (rank == 0) sh.cnt[wv][d] = base + __popcll(m);   // after every peer read `base`
+    for (int i0 = lo; i0 < hi; i0 += kWave * kSteps) {
+        uint32_t keys[kSteps], idv[kSteps];
+#pragma unroll
+        for (int j = 0; j < kSteps; ++j) {
+            const int i = i0 + j * kWave + lane;
+            keys[j] = i < hi ? kin[i] : 0u;
+            idv[j] = i < hi ? (iin ? iin[i] : static_cast<uint32_t>(i)) : 0u;
+        }
+#pragma unroll
+        for (int j = 0; j < kSteps; ++j) {
+            const bool valid = i0 + j * kWave + lane < hi;
+            const uint32_t d = 255u - ((keys[j] >> shift) & 255u);
+            const uint64_t m = match_digit(d, valid);
+            const uint32_t base = valid ? sh.cnt[wv][d] : 0u;
+            const uint32_t rank = __popcll(m & ((1ull << lane) - 1ull));
+            if (valid) {
+                kout[base + rank] = keys[j];
+                iout[base + rank] = idv[j];
+                if (rank == 0) sh.cnt[wv][d] = base + __popcll(m);   // after every peer read `base`
+            }
         }
     }
     __syncthreads();
 }
 
-// Sorted (descending key, ascending id) result in (key_a, id_a).
+// Sorted (descending key, ascending position) result in (key_a, id_a).  have_ids: id_a holds the
+// entries' ids (in ascending order for equal keys to come out by ascending id); else ids 0..n-1.
 __device__ void sort_desc(uint32_t* key_a, uint32_t* key_b, uint32_t* id_a, uint32_t* id_b, int n,
-                          BlockShared& sh, int tid, int lane, int wv) {
-    radix_pass(key_a, nullptr, key_b, id_b, n, 0, sh, tid, lane, wv);
+                          bool have_ids, BlockShared& sh, int tid, int lane, int wv) {
+    radix_pass(key_a, have_ids ? id_a : nullptr, key_b, id_b, n, 0, sh, tid, lane, wv);
     radix_pass(key_b, id_b, key_a, id_a, n, 8, sh, tid, lane, wv);
     radix_pass(key_a, id_a, key_b, id_b, n, 16, sh, tid, lane, wv);
     radix_pass(key_b, id_b, key_a, id_a, n, 24, sh, tid, lane, wv);
@@ -225,74 +261,237 @@ enum { kReach = 0, kExceed = 1, kExceedScaled = 2 };
 template <int MODE>
 __device__ int find_first(const uint32_t* __restrict__ pbits, int limit, float thr, BlockShared& sh,
                           int lane, int wv, double* total_out) {
-    const int seg = ((limit + kSampBlock - 1) / kSampBlock) * kWave;
-    const int lo = min(limit, wv * seg), hi = min(limit, lo + seg);
-    double s = 0.0;
-    for (int i = lo + lane; i < hi; i += kWave) s += static_cast<double>(__uint_as_float(pbits[i]));
-    s = wave_sum_f64(s);
-    if (lane == 0) sh.f64[wv] = s;
-    __syncthreads();
-    double base = 0.0, total = 0.0;
+    // Narrow the range 16-fold per level: every wave sums one sub-range (coalesced, batched
+    // loads), the first sub-range whose end satisfies the rule holds the answer; the last
+    // <= 64 entries are scanned by lane.  Sums are double; only the compared value is rounded.
+    int lo = 0, hi = limit;
+    double base = 0.0;
+    float x = thr;
+    bool top = true;
+    while (top || hi - lo > kWave) {
+        const int span = hi - lo;
+        const int sub = ((span + kSampWaves * kWave - 1) / (kSampWaves * kWave)) * kWave;
+        const int wlo = min(hi, lo + wv * sub), whi = min(hi, wlo + sub);
+        double s = 0.0;
+        for (int i0 = wlo + lane; i0 < whi; i0 += kWave * kLoads) {
+            uint32_t b[kLoads];
 #pragma unroll
-    for (int w = 0; w < kSampWaves; ++w) {
-        if (w < wv) base += sh.f64[w];
-        total += sh.f64[w];
-    }
-    const float x = MODE == kExceedScaled ? thr * static_cast<float>(total) : thr;
-    int cand = limit;
-    double acc = base;
-    for (int i0 = lo; i0 < hi; i0 += kWave) {
-        const int i = i0 + lane;
-        double incl = i < hi ? static_cast<double>(__uint_as_float(pbits[i])) : 0.0;
+            for (int j = 0; j < kLoads; ++j) b[j] = i0 + j * kWave < whi ? pbits[i0 + j * kWave] : 0u;
 #pragma unroll
-        for (int off = 1; off < kWave; off <<= 1) {
-            const double o = __shfl_up(incl, off, kWave);
-            if (lane >= off) incl += o;
+            for (int j = 0; j < kLoads; ++j) s += static_cast<double>(__uint_as_float(b[j]));
         }
-        const float cum = static_cast<float>(acc + incl);
-        const bool hit = i < hi && (MODE == kReach ? cum >= x : x < cum);
-        const uint64_t b = __ballot(hit);
-        if (b) {
-            cand = i0 + __ffsll(static_cast<long long>(b)) - 1;
-            break;
-        }
-        acc += __shfl(incl, kWave - 1, kWave);
-    }
-    if (lane == 0) sh.i32[wv] = cand;
-    __syncthreads();
-    int r = limit;
+        s = wave_sum_f64(s);
+        if (lane == 0) sh.f64[wv] = s;
+        __syncthreads();
+        if (top) {
+            double total = 0.0;
 #pragma unroll
-    for (int w = 0; w < kSampWaves; ++w) r = min(r, sh.i32[w]);
-    __syncthreads();
-    *total_out = total;
-    return r;
+            for (int w = 0; w < kSampWaves; ++w) total += sh.f64[w];
+            *total_out = total;
+            if (MODE == kExceedScaled) x = thr * static_cast<float>(total);
+        }
+        int pick = -1;
+        double before = base, run = base;
+#pragma unroll
+        for (int w = 0; w < kSampWaves; ++w) {
+            run += sh.f64[w];
+            const float cum = static_cast<float>(run);
+            const bool hit = MODE == kReach ? cum >= x : x < cum;
+            if (hit && pick < 0) pick = w;
+            if (pick < 0) before = run;
+        }
+        __syncthreads();
+        if (pick < 0) {
+            if (top) return limit;      // the rule is never met
+            return hi - 1;              // (re-associated sums disagreeing in the last bit)
+        }
+        base = before;
+        lo = min(hi, lo + pick * sub);
+        hi = min(hi, lo + sub);
+        top = false;
+    }
+    const int i = lo + lane;
+    double incl = i < hi ? static_cast<double>(__uint_as_float(pbits[i])) : 0.0;
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+        const double o = __shfl_up(incl, off, kWave);
+        if (lane >= off) incl += o;
+    }
+    const float cum = static_cast<float>(base + incl);
+    const uint64_t b = __ballot(i < hi && (MODE == kReach ? cum >= x : x < cum));
+    return b ? lo + __ffsll(static_cast<long long>(b)) - 1 : hi - 1;
 }
 
-// p = softmax(row / T) as float bit patterns in `out`; returns the number of entries with p > 0.
-__device__ int softmax_to_bits(const float* row, int V, float mx, float temperature, uint32_t* out,
-                               BlockShared& sh, int tid, int lane, int wv) {
+// p = softmax(row / T) as float bit patterns in `out`.  Also: the number of entries with p > 0,
+// their sum, the largest p, and (HIST) a histogram of count and mass over the buckets.
+struct SoftmaxStats {
+    int n_pos;
+    double total;
+    uint32_t max_bits;
+};
+template <bool HIST>
+__device__ SoftmaxStats softmax_to_bits(const float* row, int V, float mx, float temperature,
+                                        uint32_t* out, BlockShared& sh, int tid, int lane, int wv) {
     const float inv_t = 1.0f / fmaxf(temperature, 1e-5f);
     double s = 0.0;
-    for (int v = tid; v < V; v += kSampBlock) {
-        const float e = expf((row[v] - mx) * inv_t);
-        out[v] = __float_as_uint(e);
-        s += static_cast<double>(e);
+    for (int v0 = tid; v0 < V; v0 += kSampBlock * kLoads) {
+        float x[kLoads];
+#pragma unroll
+        for (int j = 0; j < kLoads; ++j) {
+            const int v = v0 + j * kSampBlock;
+            x[j] = v < V ? row[v] : 0.f;
+        }
+#pragma unroll
+        for (int j = 0; j < kLoads; ++j) {
+            const int v = v0 + j * kSampBlock;
+            if (v < V) {
+                const float e = expf((x[j] - mx) * inv_t);
+                out[v] = __float_as_uint(e);
+                s += static_cast<double>(e);
+            }
+        }
     }
     const double sum = block_sum_f64(s, sh, lane, wv);
     const float inv_sum = static_cast<float>(1.0 / fmax(1e-30, sum));
     int pos = 0;
-    for (int v = tid; v < V; v += kSampBlock) {
-        const float p = __uint_as_float(out[v]) * inv_sum;
-        out[v] = __float_as_uint(p);
-        pos += p > 0.0f;
+    double ps = 0.0;
+    uint32_t mb = 0u;
+    // p_max = e_max * inv_sum with e_max = expf(0) = 1 (the row maximum), known before the pass
+    const uint32_t top_bits = __float_as_uint(inv_sum);
+    uint32_t lc[kLevels];
+    float lm[kLevels];
+#pragma unroll
+    for (int j = 0; j < kLevels; ++j) {
+        lc[j] = 0u;
+        lm[j] = 0.f;
     }
-    return block_sum_i32(pos, sh, lane, wv);
+    for (int v0 = tid; v0 < V; v0 += kSampBlock * kLoads) {
+        uint32_t eb[kLoads];
+#pragma unroll
+        for (int j = 0; j < kLoads; ++j) {
+            const int v = v0 + j * kSampBlock;
+            eb[j] = v < V ? out[v] : 0u;
+        }
+#pragma unroll
+        for (int j = 0; j < kLoads; ++j) {
+            const int v = v0 + j * kSampBlock;
+            if (v >= V) continue;
+            const float p = __uint_as_float(eb[j]) * inv_sum;
+            const uint32_t bits = __float_as_uint(p);
+            out[v] = bits;
+            if (p > 0.0f) {
+                ++pos;
+                ps += static_cast<double>(p);
+                mb = max(mb, bits);
+                if (HIST) {
+#pragma unroll
+                    for (int j = 0; j < kLevels; ++j) {
+                        const bool in = bits + (j + 1) * kLevelStep >= top_bits;
+                        lc[j] += in;
+                        lm[j] += in ? p : 0.f;
+                    }
+                }
+            }
+        }
+    }
+    SoftmaxStats st;
+    st.n_pos = block_sum_i32(pos, sh, lane, wv);
+    st.total = block_sum_f64(ps, sh, lane, wv);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) mb = max(mb, static_cast<uint32_t>(__shfl_xor(mb, off, kWave)));
+    if (lane == 0) sh.u32[wv] = mb;
+    __syncthreads();
+    mb = 0u;
+#pragma unroll
+    for (int w = 0; w < kSampWaves; ++w) mb = max(mb, sh.u32[w]);
+    __syncthreads();
+    st.max_bits = mb;
+    if (HIST) {
+#pragma unroll
+        for (int j = 0; j < kLevels; ++j) {
+            uint32_t c = lc[j];
+            float m = lm[j];
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) {
+                c += __shfl_xor(c, off, kWave);
+                m += __shfl_xor(m, off, kWave);
+            }
+            if (lane == 0) {
+                sh.lcnt[wv][j] = c;
+                sh.lmass[wv][j] = m;
+            }
+        }
+        __syncthreads();
+    }
+    return st;
+}
+
+// Entries with bits >= floor_bits, in index order, into (kout, iout); returns how many.
+__device__ int compact_ge(const uint32_t* __restrict__ kin, uint32_t floor_bits,
+                          uint32_t* __restrict__ kout, uint32_t* __restrict__ iout, int n,
+                          BlockShared& sh, int lane, int wv) {
+    const int seg = ((n + kSampBlock - 1) / kSampBlock) * kWave;
+    const int lo = min(n, wv * seg), hi = min(n, lo + seg);
+    constexpr int kSteps = 16;
+    int c = 0;
+    for (int i0 = lo; i0 < hi; i0 += kWave * kSteps) {
+        uint32_t keys[kSteps];
+#pragma unroll
+        for (int j = 0; j < kSteps; ++j) {
+            const int i = i0 + j * kWave + lane;
+            keys[j] = i < hi ? kin[i] : 0u;
+        }
+#pragma unroll
+        for (int j = 0; j < kSteps; ++j)
+            c += __popcll(__ballot(i0 + j * kWave + lane < hi && keys[j] >= floor_bits));
+    }
+    if (lane == 0) sh.i32[wv] = c;
+    __syncthreads();
+    int base = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < kSampWaves; ++w) {
+        if (w < wv) base += sh.i32[w];
+        total += sh.i32[w];
+    }
+    __syncthreads();
+    for (int i0 = lo; i0 < hi; i0 += kWave * kSteps) {
+        uint32_t keys[kSteps];
+#pragma unroll
+        for (int j = 0; j < kSteps; ++j) {
+            const int i = i0 + j * kWave + lane;
+            keys[j] = i < hi ? kin[i] : 0u;
+        }
+#pragma unroll
+        for (int j = 0; j < kSteps; ++j) {
+            const int i = i0 + j * kWave + lane;
+            const bool take = i < hi && keys[j] >= floor_bits;
+            const uint64_t b = __ballot(take);
+            if (take) {
+                const int at = base + __popcll(b & ((1ull << lane) - 1ull));
+                kout[at] = keys[j];
+                iout[at] = static_cast<uint32_t>(i);
+            }
+            base += __popcll(b);
+        }
+    }
+    __syncthreads();
+    return total;
 }
 
 __device__ float log_sum_exp(const float* row, int V, float mx, BlockShared& sh, int tid, int lane,
                              int wv) {
     double s = 0.0;
-    for (int v = tid; v < V; v += kSampBlock) s += exp(static_cast<double>(row[v] - mx));
+    for (int v0 = tid; v0 < V; v0 += kSampBlock * kLoads) {
+        float x[kLoads];
+#pragma unroll
+        for (int j = 0; j < kLoads; ++j) {
+            const int v = v0 + j * kSampBlock;
+            x[j] = v < V ? row[v] : -INFINITY;
+        }
+#pragma unroll
+        for (int j = 0; j < kLoads; ++j)
+            if (v0 + j * kSampBlock < V) s += exp(static_cast<double>(x[j] - mx));
+    }
     const double sum = block_sum_f64(s, sh, lane, wv);
     return mx + static_cast<float>(log(fmax(1e-30, sum)));
 }
@@ -317,9 +516,19 @@ __global__ __launch_bounds__(kSampBlock) void sample_kernel(SampleArgs a) {
     if (kind == PIE_HIP_SAMPLER_ENTROPY) {
         const float lse = log_sum_exp(row, V, mx, sh, tid, lane, wv);
         double h = 0.0;
-        for (int v = tid; v < V; v += kSampBlock) {
-            const float lp = row[v] - lse;
-            h -= exp(static_cast<double>(lp)) * static_cast<double>(lp);
+        for (int v0 = tid; v0 < V; v0 += kSampBlock * kLoads) {
+            float x[kLoads];
+#pragma unroll
+            for (int j = 0; j < kLoads; ++j) {
+                const int v = v0 + j * kSampBlock;
+                x[j] = v < V ? row[v] : 0.f;
+            }
+#pragma unroll
+            for (int j = 0; j < kLoads; ++j)
+                if (v0 + j * kSampBlock < V) {
+                    const float lp = x[j] - lse;
+                    h -= exp(static_cast<double>(lp)) * static_cast<double>(lp);
+                }
         }
         const double H = block_sum_f64(h, sh, lane, wv);
         if (tid == 0 && o1 > o0) a.values[o0] = static_cast<float>(H);
@@ -333,9 +542,8 @@ __global__ __launch_bounds__(kSampBlock) void sample_kernel(SampleArgs a) {
     const float temperature = a.temperature[s];
 
     if (kind == PIE_HIP_SAMPLER_DIST) {
-        softmax_to_bits(row, V, mx, temperature, ka, sh, tid, lane, wv);
-        __syncthreads();
-        sort_desc(ka, kb, ia, ib, V, sh, tid, lane, wv);
+        softmax_to_bits<false>(row, V, mx, temperature, ka, sh, tid, lane, wv);
+        sort_desc(ka, kb, ia, ib, V, false, sh, tid, lane, wv);
         const int k = min(o1 - o0, V);
         for (int i = tid; i < k; i += kSampBlock) {
             a.values[o0 + i] = __uint_as_float(ka[i]);
@@ -349,46 +557,92 @@ __global__ __launch_bounds__(kSampBlock) void sample_kernel(SampleArgs a) {
         if (tid == 0) a.tokens[s] = static_cast<uint32_t>(amax);
         return;
     }
-    const int n_pos = softmax_to_bits(row, V, mx, temperature, ka, sh, tid, lane, wv);
-    __syncthreads();
     const float u = a.uniform[s];
     double total;
     if (kind == PIE_HIP_SAMPLER_MULTINOMIAL) {
+        softmax_to_bits<false>(row, V, mx, temperature, ka, sh, tid, lane, wv);
         const int tok = find_first<kExceed>(ka, V, u, sh, lane, wv, &total);
         if (tid == 0) a.tokens[s] = static_cast<uint32_t>(tok < V ? tok : amax);
         return;
     }
+    const SoftmaxStats st = softmax_to_bits<true>(row, V, mx, temperature, ka, sh, tid, lane, wv);
+    const int n_pos = st.n_pos;
     if (n_pos == 0) {
         if (tid == 0) a.tokens[s] = 0u;
         return;
     }
-    sort_desc(ka, kb, ia, ib, V, sh, tid, lane, wv);
-    int keep = n_pos;
+    // What the draw can touch is a head of the descending order: the first top_k entries, the
+    // prefix reaching top_p, the entries above the min-p threshold, or (nothing restricting)
+    // the prefix whose mass exceeds u * total.  Any set {p >= t} containing that head gives
+    // the same result as the whole vocabulary, so only such a set is compacted and sorted;
+    // t is the first of the levels p_max * 2^(-3j) that covers the need (exact for min-p).
     const bool wants_k = kind == PIE_HIP_SAMPLER_TOP_K || kind == PIE_HIP_SAMPLER_TOP_K_TOP_P;
     const bool wants_p = kind == PIE_HIP_SAMPLER_TOP_P || kind == PIE_HIP_SAMPLER_TOP_K_TOP_P;
-    if (wants_k) {
-        const uint32_t k = a.top_k[s];
-        if (k != 0u && k < static_cast<uint32_t>(keep)) keep = static_cast<int>(k);
+    const uint32_t top_k = a.top_k[s];
+    const float thr_p = fminf(fmaxf(a.top_p[s], 0.0f), 1.0f);
+    const float thr_m = a.min_p[s] * __uint_as_float(st.max_bits);
+    int need_count = 0;
+    float need_mass = 0.f;
+    uint32_t floor_bits = 0u;     // nonzero: the exact lower bound of the kept entries (min-p)
+    bool keep_all = false;
+    if (wants_k && top_k != 0u) need_count = static_cast<int>(min(top_k, static_cast<uint32_t>(n_pos)));
+    else if (wants_p && thr_p < 1.0f) need_mass = thr_p;
+    else if (kind == PIE_HIP_SAMPLER_MIN_P && thr_m > 0.0f && thr_m <= __uint_as_float(st.max_bits))
+        floor_bits = __float_as_uint(thr_m);
+    else {
+        keep_all = true;
+        need_mass = u * static_cast<float>(st.total);
     }
-    if (wants_p) {
-        const float thr = fminf(fmaxf(a.top_p[s], 0.0f), 1.0f);
-        if (thr < 1.0f) {
-            const int i = find_first<kReach>(ka, keep, thr, sh, lane, wv, &total);
-            if (i < keep) keep = i + 1;
+    for (int attempt = 0; attempt < 2; ++attempt) {
+        uint32_t t_bits = 1u;     // every positive entry
+        if (floor_bits) t_bits = floor_bits;
+        else if (attempt == 0) {
+            // the first level whose candidates cover the need (every thread computes the same)
+            const uint32_t top_bits = st.max_bits;
+            for (int j = 0; j < kLevels; ++j) {
+                uint32_t cc = 0u;
+                float cm = 0.f;
+#pragma unroll
+                for (int w = 0; w < kSampWaves; ++w) {
+                    cc += sh.lcnt[w][j];
+                    cm += sh.lmass[w][j];
+                }
+                const bool enough = need_count > 0 ? cc >= static_cast<uint32_t>(need_count)
+                                                   : cm >= need_mass + 1e-4f;
+                if (enough && top_bits > (j + 1) * kLevelStep) {
+                    t_bits = top_bits - (j + 1) * kLevelStep;
+                    break;
+                }
+            }
         }
+        const int m = compact_ge(ka, t_bits, kb, ib, V, sh, lane, wv);
+        const bool whole = m == n_pos;
+        sort_desc(kb, ka, ib, ia, m, true, sh, tid, lane, wv);   // note: overwrites ka
+        bool ok = true;
+        uint32_t tok = 0u;
+        if (keep_all) {
+            const int i = find_first<kExceed>(kb, m, need_mass, sh, lane, wv, &total);
+            ok = i < m || whole;
+            tok = ib[i < m ? i : m - 1];
+        } else {
+            int keep = m;
+            if (need_count > 0) keep = min(need_count, m);
+            if (wants_p && thr_p < 1.0f) {
+                const int i = find_first<kReach>(kb, keep, thr_p, sh, lane, wv, &total);
+                if (i < keep) keep = i + 1;
+                else ok = whole || need_count > 0;   // the prefix must end inside the candidates
+            }
+            const int i = find_first<kExceedScaled>(kb, keep, u, sh, lane, wv, &total);
+            tok = total <= 0.0 ? ib[0] : ib[i < keep ? i : keep - 1];
+        }
+        if (ok || attempt == 1) {
+            if (tid == 0) a.tokens[s] = tok;
+            return;
+        }
+        // the histogram's float masses misjudged the head: rebuild p (the sort used its buffer)
+        // and take every positive entry
+        softmax_to_bits<false>(row, V, mx, temperature, ka, sh, tid, lane, wv);
     }
-    if (kind == PIE_HIP_SAMPLER_MIN_P) {
-        const float thr = a.min_p[s] * __uint_as_float(ka[0]);
-        int c = 0;
-        for (int i = tid; i < keep; i += kSampBlock) c += __uint_as_float(ka[i]) >= thr;
-        const int cut = block_sum_i32(c, sh, lane, wv);   // sorted: the passing entries are a prefix
-        if (cut > 0) keep = cut;
-    }
-    const int i = find_first<kExceedScaled>(ka, keep, u, sh, lane, wv, &total);
-    uint32_t tok;
-    if (total <= 0.0) tok = ia[0];
-    else tok = ia[i < keep ? i : keep - 1];
-    if (tid == 0) a.tokens[s] = tok;
 }
 
 // Sampled rows of the bf16 logits -> f32, BRLE logit mask applied.  bounds: per slot, the
