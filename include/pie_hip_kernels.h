@@ -196,6 +196,29 @@ int pie_hip_moe_combine(const uint16_t* y_routes_bf16, const int32_t* route_pos,
                         int hidden, int add, void* stream);
 
 /*
+ * Custom attention masks for the per-row form.  pie_hip_attn_mask_bitmap turns per-row BRLE
+ * runs into one u16 per 16-token unit (bit t = key 16*unit + t visible): run_bounds holds each
+ * row's cumulative run ends, [run_bounds_indptr[r], run_bounds_indptr[r+1]); runs alternate
+ * hidden / visible from key 0, keys past the last run are hidden, a row without runs sees its
+ * whole window; no key at or past row_kv_len[r] (= the row's position + 1) is ever visible, and
+ * window > 0 also hides keys below row_kv_len[r] - window
+ * (build_attn_mask_f16, driver/portable/src/plan.cpp:54-94).  bitmap: [num_rows, stride_units],
+ * stride_units >= ceil(max_kv_len / 16).
+ * pie_hip_attn_rows_paged_masked is pie_hip_attn_rows_paged restricted to the visible keys; a
+ * row with no visible key gives o = 0, lse = -inf.
+ */
+int pie_hip_attn_mask_bitmap(const uint32_t* run_bounds, const int32_t* run_bounds_indptr,
+                             const int32_t* row_kv_len, int window, uint16_t* bitmap, int num_rows,
+                             int stride_units, void* stream);
+int pie_hip_attn_rows_paged_masked(const uint16_t* q, const uint16_t* k_pages, const uint16_t* v_pages,
+                                   uint16_t* o, float* lse, const uint32_t* kv_page_indices,
+                                   const uint32_t* row_page_begin, const int32_t* row_kv_len,
+                                   const uint16_t* mask_bitmap, int mask_stride_units, int num_rows,
+                                   int num_q_heads, int num_kv_heads, int head_dim, int page_size,
+                                   float sm_scale, int max_kv_len, void* workspace,
+                                   size_t workspace_bytes, void* stream);
+
+/*
  * Sampling beyond greedy argmax, one slot = one sampled logits row.
  *
  * pie_hip_sample_gather_logits: out[s, :] = f32(logits[rows[s], :]) (rows == NULL: row s), with

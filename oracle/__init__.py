@@ -319,6 +319,46 @@ def moe_combine(y_routes_bf16, topk_w, out_bf16=None):
     return out
 
 
+def brle_allow(runs, pos: int, n_kv: int, window: int = 0) -> np.ndarray:
+    """uint8 [n_kv]: keys visible to a token at `pos` carrying the BRLE `runs`
+    (build_attn_mask_f16, driver/portable/src/plan.cpp:54-94)."""
+    r = _c(np.asarray(runs, np.uint32), np.uint32)
+    out = np.zeros(max(n_kv, 1), np.uint8)
+    lib().orc_brle_allow(_p(r), C.c_size_t(r.size), C.c_int(pos), C.c_int(n_kv), C.c_int(window), _p(out))
+    return out[:n_kv]
+
+
+def attn_rows_masked(q_bf16, k_pages, v_pages, page_indices, row_begin, row_len, hq, hk, d, ps,
+                     allow_rows, sm_scale=-1.0, mode=2):
+    """Per-row extents with per-row visibility: allow_rows[r] is None or a uint8 array over the
+    row's keys.  Returns (o_f32, o_bf16, lse)."""
+    q = _c(q_bf16, np.uint16)
+    rows = q.shape[0]
+    kp, vp_ = _c(k_pages, np.uint16), _c(v_pages, np.uint16)
+    pi = _c(np.asarray(page_indices, np.uint32), np.uint32)
+    rb = _c(np.asarray(row_begin, np.uint32), np.uint32)
+    rl = _c(np.asarray(row_len, np.int32), np.int32)
+    offs, chunks, at = [], [], 0
+    for r in range(rows):
+        if allow_rows[r] is None:
+            offs.append(-1)
+        else:
+            a = np.asarray(allow_rows[r], np.uint8)
+            assert a.size >= rl[r]
+            chunks.append(a)
+            offs.append(at)
+            at += a.size
+    allow = _c(np.concatenate(chunks) if chunks else np.zeros(1, np.uint8), np.uint8)
+    off = _c(np.asarray(offs, np.int64), np.int64)
+    o32 = np.zeros((rows, hq, d), np.float32)
+    o16 = np.zeros((rows, hq, d), np.uint16)
+    lse = np.zeros((rows, hq), np.float32)
+    lib().orc_attn_rows_masked(_p(q), _p(kp), _p(vp_), _p(o32), _p(o16), _p(lse), _p(pi), _p(rb), _p(rl),
+                               C.c_int(rows), C.c_int(hq), C.c_int(hk), C.c_int(d), C.c_int(ps),
+                               C.c_float(sm_scale), C.c_int(mode), _p(allow), _p(off))
+    return o32, o16, lse
+
+
 # ---------------------------------------------------------------- samplers
 SAMPLER_KINDS = {"multinomial": 0, "top_k": 1, "top_p": 2, "min_p": 3, "top_k_top_p": 4,
                  "dist": 6, "raw_logits": 7, "logprob": 8, "logprobs": 9, "entropy": 10}

@@ -100,8 +100,11 @@ class OracleModel:
         self._vp = (C.c_void_p * L)(*[a.ctypes.data for a in self.v_pages])
 
     def forward(self, token_ids, position_ids, kv_page_indices, kv_page_indptr, kv_last_page_lens,
-                qo_indptr, sampling_indices=None, sampling_indptr=None, want_logits=False):
-        """One forward pass; returns (tokens per sampled row, logits bf16 bits or None, plan)."""
+                qo_indptr, sampling_indices=None, sampling_indptr=None, want_logits=False,
+                masks=None, window: int = 0):
+        """One forward pass; returns (tokens per sampled row, logits bf16 bits or None, plan).
+        masks: optional per-token BRLE run lists (custom attention masks,
+        driver/portable/src/plan.cpp:54-94); an empty list = plain causal."""
         R = len(qo_indptr) - 1
         if sampling_indices is None:
             qo = np.asarray(qo_indptr, np.int64)
@@ -121,10 +124,22 @@ class OracleModel:
         out = np.zeros(max(S, 1), np.uint32)
         logits = np.zeros((max(S, 1), self.cfg["vocab"]), np.uint16) if want_logits else None
         vp = lambda a: C.c_void_p(a.ctypes.data)
+        allow = allow_off = None
+        if masks is not None:
+            from oracle import brle_allow
+            offs, chunks, at = [], [], 0
+            for i in range(N):
+                chunks.append(brle_allow(masks[i], int(pos[i]), int(rl[i]), window))
+                offs.append(at)
+                at += int(rl[i])
+            allow = np.ascontiguousarray(np.concatenate(chunks) if chunks else np.zeros(1, np.uint8))
+            allow_off = np.ascontiguousarray(np.asarray(offs, np.int64))
         lib().orc_llama_forward(C.byref(self._m), self._kp, self._vp, vp(tok), vp(pos), vp(slots),
                                 vp(rb), vp(rl), vp(pages), C.c_int(N), vp(sr), C.c_int(S),
                                 C.c_int(self.cfg["page_size"]), vp(out),
-                                vp(logits) if want_logits else None)
+                                vp(logits) if want_logits else None,
+                                vp(allow) if allow is not None else None,
+                                vp(allow_off) if allow_off is not None else None)
         return out[:S], (logits[:S] if want_logits else None), p
 
     def generate(self, prompt, max_new: int, replicate: int = 1, want_logits=False):

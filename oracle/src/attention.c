@@ -11,13 +11,28 @@
  * ((page*page_size + slot)*hk + h)*d + j, the same address the portable driver's
  * per-slot rows give (driver/portable/src/kv_cache.hpp:5-17).
  *
+ *   custom masks                    driver/portable/src/plan.cpp:54-94 (build_attn_mask_f16):
+ *                                   key j is visible to a token at position p iff
+ *                                   max(0, p - window + 1) <= j <= min(n_kv - 1, p) and, when
+ *                                   the token carries BRLE runs, j lies in a true run (runs
+ *                                   alternate false/true from position 0; a mask cannot unmask
+ *                                   the future or reach past its last run)
+ *
  * Pinned by tests/test_oracle_attention.py: dense numpy fp64 softmax attention over
  * the gathered rows, page-permutation invariance, forked-prefix equality, the LSE
- * definition, the zero-length case and the causal limit on small brute-force cases.
+ * definition, the zero-length case, the causal limit on small brute-force cases, and masked
+ * rows against dense attention over the allowed keys only.
  */
 #include <stdlib.h>
+#include <string.h>
 
 #include "oracle_common.h"
+
+void orc_attn_rows_masked(const uint16_t* q, const uint16_t* k_pages, const uint16_t* v_pages,
+                          float* o_f32, uint16_t* o_bf16, float* lse, const uint32_t* page_indices,
+                          const uint32_t* row_begin, const int32_t* row_len, int rows, int hq,
+                          int hk, int d, int ps, float sm_scale, int mode, const uint8_t* allow,
+                          const int64_t* allow_off);
 
 static int orc_kv_len(const uint32_t* indptr, const uint32_t* last_lens, int r, int ps) {
     const int pages = (int)(indptr[r + 1] - indptr[r]);
@@ -33,7 +48,7 @@ static int orc_kv_len(const uint32_t* indptr, const uint32_t* last_lens, int r, 
 static void orc_attn_row(const uint16_t* q_row, const uint16_t* k_pages, const uint16_t* v_pages,
                          float* o_f32, uint16_t* o_bf16, float* lse, const uint32_t* page_indices,
                          uint32_t pg_lo, int lim, int hq, int hk, int d, int ps, float scale,
-                         int mode, double* w) {
+                         int mode, double* w, const uint8_t* allow) {
     const int gqa = hq / hk;
     for (int h = 0; h < hq; ++h) {
         const int kvh = h / gqa;
@@ -55,8 +70,17 @@ static void orc_attn_row(const uint16_t* q_row, const uint16_t* k_pages, const u
                          (double)orc_bf16_to_f32(k_pages[koff + e]);
                 dot = f * (double)scale;
             }
+            if (allow && !allow[j]) dot = -INFINITY;
             w[j] = dot;
             if (dot > row_max) row_max = dot;
+        }
+        if (row_max == -INFINITY) {   /* no visible key: zero output, lse = -inf */
+            for (int e = 0; e < d; ++e) {
+                o_f32[qoff + e] = 0.f;
+                if (o_bf16) o_bf16[qoff + e] = 0;
+            }
+            if (lse) lse[h] = -INFINITY;
+            continue;
         }
         double z = 0.0;
         float zf = 0.f;
@@ -116,7 +140,7 @@ void orc_attn_paged(const uint16_t* q, const uint16_t* k_pages, const uint16_t* 
             const size_t row = (size_t)(q_lo + qi) * hq;
             orc_attn_row(q + row * d, k_pages, v_pages, o_f32 + row * d,
                          o_bf16 ? o_bf16 + row * d : NULL, lse ? lse + row : NULL, page_indices,
-                         page_indptr[r], lim, hq, hk, d, ps, scale, mode, w);
+                         page_indptr[r], lim, hq, hk, d, ps, scale, mode, w, NULL);
         }
         free(w);
     }
@@ -131,6 +155,17 @@ void orc_attn_rows(const uint16_t* q, const uint16_t* k_pages, const uint16_t* v
                    float* o_f32, uint16_t* o_bf16, float* lse, const uint32_t* page_indices,
                    const uint32_t* row_begin, const int32_t* row_len, int rows, int hq, int hk,
                    int d, int ps, float sm_scale, int mode) {
+    orc_attn_rows_masked(q, k_pages, v_pages, o_f32, o_bf16, lse, page_indices, row_begin, row_len,
+                         rows, hq, hk, d, ps, sm_scale, mode, NULL, NULL);
+}
+
+/* The same with per-row visibility: row r's key j is visible iff allow[allow_off[r] + j] != 0
+ * (allow_off[r] < 0 or allow == NULL: every key below row_len[r]). */
+void orc_attn_rows_masked(const uint16_t* q, const uint16_t* k_pages, const uint16_t* v_pages,
+                          float* o_f32, uint16_t* o_bf16, float* lse, const uint32_t* page_indices,
+                          const uint32_t* row_begin, const int32_t* row_len, int rows, int hq,
+                          int hk, int d, int ps, float sm_scale, int mode, const uint8_t* allow,
+                          const int64_t* allow_off) {
     const float scale = sm_scale > 0.f ? sm_scale : 1.0f / sqrtf((float)d);
 #pragma omp parallel for schedule(dynamic)
     for (int r = 0; r < rows; ++r) {
@@ -139,8 +174,33 @@ void orc_attn_rows(const uint16_t* q, const uint16_t* k_pages, const uint16_t* v
         const size_t row = (size_t)r * hq;
         orc_attn_row(q + row * d, k_pages, v_pages, o_f32 + row * d,
                      o_bf16 ? o_bf16 + row * d : NULL, lse ? lse + row : NULL, page_indices,
-                     row_begin[r], lim, hq, hk, d, ps, scale, mode, w);
+                     row_begin[r], lim, hq, hk, d, ps, scale, mode, w,
+                     (allow && allow_off && allow_off[r] >= 0) ? allow + allow_off[r] : NULL);
         free(w);
+    }
+}
+
+/* Visibility of keys 0..n_kv-1 for a token at position `pos` (build_attn_mask_f16,
+ * driver/portable/src/plan.cpp:54-94).  n_runs == 0: the causal window alone. */
+void orc_brle_allow(const uint32_t* runs, size_t n_runs, int pos, int n_kv, int window,
+                    uint8_t* out) {
+    memset(out, 0, (size_t)(n_kv > 0 ? n_kv : 0));
+    const int hi = pos < n_kv - 1 ? pos : n_kv - 1;
+    int lo = window > 0 ? pos - window + 1 : 0;
+    if (lo < 0) lo = 0;
+    if (n_runs == 0) {
+        for (int j = lo; j <= hi; ++j) out[j] = 1;
+        return;
+    }
+    int is_true = 0;
+    int64_t p = 0;
+    for (size_t k = 0; k < n_runs && p <= hi; ++k) {
+        int64_t end = p + (int64_t)runs[k];
+        if (end > hi + 1) end = hi + 1;
+        if (is_true)
+            for (int64_t j = p > lo ? p : lo; j < end; ++j) out[j] = 1;
+        p = end;
+        is_true = !is_true;
     }
 }
 

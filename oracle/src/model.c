@@ -127,13 +127,15 @@ static void orc_moe_ffn(const OrcModel* m, int l, const uint16_t* xn, uint16_t* 
 /*
  * tokens/positions/kv_slots/row_begin/row_len: [N] as produced by the planner; k_pages/v_pages:
  * [L] pools [pages, ps, hk, d], updated in place; sample_rows [S] -> out_tokens [S] and, when
- * non-NULL, logits_bf16 [S, V].
+ * non-NULL, logits_bf16 [S, V].  allow / allow_off: optional per-row key visibility (custom
+ * attention masks), as orc_attn_rows_masked takes them.
  */
 void orc_llama_forward(const OrcModel* m, uint16_t* const* k_pages, uint16_t* const* v_pages,
                        const uint32_t* tokens, const int32_t* positions, const int64_t* kv_slots,
                        const uint32_t* row_begin, const int32_t* row_len,
                        const uint32_t* page_indices, int N, const uint32_t* sample_rows, int S,
-                       int page_size, uint32_t* out_tokens, uint16_t* logits_bf16) {
+                       int page_size, uint32_t* out_tokens, uint16_t* logits_bf16,
+                       const uint8_t* allow, const int64_t* allow_off) {
     const int H = m->hidden, d = m->head_dim, hq = m->q_heads, hk = m->kv_heads;
     const int I = m->intermediate, V = m->vocab;
     const int qkv_dim = (hq + 2 * hk) * d;
@@ -155,8 +157,8 @@ void orc_llama_forward(const OrcModel* m, uint16_t* const* k_pages, uint16_t* co
         orc_qkv_rope_kvwrite(qkv, q, k_pages[l], v_pages[l], m->has_qk_norm ? m->q_norm[l] : NULL,
                              m->has_qk_norm ? m->k_norm[l] : NULL, tab, kv_slots, N, hq, hk, d,
                              m->rope_interleaved, m->rms_eps);
-        orc_attn_rows(q, k_pages[l], v_pages[l], attn_f, attn, NULL, page_indices, row_begin, row_len,
-                      N, hq, hk, d, page_size, -1.f, 0);
+        orc_attn_rows_masked(q, k_pages[l], v_pages[l], attn_f, attn, NULL, page_indices, row_begin,
+                             row_len, N, hq, hk, d, page_size, -1.f, 0, allow, allow_off);
         orc_linear(m, &m->wo[l], attn, x, N, H, hq * d, 1);
         orc_rmsnorm(x, NULL, m->ffn_norm[l], xn, N, H, m->rms_eps);
         if (m->num_experts > 0) {

@@ -31,6 +31,13 @@ void orc_attn_rows(const uint16_t* q, const uint16_t* k_pages, const uint16_t* v
                    float* o_f32, uint16_t* o_bf16, float* lse, const uint32_t* page_indices,
                    const uint32_t* row_begin, const int32_t* row_len, int rows, int hq, int hk,
                    int d, int ps, float sm_scale, int mode);
+void orc_attn_rows_masked(const uint16_t* q, const uint16_t* k_pages, const uint16_t* v_pages,
+                          float* o_f32, uint16_t* o_bf16, float* lse, const uint32_t* page_indices,
+                          const uint32_t* row_begin, const int32_t* row_len, int rows, int hq,
+                          int hk, int d, int ps, float sm_scale, int mode, const uint8_t* allow,
+                          const int64_t* allow_off);
+void orc_brle_allow(const uint32_t* runs, size_t n_runs, int pos, int n_kv, int window,
+                    uint8_t* out);
 void orc_topk_softmax(const uint16_t* logits, int32_t* topk_idx, float* topk_w, int N, int E, int K);
 void orc_moe_combine(const uint16_t* y_routes, const float* topk_w, uint16_t* out, int N, int K,
                      int H, int add);

@@ -72,19 +72,22 @@ struct UnitRegs {
     static constexpr int IPU = kUnitTokens / TPI;    // load instructions per unit
     u32x4_t k[IPU];
     u32x4_t v[IPU];
+    uint32_t mask;   // MASKED kernels: bit t = token t of the unit is visible
 };
 
 // part_o  [R, hq, nsplit, D] f32 (unnormalised), part_ml [R, hq, nsplit, 2] f32 (max, sum),
 // both in units where scores were multiplied by scale*log2(e).
-template <int D, int GQA>
+// MASKED: mask_bits [rows, mask_stride] u16, one word per 16-token unit (custom attention
+// masks); hidden tokens are dropped like the slots past the context.
+template <int D, int GQA, bool MASKED>
 __global__ __launch_bounds__(kAttnBlock) void attn_decode_split_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_pages,
     const uint16_t* __restrict__ v_pages, const uint32_t* __restrict__ page_indices,
     const uint32_t* __restrict__ page_indptr, const uint32_t* __restrict__ last_lens,
     const uint32_t* __restrict__ row_begin, const int32_t* __restrict__ row_len,
     float* __restrict__ part_o, float* __restrict__ part_ml, uint16_t* __restrict__ o_direct,
-    float* __restrict__ lse, int hq, int hk, int ps, int units_per_split, int nsplit,
-    float scale_log2e) {
+    float* __restrict__ lse, const uint16_t* __restrict__ mask_bits, int mask_stride, int hq,
+    int hk, int ps, int units_per_split, int nsplit, float scale_log2e) {
     using U = UnitRegs<D, GQA>;
     constexpr int LPR = U::LPR, TPI = U::TPI, IPU = U::IPU;
     const int kvh = blockIdx.x, split = blockIdx.y, r = blockIdx.z;  // kv heads of the same tokens are dispatched together
@@ -120,6 +123,7 @@ __global__ __launch_bounds__(kAttnBlock) void attn_decode_split_kernel(
             u.k[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(k_pages + off));
             u.v[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(v_pages + off));
         }
+        if (MASKED) u.mask = mask_bits[static_cast<size_t>(r) * mask_stride + unit];
     };
 
     float m[GQA], l[GQA], o[GQA][8];
@@ -150,6 +154,16 @@ __global__ __launch_bounds__(kAttnBlock) void attn_decode_split_kernel(
 #pragma unroll
             for (int i = 0; i < IPU; ++i) {
                 if (tok0 + i * TPI + grp >= kv_len) {
+#pragma unroll
+                    for (int h = 0; h < GQA; ++h) s[i][h] = -INFINITY;
+                    u.v[i] = u32x4_t{0u, 0u, 0u, 0u};
+                }
+            }
+        }
+        if (MASKED && u.mask != 0xFFFFu) {
+#pragma unroll
+            for (int i = 0; i < IPU; ++i) {
+                if (!((u.mask >> (i * TPI + grp)) & 1u)) {
 #pragma unroll
                     for (int h = 0; h < GQA; ++h) s[i][h] = -INFINITY;
                     u.v[i] = u32x4_t{0u, 0u, 0u, 0u};
@@ -381,22 +395,22 @@ SplitPlan plan_splits(int R, int hk, int max_kv_len) {
     return {static_cast<int>(ups), nsplit};
 }
 
-template <int D, int GQA>
+template <int D, int GQA, bool MASKED>
 int launch_decode(const uint16_t* q, const uint16_t* k_pages, const uint16_t* v_pages, uint16_t* o,
                   float* lse, const uint32_t* page_indices, const uint32_t* page_indptr,
                   const uint32_t* last_lens, const uint32_t* row_begin, const int32_t* row_len,
                   int R, int hq, int hk, int ps, float sm_scale,
-                  int max_kv_len, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+                  int max_kv_len, void* workspace, size_t workspace_bytes, const uint16_t* mask_bits,
+                  int mask_stride, hipStream_t stream) {
     const SplitPlan plan = plan_splits(R, hk, max_kv_len);
     const float scale_log2e = sm_scale * 1.4426950408889634f;
     if (plan.nsplit == 1) {
         hipLaunchKernelGGL((attn_decode_clear_empty_kernel<D>), dim3(R * hq), dim3(D), 0, stream,
                            page_indptr, last_lens, row_begin, row_len, o, lse, hq, ps);
-        hipLaunchKernelGGL((attn_decode_split_kernel<D, GQA>), dim3(hk, 1, R), dim3(kAttnBlock), 0,
-                           stream, q, k_pages, v_pages, page_indices, page_indptr, last_lens,
-                           row_begin, row_len, nullptr, nullptr, o, lse, hq, hk, ps,
-                           plan.units_per_split, 1,
-                           scale_log2e);
+        hipLaunchKernelGGL((attn_decode_split_kernel<D, GQA, MASKED>), dim3(hk, 1, R),
+                           dim3(kAttnBlock), 0, stream, q, k_pages, v_pages, page_indices,
+                           page_indptr, last_lens, row_begin, row_len, nullptr, nullptr, o, lse,
+                           mask_bits, mask_stride, hq, hk, ps, plan.units_per_split, 1, scale_log2e);
         return launch_status();
     }
     const size_t n_part = static_cast<size_t>(R) * hq * plan.nsplit;
@@ -404,10 +418,10 @@ int launch_decode(const uint16_t* q, const uint16_t* k_pages, const uint16_t* v_
     if (!workspace || workspace_bytes < need) return PIE_HIP_ERR_INVALID;
     float* part_o = static_cast<float*>(workspace);
     float* part_ml = part_o + n_part * D;
-    hipLaunchKernelGGL((attn_decode_split_kernel<D, GQA>), dim3(hk, plan.nsplit, R),
+    hipLaunchKernelGGL((attn_decode_split_kernel<D, GQA, MASKED>), dim3(hk, plan.nsplit, R),
                        dim3(kAttnBlock), 0, stream, q, k_pages, v_pages, page_indices, page_indptr,
-                       last_lens, row_begin, row_len, part_o, part_ml, nullptr, nullptr, hq, hk, ps,
-                       plan.units_per_split, plan.nsplit, scale_log2e);
+                       last_lens, row_begin, row_len, part_o, part_ml, nullptr, nullptr, mask_bits,
+                       mask_stride, hq, hk, ps, plan.units_per_split, plan.nsplit, scale_log2e);
     hipLaunchKernelGGL((attn_decode_merge_kernel<D>), dim3(R * hq), dim3(D), 0, stream, part_o,
                        part_ml, page_indptr, last_lens, row_begin, row_len, o, lse, hq, ps,
                        plan.units_per_split,
@@ -435,7 +449,9 @@ int attn_dispatch(const uint16_t* q, const uint16_t* k_pages, const uint16_t* v_
                   const uint32_t* kv_last_page_lens, const uint32_t* row_begin,
                   const int32_t* row_len, int num_rows, int num_q_heads, int num_kv_heads,
                   int head_dim, int page_size, float sm_scale, int max_kv_len, void* workspace,
-                  size_t workspace_bytes, void* stream) {
+                  size_t workspace_bytes, void* stream, const uint16_t* mask_bits = nullptr,
+                  int mask_stride = 0) {
+    if (mask_bits && mask_stride < (max_kv_len + kUnitTokens - 1) / kUnitTokens) return PIE_HIP_ERR_INVALID;
     if (!q || !k_pages || !v_pages || !o || !kv_page_indices || num_rows <= 0 ||
         num_q_heads <= 0 || num_kv_heads <= 0 || page_size <= 0 || max_kv_len < 0)
         return PIE_HIP_ERR_INVALID;
@@ -446,11 +462,19 @@ int attn_dispatch(const uint16_t* q, const uint16_t* k_pages, const uint16_t* v_
     const int gqa = num_q_heads / num_kv_heads;
     hipStream_t st = static_cast<hipStream_t>(stream);
 #define PIE_ATTN_CASE(DD, GG)                                                                  \
-    if (head_dim == DD && gqa == GG)                                                           \
-        return launch_decode<DD, GG>(q, k_pages, v_pages, o, lse, kv_page_indices,             \
-                                     kv_page_indptr, kv_last_page_lens, row_begin, row_len,    \
-                                     num_rows, num_q_heads, num_kv_heads, page_size, scale,    \
-                                     max_kv_len, workspace, workspace_bytes, st);
+    if (head_dim == DD && gqa == GG) {                                                         \
+        if (mask_bits)                                                                         \
+            return launch_decode<DD, GG, true>(                                                \
+                q, k_pages, v_pages, o, lse, kv_page_indices, kv_page_indptr,                  \
+                kv_last_page_lens, row_begin, row_len, num_rows, num_q_heads, num_kv_heads,    \
+                page_size, scale, max_kv_len, workspace, workspace_bytes, mask_bits,           \
+                mask_stride, st);                                                              \
+        return launch_decode<DD, GG, false>(q, k_pages, v_pages, o, lse, kv_page_indices,      \
+                                            kv_page_indptr, kv_last_page_lens, row_begin,      \
+                                            row_len, num_rows, num_q_heads, num_kv_heads,      \
+                                            page_size, scale, max_kv_len, workspace,           \
+                                            workspace_bytes, nullptr, 0, st);                  \
+    }
     PIE_ATTN_CASE(128, 1)
     PIE_ATTN_CASE(128, 2)
     PIE_ATTN_CASE(128, 4)
@@ -493,4 +517,71 @@ extern "C" int pie_hip_attn_rows_paged(const uint16_t* q, const uint16_t* k_page
                                   row_page_begin, row_kv_len, num_rows, num_q_heads, num_kv_heads,
                                   head_dim, page_size, sm_scale, max_kv_len, workspace,
                                   workspace_bytes, stream);
+}
+
+namespace pie_hip {
+namespace {
+
+// One thread per (row, 16-token unit): bit t = key 16*unit + t is visible to the row.
+// bounds: per row the cumulative ends of its BRLE runs (run j covers [bounds[j-1], bounds[j])
+// and is a visible run when j is odd); a row without runs sees its whole causal window.
+__global__ __launch_bounds__(256) void attn_mask_bitmap_kernel(
+    const uint32_t* __restrict__ bounds, const int32_t* __restrict__ bounds_indptr,
+    const int32_t* __restrict__ row_kv_len, int window, uint16_t* __restrict__ bitmap, int rows,
+    int stride) {
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= rows * stride) return;
+    const int r = idx / stride, unit = idx - r * stride;
+    const int kv_len = row_kv_len[r];                      // visible keys end at the row's position
+    const int lo = window > 0 ? max(0, kv_len - window) : 0;
+    const int b0 = bounds_indptr[r], b1 = bounds_indptr[r + 1];
+    uint32_t word = 0u;
+    for (int t = 0; t < kUnitTokens; ++t) {
+        const int j = unit * kUnitTokens + t;
+        bool vis = j < kv_len && j >= lo;
+        if (vis && b1 > b0) {
+            int a = b0, b = b1;   // first run whose end is past j
+            while (a < b) {
+                const int mid = (a + b) >> 1;
+                if (bounds[mid] > static_cast<uint32_t>(j)) b = mid;
+                else a = mid + 1;
+            }
+            vis = a < b1 && ((a - b0) & 1);
+        }
+        word |= static_cast<uint32_t>(vis) << t;
+    }
+    bitmap[idx] = static_cast<uint16_t>(word);
+}
+
+}  // namespace
+}  // namespace pie_hip
+
+extern "C" int pie_hip_attn_mask_bitmap(const uint32_t* run_bounds, const int32_t* run_bounds_indptr,
+                                        const int32_t* row_kv_len, int window, uint16_t* bitmap,
+                                        int num_rows, int stride_units, void* stream) {
+    using namespace pie_hip;
+    if (!run_bounds_indptr || !row_kv_len || !bitmap || num_rows <= 0 || stride_units <= 0)
+        return PIE_HIP_ERR_INVALID;
+    const long long n = static_cast<long long>(num_rows) * stride_units;
+    if (n > 0x7FFFFFFFll) return PIE_HIP_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(attn_mask_bitmap_kernel, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), run_bounds, run_bounds_indptr, row_kv_len,
+                       window, bitmap, num_rows, stride_units);
+    return launch_status();
+}
+
+extern "C" int pie_hip_attn_rows_paged_masked(const uint16_t* q, const uint16_t* k_pages,
+                                              const uint16_t* v_pages, uint16_t* o, float* lse,
+                                              const uint32_t* kv_page_indices,
+                                              const uint32_t* row_page_begin,
+                                              const int32_t* row_kv_len, const uint16_t* mask_bitmap,
+                                              int mask_stride_units, int num_rows, int num_q_heads,
+                                              int num_kv_heads, int head_dim, int page_size,
+                                              float sm_scale, int max_kv_len, void* workspace,
+                                              size_t workspace_bytes, void* stream) {
+    if (!row_page_begin || !row_kv_len || !mask_bitmap) return PIE_HIP_ERR_INVALID;
+    return pie_hip::attn_dispatch(q, k_pages, v_pages, o, lse, kv_page_indices, nullptr, nullptr,
+                                  row_page_begin, row_kv_len, num_rows, num_q_heads, num_kv_heads,
+                                  head_dim, page_size, sm_scale, max_kv_len, workspace,
+                                  workspace_bytes, stream, mask_bitmap, mask_stride_units);
 }

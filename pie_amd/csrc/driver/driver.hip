@@ -270,8 +270,6 @@ struct PieHipDriver {
         try {
             auto t0 = clk::now();
             const BatchPlan plan = plan_forward(f, exec->page_size(), exec->total_pages());
-            if (plan.has_user_masks)
-                throw std::runtime_error("forward: custom attention masks are not supported by this driver yet");
             if (R > cfg.batching.max_forward_requests)
                 throw std::runtime_error("forward: batch exceeds max_forward_requests");
             const uint32_t plan_us = us_since(t0);

@@ -181,6 +181,7 @@ Executor::~Executor() {
                     static_cast<void*>(moe_offsets_), static_cast<void*>(moe_route_token_),
                     static_cast<void*>(moe_route_pos_)})
         if (p) (void)hipFree(p);
+    for (Growable* g : {&mask_in_host_, &mask_in_dev_, &mask_bitmap_}) g->release();
     for (Growable* g : {&samp_f32_, &samp_ws_, &samp_in_dev_, &samp_in_host_, &samp_out_dev_, &samp_out_host_})
         g->release();
     if (in_host_) (void)hipHostFree(in_host_);
@@ -279,9 +280,16 @@ void Executor::body(int N, int S, int max_kv_len) {
                                                 rope_tab_, slots, N, hq, hk, d, m.rope_interleaved,
                                                 m.rms_eps, s));
         }
-        PIE_KERNEL(pie_hip_attn_rows_paged(q_, k_pool_[l], v_pool_[l], attn_, nullptr, pages,
-                                           row_begin, row_len, N, hq, hk, d, page_size_, -1.f,
-                                           max_kv_len, attn_ws_, attn_ws_bytes_, s));
+        if (masked_) {
+            PIE_KERNEL(pie_hip_attn_rows_paged_masked(
+                q_, k_pool_[l], v_pool_[l], attn_, nullptr, pages, row_begin, row_len,
+                static_cast<const uint16_t*>(mask_bitmap_.ptr), mask_stride_, N, hq, hk, d, page_size_,
+                -1.f, max_kv_len, attn_ws_, attn_ws_bytes_, s));
+        } else {
+            PIE_KERNEL(pie_hip_attn_rows_paged(q_, k_pool_[l], v_pool_[l], attn_, nullptr, pages,
+                                               row_begin, row_len, N, hq, hk, d, page_size_, -1.f,
+                                               max_kv_len, attn_ws_, attn_ws_bytes_, s));
+        }
         linear_fused(w.wo, attn_, nullptr, m.rms_eps, x_, N, 1, 0, xn_, s);
         if (model_.is_moe()) {
             moe_block(w, N, s);
@@ -347,6 +355,39 @@ float pcg32_first_uniform(uint64_t seed) {
 }
 
 }  // namespace
+
+// Custom attention masks: each row's BRLE runs become cumulative bounds, the device expands
+// them into one visibility word per 16-token unit, and the layers' attention reads that.
+void Executor::prepare_masks(const BatchPlan& plan) {
+    const int N = plan.N;
+    std::vector<int32_t> indptr(static_cast<size_t>(N) + 1, 0);
+    std::vector<uint32_t> bounds;
+    for (int i = 0; i < N; ++i) {
+        uint64_t acc = 0;
+        for (uint32_t len : plan.row_mask_runs[i]) {
+            acc = std::min<uint64_t>(acc + len, 0xFFFFFFFFull);
+            bounds.push_back(static_cast<uint32_t>(acc));
+        }
+        indptr[i + 1] = static_cast<int32_t>(bounds.size());
+    }
+    const size_t off_bounds = align_up(4ull * (N + 1), 16);
+    const size_t total = off_bounds + 4ull * std::max<size_t>(bounds.size(), 1);
+    mask_in_host_.pinned = true;
+    mask_in_host_.ensure(total);
+    mask_in_dev_.ensure(total);
+    mask_stride_ = std::max(1, (plan.max_kv_len + 15) / 16);
+    mask_bitmap_.ensure(static_cast<size_t>(N) * mask_stride_ * sizeof(uint16_t));
+    auto* h = static_cast<unsigned char*>(mask_in_host_.ptr);
+    std::memcpy(h, indptr.data(), 4ull * (N + 1));
+    if (!bounds.empty()) std::memcpy(h + off_bounds, bounds.data(), 4ull * bounds.size());
+    PIE_HIP_CHECK(hipMemcpyAsync(mask_in_dev_.ptr, h, total, hipMemcpyHostToDevice, stream_));
+    const auto* dv = static_cast<const unsigned char*>(mask_in_dev_.ptr);
+    const Inputs lay = input_layout(N, static_cast<int>(plan.sample_rows.size()));   // this forward's staging layout
+    const auto* row_len = reinterpret_cast<const int32_t*>(in_dev_ + lay.off_row_len);
+    PIE_KERNEL(pie_hip_attn_mask_bitmap(reinterpret_cast<const uint32_t*>(dv + off_bounds),
+                                        reinterpret_cast<const int32_t*>(dv), row_len, 0,
+                                        static_cast<uint16_t*>(mask_bitmap_.ptr), N, mask_stride_, stream_));
+}
 
 // Host half of the sampler stage: per-slot parameter arrays, uniforms, payload ranges, BRLE
 // bounds — staged in pinned memory and sent to the device ahead of the forward body.
@@ -522,6 +563,8 @@ void Executor::forward(const BatchPlan& plan, std::vector<uint32_t>& tokens_out,
     if (S) std::memcpy(in_host_ + in.off_sample_rows, plan.sample_rows.data(), static_cast<size_t>(S) * 4);
     std::memcpy(in_host_ + in.off_pages, plan.page_indices.data(), plan.page_indices.size() * 4);
     PIE_HIP_CHECK(hipMemcpyAsync(in_dev_, in_host_, used, hipMemcpyHostToDevice, stream_));
+    masked_ = plan.has_user_masks;
+    if (masked_) prepare_masks(plan);
     const bool sampling = !plan.all_greedy && S > 0;
     const int chunk = static_cast<int>(std::min<size_t>(max_tokens_, 2 * static_cast<size_t>(cfg_.batching.max_forward_requests)));
     samp_gather_in_body_ = false;

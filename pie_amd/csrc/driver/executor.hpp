@@ -78,6 +78,7 @@ class Executor {
 
   private:
     void body(int N, int S, int max_kv_len);
+    void prepare_masks(const BatchPlan& plan);
     void prepare_samplers(const BatchPlan& plan);
     void enqueue_samplers();
     void collect_samplers(const BatchPlan& plan, SampleOutputs& out);
@@ -125,6 +126,10 @@ class Executor {
         void ensure(size_t bytes);
         void release();
     };
+    // custom attention masks of the current forward (never part of a captured graph)
+    Growable mask_in_host_, mask_in_dev_, mask_bitmap_;
+    int mask_stride_ = 0;
+    bool masked_ = false;
     Growable samp_f32_, samp_ws_, samp_in_dev_, samp_in_host_, samp_out_dev_, samp_out_host_;
     struct SampLayout {
         size_t kind, temperature, top_k, top_p, min_p, uniform, out_indptr, labels, bounds_indptr,

@@ -52,6 +52,7 @@ struct BatchPlan {
     std::vector<uint32_t> label_ids;         // Logprob / Logprobs labels of all slots
     std::vector<std::vector<uint32_t>> logit_mask_runs;  // [R] BRLE runs (empty = no constraint)
     std::vector<std::vector<uint32_t>> draft_tokens;     // [R] speculative drafts to verify
+    std::vector<std::vector<uint32_t>> row_mask_runs;    // [N] when has_user_masks: BRLE runs per token row
     int max_kv_len = 0;
     bool pure_decode = false;  // every request has exactly one token row, no user masks
     bool all_greedy = false;   // every sampling slot is a token sampler with temperature ~ 0
@@ -153,6 +154,17 @@ inline BatchPlan plan_forward(const PieForwardRequestDesc& f, int page_size, int
                        f.spec_indptr.ptr[R] > f.spec_position_ids.len))
         throw std::runtime_error("plan: spec_indptr exceeds the draft arrays");
     p.has_user_masks = !masks_are_synthesised_causal(f);
+    if (p.has_user_masks) {
+        // one BRLE per token row over its keys [0, position]; no runs = plain causal
+        // (driver/portable/src/plan.cpp:54-94, :296-334)
+        if (f.masks.len != static_cast<size_t>(N))
+            throw std::runtime_error("plan: custom attention masks must be one per token row");
+        p.row_mask_runs.resize(N);
+        for (int i = 0; i < N; ++i) {
+            const PieBrleDesc& m = f.masks.ptr[i];
+            p.row_mask_runs[i].assign(m.buffer.ptr, m.buffer.ptr + m.buffer.len);
+        }
+    }
     p.pure_decode = !p.has_user_masks;
     p.all_greedy = true;
 

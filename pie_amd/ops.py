@@ -588,3 +588,59 @@ def sample(logits_f32: torch.Tensor, kinds, temperature, top_k, top_p, min_p, un
                             _ptr(values), _ptr(ids), _ptr(ws), C.c_size_t(need), S, V, _stream()),
            "pie_hip_sample")
     return tokens, values, ids, indptr
+
+
+# ---------------------------------------------------------------- per-row attention (prefill / mixed)
+def attn_mask_bitmap(mask_runs, row_kv_len: torch.Tensor, max_kv_len: int, window: int = 0):
+    """u16 [rows, ceil(max_kv_len/16)] visibility words from per-row BRLE runs
+    (build_attn_mask_f16, driver/portable/src/plan.cpp:54-94).  Returns (bitmap, stride)."""
+    _dev(row_kv_len, torch.int32, "row_kv_len")
+    rows = row_kv_len.numel()
+    if len(mask_runs) != rows:
+        raise KernelError("one run list per row expected")
+    bounds, indptr = brle_bounds(mask_runs, row_kv_len.device)
+    if indptr is None:
+        indptr = torch.zeros(rows + 1, dtype=torch.int32, device=row_kv_len.device)
+        bounds = torch.zeros(1, dtype=torch.int32, device=row_kv_len.device)
+    stride = max(1, (max_kv_len + 15) // 16)
+    bitmap = torch.empty((rows, stride), dtype=torch.int16, device=row_kv_len.device)
+    _check(kernels().pie_hip_attn_mask_bitmap(_ptr(bounds), _ptr(indptr), _ptr(row_kv_len), window,
+                                              _ptr(bitmap), rows, stride, _stream()),
+           "pie_hip_attn_mask_bitmap")
+    return bitmap, stride
+
+
+def attention_rows_paged(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
+                         kv_page_indices: torch.Tensor, row_page_begin: torch.Tensor,
+                         row_kv_len: torch.Tensor, max_kv_len: int, mask_runs=None, window: int = 0,
+                         lse: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """o[rows, hq, d]: query row r over the first row_kv_len[r] keys of the page list starting at
+    kv_page_indices[row_page_begin[r]]; with `mask_runs` (per-row BRLE) or `window`, over the
+    visible keys only."""
+    _dev(q, torch.bfloat16, "q")
+    _dev(k_pages, torch.bfloat16, "k_pages")
+    for name, t in (("kv_page_indices", kv_page_indices), ("row_page_begin", row_page_begin),
+                    ("row_kv_len", row_kv_len)):
+        _dev(t, torch.int32, name)
+    rows, hq, d = q.shape
+    _, ps, hk, _ = k_pages.shape
+    o = torch.empty_like(q)
+    need = attn_decode_workspace_bytes(rows, hq, hk, d, max_kv_len)
+    ws = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)
+    k = kernels()
+    if mask_runs is None and window <= 0:
+        st = k.pie_hip_attn_rows_paged(_ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(o), _ptr(lse),
+                                       _ptr(kv_page_indices), _ptr(row_page_begin), _ptr(row_kv_len),
+                                       rows, hq, hk, d, ps, C.c_float(-1.0), max_kv_len, _ptr(ws),
+                                       C.c_size_t(need), _stream())
+        _check(st, "pie_hip_attn_rows_paged")
+        return o
+    bitmap, stride = attn_mask_bitmap(mask_runs if mask_runs is not None else [[]] * rows,
+                                      row_kv_len, max_kv_len, window)
+    st = k.pie_hip_attn_rows_paged_masked(_ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(o), _ptr(lse),
+                                          _ptr(kv_page_indices), _ptr(row_page_begin),
+                                          _ptr(row_kv_len), _ptr(bitmap), stride, rows, hq, hk, d, ps,
+                                          C.c_float(-1.0), max_kv_len, _ptr(ws), C.c_size_t(need),
+                                          _stream())
+    _check(st, "pie_hip_attn_rows_paged_masked")
+    return o

@@ -167,3 +167,45 @@ def test_back_to_back_calls_share_workspace(gpu, oracle):
     torch.cuda.synchronize()
     for it, o in outs:
         assert np.array_equal(o.view(torch.uint16).cpu().numpy(), cases[it % 3][0]), it
+
+
+@pytest.mark.parametrize("hq,hk,d", [(8, 2, 128), (4, 4, 64)])
+def test_rows_with_custom_masks_match_oracle(gpu, oracle, hq, hk, d):
+    """Per-row extents with BRLE masks and a sliding window: visible keys only, rows with no
+    visible key give zeros, unmasked rows equal the unmasked entry point."""
+    import torch
+
+    from pie_amd import ops
+
+    rng = np.random.default_rng(55 + d)
+    ps = 16
+    ctx = [300, 77, 1100]
+    b = make_paged_batch(rng, ctx, hk, d, ps, f32_to_bf16=oracle.f32_to_bf16)
+    # rows: (request, position)
+    rows = [(0, 299), (0, 150), (1, 76), (1, 10), (2, 1099), (2, 600), (2, 0), (0, 40)]
+    runs = [[], [10, 50, 20, 1000], [0, 1, 70, 6], [11, 5], [500, 1, 300, 299], [0, 601], [1, 4], [0, 3, 30, 8]]
+    row_begin = np.array([b["page_indptr"][r] for r, _ in rows], np.int32)
+    row_len = np.array([p + 1 for _, p in rows], np.int32)
+    q = oracle.f32_to_bf16(rng.standard_normal((len(rows), hq, d)).astype(np.float32))
+    dev = lambda a, dt=None: (lambda t: t.view(dt) if dt is not None else t)(
+        torch.from_numpy(np.ascontiguousarray(a)).to(gpu))
+    args = (dev(q, torch.bfloat16), dev(b["k_pages"], torch.bfloat16), dev(b["v_pages"], torch.bfloat16),
+            dev(b["page_indices"].view(np.int32)), dev(row_begin), dev(row_len), int(row_len.max()))
+    for window in (0, 64):
+        lse = torch.empty((len(rows), hq), dtype=torch.float32, device=gpu)
+        o = ops.attention_rows_paged(*args, mask_runs=runs, window=window, lse=lse)
+        torch.cuda.synchronize()
+        got = oracle.bf16_to_f32(o.view(torch.uint16).cpu().numpy()).astype(np.float64)
+        allow = [oracle.brle_allow(runs[i], rows[i][1], int(row_len[i]), window) for i in range(len(rows))]
+        truth, _, lse64 = oracle.attn_rows_masked(q, b["k_pages"], b["v_pages"], b["page_indices"],
+                                                  row_begin, row_len, hq, hk, d, ps, allow)
+        tol = 2.0 ** -8 * np.maximum(np.abs(truth), np.abs(got)) + 1e-4
+        assert np.all(np.abs(got - truth) <= tol)
+        fin = np.isfinite(lse64)
+        lg = lse.cpu().numpy()
+        assert np.array_equal(np.isneginf(lg), ~fin) and np.allclose(lg[fin], lse64[fin], atol=1e-4)
+        assert not allow[3].any() and np.all(got[3] == 0)          # runs end before any visible key
+    # no masks, no window: bit-identical to the unmasked entry point
+    plain = ops.attention_rows_paged(*args)
+    masked = ops.attention_rows_paged(*args, mask_runs=[[]] * len(rows))
+    assert torch.equal(plain.view(torch.uint16), masked.view(torch.uint16))

@@ -189,11 +189,11 @@ def test_forward_failures_return_empty_response(gpu):
         ok = dict(token_ids=[1], position_ids=[0], kv_page_indices=[0], kv_page_indptr=[0, 1],
                   kv_last_page_lens=[1], qo_indptr=[0, 1])
         # out-of-range page id, position past the context, a sampler kind without an
-        # implementation (Embedding), user mask
+        # implementation (Embedding), attention masks that are not one per token row
         for bad in (dict(kv_page_indices=[9999]), dict(position_ids=[5]),
                     dict(samplers=[dict(kind=5, temperature=0.8)], sampling_indices=[0],
                          sampling_indptr=[0, 1], sampler_indptr=[0, 1]),
-                    dict(masks=[[1, 0]])):
+                    dict(masks=[[0, 1], [0, 1]])):
             args = dict(ok)
             args.update(bad)
             res = d.forward(drvmod.ForwardFrame(**args))
@@ -261,3 +261,52 @@ def test_run_inproc_serve_loop(gpu, tmp_path):
     # a missing config is an error return, not a crash
     argv2 = (C.c_char_p * 1)(b"pie-driver-hip")
     assert drvmod.lib().pie_driver_hip_run_inproc(1, argv2, 0, ready, None, vt) == -1
+
+
+def test_custom_attention_masks_match_oracle(gpu, oracle):
+    """Prefill and a decode step under per-token BRLE attention masks
+    (build_attn_mask_f16, driver/portable/src/plan.cpp:54-94) against the oracle model."""
+    from pie_amd import driver as drvmod
+
+    kw = dict(quant="int8")
+    cfg = full_cfg(**kw)
+    V, ps = cfg["vocab"], cfg["page_size"]
+    rng = np.random.default_rng(93)
+    n = 45
+    prompt = rng.integers(0, V, n)
+    masks = []
+    for i in range(n):
+        if i % 4 == 0:
+            masks.append([])                              # no runs: plain causal
+        elif i % 4 == 1:
+            masks.append([0, i + 1])                      # the synthesised causal shape
+        else:
+            a = int(rng.integers(0, i + 1))
+            b = int(rng.integers(1, 8))
+            masks.append([a, b, int(rng.integers(0, 5)), n])   # a hole pattern, clipped at i
+    masks[7] = [0, 1, 100]                                # only key 0
+    with drvmod.Driver(toml_config(**kw)) as d:
+        om, _ = oracle_model_from_driver(d, cfg)
+        npg = (n + ps - 1) // ps
+        args = dict(token_ids=prompt, position_ids=np.arange(n), kv_page_indices=np.arange(npg),
+                    kv_page_indptr=[0, npg], kv_last_page_lens=[n - (npg - 1) * ps], qo_indptr=[0, n],
+                    sampling_indices=[n - 1, 7, 20], sampling_indptr=[0, 3])
+        res = d.forward(drvmod.ForwardFrame(**args, masks=masks))
+        assert res.num_requests == 1 and len(res.tokens) == 3
+        otok, olog, _ = om.forward(**args, masks=masks, want_logits=True)
+        glog = d.export_tensor("debug.logits", np.uint16).reshape(-1, V)
+        for i in range(3):
+            check_step(oracle, glog[i], olog[i], res.tokens[i], otok[i])
+        masked_row7 = olog[1].copy()
+        # a decode step that hides the first half of the context
+        step = dict(token_ids=[int(res.tokens[0])], position_ids=[n], kv_page_indices=np.arange(npg),
+                    kv_page_indptr=[0, npg], kv_last_page_lens=[n + 1 - (npg - 1) * ps], qo_indptr=[0, 1])
+        m = [[n // 2, n]]
+        res = d.forward(drvmod.ForwardFrame(**step, masks=m))
+        otok, olog, _ = om.forward(**step, masks=m, want_logits=True)
+        glog = d.export_tensor("debug.logits", np.uint16).reshape(-1, V)
+        check_step(oracle, glog[0], olog[0], res.tokens[0], otok[0])
+        # the masks matter: without them the oracle gives different logits on a masked row
+        # (last: this run overwrites the oracle's KV pool)
+        _, plain, _ = om.forward(**args, want_logits=True)
+        assert cosine(oracle.bf16_to_f32(plain[1]), oracle.bf16_to_f32(masked_row7)) < 0.999

@@ -136,3 +136,49 @@ def test_kv_write_slots(oracle):
             assert np.array_equal(vp[pages[pos // ps], pos % ps], vc[qo[r] + i])
             written += 1
     assert np.count_nonzero(kp.reshape(-1, hk * d).any(axis=1)) == written
+
+
+def test_brle_visibility_follows_the_mask_builder(oracle):
+    """build_attn_mask_f16 (driver/portable/src/plan.cpp:54-94) on hand-worked rows."""
+    b = lambda runs, pos, n_kv, w=0: list(oracle.brle_allow(runs, pos, n_kv, w))
+    assert b([], 3, 6) == [1, 1, 1, 1, 0, 0]                       # plain causal
+    assert b([], 3, 6, 2) == [0, 0, 1, 1, 0, 0]                    # sliding window of 2
+    assert b([0, 4], 3, 6) == [1, 1, 1, 1, 0, 0]                   # the synthesised causal shape
+    assert b([1, 2, 1, 5], 5, 8) == [0, 1, 1, 0, 1, 1, 0, 0]       # holes; nothing past pos
+    assert b([0, 2], 5, 8) == [1, 1, 0, 0, 0, 0, 0, 0]             # past the last run: hidden
+    assert b([0, 100], 2, 8) == [1, 1, 1, 0, 0, 0, 0, 0]           # a mask cannot unmask the future
+    assert b([2, 3], 9, 4) == [0, 0, 1, 1]                         # clipped to the context
+    assert b([0, 6], 5, 8, 3) == [0, 0, 0, 1, 1, 1, 0, 0]          # window clips a true run
+
+
+def test_masked_rows_equal_dense_attention_over_the_allowed_keys(oracle):
+    from paged_cases import make_paged_batch
+
+    rng = np.random.default_rng(77)
+    hq, hk, d, ps = 4, 2, 64, 16
+    ctx = [37, 20]
+    b = make_paged_batch(rng, ctx, hk, d, ps, f32_to_bf16=oracle.f32_to_bf16)
+    # rows: three queries of request 0 (positions 30, 33, 36) and one of request 1
+    row_begin = [int(b["page_indptr"][0])] * 3 + [int(b["page_indptr"][1])]
+    row_len = [31, 34, 37, 20]
+    q = oracle.f32_to_bf16(rng.standard_normal((4, hq, d)).astype(np.float32))
+    allow = [oracle.brle_allow([3, 10, 5, 40], 30, 31), None,
+             oracle.brle_allow([0, 1, 35, 1], 36, 37), np.zeros(20, np.uint8)]
+    o32, _, lse = oracle.attn_rows_masked(q, b["k_pages"], b["v_pages"], b["page_indices"], row_begin,
+                                          row_len, hq, hk, d, ps, allow)
+    kf, vf = oracle.bf16_to_f32(b["k_pages"]).astype(np.float64), oracle.bf16_to_f32(b["v_pages"]).astype(np.float64)
+    qf = oracle.bf16_to_f32(q).astype(np.float64)
+    for r in range(4):
+        pages = b["page_indices"][row_begin[r]:]
+        keys = np.array([pages[j // ps] * ps + j % ps for j in range(row_len[r])])
+        vis = np.ones(row_len[r], bool) if allow[r] is None else allow[r][:row_len[r]].astype(bool)
+        for h in range(hq):
+            K = kf.reshape(-1, hk, d)[keys[vis], h // (hq // hk)]
+            Vv = vf.reshape(-1, hk, d)[keys[vis], h // (hq // hk)]
+            if not vis.any():
+                assert np.all(o32[r, h] == 0) and np.isneginf(lse[r, h])
+                continue
+            s = K @ qf[r, h] / np.sqrt(d)
+            p = np.exp(s - s.max())
+            assert np.allclose(o32[r, h], (p / p.sum()) @ Vv, rtol=1e-5, atol=1e-6)
+            assert abs(lse[r, h] - (np.log(p.sum()) + s.max())) < 1e-4
