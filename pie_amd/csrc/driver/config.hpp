@@ -38,6 +38,10 @@ struct ModelConfig {
     std::uint64_t seed = 0x9E3779B97F4A7C15ull;
     float init_std = 0.02f;
     float router_std = 0.f;  // MoE router rows; 0 = init_std
+    // `[model] hf_path` (portable driver's key) or `snapshot_dir` (CUDA driver's key): a Hugging
+    // Face snapshot directory; its config.json then fixes the shape fields above and the weights
+    // come from its safetensors files instead of the synthetic initialiser
+    std::string checkpoint_dir;
 };
 
 struct BatchingConfig {
@@ -133,6 +137,34 @@ inline std::map<std::string, std::map<std::string, std::string>> parse_toml_lite
     return out;
 }
 
+// Shape and range checks, defaults that depend on other fields.
+inline void finalize_config(DriverConfig& c) {
+    auto& m = c.model;
+    if (m.hidden <= 0 || m.layers <= 0 || m.q_heads <= 0 || m.kv_heads <= 0 || m.vocab <= 0)
+        throw std::runtime_error("config: [model] needs hidden, layers, q_heads, kv_heads, vocab");
+    if (m.head_dim <= 0) m.head_dim = m.hidden / m.q_heads;
+    if (m.q_heads % m.kv_heads != 0) throw std::runtime_error("config: q_heads must be a multiple of kv_heads");
+    const bool moe = m.arch == "qwen3_moe";
+    if (m.arch != "llama3" && m.arch != "qwen3" && !moe)
+        throw std::runtime_error("config: unsupported arch '" + m.arch + "'");
+    if (moe) {
+        if (m.num_experts <= 0 || m.top_k <= 0 || m.expert_intermediate <= 0 || m.top_k > m.num_experts)
+            throw std::runtime_error("config: qwen3_moe needs num_experts, top_k, expert_intermediate");
+    } else if (m.intermediate <= 0) {
+        throw std::runtime_error("config: [model] needs intermediate");
+    }
+    if (m.quant != "int4b8" && m.quant != "int8" && m.quant != "fp8" && m.quant != "bf16")
+        throw std::runtime_error("config: unsupported quant '" + m.quant + "'");
+    if (m.scale_dtype != "bf16" && m.scale_dtype != "f32")
+        throw std::runtime_error("config: scale_dtype must be bf16 or f32");
+    if (m.rope_interleaved < 0) m.rope_interleaved = (m.arch == "llama3") ? 1 : 0;
+    const auto& b = c.batching;
+    if (b.kv_page_size <= 0 || b.kv_page_size % 16 != 0)
+        throw std::runtime_error("config: kv_page_size must be a positive multiple of 16");
+    if (b.total_pages <= 0 || b.max_forward_tokens <= 0 || b.max_forward_requests <= 0)
+        throw std::runtime_error("config: [batching] sizes must be positive");
+}
+
 inline DriverConfig parse_config_text(const std::string& text) {
     using namespace detail;
     DriverConfig c;
@@ -169,6 +201,7 @@ inline DriverConfig parse_config_text(const std::string& text) {
                 else if (k == "seed") m.seed = (std::uint64_t)to_int(v, key);
                 else if (k == "init_std") m.init_std = (float)to_float(v, key);
                 else if (k == "router_std") m.router_std = (float)to_float(v, key);
+                else if (k == "hf_path" || k == "snapshot_dir") m.checkpoint_dir = v;
                 // other [model] keys (paths, dtype hints) belong to loaders this driver lacks
             } else if (sec == "batching") {
                 auto& b = c.batching;
@@ -186,30 +219,7 @@ inline DriverConfig parse_config_text(const std::string& text) {
             }
         }
     }
-    auto& m = c.model;
-    if (m.hidden <= 0 || m.layers <= 0 || m.q_heads <= 0 || m.kv_heads <= 0 || m.vocab <= 0)
-        throw std::runtime_error("config: [model] needs hidden, layers, q_heads, kv_heads, vocab");
-    if (m.head_dim <= 0) m.head_dim = m.hidden / m.q_heads;
-    if (m.q_heads % m.kv_heads != 0) throw std::runtime_error("config: q_heads must be a multiple of kv_heads");
-    const bool moe = m.arch == "qwen3_moe";
-    if (m.arch != "llama3" && m.arch != "qwen3" && !moe)
-        throw std::runtime_error("config: unsupported arch '" + m.arch + "'");
-    if (moe) {
-        if (m.num_experts <= 0 || m.top_k <= 0 || m.expert_intermediate <= 0 || m.top_k > m.num_experts)
-            throw std::runtime_error("config: qwen3_moe needs num_experts, top_k, expert_intermediate");
-    } else if (m.intermediate <= 0) {
-        throw std::runtime_error("config: [model] needs intermediate");
-    }
-    if (m.quant != "int4b8" && m.quant != "int8" && m.quant != "fp8" && m.quant != "bf16")
-        throw std::runtime_error("config: unsupported quant '" + m.quant + "'");
-    if (m.scale_dtype != "bf16" && m.scale_dtype != "f32")
-        throw std::runtime_error("config: scale_dtype must be bf16 or f32");
-    if (m.rope_interleaved < 0) m.rope_interleaved = (m.arch == "llama3") ? 1 : 0;
-    const auto& b = c.batching;
-    if (b.kv_page_size <= 0 || b.kv_page_size % 16 != 0)
-        throw std::runtime_error("config: kv_page_size must be a positive multiple of 16");
-    if (b.total_pages <= 0 || b.max_forward_tokens <= 0 || b.max_forward_requests <= 0)
-        throw std::runtime_error("config: [batching] sizes must be positive");
+    if (c.model.checkpoint_dir.empty()) finalize_config(c);   // else after config.json is applied
     return c;
 }
 

@@ -22,6 +22,7 @@
 #include "model.hpp"
 #include "pie_driver_abi.h"
 #include "planner.hpp"
+#include "snapshot.hpp"
 
 using namespace pie_hip_driver;
 
@@ -207,6 +208,17 @@ std::string json_escape(const std::string& s) {
 
 }  // namespace
 
+// TOML, then (with `[model] hf_path` / `snapshot_dir`) the snapshot's config.json for the shape.
+static DriverConfig load_driver_config(const std::string& src) {
+    DriverConfig c = load_config(src);
+    if (!c.model.checkpoint_dir.empty()) {
+        apply_hf_config(c.model, c.model.checkpoint_dir);
+        finalize_config(c);
+        if (c.runtime.snapshot_dir.empty()) c.runtime.snapshot_dir = c.model.checkpoint_dir;
+    }
+    return c;
+}
+
 struct PieHipDriver {
     DriverConfig cfg;
     Model model;
@@ -227,7 +239,8 @@ struct PieHipDriver {
         if (hipStreamCreateWithFlags(&s, hipStreamNonBlocking) != hipSuccess)
             throw std::runtime_error("cannot create a HIP stream");
         try {
-            model.init_synthetic(cfg.model, s);
+            if (cfg.model.checkpoint_dir.empty()) model.init_synthetic(cfg.model, s);
+            else model.load_snapshot(cfg.model, s);
         } catch (...) {
             (void)hipStreamDestroy(s);
             throw;
@@ -390,7 +403,7 @@ PieSamplerDesc greedy_sampler() {
 extern "C" PieHipDriver* pie_hip_driver_create(const char* config_toml, char* err, size_t err_cap) {
     try {
         if (!config_toml) throw std::runtime_error("null config");
-        return new PieHipDriver(load_config(config_toml));
+        return new PieHipDriver(load_driver_config(config_toml));
     } catch (const std::exception& e) {
         set_err(err, err_cap, e.what());
         return nullptr;
@@ -640,7 +653,7 @@ extern "C" int pie_driver_hip_run_inproc(int argc, char** argv, int install_sign
             std::signal(SIGTERM, [](int) { g_stop.store(true); });
         }
         g_stop.store(false, std::memory_order_release);
-        PieHipDriver driver(load_config(config_path));
+        PieHipDriver driver(load_driver_config(config_path));
         if (ready_cb) ready_cb(driver.caps.c_str(), ready_ctx);
         if (driver.cfg.runtime.verbose) std::fprintf(stderr, "[pie-driver-hip] serving on in-process channel\n");
         PieResponseFrameDesc resp;
@@ -666,6 +679,45 @@ extern "C" int pie_driver_hip_run_inproc(int argc, char** argv, int install_sign
         return -1;
     } catch (...) {
         std::fprintf(stderr, "[pie-driver-hip] fatal: unknown error\n");
+        return -1;
+    }
+}
+
+// Host-only snapshot hook: reads `<dir>/config.json` and the safetensors headers and writes a
+// JSON summary {"arch", the shape fields, "tensors": {name: {"dtype", "shape", "bytes",
+// "first_bytes": [up to 8 leading data bytes]}}} into out.  Returns its length, or -1 with the
+// reader's message in err.  No GPU is touched.
+extern "C" long long pie_hip_driver_snapshot_info(const char* dir, char* out, size_t out_cap,
+                                                  char* err, size_t err_cap) {
+    try {
+        if (!dir || !out) throw std::runtime_error("null argument");
+        ModelConfig m;
+        apply_hf_config(m, dir);
+        const Snapshot snap(dir);
+        std::ostringstream j;
+        j << "{\"arch\":\"" << m.arch << "\",\"hidden\":" << m.hidden << ",\"layers\":" << m.layers
+          << ",\"q_heads\":" << m.q_heads << ",\"kv_heads\":" << m.kv_heads << ",\"head_dim\":" << m.head_dim
+          << ",\"intermediate\":" << m.intermediate << ",\"vocab\":" << m.vocab
+          << ",\"rms_eps\":" << m.rms_eps << ",\"rope_theta\":" << m.rope_theta
+          << ",\"rope_factor\":" << m.rope_factor << ",\"tie_embeddings\":" << (m.tie_embeddings ? "true" : "false")
+          << ",\"num_experts\":" << m.num_experts << ",\"top_k\":" << m.top_k
+          << ",\"expert_intermediate\":" << m.expert_intermediate << ",\"tensors\":{";
+        bool first = true;
+        for (const auto& [name, t] : snap.tensors()) {
+            j << (first ? "" : ",") << "\"" << json_escape(name) << "\":{\"dtype\":\"" << t.dtype << "\",\"shape\":[";
+            for (size_t i = 0; i < t.shape.size(); ++i) j << (i ? "," : "") << t.shape[i];
+            j << "],\"bytes\":" << t.bytes << ",\"first_bytes\":[";
+            for (size_t i = 0; i < std::min<size_t>(8, t.bytes); ++i) j << (i ? "," : "") << static_cast<int>(t.data[i]);
+            j << "]}";
+            first = false;
+        }
+        j << "}}";
+        const std::string text = j.str();
+        if (text.size() + 1 > out_cap) throw std::runtime_error("output buffer too small");
+        std::memcpy(out, text.c_str(), text.size() + 1);
+        return static_cast<long long>(text.size());
+    } catch (const std::exception& e) {
+        set_err(err, err_cap, e.what());
         return -1;
     }
 }

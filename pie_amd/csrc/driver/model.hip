@@ -4,6 +4,7 @@
 #include <stdexcept>
 
 #include "pie_hip_kernels.h"
+#include "snapshot.hpp"
 
 namespace pie_hip_driver {
 
@@ -119,26 +120,29 @@ void* Model::alloc(size_t bytes, const std::string& name) {
     return p;
 }
 
-void Model::make_linear(Linear& lin, int N, int K, const std::string& name, std::uint64_t seed,
-                        hipStream_t stream) {
+void Model::prepare_linear(Linear& lin, int N, int K, const std::string& name) {
     lin.kind = quant_;
     lin.N = N;
     lin.K = K;
     lin.group = cfg_.group_size;
     lin.scale_bf16 = cfg_.scale_dtype == "bf16";
-    const size_t nk = static_cast<size_t>(N) * K;
     if (quant_ == Quant::Int4b8 && (K % lin.group != 0 || lin.group % 32 != 0))
         throw std::runtime_error("model: int4b8 needs K % group == 0 and group % 32 == 0 (" + name + ")");
     lin.data = alloc(lin.data_bytes(), name + ".data");
     if (lin.scale_bytes()) lin.scale = alloc(lin.scale_bytes(), name + ".scale");
     decode_bytes_ += lin.data_bytes() + lin.scale_bytes();
+    if (quant_ != Quant::Bf16 && static_cast<size_t>(N) * K > tmp_elems_)
+        throw std::runtime_error("model: scratch too small for " + name);
+}
+
+// [N, K] bf16 in the scratch buffer -> the linear's storage format.
+void Model::quantise_scratch(Linear& lin, const std::string& name, hipStream_t stream) {
+    const int N = lin.N, K = lin.K;
+    int st = 0;
     if (quant_ == Quant::Bf16) {
-        fill_normal(static_cast<uint16_t*>(lin.data), nk, seed, 0.f, cfg_.init_std, stream);
+        PIE_HIP_CHECK(hipMemcpyAsync(lin.data, tmp_bf16_, lin.data_bytes(), hipMemcpyDeviceToDevice, stream));
         return;
     }
-    if (nk > tmp_elems_) throw std::runtime_error("model: scratch too small for " + name);
-    fill_normal(tmp_bf16_, nk, seed, 0.f, cfg_.init_std, stream);
-    int st = 0;
     if (quant_ == Quant::Int4b8) {
         st = pie_hip_quant_int4b8_group(tmp_bf16_, static_cast<uint32_t*>(lin.data),
                                         static_cast<uint16_t*>(lin.scale), N, K, lin.group, stream);
@@ -157,6 +161,18 @@ void Model::make_linear(Linear& lin, int N, int K, const std::string& name, std:
         }
     }
     if (st != 0) throw std::runtime_error("model: quantiser failed for " + name);
+}
+
+void Model::make_linear(Linear& lin, int N, int K, const std::string& name, std::uint64_t seed,
+                        hipStream_t stream) {
+    prepare_linear(lin, N, K, name);
+    const size_t nk = static_cast<size_t>(N) * K;
+    if (quant_ == Quant::Bf16) {
+        fill_normal(static_cast<uint16_t*>(lin.data), nk, seed, 0.f, cfg_.init_std, stream);
+        return;
+    }
+    fill_normal(tmp_bf16_, nk, seed, 0.f, cfg_.init_std, stream);
+    quantise_scratch(lin, name, stream);
 }
 
 // Re-orders the rows of a fused gate/up projection from (all gate rows, all up rows) to
@@ -254,6 +270,198 @@ void Model::init_synthetic(const ModelConfig& cfg, hipStream_t stream) {
             interleave_gate_up(w.wgu, E, stream);
             make_linear(w.wdown, E * H, I, p + "wdown", next_seed(), stream);
             // a batch-1 decode step touches top_k of the E experts
+            const size_t all = decode_bytes_ - before;
+            decode_bytes_ = before + all / E * cfg.top_k + static_cast<size_t>(E) * H * 2;
+        }
+    }
+    PIE_HIP_CHECK(hipStreamSynchronize(stream));
+    (void)hipFree(tmp_bf16_);
+    tmp_bf16_ = nullptr;
+}
+
+namespace {
+
+// Widens / narrows a checkpoint tensor to bf16 bits on the host when it is not bf16 already.
+const uint16_t* as_bf16(const StTensor& t, std::vector<uint16_t>& staging) {
+    const size_t n = static_cast<size_t>(t.elems());
+    if (t.dtype == "BF16") {
+        if (t.bytes != n * 2) throw std::runtime_error("snapshot: BF16 tensor with a wrong byte count");
+        return reinterpret_cast<const uint16_t*>(t.data);
+    }
+    staging.resize(n);
+    auto rne = [](float f) {
+        uint32_t u;
+        std::memcpy(&u, &f, 4);
+        if ((u & 0x7FFFFFFFu) > 0x7F800000u) return static_cast<uint16_t>((u >> 16) | 0x40u);
+        return static_cast<uint16_t>((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
+    };
+    if (t.dtype == "F32") {
+        if (t.bytes != n * 4) throw std::runtime_error("snapshot: F32 tensor with a wrong byte count");
+        for (size_t i = 0; i < n; ++i) {
+            float f;
+            std::memcpy(&f, t.data + 4 * i, 4);
+            staging[i] = rne(f);
+        }
+    } else if (t.dtype == "F16") {
+        if (t.bytes != n * 2) throw std::runtime_error("snapshot: F16 tensor with a wrong byte count");
+        for (size_t i = 0; i < n; ++i) {
+            uint16_t h;
+            std::memcpy(&h, t.data + 2 * i, 2);
+            const uint32_t sign = (h & 0x8000u) << 16, exp = (h >> 10) & 0x1Fu, man = h & 0x3FFu;
+            uint32_t u;
+            if (exp == 0) {
+                if (man == 0) u = sign;
+                else {   // subnormal half: normalise
+                    int e = -1;
+                    uint32_t m2 = man;
+                    do { ++e; m2 <<= 1; } while (!(m2 & 0x400u));
+                    u = sign | ((127 - 15 - e) << 23) | ((m2 & 0x3FFu) << 13);
+                }
+            } else if (exp == 31) u = sign | 0x7F800000u | (man << 13);
+            else u = sign | ((exp + 112) << 23) | (man << 13);
+            float f;
+            std::memcpy(&f, &u, 4);
+            staging[i] = rne(f);
+        }
+    } else {
+        throw std::runtime_error("snapshot: dtype " + t.dtype + " is not a floating weight");
+    }
+    return staging.data();
+}
+
+void expect_shape(const StTensor& t, const std::string& name, int64_t rows, int64_t cols) {
+    const bool ok = cols < 0 ? (t.shape.size() == 1 && t.shape[0] == rows)
+                             : (t.shape.size() == 2 && t.shape[0] == rows && t.shape[1] == cols);
+    if (!ok) throw std::runtime_error("snapshot: tensor '" + name + "' has an unexpected shape");
+}
+
+}  // namespace
+
+void Model::load_snapshot(const ModelConfig& cfg, hipStream_t stream) {
+    cfg_ = cfg;
+    quant_ = parse_quant(cfg.quant);
+    const Snapshot snap(cfg.checkpoint_dir);
+    const int H = cfg.hidden, d = cfg.head_dim, hq = cfg.q_heads, hk = cfg.kv_heads;
+    const int V = cfg.vocab, L = cfg.layers;
+    const bool moe = is_moe();
+    const int I = moe ? cfg.expert_intermediate : cfg.intermediate;
+    const int E = moe ? cfg.num_experts : 1;
+    if (H % 32 != 0 || d % 8 != 0 || I % 32 != 0 || V % 8 != 0)
+        throw std::runtime_error("model: hidden/intermediate must be multiples of 32, head_dim and vocab of 8");
+
+    size_t biggest = static_cast<size_t>((hq + 2 * hk) * d) * H;
+    biggest = std::max(biggest, static_cast<size_t>(2 * I) * H * E);
+    biggest = std::max(biggest, static_cast<size_t>(H) * hq * d);
+    tmp_elems_ = biggest;
+    PIE_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&tmp_bf16_), biggest * 2));
+    std::vector<uint16_t> staging;
+
+    // rows of a checkpoint tensor -> device bf16 at `dst` (+ row offset)
+    auto upload = [&](const std::string& name, uint16_t* dst, int64_t rows, int64_t cols) {
+        const StTensor& t = snap.at(name);
+        expect_shape(t, name, rows, cols);
+        const uint16_t* src = as_bf16(t, staging);
+        PIE_HIP_CHECK(hipMemcpyAsync(dst, src, static_cast<size_t>(t.elems()) * 2, hipMemcpyHostToDevice, stream));
+        PIE_HIP_CHECK(hipStreamSynchronize(stream));   // `staging` is reused by the next tensor
+    };
+    auto vector_param = [&](const std::string& src, const std::string& name, int n) {
+        auto* p = static_cast<uint16_t*>(alloc(static_cast<size_t>(n) * 2, name));
+        upload(src, p, n, -1);
+        return p;
+    };
+
+    embed = static_cast<uint16_t*>(alloc(static_cast<size_t>(V) * H * 2, "embed"));
+    upload("model.embed_tokens.weight", embed, V, H);
+    if (cfg.tie_embeddings || !snap.find("lm_head.weight")) {
+        lm_head = embed;
+        names_["lm_head"] = names_["embed"];
+    } else {
+        lm_head = static_cast<uint16_t*>(alloc(static_cast<size_t>(V) * H * 2, "lm_head"));
+        upload("lm_head.weight", lm_head, V, H);
+    }
+    decode_bytes_ += static_cast<size_t>(V) * H * 2;
+    final_norm = vector_param("model.norm.weight", "final_norm", H);
+    const std::vector<float> f = rope_inv_freq(cfg);
+    inv_freq = static_cast<float*>(alloc(f.size() * 4, "inv_freq"));
+    PIE_HIP_CHECK(hipMemcpyAsync(inv_freq, f.data(), f.size() * 4, hipMemcpyHostToDevice, stream));
+    PIE_HIP_CHECK(hipStreamSynchronize(stream));
+
+    // One fused linear from several checkpoint projections, rows concatenated in order.
+    struct Part {
+        std::string prefix;   // e.g. "model.layers.0.self_attn.q_proj"
+        int rows;
+    };
+    auto fused = [&](Linear& lin, const std::vector<Part>& parts, int K, const std::string& name) {
+        int N = 0;
+        for (const Part& p : parts) N += p.rows;
+        prepare_linear(lin, N, K, name);
+        const bool packed = snap.find(parts[0].prefix + ".weight_packed") != nullptr;
+        if (packed) {
+            // compressed-tensors pack-quantized int4: nibble j of word w = element 8w + j,
+            // stored value + 8 (the layout of driver/cuda/src/kernels/dequant_wna16.cu:31-36)
+            if (quant_ != Quant::Int4b8)
+                throw std::runtime_error("snapshot: '" + name + "' is packed int4; set quant = \"int4b8\"");
+            size_t row = 0;
+            for (const Part& p : parts) {
+                const StTensor& w = snap.at(p.prefix + ".weight_packed");
+                const StTensor& sc = snap.at(p.prefix + ".weight_scale");
+                if (w.dtype != "I32" && w.dtype != "U32") throw std::runtime_error("snapshot: weight_packed must be I32");
+                expect_shape(w, p.prefix + ".weight_packed", p.rows, K / 8);
+                expect_shape(sc, p.prefix + ".weight_scale", p.rows, K / lin.group);
+                PIE_HIP_CHECK(hipMemcpyAsync(static_cast<uint8_t*>(lin.data) + row * (K / 2), w.data, w.bytes,
+                                             hipMemcpyHostToDevice, stream));
+                const uint16_t* sb = as_bf16(sc, staging);
+                PIE_HIP_CHECK(hipMemcpyAsync(static_cast<uint16_t*>(lin.scale) + row * (K / lin.group), sb,
+                                             static_cast<size_t>(sc.elems()) * 2, hipMemcpyHostToDevice, stream));
+                PIE_HIP_CHECK(hipStreamSynchronize(stream));
+                row += p.rows;
+            }
+            return;
+        }
+        uint16_t* dst = quant_ == Quant::Bf16 ? static_cast<uint16_t*>(lin.data) : tmp_bf16_;
+        size_t row = 0;
+        for (const Part& p : parts) {
+            upload(p.prefix + ".weight", dst + row * K, p.rows, K);
+            row += p.rows;
+        }
+        if (quant_ != Quant::Bf16) quantise_scratch(lin, name, stream);
+    };
+
+    layers.resize(L);
+    for (int l = 0; l < L; ++l) {
+        LayerWeights& w = layers[l];
+        const std::string p = "layers." + std::to_string(l) + ".";
+        const std::string hf = "model.layers." + std::to_string(l) + ".";
+        w.attn_norm = vector_param(hf + "input_layernorm.weight", p + "attn_norm", H);
+        w.ffn_norm = vector_param(hf + "post_attention_layernorm.weight", p + "ffn_norm", H);
+        if (has_qk_norm()) {
+            w.q_norm = vector_param(hf + "self_attn.q_norm.weight", p + "q_norm", d);
+            w.k_norm = vector_param(hf + "self_attn.k_norm.weight", p + "k_norm", d);
+        }
+        fused(w.wqkv, {{hf + "self_attn.q_proj", hq * d}, {hf + "self_attn.k_proj", hk * d},
+                       {hf + "self_attn.v_proj", hk * d}}, H, p + "wqkv");
+        fused(w.wo, {{hf + "self_attn.o_proj", H}}, hq * d, p + "wo");
+        if (!moe) {
+            fused(w.wgu, {{hf + "mlp.gate_proj", I}, {hf + "mlp.up_proj", I}}, H, p + "wgu");
+            interleave_gate_up(w.wgu, 1, stream);
+            fused(w.wdown, {{hf + "mlp.down_proj", H}}, I, p + "wdown");
+        } else {
+            w.router.kind = Quant::Bf16;
+            w.router.N = E;
+            w.router.K = H;
+            w.router.data = alloc(static_cast<size_t>(E) * H * 2, p + "router");
+            upload(hf + "mlp.gate.weight", static_cast<uint16_t*>(w.router.data), E, H);
+            std::vector<Part> gu, down;
+            for (int e = 0; e < E; ++e) {
+                const std::string ex = hf + "mlp.experts." + std::to_string(e) + ".";
+                gu.push_back({ex + "gate_proj", I});
+                gu.push_back({ex + "up_proj", I});
+                down.push_back({ex + "down_proj", H});
+            }
+            const size_t before = decode_bytes_;
+            fused(w.wgu, gu, H, p + "wgu");
+            interleave_gate_up(w.wgu, E, stream);
+            fused(w.wdown, down, I, p + "wdown");
             const size_t all = decode_bytes_ - before;
             decode_bytes_ = before + all / E * cfg.top_k + static_cast<size_t>(E) * H * 2;
         }

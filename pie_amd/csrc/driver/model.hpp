@@ -73,6 +73,12 @@ class Model {
     // N(0, init_std) rounded to bf16, then quantised by the library's quantiser kernels.
     void init_synthetic(const ModelConfig& cfg, hipStream_t stream);
 
+    // The same layout filled from a Hugging Face snapshot (cfg.checkpoint_dir): bf16 / f16 / f32
+    // `*.weight` tensors are fused (q|k|v rows, gate/up interleaved, experts stacked) and
+    // quantised on the device to cfg.quant; compressed-tensors int4 checkpoints
+    // (`weight_packed` int32 [N, K/8] + `weight_scale` [N, K/group]) are taken as stored.
+    void load_snapshot(const ModelConfig& cfg, hipStream_t stream);
+
     const ModelConfig& cfg() const { return cfg_; }
     bool is_moe() const { return cfg_.arch == "qwen3_moe"; }
     bool has_qk_norm() const { return cfg_.arch != "llama3"; }
@@ -92,6 +98,8 @@ class Model {
     void* alloc(size_t bytes, const std::string& name);
     void make_linear(Linear& lin, int N, int K, const std::string& name, std::uint64_t seed,
                      hipStream_t stream);
+    void prepare_linear(Linear& lin, int N, int K, const std::string& name);
+    void quantise_scratch(Linear& lin, const std::string& name, hipStream_t stream);
     void interleave_gate_up(Linear& lin, int blocks, hipStream_t stream);
     ModelConfig cfg_;
     Quant quant_ = Quant::Bf16;

@@ -395,6 +395,22 @@ class Driver:
         return arr
 
 
+def snapshot_info(directory: str) -> dict:
+    """Host-only: what the driver's snapshot reader sees in a Hugging Face checkpoint directory
+    (config.json fields as the driver maps them, and every safetensors entry)."""
+    import json
+
+    out = C.create_string_buffer(8 << 20)
+    err = C.create_string_buffer(1024)
+    f = lib().pie_hip_driver_snapshot_info
+    f.restype = C.c_longlong
+    f.argtypes = [C.c_char_p, C.c_char_p, C.c_size_t, C.c_char_p, C.c_size_t]
+    n = f(directory.encode(), out, len(out), err, len(err))
+    if n < 0:
+        raise RuntimeError(f"pie_hip_driver_snapshot_info: {err.value.decode()}")
+    return json.loads(out.value.decode())
+
+
 def plan(frame: ForwardFrame, page_size: int, total_pages: int) -> dict:
     """Runs the driver's host-side planner (no GPU) and returns its integer plan."""
     f = frame.frame.payload.forward
