@@ -305,19 +305,30 @@ struct PieHipDriver {
         }
     }
 
+    // Status codes and checks of driver/portable/src/service/inproc_service.cpp:82-203: a length
+    // mismatch is a failure (5), host copies without a swap pool are unsupported (4), an id
+    // outside its pool is out of range (3); pairs before a bad one have been copied.
     int copy(const PieCopyRequestDesc& c, uint32_t method) {
         if (c.srcs.len != c.dsts.len) return PIE_STATUS_FAILED;
         if (method >= PIE_METHOD_COPY_RS_D2H) return PIE_STATUS_UNSUPPORTED;  // no recurrent state
-        const uint32_t total = static_cast<uint32_t>(exec->total_pages());
+        const uint32_t dev = static_cast<uint32_t>(exec->total_pages());
+        const uint32_t host = static_cast<uint32_t>(exec->cpu_pages());
+        if (method != PIE_METHOD_COPY_KV_D2D && host == 0) return PIE_STATUS_UNSUPPORTED;
+        const uint32_t src_cap = (method == PIE_METHOD_COPY_KV_D2H || method == PIE_METHOD_COPY_KV_D2D) ? dev : host;
+        const uint32_t dst_cap = (method == PIE_METHOD_COPY_KV_H2D || method == PIE_METHOD_COPY_KV_D2D) ? dev : host;
+        size_t good = 0;
+        while (good < c.srcs.len && c.srcs.ptr[good] < src_cap && c.dsts.ptr[good] < dst_cap) ++good;
         switch (method) {
             case PIE_METHOD_COPY_KV_D2D:
-                for (size_t i = 0; i < c.srcs.len; ++i)
-                    if (c.srcs.ptr[i] >= total || c.dsts.ptr[i] >= total) return PIE_STATUS_OUT_OF_RANGE;
+                if (good != c.srcs.len) return PIE_STATUS_OUT_OF_RANGE;
                 exec->copy_pages_d2d(c.srcs.ptr, c.dsts.ptr, c.srcs.len);
                 return PIE_STATUS_OK;
-            default:
-                return PIE_STATUS_UNSUPPORTED;  // no host swap pool (cpu_pages = 0)
+            case PIE_METHOD_COPY_KV_D2H: exec->copy_pages_d2h(c.srcs.ptr, c.dsts.ptr, good); break;
+            case PIE_METHOD_COPY_KV_H2D: exec->copy_pages_h2d(c.srcs.ptr, c.dsts.ptr, good); break;
+            case PIE_METHOD_COPY_KV_H2H: exec->copy_pages_h2h(c.srcs.ptr, c.dsts.ptr, good); break;
+            default: return PIE_STATUS_UNSUPPORTED;
         }
+        return good == c.srcs.len ? PIE_STATUS_OK : PIE_STATUS_OUT_OF_RANGE;
     }
 
     void handle(const PieFrameDesc& frame, PieResponseFrameDesc& out) {

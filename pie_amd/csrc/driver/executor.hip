@@ -123,6 +123,12 @@ Executor::Executor(const DriverConfig& cfg, Model& model) : cfg_(cfg), model_(mo
     max_tokens_ = cfg.batching.max_forward_tokens;
     max_page_refs_ = 4 * total_pages_ + max_tokens_;
     alloc_kv();
+    cpu_pages_ = std::max(0, cfg.batching.cpu_pages);
+    if (cpu_pages_ > 0) {
+        const size_t bytes = static_cast<size_t>(model.cfg().layers) * 2 * cpu_pages_ * page_bytes();
+        PIE_HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&swap_pool_), bytes, hipHostMallocDefault));
+        std::memset(swap_pool_, 0, bytes);
+    }
 
     const ModelConfig& m = model.cfg();
     const size_t T = static_cast<size_t>(max_tokens_);
@@ -184,6 +190,7 @@ Executor::~Executor() {
     for (Growable* g : {&mask_in_host_, &mask_in_dev_, &mask_bitmap_}) g->release();
     for (Growable* g : {&samp_f32_, &samp_ws_, &samp_in_dev_, &samp_in_host_, &samp_out_dev_, &samp_out_host_})
         g->release();
+    if (swap_pool_) (void)hipHostFree(swap_pool_);
     if (in_host_) (void)hipHostFree(in_host_);
     if (out_host_) (void)hipHostFree(out_host_);
     if (stream_) (void)hipStreamDestroy(stream_);
@@ -617,6 +624,45 @@ void Executor::forward(const BatchPlan& plan, std::vector<uint32_t>& tokens_out,
     }
     const int cap = static_cast<int>(std::min<size_t>(max_tokens_, 2 * static_cast<size_t>(cfg_.batching.max_forward_requests)));
     last_logit_rows_ = S == 0 ? 0 : ((S - 1) % cap) + 1;
+}
+
+void Executor::copy_pages_d2h(const uint32_t* dev_srcs, const uint32_t* host_dsts, size_t n) {
+    const size_t pb = page_bytes();
+    for (size_t i = 0; i < n; ++i)
+        for (size_t l = 0; l < k_pool_.size(); ++l) {
+            const size_t off = static_cast<size_t>(dev_srcs[i]) * pb;
+            PIE_HIP_CHECK(hipMemcpyAsync(swap_slot(static_cast<int>(l), 0, host_dsts[i]),
+                                         reinterpret_cast<const unsigned char*>(k_pool_[l]) + off, pb,
+                                         hipMemcpyDeviceToHost, stream_));
+            PIE_HIP_CHECK(hipMemcpyAsync(swap_slot(static_cast<int>(l), 1, host_dsts[i]),
+                                         reinterpret_cast<const unsigned char*>(v_pool_[l]) + off, pb,
+                                         hipMemcpyDeviceToHost, stream_));
+        }
+    PIE_HIP_CHECK(hipStreamSynchronize(stream_));
+}
+
+void Executor::copy_pages_h2d(const uint32_t* host_srcs, const uint32_t* dev_dsts, size_t n) {
+    const size_t pb = page_bytes();
+    for (size_t i = 0; i < n; ++i)
+        for (size_t l = 0; l < k_pool_.size(); ++l) {
+            const size_t off = static_cast<size_t>(dev_dsts[i]) * pb;
+            PIE_HIP_CHECK(hipMemcpyAsync(reinterpret_cast<unsigned char*>(k_pool_[l]) + off,
+                                         swap_slot(static_cast<int>(l), 0, host_srcs[i]), pb,
+                                         hipMemcpyHostToDevice, stream_));
+            PIE_HIP_CHECK(hipMemcpyAsync(reinterpret_cast<unsigned char*>(v_pool_[l]) + off,
+                                         swap_slot(static_cast<int>(l), 1, host_srcs[i]), pb,
+                                         hipMemcpyHostToDevice, stream_));
+        }
+    PIE_HIP_CHECK(hipStreamSynchronize(stream_));
+}
+
+void Executor::copy_pages_h2h(const uint32_t* srcs, const uint32_t* dsts, size_t n) {
+    const size_t pb = page_bytes();
+    for (size_t i = 0; i < n; ++i)
+        for (size_t l = 0; l < k_pool_.size(); ++l)
+            for (int kv = 0; kv < 2; ++kv)
+                std::memmove(swap_slot(static_cast<int>(l), kv, dsts[i]),
+                             swap_slot(static_cast<int>(l), kv, srcs[i]), pb);
 }
 
 void Executor::copy_pages_d2d(const uint32_t* srcs, const uint32_t* dsts, size_t n) {

@@ -62,6 +62,13 @@ class Executor {
 
     // KV page copies inside the device pool (every layer, K and V).
     void copy_pages_d2d(const uint32_t* srcs, const uint32_t* dsts, size_t n);
+    // Host swap pool (`[batching] cpu_pages` pinned pages per layer for K and for V,
+    // driver/portable/src/host_swap_pool.cpp): device page -> host slot, back, host -> host.
+    // Callers check the ids against total_pages() / cpu_pages() first.
+    void copy_pages_d2h(const uint32_t* dev_srcs, const uint32_t* host_dsts, size_t n);
+    void copy_pages_h2d(const uint32_t* host_srcs, const uint32_t* dev_dsts, size_t n);
+    void copy_pages_h2h(const uint32_t* srcs, const uint32_t* dsts, size_t n);
+    int cpu_pages() const { return cpu_pages_; }
 
     int total_pages() const { return total_pages_; }
     int page_size() const { return page_size_; }
@@ -91,6 +98,11 @@ class Executor {
     int total_pages_ = 0, page_size_ = 0, max_tokens_ = 0, max_page_refs_ = 0;
 
     std::vector<uint16_t*> k_pool_, v_pool_;  // per layer [pages, ps, hk, d]
+    unsigned char* swap_pool_ = nullptr;       // pinned: [layer][K|V][cpu_pages] pages
+    int cpu_pages_ = 0;
+    unsigned char* swap_slot(int layer, int kv, uint32_t slot) const {
+        return swap_pool_ + ((static_cast<size_t>(layer) * 2 + kv) * cpu_pages_ + slot) * page_bytes();
+    }
     // activations
     uint16_t *x_ = nullptr, *xn_ = nullptr, *qkv_ = nullptr, *q_ = nullptr, *attn_ = nullptr;
     uint16_t *gu_ = nullptr, *act_ = nullptr, *xs_ = nullptr, *logits_ = nullptr;

@@ -310,3 +310,35 @@ def test_custom_attention_masks_match_oracle(gpu, oracle):
         # (last: this run overwrites the oracle's KV pool)
         _, plain, _ = om.forward(**args, want_logits=True)
         assert cosine(oracle.bf16_to_f32(plain[1]), oracle.bf16_to_f32(masked_row7)) < 0.999
+
+
+def test_host_swap_pool_round_trip(gpu, oracle):
+    """Copy D2H / H2H / H2D of KV pages through the pinned swap pool
+    (driver/portable/src/service/inproc_service.cpp:82-203): a context swapped out and back into
+    other device pages decodes bit-identically; status codes of the error cases."""
+    from pie_amd import driver as drvmod
+
+    cfg = full_cfg(cpu_pages=4)
+    ps, V = cfg["page_size"], cfg["vocab"]
+    rng = np.random.default_rng(95)
+    prompt = rng.integers(0, V, 27)          # pages 0 and 1
+    with drvmod.Driver(toml_config(cpu_pages=4)) as d:
+        assert d.capabilities()["swap_pool_size"] == 4
+        t0 = d.forward(drvmod.ForwardFrame(prompt, np.arange(27), [0, 1], [0, 2], [11], [0, 27])).tokens[0]
+        step = lambda pages: d.forward(drvmod.ForwardFrame([t0], [27], pages, [0, 2], [12], [0, 1]))
+        status = lambda fr: d.handle(fr).payload.status.status
+        assert status(drvmod.copy_frame(0, [0, 1], [2, 3])) == 0          # device 0,1 -> host 2,3
+        assert status(drvmod.copy_frame(3, [2, 3], [0, 1])) == 0          # host 2,3 -> host 0,1
+        assert status(drvmod.copy_frame(1, [0, 1], [5, 6])) == 0          # host 0,1 -> device 5,6
+        a = step([0, 1])
+        la = d.export_tensor("debug.logits", np.uint16)[:V].copy()
+        # undo the decode write on the copy's source... the copies were taken before it: decode on them
+        b = step([5, 6])
+        lb = d.export_tensor("debug.logits", np.uint16)[:V].copy()
+        assert a.tokens == b.tokens and np.array_equal(la, lb)
+        assert status(drvmod.copy_frame(0, [0], [4])) == 3                # host slot out of range
+        assert status(drvmod.copy_frame(1, [0], [9999])) == 3             # device page out of range
+        assert status(drvmod.copy_frame(3, [0, 1], [2])) == 5             # length mismatch
+    with drvmod.Driver(toml_config()) as d:                                # no pool
+        for direction in (0, 1, 3):
+            assert d.handle(drvmod.copy_frame(direction, [0], [0])).payload.status.status == 4
