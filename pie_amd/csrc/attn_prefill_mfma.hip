@@ -1,0 +1,302 @@
+// Prefill attention over paged KV on the matrix cores (gfx950, v_mfma_f32_16x16x32_bf16).
+//
+//   o[row, h, :] = softmax_j( q[row, h, :] . K[j, kvh, :] * scale ) . V[j, kvh, :],  j < row_kv_len[row]
+// for tiles of consecutive query rows that share one page list (the tokens of one prefill
+// chunk): same result contract as pie_hip_attn_rows_paged, i.e. the causal prefill branch of
+// the reference's paged kernel (driver/cuda/src/ops/attention_naive_paged.cu:148-317) and of
+// build_request_flash_attn (driver/portable/src/graph_common.cpp:347-396).
+//
+// One block (4 waves) = one tile x one kv head = 128 (token, q head) rows, 32 per wave as two
+// 16-row MFMA tiles.  Keys advance 32 at a time:
+//   S^T[key, query]  = K . Q^T     A = K fragment from LDS (row = key, k = d),  B = Q fragment kept
+//                                  in registers (col = query, k = d)
+//   O^T[d, query]   += V^T . P^T   A = V^T fragment from LDS (row = d, k = key), B = P in registers
+// Both products put the query on the lane%16 axis, so the online-softmax state (max, sum,
+// rescale) is per lane and the probabilities leave the first product already in the register
+// layout the second one consumes — with the 32 keys of a step in the order
+// [4g..4g+3, 16+4g..16+4g+3] per 16-lane group g, which is the order V^T is laid out in LDS.
+// K rows are padded to 272 B and V^T rows to 80 B: every 16-byte operand read of 16 lanes
+// touches 64 distinct banks.  The next step's K/V are requested from HBM before the current
+// step is multiplied.  Probabilities are rounded to bf16 for the second product (fp32
+// accumulators), and the normaliser sums those rounded values.
+#include "common.hip.h"
+
+namespace pie_hip {
+namespace {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+
+constexpr int kTileWaves = 4;
+constexpr int kTileThreads = kTileWaves * kWave;
+constexpr int kStepKeys = 32;
+constexpr int kBlockRows = 128;           // (token, head) rows per block
+constexpr int kVtStride = kStepKeys + 8;  // bf16 elements per V^T row (80 B)
+
+// slot of key kappa (0..31) inside a V^T row
+__device__ __forceinline__ int vt_slot(int kappa) {
+    return kappa < 16 ? 8 * (kappa >> 2) + (kappa & 3) : 8 * ((kappa - 16) >> 2) + 4 + (kappa & 3);
+}
+
+template <int D, int GQA>
+__global__ __launch_bounds__(kTileThreads) void attn_prefill_tile_kernel(
+    const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_pages,
+    const uint16_t* __restrict__ v_pages, uint16_t* __restrict__ o,
+    const uint32_t* __restrict__ page_indices, const uint32_t* __restrict__ row_begin,
+    const int32_t* __restrict__ row_len, const int32_t* __restrict__ tile_start,
+    const int32_t* __restrict__ tile_rows, int hq, int hk, int ps, float scale_log2e) {
+    constexpr int TQ = kBlockRows / GQA;   // query tokens per tile
+    constexpr int KS = D / 32;             // k steps of the first product
+    constexpr int DT = D / 16;             // d tiles of the second product
+    constexpr int LPR = D / 8;             // 16-byte pieces per K/V row
+    constexpr int KSTRIDE = D + 8;         // bf16 elements per K row in LDS
+    constexpr int PIECES = kStepKeys * LPR / kTileThreads;   // 16-byte pieces per thread per matrix
+    static_assert(PIECES >= 1 && (PIECES % 2 == 0 || PIECES == 1), "piece mapping");
+
+    __shared__ __attribute__((aligned(16))) uint16_t Ks[kStepKeys * KSTRIDE];
+    __shared__ __attribute__((aligned(16))) uint16_t Vt[D * kVtStride];
+    __shared__ int s_kmax;
+
+    const int tile = blockIdx.x, kvh = blockIdx.y;
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wv = tid / kWave;
+    const int l16 = lane & 15, g = lane >> 4;
+    const int s0 = tile_start[tile], n_rows = tile_rows[tile];
+    const uint32_t pg_lo = row_begin[s0];
+
+    if (tid == 0) s_kmax = 0;
+    __syncthreads();
+    if (tid < n_rows) atomicMax(&s_kmax, row_len[s0 + tid]);
+    __syncthreads();
+    const int kmax = s_kmax;
+
+    // this lane's two query rows (one per 16-row tile of the wave)
+    int my_len[2], my_row[2], my_head[2];
+    bf16x8_t qf[2][KS];
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt) {
+        const int m = wv * 32 + qt * 16 + l16;
+        const int h = m / TQ, t = m % TQ;
+        const bool valid = t < n_rows;
+        my_row[qt] = s0 + (valid ? t : 0);
+        my_head[qt] = kvh * GQA + h;
+        my_len[qt] = valid ? row_len[my_row[qt]] : 0;
+        const uint16_t* qp = q + (static_cast<size_t>(my_row[qt]) * hq + my_head[qt]) * D + 8 * g;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            u32x4_t v = *reinterpret_cast<const u32x4_t*>(qp + 32 * ks);
+            if (!valid) v = u32x4_t{0u, 0u, 0u, 0u};
+            qf[qt][ks] = __builtin_bit_cast(bf16x8_t, v);
+        }
+    }
+
+    // K/V staging: thread -> (key pair kp, 16-byte piece dc) so that two adjacent keys of one
+    // piece meet in one thread (their V values pack into 4-byte LDS writes)
+    constexpr int PAIRS = kStepKeys / 2;
+    u32x4_t kreg[PIECES], vreg[PIECES];
+    auto piece_of = [&](int u, int& key, int& dc) {
+        if (PIECES == 1) {   // D = 64: one piece per thread
+            key = tid % kStepKeys;
+            dc = tid / kStepKeys;
+            return;
+        }
+        // pieces of one thread: (pair, dc) pairs p = tid + kTileThreads * (u / 2); key = 2 * pair + (u & 1)
+        const int p = tid + kTileThreads * (u >> 1);
+        const int pair = p % PAIRS;
+        dc = p / PAIRS;
+        key = 2 * pair + (u & 1);
+    };
+    auto issue = [&](int j0) {
+#pragma unroll
+        for (int u = 0; u < PIECES; ++u) {
+            int key, dc;
+            piece_of(u, key, dc);
+            const int j = min(j0 + key, kmax - 1);
+            const uint32_t pid = page_indices[pg_lo + j / ps];
+            const size_t off = ((static_cast<size_t>(pid) * ps + j % ps) * hk + kvh) * D + dc * 8;
+            kreg[u] = *reinterpret_cast<const u32x4_t*>(k_pages + off);
+            vreg[u] = *reinterpret_cast<const u32x4_t*>(v_pages + off);
+        }
+    };
+    auto stage = [&]() {
+#pragma unroll
+        for (int u = 0; u < PIECES; ++u) {
+            int key, dc;
+            piece_of(u, key, dc);
+            *reinterpret_cast<u32x4_t*>(&Ks[key * KSTRIDE + dc * 8]) = kreg[u];
+        }
+#pragma unroll
+        for (int u = 0; u + 1 < PIECES || (PIECES == 1 && u == 0); u += 2) {
+            int key, dc;
+            piece_of(u, key, dc);
+            const int slot = vt_slot(key);
+            if constexpr (PIECES == 1) {
+                const uint32_t w[4] = {vreg[0].x, vreg[0].y, vreg[0].z, vreg[0].w};
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    Vt[(dc * 8 + e) * kVtStride + slot] = static_cast<uint16_t>(w[e >> 1] >> (16 * (e & 1)));
+            } else {
+                const uint32_t a[4] = {vreg[u].x, vreg[u].y, vreg[u].z, vreg[u].w};
+                const uint32_t b[4] = {vreg[u + 1].x, vreg[u + 1].y, vreg[u + 1].z, vreg[u + 1].w};
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const uint32_t lo = (a[e >> 1] >> (16 * (e & 1))) & 0xFFFFu;
+                    const uint32_t hi = (b[e >> 1] >> (16 * (e & 1))) & 0xFFFFu;
+                    *reinterpret_cast<uint32_t*>(&Vt[(dc * 8 + e) * kVtStride + slot]) = lo | (hi << 16);
+                }
+            }
+        }
+    };
+
+    f32x4_t acc[2][DT];
+    float mx[2], lsum[2];
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt) {
+        mx[qt] = -INFINITY;
+        lsum[qt] = 0.f;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) acc[qt][dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    }
+
+    if (kmax > 0) issue(0);
+    for (int j0 = 0; j0 < kmax; j0 += kStepKeys) {
+        __syncthreads();   // the previous step's LDS reads are done
+        stage();
+        __syncthreads();
+        if (j0 + kStepKeys < kmax) issue(j0 + kStepKeys);
+
+        // S^T = K . Q^T for both query tiles
+        f32x4_t st[2][2];
+#pragma unroll
+        for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+            for (int nt = 0; nt < 2; ++nt) st[qt][nt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+            for (int nt = 0; nt < 2; ++nt) {
+                const bf16x8_t kf = __builtin_bit_cast(
+                    bf16x8_t, *reinterpret_cast<const u32x4_t*>(&Ks[(16 * nt + l16) * KSTRIDE + 32 * ks + 8 * g]));
+#pragma unroll
+                for (int qt = 0; qt < 2; ++qt)
+                    st[qt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[qt][ks], st[qt][nt], 0, 0, 0);
+            }
+        }
+        // online softmax per query (= per lane%16); the 8 keys of this lane: 16nt + 4g + r
+        bf16x8_t pf[2];
+#pragma unroll
+        for (int qt = 0; qt < 2; ++qt) {
+            float s[8];
+            float m_new = mx[qt];
+#pragma unroll
+            for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int key = j0 + 16 * nt + 4 * g + r;
+                    const float v = key < my_len[qt] ? st[qt][nt][r] * scale_log2e : -INFINITY;
+                    s[4 * nt + r] = v;
+                    m_new = fmaxf(m_new, v);
+                }
+            m_new = fmaxf(m_new, __shfl_xor(m_new, 16, kWave));
+            m_new = fmaxf(m_new, __shfl_xor(m_new, 32, kWave));
+            const float safe = m_new == -INFINITY ? 0.f : m_new;
+            const float alpha = exp2f(mx[qt] - safe);
+            mx[qt] = m_new;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) s[e] = exp2f(s[e] - safe);
+            const u32x4_t packed = {pack_bf16x2(s[0], s[1]), pack_bf16x2(s[2], s[3]),
+                                    pack_bf16x2(s[4], s[5]), pack_bf16x2(s[6], s[7])};
+            pf[qt] = __builtin_bit_cast(bf16x8_t, packed);
+            // the normaliser sums the rounded weights, the ones that multiply V: the output stays
+            // an exact weighted mean of V rows
+            float sum = 0.f;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) sum += bf16_lo(packed[e]) + bf16_hi(packed[e]);
+            lsum[qt] = lsum[qt] * alpha + sum;
+            if (alpha != 1.0f) {
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) acc[qt][dt] *= alpha;
+            }
+        }
+        // O^T += V^T . P^T
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            const bf16x8_t vf = __builtin_bit_cast(
+                bf16x8_t, *reinterpret_cast<const u32x4_t*>(&Vt[(16 * dt + l16) * kVtStride + 8 * g]));
+#pragma unroll
+            for (int qt = 0; qt < 2; ++qt)
+                acc[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[qt], acc[qt][dt], 0, 0, 0);
+        }
+    }
+
+    // normalise and store: this lane holds, for its query, d = 16 dt + 4 g + r
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt) {
+        float l = lsum[qt];
+        l += __shfl_xor(l, 16, kWave);
+        l += __shfl_xor(l, 32, kWave);
+        const int m = wv * 32 + qt * 16 + l16;
+        if (m % TQ >= n_rows) continue;
+        const float inv = l > 0.f ? 1.0f / l : 0.f;
+        uint16_t* op = o + (static_cast<size_t>(my_row[qt]) * hq + my_head[qt]) * D + 4 * g;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            const f32x4_t a = acc[qt][dt];
+            const u32x2_t w = {pack_bf16x2(a[0] * inv, a[1] * inv), pack_bf16x2(a[2] * inv, a[3] * inv)};
+            *reinterpret_cast<u32x2_t*>(op + 16 * dt) = w;
+        }
+    }
+}
+
+template <int D, int GQA>
+int launch_tiles(const uint16_t* q, const uint16_t* k_pages, const uint16_t* v_pages, uint16_t* o,
+                 const uint32_t* page_indices, const uint32_t* row_begin, const int32_t* row_len,
+                 const int32_t* tile_start, const int32_t* tile_rows, int num_tiles, int hq, int hk,
+                 int ps, float scale, hipStream_t stream) {
+    hipLaunchKernelGGL((attn_prefill_tile_kernel<D, GQA>), dim3(num_tiles, hk), dim3(kTileThreads), 0,
+                       stream, q, k_pages, v_pages, o, page_indices, row_begin, row_len, tile_start,
+                       tile_rows, hq, hk, ps, scale * 1.4426950408889634f);
+    return launch_status();
+}
+
+}  // namespace
+}  // namespace pie_hip
+
+extern "C" int pie_hip_attn_prefill_tile_rows(int num_q_heads, int num_kv_heads) {
+    if (num_q_heads <= 0 || num_kv_heads <= 0 || num_q_heads % num_kv_heads != 0) return 0;
+    const int gqa = num_q_heads / num_kv_heads;
+    if (gqa != 1 && gqa != 2 && gqa != 4 && gqa != 8) return 0;
+    return pie_hip::kBlockRows / gqa;
+}
+
+extern "C" int pie_hip_attn_prefill_tiles(const uint16_t* q, const uint16_t* k_pages,
+                                          const uint16_t* v_pages, uint16_t* o,
+                                          const uint32_t* kv_page_indices,
+                                          const uint32_t* row_page_begin, const int32_t* row_kv_len,
+                                          const int32_t* tile_row_start, const int32_t* tile_num_rows,
+                                          int num_tiles, int num_q_heads, int num_kv_heads,
+                                          int head_dim, int page_size, float sm_scale, void* stream) {
+    using namespace pie_hip;
+    if (!q || !k_pages || !v_pages || !o || !kv_page_indices || !row_page_begin || !row_kv_len ||
+        !tile_row_start || !tile_num_rows || num_tiles <= 0 || page_size <= 0)
+        return PIE_HIP_ERR_INVALID;
+    if (pie_hip_attn_prefill_tile_rows(num_q_heads, num_kv_heads) == 0 || page_size % 2 != 0 ||
+        num_tiles > 0x7FFFFFFF / 2 || num_kv_heads > 65535)
+        return PIE_HIP_ERR_UNSUPPORTED;
+    const float scale = sm_scale > 0.f ? sm_scale : 1.0f / sqrtf(static_cast<float>(head_dim));
+    const int gqa = num_q_heads / num_kv_heads;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+#define PIE_TILE_CASE(DD, GG)                                                                       \
+    if (head_dim == DD && gqa == GG)                                                                \
+        return launch_tiles<DD, GG>(q, k_pages, v_pages, o, kv_page_indices, row_page_begin,        \
+                                    row_kv_len, tile_row_start, tile_num_rows, num_tiles,           \
+                                    num_q_heads, num_kv_heads, page_size, scale, st);
+    PIE_TILE_CASE(128, 1)
+    PIE_TILE_CASE(128, 2)
+    PIE_TILE_CASE(128, 4)
+    PIE_TILE_CASE(128, 8)
+    PIE_TILE_CASE(64, 1)
+    PIE_TILE_CASE(64, 2)
+    PIE_TILE_CASE(64, 4)
+    PIE_TILE_CASE(64, 8)
+#undef PIE_TILE_CASE
+    return PIE_HIP_ERR_UNSUPPORTED;
+}

@@ -644,3 +644,30 @@ def attention_rows_paged(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
                                           _stream())
     _check(st, "pie_hip_attn_rows_paged_masked")
     return o
+
+
+def attn_prefill_tile_rows(hq: int, hk: int) -> int:
+    """Most query rows one tile of `attention_prefill_tiles` may hold (0: unsupported head ratio)."""
+    return int(kernels().pie_hip_attn_prefill_tile_rows(hq, hk))
+
+
+def attention_prefill_tiles(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
+                            kv_page_indices: torch.Tensor, row_page_begin: torch.Tensor,
+                            row_kv_len: torch.Tensor, tile_row_start: torch.Tensor,
+                            tile_num_rows: torch.Tensor) -> torch.Tensor:
+    """Matrix-core prefill attention over tiles of consecutive rows that share a page list."""
+    _dev(q, torch.bfloat16, "q")
+    _dev(k_pages, torch.bfloat16, "k_pages")
+    for name, t in (("kv_page_indices", kv_page_indices), ("row_page_begin", row_page_begin),
+                    ("row_kv_len", row_kv_len), ("tile_row_start", tile_row_start),
+                    ("tile_num_rows", tile_num_rows)):
+        _dev(t, torch.int32, name)
+    rows, hq, d = q.shape
+    _, ps, hk, _ = k_pages.shape
+    o = torch.zeros_like(q)
+    st = kernels().pie_hip_attn_prefill_tiles(_ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(o),
+                                              _ptr(kv_page_indices), _ptr(row_page_begin),
+                                              _ptr(row_kv_len), _ptr(tile_row_start), _ptr(tile_num_rows),
+                                              tile_row_start.numel(), hq, hk, d, ps, C.c_float(-1.0), _stream())
+    _check(st, "pie_hip_attn_prefill_tiles")
+    return o
