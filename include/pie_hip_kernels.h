@@ -199,10 +199,11 @@ int pie_hip_moe_combine(const uint16_t* y_routes_bf16, const int32_t* route_pos,
  * Prefill attention on the matrix cores: the result contract of pie_hip_attn_rows_paged for
  * query rows grouped into tiles.  Tile i covers rows tile_row_start[i] .. + tile_num_rows[i]
  * (consecutive rows that share one page list, i.e. row_page_begin is equal across the tile;
- * at most pie_hip_attn_prefill_tile_rows(hq, hk) = 128 / (hq/hk) rows); each row still sees
- * its own first row_kv_len[row] keys.  Probabilities are rounded to bf16 before they multiply V
+ * at most rows_per_tile rows, which is pie_hip_attn_prefill_tile_rows(hq, hk) = 128 / (hq/hk)
+ * or half of it — the smaller tile doubles the number of blocks for small batches); each row
+ * still sees its own first row_kv_len[row] keys.  Probabilities are rounded to bf16 before they multiply V
  * (fp32 softmax sums and accumulators), so results agree with the per-row kernel to about one
- * bf16 step rather than bit for bit.  d in {64,128}, hq/hk in {1,2,4,8}, page_size even.
+ * bf16 step rather than bit for bit.  d in {64,128}, hq/hk in {1,2,4,8}, page_size % 16 == 0.
  * Reference: the causal prefill branch of launch_attention_naive_paged_prefill,
  * driver/cuda/src/ops/attention_naive_paged.cu:148-317; per-request flash attention of the
  * portable driver, driver/portable/src/graph_common.cpp:347-396.
@@ -212,8 +213,8 @@ int pie_hip_attn_prefill_tiles(const uint16_t* q, const uint16_t* k_pages, const
                                uint16_t* o, const uint32_t* kv_page_indices,
                                const uint32_t* row_page_begin, const int32_t* row_kv_len,
                                const int32_t* tile_row_start, const int32_t* tile_num_rows,
-                               int num_tiles, int num_q_heads, int num_kv_heads, int head_dim,
-                               int page_size, float sm_scale, void* stream);
+                               int num_tiles, int rows_per_tile, int num_q_heads, int num_kv_heads,
+                               int head_dim, int page_size, float sm_scale, void* stream);
 
 /*
  * Custom attention masks for the per-row form.  pie_hip_attn_mask_bitmap turns per-row BRLE

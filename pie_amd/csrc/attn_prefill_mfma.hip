@@ -37,14 +37,16 @@ __device__ __forceinline__ int vt_slot(int kappa) {
     return kappa < 16 ? 8 * (kappa >> 2) + (kappa & 3) : 8 * ((kappa - 16) >> 2) + 4 + (kappa & 3);
 }
 
-template <int D, int GQA>
+// QT: 16-row MFMA tiles per wave (2: 128 rows per block, K/V fragments read once per two tiles;
+// 1: 64 rows per block, twice the blocks for small batches).
+template <int D, int GQA, int QT>
 __global__ __launch_bounds__(kTileThreads) void attn_prefill_tile_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_pages,
     const uint16_t* __restrict__ v_pages, uint16_t* __restrict__ o,
     const uint32_t* __restrict__ page_indices, const uint32_t* __restrict__ row_begin,
     const int32_t* __restrict__ row_len, const int32_t* __restrict__ tile_start,
     const int32_t* __restrict__ tile_rows, int hq, int hk, int ps, float scale_log2e) {
-    constexpr int TQ = kBlockRows / GQA;   // query tokens per tile
+    constexpr int TQ = 32 * QT * kTileWaves / (2 * GQA);   // query tokens per tile: 64 QT / GQA
     constexpr int KS = D / 32;             // k steps of the first product
     constexpr int DT = D / 16;             // d tiles of the second product
     constexpr int LPR = D / 8;             // 16-byte pieces per K/V row
@@ -69,11 +71,11 @@ __global__ __launch_bounds__(kTileThreads) void attn_prefill_tile_kernel(
     const int kmax = s_kmax;
 
     // this lane's two query rows (one per 16-row tile of the wave)
-    int my_len[2], my_row[2], my_head[2];
-    bf16x8_t qf[2][KS];
+    int my_len[QT], my_row[QT], my_head[QT];
+    bf16x8_t qf[QT][KS];
 #pragma unroll
-    for (int qt = 0; qt < 2; ++qt) {
-        const int m = wv * 32 + qt * 16 + l16;
+    for (int qt = 0; qt < QT; ++qt) {
+        const int m = wv * 16 * QT + qt * 16 + l16;
         const int h = m / TQ, t = m % TQ;
         const bool valid = t < n_rows;
         my_row[qt] = s0 + (valid ? t : 0);
@@ -91,7 +93,8 @@ __global__ __launch_bounds__(kTileThreads) void attn_prefill_tile_kernel(
     // K/V staging: thread -> (key pair kp, 16-byte piece dc) so that two adjacent keys of one
     // piece meet in one thread (their V values pack into 4-byte LDS writes)
     constexpr int PAIRS = kStepKeys / 2;
-    u32x4_t kreg[PIECES], vreg[PIECES];
+    constexpr int PF = 2;   // steps of K/V in flight
+    u32x4_t kreg[PF][PIECES], vreg[PF][PIECES];
     auto piece_of = [&](int u, int& key, int& dc) {
         if (PIECES == 1) {   // D = 64: one piece per thread
             key = tid % kStepKeys;
@@ -104,69 +107,75 @@ __global__ __launch_bounds__(kTileThreads) void attn_prefill_tile_kernel(
         dc = p / PAIRS;
         key = 2 * pair + (u & 1);
     };
-    auto issue = [&](int j0) {
+    // a 32-key step touches at most two pages (page_size % 16 == 0): their ids come through
+    // scalar loads, so the vector-memory queue holds K/V loads only, in step order
+    auto issue = [&](int slot, int j0) {
+        const int ja = min(j0, kmax - 1), jb = min(j0 + kStepKeys - 1, kmax - 1);
+        const int page_a = ja / ps;
+        const uint32_t pid_a = __builtin_amdgcn_readfirstlane(page_indices[pg_lo + page_a]);
+        const uint32_t pid_b = __builtin_amdgcn_readfirstlane(page_indices[pg_lo + jb / ps]);
 #pragma unroll
         for (int u = 0; u < PIECES; ++u) {
             int key, dc;
             piece_of(u, key, dc);
             const int j = min(j0 + key, kmax - 1);
-            const uint32_t pid = page_indices[pg_lo + j / ps];
-            const size_t off = ((static_cast<size_t>(pid) * ps + j % ps) * hk + kvh) * D + dc * 8;
-            kreg[u] = *reinterpret_cast<const u32x4_t*>(k_pages + off);
-            vreg[u] = *reinterpret_cast<const u32x4_t*>(v_pages + off);
+            const int page = j / ps;
+            const uint32_t pid = page == page_a ? pid_a : pid_b;
+            const size_t off = ((static_cast<size_t>(pid) * ps + (j - page * ps)) * hk + kvh) * D + dc * 8;
+            kreg[slot][u] = *reinterpret_cast<const u32x4_t*>(k_pages + off);
+            vreg[slot][u] = *reinterpret_cast<const u32x4_t*>(v_pages + off);
         }
     };
-    auto stage = [&]() {
+    auto stage = [&](int slot) {
 #pragma unroll
         for (int u = 0; u < PIECES; ++u) {
             int key, dc;
             piece_of(u, key, dc);
-            *reinterpret_cast<u32x4_t*>(&Ks[key * KSTRIDE + dc * 8]) = kreg[u];
+            *reinterpret_cast<u32x4_t*>(&Ks[key * KSTRIDE + dc * 8]) = kreg[slot][u];
         }
 #pragma unroll
         for (int u = 0; u + 1 < PIECES || (PIECES == 1 && u == 0); u += 2) {
             int key, dc;
             piece_of(u, key, dc);
-            const int slot = vt_slot(key);
+            const int col = vt_slot(key);
             if constexpr (PIECES == 1) {
-                const uint32_t w[4] = {vreg[0].x, vreg[0].y, vreg[0].z, vreg[0].w};
+                const uint32_t w[4] = {vreg[slot][0].x, vreg[slot][0].y, vreg[slot][0].z, vreg[slot][0].w};
 #pragma unroll
                 for (int e = 0; e < 8; ++e)
-                    Vt[(dc * 8 + e) * kVtStride + slot] = static_cast<uint16_t>(w[e >> 1] >> (16 * (e & 1)));
+                    Vt[(dc * 8 + e) * kVtStride + col] = static_cast<uint16_t>(w[e >> 1] >> (16 * (e & 1)));
             } else {
-                const uint32_t a[4] = {vreg[u].x, vreg[u].y, vreg[u].z, vreg[u].w};
-                const uint32_t b[4] = {vreg[u + 1].x, vreg[u + 1].y, vreg[u + 1].z, vreg[u + 1].w};
+                const uint32_t a[4] = {vreg[slot][u].x, vreg[slot][u].y, vreg[slot][u].z, vreg[slot][u].w};
+                const uint32_t b[4] = {vreg[slot][u + 1].x, vreg[slot][u + 1].y, vreg[slot][u + 1].z, vreg[slot][u + 1].w};
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
                     const uint32_t lo = (a[e >> 1] >> (16 * (e & 1))) & 0xFFFFu;
                     const uint32_t hi = (b[e >> 1] >> (16 * (e & 1))) & 0xFFFFu;
-                    *reinterpret_cast<uint32_t*>(&Vt[(dc * 8 + e) * kVtStride + slot]) = lo | (hi << 16);
+                    *reinterpret_cast<uint32_t*>(&Vt[(dc * 8 + e) * kVtStride + col]) = lo | (hi << 16);
                 }
             }
         }
     };
 
-    f32x4_t acc[2][DT];
-    float mx[2], lsum[2];
+    f32x4_t acc[QT][DT];
+    float mx[QT], lsum[QT];
 #pragma unroll
-    for (int qt = 0; qt < 2; ++qt) {
+    for (int qt = 0; qt < QT; ++qt) {
         mx[qt] = -INFINITY;
         lsum[qt] = 0.f;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) acc[qt][dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     }
 
-    if (kmax > 0) issue(0);
-    for (int j0 = 0; j0 < kmax; j0 += kStepKeys) {
+    auto step = [&](int slot, int j0) {
         __syncthreads();   // the previous step's LDS reads are done
-        stage();
+        stage(slot);
         __syncthreads();
-        if (j0 + kStepKeys < kmax) issue(j0 + kStepKeys);
+        if (j0 + PF * kStepKeys < kmax) issue(slot, j0 + PF * kStepKeys);
 
         // S^T = K . Q^T for both query tiles
-        f32x4_t st[2][2];
+        f32x4_t st[QT][2];
 #pragma unroll
-        for (int qt = 0; qt < 2; ++qt)
+        for (int qt = 0; qt < QT; ++qt)
 #pragma unroll
             for (int nt = 0; nt < 2; ++nt) st[qt][nt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -176,14 +185,14 @@ __global__ __launch_bounds__(kTileThreads) void attn_prefill_tile_kernel(
                 const bf16x8_t kf = __builtin_bit_cast(
                     bf16x8_t, *reinterpret_cast<const u32x4_t*>(&Ks[(16 * nt + l16) * KSTRIDE + 32 * ks + 8 * g]));
 #pragma unroll
-                for (int qt = 0; qt < 2; ++qt)
+                for (int qt = 0; qt < QT; ++qt)
                     st[qt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[qt][ks], st[qt][nt], 0, 0, 0);
             }
         }
         // online softmax per query (= per lane%16); the 8 keys of this lane: 16nt + 4g + r
-        bf16x8_t pf[2];
+        bf16x8_t pf[QT];
 #pragma unroll
-        for (int qt = 0; qt < 2; ++qt) {
+        for (int qt = 0; qt < QT; ++qt) {
             float s[8];
             float m_new = mx[qt];
 #pragma unroll
@@ -222,18 +231,25 @@ __global__ __launch_bounds__(kTileThreads) void attn_prefill_tile_kernel(
             const bf16x8_t vf = __builtin_bit_cast(
                 bf16x8_t, *reinterpret_cast<const u32x4_t*>(&Vt[(16 * dt + l16) * kVtStride + 8 * g]));
 #pragma unroll
-            for (int qt = 0; qt < 2; ++qt)
+            for (int qt = 0; qt < QT; ++qt)
                 acc[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[qt], acc[qt][dt], 0, 0, 0);
         }
+    };
+
+    if (kmax > 0) issue(0, 0);
+    if (kmax > kStepKeys) issue(1, kStepKeys);
+    for (int j0 = 0; j0 < kmax; j0 += PF * kStepKeys) {   // unrolled by PF: compile-time register slots
+        step(0, j0);
+        if (j0 + kStepKeys < kmax) step(1, j0 + kStepKeys);
     }
 
     // normalise and store: this lane holds, for its query, d = 16 dt + 4 g + r
 #pragma unroll
-    for (int qt = 0; qt < 2; ++qt) {
+    for (int qt = 0; qt < QT; ++qt) {
         float l = lsum[qt];
         l += __shfl_xor(l, 16, kWave);
         l += __shfl_xor(l, 32, kWave);
-        const int m = wv * 32 + qt * 16 + l16;
+        const int m = wv * 16 * QT + qt * 16 + l16;
         if (m % TQ >= n_rows) continue;
         const float inv = l > 0.f ? 1.0f / l : 0.f;
         uint16_t* op = o + (static_cast<size_t>(my_row[qt]) * hq + my_head[qt]) * D + 4 * g;
@@ -246,12 +262,12 @@ __global__ __launch_bounds__(kTileThreads) void attn_prefill_tile_kernel(
     }
 }
 
-template <int D, int GQA>
+template <int D, int GQA, int QT>
 int launch_tiles(const uint16_t* q, const uint16_t* k_pages, const uint16_t* v_pages, uint16_t* o,
                  const uint32_t* page_indices, const uint32_t* row_begin, const int32_t* row_len,
                  const int32_t* tile_start, const int32_t* tile_rows, int num_tiles, int hq, int hk,
                  int ps, float scale, hipStream_t stream) {
-    hipLaunchKernelGGL((attn_prefill_tile_kernel<D, GQA>), dim3(num_tiles, hk), dim3(kTileThreads), 0,
+    hipLaunchKernelGGL((attn_prefill_tile_kernel<D, GQA, QT>), dim3(num_tiles, hk), dim3(kTileThreads), 0,
                        stream, q, k_pages, v_pages, o, page_indices, row_begin, row_len, tile_start,
                        tile_rows, hq, hk, ps, scale * 1.4426950408889634f);
     return launch_status();
@@ -272,23 +288,31 @@ extern "C" int pie_hip_attn_prefill_tiles(const uint16_t* q, const uint16_t* k_p
                                           const uint32_t* kv_page_indices,
                                           const uint32_t* row_page_begin, const int32_t* row_kv_len,
                                           const int32_t* tile_row_start, const int32_t* tile_num_rows,
-                                          int num_tiles, int num_q_heads, int num_kv_heads,
-                                          int head_dim, int page_size, float sm_scale, void* stream) {
+                                          int num_tiles, int rows_per_tile, int num_q_heads,
+                                          int num_kv_heads, int head_dim, int page_size,
+                                          float sm_scale, void* stream) {
     using namespace pie_hip;
     if (!q || !k_pages || !v_pages || !o || !kv_page_indices || !row_page_begin || !row_kv_len ||
         !tile_row_start || !tile_num_rows || num_tiles <= 0 || page_size <= 0)
         return PIE_HIP_ERR_INVALID;
-    if (pie_hip_attn_prefill_tile_rows(num_q_heads, num_kv_heads) == 0 || page_size % 2 != 0 ||
-        num_tiles > 0x7FFFFFFF / 2 || num_kv_heads > 65535)
+    const int cap = pie_hip_attn_prefill_tile_rows(num_q_heads, num_kv_heads);
+    if (cap == 0 || page_size % 16 != 0 || num_tiles > 0x7FFFFFFF / 2 || num_kv_heads > 65535)
         return PIE_HIP_ERR_UNSUPPORTED;
+    if (rows_per_tile != cap && rows_per_tile * 2 != cap) return PIE_HIP_ERR_UNSUPPORTED;
+    const bool big = rows_per_tile == cap;
     const float scale = sm_scale > 0.f ? sm_scale : 1.0f / sqrtf(static_cast<float>(head_dim));
     const int gqa = num_q_heads / num_kv_heads;
     hipStream_t st = static_cast<hipStream_t>(stream);
 #define PIE_TILE_CASE(DD, GG)                                                                       \
     if (head_dim == DD && gqa == GG)                                                                \
-        return launch_tiles<DD, GG>(q, k_pages, v_pages, o, kv_page_indices, row_page_begin,        \
-                                    row_kv_len, tile_row_start, tile_num_rows, num_tiles,           \
-                                    num_q_heads, num_kv_heads, page_size, scale, st);
+        return big ? launch_tiles<DD, GG, 2>(q, k_pages, v_pages, o, kv_page_indices,               \
+                                             row_page_begin, row_kv_len, tile_row_start,            \
+                                             tile_num_rows, num_tiles, num_q_heads, num_kv_heads,   \
+                                             page_size, scale, st)                                  \
+                   : launch_tiles<DD, GG, 1>(q, k_pages, v_pages, o, kv_page_indices,               \
+                                             row_page_begin, row_kv_len, tile_row_start,            \
+                                             tile_num_rows, num_tiles, num_q_heads, num_kv_heads,   \
+                                             page_size, scale, st);
     PIE_TILE_CASE(128, 1)
     PIE_TILE_CASE(128, 2)
     PIE_TILE_CASE(128, 4)

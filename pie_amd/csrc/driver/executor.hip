@@ -187,7 +187,7 @@ Executor::~Executor() {
                     static_cast<void*>(moe_offsets_), static_cast<void*>(moe_route_token_),
                     static_cast<void*>(moe_route_pos_)})
         if (p) (void)hipFree(p);
-    for (Growable* g : {&mask_in_host_, &mask_in_dev_, &mask_bitmap_}) g->release();
+    for (Growable* g : {&mask_in_host_, &mask_in_dev_, &mask_bitmap_, &tile_in_host_, &tile_in_dev_}) g->release();
     for (Growable* g : {&samp_f32_, &samp_ws_, &samp_in_dev_, &samp_in_host_, &samp_out_dev_, &samp_out_host_})
         g->release();
     if (swap_pool_) (void)hipHostFree(swap_pool_);
@@ -287,7 +287,12 @@ void Executor::body(int N, int S, int max_kv_len) {
                                                 rope_tab_, slots, N, hq, hk, d, m.rope_interleaved,
                                                 m.rms_eps, s));
         }
-        if (masked_) {
+        if (n_tiles_ > 0) {
+            const auto* td = static_cast<const int32_t*>(tile_in_dev_.ptr);
+            PIE_KERNEL(pie_hip_attn_prefill_tiles(q_, k_pool_[l], v_pool_[l], attn_, pages, row_begin,
+                                                  row_len, td, td + n_tiles_, n_tiles_, tile_rows_, hq,
+                                                  hk, d, page_size_, -1.f, s));
+        } else if (masked_) {
             PIE_KERNEL(pie_hip_attn_rows_paged_masked(
                 q_, k_pool_[l], v_pool_[l], attn_, nullptr, pages, row_begin, row_len,
                 static_cast<const uint16_t*>(mask_bitmap_.ptr), mask_stride_, N, hq, hk, d, page_size_,
@@ -362,6 +367,40 @@ float pcg32_first_uniform(uint64_t seed) {
 }
 
 }  // namespace
+
+// Prefill-shaped batches (every request brings at least 8 query rows, no custom masks) run
+// their attention on the matrix cores: rows are cut into tiles of consecutive rows of one
+// request.  Batches with single-row requests keep the per-row kernel, whose split-K spreads a
+// long context over the machine.
+void Executor::prepare_tiles(const BatchPlan& plan) {
+    n_tiles_ = 0;
+    const ModelConfig& m = model_.cfg();
+    int cap = pie_hip_attn_prefill_tile_rows(m.q_heads, m.kv_heads);
+    if (cap <= 0 || plan.has_user_masks || page_size_ % 16 != 0 || (m.head_dim != 64 && m.head_dim != 128)) return;
+    long long blocks = 0;
+    for (int r = 0; r < plan.R; ++r) {
+        const int n = plan.qo_indptr[r + 1] - plan.qo_indptr[r];
+        if (n < 8) return;
+        blocks += static_cast<long long>((n + cap - 1) / cap) * m.kv_heads;
+    }
+    if (blocks < 512) cap /= 2;   // fewer than two full-size blocks per CU: halve the tiles
+    tile_rows_ = cap;
+    std::vector<int32_t> start, rows;
+    for (int r = 0; r < plan.R; ++r)
+        for (int t0 = plan.qo_indptr[r]; t0 < plan.qo_indptr[r + 1]; t0 += cap) {
+            start.push_back(t0);
+            rows.push_back(std::min(cap, plan.qo_indptr[r + 1] - t0));
+        }
+    const size_t n = start.size(), bytes = 8 * n;
+    tile_in_host_.pinned = true;
+    tile_in_host_.ensure(bytes);
+    tile_in_dev_.ensure(bytes);
+    auto* h = static_cast<int32_t*>(tile_in_host_.ptr);
+    std::memcpy(h, start.data(), 4 * n);
+    std::memcpy(h + n, rows.data(), 4 * n);
+    PIE_HIP_CHECK(hipMemcpyAsync(tile_in_dev_.ptr, h, bytes, hipMemcpyHostToDevice, stream_));
+    n_tiles_ = static_cast<int>(n);
+}
 
 // Custom attention masks: each row's BRLE runs become cumulative bounds, the device expands
 // them into one visibility word per 16-token unit, and the layers' attention reads that.
@@ -572,6 +611,7 @@ void Executor::forward(const BatchPlan& plan, std::vector<uint32_t>& tokens_out,
     PIE_HIP_CHECK(hipMemcpyAsync(in_dev_, in_host_, used, hipMemcpyHostToDevice, stream_));
     masked_ = plan.has_user_masks;
     if (masked_) prepare_masks(plan);
+    prepare_tiles(plan);
     const bool sampling = !plan.all_greedy && S > 0;
     const int chunk = static_cast<int>(std::min<size_t>(max_tokens_, 2 * static_cast<size_t>(cfg_.batching.max_forward_requests)));
     samp_gather_in_body_ = false;

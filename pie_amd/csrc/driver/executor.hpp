@@ -86,6 +86,7 @@ class Executor {
   private:
     void body(int N, int S, int max_kv_len);
     void prepare_masks(const BatchPlan& plan);
+    void prepare_tiles(const BatchPlan& plan);
     void prepare_samplers(const BatchPlan& plan);
     void enqueue_samplers();
     void collect_samplers(const BatchPlan& plan, SampleOutputs& out);
@@ -138,6 +139,9 @@ class Executor {
         void ensure(size_t bytes);
         void release();
     };
+    // query-row tiles of the current forward for the matrix-core prefill attention (0 = per-row kernel)
+    Growable tile_in_host_, tile_in_dev_;
+    int n_tiles_ = 0, tile_rows_ = 0;
     // custom attention masks of the current forward (never part of a captured graph)
     Growable mask_in_host_, mask_in_dev_, mask_bitmap_;
     int mask_stride_ = 0;

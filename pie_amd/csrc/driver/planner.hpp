@@ -45,6 +45,7 @@ struct BatchPlan {
     std::vector<uint32_t> row_page_begin;  // [N] first entry of the row's page list
     std::vector<int32_t> row_kv_len;       // [N] keys visible to the row: min(seq_len, pos+1)
     std::vector<int32_t> seq_len;          // [R]
+    std::vector<int32_t> qo_indptr;        // [R+1] token rows of each request
     std::vector<uint32_t> page_indices;    // copy of the wire list (uploaded as is)
     std::vector<int32_t> sample_rows;      // global token rows to sample, request-major
     std::vector<int32_t> sample_indptr;    // [R+1]
@@ -142,6 +143,7 @@ inline BatchPlan plan_forward(const PieForwardRequestDesc& f, int page_size, int
     p.row_page_begin.resize(N);
     p.row_kv_len.resize(N);
     p.seq_len.resize(R);
+    p.qo_indptr.assign(f.qo_indptr.ptr, f.qo_indptr.ptr + R + 1);
     p.page_indices.assign(f.kv_page_indices.ptr, f.kv_page_indices.ptr + f.kv_page_indices.len);
     p.sample_indptr.assign(1, 0);
     p.logit_mask_runs.resize(R);

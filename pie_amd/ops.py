@@ -654,8 +654,9 @@ def attn_prefill_tile_rows(hq: int, hk: int) -> int:
 def attention_prefill_tiles(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                             kv_page_indices: torch.Tensor, row_page_begin: torch.Tensor,
                             row_kv_len: torch.Tensor, tile_row_start: torch.Tensor,
-                            tile_num_rows: torch.Tensor) -> torch.Tensor:
-    """Matrix-core prefill attention over tiles of consecutive rows that share a page list."""
+                            tile_num_rows: torch.Tensor, rows_per_tile: Optional[int] = None) -> torch.Tensor:
+    """Matrix-core prefill attention over tiles of consecutive rows that share a page list.
+    rows_per_tile: `attn_prefill_tile_rows(hq, hk)` (default) or half of it."""
     _dev(q, torch.bfloat16, "q")
     _dev(k_pages, torch.bfloat16, "k_pages")
     for name, t in (("kv_page_indices", kv_page_indices), ("row_page_begin", row_page_begin),
@@ -668,6 +669,8 @@ def attention_prefill_tiles(q: torch.Tensor, k_pages: torch.Tensor, v_pages: tor
     st = kernels().pie_hip_attn_prefill_tiles(_ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(o),
                                               _ptr(kv_page_indices), _ptr(row_page_begin),
                                               _ptr(row_kv_len), _ptr(tile_row_start), _ptr(tile_num_rows),
-                                              tile_row_start.numel(), hq, hk, d, ps, C.c_float(-1.0), _stream())
+                                              tile_row_start.numel(),
+                                              rows_per_tile or attn_prefill_tile_rows(hq, hk), hq, hk, d,
+                                              ps, C.c_float(-1.0), _stream())
     _check(st, "pie_hip_attn_prefill_tiles")
     return o

@@ -22,9 +22,10 @@ def build_rows(b, ctx, chunks, tile_rows):
             np.array([t[0] for t in tiles], np.int32), np.array([t[1] for t in tiles], np.int32))
 
 
+@pytest.mark.parametrize("half", [False, True])
 @pytest.mark.parametrize("hq,hk,d,ps", [(8, 2, 128, 16), (8, 1, 128, 32), (4, 2, 64, 16), (4, 4, 64, 16),
-                                        (32, 8, 128, 16)])
-def test_tiles_match_oracle_and_row_kernel(gpu, oracle, hq, hk, d, ps):
+                                        (32, 8, 128, 16), (8, 2, 128, 48)])
+def test_tiles_match_oracle_and_row_kernel(gpu, oracle, hq, hk, d, ps, half):
     import torch
 
     from pie_amd import ops
@@ -34,6 +35,8 @@ def test_tiles_match_oracle_and_row_kernel(gpu, oracle, hq, hk, d, ps):
     b = make_paged_batch(rng, ctx, hk, d, ps, f32_to_bf16=oracle.f32_to_bf16)
     tr = ops.attn_prefill_tile_rows(hq, hk)
     assert tr == 128 // (hq // hk)
+    if half:
+        tr //= 2
     # a later chunk of a long prompt, a whole short prompt, a prompt shorter than a tile, one token
     chunks = [(120, 80), (0, 75), (0, 33), (0, 1)]
     row_begin, row_len, tile_start, tile_n = build_rows(b, ctx, chunks, tr)
@@ -43,7 +46,7 @@ def test_tiles_match_oracle_and_row_kernel(gpu, oracle, hq, hk, d, ps):
         torch.from_numpy(np.ascontiguousarray(a)).to(gpu))
     args = (dev(q, torch.bfloat16), dev(b["k_pages"], torch.bfloat16), dev(b["v_pages"], torch.bfloat16),
             dev(b["page_indices"].view(np.int32)), dev(row_begin), dev(row_len))
-    o = ops.attention_prefill_tiles(*args, dev(tile_start), dev(tile_n))
+    o = ops.attention_prefill_tiles(*args, dev(tile_start), dev(tile_n), rows_per_tile=tr)
     torch.cuda.synchronize()
     got_bits = o.view(torch.uint16).cpu().numpy()
     got = oracle.bf16_to_f32(got_bits).astype(np.float64)
