@@ -374,7 +374,7 @@ def main():
     pages_per_ctx = (args.prompt + max_new + page_size - 1) // page_size
     total_pages = pages_per_ctx * args.batch + 8
     model, label = (MODEL, None) if args.model == "llama8b-w4a16" else OTHER_MODELS[args.model]
-    cfg_text = toml(model, page_size, total_pages, 512, max(16, args.batch))
+    cfg_text = toml(model, page_size, total_pages, 2048, max(16, args.batch))
     hip = Hip()
     rng = np.random.default_rng(2048)
     prompt = rng.integers(0, model["vocab"], args.prompt)

@@ -10,8 +10,9 @@
 // integer / e4m3 value itself, exact in bf16, with the row scale applied to the fp32 sum),
 // bf16 x bf16 products, fp32 accumulation, one rounding at the end.
 //
-// Tiling: a 128 x 128 output tile per block of four waves, each wave a 64 x 64 quadrant held as
-// 4 x 4 accumulators of v_mfma_f32_16x16x32_bf16; K advances 64 at a time.
+// Tiling: a 128 x 128 (or, for large M, 256 x 128) output tile per block of four waves, each wave
+// a 64 x 64 (128 x 64) quadrant held as 4 x 4 (8 x 4) accumulators of v_mfma_f32_16x16x32_bf16; K
+// advances 64 at a time.
 //   * activations (and bf16 weights) travel global -> LDS directly (global_load_lds_dwordx4,
 //     no registers) into a ring of three stages, issued two K steps ahead; every wave waits
 //     for its own transfers with an explicit vmcnt and the block meets at one barrier per step;
@@ -36,6 +37,7 @@ constexpr int BM = 128, BN = 128, BK = 64;
 constexpr int kThreads = 256;
 constexpr int kTileVecs = BM * (BK / 8);   // 16-byte vectors per bf16 tile (16 KiB)
 constexpr int kStages = 3;
+constexpr int kMaxMT = 8;   // 16-row activation tiles per wave, at most
 
 #define PIE_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
 
@@ -158,29 +160,43 @@ struct GBf16 {
 // s_waitcnt with vmcnt(n) (n < 16) and lgkmcnt(0), expcnt untouched (gfx9 encoding)
 #define PIE_WAIT_VM_LGKM0(n) __builtin_amdgcn_s_waitcnt(0x0070 | (n))
 
+// MT: 16-row activation tiles per wave.  4: a 128 x 128 block tile (64 x 64 per wave); 8: a
+// 256 x 128 block tile (128 x 64 per wave) — 12 operand reads feed 32 MFMAs instead of 8 for 16,
+// which moves the kernel from LDS-bound to MFMA-bound when M is large enough to fill the
+// machine with the bigger tiles.
+template <class Base, int MT_>
+struct Shape : Base {
+    static constexpr int kMT = MT_;
+};
+
 template <class F>
 __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(const GemmArgs a) {
+    constexpr int MT = F::kMT;
+    constexpr int BMv = 32 * MT;                 // activation rows per block
+    constexpr int kATileVecs = BMv * (BK / 8);   // 16-byte vectors per activation stage
     extern __shared__ __align__(16) unsigned char smem[];
-    u32x4_t* lds_a = reinterpret_cast<u32x4_t*>(smem);            // [kStages][tile]
-    u32x4_t* lds_b = lds_a + kStages * kTileVecs;                 // direct: [kStages][tile]; else [2][tile]
+    u32x4_t* lds_a = reinterpret_cast<u32x4_t*>(smem);            // [kStages][A tile]
+    u32x4_t* lds_b = lds_a + kStages * kATileVecs;                // direct: [kStages][tile]; else [2][tile]
     const int tid = threadIdx.x, lane = tid & (kWave - 1);
     const int wv = __builtin_amdgcn_readfirstlane(tid / kWave);
     const int j = lane & 15, q = lane >> 4;
     const int wm = wv >> 1, wn = wv & 1;
     const int M = a.M, N = a.N, K = a.K;
-    const int n0 = blockIdx.x * BN, m0 = blockIdx.y * BM;
+    const int n0 = blockIdx.x * BN, m0 = blockIdx.y * BMv;
     const int nk = K / BK;
 
     // direct transfers: wave w moves the 1 KiB chunks ci = 4u + w (8 tile rows each); lane p
     // lands at chunk position p = (row ci*8 + p/8, slot p%8), which holds granule slot ^ key(row)
-    const uint16_t* aptr[4];
+    const uint16_t* aptr[kMaxMT];   // (fixed bounds: arrays sized by the template value kept the
+                                    // host side from emitting the kernel stubs)
     const uint16_t* bptr[4];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < MT; ++u) {
         const int r = (u * 4 + wv) * 8 + (lane >> 3);
         const int g = (lane & 7) ^ ((r >> 1) & 7);
         aptr[u] = a.act + static_cast<size_t>(min(m0 + r, M - 1)) * K + g * 8;
-        bptr[u] = reinterpret_cast<const uint16_t*>(a.w) + static_cast<size_t>(min(n0 + r, N - 1)) * K + g * 8;
+        if (u < 4)
+            bptr[u] = reinterpret_cast<const uint16_t*>(a.w) + static_cast<size_t>(min(n0 + r, N - 1)) * K + g * 8;
     }
     auto issue_direct = [&](int kt) {
         const int k0 = min(kt, nk - 1) * BK;
@@ -191,16 +207,16 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(const GemmArgs a) {
                 __builtin_amdgcn_global_load_lds(bptr[u] + k0, PIE_LDS_PTR(lds_b + st * kTileVecs + (u * 4 + wv) * 64), 16, 0, 0);
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u)
-            __builtin_amdgcn_global_load_lds(aptr[u] + k0, PIE_LDS_PTR(lds_a + st * kTileVecs + (u * 4 + wv) * 64), 16, 0, 0);
+        for (int u = 0; u < MT; ++u)
+            __builtin_amdgcn_global_load_lds(aptr[u] + k0, PIE_LDS_PTR(lds_a + st * kATileVecs + (u * 4 + wv) * 64), 16, 0, 0);
     };
     const int wrow = tid >> 1;
     const int wn_glob = min(n0 + wrow, N - 1);
     auto load_w = [&](int kt) { return F::load(a, wn_glob, min(kt, nk - 1) * BK, tid); };
 
-    f32x4_t acc[4][4];
+    f32x4_t acc[kMaxMT][4];
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt)
+    for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int nt = 0; nt < 4; ++nt) acc[mt][nt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
@@ -225,8 +241,8 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(const GemmArgs a) {
             // Transfers of step kt are complete when at most the operations issued after them
             // are outstanding: the previous iteration's weight loads and its 4 (8) transfers.
             __builtin_amdgcn_sched_barrier(0);
-            if (F::kDirect) PIE_WAIT_VM_LGKM0(8);
-            else PIE_WAIT_VM_LGKM0(4 + F::kLoads);
+            if (F::kDirect) PIE_WAIT_VM_LGKM0(4 + MT);
+            else PIE_WAIT_VM_LGKM0(MT + F::kLoads);
             __builtin_amdgcn_s_barrier();
             __builtin_amdgcn_sched_barrier(0);
             rr[i] = load_w(kt + kStages);   // slot i held step kt, already written to LDS
@@ -235,20 +251,19 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(const GemmArgs a) {
             __builtin_amdgcn_sched_barrier(0);
 
             if (kt < nk) {
-                const u32x4_t* A = lds_a + i * kTileVecs + (wm * 64 + j) * 8;
+                const u32x4_t* A = lds_a + i * kATileVecs + (wm * 16 * MT + j) * 8;
                 const u32x4_t* B = lds_b + (F::kDirect ? i : (kt & 1)) * kTileVecs + (wn * 64 + j) * 8;
                 const int key = j >> 1;   // swizzle key of rows base16 + j
 #pragma unroll
                 for (int ks = 0; ks < BK / 32; ++ks) {
-                    bf16x8_t af[4], bfr[4];
+                    bf16x8_t af[kMaxMT], bfr[4];
                     const int slot = (ks * 4 + q) ^ key;
 #pragma unroll
-                    for (int t = 0; t < 4; ++t) {
-                        af[t] = __builtin_bit_cast(bf16x8_t, A[t * 16 * 8 + slot]);
-                        bfr[t] = __builtin_bit_cast(bf16x8_t, B[t * 16 * 8 + slot]);
-                    }
+                    for (int t = 0; t < MT; ++t) af[t] = __builtin_bit_cast(bf16x8_t, A[t * 16 * 8 + slot]);
 #pragma unroll
-                    for (int mt = 0; mt < 4; ++mt)
+                    for (int t = 0; t < 4; ++t) bfr[t] = __builtin_bit_cast(bf16x8_t, B[t * 16 * 8 + slot]);
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
                         for (int nt = 0; nt < 4; ++nt)
                             acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[mt], bfr[nt], acc[mt][nt], 0, 0, 0);
@@ -271,10 +286,10 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(const GemmArgs a) {
                                  : reinterpret_cast<const float*>(a.scale)[nc];
         }
 #pragma unroll
-        for (int mt = 0; mt < 4; ++mt)
+        for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const int m = m0 + wm * 64 + mt * 16 + 4 * q + r;
+                const int m = m0 + wm * 16 * MT + mt * 16 + 4 * q + r;
                 float v = acc[mt][nt][r] * rs;
                 const bool ok = m < M && n < N;
                 if (a.swiglu) {
@@ -294,17 +309,34 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(const GemmArgs a) {
     }
 }
 
-template <class F>
-int launch_gemm(const GemmArgs& a, hipStream_t stream) {
-    constexpr size_t smem = static_cast<size_t>(kStages + (F::kDirect ? kStages : 2)) * kTileVecs * sizeof(u32x4_t);
+template <class F, int MT>
+int launch_gemm_mt(const GemmArgs& a, hipStream_t stream) {
+    constexpr int BMv = 32 * MT;
+    constexpr size_t smem = (static_cast<size_t>(kStages) * BMv * (BK / 8) +
+                             static_cast<size_t>(F::kDirect ? kStages : 2) * kTileVecs) * sizeof(u32x4_t);
     static const hipError_t attr =
-        hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_mfma_kernel<F>),
+        hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_mfma_kernel<Shape<F, MT>>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
     if (attr != hipSuccess) return PIE_HIP_ERR_LAUNCH;
-    const dim3 grid((a.N + BN - 1) / BN, (a.M + BM - 1) / BM);
+    const dim3 grid((a.N + BN - 1) / BN, (a.M + BMv - 1) / BMv);
     if (grid.y > 65535) return PIE_HIP_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL(gemm_mfma_kernel<F>, grid, dim3(kThreads), smem, stream, a);
+    hipLaunchKernelGGL((gemm_mfma_kernel<Shape<F, MT>>), grid, dim3(kThreads), smem, stream, a);
     return launch_status();
+}
+
+// Measured at M = 2048 (MI355X): with both operands direct-to-LDS (bf16 weights) a 256-row tile
+// takes 1.66x the time of a 128-row tile for twice the work (790-930 against 650-820 TFLOP/s);
+// with quantised weights the decode-and-store stage, not the operand reads, sets the pace and
+// the taller tile gains nothing (int4 650-710 either way, fp8 slower), so those keep 128 rows.
+// PIE_HIP_GEMM_MT=4|8 forces a shape (measurement hook).
+template <class F>
+int launch_gemm(const GemmArgs& a, hipStream_t stream) {
+    static const int forced = [] { const char* e = getenv("PIE_HIP_GEMM_MT"); return e ? atoi(e) : 0; }();
+    const long long nt = (a.N + BN - 1) / BN;
+    const long long t4 = nt * ((a.M + 127) / 128), t8 = nt * ((a.M + 255) / 256);
+    const double c4 = static_cast<double>((t4 + 255) / 256), c8 = 1.66 * static_cast<double>((t8 + 255) / 256);
+    const bool tall = forced ? forced == 8 : (F::kDirect && a.M > 128 && c8 < c4);
+    return tall ? launch_gemm_mt<F, 8>(a, stream) : launch_gemm_mt<F, 4>(a, stream);
 }
 
 }  // namespace
