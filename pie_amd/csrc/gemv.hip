@@ -44,6 +44,7 @@ namespace {
 constexpr int kBlock = 256;  // 4 waves: one per SIMD of a CU
 constexpr int kWavesPerBlock = kBlock / kWave;
 constexpr int kNumCU = 256;
+constexpr int kUnits = 2;   // work units in flight per wave
 
 typedef float f32x2_t __attribute__((ext_vector_type(2)));
 
@@ -104,17 +105,37 @@ struct FmtInt4 {
                  bf16_lo(xs[i].z) + bf16_hi(xs[i].z) + bf16_lo(xs[i].w) + bf16_hi(xs[i].w);
         return s;
     }
+    // the same staging from a register: v = activations 8*sv .. 8*sv + 7 of a row
+    static __device__ __forceinline__ void stage_vec(u32x4_t* xrow, int sv, const u32x4_t v) {
+        const int c = sv >> 8, l = (sv & 255) >> 2, i = sv & 3;
+        u32x4_t p;
+        p.x = (v.x & 0xFFFFu) | (v.z << 16);
+        p.y = (v.x >> 16) | (v.z & 0xFFFF0000u);
+        p.z = (v.y & 0xFFFFu) | (v.w << 16);
+        p.w = (v.y >> 16) | (v.w & 0xFFFF0000u);
+        xrow[(c * XV + i) * kWave + l] = p;
+    }
     static __device__ __forceinline__ float dot(const u32x4_t w, const u32x4_t* xs, float p) {
         const uint32_t kMask = 0x000F000Fu;
         uint32_t k128 = 0x43004300u;  // (128.0bf16, 128.0bf16), kept in a VGPR for and_or
         asm volatile("" : "+v"(k128));
+        // all sixteen pairs first, then the dot products: a dot product issued right behind the
+        // instruction that made its operand costs a wait state
+        uint32_t t[16];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const uint32_t v = w[i];
-            p = dot2_bf16(xs[i].x, and_or(v, kMask, k128), p);
-            p = dot2_bf16(xs[i].y, and_or(v >> 4, kMask, k128), p);
-            p = dot2_bf16(xs[i].z, and_or(v >> 8, kMask, k128), p);
-            p = dot2_bf16(xs[i].w, and_or(v >> 12, kMask, k128), p);
+            t[4 * i + 0] = and_or(v, kMask, k128);
+            t[4 * i + 1] = and_or(v >> 4, kMask, k128);
+            t[4 * i + 2] = and_or(v >> 8, kMask, k128);
+            t[4 * i + 3] = and_or(v >> 12, kMask, k128);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            p = dot2_bf16(xs[i].x, t[4 * i + 0], p);
+            p = dot2_bf16(xs[i].y, t[4 * i + 1], p);
+            p = dot2_bf16(xs[i].z, t[4 * i + 2], p);
+            p = dot2_bf16(xs[i].w, t[4 * i + 3], p);
         }
         return p;
     }
@@ -128,6 +149,9 @@ struct FmtBf16 {
         return ld.load8(k0);
     }
     static __device__ __forceinline__ float sum_x(const u32x4_t*) { return 0.f; }
+    static __device__ __forceinline__ void stage_vec(u32x4_t* xrow, int sv, const u32x4_t v) {
+        xrow[sv] = v;   // (chunk sv / 64, lane sv % 64)
+    }
     static __device__ __forceinline__ float dot(const u32x4_t w, const u32x4_t* xs, float p) {
         p = dot2_bf16(xs[0].x, w.x, p);
         p = dot2_bf16(xs[0].y, w.y, p);
@@ -151,6 +175,11 @@ struct FmtF32Act {
             s += __uint_as_float(xs[i].x) + __uint_as_float(xs[i].y) + __uint_as_float(xs[i].z) +
                  __uint_as_float(xs[i].w);
         return s;
+    }
+    static __device__ __forceinline__ void stage_vec(u32x4_t* xrow, int sv, const u32x4_t v) {
+        const int c = sv >> 7, l = (sv & 127) >> 1, h = sv & 1;
+        xrow[(c * XV + 2 * h) * kWave + l] = u32x4_t{v.x << 16, v.x & 0xFFFF0000u, v.y << 16, v.y & 0xFFFF0000u};
+        xrow[(c * XV + 2 * h + 1) * kWave + l] = u32x4_t{v.z << 16, v.z & 0xFFFF0000u, v.w << 16, v.w & 0xFFFF0000u};
     }
 };
 
@@ -227,6 +256,7 @@ struct GemvArgs {
     uint16_t* k_pages;
     uint16_t* v_pages;
     int hq, hk, d;
+    int g_shift;  // log2(G) when G is a power of two, else -1 (set by dispatch)
 };
 
 // ROPE: the q|k|v epilogue (rotation + KV write); its per-lane cos / sin / slot ride with every
@@ -261,18 +291,22 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
 
     // Branch-free loads: lanes past K re-read lane 0's piece and are masked out in compute;
     // rows past the slice re-read its last row and are dropped at the store.
-    auto issue = [&](Unit<R>& u, int g, int c) {
+    // (`live` false: a unit past the end of the slice; every lane then re-reads one 16-byte
+    // piece, so the request costs a single cache line)
+    auto issue = [&](Unit<R>& u, int g, int c, bool live) {
         const int kbase = c * kChunkK + lane * WPP;
         const bool valid = kbase < K;
-        const int piece = valid ? c * kWave + lane : 0;
+        const int piece = (valid && live) ? c * kWave + lane : 0;
+        int gidx = 0;   // scale group of this lane's piece
+        if constexpr (F::kGroupScale)
+            gidx = (valid && live) ? (a.g_shift >= 0 ? kbase >> a.g_shift : kbase / a.G) : 0;
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const int row = min(row_begin + g * R + r, row_end - 1);
+            const int row = live ? min(row_begin + g * R + r, row_end - 1) : row_begin;
             u.w[r] = __builtin_nontemporal_load(a.w + static_cast<size_t>(row) * row_stride_v4 +
                                                 piece);
             if constexpr (F::kGroupScale)
-                u.gs[r] = a.gscale[static_cast<size_t>(row) * groups_per_row +
-                                   (valid ? kbase / a.G : 0)];
+                u.gs[r] = a.gscale[static_cast<size_t>(row) * groups_per_row + gidx];
         }
         // Every unit prefetches what the lane that finishes an output needs, so the
         // epilogue never stalls the pipeline (only the last chunk's values are used).
@@ -281,8 +315,10 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
         const int per = pairs ? (R / 2) * M : R * M;
         const int li = lane < per ? lane / M : 0;
         const int lm = lane < per ? lane % M : 0;
-        const int lrow = pairs ? min(row_begin + g * R + 2 * li, row_end - 2)
-                               : min(row_begin + g * R + li, row_end - 1);
+        // (a wave whose slice is empty has no live unit: row_end - 1 may be -1 there)
+        const int lrow = !live ? row_begin
+                         : pairs ? min(row_begin + g * R + 2 * li, row_end - 2)
+                                 : min(row_begin + g * R + li, row_end - 1);
         u.prev = a.y[pairs ? 0 : static_cast<size_t>(lm) * N + lrow];
         if constexpr (F::kRowScale) {
             u.rs = F::load(a.rscale, lrow);
@@ -297,13 +333,107 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
         }
     };
 
-    Unit<R> ua, ub;
-    if (nunits > 0) issue(ua, 0, 0);
+    // kUnits work units are requested before the activations are staged and stay in flight
+    // from then on.  (Measured: deeper rings than two lose on every decode shape of an 8B
+    // model, 1.84 / 1.94 / 2.03 ms per decode step for 2 / 3 / 4 units.)
+    Unit<R> un[kUnits];
+    int ug[kUnits], uc[kUnits];
+    int next_g = 0, next_c = 0, issued = 0;
+    auto issue_next = [&](Unit<R>& u, int& og, int& oc) {
+        og = next_g;
+        oc = next_c;
+        issue(u, next_g, next_c, issued < nunits);
+        ++issued;
+        if (++next_c == nchunks) {
+            next_c = 0;
+            ++next_g;
+        }
+    };
+    // Activation rows short enough to sit in registers (8 vectors of 16 bytes per thread) are
+    // requested before the weights: memory operations return in order, so a prologue that
+    // loads activations after the first weight requests starts only when those have arrived
+    // from HBM.  Longer rows keep the two-pass prologue below.
+    constexpr int kPreJ = 8 / M;
+    const int nv = K / 8, nvp = nchunks * (kChunkK / 8);   // real / padded source vectors per row
+    const bool pre = nvp <= kPreJ * kBlock;
+    u32x4_t xr[kPreJ * M], nw[kPreJ];
+    if (pre) {
+#pragma unroll
+        for (int jj = 0; jj < kPreJ; ++jj) {
+            const int sv = tid + jj * kBlock;
+            const int svc = min(sv, nv - 1);
+#pragma unroll
+            for (int m = 0; m < M; ++m) {
+                const u32x4_t v = *reinterpret_cast<const u32x4_t*>(a.act + static_cast<size_t>(m) * K + svc * 8);
+                xr[jj * M + m] = sv < nv ? v : u32x4_t{0u, 0u, 0u, 0u};
+            }
+            if (a.norm_w) nw[jj] = *reinterpret_cast<const u32x4_t*>(a.norm_w + svc * 8);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < kUnits; ++i) issue_next(un[i], ug[i], uc[i]);
 
-    // Optional fused RMSNorm: sum of squares of each activation row (fp32), block-reduced.
     float inv_rms[M];
 #pragma unroll
     for (int m = 0; m < M; ++m) inv_rms[m] = 1.f;
+    if (pre) {
+        // ---- activations from registers (requested before the weights) ----
+        if (a.norm_w) {
+            float* red = lds_sx;  // free until the sums are written below
+#pragma unroll
+            for (int m = 0; m < M; ++m) {
+                float local = 0.f;
+#pragma unroll
+                for (int jj = 0; jj < kPreJ; ++jj) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const float lo = bf16_lo(xr[jj * M + m][i]), hi = bf16_hi(xr[jj * M + m][i]);
+                        local += lo * lo + hi * hi;
+                    }
+                }
+                local = wave_sum_dpp(local);
+                if (lane == 0) red[m * kWavesPerBlock + wv] = local;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int m = 0; m < M; ++m) {
+                float t = 0.f;
+#pragma unroll
+                for (int w = 0; w < kWavesPerBlock; ++w) t += red[m * kWavesPerBlock + w];
+                inv_rms[m] = rsqrtf(t / static_cast<float>(K) + a.eps);
+            }
+            __syncthreads();
+        }
+#pragma unroll
+        for (int jj = 0; jj < kPreJ; ++jj) {
+            const int sv = tid + jj * kBlock;
+            if (sv < nvp) {
+#pragma unroll
+                for (int m = 0; m < M; ++m) {
+                    u32x4_t v = xr[jj * M + m];
+                    if (a.norm_w) {
+                        const ActLoader ld{nullptr, a.norm_w, inv_rms[m]};
+                        v = u32x4_t{ld.norm2(v.x, nw[jj].x), ld.norm2(v.y, nw[jj].y),
+                                    ld.norm2(v.z, nw[jj].z), ld.norm2(v.w, nw[jj].w)};
+                    }
+                    F::stage_vec(lds_x + m * vec_per_m, sv, v);
+                    if (F::kBias != 0.f) {
+                        // the WPP / 8 neighbouring lanes that hold one piece's activations add
+                        // their sums (a piece never straddles a quad)
+                        float sx = bf16_lo(v.x) + bf16_hi(v.x) + bf16_lo(v.y) + bf16_hi(v.y) +
+                                   bf16_lo(v.z) + bf16_hi(v.z) + bf16_lo(v.w) + bf16_hi(v.w);
+                        constexpr int kPer = WPP / 8;   // 4 (int4) or 2 (byte formats)
+                        sx = dpp_add_f32<0xB1>(sx);                      // quad_perm [1,0,3,2]
+                        if (kPer == 4) sx = dpp_add_f32<0x4E>(sx);       // quad_perm [2,3,0,1]
+                        const int piece = sv / kPer;   // = chunk * 64 + lane
+                        if ((sv & (kPer - 1)) == 0) lds_sx[m * nchunks * kWave + piece] = sx;
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    } else {
+    // Optional fused RMSNorm: sum of squares of each activation row (fp32), block-reduced.
     if (a.norm_w) {
         float* red = lds_sx;  // free until the sum_x pass below
 #pragma unroll
@@ -363,6 +493,7 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
             lds_sx[j] = F::sum_x(xs);
         }
         __syncthreads();
+    }
     }
 
     float acc[R][M];
@@ -466,26 +597,15 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
         }
     };
 
-    // Two-deep software pipeline over (row group, chunk) units.  Loads are issued
-    // unconditionally (past the end they re-request the last unit) so the wait
-    // before each compute only covers the unit it consumes.
-    const int last_g = ngroups - 1, last_c = nchunks - 1;
-    auto advance = [&](int& gg, int& cc) {
-        if (gg == last_g && cc == last_c) return;
-        if (++cc == nchunks) { cc = 0; ++gg; }
-    };
-    int g = 0, c = 0;  // coordinates of the unit held in `ua`
-    for (int u = 0; u < nunits; u += 2) {
-        int g1 = g, c1 = c;
-        advance(g1, c1);
-        int g2 = g1, c2 = c1;
-        advance(g2, c2);
-        issue(ub, g1, c1);
-        compute(ua, g, c);
-        issue(ua, g2, c2);
-        if (u + 1 < nunits) compute(ub, g1, c1);
-        g = g2;
-        c = c2;
+    // Ring of kUnits units: a unit's registers are requested again as soon as it has been
+    // reduced.  Loads are issued unconditionally so the wait before each compute only covers
+    // the unit it consumes.
+    for (int u = 0; u < nunits; u += kUnits) {
+#pragma unroll
+        for (int i = 0; i < kUnits; ++i) {
+            if (u + i < nunits) compute(un[i], ug[i], uc[i]);
+            issue_next(un[i], ug[i], uc[i]);
+        }
     }
 }
 
@@ -541,6 +661,7 @@ int dispatch(GemvArgs a, int M, int rows_per_wave, int waves_per_simd, hipStream
     // Measured on MI355X: two resident waves per SIMD, each walking its slice four rows
     // at a time (fewer when the slice is shorter), is within a few percent of the best
     // (rows, waves) pair for every decode shape of an 8B-class model.
+    a.g_shift = (a.G > 0 && (a.G & (a.G - 1)) == 0) ? __builtin_ctz(static_cast<unsigned>(a.G)) : -1;
     if (waves_per_simd <= 0) waves_per_simd = 2;
     if (waves_per_simd > 8) return PIE_HIP_ERR_INVALID;
     if (rows_per_wave <= 0) {
