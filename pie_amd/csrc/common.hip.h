@@ -67,6 +67,42 @@ __device__ __forceinline__ float wave_sum_dpp(float v) {
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov_f32(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+
+// Wave64 sums of NV (2 or 4) values at once: lane i < NV ends with the total of v[i] (every
+// lane ends with the total of value `lane' & (NV - 1)`, lane' = lane with its low two bits
+// flipped in odd quads).  The first log2(NV) butterfly steps halve the number of values a lane
+// carries instead of adding NV separate butterflies: each lane keeps the values whose index
+// bit matches its lane bit and sends the others to its partner.  Odd quads use the mirrored
+// assignment so that the two mirror steps (lane ^ 7, lane ^ 15) pair lanes that carry the same
+// value; rows are folded with the 16- and 32-lane swaps.  Every value is added over the same
+// tree as wave_sum_dpp uses, so the totals are bit-identical to NV separate wave_sum_dpp calls.
+template <int NV>
+__device__ __forceinline__ float wave_sum_multi(const float* v, int lane) {
+    static_assert(NV == 2 || NV == 4, "two or four values");
+    const int lp = (lane & 4) ? lane ^ 3 : lane;
+    const bool b0 = lp & 1;
+    float x;
+    if (NV == 4) {
+        const float a = (b0 ? v[1] : v[0]) + dpp_mov_f32<0xB1>(b0 ? v[0] : v[1]);   // lane ^ 1
+        const float b = (b0 ? v[3] : v[2]) + dpp_mov_f32<0xB1>(b0 ? v[2] : v[3]);
+        const bool b1 = lp & 2;
+        x = (b1 ? b : a) + dpp_mov_f32<0x4E>(b1 ? a : b);                           // lane ^ 2
+    } else {
+        x = (b0 ? v[1] : v[0]) + dpp_mov_f32<0xB1>(b0 ? v[0] : v[1]);
+        x = dpp_add_f32<0x4E>(x);
+    }
+    x = dpp_add_f32<0x141>(x);   // row_half_mirror (lane ^ 7)
+    x = dpp_add_f32<0x140>(x);   // row_mirror (lane ^ 15)
+    const auto r16 = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    x = __uint_as_float(r16[0]) + __uint_as_float(r16[1]);   // rows 0+1, 2+3
+    const auto r32 = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(r32[0]) + __uint_as_float(r32[1]);
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);

@@ -523,13 +523,25 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
             }
         }
         if (c == nchunks - 1) {
+            // One activation row and 2-4 weight rows (single-sequence decode): the R sums are
+            // reduced together and lane r holds row r's total.  Otherwise one butterfly each.
+            constexpr bool kMulti = M == 1 && R >= 2;
             float tot[R][M];
+            float multi = 0.f;
+            if constexpr (kMulti) {
+                const float vals[4] = {acc[0][0], acc[1][0], R > 2 ? acc[R > 2 ? 2 : 0][0] : 0.f,
+                                       R > 3 ? acc[R > 3 ? 3 : 0][0] : 0.f};
+                multi = wave_sum_multi<(R > 2 ? 4 : 2)>(vals, lane);
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
+                for (int r = 0; r < R; ++r) acc[r][0] = 0.f;
+            } else {
 #pragma unroll
-                for (int m = 0; m < M; ++m) {
-                    tot[r][m] = wave_sum_dpp(acc[r][m]);
-                    acc[r][m] = 0.f;
+                for (int r = 0; r < R; ++r) {
+#pragma unroll
+                    for (int m = 0; m < M; ++m) {
+                        tot[r][m] = wave_sum_dpp(acc[r][m]);
+                        acc[r][m] = 0.f;
+                    }
                 }
             }
             if (pairs) {
@@ -537,13 +549,18 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
                     // lane p*M + m finishes pair p: g and u are rounded to bf16 first, as the
                     // unfused projection would store them (swiglu.cu:18-21 reads bf16 inputs)
                     float gv = 0.f, uv = 0.f;
+                    if constexpr (kMulti) {
+                        gv = dpp_mov_f32<0x88>(multi);   // quad_perm [0,2,0,2]: lane p <- lane 2p
+                        uv = dpp_mov_f32<0xDD>(multi);   // quad_perm [1,3,1,3]: lane p <- lane 2p + 1
+                    } else {
 #pragma unroll
-                    for (int pr = 0; pr < R / 2; ++pr) {
+                        for (int pr = 0; pr < R / 2; ++pr) {
 #pragma unroll
-                        for (int m = 0; m < M; ++m) {
-                            if (lane == pr * M + m) {
-                                gv = tot[2 * pr][m];
-                                uv = tot[2 * pr + 1][m];
+                            for (int m = 0; m < M; ++m) {
+                                if (lane == pr * M + m) {
+                                    gv = tot[2 * pr][m];
+                                    uv = tot[2 * pr + 1][m];
+                                }
                             }
                         }
                     }
@@ -562,7 +579,8 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
                         } else {
                             // the projection's bf16 values, then the rotation of
                             // qkv_rope_kvwrite_kernel with the same operations and rounding
-                            const int head = row / a.d, dd = row - head * a.d;
+                            const int head = row >> __builtin_ctz(static_cast<unsigned>(a.d));   // (power of two)
+                            const int dd = row & (a.d - 1);
                             const int slot = u.slot;
                             if (head < a.hq + a.hk) {
                                 const float c = u.rc, sn = u.rsn;
@@ -580,11 +598,15 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
                 }
             } else {
                 float mine = 0.f;
+                if constexpr (kMulti) {
+                    mine = multi;
+                } else {
 #pragma unroll
-                for (int r = 0; r < R; ++r) {
+                    for (int r = 0; r < R; ++r) {
 #pragma unroll
-                    for (int m = 0; m < M; ++m) {
-                        if (lane == r * M + m) mine = tot[r][m];
+                        for (int m = 0; m < M; ++m) {
+                            if (lane == r * M + m) mine = tot[r][m];
+                        }
                     }
                 }
                 const int row = row_begin + g * R + lane / M;
