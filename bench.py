@@ -282,24 +282,34 @@ def cpu_baseline(drv, model, page_size, total_pages, n_prompt, gpu_tokens, budge
     for l in range(model["layers"]):
         om.k_pages[l][...] = drv.export_tensor(f"kv.k.{l}", np.uint16).reshape(om.k_pages[l].shape)
         om.v_pages[l][...] = drv.export_tensor(f"kv.v.{l}", np.uint16).reshape(om.v_pages[l].shape)
-    steps, matched, t_total = 0, 0, 0.0
+    import oracle
+
+    steps, matched, near_ties, t_total = 0, 0, 0, 0.0
     tok = int(gpu_tokens[0])
     while steps < len(gpu_tokens) - 1 and (steps < 2 or t_total < budget_s):
         pos = n_prompt + steps
         npg = (pos + 1 + page_size - 1) // page_size
         t0 = time.perf_counter()
-        out, _, _ = om.forward([tok], [pos], np.arange(npg), [0, npg],
-                               [pos + 1 - (npg - 1) * page_size], [0, 1])
+        out, logits, _ = om.forward([tok], [pos], np.arange(npg), [0, npg],
+                                    [pos + 1 - (npg - 1) * page_size], [0, 1], want_logits=True)
         t_total += time.perf_counter() - t0
         steps += 1
-        matched += int(int(out[0]) == int(gpu_tokens[steps]))
+        if int(out[0]) == int(gpu_tokens[steps]):
+            matched += 1
+        else:
+            # a mismatch only counts where the oracle's own top-2 logits are clearly apart
+            # (the parity tests' bar: gap above 2^-6 of the top logit)
+            lg = oracle.bf16_to_f32(np.asarray(logits).reshape(-1))
+            top2 = np.partition(lg, -2)[-2:]
+            near_ties += int(float(top2[1] - top2[0]) <= 2.0 ** -6 * max(abs(float(top2[1])), 1e-30))
         tok = int(gpu_tokens[steps])  # teacher-forced: every step is compared on the same context
     cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
     return dict(value=steps / t_total, unit="tokens/s", cores=cores, kind="port",
                 sample=f"{steps} batch-1 decode steps of the same model at context {n_prompt}+, "
                        "oracle (C restatement of the reference forward pass, OpenMP over rows) "
                        "fed the GPU's weights and prefilled KV pages",
-                greedy_tokens_matched=matched, greedy_tokens_compared=steps)
+                greedy_tokens_matched=matched, greedy_tokens_compared=steps,
+                mismatches_at_oracle_near_ties=near_ties)
 
 
 # HBM bytes per GEMV launch, averaged over the model's four int4 linears at M = 1, from two

@@ -15,11 +15,12 @@
 //     balanced slice of the output rows, so all CUs start and finish together;
 //   * a wave walks its slice R rows at a time; every lane streams 16-byte pieces of
 //     each row, so one wave instruction covers 1 KiB of a row, fully coalesced.
-//     Loads are branch-free and issued one work unit (R rows x one 1 KiB chunk)
+//     Loads are branch-free and run a ring of two work units (R rows x one 1 KiB chunk)
 //     ahead of the arithmetic, so 2R independent 16 B loads per lane are in flight
 //     while the previous unit is being reduced;
-//   * the first unit is requested before the activation row is staged, so the
-//     HBM latency of the weights overlaps the LDS staging;
+//   * the first units are requested before the activation row is staged, so the
+//     HBM latency of the weights overlaps the LDS staging; the activations themselves
+//     are requested even earlier (vector memory operations return in order);
 //   * activations are staged once per block into LDS in exactly the order the
 //     format's in-register decode produces weights, laid out so a lane's 16 B LDS
 //     reads are conflict free;
@@ -32,7 +33,8 @@
 //     conversion instruction decodes them, with -128*sum(x) preset the same way;
 //   * fp8: the packed e4m3 -> f32 conversion instruction decodes two weights each;
 //   * bf16: weights feed v_dot2_f32_bf16 directly;
-//   * a wave64 butterfly finishes the row; the lane that stores an output has
+//   * a wave64 butterfly finishes the row (one shared butterfly for the 2-4 rows of a
+//     step when there is a single activation row); the lane that stores an output has
 //     prefetched the residual / row scale it needs with the unit's loads.
 #include <hip/hip_ext.h>
 
