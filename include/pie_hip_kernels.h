@@ -143,12 +143,28 @@ int pie_hip_gemm_skinny(int format, const uint16_t* act_bf16, const void* weight
  * (driver/cuda/src/kernels/dequant_wna16.cu:11-38) followed by a bf16 GEMM
  * (driver/cuda/src/ops/gemm.cpp:1213-1236); int8 / fp8 values are exact in bf16 and their row
  * scale multiplies the fp32 sum — then bf16 x bf16 products, fp32 accumulation, one rounding.
- * 128 x 128 x 64 tiles, v_mfma_f32_16x16x32_bf16.  Requirements: K % 64 == 0; int4b8
+ * 128 x 128 x 64 tiles (64 x 128 for M <= 64, 256 x 128 for bf16 weights at large M),
+ * v_mfma_f32_16x16x32_bf16.  Requirements: K % 64 == 0; int4b8
  * group_size a power of two >= 32 dividing K.
  */
 int pie_hip_gemm_mfma(int format, const uint16_t* act_bf16, const void* weight, const void* scale,
                       int scale_is_bf16, int group_size, uint16_t* y_bf16, int M, int N, int K,
                       int beta, int swiglu, void* stream);
+
+/*
+ * The same GEMM for a decode batch (M <= 128 rows), where the output has too few 128-column
+ * tiles to fill the machine: K is split into shares, one block per (tile, share), fp32 partial
+ * sums go to `workspace` and a second kernel adds them and applies beta / swiglu.  Same
+ * evaluation order per share; the shares are added in fp32 in ascending K.
+ * pie_hip_gemm_mfma_workspace_bytes(M, N, K) is the workspace this shape needs (0: the shape is
+ * not split and the call is pie_hip_gemm_mfma).  Role in the reference: cuBLASLt's split-K
+ * heuristics inside gemm_act_x_w for small M (driver/cuda/src/ops/gemm.cpp:1414-1583).
+ */
+size_t pie_hip_gemm_mfma_workspace_bytes(int M, int N, int K);
+int pie_hip_gemm_mfma_splitk(int format, const uint16_t* act_bf16, const void* weight,
+                             const void* scale, int scale_is_bf16, int group_size,
+                             uint16_t* y_bf16, int M, int N, int K, int beta, int swiglu,
+                             void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * MoE grouped weight-only GEMM: one skinny problem per expert in a single launch.

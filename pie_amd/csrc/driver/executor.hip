@@ -51,15 +51,29 @@ int fmt_code(Quant q) {
     }
 }
 
-// Measured cost models (MI355X, microseconds): the skinny GEMM streams the weights once per 16
-// rows at ~2.4 TB/s plus ~4 us per pass; the tiled GEMM walks K in 64-wide steps of ~1 us
-// while its 128 x 128 tiles fit the machine (512 resident blocks), longer in proportion beyond.
-bool tiled_gemm_is_faster(const Linear& w, int M) {
-    if (w.K % 64 != 0 || M < 48) return false;
-    const double skinny = ((M + 15) / 16) * (4.0 + static_cast<double>(w.data_bytes()) / 2.4e6);
-    const double tiles = static_cast<double>((w.N + 127) / 128) * ((M + 127) / 128);
-    const double gemm = (w.K / 64) * 0.97 * std::max(1.0, tiles / 512.0);
-    return gemm < skinny;
+// Measured cost models (MI355X, microseconds, int4 8B-class shapes at 16-128 rows).  Skinny GEMM:
+// ~5 us + the weights at ~2.8 TB/s for the first 16-row pass, each further (side-by-side) pass
+// adding 85 % of that stream.  Tiled GEMM: K in 64-wide steps of ~0.72 us with 64-row block
+// tiles (M <= 64), ~0.98 us with 128-row tiles, while the tiles fit the machine (512 resident
+// blocks).  Split-K tiled GEMM: the steps of one share (+3 of prologue) at 1.25 / 1.6 us with two
+// blocks per CU, per round of 512 blocks, plus ~15 us for the second kernel and the partials.
+enum class GemmPath { Skinny, Tiled, TiledSplitK };
+GemmPath pick_gemm(const Linear& w, int M, size_t ws_bytes) {
+    if (w.K % 64 != 0 || M < 17) return GemmPath::Skinny;
+    const int passes = (M + 15) / 16;
+    const double skinny = 5.0 + static_cast<double>(w.data_bytes()) / 2.8e6 * (1.0 + 0.85 * (passes - 1));
+    const int steps = w.K / 64;
+    const double tiles = static_cast<double>((w.N + 127) / 128) * (M <= 64 ? 1 : (M + 127) / 128);
+    const double tiled = 2.0 + steps * (M <= 64 ? 0.72 : 0.98) * std::max(1.0, tiles / 512.0);
+    double split = 1e30;
+    const size_t need = M <= 128 ? pie_hip_gemm_mfma_workspace_bytes(M, w.N, w.K) : 0;
+    if (need && need <= ws_bytes) {
+        const int shares = static_cast<int>(need / (static_cast<size_t>(M) * w.N * sizeof(float)));
+        const int per = (steps + shares - 1) / shares;
+        split = 15.0 + (per + 3) * (M <= 64 ? 1.25 : 1.6) * std::ceil(tiles * shares / 512.0);
+    }
+    if (split < skinny && split < tiled) return GemmPath::TiledSplitK;
+    return tiled < skinny ? GemmPath::Tiled : GemmPath::Skinny;
 }
 
 // y = epilogue(rmsnorm?(act) · W^T) by the weight's storage format — the dispatcher role of
@@ -69,7 +83,8 @@ bool tiled_gemm_is_faster(const Linear& w, int M) {
 // weights once per 16 rows, or the tiled matrix-core GEMM where its cost model wins; shapes those do
 // not take fall back to the GEMV path.
 void linear_fused(const Linear& w, const uint16_t* act, const uint16_t* norm_w, float eps,
-                  uint16_t* y, int M, int beta, int swiglu, uint16_t* norm_tmp, hipStream_t s) {
+                  uint16_t* y, int M, int beta, int swiglu, uint16_t* norm_tmp, void* gemm_ws,
+                  size_t gemm_ws_bytes, hipStream_t s) {
     const int fmt = fmt_code(w.kind);
     const int sbf = w.scale_bf16 ? 1 : 0;
     if (M > 4) {
@@ -78,10 +93,15 @@ void linear_fused(const Linear& w, const uint16_t* act, const uint16_t* norm_w, 
             PIE_KERNEL(pie_hip_rmsnorm(act, norm_w, norm_tmp, M, w.K, eps, s));
             a = norm_tmp;
         }
-        if (tiled_gemm_is_faster(w, M)) {
-            // compute-bound: the tiled GEMM (weights dequantised to bf16 while staged)
-            const int sg = pie_hip_gemm_mfma(fmt, a, w.data, w.scale, sbf, w.group, y, M, w.N, w.K,
-                                             beta, swiglu, s);
+        const GemmPath path = pick_gemm(w, M, gemm_ws_bytes);
+        if (path != GemmPath::Skinny) {
+            // the tiled GEMM (weights dequantised to bf16 while staged), in K shares for a
+            // decode batch whose output has few tiles
+            const int sg = path == GemmPath::TiledSplitK
+                               ? pie_hip_gemm_mfma_splitk(fmt, a, w.data, w.scale, sbf, w.group, y, M, w.N,
+                                                          w.K, beta, swiglu, gemm_ws, gemm_ws_bytes, s)
+                               : pie_hip_gemm_mfma(fmt, a, w.data, w.scale, sbf, w.group, y, M, w.N, w.K,
+                                                   beta, swiglu, s);
             if (sg == PIE_HIP_OK) return;
             if (sg != PIE_HIP_ERR_UNSUPPORTED) PIE_KERNEL(sg);
         }
@@ -164,6 +184,16 @@ Executor::Executor(const DriverConfig& cfg, Model& model) : cfg_(cfg), model_(mo
     // rows * splits <= 3072/hk + rows.
     attn_ws_bytes_ = (3072 / static_cast<size_t>(hk) + 1 + T) * hq * (d + 2) * sizeof(float);
     PIE_HIP_CHECK(hipMalloc(&attn_ws_, attn_ws_bytes_));
+    // fp32 partials of the split-K GEMM for decode batches of up to 128 rows (dense layers)
+    if (!model.layers.empty()) {
+        const LayerWeights& l0 = model.layers[0];
+        for (const Linear* w : {&l0.wqkv, &l0.wo, &l0.wgu, &l0.wdown})
+            for (int rows : {64, 128})
+                if (w->data && w->K % 64 == 0)
+                    gemm_ws_bytes_ = std::max(gemm_ws_bytes_, pie_hip_gemm_mfma_workspace_bytes(rows, w->N, w->K));
+        gemm_ws_bytes_ = std::min<size_t>(gemm_ws_bytes_, size_t(64) << 20);
+        if (gemm_ws_bytes_) PIE_HIP_CHECK(hipMalloc(&gemm_ws_, gemm_ws_bytes_));
+    }
 
     in_ = input_layout(max_tokens_, max_tokens_);
     in_.total = align_up(in_.off_pages + static_cast<size_t>(max_page_refs_) * 4, 256);
@@ -180,7 +210,7 @@ Executor::~Executor() {
     for (void* p : {static_cast<void*>(x_), static_cast<void*>(xn_), static_cast<void*>(qkv_),
                     static_cast<void*>(q_), static_cast<void*>(attn_), static_cast<void*>(gu_),
                     static_cast<void*>(act_), static_cast<void*>(xs_), static_cast<void*>(logits_),
-                    static_cast<void*>(rope_tab_), static_cast<void*>(out_tokens_), attn_ws_,
+                    static_cast<void*>(rope_tab_), static_cast<void*>(out_tokens_), attn_ws_, gemm_ws_,
                     static_cast<void*>(in_dev_), static_cast<void*>(copy_ids_),
                     static_cast<void*>(moe_y_), static_cast<void*>(moe_logits_),
                     static_cast<void*>(moe_idx_), static_cast<void*>(moe_w_),
@@ -244,7 +274,7 @@ void Executor::moe_block(const LayerWeights& w, int N, hipStream_t s) {
     const int fmt = fmt_code(w.wgu.kind);
     const int sbf = w.wgu.scale_bf16 ? 1 : 0;
     PIE_KERNEL(pie_hip_rmsnorm(x_, w.ffn_norm, xn_, N, H, m.rms_eps, s));
-    linear_fused(w.router, xn_, nullptr, m.rms_eps, moe_logits_, N, 0, 0, nullptr, s);
+    linear_fused(w.router, xn_, nullptr, m.rms_eps, moe_logits_, N, 0, 0, nullptr, gemm_ws_, gemm_ws_bytes_, s);
     PIE_KERNEL(pie_hip_moe_route(moe_logits_, moe_idx_, moe_w_, moe_offsets_, moe_route_token_,
                                  moe_route_pos_, N, E, K, s));
     const int hint = std::max(1, std::min(N, 2 * ((N * K + E - 1) / E)));
@@ -282,7 +312,7 @@ void Executor::body(int N, int S, int max_kv_len) {
                                               w.wqkv.group, N, H, rope_tab_, slots, q_, k_pool_[l],
                                               v_pool_[l], hq, hk, d, s));
         } else {
-            linear_fused(w.wqkv, x_, w.attn_norm, m.rms_eps, qkv_, N, 0, 0, xn_, s);
+            linear_fused(w.wqkv, x_, w.attn_norm, m.rms_eps, qkv_, N, 0, 0, xn_, gemm_ws_, gemm_ws_bytes_, s);
             PIE_KERNEL(pie_hip_qkv_rope_kvwrite(qkv_, q_, k_pool_[l], v_pool_[l], w.q_norm, w.k_norm,
                                                 rope_tab_, slots, N, hq, hk, d, m.rope_interleaved,
                                                 m.rms_eps, s));
@@ -302,13 +332,13 @@ void Executor::body(int N, int S, int max_kv_len) {
                                                row_begin, row_len, N, hq, hk, d, page_size_, -1.f,
                                                max_kv_len, attn_ws_, attn_ws_bytes_, s));
         }
-        linear_fused(w.wo, attn_, nullptr, m.rms_eps, x_, N, 1, 0, xn_, s);
+        linear_fused(w.wo, attn_, nullptr, m.rms_eps, x_, N, 1, 0, xn_, gemm_ws_, gemm_ws_bytes_, s);
         if (model_.is_moe()) {
             moe_block(w, N, s);
             continue;
         }
-        linear_fused(w.wgu, x_, w.ffn_norm, m.rms_eps, act_, N, 0, 1, xn_, s);
-        linear_fused(w.wdown, act_, nullptr, m.rms_eps, x_, N, 1, 0, xn_, s);
+        linear_fused(w.wgu, x_, w.ffn_norm, m.rms_eps, act_, N, 0, 1, xn_, gemm_ws_, gemm_ws_bytes_, s);
+        linear_fused(w.wdown, act_, nullptr, m.rms_eps, x_, N, 1, 0, xn_, gemm_ws_, gemm_ws_bytes_, s);
     }
     // lm_head only on the sampled rows (driver/portable/src/graph_qwen3.cpp:867-896)
     const int cap = static_cast<int>(std::min<size_t>(max_tokens_, 2 * static_cast<size_t>(cfg_.batching.max_forward_requests)));
@@ -320,7 +350,7 @@ void Executor::body(int N, int S, int max_kv_len) {
         head.data = model_.lm_head;
         head.N = m.vocab;
         head.K = H;
-        linear_fused(head, xs_, model_.final_norm, m.rms_eps, logits_, n, 0, 0, xn_, s);
+        linear_fused(head, xs_, model_.final_norm, m.rms_eps, logits_, n, 0, 0, xn_, gemm_ws_, gemm_ws_bytes_, s);
         PIE_KERNEL(pie_hip_argmax(logits_, out_tokens_ + s0, n, m.vocab, s));
         if (samp_gather_in_body_) {   // more sampled rows than one chunk: keep each chunk's f32 rows
             const auto* in = static_cast<const unsigned char*>(samp_in_dev_.ptr);

@@ -116,6 +116,8 @@ class Executor {
     uint32_t* out_tokens_ = nullptr;
     void* attn_ws_ = nullptr;
     size_t attn_ws_bytes_ = 0;
+    void* gemm_ws_ = nullptr;      // split-K partial sums of the tiled GEMM
+    size_t gemm_ws_bytes_ = 0;
     uint32_t* copy_ids_ = nullptr;  // staging for page-copy id lists
     size_t copy_ids_cap_ = 0;
 

@@ -47,6 +47,7 @@ struct GemmArgs {
     const unsigned char* scale;
     uint16_t* y;
     int M, N, K, g_shift, beta, swiglu, scale_is_bf16;
+    float* partial;   // split-K: fp32 [gridDim.z][M][N] partial sums (row scale applied), else null
 };
 
 __device__ __forceinline__ uint32_t pack_trunc(float lo, float hi) {
@@ -183,7 +184,11 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(const GemmArgs a) {
     const int wm = wv >> 1, wn = wv & 1;
     const int M = a.M, N = a.N, K = a.K;
     const int n0 = blockIdx.x * BN, m0 = blockIdx.y * BMv;
-    const int nk = K / BK;
+    // split-K: block z owns the K steps [kbeg, kbeg + nk) (the host makes every share non-empty)
+    const int nk_all = K / BK;
+    const int per_split = (nk_all + static_cast<int>(gridDim.z) - 1) / static_cast<int>(gridDim.z);
+    const int kbeg = blockIdx.z * per_split;
+    const int nk = min(per_split, nk_all - kbeg);
 
     // direct transfers: wave w moves the 1 KiB chunks ci = 4u + w (8 tile rows each); lane p
     // lands at chunk position p = (row ci*8 + p/8, slot p%8), which holds granule slot ^ key(row)
@@ -191,15 +196,15 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(const GemmArgs a) {
                                     // host side from emitting the kernel stubs)
     const uint16_t* bptr[4];
 #pragma unroll
-    for (int u = 0; u < MT; ++u) {
+    for (int u = 0; u < (MT > 4 ? MT : 4); ++u) {
         const int r = (u * 4 + wv) * 8 + (lane >> 3);
         const int g = (lane & 7) ^ ((r >> 1) & 7);
-        aptr[u] = a.act + static_cast<size_t>(min(m0 + r, M - 1)) * K + g * 8;
+        if (u < MT) aptr[u] = a.act + static_cast<size_t>(min(m0 + r, M - 1)) * K + g * 8;
         if (u < 4)
             bptr[u] = reinterpret_cast<const uint16_t*>(a.w) + static_cast<size_t>(min(n0 + r, N - 1)) * K + g * 8;
     }
     auto issue_direct = [&](int kt) {
-        const int k0 = min(kt, nk - 1) * BK;
+        const int k0 = (kbeg + min(kt, nk - 1)) * BK;
         const int st = kt % kStages;
         if (F::kDirect) {
 #pragma unroll
@@ -212,7 +217,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(const GemmArgs a) {
     };
     const int wrow = tid >> 1;
     const int wn_glob = min(n0 + wrow, N - 1);
-    auto load_w = [&](int kt) { return F::load(a, wn_glob, min(kt, nk - 1) * BK, tid); };
+    auto load_w = [&](int kt) { return F::load(a, wn_glob, (kbeg + min(kt, nk - 1)) * BK, tid); };
 
     f32x4_t acc[kMaxMT][4];
 #pragma unroll
@@ -292,7 +297,9 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(const GemmArgs a) {
                 const int m = m0 + wm * 16 * MT + mt * 16 + 4 * q + r;
                 float v = acc[mt][nt][r] * rs;
                 const bool ok = m < M && n < N;
-                if (a.swiglu) {
+                if (a.partial) {
+                    if (ok) a.partial[(static_cast<size_t>(blockIdx.z) * M + m) * N + n] = v;
+                } else if (a.swiglu) {
                     const float gb = bf16_bits_to_f32(f32_to_bf16_bits(v));
                     const float other = __int_as_float(__builtin_amdgcn_update_dpp(
                         0, __float_as_int(gb), 0xB1, 0xF, 0xF, true));  // quad_perm [1,0,3,2]
@@ -309,8 +316,38 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(const GemmArgs a) {
     }
 }
 
+// Sums the split-K partials and applies the epilogue the single-pass kernel would have applied
+// (residual add, or SwiGLU over adjacent (gate, up) columns with both rounded to bf16 first).
+__global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* partial, uint16_t* y,
+                                                                 int M, int N, int splits, int beta,
+                                                                 int swiglu) {
+    const int nout = swiglu ? N / 2 : N;
+    const size_t idx = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (idx >= static_cast<size_t>(M) * nout) return;
+    const int m = static_cast<int>(idx / nout), c = static_cast<int>(idx % nout);
+    const size_t plane = static_cast<size_t>(M) * N;
+    if (swiglu) {
+        const float* p = partial + static_cast<size_t>(m) * N + 2 * c;
+        float g = 0.f, u = 0.f;
+        for (int z = 0; z < splits; ++z) {
+            g += p[z * plane];
+            u += p[z * plane + 1];
+        }
+        const float gb = bf16_bits_to_f32(f32_to_bf16_bits(g));
+        const float ub = bf16_bits_to_f32(f32_to_bf16_bits(u));
+        const float silu = gb / (1.f + expf(-gb));
+        y[idx] = f32_to_bf16_bits(silu * ub);
+    } else {
+        const float* p = partial + static_cast<size_t>(m) * N + c;
+        float v = 0.f;
+        for (int z = 0; z < splits; ++z) v += p[z * plane];
+        if (beta) v += bf16_bits_to_f32(y[idx]);
+        y[idx] = f32_to_bf16_bits(v);
+    }
+}
+
 template <class F, int MT>
-int launch_gemm_mt(const GemmArgs& a, hipStream_t stream) {
+int launch_gemm_mt(const GemmArgs& a, int splits, hipStream_t stream) {
     constexpr int BMv = 32 * MT;
     constexpr size_t smem = (static_cast<size_t>(kStages) * BMv * (BK / 8) +
                              static_cast<size_t>(F::kDirect ? kStages : 2) * kTileVecs) * sizeof(u32x4_t);
@@ -318,7 +355,7 @@ int launch_gemm_mt(const GemmArgs& a, hipStream_t stream) {
         hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_mfma_kernel<Shape<F, MT>>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
     if (attr != hipSuccess) return PIE_HIP_ERR_LAUNCH;
-    const dim3 grid((a.N + BN - 1) / BN, (a.M + BMv - 1) / BMv);
+    const dim3 grid((a.N + BN - 1) / BN, (a.M + BMv - 1) / BMv, splits);
     if (grid.y > 65535) return PIE_HIP_ERR_UNSUPPORTED;
     hipLaunchKernelGGL((gemm_mfma_kernel<Shape<F, MT>>), grid, dim3(kThreads), smem, stream, a);
     return launch_status();
@@ -332,21 +369,51 @@ int launch_gemm_mt(const GemmArgs& a, hipStream_t stream) {
 template <class F>
 int launch_gemm(const GemmArgs& a, hipStream_t stream) {
     static const int forced = [] { const char* e = getenv("PIE_HIP_GEMM_MT"); return e ? atoi(e) : 0; }();
+    if (a.M <= 64 && !forced) return launch_gemm_mt<F, 2>(a, 1, stream);   // 64-row block tiles
     const long long nt = (a.N + BN - 1) / BN;
     const long long t4 = nt * ((a.M + 127) / 128), t8 = nt * ((a.M + 255) / 256);
     const double c4 = static_cast<double>((t4 + 255) / 256), c8 = 1.66 * static_cast<double>((t8 + 255) / 256);
     const bool tall = forced ? forced == 8 : (F::kDirect && a.M > 128 && c8 < c4);
-    return tall ? launch_gemm_mt<F, 8>(a, stream) : launch_gemm_mt<F, 4>(a, stream);
+    return tall ? launch_gemm_mt<F, 8>(a, 1, stream) : launch_gemm_mt<F, 4>(a, 1, stream);
+}
+
+// Few output tiles (M up to 128 rows of a decode batch): a block per (tile, K share) so that
+// the machine is full and each block's serial K loop is short; fp32 partials meet in a second
+// kernel.  Returns the number of K shares for a shape, 1 = not worth splitting.
+int splitk_shares(int M, int N, int K) {
+    if (M > 128) return 1;
+    const long long tiles = static_cast<long long>((N + BN - 1) / BN) * (M > 64 ? (M + 127) / 128 : 1);
+    const int nk_all = K / BK;
+    long long want = 1024 / tiles;
+    if (want > 16) want = 16;
+    if (want > nk_all / 4) want = nk_all / 4;
+    if (want < 2) return 1;
+    const int per = (nk_all + static_cast<int>(want) - 1) / static_cast<int>(want);
+    return (nk_all + per - 1) / per;   // every share non-empty
+}
+
+template <class F>
+int launch_gemm_splitk(GemmArgs a, int splits, float* ws, hipStream_t stream) {
+    const int beta = a.beta, swiglu = a.swiglu;
+    a.partial = ws;
+    a.beta = 0;
+    a.swiglu = 0;
+    const int st = a.M <= 64 ? launch_gemm_mt<F, 2>(a, splits, stream) : launch_gemm_mt<F, 4>(a, splits, stream);
+    if (st != PIE_HIP_OK) return st;
+    const size_t outs = static_cast<size_t>(a.M) * (swiglu ? a.N / 2 : a.N);
+    hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3(static_cast<unsigned>((outs + 255) / 256)), dim3(256), 0,
+                       stream, ws, a.y, a.M, a.N, splits, beta, swiglu);
+    return launch_status();
 }
 
 }  // namespace
 }  // namespace pie_hip
 
-extern "C" int pie_hip_gemm_mfma(int format, const uint16_t* act_bf16, const void* weight,
-                                 const void* scale, int scale_is_bf16, int group_size,
-                                 uint16_t* y_bf16, int M, int N, int K, int beta, int swiglu,
-                                 void* stream) {
-    using namespace pie_hip;
+namespace pie_hip {
+namespace {
+int gemm_entry(int format, const uint16_t* act_bf16, const void* weight, const void* scale,
+               int scale_is_bf16, int group_size, uint16_t* y_bf16, int M, int N, int K, int beta,
+               int swiglu, void* workspace, size_t workspace_bytes, void* stream) {
     if (!act_bf16 || !weight || !y_bf16 || M <= 0 || N <= 0 || K <= 0) return PIE_HIP_ERR_INVALID;
     if (format != PIE_HIP_FMT_BF16 && !scale) return PIE_HIP_ERR_INVALID;
     if (K % BK != 0) return PIE_HIP_ERR_UNSUPPORTED;
@@ -363,16 +430,53 @@ extern "C" int pie_hip_gemm_mfma(int format, const uint16_t* act_bf16, const voi
     a.swiglu = swiglu ? 1 : 0;
     a.scale_is_bf16 = scale_is_bf16;
     hipStream_t st = static_cast<hipStream_t>(stream);
+    if (format == PIE_HIP_FMT_INT4B8) {
+        // a 32-value run of one row must lie inside one scale group
+        if (group_size < 32 || (group_size & (group_size - 1)) != 0 || K % group_size != 0)
+            return PIE_HIP_ERR_UNSUPPORTED;
+        a.g_shift = __builtin_ctz(static_cast<unsigned>(group_size));
+    }
+    const int splits = workspace ? splitk_shares(M, N, K) : 1;
+    if (splits > 1) {
+        if (workspace_bytes < static_cast<size_t>(splits) * M * N * sizeof(float)) return PIE_HIP_ERR_INVALID;
+        float* ws = static_cast<float*>(workspace);
+        switch (format) {
+            case PIE_HIP_FMT_INT4B8: return launch_gemm_splitk<GInt4>(a, splits, ws, st);
+            case PIE_HIP_FMT_INT8: return launch_gemm_splitk<GInt8>(a, splits, ws, st);
+            case PIE_HIP_FMT_FP8: return launch_gemm_splitk<GFp8>(a, splits, ws, st);
+            case PIE_HIP_FMT_BF16: return launch_gemm_splitk<GBf16>(a, splits, ws, st);
+            default: return PIE_HIP_ERR_INVALID;
+        }
+    }
     switch (format) {
-        case PIE_HIP_FMT_INT4B8:
-            // a 32-value run of one row must lie inside one scale group
-            if (group_size < 32 || (group_size & (group_size - 1)) != 0 || K % group_size != 0)
-                return PIE_HIP_ERR_UNSUPPORTED;
-            a.g_shift = __builtin_ctz(static_cast<unsigned>(group_size));
-            return launch_gemm<GInt4>(a, st);
+        case PIE_HIP_FMT_INT4B8: return launch_gemm<GInt4>(a, st);
         case PIE_HIP_FMT_INT8: return launch_gemm<GInt8>(a, st);
         case PIE_HIP_FMT_FP8: return launch_gemm<GFp8>(a, st);
         case PIE_HIP_FMT_BF16: return launch_gemm<GBf16>(a, st);
         default: return PIE_HIP_ERR_INVALID;
     }
+}
+}  // namespace
+}  // namespace pie_hip
+
+extern "C" int pie_hip_gemm_mfma(int format, const uint16_t* act_bf16, const void* weight,
+                                 const void* scale, int scale_is_bf16, int group_size,
+                                 uint16_t* y_bf16, int M, int N, int K, int beta, int swiglu,
+                                 void* stream) {
+    return pie_hip::gemm_entry(format, act_bf16, weight, scale, scale_is_bf16, group_size, y_bf16, M, N,
+                               K, beta, swiglu, nullptr, 0, stream);
+}
+
+extern "C" size_t pie_hip_gemm_mfma_workspace_bytes(int M, int N, int K) {
+    if (M <= 0 || N <= 0 || K <= 0 || K % pie_hip::BK != 0) return 0;
+    const int splits = pie_hip::splitk_shares(M, N, K);
+    return splits > 1 ? static_cast<size_t>(splits) * M * N * sizeof(float) : 0;
+}
+
+extern "C" int pie_hip_gemm_mfma_splitk(int format, const uint16_t* act_bf16, const void* weight,
+                                        const void* scale, int scale_is_bf16, int group_size,
+                                        uint16_t* y_bf16, int M, int N, int K, int beta, int swiglu,
+                                        void* workspace, size_t workspace_bytes, void* stream) {
+    return pie_hip::gemm_entry(format, act_bf16, weight, scale, scale_is_bf16, group_size, y_bf16, M, N,
+                               K, beta, swiglu, workspace, workspace_bytes, stream);
 }

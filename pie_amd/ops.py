@@ -463,8 +463,11 @@ def moe_combine(y_routes: torch.Tensor, route_pos: torch.Tensor, topk_w: torch.T
 
 
 def gemm_mfma(act: torch.Tensor, w: WeightView, y: Optional[torch.Tensor] = None, beta: int = 0,
-              swiglu: bool = False) -> torch.Tensor:
-    """Tiled matrix-core GEMM for large M (weights dequantised to bf16 while staged)."""
+              swiglu: bool = False, split_k: bool = False,
+              workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Tiled matrix-core GEMM for large M (weights dequantised to bf16 while staged).
+    split_k: the decode-batch form (K shares + fp32 partials in `workspace`, allocated here
+    when not given)."""
     _dev(act, torch.bfloat16, "act")
     M, K = act.shape
     if K != w.K:
@@ -478,11 +481,31 @@ def gemm_mfma(act: torch.Tensor, w: WeightView, y: Optional[torch.Tensor] = None
     if tuple(y.shape) != (M, n_out):
         raise KernelError("y shape mismatch")
     scale_is_bf16 = int(w.scale is not None and w.scale.dtype == torch.bfloat16)
-    st = kernels().pie_hip_gemm_mfma(FMT[w.kind], _ptr(act), _ptr(w.data), _ptr(w.scale),
-                                     scale_is_bf16, w.group_size, _ptr(y), M, w.N, K, beta,
-                                     int(swiglu), _stream())
+    lib = kernels()
+    if split_k:
+        lib.pie_hip_gemm_mfma_workspace_bytes.restype = C.c_size_t
+        need = int(lib.pie_hip_gemm_mfma_workspace_bytes(M, w.N, K))
+        if need:
+            if workspace is None:
+                workspace = torch.empty(need, dtype=torch.uint8, device=act.device)
+            if workspace.numel() * workspace.element_size() < need:
+                raise KernelError("workspace too small")
+            st = lib.pie_hip_gemm_mfma_splitk(FMT[w.kind], _ptr(act), _ptr(w.data), _ptr(w.scale),
+                                              scale_is_bf16, w.group_size, _ptr(y), M, w.N, K, beta,
+                                              int(swiglu), _ptr(workspace), C.c_size_t(need), _stream())
+            _check(st, "pie_hip_gemm_mfma_splitk")
+            return y
+    st = lib.pie_hip_gemm_mfma(FMT[w.kind], _ptr(act), _ptr(w.data), _ptr(w.scale),
+                               scale_is_bf16, w.group_size, _ptr(y), M, w.N, K, beta,
+                               int(swiglu), _stream())
     _check(st, "pie_hip_gemm_mfma")
     return y
+
+
+def gemm_mfma_workspace_bytes(M: int, N: int, K: int) -> int:
+    lib = kernels()
+    lib.pie_hip_gemm_mfma_workspace_bytes.restype = C.c_size_t
+    return int(lib.pie_hip_gemm_mfma_workspace_bytes(M, N, K))
 
 
 def qkv_rope_fused(act: torch.Tensor, w: WeightView, table: torch.Tensor, kv_slots: torch.Tensor,
