@@ -376,6 +376,47 @@ int pie_hip_attn_rows_paged(const uint16_t* q, const uint16_t* k_pages, const ui
                             int page_size, float sm_scale, int max_kv_len, void* workspace,
                             size_t workspace_bytes, void* stream);
 
+/*
+ * KV-cache storage formats of the pool (the CUDA driver's kv_cache_dtype values,
+ * driver/cuda/src/kv_cache_format.cpp:46-110).  One-byte formats keep the bf16 layout
+ * [pages, page_size, hk, d] with one byte per element; the per-token-head formats add fp32 side
+ * scales [pages, page_size, hk] for K and for V.  fp8_e5m2 and the fp4 block formats are not
+ * implemented (PIE_HIP_ERR_UNSUPPORTED).
+ */
+enum {
+    PIE_HIP_KV_BF16 = 0,
+    PIE_HIP_KV_FP8_E4M3 = 1,             /* saturating cast of the value, no scales */
+    PIE_HIP_KV_INT8_PER_TOKEN_HEAD = 2,  /* scale = absmax/127, code = rint(x / scale) */
+    PIE_HIP_KV_FP8_PER_TOKEN_HEAD = 3    /* scale = absmax/448, code = e4m3(x / scale) */
+};
+
+/*
+ * pie_hip_attn_rows_paged over a pool in a one-byte format: every K / V element is
+ * float(code) * scale as load_kv_scalar reads it (driver/cuda/src/ops/attention_naive_paged.cu:56-112),
+ * everything else as for bf16 pools.  k_scales / v_scales: required for the per-token-head
+ * formats, NULL for PIE_HIP_KV_FP8_E4M3.  Custom masks are not available with these formats.
+ */
+int pie_hip_attn_rows_paged_kvq(int kv_format, const uint16_t* q, const void* k_pages,
+                                const void* v_pages, const float* k_scales, const float* v_scales,
+                                uint16_t* o, float* lse, const uint32_t* kv_page_indices,
+                                const uint32_t* row_page_begin, const int32_t* row_kv_len,
+                                int num_rows, int num_q_heads, int num_kv_heads, int head_dim,
+                                int page_size, float sm_scale, int max_kv_len, void* workspace,
+                                size_t workspace_bytes, void* stream);
+
+/*
+ * Quantising KV write: this step's K and V rows [num_tokens, hk, d] bf16 (after RoPE) go to
+ * slot kv_slots[t] of a one-byte pool (slot < 0: skipped).  Per-token-head formats:
+ * scale = absmax / qmax (qmax 127 / 448; 1 for an all-zero row), code = x * (1/scale) rounded
+ * to nearest even, clamped / saturated; PIE_HIP_KV_FP8_E4M3: the saturating cast of x.
+ * Reference: write_kv_per_token_head_kernel and write_kv_fp8_per_tensor_kernel,
+ * driver/cuda/src/kernels/kv_paged.cu:155-297.
+ */
+int pie_hip_kv_write_quant(int kv_format, const uint16_t* k_rows, const uint16_t* v_rows,
+                           const int64_t* kv_slots, void* k_pages, void* v_pages, float* k_scales,
+                           float* v_scales, int num_tokens, int num_kv_heads, int head_dim,
+                           void* stream);
+
 /* ---- per-layer kernels of the llama-like decoder ---------------------------- */
 
 /* y[n,:] = table[token_ids[n],:]; ids >= vocab read row 0.

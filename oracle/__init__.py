@@ -328,6 +328,41 @@ def brle_allow(runs, pos: int, n_kv: int, window: int = 0) -> np.ndarray:
     return out[:n_kv]
 
 
+KV_FORMATS = {"bf16": 0, "fp8_e4m3": 1, "int8_per_token_head": 2, "fp8_per_token_head": 3}
+
+
+def kv_quant_rows(x_bf16, fmt: str):
+    """KV-cache quantisation of (token, head) rows [rows, d] bf16
+    (driver/cuda/src/kernels/kv_paged.cu:155-297).  Returns (codes u8 [rows, d], scales f32 [rows]
+    or None for fp8_e4m3, dequantised f32 [rows, d] = float(code) * scale)."""
+    x = _c(x_bf16, np.uint16)
+    rows, d = x.shape
+    codes = np.zeros((rows, d), np.uint8)
+    scales = np.ones(rows, np.float32)
+    deq = np.zeros((rows, d), np.float32)
+    lib().orc_kv_quant_rows(_p(x), _p(codes), _p(scales), _p(deq), C.c_int(rows), C.c_int(d),
+                            C.c_int(KV_FORMATS[fmt]))
+    return codes, (None if fmt == "fp8_e4m3" else scales), deq
+
+
+def attn_rows_f32kv(q_bf16, k_pages_f32, v_pages_f32, page_indices, row_begin, row_len, hq, hk, d, ps,
+                    sm_scale=-1.0, mode=2):
+    """attn_rows over pools of dequantised f32 K / V values (one-byte KV-cache formats)."""
+    q = _c(q_bf16, np.uint16)
+    rows = q.shape[0]
+    kp, vp_ = _c(k_pages_f32, np.float32), _c(v_pages_f32, np.float32)
+    pi = _c(np.asarray(page_indices, np.uint32), np.uint32)
+    rb = _c(np.asarray(row_begin, np.uint32), np.uint32)
+    rl = _c(np.asarray(row_len, np.int32), np.int32)
+    o32 = np.zeros((rows, hq, d), np.float32)
+    o16 = np.zeros((rows, hq, d), np.uint16)
+    lse = np.zeros((rows, hq), np.float32)
+    lib().orc_attn_rows_f32kv(_p(q), _p(kp), _p(vp_), _p(o32), _p(o16), _p(lse), _p(pi), _p(rb), _p(rl),
+                              C.c_int(rows), C.c_int(hq), C.c_int(hk), C.c_int(d), C.c_int(ps),
+                              C.c_float(sm_scale), C.c_int(mode), None, None)
+    return o32, o16, lse
+
+
 def attn_rows_masked(q_bf16, k_pages, v_pages, page_indices, row_begin, row_len, hq, hk, d, ps,
                      allow_rows, sm_scale=-1.0, mode=2):
     """Per-row extents with per-row visibility: allow_rows[r] is None or a uint8 array over the

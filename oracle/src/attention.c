@@ -45,7 +45,13 @@ static int orc_kv_len(const uint32_t* indptr, const uint32_t* last_lens, int r, 
  * page_indices[pg_lo].  mode 0: fp32 two-pass softmax in the reference's order
  * (attention_naive_paged.cu:362-447); mode 2: fp64.
  */
-static void orc_attn_row(const uint16_t* q_row, const uint16_t* k_pages, const uint16_t* v_pages,
+/* K / V element: bf16 pool, or (kv_f32) a pool of already dequantised f32 values — the
+ * float(code) * scale of load_kv_scalar, attention_naive_paged.cu:56-112 */
+static inline float orc_kv_at(const void* pages, int kv_f32, size_t idx) {
+    return kv_f32 ? ((const float*)pages)[idx] : orc_bf16_to_f32(((const uint16_t*)pages)[idx]);
+}
+
+static void orc_attn_row(const uint16_t* q_row, const void* k_pages, const void* v_pages, int kv_f32,
                          float* o_f32, uint16_t* o_bf16, float* lse, const uint32_t* page_indices,
                          uint32_t pg_lo, int lim, int hq, int hk, int d, int ps, float scale,
                          int mode, double* w, const uint8_t* allow) {
@@ -61,13 +67,13 @@ static void orc_attn_row(const uint16_t* q_row, const uint16_t* k_pages, const u
             if (mode == 0) {
                 float f = 0.f;
                 for (int e = 0; e < d; ++e)
-                    f += orc_bf16_to_f32(q_row[qoff + e]) * orc_bf16_to_f32(k_pages[koff + e]);
+                    f += orc_bf16_to_f32(q_row[qoff + e]) * orc_kv_at(k_pages, kv_f32, koff + e);
                 dot = (double)(f * scale);
             } else {
                 double f = 0.0;
                 for (int e = 0; e < d; ++e)
                     f += (double)orc_bf16_to_f32(q_row[qoff + e]) *
-                         (double)orc_bf16_to_f32(k_pages[koff + e]);
+                         (double)orc_kv_at(k_pages, kv_f32, koff + e);
                 dot = f * (double)scale;
             }
             if (allow && !allow[j]) dot = -INFINITY;
@@ -101,7 +107,7 @@ static void orc_attn_row(const uint16_t* q_row, const uint16_t* k_pages, const u
             for (int j = 0; j < lim; ++j) {
                 const uint32_t pid = page_indices[pg_lo + j / ps];
                 const size_t voff = (((size_t)pid * ps + j % ps) * hk + kvh) * d;
-                const float v = orc_bf16_to_f32(v_pages[voff + e]);
+                const float v = orc_kv_at(v_pages, kv_f32, voff + e);
                 if (mode == 0) accf = fmaf(v, (float)w[j], accf);
                 else acc += (double)v * w[j];
             }
@@ -138,7 +144,7 @@ void orc_attn_paged(const uint16_t* q, const uint16_t* k_pages, const uint16_t* 
             if (lim > kv_total) lim = kv_total;
             if (lim < 0) lim = 0;
             const size_t row = (size_t)(q_lo + qi) * hq;
-            orc_attn_row(q + row * d, k_pages, v_pages, o_f32 + row * d,
+            orc_attn_row(q + row * d, k_pages, v_pages, 0, o_f32 + row * d,
                          o_bf16 ? o_bf16 + row * d : NULL, lse ? lse + row : NULL, page_indices,
                          page_indptr[r], lim, hq, hk, d, ps, scale, mode, w, NULL);
         }
@@ -172,7 +178,7 @@ void orc_attn_rows_masked(const uint16_t* q, const uint16_t* k_pages, const uint
         const int lim = row_len[r] > 0 ? row_len[r] : 0;
         double* w = (double*)malloc(sizeof(double) * (size_t)(lim > 0 ? lim : 1));
         const size_t row = (size_t)r * hq;
-        orc_attn_row(q + row * d, k_pages, v_pages, o_f32 + row * d,
+        orc_attn_row(q + row * d, k_pages, v_pages, 0, o_f32 + row * d,
                      o_bf16 ? o_bf16 + row * d : NULL, lse ? lse + row : NULL, page_indices,
                      row_begin[r], lim, hq, hk, d, ps, scale, mode, w,
                      (allow && allow_off && allow_off[r] >= 0) ? allow + allow_off[r] : NULL);
@@ -223,6 +229,68 @@ void orc_kv_write(const uint16_t* k_curr, const uint16_t* v_curr, uint16_t* k_pa
             const size_t dst = ((size_t)pid * ps + abs_pos % ps) * row;
             memcpy(k_pages + dst, k_curr + (size_t)(q_lo + i) * row, row * 2);
             memcpy(v_pages + dst, v_curr + (size_t)(q_lo + i) * row, row * 2);
+        }
+    }
+}
+
+
+/* orc_attn_rows_masked over pools of dequantised f32 values (one-byte KV-cache formats). */
+void orc_attn_rows_f32kv(const uint16_t* q, const float* k_pages, const float* v_pages,
+                         float* o_f32, uint16_t* o_bf16, float* lse, const uint32_t* page_indices,
+                         const uint32_t* row_begin, const int32_t* row_len, int rows, int hq,
+                         int hk, int d, int ps, float sm_scale, int mode, const uint8_t* allow,
+                         const int64_t* allow_off) {
+    const float scale = sm_scale > 0.f ? sm_scale : 1.0f / sqrtf((float)d);
+#pragma omp parallel for schedule(dynamic)
+    for (int r = 0; r < rows; ++r) {
+        const int lim = row_len[r] > 0 ? row_len[r] : 0;
+        double* w = (double*)malloc(sizeof(double) * (size_t)(lim > 0 ? lim : 1));
+        const size_t row = (size_t)r * hq;
+        orc_attn_row(q + row * d, k_pages, v_pages, 1, o_f32 + row * d,
+                     o_bf16 ? o_bf16 + row * d : NULL, lse ? lse + row : NULL, page_indices,
+                     row_begin[r], lim, hq, hk, d, ps, scale, mode, w,
+                     (allow && allow_off && allow_off[r] >= 0) ? allow + allow_off[r] : NULL);
+        free(w);
+    }
+}
+
+/*
+ * KV-cache quantisation of `rows` (token, head) rows of d bf16 values
+ * (driver/cuda/src/kernels/kv_paged.cu:155-297).
+ *   fmt 1 (fp8_e4m3):            code = e4m3_satfinite(x); scales untouched
+ *   fmt 2 (int8_per_token_head): scale = absmax/127 (1 when absmax == 0), inv = 1/scale,
+ *                                code = clamp(rintf(x * inv), -128, 127)
+ *   fmt 3 (fp8_per_token_head):  scale = absmax/448 (1 when 0), code = e4m3_satfinite(x * inv)
+ * dequant (optional, f32): float(code) * scale, as the attention kernels read it.
+ */
+uint8_t orc_f32_to_fp8_e4m3(float f);
+float orc_fp8_e4m3_to_f32(uint8_t v);
+void orc_kv_quant_rows(const uint16_t* x, uint8_t* codes, float* scales, float* dequant, int rows,
+                       int d, int fmt) {
+    for (int r = 0; r < rows; ++r) {
+        const uint16_t* src = x + (size_t)r * d;
+        float scale = 1.f, inv = 1.f;
+        if (fmt != 1) {
+            float amax = 0.f;
+            for (int j = 0; j < d; ++j) amax = fmaxf(amax, fabsf(orc_bf16_to_f32(src[j])));
+            scale = amax > 0.f ? amax / (fmt == 2 ? 127.f : 448.f) : 1.f;
+            inv = 1.f / scale;
+            if (scales) scales[r] = scale;
+        }
+        for (int j = 0; j < d; ++j) {
+            const float f = orc_bf16_to_f32(src[j]) * inv;
+            float val;
+            if (fmt == 2) {
+                int qv = (int)rintf(f);
+                qv = qv > 127 ? 127 : (qv < -128 ? -128 : qv);
+                codes[(size_t)r * d + j] = (uint8_t)(int8_t)qv;
+                val = (float)qv;
+            } else {
+                const uint8_t c = orc_f32_to_fp8_e4m3(f);
+                codes[(size_t)r * d + j] = c;
+                val = orc_fp8_e4m3_to_f32(c);
+            }
+            if (dequant) dequant[(size_t)r * d + j] = val * scale;
         }
     }
 }

@@ -65,13 +65,68 @@ __device__ __forceinline__ RowExtent row_extent(const uint32_t* __restrict__ pag
     return {lo, npages > 0 ? (npages - 1) * ps + static_cast<int>(last_lens[r]) : 0};
 }
 
-template <int D, int GQA>
+// KV storage of the pool (driver/cuda/src/kv_cache_format.hpp:11-17): bf16; one-byte e4m3 with
+// optional fp32 scales per (token, kv head) — "fp8_e4m3" stores casts, "fp8_per_token_head"
+// stores x / scale; int8 with such scales.  A lane still owns 8 elements of a row: 16 bytes of
+// bf16 or 8 bytes of a one-byte format.  Values are decoded as the reference's load_kv_scalar
+// does (driver/cuda/src/ops/attention_naive_paged.cu:56-112): float(code) * scale.
+constexpr int kKvBf16 = 0, kKvFp8 = 1, kKvInt8 = 2;
+
+template <int KVF>
+struct KvVec {
+    using type = u32x4_t;
+};
+template <>
+struct KvVec<kKvFp8> {
+    using type = u32x2_t;
+};
+template <>
+struct KvVec<kKvInt8> {
+    using type = u32x2_t;
+};
+
+__device__ __forceinline__ uint32_t kv_pack_trunc(float lo, float hi) {
+    return __builtin_amdgcn_perm(__float_as_uint(hi), __float_as_uint(lo), 0x07060302u);
+}
+// 8 stored elements -> 8 floats / 4 bf16 pairs (every code is exact in bf16)
+template <int KVF>
+__device__ __forceinline__ void kv_decode_f32(const typename KvVec<KVF>::type r, float* f) {
+    if constexpr (KVF == kKvBf16) {
+        f[0] = bf16_lo(r.x); f[1] = bf16_hi(r.x); f[2] = bf16_lo(r.y); f[3] = bf16_hi(r.y);
+        f[4] = bf16_lo(r.z); f[5] = bf16_hi(r.z); f[6] = bf16_lo(r.w); f[7] = bf16_hi(r.w);
+    } else if constexpr (KVF == kKvFp8) {
+        typedef float f32x2_t __attribute__((ext_vector_type(2)));
+        const f32x2_t a = __builtin_amdgcn_cvt_pk_f32_fp8(r.x, false), b = __builtin_amdgcn_cvt_pk_f32_fp8(r.x, true);
+        const f32x2_t c = __builtin_amdgcn_cvt_pk_f32_fp8(r.y, false), d = __builtin_amdgcn_cvt_pk_f32_fp8(r.y, true);
+        f[0] = a.x; f[1] = a.y; f[2] = b.x; f[3] = b.y; f[4] = c.x; f[5] = c.y; f[6] = d.x; f[7] = d.y;
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            f[e] = static_cast<float>(static_cast<int8_t>(r.x >> (8 * e)));
+            f[4 + e] = static_cast<float>(static_cast<int8_t>(r.y >> (8 * e)));
+        }
+    }
+}
+template <int KVF>
+__device__ __forceinline__ u32x4_t kv_decode_bf16(const typename KvVec<KVF>::type r) {
+    if constexpr (KVF == kKvBf16) {
+        return r;
+    } else {
+        float f[8];
+        kv_decode_f32<KVF>(r, f);
+        return u32x4_t{kv_pack_trunc(f[0], f[1]), kv_pack_trunc(f[2], f[3]), kv_pack_trunc(f[4], f[5]),
+                       kv_pack_trunc(f[6], f[7])};
+    }
+}
+
+template <int D, int GQA, int KVF = kKvBf16>
 struct UnitRegs {
     static constexpr int LPR = D / 8;
     static constexpr int TPI = kWave / LPR;          // tokens per load instruction
     static constexpr int IPU = kUnitTokens / TPI;    // load instructions per unit
-    u32x4_t k[IPU];
-    u32x4_t v[IPU];
+    typename KvVec<KVF>::type k[IPU];
+    typename KvVec<KVF>::type v[IPU];
+    float ks[IPU], vs[IPU];   // one-byte formats: the (token, kv head) scales
     uint32_t mask;   // MASKED kernels: bit t = token t of the unit is visible
 };
 
@@ -79,17 +134,22 @@ struct UnitRegs {
 // both in units where scores were multiplied by scale*log2(e).
 // MASKED: mask_bits [rows, mask_stride] u16, one word per 16-token unit (custom attention
 // masks); hidden tokens are dropped like the slots past the context.
-template <int D, int GQA, bool MASKED>
+template <int D, int GQA, bool MASKED, int KVF = kKvBf16>
 __global__ __launch_bounds__(kAttnBlock) void attn_decode_split_kernel(
-    const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_pages,
-    const uint16_t* __restrict__ v_pages, const uint32_t* __restrict__ page_indices,
+    const uint16_t* __restrict__ q, const void* __restrict__ k_pages_raw,
+    const void* __restrict__ v_pages_raw, const float* __restrict__ k_scales,
+    const float* __restrict__ v_scales, const uint32_t* __restrict__ page_indices,
     const uint32_t* __restrict__ page_indptr, const uint32_t* __restrict__ last_lens,
     const uint32_t* __restrict__ row_begin, const int32_t* __restrict__ row_len,
     float* __restrict__ part_o, float* __restrict__ part_ml, uint16_t* __restrict__ o_direct,
     float* __restrict__ lse, const uint16_t* __restrict__ mask_bits, int mask_stride, int hq,
     int hk, int ps, int units_per_split, int nsplit, float scale_log2e) {
-    using U = UnitRegs<D, GQA>;
+    using U = UnitRegs<D, GQA, KVF>;
+    using KV = typename KvVec<KVF>::type;
     constexpr int LPR = U::LPR, TPI = U::TPI, IPU = U::IPU;
+    constexpr int kElemBytes = KVF == kKvBf16 ? 2 : 1;
+    const unsigned char* k_pages = static_cast<const unsigned char*>(k_pages_raw);
+    const unsigned char* v_pages = static_cast<const unsigned char*>(v_pages_raw);
     const int kvh = blockIdx.x, split = blockIdx.y, r = blockIdx.z;  // kv heads of the same tokens are dispatched together
     const int tid = threadIdx.x, lane = tid & (kWave - 1);
     const int wv = __builtin_amdgcn_readfirstlane(tid / kWave);  // wave-uniform -> SGPR
@@ -115,13 +175,18 @@ __global__ __launch_bounds__(kAttnBlock) void attn_decode_split_kernel(
         const int tok0 = unit * kUnitTokens;
         const int page = tok0 / ps;
         const uint32_t pid = page_indices[pg_lo + page];
-        const size_t base =
-            ((static_cast<size_t>(pid) * ps + (tok0 - page * ps)) * hk + kvh) * D + dl * 8;
+        const size_t slot0 = static_cast<size_t>(pid) * ps + (tok0 - page * ps);
+        const size_t base = (slot0 * hk + kvh) * D + dl * 8;
 #pragma unroll
         for (int i = 0; i < IPU; ++i) {
-            const size_t off = base + static_cast<size_t>(i * TPI + grp) * row_stride;
-            u.k[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(k_pages + off));
-            u.v[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(v_pages + off));
+            const size_t off = (base + static_cast<size_t>(i * TPI + grp) * row_stride) * kElemBytes;
+            u.k[i] = __builtin_nontemporal_load(reinterpret_cast<const KV*>(k_pages + off));
+            u.v[i] = __builtin_nontemporal_load(reinterpret_cast<const KV*>(v_pages + off));
+            if constexpr (KVF != kKvBf16) {
+                const size_t th = (slot0 + i * TPI + grp) * hk + kvh;
+                u.ks[i] = k_scales ? k_scales[th] : 1.f;
+                u.vs[i] = v_scales ? v_scales[th] : 1.f;
+            }
         }
         if (MASKED) u.mask = mask_bits[static_cast<size_t>(r) * mask_stride + unit];
     };
@@ -140,14 +205,16 @@ __global__ __launch_bounds__(kAttnBlock) void attn_decode_split_kernel(
         float s[IPU][GQA];
 #pragma unroll
         for (int i = 0; i < IPU; ++i) {
+            const u32x4_t kb = kv_decode_bf16<KVF>(u.k[i]);
+            const float sc = KVF == kKvBf16 ? scale_log2e : scale_log2e * u.ks[i];
 #pragma unroll
             for (int h = 0; h < GQA; ++h) {
                 float p = 0.f;
-                p = dot2_bf16(u.k[i].x, qv[h].x, p);
-                p = dot2_bf16(u.k[i].y, qv[h].y, p);
-                p = dot2_bf16(u.k[i].z, qv[h].z, p);
-                p = dot2_bf16(u.k[i].w, qv[h].w, p);
-                s[i][h] = token_lanes_sum<LPR>(p) * scale_log2e;
+                p = dot2_bf16(kb.x, qv[h].x, p);
+                p = dot2_bf16(kb.y, qv[h].y, p);
+                p = dot2_bf16(kb.z, qv[h].z, p);
+                p = dot2_bf16(kb.w, qv[h].w, p);
+                s[i][h] = token_lanes_sum<LPR>(p) * sc;
             }
         }
         if (tok0 + kUnitTokens > kv_len) {  // tail unit: drop slots past the context
@@ -156,7 +223,8 @@ __global__ __launch_bounds__(kAttnBlock) void attn_decode_split_kernel(
                 if (tok0 + i * TPI + grp >= kv_len) {
 #pragma unroll
                     for (int h = 0; h < GQA; ++h) s[i][h] = -INFINITY;
-                    u.v[i] = u32x4_t{0u, 0u, 0u, 0u};
+                    u.v[i] = KV{};
+                    u.vs[i] = 0.f;
                 }
             }
         }
@@ -166,7 +234,8 @@ __global__ __launch_bounds__(kAttnBlock) void attn_decode_split_kernel(
                 if (!((u.mask >> (i * TPI + grp)) & 1u)) {
 #pragma unroll
                     for (int h = 0; h < GQA; ++h) s[i][h] = -INFINITY;
-                    u.v[i] = u32x4_t{0u, 0u, 0u, 0u};
+                    u.v[i] = KV{};
+                    u.vs[i] = 0.f;
                 }
             }
         }
@@ -198,14 +267,13 @@ __global__ __launch_bounds__(kAttnBlock) void attn_decode_split_kernel(
 #pragma unroll
         for (int i = 0; i < IPU; ++i) {
             float vf[8];
-            vf[0] = bf16_lo(u.v[i].x); vf[1] = bf16_hi(u.v[i].x);
-            vf[2] = bf16_lo(u.v[i].y); vf[3] = bf16_hi(u.v[i].y);
-            vf[4] = bf16_lo(u.v[i].z); vf[5] = bf16_hi(u.v[i].z);
-            vf[6] = bf16_lo(u.v[i].w); vf[7] = bf16_hi(u.v[i].w);
+            kv_decode_f32<KVF>(u.v[i], vf);
 #pragma unroll
-            for (int h = 0; h < GQA; ++h)
+            for (int h = 0; h < GQA; ++h) {
+                const float pw = KVF == kKvBf16 ? s[i][h] : s[i][h] * u.vs[i];
 #pragma unroll
-                for (int e = 0; e < 8; ++e) o[h][e] = fmaf(s[i][h], vf[e], o[h][e]);
+                for (int e = 0; e < 8; ++e) o[h][e] = fmaf(pw, vf[e], o[h][e]);
+            }
         }
     };
 
@@ -395,9 +463,9 @@ SplitPlan plan_splits(int R, int hk, int max_kv_len) {
     return {static_cast<int>(ups), nsplit};
 }
 
-template <int D, int GQA, bool MASKED>
-int launch_decode(const uint16_t* q, const uint16_t* k_pages, const uint16_t* v_pages, uint16_t* o,
-                  float* lse, const uint32_t* page_indices, const uint32_t* page_indptr,
+template <int D, int GQA, bool MASKED, int KVF = kKvBf16>
+int launch_decode(const uint16_t* q, const void* k_pages, const void* v_pages,
+                  const float* k_scales, const float* v_scales, uint16_t* o, float* lse, const uint32_t* page_indices, const uint32_t* page_indptr,
                   const uint32_t* last_lens, const uint32_t* row_begin, const int32_t* row_len,
                   int R, int hq, int hk, int ps, float sm_scale,
                   int max_kv_len, void* workspace, size_t workspace_bytes, const uint16_t* mask_bits,
@@ -407,8 +475,8 @@ int launch_decode(const uint16_t* q, const uint16_t* k_pages, const uint16_t* v_
     if (plan.nsplit == 1) {
         hipLaunchKernelGGL((attn_decode_clear_empty_kernel<D>), dim3(R * hq), dim3(D), 0, stream,
                            page_indptr, last_lens, row_begin, row_len, o, lse, hq, ps);
-        hipLaunchKernelGGL((attn_decode_split_kernel<D, GQA, MASKED>), dim3(hk, 1, R),
-                           dim3(kAttnBlock), 0, stream, q, k_pages, v_pages, page_indices,
+        hipLaunchKernelGGL((attn_decode_split_kernel<D, GQA, MASKED, KVF>), dim3(hk, 1, R),
+                           dim3(kAttnBlock), 0, stream, q, k_pages, v_pages, k_scales, v_scales, page_indices,
                            page_indptr, last_lens, row_begin, row_len, nullptr, nullptr, o, lse,
                            mask_bits, mask_stride, hq, hk, ps, plan.units_per_split, 1, scale_log2e);
         return launch_status();
@@ -418,8 +486,8 @@ int launch_decode(const uint16_t* q, const uint16_t* k_pages, const uint16_t* v_
     if (!workspace || workspace_bytes < need) return PIE_HIP_ERR_INVALID;
     float* part_o = static_cast<float*>(workspace);
     float* part_ml = part_o + n_part * D;
-    hipLaunchKernelGGL((attn_decode_split_kernel<D, GQA, MASKED>), dim3(hk, plan.nsplit, R),
-                       dim3(kAttnBlock), 0, stream, q, k_pages, v_pages, page_indices, page_indptr,
+    hipLaunchKernelGGL((attn_decode_split_kernel<D, GQA, MASKED, KVF>), dim3(hk, plan.nsplit, R),
+                       dim3(kAttnBlock), 0, stream, q, k_pages, v_pages, k_scales, v_scales, page_indices, page_indptr,
                        last_lens, row_begin, row_len, part_o, part_ml, nullptr, nullptr, mask_bits,
                        mask_stride, hq, hk, ps, plan.units_per_split, plan.nsplit, scale_log2e);
     hipLaunchKernelGGL((attn_decode_merge_kernel<D>), dim3(R * hq), dim3(D), 0, stream, part_o,
@@ -444,13 +512,14 @@ extern "C" size_t pie_hip_attn_decode_workspace_bytes(int num_requests, int num_
 
 namespace pie_hip {
 namespace {
-int attn_dispatch(const uint16_t* q, const uint16_t* k_pages, const uint16_t* v_pages, uint16_t* o,
+int attn_dispatch(const uint16_t* q, const void* k_pages, const void* v_pages, uint16_t* o,
                   float* lse, const uint32_t* kv_page_indices, const uint32_t* kv_page_indptr,
                   const uint32_t* kv_last_page_lens, const uint32_t* row_begin,
                   const int32_t* row_len, int num_rows, int num_q_heads, int num_kv_heads,
                   int head_dim, int page_size, float sm_scale, int max_kv_len, void* workspace,
                   size_t workspace_bytes, void* stream, const uint16_t* mask_bits = nullptr,
-                  int mask_stride = 0) {
+                  int mask_stride = 0, int kv_format = PIE_HIP_KV_BF16, const float* k_scales = nullptr,
+                  const float* v_scales = nullptr) {
     if (mask_bits && mask_stride < (max_kv_len + kUnitTokens - 1) / kUnitTokens) return PIE_HIP_ERR_INVALID;
     if (!q || !k_pages || !v_pages || !o || !kv_page_indices || num_rows <= 0 ||
         num_q_heads <= 0 || num_kv_heads <= 0 || page_size <= 0 || max_kv_len < 0)
@@ -461,15 +530,36 @@ int attn_dispatch(const uint16_t* q, const uint16_t* k_pages, const uint16_t* v_
     const float scale = sm_scale > 0.f ? sm_scale : 1.0f / sqrtf(static_cast<float>(head_dim));
     const int gqa = num_q_heads / num_kv_heads;
     hipStream_t st = static_cast<hipStream_t>(stream);
+    // one-byte KV formats: plain rows only (no custom-mask instantiation), per-(token, head)
+    // scales required for int8 and the scaled fp8 form, absent for plain fp8 casts
+    if (kv_format != PIE_HIP_KV_BF16) {
+        if (mask_bits) return PIE_HIP_ERR_UNSUPPORTED;
+        const bool scaled = kv_format == PIE_HIP_KV_INT8_PER_TOKEN_HEAD || kv_format == PIE_HIP_KV_FP8_PER_TOKEN_HEAD;
+        if (kv_format != PIE_HIP_KV_FP8_E4M3 && !scaled) return PIE_HIP_ERR_UNSUPPORTED;
+        if (scaled != (k_scales != nullptr) || scaled != (v_scales != nullptr)) return PIE_HIP_ERR_INVALID;
+    }
 #define PIE_ATTN_CASE(DD, GG)                                                                  \
     if (head_dim == DD && gqa == GG) {                                                         \
+        if (kv_format == PIE_HIP_KV_INT8_PER_TOKEN_HEAD)                                       \
+            return launch_decode<DD, GG, false, kKvInt8>(                                      \
+                q, k_pages, v_pages, k_scales, v_scales, o, lse, kv_page_indices,              \
+                kv_page_indptr, kv_last_page_lens, row_begin, row_len, num_rows, num_q_heads,  \
+                num_kv_heads, page_size, scale, max_kv_len, workspace, workspace_bytes,        \
+                nullptr, 0, st);                                                               \
+        if (kv_format != PIE_HIP_KV_BF16)                                                      \
+            return launch_decode<DD, GG, false, kKvFp8>(                                       \
+                q, k_pages, v_pages, k_scales, v_scales, o, lse, kv_page_indices,              \
+                kv_page_indptr, kv_last_page_lens, row_begin, row_len, num_rows, num_q_heads,  \
+                num_kv_heads, page_size, scale, max_kv_len, workspace, workspace_bytes,        \
+                nullptr, 0, st);                                                               \
         if (mask_bits)                                                                         \
             return launch_decode<DD, GG, true>(                                                \
-                q, k_pages, v_pages, o, lse, kv_page_indices, kv_page_indptr,                  \
+                q, k_pages, v_pages, nullptr, nullptr, o, lse, kv_page_indices, kv_page_indptr, \
                 kv_last_page_lens, row_begin, row_len, num_rows, num_q_heads, num_kv_heads,    \
                 page_size, scale, max_kv_len, workspace, workspace_bytes, mask_bits,           \
                 mask_stride, st);                                                              \
-        return launch_decode<DD, GG, false>(q, k_pages, v_pages, o, lse, kv_page_indices,      \
+        return launch_decode<DD, GG, false>(q, k_pages, v_pages, nullptr, nullptr, o, lse,     \
+                                            kv_page_indices,                                   \
                                             kv_page_indptr, kv_last_page_lens, row_begin,      \
                                             row_len, num_rows, num_q_heads, num_kv_heads,      \
                                             page_size, scale, max_kv_len, workspace,           \
@@ -517,6 +607,96 @@ extern "C" int pie_hip_attn_rows_paged(const uint16_t* q, const uint16_t* k_page
                                   row_page_begin, row_kv_len, num_rows, num_q_heads, num_kv_heads,
                                   head_dim, page_size, sm_scale, max_kv_len, workspace,
                                   workspace_bytes, stream);
+}
+
+extern "C" int pie_hip_attn_rows_paged_kvq(int kv_format, const uint16_t* q, const void* k_pages,
+                                           const void* v_pages, const float* k_scales,
+                                           const float* v_scales, uint16_t* o, float* lse,
+                                           const uint32_t* kv_page_indices,
+                                           const uint32_t* row_page_begin,
+                                           const int32_t* row_kv_len, int num_rows,
+                                           int num_q_heads, int num_kv_heads, int head_dim,
+                                           int page_size, float sm_scale, int max_kv_len,
+                                           void* workspace, size_t workspace_bytes, void* stream) {
+    if (!row_page_begin || !row_kv_len) return PIE_HIP_ERR_INVALID;
+    return pie_hip::attn_dispatch(q, k_pages, v_pages, o, lse, kv_page_indices, nullptr, nullptr,
+                                  row_page_begin, row_kv_len, num_rows, num_q_heads, num_kv_heads,
+                                  head_dim, page_size, sm_scale, max_kv_len, workspace,
+                                  workspace_bytes, stream, nullptr, 0, kv_format, k_scales, v_scales);
+}
+
+namespace pie_hip {
+namespace {
+
+// Writes this step's K / V rows [N, hk, d] bf16 into a one-byte pool at the tokens' slots:
+// one wave per (token, kv head).  Per-(token, head) formats: scale = absmax / qmax (1 for an
+// all-zero row), code = x * (1 / scale) rounded to nearest even and clamped (int8: [-128, 127];
+// e4m3: saturating at 448); plain fp8: the saturating cast of x itself.  The arithmetic of
+// write_kv_per_token_head_kernel / write_kv_fp8_per_tensor_kernel,
+// driver/cuda/src/kernels/kv_paged.cu:155-297.
+__global__ __launch_bounds__(256) void kv_write_quant_kernel(
+    const uint16_t* __restrict__ k_src, const uint16_t* __restrict__ v_src,
+    const int64_t* __restrict__ kv_slots, unsigned char* __restrict__ k_pages,
+    unsigned char* __restrict__ v_pages, float* __restrict__ k_scales,
+    float* __restrict__ v_scales, int n_rows, int hk, int d, int kv_format) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int row = blockIdx.x * (256 / kWave) + threadIdx.x / kWave;   // (token, head)
+    if (row >= n_rows) return;
+    const int t = row / hk, h = row - t * hk;
+    const int64_t slot = kv_slots[t];
+    if (slot < 0) return;
+    const size_t src = static_cast<size_t>(row) * d;
+    const size_t th = static_cast<size_t>(slot) * hk + h;
+    const bool scaled = kv_format != PIE_HIP_KV_FP8_E4M3;
+    const float qmax = kv_format == PIE_HIP_KV_INT8_PER_TOKEN_HEAD ? 127.f : 448.f;
+#pragma unroll
+    for (int which = 0; which < 2; ++which) {
+        const uint16_t* x = which ? v_src : k_src;
+        unsigned char* dst = (which ? v_pages : k_pages) + th * d;
+        float inv = 1.f;
+        if (scaled) {
+            float amax = 0.f;
+            for (int j = lane; j < d; j += kWave) amax = fmaxf(amax, fabsf(bf16_bits_to_f32(x[src + j])));
+            amax = wave_max(amax);
+            const float scale = amax > 0.f ? amax / qmax : 1.f;
+            inv = 1.f / scale;
+            if (lane == 0) (which ? v_scales : k_scales)[th] = scale;
+        }
+        for (int j = lane; j < d; j += kWave) {
+            const float f = bf16_bits_to_f32(x[src + j]) * inv;
+            if (kv_format == PIE_HIP_KV_INT8_PER_TOKEN_HEAD) {
+                int qv = static_cast<int>(rintf(f));
+                qv = qv > 127 ? 127 : (qv < -128 ? -128 : qv);
+                dst[j] = static_cast<unsigned char>(static_cast<int8_t>(qv));
+            } else {
+                const float c = fminf(fmaxf(f, -448.f), 448.f);
+                dst[j] = static_cast<unsigned char>(__builtin_amdgcn_cvt_pk_fp8_f32(c, c, 0, false) & 0xFF);
+            }
+        }
+    }
+}
+
+}  // namespace
+}  // namespace pie_hip
+
+extern "C" int pie_hip_kv_write_quant(int kv_format, const uint16_t* k_rows, const uint16_t* v_rows,
+                                      const int64_t* kv_slots, void* k_pages, void* v_pages,
+                                      float* k_scales, float* v_scales, int num_tokens,
+                                      int num_kv_heads, int head_dim, void* stream) {
+    using namespace pie_hip;
+    if (!k_rows || !v_rows || !kv_slots || !k_pages || !v_pages || num_tokens < 0 || num_kv_heads <= 0 ||
+        head_dim <= 0)
+        return PIE_HIP_ERR_INVALID;
+    const bool scaled = kv_format == PIE_HIP_KV_INT8_PER_TOKEN_HEAD || kv_format == PIE_HIP_KV_FP8_PER_TOKEN_HEAD;
+    if (kv_format != PIE_HIP_KV_FP8_E4M3 && !scaled) return PIE_HIP_ERR_UNSUPPORTED;
+    if (scaled && (!k_scales || !v_scales)) return PIE_HIP_ERR_INVALID;
+    if (num_tokens == 0) return PIE_HIP_OK;
+    const int rows = num_tokens * num_kv_heads;
+    hipLaunchKernelGGL(kv_write_quant_kernel, dim3((rows + 3) / 4), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), k_rows, v_rows, kv_slots,
+                       static_cast<unsigned char*>(k_pages), static_cast<unsigned char*>(v_pages), k_scales,
+                       v_scales, rows, num_kv_heads, head_dim, kv_format);
+    return launch_status();
 }
 
 namespace pie_hip {

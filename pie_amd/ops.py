@@ -697,3 +697,68 @@ def attention_prefill_tiles(q: torch.Tensor, k_pages: torch.Tensor, v_pages: tor
                                               ps, C.c_float(-1.0), _stream())
     _check(st, "pie_hip_attn_prefill_tiles")
     return o
+
+
+KV_FORMATS = {"bf16": 0, "fp8_e4m3": 1, "int8_per_token_head": 2, "fp8_per_token_head": 3}
+
+
+def kv_write_quant(fmt: str, k_rows: torch.Tensor, v_rows: torch.Tensor, kv_slots: torch.Tensor,
+                   k_pages: torch.Tensor, v_pages: torch.Tensor,
+                   k_scales: Optional[torch.Tensor] = None,
+                   v_scales: Optional[torch.Tensor] = None) -> None:
+    """Quantising KV write of rows [N, hk, d] bf16 into one-byte pools [pages, ps, hk, d]
+    (+ f32 scales [pages, ps, hk] for the per-token-head formats)."""
+    _dev(k_rows, torch.bfloat16, "k_rows")
+    _dev(v_rows, torch.bfloat16, "v_rows")
+    _dev(kv_slots, torch.int64, "kv_slots")
+    N, hk, d = k_rows.shape
+    if tuple(v_rows.shape) != (N, hk, d) or kv_slots.numel() != N:
+        raise KernelError("shape mismatch")
+    for t in (k_pages, v_pages):
+        if t.element_size() != 1 or not t.is_contiguous() or t.shape[-2:] != (hk, d):
+            raise KernelError("pools must be contiguous one-byte [pages, ps, hk, d]")
+    if N and int(kv_slots.max()) >= k_pages.numel() // (hk * d):
+        raise KernelError("kv slot out of range")
+    for sc in (k_scales, v_scales):
+        if sc is not None:
+            _dev(sc, torch.float32, "scales")
+            if sc.numel() != k_pages.numel() // d:
+                raise KernelError("scales must be [pages, ps, hk]")
+    _check(kernels().pie_hip_kv_write_quant(KV_FORMATS[fmt], _ptr(k_rows), _ptr(v_rows), _ptr(kv_slots),
+                                            _ptr(k_pages), _ptr(v_pages), _ptr(k_scales), _ptr(v_scales),
+                                            N, hk, d, _stream()), "pie_hip_kv_write_quant")
+
+
+def attention_rows_paged_kvq(fmt: str, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
+                             k_scales: Optional[torch.Tensor], v_scales: Optional[torch.Tensor],
+                             kv_page_indices: torch.Tensor, row_page_begin: torch.Tensor,
+                             row_kv_len: torch.Tensor, lse: bool = False):
+    """Per-row paged attention over a one-byte KV pool.  q [rows, hq, d] bf16."""
+    _dev(q, torch.bfloat16, "q")
+    rows, hq, d = q.shape
+    ps, hk = k_pages.shape[1], k_pages.shape[2]
+    if k_pages.element_size() != 1 or v_pages.element_size() != 1:
+        raise KernelError("one-byte pools expected")
+    _dev(kv_page_indices, torch.int32, "kv_page_indices")
+    _dev(row_page_begin, torch.int32, "row_page_begin")
+    _dev(row_kv_len, torch.int32, "row_kv_len")
+    if rows == 0:
+        return torch.empty_like(q), None
+    max_kv = int(row_kv_len.max())
+    npages = (row_kv_len.to(torch.int64) + ps - 1) // ps
+    if int((row_page_begin.to(torch.int64) + npages).max()) > kv_page_indices.numel():
+        raise KernelError("row extent runs past the page list")
+    if kv_page_indices.numel() and int(kv_page_indices.max()) >= k_pages.shape[0]:
+        raise KernelError("page id out of range")
+    o = torch.empty_like(q)
+    lse_t = torch.empty((rows, hq), dtype=torch.float32, device=q.device) if lse else None
+    lib = kernels()
+    lib.pie_hip_attn_decode_workspace_bytes.restype = C.c_size_t
+    need = int(lib.pie_hip_attn_decode_workspace_bytes(rows, hq, hk, d, max_kv))
+    ws = torch.empty(max(need, 1), dtype=torch.uint8, device=q.device)
+    _check(lib.pie_hip_attn_rows_paged_kvq(KV_FORMATS[fmt], _ptr(q), _ptr(k_pages), _ptr(v_pages),
+                                           _ptr(k_scales), _ptr(v_scales), _ptr(o), _ptr(lse_t),
+                                           _ptr(kv_page_indices), _ptr(row_page_begin), _ptr(row_kv_len),
+                                           rows, hq, hk, d, ps, C.c_float(-1.0), max_kv, _ptr(ws),
+                                           C.c_size_t(need), _stream()), "pie_hip_attn_rows_paged_kvq")
+    return o, lse_t

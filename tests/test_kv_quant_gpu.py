@@ -1,0 +1,99 @@
+"""GPU parity for the one-byte KV-cache formats: the quantising KV write is bit-exact against the
+oracle (codes and scales), and paged attention over such pools matches the oracle's attention
+over the dequantised values (float(code) * scale)."""
+import numpy as np
+import pytest
+
+from gpu_util import dev
+from paged_cases import make_paged_batch
+
+pytestmark = pytest.mark.gpu
+
+FORMATS = ["fp8_e4m3", "int8_per_token_head", "fp8_per_token_head"]
+
+
+@pytest.mark.parametrize("fmt", FORMATS)
+@pytest.mark.parametrize("hk,d", [(8, 128), (2, 64), (3, 96)])
+def test_kv_write_quant_bit_exact(gpu, oracle, fmt, hk, d):
+    import torch
+    from pie_amd import ops
+
+    rng = np.random.default_rng(40 + hk + d)
+    N, pages, ps = 37, 9, 16
+    k = oracle.f32_to_bf16((rng.standard_normal((N, hk, d)) * rng.uniform(0.05, 20, (N, hk, 1))).astype(np.float32))
+    v = oracle.f32_to_bf16(rng.standard_normal((N, hk, d)).astype(np.float32))
+    k[3] = 0                                                   # an all-zero token
+    slots = rng.permutation(pages * ps)[:N].astype(np.int64)
+    slots[5] = -1                                              # a token without a slot
+    kp = torch.full((pages, ps, hk, d), 0x55, dtype=torch.uint8, device=gpu)
+    vp = torch.full((pages, ps, hk, d), 0x55, dtype=torch.uint8, device=gpu)
+    scaled = fmt != "fp8_e4m3"
+    ks = torch.full((pages, ps, hk), -7.0, dtype=torch.float32, device=gpu) if scaled else None
+    vs = torch.full((pages, ps, hk), -7.0, dtype=torch.float32, device=gpu) if scaled else None
+    ops.kv_write_quant(fmt, dev(k, gpu, torch.bfloat16), dev(v, gpu, torch.bfloat16), dev(slots, gpu),
+                       kp, vp, ks, vs)
+    torch.cuda.synchronize()
+    for src, pool, sc in ((k, kp, ks), (v, vp, vs)):
+        codes, scales, _ = oracle.kv_quant_rows(src.reshape(N * hk, d), fmt)
+        want = np.full((pages * ps, hk, d), 0x55, np.uint8)
+        want_s = np.full((pages * ps, hk), -7.0, np.float32)
+        for t in range(N):
+            if slots[t] >= 0:
+                want[slots[t]] = codes.reshape(N, hk, d)[t]
+                if scaled:
+                    want_s[slots[t]] = scales.reshape(N, hk)[t]
+        assert np.array_equal(pool.cpu().numpy().reshape(pages * ps, hk, d), want)
+        if scaled:
+            assert np.array_equal(sc.cpu().numpy().reshape(pages * ps, hk), want_s)
+
+
+@pytest.mark.parametrize("fmt", FORMATS)
+@pytest.mark.parametrize("hq,hk,d,ps", [(32, 8, 128, 16), (8, 8, 128, 32), (16, 2, 64, 16), (4, 4, 64, 16)])
+def test_attention_over_quantised_pool_matches_oracle(gpu, oracle, fmt, hq, hk, d, ps):
+    import torch
+    from pie_amd import ops
+
+    rng = np.random.default_rng(50 + hq + d + ps)
+    ctx = [1, 15, 16, 17, 33, 100, 257, 0, 1500, 5]
+    b = make_paged_batch(rng, ctx, hk, d, ps, shared_prefix_tokens=2 * ps, shared_fraction=0.3,
+                         f32_to_bf16=oracle.f32_to_bf16)
+    P = b["num_pages"]
+    q = oracle.f32_to_bf16(rng.standard_normal((len(ctx), hq, d)).astype(np.float32))
+    pools = {}
+    for name in ("k_pages", "v_pages"):
+        codes, scales, deq = oracle.kv_quant_rows(b[name].reshape(P * ps * hk, d), fmt)
+        pools[name] = (codes.reshape(P, ps, hk, d), None if scales is None else scales.reshape(P, ps, hk),
+                       deq.reshape(P, ps, hk, d))
+    begin, lens = b["page_indptr"][:-1].astype(np.int32), np.asarray(ctx, np.int32)
+    sc = lambda s: None if s is None else dev(s, gpu)
+    o, lse = ops.attention_rows_paged_kvq(
+        fmt, dev(q, gpu, torch.bfloat16), dev(pools["k_pages"][0], gpu), dev(pools["v_pages"][0], gpu),
+        sc(pools["k_pages"][1]), sc(pools["v_pages"][1]), dev(b["page_indices"].view(np.int32), gpu),
+        dev(begin, gpu), dev(lens, gpu), lse=True)
+    torch.cuda.synchronize()
+    truth, _, lse64 = oracle.attn_rows_f32kv(q, pools["k_pages"][2], pools["v_pages"][2], b["page_indices"],
+                                             begin, lens, hq, hk, d, ps, mode=2)
+    got = oracle.bf16_to_f32(o.view(torch.uint16).cpu().numpy()).astype(np.float64)
+    # one bf16 rounding of the output + fp32 softmax / accumulation error, as for bf16 pools
+    tol = 2.0 ** -8 * np.maximum(np.abs(truth), np.abs(got)) + 1e-4
+    err = np.abs(got - truth)
+    assert np.all(err <= tol), f"worst {np.max(err / tol):.2f}x tol"
+    lse_g = lse.cpu().numpy()
+    fin = np.isfinite(lse64)
+    assert np.array_equal(np.isneginf(lse_g), np.isneginf(lse64))
+    assert np.allclose(lse_g[fin], lse64[fin], rtol=0, atol=2e-4)
+
+
+def test_quantised_pool_argument_checks(gpu):
+    import torch
+    from pie_amd import ops
+
+    q = torch.zeros((1, 8, 128), dtype=torch.bfloat16, device=gpu)
+    pool = torch.zeros((2, 16, 2, 128), dtype=torch.uint8, device=gpu)
+    idx = torch.zeros(1, dtype=torch.int32, device=gpu)
+    one = torch.ones(1, dtype=torch.int32, device=gpu)
+    with pytest.raises(ops.KernelError):   # per-token-head formats need their scales
+        ops.attention_rows_paged_kvq("int8_per_token_head", q, pool, pool, None, None, idx, idx, one)
+    sc = torch.ones((2, 16, 2), dtype=torch.float32, device=gpu)
+    with pytest.raises(ops.KernelError):   # plain fp8 takes none
+        ops.attention_rows_paged_kvq("fp8_e4m3", q, pool, pool, sc, sc, idx, idx, one)

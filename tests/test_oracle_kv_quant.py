@@ -1,0 +1,131 @@
+"""Pins for the oracle's KV-cache quantiser (driver/cuda/src/kernels/kv_paged.cu:155-297) and the
+f32-pool attention it feeds: the reference test's own source pattern and bars
+(driver/cuda/tests/test_kv_cache_quant.cu:34-40, :98-160, :230-262), independent numpy / torch
+evaluations of the same rules, and hand-worked rounding cases."""
+import numpy as np
+import pytest
+import torch
+
+from paged_cases import make_paged_batch
+
+FORMATS = ["fp8_e4m3", "int8_per_token_head", "fp8_per_token_head"]
+
+
+def reference_source(value: bool):
+    """source_value() of the reference test: 2 tokens x 2 heads x 17 dims."""
+    t, h, d = np.meshgrid(np.arange(2), np.arange(2), np.arange(17), indexing="ij")
+    sign = np.where((t + h + d + (1 if value else 0)) & 1, -1.0, 1.0)
+    base = 0.03 * (d - 8) + 0.11 * (h + 1) + 0.17 * (t + 1)
+    return (sign * base).astype(np.float32).reshape(4, 17)
+
+
+def e4m3_qdq(x):
+    """Saturating round-to-nearest-even e4m3fn through torch (independent of the oracle)."""
+    t = torch.from_numpy(np.clip(x, -448.0, 448.0).astype(np.float32))
+    return t.to(torch.float8_e4m3fn).to(torch.float32).numpy()
+
+
+def independent_qdq(xf, fmt):
+    """expected_qdq / expected_scale of the reference test, evaluated with numpy."""
+    if fmt == "fp8_e4m3":
+        return e4m3_qdq(xf), None
+    qmax = np.float32(127.0 if fmt.startswith("int8") else 448.0)
+    amax = np.abs(xf).max(axis=1)
+    scale = np.where(amax > 0, amax / qmax, np.float32(1.0)).astype(np.float32)
+    if fmt.startswith("int8"):
+        q = np.clip(np.rint(xf / scale[:, None]), -128, 127).astype(np.float32)
+        return q * scale[:, None], scale
+    return e4m3_qdq(xf / scale[:, None]) * scale[:, None], scale
+
+
+@pytest.mark.parametrize("fmt", FORMATS)
+@pytest.mark.parametrize("value", [False, True])
+def test_reference_pattern_within_reference_bars(oracle, fmt, value):
+    x = oracle.f32_to_bf16(reference_source(value))
+    xf = oracle.bf16_to_f32(x)
+    codes, scales, deq = oracle.kv_quant_rows(x, fmt)
+    want, want_scale = independent_qdq(xf, fmt)
+    assert np.max(np.abs(deq - want)) <= 0.02          # the reference test's bar
+    if want_scale is not None:
+        assert np.max(np.abs(scales - want_scale)) <= 1e-5
+        assert np.array_equal(scales, want_scale)      # same fp32 division
+    else:
+        assert scales is None
+
+
+@pytest.mark.parametrize("fmt", FORMATS)
+def test_codes_equal_an_independent_evaluation(oracle, fmt):
+    """The kernel's exact arithmetic: x * (1 / scale) in fp32, then rint / the e4m3 cast."""
+    rng = np.random.default_rng(11)
+    x = oracle.f32_to_bf16((rng.standard_normal((64, 128)) * rng.uniform(0.01, 30, (64, 1))).astype(np.float32))
+    xf = oracle.bf16_to_f32(x)
+    codes, scales, deq = oracle.kv_quant_rows(x, fmt)
+    if fmt == "fp8_e4m3":
+        scale = np.ones(64, np.float32)
+    else:
+        qmax = np.float32(127.0 if fmt.startswith("int8") else 448.0)
+        scale = (np.abs(xf).max(axis=1) / qmax).astype(np.float32)
+        assert np.array_equal(scales, scale)
+    pre = xf * (np.float32(1.0) / scale)[:, None]
+    if fmt.startswith("int8"):
+        want = np.clip(np.rint(pre), -128, 127)
+        assert np.array_equal(codes.view(np.int8).astype(np.float32), want)
+        assert np.array_equal(deq, want.astype(np.float32) * scale[:, None])
+        assert np.all(np.abs(codes.view(np.int8)).max(axis=1) == 127)     # the absmax element
+    else:
+        want = e4m3_qdq(pre)
+        got = torch.from_numpy(codes.copy()).view(torch.float8_e4m3fn).to(torch.float32).numpy()
+        assert np.array_equal(got, want)
+        assert np.array_equal(deq, want * scale[:, None])
+        if fmt == "fp8_per_token_head":
+            assert np.all(np.abs(got).max(axis=1) == 448.0)
+
+
+def test_hand_worked_rounding_and_zero_rows(oracle):
+    # scale = 127 * 2^-7 / 127 = 2^-7 exactly; 2.5 and 3.5 steps round to even, -0.5 steps to -0
+    row = np.array([127, 2.5, 3.5, -2.5, -0.5, 0.4375, 126.5, -127] + [0] * 8, np.float32) * 2.0 ** -7
+    x = oracle.f32_to_bf16(np.stack([row, np.zeros(16, np.float32)]))
+    assert np.array_equal(oracle.bf16_to_f32(x)[0], row)           # all exact in bf16
+    codes, scales, deq = oracle.kv_quant_rows(x, "int8_per_token_head")
+    assert scales[0] == 2.0 ** -7 and scales[1] == 1.0              # all-zero row: scale 1
+    assert list(codes.view(np.int8)[0][:8]) == [127, 2, 4, -2, 0, 0, 126, -127]
+    assert not codes[1].any() and not deq[1].any()
+    codes, scales, _ = oracle.kv_quant_rows(x, "fp8_per_token_head")
+    assert scales[0] == np.float32(127 * 2.0 ** -7) / np.float32(448.0) and scales[1] == 1.0
+    assert codes[0][0] == 0x7E and codes[0][7] == 0xFE              # +-448
+    # plain fp8: values beyond 448 saturate, NaN-free
+    big = oracle.f32_to_bf16(np.array([[1000.0, -1000.0, 448.0, 0.0625, 0.0]], np.float32))
+    codes, scales, deq = oracle.kv_quant_rows(big, "fp8_e4m3")
+    assert scales is None and list(deq[0]) == [448.0, -448.0, 448.0, 0.0625, 0.0]
+
+
+def test_attention_over_f32_pools_equals_dense_attention(oracle):
+    """The f32-pool attention against numpy fp64 softmax attention over gathered rows, and
+    against the bf16-pool oracle when the pools hold the same values."""
+    rng = np.random.default_rng(5)
+    hq, hk, d, ps = 8, 2, 64, 16
+    ctx = [1, 17, 40, 0, 100]
+    b = make_paged_batch(rng, ctx, hk, d, ps, f32_to_bf16=oracle.f32_to_bf16)
+    q = oracle.f32_to_bf16(rng.standard_normal((len(ctx), hq, d)).astype(np.float32))
+    kf, vf = oracle.bf16_to_f32(b["k_pages"]), oracle.bf16_to_f32(b["v_pages"])
+    begin, lens = b["page_indptr"][:-1], np.asarray(ctx, np.int32)
+    o32, _, lse = oracle.attn_rows_f32kv(q, kf, vf, b["page_indices"], begin, lens, hq, hk, d, ps)
+    ref32, _, ref_lse = oracle.attn_rows_masked(q, b["k_pages"], b["v_pages"], b["page_indices"], begin,
+                                                lens, hq, hk, d, ps, [None] * len(ctx), mode=2)
+    assert np.array_equal(o32, ref32) and np.array_equal(lse, ref_lse)
+    # a scaled pool: dense fp64 attention over the gathered dequantised rows
+    kf2 = (kf * 0.37).astype(np.float32)
+    o32, _, _ = oracle.attn_rows_f32kv(q, kf2, vf, b["page_indices"], begin, lens, hq, hk, d, ps)
+    qf = oracle.bf16_to_f32(q).astype(np.float64)
+    for r, n in enumerate(ctx):
+        if n == 0:
+            assert not o32[r].any()
+            continue
+        pages = b["page_indices"][int(begin[r]):int(begin[r]) + (n + ps - 1) // ps]
+        K = kf2[pages].reshape(-1, hk, d)[:n].astype(np.float64)
+        V = vf[pages].reshape(-1, hk, d)[:n].astype(np.float64)
+        for h in range(hq):
+            s = K[:, h // (hq // hk)] @ qf[r, h] / np.sqrt(d)
+            p = np.exp(s - s.max())
+            want = (p / p.sum()) @ V[:, h // (hq // hk)]
+            assert np.allclose(o32[r, h], want, rtol=1e-6, atol=1e-6)
