@@ -98,6 +98,15 @@ class OracleModel:
         self.v_pages = [np.zeros(shape, np.uint16) for _ in range(L)]
         self._kp = (C.c_void_p * L)(*[a.ctypes.data for a in self.k_pages])
         self._vp = (C.c_void_p * L)(*[a.ctypes.data for a in self.v_pages])
+        # one-byte KV-cache formats: pools of the dequantised values the attention reads back
+        from oracle import KV_FORMATS
+        kv_dtype = cfg.get("kv_cache_dtype", "bf16")
+        self.kv_format = KV_FORMATS["bf16" if kv_dtype in ("auto", "bfloat16") else kv_dtype]
+        if self.kv_format:
+            self.k_f32 = [np.zeros(shape, np.float32) for _ in range(L)]
+            self.v_f32 = [np.zeros(shape, np.float32) for _ in range(L)]
+            self._kf = (C.c_void_p * L)(*[a.ctypes.data for a in self.k_f32])
+            self._vf = (C.c_void_p * L)(*[a.ctypes.data for a in self.v_f32])
 
     def forward(self, token_ids, position_ids, kv_page_indices, kv_page_indptr, kv_last_page_lens,
                 qo_indptr, sampling_indices=None, sampling_indptr=None, want_logits=False,
@@ -134,6 +143,13 @@ class OracleModel:
                 at += int(rl[i])
             allow = np.ascontiguousarray(np.concatenate(chunks) if chunks else np.zeros(1, np.uint8))
             allow_off = np.ascontiguousarray(np.asarray(offs, np.int64))
+        if self.kv_format:
+            assert masks is None, "custom masks are not available with one-byte KV formats"
+            lib().orc_llama_forward_kvq(C.byref(self._m), C.c_int(self.kv_format), self._kf, self._vf,
+                                        vp(tok), vp(pos), vp(slots), vp(rb), vp(rl), vp(pages), C.c_int(N),
+                                        vp(sr), C.c_int(S), C.c_int(self.cfg["page_size"]), vp(out),
+                                        vp(logits) if want_logits else None)
+            return out[:S], (logits[:S] if want_logits else None), p
         lib().orc_llama_forward(C.byref(self._m), self._kp, self._vp, vp(tok), vp(pos), vp(slots),
                                 vp(rb), vp(rl), vp(pages), C.c_int(N), vp(sr), C.c_int(S),
                                 C.c_int(self.cfg["page_size"]), vp(out),

@@ -20,6 +20,7 @@
  * driver/cuda/tests/parity_qwen3.py:160-181).
  */
 #include <stdlib.h>
+#include <string.h>
 
 #include "oracle_api.h"
 
@@ -130,7 +131,20 @@ static void orc_moe_ffn(const OrcModel* m, int l, const uint16_t* xn, uint16_t* 
  * non-NULL, logits_bf16 [S, V].  allow / allow_off: optional per-row key visibility (custom
  * attention masks), as orc_attn_rows_masked takes them.
  */
-void orc_llama_forward(const OrcModel* m, uint16_t* const* k_pages, uint16_t* const* v_pages,
+void orc_kv_quant_rows(const uint16_t* x, uint8_t* codes, float* scales, float* dequant, int rows,
+                       int d, int fmt);
+void orc_attn_rows_f32kv(const uint16_t* q, const float* k_pages, const float* v_pages,
+                         float* o_f32, uint16_t* o_bf16, float* lse, const uint32_t* page_indices,
+                         const uint32_t* row_begin, const int32_t* row_len, int rows, int hq,
+                         int hk, int d, int ps, float sm_scale, int mode, const uint8_t* allow,
+                         const int64_t* allow_off);
+
+/* kv_format != 0: a one-byte KV-cache format (1 fp8_e4m3, 2 int8_per_token_head,
+ * 3 fp8_per_token_head).  The step's rotated K / V rows are quantised per (token, head) as
+ * kv_paged.cu:155-297 does and the pools k_f32 / v_f32 [L][pages, ps, hk, d] hold the values the
+ * attention reads back, float(code) * scale (attention_naive_paged.cu:56-112). */
+static void orc_llama_forward_impl(const OrcModel* m, uint16_t* const* k_pages, uint16_t* const* v_pages,
+                       int kv_format, float* const* k_f32, float* const* v_f32,
                        const uint32_t* tokens, const int32_t* positions, const int64_t* kv_slots,
                        const uint32_t* row_begin, const int32_t* row_len,
                        const uint32_t* page_indices, int N, const uint32_t* sample_rows, int S,
@@ -148,17 +162,46 @@ void orc_llama_forward(const OrcModel* m, uint16_t* const* k_pages, uint16_t* co
     uint16_t* gu = (uint16_t*)malloc((size_t)N * 2 * I * 2);
     uint16_t* act = (uint16_t*)malloc((size_t)N * I * 2);
     float* tab = (float*)malloc((size_t)N * d * 4);
+    const size_t kvrow = (size_t)hk * d;
+    uint16_t *k_rows = NULL, *v_rows = NULL;
+    uint8_t* codes = NULL;
+    float *scales = NULL, *deq = NULL;
+    int64_t* iota = NULL;
+    if (kv_format) {
+        k_rows = (uint16_t*)malloc((size_t)N * kvrow * 2);
+        v_rows = (uint16_t*)malloc((size_t)N * kvrow * 2);
+        codes = (uint8_t*)malloc((size_t)N * kvrow);
+        scales = (float*)malloc((size_t)N * hk * 4);
+        deq = (float*)malloc((size_t)N * kvrow * 4);
+        iota = (int64_t*)malloc((size_t)N * 8);
+        for (int i = 0; i < N; ++i) iota[i] = i;
+    }
 
     orc_embed(tokens, m->embed, x, N, H, V);
     orc_rope_table(positions, m->inv_freq, tab, N, d);
     for (int l = 0; l < m->layers; ++l) {
         orc_rmsnorm(x, NULL, m->attn_norm[l], xn, N, H, m->rms_eps);
         orc_linear(m, &m->wqkv[l], xn, qkv, N, qkv_dim, H, 0);
-        orc_qkv_rope_kvwrite(qkv, q, k_pages[l], v_pages[l], m->has_qk_norm ? m->q_norm[l] : NULL,
-                             m->has_qk_norm ? m->k_norm[l] : NULL, tab, kv_slots, N, hq, hk, d,
-                             m->rope_interleaved, m->rms_eps);
-        orc_attn_rows_masked(q, k_pages[l], v_pages[l], attn_f, attn, NULL, page_indices, row_begin,
-                             row_len, N, hq, hk, d, page_size, -1.f, 0, allow, allow_off);
+        if (kv_format) {
+            orc_qkv_rope_kvwrite(qkv, q, k_rows, v_rows, m->has_qk_norm ? m->q_norm[l] : NULL,
+                                 m->has_qk_norm ? m->k_norm[l] : NULL, tab, iota, N, hq, hk, d,
+                                 m->rope_interleaved, m->rms_eps);
+            for (int kv = 0; kv < 2; ++kv) {
+                orc_kv_quant_rows(kv ? v_rows : k_rows, codes, scales, deq, N * hk, d, kv_format);
+                float* pool = kv ? v_f32[l] : k_f32[l];
+                for (int t = 0; t < N; ++t)
+                    if (kv_slots[t] >= 0)
+                        memcpy(pool + (size_t)kv_slots[t] * kvrow, deq + (size_t)t * kvrow, kvrow * 4);
+            }
+            orc_attn_rows_f32kv(q, k_f32[l], v_f32[l], attn_f, attn, NULL, page_indices, row_begin,
+                                row_len, N, hq, hk, d, page_size, -1.f, 0, allow, allow_off);
+        } else {
+            orc_qkv_rope_kvwrite(qkv, q, k_pages[l], v_pages[l], m->has_qk_norm ? m->q_norm[l] : NULL,
+                                 m->has_qk_norm ? m->k_norm[l] : NULL, tab, kv_slots, N, hq, hk, d,
+                                 m->rope_interleaved, m->rms_eps);
+            orc_attn_rows_masked(q, k_pages[l], v_pages[l], attn_f, attn, NULL, page_indices, row_begin,
+                                 row_len, N, hq, hk, d, page_size, -1.f, 0, allow, allow_off);
+        }
         orc_linear(m, &m->wo[l], attn, x, N, H, hq * d, 1);
         orc_rmsnorm(x, NULL, m->ffn_norm[l], xn, N, H, m->rms_eps);
         if (m->num_experts > 0) {
@@ -184,4 +227,26 @@ void orc_llama_forward(const OrcModel* m, uint16_t* const* k_pages, uint16_t* co
         if (!logits_bf16) free(lg);
     }
     free(x); free(xn); free(qkv); free(q); free(attn); free(attn_f); free(gu); free(act); free(tab);
+    free(k_rows); free(v_rows); free(codes); free(scales); free(deq); free(iota);
+}
+
+void orc_llama_forward(const OrcModel* m, uint16_t* const* k_pages, uint16_t* const* v_pages,
+                       const uint32_t* tokens, const int32_t* positions, const int64_t* kv_slots,
+                       const uint32_t* row_begin, const int32_t* row_len,
+                       const uint32_t* page_indices, int N, const uint32_t* sample_rows, int S,
+                       int page_size, uint32_t* out_tokens, uint16_t* logits_bf16,
+                       const uint8_t* allow, const int64_t* allow_off) {
+    orc_llama_forward_impl(m, k_pages, v_pages, 0, NULL, NULL, tokens, positions, kv_slots, row_begin,
+                           row_len, page_indices, N, sample_rows, S, page_size, out_tokens,
+                           logits_bf16, allow, allow_off);
+}
+
+void orc_llama_forward_kvq(const OrcModel* m, int kv_format, float* const* k_f32, float* const* v_f32,
+                           const uint32_t* tokens, const int32_t* positions, const int64_t* kv_slots,
+                           const uint32_t* row_begin, const int32_t* row_len,
+                           const uint32_t* page_indices, int N, const uint32_t* sample_rows, int S,
+                           int page_size, uint32_t* out_tokens, uint16_t* logits_bf16) {
+    orc_llama_forward_impl(m, NULL, NULL, kv_format, k_f32, v_f32, tokens, positions, kv_slots,
+                           row_begin, row_len, page_indices, N, sample_rows, S, page_size, out_tokens,
+                           logits_bf16, NULL, NULL);
 }

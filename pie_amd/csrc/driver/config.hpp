@@ -11,6 +11,7 @@
 #include <map>
 #include <sstream>
 #include <stdexcept>
+#include <cctype>
 #include <string>
 
 namespace pie_hip_driver {
@@ -50,6 +51,9 @@ struct BatchingConfig {
     int max_forward_tokens = 10240;
     int max_forward_requests = 512;
     int cpu_pages = 0;
+    // KV-cache storage (driver/cuda/src/config.hpp:66, kv_cache_format.cpp:46-110): auto | bf16 |
+    // bfloat16 | fp8_e4m3 | int8_per_token_head | fp8_per_token_head
+    std::string kv_cache_dtype = "auto";
 };
 
 struct RuntimeConfig {
@@ -137,6 +141,23 @@ inline std::map<std::string, std::map<std::string, std::string>> parse_toml_lite
     return out;
 }
 
+// The kernel library's PIE_HIP_KV_* code of a kv_cache_dtype value; the reference's other values
+// (fp8_e5m2, fp4_e2m1, nvfp4) are recognised and refused, anything else is invalid
+// (driver/cuda/src/kv_cache_format.cpp:105-108).
+inline int kv_format_code(const std::string& value) {
+    std::string v;
+    for (char ch : value) v.push_back(static_cast<char>(std::tolower(static_cast<unsigned char>(ch))));
+    if (v.empty() || v == "auto" || v == "bf16" || v == "bfloat16") return 0;
+    if (v == "fp8_e4m3") return 1;
+    if (v == "int8_per_token_head") return 2;
+    if (v == "fp8_per_token_head") return 3;
+    if (v == "fp8_e5m2" || v == "fp4_e2m1" || v == "nvfp4")
+        throw std::runtime_error("config: kv_cache_dtype '" + value + "' is not implemented by this driver");
+    throw std::runtime_error("invalid kv_cache_dtype '" + value +
+                             "'; expected one of: auto, bf16, bfloat16, fp8_e4m3, fp8_e5m2, "
+                             "int8_per_token_head, fp8_per_token_head, fp4_e2m1, nvfp4");
+}
+
 // Shape and range checks, defaults that depend on other fields.
 inline void finalize_config(DriverConfig& c) {
     auto& m = c.model;
@@ -163,6 +184,7 @@ inline void finalize_config(DriverConfig& c) {
         throw std::runtime_error("config: kv_page_size must be a positive multiple of 16");
     if (b.total_pages <= 0 || b.max_forward_tokens <= 0 || b.max_forward_requests <= 0)
         throw std::runtime_error("config: [batching] sizes must be positive");
+    (void)kv_format_code(b.kv_cache_dtype);
 }
 
 inline DriverConfig parse_config_text(const std::string& text) {
@@ -210,6 +232,7 @@ inline DriverConfig parse_config_text(const std::string& text) {
                 else if (k == "max_forward_tokens") b.max_forward_tokens = (int)to_int(v, key);
                 else if (k == "max_forward_requests") b.max_forward_requests = (int)to_int(v, key);
                 else if (k == "cpu_pages") b.cpu_pages = (int)to_int(v, key);
+                else if (k == "kv_cache_dtype") b.kv_cache_dtype = v;
                 else throw std::runtime_error("config: unknown [batching] key '" + k + "'");
             } else if (sec == "runtime") {
                 auto& r = c.runtime;

@@ -142,10 +142,12 @@ Executor::Executor(const DriverConfig& cfg, Model& model) : cfg_(cfg), model_(mo
     total_pages_ = cfg.batching.total_pages;
     max_tokens_ = cfg.batching.max_forward_tokens;
     max_page_refs_ = 4 * total_pages_ + max_tokens_;
+    kv_format_ = kv_format_code(cfg.batching.kv_cache_dtype);
     alloc_kv();
     cpu_pages_ = std::max(0, cfg.batching.cpu_pages);
     if (cpu_pages_ > 0) {
-        const size_t bytes = static_cast<size_t>(model.cfg().layers) * 2 * cpu_pages_ * page_bytes();
+        const size_t bytes = static_cast<size_t>(model.cfg().layers) * 2 * cpu_pages_ *
+                             (page_bytes() + scale_page_bytes());
         PIE_HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&swap_pool_), bytes, hipHostMallocDefault));
         std::memset(swap_pool_, 0, bytes);
     }
@@ -184,6 +186,14 @@ Executor::Executor(const DriverConfig& cfg, Model& model) : cfg_(cfg), model_(mo
     // rows * splits <= 3072/hk + rows.
     attn_ws_bytes_ = (3072 / static_cast<size_t>(hk) + 1 + T) * hq * (d + 2) * sizeof(float);
     PIE_HIP_CHECK(hipMalloc(&attn_ws_, attn_ws_bytes_));
+    if (kv_format_ != PIE_HIP_KV_BF16) {
+        k_rows_ = dmalloc<uint16_t>(T * hk * d);
+        v_rows_ = dmalloc<uint16_t>(T * hk * d);
+        iota_slots_ = dmalloc<int64_t>(T);
+        std::vector<int64_t> iota(T);
+        for (size_t i = 0; i < T; ++i) iota[i] = static_cast<int64_t>(i);
+        PIE_HIP_CHECK(hipMemcpy(iota_slots_, iota.data(), T * sizeof(int64_t), hipMemcpyHostToDevice));
+    }
     // fp32 partials of the split-K GEMM for decode batches of up to 128 rows (dense layers)
     if (!model.layers.empty()) {
         const LayerWeights& l0 = model.layers[0];
@@ -215,8 +225,11 @@ Executor::~Executor() {
                     static_cast<void*>(moe_y_), static_cast<void*>(moe_logits_),
                     static_cast<void*>(moe_idx_), static_cast<void*>(moe_w_),
                     static_cast<void*>(moe_offsets_), static_cast<void*>(moe_route_token_),
-                    static_cast<void*>(moe_route_pos_)})
+                    static_cast<void*>(moe_route_pos_), static_cast<void*>(k_rows_),
+                    static_cast<void*>(v_rows_), static_cast<void*>(iota_slots_)})
         if (p) (void)hipFree(p);
+    for (auto* p : k_scale_pool_) (void)hipFree(p);
+    for (auto* p : v_scale_pool_) (void)hipFree(p);
     for (Growable* g : {&mask_in_host_, &mask_in_dev_, &mask_bitmap_, &tile_in_host_, &tile_in_dev_}) g->release();
     for (Growable* g : {&samp_f32_, &samp_ws_, &samp_in_dev_, &samp_in_host_, &samp_out_dev_, &samp_out_host_})
         g->release();
@@ -226,9 +239,15 @@ Executor::~Executor() {
     if (stream_) (void)hipStreamDestroy(stream_);
 }
 
+// Page sizes of the storage formats: kv_bytes_per_page / scale_bytes_per_page,
+// driver/cuda/src/kv_cache_format.cpp:27-49.
 size_t Executor::page_bytes() const {
     const ModelConfig& m = model_.cfg();
-    return static_cast<size_t>(page_size_) * m.kv_heads * m.head_dim * 2;
+    return static_cast<size_t>(page_size_) * m.kv_heads * m.head_dim * (kv_format_ == PIE_HIP_KV_BF16 ? 2 : 1);
+}
+size_t Executor::scale_page_bytes() const {
+    const bool scaled = kv_format_ == PIE_HIP_KV_INT8_PER_TOKEN_HEAD || kv_format_ == PIE_HIP_KV_FP8_PER_TOKEN_HEAD;
+    return scaled ? static_cast<size_t>(page_size_) * model_.cfg().kv_heads * sizeof(float) : 0;
 }
 
 // Allocate the pool; on out-of-memory halve the page count down to 64 pages
@@ -237,6 +256,7 @@ void Executor::alloc_kv() {
     const int L = model_.cfg().layers;
     for (;;) {
         const size_t bytes = page_bytes() * static_cast<size_t>(total_pages_);
+        const size_t sbytes = scale_page_bytes() * static_cast<size_t>(total_pages_);
         bool ok = true;
         for (int l = 0; l < L && ok; ++l) {
             void *k = nullptr, *v = nullptr;
@@ -244,12 +264,22 @@ void Executor::alloc_kv() {
             k_pool_.push_back(static_cast<uint16_t*>(k));
             if (hipMalloc(&v, bytes) != hipSuccess) { ok = false; break; }
             v_pool_.push_back(static_cast<uint16_t*>(v));
+            if (sbytes) {
+                if (hipMalloc(&k, sbytes) != hipSuccess) { ok = false; break; }
+                k_scale_pool_.push_back(static_cast<float*>(k));
+                if (hipMalloc(&v, sbytes) != hipSuccess) { ok = false; break; }
+                v_scale_pool_.push_back(static_cast<float*>(v));
+            }
         }
         if (ok) {
             // Pages start zeroed so slots no request has written hold finite values.
             for (int l = 0; l < L; ++l) {
                 PIE_HIP_CHECK(hipMemsetAsync(k_pool_[l], 0, bytes, stream_));
                 PIE_HIP_CHECK(hipMemsetAsync(v_pool_[l], 0, bytes, stream_));
+                if (sbytes) {
+                    PIE_HIP_CHECK(hipMemsetAsync(k_scale_pool_[l], 0, sbytes, stream_));
+                    PIE_HIP_CHECK(hipMemsetAsync(v_scale_pool_[l], 0, sbytes, stream_));
+                }
             }
             PIE_HIP_CHECK(hipStreamSynchronize(stream_));
             return;
@@ -257,8 +287,12 @@ void Executor::alloc_kv() {
         (void)hipGetLastError();
         for (auto* p : k_pool_) (void)hipFree(p);
         for (auto* p : v_pool_) (void)hipFree(p);
+        for (auto* p : k_scale_pool_) (void)hipFree(p);
+        for (auto* p : v_scale_pool_) (void)hipFree(p);
         k_pool_.clear();
         v_pool_.clear();
+        k_scale_pool_.clear();
+        v_scale_pool_.clear();
         if (total_pages_ <= 64) throw std::runtime_error("executor: cannot allocate the KV pool");
         total_pages_ = std::max(64, total_pages_ / 2);
     }
@@ -305,7 +339,18 @@ void Executor::body(int N, int S, int max_kv_len) {
     PIE_KERNEL(pie_hip_rope_table(positions, model_.inv_freq, rope_tab_, N, d, s));
     for (int l = 0; l < m.layers; ++l) {
         const LayerWeights& w = model_.layers[l];
-        if (N <= 4 && m.rope_interleaved && !w.q_norm && (d & (d - 1)) == 0) {
+        const bool kvq = kv_format_ != PIE_HIP_KV_BF16;
+        float* ksc = kvq && !k_scale_pool_.empty() ? k_scale_pool_[l] : nullptr;
+        float* vsc = kvq && !v_scale_pool_.empty() ? v_scale_pool_[l] : nullptr;
+        if (kvq) {
+            // one-byte pools: the rotated K / V rows of this step are staged as bf16 rows (row t
+            // in "slot" t) and quantised into the tokens' real slots
+            linear_fused(w.wqkv, x_, w.attn_norm, m.rms_eps, qkv_, N, 0, 0, xn_, gemm_ws_, gemm_ws_bytes_, s);
+            PIE_KERNEL(pie_hip_qkv_rope_kvwrite(qkv_, q_, k_rows_, v_rows_, w.q_norm, w.k_norm, rope_tab_,
+                                                iota_slots_, N, hq, hk, d, m.rope_interleaved, m.rms_eps, s));
+            PIE_KERNEL(pie_hip_kv_write_quant(kv_format_, k_rows_, v_rows_, slots, k_pool_[l], v_pool_[l],
+                                              ksc, vsc, N, hk, d, s));
+        } else if (N <= 4 && m.rope_interleaved && !w.q_norm && (d & (d - 1)) == 0) {
             // decode rows of llama-type layers: rotation and KV write ride in the projection
             PIE_KERNEL(pie_hip_qkv_rope_fused(fmt_code(w.wqkv.kind), x_, w.attn_norm, m.rms_eps,
                                               w.wqkv.data, w.wqkv.scale, w.wqkv.scale_bf16 ? 1 : 0,
@@ -317,7 +362,12 @@ void Executor::body(int N, int S, int max_kv_len) {
                                                 rope_tab_, slots, N, hq, hk, d, m.rope_interleaved,
                                                 m.rms_eps, s));
         }
-        if (n_tiles_ > 0) {
+        if (kvq) {
+            if (masked_) throw std::runtime_error("executor: custom attention masks need a bf16 KV cache");
+            PIE_KERNEL(pie_hip_attn_rows_paged_kvq(kv_format_, q_, k_pool_[l], v_pool_[l], ksc, vsc, attn_,
+                                                   nullptr, pages, row_begin, row_len, N, hq, hk, d,
+                                                   page_size_, -1.f, max_kv_len, attn_ws_, attn_ws_bytes_, s));
+        } else if (n_tiles_ > 0) {
             const auto* td = static_cast<const int32_t*>(tile_in_dev_.ptr);
             PIE_KERNEL(pie_hip_attn_prefill_tiles(q_, k_pool_[l], v_pool_[l], attn_, pages, row_begin,
                                                   row_len, td, td + n_tiles_, n_tiles_, tile_rows_, hq,
@@ -407,6 +457,7 @@ void Executor::prepare_tiles(const BatchPlan& plan) {
     const ModelConfig& m = model_.cfg();
     int cap = pie_hip_attn_prefill_tile_rows(m.q_heads, m.kv_heads);
     if (cap <= 0 || plan.has_user_masks || page_size_ % 16 != 0 || (m.head_dim != 64 && m.head_dim != 128)) return;
+    if (kv_format_ != PIE_HIP_KV_BF16) return;   // the tile kernel reads bf16 pools only
     long long blocks = 0;
     for (int r = 0; r < plan.R; ++r) {
         const int n = plan.qo_indptr[r + 1] - plan.qo_indptr[r];
@@ -696,38 +747,45 @@ void Executor::forward(const BatchPlan& plan, std::vector<uint32_t>& tokens_out,
     last_logit_rows_ = S == 0 ? 0 : ((S - 1) % cap) + 1;
 }
 
+// A swap-pool slot holds a page's K (or V) bytes followed by its fp32 scales (scaled formats).
 void Executor::copy_pages_d2h(const uint32_t* dev_srcs, const uint32_t* host_dsts, size_t n) {
-    const size_t pb = page_bytes();
+    const size_t pb = page_bytes(), sb = scale_page_bytes();
     for (size_t i = 0; i < n; ++i)
-        for (size_t l = 0; l < k_pool_.size(); ++l) {
-            const size_t off = static_cast<size_t>(dev_srcs[i]) * pb;
-            PIE_HIP_CHECK(hipMemcpyAsync(swap_slot(static_cast<int>(l), 0, host_dsts[i]),
-                                         reinterpret_cast<const unsigned char*>(k_pool_[l]) + off, pb,
-                                         hipMemcpyDeviceToHost, stream_));
-            PIE_HIP_CHECK(hipMemcpyAsync(swap_slot(static_cast<int>(l), 1, host_dsts[i]),
-                                         reinterpret_cast<const unsigned char*>(v_pool_[l]) + off, pb,
-                                         hipMemcpyDeviceToHost, stream_));
-        }
+        for (size_t l = 0; l < k_pool_.size(); ++l)
+            for (int kv = 0; kv < 2; ++kv) {
+                unsigned char* dst = swap_slot(static_cast<int>(l), kv, host_dsts[i]);
+                const auto* pool = reinterpret_cast<const unsigned char*>(kv ? v_pool_[l] : k_pool_[l]);
+                PIE_HIP_CHECK(hipMemcpyAsync(dst, pool + static_cast<size_t>(dev_srcs[i]) * pb, pb,
+                                             hipMemcpyDeviceToHost, stream_));
+                if (sb) {
+                    const auto* sc = reinterpret_cast<const unsigned char*>(kv ? v_scale_pool_[l] : k_scale_pool_[l]);
+                    PIE_HIP_CHECK(hipMemcpyAsync(dst + pb, sc + static_cast<size_t>(dev_srcs[i]) * sb, sb,
+                                                 hipMemcpyDeviceToHost, stream_));
+                }
+            }
     PIE_HIP_CHECK(hipStreamSynchronize(stream_));
 }
 
 void Executor::copy_pages_h2d(const uint32_t* host_srcs, const uint32_t* dev_dsts, size_t n) {
-    const size_t pb = page_bytes();
+    const size_t pb = page_bytes(), sb = scale_page_bytes();
     for (size_t i = 0; i < n; ++i)
-        for (size_t l = 0; l < k_pool_.size(); ++l) {
-            const size_t off = static_cast<size_t>(dev_dsts[i]) * pb;
-            PIE_HIP_CHECK(hipMemcpyAsync(reinterpret_cast<unsigned char*>(k_pool_[l]) + off,
-                                         swap_slot(static_cast<int>(l), 0, host_srcs[i]), pb,
-                                         hipMemcpyHostToDevice, stream_));
-            PIE_HIP_CHECK(hipMemcpyAsync(reinterpret_cast<unsigned char*>(v_pool_[l]) + off,
-                                         swap_slot(static_cast<int>(l), 1, host_srcs[i]), pb,
-                                         hipMemcpyHostToDevice, stream_));
-        }
+        for (size_t l = 0; l < k_pool_.size(); ++l)
+            for (int kv = 0; kv < 2; ++kv) {
+                const unsigned char* src = swap_slot(static_cast<int>(l), kv, host_srcs[i]);
+                auto* pool = reinterpret_cast<unsigned char*>(kv ? v_pool_[l] : k_pool_[l]);
+                PIE_HIP_CHECK(hipMemcpyAsync(pool + static_cast<size_t>(dev_dsts[i]) * pb, src, pb,
+                                             hipMemcpyHostToDevice, stream_));
+                if (sb) {
+                    auto* sc = reinterpret_cast<unsigned char*>(kv ? v_scale_pool_[l] : k_scale_pool_[l]);
+                    PIE_HIP_CHECK(hipMemcpyAsync(sc + static_cast<size_t>(dev_dsts[i]) * sb, src + pb, sb,
+                                                 hipMemcpyHostToDevice, stream_));
+                }
+            }
     PIE_HIP_CHECK(hipStreamSynchronize(stream_));
 }
 
 void Executor::copy_pages_h2h(const uint32_t* srcs, const uint32_t* dsts, size_t n) {
-    const size_t pb = page_bytes();
+    const size_t pb = page_bytes() + scale_page_bytes();
     for (size_t i = 0; i < n; ++i)
         for (size_t l = 0; l < k_pool_.size(); ++l)
             for (int kv = 0; kv < 2; ++kv)
@@ -751,6 +809,12 @@ void Executor::copy_pages_d2d(const uint32_t* srcs, const uint32_t* dsts, size_t
                                              cnt, page_bytes(), stream_));
             PIE_KERNEL(pie_hip_copy_kv_pages(v_pool_[l], copy_ids_ + i, copy_ids_ + copy_ids_cap_ + i,
                                              cnt, page_bytes(), stream_));
+            if (scale_page_bytes()) {
+                PIE_KERNEL(pie_hip_copy_kv_pages(k_scale_pool_[l], copy_ids_ + i, copy_ids_ + copy_ids_cap_ + i,
+                                                 cnt, scale_page_bytes(), stream_));
+                PIE_KERNEL(pie_hip_copy_kv_pages(v_scale_pool_[l], copy_ids_ + i, copy_ids_ + copy_ids_cap_ + i,
+                                                 cnt, scale_page_bytes(), stream_));
+            }
         }
     }
     PIE_HIP_CHECK(hipStreamSynchronize(stream_));

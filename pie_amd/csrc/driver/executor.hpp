@@ -72,7 +72,9 @@ class Executor {
 
     int total_pages() const { return total_pages_; }
     int page_size() const { return page_size_; }
-    size_t page_bytes() const;
+    size_t page_bytes() const;         // K (or V) bytes of one page in the pool's storage format
+    size_t scale_page_bytes() const;   // fp32 side scales of one page (0 without them)
+    int kv_format() const { return kv_format_; }
     hipStream_t stream() const { return stream_; }
     int graphs_cached() const { return static_cast<int>(graphs_.size()); }
     // Logits [rows, vocab] bf16 of the last forward's (last chunk of) sampled rows; debug/test hook.
@@ -98,11 +100,16 @@ class Executor {
     hipStream_t stream_ = nullptr;
     int total_pages_ = 0, page_size_ = 0, max_tokens_ = 0, max_page_refs_ = 0;
 
-    std::vector<uint16_t*> k_pool_, v_pool_;  // per layer [pages, ps, hk, d]
-    unsigned char* swap_pool_ = nullptr;       // pinned: [layer][K|V][cpu_pages] pages
+    std::vector<uint16_t*> k_pool_, v_pool_;  // per layer [pages, ps, hk, d] (bf16 or one byte per element)
+    int kv_format_ = 0;                        // PIE_HIP_KV_*
+    std::vector<float*> k_scale_pool_, v_scale_pool_;   // per layer [pages, ps, hk], scaled formats
+    uint16_t *k_rows_ = nullptr, *v_rows_ = nullptr;     // this step's rotated K / V rows before quantisation
+    int64_t* iota_slots_ = nullptr;                      // 0, 1, 2, ...: row t of k_rows_ is "slot" t
+    unsigned char* swap_pool_ = nullptr;       // pinned: [layer][K|V][cpu_pages] pages (+ their scales)
     int cpu_pages_ = 0;
     unsigned char* swap_slot(int layer, int kv, uint32_t slot) const {
-        return swap_pool_ + ((static_cast<size_t>(layer) * 2 + kv) * cpu_pages_ + slot) * page_bytes();
+        return swap_pool_ + ((static_cast<size_t>(layer) * 2 + kv) * cpu_pages_ + slot) *
+                                (page_bytes() + scale_page_bytes());
     }
     // activations
     uint16_t *x_ = nullptr, *xn_ = nullptr, *qkv_ = nullptr, *q_ = nullptr, *attn_ = nullptr;
