@@ -55,7 +55,8 @@ OTHER_MODELS = {
 }
 
 
-def toml(model: dict, page_size: int, total_pages: int, max_tokens: int, max_requests: int) -> str:
+def toml(model: dict, page_size: int, total_pages: int, max_tokens: int, max_requests: int,
+         kv_cache_dtype: str = "auto") -> str:
     lines = ["[model]"]
     for k, v in model.items():
         if isinstance(v, bool):
@@ -64,7 +65,7 @@ def toml(model: dict, page_size: int, total_pages: int, max_tokens: int, max_req
             lines.append(f'{k} = "{v}"' if isinstance(v, str) else f"{k} = {v}")
     lines += ["[batching]", f"kv_page_size = {page_size}", f"total_pages = {total_pages}",
               f"max_forward_tokens = {max_tokens}", f"max_forward_requests = {max_requests}",
-              "[runtime]", "use_graphs = true"]
+              f'kv_cache_dtype = "{kv_cache_dtype}"', "[runtime]", "use_graphs = true"]
     return "\n".join(lines) + "\n"
 
 
@@ -207,10 +208,26 @@ def attention_extra():
     t = time_graph(lambda: ops.attention_paged_decode(q, kp, vp, pi, pp, ll, maxlen, o=o, workspace=ws), 10)
     alg = int(ctx.sum()) * 2 * hk * d * 2 + R * hq * d * 2 * 2
     dedup = alg - 15 * 1024 * 2 * hk * d * 2
+    # the same batch over one-byte pools (codes + fp32 scales per (token, head))
+    rb = torch.tensor(indptr[:-1], dtype=torch.int32, device=dev)
+    rl = torch.from_numpy(ctx.astype(np.int32)).to(dev)
+    one_byte = {}
+    for fmt in ("fp8_per_token_head", "int8_per_token_head"):
+        k8 = torch.randint(0, 120, (total, ps, hk, d), dtype=torch.uint8, device=dev)
+        v8 = torch.randint(0, 120, (total, ps, hk, d), dtype=torch.uint8, device=dev)
+        ks = torch.rand(total, ps, hk, device=dev) * 0.01 + 0.001
+        vs = torch.rand(total, ps, hk, device=dev) * 0.01 + 0.001
+        fn = lambda: ops.attention_rows_paged_kvq(fmt, q, k8, v8, ks, vs, pi, rb, rl, max_kv_len=maxlen,
+                                                  o=o, workspace=ws)
+        fn()
+        tq = time_graph(fn, 10)
+        algq = int(ctx.sum()) * 2 * hk * (d + 4) + R * hq * d * 2 * 2
+        one_byte[fmt] = dict(us=round(tq * 1e6, 1), algorithmic_bytes=algq, gbps=round(algq / tq / 1e9, 1),
+                             frac_of_hbm_peak=round(algq / tq / 1e9 / HBM_PEAK_GBPS, 4))
     return dict(workload="decode attention 32q/8kv d128 page16 batch64 ctx U[512,8192] 25% forked 1024 prefix",
                 us=round(t * 1e6, 1), algorithmic_bytes=alg, gbps=round(alg / t / 1e9, 1),
                 frac_of_hbm_peak=round(alg / t / 1e9 / HBM_PEAK_GBPS, 4),
-                dedup_bytes=dedup, note="split kernel + merge kernel per call")
+                dedup_bytes=dedup, note="split kernel + merge kernel per call", one_byte_kv=one_byte)
 
 
 def w4a16_sweep_extra():
@@ -355,6 +372,9 @@ def main():
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--kv-cache-dtype", default="auto",
+                    choices=["auto", "bf16", "fp8_e4m3", "int8_per_token_head", "fp8_per_token_head"],
+                    help="KV-cache storage of the driver under test (the headline run keeps bf16)")
     ap.add_argument("--no-extra", action="store_true")
     ap.add_argument("--model", default="llama8b-w4a16", choices=["llama8b-w4a16", *OTHER_MODELS])
     ap.add_argument("--sampler", default="greedy", choices=["greedy", "top_p", "top_k", "min_p", "multinomial"],
@@ -384,7 +404,7 @@ def main():
     pages_per_ctx = (args.prompt + max_new + page_size - 1) // page_size
     total_pages = pages_per_ctx * args.batch + 8
     model, label = (MODEL, None) if args.model == "llama8b-w4a16" else OTHER_MODELS[args.model]
-    cfg_text = toml(model, page_size, total_pages, 2048, max(16, args.batch))
+    cfg_text = toml(model, page_size, total_pages, 2048, max(16, args.batch), args.kv_cache_dtype)
     hip = Hip()
     rng = np.random.default_rng(2048)
     prompt = rng.integers(0, model["vocab"], args.prompt)

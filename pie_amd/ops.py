@@ -732,8 +732,12 @@ def kv_write_quant(fmt: str, k_rows: torch.Tensor, v_rows: torch.Tensor, kv_slot
 def attention_rows_paged_kvq(fmt: str, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                              k_scales: Optional[torch.Tensor], v_scales: Optional[torch.Tensor],
                              kv_page_indices: torch.Tensor, row_page_begin: torch.Tensor,
-                             row_kv_len: torch.Tensor, lse: bool = False):
-    """Per-row paged attention over a one-byte KV pool.  q [rows, hq, d] bf16."""
+                             row_kv_len: torch.Tensor, lse: bool = False,
+                             max_kv_len: Optional[int] = None, o: Optional[torch.Tensor] = None,
+                             workspace: Optional[torch.Tensor] = None):
+    """Per-row paged attention over a one-byte KV pool.  q [rows, hq, d] bf16.  With
+    max_kv_len, o and workspace given the call neither synchronises nor allocates (graph
+    capture); the extents are then the caller's responsibility."""
     _dev(q, torch.bfloat16, "q")
     rows, hq, d = q.shape
     ps, hk = k_pages.shape[1], k_pages.shape[2]
@@ -744,18 +748,24 @@ def attention_rows_paged_kvq(fmt: str, q: torch.Tensor, k_pages: torch.Tensor, v
     _dev(row_kv_len, torch.int32, "row_kv_len")
     if rows == 0:
         return torch.empty_like(q), None
-    max_kv = int(row_kv_len.max())
-    npages = (row_kv_len.to(torch.int64) + ps - 1) // ps
-    if int((row_page_begin.to(torch.int64) + npages).max()) > kv_page_indices.numel():
-        raise KernelError("row extent runs past the page list")
-    if kv_page_indices.numel() and int(kv_page_indices.max()) >= k_pages.shape[0]:
-        raise KernelError("page id out of range")
-    o = torch.empty_like(q)
+    if max_kv_len is None:
+        max_kv = int(row_kv_len.max())
+        npages = (row_kv_len.to(torch.int64) + ps - 1) // ps
+        if int((row_page_begin.to(torch.int64) + npages).max()) > kv_page_indices.numel():
+            raise KernelError("row extent runs past the page list")
+        if kv_page_indices.numel() and int(kv_page_indices.max()) >= k_pages.shape[0]:
+            raise KernelError("page id out of range")
+    else:
+        max_kv = int(max_kv_len)
+    if o is None:
+        o = torch.empty_like(q)
     lse_t = torch.empty((rows, hq), dtype=torch.float32, device=q.device) if lse else None
     lib = kernels()
     lib.pie_hip_attn_decode_workspace_bytes.restype = C.c_size_t
     need = int(lib.pie_hip_attn_decode_workspace_bytes(rows, hq, hk, d, max_kv))
-    ws = torch.empty(max(need, 1), dtype=torch.uint8, device=q.device)
+    ws = workspace if workspace is not None else torch.empty(max(need, 1), dtype=torch.uint8, device=q.device)
+    if ws.numel() < need:
+        raise KernelError("workspace too small")
     _check(lib.pie_hip_attn_rows_paged_kvq(KV_FORMATS[fmt], _ptr(q), _ptr(k_pages), _ptr(v_pages),
                                            _ptr(k_scales), _ptr(v_scales), _ptr(o), _ptr(lse_t),
                                            _ptr(kv_page_indices), _ptr(row_page_begin), _ptr(row_kv_len),
