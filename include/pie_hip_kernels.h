@@ -186,6 +186,30 @@ int pie_hip_moe_grouped_gemm(int format, const uint16_t* act_bf16, const int32_t
                              uint16_t* y_bf16, int N, int K, int swiglu, void* stream);
 
 /*
+ * Tile-major weight layout for the skinny and grouped GEMMs.  The 16 bytes that lane (j, q) of a
+ * wave loads for the 16-row tile t and K block b — byte 64 b + 16 q of row 16 t + j in the
+ * row-major [N, K] matrix — are stored at byte ((t * nb + b) * 64 + 16 q + j) * 16, nb =
+ * row_bytes / 64, so every wave load is 1 KiB contiguous instead of 16 rows x 64 bytes (rows past
+ * N are zero; dst holds ceil(N/16) * 16 * row_bytes bytes).  int4 group scales [N, groups] become
+ * [tile][group][16 rows].  Built once at load; the values and their evaluation order are those of
+ * the row-major entry points, bit for bit.  Role in the reference: Marlin's offline weight
+ * repack (driver/cuda/third_party/marlin/marlin_wrapper.hpp:39-51).
+ */
+int pie_hip_repack_mfma_tiles(const void* src, void* dst, int N, size_t row_bytes, void* stream);
+int pie_hip_repack_scale_tiles(const uint16_t* src, uint16_t* dst, int N, int groups, void* stream);
+/* pie_hip_gemm_skinny / pie_hip_moe_grouped_gemm over weights (and int4 group scales) in that
+ * layout; every other argument as there (expert strides in bytes of the tiled buffers). */
+int pie_hip_gemm_skinny_tiled(int format, const uint16_t* act_bf16, const void* weight,
+                        const void* scale, int scale_is_bf16, int group_size, uint16_t* y_bf16,
+                        int M, int N, int K, int beta, int swiglu, void* stream);
+int pie_hip_moe_grouped_gemm_tiled(int format, const uint16_t* act_bf16, const int32_t* route_act_rows,
+                             const int32_t* expert_offsets, int num_experts,
+                             int max_rows_per_expert, const void* weights,
+                             size_t weight_stride_bytes, const void* scales,
+                             size_t scale_stride_bytes, int scale_is_bf16, int group_size,
+                             uint16_t* y_bf16, int N, int K, int swiglu, void* stream);
+
+/*
  * MoE routing: per token softmax over router_logits[t, 0..E) (bf16 in, fp32 inside), top_k by
  * repeated argmax with exclusion (ties to the lowest expert index), weights renormalised to
  * sum 1 — topk_softmax_bf16_kernel, driver/cuda/src/kernels/topk_softmax.cu:19-86 (graph form:

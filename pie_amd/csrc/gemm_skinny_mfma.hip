@@ -109,6 +109,7 @@ struct SkinnyArgs {
     int M;                      // rows when offsets == null
     int N, K, G, g_shift, beta, swiglu, scale_is_bf16;
     int m_split;                // dense only: blockIdx.y = 16-row pass
+    int tiled;                  // weights (and int4 group scales) in the tile-major layout
     size_t w_stride, scale_stride;  // bytes between problems
 };
 
@@ -154,22 +155,29 @@ __global__ __launch_bounds__(KP* kWave) void skinny_kernel(const SkinnyArgs a) {
     const unsigned char* wbase = a.w + static_cast<size_t>(p) * a.w_stride;
     const unsigned char* sbase = a.scale ? a.scale + static_cast<size_t>(p) * a.scale_stride : nullptr;
     const uint16_t* gsbase = reinterpret_cast<const uint16_t*>(sbase);
-    const int groups = F::kGroupScale ? K >> a.g_shift : 0;
     const int blk_shift = a.g_shift - (F::kGroupScale ? 7 : 0);   // 16-byte blocks per scale group, log2
+    // Weight addressing.  Row-major [N, K]: lane (j, q) reads 16 bytes of row 16*tile + j at byte
+    // 64*b + 16*q of the row.  Tile-major: the same 16 bytes sit at ((tile*nb + b)*64 + lane)*16,
+    // so one wave load is 1 KiB contiguous and consecutive b are consecutive KiB.
+    const int nb = K / LK;                      // 16-byte blocks along K per lane quad
+    const int groups = F::kGroupScale ? K >> a.g_shift : 0;
+    const size_t bstride = a.tiled ? 1024 : static_cast<size_t>(LK) * F::kBytesPer2K / 2;
+    const int gstride = a.tiled ? 16 : 1;       // int4 scales: tile-major [tile][group][16 rows]
     const unsigned char* wptr[NG];
-    int nrow[NG];
+    int nrow[NG];                               // (scale row offset)
     float row_scale[NG];
 #pragma unroll
     for (int i = 0; i < NG; ++i) {
-        const int n = min(min(tile0 + i, T - 1) * 16 + j, N - 1);
-        nrow[i] = n;
-        wptr[i] = wbase + static_cast<size_t>(n) * row_bytes + static_cast<size_t>(q) * KPL * F::kBytesPer2K / 2;
+        const int tile = min(tile0 + i, T - 1);
+        const int n = min(tile * 16 + j, N - 1);
+        nrow[i] = a.tiled ? tile * 16 * groups + j : n * groups;   // offset of the row's first group scale
+        wptr[i] = a.tiled ? wbase + static_cast<size_t>(tile) * nb * 1024 + static_cast<size_t>(lane) * 16
+                          : wbase + static_cast<size_t>(n) * row_bytes + static_cast<size_t>(q) * KPL * F::kBytesPer2K / 2;
         row_scale[i] = 1.f;
         if (!F::kGroupScale && sbase)
             row_scale[i] = a.scale_is_bf16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(sbase)[n])
                                            : reinterpret_cast<const float*>(sbase)[n];
     }
-    const int nb = K / LK;                      // 16-byte blocks along K per lane quad
     const int nchunks = (K + CK - 1) / CK;
     const bf16x8_t ones = __builtin_bit_cast(bf16x8_t, u32x4_t{0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u});
     const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
@@ -180,8 +188,8 @@ __global__ __launch_bounds__(KP* kWave) void skinny_kernel(const SkinnyArgs a) {
 #pragma unroll
         for (int h = 0; h < WL; ++h) {
             const int b = min(b0 + h, nb - 1);
-            sl.w[h] = *reinterpret_cast<const u32x4_t*>(wp + static_cast<size_t>(b) * LK * F::kBytesPer2K / 2);
-            sl.gs[h] = F::kGroupScale ? gsbase[static_cast<size_t>(n) * groups + (b >> blk_shift)] : uint16_t(0);
+            sl.w[h] = *reinterpret_cast<const u32x4_t*>(wp + static_cast<size_t>(b) * bstride);
+            sl.gs[h] = F::kGroupScale ? gsbase[static_cast<size_t>(n) + static_cast<size_t>(b >> blk_shift) * gstride] : uint16_t(0);
         }
         return sl;
     };
@@ -410,6 +418,37 @@ int launch_skinny(SkinnyArgs a, int problems, hipStream_t stream) {
     return launch_cfg<F, 4, CK, 1, 4, 1>(a, problems, stream);
 }
 
+// Tile-major weight layout: the 16 bytes lane (j, q) of a wave loads for tile t (rows 16t..16t+15)
+// and K block b — byte 64 b + 16 q of row 16 t + j — move to ((t*nb + b)*64 + 16 q + j)*16, so a
+// wave's load is 1 KiB contiguous.  One thread per 16-byte block of the destination; rows past N
+// are zero.
+__global__ __launch_bounds__(256) void repack_tiles_kernel(const u32x4_t* __restrict__ src,
+                                                           u32x4_t* __restrict__ dst, int N, int nb,
+                                                           size_t total) {
+    const size_t idx = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (idx >= total) return;
+    const int lane = static_cast<int>(idx & 63);
+    const size_t tb = idx >> 6;
+    const int b = static_cast<int>(tb % nb);
+    const size_t tile = tb / nb;
+    const size_t n = tile * 16 + (lane & 15);
+    u32x4_t v = {0u, 0u, 0u, 0u};
+    if (n < static_cast<size_t>(N)) v = src[n * (static_cast<size_t>(nb) * 4) + b * 4 + (lane >> 4)];
+    dst[idx] = v;
+}
+// int4 group scales [N, groups] -> [tile][group][16 rows]
+__global__ __launch_bounds__(256) void repack_scale_tiles_kernel(const uint16_t* __restrict__ src,
+                                                                 uint16_t* __restrict__ dst, int N,
+                                                                 int groups, size_t total) {
+    const size_t idx = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (idx >= total) return;
+    const int j = static_cast<int>(idx & 15);
+    const size_t tg = idx >> 4;
+    const int g = static_cast<int>(tg % groups);
+    const size_t n = (tg / groups) * 16 + j;
+    dst[idx] = n < static_cast<size_t>(N) ? src[n * groups + g] : uint16_t(0);
+}
+
 int dispatch_skinny(int format, const SkinnyArgs& a, int problems, hipStream_t st) {
     switch (format) {
         case PIE_HIP_FMT_INT4B8: return launch_skinny<SkInt4>(a, problems, st);
@@ -473,4 +512,81 @@ extern "C" int pie_hip_moe_grouped_gemm(int format, const uint16_t* act_bf16,
     a.w_stride = weight_stride_bytes;
     a.scale_stride = scale_stride_bytes;
     return dispatch_skinny(format, a, num_experts, static_cast<hipStream_t>(stream));
+}
+
+// ---- the same two entry points over weights in the tile-major layout ----------------------
+extern "C" int pie_hip_gemm_skinny_tiled(int format, const uint16_t* act_bf16, const void* weight,
+                                   const void* scale, int scale_is_bf16, int group_size,
+                                   uint16_t* y_bf16, int M, int N, int K, int beta, int swiglu,
+                                   void* stream) {
+    using namespace pie_hip;
+    if (!act_bf16 || !weight || !y_bf16 || M <= 0) return PIE_HIP_ERR_INVALID;
+    if (format != PIE_HIP_FMT_BF16 && !scale) return PIE_HIP_ERR_INVALID;
+    SkinnyArgs a{};
+    a.act = act_bf16;
+    a.w = static_cast<const unsigned char*>(weight);
+    a.scale = static_cast<const unsigned char*>(scale);
+    a.y = y_bf16;
+    a.M = M;
+    a.N = N;
+    a.K = K;
+    a.G = group_size;
+    a.beta = beta;
+    a.swiglu = swiglu ? 1 : 0;
+    a.scale_is_bf16 = scale_is_bf16;
+    a.tiled = 1;
+    return dispatch_skinny(format, a, 1, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int pie_hip_moe_grouped_gemm_tiled(int format, const uint16_t* act_bf16,
+                                        const int32_t* route_act_rows,
+                                        const int32_t* expert_offsets, int num_experts,
+                                        int max_rows_per_expert, const void* weights,
+                                        size_t weight_stride_bytes, const void* scales,
+                                        size_t scale_stride_bytes, int scale_is_bf16,
+                                        int group_size, uint16_t* y_bf16, int N, int K, int swiglu,
+                                        void* stream) {
+    using namespace pie_hip;
+    if (!act_bf16 || !expert_offsets || !weights || !y_bf16 || num_experts <= 0 ||
+        max_rows_per_expert <= 0)
+        return PIE_HIP_ERR_INVALID;
+    if (format != PIE_HIP_FMT_BF16 && !scales) return PIE_HIP_ERR_INVALID;
+    SkinnyArgs a{};
+    a.act = act_bf16;
+    a.act_rows = route_act_rows;
+    a.w = static_cast<const unsigned char*>(weights);
+    a.scale = static_cast<const unsigned char*>(scales);
+    a.y = y_bf16;
+    a.offsets = expert_offsets;
+    a.N = N;
+    a.K = K;
+    a.G = group_size;
+    a.swiglu = swiglu ? 1 : 0;
+    a.scale_is_bf16 = scale_is_bf16;
+    a.tiled = 1;
+    a.w_stride = weight_stride_bytes;
+    a.scale_stride = scale_stride_bytes;
+    return dispatch_skinny(format, a, num_experts, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int pie_hip_repack_mfma_tiles(const void* src, void* dst, int N, size_t row_bytes,
+                                         void* stream) {
+    if (!src || !dst || N <= 0 || row_bytes == 0) return PIE_HIP_ERR_INVALID;
+    if (row_bytes % 64 != 0) return PIE_HIP_ERR_UNSUPPORTED;
+    const int nb = static_cast<int>(row_bytes / 64);
+    const size_t total = static_cast<size_t>((N + 15) / 16) * nb * 64;
+    if ((total + 255) / 256 > 0x7FFFFFFFull) return PIE_HIP_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(pie_hip::repack_tiles_kernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256),
+                       0, static_cast<hipStream_t>(stream), static_cast<const pie_hip::u32x4_t*>(src),
+                       static_cast<pie_hip::u32x4_t*>(dst), N, nb, total);
+    return pie_hip::launch_status();
+}
+
+extern "C" int pie_hip_repack_scale_tiles(const uint16_t* src, uint16_t* dst, int N, int groups,
+                                          void* stream) {
+    if (!src || !dst || N <= 0 || groups <= 0) return PIE_HIP_ERR_INVALID;
+    const size_t total = static_cast<size_t>((N + 15) / 16) * groups * 16;
+    hipLaunchKernelGGL(pie_hip::repack_scale_tiles_kernel, dim3(static_cast<unsigned>((total + 255) / 256)),
+                       dim3(256), 0, static_cast<hipStream_t>(stream), src, dst, N, groups, total);
+    return pie_hip::launch_status();
 }

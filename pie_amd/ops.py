@@ -363,10 +363,30 @@ def linear_fused(act: torch.Tensor, w: WeightView, norm_weight: Optional[torch.T
     return y
 
 
+def repack_mfma_tiles(w: WeightView) -> WeightView:
+    """The weight (and int4 group scales) in the skinny GEMM's tile-major layout: a WeightView
+    whose kind carries the suffix '+tiled' for gemm_skinny / moe_grouped_gemm."""
+    rows = w.data.shape[0] if w.data.dim() == 2 else w.data.shape[0] * w.data.shape[1]
+    flat = w.data.reshape(rows, -1).contiguous()
+    row_bytes = flat.shape[1] * flat.element_size()
+    dst = torch.empty(((rows + 15) // 16 * 16, flat.shape[1]), dtype=flat.dtype, device=flat.device)
+    _check(kernels().pie_hip_repack_mfma_tiles(_ptr(flat), _ptr(dst), rows, C.c_size_t(row_bytes), _stream()),
+           "pie_hip_repack_mfma_tiles")
+    scale = w.scale
+    if w.kind == "int4b8":
+        sf = w.scale.reshape(rows, -1).contiguous()
+        _dev(sf, torch.bfloat16, "scale")
+        scale = torch.empty(((rows + 15) // 16 * 16, sf.shape[1]), dtype=torch.bfloat16, device=sf.device)
+        _check(kernels().pie_hip_repack_scale_tiles(_ptr(sf), _ptr(scale), rows, sf.shape[1], _stream()),
+               "pie_hip_repack_scale_tiles")
+    return WeightView(w.kind + "+tiled", dst, scale, w.group_size, w.N, w.K)
+
+
 def gemm_skinny(act: torch.Tensor, w: WeightView, y: Optional[torch.Tensor] = None, beta: int = 0,
                 swiglu: bool = False) -> torch.Tensor:
     """Matrix-core weight-only GEMM for a handful to a few dozen activation rows (same contract as
-    `linear_fused` without the norm)."""
+    `linear_fused` without the norm).  A WeightView from repack_mfma_tiles runs the tile-major
+    entry point."""
     _dev(act, torch.bfloat16, "act")
     M, K = act.shape
     if K != w.K:
@@ -380,9 +400,10 @@ def gemm_skinny(act: torch.Tensor, w: WeightView, y: Optional[torch.Tensor] = No
     if tuple(y.shape) != (M, n_out):
         raise KernelError("y shape mismatch")
     scale_is_bf16 = int(w.scale is not None and w.scale.dtype == torch.bfloat16)
-    st = kernels().pie_hip_gemm_skinny(FMT[w.kind], _ptr(act), _ptr(w.data), _ptr(w.scale),
-                                       scale_is_bf16, w.group_size, _ptr(y), M, w.N, K, beta,
-                                       int(swiglu), _stream())
+    tiled = w.kind.endswith("+tiled")
+    fn = kernels().pie_hip_gemm_skinny_tiled if tiled else kernels().pie_hip_gemm_skinny
+    st = fn(FMT[w.kind.split("+")[0]], _ptr(act), _ptr(w.data), _ptr(w.scale), scale_is_bf16, w.group_size,
+            _ptr(y), M, w.N, K, beta, int(swiglu), _stream())
     _check(st, "pie_hip_gemm_skinny")
     return y
 
@@ -391,7 +412,8 @@ def moe_grouped_gemm(act: torch.Tensor, route_act_rows: Optional[torch.Tensor],
                      expert_offsets: torch.Tensor, kind: str, weights: torch.Tensor,
                      scales: Optional[torch.Tensor], N: int, K: int, rows_hint: int,
                      group_size: int = 0, swiglu: bool = False,
-                     y: Optional[torch.Tensor] = None, num_routes: Optional[int] = None) -> torch.Tensor:
+                     y: Optional[torch.Tensor] = None, num_routes: Optional[int] = None,
+                     tiled: bool = False) -> torch.Tensor:
     """One skinny GEMM per expert in a single launch.  `weights` is [E, N, K] in the format's
     element type (int4b8: [E, N, K/8] words), `scales` [E, N] (int4b8: [E, N, K/G]);
     `expert_offsets` int32 [E+1] are the first route row of each expert (routes sorted by expert);
@@ -420,7 +442,8 @@ def moe_grouped_gemm(act: torch.Tensor, route_act_rows: Optional[torch.Tensor],
     wstride = weights[0].numel() * weights.element_size()
     sstride = 0 if scales is None else scales[0].numel() * scales.element_size()
     scale_is_bf16 = int(scales is not None and scales.dtype == torch.bfloat16)
-    st = kernels().pie_hip_moe_grouped_gemm(
+    fn = kernels().pie_hip_moe_grouped_gemm_tiled if tiled else kernels().pie_hip_moe_grouped_gemm
+    st = fn(
         FMT[kind], _ptr(act), _ptr(route_act_rows), _ptr(expert_offsets), E, int(rows_hint),
         _ptr(weights), C.c_size_t(wstride), _ptr(scales), C.c_size_t(sstride), scale_is_bf16,
         group_size, _ptr(y), N, K, int(swiglu), _stream())

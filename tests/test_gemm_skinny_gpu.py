@@ -146,3 +146,73 @@ def test_moe_grouped_gemm_matches_per_expert_oracle(gpu, oracle, kind, swiglu):
     assert got.shape == ref.shape
     assert close_to_oracle(oracle, got, ref, rel=2.0 ** -6)
     assert (ulp_diff(got, ref) <= 1).mean() > 0.97
+
+
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("N,K", [(80, 1024), (100, 512), (12304, 512)])
+def test_tile_major_repack_is_the_documented_permutation(gpu, oracle, kind, N, K):
+    """dst[((t*nb + b)*64 + 16q + j)*16 ..] = the 16 bytes at byte 64b + 16q of row 16t + j; rows
+    past N are zero; int4 group scales become [tile][group][16]."""
+    import torch
+    from pie_amd import ops
+
+    rng = np.random.default_rng(330 + N)
+    wd, mk = make_weight(oracle, rng, kind, N, K)
+    w = mk(gpu)
+    t = ops.repack_mfma_tiles(w)
+    src = w.data.contiguous().view(torch.uint8).cpu().numpy().reshape(N, -1)
+    row_bytes = src.shape[1]
+    nb, tiles = row_bytes // 64, (N + 15) // 16
+    padded = np.zeros((tiles * 16, row_bytes), np.uint8)
+    padded[:N] = src
+    want = padded.reshape(tiles, 16, nb, 4, 16).transpose(0, 2, 3, 1, 4)      # [t][b][q][j][16 bytes]
+    assert np.array_equal(t.data.view(torch.uint8).cpu().numpy().reshape(-1), want.reshape(-1))
+    if kind == "int4b8":
+        sc = w.scale.view(torch.uint16).cpu().numpy()
+        ps = np.zeros((tiles * 16, sc.shape[1]), np.uint16)
+        ps[:N] = sc
+        want_s = ps.reshape(tiles, 16, -1).transpose(0, 2, 1)                 # [t][g][j]
+        assert np.array_equal(t.scale.view(torch.uint16).cpu().numpy().reshape(-1), want_s.reshape(-1))
+
+
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("M,N,K", [(5, 64, 512), (16, 256, 4096), (17, 100, 2048), (45, 48, 512),
+                                   (8, 12304, 512), (20, 24592, 512)])
+def test_skinny_over_tile_major_weights_is_bit_identical(gpu, oracle, kind, M, N, K):
+    """Same values, same evaluation order: only the addresses of the weight loads change."""
+    import torch
+    from pie_amd import ops
+
+    rng = np.random.default_rng(340 + M + N)
+    wd, mk = make_weight(oracle, rng, kind, N, K)
+    w = mk(gpu)
+    x = dev(oracle.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32)), gpu, torch.bfloat16)
+    a = bits(ops.gemm_skinny(x, w))
+    b = bits(ops.gemm_skinny(x, ops.repack_mfma_tiles(w)))
+    assert np.array_equal(a, b)
+    assert close_to_oracle(oracle, b, oracle_linear(oracle, wd, bits(x)))
+
+
+@pytest.mark.parametrize("kind", ["fp8", "int4b8", "bf16"])
+@pytest.mark.parametrize("swiglu", [False, True])
+def test_moe_grouped_gemm_over_tile_major_experts_is_bit_identical(gpu, oracle, kind, swiglu):
+    import torch
+    from pie_amd import ops
+
+    rng = np.random.default_rng(350)
+    E, N, K, T = 6, 96, 512, 20
+    counts = np.array([3, 0, 21, 1, 0, 7])
+    offs = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    rows = rng.integers(0, T, size=int(offs[-1])).astype(np.int32)
+    x = dev(oracle.f32_to_bf16(rng.standard_normal((T, K)).astype(np.float32)), gpu, torch.bfloat16)
+    views = [make_weight(oracle, rng, kind, N, K)[1](gpu) for _ in range(E)]
+    wstack = torch.stack([v.data for v in views]).contiguous()
+    sstack = None if views[0].scale is None else torch.stack([v.scale for v in views]).contiguous()
+    args = dict(rows_hint=16, group_size=views[0].group_size, swiglu=swiglu)
+    a = bits(ops.moe_grouped_gemm(x, dev(rows, gpu), dev(offs, gpu), kind, wstack, sstack, N, K, **args))
+    tiled = ops.repack_mfma_tiles(ops.WeightView(kind, wstack, sstack, views[0].group_size, E * N, K))
+    ws = tiled.data.reshape(E, N, -1)
+    ss = tiled.scale if kind != "int4b8" else tiled.scale.reshape(E, N, -1)
+    ss = sstack if kind != "int4b8" else ss
+    b = bits(ops.moe_grouped_gemm(x, dev(rows, gpu), dev(offs, gpu), kind, ws, ss, N, K, tiled=True, **args))
+    assert np.array_equal(a, b)
