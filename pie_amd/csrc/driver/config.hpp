@@ -59,6 +59,9 @@ struct BatchingConfig {
 struct RuntimeConfig {
     bool verbose = false;
     bool use_graphs = true;
+    // a second copy of every decoder linear in the skinny GEMM's tile-major layout (doubles the
+    // weight memory, ~25 % off the 5-32-row and MoE grouped GEMMs)
+    bool tiled_weights = true;
     std::string snapshot_dir;
 };
 
@@ -238,6 +241,7 @@ inline DriverConfig parse_config_text(const std::string& text) {
                 auto& r = c.runtime;
                 if (k == "verbose") r.verbose = to_bool(v, key);
                 else if (k == "use_graphs") r.use_graphs = to_bool(v, key);
+                else if (k == "tiled_weights") r.tiled_weights = to_bool(v, key);
                 else if (k == "snapshot_dir") r.snapshot_dir = v;
             }
         }

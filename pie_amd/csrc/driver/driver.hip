@@ -241,6 +241,7 @@ struct PieHipDriver {
         try {
             if (cfg.model.checkpoint_dir.empty()) model.init_synthetic(cfg.model, s);
             else model.load_snapshot(cfg.model, s);
+            if (cfg.runtime.tiled_weights) model.build_tiled_copies(s);
         } catch (...) {
             (void)hipStreamDestroy(s);
             throw;

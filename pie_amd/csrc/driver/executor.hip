@@ -52,8 +52,8 @@ int fmt_code(Quant q) {
 }
 
 // Measured cost models (MI355X, microseconds, int4 8B-class shapes at 16-128 rows).  Skinny GEMM:
-// ~5 us + the weights at ~2.8 TB/s for the first 16-row pass, each further (side-by-side) pass
-// adding 85 % of that stream.  Tiled GEMM: K in 64-wide steps of ~0.72 us with 64-row block
+// ~5 us + the weights at ~2.8 TB/s (3.3 TB/s from the tile-major copy) for the first 16-row pass,
+// each further (side-by-side) pass adding 85 % (80 %) of that stream.  Tiled GEMM: K in 64-wide steps of ~0.72 us with 64-row block
 // tiles (M <= 64), ~0.98 us with 128-row tiles, while the tiles fit the machine (512 resident
 // blocks).  Split-K tiled GEMM: the steps of one share (+3 of prologue) at 1.25 / 1.6 us with two
 // blocks per CU, per round of 512 blocks, plus ~15 us for the second kernel and the partials.
@@ -61,7 +61,9 @@ enum class GemmPath { Skinny, Tiled, TiledSplitK };
 GemmPath pick_gemm(const Linear& w, int M, size_t ws_bytes) {
     if (w.K % 64 != 0 || M < 17) return GemmPath::Skinny;
     const int passes = (M + 15) / 16;
-    const double skinny = 5.0 + static_cast<double>(w.data_bytes()) / 2.8e6 * (1.0 + 0.85 * (passes - 1));
+    const double skinny = w.data_tiled
+                              ? 5.0 + static_cast<double>(w.data_bytes()) / 3.3e6 * (1.0 + 0.80 * (passes - 1))
+                              : 5.0 + static_cast<double>(w.data_bytes()) / 2.8e6 * (1.0 + 0.85 * (passes - 1));
     const int steps = w.K / 64;
     const double tiles = static_cast<double>((w.N + 127) / 128) * (M <= 64 ? 1 : (M + 127) / 128);
     const double tiled = 2.0 + steps * (M <= 64 ? 0.72 : 0.98) * std::max(1.0, tiles / 512.0);
@@ -105,8 +107,11 @@ void linear_fused(const Linear& w, const uint16_t* act, const uint16_t* norm_w, 
             if (sg == PIE_HIP_OK) return;
             if (sg != PIE_HIP_ERR_UNSUPPORTED) PIE_KERNEL(sg);
         }
-        const int st = pie_hip_gemm_skinny(fmt, a, w.data, w.scale, sbf, w.group, y, M, w.N, w.K,
-                                           beta, swiglu, s);
+        const int st = w.data_tiled
+                           ? pie_hip_gemm_skinny_tiled(fmt, a, w.data_tiled, w.scale_tiled ? w.scale_tiled : w.scale,
+                                                       sbf, w.group, y, M, w.N, w.K, beta, swiglu, s)
+                           : pie_hip_gemm_skinny(fmt, a, w.data, w.scale, sbf, w.group, y, M, w.N, w.K, beta,
+                                                 swiglu, s);
         if (st == PIE_HIP_OK) return;
         if (st != PIE_HIP_ERR_UNSUPPORTED) PIE_KERNEL(st);
         PIE_KERNEL(pie_hip_linear_fused(fmt, a, nullptr, eps, w.data, w.scale, sbf, w.group, y, M,
@@ -312,13 +317,17 @@ void Executor::moe_block(const LayerWeights& w, int N, hipStream_t s) {
     PIE_KERNEL(pie_hip_moe_route(moe_logits_, moe_idx_, moe_w_, moe_offsets_, moe_route_token_,
                                  moe_route_pos_, N, E, K, s));
     const int hint = std::max(1, std::min(N, 2 * ((N * K + E - 1) / E)));
-    PIE_KERNEL(pie_hip_moe_grouped_gemm(fmt, xn_, moe_route_token_, moe_offsets_, E, hint, w.wgu.data,
-                                        w.wgu.data_bytes() / E, w.wgu.scale, w.wgu.scale_bytes() / E,
-                                        sbf, w.wgu.group, act_, 2 * Ie, H, 1, s));
-    PIE_KERNEL(pie_hip_moe_grouped_gemm(fmt, act_, nullptr, moe_offsets_, E, hint, w.wdown.data,
-                                        w.wdown.data_bytes() / E, w.wdown.scale,
-                                        w.wdown.scale_bytes() / E, sbf, w.wdown.group, moe_y_, H, Ie,
-                                        0, s));
+    // experts stacked along the rows: the tile-major copy of the stack keeps expert e at the same
+    // byte stride (every expert has a multiple of 16 rows)
+    const bool tiled = w.wgu.data_tiled && w.wdown.data_tiled && (2 * Ie) % 16 == 0 && H % 16 == 0;
+    auto grouped = tiled ? pie_hip_moe_grouped_gemm_tiled : pie_hip_moe_grouped_gemm;
+    auto wptr = [&](const Linear& l) { return tiled ? l.data_tiled : l.data; };
+    auto sptr = [&](const Linear& l) { return tiled && l.scale_tiled ? l.scale_tiled : l.scale; };
+    PIE_KERNEL(grouped(fmt, xn_, moe_route_token_, moe_offsets_, E, hint, wptr(w.wgu),
+                       w.wgu.data_bytes() / E, sptr(w.wgu), w.wgu.scale_bytes() / E, sbf, w.wgu.group,
+                       act_, 2 * Ie, H, 1, s));
+    PIE_KERNEL(grouped(fmt, act_, nullptr, moe_offsets_, E, hint, wptr(w.wdown), w.wdown.data_bytes() / E,
+                       sptr(w.wdown), w.wdown.scale_bytes() / E, sbf, w.wdown.group, moe_y_, H, Ie, 0, s));
     PIE_KERNEL(pie_hip_moe_combine(moe_y_, moe_route_pos_, moe_w_, x_, N, K, H, 1, s));
 }
 

@@ -112,6 +112,26 @@ Model::~Model() {
     for (void* p : allocs_) (void)hipFree(p);
 }
 
+void Model::build_tiled_copies(hipStream_t stream) {
+    for (LayerWeights& l : layers)
+        for (Linear* w : {&l.wqkv, &l.wo, &l.wgu, &l.wdown}) {
+            if (!w->data || w->data_tiled || w->N <= 0 || w->N % 16 != 0) continue;
+            const size_t row_bytes = w->data_bytes() / static_cast<size_t>(w->N);
+            if (row_bytes % 64 != 0) continue;
+            w->data_tiled = alloc(w->data_bytes(), "");
+            if (pie_hip_repack_mfma_tiles(w->data, w->data_tiled, w->N, row_bytes, stream) != PIE_HIP_OK)
+                throw std::runtime_error("model: weight repack failed");
+            if (w->kind == Quant::Int4b8) {
+                w->scale_tiled = alloc(w->scale_bytes(), "");
+                if (pie_hip_repack_scale_tiles(static_cast<const uint16_t*>(w->scale),
+                                               static_cast<uint16_t*>(w->scale_tiled), w->N, w->K / w->group,
+                                               stream) != PIE_HIP_OK)
+                    throw std::runtime_error("model: scale repack failed");
+            }
+        }
+    PIE_HIP_CHECK(hipStreamSynchronize(stream));
+}
+
 void* Model::alloc(size_t bytes, const std::string& name) {
     void* p = nullptr;
     PIE_HIP_CHECK(hipMalloc(&p, bytes ? bytes : 16));

@@ -31,6 +31,9 @@ struct Linear {
     void* scale = nullptr;  // int4: bf16 [N, K/G]; int8/fp8: f32 or bf16 [N]; bf16: null
     bool scale_bf16 = true;
     int N = 0, K = 0, group = 0;
+    // optional copies in the skinny GEMM's tile-major layout (pie_hip_repack_mfma_tiles)
+    void* data_tiled = nullptr;
+    void* scale_tiled = nullptr;   // int4 group scales; other formats keep `scale`
     size_t data_bytes() const {
         const size_t nk = static_cast<size_t>(N) * K;
         switch (kind) {
@@ -78,6 +81,9 @@ class Model {
     // quantised on the device to cfg.quant; compressed-tensors int4 checkpoints
     // (`weight_packed` int32 [N, K/8] + `weight_scale` [N, K/group]) are taken as stored.
     void load_snapshot(const ModelConfig& cfg, hipStream_t stream);
+
+    // Builds the tile-major copies of every decoder linear whose shape the skinny GEMM takes.
+    void build_tiled_copies(hipStream_t stream);
 
     const ModelConfig& cfg() const { return cfg_; }
     bool is_moe() const { return cfg_.arch == "qwen3_moe"; }
