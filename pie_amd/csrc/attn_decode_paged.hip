@@ -358,6 +358,238 @@ __global__ __launch_bounds__(kAttnBlock) void attn_decode_split_kernel(
     }
 }
 
+// ---- the same split on the matrix cores (bf16 pools, no custom mask) ------------------------
+// One block = one (row, kv head, split) as above; each of the four waves walks every fourth
+// 32-key step of the split on its own (own K/V loads, own LDS region, own online-softmax state;
+// no block barrier inside the loop):
+//   S^T[key, query] = K . Q^T      A = K rows straight from HBM in the operand layout (lane l16 =
+//                                  key, k = 8 consecutive d), B = the GQA query heads of the row
+//                                  in the first GQA of 16 columns (the rest are zero)
+//   O^T[d, query]  += V^T . P^T    A = V^T from the wave's LDS region, B = P from registers
+// The query sits on the lane%16 axis of both accumulators, so max / sum / rescale are per lane
+// and cost two cross-lane steps per 32 keys instead of four per key and head.  The keys of a
+// step leave the first product in the order [4g..4g+3, 16+4g..16+4g+3] per 16-lane group g —
+// the order V^T is laid out in LDS (rows padded to 80 B: conflict-free operand reads).
+// Probabilities enter the second product as a bf16 pair (hi + lo), i.e. with 16 mantissa bits,
+// so the result keeps the accuracy of the fp32 kernel above.
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+constexpr int kMStepKeys = 32;
+constexpr int kMVtStride = kMStepKeys + 8;
+
+template <int D, int GQA>
+__global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
+    const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_pages,
+    const uint16_t* __restrict__ v_pages, const uint32_t* __restrict__ page_indices,
+    const uint32_t* __restrict__ page_indptr, const uint32_t* __restrict__ last_lens,
+    const uint32_t* __restrict__ row_begin, const int32_t* __restrict__ row_len,
+    float* __restrict__ part_o, float* __restrict__ part_ml, uint16_t* __restrict__ o_direct,
+    float* __restrict__ lse, int hq, int hk, int ps, int ps_shift, int units_per_split, int nsplit,
+    float scale_log2e) {
+    constexpr int KS = D / 32;                 // k steps of the first product
+    constexpr int DT = D / 16;                 // d tiles of the second product
+    constexpr int LPR = D / 8;                 // 16-byte pieces per K/V row
+    constexpr int VC = 16 * LPR / kWave;       // (key pair, piece) combos per lane per step
+    constexpr int PF = 2;                      // steps of K/V in flight per wave
+    static_assert(GQA <= 16 && VC >= 1, "shape");
+    __shared__ __attribute__((aligned(16))) uint16_t vt_all[kAttnWaves][D * kMVtStride];
+    __shared__ float sm_m[kAttnWaves][16];
+    __shared__ float sm_l[kAttnWaves][16];
+    static_assert(sizeof(float) * GQA * D <= sizeof(uint16_t) * D * kMVtStride, "per-wave output fits its V^T region");
+
+    const int kvh = blockIdx.x, split = blockIdx.y, r = blockIdx.z;
+    const int tid = threadIdx.x, lane = tid & (kWave - 1);
+    const int wv = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const int l16 = lane & 15, g = lane >> 4;
+
+    const RowExtent ext = row_extent(page_indptr, last_lens, row_begin, row_len, r, ps);
+    const uint32_t pg_lo = ext.pg_lo;
+    const int kv_len = ext.kv_len;
+    const int nunits = (kv_len + kUnitTokens - 1) / kUnitTokens;
+    const int u_begin = split * units_per_split;
+    if (u_begin >= nunits) return;
+    const int k_begin = u_begin * kUnitTokens;
+    const int k_end = min(min(u_begin + units_per_split, nunits) * kUnitTokens, kv_len);
+
+    // Q^T fragment: column l16 = query head l16 of this kv head's group (zero beyond GQA)
+    bf16x8_t qf[KS];
+    {
+        const bool valid = l16 < GQA;
+        const uint16_t* qp = q + (static_cast<size_t>(r) * hq + kvh * GQA + (valid ? l16 : 0)) * D + 8 * g;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            u32x4_t v = *reinterpret_cast<const u32x4_t*>(qp + 32 * ks);
+            if (!valid) v = u32x4_t{0u, 0u, 0u, 0u};
+            qf[ks] = __builtin_bit_cast(bf16x8_t, v);
+        }
+    }
+
+    uint16_t* Vt = vt_all[wv];
+    u32x4_t kreg[PF][2 * KS], vreg[PF][2 * VC];
+    // A 32-key step starts on a multiple of 16 and touches at most two pages (page_size % 16 == 0);
+    // their ids come through scalar loads.  Keys past the split repeat its last key (finite
+    // data; their probabilities are zero).
+    auto issue = [&](int slot, int j0) {
+        const int ja = min(j0, k_end - 1);
+        const int page_a = ps_shift >= 0 ? ja >> ps_shift : ja / ps;
+        const int pa_end = (page_a + 1) * ps;
+        const int jb = min(j0 + kMStepKeys - 1, k_end - 1);
+        const uint32_t pid_a = __builtin_amdgcn_readfirstlane(page_indices[pg_lo + page_a]);
+        const uint32_t pid_b = __builtin_amdgcn_readfirstlane(page_indices[pg_lo + page_a + (jb >= pa_end ? 1 : 0)]);
+        auto row_off = [&](int key) {
+            const int j = min(j0 + key, k_end - 1);
+            const bool in_a = j < pa_end;
+            const size_t slot_idx = static_cast<size_t>(in_a ? pid_a : pid_b) * ps + (j - (in_a ? pa_end - ps : pa_end));
+            return (slot_idx * hk + kvh) * D;
+        };
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt) {
+            const size_t off = row_off(16 * nt + l16) + 8 * g;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+                kreg[slot][nt * KS + ks] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(k_pages + off + 32 * ks));
+        }
+#pragma unroll
+        for (int c = 0; c < VC; ++c) {
+            const int pidx = lane + kWave * c;
+            const int pair = pidx & 15, dc = pidx >> 4;
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+                vreg[slot][2 * c + u] = __builtin_nontemporal_load(
+                    reinterpret_cast<const u32x4_t*>(v_pages + row_off(2 * pair + u) + dc * 8));
+        }
+    };
+    // V rows -> V^T in the wave's LDS region: two adjacent keys of one piece meet in one lane and
+    // leave as 4-byte writes (slot of key kappa: 8*(kappa%16/4) + kappa%4, +4 for kappa >= 16)
+    auto stage = [&](int slot) {
+#pragma unroll
+        for (int c = 0; c < VC; ++c) {
+            const int pidx = lane + kWave * c;
+            const int pair = pidx & 15, dc = pidx >> 4;
+            const int kappa = 2 * pair;
+            const int col = kappa < 16 ? 8 * (kappa >> 2) + (kappa & 3) : 8 * ((kappa - 16) >> 2) + 4 + (kappa & 3);
+            const u32x4_t a = vreg[slot][2 * c], b = vreg[slot][2 * c + 1];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const uint32_t lo = (a[e >> 1] >> (16 * (e & 1))) & 0xFFFFu;
+                const uint32_t hi = (b[e >> 1] >> (16 * (e & 1))) & 0xFFFFu;
+                *reinterpret_cast<uint32_t*>(&Vt[(dc * 8 + e) * kMVtStride + col]) = lo | (hi << 16);
+            }
+        }
+    };
+
+    f32x4_t acc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) acc[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    float mx = -INFINITY, lsum = 0.f;
+
+    constexpr int kStride = kAttnWaves * kMStepKeys;   // keys between two steps of one wave
+    auto step = [&](int slot, int j0) {
+        stage(slot);
+        f32x4_t st[2] = {f32x4_t{0.f, 0.f, 0.f, 0.f}, f32x4_t{0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+            for (int nt = 0; nt < 2; ++nt)
+                st[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                    __builtin_bit_cast(bf16x8_t, kreg[slot][nt * KS + ks]), qf[ks], st[nt], 0, 0, 0);
+        if (j0 + PF * kStride < k_end) issue(slot, j0 + PF * kStride);
+
+        // online softmax of query l16 over this lane's keys 16nt + 4g + r
+        float sv[8];
+        float m_new = mx;
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) {
+                const int key = j0 + 16 * nt + 4 * g + rr;
+                const float v = key < k_end ? st[nt][rr] * scale_log2e : -INFINITY;
+                sv[4 * nt + rr] = v;
+                m_new = fmaxf(m_new, v);
+            }
+        m_new = fmaxf(m_new, __shfl_xor(m_new, 16, kWave));
+        m_new = fmaxf(m_new, __shfl_xor(m_new, 32, kWave));
+        const float safe = m_new == -INFINITY ? 0.f : m_new;
+        const float alpha = exp2f(mx - safe);
+        mx = m_new;
+        float sum = 0.f;
+        uint32_t hi[4], lo[4];
+#pragma unroll
+        for (int e = 0; e < 8; e += 2) {
+            const float p0 = exp2f(sv[e] - safe), p1 = exp2f(sv[e + 1] - safe);
+            sum += p0 + p1;
+            // p = hi + lo with both parts bf16: hi by truncation, lo = bf16(p - hi)
+            const uint32_t b0 = __float_as_uint(p0) & 0xFFFF0000u, b1 = __float_as_uint(p1) & 0xFFFF0000u;
+            hi[e >> 1] = (b0 >> 16) | b1;
+            lo[e >> 1] = pack_bf16x2(p0 - __uint_as_float(b0), p1 - __uint_as_float(b1));
+        }
+        lsum = lsum * alpha + sum;
+        if (__any(alpha != 1.0f)) {
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) acc[dt] *= alpha;
+        }
+        const bf16x8_t p_hi = __builtin_bit_cast(bf16x8_t, u32x4_t{hi[0], hi[1], hi[2], hi[3]});
+        const bf16x8_t p_lo = __builtin_bit_cast(bf16x8_t, u32x4_t{lo[0], lo[1], lo[2], lo[3]});
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            const bf16x8_t vf = __builtin_bit_cast(
+                bf16x8_t, *reinterpret_cast<const u32x4_t*>(&Vt[(16 * dt + l16) * kMVtStride + 8 * g]));
+            acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, p_hi, acc[dt], 0, 0, 0);
+            acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, p_lo, acc[dt], 0, 0, 0);
+        }
+    };
+
+    const int first = k_begin + wv * kMStepKeys;
+    if (first < k_end) issue(0, first);
+    if (first + kStride < k_end) issue(1, first + kStride);
+    for (int j0 = first; j0 < k_end; j0 += PF * kStride) {
+        step(0, j0);
+        if (j0 + kStride < k_end) step(1, j0 + kStride);
+    }
+
+    // this wave's result into its own LDS region (as floats), then the four waves are merged
+    lsum += __shfl_xor(lsum, 16, kWave);
+    lsum += __shfl_xor(lsum, 32, kWave);
+    float* so = reinterpret_cast<float*>(Vt);   // [GQA][D]
+    if (l16 < GQA) {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) so[l16 * D + 16 * dt + 4 * g + rr] = acc[dt][rr];
+        if (g == 0) {
+            sm_m[wv][l16] = mx;
+            sm_l[wv][l16] = lsum;
+        }
+    }
+    __syncthreads();
+    for (int idx = tid; idx < GQA * D; idx += kAttnBlock) {
+        const int h = idx / D, dd = idx - h * D;
+        float m_all = sm_m[0][h];
+#pragma unroll
+        for (int w = 1; w < kAttnWaves; ++w) m_all = fmaxf(m_all, sm_m[w][h]);
+        const float safe = (m_all == -INFINITY) ? 0.f : m_all;
+        float ov = 0.f, ls = 0.f;
+#pragma unroll
+        for (int w = 0; w < kAttnWaves; ++w) {
+            const float a = exp2f(sm_m[w][h] - safe);
+            ov += reinterpret_cast<const float*>(vt_all[w])[h * D + dd] * a;
+            ls += sm_l[w][h] * a;
+        }
+        const int head = kvh * GQA + h;
+        const size_t rh = static_cast<size_t>(r) * hq + head;
+        if (o_direct) {
+            o_direct[rh * D + dd] = f32_to_bf16_bits(ls > 0.f ? ov / ls : 0.f);
+            if (lse && dd == 0)
+                lse[rh] = ls > 0.f ? (logf(ls) + m_all * 0.6931471805599453f) : -INFINITY;
+        } else {
+            part_o[(rh * nsplit + split) * D + dd] = ov;
+            if (dd == 0) {
+                part_ml[(rh * nsplit + split) * 2 + 0] = m_all;
+                part_ml[(rh * nsplit + split) * 2 + 1] = ls;
+            }
+        }
+    }
+}
+
 // One block per (request, q head): combine the splits that exist for this request.  Two
 // parallel phases instead of a serial walk over splits: (1) the (max, sum) pairs of all splits
 // are loaded at once and reduced to per-split weights in LDS, (2) each thread sums its output
@@ -472,6 +704,43 @@ int launch_decode(const uint16_t* q, const void* k_pages, const void* v_pages,
                   int mask_stride, hipStream_t stream) {
     const SplitPlan plan = plan_splits(R, hk, max_kv_len);
     const float scale_log2e = sm_scale * 1.4426950408889634f;
+    if constexpr (!MASKED && KVF == kKvBf16) {
+        // bf16 pools without a custom mask.  Measured (MI355X, 8B / 30B-A3B decode steps): the
+        // matrix-core kernel wins with eight query heads per kv head (MoE batch 64: 9.07 against
+        // 9.78 ms per step) and for small batches (batch 1: 1.815 against 1.860 ms, batch 16 even);
+        // with four heads per kv head and many rows the dot-product kernel's whole-row loads win
+        // (batch 64: 7.75 against 8.52 ms; 4.96 against 4.04 TB/s on 64 rows of 512-8192 keys).
+        // PIE_HIP_ATTN_VALU = 1 / 0 forces one or the other (measurement hook).
+        static const int forced = [] { const char* e = getenv("PIE_HIP_ATTN_VALU"); return e ? (atoi(e) ? 1 : 0) : -1; }();
+        const bool mfma = forced >= 0 ? forced == 0 : (GQA >= 8 || R <= 16);
+        if (mfma) {
+            const int ps_shift = (ps & (ps - 1)) == 0 ? __builtin_ctz(static_cast<unsigned>(ps)) : -1;
+            const uint16_t* kp = static_cast<const uint16_t*>(k_pages);
+            const uint16_t* vp = static_cast<const uint16_t*>(v_pages);
+            if (plan.nsplit == 1) {
+                hipLaunchKernelGGL((attn_decode_clear_empty_kernel<D>), dim3(R * hq), dim3(D), 0, stream,
+                                   page_indptr, last_lens, row_begin, row_len, o, lse, hq, ps);
+                hipLaunchKernelGGL((attn_decode_mfma_kernel<D, GQA>), dim3(hk, 1, R), dim3(kAttnBlock), 0,
+                                   stream, q, kp, vp, page_indices, page_indptr, last_lens, row_begin, row_len,
+                                   nullptr, nullptr, o, lse, hq, hk, ps, ps_shift, plan.units_per_split, 1,
+                                   scale_log2e);
+                return launch_status();
+            }
+            const size_t n_part = static_cast<size_t>(R) * hq * plan.nsplit;
+            const size_t need = n_part * (D + 2) * sizeof(float);
+            if (!workspace || workspace_bytes < need) return PIE_HIP_ERR_INVALID;
+            float* part_o = static_cast<float*>(workspace);
+            float* part_ml = part_o + n_part * D;
+            hipLaunchKernelGGL((attn_decode_mfma_kernel<D, GQA>), dim3(hk, plan.nsplit, R), dim3(kAttnBlock), 0,
+                               stream, q, kp, vp, page_indices, page_indptr, last_lens, row_begin, row_len,
+                               part_o, part_ml, nullptr, nullptr, hq, hk, ps, ps_shift, plan.units_per_split,
+                               plan.nsplit, scale_log2e);
+            hipLaunchKernelGGL((attn_decode_merge_kernel<D>), dim3(R * hq), dim3(D), 0, stream, part_o,
+                               part_ml, page_indptr, last_lens, row_begin, row_len, o, lse, hq, ps,
+                               plan.units_per_split, plan.nsplit);
+            return launch_status();
+        }
+    }
     if (plan.nsplit == 1) {
         hipLaunchKernelGGL((attn_decode_clear_empty_kernel<D>), dim3(R * hq), dim3(D), 0, stream,
                            page_indptr, last_lens, row_begin, row_len, o, lse, hq, ps);

@@ -205,7 +205,11 @@ def test_rows_with_custom_masks_match_oracle(gpu, oracle, hq, hk, d):
         lg = lse.cpu().numpy()
         assert np.array_equal(np.isneginf(lg), ~fin) and np.allclose(lg[fin], lse64[fin], atol=1e-4)
         assert not allow[3].any() and np.all(got[3] == 0)          # runs end before any visible key
-    # no masks, no window: bit-identical to the unmasked entry point
-    plain = ops.attention_rows_paged(*args)
-    masked = ops.attention_rows_paged(*args, mask_runs=[[]] * len(rows))
-    assert torch.equal(plain.view(torch.uint16), masked.view(torch.uint16))
+    # no masks, no window: the unmasked entry point's result (that one runs the matrix-core
+    # kernel, the masked one the dot-product kernel: same values to a bf16 step)
+    plain = ops.attention_rows_paged(*args).view(torch.uint16).cpu().numpy().astype(np.int32)
+    masked = ops.attention_rows_paged(*args, mask_runs=[[]] * len(rows)).view(torch.uint16).cpu().numpy().astype(np.int32)
+    same_sign = (plain >> 15) == (masked >> 15)
+    assert (np.abs(plain - masked)[same_sign] <= 1).mean() > 0.99
+    pf, mf = oracle.bf16_to_f32(plain.astype(np.uint16)), oracle.bf16_to_f32(masked.astype(np.uint16))
+    assert np.all(np.abs(pf - mf) <= 2.0 ** -7 * np.maximum(np.abs(pf), np.abs(mf)) + 2e-4)
