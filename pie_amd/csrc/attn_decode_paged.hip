@@ -362,9 +362,9 @@ __global__ __launch_bounds__(kAttnBlock) void attn_decode_split_kernel(
 // One block = one (row, kv head, split) as above; each of the four waves walks every fourth
 // 32-key step of the split on its own (own K/V loads, own LDS region, own online-softmax state;
 // no block barrier inside the loop):
-//   S^T[key, query] = K . Q^T      A = K rows straight from HBM in the operand layout (lane l16 =
-//                                  key, k = 8 consecutive d), B = the GQA query heads of the row
-//                                  in the first GQA of 16 columns (the rest are zero)
+//   S^T[key, query] = K . Q^T      A = K fragment from the wave's LDS region (row = key, k = d; rows
+//                                  padded to D + 8), B = the GQA query heads of the row in the
+//                                  first GQA of 16 columns (the rest are zero)
 //   O^T[d, query]  += V^T . P^T    A = V^T from the wave's LDS region, B = P from registers
 // The query sits on the lane%16 axis of both accumulators, so max / sum / rescale are per lane
 // and cost two cross-lane steps per 32 keys instead of four per key and head.  The keys of a
@@ -391,7 +391,9 @@ __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
     constexpr int VC = 16 * LPR / kWave;       // (key pair, piece) combos per lane per step
     constexpr int PF = 2;                      // steps of K/V in flight per wave
     static_assert(GQA <= 16 && VC >= 1, "shape");
+    constexpr int KSTRIDE = D + 8;             // bf16 elements per K row in LDS (padded: conflict-free reads)
     __shared__ __attribute__((aligned(16))) uint16_t vt_all[kAttnWaves][D * kMVtStride];
+    __shared__ __attribute__((aligned(16))) uint16_t ks_all[kAttnWaves][kMStepKeys * KSTRIDE];
     __shared__ float sm_m[kAttnWaves][16];
     __shared__ float sm_l[kAttnWaves][16];
     static_assert(sizeof(float) * GQA * D <= sizeof(uint16_t) * D * kMVtStride, "per-wave output fits its V^T region");
@@ -424,7 +426,14 @@ __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
     }
 
     uint16_t* Vt = vt_all[wv];
+    uint16_t* Ks = ks_all[wv];
+    // K loads: whole rows, LPR adjacent lanes per key (kWave / LPR keys per instruction)
+    constexpr int KPI = kWave / LPR;
     u32x4_t kreg[PF][2 * KS], vreg[PF][2 * VC];
+    // V loads: combo c of a lane = (key pair, 16-byte piece); eight adjacent lanes take eight
+    // adjacent pieces (128 contiguous bytes of a row)
+    auto v_piece = [&](int c) { return (lane & 7) + 8 * (c % (LPR / 8)); };
+    auto v_pair = [&](int c) { return (lane >> 3) + 8 * (c / (LPR / 8)); };
     // A 32-key step starts on a multiple of 16 and touches at most two pages (page_size % 16 == 0);
     // their ids come through scalar loads.  Keys past the split repeat its last key (finite
     // data; their probabilities are zero).
@@ -442,16 +451,12 @@ __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
             return (slot_idx * hk + kvh) * D;
         };
 #pragma unroll
-        for (int nt = 0; nt < 2; ++nt) {
-            const size_t off = row_off(16 * nt + l16) + 8 * g;
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks)
-                kreg[slot][nt * KS + ks] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(k_pages + off + 32 * ks));
-        }
+        for (int i = 0; i < 2 * KS; ++i)
+            kreg[slot][i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(
+                k_pages + row_off(lane / LPR + KPI * i) + (lane % LPR) * 8));
 #pragma unroll
         for (int c = 0; c < VC; ++c) {
-            const int pidx = lane + kWave * c;
-            const int pair = pidx & 15, dc = pidx >> 4;
+            const int pair = v_pair(c), dc = v_piece(c);
 #pragma unroll
             for (int u = 0; u < 2; ++u)
                 vreg[slot][2 * c + u] = __builtin_nontemporal_load(
@@ -462,9 +467,11 @@ __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
     // leave as 4-byte writes (slot of key kappa: 8*(kappa%16/4) + kappa%4, +4 for kappa >= 16)
     auto stage = [&](int slot) {
 #pragma unroll
+        for (int i = 0; i < 2 * KS; ++i)
+            *reinterpret_cast<u32x4_t*>(&Ks[(lane / LPR + KPI * i) * KSTRIDE + (lane % LPR) * 8]) = kreg[slot][i];
+#pragma unroll
         for (int c = 0; c < VC; ++c) {
-            const int pidx = lane + kWave * c;
-            const int pair = pidx & 15, dc = pidx >> 4;
+            const int pair = v_pair(c), dc = v_piece(c);
             const int kappa = 2 * pair;
             const int col = kappa < 16 ? 8 * (kappa >> 2) + (kappa & 3) : 8 * ((kappa - 16) >> 2) + 4 + (kappa & 3);
             const u32x4_t a = vreg[slot][2 * c], b = vreg[slot][2 * c + 1];
@@ -491,7 +498,9 @@ __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
 #pragma unroll
             for (int nt = 0; nt < 2; ++nt)
                 st[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                    __builtin_bit_cast(bf16x8_t, kreg[slot][nt * KS + ks]), qf[ks], st[nt], 0, 0, 0);
+                    __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(
+                                                     &Ks[(16 * nt + l16) * KSTRIDE + 32 * ks + 8 * g])),
+                    qf[ks], st[nt], 0, 0, 0);
         if (j0 + PF * kStride < k_end) issue(slot, j0 + PF * kStride);
 
         // online softmax of query l16 over this lane's keys 16nt + 4g + r
@@ -705,14 +714,13 @@ int launch_decode(const uint16_t* q, const void* k_pages, const void* v_pages,
     const SplitPlan plan = plan_splits(R, hk, max_kv_len);
     const float scale_log2e = sm_scale * 1.4426950408889634f;
     if constexpr (!MASKED && KVF == kKvBf16) {
-        // bf16 pools without a custom mask.  Measured (MI355X, 8B / 30B-A3B decode steps): the
-        // matrix-core kernel wins with eight query heads per kv head (MoE batch 64: 9.07 against
-        // 9.78 ms per step) and for small batches (batch 1: 1.815 against 1.860 ms, batch 16 even);
-        // with four heads per kv head and many rows the dot-product kernel's whole-row loads win
-        // (batch 64: 7.75 against 8.52 ms; 4.96 against 4.04 TB/s on 64 rows of 512-8192 keys).
+        // bf16 pools without a custom mask run on the matrix cores.  Measured (MI355X, 8B / 30B-A3B
+        // decode steps, four / eight query heads per kv head), matrix-core against dot-product
+        // kernel: batch 1 1.808 / 1.860 ms, batch 8 2.68 / 2.80, batch 32 4.07 / 4.13, batch 64 at
+        // 2048 keys 7.53 / 7.72, MoE batch 64 7.98 / 8.80; 64 rows of 512-8192 keys 5.61 / 4.96 TB/s.
         // PIE_HIP_ATTN_VALU = 1 / 0 forces one or the other (measurement hook).
         static const int forced = [] { const char* e = getenv("PIE_HIP_ATTN_VALU"); return e ? (atoi(e) ? 1 : 0) : -1; }();
-        const bool mfma = forced >= 0 ? forced == 0 : (GQA >= 8 || R <= 16);
+        const bool mfma = forced >= 0 ? forced == 0 : true;
         if (mfma) {
             const int ps_shift = (ps & (ps - 1)) == 0 ? __builtin_ctz(static_cast<unsigned>(ps)) : -1;
             const uint16_t* kp = static_cast<const uint16_t*>(k_pages);
