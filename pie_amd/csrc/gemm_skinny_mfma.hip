@@ -47,6 +47,17 @@ struct SkInt4 {
     static constexpr int kPerLane = 32, kSteps = 4, kBytesPer2K = 1;
     static constexpr float kBias = -136.f;
     static constexpr bool kGroupScale = true;
+    // (128.0bf16, 128.0bf16) held in a VGPR for and_or: made once per kernel, opaque to the compiler
+    static __device__ __forceinline__ uint32_t magic() {
+        uint32_t k128 = 0x43004300u;
+        asm volatile("" : "+v"(k128));
+        return k128;
+    }
+    static __device__ __forceinline__ u32x4_t decode(const u32x4_t w, int s, uint32_t k128) {
+        const uint32_t v = w[s];
+        return u32x4_t{and_or(v, 0x000F000Fu, k128), and_or(v >> 4, 0x000F000Fu, k128),
+                       and_or(v >> 8, 0x000F000Fu, k128), and_or(v >> 12, 0x000F000Fu, k128)};
+    }
     static __device__ __forceinline__ u32x4_t decode(const u32x4_t w, int s) {
         uint32_t k128 = 0x43004300u;
         asm volatile("" : "+v"(k128));
@@ -66,6 +77,8 @@ struct SkFp8 {
     static constexpr int kPerLane = 16, kSteps = 2, kBytesPer2K = 2;
     static constexpr float kBias = 0.f;
     static constexpr bool kGroupScale = false;
+    static __device__ __forceinline__ uint32_t magic() { return 0u; }
+    static __device__ __forceinline__ u32x4_t decode(const u32x4_t w, int s, uint32_t) { return decode(w, s); }
     static __device__ __forceinline__ u32x4_t decode(const u32x4_t w, int s) {
         const uint32_t a = w[2 * s], b = w[2 * s + 1];
         const f32x2_t a0 = __builtin_amdgcn_cvt_pk_f32_fp8(a, false);
@@ -85,6 +98,8 @@ struct SkInt8 {
         return pack_hi16(static_cast<float>((u >> lo_shift) & 0xFFu),
                          static_cast<float>((u >> (lo_shift + 8)) & 0xFFu));
     }
+    static __device__ __forceinline__ uint32_t magic() { return 0u; }
+    static __device__ __forceinline__ u32x4_t decode(const u32x4_t w, int s, uint32_t) { return decode(w, s); }
     static __device__ __forceinline__ u32x4_t decode(const u32x4_t w, int s) {
         const uint32_t a = w[2 * s] ^ 0x80808080u, b = w[2 * s + 1] ^ 0x80808080u;
         return u32x4_t{two(a, 0), two(a, 16), two(b, 0), two(b, 16)};
@@ -95,6 +110,8 @@ struct SkBf16 {
     static constexpr int kPerLane = 8, kSteps = 1, kBytesPer2K = 4;
     static constexpr float kBias = 0.f;
     static constexpr bool kGroupScale = false;
+    static __device__ __forceinline__ uint32_t magic() { return 0u; }
+    static __device__ __forceinline__ u32x4_t decode(const u32x4_t w, int, uint32_t) { return w; }
     static __device__ __forceinline__ u32x4_t decode(const u32x4_t w, int) { return w; }
     static __device__ __forceinline__ u32x4_t order(const u32x4_t v) { return v; }
 };
@@ -124,7 +141,7 @@ struct WSlot {
 // KP waves split K; CK k-values of activations per LDS chunk; NG tiles of 16 weight rows per
 // block; PW ring slots of WL adjacent 16-byte weight blocks in flight per lane (WL = 2: a
 // wave's two loads of a step cover whole 128-byte lines of each of its 16 rows).
-template <class F, int KP, int CK, int NG, int PW, int WL>
+template <class F, int KP, int CK, int NG, int PW, int WL, bool TILED>
 __global__ __launch_bounds__(KP* kWave) void skinny_kernel(const SkinnyArgs a) {
     constexpr int KPL = F::kPerLane, S = F::kSteps;
     constexpr int LK = 4 * KPL;               // k covered by one wave-wide 16-byte load
@@ -161,18 +178,22 @@ __global__ __launch_bounds__(KP* kWave) void skinny_kernel(const SkinnyArgs a) {
     // so one wave load is 1 KiB contiguous and consecutive b are consecutive KiB.
     const int nb = K / LK;                      // 16-byte blocks along K per lane quad
     const int groups = F::kGroupScale ? K >> a.g_shift : 0;
-    const size_t bstride = a.tiled ? 1024 : static_cast<size_t>(LK) * F::kBytesPer2K / 2;
-    const int gstride = a.tiled ? 16 : 1;       // int4 scales: tile-major [tile][group][16 rows]
+    constexpr size_t bstride = TILED ? 1024 : static_cast<size_t>(LK) * F::kBytesPer2K / 2;
+    constexpr int gstride = TILED ? 16 : 1;     // int4 scales: tile-major [tile][group][16 rows]
+    // tile-major: everything but the lane's own 16 bytes (2 bytes of a scale row) is uniform
+    // over the wave, so the addresses are scalar bases plus one constant vector offset
     const unsigned char* wptr[NG];
     int nrow[NG];                               // (scale row offset)
+    const unsigned lane16 = TILED ? static_cast<unsigned>(lane) * 16u : 0u;
+    const unsigned j2 = TILED ? static_cast<unsigned>(j) : 0u;
     float row_scale[NG];
 #pragma unroll
     for (int i = 0; i < NG; ++i) {
         const int tile = min(tile0 + i, T - 1);
         const int n = min(tile * 16 + j, N - 1);
-        nrow[i] = a.tiled ? tile * 16 * groups + j : n * groups;   // offset of the row's first group scale
-        wptr[i] = a.tiled ? wbase + static_cast<size_t>(tile) * nb * 1024 + static_cast<size_t>(lane) * 16
-                          : wbase + static_cast<size_t>(n) * row_bytes + static_cast<size_t>(q) * KPL * F::kBytesPer2K / 2;
+        nrow[i] = TILED ? tile * 16 * groups : n * groups;   // offset of the row's first group scale
+        wptr[i] = TILED ? wbase + static_cast<size_t>(tile) * nb * 1024
+                        : wbase + static_cast<size_t>(n) * row_bytes + static_cast<size_t>(q) * KPL * F::kBytesPer2K / 2;
         row_scale[i] = 1.f;
         if (!F::kGroupScale && sbase)
             row_scale[i] = a.scale_is_bf16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(sbase)[n])
@@ -188,8 +209,8 @@ __global__ __launch_bounds__(KP* kWave) void skinny_kernel(const SkinnyArgs a) {
 #pragma unroll
         for (int h = 0; h < WL; ++h) {
             const int b = min(b0 + h, nb - 1);
-            sl.w[h] = *reinterpret_cast<const u32x4_t*>(wp + static_cast<size_t>(b) * bstride);
-            sl.gs[h] = F::kGroupScale ? gsbase[static_cast<size_t>(n) + static_cast<size_t>(b >> blk_shift) * gstride] : uint16_t(0);
+            sl.w[h] = *reinterpret_cast<const u32x4_t*>(wp + static_cast<size_t>(b) * bstride + lane16);
+            sl.gs[h] = F::kGroupScale ? (gsbase + static_cast<size_t>(n) + static_cast<size_t>(b >> blk_shift) * gstride)[j2] : uint16_t(0);
         }
         return sl;
     };
@@ -368,20 +389,293 @@ __global__ __launch_bounds__(KP* kWave) void skinny_kernel(const SkinnyArgs a) {
     }
 }
 
-template <class F, int KP, int CK, int NG, int PW, int WL>
-int launch_cfg(const SkinnyArgs& a, int problems, hipStream_t stream) {
+// ---- wave-private form (tile-major weights) -------------------------------------------------
+// The form above shares each staged activation chunk among the waves of a block and pays two
+// block barriers per chunk; with four waves splitting K that also caps a CU at a few waves.
+// Here a wave owns its work outright: NG tiles of 16 weight rows times one contiguous K slice,
+// its own LDS region for the activations of that slice (256 k-values at a time, loaded one
+// chunk ahead into registers), its own ring of weight loads.  Nothing synchronises inside the
+// K loop; the KP = 1 << kp_shift waves that share a tile group meet once, in LDS, at the end.
+// A block is kSwWaves waves = kSwWaves / KP tile groups.
+constexpr int kSwWaves = 8;
+constexpr int kSwChunk = 256;                       // k-values per staged chunk
+constexpr int kSwStride = kSwChunk / 8 + 1;         // 16-byte vectors per staged row (padded)
+constexpr int kSwRegion = 16 * kSwStride;           // vectors per wave region
+
+struct WOne {
+    u32x4_t w;
+    uint16_t gs;
+};
+
+template <class F, int NG>
+__global__ __launch_bounds__(kSwWaves* kWave, NG == 1 ? 4 : 2) void skinny_wave_kernel(const SkinnyArgs a, const int kp_shift) {
+    constexpr int KPL = F::kPerLane, S = F::kSteps;
+    constexpr int LK = 4 * KPL;                     // k covered by one wave-wide 16-byte load (a block)
+    constexpr int CB = kSwChunk / LK;               // blocks per chunk
+    constexpr int NS = NG * CB;                     // steps per chunk, tile-major order
+    constexpr int PF = NS < 8 ? NS : 8;             // weight loads in flight per lane (deeper rings cost the occupancy that pays more)
+    constexpr int CU = NS >= PF ? 1 : PF / NS;      // chunks per trip: ring slots stay compile-time
+    constexpr int SV = kSwRegion / kSwStride * (kSwChunk / 8) / kWave;   // staged vectors per lane and chunk
+    constexpr bool kBiased = F::kBias != 0.f;
+    constexpr bool kRowBias = kBiased && !F::kGroupScale;
+    static_assert((NS % PF == 0 || PF % NS == 0) && SV == 8, "ring and staging shapes");
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int tid = threadIdx.x, lane = tid & (kWave - 1);
+    const int wv = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const int j = lane & 15, q = lane >> 4;
+    u32x4_t* lds_a = reinterpret_cast<u32x4_t*>(smem) + wv * kSwRegion;
+    float* red = reinterpret_cast<float*>(smem);
+    constexpr int kRegionF = kSwRegion * 4;
+    const int KP = 1 << kp_shift;
+    const int ks = wv & (KP - 1);
+    const int N = a.N, K = a.K;
+    const int p = a.offsets ? blockIdx.y : 0;
+    const int r0 = a.offsets ? a.offsets[p] : (a.m_split ? blockIdx.y * 16 : 0);
+    const int r1 = a.offsets ? a.offsets[p + 1] : (a.m_split ? min(a.M, r0 + 16) : a.M);
+    if (r1 <= r0) return;
+
+    const int T = (N + 15) / 16;
+    const int tile0 = (blockIdx.x * (kSwWaves >> kp_shift) + (wv >> kp_shift)) * NG;
+    const unsigned char* wbase = a.w + static_cast<size_t>(p) * a.w_stride;
+    const unsigned char* sbase = a.scale ? a.scale + static_cast<size_t>(p) * a.scale_stride : nullptr;
+    const uint16_t* gsbase = reinterpret_cast<const uint16_t*>(sbase);
+    const int blk_shift = a.g_shift - (F::kGroupScale ? 7 : 0);
+    const int nb = K / LK;
+    const int groups = F::kGroupScale ? K >> a.g_shift : 0;
+    // this wave's K slice, in whole chunks
+    const int nch_all = nb / CB;                    // the launcher takes whole chunks only
+    const int per = (nch_all + KP - 1) >> kp_shift;
+    const int ch_lo = ks * per;
+    const int nch = max(0, min(nch_all, ch_lo + per) - ch_lo);
+    const int b_lo = ch_lo * CB;
+
+    const unsigned char* wt[NG];
+    const uint16_t* st[NG];
+    float row_scale[NG];
+#pragma unroll
+    for (int i = 0; i < NG; ++i) {
+        const int tile = min(tile0 + i, T - 1);
+        wt[i] = wbase + static_cast<size_t>(tile) * nb * 1024;
+        st[i] = gsbase + static_cast<size_t>(tile) * 16 * groups;
+        row_scale[i] = 1.f;
+        const int n = min(tile * 16 + j, N - 1);
+        if (!F::kGroupScale && sbase)
+            row_scale[i] = a.scale_is_bf16 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(sbase)[n])
+                                           : reinterpret_cast<const float*>(sbase)[n];
+    }
+    const unsigned lane16 = static_cast<unsigned>(lane) * 16u;
+    const uint32_t magic = F::magic();
+    const bf16x8_t ones = __builtin_bit_cast(bf16x8_t, u32x4_t{0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u});
+    const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
+
+    // step `lin` of chunk c: tile lin / CB, block lin % CB of the chunk
+    auto load_w = [&](int c, int lin) {
+        const int b = min(b_lo + c * CB + lin % CB, nb - 1);
+        WOne sl;
+        sl.w = *reinterpret_cast<const u32x4_t*>(wt[lin / CB] + static_cast<size_t>(b) * 1024 + lane16);
+        sl.gs = F::kGroupScale ? (st[lin / CB] + static_cast<size_t>(b >> blk_shift) * 16)[j] : uint16_t(0);
+        return sl;
+    };
+
+    // staging: a wave-wide load covers 512 bytes of each of two activation rows
+    const int srow = lane >> 5, svec = lane & 31;
+
+    for (int mt0 = r0; mt0 < r1; mt0 += 16) {
+        int arow[SV];   // rows past the problem repeat its last row and are never stored
+#pragma unroll
+        for (int u = 0; u < SV; ++u) {
+            const int row = min(mt0 + srow + 2 * u, r1 - 1);
+            arow[u] = a.act_rows ? a.act_rows[row] : row;
+        }
+        u32x4_t stg[SV];
+        auto stage_load = [&](int c) {
+            const int k0 = min((b_lo + c * CB) * LK + svec * 8, K - 8);
+#pragma unroll
+            for (int u = 0; u < SV; ++u)
+                stg[u] = *reinterpret_cast<const u32x4_t*>(a.act + static_cast<size_t>(arow[u]) * K + k0);
+        };
+        auto stage_store = [&]() {
+#pragma unroll
+            for (int u = 0; u < SV; ++u) lds_a[(srow + 2 * u) * kSwStride + svec] = F::order(stg[u]);
+        };
+
+        f32x4_t acc[NG], sxs[F::kGroupScale ? CB : 1], sxt = zero4;
+#pragma unroll
+        for (int i = 0; i < NG; ++i) acc[i] = zero4;
+
+        WOne ring[PF];
+#pragma unroll
+        for (int l = 0; l < PF; ++l) ring[l] = load_w(l / NS, l % NS);
+        stage_load(0);
+        stage_store();
+
+        auto step = [&](const WOne& cur, int ng, int blk) {
+            const int vbase = blk * (LK / 8) + q * S;
+            const int sxi = F::kGroupScale ? blk : 0;
+            bf16x8_t ax[S];
+#pragma unroll
+            for (int s = 0; s < S; ++s) ax[s] = __builtin_bit_cast(bf16x8_t, lds_a[j * kSwStride + vbase + s]);
+            f32x4_t part = zero4;
+#pragma unroll
+            for (int s = 0; s < S; ++s) {
+                const bf16x8_t bw = __builtin_bit_cast(bf16x8_t, F::decode(cur.w, s, magic));
+                if (kBiased && ng == 0) {
+                    if (F::kGroupScale)
+                        sxs[sxi] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax[s], ones, s == 0 ? zero4 : sxs[sxi], 0, 0, 0);
+                    else
+                        sxt = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax[s], ones, sxt, 0, 0, 0);
+                }
+                if (F::kGroupScale)
+                    part = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax[s], bw, part, 0, 0, 0);
+                else
+                    acc[ng] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax[s], bw, acc[ng], 0, 0, 0);
+            }
+            if (F::kGroupScale) {
+                if (ng == 0) sxs[sxi] = sxs[sxi] * F::kBias;
+                const float sc = bf16_bits_to_f32(cur.gs);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[ng][r] = fmaf(sc, part[r] + sxs[sxi][r], acc[ng][r]);
+            }
+        };
+
+        for (int c0 = 0; c0 < nch; c0 += CU) {
+#pragma unroll
+            for (int cu = 0; cu < CU; ++cu) {
+                const int c = c0 + cu;
+                stage_load(c + 1);   // (past the slice: a clamped, unused repeat)
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int lin = 0; lin < NS; ++lin) {
+                    const int slot = (cu * NS + lin) % PF;
+                    // consume the slot, then refill it (a ring ahead of its next use).  In this
+                    // order the old and the new value never live at once, so the slot keeps its
+                    // registers around the loop; refilling first makes the compiler copy the ring
+                    // at the loop end, which waits for every load in flight.  The scheduling
+                    // barriers keep the order (left alone, the scheduler also gathers all loads
+                    // of a chunk behind all of its arithmetic).
+                    step(ring[slot], lin / CB, lin % CB);   // K is whole chunks: no step is partial
+                    __builtin_amdgcn_sched_barrier(0);
+                    ring[slot] = load_w(c + (lin + PF) / NS, (lin + PF) % NS);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                stage_store();
+            }
+        }
+
+        // ---- the KP waves of a tile group meet; work item (tile i, accumulator row rr) ----
+        __syncthreads();
+        float* mine = red + static_cast<size_t>(wv) * kRegionF;
+#pragma unroll
+        for (int i = 0; i < NG; ++i)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) mine[(i * 4 + r) * kWave + lane] = acc[i][r];
+        if (kRowBias) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) mine[(NG * 4 + r) * kWave + lane] = sxt[r];
+        }
+        __syncthreads();
+        const float* grp = red + static_cast<size_t>(wv - ks) * kRegionF;
+        auto total = [&](int item, int rr) {
+            float v = 0.f;
+            for (int w = 0; w < KP; ++w) v += grp[static_cast<size_t>(w) * kRegionF + (item * 4 + rr) * kWave + lane];
+            return v;
+        };
+        const int nout = a.swiglu ? N / 2 : N;
+        for (int id = ks; id < NG * 4; id += KP) {
+            const int i = id >> 2, rr = id & 3;
+            const int m = mt0 + 4 * q + rr;
+            const float bias = kRowBias ? F::kBias * total(NG, rr) : 0.f;
+            float rs = row_scale[0];
+#pragma unroll
+            for (int t = 1; t < NG; ++t) rs = i == t ? row_scale[t] : rs;
+            const int n = (tile0 + i) * 16 + j;
+            const bool ok = m < r1 && n < N;
+            float v = (total(i, rr) + bias) * rs;
+            if (a.swiglu) {
+                const float gb = bf16_bits_to_f32(f32_to_bf16_bits(v));
+                const float other = __int_as_float(__builtin_amdgcn_update_dpp(
+                    0, __float_as_int(gb), 0xB1, 0xF, 0xF, true));  // quad_perm [1,0,3,2]
+                if ((j & 1) == 0 && ok) {
+                    const float silu = gb / (1.f + expf(-gb));
+                    a.y[static_cast<size_t>(m) * nout + n / 2] = f32_to_bf16_bits(silu * other);
+                }
+            } else if (ok) {
+                const size_t o = static_cast<size_t>(m) * nout + n;
+                if (a.beta) v += bf16_bits_to_f32(a.y[o]);
+                a.y[o] = f32_to_bf16_bits(v);
+            }
+        }
+        __syncthreads();   // the regions go back to staging
+    }
+}
+
+template <class F, int NG>
+int launch_wave_cfg(const SkinnyArgs& a, int problems, int kp_shift, hipStream_t stream) {
+    constexpr size_t smem = static_cast<size_t>(kSwWaves) * kSwRegion * 16;
+    static const hipError_t attr = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(&skinny_wave_kernel<F, NG>),
+        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
+    if (attr != hipSuccess) return PIE_HIP_ERR_LAUNCH;
+    const int tgroups = ((a.N + 15) / 16 + NG - 1) / NG;
+    const int per_block = kSwWaves >> kp_shift;
+    const dim3 grid((tgroups + per_block - 1) / per_block, a.m_split ? (a.M + 15) / 16 : problems);
+    hipLaunchKernelGGL((skinny_wave_kernel<F, NG>), grid, dim3(kSwWaves * kWave), smem, stream, a, kp_shift);
+    return launch_status();
+}
+
+// Tiles per wave and K split: the most tiles per wave (activation staging and the bias MFMAs
+// are paid once per chunk, whatever the tile count) that still gives the machine about eight
+// waves per CU.
+template <class F>
+int launch_wave(const SkinnyArgs& a, int problems, hipStream_t stream) {
+    constexpr int LK = 4 * F::kPerLane, CB = kSwChunk / LK;
+    const int nch_all = (a.K / LK + CB - 1) / CB;
+    const long mult = a.m_split ? (a.M + 15) / 16 : problems;
+    const long tiles = (a.N + 15) / 16;
+    static const int force_ng = [] { const char* e = getenv("PIE_SKINNY_NG"); return e ? atoi(e) : 0; }();
+    static const int force_kp = [] { const char* e = getenv("PIE_SKINNY_KP"); return e ? atoi(e) : -1; }();
+    constexpr long kWant = 2048;
+    int ng = 1, kp_shift = 3;
+    for (int cand = 4; cand >= 1; cand >>= 1) {
+        const long groups = (tiles + cand - 1) / cand * mult;
+        int sh = 0;
+        while (sh < 3 && (groups << sh) * 4 < kWant * 3) ++sh;
+        while (sh > 0 && (1 << sh) > nch_all) --sh;
+        if ((groups << sh) * 4 >= kWant * 3 || cand == 1) {
+            ng = cand;
+            kp_shift = sh;
+            break;
+        }
+    }
+    if (force_ng) ng = force_ng;
+    if (force_kp >= 0) kp_shift = force_kp;
+    switch (ng) {
+        case 4: return launch_wave_cfg<F, 4>(a, problems, kp_shift, stream);
+        case 2: return launch_wave_cfg<F, 2>(a, problems, kp_shift, stream);
+        default: return launch_wave_cfg<F, 1>(a, problems, kp_shift, stream);
+    }
+}
+
+template <class F, int KP, int CK, int NG, int PW, int WL, bool TILED>
+int launch_cfg_t(const SkinnyArgs& a, int problems, hipStream_t stream) {
     constexpr bool kRowBias = F::kBias != 0.f && !F::kGroupScale;
     constexpr size_t kStage = static_cast<size_t>(16) * (CK / 8 + 1) * 16;
     constexpr size_t kRed = static_cast<size_t>(KP) * (NG + (kRowBias ? 1 : 0)) * 4 * kWave * sizeof(float);
     constexpr size_t smem = kStage > kRed ? kStage : kRed;
     static const hipError_t attr = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(&skinny_kernel<F, KP, CK, NG, PW, WL>),
+        reinterpret_cast<const void*>(&skinny_kernel<F, KP, CK, NG, PW, WL, TILED>),
         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
     if (attr != hipSuccess) return PIE_HIP_ERR_LAUNCH;
     const int tiles = (a.N + 15) / 16;
     const dim3 grid((tiles + NG - 1) / NG, a.m_split ? (a.M + 15) / 16 : problems);
-    hipLaunchKernelGGL((skinny_kernel<F, KP, CK, NG, PW, WL>), grid, dim3(KP * kWave), smem, stream, a);
+    hipLaunchKernelGGL((skinny_kernel<F, KP, CK, NG, PW, WL, TILED>), grid, dim3(KP * kWave), smem, stream, a);
     return launch_status();
+}
+
+template <class F, int KP, int CK, int NG, int PW, int WL>
+int launch_cfg(const SkinnyArgs& a, int problems, hipStream_t stream) {
+    return a.tiled ? launch_cfg_t<F, KP, CK, NG, PW, WL, true>(a, problems, stream)
+                   : launch_cfg_t<F, KP, CK, NG, PW, WL, false>(a, problems, stream);
 }
 
 template <class F>
@@ -408,6 +702,12 @@ int launch_skinny(SkinnyArgs a, int problems, hipStream_t stream) {
     // and wave) when K allows.
     const long tiles = static_cast<long>((a.N + 15) / 16) * (a.m_split ? (a.M + 15) / 16 : problems);
     constexpr int W8 = (CK / (8 * LK) >= 2) ? 2 : 1;   // loads per step with eight waves
+    static const bool old_form = getenv("PIE_SKINNY_OLD") != nullptr;
+    // dense tile-major launches take the wave-private form (measured, 8B decode steps of 8 / 16 /
+    // 32 / 64 rows: 2.43 / 2.78 / 3.42 / 5.18 ms against 2.75 / 2.95 / 4.07 / 5.64); the grouped
+    // MoE launches stay with the block-shared form, whose eight tiles per staged chunk halve the
+    // activation traffic (30B-A3B, 64 rows: 7.9 against 11.0 ms per step)
+    if (a.tiled && !a.offsets && !old_form && a.K % kSwChunk == 0) return launch_wave<F>(a, problems, stream);
     if (a.K % (8 * LK) == 0) {
         if (tiles / 8 >= 448) return launch_cfg<F, 4, CK, 8, 4, 2>(a, problems, stream);
         if (tiles / 4 >= 448) return launch_cfg<F, 4, CK, 4, 4, 2>(a, problems, stream);

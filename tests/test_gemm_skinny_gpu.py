@@ -177,9 +177,13 @@ def test_tile_major_repack_is_the_documented_permutation(gpu, oracle, kind, N, K
 
 @pytest.mark.parametrize("kind", KINDS)
 @pytest.mark.parametrize("M,N,K", [(5, 64, 512), (16, 256, 4096), (17, 100, 2048), (45, 48, 512),
-                                   (8, 12304, 512), (20, 24592, 512)])
-def test_skinny_over_tile_major_weights_is_bit_identical(gpu, oracle, kind, M, N, K):
-    """Same values, same evaluation order: only the addresses of the weight loads change."""
+                                   (8, 12304, 512), (20, 24592, 512),
+                                   # long K: seven chunks per K slice; 1536: a K slice left empty
+                                   (6, 64, 14336), (32, 1040, 1536), (1, 4096, 4096), (3, 8192, 1024)])
+def test_skinny_over_tile_major_weights_matches_oracle_and_row_major(gpu, oracle, kind, M, N, K):
+    """Tile-major weights run the wave-private kernel (another split of K, so another sum order):
+    same bar against the oracle as the row-major path, and within one bf16 step of that path on
+    almost every element."""
     import torch
     from pie_amd import ops
 
@@ -189,18 +193,39 @@ def test_skinny_over_tile_major_weights_is_bit_identical(gpu, oracle, kind, M, N
     x = dev(oracle.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32)), gpu, torch.bfloat16)
     a = bits(ops.gemm_skinny(x, w))
     b = bits(ops.gemm_skinny(x, ops.repack_mfma_tiles(w)))
-    assert np.array_equal(a, b)
-    assert close_to_oracle(oracle, b, oracle_linear(oracle, wd, bits(x)))
+    ref = oracle_linear(oracle, wd, bits(x))
+    assert close_to_oracle(oracle, b, ref)
+    assert (ulp_diff(b, ref) <= 1).mean() > 0.98
+    assert (ulp_diff(a, b) <= 1).mean() > 0.98
+
+
+@pytest.mark.parametrize("kind", KINDS)
+def test_skinny_tile_major_one_hot_rows_are_exact(gpu, oracle, kind):
+    """One-hot activations over tile-major weights: y[m, n] is bf16(dequantised w[n, k_m]) exactly,
+    whatever K slice and chunk k_m falls in."""
+    import torch
+    from pie_amd import ops
+
+    rng = np.random.default_rng(341)
+    M, N, K = 16, 96, 4096
+    wd, mk = make_weight(oracle, rng, kind, N, K)
+    ks = np.array([0, 1, 7, 8, 31, 127, 128, 255, 256, 511, 512, 1023, 2048, 3000, 4094, 4095])
+    x = np.zeros((M, K), dtype=np.float32)
+    x[np.arange(M), ks] = 1.0
+    xb = oracle.f32_to_bf16(x)
+    got = bits(ops.gemm_skinny(dev(xb, gpu, torch.bfloat16), ops.repack_mfma_tiles(mk(gpu))))
+    ref = oracle_linear(oracle, wd, xb)
+    assert np.array_equal(got, ref)
 
 
 @pytest.mark.parametrize("kind", ["fp8", "int4b8", "bf16"])
 @pytest.mark.parametrize("swiglu", [False, True])
-def test_moe_grouped_gemm_over_tile_major_experts_is_bit_identical(gpu, oracle, kind, swiglu):
+def test_moe_grouped_gemm_over_tile_major_experts(gpu, oracle, kind, swiglu):
     import torch
     from pie_amd import ops
 
     rng = np.random.default_rng(350)
-    E, N, K, T = 6, 96, 512, 20
+    E, N, K, T = 6, 96, 1024, 20
     counts = np.array([3, 0, 21, 1, 0, 7])
     offs = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
     rows = rng.integers(0, T, size=int(offs[-1])).astype(np.int32)
@@ -215,4 +240,7 @@ def test_moe_grouped_gemm_over_tile_major_experts_is_bit_identical(gpu, oracle, 
     ss = tiled.scale if kind != "int4b8" else tiled.scale.reshape(E, N, -1)
     ss = sstack if kind != "int4b8" else ss
     b = bits(ops.moe_grouped_gemm(x, dev(rows, gpu), dev(offs, gpu), kind, ws, ss, N, K, tiled=True, **args))
-    assert np.array_equal(a, b)
+    # the row-major path is checked against the per-expert oracle above; the tile-major kernel
+    # splits K differently, so its sums differ from it in order only
+    assert a.shape == b.shape
+    assert (ulp_diff(a, b) <= 1).mean() > 0.98 and close_to_oracle(oracle, b, a)
