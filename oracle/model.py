@@ -143,6 +143,17 @@ class OracleModel:
                 at += int(rl[i])
             allow = np.ascontiguousarray(np.concatenate(chunks) if chunks else np.zeros(1, np.uint8))
             allow_off = np.ascontiguousarray(np.asarray(offs, np.int64))
+        lib().orc_router_gap_reset()
+        try:
+            return self._forward_call(tok, pos, slots, rb, rl, pages, N, sr, S, out, logits, want_logits,
+                                      masks, allow, allow_off, p)
+        finally:
+            lib().orc_router_gap_get.restype = C.c_float
+            self._router_gap = float(lib().orc_router_gap_get())
+
+    def _forward_call(self, tok, pos, slots, rb, rl, pages, N, sr, S, out, logits, want_logits, masks,
+                      allow, allow_off, p):
+        vp = lambda a: C.c_void_p(a.ctypes.data)
         if self.kv_format:
             assert masks is None, "custom masks are not available with one-byte KV formats"
             lib().orc_llama_forward_kvq(C.byref(self._m), C.c_int(self.kv_format), self._kf, self._vf,
@@ -158,10 +169,17 @@ class OracleModel:
                                 vp(allow_off) if allow_off is not None else None)
         return out[:S], (logits[:S] if want_logits else None), p
 
+    def router_gap(self) -> float:
+        """Smallest gap between the last chosen and the first rejected router logit, relative to
+        the token's largest logit magnitude, in the most recent forward (huge for dense models):
+        near bf16 resolution, another summation order may route a token to another expert."""
+        return self._router_gap
+
     def generate(self, prompt, max_new: int, replicate: int = 1, want_logits=False):
         """Greedy generation over contiguous page ranges, one prefill per context and one
         multi-request decode forward per step.  Returns tokens [replicate, max_new] (and the
-        per-step logits of context 0 when asked)."""
+        per-step logits of context 0 when asked); `last_router_gaps` holds router_gap() of the
+        prefill and of each decode step."""
         ps = self.cfg["page_size"]
         n_prompt = len(prompt)
         ppc = (n_prompt + max_new + ps - 1) // ps
@@ -173,6 +191,8 @@ class OracleModel:
                                     [n_prompt - (npg - 1) * ps], [0, n_prompt],
                                     want_logits=want_logits and c == 0)
             toks[c, 0] = t[0]
+            if c == 0:
+                self.last_router_gaps = [self.router_gap()]
             if want_logits and c == 0:
                 logit_trace.append(lg[0])
         for s in range(1, max_new):
@@ -184,6 +204,7 @@ class OracleModel:
                                     [pos + 1 - (npg - 1) * ps] * replicate,
                                     np.arange(replicate + 1), want_logits=want_logits)
             toks[:, s] = t
+            self.last_router_gaps.append(self.router_gap())
             if want_logits:
                 logit_trace.append(lg[0])
         return (toks, logit_trace) if want_logits else toks

@@ -19,6 +19,7 @@
  * transformer on a tiny model (cosine of the logits, the tolerance precedent of
  * driver/cuda/tests/parity_qwen3.py:160-181).
  */
+#include <math.h>
 #include <stdlib.h>
 #include <string.h>
 
@@ -98,6 +99,33 @@ static OrcLinear orc_expert_slice(const OrcModel* m, const OrcLinear* w, int e, 
     return s;
 }
 
+/* Test diagnostic: the smallest gap between the last selected and the first rejected router
+ * logit, relative to the largest logit magnitude of that token, over every (layer, token) routed
+ * since the last reset.  A gap at bf16 resolution
+ * means another summation order may pick another expert there: the parity tests flag such a
+ * forward as a near-tie instead of holding it to the logit bar. */
+static float g_router_min_gap = 3.4e38f;
+void orc_router_gap_reset(void) { g_router_min_gap = 3.4e38f; }
+float orc_router_gap_get(void) { return g_router_min_gap; }
+static void orc_router_gap_note(const uint16_t* logits, int N, int E, int K) {
+    if (K >= E) return;
+    for (int n = 0; n < N; ++n) {
+        float v[512];
+        for (int j = 0; j < E; ++j) v[j] = orc_bf16_to_f32(logits[(size_t)n * E + j]);
+        for (int k = 0; k <= K; ++k) { /* partial selection sort: v[0..K] descending */
+            int b = k;
+            for (int j = k + 1; j < E; ++j)
+                if (v[j] > v[b]) b = j;
+            const float t = v[k]; v[k] = v[b]; v[b] = t;
+        }
+        float mag = 0.f; /* the row's largest magnitude: the error of a logit scales with the
+                            size of the sum's terms, not with the logit's own value */
+        for (int j = 0; j < E; ++j) mag = fabsf(v[j]) > mag ? fabsf(v[j]) : mag;
+        const float gap = (v[K - 1] - v[K]) / (mag > 1e-20f ? mag : 1e-20f);
+        if (gap < g_router_min_gap) g_router_min_gap = gap;
+    }
+}
+
 /* x[t] += sum_k w[t,k] * down_e(swiglu(gateup_e(xn[t]))) over the token's top-k experts. */
 static void orc_moe_ffn(const OrcModel* m, int l, const uint16_t* xn, uint16_t* x, int N) {
     const int H = m->hidden, E = m->num_experts, K = m->top_k, Ie = m->expert_intermediate;
@@ -108,6 +136,7 @@ static void orc_moe_ffn(const OrcModel* m, int l, const uint16_t* xn, uint16_t* 
     uint16_t* yr = (uint16_t*)malloc((size_t)N * K * H * 2);
     orc_gemm_bf16(xn, m->router[l], NULL, lf, logits, NULL, N, E, H, 0, 0);
     orc_topk_softmax(logits, idx, wts, N, E, K);
+    orc_router_gap_note(logits, N, E, K);
 #pragma omp parallel for schedule(dynamic)
     for (int r = 0; r < N * K; ++r) {
         const int t = r / K, e = idx[r];

@@ -52,8 +52,9 @@ int fmt_code(Quant q) {
 }
 
 // Measured cost models (MI355X, microseconds, int4 8B-class shapes at 16-128 rows).  Skinny GEMM:
-// ~5 us + the weights at ~2.8 TB/s (3.3 TB/s from the tile-major copy) for the first 16-row pass,
-// each further (side-by-side) pass adding 85 % (80 %) of that stream.  Tiled GEMM: K in 64-wide steps of ~0.72 us with 64-row block
+// ~5 us + the weights at ~2.8 TB/s for the first 16-row pass, each further (side-by-side) pass
+// adding 85 % of that stream; from the tile-major copy (wave-private form) ~3.8 TB/s and 52 % per
+// further pass, the pass count rounded up to a power of two.  Tiled GEMM: K in 64-wide steps of ~0.72 us with 64-row block
 // tiles (M <= 64), ~0.98 us with 128-row tiles, while the tiles fit the machine (512 resident
 // blocks).  Split-K tiled GEMM: the steps of one share (+3 of prologue) at 1.25 / 1.6 us with two
 // blocks per CU, per round of 512 blocks, plus ~15 us for the second kernel and the partials.
@@ -61,8 +62,10 @@ enum class GemmPath { Skinny, Tiled, TiledSplitK };
 GemmPath pick_gemm(const Linear& w, int M, size_t ws_bytes) {
     if (w.K % 64 != 0 || M < 17) return GemmPath::Skinny;
     const int passes = (M + 15) / 16;
+    int p2 = 1;   // the wave-private form runs its passes side by side: cost steps at powers of two
+    while (p2 < passes) p2 <<= 1;
     const double skinny = w.data_tiled
-                              ? 5.0 + static_cast<double>(w.data_bytes()) / 3.3e6 * (1.0 + 0.80 * (passes - 1))
+                              ? 5.0 + static_cast<double>(w.data_bytes()) / 3.8e6 * (1.0 + 0.52 * (p2 - 1))
                               : 5.0 + static_cast<double>(w.data_bytes()) / 2.8e6 * (1.0 + 0.85 * (passes - 1));
     const int steps = w.K / 64;
     const double tiles = static_cast<double>((w.N + 127) / 128) * (M <= 64 ? 1 : (M + 127) / 128);

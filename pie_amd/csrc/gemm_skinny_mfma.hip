@@ -634,14 +634,16 @@ int launch_wave(const SkinnyArgs& a, int problems, hipStream_t stream) {
     const long tiles = (a.N + 15) / 16;
     static const int force_ng = [] { const char* e = getenv("PIE_SKINNY_NG"); return e ? atoi(e) : 0; }();
     static const int force_kp = [] { const char* e = getenv("PIE_SKINNY_KP"); return e ? atoi(e) : -1; }();
-    constexpr long kWant = 2048;
-    int ng = 1, kp_shift = 3;
+    // a CU holds one block of eight waves (two with one tile per wave: fewer registers).  Take
+    // the most tiles per wave whose K split still puts >= 1100 waves on the machine without
+    // going past what is resident at once (a second round of blocks costs more than idle CUs).
+    int ng = 1, kp_shift = 0;
     for (int cand = 4; cand >= 1; cand >>= 1) {
         const long groups = (tiles + cand - 1) / cand * mult;
+        const long cap = 256L * (cand == 1 ? 16 : 8);
         int sh = 0;
-        while (sh < 3 && (groups << sh) * 4 < kWant * 3) ++sh;
-        while (sh > 0 && (1 << sh) > nch_all) --sh;
-        if ((groups << sh) * 4 >= kWant * 3 || cand == 1) {
+        while (sh < 3 && (groups << (sh + 1)) <= cap && (2 << sh) <= nch_all) ++sh;
+        if ((groups << sh) >= 1100 || cand == 1) {
             ng = cand;
             kp_shift = sh;
             break;

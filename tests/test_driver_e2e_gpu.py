@@ -34,26 +34,36 @@ def teacher_forced_compare(oracle, drvmod, d, om, cfg, prompt, max_new, replicat
         assert res.num_requests == 1 and len(res.tokens) == 1
         if c == 0:
             lg = d.export_tensor("debug.logits", np.uint16).reshape(-1, V)[0]
-            near_ties += check_step(oracle, lg, otrace[0], res.tokens[0], otoks[0, 0], **bars)
+            near_ties += check_step(oracle, lg, otrace[0], res.tokens[0], otoks[0, 0],
+                                    router_gap=om.last_router_gaps[0], **bars)
     for s in range(1, max_new):
         pos = n_prompt + s - 1
         res = d.forward(step_frames(drvmod, otoks[:, s - 1], pos, replicate, ppc, ps))
         assert res.num_requests == replicate and res.tokens_indptr == list(range(replicate + 1))
         lg = d.export_tensor("debug.logits", np.uint16).reshape(-1, V)
-        near_ties += check_step(oracle, lg[0], otrace[s], res.tokens[0], otoks[0, s], **bars)
+        near_ties += check_step(oracle, lg[0], otrace[s], res.tokens[0], otoks[0, s],
+                                router_gap=om.last_router_gaps[s], **bars)
         # every replica holds the same context: identical tokens
         assert len(set(res.tokens)) == 1
     return otoks, near_ties
 
 
 def check_step(oracle, gpu_logit_bits, orc_logit_bits, gpu_tok, orc_tok, cos_min=0.9999, rel=0.02,
-               tie=2.0 ** -6):
+               tie=2.0 ** -6, router_gap=float("inf")):
     g = oracle.bf16_to_f32(gpu_logit_bits)
     o = oracle.bf16_to_f32(orc_logit_bits)
+    # MoE: where the oracle's router logits separate the last chosen expert from the first
+    # rejected one by no more than two bf16 steps of the row's largest logit, another fp32
+    # summation order upstream may route a token of this forward to another expert.  Such a step
+    # counts as a near-tie and is held to a looser logit bar (one expert of top_k swapped for its
+    # neighbour), never skipped.
+    router_tie = router_gap <= 2.0 ** -7
+    if router_tie:
+        cos_min, rel = min(cos_min, 0.995), max(rel, 0.15)
     assert cosine(g, o) >= cos_min
     assert np.max(np.abs(g - o)) <= rel * np.max(np.abs(o)) + 1e-3
     top2 = np.sort(o)[-2:]
-    near_tie = (top2[1] - top2[0]) <= tie * abs(top2[1]) + 1e-6
+    near_tie = router_tie or (top2[1] - top2[0]) <= tie * abs(top2[1]) + 1e-6
     if not near_tie:
         assert int(gpu_tok) == int(orc_tok)
     # the token the driver returns is the argmax of its own logits, first index on ties

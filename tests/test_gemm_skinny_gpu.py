@@ -71,19 +71,21 @@ def test_skinny_one_hot_rows_are_exact(gpu, oracle, kind):
 
 
 @pytest.mark.parametrize("kind", ["int4b8", "fp8"])
-def test_skinny_beta_and_swiglu(gpu, oracle, kind):
+@pytest.mark.parametrize("tiled,M", [(False, 12), (True, 12), (True, 37)])
+def test_skinny_beta_and_swiglu(gpu, oracle, kind, tiled, M):
     import torch
     from pie_amd import ops
 
     rng = np.random.default_rng(313)
-    M, I, K = 12, 192, 1024
+    I, K = 192, 1024
     wd, mk = make_weight(oracle, rng, kind, 2 * I, K)
     x = oracle.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32))
     xg = dev(x, gpu, torch.bfloat16)
     w = mk(gpu)
+    lay = ops.repack_mfma_tiles if tiled else (lambda v: v)
     # residual accumulate
     y0 = oracle.f32_to_bf16(rng.standard_normal((M, 2 * I)).astype(np.float32))
-    got = bits(ops.gemm_skinny(xg, w, y=dev(y0, gpu, torch.bfloat16).clone(), beta=1))
+    got = bits(ops.gemm_skinny(xg, lay(w), y=dev(y0, gpu, torch.bfloat16).clone(), beta=1))
     ref = oracle_linear(oracle, wd, x, y_in=y0)
     assert close_to_oracle(oracle, got, ref) and (ulp_diff(got, ref) <= 1).mean() > 0.98
     # swiglu epilogue over interleaved rows
@@ -92,12 +94,12 @@ def test_skinny_beta_and_swiglu(gpu, oracle, kind):
     idx = torch.from_numpy(perm).to(gpu)
     wi = ops.WeightView(w.kind, w.data[idx].contiguous(), w.scale[idx].contiguous(), w.group_size,
                         w.N, w.K)
-    fused = bits(ops.gemm_skinny(xg, wi, swiglu=True))
+    fused = bits(ops.gemm_skinny(xg, lay(wi), swiglu=True))
     assert fused.shape == (M, I)
-    unfused = bits(ops.swiglu_bf16(ops.gemm_skinny(xg, w)))
+    unfused = bits(ops.swiglu_bf16(ops.gemm_skinny(xg, lay(w))))
     assert np.array_equal(fused, unfused)
     with pytest.raises(ops.KernelError):
-        ops.gemm_skinny(xg, wi, y=torch.zeros(M, I, device=gpu, dtype=torch.bfloat16), beta=1,
+        ops.gemm_skinny(xg, lay(wi), y=torch.zeros(M, I, device=gpu, dtype=torch.bfloat16), beta=1,
                         swiglu=True)
 
 
@@ -179,7 +181,9 @@ def test_tile_major_repack_is_the_documented_permutation(gpu, oracle, kind, N, K
 @pytest.mark.parametrize("M,N,K", [(5, 64, 512), (16, 256, 4096), (17, 100, 2048), (45, 48, 512),
                                    (8, 12304, 512), (20, 24592, 512),
                                    # long K: seven chunks per K slice; 1536: a K slice left empty
-                                   (6, 64, 14336), (32, 1040, 1536), (1, 4096, 4096), (3, 8192, 1024)])
+                                   (6, 64, 14336), (32, 1040, 1536), (1, 4096, 4096), (3, 8192, 1024),
+                                   # fewer rows than a tile (a router), two passes over small matrices
+                                   (21, 8, 512), (21, 768, 512), (21, 512, 512), (130, 72, 1024)])
 def test_skinny_over_tile_major_weights_matches_oracle_and_row_major(gpu, oracle, kind, M, N, K):
     """Tile-major weights run the wave-private kernel (another split of K, so another sum order):
     same bar against the oracle as the row-major path, and within one bf16 step of that path on

@@ -88,3 +88,38 @@ def test_oracle_moe_forward_matches_dense_fp64(oracle, quant):
         assert lo @ rl / (np.linalg.norm(lo) * np.linalg.norm(rl)) >= 0.9995, i
         good += 1
     assert good >= 5
+
+
+def test_router_gap_reports_the_selection_margin(oracle):
+    """router_gap() = (last chosen - first rejected router logit) / the token's largest logit
+    magnitude, minimum over layers and tokens.  Router rows c_e * u with c = +-powers of two make
+    every logit an exact multiple c_e * (u . x): whatever x is (either sign of u . x), the margin
+    between the 2nd and 3rd is exactly 1/4 of the largest; identical rows give 0; a dense model
+    reports no margin at all."""
+    from oracle.model import OracleModel
+
+    cfg = dict(hidden=128, layers=2, q_heads=4, kv_heads=2, head_dim=32, intermediate=0, vocab=200,
+               rms_eps=1e-5, rope_interleaved=0, qk_norm=True, quant="bf16", group_size=64,
+               page_size=4, total_pages=16, num_experts=6, top_k=2, expert_intermediate=64)
+    rng = np.random.default_rng(403)
+    t = make_tensors(oracle, rng, cfg)
+    u = oracle.bf16_to_f32(oracle.f32_to_bf16(rng.standard_normal(128).astype(np.float32)))
+    c = np.array([4, 2, 1, -1, -2, -4], np.float32)
+    for l in range(2):
+        t[f"layers.{l}.router"] = oracle.f32_to_bf16(c[:, None] * u[None, :])
+    om = OracleModel(cfg, t)
+    prompt = rng.integers(0, cfg["vocab"], 5)
+    om.forward(prompt, np.arange(5), [3, 7], [0, 2], [1], [0, 5])
+    assert om.router_gap() == 0.25
+    for l in range(2):
+        t[f"layers.{l}.router"] = oracle.f32_to_bf16(np.tile(u, (6, 1)))
+    om = OracleModel(cfg, t)
+    om.forward(prompt, np.arange(5), [3, 7], [0, 2], [1], [0, 5])
+    assert om.router_gap() == 0.0
+    toks = om.generate(prompt, 3)
+    assert len(om.last_router_gaps) == 3 and toks.shape == (1, 3)
+
+    dense = dict(cfg, num_experts=0, top_k=0, expert_intermediate=0, intermediate=64)
+    od = OracleModel(dense, make_tensors(oracle, rng, dense))
+    od.forward(prompt, np.arange(5), [3, 7], [0, 2], [1], [0, 5])
+    assert od.router_gap() > 1e30
