@@ -481,6 +481,11 @@ __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 ? 4 : 2) void skinny_wave_
     const int srow = lane >> 5, svec = lane & 31;
 
     for (int mt0 = r0; mt0 < r1; mt0 += 16) {
+        // a pass of at most eight rows stages eight: the activations are re-read by every tile
+        // group, so their traffic matters as much as the weights'.  Accumulator rows 8..15 then
+        // repeat rows 0..7 and are never stored.
+        const bool r8 = r1 - mt0 <= 8;
+        const int jr = r8 ? (j & 7) : j;
         int arow[SV];   // rows past the problem repeat its last row and are never stored
 #pragma unroll
         for (int u = 0; u < SV; ++u) {
@@ -492,11 +497,13 @@ __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 ? 4 : 2) void skinny_wave_
             const int k0 = min((b_lo + c * CB) * LK + svec * 8, K - 8);
 #pragma unroll
             for (int u = 0; u < SV; ++u)
-                stg[u] = *reinterpret_cast<const u32x4_t*>(a.act + static_cast<size_t>(arow[u]) * K + k0);
+                if (u < SV / 2 || !r8)
+                    stg[u] = *reinterpret_cast<const u32x4_t*>(a.act + static_cast<size_t>(arow[u]) * K + k0);
         };
         auto stage_store = [&]() {
 #pragma unroll
-            for (int u = 0; u < SV; ++u) lds_a[(srow + 2 * u) * kSwStride + svec] = F::order(stg[u]);
+            for (int u = 0; u < SV; ++u)
+                if (u < SV / 2 || !r8) lds_a[(srow + 2 * u) * kSwStride + svec] = F::order(stg[u]);
         };
 
         f32x4_t acc[NG], sxs[F::kGroupScale ? CB : 1], sxt = zero4;
@@ -514,7 +521,7 @@ __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 ? 4 : 2) void skinny_wave_
             const int sxi = F::kGroupScale ? blk : 0;
             bf16x8_t ax[S];
 #pragma unroll
-            for (int s = 0; s < S; ++s) ax[s] = __builtin_bit_cast(bf16x8_t, lds_a[j * kSwStride + vbase + s]);
+            for (int s = 0; s < S; ++s) ax[s] = __builtin_bit_cast(bf16x8_t, lds_a[jr * kSwStride + vbase + s]);
             f32x4_t part = zero4;
 #pragma unroll
             for (int s = 0; s < S; ++s) {
@@ -709,7 +716,8 @@ int launch_skinny(SkinnyArgs a, int problems, hipStream_t stream) {
     // 32 / 64 rows: 2.43 / 2.78 / 3.42 / 5.18 ms against 2.75 / 2.95 / 4.07 / 5.64); the grouped
     // MoE launches stay with the block-shared form, whose eight tiles per staged chunk halve the
     // activation traffic (30B-A3B, 64 rows: 7.9 against 11.0 ms per step)
-    if (a.tiled && !a.offsets && !old_form && a.K % kSwChunk == 0) return launch_wave<F>(a, problems, stream);
+    static const bool grouped_wave = getenv("PIE_SKINNY_GROUPED_WAVE") != nullptr;
+    if (a.tiled && (!a.offsets || grouped_wave) && !old_form && a.K % kSwChunk == 0) return launch_wave<F>(a, problems, stream);
     if (a.K % (8 * LK) == 0) {
         if (tiles / 8 >= 448) return launch_cfg<F, 4, CK, 8, 4, 2>(a, problems, stream);
         if (tiles / 4 >= 448) return launch_cfg<F, 4, CK, 4, 4, 2>(a, problems, stream);
