@@ -234,7 +234,8 @@ def w4a16_sweep_extra():
     """The W4A16 GEMM sweep of BASELINE's second config: (K, N) x M, int4b8 group 128.  Each
     (shape, M) is timed from a HIP graph that walks a ring of weight copies larger than the
     256 MB last-level cache, so every launch streams its weights from HBM.  M <= 4 runs the GEMV,
-    above that the faster of the skinny and the tiled matrix-core GEMM (both reported)."""
+    above that the faster of the skinny and the tiled matrix-core GEMM (both reported); the skinny
+    GEMM reads tile-major copies of the weights, as the driver's decoder linears do."""
     import torch
 
     from pie_amd import ops
@@ -248,6 +249,7 @@ def w4a16_sweep_extra():
         ring = [ops.int4b8_view(torch.randint(-2**31, 2**31 - 1, (N, K // 8), dtype=torch.int32, device=dev),
                                 (torch.rand(N, K // G, device=dev) * 0.015 + 0.005).bfloat16(), G)
                 for _ in range(ncopy)]
+        tiled_ring = [ops.repack_mfma_tiles(w) for w in ring]
         for M in (1, 8, 32, 128, 2048):
             act = torch.randn(M, K, device=dev).bfloat16()
             y = torch.empty(M, N, device=dev, dtype=torch.bfloat16)
@@ -260,11 +262,12 @@ def w4a16_sweep_extra():
                 kernels["tiled"] = ops.gemm_mfma
             res = {}
             for name, fn in kernels.items():
-                t = time_graph(lambda: fn(act, ring[next(it) % ncopy], y=y), ncopy, reps=3)
+                src = tiled_ring if name == "skinny" else ring
+                t = time_graph(lambda: fn(act, src[next(it) % ncopy], y=y), ncopy, reps=3)
                 res[name] = dict(us=round(t * 1e6, 1), gbps=round(alg / t / 1e9, 1),
                                  tflops=round(2.0 * M * N * K / t / 1e12, 1))
             out[f"K{K}_N{N}_M{M}"] = res
-        del ring
+        del ring, tiled_ring
         torch.cuda.empty_cache()
     return out
 

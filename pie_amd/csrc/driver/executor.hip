@@ -64,8 +64,10 @@ GemmPath pick_gemm(const Linear& w, int M, size_t ws_bytes) {
     const int passes = (M + 15) / 16;
     int p2 = 1;   // the wave-private form runs its passes side by side: cost steps at powers of two
     while (p2 < passes) p2 <<= 1;
+    // (past eight passes the machine is full: the cost grows in proportion)
+    const double wave_form = p2 <= 8 ? 1.0 + 0.52 * (p2 - 1) : (1.0 + 0.52 * 7) * passes / 8.0;
     const double skinny = w.data_tiled
-                              ? 5.0 + static_cast<double>(w.data_bytes()) / 3.8e6 * (1.0 + 0.52 * (p2 - 1))
+                              ? 5.0 + static_cast<double>(w.data_bytes()) / 3.8e6 * wave_form
                               : 5.0 + static_cast<double>(w.data_bytes()) / 2.8e6 * (1.0 + 0.85 * (passes - 1));
     const int steps = w.K / 64;
     const double tiles = static_cast<double>((w.N + 127) / 128) * (M <= 64 ? 1 : (M + 127) / 128);
