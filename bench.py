@@ -305,6 +305,7 @@ def cpu_baseline(drv, model, page_size, total_pages, n_prompt, gpu_tokens, budge
     import oracle
 
     steps, matched, near_ties, t_total = 0, 0, 0, 0.0
+    margins = []   # per mismatch: how far below its own choice the oracle ranks the GPU's token
     tok = int(gpu_tokens[0])
     while steps < len(gpu_tokens) - 1 and (steps < 2 or t_total < budget_s):
         pos = n_prompt + steps
@@ -322,6 +323,8 @@ def cpu_baseline(drv, model, page_size, total_pages, n_prompt, gpu_tokens, budge
             lg = oracle.bf16_to_f32(np.asarray(logits).reshape(-1))
             top2 = np.partition(lg, -2)[-2:]
             near_ties += int(float(top2[1] - top2[0]) <= 2.0 ** -6 * max(abs(float(top2[1])), 1e-30))
+            top = float(lg[int(out[0])])
+            margins.append(round((top - float(lg[int(gpu_tokens[steps])])) / max(abs(top), 1e-30), 5))
         tok = int(gpu_tokens[steps])  # teacher-forced: every step is compared on the same context
     cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
     return dict(value=steps / t_total, unit="tokens/s", cores=cores, kind="port",
@@ -329,7 +332,8 @@ def cpu_baseline(drv, model, page_size, total_pages, n_prompt, gpu_tokens, budge
                        "oracle (C restatement of the reference forward pass, OpenMP over rows) "
                        "fed the GPU's weights and prefilled KV pages",
                 greedy_tokens_matched=matched, greedy_tokens_compared=steps,
-                mismatches_at_oracle_near_ties=near_ties)
+                mismatches_at_oracle_near_ties=near_ties,
+                mismatch_margins_rel_to_top_logit=margins)
 
 
 # HBM bytes per GEMV launch, averaged over the model's four int4 linears at M = 1, from two
