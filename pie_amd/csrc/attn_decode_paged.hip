@@ -376,10 +376,11 @@ typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 constexpr int kMStepKeys = 32;
 constexpr int kMVtStride = kMStepKeys + 8;
 
-template <int D, int GQA>
+template <int D, int GQA, int KVF = kKvBf16>
 __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
-    const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_pages,
-    const uint16_t* __restrict__ v_pages, const uint32_t* __restrict__ page_indices,
+    const uint16_t* __restrict__ q, const void* __restrict__ k_pages_raw,
+    const void* __restrict__ v_pages_raw, const float* __restrict__ k_scales,
+    const float* __restrict__ v_scales, const uint32_t* __restrict__ page_indices,
     const uint32_t* __restrict__ page_indptr, const uint32_t* __restrict__ last_lens,
     const uint32_t* __restrict__ row_begin, const int32_t* __restrict__ row_len,
     float* __restrict__ part_o, float* __restrict__ part_ml, uint16_t* __restrict__ o_direct,
@@ -387,15 +388,28 @@ __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
     float scale_log2e) {
     constexpr int KS = D / 32;                 // k steps of the first product
     constexpr int DT = D / 16;                 // d tiles of the second product
-    constexpr int LPR = D / 8;                 // 16-byte pieces per K/V row
+    // One-byte pools: the codes become bf16 (exactly) on the way into the wave's LDS regions, the
+    // per-(token, kv head) scales multiply the scores (K) and the probabilities (V) — the
+    // arithmetic of the dot-product kernel above, float(code) * scale.
+    constexpr bool Q8 = KVF != kKvBf16;
+    constexpr int EB = Q8 ? 1 : 2;             // stored bytes per element
+    constexpr int LPR = D * EB / 16;           // 16-byte pieces per stored K/V row
+    constexpr int NK = kMStepKeys * LPR / kWave;   // K load instructions per step
     constexpr int VC = 16 * LPR / kWave;       // (key pair, piece) combos per lane per step
+    constexpr int PG = LPR < 8 ? LPR : 8;      // adjacent lanes that take adjacent V pieces
     constexpr int PF = 2;                      // steps of K/V in flight per wave
-    static_assert(GQA <= 16 && VC >= 1, "shape");
+    static_assert(GQA <= 16 && VC >= 1 && NK >= 1, "shape");
+    const unsigned char* k_pages = static_cast<const unsigned char*>(k_pages_raw);
+    const unsigned char* v_pages = static_cast<const unsigned char*>(v_pages_raw);
     constexpr int KSTRIDE = D + 8;             // bf16 elements per K row in LDS (padded: conflict-free reads)
-    __shared__ __attribute__((aligned(16))) uint16_t vt_all[kAttnWaves][D * kMVtStride];
+    // V^T rows are 80 bytes; every 16 rows the region skips another 32 bytes, so the eight pieces
+    // (row groups) a staging write touches start in different banks
+    __shared__ __attribute__((aligned(16))) uint16_t vt_all[kAttnWaves][D * kMVtStride + D];
+    auto vt_at = [](int row, int col) { return row * kMVtStride + (row >> 4) * 16 + col; };
     __shared__ __attribute__((aligned(16))) uint16_t ks_all[kAttnWaves][kMStepKeys * KSTRIDE];
     __shared__ float sm_m[kAttnWaves][16];
     __shared__ float sm_l[kAttnWaves][16];
+    __shared__ __attribute__((aligned(16))) float sc_all[Q8 ? kAttnWaves : 1][kWave];   // K | V scales of a step
     static_assert(sizeof(float) * GQA * D <= sizeof(uint16_t) * D * kMVtStride, "per-wave output fits its V^T region");
 
     const int kvh = blockIdx.x, split = blockIdx.y, r = blockIdx.z;
@@ -429,11 +443,17 @@ __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
     uint16_t* Ks = ks_all[wv];
     // K loads: whole rows, LPR adjacent lanes per key (kWave / LPR keys per instruction)
     constexpr int KPI = kWave / LPR;
-    u32x4_t kreg[PF][2 * KS], vreg[PF][2 * VC];
+    u32x4_t kreg[PF][NK], vreg[PF][2 * VC];
+    float sreg[PF];   // one-byte pools: lane < 32 holds the K scale of key `lane`, the others V's
     // V loads: combo c of a lane = (key pair, 16-byte piece); eight adjacent lanes take eight
     // adjacent pieces (128 contiguous bytes of a row)
-    auto v_piece = [&](int c) { return (lane & 7) + 8 * (c % (LPR / 8)); };
-    auto v_pair = [&](int c) { return (lane >> 3) + 8 * (c / (LPR / 8)); };
+    auto v_piece = [&](int c) { return (lane % PG) + PG * (c % (LPR / PG)); };
+    // key pairs of one instruction: (0,1,8,9,2,3,10,11) + 4c', whose V^T columns are words 0..7
+    // (8..15) of a row — with the row-group skew every lane of a staging write has its own bank
+    auto v_pair = [&](int c) {
+        const int i = lane / PG;
+        return (i & 1) + 2 * ((i >> 2) & 1) + 8 * ((i >> 1) & 1) + 4 * ((i >> 3) + (kWave / PG / 8) * (c / (LPR / PG)));
+    };
     // A 32-key step starts on a multiple of 16 and touches at most two pages (page_size % 16 == 0);
     // their ids come through scalar loads.  Keys past the split repeat its last key (finite
     // data; their probabilities are zero).
@@ -444,44 +464,70 @@ __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
         const int jb = min(j0 + kMStepKeys - 1, k_end - 1);
         const uint32_t pid_a = __builtin_amdgcn_readfirstlane(page_indices[pg_lo + page_a]);
         const uint32_t pid_b = __builtin_amdgcn_readfirstlane(page_indices[pg_lo + page_a + (jb >= pa_end ? 1 : 0)]);
-        auto row_off = [&](int key) {
+        auto row_th = [&](int key) {   // (token slot, kv head) index of a key of the step
             const int j = min(j0 + key, k_end - 1);
             const bool in_a = j < pa_end;
             const size_t slot_idx = static_cast<size_t>(in_a ? pid_a : pid_b) * ps + (j - (in_a ? pa_end - ps : pa_end));
-            return (slot_idx * hk + kvh) * D;
+            return slot_idx * hk + kvh;
         };
 #pragma unroll
-        for (int i = 0; i < 2 * KS; ++i)
+        for (int i = 0; i < NK; ++i)
             kreg[slot][i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(
-                k_pages + row_off(lane / LPR + KPI * i) + (lane % LPR) * 8));
+                k_pages + row_th(lane / LPR + KPI * i) * (D * EB) + (lane % LPR) * 16));
 #pragma unroll
         for (int c = 0; c < VC; ++c) {
             const int pair = v_pair(c), dc = v_piece(c);
 #pragma unroll
             for (int u = 0; u < 2; ++u)
                 vreg[slot][2 * c + u] = __builtin_nontemporal_load(
-                    reinterpret_cast<const u32x4_t*>(v_pages + row_off(2 * pair + u) + dc * 8));
+                    reinterpret_cast<const u32x4_t*>(v_pages + row_th(2 * pair + u) * (D * EB) + dc * 16));
+        }
+        if constexpr (Q8) {
+            const float* sp = lane < kMStepKeys ? k_scales : v_scales;
+            sreg[slot] = sp ? sp[row_th(lane & (kMStepKeys - 1))] : 1.f;
         }
     };
     // V rows -> V^T in the wave's LDS region: two adjacent keys of one piece meet in one lane and
     // leave as 4-byte writes (slot of key kappa: 8*(kappa%16/4) + kappa%4, +4 for kappa >= 16)
     auto stage = [&](int slot) {
 #pragma unroll
-        for (int i = 0; i < 2 * KS; ++i)
-            *reinterpret_cast<u32x4_t*>(&Ks[(lane / LPR + KPI * i) * KSTRIDE + (lane % LPR) * 8]) = kreg[slot][i];
+        for (int i = 0; i < NK; ++i) {
+            uint16_t* dst = &Ks[(lane / LPR + KPI * i) * KSTRIDE + (lane % LPR) * (16 / EB)];
+            if constexpr (!Q8) {
+                *reinterpret_cast<u32x4_t*>(dst) = kreg[slot][i];
+            } else {   // 16 codes -> 16 bf16
+                const u32x4_t w = kreg[slot][i];
+                *reinterpret_cast<u32x4_t*>(dst) = kv_decode_bf16<KVF>(u32x2_t{w.x, w.y});
+                *reinterpret_cast<u32x4_t*>(dst + 8) = kv_decode_bf16<KVF>(u32x2_t{w.z, w.w});
+            }
+        }
 #pragma unroll
         for (int c = 0; c < VC; ++c) {
             const int pair = v_pair(c), dc = v_piece(c);
             const int kappa = 2 * pair;
             const int col = kappa < 16 ? 8 * (kappa >> 2) + (kappa & 3) : 8 * ((kappa - 16) >> 2) + 4 + (kappa & 3);
             const u32x4_t a = vreg[slot][2 * c], b = vreg[slot][2 * c + 1];
+            if constexpr (!Q8) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const uint32_t lo = (a[e >> 1] >> (16 * (e & 1))) & 0xFFFFu;
-                const uint32_t hi = (b[e >> 1] >> (16 * (e & 1))) & 0xFFFFu;
-                *reinterpret_cast<uint32_t*>(&Vt[(dc * 8 + e) * kMVtStride + col]) = lo | (hi << 16);
+                for (int e = 0; e < 8; ++e) {
+                    const uint32_t lo = (a[e >> 1] >> (16 * (e & 1))) & 0xFFFFu;
+                    const uint32_t hi = (b[e >> 1] >> (16 * (e & 1))) & 0xFFFFu;
+                    *reinterpret_cast<uint32_t*>(&Vt[vt_at(dc * 8 + e, col)]) = lo | (hi << 16);
+                }
+            } else {   // 16 elements of two adjacent keys: (bf16(a_e), bf16(b_e)) pairs
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    float fa[8], fb[8];
+                    kv_decode_f32<KVF>(u32x2_t{a[2 * h], a[2 * h + 1]}, fa);
+                    kv_decode_f32<KVF>(u32x2_t{b[2 * h], b[2 * h + 1]}, fb);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        *reinterpret_cast<uint32_t*>(&Vt[vt_at(dc * 16 + 8 * h + e, col)]) =
+                            kv_pack_trunc(fa[e], fb[e]);
+                }
             }
         }
+        if constexpr (Q8) sc_all[wv][lane] = sreg[slot];
     };
 
     f32x4_t acc[DT];
@@ -501,6 +547,15 @@ __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
                     __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(
                                                      &Ks[(16 * nt + l16) * KSTRIDE + 32 * ks + 8 * g])),
                     qf[ks], st[nt], 0, 0, 0);
+        // (one-byte pools) the scales of this lane's keys, before the slot is refilled
+        f32x4_t ksc[2], vsc[2];
+        if constexpr (Q8) {
+#pragma unroll
+            for (int nt = 0; nt < 2; ++nt) {
+                ksc[nt] = *reinterpret_cast<const f32x4_t*>(&sc_all[wv][16 * nt + 4 * g]);
+                vsc[nt] = *reinterpret_cast<const f32x4_t*>(&sc_all[wv][kMStepKeys + 16 * nt + 4 * g]);
+            }
+        }
         if (j0 + PF * kStride < k_end) issue(slot, j0 + PF * kStride);
 
         // online softmax of query l16 over this lane's keys 16nt + 4g + r
@@ -511,7 +566,8 @@ __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
 #pragma unroll
             for (int rr = 0; rr < 4; ++rr) {
                 const int key = j0 + 16 * nt + 4 * g + rr;
-                const float v = key < k_end ? st[nt][rr] * scale_log2e : -INFINITY;
+                const float sc = Q8 ? scale_log2e * ksc[nt][rr] : scale_log2e;
+                const float v = key < k_end ? st[nt][rr] * sc : -INFINITY;
                 sv[4 * nt + rr] = v;
                 m_new = fmaxf(m_new, v);
             }
@@ -524,8 +580,12 @@ __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
         uint32_t hi[4], lo[4];
 #pragma unroll
         for (int e = 0; e < 8; e += 2) {
-            const float p0 = exp2f(sv[e] - safe), p1 = exp2f(sv[e + 1] - safe);
+            float p0 = exp2f(sv[e] - safe), p1 = exp2f(sv[e + 1] - safe);
             sum += p0 + p1;
+            if constexpr (Q8) {   // V = float(code) * scale: the scale rides on the probability
+                p0 *= vsc[e >> 2][e & 3];
+                p1 *= vsc[e >> 2][(e & 3) + 1];
+            }
             // p = hi + lo with both parts bf16: hi by truncation, lo = bf16(p - hi)
             const uint32_t b0 = __float_as_uint(p0) & 0xFFFF0000u, b1 = __float_as_uint(p1) & 0xFFFF0000u;
             hi[e >> 1] = (b0 >> 16) | b1;
@@ -541,7 +601,7 @@ __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
             const bf16x8_t vf = __builtin_bit_cast(
-                bf16x8_t, *reinterpret_cast<const u32x4_t*>(&Vt[(16 * dt + l16) * kMVtStride + 8 * g]));
+                bf16x8_t, *reinterpret_cast<const u32x4_t*>(&Vt[vt_at(16 * dt + l16, 8 * g)]));
             acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, p_hi, acc[dt], 0, 0, 0);
             acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, p_lo, acc[dt], 0, 0, 0);
         }
@@ -713,8 +773,8 @@ int launch_decode(const uint16_t* q, const void* k_pages, const void* v_pages,
                   int mask_stride, hipStream_t stream) {
     const SplitPlan plan = plan_splits(R, hk, max_kv_len);
     const float scale_log2e = sm_scale * 1.4426950408889634f;
-    if constexpr (!MASKED && KVF == kKvBf16) {
-        // bf16 pools without a custom mask run on the matrix cores.  Measured (MI355X, 8B / 30B-A3B
+    if constexpr (!MASKED) {
+        // Rows without a custom mask run on the matrix cores (bf16 and one-byte pools).  Measured (MI355X, 8B / 30B-A3B
         // decode steps, four / eight query heads per kv head), matrix-core against dot-product
         // kernel: batch 1 1.808 / 1.860 ms, batch 8 2.68 / 2.80, batch 32 4.07 / 4.13, batch 64 at
         // 2048 keys 7.53 / 7.72, MoE batch 64 7.98 / 8.80; 64 rows of 512-8192 keys 5.61 / 4.96 TB/s.
@@ -723,13 +783,12 @@ int launch_decode(const uint16_t* q, const void* k_pages, const void* v_pages,
         const bool mfma = forced >= 0 ? forced == 0 : true;
         if (mfma) {
             const int ps_shift = (ps & (ps - 1)) == 0 ? __builtin_ctz(static_cast<unsigned>(ps)) : -1;
-            const uint16_t* kp = static_cast<const uint16_t*>(k_pages);
-            const uint16_t* vp = static_cast<const uint16_t*>(v_pages);
             if (plan.nsplit == 1) {
                 hipLaunchKernelGGL((attn_decode_clear_empty_kernel<D>), dim3(R * hq), dim3(D), 0, stream,
                                    page_indptr, last_lens, row_begin, row_len, o, lse, hq, ps);
-                hipLaunchKernelGGL((attn_decode_mfma_kernel<D, GQA>), dim3(hk, 1, R), dim3(kAttnBlock), 0,
-                                   stream, q, kp, vp, page_indices, page_indptr, last_lens, row_begin, row_len,
+                hipLaunchKernelGGL((attn_decode_mfma_kernel<D, GQA, KVF>), dim3(hk, 1, R), dim3(kAttnBlock), 0,
+                                   stream, q, k_pages, v_pages, k_scales, v_scales, page_indices, page_indptr,
+                                   last_lens, row_begin, row_len,
                                    nullptr, nullptr, o, lse, hq, hk, ps, ps_shift, plan.units_per_split, 1,
                                    scale_log2e);
                 return launch_status();
@@ -739,8 +798,9 @@ int launch_decode(const uint16_t* q, const void* k_pages, const void* v_pages,
             if (!workspace || workspace_bytes < need) return PIE_HIP_ERR_INVALID;
             float* part_o = static_cast<float*>(workspace);
             float* part_ml = part_o + n_part * D;
-            hipLaunchKernelGGL((attn_decode_mfma_kernel<D, GQA>), dim3(hk, plan.nsplit, R), dim3(kAttnBlock), 0,
-                               stream, q, kp, vp, page_indices, page_indptr, last_lens, row_begin, row_len,
+            hipLaunchKernelGGL((attn_decode_mfma_kernel<D, GQA, KVF>), dim3(hk, plan.nsplit, R), dim3(kAttnBlock), 0,
+                               stream, q, k_pages, v_pages, k_scales, v_scales, page_indices, page_indptr,
+                               last_lens, row_begin, row_len,
                                part_o, part_ml, nullptr, nullptr, hq, hk, ps, ps_shift, plan.units_per_split,
                                plan.nsplit, scale_log2e);
             hipLaunchKernelGGL((attn_decode_merge_kernel<D>), dim3(R * hq), dim3(D), 0, stream, part_o,
