@@ -376,7 +376,7 @@ typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 constexpr int kMStepKeys = 32;
 constexpr int kMVtStride = kMStepKeys + 8;
 
-template <int D, int GQA, int KVF = kKvBf16>
+template <int D, int GQA, int KVF = kKvBf16, bool MASKED = false>
 __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
     const uint16_t* __restrict__ q, const void* __restrict__ k_pages_raw,
     const void* __restrict__ v_pages_raw, const float* __restrict__ k_scales,
@@ -384,8 +384,8 @@ __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
     const uint32_t* __restrict__ page_indptr, const uint32_t* __restrict__ last_lens,
     const uint32_t* __restrict__ row_begin, const int32_t* __restrict__ row_len,
     float* __restrict__ part_o, float* __restrict__ part_ml, uint16_t* __restrict__ o_direct,
-    float* __restrict__ lse, int hq, int hk, int ps, int ps_shift, int units_per_split, int nsplit,
-    float scale_log2e) {
+    float* __restrict__ lse, const uint16_t* __restrict__ mask_bits, int mask_stride, int hq, int hk,
+    int ps, int ps_shift, int units_per_split, int nsplit, float scale_log2e) {
     constexpr int KS = D / 32;                 // k steps of the first product
     constexpr int DT = D / 16;                 // d tiles of the second product
     // One-byte pools: the codes become bf16 (exactly) on the way into the wave's LDS regions, the
@@ -445,6 +445,7 @@ __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
     constexpr int KPI = kWave / LPR;
     u32x4_t kreg[PF][NK], vreg[PF][2 * VC];
     float sreg[PF];   // one-byte pools: lane < 32 holds the K scale of key `lane`, the others V's
+    uint32_t mreg[PF];   // MASKED: the visibility words of the step's two 16-token units
     // V loads: combo c of a lane = (key pair, 16-byte piece); eight adjacent lanes take eight
     // adjacent pieces (128 contiguous bytes of a row)
     auto v_piece = [&](int c) { return (lane % PG) + PG * (c % (LPR / PG)); };
@@ -485,6 +486,11 @@ __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
         if constexpr (Q8) {
             const float* sp = lane < kMStepKeys ? k_scales : v_scales;
             sreg[slot] = sp ? sp[row_th(lane & (kMStepKeys - 1))] : 1.f;
+        }
+        if constexpr (MASKED) {   // (the second unit may lie past the context: its keys are dropped anyway)
+            const uint16_t* mrow = mask_bits + static_cast<size_t>(r) * mask_stride;
+            const int u0 = j0 / kUnitTokens;
+            mreg[slot] = static_cast<uint32_t>(mrow[u0]) | (static_cast<uint32_t>(mrow[min(u0 + 1, nunits - 1)]) << 16);
         }
     };
     // V rows -> V^T in the wave's LDS region: two adjacent keys of one piece meet in one lane and
@@ -556,6 +562,7 @@ __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
                 vsc[nt] = *reinterpret_cast<const f32x4_t*>(&sc_all[wv][kMStepKeys + 16 * nt + 4 * g]);
             }
         }
+        const uint32_t vis = MASKED ? mreg[slot] : 0xFFFFFFFFu;   // bit 16nt + t: key t of unit nt visible
         if (j0 + PF * kStride < k_end) issue(slot, j0 + PF * kStride);
 
         // online softmax of query l16 over this lane's keys 16nt + 4g + r
@@ -567,7 +574,8 @@ __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
             for (int rr = 0; rr < 4; ++rr) {
                 const int key = j0 + 16 * nt + 4 * g + rr;
                 const float sc = Q8 ? scale_log2e * ksc[nt][rr] : scale_log2e;
-                const float v = key < k_end ? st[nt][rr] * sc : -INFINITY;
+                const bool seen = key < k_end && (!MASKED || ((vis >> (16 * nt + 4 * g + rr)) & 1u));
+                const float v = seen ? st[nt][rr] * sc : -INFINITY;
                 sv[4 * nt + rr] = v;
                 m_new = fmaxf(m_new, v);
             }
@@ -773,8 +781,8 @@ int launch_decode(const uint16_t* q, const void* k_pages, const void* v_pages,
                   int mask_stride, hipStream_t stream) {
     const SplitPlan plan = plan_splits(R, hk, max_kv_len);
     const float scale_log2e = sm_scale * 1.4426950408889634f;
-    if constexpr (!MASKED) {
-        // Rows without a custom mask run on the matrix cores (bf16 and one-byte pools).  Measured (MI355X, 8B / 30B-A3B
+    {
+        // The matrix-core kernel: bf16 and one-byte pools, rows with and without a custom mask.  Measured (MI355X, 8B / 30B-A3B
         // decode steps, four / eight query heads per kv head), matrix-core against dot-product
         // kernel: batch 1 1.808 / 1.860 ms, batch 8 2.68 / 2.80, batch 32 4.07 / 4.13, batch 64 at
         // 2048 keys 7.53 / 7.72, MoE batch 64 7.98 / 8.80; 64 rows of 512-8192 keys 5.61 / 4.96 TB/s.
@@ -786,11 +794,11 @@ int launch_decode(const uint16_t* q, const void* k_pages, const void* v_pages,
             if (plan.nsplit == 1) {
                 hipLaunchKernelGGL((attn_decode_clear_empty_kernel<D>), dim3(R * hq), dim3(D), 0, stream,
                                    page_indptr, last_lens, row_begin, row_len, o, lse, hq, ps);
-                hipLaunchKernelGGL((attn_decode_mfma_kernel<D, GQA, KVF>), dim3(hk, 1, R), dim3(kAttnBlock), 0,
+                hipLaunchKernelGGL((attn_decode_mfma_kernel<D, GQA, KVF, MASKED>), dim3(hk, 1, R), dim3(kAttnBlock), 0,
                                    stream, q, k_pages, v_pages, k_scales, v_scales, page_indices, page_indptr,
                                    last_lens, row_begin, row_len,
-                                   nullptr, nullptr, o, lse, hq, hk, ps, ps_shift, plan.units_per_split, 1,
-                                   scale_log2e);
+                                   nullptr, nullptr, o, lse, mask_bits, mask_stride, hq, hk, ps, ps_shift,
+                                   plan.units_per_split, 1, scale_log2e);
                 return launch_status();
             }
             const size_t n_part = static_cast<size_t>(R) * hq * plan.nsplit;
@@ -798,11 +806,11 @@ int launch_decode(const uint16_t* q, const void* k_pages, const void* v_pages,
             if (!workspace || workspace_bytes < need) return PIE_HIP_ERR_INVALID;
             float* part_o = static_cast<float*>(workspace);
             float* part_ml = part_o + n_part * D;
-            hipLaunchKernelGGL((attn_decode_mfma_kernel<D, GQA, KVF>), dim3(hk, plan.nsplit, R), dim3(kAttnBlock), 0,
+            hipLaunchKernelGGL((attn_decode_mfma_kernel<D, GQA, KVF, MASKED>), dim3(hk, plan.nsplit, R), dim3(kAttnBlock), 0,
                                stream, q, k_pages, v_pages, k_scales, v_scales, page_indices, page_indptr,
                                last_lens, row_begin, row_len,
-                               part_o, part_ml, nullptr, nullptr, hq, hk, ps, ps_shift, plan.units_per_split,
-                               plan.nsplit, scale_log2e);
+                               part_o, part_ml, nullptr, nullptr, mask_bits, mask_stride, hq, hk, ps, ps_shift,
+                               plan.units_per_split, plan.nsplit, scale_log2e);
             hipLaunchKernelGGL((attn_decode_merge_kernel<D>), dim3(R * hq), dim3(D), 0, stream, part_o,
                                part_ml, page_indptr, last_lens, row_begin, row_len, o, lse, hq, ps,
                                plan.units_per_split, plan.nsplit);
