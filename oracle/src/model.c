@@ -126,6 +126,14 @@ static void orc_router_gap_note(const uint16_t* logits, int N, int E, int K) {
     }
 }
 
+/* Test diagnostic: when set, row 0 of the last layer's intermediates of the next forward is
+ * copied out: q after RoPE [hq*d], attention output [hq*d], SwiGLU output [I] (dense models),
+ * residual stream after the layer [H].  Any pointer may be NULL. */
+static uint16_t *g_cap_q = NULL, *g_cap_attn = NULL, *g_cap_act = NULL, *g_cap_x = NULL;
+void orc_debug_capture(uint16_t* q, uint16_t* attn, uint16_t* act, uint16_t* x) {
+    g_cap_q = q; g_cap_attn = attn; g_cap_act = act; g_cap_x = x;
+}
+
 /* x[t] += sum_k w[t,k] * down_e(swiglu(gateup_e(xn[t]))) over the token's top-k experts. */
 static void orc_moe_ffn(const OrcModel* m, int l, const uint16_t* xn, uint16_t* x, int N) {
     const int H = m->hidden, E = m->num_experts, K = m->top_k, Ie = m->expert_intermediate;
@@ -239,6 +247,12 @@ static void orc_llama_forward_impl(const OrcModel* m, uint16_t* const* k_pages, 
             orc_linear(m, &m->wgu[l], xn, gu, N, 2 * I, H, 0);
             orc_swiglu(gu, act, N, I);
             orc_linear(m, &m->wdown[l], act, x, N, H, I, 1);
+        }
+        if (l == m->layers - 1) {
+            if (g_cap_q) memcpy(g_cap_q, q, (size_t)hq * d * 2);
+            if (g_cap_attn) memcpy(g_cap_attn, attn, (size_t)hq * d * 2);
+            if (g_cap_act && m->num_experts == 0) memcpy(g_cap_act, act, (size_t)I * 2);
+            if (g_cap_x) memcpy(g_cap_x, x, (size_t)H * 2);
         }
     }
     if (S > 0) {

@@ -456,6 +456,20 @@ extern "C" size_t pie_hip_driver_export_tensor(PieHipDriver* d, const char* name
         return bytes;
     }
     const std::string nm(name);
+    if (nm.rfind("debug.", 0) == 0) {
+        const uint16_t* buf = d->exec->debug_buffer(nm.substr(6));
+        if (!buf) return 0;
+        const auto& mc = d->cfg.model;
+        const size_t elems = nm == "debug.x" ? mc.hidden
+                             : nm == "debug.act" ? (mc.num_experts > 0 ? mc.expert_intermediate : mc.intermediate)
+                                                 : static_cast<size_t>(mc.q_heads) * mc.head_dim;
+        const size_t bytes = elems * 2;
+        if (dst) {
+            const size_t n = bytes < cap ? bytes : cap;
+            if (hipMemcpy(dst, buf, n, hipMemcpyDeviceToHost) != hipSuccess) return 0;
+        }
+        return bytes;
+    }
     if (nm.rfind("kv.k.", 0) == 0 || nm.rfind("kv.v.", 0) == 0) {
         const int l = std::atoi(nm.c_str() + 5);
         const uint16_t* pool = d->exec->kv_pool(nm[3] == 'k', l);

@@ -79,6 +79,15 @@ class Executor {
     int graphs_cached() const { return static_cast<int>(graphs_.size()); }
     // Logits [rows, vocab] bf16 of the last forward's (last chunk of) sampled rows; debug/test hook.
     const uint16_t* last_logits() const { return logits_; }
+    // Row 0 of the last layer's intermediates after a forward (debug/test hook): "x" residual
+    // stream, "q" rotated queries, "attn" attention output, "act" SwiGLU output.
+    const uint16_t* debug_buffer(const std::string& what) const {
+        if (what == "x") return x_;
+        if (what == "q") return q_;
+        if (what == "attn") return attn_;
+        if (what == "act") return act_;
+        return nullptr;
+    }
     int last_logit_rows() const { return last_logit_rows_; }
     const uint16_t* kv_pool(bool k, int layer) const {
         if (layer < 0 || layer >= static_cast<int>(k_pool_.size())) return nullptr;

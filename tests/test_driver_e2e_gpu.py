@@ -431,3 +431,43 @@ def test_custom_masks_are_refused_with_a_one_byte_kv_cache(gpu):
     for bad, msg in (("fp8_e5m2", "not implemented"), ("turboquant", "invalid kv_cache_dtype")):
         with pytest.raises(Exception, match=msg):
             drvmod.Driver(toml_config(kv_cache_dtype=bad))
+
+
+@pytest.mark.parametrize("kw", [dict(quant="int4b8"), dict(arch="qwen3", quant="bf16", head_dim=128, q_heads=4,
+                                                           kv_heads=1, rope_theta=1e6)],
+                         ids=["llama3-int4b8", "qwen3-bf16"])
+def test_last_layer_intermediates_match_oracle(gpu, oracle, kw):
+    """Beyond the logits: row 0 of the last layer's rotated queries, attention output, SwiGLU
+    output and residual stream of a decode step against the oracle's (`orc_debug_capture`).
+    Each is a bf16 vector a few rounding points downstream of identical inputs: cosine >= 0.9999
+    and at most a few bf16 steps apart anywhere."""
+    import ctypes as C
+    from pie_amd import driver as drvmod
+
+    cfg = full_cfg(**kw)
+    ps = cfg["page_size"]
+    rng = np.random.default_rng(95)
+    prompt = rng.integers(0, cfg["vocab"], 19)
+    H, I, QD = cfg["hidden"], cfg["intermediate"], cfg["q_heads"] * cfg["head_dim"]
+    with drvmod.Driver(toml_config(**kw)) as d:
+        om, _ = oracle_model_from_driver(d, cfg)
+        n, npg = len(prompt), (len(prompt) + ps - 1) // ps
+        fr = (prompt, np.arange(n), np.arange(npg), [0, npg], [n - (npg - 1) * ps], [0, n])
+        tok = int(d.forward(drvmod.ForwardFrame(*fr)).tokens[0])
+        assert int(om.forward(*fr)[0][0]) == tok
+        step = ([tok], [n], np.arange(npg + 1)[: (n + ps) // ps], [0, (n + ps) // ps], [n + 1 - ((n + ps) // ps - 1) * ps], [0, 1])
+        d.forward(drvmod.ForwardFrame(*step))
+        got = {k: d.export_tensor("debug." + k, np.uint16) for k in ("q", "attn", "act", "x")}
+        cap = dict(q=np.zeros(QD, np.uint16), attn=np.zeros(QD, np.uint16), act=np.zeros(I, np.uint16),
+                   x=np.zeros(H, np.uint16))
+        lib = oracle.lib()
+        lib.orc_debug_capture(*[C.c_void_p(cap[k].ctypes.data) for k in ("q", "attn", "act", "x")])
+        try:
+            om.forward(*step)
+        finally:
+            lib.orc_debug_capture(None, None, None, None)
+    for k in ("q", "attn", "act", "x"):
+        g, o = oracle.bf16_to_f32(got[k][: len(cap[k])]), oracle.bf16_to_f32(cap[k])
+        assert len(got[k]) == len(cap[k]) and np.any(o != 0), k
+        assert cosine(g, o) >= 0.9999, (k, cosine(g, o))
+        assert np.max(np.abs(g - o)) <= 2.0 ** -5 * np.max(np.abs(o)) + 1e-3, k
