@@ -254,7 +254,10 @@ int pie_hip_driver_generate(PieHipDriver* d, const uint32_t* prompt, int n_promp
                             int replicate, int warmup, uint32_t* out_tokens, double* timings_us,
                             char* err, size_t err_cap);
 /* Copy a named tensor to host memory (test/bench hook): model weights by name, "kv.k.<l>" /
- * "kv.v.<l>" (layer l's page pool) and "debug.logits" (last forward's sampled-row logits).
+ * "kv.v.<l>" (layer l's page pool), "debug.logits" (last forward's sampled-row logits) and
+ * row 0 of the last layer's intermediates of the last forward: "debug.q" (rotated queries,
+ * q_heads * head_dim bf16), "debug.attn" (attention output), "debug.act" (SwiGLU output) and
+ * "debug.x" (residual stream after the layer).
  * Returns the byte size, 0 if the tensor does not exist; copies min(size, cap) bytes when dst
  * is non-null. */
 size_t pie_hip_driver_export_tensor(PieHipDriver* d, const char* name, void* dst, size_t cap);
