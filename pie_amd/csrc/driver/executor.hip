@@ -94,7 +94,18 @@ void linear_fused(const Linear& w, const uint16_t* act, const uint16_t* norm_w, 
                   size_t gemm_ws_bytes, hipStream_t s) {
     const int fmt = fmt_code(w.kind);
     const int sbf = w.scale_bf16 ? 1 : 0;
-    if (M > 4) {
+    // Two to four rows: the GEMV pays its dot products once per row (8B shapes, 1..4 rows: gate|up
+    // 16.7 / 21.6 / 26.7 / 31.8 us, down 11.3 / 15.9 / 26.1 / 29.7), the skinny GEMM over the
+    // tile-major copy does not (19 / 12.7 us at any of them) but needs the norm as its own launch
+    // (~4.8 us).  Measured costs decide; without a tile-major copy the GEMV keeps all four.
+    bool gemv = M <= 4;
+    if (gemv && M >= 2 && w.data_tiled) {
+        const double bytes = static_cast<double>(w.data_bytes());
+        const double t_gemv = 5.0 + bytes / 5.5e6 * (1.0 + 0.5 * (M - 1));
+        const double t_skinny = 5.0 + bytes / 3.9e6 + (norm_w ? 4.8 : 0.0);
+        gemv = t_gemv <= t_skinny;
+    }
+    if (!gemv) {
         const uint16_t* a = act;
         if (norm_w) {
             PIE_KERNEL(pie_hip_rmsnorm(act, norm_w, norm_tmp, M, w.K, eps, s));
