@@ -202,6 +202,17 @@ int pie_hip_repack_scale_tiles(const uint16_t* src, uint16_t* dst, int N, int gr
 int pie_hip_gemm_skinny_tiled(int format, const uint16_t* act_bf16, const void* weight,
                         const void* scale, int scale_is_bf16, int group_size, uint16_t* y_bf16,
                         int M, int N, int K, int beta, int swiglu, void* stream);
+/* pie_hip_qkv_rope_fused for more rows than the GEMV takes (a decode batch): the q|k|v projection
+ * over tile-major weights with interleaved RoPE and the KV-cache write in its epilogue.  act_bf16
+ * is the normalised activation [M, K]; values are those of pie_hip_gemm_skinny_tiled followed by
+ * pie_hip_qkv_rope_kvwrite (interleaved = 1, no q/k norm), every intermediate rounded to bf16 at
+ * the same points.  Same reference role: the qkv gemm + qkv_decode_qk_norm_rope_write_kv_kernel
+ * pair of driver/cuda/src/model/llama_like.cpp:370-470.  head_dim a power of two, K % 256 == 0. */
+int pie_hip_qkv_rope_skinny_tiled(int format, const uint16_t* act_bf16, const void* weight,
+                                  const void* scale, int scale_is_bf16, int group_size, int M, int K,
+                                  const float* rope_table, const int64_t* kv_slots, uint16_t* q_out,
+                                  uint16_t* k_pages, uint16_t* v_pages, int num_q_heads,
+                                  int num_kv_heads, int head_dim, void* stream);
 int pie_hip_moe_grouped_gemm_tiled(int format, const uint16_t* act_bf16, const int32_t* route_act_rows,
                              const int32_t* expert_offsets, int num_experts,
                              int max_rows_per_expert, const void* weights,

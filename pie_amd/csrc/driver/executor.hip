@@ -382,10 +382,25 @@ void Executor::body(int N, int S, int max_kv_len) {
                                               w.wqkv.group, N, H, rope_tab_, slots, q_, k_pool_[l],
                                               v_pool_[l], hq, hk, d, s));
         } else {
-            linear_fused(w.wqkv, x_, w.attn_norm, m.rms_eps, qkv_, N, 0, 0, xn_, gemm_ws_, gemm_ws_bytes_, s);
-            PIE_KERNEL(pie_hip_qkv_rope_kvwrite(qkv_, q_, k_pool_[l], v_pool_[l], w.q_norm, w.k_norm,
-                                                rope_tab_, slots, N, hq, hk, d, m.rope_interleaved,
-                                                m.rms_eps, s));
+            // a decode batch of llama-type layers on the skinny GEMM: rotation and KV write ride
+            // in its epilogue too (one launch less per layer)
+            bool done = false;
+            if (m.rope_interleaved && !w.q_norm && (d & (d - 1)) == 0 && w.wqkv.data_tiled &&
+                pick_gemm(w.wqkv, N, gemm_ws_bytes_) == GemmPath::Skinny) {
+                PIE_KERNEL(pie_hip_rmsnorm(x_, w.attn_norm, xn_, N, H, m.rms_eps, s));
+                const int st = pie_hip_qkv_rope_skinny_tiled(
+                    fmt_code(w.wqkv.kind), xn_, w.wqkv.data_tiled,
+                    w.wqkv.scale_tiled ? w.wqkv.scale_tiled : w.wqkv.scale, w.wqkv.scale_bf16 ? 1 : 0,
+                    w.wqkv.group, N, H, rope_tab_, slots, q_, k_pool_[l], v_pool_[l], hq, hk, d, s);
+                if (st == PIE_HIP_OK) done = true;
+                else if (st != PIE_HIP_ERR_UNSUPPORTED) PIE_KERNEL(st);
+            }
+            if (!done) {
+                linear_fused(w.wqkv, x_, w.attn_norm, m.rms_eps, qkv_, N, 0, 0, xn_, gemm_ws_, gemm_ws_bytes_, s);
+                PIE_KERNEL(pie_hip_qkv_rope_kvwrite(qkv_, q_, k_pool_[l], v_pool_[l], w.q_norm, w.k_norm,
+                                                    rope_tab_, slots, N, hq, hk, d, m.rope_interleaved,
+                                                    m.rms_eps, s));
+            }
         }
         if (kvq) {
             if (masked_) throw std::runtime_error("executor: custom attention masks need a bf16 KV cache");

@@ -128,6 +128,14 @@ struct SkinnyArgs {
     int m_split;                // dense only: blockIdx.y = 16-row pass
     int tiled;                  // weights (and int4 group scales) in the tile-major layout
     size_t w_stride, scale_stride;  // bytes between problems
+    // q|k|v epilogue of the wave-private form (rope_table != null): rows of W are the q, k and
+    // v heads; adjacent output pairs of q and k heads are rotated, q goes to y [rows, hq*d], k
+    // and v to slot kv_slots[row] of the page pools
+    const float* rope_table;    // [rows, d]: cos (d/2) then sin (d/2) per row
+    const int64_t* kv_slots;    // [rows]; negative: the row writes no K/V
+    uint16_t* k_pages;
+    uint16_t* v_pages;
+    int hq, hk, d;
 };
 
 constexpr int gcd_c(int a, int b) { return b == 0 ? a : gcd_c(b, a % b); }
@@ -598,7 +606,30 @@ __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 ? 4 : 2) void skinny_wave_
             const int n = (tile0 + i) * 16 + j;
             const bool ok = m < r1 && n < N;
             float v = (total(i, rr) + bias) * rs;
-            if (a.swiglu) {
+            if (a.rope_table) {
+                // the projection's bf16 values, then the rotation of qkv_rope_kvwrite_kernel with
+                // the same operations and rounding; columns (n, n + 1) sit in adjacent lanes
+                const float gb = bf16_bits_to_f32(f32_to_bf16_bits(v));
+                const float ub = __int_as_float(__builtin_amdgcn_update_dpp(
+                    0, __float_as_int(gb), 0xB1, 0xF, 0xF, true));  // quad_perm [1,0,3,2]
+                if ((j & 1) == 0 && ok) {
+                    const int dsh = __builtin_ctz(static_cast<unsigned>(a.d));   // head_dim is a power of two
+                    const int head = n >> dsh, dd = n & (a.d - 1);
+                    const int64_t slot = a.kv_slots[m];
+                    if (head < a.hq + a.hk) {
+                        const float* tab = a.rope_table + static_cast<size_t>(m) * a.d + (dd >> 1);
+                        const float c = tab[0], sn = tab[a.d >> 1];
+                        const uint32_t out = pack_bf16x2(gb * c - ub * sn, ub * c + gb * sn);
+                        if (head < a.hq)
+                            *reinterpret_cast<uint32_t*>(a.y + (static_cast<size_t>(m) * a.hq + head) * a.d + dd) = out;
+                        else if (slot >= 0)
+                            *reinterpret_cast<uint32_t*>(a.k_pages + (static_cast<size_t>(slot) * a.hk + (head - a.hq)) * a.d + dd) = out;
+                    } else if (slot >= 0) {
+                        *reinterpret_cast<uint32_t*>(a.v_pages + (static_cast<size_t>(slot) * a.hk + (head - a.hq - a.hk)) * a.d + dd) =
+                            pack_bf16x2(gb, ub);
+                    }
+                }
+            } else if (a.swiglu) {
                 const float gb = bf16_bits_to_f32(f32_to_bf16_bits(v));
                 const float other = __int_as_float(__builtin_amdgcn_update_dpp(
                     0, __float_as_int(gb), 0xB1, 0xF, 0xF, true));  // quad_perm [1,0,3,2]
@@ -716,6 +747,7 @@ int launch_skinny(SkinnyArgs a, int problems, hipStream_t stream) {
     // 32 / 64 rows: 2.43 / 2.78 / 3.42 / 5.18 ms against 2.75 / 2.95 / 4.07 / 5.64); the grouped
     // MoE launches stay with the block-shared form, whose eight tiles per staged chunk halve the
     // activation traffic (30B-A3B, 64 rows: 7.9 against 11.0 ms per step)
+    if (a.rope_table) return launch_wave<F>(a, problems, stream);   // (entry point checked K)
     static const bool grouped_wave = getenv("PIE_SKINNY_GROUPED_WAVE") != nullptr;
     if (a.tiled && (!a.offsets || grouped_wave) && !old_form && a.K % kSwChunk == 0) return launch_wave<F>(a, problems, stream);
     if (a.K % (8 * LK) == 0) {
@@ -845,6 +877,42 @@ extern "C" int pie_hip_gemm_skinny_tiled(int format, const uint16_t* act_bf16, c
     a.swiglu = swiglu ? 1 : 0;
     a.scale_is_bf16 = scale_is_bf16;
     a.tiled = 1;
+    return dispatch_skinny(format, a, 1, static_cast<hipStream_t>(stream));
+}
+
+// q|k|v projection over tile-major weights with RoPE and the KV write in the epilogue (more rows
+// than the GEMV form takes): values of pie_hip_gemm_skinny_tiled followed by
+// pie_hip_qkv_rope_kvwrite with interleaved = 1 and no q/k norm.
+extern "C" int pie_hip_qkv_rope_skinny_tiled(int format, const uint16_t* act_bf16, const void* weight,
+                                             const void* scale, int scale_is_bf16, int group_size,
+                                             int M, int K, const float* rope_table,
+                                             const int64_t* kv_slots, uint16_t* q_out,
+                                             uint16_t* k_pages, uint16_t* v_pages, int num_q_heads,
+                                             int num_kv_heads, int head_dim, void* stream) {
+    using namespace pie_hip;
+    if (!act_bf16 || !weight || !rope_table || !kv_slots || !q_out || !k_pages || !v_pages || M <= 0 ||
+        num_q_heads <= 0 || num_kv_heads <= 0 || head_dim <= 0)
+        return PIE_HIP_ERR_INVALID;
+    if (format != PIE_HIP_FMT_BF16 && !scale) return PIE_HIP_ERR_INVALID;
+    if ((head_dim & (head_dim - 1)) != 0 || head_dim % 16 != 0 || K % kSwChunk != 0) return PIE_HIP_ERR_UNSUPPORTED;
+    SkinnyArgs a{};
+    a.act = act_bf16;
+    a.w = static_cast<const unsigned char*>(weight);
+    a.scale = static_cast<const unsigned char*>(scale);
+    a.y = q_out;
+    a.M = M;
+    a.N = (num_q_heads + 2 * num_kv_heads) * head_dim;
+    a.K = K;
+    a.G = group_size;
+    a.scale_is_bf16 = scale_is_bf16;
+    a.tiled = 1;
+    a.rope_table = rope_table;
+    a.kv_slots = kv_slots;
+    a.k_pages = k_pages;
+    a.v_pages = v_pages;
+    a.hq = num_q_heads;
+    a.hk = num_kv_heads;
+    a.d = head_dim;
     return dispatch_skinny(format, a, 1, static_cast<hipStream_t>(stream));
 }
 

@@ -555,6 +555,31 @@ def qkv_rope_fused(act: torch.Tensor, w: WeightView, table: torch.Tensor, kv_slo
     return q_out
 
 
+def qkv_rope_skinny_tiled(act: torch.Tensor, w: WeightView, table: torch.Tensor, kv_slots: torch.Tensor,
+                          k_pages: torch.Tensor, v_pages: torch.Tensor, hq: int, hk: int, d: int) -> torch.Tensor:
+    """q|k|v projection over tile-major weights + interleaved RoPE + KV-cache write for a decode
+    batch (act already normalised).  Returns q [M, hq, d]; k / v land in their slots."""
+    _dev(act, torch.bfloat16, "act")
+    _dev(table, torch.float32, "rope_table")
+    _dev(kv_slots, torch.int64, "kv_slots")
+    _dev(k_pages, torch.bfloat16, "k_pages")
+    _dev(v_pages, torch.bfloat16, "v_pages")
+    if not w.kind.endswith("+tiled"):
+        raise KernelError("tile-major weights expected (repack_mfma_tiles)")
+    M, K = act.shape
+    if K != w.K or w.N != (hq + 2 * hk) * d or tuple(table.shape) != (M, d) or kv_slots.numel() != M:
+        raise KernelError("shape mismatch")
+    if M and int(kv_slots.max()) >= k_pages.numel() // (hk * d):
+        raise KernelError("kv slot out of range")
+    q_out = torch.empty((M, hq, d), dtype=torch.bfloat16, device=act.device)
+    scale_is_bf16 = int(w.scale is not None and w.scale.dtype == torch.bfloat16)
+    _check(kernels().pie_hip_qkv_rope_skinny_tiled(
+        FMT[w.kind[:-len("+tiled")]], _ptr(act), _ptr(w.data), _ptr(w.scale), scale_is_bf16, w.group_size,
+        M, K, _ptr(table), _ptr(kv_slots), _ptr(q_out), _ptr(k_pages), _ptr(v_pages), hq, hk, d,
+        _stream()), "pie_hip_qkv_rope_skinny_tiled")
+    return q_out
+
+
 # ---------------------------------------------------------------- sampling
 SAMPLER_KINDS = {"multinomial": 0, "top_k": 1, "top_p": 2, "min_p": 3, "top_k_top_p": 4,
                  "dist": 6, "raw_logits": 7, "logprob": 8, "logprobs": 9, "entropy": 10}

@@ -248,3 +248,32 @@ def test_moe_grouped_gemm_over_tile_major_experts(gpu, oracle, kind, swiglu):
     # splits K differently, so its sums differ from it in order only
     assert a.shape == b.shape
     assert (ulp_diff(a, b) <= 1).mean() > 0.98 and close_to_oracle(oracle, b, a)
+
+
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("M,hq,hk,d,K", [(5, 8, 2, 64, 512), (16, 4, 4, 128, 1024), (37, 32, 8, 128, 4096)])
+def test_qkv_rope_epilogue_of_the_skinny_gemm_equals_projection_then_rope_kernel(gpu, oracle, kind, M, hq, hk,
+                                                                                 d, K):
+    """A decode batch's q|k|v projection with RoPE and the KV write in the skinny GEMM's epilogue:
+    exactly the bytes of the same projection followed by the rope + KV-write kernel — q, and the
+    touched K / V slots (one token without a slot)."""
+    import torch
+    from pie_amd import ops
+
+    rng = np.random.default_rng(360 + M + hq)
+    N = (hq + 2 * hk) * d
+    wd, mk = make_weight(oracle, rng, kind, N, K)
+    wt = ops.repack_mfma_tiles(mk(gpu))
+    x = dev(oracle.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32)), gpu, torch.bfloat16)
+    pos = rng.integers(0, 500, M).astype(np.int32)
+    tab = ops.rope_table(dev(pos, gpu), dev(oracle.rope_inv_freq(d, 10000.0), gpu), d)
+    slots = rng.permutation(64)[:M].astype(np.int64)
+    slots[1] = -1
+    sg = dev(slots, gpu)
+    pools = [torch.full((64, hk, d), 0.5, device=gpu, dtype=torch.bfloat16) for _ in range(4)]
+    q1 = ops.qkv_rope_skinny_tiled(x, wt, tab, sg, pools[0], pools[1], hq, hk, d)
+    q2 = ops.qkv_rope_kvwrite(ops.gemm_skinny(x, wt), pools[2], pools[3], tab, sg, hq, hk, d, True)
+    assert np.array_equal(bits(q1), bits(q2))
+    assert np.array_equal(bits(pools[0]), bits(pools[2]))
+    assert np.array_equal(bits(pools[1]), bits(pools[3]))
+    assert not np.all(bits(pools[0]) == bits(torch.full((64, hk, d), 0.5, device=gpu, dtype=torch.bfloat16)))
