@@ -7,7 +7,7 @@ import scipy.stats
 
 
 def test_pcg32_matches_the_published_demo_sequence(oracle):
-    # pcg32_srandom_r(&rng, 42u, 54u) of the PCG reference implementation (pcg32-demo, round 1)
+    # pcg32_srandom_r(&rng, 42u, 54u) of the PCG reference implementation (the first sequence pcg32-demo prints)
     want = [0xa15c02b7, 0x7b47f409, 0xba1d3330, 0x83d2f293, 0xbfa4784b, 0xcbed606e]
     assert [int(x) for x in oracle.pcg32_sequence(42, 54, 6)] == want
 
