@@ -471,3 +471,21 @@ def test_last_layer_intermediates_match_oracle(gpu, oracle, kw):
         assert len(got[k]) == len(cap[k]) and np.any(o != 0), k
         assert cosine(g, o) >= 0.9999, (k, cosine(g, o))
         assert np.max(np.abs(g - o)) <= 2.0 ** -5 * np.max(np.abs(o)) + 1e-3, k
+
+
+@pytest.mark.parametrize("kw", [dict(quant="int4b8"), dict(quant="fp8"),
+                                dict(arch="qwen3", quant="int4b8", head_dim=128, q_heads=4, kv_heads=1,
+                                     rope_theta=1e6)], ids=["llama3-int4b8", "llama3-fp8", "qwen3-int4b8"])
+@pytest.mark.parametrize("replicate", [3, 4, 7])
+def test_small_decode_batches_match_oracle(gpu, oracle, kw, replicate):
+    """Three, four and seven identical contexts: the rows where each linear is sent to the GEMV or
+    to the skinny GEMM by cost (and the q|k|v epilogue changes kernels) against the oracle."""
+    from pie_amd import driver as drvmod
+
+    cfg = full_cfg(**kw)
+    rng = np.random.default_rng(96)
+    prompt = rng.integers(0, cfg["vocab"], 13)
+    with drvmod.Driver(toml_config(**kw, total_pages=96)) as d:
+        om, _ = oracle_model_from_driver(d, dict(cfg, total_pages=96))
+        _, near = teacher_forced_compare(oracle, drvmod, d, om, cfg, prompt, 6, replicate)
+        assert near <= 3
