@@ -686,13 +686,24 @@ __global__ __launch_bounds__(D) void attn_decode_merge_kernel(
     const int r = rh / hq;
     const int dd = threadIdx.x;
     const int lane = dd & (kWave - 1), wv = dd / kWave;
+    const float* ml = part_ml + static_cast<size_t>(rh) * nsplit * 2;
+    const float* po = part_o + static_cast<size_t>(rh) * nsplit * D + dd;
+    // Everything the block needs is requested at once — the row's extent, the (max, sum) pairs
+    // and the first kPre partial outputs of every split slot, used or not (the workspace holds
+    // nsplit slots per row; unused ones are masked below) — so the kernel waits for memory once
+    // instead of three times in a row.
+    constexpr int kPre = 24;
+    float pre[kPre];
+#pragma unroll
+    for (int s = 0; s < kPre; ++s) pre[s] = s < nsplit ? po[static_cast<size_t>(s) * D] : 0.f;
+    float2 mine_ml = make_float2(-INFINITY, 0.f);
+    if (dd < nsplit) mine_ml = *reinterpret_cast<const float2*>(ml + 2 * dd);
     const int kv_len = row_extent(page_indptr, last_lens, row_begin, row_len, r, ps).kv_len;
     const int nunits = (kv_len + kUnitTokens - 1) / kUnitTokens;
     const int ns = min(nsplit, (nunits + units_per_split - 1) / units_per_split);
-    const float* ml = part_ml + static_cast<size_t>(rh) * nsplit * 2;
 
-    float mloc = -INFINITY;
-    for (int s = dd; s < ns; s += D) mloc = fmaxf(mloc, ml[2 * s]);
+    float mloc = dd < ns ? mine_ml.x : -INFINITY;
+    for (int s = dd + D; s < ns; s += D) mloc = fmaxf(mloc, ml[2 * s]);
     mloc = wave_max(mloc);
     if (lane == 0) s_red[wv] = mloc;
     __syncthreads();
@@ -701,7 +712,12 @@ __global__ __launch_bounds__(D) void attn_decode_merge_kernel(
     for (int w = 1; w < D / kWave; ++w) mx = fmaxf(mx, s_red[w]);
     const float safe = (mx == -INFINITY) ? 0.f : mx;
     float lloc = 0.f;
-    for (int s = dd; s < ns; s += D) {
+    if (dd < ns) {
+        const float a = exp2f(mine_ml.x - safe);
+        s_w[dd] = a;
+        lloc = mine_ml.y * a;
+    }
+    for (int s = dd + D; s < ns; s += D) {
         const float a = exp2f(ml[2 * s] - safe);
         s_w[s] = a;
         lloc += ml[2 * s + 1] * a;
@@ -713,16 +729,30 @@ __global__ __launch_bounds__(D) void attn_decode_merge_kernel(
 #pragma unroll
     for (int w = 0; w < D / kWave; ++w) ls += s_red[D / kWave + w];
 
-    const float* po = part_o + static_cast<size_t>(rh) * nsplit * D + dd;
+    // the sum over splits keeps its order: four interleaved accumulators over s = 0, 1, 2, ...
     float acc0 = 0.f, acc1 = 0.f, acc2 = 0.f, acc3 = 0.f;
     int s = 0;
+#pragma unroll
+    for (int b = 0; b < kPre; b += 4) {
+        if (b + 4 <= ns) {
+            acc0 = fmaf(pre[b], s_w[b], acc0);
+            acc1 = fmaf(pre[b + 1], s_w[b + 1], acc1);
+            acc2 = fmaf(pre[b + 2], s_w[b + 2], acc2);
+            acc3 = fmaf(pre[b + 3], s_w[b + 3], acc3);
+            s = b + 4;
+        }
+    }
     for (; s + 4 <= ns; s += 4) {
         acc0 = fmaf(po[static_cast<size_t>(s) * D], s_w[s], acc0);
         acc1 = fmaf(po[static_cast<size_t>(s + 1) * D], s_w[s + 1], acc1);
         acc2 = fmaf(po[static_cast<size_t>(s + 2) * D], s_w[s + 2], acc2);
         acc3 = fmaf(po[static_cast<size_t>(s + 3) * D], s_w[s + 3], acc3);
     }
-    for (; s < ns; ++s) acc0 = fmaf(po[static_cast<size_t>(s) * D], s_w[s], acc0);
+    // the last one to three splits, in order (s = ns rounded down to a multiple of four here)
+#pragma unroll
+    for (int b = 0; b < kPre; ++b)
+        if (b >= s && b < ns) acc0 = fmaf(pre[b], s_w[b], acc0);
+    for (int t = max(s, kPre); t < ns; ++t) acc0 = fmaf(po[static_cast<size_t>(t) * D], s_w[t], acc0);
     const float ov = (acc0 + acc1) + (acc2 + acc3);
     o[static_cast<size_t>(rh) * D + dd] = f32_to_bf16_bits(ls > 0.f ? ov / ls : 0.f);
     if (lse && dd == 0) lse[rh] = ls > 0.f ? (logf(ls) + mx * 0.6931471805599453f) : -INFINITY;
