@@ -451,6 +451,18 @@ int pie_hip_kv_write_quant(int kv_format, const uint16_t* k_rows, const uint16_t
                            const int64_t* kv_slots, void* k_pages, void* v_pages, float* k_scales,
                            float* v_scales, int num_tokens, int num_kv_heads, int head_dim,
                            void* stream);
+/* pie_hip_qkv_rope_kvwrite and pie_hip_kv_write_quant in one launch for one-byte pools: every
+ * (token, head) of the packed q|k|v rows is rotated (optional per-head q/k RMSNorm, either
+ * pairing) and rounded to bf16 as by pie_hip_qkv_rope_kvwrite; q goes to q_out, the K and V
+ * heads are quantised from those bf16 values into the token's slot with the arithmetic of
+ * pie_hip_kv_write_quant (driver/cuda/src/kernels/kv_paged.cu:155-297) — the same bytes and
+ * scales as the two calls in a row.  head_dim <= 256. */
+int pie_hip_qkv_rope_kvwrite_quant(int kv_format, const uint16_t* packed_qkv, uint16_t* q_out,
+                                   void* k_pages, void* v_pages, float* k_scales, float* v_scales,
+                                   const uint16_t* q_norm_weight, const uint16_t* k_norm_weight,
+                                   const float* rope_table, const int64_t* kv_slots, int num_tokens,
+                                   int num_q_heads, int num_kv_heads, int head_dim, int interleaved,
+                                   float eps, void* stream);
 
 /* ---- per-layer kernels of the llama-like decoder ---------------------------- */
 

@@ -1051,8 +1051,134 @@ __global__ __launch_bounds__(256) void kv_write_quant_kernel(
     }
 }
 
+// The same quantiser behind the RoPE stage: one wave per (token, head) of a packed q|k|v row
+// rotates its head as qkv_rope_kvwrite_kernel does (optional per-head RMSNorm, both pairings),
+// rounds to bf16 — the values the two-kernel path stages as rows — and, for K and V heads,
+// quantises them from registers into the token's slot.  q heads go to q_out.
+template <int ITER>   // pairs per lane: head_dim <= 128 * ITER
+__global__ __launch_bounds__(64) void qkv_rope_kvwrite_quant_kernel(
+    const uint16_t* __restrict__ packed, uint16_t* __restrict__ q_out,
+    unsigned char* __restrict__ k_pages, unsigned char* __restrict__ v_pages,
+    float* __restrict__ k_scales, float* __restrict__ v_scales,
+    const uint16_t* __restrict__ q_norm_w, const uint16_t* __restrict__ k_norm_w,
+    const float* __restrict__ rope_table, const int64_t* __restrict__ kv_slots, int hq, int hk,
+    int d, int interleaved, float eps, int kv_format) {
+    const int n = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+    const int half = d / 2;
+    const size_t stride = static_cast<size_t>(hq + 2 * hk) * d;
+    const uint16_t* src = packed + n * stride + static_cast<size_t>(head) * d;
+    const bool is_q = head < hq, is_k = !is_q && head < hq + hk;
+    const int64_t slot = kv_slots[n];
+    if (!is_q && slot < 0) return;  // token without a KV slot
+    // this lane's pairs (ia, ib) and their bf16 values after the optional norm and rotation
+    float va[ITER], vb[ITER];
+    const uint16_t* nw = is_q ? q_norm_w : (is_k ? k_norm_w : nullptr);
+    float inv_rms = 1.f;
+    if (nw) {
+        float local = 0.f;
+        for (int i = lane; i < d; i += kWave) {
+            const float v = bf16_bits_to_f32(src[i]);
+            local += v * v;
+        }
+        inv_rms = rsqrtf(wave_sum(local) / static_cast<float>(d) + eps);
+    }
+    const float* tab = rope_table + static_cast<size_t>(n) * d;
+#pragma unroll
+    for (int it = 0; it < ITER; ++it) {
+        const int i = lane + it * kWave;
+        va[it] = vb[it] = 0.f;
+        if (i < half) {
+            const int ia = interleaved ? 2 * i : i, ib = interleaved ? 2 * i + 1 : i + half;
+            float a = bf16_bits_to_f32(src[ia]), b = bf16_bits_to_f32(src[ib]);
+            if (is_q || is_k) {
+                if (nw) {
+                    a = a * inv_rms * bf16_bits_to_f32(nw[ia]);
+                    b = b * inv_rms * bf16_bits_to_f32(nw[ib]);
+                }
+                const float c = tab[i], sn = tab[i + half];
+                const float ra = a * c - b * sn, rb = b * c + a * sn;
+                a = bf16_bits_to_f32(f32_to_bf16_bits(ra));
+                b = bf16_bits_to_f32(f32_to_bf16_bits(rb));
+            }
+            va[it] = a;
+            vb[it] = b;
+            if (is_q) {
+                uint16_t* dst = q_out + (static_cast<size_t>(n) * hq + head) * d;
+                dst[ia] = f32_to_bf16_bits(a);
+                dst[ib] = f32_to_bf16_bits(b);
+            }
+        }
+    }
+    if (is_q) return;
+    const int h = is_k ? head - hq : head - hq - hk;
+    const size_t th = static_cast<size_t>(slot) * hk + h;
+    unsigned char* dst = (is_k ? k_pages : v_pages) + th * d;
+    const bool scaled = kv_format != PIE_HIP_KV_FP8_E4M3;
+    const float qmax = kv_format == PIE_HIP_KV_INT8_PER_TOKEN_HEAD ? 127.f : 448.f;
+    float inv = 1.f;
+    if (scaled) {
+        float amax = 0.f;
+#pragma unroll
+        for (int it = 0; it < ITER; ++it) amax = fmaxf(amax, fmaxf(fabsf(va[it]), fabsf(vb[it])));
+        amax = wave_max(amax);
+        const float scale = amax > 0.f ? amax / qmax : 1.f;
+        inv = 1.f / scale;
+        if (lane == 0) (is_k ? k_scales : v_scales)[th] = scale;
+    }
+    auto code = [&](float x) {
+        const float f = x * inv;
+        if (kv_format == PIE_HIP_KV_INT8_PER_TOKEN_HEAD) {
+            int qv = static_cast<int>(rintf(f));
+            qv = qv > 127 ? 127 : (qv < -128 ? -128 : qv);
+            return static_cast<unsigned char>(static_cast<int8_t>(qv));
+        }
+        const float c = fminf(fmaxf(f, -448.f), 448.f);
+        return static_cast<unsigned char>(__builtin_amdgcn_cvt_pk_fp8_f32(c, c, 0, false) & 0xFF);
+    };
+#pragma unroll
+    for (int it = 0; it < ITER; ++it) {
+        const int i = lane + it * kWave;
+        if (i < half) {
+            const int ia = interleaved ? 2 * i : i, ib = interleaved ? 2 * i + 1 : i + half;
+            dst[ia] = code(va[it]);
+            dst[ib] = code(vb[it]);
+        }
+    }
+}
+
 }  // namespace
 }  // namespace pie_hip
+
+extern "C" int pie_hip_qkv_rope_kvwrite_quant(int kv_format, const uint16_t* packed_qkv, uint16_t* q_out,
+                                              void* k_pages, void* v_pages, float* k_scales,
+                                              float* v_scales, const uint16_t* q_norm_weight,
+                                              const uint16_t* k_norm_weight, const float* rope_table,
+                                              const int64_t* kv_slots, int num_tokens, int num_q_heads,
+                                              int num_kv_heads, int head_dim, int interleaved, float eps,
+                                              void* stream) {
+    using namespace pie_hip;
+    if (!packed_qkv || !q_out || !k_pages || !v_pages || !rope_table || !kv_slots || num_tokens <= 0 ||
+        num_q_heads <= 0 || num_kv_heads <= 0 || head_dim <= 0)
+        return PIE_HIP_ERR_INVALID;
+    if (!q_norm_weight != !k_norm_weight) return PIE_HIP_ERR_INVALID;
+    const bool scaled = kv_format == PIE_HIP_KV_INT8_PER_TOKEN_HEAD || kv_format == PIE_HIP_KV_FP8_PER_TOKEN_HEAD;
+    if (kv_format != PIE_HIP_KV_FP8_E4M3 && !scaled) return PIE_HIP_ERR_UNSUPPORTED;
+    if (scaled && (!k_scales || !v_scales)) return PIE_HIP_ERR_INVALID;
+    if (head_dim % 8 != 0 || head_dim > 256 || num_q_heads + 2 * num_kv_heads > 65535) return PIE_HIP_ERR_UNSUPPORTED;
+    const dim3 grid(num_tokens, num_q_heads + 2 * num_kv_heads);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    unsigned char* kp = static_cast<unsigned char*>(k_pages);
+    unsigned char* vp = static_cast<unsigned char*>(v_pages);
+    if (head_dim <= 128)
+        hipLaunchKernelGGL(qkv_rope_kvwrite_quant_kernel<1>, grid, dim3(64), 0, st, packed_qkv, q_out, kp, vp,
+                           k_scales, v_scales, q_norm_weight, k_norm_weight, rope_table, kv_slots,
+                           num_q_heads, num_kv_heads, head_dim, interleaved, eps, kv_format);
+    else
+        hipLaunchKernelGGL(qkv_rope_kvwrite_quant_kernel<2>, grid, dim3(64), 0, st, packed_qkv, q_out, kp, vp,
+                           k_scales, v_scales, q_norm_weight, k_norm_weight, rope_table, kv_slots,
+                           num_q_heads, num_kv_heads, head_dim, interleaved, eps, kv_format);
+    return launch_status();
+}
 
 extern "C" int pie_hip_kv_write_quant(int kv_format, const uint16_t* k_rows, const uint16_t* v_rows,
                                       const int64_t* kv_slots, void* k_pages, void* v_pages,

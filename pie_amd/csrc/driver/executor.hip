@@ -371,10 +371,18 @@ void Executor::body(int N, int S, int max_kv_len) {
             // one-byte pools: the rotated K / V rows of this step are staged as bf16 rows (row t
             // in "slot" t) and quantised into the tokens' real slots
             linear_fused(w.wqkv, x_, w.attn_norm, m.rms_eps, qkv_, N, 0, 0, xn_, gemm_ws_, gemm_ws_bytes_, s);
-            PIE_KERNEL(pie_hip_qkv_rope_kvwrite(qkv_, q_, k_rows_, v_rows_, w.q_norm, w.k_norm, rope_tab_,
-                                                iota_slots_, N, hq, hk, d, m.rope_interleaved, m.rms_eps, s));
-            PIE_KERNEL(pie_hip_kv_write_quant(kv_format_, k_rows_, v_rows_, slots, k_pool_[l], v_pool_[l],
-                                              ksc, vsc, N, hk, d, s));
+            // rotation and quantising write in one launch; head dims past 256 take the two kernels
+            const int st = pie_hip_qkv_rope_kvwrite_quant(kv_format_, qkv_, q_, k_pool_[l], v_pool_[l], ksc, vsc,
+                                                          w.q_norm, w.k_norm, rope_tab_, slots, N, hq, hk, d,
+                                                          m.rope_interleaved, m.rms_eps, s);
+            if (st == PIE_HIP_ERR_UNSUPPORTED) {
+                PIE_KERNEL(pie_hip_qkv_rope_kvwrite(qkv_, q_, k_rows_, v_rows_, w.q_norm, w.k_norm, rope_tab_,
+                                                    iota_slots_, N, hq, hk, d, m.rope_interleaved, m.rms_eps, s));
+                PIE_KERNEL(pie_hip_kv_write_quant(kv_format_, k_rows_, v_rows_, slots, k_pool_[l], v_pool_[l],
+                                                  ksc, vsc, N, hk, d, s));
+            } else {
+                PIE_KERNEL(st);
+            }
         } else if (N <= 4 && m.rope_interleaved && !w.q_norm && (d & (d - 1)) == 0) {
             // decode rows of llama-type layers: rotation and KV write ride in the projection
             PIE_KERNEL(pie_hip_qkv_rope_fused(fmt_code(w.wqkv.kind), x_, w.attn_norm, m.rms_eps,

@@ -777,6 +777,36 @@ def kv_write_quant(fmt: str, k_rows: torch.Tensor, v_rows: torch.Tensor, kv_slot
                                             N, hk, d, _stream()), "pie_hip_kv_write_quant")
 
 
+def qkv_rope_kvwrite_quant(fmt: str, packed: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
+                           k_scales: Optional[torch.Tensor], v_scales: Optional[torch.Tensor],
+                           table: torch.Tensor, kv_slots: torch.Tensor, hq: int, hk: int, d: int,
+                           interleaved: bool, q_norm_w=None, k_norm_w=None, eps: float = 1e-6) -> torch.Tensor:
+    """RoPE (+ optional per-head q/k norm) and the quantising KV write in one launch over packed
+    q|k|v rows [N, (hq + 2 hk) d]; returns q [N, hq, d]."""
+    _dev(packed, torch.bfloat16, "packed")
+    _dev(table, torch.float32, "rope_table")
+    _dev(kv_slots, torch.int64, "kv_slots")
+    N = packed.shape[0]
+    if packed.shape[1] != (hq + 2 * hk) * d or tuple(table.shape) != (N, d) or kv_slots.numel() != N:
+        raise KernelError("shape mismatch")
+    for t in (k_pages, v_pages):
+        if t.element_size() != 1 or not t.is_contiguous() or t.shape[-2:] != (hk, d):
+            raise KernelError("pools must be contiguous one-byte [pages, ps, hk, d]")
+    if N and int(kv_slots.max()) >= k_pages.numel() // (hk * d):
+        raise KernelError("kv slot out of range")
+    for sc in (k_scales, v_scales):
+        if sc is not None:
+            _dev(sc, torch.float32, "scales")
+            if sc.numel() != k_pages.numel() // d:
+                raise KernelError("scales must be [pages, ps, hk]")
+    q_out = torch.empty((N, hq, d), dtype=torch.bfloat16, device=packed.device)
+    _check(kernels().pie_hip_qkv_rope_kvwrite_quant(
+        KV_FORMATS[fmt], _ptr(packed), _ptr(q_out), _ptr(k_pages), _ptr(v_pages), _ptr(k_scales),
+        _ptr(v_scales), _ptr(q_norm_w), _ptr(k_norm_w), _ptr(table), _ptr(kv_slots), N, hq, hk, d,
+        int(interleaved), C.c_float(eps), _stream()), "pie_hip_qkv_rope_kvwrite_quant")
+    return q_out
+
+
 def attention_rows_paged_kvq(fmt: str, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                              k_scales: Optional[torch.Tensor], v_scales: Optional[torch.Tensor],
                              kv_page_indices: torch.Tensor, row_page_begin: torch.Tensor,

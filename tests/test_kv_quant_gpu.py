@@ -97,3 +97,51 @@ def test_quantised_pool_argument_checks(gpu):
     sc = torch.ones((2, 16, 2), dtype=torch.float32, device=gpu)
     with pytest.raises(ops.KernelError):   # plain fp8 takes none
         ops.attention_rows_paged_kvq("fp8_e4m3", q, pool, pool, sc, sc, idx, idx, one)
+
+
+@pytest.mark.parametrize("fmt", FORMATS)
+@pytest.mark.parametrize("hq,hk,d,interleaved,qk_norm", [(8, 2, 128, True, False), (4, 4, 64, False, True),
+                                                        (4, 1, 256, False, False), (6, 3, 96, True, True)])
+def test_rope_and_quantising_write_in_one_launch_equal_the_two_kernels(gpu, oracle, fmt, hq, hk, d,
+                                                                       interleaved, qk_norm):
+    """RoPE + quantising KV write fused: q, codes and scales are the bytes of the rope kernel
+    (into staged bf16 rows) followed by the quantising write (both pinned against the oracle)."""
+    import torch
+    from pie_amd import ops
+
+    rng = np.random.default_rng(60 + hq + d)
+    N, pages, ps = 21, 6, 16
+    packed = dev(oracle.f32_to_bf16((rng.standard_normal((N, (hq + 2 * hk) * d)) * 3).astype(np.float32)), gpu,
+                 torch.bfloat16)
+    pos = rng.integers(0, 3000, N).astype(np.int32)
+    tab = ops.rope_table(dev(pos, gpu), dev(oracle.rope_inv_freq(d, 500000.0), gpu), d)
+    slots = rng.permutation(pages * ps)[:N].astype(np.int64)
+    slots[2] = -1
+    sg = dev(slots, gpu)
+    qn = dev(oracle.f32_to_bf16(rng.uniform(0.5, 1.5, d).astype(np.float32)), gpu, torch.bfloat16) if qk_norm else None
+    kn = dev(oracle.f32_to_bf16(rng.uniform(0.5, 1.5, d).astype(np.float32)), gpu, torch.bfloat16) if qk_norm else None
+    scaled = fmt != "fp8_e4m3"
+
+    def pools():
+        kp = torch.full((pages, ps, hk, d), 0x55, dtype=torch.uint8, device=gpu)
+        vp = torch.full((pages, ps, hk, d), 0x55, dtype=torch.uint8, device=gpu)
+        ks = torch.full((pages, ps, hk), -7.0, dtype=torch.float32, device=gpu) if scaled else None
+        vs = torch.full((pages, ps, hk), -7.0, dtype=torch.float32, device=gpu) if scaled else None
+        return kp, vp, ks, vs
+
+    a = pools()
+    q1 = ops.qkv_rope_kvwrite_quant(fmt, packed, a[0], a[1], a[2], a[3], tab, sg, hq, hk, d, interleaved, qn, kn,
+                                    eps=1e-6)
+    # two kernels: rotated K / V as bf16 rows (row t in slot t), then the quantising write
+    k_rows = torch.zeros((N, hk, d), dtype=torch.bfloat16, device=gpu)
+    v_rows = torch.zeros((N, hk, d), dtype=torch.bfloat16, device=gpu)
+    iota = dev(np.arange(N, dtype=np.int64), gpu)
+    q2 = ops.qkv_rope_kvwrite(packed, k_rows, v_rows, tab, iota, hq, hk, d, interleaved, qn, kn, eps=1e-6)
+    b = pools()
+    ops.kv_write_quant(fmt, k_rows, v_rows, sg, b[0], b[1], b[2], b[3])
+    torch.cuda.synchronize()
+    assert torch.equal(q1.view(torch.int16), q2.view(torch.int16))
+    for x, y in zip(a, b):
+        if x is not None:
+            assert torch.equal(x, y)
+    assert not torch.all(a[0] == 0x55)
