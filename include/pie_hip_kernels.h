@@ -438,6 +438,17 @@ int pie_hip_attn_rows_paged_kvq(int kv_format, const uint16_t* q, const void* k_
                                 int num_rows, int num_q_heads, int num_kv_heads, int head_dim,
                                 int page_size, float sm_scale, int max_kv_len, void* workspace,
                                 size_t workspace_bytes, void* stream);
+/* The same over rows with custom attention masks: mask_bitmap as for
+ * pie_hip_attn_rows_paged_masked (one visibility word per row and 16-token unit). */
+int pie_hip_attn_rows_paged_kvq_masked(int kv_format, const uint16_t* q, const void* k_pages,
+                                       const void* v_pages, const float* k_scales,
+                                       const float* v_scales, uint16_t* o, float* lse,
+                                       const uint32_t* kv_page_indices,
+                                       const uint32_t* row_page_begin, const int32_t* row_kv_len,
+                                       const uint16_t* mask_bitmap, int mask_stride_units,
+                                       int num_rows, int num_q_heads, int num_kv_heads, int head_dim,
+                                       int page_size, float sm_scale, int max_kv_len,
+                                       void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * Quantising KV write: this step's K and V rows [num_tokens, hk, d] bf16 (after RoPE) go to

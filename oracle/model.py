@@ -155,11 +155,12 @@ class OracleModel:
                       allow, allow_off, p):
         vp = lambda a: C.c_void_p(a.ctypes.data)
         if self.kv_format:
-            assert masks is None, "custom masks are not available with one-byte KV formats"
             lib().orc_llama_forward_kvq(C.byref(self._m), C.c_int(self.kv_format), self._kf, self._vf,
                                         vp(tok), vp(pos), vp(slots), vp(rb), vp(rl), vp(pages), C.c_int(N),
                                         vp(sr), C.c_int(S), C.c_int(self.cfg["page_size"]), vp(out),
-                                        vp(logits) if want_logits else None)
+                                        vp(logits) if want_logits else None,
+                                        vp(allow) if allow is not None else None,
+                                        vp(allow_off) if allow_off is not None else None)
             return out[:S], (logits[:S] if want_logits else None), p
         lib().orc_llama_forward(C.byref(self._m), self._kp, self._vp, vp(tok), vp(pos), vp(slots),
                                 vp(rb), vp(rl), vp(pages), C.c_int(N), vp(sr), C.c_int(S),

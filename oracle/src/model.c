@@ -288,8 +288,9 @@ void orc_llama_forward_kvq(const OrcModel* m, int kv_format, float* const* k_f32
                            const uint32_t* tokens, const int32_t* positions, const int64_t* kv_slots,
                            const uint32_t* row_begin, const int32_t* row_len,
                            const uint32_t* page_indices, int N, const uint32_t* sample_rows, int S,
-                           int page_size, uint32_t* out_tokens, uint16_t* logits_bf16) {
+                           int page_size, uint32_t* out_tokens, uint16_t* logits_bf16,
+                           const uint8_t* allow, const int64_t* allow_off) {
     orc_llama_forward_impl(m, NULL, NULL, kv_format, k_f32, v_f32, tokens, positions, kv_slots,
                            row_begin, row_len, page_indices, N, sample_rows, S, page_size, out_tokens,
-                           logits_bf16, NULL, NULL);
+                           logits_bf16, allow, allow_off);
 }

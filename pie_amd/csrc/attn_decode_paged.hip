@@ -905,22 +905,33 @@ int attn_dispatch(const uint16_t* q, const void* k_pages, const void* v_pages, u
     const float scale = sm_scale > 0.f ? sm_scale : 1.0f / sqrtf(static_cast<float>(head_dim));
     const int gqa = num_q_heads / num_kv_heads;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    // one-byte KV formats: plain rows only (no custom-mask instantiation), per-(token, head)
-    // scales required for int8 and the scaled fp8 form, absent for plain fp8 casts
+    // one-byte KV formats: per-(token, head) scales required for int8 and the scaled fp8 form,
+    // absent for plain fp8 casts
     if (kv_format != PIE_HIP_KV_BF16) {
-        if (mask_bits) return PIE_HIP_ERR_UNSUPPORTED;
         const bool scaled = kv_format == PIE_HIP_KV_INT8_PER_TOKEN_HEAD || kv_format == PIE_HIP_KV_FP8_PER_TOKEN_HEAD;
         if (kv_format != PIE_HIP_KV_FP8_E4M3 && !scaled) return PIE_HIP_ERR_UNSUPPORTED;
         if (scaled != (k_scales != nullptr) || scaled != (v_scales != nullptr)) return PIE_HIP_ERR_INVALID;
     }
 #define PIE_ATTN_CASE(DD, GG)                                                                  \
     if (head_dim == DD && gqa == GG) {                                                         \
+        if (kv_format == PIE_HIP_KV_INT8_PER_TOKEN_HEAD && mask_bits)                          \
+            return launch_decode<DD, GG, true, kKvInt8>(                                       \
+                q, k_pages, v_pages, k_scales, v_scales, o, lse, kv_page_indices,              \
+                kv_page_indptr, kv_last_page_lens, row_begin, row_len, num_rows, num_q_heads,  \
+                num_kv_heads, page_size, scale, max_kv_len, workspace, workspace_bytes,        \
+                mask_bits, mask_stride, st);                                                   \
         if (kv_format == PIE_HIP_KV_INT8_PER_TOKEN_HEAD)                                       \
             return launch_decode<DD, GG, false, kKvInt8>(                                      \
                 q, k_pages, v_pages, k_scales, v_scales, o, lse, kv_page_indices,              \
                 kv_page_indptr, kv_last_page_lens, row_begin, row_len, num_rows, num_q_heads,  \
                 num_kv_heads, page_size, scale, max_kv_len, workspace, workspace_bytes,        \
                 nullptr, 0, st);                                                               \
+        if (kv_format != PIE_HIP_KV_BF16 && mask_bits)                                         \
+            return launch_decode<DD, GG, true, kKvFp8>(                                        \
+                q, k_pages, v_pages, k_scales, v_scales, o, lse, kv_page_indices,              \
+                kv_page_indptr, kv_last_page_lens, row_begin, row_len, num_rows, num_q_heads,  \
+                num_kv_heads, page_size, scale, max_kv_len, workspace, workspace_bytes,        \
+                mask_bits, mask_stride, st);                                                   \
         if (kv_format != PIE_HIP_KV_BF16)                                                      \
             return launch_decode<DD, GG, false, kKvFp8>(                                       \
                 q, k_pages, v_pages, k_scales, v_scales, o, lse, kv_page_indices,              \
@@ -998,6 +1009,24 @@ extern "C" int pie_hip_attn_rows_paged_kvq(int kv_format, const uint16_t* q, con
                                   row_page_begin, row_kv_len, num_rows, num_q_heads, num_kv_heads,
                                   head_dim, page_size, sm_scale, max_kv_len, workspace,
                                   workspace_bytes, stream, nullptr, 0, kv_format, k_scales, v_scales);
+}
+
+extern "C" int pie_hip_attn_rows_paged_kvq_masked(int kv_format, const uint16_t* q, const void* k_pages,
+                                                  const void* v_pages, const float* k_scales,
+                                                  const float* v_scales, uint16_t* o, float* lse,
+                                                  const uint32_t* kv_page_indices,
+                                                  const uint32_t* row_page_begin,
+                                                  const int32_t* row_kv_len, const uint16_t* mask_bitmap,
+                                                  int mask_stride_units, int num_rows, int num_q_heads,
+                                                  int num_kv_heads, int head_dim, int page_size,
+                                                  float sm_scale, int max_kv_len, void* workspace,
+                                                  size_t workspace_bytes, void* stream) {
+    if (!row_page_begin || !row_kv_len || !mask_bitmap || mask_stride_units <= 0) return PIE_HIP_ERR_INVALID;
+    return pie_hip::attn_dispatch(q, k_pages, v_pages, o, lse, kv_page_indices, nullptr, nullptr,
+                                  row_page_begin, row_kv_len, num_rows, num_q_heads, num_kv_heads,
+                                  head_dim, page_size, sm_scale, max_kv_len, workspace,
+                                  workspace_bytes, stream, mask_bitmap, mask_stride_units, kv_format,
+                                  k_scales, v_scales);
 }
 
 namespace pie_hip {

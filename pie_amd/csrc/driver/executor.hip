@@ -410,8 +410,12 @@ void Executor::body(int N, int S, int max_kv_len) {
                                                     m.rms_eps, s));
             }
         }
-        if (kvq) {
-            if (masked_) throw std::runtime_error("executor: custom attention masks need a bf16 KV cache");
+        if (kvq && masked_) {
+            PIE_KERNEL(pie_hip_attn_rows_paged_kvq_masked(
+                kv_format_, q_, k_pool_[l], v_pool_[l], ksc, vsc, attn_, nullptr, pages, row_begin, row_len,
+                static_cast<const uint16_t*>(mask_bitmap_.ptr), mask_stride_, N, hq, hk, d, page_size_, -1.f,
+                max_kv_len, attn_ws_, attn_ws_bytes_, s));
+        } else if (kvq) {
             PIE_KERNEL(pie_hip_attn_rows_paged_kvq(kv_format_, q_, k_pool_[l], v_pool_[l], ksc, vsc, attn_,
                                                    nullptr, pages, row_begin, row_len, N, hq, hk, d,
                                                    page_size_, -1.f, max_kv_len, attn_ws_, attn_ws_bytes_, s));

@@ -419,15 +419,55 @@ def test_page_copies_carry_one_byte_pages_and_their_scales(gpu, oracle, kv_dtype
             assert tk == outs[0][0] and np.array_equal(lg, outs[0][1])
 
 
-def test_custom_masks_are_refused_with_a_one_byte_kv_cache(gpu):
+@pytest.mark.parametrize("kv", ["fp8_per_token_head", "int8_per_token_head"])
+def test_custom_masks_over_a_one_byte_kv_cache_match_oracle(gpu, oracle, kv):
+    """Per-token BRLE masks with one-byte KV pools: prefill rows and a decode step against the
+    oracle model reading the same quantised values (the bars of the one-byte generation test)."""
     from pie_amd import driver as drvmod
 
-    with drvmod.Driver(toml_config(kv_cache_dtype="fp8_per_token_head")) as d:
-        toks = np.arange(5)
-        fr = drvmod.ForwardFrame(toks, np.arange(5), [0], [0, 1], [5], [0, 5],
-                                 masks=[[0, 1, 1, 5] for _ in range(5)])   # key 1 hidden
-        assert d.forward(fr).num_requests == 0
-        assert d.forward(drvmod.ForwardFrame(toks, np.arange(5), [0], [0, 1], [5], [0, 5])).num_requests == 1
+    kw = dict(quant="int8", kv_cache_dtype=kv)
+    cfg = full_cfg(**kw)
+    V, ps = cfg["vocab"], cfg["page_size"]
+    rng = np.random.default_rng(97)
+    n = 37
+    prompt = rng.integers(0, V, n)
+    masks = []
+    for i in range(n):
+        if i % 3 == 0:
+            masks.append([])                              # plain causal
+        else:
+            a = int(rng.integers(0, i + 1))
+            masks.append([a, int(rng.integers(1, 8)), int(rng.integers(0, 5)), n])
+    masks[5] = [0, 1, 100]                                # only key 0
+    bars = dict(cos_min=0.998, rel=0.1, tie=2.0 ** -4)
+    with drvmod.Driver(toml_config(**kw)) as d:
+        om, _ = oracle_model_from_driver(d, cfg)
+        npg = (n + ps - 1) // ps
+        args = dict(token_ids=prompt, position_ids=np.arange(n), kv_page_indices=np.arange(npg),
+                    kv_page_indptr=[0, npg], kv_last_page_lens=[n - (npg - 1) * ps], qo_indptr=[0, n],
+                    sampling_indices=[n - 1, 5, 20], sampling_indptr=[0, 3])
+        res = d.forward(drvmod.ForwardFrame(**args, masks=masks))
+        assert res.num_requests == 1 and len(res.tokens) == 3
+        otok, olog, _ = om.forward(**args, masks=masks, want_logits=True)
+        glog = d.export_tensor("debug.logits", np.uint16).reshape(-1, V)
+        for i in range(3):
+            check_step(oracle, glog[i], olog[i], res.tokens[i], otok[i], **bars)
+        step = dict(token_ids=[int(otok[0])], position_ids=[n], kv_page_indices=np.arange(npg),
+                    kv_page_indptr=[0, npg], kv_last_page_lens=[n + 1 - (npg - 1) * ps], qo_indptr=[0, 1])
+        m = [[n // 2, n]]
+        res = d.forward(drvmod.ForwardFrame(**step, masks=m))
+        otok2, olog2, _ = om.forward(**step, masks=m, want_logits=True)
+        glog2 = d.export_tensor("debug.logits", np.uint16).reshape(-1, V)
+        check_step(oracle, glog2[0], olog2[0], res.tokens[0], otok2[0], **bars)
+        # the mask matters: the unmasked step gives other logits
+        res3 = d.forward(drvmod.ForwardFrame(**step))
+        glog3 = d.export_tensor("debug.logits", np.uint16).reshape(-1, V)
+        assert cosine(oracle.bf16_to_f32(glog3[0]), oracle.bf16_to_f32(glog2[0])) < 0.9999
+
+
+def test_unknown_kv_cache_dtypes_are_refused(gpu):
+    from pie_amd import driver as drvmod
+
     for bad, msg in (("fp8_e5m2", "not implemented"), ("turboquant", "invalid kv_cache_dtype")):
         with pytest.raises(Exception, match=msg):
             drvmod.Driver(toml_config(kv_cache_dtype=bad))
