@@ -266,6 +266,17 @@ int pie_hip_attn_prefill_tiles(const uint16_t* q, const uint16_t* k_pages, const
                                const int32_t* tile_row_start, const int32_t* tile_num_rows,
                                int num_tiles, int rows_per_tile, int num_q_heads, int num_kv_heads,
                                int head_dim, int page_size, float sm_scale, void* stream);
+/* The same over one-byte KV pools (kv_format / k_scales / v_scales as for
+ * pie_hip_attn_rows_paged_kvq; PIE_HIP_KV_BF16 with null scales is pie_hip_attn_prefill_tiles):
+ * codes are decoded exactly into the bf16 tiles, the K scale multiplies the score and the V
+ * scale the rounded probability. */
+int pie_hip_attn_prefill_tiles_kvq(int kv_format, const uint16_t* q, const void* k_pages,
+                                   const void* v_pages, const float* k_scales, const float* v_scales,
+                                   uint16_t* o, const uint32_t* kv_page_indices,
+                                   const uint32_t* row_page_begin, const int32_t* row_kv_len,
+                                   const int32_t* tile_row_start, const int32_t* tile_num_rows,
+                                   int num_tiles, int rows_per_tile, int num_q_heads, int num_kv_heads,
+                                   int head_dim, int page_size, float sm_scale, void* stream);
 
 /*
  * Custom attention masks for the per-row form.  pie_hip_attn_mask_bitmap turns per-row BRLE

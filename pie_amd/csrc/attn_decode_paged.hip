@@ -65,60 +65,6 @@ __device__ __forceinline__ RowExtent row_extent(const uint32_t* __restrict__ pag
     return {lo, npages > 0 ? (npages - 1) * ps + static_cast<int>(last_lens[r]) : 0};
 }
 
-// KV storage of the pool (driver/cuda/src/kv_cache_format.hpp:11-17): bf16; one-byte e4m3 with
-// optional fp32 scales per (token, kv head) — "fp8_e4m3" stores casts, "fp8_per_token_head"
-// stores x / scale; int8 with such scales.  A lane still owns 8 elements of a row: 16 bytes of
-// bf16 or 8 bytes of a one-byte format.  Values are decoded as the reference's load_kv_scalar
-// does (driver/cuda/src/ops/attention_naive_paged.cu:56-112): float(code) * scale.
-constexpr int kKvBf16 = 0, kKvFp8 = 1, kKvInt8 = 2;
-
-template <int KVF>
-struct KvVec {
-    using type = u32x4_t;
-};
-template <>
-struct KvVec<kKvFp8> {
-    using type = u32x2_t;
-};
-template <>
-struct KvVec<kKvInt8> {
-    using type = u32x2_t;
-};
-
-__device__ __forceinline__ uint32_t kv_pack_trunc(float lo, float hi) {
-    return __builtin_amdgcn_perm(__float_as_uint(hi), __float_as_uint(lo), 0x07060302u);
-}
-// 8 stored elements -> 8 floats / 4 bf16 pairs (every code is exact in bf16)
-template <int KVF>
-__device__ __forceinline__ void kv_decode_f32(const typename KvVec<KVF>::type r, float* f) {
-    if constexpr (KVF == kKvBf16) {
-        f[0] = bf16_lo(r.x); f[1] = bf16_hi(r.x); f[2] = bf16_lo(r.y); f[3] = bf16_hi(r.y);
-        f[4] = bf16_lo(r.z); f[5] = bf16_hi(r.z); f[6] = bf16_lo(r.w); f[7] = bf16_hi(r.w);
-    } else if constexpr (KVF == kKvFp8) {
-        typedef float f32x2_t __attribute__((ext_vector_type(2)));
-        const f32x2_t a = __builtin_amdgcn_cvt_pk_f32_fp8(r.x, false), b = __builtin_amdgcn_cvt_pk_f32_fp8(r.x, true);
-        const f32x2_t c = __builtin_amdgcn_cvt_pk_f32_fp8(r.y, false), d = __builtin_amdgcn_cvt_pk_f32_fp8(r.y, true);
-        f[0] = a.x; f[1] = a.y; f[2] = b.x; f[3] = b.y; f[4] = c.x; f[5] = c.y; f[6] = d.x; f[7] = d.y;
-    } else {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            f[e] = static_cast<float>(static_cast<int8_t>(r.x >> (8 * e)));
-            f[4 + e] = static_cast<float>(static_cast<int8_t>(r.y >> (8 * e)));
-        }
-    }
-}
-template <int KVF>
-__device__ __forceinline__ u32x4_t kv_decode_bf16(const typename KvVec<KVF>::type r) {
-    if constexpr (KVF == kKvBf16) {
-        return r;
-    } else {
-        float f[8];
-        kv_decode_f32<KVF>(r, f);
-        return u32x4_t{kv_pack_trunc(f[0], f[1]), kv_pack_trunc(f[2], f[3]), kv_pack_trunc(f[4], f[5]),
-                       kv_pack_trunc(f[6], f[7])};
-    }
-}
-
 template <int D, int GQA, int KVF = kKvBf16>
 struct UnitRegs {
     static constexpr int LPR = D / 8;

@@ -39,10 +39,14 @@ __device__ __forceinline__ int vt_slot(int kappa) {
 
 // QT: 16-row MFMA tiles per wave (2: 128 rows per block, K/V fragments read once per two tiles;
 // 1: 64 rows per block, twice the blocks for small batches).
-template <int D, int GQA, int QT>
+// KVF: one-byte pools (the codes become bf16 — exactly — on the way into the LDS tiles, one
+// 16-code piece per thread and matrix; the step's per-(token, kv head) scales sit in LDS and
+// multiply the scores (K) and the probabilities (V): float(code) * scale as in the row kernels).
+template <int D, int GQA, int QT, int KVF = kKvBf16>
 __global__ __launch_bounds__(kTileThreads) void attn_prefill_tile_kernel(
-    const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_pages,
-    const uint16_t* __restrict__ v_pages, uint16_t* __restrict__ o,
+    const uint16_t* __restrict__ q, const void* __restrict__ k_pages_raw,
+    const void* __restrict__ v_pages_raw, const float* __restrict__ k_scales,
+    const float* __restrict__ v_scales, uint16_t* __restrict__ o,
     const uint32_t* __restrict__ page_indices, const uint32_t* __restrict__ row_begin,
     const int32_t* __restrict__ row_len, const int32_t* __restrict__ tile_start,
     const int32_t* __restrict__ tile_rows, int hq, int hk, int ps, float scale_log2e) {
@@ -51,8 +55,16 @@ __global__ __launch_bounds__(kTileThreads) void attn_prefill_tile_kernel(
     constexpr int DT = D / 16;             // d tiles of the second product
     constexpr int LPR = D / 8;             // 16-byte pieces per K/V row
     constexpr int KSTRIDE = D + 8;         // bf16 elements per K row in LDS
-    constexpr int PIECES = kStepKeys * LPR / kTileThreads;   // 16-byte pieces per thread per matrix
+    constexpr bool Q8 = KVF != kKvBf16;
+    constexpr int LPRQ = D / 16;           // 16-code pieces per one-byte row
+    constexpr int PIECES = Q8 ? 1 : kStepKeys * LPR / kTileThreads;   // 16-byte pieces per thread per matrix
     static_assert(PIECES >= 1 && (PIECES % 2 == 0 || PIECES == 1), "piece mapping");
+    static_assert(kStepKeys * LPRQ <= kTileThreads, "one-byte pieces fit one per thread");
+    const uint16_t* k_pages = static_cast<const uint16_t*>(k_pages_raw);
+    const uint16_t* v_pages = static_cast<const uint16_t*>(v_pages_raw);
+    const unsigned char* k_bytes = static_cast<const unsigned char*>(k_pages_raw);
+    const unsigned char* v_bytes = static_cast<const unsigned char*>(v_pages_raw);
+    __shared__ __attribute__((aligned(16))) float s_sc[Q8 ? 2 * kStepKeys : 1];   // K | V scales of a step
 
     __shared__ __attribute__((aligned(16))) uint16_t Ks[kStepKeys * KSTRIDE];
     __shared__ __attribute__((aligned(16))) uint16_t Vt[D * kVtStride];
@@ -95,7 +107,13 @@ __global__ __launch_bounds__(kTileThreads) void attn_prefill_tile_kernel(
     constexpr int PAIRS = kStepKeys / 2;
     constexpr int PF = 2;   // steps of K/V in flight
     u32x4_t kreg[PF][PIECES], vreg[PF][PIECES];
+    float sreg[PF];   // one-byte pools: thread t < 32 holds the K scale of key t, t < 64 V's
     auto piece_of = [&](int u, int& key, int& dc) {
+        if constexpr (Q8) {   // thread -> (key, 16-code piece); threads past the tile idle
+            key = tid % kStepKeys;
+            dc = tid / kStepKeys;
+            return;
+        }
         if (PIECES == 1) {   // D = 64: one piece per thread
             key = tid % kStepKeys;
             dc = tid / kStepKeys;
@@ -114,19 +132,57 @@ __global__ __launch_bounds__(kTileThreads) void attn_prefill_tile_kernel(
         const int page_a = ja / ps;
         const uint32_t pid_a = __builtin_amdgcn_readfirstlane(page_indices[pg_lo + page_a]);
         const uint32_t pid_b = __builtin_amdgcn_readfirstlane(page_indices[pg_lo + jb / ps]);
+        auto token_head = [&](int key) {
+            const int j = min(j0 + key, kmax - 1);
+            const int page = j / ps;
+            const uint32_t pid = page == page_a ? pid_a : pid_b;
+            return (static_cast<size_t>(pid) * ps + (j - page * ps)) * hk + kvh;
+        };
+        if constexpr (Q8) {
+            int key, dc;
+            piece_of(0, key, dc);
+            if (dc < LPRQ) {
+                const size_t off = token_head(key) * D + dc * 16;
+                kreg[slot][0] = *reinterpret_cast<const u32x4_t*>(k_bytes + off);
+                vreg[slot][0] = *reinterpret_cast<const u32x4_t*>(v_bytes + off);
+            }
+            if (tid < 2 * kStepKeys) {
+                const float* sp = tid < kStepKeys ? k_scales : v_scales;
+                sreg[slot] = sp ? sp[token_head(tid % kStepKeys)] : 1.f;
+            }
+            return;
+        }
 #pragma unroll
         for (int u = 0; u < PIECES; ++u) {
             int key, dc;
             piece_of(u, key, dc);
-            const int j = min(j0 + key, kmax - 1);
-            const int page = j / ps;
-            const uint32_t pid = page == page_a ? pid_a : pid_b;
-            const size_t off = ((static_cast<size_t>(pid) * ps + (j - page * ps)) * hk + kvh) * D + dc * 8;
+            const size_t off = token_head(key) * D + dc * 8;
             kreg[slot][u] = *reinterpret_cast<const u32x4_t*>(k_pages + off);
             vreg[slot][u] = *reinterpret_cast<const u32x4_t*>(v_pages + off);
         }
     };
     auto stage = [&](int slot) {
+        if constexpr (Q8) {
+            int key, dc;
+            piece_of(0, key, dc);
+            if (dc < LPRQ) {
+                const u32x4_t kw = kreg[slot][0], vw = vreg[slot][0];
+                uint16_t* kd = &Ks[key * KSTRIDE + dc * 16];
+                *reinterpret_cast<u32x4_t*>(kd) = kv_decode_bf16<KVF>(u32x2_t{kw.x, kw.y});
+                *reinterpret_cast<u32x4_t*>(kd + 8) = kv_decode_bf16<KVF>(u32x2_t{kw.z, kw.w});
+                const int col = vt_slot(key);
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    float f[8];
+                    kv_decode_f32<KVF>(u32x2_t{vw[2 * h], vw[2 * h + 1]}, f);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        Vt[(dc * 16 + 8 * h + e) * kVtStride + col] = static_cast<uint16_t>(__float_as_uint(f[e]) >> 16);
+                }
+            }
+            if (tid < 2 * kStepKeys) s_sc[tid] = sreg[slot];
+            return;
+        }
 #pragma unroll
         for (int u = 0; u < PIECES; ++u) {
             int key, dc;
@@ -170,6 +226,15 @@ __global__ __launch_bounds__(kTileThreads) void attn_prefill_tile_kernel(
         __syncthreads();   // the previous step's LDS reads are done
         stage(slot);
         __syncthreads();
+        // (one-byte pools) the scales of this lane's keys 16nt + 4g + r
+        f32x4_t ksc[2], vsc[2];
+        if constexpr (Q8) {
+#pragma unroll
+            for (int nt = 0; nt < 2; ++nt) {
+                ksc[nt] = *reinterpret_cast<const f32x4_t*>(&s_sc[16 * nt + 4 * g]);
+                vsc[nt] = *reinterpret_cast<const f32x4_t*>(&s_sc[kStepKeys + 16 * nt + 4 * g]);
+            }
+        }
         if (j0 + PF * kStepKeys < kmax) issue(slot, j0 + PF * kStepKeys);
 
         // S^T = K . Q^T for both query tiles
@@ -200,7 +265,8 @@ __global__ __launch_bounds__(kTileThreads) void attn_prefill_tile_kernel(
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const int key = j0 + 16 * nt + 4 * g + r;
-                    const float v = key < my_len[qt] ? st[qt][nt][r] * scale_log2e : -INFINITY;
+                    const float sc = Q8 ? scale_log2e * ksc[nt][r] : scale_log2e;
+                    const float v = key < my_len[qt] ? st[qt][nt][r] * sc : -INFINITY;
                     s[4 * nt + r] = v;
                     m_new = fmaxf(m_new, v);
                 }
@@ -213,7 +279,17 @@ __global__ __launch_bounds__(kTileThreads) void attn_prefill_tile_kernel(
             for (int e = 0; e < 8; ++e) s[e] = exp2f(s[e] - safe);
             const u32x4_t packed = {pack_bf16x2(s[0], s[1]), pack_bf16x2(s[2], s[3]),
                                     pack_bf16x2(s[4], s[5]), pack_bf16x2(s[6], s[7])};
-            pf[qt] = __builtin_bit_cast(bf16x8_t, packed);
+            if constexpr (Q8) {
+                // V = float(code) * scale: the rounded weight times the key's scale multiplies the codes
+                const u32x4_t scaled = {
+                    pack_bf16x2(bf16_lo(packed[0]) * vsc[0][0], bf16_hi(packed[0]) * vsc[0][1]),
+                    pack_bf16x2(bf16_lo(packed[1]) * vsc[0][2], bf16_hi(packed[1]) * vsc[0][3]),
+                    pack_bf16x2(bf16_lo(packed[2]) * vsc[1][0], bf16_hi(packed[2]) * vsc[1][1]),
+                    pack_bf16x2(bf16_lo(packed[3]) * vsc[1][2], bf16_hi(packed[3]) * vsc[1][3])};
+                pf[qt] = __builtin_bit_cast(bf16x8_t, scaled);
+            } else {
+                pf[qt] = __builtin_bit_cast(bf16x8_t, packed);
+            }
             // the normaliser sums the rounded weights, the ones that multiply V: the output stays
             // an exact weighted mean of V rows
             float sum = 0.f;
@@ -263,13 +339,25 @@ __global__ __launch_bounds__(kTileThreads) void attn_prefill_tile_kernel(
 }
 
 template <int D, int GQA, int QT>
-int launch_tiles(const uint16_t* q, const uint16_t* k_pages, const uint16_t* v_pages, uint16_t* o,
+int launch_tiles(int kv_format, const uint16_t* q, const void* k_pages, const void* v_pages,
+                 const float* k_scales, const float* v_scales, uint16_t* o,
                  const uint32_t* page_indices, const uint32_t* row_begin, const int32_t* row_len,
                  const int32_t* tile_start, const int32_t* tile_rows, int num_tiles, int hq, int hk,
                  int ps, float scale, hipStream_t stream) {
-    hipLaunchKernelGGL((attn_prefill_tile_kernel<D, GQA, QT>), dim3(num_tiles, hk), dim3(kTileThreads), 0,
-                       stream, q, k_pages, v_pages, o, page_indices, row_begin, row_len, tile_start,
-                       tile_rows, hq, hk, ps, scale * 1.4426950408889634f);
+    const dim3 grid(num_tiles, hk);
+    const float sl = scale * 1.4426950408889634f;
+    if (kv_format == PIE_HIP_KV_BF16)
+        hipLaunchKernelGGL((attn_prefill_tile_kernel<D, GQA, QT, kKvBf16>), grid, dim3(kTileThreads), 0, stream, q,
+                           k_pages, v_pages, k_scales, v_scales, o, page_indices, row_begin, row_len,
+                           tile_start, tile_rows, hq, hk, ps, sl);
+    else if (kv_format == PIE_HIP_KV_INT8_PER_TOKEN_HEAD)
+        hipLaunchKernelGGL((attn_prefill_tile_kernel<D, GQA, QT, kKvInt8>), grid, dim3(kTileThreads), 0, stream, q,
+                           k_pages, v_pages, k_scales, v_scales, o, page_indices, row_begin, row_len,
+                           tile_start, tile_rows, hq, hk, ps, sl);
+    else
+        hipLaunchKernelGGL((attn_prefill_tile_kernel<D, GQA, QT, kKvFp8>), grid, dim3(kTileThreads), 0, stream, q,
+                           k_pages, v_pages, k_scales, v_scales, o, page_indices, row_begin, row_len,
+                           tile_start, tile_rows, hq, hk, ps, sl);
     return launch_status();
 }
 
@@ -283,18 +371,24 @@ extern "C" int pie_hip_attn_prefill_tile_rows(int num_q_heads, int num_kv_heads)
     return pie_hip::kBlockRows / gqa;
 }
 
-extern "C" int pie_hip_attn_prefill_tiles(const uint16_t* q, const uint16_t* k_pages,
-                                          const uint16_t* v_pages, uint16_t* o,
-                                          const uint32_t* kv_page_indices,
-                                          const uint32_t* row_page_begin, const int32_t* row_kv_len,
-                                          const int32_t* tile_row_start, const int32_t* tile_num_rows,
-                                          int num_tiles, int rows_per_tile, int num_q_heads,
-                                          int num_kv_heads, int head_dim, int page_size,
-                                          float sm_scale, void* stream) {
+extern "C" int pie_hip_attn_prefill_tiles_kvq(int kv_format, const uint16_t* q, const void* k_pages,
+                                              const void* v_pages, const float* k_scales,
+                                              const float* v_scales, uint16_t* o,
+                                              const uint32_t* kv_page_indices,
+                                              const uint32_t* row_page_begin, const int32_t* row_kv_len,
+                                              const int32_t* tile_row_start, const int32_t* tile_num_rows,
+                                              int num_tiles, int rows_per_tile, int num_q_heads,
+                                              int num_kv_heads, int head_dim, int page_size,
+                                              float sm_scale, void* stream) {
     using namespace pie_hip;
     if (!q || !k_pages || !v_pages || !o || !kv_page_indices || !row_page_begin || !row_kv_len ||
         !tile_row_start || !tile_num_rows || num_tiles <= 0 || page_size <= 0)
         return PIE_HIP_ERR_INVALID;
+    {
+        const bool scaled = kv_format == PIE_HIP_KV_INT8_PER_TOKEN_HEAD || kv_format == PIE_HIP_KV_FP8_PER_TOKEN_HEAD;
+        if (kv_format != PIE_HIP_KV_BF16 && kv_format != PIE_HIP_KV_FP8_E4M3 && !scaled) return PIE_HIP_ERR_UNSUPPORTED;
+        if (scaled != (k_scales != nullptr) || scaled != (v_scales != nullptr)) return PIE_HIP_ERR_INVALID;
+    }
     const int cap = pie_hip_attn_prefill_tile_rows(num_q_heads, num_kv_heads);
     if (cap == 0 || page_size % 16 != 0 || num_tiles > 0x7FFFFFFF / 2 || num_kv_heads > 65535)
         return PIE_HIP_ERR_UNSUPPORTED;
@@ -305,14 +399,14 @@ extern "C" int pie_hip_attn_prefill_tiles(const uint16_t* q, const uint16_t* k_p
     hipStream_t st = static_cast<hipStream_t>(stream);
 #define PIE_TILE_CASE(DD, GG)                                                                       \
     if (head_dim == DD && gqa == GG)                                                                \
-        return big ? launch_tiles<DD, GG, 2>(q, k_pages, v_pages, o, kv_page_indices,               \
-                                             row_page_begin, row_kv_len, tile_row_start,            \
-                                             tile_num_rows, num_tiles, num_q_heads, num_kv_heads,   \
-                                             page_size, scale, st)                                  \
-                   : launch_tiles<DD, GG, 1>(q, k_pages, v_pages, o, kv_page_indices,               \
-                                             row_page_begin, row_kv_len, tile_row_start,            \
-                                             tile_num_rows, num_tiles, num_q_heads, num_kv_heads,   \
-                                             page_size, scale, st);
+        return big ? launch_tiles<DD, GG, 2>(kv_format, q, k_pages, v_pages, k_scales, v_scales, o, \
+                                             kv_page_indices, row_page_begin, row_kv_len,           \
+                                             tile_row_start, tile_num_rows, num_tiles, num_q_heads, \
+                                             num_kv_heads, page_size, scale, st)                    \
+                   : launch_tiles<DD, GG, 1>(kv_format, q, k_pages, v_pages, k_scales, v_scales, o, \
+                                             kv_page_indices, row_page_begin, row_kv_len,           \
+                                             tile_row_start, tile_num_rows, num_tiles, num_q_heads, \
+                                             num_kv_heads, page_size, scale, st);
     PIE_TILE_CASE(128, 1)
     PIE_TILE_CASE(128, 2)
     PIE_TILE_CASE(128, 4)
@@ -323,4 +417,18 @@ extern "C" int pie_hip_attn_prefill_tiles(const uint16_t* q, const uint16_t* k_p
     PIE_TILE_CASE(64, 8)
 #undef PIE_TILE_CASE
     return PIE_HIP_ERR_UNSUPPORTED;
+}
+
+extern "C" int pie_hip_attn_prefill_tiles(const uint16_t* q, const uint16_t* k_pages,
+                                          const uint16_t* v_pages, uint16_t* o,
+                                          const uint32_t* kv_page_indices,
+                                          const uint32_t* row_page_begin, const int32_t* row_kv_len,
+                                          const int32_t* tile_row_start, const int32_t* tile_num_rows,
+                                          int num_tiles, int rows_per_tile, int num_q_heads,
+                                          int num_kv_heads, int head_dim, int page_size,
+                                          float sm_scale, void* stream) {
+    return pie_hip_attn_prefill_tiles_kvq(PIE_HIP_KV_BF16, q, k_pages, v_pages, nullptr, nullptr, o,
+                                          kv_page_indices, row_page_begin, row_kv_len, tile_row_start,
+                                          tile_num_rows, num_tiles, rows_per_tile, num_q_heads,
+                                          num_kv_heads, head_dim, page_size, sm_scale, stream);
 }

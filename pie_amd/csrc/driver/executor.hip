@@ -410,7 +410,12 @@ void Executor::body(int N, int S, int max_kv_len) {
                                                     m.rms_eps, s));
             }
         }
-        if (kvq && masked_) {
+        if (kvq && n_tiles_ > 0 && !masked_) {
+            const auto* td = static_cast<const int32_t*>(tile_in_dev_.ptr);
+            PIE_KERNEL(pie_hip_attn_prefill_tiles_kvq(kv_format_, q_, k_pool_[l], v_pool_[l], ksc, vsc, attn_,
+                                                      pages, row_begin, row_len, td, td + n_tiles_, n_tiles_,
+                                                      tile_rows_, hq, hk, d, page_size_, -1.f, s));
+        } else if (kvq && masked_) {
             PIE_KERNEL(pie_hip_attn_rows_paged_kvq_masked(
                 kv_format_, q_, k_pool_[l], v_pool_[l], ksc, vsc, attn_, nullptr, pages, row_begin, row_len,
                 static_cast<const uint16_t*>(mask_bitmap_.ptr), mask_stride_, N, hq, hk, d, page_size_, -1.f,
@@ -509,7 +514,6 @@ void Executor::prepare_tiles(const BatchPlan& plan) {
     const ModelConfig& m = model_.cfg();
     int cap = pie_hip_attn_prefill_tile_rows(m.q_heads, m.kv_heads);
     if (cap <= 0 || plan.has_user_masks || page_size_ % 16 != 0 || (m.head_dim != 64 && m.head_dim != 128)) return;
-    if (kv_format_ != PIE_HIP_KV_BF16) return;   // the tile kernel reads bf16 pools only
     long long blocks = 0;
     for (int r = 0; r < plan.R; ++r) {
         const int n = plan.qo_indptr[r + 1] - plan.qo_indptr[r];

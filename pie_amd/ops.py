@@ -750,6 +750,32 @@ def attention_prefill_tiles(q: torch.Tensor, k_pages: torch.Tensor, v_pages: tor
 KV_FORMATS = {"bf16": 0, "fp8_e4m3": 1, "int8_per_token_head": 2, "fp8_per_token_head": 3}
 
 
+def attention_prefill_tiles_kvq(fmt: str, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
+                                k_scales: Optional[torch.Tensor], v_scales: Optional[torch.Tensor],
+                                kv_page_indices: torch.Tensor, row_page_begin: torch.Tensor,
+                                row_kv_len: torch.Tensor, tile_row_start: torch.Tensor,
+                                tile_num_rows: torch.Tensor, rows_per_tile: Optional[int] = None) -> torch.Tensor:
+    """`attention_prefill_tiles` over one-byte pools [pages, ps, hk, d] (+ f32 scales [pages, ps, hk])."""
+    _dev(q, torch.bfloat16, "q")
+    for name, t in (("kv_page_indices", kv_page_indices), ("row_page_begin", row_page_begin),
+                    ("row_kv_len", row_kv_len), ("tile_row_start", tile_row_start),
+                    ("tile_num_rows", tile_num_rows)):
+        _dev(t, torch.int32, name)
+    for t in (k_pages, v_pages):
+        if t.element_size() != 1 or not t.is_contiguous():
+            raise KernelError("pools must be contiguous one-byte [pages, ps, hk, d]")
+    rows, hq, d = q.shape
+    _, ps, hk, _ = k_pages.shape
+    o = torch.zeros_like(q)
+    st = kernels().pie_hip_attn_prefill_tiles_kvq(
+        KV_FORMATS[fmt], _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(k_scales), _ptr(v_scales), _ptr(o),
+        _ptr(kv_page_indices), _ptr(row_page_begin), _ptr(row_kv_len), _ptr(tile_row_start),
+        _ptr(tile_num_rows), tile_row_start.numel(), rows_per_tile or attn_prefill_tile_rows(hq, hk), hq, hk,
+        d, ps, C.c_float(-1.0), _stream())
+    _check(st, "pie_hip_attn_prefill_tiles_kvq")
+    return o
+
+
 def kv_write_quant(fmt: str, k_rows: torch.Tensor, v_rows: torch.Tensor, kv_slots: torch.Tensor,
                    k_pages: torch.Tensor, v_pages: torch.Tensor,
                    k_scales: Optional[torch.Tensor] = None,

@@ -64,3 +64,46 @@ def test_tiles_match_oracle_and_row_kernel(gpu, oracle, hq, hk, d, ps, half):
     assert np.all(np.abs(got - rowf) <= 2.0 ** -7 * np.maximum(np.abs(rowf), np.abs(got)) + 8e-3)
     ulp = np.abs(got_bits.astype(np.int32) - row.astype(np.int32))
     assert (ulp <= 1).mean() > 0.85
+
+
+@pytest.mark.parametrize("fmt", ["fp8_e4m3", "int8_per_token_head", "fp8_per_token_head"])
+@pytest.mark.parametrize("hq,hk,d,ps", [(8, 2, 128, 16), (4, 4, 64, 16), (32, 8, 128, 32)])
+def test_tiles_over_one_byte_pools_match_the_row_kernel(gpu, oracle, fmt, hq, hk, d, ps):
+    """The tile kernel over quantised pools against the per-row kernel over the same pools (itself
+    held to the oracle in test_kv_quant_gpu.py): same codes, same scales, probabilities rounded to
+    bf16 in the tile kernel only."""
+    import torch
+
+    from pie_amd import ops
+
+    rng = np.random.default_rng(70 + hq + d)
+    ctx = [200, 75, 33, 1]
+    b = make_paged_batch(rng, ctx, hk, d, ps, f32_to_bf16=oracle.f32_to_bf16)
+    tr = ops.attn_prefill_tile_rows(hq, hk)
+    chunks = [(120, 80), (0, 75), (0, 33), (0, 1)]
+    row_begin, row_len, tile_start, tile_n = build_rows(b, ctx, chunks, tr)
+    rows = len(row_begin)
+    q = oracle.f32_to_bf16(rng.standard_normal((rows, hq, d)).astype(np.float32))
+    dev = lambda a, dt=None: (lambda t: t.view(dt) if dt is not None else t)(
+        torch.from_numpy(np.ascontiguousarray(a)).to(gpu))
+    # quantise the bf16 pools slot by slot with the library's own write kernel
+    pages = b["k_pages"].shape[0]
+    kp = torch.zeros((pages, ps, hk, d), dtype=torch.uint8, device=gpu)
+    vp = torch.zeros_like(kp)
+    scaled = fmt != "fp8_e4m3"
+    ks = torch.ones((pages, ps, hk), dtype=torch.float32, device=gpu) if scaled else None
+    vs = torch.ones((pages, ps, hk), dtype=torch.float32, device=gpu) if scaled else None
+    slots = dev(np.arange(pages * ps, dtype=np.int64))
+    ops.kv_write_quant(fmt, dev(b["k_pages"], torch.bfloat16).reshape(pages * ps, hk, d),
+                       dev(b["v_pages"], torch.bfloat16).reshape(pages * ps, hk, d), slots, kp, vp, ks, vs)
+    qd, pi, rb, rl = dev(q, torch.bfloat16), dev(b["page_indices"].view(np.int32)), dev(row_begin), dev(row_len)
+    o = ops.attention_prefill_tiles_kvq(fmt, qd, kp, vp, ks, vs, pi, rb, rl, dev(tile_start), dev(tile_n),
+                                        rows_per_tile=tr)
+    ref = ops.attention_rows_paged_kvq(fmt, qd, kp, vp, ks, vs, pi, rb, rl)[0]
+    torch.cuda.synchronize()
+    got = oracle.bf16_to_f32(o.view(torch.uint16).cpu().numpy()).astype(np.float64)
+    want = oracle.bf16_to_f32(ref.view(torch.uint16).cpu().numpy()).astype(np.float64)
+    tol = 2.0 ** -7 * np.maximum(np.abs(want), np.abs(got)) + 6e-3
+    err = np.abs(got - want)
+    assert np.all(err <= tol), f"worst {np.max(err / tol):.2f}x tol"
+    assert np.linalg.norm(got - want) <= 4e-3 * np.linalg.norm(want)
