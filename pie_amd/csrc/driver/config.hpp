@@ -62,6 +62,10 @@ struct RuntimeConfig {
     // a second copy of every decoder linear in the skinny GEMM's tile-major layout (doubles the
     // weight memory, ~25 % off the 5-32-row and MoE grouped GEMMs)
     bool tiled_weights = true;
+    // one synthetic full-size prefill chunk and a decode step at start-up, so that the first
+    // request does not pay one-time costs (measured: 58 ms cold against 47 ms for a 2048-token
+    // prefill of an 8B model); writes only KV pages nobody owns yet
+    bool warmup = true;
     std::string snapshot_dir;
 };
 
@@ -242,6 +246,7 @@ inline DriverConfig parse_config_text(const std::string& text) {
                 if (k == "verbose") r.verbose = to_bool(v, key);
                 else if (k == "use_graphs") r.use_graphs = to_bool(v, key);
                 else if (k == "tiled_weights") r.tiled_weights = to_bool(v, key);
+                else if (k == "warmup") r.warmup = to_bool(v, key);
                 else if (k == "snapshot_dir") r.snapshot_dir = v;
             }
         }

@@ -412,10 +412,29 @@ PieSamplerDesc greedy_sampler() {
 
 }  // namespace
 
+// Start-up warm-up ([runtime] warmup): the generation harness on a synthetic prompt of one full
+// prefill chunk plus two decode steps.  Best effort: a pool too small for it skips it.
+static void warm_up(PieHipDriver* d) {
+    if (!d->cfg.runtime.warmup) return;
+    const long long room = static_cast<long long>(d->exec->total_pages()) * d->exec->page_size() - 4;
+    const int n = static_cast<int>(std::min<long long>(d->cfg.batching.max_forward_tokens, room));
+    if (n <= 0) return;
+    std::vector<uint32_t> prompt(n);
+    for (int i = 0; i < n; ++i) prompt[i] = static_cast<uint32_t>(i % std::max(1, d->cfg.model.vocab));
+    uint32_t out[3];
+    double tm[4];
+    char err[256];
+    const int rc = pie_hip_driver_generate(d, prompt.data(), n, 3, 1, 0, out, tm, err, sizeof(err));
+    if (rc != 0 && d->cfg.runtime.verbose) std::fprintf(stderr, "[pie-driver-hip] warm-up skipped: %s\n", err);
+    d->last_error.clear();
+}
+
 extern "C" PieHipDriver* pie_hip_driver_create(const char* config_toml, char* err, size_t err_cap) {
     try {
         if (!config_toml) throw std::runtime_error("null config");
-        return new PieHipDriver(load_driver_config(config_toml));
+        PieHipDriver* d = new PieHipDriver(load_driver_config(config_toml));
+        warm_up(d);
+        return d;
     } catch (const std::exception& e) {
         set_err(err, err_cap, e.what());
         return nullptr;
@@ -680,6 +699,7 @@ extern "C" int pie_driver_hip_run_inproc(int argc, char** argv, int install_sign
         }
         g_stop.store(false, std::memory_order_release);
         PieHipDriver driver(load_driver_config(config_path));
+        warm_up(&driver);
         if (ready_cb) ready_cb(driver.caps.c_str(), ready_ctx);
         if (driver.cfg.runtime.verbose) std::fprintf(stderr, "[pie-driver-hip] serving on in-process channel\n");
         PieResponseFrameDesc resp;
