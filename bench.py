@@ -382,8 +382,18 @@ def pmc_workload():
         for i in range(12):
             ops.linear_fused(act, ws[i % 6], y=y)
         torch.cuda.synchronize()
+        if N == 2 * I:
+            # the same matrices in the tile-major layout under the skinny GEMM at 16 rows
+            tiled = [ops.repack_mfma_tiles(w) for w in ws]
+            act16 = torch.randn(16, K, device=dev).bfloat16()
+            y16 = torch.empty(16, N, device=dev, dtype=torch.bfloat16)
+            for i in range(12):
+                ops.gemm_skinny(act16, tiled[i % 6], y=y16)
+            torch.cuda.synchronize()
+            del tiled
         del ws
-    print(json.dumps({"pmc_workload": "4 x 256 MiB copy, 12 launches of each int4 GEMV shape at M=1"}))
+    print(json.dumps({"pmc_workload": "4 x 256 MiB copy, 12 launches of each int4 GEMV shape at M=1, "
+                                      "12 launches of the skinny GEMM at M=16 on the gate|up shape"}))
 
 
 def main():
