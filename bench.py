@@ -343,7 +343,8 @@ def cpu_baseline(drv, model, page_size, total_pages, n_prompt, gpu_tokens, budge
     return dict(value=steps / t_total, unit="tokens/s", cores=cores, kind="port",
                 sample=f"{steps} batch-1 decode steps of the same model at context {n_prompt}+, "
                        "oracle (C restatement of the reference forward pass, OpenMP over rows) "
-                       "fed the GPU's weights and prefilled KV pages",
+                       "fed the GPU's weights and prefilled KV pages; every compared step is also replayed "
+                       "through the driver boundary for its logits",
                 greedy_tokens_matched=matched, greedy_tokens_compared=steps,
                 mismatches_at_oracle_near_ties=near_ties,
                 mismatch_margins_rel_to_top_logit=margins,
