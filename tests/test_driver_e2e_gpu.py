@@ -529,3 +529,18 @@ def test_small_decode_batches_match_oracle(gpu, oracle, kw, replicate):
         om, _ = oracle_model_from_driver(d, dict(cfg, total_pages=96))
         _, near = teacher_forced_compare(oracle, drvmod, d, om, cfg, prompt, 6, replicate)
         assert near <= 3
+
+
+def test_start_up_warm_up_changes_no_result(gpu):
+    """[runtime] warmup runs a synthetic chunk over unowned pages at start-up: with it on or off
+    the same request gives the same tokens and the same logits, bit for bit."""
+    from pie_amd import driver as drvmod
+
+    rng = np.random.default_rng(98)
+    prompt = rng.integers(0, 2048, 23)
+    outs = []
+    for warm in (True, False):
+        with drvmod.Driver(toml_config(warmup=warm)) as d:
+            toks, _ = d.generate(prompt, 6, replicate=2)
+            outs.append((toks.copy(), d.export_tensor("debug.logits", np.uint16).copy()))
+    assert np.array_equal(outs[0][0], outs[1][0]) and np.array_equal(outs[0][1], outs[1][1])
