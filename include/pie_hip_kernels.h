@@ -423,6 +423,26 @@ int pie_hip_attn_rows_paged(const uint16_t* q, const uint16_t* k_pages, const ui
                             size_t workspace_bytes, void* stream);
 
 /*
+ * pie_hip_attn_rows_paged without a workspace argument and without any allocation, for callers
+ * that cannot allocate device memory: code running under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  It has no counterpart in the reference.  The split partials
+ * go to a device array built into the library, PIE_HIP_ATTN_STATIC_SCRATCH_BYTES per GPU, held
+ * until the process ends; a batch whose partials
+ * (pie_hip_attn_decode_workspace_bytes(num_rows, ...)) exceed it is refused with
+ * PIE_HIP_ERR_UNSUPPORTED and a message on stderr.  Same kernels and results as
+ * pie_hip_attn_rows_paged, bit for bit.  All calls on one GPU share that GPU's array: calls
+ * that overlap on one GPU (different streams, or threads) race; serialise them.  The first call
+ * on a device looks up the array's address (no allocation, but make it outside graph capture).
+ */
+#define PIE_HIP_ATTN_STATIC_SCRATCH_BYTES (16u << 20)
+int pie_hip_attn_rows_paged_static(const uint16_t* q, const uint16_t* k_pages,
+                                   const uint16_t* v_pages, uint16_t* o, float* lse,
+                                   const uint32_t* kv_page_indices, const uint32_t* row_page_begin,
+                                   const int32_t* row_kv_len, int num_rows, int num_q_heads,
+                                   int num_kv_heads, int head_dim, int page_size, float sm_scale,
+                                   int max_kv_len, void* stream);
+
+/*
  * KV-cache storage formats of the pool (the CUDA driver's kv_cache_dtype values,
  * driver/cuda/src/kv_cache_format.cpp:46-110).  One-byte formats keep the bf16 layout
  * [pages, page_size, hk, d] with one byte per element; the per-token-head formats add fp32 side

@@ -23,6 +23,9 @@
 //   * the next unit's K and V rows are requested before the current unit is
 //     reduced, so 2 x (K+V) = 16 KiB per wave is in flight;
 //   * a second, tiny kernel merges the splits (skipped when there is one split).
+#include <cstdio>
+#include <mutex>
+
 #include "common.hip.h"
 
 namespace pie_hip {
@@ -939,6 +942,70 @@ extern "C" int pie_hip_attn_rows_paged(const uint16_t* q, const uint16_t* k_page
                                   row_page_begin, row_kv_len, num_rows, num_q_heads, num_kv_heads,
                                   head_dim, page_size, sm_scale, max_kv_len, workspace,
                                   workspace_bytes, stream);
+}
+
+// ---------------------------------------------------------------------------------------------
+// pie_hip_attn_rows_paged for callers that cannot allocate: the split partials live in a
+// file-scope device array instead of a caller workspace.  Each GPU holds its own copy of the
+// array at its own address; the address is looked up once per device and kept.
+namespace pie_hip {
+namespace {
+constexpr size_t kStaticScratchBytes = PIE_HIP_ATTN_STATIC_SCRATCH_BYTES;
+constexpr int kStaticScratchMaxDevices = 64;
+}  // namespace
+}  // namespace pie_hip
+
+static __device__ __align__(256) unsigned char scratch[pie_hip::kStaticScratchBytes];
+
+namespace pie_hip {
+namespace {
+std::mutex g_scratch_mu;
+void* g_scratch_ptr[kStaticScratchMaxDevices] = {};
+
+// The device-side address of `scratch` on the current device (nullptr on failure).
+void* static_scratch_for_current_device() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kStaticScratchMaxDevices) return nullptr;
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        g_scratch_ptr[dev] = p;
+    }
+    return g_scratch_ptr[dev];
+}
+}  // namespace
+}  // namespace pie_hip
+
+extern "C" int pie_hip_attn_rows_paged_static(const uint16_t* q, const uint16_t* k_pages,
+                                              const uint16_t* v_pages, uint16_t* o, float* lse,
+                                              const uint32_t* kv_page_indices,
+                                              const uint32_t* row_page_begin,
+                                              const int32_t* row_kv_len, int num_rows,
+                                              int num_q_heads, int num_kv_heads, int head_dim,
+                                              int page_size, float sm_scale, int max_kv_len,
+                                              void* stream) {
+    if (!row_page_begin || !row_kv_len) return PIE_HIP_ERR_INVALID;
+    const size_t need = pie_hip_attn_decode_workspace_bytes(num_rows, num_q_heads, num_kv_heads,
+                                                            head_dim, max_kv_len);
+    if (need > pie_hip::kStaticScratchBytes) {
+        fprintf(stderr,
+                "pie_hip_attn_rows_paged_static: %d rows x %d heads over up to %d keys need %zu bytes of "
+                "split partials, the built-in scratch holds %zu\n",
+                num_rows, num_q_heads, max_kv_len, need, pie_hip::kStaticScratchBytes);
+        return PIE_HIP_ERR_UNSUPPORTED;
+    }
+    void* ws = pie_hip::static_scratch_for_current_device();
+    if (!ws) return PIE_HIP_ERR_LAUNCH;
+    // Every partial slot the merge reads is written by the split kernel of the same call, so
+    // nothing in the array has to start at zero.
+    return pie_hip::attn_dispatch(q, k_pages, v_pages, o, lse, kv_page_indices, nullptr, nullptr,
+                                  row_page_begin, row_kv_len, num_rows, num_q_heads, num_kv_heads,
+                                  head_dim, page_size, sm_scale, max_kv_len, ws,
+                                  pie_hip::kStaticScratchBytes, stream);
 }
 
 extern "C" int pie_hip_attn_rows_paged_kvq(int kv_format, const uint16_t* q, const void* k_pages,

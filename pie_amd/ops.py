@@ -717,6 +717,34 @@ def attention_rows_paged(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
     return o
 
 
+ATTN_STATIC_SCRATCH_BYTES = 16 << 20
+
+
+def attention_rows_paged_static(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
+                                kv_page_indices: torch.Tensor, row_page_begin: torch.Tensor,
+                                row_kv_len: torch.Tensor, max_kv_len: int, o: torch.Tensor,
+                                lse: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """`attention_rows_paged` through the entry point that allocates nothing: the caller brings
+    the output `o`, the split partials live in the library's built-in per-GPU scratch array
+    (ATTN_STATIC_SCRATCH_BYTES; larger batches raise).  No tensor is created here."""
+    _dev(q, torch.bfloat16, "q")
+    _dev(k_pages, torch.bfloat16, "k_pages")
+    _dev(o, torch.bfloat16, "o")
+    for name, t in (("kv_page_indices", kv_page_indices), ("row_page_begin", row_page_begin),
+                    ("row_kv_len", row_kv_len)):
+        _dev(t, torch.int32, name)
+    rows, hq, d = q.shape
+    _, ps, hk, _ = k_pages.shape
+    if o.shape != q.shape:
+        raise KernelError("o must have q's shape")
+    st = kernels().pie_hip_attn_rows_paged_static(
+        _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(o), _ptr(lse), _ptr(kv_page_indices),
+        _ptr(row_page_begin), _ptr(row_kv_len), rows, hq, hk, d, ps, C.c_float(-1.0), max_kv_len,
+        _stream())
+    _check(st, "pie_hip_attn_rows_paged_static")
+    return o
+
+
 def attn_prefill_tile_rows(hq: int, hk: int) -> int:
     """Most query rows one tile of `attention_prefill_tiles` may hold (0: unsupported head ratio)."""
     return int(kernels().pie_hip_attn_prefill_tile_rows(hq, hk))
