@@ -26,6 +26,11 @@
 extern "C" {
 #endif
 
+/* RoPE pairings of the rotation kernels and fused epilogues */
+#define PIE_HIP_ROPE_HALF 0
+#define PIE_HIP_ROPE_ADJACENT 1
+#define PIE_HIP_ROPE_HALF_PAIRED_ROWS 2
+
 #define PIE_HIP_OK 0
 #define PIE_HIP_ERR_INVALID 1     /* null pointer, non-positive size, bad enum   */
 #define PIE_HIP_ERR_UNSUPPORTED 2 /* shape the kernels do not cover              */
@@ -107,7 +112,12 @@ int pie_hip_linear_fused(int format, const uint16_t* act_bf16, const uint16_t* n
  * driver/cuda/src/kernels/rope.cu:14-33), q goes to q_out [M, hq*d], k and v to slot
  * kv_slots[m] of the paged pools (NHD addressing, driver/cuda/src/kernels/split_packed.cu:116-138).
  * Values are those of pie_hip_linear_fused followed by pie_hip_qkv_rope_kvwrite with
- * interleaved = 1 and no q/k norm (every intermediate rounded to bf16 at the same points).
+ * interleaved = pairing and no q/k norm (every intermediate rounded to bf16 at the same points).
+ * pairing = PIE_HIP_ROPE_ADJACENT: as described.  pairing = PIE_HIP_ROPE_HALF_PAIRED_ROWS: the
+ * half-split pairing of Llama / Qwen checkpoints (i, i + d/2; driver/cuda/src/kernels/rope.cu:10-21)
+ * over weights whose q / k rows were re-ordered at load so that rows (2i, 2i+1) of a head are
+ * that pair; the rotated values are written to positions i and i + d/2, so q_out and the pools
+ * hold what the unpermuted projection followed by half-split RoPE gives, bit for bit.
  * Replaces the qkv gemm + qkv_decode_qk_norm_rope_write_kv_kernel pair of
  * driver/cuda/src/model/llama_like.cpp:370-470 for llama-type decode.  head_dim a power of two,
  * M <= 4 per weight pass like the GEMV.
@@ -117,7 +127,7 @@ int pie_hip_qkv_rope_fused(int format, const uint16_t* act_bf16, const uint16_t*
                            int group_size, int M, int K, const float* rope_table,
                            const int64_t* kv_slots, uint16_t* q_out, uint16_t* k_pages,
                            uint16_t* v_pages, int num_q_heads, int num_kv_heads, int head_dim,
-                           void* stream);
+                           int pairing, void* stream);
 
 /*
  * Weight-only GEMM for a handful to a few dozen activation rows on the matrix cores:
@@ -205,14 +215,14 @@ int pie_hip_gemm_skinny_tiled(int format, const uint16_t* act_bf16, const void* 
 /* pie_hip_qkv_rope_fused for more rows than the GEMV takes (a decode batch): the q|k|v projection
  * over tile-major weights with interleaved RoPE and the KV-cache write in its epilogue.  act_bf16
  * is the normalised activation [M, K]; values are those of pie_hip_gemm_skinny_tiled followed by
- * pie_hip_qkv_rope_kvwrite (interleaved = 1, no q/k norm), every intermediate rounded to bf16 at
+ * pie_hip_qkv_rope_kvwrite (interleaved = pairing, 1 or 2; no q/k norm), every intermediate rounded to bf16 at
  * the same points.  Same reference role: the qkv gemm + qkv_decode_qk_norm_rope_write_kv_kernel
  * pair of driver/cuda/src/model/llama_like.cpp:370-470.  head_dim a power of two, K % 256 == 0. */
 int pie_hip_qkv_rope_skinny_tiled(int format, const uint16_t* act_bf16, const void* weight,
                                   const void* scale, int scale_is_bf16, int group_size, int M, int K,
                                   const float* rope_table, const int64_t* kv_slots, uint16_t* q_out,
                                   uint16_t* k_pages, uint16_t* v_pages, int num_q_heads,
-                                  int num_kv_heads, int head_dim, void* stream);
+                                  int num_kv_heads, int head_dim, int pairing, void* stream);
 int pie_hip_moe_grouped_gemm_tiled(int format, const uint16_t* act_bf16, const int32_t* route_act_rows,
                              const int32_t* expert_offsets, int num_experts,
                              int max_rows_per_expert, const void* weights,
@@ -536,7 +546,11 @@ int pie_hip_rope_table(const int32_t* positions, const float* inv_freq, float* t
  * weights or neither) and RoPE to q and k, write q to q_out[N, hq, d], and write k (rotated)
  * and v (copied) into the KV pool [pages, page_size, hk, d] at physical slot
  * kv_slots[n] = page*page_size + offset (negative = token has no slot).  One bf16 rounding at
- * the store.  interleaved: 0 pairs (i, i+d/2), 1 pairs (2i, 2i+1).
+ * the store.  interleaved: PIE_HIP_ROPE_HALF (0) pairs (i, i+d/2), PIE_HIP_ROPE_ADJACENT (1) pairs
+ * (2i, 2i+1), PIE_HIP_ROPE_HALF_PAIRED_ROWS (2): the q / k rows of the projection were re-ordered
+ * at load so that elements (2i, 2i+1) of packed_qkv hold the half-split pair (i, i+d/2); they are
+ * rotated as that pair and written to positions i and i+d/2 (V rows are as stored) — the output
+ * of mode 0 over the original row order, bit for bit.
  * Reference: launch_qkv_decode_qk_norm_rope_write_kv_bf16,
  * driver/cuda/src/kernels/split_packed.hpp:34-57, split_packed.cu:62-178; slot arithmetic of
  * driver/portable/src/plan.hpp:36-45 is done by the caller.

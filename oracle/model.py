@@ -177,38 +177,52 @@ class OracleModel:
         return self._router_gap
 
     def generate(self, prompt, max_new: int, replicate: int = 1, want_logits=False):
-        """Greedy generation over contiguous page ranges, one prefill per context and one
-        multi-request decode forward per step.  Returns tokens [replicate, max_new] (and the
-        per-step logits of context 0 when asked); `last_router_gaps` holds router_gap() of the
-        prefill and of each decode step."""
+        """Greedy generation of `replicate` copies of one prompt (see generate_ragged).  Returns
+        tokens [replicate, max_new] (and the per-step logits of context 0 when asked)."""
+        out = self.generate_ragged([prompt] * replicate, max_new, want_logits=want_logits)
+        if want_logits:
+            return out[0], [step[0] for step in out[1]]
+        return out
+
+    def generate_ragged(self, prompts, max_new: int, want_logits=False):
+        """Greedy generation of several contexts with their own prompts (any lengths) over
+        contiguous page ranges: one prefill per context, then one multi-request decode forward
+        per step in which every request sits at its own position with its own page count —
+        the loop of the reference's offline harness
+        (driver/portable/src/executor/executor.cpp:1439-1597) over a ragged batch.  Returns tokens
+        [R, max_new] and, when asked, trace[step][r] = logits (bf16 bits) of context r;
+        `prefill_router_gaps[r]` holds router_gap() of context r's prefill, `last_router_gaps` the
+        smallest of those followed by the gap of each decode step."""
         ps = self.cfg["page_size"]
-        n_prompt = len(prompt)
-        ppc = (n_prompt + max_new + ps - 1) // ps
-        toks = np.zeros((replicate, max_new), np.uint32)
-        logit_trace = []
-        for c in range(replicate):
-            npg = (n_prompt + ps - 1) // ps
-            t, lg, _ = self.forward(prompt, np.arange(n_prompt), np.arange(npg) + c * ppc, [0, npg],
-                                    [n_prompt - (npg - 1) * ps], [0, n_prompt],
-                                    want_logits=want_logits and c == 0)
+        R = len(prompts)
+        lens = [len(p) for p in prompts]
+        ppc = (max(lens) + max_new + ps - 1) // ps
+        toks = np.zeros((R, max_new), np.uint32)
+        trace = [[None] * R for _ in range(max_new)]
+        self.prefill_router_gaps = []
+        for c, prompt in enumerate(prompts):
+            n = lens[c]
+            npg = (n + ps - 1) // ps
+            t, lg, _ = self.forward(prompt, np.arange(n), np.arange(npg) + c * ppc, [0, npg],
+                                    [n - (npg - 1) * ps], [0, n], want_logits=want_logits)
             toks[c, 0] = t[0]
-            if c == 0:
-                self.last_router_gaps = [self.router_gap()]
-            if want_logits and c == 0:
-                logit_trace.append(lg[0])
+            self.prefill_router_gaps.append(self.router_gap())
+            if want_logits:
+                trace[0][c] = lg[0]
+        self.last_router_gaps = [min(self.prefill_router_gaps)]
         for s in range(1, max_new):
-            pos = n_prompt + s - 1
-            npg = (pos + 1 + ps - 1) // ps
-            pages = np.concatenate([np.arange(npg) + c * ppc for c in range(replicate)])
-            t, lg, _ = self.forward(toks[:, s - 1], [pos] * replicate, pages,
-                                    np.arange(replicate + 1) * npg,
-                                    [pos + 1 - (npg - 1) * ps] * replicate,
-                                    np.arange(replicate + 1), want_logits=want_logits)
+            pos = [n + s - 1 for n in lens]
+            npg = [(p + 1 + ps - 1) // ps for p in pos]
+            pages = np.concatenate([np.arange(g) + c * ppc for c, g in enumerate(npg)])
+            t, lg, _ = self.forward(toks[:, s - 1], pos, pages, np.concatenate([[0], np.cumsum(npg)]),
+                                    [p + 1 - (g - 1) * ps for p, g in zip(pos, npg)],
+                                    np.arange(R + 1), want_logits=want_logits)
             toks[:, s] = t
             self.last_router_gaps.append(self.router_gap())
             if want_logits:
-                logit_trace.append(lg[0])
-        return (toks, logit_trace) if want_logits else toks
+                for c in range(R):
+                    trace[s][c] = lg[c]
+        return (toks, trace) if want_logits else toks
 
 
 _DATA_DTYPE = {"int4b8": np.uint32, "int8": np.int8, "fp8": np.uint8, "bf16": np.uint16}
@@ -221,6 +235,21 @@ def model_from_driver(drv, cfg: dict):
     page_size, total_pages.  Returns (model, tensors)."""
     L, quant = cfg["layers"], cfg["quant"]
     t = {}
+    # the driver may keep the q / k rows of wqkv re-ordered (rows (2i, 2i+1) of a head = the
+    # half-split pair (i, i + d/2)); the oracle uses the checkpoint's row order
+    paired = drv.export_tensor("info.qk_rows_paired", np.int32)
+    paired = bool(paired is not None and paired[0])
+    interleaved = drv.export_tensor("info.rope_interleaved", np.int32)
+    interleaved = int(interleaved[0]) if interleaved is not None else 0
+    d_, hq_, hk_ = cfg["head_dim"], cfg["q_heads"], cfg["kv_heads"]
+    inv_pair = np.arange((hq_ + 2 * hk_) * d_)
+    if paired:
+        # stored row h*d + 2i = original row h*d + i, stored row h*d + 2i + 1 = original h*d + d/2 + i
+        head = np.empty(d_, np.int64)
+        head[:d_ // 2] = 2 * np.arange(d_ // 2)
+        head[d_ // 2:] = 2 * np.arange(d_ // 2) + 1
+        for h in range(hq_ + hk_):
+            inv_pair[h * d_:(h + 1) * d_] = h * d_ + head
     for name in ("embed", "lm_head", "final_norm"):
         t[name] = drv.export_tensor(name, np.uint16)
     t["inv_freq"] = drv.export_tensor("inv_freq", np.float32)
@@ -249,12 +278,17 @@ def model_from_driver(drv, cfg: dict):
                 data = canon(data)
                 if sc is not None:
                     sc = canon(sc)
+            if w == "wqkv" and paired:
+                rows = len(inv_pair)
+                data = data.reshape(rows, -1)[inv_pair].reshape(-1)
+                if sc is not None:
+                    sc = sc.reshape(rows, -1)[inv_pair].reshape(-1)
             t[p + w + ".data"] = data
             if sc is not None:
                 t[p + w + ".scale"] = sc
     ocfg = dict(hidden=cfg["hidden"], layers=L, q_heads=cfg["q_heads"], kv_heads=cfg["kv_heads"],
                 head_dim=cfg["head_dim"], intermediate=cfg["intermediate"], vocab=cfg["vocab"],
-                rms_eps=cfg.get("rms_eps", 1e-5), rope_interleaved=1 if cfg["arch"] == "llama3" else 0,
+                rms_eps=cfg.get("rms_eps", 1e-5), rope_interleaved=interleaved,
                 qk_norm=cfg["arch"] != "llama3", quant=quant, group_size=cfg.get("group_size", 128),
                 page_size=cfg["page_size"], total_pages=cfg["total_pages"])
     if cfg["arch"] == "qwen3_moe":

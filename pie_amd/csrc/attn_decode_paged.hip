@@ -1130,12 +1130,16 @@ __global__ __launch_bounds__(64) void qkv_rope_kvwrite_quant_kernel(
         const int i = lane + it * kWave;
         va[it] = vb[it] = 0.f;
         if (i < half) {
-            const int ia = interleaved ? 2 * i : i, ib = interleaved ? 2 * i + 1 : i + half;
+            // (interleaved = 2: q / k rows re-ordered at load, elements (2i, 2i+1) hold the
+            // half-split pair (i, i+d/2) and go back to those positions; V rows are as stored)
+            const int pin = (interleaved == 2 && !(is_q || is_k)) ? 0 : interleaved;
+            const int ia = pin ? 2 * i : i, ib = pin ? 2 * i + 1 : i + half;
+            const int oa = pin == 1 ? 2 * i : i, ob = pin == 1 ? 2 * i + 1 : i + half;
             float a = bf16_bits_to_f32(src[ia]), b = bf16_bits_to_f32(src[ib]);
             if (is_q || is_k) {
                 if (nw) {
-                    a = a * inv_rms * bf16_bits_to_f32(nw[ia]);
-                    b = b * inv_rms * bf16_bits_to_f32(nw[ib]);
+                    a = a * inv_rms * bf16_bits_to_f32(nw[oa]);
+                    b = b * inv_rms * bf16_bits_to_f32(nw[ob]);
                 }
                 const float c = tab[i], sn = tab[i + half];
                 const float ra = a * c - b * sn, rb = b * c + a * sn;
@@ -1146,8 +1150,8 @@ __global__ __launch_bounds__(64) void qkv_rope_kvwrite_quant_kernel(
             vb[it] = b;
             if (is_q) {
                 uint16_t* dst = q_out + (static_cast<size_t>(n) * hq + head) * d;
-                dst[ia] = f32_to_bf16_bits(a);
-                dst[ib] = f32_to_bf16_bits(b);
+                dst[oa] = f32_to_bf16_bits(a);
+                dst[ob] = f32_to_bf16_bits(b);
             }
         }
     }
@@ -1181,9 +1185,9 @@ __global__ __launch_bounds__(64) void qkv_rope_kvwrite_quant_kernel(
     for (int it = 0; it < ITER; ++it) {
         const int i = lane + it * kWave;
         if (i < half) {
-            const int ia = interleaved ? 2 * i : i, ib = interleaved ? 2 * i + 1 : i + half;
-            dst[ia] = code(va[it]);
-            dst[ib] = code(vb[it]);
+            const bool adjacent = interleaved == 1;
+            dst[adjacent ? 2 * i : i] = code(va[it]);
+            dst[adjacent ? 2 * i + 1 : i + half] = code(vb[it]);
         }
     }
 }

@@ -26,7 +26,7 @@ struct ModelConfig {
     // llama3 wavelength-band RoPE scaling; factor <= 0 disables it
     float rope_factor = 0.f, rope_low_freq_factor = 1.f, rope_high_freq_factor = 4.f;
     int rope_original_max_pos = 8192;
-    int rope_interleaved = -1;  // -1: by arch (llama3 -> adjacent pairs, others -> half split)
+    int rope_interleaved = -1;  // -1: half split, the pairing of Llama / Mistral / Qwen checkpoints
     bool tie_embeddings = false;
     // storage format of the decoder linears: "int4b8" | "int8" | "fp8" | "bf16"
     std::string quant = "int4b8";
@@ -185,7 +185,9 @@ inline void finalize_config(DriverConfig& c) {
         throw std::runtime_error("config: unsupported quant '" + m.quant + "'");
     if (m.scale_dtype != "bf16" && m.scale_dtype != "f32")
         throw std::runtime_error("config: scale_dtype must be bf16 or f32");
-    if (m.rope_interleaved < 0) m.rope_interleaved = (m.arch == "llama3") ? 1 : 0;
+    // (i, i + d/2) pairs for every architecture here, as the reference rotates them
+    // (driver/cuda/src/kernels/rope.cu:10-21 keeps adjacent pairs for GLM only)
+    if (m.rope_interleaved < 0) m.rope_interleaved = 0;
     const auto& b = c.batching;
     if (b.kv_page_size <= 0 || b.kv_page_size % 16 != 0)
         throw std::runtime_error("config: kv_page_size must be a positive multiple of 16");

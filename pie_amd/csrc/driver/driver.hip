@@ -216,6 +216,12 @@ static DriverConfig load_driver_config(const std::string& src) {
         finalize_config(c);
         if (c.runtime.snapshot_dir.empty()) c.runtime.snapshot_dir = c.model.checkpoint_dir;
     }
+    // The routing kernel always divides the top-k probabilities by their sum
+    // (driver/portable/src/graph_common.cpp:279-283 does so only under norm_topk): a model that
+    // asks for raw probabilities would get other expert weights without a word.
+    if (c.model.arch == "qwen3_moe" && !c.model.norm_topk)
+        throw std::runtime_error("config: norm_topk = false (norm_topk_prob) is not implemented: "
+                                 "router weights are always renormalised over the top-k experts");
     return c;
 }
 
@@ -475,6 +481,12 @@ extern "C" size_t pie_hip_driver_export_tensor(PieHipDriver* d, const char* name
         return bytes;
     }
     const std::string nm(name);
+    if (nm == "info.qk_rows_paired" || nm == "info.rope_interleaved") {   // one int32
+        const int32_t v = nm == "info.qk_rows_paired" ? (d->model.qk_rows_paired() ? 1 : 0)
+                                                      : d->cfg.model.rope_interleaved;
+        if (dst && cap >= sizeof(v)) std::memcpy(dst, &v, sizeof(v));
+        return sizeof(v);
+    }
     if (nm.rfind("debug.", 0) == 0) {
         const uint16_t* buf = d->exec->debug_buffer(nm.substr(6));
         if (!buf) return 0;

@@ -203,6 +203,7 @@ Executor::Executor(const DriverConfig& cfg, Model& model) : cfg_(cfg), model_(mo
     xs_ = dmalloc<uint16_t>(srows * H);
     logits_ = dmalloc<uint16_t>(srows * m.vocab);
     out_tokens_ = dmalloc<uint32_t>(T);
+    out_cap_ = T;
     // Bound of the split-K partial buffers over every (rows, context) the planner can pick:
     // rows * splits <= 3072/hk + rows.
     attn_ws_bytes_ = (3072 / static_cast<size_t>(hk) + 1 + T) * hq * (d + 2) * sizeof(float);
@@ -362,6 +363,11 @@ void Executor::body(int N, int S, int max_kv_len) {
 
     PIE_KERNEL(pie_hip_embed(tokens, model_.embed, x_, N, H, m.vocab, s));
     PIE_KERNEL(pie_hip_rope_table(positions, model_.inv_freq, rope_tab_, N, d, s));
+    // RoPE pairing as the rotation kernels take it: adjacent pairs, half-split pairs, or
+    // half-split pairs over projection rows re-ordered at load (then the fused epilogues apply)
+    const int pairing = m.rope_interleaved ? PIE_HIP_ROPE_ADJACENT
+                        : model_.qk_rows_paired() ? PIE_HIP_ROPE_HALF_PAIRED_ROWS : PIE_HIP_ROPE_HALF;
+    const bool fused_rope = pairing != PIE_HIP_ROPE_HALF && (d & (d - 1)) == 0;
     for (int l = 0; l < m.layers; ++l) {
         const LayerWeights& w = model_.layers[l];
         const bool kvq = kv_format_ != PIE_HIP_KV_BF16;
@@ -374,40 +380,39 @@ void Executor::body(int N, int S, int max_kv_len) {
             // rotation and quantising write in one launch; head dims past 256 take the two kernels
             const int st = pie_hip_qkv_rope_kvwrite_quant(kv_format_, qkv_, q_, k_pool_[l], v_pool_[l], ksc, vsc,
                                                           w.q_norm, w.k_norm, rope_tab_, slots, N, hq, hk, d,
-                                                          m.rope_interleaved, m.rms_eps, s);
+                                                          pairing, m.rms_eps, s);
             if (st == PIE_HIP_ERR_UNSUPPORTED) {
                 PIE_KERNEL(pie_hip_qkv_rope_kvwrite(qkv_, q_, k_rows_, v_rows_, w.q_norm, w.k_norm, rope_tab_,
-                                                    iota_slots_, N, hq, hk, d, m.rope_interleaved, m.rms_eps, s));
+                                                    iota_slots_, N, hq, hk, d, pairing, m.rms_eps, s));
                 PIE_KERNEL(pie_hip_kv_write_quant(kv_format_, k_rows_, v_rows_, slots, k_pool_[l], v_pool_[l],
                                                   ksc, vsc, N, hk, d, s));
             } else {
                 PIE_KERNEL(st);
             }
-        } else if (N <= 4 && m.rope_interleaved && !w.q_norm && (d & (d - 1)) == 0) {
+        } else if (N <= 4 && fused_rope && !w.q_norm) {
             // decode rows of llama-type layers: rotation and KV write ride in the projection
             PIE_KERNEL(pie_hip_qkv_rope_fused(fmt_code(w.wqkv.kind), x_, w.attn_norm, m.rms_eps,
                                               w.wqkv.data, w.wqkv.scale, w.wqkv.scale_bf16 ? 1 : 0,
                                               w.wqkv.group, N, H, rope_tab_, slots, q_, k_pool_[l],
-                                              v_pool_[l], hq, hk, d, s));
+                                              v_pool_[l], hq, hk, d, pairing, s));
         } else {
             // a decode batch of llama-type layers on the skinny GEMM: rotation and KV write ride
             // in its epilogue too (one launch less per layer)
             bool done = false;
-            if (m.rope_interleaved && !w.q_norm && (d & (d - 1)) == 0 && w.wqkv.data_tiled &&
+            if (fused_rope && !w.q_norm && w.wqkv.data_tiled &&
                 pick_gemm(w.wqkv, N, gemm_ws_bytes_) == GemmPath::Skinny) {
                 PIE_KERNEL(pie_hip_rmsnorm(x_, w.attn_norm, xn_, N, H, m.rms_eps, s));
                 const int st = pie_hip_qkv_rope_skinny_tiled(
                     fmt_code(w.wqkv.kind), xn_, w.wqkv.data_tiled,
                     w.wqkv.scale_tiled ? w.wqkv.scale_tiled : w.wqkv.scale, w.wqkv.scale_bf16 ? 1 : 0,
-                    w.wqkv.group, N, H, rope_tab_, slots, q_, k_pool_[l], v_pool_[l], hq, hk, d, s);
+                    w.wqkv.group, N, H, rope_tab_, slots, q_, k_pool_[l], v_pool_[l], hq, hk, d, pairing, s);
                 if (st == PIE_HIP_OK) done = true;
                 else if (st != PIE_HIP_ERR_UNSUPPORTED) PIE_KERNEL(st);
             }
             if (!done) {
                 linear_fused(w.wqkv, x_, w.attn_norm, m.rms_eps, qkv_, N, 0, 0, xn_, gemm_ws_, gemm_ws_bytes_, s);
                 PIE_KERNEL(pie_hip_qkv_rope_kvwrite(qkv_, q_, k_pool_[l], v_pool_[l], w.q_norm, w.k_norm,
-                                                    rope_tab_, slots, N, hq, hk, d, m.rope_interleaved,
-                                                    m.rms_eps, s));
+                                                    rope_tab_, slots, N, hq, hk, d, pairing, m.rms_eps, s));
             }
         }
         if (kvq && n_tiles_ > 0 && !masked_) {
@@ -726,6 +731,22 @@ void Executor::collect_samplers(const BatchPlan& plan, SampleOutputs& out) {
     out.out_indptr.assign(ip, ip + S + 1);
 }
 
+// Captured graphs hold the old buffer's address: they are dropped with it.
+void Executor::grow_outputs(size_t slots) {
+    PIE_HIP_CHECK(hipStreamSynchronize(stream_));
+    for (auto& kv : graphs_) (void)hipGraphExecDestroy(kv.second);
+    graphs_.clear();
+    const size_t cap = std::max(slots, 2 * out_cap_);
+    (void)hipFree(out_tokens_);
+    out_tokens_ = nullptr;
+    (void)hipHostFree(out_host_);
+    out_host_ = nullptr;
+    out_cap_ = 0;
+    out_tokens_ = dmalloc<uint32_t>(cap);
+    PIE_HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&out_host_), cap * 4, hipHostMallocDefault));
+    out_cap_ = cap;
+}
+
 void Executor::forward(const BatchPlan& plan, std::vector<uint32_t>& tokens_out,
                        ForwardTimings* t, SampleOutputs* samples) {
     const int N = plan.N, S = static_cast<int>(plan.sample_rows.size());
@@ -733,6 +754,9 @@ void Executor::forward(const BatchPlan& plan, std::vector<uint32_t>& tokens_out,
     if (N > max_tokens_) throw std::runtime_error("executor: batch exceeds max_forward_tokens");
     if (static_cast<int>(plan.page_indices.size()) > max_page_refs_)
         throw std::runtime_error("executor: batch exceeds the page reference capacity");
+    // A request may put several samplers on one row, so the sampling slots can outnumber the
+    // rows: the token buffers follow the slot count.
+    if (static_cast<size_t>(S) > out_cap_) grow_outputs(static_cast<size_t>(S));
 
     auto t0 = clk::now();
     const Inputs in = input_layout(N, S);

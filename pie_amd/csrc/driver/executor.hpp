@@ -96,6 +96,7 @@ class Executor {
 
   private:
     void body(int N, int S, int max_kv_len);
+    void grow_outputs(size_t slots);
     void prepare_masks(const BatchPlan& plan);
     void prepare_tiles(const BatchPlan& plan);
     void prepare_samplers(const BatchPlan& plan);
@@ -130,6 +131,7 @@ class Executor {
     float* moe_w_ = nullptr;
     float* rope_tab_ = nullptr;
     uint32_t* out_tokens_ = nullptr;
+    size_t out_cap_ = 0;   // sampling slots out_tokens_ / out_host_ hold
     void* attn_ws_ = nullptr;
     size_t attn_ws_bytes_ = 0;
     void* gemm_ws_ = nullptr;      // split-K partial sums of the tiled GEMM

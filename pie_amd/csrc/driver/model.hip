@@ -200,22 +200,40 @@ void Model::make_linear(Linear& lin, int N, int K, const std::string& name, std:
 // kernel pairs up.  A pure row permutation of the canonical [N, K] layout: data and scales move
 // together, no value changes.
 void Model::interleave_gate_up(Linear& lin, int blocks, hipStream_t stream) {
-    const size_t half = static_cast<size_t>(lin.N) / blocks / 2;
+    interleave_row_blocks(lin, static_cast<size_t>(lin.N) / blocks / 2, static_cast<size_t>(lin.N), stream);
+}
+
+// Inside every block of 2*half rows among the first `rows` rows: row 2i <- row i, row 2i+1 <-
+// row half + i; data and scales together, later rows untouched.
+void Model::interleave_row_blocks(Linear& lin, size_t half, size_t rows, hipStream_t stream) {
     auto permute = [&](void* buf, size_t bytes) {
-        if (!buf || bytes == 0) return;
+        if (!buf || bytes == 0 || rows == 0) return;
         const size_t row_bytes = bytes / lin.N;
+        const size_t part = rows * row_bytes;
         void* tmp = nullptr;
-        PIE_HIP_CHECK(hipMalloc(&tmp, bytes));
+        PIE_HIP_CHECK(hipMalloc(&tmp, part));
         hipLaunchKernelGGL(interleave_rows_kernel, dim3(2048), dim3(256), 0, stream,
                            static_cast<const unsigned char*>(buf), static_cast<unsigned char*>(tmp),
-                           half, row_bytes, static_cast<size_t>(lin.N));
+                           half, row_bytes, rows);
         PIE_HIP_CHECK(hipGetLastError());
-        PIE_HIP_CHECK(hipMemcpyAsync(buf, tmp, bytes, hipMemcpyDeviceToDevice, stream));
+        PIE_HIP_CHECK(hipMemcpyAsync(buf, tmp, part, hipMemcpyDeviceToDevice, stream));
         PIE_HIP_CHECK(hipStreamSynchronize(stream));
         (void)hipFree(tmp);
     };
     permute(lin.data, lin.data_bytes());
     permute(lin.scale, lin.scale_bytes());
+}
+
+// Half-split RoPE (pairs (i, i + d/2), driver/cuda/src/kernels/rope.cu:10-21) without a per-head
+// q/k norm: the q and k rows of the fused projection are re-ordered so that a pair's two outputs
+// are neighbours, which lets the projection kernels rotate them in their epilogue; the stores
+// put them back at i and i + d/2, so q and the KV pool hold what the original row order gives.
+void Model::pair_qk_rows(hipStream_t stream) {
+    const int d = cfg_.head_dim;
+    if (cfg_.rope_interleaved || has_qk_norm() || d < 2 || (d & (d - 1)) != 0) return;
+    const size_t rows = static_cast<size_t>(cfg_.q_heads + cfg_.kv_heads) * d;
+    for (LayerWeights& l : layers) interleave_row_blocks(l.wqkv, static_cast<size_t>(d) / 2, rows, stream);
+    qk_rows_paired_ = true;
 }
 
 void Model::init_synthetic(const ModelConfig& cfg, hipStream_t stream) {
@@ -297,6 +315,7 @@ void Model::init_synthetic(const ModelConfig& cfg, hipStream_t stream) {
     PIE_HIP_CHECK(hipStreamSynchronize(stream));
     (void)hipFree(tmp_bf16_);
     tmp_bf16_ = nullptr;
+    pair_qk_rows(stream);
 }
 
 namespace {
@@ -428,6 +447,9 @@ void Model::load_snapshot(const ModelConfig& cfg, hipStream_t stream) {
                 if (w.dtype != "I32" && w.dtype != "U32") throw std::runtime_error("snapshot: weight_packed must be I32");
                 expect_shape(w, p.prefix + ".weight_packed", p.rows, K / 8);
                 expect_shape(sc, p.prefix + ".weight_scale", p.rows, K / lin.group);
+                if (w.bytes != static_cast<size_t>(p.rows) * (K / 2) ||
+                    (row + p.rows) * (static_cast<size_t>(K) / 2) > lin.data_bytes())
+                    throw std::runtime_error("snapshot: '" + p.prefix + ".weight_packed' does not fit its rows");
                 PIE_HIP_CHECK(hipMemcpyAsync(static_cast<uint8_t*>(lin.data) + row * (K / 2), w.data, w.bytes,
                                              hipMemcpyHostToDevice, stream));
                 const uint16_t* sb = as_bf16(sc, staging);
@@ -489,6 +511,7 @@ void Model::load_snapshot(const ModelConfig& cfg, hipStream_t stream) {
     PIE_HIP_CHECK(hipStreamSynchronize(stream));
     (void)hipFree(tmp_bf16_);
     tmp_bf16_ = nullptr;
+    pair_qk_rows(stream);
 }
 
 }  // namespace pie_hip_driver

@@ -88,6 +88,10 @@ class Model {
     const ModelConfig& cfg() const { return cfg_; }
     bool is_moe() const { return cfg_.arch == "qwen3_moe"; }
     bool has_qk_norm() const { return cfg_.arch != "llama3"; }
+    // True when the q and k rows of every layer's wqkv were re-ordered at load so that rows
+    // (2i, 2i+1) of a head hold the half-split RoPE pair (i, i + d/2): the fused projection
+    // epilogues then rotate neighbouring outputs and store them at i and i + d/2.
+    bool qk_rows_paired() const { return qk_rows_paired_; }
     Quant quant() const { return quant_; }
 
     uint16_t* embed = nullptr;
@@ -107,6 +111,9 @@ class Model {
     void prepare_linear(Linear& lin, int N, int K, const std::string& name);
     void quantise_scratch(Linear& lin, const std::string& name, hipStream_t stream);
     void interleave_gate_up(Linear& lin, int blocks, hipStream_t stream);
+    void interleave_row_blocks(Linear& lin, size_t half, size_t rows, hipStream_t stream);
+    void pair_qk_rows(hipStream_t stream);
+    bool qk_rows_paired_ = false;
     ModelConfig cfg_;
     Quant quant_ = Quant::Bf16;
     std::vector<void*> allocs_;

@@ -175,6 +175,15 @@ inline Json parse_json_file(const std::string& path) {
 }
 
 // ---- safetensors --------------------------------------------------------------------------
+// Bytes per element of a safetensors dtype name (0: not a dtype of that format).
+inline size_t st_dtype_size(const std::string& dt) {
+    if (dt == "F64" || dt == "I64" || dt == "U64") return 8;
+    if (dt == "F32" || dt == "I32" || dt == "U32") return 4;
+    if (dt == "BF16" || dt == "F16" || dt == "I16" || dt == "U16") return 2;
+    if (dt == "I8" || dt == "U8" || dt == "BOOL" || dt == "F8_E4M3" || dt == "F8_E5M2") return 1;
+    return 0;
+}
+
 struct StTensor {
     std::string dtype;            // "BF16", "F16", "F32", "I32", "U8", "I8", "F8_E4M3", ...
     std::vector<int64_t> shape;
@@ -250,11 +259,35 @@ class Snapshot {
             const Json* off = kv.second.get("data_offsets");
             if (!dt || !sh || !off || off->arr.size() != 2)
                 throw std::runtime_error("snapshot: malformed entry '" + kv.first + "'");
+            // Nothing in the header is trusted: kinds, dtype names, dimensions (whole, >= 0, no
+            // overflow of the element count), offsets inside the file, and a byte count that is
+            // exactly elements * element size — later copies size themselves from these.
+            if (dt->kind != Json::String || sh->kind != Json::Array || off->kind != Json::Array ||
+                off->arr[0].kind != Json::Number || off->arr[1].kind != Json::Number)
+                throw std::runtime_error("snapshot: malformed entry '" + kv.first + "'");
             StTensor t;
             t.dtype = dt->str;
-            for (const Json& s : sh->arr) t.shape.push_back(static_cast<int64_t>(s.num));
+            const size_t esize = st_dtype_size(t.dtype);
+            if (esize == 0) throw std::runtime_error("snapshot: unknown dtype '" + t.dtype + "' in '" + kv.first + "'");
+            uint64_t elems = 1;
+            for (const Json& s : sh->arr) {
+                if (s.kind != Json::Number || !(s.num >= 0.0) || s.num > 9.0e15 ||
+                    s.num != static_cast<double>(static_cast<int64_t>(s.num)))
+                    throw std::runtime_error("snapshot: bad dimension in '" + kv.first + "'");
+                const uint64_t dim = static_cast<uint64_t>(s.num);
+                if (dim != 0 && elems > (uint64_t(1) << 62) / dim)
+                    throw std::runtime_error("snapshot: element count of '" + kv.first + "' overflows");
+                elems *= dim;
+                t.shape.push_back(static_cast<int64_t>(dim));
+            }
+            auto whole = [](double v) { return v >= 0.0 && v <= 9.0e15 && v == static_cast<double>(static_cast<uint64_t>(v)); };
+            if (!whole(off->arr[0].num) || !whole(off->arr[1].num))
+                throw std::runtime_error("snapshot: offsets of '" + kv.first + "' out of range");
             const uint64_t b = static_cast<uint64_t>(off->arr[0].num), e = static_cast<uint64_t>(off->arr[1].num);
             if (b > e || e > data_bytes) throw std::runtime_error("snapshot: offsets of '" + kv.first + "' out of range");
+            if (e - b != elems * esize)
+                throw std::runtime_error("snapshot: '" + kv.first + "' holds " + std::to_string(e - b) +
+                                         " bytes, its shape and dtype need " + std::to_string(elems * esize));
             t.data = data0 + b;
             t.bytes = e - b;
             tensors_[kv.first] = std::move(t);

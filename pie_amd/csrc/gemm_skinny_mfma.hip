@@ -136,6 +136,7 @@ struct SkinnyArgs {
     uint16_t* k_pages;
     uint16_t* v_pages;
     int hq, hk, d;
+    int half_out;   // q / k rows re-ordered at load: pair (2i, 2i+1) goes to positions (i, i + d/2)
 };
 
 constexpr int gcd_c(int a, int b) { return b == 0 ? a : gcd_c(b, a % b); }
@@ -620,10 +621,16 @@ __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 ? 4 : 2) void skinny_wave_
                         const float* tab = a.rope_table + static_cast<size_t>(m) * a.d + (dd >> 1);
                         const float c = tab[0], sn = tab[a.d >> 1];
                         const uint32_t out = pack_bf16x2(gb * c - ub * sn, ub * c + gb * sn);
-                        if (head < a.hq)
-                            *reinterpret_cast<uint32_t*>(a.y + (static_cast<size_t>(m) * a.hq + head) * a.d + dd) = out;
-                        else if (slot >= 0)
-                            *reinterpret_cast<uint32_t*>(a.k_pages + (static_cast<size_t>(slot) * a.hk + (head - a.hq)) * a.d + dd) = out;
+                        uint16_t* dst = head < a.hq ? a.y + (static_cast<size_t>(m) * a.hq + head) * a.d
+                                                    : a.k_pages + (static_cast<size_t>(slot) * a.hk + (head - a.hq)) * a.d;
+                        if (head < a.hq || slot >= 0) {
+                            if (a.half_out) {
+                                dst[dd >> 1] = static_cast<uint16_t>(out & 0xFFFFu);
+                                dst[(dd >> 1) + (a.d >> 1)] = static_cast<uint16_t>(out >> 16);
+                            } else {
+                                *reinterpret_cast<uint32_t*>(dst + dd) = out;
+                            }
+                        }
                     } else if (slot >= 0) {
                         *reinterpret_cast<uint32_t*>(a.v_pages + (static_cast<size_t>(slot) * a.hk + (head - a.hq - a.hk)) * a.d + dd) =
                             pack_bf16x2(gb, ub);
@@ -882,16 +889,16 @@ extern "C" int pie_hip_gemm_skinny_tiled(int format, const uint16_t* act_bf16, c
 
 // q|k|v projection over tile-major weights with RoPE and the KV write in the epilogue (more rows
 // than the GEMV form takes): values of pie_hip_gemm_skinny_tiled followed by
-// pie_hip_qkv_rope_kvwrite with interleaved = 1 and no q/k norm.
+// pie_hip_qkv_rope_kvwrite with interleaved = pairing (1 or 2) and no q/k norm.
 extern "C" int pie_hip_qkv_rope_skinny_tiled(int format, const uint16_t* act_bf16, const void* weight,
                                              const void* scale, int scale_is_bf16, int group_size,
                                              int M, int K, const float* rope_table,
                                              const int64_t* kv_slots, uint16_t* q_out,
                                              uint16_t* k_pages, uint16_t* v_pages, int num_q_heads,
-                                             int num_kv_heads, int head_dim, void* stream) {
+                                             int num_kv_heads, int head_dim, int pairing, void* stream) {
     using namespace pie_hip;
     if (!act_bf16 || !weight || !rope_table || !kv_slots || !q_out || !k_pages || !v_pages || M <= 0 ||
-        num_q_heads <= 0 || num_kv_heads <= 0 || head_dim <= 0)
+        num_q_heads <= 0 || num_kv_heads <= 0 || head_dim <= 0 || (pairing != 1 && pairing != 2))
         return PIE_HIP_ERR_INVALID;
     if (format != PIE_HIP_FMT_BF16 && !scale) return PIE_HIP_ERR_INVALID;
     if ((head_dim & (head_dim - 1)) != 0 || head_dim % 16 != 0 || K % kSwChunk != 0) return PIE_HIP_ERR_UNSUPPORTED;
@@ -913,6 +920,7 @@ extern "C" int pie_hip_qkv_rope_skinny_tiled(int format, const uint16_t* act_bf1
     a.hq = num_q_heads;
     a.hk = num_kv_heads;
     a.d = head_dim;
+    a.half_out = pairing == 2;
     return dispatch_skinny(format, a, 1, static_cast<hipStream_t>(stream));
 }
 

@@ -259,6 +259,9 @@ struct GemvArgs {
     uint16_t* v_pages;
     int hq, hk, d;
     int g_shift;  // log2(G) when G is a power of two, else -1 (set by dispatch)
+    // qkv epilogue: 1 when the q / k rows were re-ordered at load so that rows (2i, 2i+1) of a
+    // head hold the half-split pair (i, i + d/2); the rotated pair goes back to those positions
+    int half_out;
 };
 
 // ROPE: the q|k|v epilogue (rotation + KV write); its per-lane cos / sin / slot ride with every
@@ -587,10 +590,17 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
                             if (head < a.hq + a.hk) {
                                 const float c = u.rc, sn = u.rsn;
                                 const uint32_t out = pack_bf16x2(gb * c - ub * sn, ub * c + gb * sn);
-                                if (head < a.hq)
-                                    *reinterpret_cast<uint32_t*>(a.y + (static_cast<size_t>(m) * a.hq + head) * a.d + dd) = out;
-                                else if (slot >= 0)
-                                    *reinterpret_cast<uint32_t*>(a.k_pages + (static_cast<size_t>(slot) * a.hk + (head - a.hq)) * a.d + dd) = out;
+                                uint16_t* dst = head < a.hq
+                                                    ? a.y + (static_cast<size_t>(m) * a.hq + head) * a.d
+                                                    : a.k_pages + (static_cast<size_t>(slot) * a.hk + (head - a.hq)) * a.d;
+                                if (head < a.hq || slot >= 0) {
+                                    if (a.half_out) {
+                                        dst[dd >> 1] = static_cast<uint16_t>(out & 0xFFFFu);
+                                        dst[(dd >> 1) + (a.d >> 1)] = static_cast<uint16_t>(out >> 16);
+                                    } else {
+                                        *reinterpret_cast<uint32_t*>(dst + dd) = out;
+                                    }
+                                }
                             } else if (slot >= 0) {
                                 *reinterpret_cast<uint32_t*>(a.v_pages + (static_cast<size_t>(slot) * a.hk + (head - a.hq - a.hk)) * a.d + dd) =
                                     pack_bf16x2(gb, ub);
@@ -822,24 +832,27 @@ extern "C" int pie_hip_linear_fused(int format, const uint16_t* act_bf16,
 }
 
 // The fused q|k|v projection of a decode step with the rotation and the KV-cache write in its
-// epilogue (interleaved RoPE, no per-head q/k norm): replaces the projection followed by
-// qkv_rope_kvwrite_kernel with identical values.
+// epilogue (no per-head q/k norm): replaces the projection followed by qkv_rope_kvwrite_kernel
+// with identical values.  pairing 1: adjacent pairs (2i, 2i+1); 2: weight rows re-ordered at load
+// so that rows (2i, 2i+1) of a q / k head are the half-split pair (i, i + d/2), written back to
+// those positions.
 extern "C" int pie_hip_qkv_rope_fused(int format, const uint16_t* act_bf16,
                                       const uint16_t* norm_weight_bf16, float eps,
                                       const void* weight, const void* scale, int scale_is_bf16,
                                       int group_size, int M, int K, const float* rope_table,
                                       const int64_t* kv_slots, uint16_t* q_out, uint16_t* k_pages,
                                       uint16_t* v_pages, int num_q_heads, int num_kv_heads,
-                                      int head_dim, void* stream) {
+                                      int head_dim, int pairing, void* stream) {
     using namespace pie_hip;
     if (!rope_table || !kv_slots || !q_out || !k_pages || !v_pages || num_q_heads <= 0 ||
-        num_kv_heads <= 0 || head_dim <= 0)
+        num_kv_heads <= 0 || head_dim <= 0 || (pairing != 1 && pairing != 2))
         return PIE_HIP_ERR_INVALID;
     if (head_dim < 2 || (head_dim & (head_dim - 1)) != 0) return PIE_HIP_ERR_UNSUPPORTED;
     const int N = (num_q_heads + 2 * num_kv_heads) * head_dim;
     GemvArgs a{act_bf16, static_cast<const u32x4_t*>(weight), nullptr, nullptr, q_out, N, K,
                group_size, 0, norm_weight_bf16, eps, 0, rope_table, kv_slots, k_pages, v_pages,
                num_q_heads, num_kv_heads, head_dim};
+    a.half_out = pairing == 2;
     hipStream_t st = static_cast<hipStream_t>(stream);
     switch (format) {
         case PIE_HIP_FMT_INT4B8:

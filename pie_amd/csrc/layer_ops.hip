@@ -115,7 +115,10 @@ __global__ void rope_table_kernel(const int32_t* __restrict__ positions,
 // driver/cuda/src/kernels/split_packed.cu:62-178; slot addressing :116-138 NHD).  The slot
 // (page*page_size + offset) is computed by the host planner from the page table, so the
 // same kernel serves decode and prefill rows.  interleaved = 0 pairs (i, i+d/2), 1 pairs
-// (2i, 2i+1) (driver/cuda/src/kernels/rope.cu:14-33).
+// (2i, 2i+1) (driver/cuda/src/kernels/rope.cu:14-33); 2: the projection's q / k rows were
+// re-ordered at load so that elements (2i, 2i+1) of its output hold the half-split pair
+// (i, i+d/2) — rotated as that pair and written to positions i and i+d/2, so q_out and the
+// pool hold exactly what interleaved = 0 gives over the original row order.
 __global__ __launch_bounds__(64) void qkv_rope_kvwrite_kernel(
     const uint16_t* __restrict__ packed, uint16_t* __restrict__ q_out,
     uint16_t* __restrict__ k_pages, uint16_t* __restrict__ v_pages,
@@ -149,15 +152,17 @@ __global__ __launch_bounds__(64) void qkv_rope_kvwrite_kernel(
                          : k_pages + (static_cast<size_t>(slot) * hk + (head - hq)) * d;
     const float* tab = rope_table + static_cast<size_t>(n) * d;
     for (int i = lane; i < half; i += kWave) {
+        // where pair i sits in the projection's row, and where it goes
         const int ia = interleaved ? 2 * i : i, ib = interleaved ? 2 * i + 1 : i + half;
+        const int oa = interleaved == 1 ? 2 * i : i, ob = interleaved == 1 ? 2 * i + 1 : i + half;
         float a = bf16_bits_to_f32(src[ia]), b = bf16_bits_to_f32(src[ib]);
         if (nw) {
-            a = a * inv_rms * bf16_bits_to_f32(nw[ia]);
-            b = b * inv_rms * bf16_bits_to_f32(nw[ib]);
+            a = a * inv_rms * bf16_bits_to_f32(nw[oa]);
+            b = b * inv_rms * bf16_bits_to_f32(nw[ob]);
         }
         const float c = tab[i], s = tab[i + half];
-        dst[ia] = f32_to_bf16_bits(a * c - b * s);
-        dst[ib] = f32_to_bf16_bits(b * c + a * s);
+        dst[oa] = f32_to_bf16_bits(a * c - b * s);
+        dst[ob] = f32_to_bf16_bits(b * c + a * s);
     }
 }
 

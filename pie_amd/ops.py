@@ -531,11 +531,26 @@ def gemm_mfma_workspace_bytes(M: int, N: int, K: int) -> int:
     return int(lib.pie_hip_gemm_mfma_workspace_bytes(M, N, K))
 
 
+def pair_qk_rows(w: WeightView, hq: int, hk: int, d: int) -> WeightView:
+    """The load-time row order of a fused q|k|v weight whose RoPE pairs are (i, i + d/2): inside
+    every q and k head, row 2i <- row i and row 2i+1 <- row i + d/2 (data and scales together;
+    V rows stay).  The fused epilogues with pairing = 2 undo it at the store."""
+    half = d // 2
+    head = torch.stack([torch.arange(half), torch.arange(half) + half], dim=1).reshape(-1)
+    idx = torch.cat([head + h * d for h in range(hq + hk)] +
+                    [torch.arange((hq + hk) * d, (hq + 2 * hk) * d)]).to(w.data.device)
+    data = w.data.reshape(w.N, -1)[idx].reshape(w.data.shape).contiguous()
+    scale = None if w.scale is None else w.scale.reshape(w.N, -1)[idx].reshape(w.scale.shape).contiguous()
+    return WeightView(w.kind, data, scale, w.group_size, w.N, w.K)
+
+
 def qkv_rope_fused(act: torch.Tensor, w: WeightView, table: torch.Tensor, kv_slots: torch.Tensor,
                    k_pages: torch.Tensor, v_pages: torch.Tensor, hq: int, hk: int, d: int,
-                   norm_weight: Optional[torch.Tensor] = None, eps: float = 1e-5) -> torch.Tensor:
-    """Fused q|k|v projection + interleaved RoPE + KV-cache write (decode rows).  Returns q
-    [M, hq, d]; k / v land in their slots of the pools."""
+                   norm_weight: Optional[torch.Tensor] = None, eps: float = 1e-5,
+                   pairing: int = 1) -> torch.Tensor:
+    """Fused q|k|v projection + RoPE + KV-cache write (decode rows).  Returns q [M, hq, d]; k / v
+    land in their slots of the pools.  pairing 1: adjacent pairs; 2: half-split pairs over
+    weights whose q / k rows were re-ordered with `pair_qk_rows`."""
     _dev(act, torch.bfloat16, "act")
     _dev(table, torch.float32, "rope_table")
     _dev(kv_slots, torch.int64, "kv_slots")
@@ -551,14 +566,16 @@ def qkv_rope_fused(act: torch.Tensor, w: WeightView, table: torch.Tensor, kv_slo
     _check(kernels().pie_hip_qkv_rope_fused(
         FMT[w.kind], _ptr(act), _ptr(norm_weight), C.c_float(eps), _ptr(w.data), _ptr(w.scale),
         scale_is_bf16, w.group_size, M, K, _ptr(table), _ptr(kv_slots), _ptr(q_out), _ptr(k_pages),
-        _ptr(v_pages), hq, hk, d, _stream()), "pie_hip_qkv_rope_fused")
+        _ptr(v_pages), hq, hk, d, pairing, _stream()), "pie_hip_qkv_rope_fused")
     return q_out
 
 
 def qkv_rope_skinny_tiled(act: torch.Tensor, w: WeightView, table: torch.Tensor, kv_slots: torch.Tensor,
-                          k_pages: torch.Tensor, v_pages: torch.Tensor, hq: int, hk: int, d: int) -> torch.Tensor:
-    """q|k|v projection over tile-major weights + interleaved RoPE + KV-cache write for a decode
-    batch (act already normalised).  Returns q [M, hq, d]; k / v land in their slots."""
+                          k_pages: torch.Tensor, v_pages: torch.Tensor, hq: int, hk: int, d: int,
+                          pairing: int = 1) -> torch.Tensor:
+    """q|k|v projection over tile-major weights + RoPE + KV-cache write for a decode batch (act
+    already normalised).  Returns q [M, hq, d]; k / v land in their slots.  pairing as for
+    `qkv_rope_fused`."""
     _dev(act, torch.bfloat16, "act")
     _dev(table, torch.float32, "rope_table")
     _dev(kv_slots, torch.int64, "kv_slots")
@@ -576,7 +593,7 @@ def qkv_rope_skinny_tiled(act: torch.Tensor, w: WeightView, table: torch.Tensor,
     _check(kernels().pie_hip_qkv_rope_skinny_tiled(
         FMT[w.kind[:-len("+tiled")]], _ptr(act), _ptr(w.data), _ptr(w.scale), scale_is_bf16, w.group_size,
         M, K, _ptr(table), _ptr(kv_slots), _ptr(q_out), _ptr(k_pages), _ptr(v_pages), hq, hk, d,
-        _stream()), "pie_hip_qkv_rope_skinny_tiled")
+        pairing, _stream()), "pie_hip_qkv_rope_skinny_tiled")
     return q_out
 
 

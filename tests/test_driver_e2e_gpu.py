@@ -10,42 +10,49 @@ from driver_util import cosine, full_cfg, oracle_model_from_driver, toml_config
 pytestmark = pytest.mark.gpu
 
 
-def step_frames(drvmod, tokens_prev, pos, replicate, ppc, ps):
-    npg = (pos + 1 + ps - 1) // ps
-    pages = np.concatenate([np.arange(npg) + c * ppc for c in range(replicate)])
-    return drvmod.ForwardFrame(tokens_prev, [pos] * replicate, pages,
-                               np.arange(replicate + 1) * npg,
-                               [pos + 1 - (npg - 1) * ps] * replicate, np.arange(replicate + 1))
+def ragged_prompts(rng, vocab, n_prompt, count):
+    """`count` distinct prompts of different lengths (the first `n_prompt` long, the others
+    shorter or longer by a few tokens, crossing page boundaries at different steps)."""
+    lens = [max(1, n_prompt + ((-1) ** c) * (3 * c + (c // 2))) for c in range(count)]
+    return [rng.integers(0, vocab, n) for n in lens]
 
 
-def teacher_forced_compare(oracle, drvmod, d, om, cfg, prompt, max_new, replicate, **bars):
-    """Feed the oracle's tokens to the GPU step by step; compare tokens and logits per step."""
+def teacher_forced_compare(oracle, drvmod, d, om, cfg, prompts, max_new, **bars):
+    """Feed the oracle's tokens to the GPU step by step — every context with its own prompt, its
+    own length and so its own position and page count in each decode batch — and compare the
+    token and the logits of EVERY request of every step.  Returns (oracle tokens, near-ties,
+    checks)."""
     ps, V = cfg["page_size"], cfg["vocab"]
-    n_prompt = len(prompt)
-    ppc = (n_prompt + max_new + ps - 1) // ps
-    otoks, otrace = om.generate(prompt, max_new, replicate, want_logits=True)
-    near_ties = 0
-    # prefill each context
-    for c in range(replicate):
-        npg = (n_prompt + ps - 1) // ps
-        fr = drvmod.ForwardFrame(prompt, np.arange(n_prompt), np.arange(npg) + c * ppc, [0, npg],
-                                 [n_prompt - (npg - 1) * ps], [0, n_prompt])
+    R = len(prompts)
+    lens = [len(p) for p in prompts]
+    ppc = (max(lens) + max_new + ps - 1) // ps
+    otoks, otrace = om.generate_ragged(prompts, max_new, want_logits=True)
+    near_ties = checks = 0
+    for c, prompt in enumerate(prompts):   # prefill each context
+        n = lens[c]
+        npg = (n + ps - 1) // ps
+        fr = drvmod.ForwardFrame(prompt, np.arange(n), np.arange(npg) + c * ppc, [0, npg],
+                                 [n - (npg - 1) * ps], [0, n])
         res = d.forward(fr)
         assert res.num_requests == 1 and len(res.tokens) == 1
-        if c == 0:
-            lg = d.export_tensor("debug.logits", np.uint16).reshape(-1, V)[0]
-            near_ties += check_step(oracle, lg, otrace[0], res.tokens[0], otoks[0, 0],
-                                    router_gap=om.last_router_gaps[0], **bars)
+        lg = d.export_tensor("debug.logits", np.uint16).reshape(-1, V)[0]
+        near_ties += check_step(oracle, lg, otrace[0][c], res.tokens[0], otoks[c, 0],
+                                router_gap=om.prefill_router_gaps[c], **bars)
+        checks += 1
     for s in range(1, max_new):
-        pos = n_prompt + s - 1
-        res = d.forward(step_frames(drvmod, otoks[:, s - 1], pos, replicate, ppc, ps))
-        assert res.num_requests == replicate and res.tokens_indptr == list(range(replicate + 1))
+        pos = [n + s - 1 for n in lens]
+        npg = [(p + 1 + ps - 1) // ps for p in pos]
+        pages = np.concatenate([np.arange(g) + c * ppc for c, g in enumerate(npg)])
+        fr = drvmod.ForwardFrame(otoks[:, s - 1], pos, pages, np.concatenate([[0], np.cumsum(npg)]),
+                                 [p + 1 - (g - 1) * ps for p, g in zip(pos, npg)], np.arange(R + 1))
+        res = d.forward(fr)
+        assert res.num_requests == R and res.tokens_indptr == list(range(R + 1))
         lg = d.export_tensor("debug.logits", np.uint16).reshape(-1, V)
-        near_ties += check_step(oracle, lg[0], otrace[s], res.tokens[0], otoks[0, s],
-                                router_gap=om.last_router_gaps[s], **bars)
-        # every replica holds the same context: identical tokens
-        assert len(set(res.tokens)) == 1
-    return otoks, near_ties
+        for c in range(R):
+            near_ties += check_step(oracle, lg[c], otrace[s][c], res.tokens[c], otoks[c, s],
+                                    router_gap=om.last_router_gaps[s], **bars)
+            checks += 1
+    return otoks, near_ties, checks
 
 
 def check_step(oracle, gpu_logit_bits, orc_logit_bits, gpu_tok, orc_tok, cos_min=0.9999, rel=0.02,
@@ -63,9 +70,14 @@ def check_step(oracle, gpu_logit_bits, orc_logit_bits, gpu_tok, orc_tok, cos_min
     assert cosine(g, o) >= cos_min
     assert np.max(np.abs(g - o)) <= rel * np.max(np.abs(o)) + 1e-3
     top2 = np.sort(o)[-2:]
-    near_tie = router_tie or (top2[1] - top2[0]) <= tie * abs(top2[1]) + 1e-6
+    margin = tie * abs(top2[1]) + 1e-6
+    near_tie = router_tie or (top2[1] - top2[0]) <= margin
     if not near_tie:
         assert int(gpu_tok) == int(orc_tok)
+    elif not router_tie:
+        # a near-tie is not skipped: the token must be one of the tied candidates, i.e. a token
+        # whose oracle logit is within the margin of the oracle's best
+        assert o[int(gpu_tok)] >= top2[1] - margin
     # the token the driver returns is the argmax of its own logits, first index on ties
     assert int(gpu_tok) == int(np.argmax(g))
     return int(near_tie)
@@ -80,6 +92,8 @@ def check_step(oracle, gpu_logit_bits, orc_logit_bits, gpu_tok, orc_tok, cos_min
     dict(arch="qwen3", quant="int4b8", head_dim=128, q_heads=4, kv_heads=1, rope_theta=1e6),
     dict(quant="int4b8", head_dim=128, q_heads=8, kv_heads=2, hidden=1024, rope_factor=8.0),
     dict(quant="int4b8", page_size=32, use_graphs=False),
+    dict(quant="int4b8", rope_interleaved=True),
+    dict(quant="bf16", rope_interleaved=True, use_graphs=False),
     dict(arch="qwen3_moe", quant="fp8", head_dim=128, q_heads=4, kv_heads=1, num_experts=8, top_k=2,
          expert_intermediate=256, router_std=0.2, intermediate=0),
     dict(arch="qwen3_moe", quant="int4b8", head_dim=128, q_heads=4, kv_heads=1, num_experts=16,
@@ -92,20 +106,22 @@ def test_greedy_generation_matches_oracle(gpu, oracle, kw):
 
     cfg = full_cfg(**kw)
     rng = np.random.default_rng(90)
-    prompt = rng.integers(0, cfg["vocab"], 21)
+    prompts = ragged_prompts(rng, cfg["vocab"], 21, 3)
     with drvmod.Driver(toml_config(**kw)) as d:
         caps = d.capabilities()
         assert caps["kv_page_size"] == cfg["page_size"] and caps["vocab_size"] == cfg["vocab"]
         om, _ = oracle_model_from_driver(d, cfg)
-        otoks, near = teacher_forced_compare(oracle, drvmod, d, om, cfg, prompt, 10, 2)
-        assert near <= 3
+        otoks, near, checks = teacher_forced_compare(oracle, drvmod, d, om, cfg, prompts, 10)
+        # (2048 nearly flat logits: about a third of the rows have a runner-up within two bf16
+        # steps of the best; those rows are held to "one of the tied candidates" by check_step)
+        assert checks == 30 and near <= 15
     # free-running generation through the driver's own harness reproduces the oracle's
     # sequence (up to the first near-tie, if any)
     with drvmod.Driver(toml_config(**kw)) as d:
-        gtoks, tm = d.generate(prompt, 10, replicate=2)
+        gtoks, tm = d.generate(prompts[0], 10, replicate=2)
         assert tm["decode_steps"] == 9 and tm["decode_device_us"] > 0
         if near == 0:
-            assert np.array_equal(gtoks, otoks)
+            assert np.array_equal(gtoks[0], otoks[0])
         assert np.array_equal(gtoks[0], gtoks[1])
 
 
@@ -191,6 +207,34 @@ def test_mixed_batch_prefill_plus_decode_and_kv_copy(gpu, oracle):
         bad = drvmod.FrameDesc()
         bad.payload.kind = 77
         assert d.handle(bad).payload.status.status == 2
+
+
+def test_more_sampling_slots_than_rows(gpu):
+    """A request may name the same row in many sampling slots (several samplers on one row, as
+    the reference's planner allows, driver/portable/src/plan.cpp:224-470): the slot count then
+    exceeds max_forward_tokens.  Every slot gets its row's greedy token, graphs and later
+    ordinary batches keep working after the token buffers have grown."""
+    from pie_amd import driver as drvmod
+
+    kw = dict(quant="int4b8", max_forward_tokens=32, max_forward_requests=4)
+    cfg = full_cfg(**kw)
+    rng = np.random.default_rng(95)
+    prompt = rng.integers(0, cfg["vocab"], 9)
+    with drvmod.Driver(toml_config(**kw)) as d:
+        base = dict(token_ids=prompt, position_ids=np.arange(9), kv_page_indices=[2], kv_page_indptr=[0, 1],
+                    kv_last_page_lens=[9], qo_indptr=[0, 9])
+        plain = d.forward(drvmod.ForwardFrame(**base))
+        # one decode step first, so a graph is cached before the buffers grow
+        step = dict(token_ids=[plain.tokens[0]], position_ids=[9], kv_page_indices=[2], kv_page_indptr=[0, 1],
+                    kv_last_page_lens=[10], qo_indptr=[0, 1])
+        t_before = d.forward(drvmod.ForwardFrame(**step)).tokens
+        slots = np.concatenate([np.full(70, 8), np.arange(9), np.full(21, 3)])   # 100 slots on 9 rows
+        res = d.forward(drvmod.ForwardFrame(**base, sampling_indices=slots, sampling_indptr=[0, len(slots)]))
+        assert res.num_requests == 1 and len(res.tokens) == len(slots)
+        for i, row in enumerate(slots):
+            assert res.tokens[i] == res.tokens[70 + row]          # same row, same token
+        assert res.tokens[0] == plain.tokens[0]
+        assert d.forward(drvmod.ForwardFrame(**step)).tokens == t_before   # the graph was rebuilt
 
 
 def test_forward_failures_return_empty_response(gpu):
@@ -379,16 +423,16 @@ def test_generation_with_one_byte_kv_cache_matches_oracle(gpu, oracle, kw, kv_dt
     kw = dict(kw, kv_cache_dtype=kv_dtype)
     cfg = full_cfg(**kw)
     rng = np.random.default_rng(97)
-    prompt = rng.integers(0, cfg["vocab"], 37)
+    prompts = ragged_prompts(rng, cfg["vocab"], 37, 2)
     with drvmod.Driver(toml_config(**kw)) as d:
         om, _ = oracle_model_from_driver(d, cfg)
-        otoks, near = teacher_forced_compare(oracle, drvmod, d, om, cfg, prompt, 8, 2, cos_min=0.998,
-                                             rel=0.1, tie=2.0 ** -4)
-        assert near < 8   # (the tiny model's logits are flat: most steps are near-ties at 2^-4)
+        otoks, near, checks = teacher_forced_compare(oracle, drvmod, d, om, cfg, prompts, 8, cos_min=0.998,
+                                                     rel=0.1, tie=2.0 ** -4)
+        assert checks == 16 and near < 16   # (the tiny model's logits are flat: most steps are near-ties at 2^-4)
     with drvmod.Driver(toml_config(**kw)) as d:
-        gtoks, _ = d.generate(prompt, 8, replicate=2)
+        gtoks, _ = d.generate(prompts[0], 8, replicate=2)
         if near == 0:
-            assert np.array_equal(gtoks, otoks)
+            assert np.array_equal(gtoks[0], otoks[0])
         assert np.array_equal(gtoks[0], gtoks[1])
 
 
@@ -473,6 +517,17 @@ def test_unknown_kv_cache_dtypes_are_refused(gpu):
             drvmod.Driver(toml_config(kv_cache_dtype=bad))
 
 
+def test_raw_router_probabilities_are_refused(gpu):
+    """norm_topk = false (config.json norm_topk_prob) asks for un-renormalised router weights,
+    which the routing kernel does not produce: start-up fails instead of computing other weights."""
+    from pie_amd import driver as drvmod
+
+    toml = toml_config(arch="qwen3_moe", quant="bf16", num_experts=4, top_k=2, expert_intermediate=64,
+                       intermediate=0).replace("top_k = 2", "top_k = 2\nnorm_topk = false")
+    with pytest.raises(Exception, match="norm_topk"):
+        drvmod.Driver(toml)
+
+
 @pytest.mark.parametrize("kw", [dict(quant="int4b8"), dict(arch="qwen3", quant="bf16", head_dim=128, q_heads=4,
                                                            kv_heads=1, rope_theta=1e6)],
                          ids=["llama3-int4b8", "qwen3-bf16"])
@@ -518,17 +573,18 @@ def test_last_layer_intermediates_match_oracle(gpu, oracle, kw):
                                      rope_theta=1e6)], ids=["llama3-int4b8", "llama3-fp8", "qwen3-int4b8"])
 @pytest.mark.parametrize("replicate", [3, 4, 7])
 def test_small_decode_batches_match_oracle(gpu, oracle, kw, replicate):
-    """Three, four and seven identical contexts: the rows where each linear is sent to the GEMV or
-    to the skinny GEMM by cost (and the q|k|v epilogue changes kernels) against the oracle."""
+    """Three, four and seven contexts with their own prompts and lengths: the rows where each
+    linear is sent to the GEMV or to the skinny GEMM by cost (and the q|k|v epilogue changes
+    kernels) against the oracle, every request of every step."""
     from pie_amd import driver as drvmod
 
     cfg = full_cfg(**kw)
     rng = np.random.default_rng(96)
-    prompt = rng.integers(0, cfg["vocab"], 13)
+    prompts = ragged_prompts(rng, cfg["vocab"], 13, replicate)
     with drvmod.Driver(toml_config(**kw, total_pages=96)) as d:
         om, _ = oracle_model_from_driver(d, dict(cfg, total_pages=96))
-        _, near = teacher_forced_compare(oracle, drvmod, d, om, cfg, prompt, 6, replicate)
-        assert near <= 3
+        _, near, checks = teacher_forced_compare(oracle, drvmod, d, om, cfg, prompts, 6)
+        assert checks == 6 * replicate and near <= checks // 2
 
 
 def test_start_up_warm_up_changes_no_result(gpu):

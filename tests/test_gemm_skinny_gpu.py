@@ -277,3 +277,11 @@ def test_qkv_rope_epilogue_of_the_skinny_gemm_equals_projection_then_rope_kernel
     assert np.array_equal(bits(pools[0]), bits(pools[2]))
     assert np.array_equal(bits(pools[1]), bits(pools[3]))
     assert not np.all(bits(pools[0]) == bits(torch.full((64, hk, d), 0.5, device=gpu, dtype=torch.bfloat16)))
+    # half-split pairing over weights with re-ordered q / k rows (pairing = 2): the bytes of the
+    # original weights followed by the half-split rope kernel
+    wp = ops.repack_mfma_tiles(ops.pair_qk_rows(mk(gpu), hq, hk, d))
+    hp = [torch.full((64, hk, d), 0.5, device=gpu, dtype=torch.bfloat16) for _ in range(4)]
+    q3 = ops.qkv_rope_skinny_tiled(x, wp, tab, sg, hp[0], hp[1], hq, hk, d, pairing=2)
+    q4 = ops.qkv_rope_kvwrite(ops.gemm_skinny(x, wt), hp[2], hp[3], tab, sg, hq, hk, d, 0)
+    assert np.array_equal(bits(q3), bits(q4))
+    assert np.array_equal(bits(hp[0]), bits(hp[2])) and np.array_equal(bits(hp[1]), bits(hp[3]))

@@ -158,6 +158,18 @@ def test_qkv_rope_epilogue_equals_projection_then_rope_kernel(gpu, oracle, kind,
     assert np.array_equal(bits(q1), bits(q2))
     assert np.array_equal(bits(pools[0]), bits(pools[2]))
     assert np.array_equal(bits(pools[1]), bits(pools[3]))
+    # half-split pairing (Llama / Qwen checkpoints): weights with re-ordered q / k rows and
+    # pairing = 2 give the bytes of the original weights followed by the half-split rope kernel;
+    # so does the rope kernel's own mode 2 over the re-ordered projection
+    wp = ops.pair_qk_rows(w, hq, hk, d)
+    hp = [torch.full((40, hk, d), 0.5, device=gpu, dtype=torch.bfloat16) for _ in range(6)]
+    q3 = ops.qkv_rope_fused(xg, wp, tab, sg, hp[0], hp[1], hq, hk, d, norm_weight=nwg, pairing=2)
+    q4 = ops.qkv_rope_kvwrite(packed, hp[2], hp[3], tab, sg, hq, hk, d, 0)
+    q5 = ops.qkv_rope_kvwrite(ops.linear_fused(xg, wp, norm_weight=nwg), hp[4], hp[5], tab, sg, hq, hk, d, 2)
+    assert np.array_equal(bits(q3), bits(q4)) and np.array_equal(bits(q5), bits(q4))
+    assert np.array_equal(bits(hp[0]), bits(hp[2])) and np.array_equal(bits(hp[1]), bits(hp[3]))
+    assert np.array_equal(bits(hp[4]), bits(hp[2])) and np.array_equal(bits(hp[5]), bits(hp[3]))
+    assert not np.array_equal(bits(q3), bits(q1))
     # and against the oracle's projection + rope
     ref_packed = oracle_linear(oracle, wd, oracle.rmsnorm(x, nw, 1e-5))
     kp = np.full((40, hk, d), oracle.f32_to_bf16(np.float32(0.5)), np.uint16)

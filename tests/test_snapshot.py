@@ -71,3 +71,49 @@ def test_reader_errors(oracle, tmp_path):
     (d / "x.safetensors").write_bytes(b"\x10\x00\x00\x00\x00\x00\x00\x00{\"a\":1}")
     with pytest.raises(RuntimeError):
         drvmod.snapshot_info(str(d))
+
+
+def _write_raw(path, header: dict, payload: bytes):
+    h = json.dumps(header).encode()
+    with open(path, "wb") as f:
+        f.write(len(h).to_bytes(8, "little") + h + payload)
+
+
+@pytest.mark.parametrize("entry,msg", [
+    (dict(dtype="BF16", shape=[4, 4], data_offsets=[0, 16]), "holds 16 bytes"),      # too few bytes for the shape
+    (dict(dtype="BF16", shape=[4, 4], data_offsets=[0, 64]), "out of range"),        # past the end of the file
+    (dict(dtype="BF16", shape=[-4, -4], data_offsets=[0, 32]), "bad dimension"),
+    (dict(dtype="BF16", shape=[2.5, 4], data_offsets=[0, 20]), "bad dimension"),
+    (dict(dtype="BF16", shape=[2 ** 40, 2 ** 40], data_offsets=[0, 32]), "overflows"),
+    (dict(dtype="Q4", shape=[4, 4], data_offsets=[0, 32]), "unknown dtype"),
+    (dict(dtype=7, shape=[4, 4], data_offsets=[0, 32]), "malformed"),
+    (dict(dtype="BF16", shape="4x4", data_offsets=[0, 32]), "malformed"),
+    (dict(dtype="BF16", shape=[4, 4], data_offsets=[-1, 31]), "out of range"),
+])
+def test_corrupt_safetensors_headers_are_refused(tmp_path, entry, msg):
+    """A header is never trusted: byte counts must equal shape x dtype size, dimensions are whole
+    and non-negative, dtypes known, offsets inside the file."""
+    from pie_amd import driver as drvmod
+
+    d = tmp_path / "corrupt"
+    os.makedirs(d)
+    (d / "config.json").write_text(json.dumps(dict(model_type="llama", hidden_size=64, num_hidden_layers=1,
+                                                   num_attention_heads=2, num_key_value_heads=1,
+                                                   intermediate_size=64, vocab_size=64)))
+    _write_raw(d / "model.safetensors", {"model.norm.weight": entry}, b"\0" * 32)
+    with pytest.raises(RuntimeError, match=msg):
+        drvmod.snapshot_info(str(d))
+
+
+def test_well_formed_raw_header_is_accepted(tmp_path):
+    from pie_amd import driver as drvmod
+
+    d = tmp_path / "fine"
+    os.makedirs(d)
+    (d / "config.json").write_text(json.dumps(dict(model_type="llama", hidden_size=64, num_hidden_layers=1,
+                                                   num_attention_heads=2, num_key_value_heads=1,
+                                                   intermediate_size=64, vocab_size=64)))
+    _write_raw(d / "model.safetensors",
+               {"model.norm.weight": dict(dtype="BF16", shape=[4, 4], data_offsets=[0, 32])}, b"\1" * 32)
+    info = drvmod.snapshot_info(str(d))
+    assert info["tensors"]["model.norm.weight"]["bytes"] == 32
