@@ -150,6 +150,9 @@ class OracleModel:
         finally:
             lib().orc_router_gap_get.restype = C.c_float
             self._router_gap = float(lib().orc_router_gap_get())
+            rows = np.zeros(max(N, 1), np.float32)
+            lib().orc_router_gap_rows(C.c_void_p(rows.ctypes.data), C.c_int(N))
+            self._router_row_gaps = rows[:N]
 
     def _forward_call(self, tok, pos, slots, rb, rl, pages, N, sr, S, out, logits, want_logits, masks,
                       allow, allow_off, p):
@@ -170,11 +173,82 @@ class OracleModel:
                                 vp(allow_off) if allow_off is not None else None)
         return out[:S], (logits[:S] if want_logits else None), p
 
+    # ---- higher-precision evaluations of the same graph (oracle/src/model_hp.c) ----
+    HP_MODES = {"P": 1, "f64": 2}
+
+    def hp_pools(self, mode: str):
+        """The KV pools of a higher-precision mode: two lists of float64 arrays
+        [pages, page_size, hk, d], created zeroed on first use."""
+        if not hasattr(self, "_hp"):
+            self._hp = {}
+        if mode not in self._hp:
+            cfg = self.cfg
+            shape = (cfg["total_pages"], cfg["page_size"], cfg["kv_heads"], cfg["head_dim"])
+            k = [np.zeros(shape, np.float64) for _ in range(cfg["layers"])]
+            v = [np.zeros(shape, np.float64) for _ in range(cfg["layers"])]
+            self._hp[mode] = (k, v, (C.c_void_p * len(k))(*[a.ctypes.data for a in k]),
+                              (C.c_void_p * len(v))(*[a.ctypes.data for a in v]))
+        return self._hp[mode][0], self._hp[mode][1]
+
+    def seed_hp_pools(self, mode: str, pages=None):
+        """Copies the bf16 pools' current contents (all pages, or the listed ones) into the
+        pools of `mode`, so that a higher-precision step starts from the same KV state."""
+        k, v = self.hp_pools(mode)
+        sel = slice(None) if pages is None else np.asarray(pages, np.int64)
+        for l in range(self.cfg["layers"]):
+            k[l][sel] = bf16_to_f32(self.k_pages[l][sel])
+            v[l][sel] = bf16_to_f32(self.v_pages[l][sel])
+
+    def forward_hp(self, mode: str, token_ids, position_ids, kv_page_indices, kv_page_indptr,
+                   kv_last_page_lens, qo_indptr, sampling_indices=None, sampling_indptr=None,
+                   masks=None, window: int = 0):
+        """The forward pass without the bf16 rounding points: mode "P" = F32 activations and an
+        F16 KV pool (the portable driver's rounding points), "f64" = double throughout (truth).
+        Uses and updates the pools of hp_pools(mode).  Returns (tokens, logits float64 [S, V],
+        plan)."""
+        R = len(qo_indptr) - 1
+        if sampling_indices is None:
+            qo = np.asarray(qo_indptr, np.int64)
+            sampling_indices = qo[1:] - qo[:-1] - 1
+            sampling_indptr = np.arange(R + 1)
+        p = plan_forward(token_ids, position_ids, kv_page_indices, kv_page_indptr,
+                         kv_last_page_lens, qo_indptr, sampling_indices, sampling_indptr,
+                         self.cfg["page_size"], self.cfg["total_pages"])
+        N, S = p["N"], len(p["sample_rows"])
+        c = lambda a, dt: np.ascontiguousarray(np.asarray(a, dt))
+        tok, pos = c(token_ids, np.uint32), c(p["positions"], np.int32)
+        slots, rb, rl = c(p["kv_slots"], np.int64), c(p["row_page_begin"], np.uint32), c(p["row_kv_len"], np.int32)
+        pages, sr = c(kv_page_indices, np.uint32), c(p["sample_rows"], np.uint32)
+        out = np.zeros(max(S, 1), np.uint32)
+        logits = np.zeros((max(S, 1), self.cfg["vocab"]), np.float64)
+        allow = allow_off = None
+        if masks is not None:
+            from oracle import brle_allow
+            offs, chunks, at = [], [], 0
+            for i in range(N):
+                chunks.append(brle_allow(masks[i], int(pos[i]), int(rl[i]), window))
+                offs.append(at)
+                at += int(rl[i])
+            allow = c(np.concatenate(chunks) if chunks else np.zeros(1, np.uint8), np.uint8)
+            allow_off = c(offs, np.int64)
+        self.hp_pools(mode)
+        _, _, kp, vp_ = self._hp[mode]
+        vp = lambda a: C.c_void_p(a.ctypes.data) if a is not None else None
+        lib().orc_llama_forward_hp(C.byref(self._m), C.c_int(self.HP_MODES[mode]), kp, vp_, vp(tok), vp(pos),
+                                   vp(slots), vp(rb), vp(rl), vp(pages), C.c_int(N), vp(sr), C.c_int(S),
+                                   C.c_int(self.cfg["page_size"]), vp(out), vp(logits), vp(allow),
+                                   vp(allow_off))
+        return out[:S], logits[:S], p
+
     def router_gap(self) -> float:
         """Smallest gap between the last chosen and the first rejected router logit, relative to
         the token's largest logit magnitude, in the most recent forward (huge for dense models):
         near bf16 resolution, another summation order may route a token to another expert."""
         return self._router_gap
+
+    def router_row_gaps(self) -> np.ndarray:
+        """router_gap() per row of the most recent forward (minimum over its layers)."""
+        return self._router_row_gaps
 
     def generate(self, prompt, max_new: int, replicate: int = 1, want_logits=False):
         """Greedy generation of `replicate` copies of one prompt (see generate_ragged).  Returns
@@ -192,7 +266,8 @@ class OracleModel:
         (driver/portable/src/executor/executor.cpp:1439-1597) over a ragged batch.  Returns tokens
         [R, max_new] and, when asked, trace[step][r] = logits (bf16 bits) of context r;
         `prefill_router_gaps[r]` holds router_gap() of context r's prefill, `last_router_gaps` the
-        smallest of those followed by the gap of each decode step."""
+        smallest of those followed by the gap of each decode step, `step_router_row_gaps[s][r]`
+        the gap of request r's own rows in step s (step 0 = its prefill)."""
         ps = self.cfg["page_size"]
         R = len(prompts)
         lens = [len(p) for p in prompts]
@@ -210,6 +285,7 @@ class OracleModel:
             if want_logits:
                 trace[0][c] = lg[0]
         self.last_router_gaps = [min(self.prefill_router_gaps)]
+        self.step_router_row_gaps = [np.asarray(self.prefill_router_gaps, np.float32)]   # [step][request]
         for s in range(1, max_new):
             pos = [n + s - 1 for n in lens]
             npg = [(p + 1 + ps - 1) // ps for p in pos]
@@ -219,6 +295,7 @@ class OracleModel:
                                     np.arange(R + 1), want_logits=want_logits)
             toks[:, s] = t
             self.last_router_gaps.append(self.router_gap())
+            self.step_router_row_gaps.append(self.router_row_gaps().copy())
             if want_logits:
                 for c in range(R):
                     trace[s][c] = lg[c]

@@ -25,34 +25,7 @@
 
 #include "oracle_api.h"
 
-typedef struct {
-    const void* data;
-    const void* scale; /* int4: bf16 [N, K/G]; int8/fp8: f32 [N]; bf16: NULL */
-} OrcLinear;
-
-typedef struct {
-    int hidden, layers, q_heads, kv_heads, head_dim, intermediate, vocab;
-    float rms_eps;
-    int rope_interleaved, has_qk_norm;
-    int quant; /* 0 int4b8, 1 int8, 2 fp8, 3 bf16 */
-    int group;
-    const uint16_t* embed;
-    const uint16_t* lm_head;
-    const uint16_t* final_norm;
-    const float* inv_freq;
-    const uint16_t* const* attn_norm; /* [L] */
-    const uint16_t* const* ffn_norm;
-    const uint16_t* const* q_norm;
-    const uint16_t* const* k_norm;
-    const OrcLinear* wqkv; /* [L] */
-    const OrcLinear* wo;
-    const OrcLinear* wgu;
-    const OrcLinear* wdown;
-    /* MoE (num_experts > 0): wgu / wdown hold the experts stacked along the rows,
-     * [E * 2*Ie, H] (per expert: gate rows then up rows) and [E * H, Ie]. */
-    int num_experts, top_k, expert_intermediate;
-    const uint16_t* const* router; /* [L] bf16 [E, H] */
-} OrcModel;
+#include "model_types.h"
 
 static void orc_linear(const OrcModel* m, const OrcLinear* w, const uint16_t* act, uint16_t* y,
                        int M, int N, int K, int beta) {
@@ -104,9 +77,17 @@ static OrcLinear orc_expert_slice(const OrcModel* m, const OrcLinear* w, int e, 
  * since the last reset.  A gap at bf16 resolution
  * means another summation order may pick another expert there: the parity tests flag such a
  * forward as a near-tie instead of holding it to the logit bar. */
+#define ORC_ROUTER_GAP_ROWS 8192
 static float g_router_min_gap = 3.4e38f;
-void orc_router_gap_reset(void) { g_router_min_gap = 3.4e38f; }
+static float g_router_row_gap[ORC_ROUTER_GAP_ROWS]; /* the same, per row of the forward (min over layers) */
+void orc_router_gap_reset(void) {
+    g_router_min_gap = 3.4e38f;
+    for (int i = 0; i < ORC_ROUTER_GAP_ROWS; ++i) g_router_row_gap[i] = 3.4e38f;
+}
 float orc_router_gap_get(void) { return g_router_min_gap; }
+void orc_router_gap_rows(float* out, int n) {
+    for (int i = 0; i < n; ++i) out[i] = i < ORC_ROUTER_GAP_ROWS ? g_router_row_gap[i] : 0.f;
+}
 static void orc_router_gap_note(const uint16_t* logits, int N, int E, int K) {
     if (K >= E) return;
     for (int n = 0; n < N; ++n) {
@@ -123,6 +104,7 @@ static void orc_router_gap_note(const uint16_t* logits, int N, int E, int K) {
         for (int j = 0; j < E; ++j) mag = fabsf(v[j]) > mag ? fabsf(v[j]) : mag;
         const float gap = (v[K - 1] - v[K]) / (mag > 1e-20f ? mag : 1e-20f);
         if (gap < g_router_min_gap) g_router_min_gap = gap;
+        if (n < ORC_ROUTER_GAP_ROWS && gap < g_router_row_gap[n]) g_router_row_gap[n] = gap;
     }
 }
 

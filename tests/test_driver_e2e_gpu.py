@@ -12,8 +12,12 @@ pytestmark = pytest.mark.gpu
 
 def ragged_prompts(rng, vocab, n_prompt, count):
     """`count` distinct prompts of different lengths (the first `n_prompt` long, the others
-    shorter or longer by a few tokens, crossing page boundaries at different steps)."""
-    lens = [max(1, n_prompt + ((-1) ** c) * (3 * c + (c // 2))) for c in range(count)]
+    shorter or longer by a few tokens, crossing page boundaries at different steps; for large
+    batches, lengths drawn from 1 .. 3 * n_prompt)."""
+    if count > 8:
+        lens = [n_prompt] + [int(n) for n in rng.integers(1, 3 * n_prompt + 1, count - 1)]
+    else:
+        lens = [max(1, n_prompt + ((-1) ** c) * (3 * c + (c // 2))) for c in range(count)]
     return [rng.integers(0, vocab, n) for n in lens]
 
 
@@ -39,6 +43,9 @@ def teacher_forced_compare(oracle, drvmod, d, om, cfg, prompts, max_new, **bars)
         near_ties += check_step(oracle, lg, otrace[0][c], res.tokens[0], otoks[c, 0],
                                 router_gap=om.prefill_router_gaps[c], **bars)
         checks += 1
+    # A request's logits depend on the routing of its own rows only, now and in the steps that
+    # wrote its KV history: the margin that matters is the smallest over the request's past.
+    gap_so_far = np.asarray(om.step_router_row_gaps[0], np.float64).copy()
     for s in range(1, max_new):
         pos = [n + s - 1 for n in lens]
         npg = [(p + 1 + ps - 1) // ps for p in pos]
@@ -48,9 +55,10 @@ def teacher_forced_compare(oracle, drvmod, d, om, cfg, prompts, max_new, **bars)
         res = d.forward(fr)
         assert res.num_requests == R and res.tokens_indptr == list(range(R + 1))
         lg = d.export_tensor("debug.logits", np.uint16).reshape(-1, V)
+        gap_so_far = np.minimum(gap_so_far, om.step_router_row_gaps[s])
         for c in range(R):
             near_ties += check_step(oracle, lg[c], otrace[s][c], res.tokens[c], otoks[c, s],
-                                    router_gap=om.last_router_gaps[s], **bars)
+                                    router_gap=gap_so_far[c], **bars)
             checks += 1
     return otoks, near_ties, checks
 
@@ -114,7 +122,9 @@ def test_greedy_generation_matches_oracle(gpu, oracle, kw):
         otoks, near, checks = teacher_forced_compare(oracle, drvmod, d, om, cfg, prompts, 10)
         # (2048 nearly flat logits: about a third of the rows have a runner-up within two bf16
         # steps of the best; those rows are held to "one of the tied candidates" by check_step)
-        assert checks == 30 and near <= 15
+        # (MoE: a request also counts as near-tie once any token of its history had a router
+        # margin at bf16 resolution; those steps are held to the looser bar, never skipped)
+        assert checks == 30 and (near <= 15 or cfg["num_experts"])
     # free-running generation through the driver's own harness reproduces the oracle's
     # sequence (up to the first near-tie, if any)
     with drvmod.Driver(toml_config(**kw)) as d:
@@ -585,6 +595,35 @@ def test_small_decode_batches_match_oracle(gpu, oracle, kw, replicate):
         om, _ = oracle_model_from_driver(d, dict(cfg, total_pages=96))
         _, near, checks = teacher_forced_compare(oracle, drvmod, d, om, cfg, prompts, 6)
         assert checks == 6 * replicate and near <= checks // 2
+
+
+@pytest.mark.parametrize("kw", [
+    dict(quant="int4b8"),
+    dict(quant="int4b8", kv_cache_dtype="fp8_per_token_head"),
+    dict(arch="qwen3_moe", quant="fp8", head_dim=128, q_heads=8, kv_heads=1, num_experts=16, top_k=4,
+         expert_intermediate=256, router_std=0.2, intermediate=0),
+    dict(arch="qwen3_moe", quant="fp8", head_dim=128, q_heads=8, kv_heads=1, num_experts=16, top_k=4,
+         expert_intermediate=256, router_std=0.2, intermediate=0, kv_cache_dtype="int8_per_token_head"),
+], ids=["llama3-int4b8", "llama3-int4b8-fp8kv", "moe-fp8", "moe-fp8-int8kv"])
+@pytest.mark.parametrize("count", [16, 64])
+def test_decode_batches_of_16_and_64_distinct_requests(gpu, oracle, kw, count):
+    """Decode batches of 16 and 64 requests, every request with its own prompt and context length
+    (1 to 39 tokens at the first step): the 16-row skinny GEMM passes (one, and four side by
+    side), the matrix-core decode attention over ragged contexts, the grouped expert GEMMs with
+    64 x top-k routes — every request of every step against the oracle."""
+    from pie_amd import driver as drvmod
+
+    kw = dict(kw, total_pages=4 * count + 8, max_forward_requests=count, max_forward_tokens=128)
+    cfg = full_cfg(**kw)
+    rng = np.random.default_rng(1000 + count)
+    prompts = ragged_prompts(rng, cfg["vocab"], 13, count)
+    bars = dict(cos_min=0.998, rel=0.1, tie=2.0 ** -4) if kw.get("kv_cache_dtype") else {}
+    with drvmod.Driver(toml_config(**kw)) as d:
+        om, _ = oracle_model_from_driver(d, cfg)
+        _, near, checks = teacher_forced_compare(oracle, drvmod, d, om, cfg, prompts, 4, **bars)
+        assert checks == 4 * count
+        if not kw.get("kv_cache_dtype") and not cfg["num_experts"]:
+            assert near <= checks // 2
 
 
 def test_start_up_warm_up_changes_no_result(gpu):

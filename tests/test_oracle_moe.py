@@ -90,6 +90,34 @@ def test_oracle_moe_forward_matches_dense_fp64(oracle, quant):
     assert good >= 5
 
 
+@pytest.mark.parametrize("quant", ["bf16", "fp8", "int4b8"])
+def test_truth_mode_moe_forward_equals_dense_fp64(oracle, quant):
+    """The double-precision forward over MoE layers (router softmax, top-k with the lowest index
+    on ties, renormalised weights, unrounded expert sums) is the numpy fp64 transformer to
+    summation-order accuracy — no routing near-tie can separate two fp64 evaluations here."""
+    from oracle.model import OracleModel
+
+    cfg = dict(hidden=128, layers=2, q_heads=4, kv_heads=2, head_dim=32, intermediate=0, vocab=200,
+               rms_eps=1e-5, rope_interleaved=0, qk_norm=True, quant=quant, group_size=64,
+               page_size=4, total_pages=16, num_experts=6, top_k=3, expert_intermediate=64)
+    rng = np.random.default_rng(404)
+    t = make_tensors(oracle, rng, cfg)
+    om, ref = OracleModel(cfg, t), DenseRef(oracle, cfg, t)
+    prompt = rng.integers(0, cfg["vocab"], 9)
+    args = dict(token_ids=prompt, position_ids=np.arange(9), kv_page_indices=[3, 7, 1], kv_page_indptr=[0, 3],
+                kv_last_page_lens=[1], qo_indptr=[0, 9], sampling_indices=np.arange(9), sampling_indptr=[0, 9])
+    toks, logits, _ = om.forward_hp("f64", **args)
+    _, lp, _ = om.forward_hp("P", **args)
+    for i, tk in enumerate(prompt):
+        ref.min_gap = 1.0
+        rl = ref.step(int(tk), i)
+        assert ref.min_gap > 1e-9
+        assert np.max(np.abs(logits[i] - rl)) <= 1e-9 * np.max(np.abs(rl)), i
+        assert int(toks[i]) == int(np.argmax(rl))
+        if ref.min_gap > 1e-4:   # F32 / F16 noise cannot flip a router decision this wide
+            assert lp[i] @ rl / (np.linalg.norm(lp[i]) * np.linalg.norm(rl)) >= 0.99999, i
+
+
 def test_router_gap_reports_the_selection_margin(oracle):
     """router_gap() = (last chosen - first rejected router logit) / the token's largest logit
     magnitude, minimum over layers and tokens.  Router rows c_e * u with c = +-powers of two make
