@@ -167,8 +167,10 @@ def time_graph(fn, n_launch: int, reps: int = 5) -> float:
     return e0.elapsed_time(e1) * 1e-3 / (reps * n_launch)
 
 
-def attention_extra():
-    """Paged decode attention on BASELINE's attention config, timed from a HIP graph."""
+def attention_case():
+    """BASELINE's attention config as device tensors plus one launcher per KV storage:
+    32 q / 8 kv heads of 128, page 16, 64 requests with contexts uniform in [512, 8192], block
+    tables a random permutation of the pool, 16 of the 64 sharing a forked 1024-token prefix."""
     import torch
 
     from pie_amd import ops
@@ -205,29 +207,65 @@ def attention_extra():
     need = ops.attn_decode_workspace_bytes(R, hq, hk, d, maxlen)
     ws = torch.empty(max(need, 16), dtype=torch.uint8, device=dev)
     o = torch.empty_like(q)
-    t = time_graph(lambda: ops.attention_paged_decode(q, kp, vp, pi, pp, ll, maxlen, o=o, workspace=ws), 10)
     alg = int(ctx.sum()) * 2 * hk * d * 2 + R * hq * d * 2 * 2
     dedup = alg - 15 * 1024 * 2 * hk * d * 2
+    launch = {"bf16": lambda: ops.attention_paged_decode(q, kp, vp, pi, pp, ll, maxlen, o=o, workspace=ws)}
     # the same batch over one-byte pools (codes + fp32 scales per (token, head))
     rb = torch.tensor(indptr[:-1], dtype=torch.int32, device=dev)
     rl = torch.from_numpy(ctx.astype(np.int32)).to(dev)
-    one_byte = {}
+    keep = []
     for fmt in ("fp8_per_token_head", "int8_per_token_head"):
         k8 = torch.randint(0, 120, (total, ps, hk, d), dtype=torch.uint8, device=dev)
         v8 = torch.randint(0, 120, (total, ps, hk, d), dtype=torch.uint8, device=dev)
         ks = torch.rand(total, ps, hk, device=dev) * 0.01 + 0.001
         vs = torch.rand(total, ps, hk, device=dev) * 0.01 + 0.001
-        fn = lambda: ops.attention_rows_paged_kvq(fmt, q, k8, v8, ks, vs, pi, rb, rl, max_kv_len=maxlen,
-                                                  o=o, workspace=ws)
-        fn()
-        tq = time_graph(fn, 10)
-        algq = int(ctx.sum()) * 2 * hk * (d + 4) + R * hq * d * 2 * 2
+        keep.append((k8, v8, ks, vs))
+        launch[fmt] = (lambda fmt=fmt, k8=k8, v8=v8, ks=ks, vs=vs:
+                       ops.attention_rows_paged_kvq(fmt, q, k8, v8, ks, vs, pi, rb, rl, max_kv_len=maxlen,
+                                                    o=o, workspace=ws))
+    algq = int(ctx.sum()) * 2 * hk * (d + 4) + R * hq * d * 2 * 2
+    return dict(launch=launch, alg=alg, dedup=dedup, alg_one_byte=algq, keep=keep)
+
+
+def attention_extra():
+    """Paged decode attention on BASELINE's attention config, timed from a HIP graph."""
+    case = attention_case()
+    t = time_graph(case["launch"]["bf16"], 10)
+    one_byte = {}
+    for fmt in ("fp8_per_token_head", "int8_per_token_head"):
+        case["launch"][fmt]()
+        tq = time_graph(case["launch"][fmt], 10)
+        algq = case["alg_one_byte"]
         one_byte[fmt] = dict(us=round(tq * 1e6, 1), algorithmic_bytes=algq, gbps=round(algq / tq / 1e9, 1),
                              frac_of_hbm_peak=round(algq / tq / 1e9 / HBM_PEAK_GBPS, 4))
+    alg = case["alg"]
     return dict(workload="decode attention 32q/8kv d128 page16 batch64 ctx U[512,8192] 25% forked 1024 prefix",
                 us=round(t * 1e6, 1), algorithmic_bytes=alg, gbps=round(alg / t / 1e9, 1),
                 frac_of_hbm_peak=round(alg / t / 1e9 / HBM_PEAK_GBPS, 4),
-                dedup_bytes=dedup, note="split kernel + merge kernel per call", one_byte_kv=one_byte)
+                dedup_bytes=case["dedup"], note="split kernel + merge kernel per call", one_byte_kv=one_byte)
+
+
+def attention_workload():
+    """What a `rocprofv3` run over the attention config needs: four 256 MiB device copies (the
+    scale of the FETCH_SIZE / WRITE_SIZE counters), then 12 eager launches of the decode
+    attention over the bf16 pool and 12 over each one-byte pool."""
+    import torch
+
+    dev = torch.device("cuda:0")
+    src = torch.empty(256 * 1024 * 1024 // 4, dtype=torch.float32, device=dev).normal_()
+    dst = torch.empty_like(src)
+    for _ in range(4):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    case = attention_case()
+    for name, fn in case["launch"].items():
+        for _ in range(12):
+            fn()
+        torch.cuda.synchronize()
+    print(json.dumps({"attention_workload": "4 x 256 MiB copy, 12 launches of the batch-64 decode attention per "
+                                            "KV storage (bf16, fp8_per_token_head, int8_per_token_head)",
+                      "algorithmic_bytes_bf16": case["alg"], "deduplicated_bytes_bf16": case["dedup"],
+                      "algorithmic_bytes_one_byte": case["alg_one_byte"]}))
 
 
 def w4a16_sweep_extra():
@@ -272,6 +310,39 @@ def w4a16_sweep_extra():
     return out
 
 
+def other_configs_extra(drvmod):
+    """Decode throughput of the other BASELINE decode configurations, each through its own driver
+    instance (created after the headline driver is closed): the 8B W4A16 model at batch 16 and 64
+    after 2048-token prefills, the 1B int8 model at batch 1 (128-token prompt, 64 steps) and the
+    30B-A3B fp8 MoE at batch 64 over 1024-token contexts."""
+    import torch
+
+    out = {}
+    cases = [("llama8b_w4a16_batch16_ctx2048", MODEL, 16, 2048, 32, 4),
+             ("llama8b_w4a16_batch64_ctx2048", MODEL, 64, 2048, 32, 4),
+             ("llama1b_int8_batch1_prompt128", OTHER_MODELS["llama1b-int8"][0], 1, 128, 64, 8),
+             ("qwen3_30b_a3b_fp8_batch64_ctx1024", OTHER_MODELS["qwen3-30b-a3b-fp8"][0], 64, 1024, 32, 4)]
+    for name, model, batch, n_prompt, steps, warm in cases:
+        page_size = 16
+        max_new = warm + steps + 1
+        pages = (n_prompt + max_new + page_size - 1) // page_size * batch + 8
+        rng = np.random.default_rng(4096 + batch)
+        prompt = rng.integers(0, model["vocab"], n_prompt)
+        t0 = time.perf_counter()
+        drv = drvmod.Driver(toml(model, page_size, pages, 2048, max(16, batch)))
+        t_init = time.perf_counter() - t0
+        try:
+            _, tm = drv.generate(prompt, max_new, replicate=batch, warmup=warm)
+        finally:
+            drv.close()
+        torch.cuda.empty_cache()
+        wall = tm["decode_wall_us"] * 1e-6
+        out[name] = dict(tokens_per_s=round(batch * tm["decode_steps"] / wall, 1),
+                         ms_per_step=round(wall / tm["decode_steps"] * 1e3, 4), steps=tm["decode_steps"],
+                         warmup=warm, init_s=round(t_init, 2), prefill_s=round(tm["prefill_us"] * 1e-6, 3))
+    return out
+
+
 def lm_head_extra(drv, model):
     import torch
 
@@ -306,6 +377,11 @@ def cpu_baseline(drv, model, page_size, total_pages, n_prompt, gpu_tokens, budge
 
     from pie_amd import driver as drvmod
 
+    # The same steps in double precision (the value both implementations approximate), from the
+    # same prefilled pages: separates rounding noise shared by both from a defect in either.
+    truth_steps = 4
+    om.seed_hp_pools("f64", pages=np.arange((n_prompt + page_size - 1) // page_size))
+    dev_gpu_truth, dev_orc_truth = [], []
     steps, matched, near_ties, t_total = 0, 0, 0, 0.0
     margins = []   # per mismatch: how far below its own choice the oracle ranks the GPU's token
     cosines, noise_rel_top, replay_diff = [], [], 0
@@ -325,6 +401,12 @@ def cpu_baseline(drv, model, page_size, total_pages, n_prompt, gpu_tokens, budge
         steps += 1
         lg = oracle.bf16_to_f32(np.asarray(logits).reshape(-1)).astype(np.float64)
         cosines.append(float(g @ lg / (np.linalg.norm(g) * np.linalg.norm(lg) + 1e-30)))
+        if steps <= truth_steps:   # (untimed)
+            _, lt, _ = om.forward_hp("f64", [tok], [pos], np.arange(npg), [0, npg], [last], [0, 1])
+            lt = lt[0]
+            one_minus_cos = lambda a: float(1.0 - a @ lt / (np.linalg.norm(a) * np.linalg.norm(lt) + 1e-30))
+            dev_gpu_truth.append(one_minus_cos(g))
+            dev_orc_truth.append(one_minus_cos(lg))
         top = float(lg[int(out[0])])
         dev_rms = float(np.sqrt(np.mean((g - lg) ** 2)))   # rms logit deviation of this step
         noise_rel_top.append(dev_rms / max(abs(top), 1e-30))
@@ -350,15 +432,29 @@ def cpu_baseline(drv, model, page_size, total_pages, n_prompt, gpu_tokens, budge
                 mismatch_margins_rel_to_top_logit=margins,
                 logit_cosine_min=round(min(cosines), 6), logit_cosine_mean=round(float(np.mean(cosines)), 6),
                 logit_rms_deviation_rel_to_top_logit=round(float(np.mean(noise_rel_top)), 5),
-                replayed_steps_with_another_token=replay_diff)
+                replayed_steps_with_another_token=replay_diff,
+                one_minus_cosine_vs_double_precision=dict(
+                    note=f"first {len(dev_gpu_truth)} compared steps re-evaluated in double precision from the "
+                         "same prefilled pages (untimed): distance of the GPU's and of the oracle's logits "
+                         "from that truth",
+                    gpu=[float(f"{v:.3e}") for v in dev_gpu_truth],
+                    oracle=[float(f"{v:.3e}") for v in dev_orc_truth]))
 
 
-# HBM bytes per GEMV launch, averaged over the model's four int4 linears at M = 1, from two
-# `rocprofv3 --pmc` runs of `bench.py --pmc-workload` (FETCH_SIZE, then WRITE_SIZE, KiB per
-# dispatch), each scaled by what the same counter reads for the 256 MiB copy in that run
-# (FETCH_SIZE reads 131 085 for 262 144 KiB: factor 2.0; WRITE_SIZE reads 262 144: factor 1.0).
-# GEMV: FETCH_SIZE 14 018.8 -> 28.71 MB, WRITE_SIZE 30.0 -> 0.03 MB; algorithmic 28.15 MB.
-GEMV_TRAFFIC_BYTES_PER_LAUNCH = 28_742_000
+def gemv_traffic_bytes_per_launch():
+    """HBM bytes per GEMV launch (average of the model's four int4 linears at M = 1) as the
+    committed `rocprofv3 --pmc` summary states them, or None when that file is missing or holds
+    no such line.  The summary is rewritten whenever the kernel is profiled again, so this figure
+    cannot outlive the kernel it was measured on unnoticed: the summary names the library build
+    it profiled."""
+    import re
+
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "gemv_w4a16_m1_hbm_traffic_pmc.md")
+    try:
+        m = re.search(r"^traffic_bytes_per_launch:\s*([0-9_]+)", open(path).read(), re.M)
+    except OSError:
+        return None
+    return int(m.group(1).replace("_", "")) if m else None
 
 
 def pmc_workload():
@@ -414,6 +510,9 @@ def main():
     ap.add_argument("--sampler", default="greedy", choices=["greedy", "top_p", "top_k", "min_p", "multinomial"],
                     help="decode-step sampler (default greedy = the headline workload); the others run "
                          "the device samplers at temperature 0.8 (top_p 0.95 / top_k 50 / min_p 0.05)")
+    ap.add_argument("--attention-workload", action="store_true",
+                    help="only launch the batch-64 decode attention of BASELINE's attention config (and a "
+                         "256 MiB copy as the counters' scale), for `rocprofv3` kernel traces and --pmc runs")
     ap.add_argument("--pmc-workload", action="store_true",
                     help="only launch what a `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE` run needs: a "
                          "256 MiB device copy (the counter's scale) and the four int4 GEMV shapes")
@@ -432,6 +531,9 @@ def main():
 
     if args.pmc_workload:
         pmc_workload()
+        return
+    if args.attention_workload:
+        attention_workload()
         return
     page_size = 16
     max_new = args.warmup + args.steps + 1
@@ -486,6 +588,9 @@ def main():
     if not args.no_cpu:
         cpu = cpu_baseline(drv, MODEL, page_size, total_pages, args.prompt, tokens[0], args.cpu_seconds)
     drv.close()
+    if not args.no_extra:
+        torch.cuda.empty_cache()
+        extra["other_configs"] = other_configs_extra(drvmod)
 
     out = {
         "metric": "decode tokens/sec @1 GPU + quant-GEMV/attention HBM GB/s as % of 8 TB/s",
@@ -500,7 +605,7 @@ def main():
         "roofline": {"bound": "hbm", "kernel": "gemv_kernel<FmtInt4> (W4A16 weight-streaming GEMV, M=1)",
                      "achieved": round(roof["achieved"], 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(roof["achieved"] / HBM_PEAK_GBPS, 4),
-                     "traffic": GEMV_TRAFFIC_BYTES_PER_LAUNCH,
+                     "traffic": gemv_traffic_bytes_per_launch(),
                      "avg_launch_us": round(roof["avg_us"], 2),
                      "algorithmic_bytes_per_launch": int(roof["bytes_per_launch"]),
                      "launches_timed": roof["launches"]},
