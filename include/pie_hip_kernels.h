@@ -130,6 +130,22 @@ int pie_hip_qkv_rope_fused(int format, const uint16_t* act_bf16, const uint16_t*
                            int pairing, void* stream);
 
 /*
+ * lm_head for greedy decode rows: logits[m, v] = bf16( rmsnorm?(act[m]) . W[v] ) for the bf16
+ * matrix W [V, H], and out_tokens[m] = argmax_v logits[m, v] over the bf16 values (the lowest
+ * index among equals, NaN never wins, an all -inf row gives 0) — pie_hip_linear_fused followed by
+ * pie_hip_argmax, bit for bit, in two launches that read the logits row only once: the GEMV
+ * keeps per-lane (largest value, row) pairs while it stores, a one-block-per-row kernel reduces
+ * them.  M <= 4 (one pass over the weights); workspace of
+ * pie_hip_lm_head_argmax_workspace_bytes(M, V) bytes, need not be cleared.
+ * Reference: lm_head_gemv_argmax_bf16 / _int8 (partial (value, index) pairs per block, then a
+ * reduce), driver/cuda/src/kernels/argmax.cu:795-935.
+ */
+size_t pie_hip_lm_head_argmax_workspace_bytes(int M, int V);
+int pie_hip_lm_head_argmax(const uint16_t* act_bf16, const uint16_t* norm_weight_bf16, float eps,
+                           const uint16_t* w_bf16, uint16_t* logits_bf16, uint32_t* out_tokens, int M,
+                           int V, int H, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * Weight-only GEMM for a handful to a few dozen activation rows on the matrix cores:
  *   y[m, n] = epilogue( sum_k act[m,k] * w(n,k) ), same formats, scales, beta and swiglu
  * contracts as pie_hip_linear_fused (no fused norm); the weights are streamed once per 16

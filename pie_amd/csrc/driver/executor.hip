@@ -204,6 +204,8 @@ Executor::Executor(const DriverConfig& cfg, Model& model) : cfg_(cfg), model_(mo
     logits_ = dmalloc<uint16_t>(srows * m.vocab);
     out_tokens_ = dmalloc<uint32_t>(T);
     out_cap_ = T;
+    amax_ws_bytes_ = pie_hip_lm_head_argmax_workspace_bytes(4, m.vocab);
+    if (amax_ws_bytes_) PIE_HIP_CHECK(hipMalloc(&amax_ws_, amax_ws_bytes_));
     // Bound of the split-K partial buffers over every (rows, context) the planner can pick:
     // rows * splits <= 3072/hk + rows.
     attn_ws_bytes_ = (3072 / static_cast<size_t>(hk) + 1 + T) * hq * (d + 2) * sizeof(float);
@@ -242,7 +244,7 @@ Executor::~Executor() {
     for (void* p : {static_cast<void*>(x_), static_cast<void*>(xn_), static_cast<void*>(qkv_),
                     static_cast<void*>(q_), static_cast<void*>(attn_), static_cast<void*>(gu_),
                     static_cast<void*>(act_), static_cast<void*>(xs_), static_cast<void*>(logits_),
-                    static_cast<void*>(rope_tab_), static_cast<void*>(out_tokens_), attn_ws_, gemm_ws_,
+                    static_cast<void*>(rope_tab_), static_cast<void*>(out_tokens_), attn_ws_, gemm_ws_, amax_ws_,
                     static_cast<void*>(in_dev_), static_cast<void*>(copy_ids_),
                     static_cast<void*>(moe_y_), static_cast<void*>(moe_logits_),
                     static_cast<void*>(moe_idx_), static_cast<void*>(moe_w_),
@@ -462,8 +464,16 @@ void Executor::body(int N, int S, int max_kv_len) {
         head.data = model_.lm_head;
         head.N = m.vocab;
         head.K = H;
-        linear_fused(head, xs_, model_.final_norm, m.rms_eps, logits_, n, 0, 0, xn_, gemm_ws_, gemm_ws_bytes_, s);
-        PIE_KERNEL(pie_hip_argmax(logits_, out_tokens_ + s0, n, m.vocab, s));
+        // up to four rows: the GEMV keeps (largest value, row) pairs while it stores the logits
+        const int fused = n <= 4 ? pie_hip_lm_head_argmax(xs_, model_.final_norm, m.rms_eps, model_.lm_head, logits_,
+                                                          out_tokens_ + s0, n, m.vocab, H, amax_ws_, amax_ws_bytes_, s)
+                                 : PIE_HIP_ERR_UNSUPPORTED;
+        if (fused == PIE_HIP_ERR_UNSUPPORTED) {
+            linear_fused(head, xs_, model_.final_norm, m.rms_eps, logits_, n, 0, 0, xn_, gemm_ws_, gemm_ws_bytes_, s);
+            PIE_KERNEL(pie_hip_argmax(logits_, out_tokens_ + s0, n, m.vocab, s));
+        } else {
+            PIE_KERNEL(fused);
+        }
         if (samp_gather_in_body_) {   // more sampled rows than one chunk: keep each chunk's f32 rows
             const auto* in = static_cast<const unsigned char*>(samp_in_dev_.ptr);
             PIE_KERNEL(pie_hip_sample_gather_logits(

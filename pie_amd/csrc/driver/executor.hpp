@@ -134,6 +134,8 @@ class Executor {
     size_t out_cap_ = 0;   // sampling slots out_tokens_ / out_host_ hold
     void* attn_ws_ = nullptr;
     size_t attn_ws_bytes_ = 0;
+    void* amax_ws_ = nullptr;      // (value, row) pairs of the lm_head GEMV's argmax stage
+    size_t amax_ws_bytes_ = 0;
     void* gemm_ws_ = nullptr;      // split-K partial sums of the tiled GEMM
     size_t gemm_ws_bytes_ = 0;
     uint32_t* copy_ids_ = nullptr;  // staging for page-copy id lists

@@ -262,6 +262,10 @@ struct GemvArgs {
     // qkv epilogue: 1 when the q / k rows were re-ordered at load so that rows (2i, 2i+1) of a
     // head hold the half-split pair (i, i + d/2); the rotated pair goes back to those positions
     int half_out;
+    // lm_head form: when set, every lane that finishes outputs also keeps the largest bf16 value
+    // it stored and its row; slot (m, wave * R + r) of amax_part receives the pair (value bits in
+    // the high word, row in the low word), for a second small kernel to reduce
+    unsigned long long* amax_part;
 };
 
 // ROPE: the q|k|v epilogue (rotation + KV write); its per-lane cos / sin / slot ride with every
@@ -341,6 +345,8 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
     // kUnits work units are requested before the activations are staged and stay in flight
     // from then on.  (Measured: deeper rings than two lose on every decode shape of an 8B
     // model, 1.84 / 1.94 / 2.03 ms per decode step for 2 / 3 / 4 units.)
+    float best_v = -INFINITY;   // lm_head form: largest output of this lane so far, and its row
+    int best_i = 0x7FFFFFFF;
     Unit<R> un[kUnits];
     int ug[kUnits], uc[kUnits];
     int next_g = 0, next_c = 0, issued = 0;
@@ -625,7 +631,15 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
                 if (lane < R * M && row < row_end) {
                     if constexpr (F::kRowScale) mine *= u.rs;
                     const float prev = a.beta ? bf16_bits_to_f32(u.prev) : 0.f;
-                    a.y[static_cast<size_t>(lane % M) * N + row] = f32_to_bf16_bits(mine + prev);
+                    const uint16_t out = f32_to_bf16_bits(mine + prev);
+                    a.y[static_cast<size_t>(lane % M) * N + row] = out;
+                    // (rows ascend inside a lane: a strict comparison keeps the first of equals;
+                    // a NaN never compares greater)
+                    const float ov = bf16_bits_to_f32(out);
+                    if (ov > best_v) {
+                        best_v = ov;
+                        best_i = row;
+                    }
                 }
             }
         }
@@ -641,6 +655,47 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
             issue_next(un[i], ug[i], uc[i]);
         }
     }
+    if (!ROPE && a.amax_part && lane < R * M)
+        a.amax_part[static_cast<size_t>(lane % M) * (total_waves * R) + wg * R + lane / M] =
+            (static_cast<unsigned long long>(__float_as_uint(best_v)) << 32) | static_cast<unsigned>(best_i);
+}
+
+// Second stage of the lm_head form: one block per activation row reduces the per-lane
+// (value, row) pairs; the largest value wins, the lowest row among equals, NaN never
+// (argmax_bf16_kernel, driver/cuda/src/kernels/argmax.cu:36-80).
+__global__ __launch_bounds__(256) void argmax_pairs_kernel(const unsigned long long* __restrict__ part,
+                                                           int count, uint32_t* __restrict__ out) {
+    __shared__ float sv[256 / kWave];
+    __shared__ int si[256 / kWave];
+    const unsigned long long* row = part + static_cast<size_t>(blockIdx.x) * count;
+    float bv = -INFINITY;
+    int bi = 0;
+    auto upd = [&](float v, int i) {
+        if (v > bv || (v == bv && i < bi)) {
+            bv = v;
+            bi = i;
+        }
+    };
+    for (int i = threadIdx.x; i < count; i += blockDim.x) {
+        const unsigned long long e = row[i];
+        upd(__uint_as_float(static_cast<uint32_t>(e >> 32)), static_cast<int>(e & 0xFFFFFFFFull));
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(bv, off, kWave);
+        const int oi = __shfl_xor(bi, off, kWave);
+        upd(ov, oi);
+    }
+    const int lane = threadIdx.x & (kWave - 1), wv = threadIdx.x / kWave;
+    if (lane == 0) {
+        sv[wv] = bv;
+        si[wv] = bi;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 256 / kWave; ++w) upd(sv[w], si[w]);
+        out[blockIdx.x] = static_cast<uint32_t>(bi == 0x7FFFFFFF ? 0 : bi);
+    }
 }
 
 // Optional per-thread event pair that brackets exactly the next GEMV kernel (set by
@@ -648,16 +703,20 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
 thread_local hipEvent_t t_start_event = nullptr;
 thread_local hipEvent_t t_stop_event = nullptr;
 
+// Blocks of a launch: the machine-sized grid, but at least one row (or row pair) per wave.
+int gemv_grid(int N, bool pairs, int waves_per_simd) {
+    int grid = kNumCU * waves_per_simd;
+    const int max_grid = (N / (pairs ? 2 : 1) + kWavesPerBlock - 1) / kWavesPerBlock;
+    return grid > max_grid ? max_grid : grid;
+}
+
 template <class F, int R, int M>
 int launch(const GemvArgs& a, int waves_per_simd, hipStream_t stream) {
     constexpr int kChunkK = kWave * F::WPP;
     const int nchunks = (a.K + kChunkK - 1) / kChunkK;
     const size_t smem = static_cast<size_t>(M) * nchunks * kWave * (F::XV * 16 + 4);
     if (smem > 64 * 1024) return PIE_HIP_ERR_UNSUPPORTED;
-    int grid = kNumCU * waves_per_simd;
-    // >= 1 row (or row pair) per wave
-    const int max_grid = (a.N / ((a.swiglu || a.rope_table) ? 2 : 1) + kWavesPerBlock - 1) / kWavesPerBlock;
-    if (grid > max_grid) grid = max_grid;
+    const int grid = gemv_grid(a.N, a.swiglu || a.rope_table, waves_per_simd);
     if (a.rope_table) {
         if constexpr (R % 2 == 0)
             hipLaunchKernelGGL((gemv_kernel<F, R, M, true>), dim3(grid), dim3(kBlock), smem, stream, a);
@@ -715,7 +774,11 @@ int dispatch(GemvArgs a, int M, int rows_per_wave, int waves_per_simd, hipStream
     uint16_t* y = a.y;
     const float* rope_table = a.rope_table;
     const int64_t* kv_slots = a.kv_slots;
+    unsigned long long* amax_part = a.amax_part;
+    const size_t amax_per_m = static_cast<size_t>(gemv_grid(a.N, a.swiglu || a.rope_table, waves_per_simd)) *
+                              kWavesPerBlock * rows_per_wave;
     for (int m0 = 0; m0 < M; m0 += mcap) {
+        if (amax_part) a.amax_part = amax_part + m0 * amax_per_m;
         const int mm = (M - m0) < mcap ? (M - m0) : mcap;
         a.act = act + static_cast<size_t>(m0) * a.K;
         a.y = y + static_cast<size_t>(m0) * (a.rope_table ? a.hq * a.d : (a.swiglu ? a.N / 2 : a.N));
@@ -795,6 +858,37 @@ extern "C" int pie_hip_gemv_bf16(const uint16_t* act_bf16, const uint16_t* w_bf1
     GemvArgs a{act_bf16, reinterpret_cast<const pie_hip::u32x4_t*>(w_bf16), nullptr, nullptr,
                y_bf16, N, K, 0, beta};
     return pie_hip::dispatch<pie_hip::FmtBf16>(a, M, 0, 0, static_cast<hipStream_t>(stream));
+}
+
+// lm_head with the greedy token in its wake: the bf16 GEMV (final RMSNorm riding in its
+// activation staging) writes the logits and per-lane (largest value, row) pairs; a one-block-per-
+// row kernel reduces the pairs.  Replaces the GEMV followed by a pass over the whole logits row
+// (lm_head_gemv_argmax_bf16, driver/cuda/src/kernels/argmax.cu:795-935: the same two stages).
+extern "C" size_t pie_hip_lm_head_argmax_workspace_bytes(int M, int V) {
+    if (M <= 0 || M > 4 || V <= 0) return 0;
+    return static_cast<size_t>(M) * pie_hip::gemv_grid(V, false, 2) * pie_hip::kWavesPerBlock * 4 * sizeof(unsigned long long);
+}
+
+extern "C" int pie_hip_lm_head_argmax(const uint16_t* act_bf16, const uint16_t* norm_weight_bf16, float eps,
+                                      const uint16_t* w_bf16, uint16_t* logits_bf16, uint32_t* out_tokens,
+                                      int M, int V, int H, void* workspace, size_t workspace_bytes,
+                                      void* stream) {
+    using namespace pie_hip;
+    if (!act_bf16 || !w_bf16 || !logits_bf16 || !out_tokens || !workspace || M <= 0 || V <= 0 || H <= 0)
+        return PIE_HIP_ERR_INVALID;
+    if (M > 4 || V < 4 * kWavesPerBlock) return PIE_HIP_ERR_UNSUPPORTED;   // one weight pass, four rows per wave
+    const size_t need = pie_hip_lm_head_argmax_workspace_bytes(M, V);
+    if (workspace_bytes < need) return PIE_HIP_ERR_INVALID;
+    GemvArgs a{act_bf16, reinterpret_cast<const u32x4_t*>(w_bf16), nullptr, nullptr, logits_bf16, V, H, 0, 0,
+               norm_weight_bf16, eps, 0};
+    a.amax_part = static_cast<unsigned long long*>(workspace);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int rc = dispatch<FmtBf16>(a, M, 4, 2, st);
+    if (rc != PIE_HIP_OK) return rc;
+    const int count = gemv_grid(V, false, 2) * kWavesPerBlock * 4;
+    hipLaunchKernelGGL(argmax_pairs_kernel, dim3(M), dim3(256), 0, st,
+                       static_cast<const unsigned long long*>(workspace), count, out_tokens);
+    return launch_status();
 }
 
 // One entry point for the fused forms the decoder layer uses: optional RMSNorm of the

@@ -316,6 +316,28 @@ def argmax_bf16(logits: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def lm_head_argmax(act: torch.Tensor, w: torch.Tensor, norm_weight: Optional[torch.Tensor] = None,
+                   eps: float = 1e-5):
+    """bf16 lm_head GEMV with the greedy token in its wake (up to four rows).  Returns
+    (logits [M, V] bf16, tokens [M] int32)."""
+    _dev(act, torch.bfloat16, "act")
+    _dev(w, torch.bfloat16, "w")
+    M, H = act.shape
+    V = w.shape[0]
+    if w.shape[1] != H:
+        raise KernelError("shape mismatch")
+    lib = kernels()
+    lib.pie_hip_lm_head_argmax_workspace_bytes.restype = C.c_size_t
+    need = int(lib.pie_hip_lm_head_argmax_workspace_bytes(M, V))
+    ws = torch.empty(max(need, 16), dtype=torch.uint8, device=act.device)
+    logits = torch.empty((M, V), dtype=torch.bfloat16, device=act.device)
+    toks = torch.empty(M, dtype=torch.int32, device=act.device)
+    _check(lib.pie_hip_lm_head_argmax(_ptr(act), _ptr(norm_weight), C.c_float(eps), _ptr(w), _ptr(logits),
+                                      _ptr(toks), M, V, H, _ptr(ws), C.c_size_t(need), _stream()),
+           "pie_hip_lm_head_argmax")
+    return logits, toks
+
+
 def copy_kv_pages(pool: torch.Tensor, srcs: torch.Tensor, dsts: torch.Tensor) -> None:
     """pool[dsts[i]] <- pool[srcs[i]] over the leading (page) dimension."""
     _dev(srcs, torch.int32, "srcs")

@@ -120,3 +120,39 @@ def test_bf16_lm_head_shape_and_greedy_token(gpu, oracle):
     top2 = np.sort(truth[0])[-2:]
     if top2[1] - top2[0] > 2.0 ** -7 * abs(top2[1]):  # not a near-tie at bf16 resolution
         assert tok == int(np.argmax(truth[0]))
+
+
+@pytest.mark.parametrize("M,V,H", [(1, 128256, 2048), (3, 32000, 4096), (4, 5000, 512), (2, 1024, 256)])
+def test_lm_head_with_argmax_equals_gemv_then_argmax(gpu, oracle, M, V, H):
+    """The fused form (GEMV that keeps per-lane (value, row) pairs + a small reduce) returns the
+    bytes of the plain GEMV with the fused norm and the token of the row argmax over them — also
+    with ties (the lowest index wins), a NaN (never wins) and an all -inf row (token 0)."""
+    import torch
+    from pie_amd import ops
+
+    rng = np.random.default_rng(70 + M)
+    w = oracle.f32_to_bf16(rng.standard_normal((V, H)).astype(np.float32) * 0.02)
+    # repeated rows make exact ties among the largest logits likely somewhere
+    w[V // 2] = w[7]
+    w[V - 1] = w[7]
+    act = oracle.f32_to_bf16(rng.standard_normal((M, H)).astype(np.float32))
+    nw = oracle.f32_to_bf16(rng.uniform(0.5, 1.5, H).astype(np.float32))
+    a, wg, nwg = dev(act, gpu, torch.bfloat16), dev(w, gpu, torch.bfloat16), dev(nw, gpu, torch.bfloat16)
+    logits, toks = ops.lm_head_argmax(a, wg, norm_weight=nwg)
+    plain = ops.linear_fused(a, ops.WeightView("bf16", wg, None, 0, V, H), norm_weight=nwg)
+    assert np.array_equal(bits(logits), bits(plain))
+    want = oracle.argmax_bf16(bits(plain))
+    assert np.array_equal(toks.cpu().numpy().astype(np.int64), np.asarray(want).astype(np.int64))
+    assert np.array_equal(toks.cpu().numpy(), ops.argmax_bf16(plain).cpu().numpy())
+    # a row that favours the duplicated weight row: its three copies tie, index 7 wins
+    act2 = np.tile(oracle.bf16_to_f32(w[7])[None, :], (M, 1)) * 8.0
+    a2 = dev(oracle.f32_to_bf16(act2.astype(np.float32)), gpu, torch.bfloat16)
+    lg2, tk2 = ops.lm_head_argmax(a2, wg)
+    l2 = oracle.bf16_to_f32(bits(lg2))
+    assert np.all(l2[:, 7] == l2[:, V // 2]) and np.all(l2[:, 7] == l2[:, V - 1])
+    assert np.all(tk2.cpu().numpy() == np.argmax(l2, axis=1)) and np.all(np.argmax(l2, axis=1) == 7)
+    # NaN activations: every logit NaN -> token 0 (nothing compares greater); inf weights: -inf rows
+    a3 = a.clone()
+    a3[0, :] = float("nan")
+    _, tk3 = ops.lm_head_argmax(a3, wg)
+    assert int(tk3[0]) == int(ops.argmax_bf16(ops.gemv_bf16(a3, wg))[0])
