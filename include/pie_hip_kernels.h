@@ -472,21 +472,22 @@ int pie_hip_attn_rows_paged_static(const uint16_t* q, const uint16_t* k_pages,
  * KV-cache storage formats of the pool (the CUDA driver's kv_cache_dtype values,
  * driver/cuda/src/kv_cache_format.cpp:46-110).  One-byte formats keep the bf16 layout
  * [pages, page_size, hk, d] with one byte per element; the per-token-head formats add fp32 side
- * scales [pages, page_size, hk] for K and for V.  fp8_e5m2 and the fp4 block formats are not
- * implemented (PIE_HIP_ERR_UNSUPPORTED).
+ * scales [pages, page_size, hk] for K and for V.  The fp4 block formats are not implemented
+ * (PIE_HIP_ERR_UNSUPPORTED).
  */
 enum {
     PIE_HIP_KV_BF16 = 0,
     PIE_HIP_KV_FP8_E4M3 = 1,             /* saturating cast of the value, no scales */
     PIE_HIP_KV_INT8_PER_TOKEN_HEAD = 2,  /* scale = absmax/127, code = rint(x / scale) */
-    PIE_HIP_KV_FP8_PER_TOKEN_HEAD = 3    /* scale = absmax/448, code = e4m3(x / scale) */
+    PIE_HIP_KV_FP8_PER_TOKEN_HEAD = 3,   /* scale = absmax/448, code = e4m3(x / scale) */
+    PIE_HIP_KV_FP8_E5M2 = 4              /* saturating e5m2 cast of the value, no scales */
 };
 
 /*
  * pie_hip_attn_rows_paged over a pool in a one-byte format: every K / V element is
  * float(code) * scale as load_kv_scalar reads it (driver/cuda/src/ops/attention_naive_paged.cu:56-112),
  * everything else as for bf16 pools.  k_scales / v_scales: required for the per-token-head
- * formats, NULL for PIE_HIP_KV_FP8_E4M3.  Custom masks are not available with these formats.
+ * formats, NULL for PIE_HIP_KV_FP8_E4M3 and PIE_HIP_KV_FP8_E5M2.  Custom masks are not available with these formats.
  */
 int pie_hip_attn_rows_paged_kvq(int kv_format, const uint16_t* q, const void* k_pages,
                                 const void* v_pages, const float* k_scales, const float* v_scales,
@@ -511,7 +512,8 @@ int pie_hip_attn_rows_paged_kvq_masked(int kv_format, const uint16_t* q, const v
  * Quantising KV write: this step's K and V rows [num_tokens, hk, d] bf16 (after RoPE) go to
  * slot kv_slots[t] of a one-byte pool (slot < 0: skipped).  Per-token-head formats:
  * scale = absmax / qmax (qmax 127 / 448; 1 for an all-zero row), code = x * (1/scale) rounded
- * to nearest even, clamped / saturated; PIE_HIP_KV_FP8_E4M3: the saturating cast of x.
+ * to nearest even, clamped / saturated; PIE_HIP_KV_FP8_E4M3 / _E5M2: the saturating cast of x
+ * (largest finite value 448 / 57344).
  * Reference: write_kv_per_token_head_kernel and write_kv_fp8_per_tensor_kernel,
  * driver/cuda/src/kernels/kv_paged.cu:155-297.
  */

@@ -328,7 +328,7 @@ def brle_allow(runs, pos: int, n_kv: int, window: int = 0) -> np.ndarray:
     return out[:n_kv]
 
 
-KV_FORMATS = {"bf16": 0, "fp8_e4m3": 1, "int8_per_token_head": 2, "fp8_per_token_head": 3}
+KV_FORMATS = {"bf16": 0, "fp8_e4m3": 1, "int8_per_token_head": 2, "fp8_per_token_head": 3, "fp8_e5m2": 4}
 
 
 def kv_quant_rows(x_bf16, fmt: str):
@@ -342,7 +342,7 @@ def kv_quant_rows(x_bf16, fmt: str):
     deq = np.zeros((rows, d), np.float32)
     lib().orc_kv_quant_rows(_p(x), _p(codes), _p(scales), _p(deq), C.c_int(rows), C.c_int(d),
                             C.c_int(KV_FORMATS[fmt]))
-    return codes, (None if fmt == "fp8_e4m3" else scales), deq
+    return codes, (None if fmt in ("fp8_e4m3", "fp8_e5m2") else scales), deq
 
 
 def attn_rows_f32kv(q_bf16, k_pages_f32, v_pages_f32, page_indices, row_begin, row_len, hq, hk, d, ps,

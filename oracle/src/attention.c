@@ -261,16 +261,55 @@ void orc_attn_rows_f32kv(const uint16_t* q, const float* k_pages, const float* v
  *   fmt 2 (int8_per_token_head): scale = absmax/127 (1 when absmax == 0), inv = 1/scale,
  *                                code = clamp(rintf(x * inv), -128, 127)
  *   fmt 3 (fp8_per_token_head):  scale = absmax/448 (1 when 0), code = e4m3_satfinite(x * inv)
+ *   fmt 4 (fp8_e5m2):            code = e5m2_satfinite(x); scales untouched
  * dequant (optional, f32): float(code) * scale, as the attention kernels read it.
  */
 uint8_t orc_f32_to_fp8_e4m3(float f);
 float orc_fp8_e4m3_to_f32(uint8_t v);
+
+/* e5m2 byte -> f32: the byte is the high half of an IEEE binary16 (1-5-2). */
+float orc_fp8_e5m2_to_f32(uint8_t v) {
+    const int sign = v >> 7, e = (v >> 2) & 0x1F, m = v & 3;
+    float r;
+    if (e == 0) r = ldexpf((float)m, -16);                 /* subnormals: m * 2^-16 */
+    else if (e == 31) r = m ? NAN : INFINITY;
+    else r = ldexpf(1.f + (float)m / 4.f, e - 15);
+    return sign ? -r : r;
+}
+
+/* f32 -> e5m2, round to nearest even, saturating to +-57344 (__NV_SATFINITE); NaN -> 0x7F.
+ * Nearest of the two neighbouring codes, the even code on a tie — found by search over the 124
+ * finite magnitudes, so the rule is the definition itself. */
+uint8_t orc_f32_to_fp8_e5m2(float f) {
+    if (f != f) return 0x7F;
+    const uint8_t sign = signbit(f) ? 0x80 : 0;
+    const float a = fabsf(f);
+    if (a >= 57344.f) return (uint8_t)(sign | 0x7B);
+    int best = 0;
+    float best_err = a;
+    for (int c = 1; c <= 0x7B; ++c) {
+        const float err = fabsf(orc_fp8_e5m2_to_f32((uint8_t)c) - a);
+        if (err < best_err || (err == best_err && (c & 1) == 0)) {
+            best = c;
+            best_err = err;
+        }
+    }
+    return (uint8_t)(sign | best);
+}
+
+void orc_fp8_e5m2_decode(const uint8_t* src, float* dst, size_t n) {
+    for (size_t i = 0; i < n; ++i) dst[i] = orc_fp8_e5m2_to_f32(src[i]);
+}
+void orc_fp8_e5m2_encode(const float* src, uint8_t* dst, size_t n) {
+    for (size_t i = 0; i < n; ++i) dst[i] = orc_f32_to_fp8_e5m2(src[i]);
+}
+
 void orc_kv_quant_rows(const uint16_t* x, uint8_t* codes, float* scales, float* dequant, int rows,
                        int d, int fmt) {
     for (int r = 0; r < rows; ++r) {
         const uint16_t* src = x + (size_t)r * d;
         float scale = 1.f, inv = 1.f;
-        if (fmt != 1) {
+        if (fmt != 1 && fmt != 4) {
             float amax = 0.f;
             for (int j = 0; j < d; ++j) amax = fmaxf(amax, fabsf(orc_bf16_to_f32(src[j])));
             scale = amax > 0.f ? amax / (fmt == 2 ? 127.f : 448.f) : 1.f;
@@ -285,6 +324,10 @@ void orc_kv_quant_rows(const uint16_t* x, uint8_t* codes, float* scales, float* 
                 qv = qv > 127 ? 127 : (qv < -128 ? -128 : qv);
                 codes[(size_t)r * d + j] = (uint8_t)(int8_t)qv;
                 val = (float)qv;
+            } else if (fmt == 4) {
+                const uint8_t c = orc_f32_to_fp8_e5m2(f);
+                codes[(size_t)r * d + j] = c;
+                val = orc_fp8_e5m2_to_f32(c);
             } else {
                 const uint8_t c = orc_f32_to_fp8_e4m3(f);
                 codes[(size_t)r * d + j] = c;

@@ -858,7 +858,7 @@ int attn_dispatch(const uint16_t* q, const void* k_pages, const void* v_pages, u
     // absent for plain fp8 casts
     if (kv_format != PIE_HIP_KV_BF16) {
         const bool scaled = kv_format == PIE_HIP_KV_INT8_PER_TOKEN_HEAD || kv_format == PIE_HIP_KV_FP8_PER_TOKEN_HEAD;
-        if (kv_format != PIE_HIP_KV_FP8_E4M3 && !scaled) return PIE_HIP_ERR_UNSUPPORTED;
+        if (kv_format != PIE_HIP_KV_FP8_E4M3 && kv_format != PIE_HIP_KV_FP8_E5M2 && !scaled) return PIE_HIP_ERR_UNSUPPORTED;
         if (scaled != (k_scales != nullptr) || scaled != (v_scales != nullptr)) return PIE_HIP_ERR_INVALID;
     }
 #define PIE_ATTN_CASE(DD, GG)                                                                  \
@@ -871,6 +871,18 @@ int attn_dispatch(const uint16_t* q, const void* k_pages, const void* v_pages, u
                 mask_bits, mask_stride, st);                                                   \
         if (kv_format == PIE_HIP_KV_INT8_PER_TOKEN_HEAD)                                       \
             return launch_decode<DD, GG, false, kKvInt8>(                                      \
+                q, k_pages, v_pages, k_scales, v_scales, o, lse, kv_page_indices,              \
+                kv_page_indptr, kv_last_page_lens, row_begin, row_len, num_rows, num_q_heads,  \
+                num_kv_heads, page_size, scale, max_kv_len, workspace, workspace_bytes,        \
+                nullptr, 0, st);                                                               \
+        if (kv_format == PIE_HIP_KV_FP8_E5M2 && mask_bits)                                     \
+            return launch_decode<DD, GG, true, kKvBf8>(                                        \
+                q, k_pages, v_pages, k_scales, v_scales, o, lse, kv_page_indices,              \
+                kv_page_indptr, kv_last_page_lens, row_begin, row_len, num_rows, num_q_heads,  \
+                num_kv_heads, page_size, scale, max_kv_len, workspace, workspace_bytes,        \
+                mask_bits, mask_stride, st);                                                   \
+        if (kv_format == PIE_HIP_KV_FP8_E5M2)                                                  \
+            return launch_decode<DD, GG, false, kKvBf8>(                                       \
                 q, k_pages, v_pages, k_scales, v_scales, o, lse, kv_page_indices,              \
                 kv_page_indptr, kv_last_page_lens, row_begin, row_len, num_rows, num_q_heads,  \
                 num_kv_heads, page_size, scale, max_kv_len, workspace, workspace_bytes,        \
@@ -1051,6 +1063,13 @@ namespace {
 // e4m3: saturating at 448); plain fp8: the saturating cast of x itself.  The arithmetic of
 // write_kv_per_token_head_kernel / write_kv_fp8_per_tensor_kernel,
 // driver/cuda/src/kernels/kv_paged.cu:155-297.
+// f32 -> e5m2 byte, round to nearest even, saturating at the largest finite value (57344), as
+// __nv_cvt_float_to_fp8(x, __NV_SATFINITE, __NV_E5M2) (driver/cuda/src/kernels/kv_paged.cu:181-184).
+__device__ __forceinline__ unsigned char f32_to_e5m2_sat(float f) {
+    const float c = fminf(fmaxf(f, -57344.f), 57344.f);
+    return static_cast<unsigned char>(__builtin_amdgcn_cvt_pk_bf8_f32(c, c, 0, false) & 0xFF);
+}
+
 __global__ __launch_bounds__(256) void kv_write_quant_kernel(
     const uint16_t* __restrict__ k_src, const uint16_t* __restrict__ v_src,
     const int64_t* __restrict__ kv_slots, unsigned char* __restrict__ k_pages,
@@ -1064,7 +1083,7 @@ __global__ __launch_bounds__(256) void kv_write_quant_kernel(
     if (slot < 0) return;
     const size_t src = static_cast<size_t>(row) * d;
     const size_t th = static_cast<size_t>(slot) * hk + h;
-    const bool scaled = kv_format != PIE_HIP_KV_FP8_E4M3;
+    const bool scaled = kv_format != PIE_HIP_KV_FP8_E4M3 && kv_format != PIE_HIP_KV_FP8_E5M2;
     const float qmax = kv_format == PIE_HIP_KV_INT8_PER_TOKEN_HEAD ? 127.f : 448.f;
 #pragma unroll
     for (int which = 0; which < 2; ++which) {
@@ -1085,6 +1104,8 @@ __global__ __launch_bounds__(256) void kv_write_quant_kernel(
                 int qv = static_cast<int>(rintf(f));
                 qv = qv > 127 ? 127 : (qv < -128 ? -128 : qv);
                 dst[j] = static_cast<unsigned char>(static_cast<int8_t>(qv));
+            } else if (kv_format == PIE_HIP_KV_FP8_E5M2) {
+                dst[j] = f32_to_e5m2_sat(f);
             } else {
                 const float c = fminf(fmaxf(f, -448.f), 448.f);
                 dst[j] = static_cast<unsigned char>(__builtin_amdgcn_cvt_pk_fp8_f32(c, c, 0, false) & 0xFF);
@@ -1159,7 +1180,7 @@ __global__ __launch_bounds__(64) void qkv_rope_kvwrite_quant_kernel(
     const int h = is_k ? head - hq : head - hq - hk;
     const size_t th = static_cast<size_t>(slot) * hk + h;
     unsigned char* dst = (is_k ? k_pages : v_pages) + th * d;
-    const bool scaled = kv_format != PIE_HIP_KV_FP8_E4M3;
+    const bool scaled = kv_format != PIE_HIP_KV_FP8_E4M3 && kv_format != PIE_HIP_KV_FP8_E5M2;
     const float qmax = kv_format == PIE_HIP_KV_INT8_PER_TOKEN_HEAD ? 127.f : 448.f;
     float inv = 1.f;
     if (scaled) {
@@ -1178,6 +1199,7 @@ __global__ __launch_bounds__(64) void qkv_rope_kvwrite_quant_kernel(
             qv = qv > 127 ? 127 : (qv < -128 ? -128 : qv);
             return static_cast<unsigned char>(static_cast<int8_t>(qv));
         }
+        if (kv_format == PIE_HIP_KV_FP8_E5M2) return f32_to_e5m2_sat(f);
         const float c = fminf(fmaxf(f, -448.f), 448.f);
         return static_cast<unsigned char>(__builtin_amdgcn_cvt_pk_fp8_f32(c, c, 0, false) & 0xFF);
     };
@@ -1208,7 +1230,7 @@ extern "C" int pie_hip_qkv_rope_kvwrite_quant(int kv_format, const uint16_t* pac
         return PIE_HIP_ERR_INVALID;
     if (!q_norm_weight != !k_norm_weight) return PIE_HIP_ERR_INVALID;
     const bool scaled = kv_format == PIE_HIP_KV_INT8_PER_TOKEN_HEAD || kv_format == PIE_HIP_KV_FP8_PER_TOKEN_HEAD;
-    if (kv_format != PIE_HIP_KV_FP8_E4M3 && !scaled) return PIE_HIP_ERR_UNSUPPORTED;
+    if (kv_format != PIE_HIP_KV_FP8_E4M3 && kv_format != PIE_HIP_KV_FP8_E5M2 && !scaled) return PIE_HIP_ERR_UNSUPPORTED;
     if (scaled && (!k_scales || !v_scales)) return PIE_HIP_ERR_INVALID;
     if (head_dim % 8 != 0 || head_dim > 256 || num_q_heads + 2 * num_kv_heads > 65535) return PIE_HIP_ERR_UNSUPPORTED;
     const dim3 grid(num_tokens, num_q_heads + 2 * num_kv_heads);
@@ -1235,7 +1257,7 @@ extern "C" int pie_hip_kv_write_quant(int kv_format, const uint16_t* k_rows, con
         head_dim <= 0)
         return PIE_HIP_ERR_INVALID;
     const bool scaled = kv_format == PIE_HIP_KV_INT8_PER_TOKEN_HEAD || kv_format == PIE_HIP_KV_FP8_PER_TOKEN_HEAD;
-    if (kv_format != PIE_HIP_KV_FP8_E4M3 && !scaled) return PIE_HIP_ERR_UNSUPPORTED;
+    if (kv_format != PIE_HIP_KV_FP8_E4M3 && kv_format != PIE_HIP_KV_FP8_E5M2 && !scaled) return PIE_HIP_ERR_UNSUPPORTED;
     if (scaled && (!k_scales || !v_scales)) return PIE_HIP_ERR_INVALID;
     if (num_tokens == 0) return PIE_HIP_OK;
     const int rows = num_tokens * num_kv_heads;

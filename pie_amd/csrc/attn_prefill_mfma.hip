@@ -17,8 +17,8 @@
 // [4g..4g+3, 16+4g..16+4g+3] per 16-lane group g, which is the order V^T is laid out in LDS.
 // K rows are padded to 272 B and V^T rows to 80 B: every 16-byte operand read of 16 lanes
 // touches 64 distinct banks.  The next step's K/V are requested from HBM before the current
-// step is multiplied.  Probabilities are rounded to bf16 for the second product (fp32
-// accumulators), and the normaliser sums those rounded values.
+// step is multiplied.  Probabilities enter the second product as a hi + lo pair of bf16 values
+// (fp32 accumulators), and the normaliser sums the unrounded values.
 #include "common.hip.h"
 
 namespace pie_hip {
@@ -255,7 +255,7 @@ __global__ __launch_bounds__(kTileThreads) void attn_prefill_tile_kernel(
             }
         }
         // online softmax per query (= per lane%16); the 8 keys of this lane: 16nt + 4g + r
-        bf16x8_t pf[QT];
+        bf16x8_t pf_hi[QT], pf_lo[QT];
 #pragma unroll
         for (int qt = 0; qt < QT; ++qt) {
             float s[8];
@@ -275,26 +275,27 @@ __global__ __launch_bounds__(kTileThreads) void attn_prefill_tile_kernel(
             const float safe = m_new == -INFINITY ? 0.f : m_new;
             const float alpha = exp2f(mx[qt] - safe);
             mx[qt] = m_new;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) s[e] = exp2f(s[e] - safe);
-            const u32x4_t packed = {pack_bf16x2(s[0], s[1]), pack_bf16x2(s[2], s[3]),
-                                    pack_bf16x2(s[4], s[5]), pack_bf16x2(s[6], s[7])};
-            if constexpr (Q8) {
-                // V = float(code) * scale: the rounded weight times the key's scale multiplies the codes
-                const u32x4_t scaled = {
-                    pack_bf16x2(bf16_lo(packed[0]) * vsc[0][0], bf16_hi(packed[0]) * vsc[0][1]),
-                    pack_bf16x2(bf16_lo(packed[1]) * vsc[0][2], bf16_hi(packed[1]) * vsc[0][3]),
-                    pack_bf16x2(bf16_lo(packed[2]) * vsc[1][0], bf16_hi(packed[2]) * vsc[1][1]),
-                    pack_bf16x2(bf16_lo(packed[3]) * vsc[1][2], bf16_hi(packed[3]) * vsc[1][3])};
-                pf[qt] = __builtin_bit_cast(bf16x8_t, scaled);
-            } else {
-                pf[qt] = __builtin_bit_cast(bf16x8_t, packed);
-            }
-            // the normaliser sums the rounded weights, the ones that multiply V: the output stays
-            // an exact weighted mean of V rows
+            // The weights reach the second product as hi + lo with both parts bf16 (hi by
+            // truncation, lo = bf16(p - hi)): 16 significant bits, so P . V keeps the accuracy of
+            // fp32 weights (the reference multiplies fp32 probabilities,
+            // driver/cuda/src/ops/attention_naive_paged.cu:148-317), and the normaliser sums the
+            // unrounded values, as the decode kernel does.
             float sum = 0.f;
+            uint32_t hi[4], lo[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) sum += bf16_lo(packed[e]) + bf16_hi(packed[e]);
+            for (int e = 0; e < 8; e += 2) {
+                float p0 = exp2f(s[e] - safe), p1 = exp2f(s[e + 1] - safe);
+                sum += p0 + p1;
+                if constexpr (Q8) {   // V = float(code) * scale: the scale rides on the weight
+                    p0 *= vsc[e >> 2][e & 3];
+                    p1 *= vsc[e >> 2][(e & 3) + 1];
+                }
+                const uint32_t b0 = __float_as_uint(p0) & 0xFFFF0000u, b1 = __float_as_uint(p1) & 0xFFFF0000u;
+                hi[e >> 1] = (b0 >> 16) | b1;
+                lo[e >> 1] = pack_bf16x2(p0 - __uint_as_float(b0), p1 - __uint_as_float(b1));
+            }
+            pf_hi[qt] = __builtin_bit_cast(bf16x8_t, u32x4_t{hi[0], hi[1], hi[2], hi[3]});
+            pf_lo[qt] = __builtin_bit_cast(bf16x8_t, u32x4_t{lo[0], lo[1], lo[2], lo[3]});
             lsum[qt] = lsum[qt] * alpha + sum;
             if (alpha != 1.0f) {
 #pragma unroll
@@ -307,8 +308,10 @@ __global__ __launch_bounds__(kTileThreads) void attn_prefill_tile_kernel(
             const bf16x8_t vf = __builtin_bit_cast(
                 bf16x8_t, *reinterpret_cast<const u32x4_t*>(&Vt[(16 * dt + l16) * kVtStride + 8 * g]));
 #pragma unroll
-            for (int qt = 0; qt < QT; ++qt)
-                acc[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[qt], acc[qt][dt], 0, 0, 0);
+            for (int qt = 0; qt < QT; ++qt) {
+                acc[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf_hi[qt], acc[qt][dt], 0, 0, 0);
+                acc[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf_lo[qt], acc[qt][dt], 0, 0, 0);
+            }
         }
     };
 
@@ -354,6 +357,10 @@ int launch_tiles(int kv_format, const uint16_t* q, const void* k_pages, const vo
         hipLaunchKernelGGL((attn_prefill_tile_kernel<D, GQA, QT, kKvInt8>), grid, dim3(kTileThreads), 0, stream, q,
                            k_pages, v_pages, k_scales, v_scales, o, page_indices, row_begin, row_len,
                            tile_start, tile_rows, hq, hk, ps, sl);
+    else if (kv_format == PIE_HIP_KV_FP8_E5M2)
+        hipLaunchKernelGGL((attn_prefill_tile_kernel<D, GQA, QT, kKvBf8>), grid, dim3(kTileThreads), 0, stream, q,
+                           k_pages, v_pages, k_scales, v_scales, o, page_indices, row_begin, row_len,
+                           tile_start, tile_rows, hq, hk, ps, sl);
     else
         hipLaunchKernelGGL((attn_prefill_tile_kernel<D, GQA, QT, kKvFp8>), grid, dim3(kTileThreads), 0, stream, q,
                            k_pages, v_pages, k_scales, v_scales, o, page_indices, row_begin, row_len,
@@ -386,7 +393,8 @@ extern "C" int pie_hip_attn_prefill_tiles_kvq(int kv_format, const uint16_t* q, 
         return PIE_HIP_ERR_INVALID;
     {
         const bool scaled = kv_format == PIE_HIP_KV_INT8_PER_TOKEN_HEAD || kv_format == PIE_HIP_KV_FP8_PER_TOKEN_HEAD;
-        if (kv_format != PIE_HIP_KV_BF16 && kv_format != PIE_HIP_KV_FP8_E4M3 && !scaled) return PIE_HIP_ERR_UNSUPPORTED;
+        if (kv_format != PIE_HIP_KV_BF16 && kv_format != PIE_HIP_KV_FP8_E4M3 && kv_format != PIE_HIP_KV_FP8_E5M2 && !scaled)
+            return PIE_HIP_ERR_UNSUPPORTED;
         if (scaled != (k_scales != nullptr) || scaled != (v_scales != nullptr)) return PIE_HIP_ERR_INVALID;
     }
     const int cap = pie_hip_attn_prefill_tile_rows(num_q_heads, num_kv_heads);

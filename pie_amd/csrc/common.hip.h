@@ -116,10 +116,10 @@ __device__ __forceinline__ float wave_max(float v) {
 
 // KV storage of the pool (driver/cuda/src/kv_cache_format.hpp:11-17): bf16; one-byte e4m3 with
 // optional fp32 scales per (token, kv head) — "fp8_e4m3" stores casts, "fp8_per_token_head"
-// stores x / scale; int8 with such scales.  A lane still owns 8 elements of a row: 16 bytes of
+// stores x / scale; int8 with such scales; one-byte e5m2 casts ("fp8_e5m2").  A lane still owns 8 elements of a row: 16 bytes of
 // bf16 or 8 bytes of a one-byte format.  Values are decoded as the reference's load_kv_scalar
 // does (driver/cuda/src/ops/attention_naive_paged.cu:56-112): float(code) * scale.
-constexpr int kKvBf16 = 0, kKvFp8 = 1, kKvInt8 = 2;
+constexpr int kKvBf16 = 0, kKvFp8 = 1, kKvInt8 = 2, kKvBf8 = 3;   // (kKvBf8: e5m2 casts, "fp8_e5m2")
 
 template <int KVF>
 struct KvVec {
@@ -131,6 +131,10 @@ struct KvVec<kKvFp8> {
 };
 template <>
 struct KvVec<kKvInt8> {
+    using type = u32x2_t;
+};
+template <>
+struct KvVec<kKvBf8> {
     using type = u32x2_t;
 };
 
@@ -147,6 +151,11 @@ __device__ __forceinline__ void kv_decode_f32(const typename KvVec<KVF>::type r,
         typedef float f32x2_t __attribute__((ext_vector_type(2)));
         const f32x2_t a = __builtin_amdgcn_cvt_pk_f32_fp8(r.x, false), b = __builtin_amdgcn_cvt_pk_f32_fp8(r.x, true);
         const f32x2_t c = __builtin_amdgcn_cvt_pk_f32_fp8(r.y, false), d = __builtin_amdgcn_cvt_pk_f32_fp8(r.y, true);
+        f[0] = a.x; f[1] = a.y; f[2] = b.x; f[3] = b.y; f[4] = c.x; f[5] = c.y; f[6] = d.x; f[7] = d.y;
+    } else if constexpr (KVF == kKvBf8) {
+        typedef float f32x2_t __attribute__((ext_vector_type(2)));
+        const f32x2_t a = __builtin_amdgcn_cvt_pk_f32_bf8(r.x, false), b = __builtin_amdgcn_cvt_pk_f32_bf8(r.x, true);
+        const f32x2_t c = __builtin_amdgcn_cvt_pk_f32_bf8(r.y, false), d = __builtin_amdgcn_cvt_pk_f32_bf8(r.y, true);
         f[0] = a.x; f[1] = a.y; f[2] = b.x; f[3] = b.y; f[4] = c.x; f[5] = c.y; f[6] = d.x; f[7] = d.y;
     } else {
 #pragma unroll

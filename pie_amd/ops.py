@@ -814,7 +814,7 @@ def attention_prefill_tiles(q: torch.Tensor, k_pages: torch.Tensor, v_pages: tor
     return o
 
 
-KV_FORMATS = {"bf16": 0, "fp8_e4m3": 1, "int8_per_token_head": 2, "fp8_per_token_head": 3}
+KV_FORMATS = {"bf16": 0, "fp8_e4m3": 1, "int8_per_token_head": 2, "fp8_per_token_head": 3, "fp8_e5m2": 4}
 
 
 def attention_prefill_tiles_kvq(fmt: str, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,

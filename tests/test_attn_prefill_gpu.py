@@ -52,26 +52,27 @@ def test_tiles_match_oracle_and_row_kernel(gpu, oracle, hq, hk, d, ps, half):
     got = oracle.bf16_to_f32(got_bits).astype(np.float64)
     truth, _, _ = oracle.attn_rows_masked(q, b["k_pages"], b["v_pages"], b["page_indices"], row_begin,
                                           row_len, hq, hk, d, ps, [None] * rows)
-    # one bf16 rounding of the output + softmax weights rounded to bf16 (2^-9 relative each,
-    # against V ~ N(0, 1))
-    tol = 2.0 ** -8 * np.maximum(np.abs(truth), np.abs(got)) + 4e-3
+    # one bf16 rounding of the output + fp32 softmax / accumulation error: the decode kernels' bar
+    # (the weights reach the second product as hi + lo bf16 pairs, 16 significant bits)
+    tol = 2.0 ** -8 * np.maximum(np.abs(truth), np.abs(got)) + 1e-4
     err = np.abs(got - truth)
     assert np.all(err <= tol), f"worst {np.max(err / tol):.2f}x tol at {np.unravel_index(np.argmax(err / tol), err.shape)}"
     row = ops.attention_rows_paged(*args, int(row_len.max())).view(torch.uint16).cpu().numpy()
     # against the per-row kernel (fp32 weights): the same bar, and mostly the same bf16 value
     # (ulp distances grow without bound for outputs near zero, so they are only counted)
     rowf = oracle.bf16_to_f32(row).astype(np.float64)
-    assert np.all(np.abs(got - rowf) <= 2.0 ** -7 * np.maximum(np.abs(rowf), np.abs(got)) + 8e-3)
+    assert np.all(np.abs(got - rowf) <= 2.0 ** -7 * np.maximum(np.abs(rowf), np.abs(got)) + 2e-4)
     ulp = np.abs(got_bits.astype(np.int32) - row.astype(np.int32))
-    assert (ulp <= 1).mean() > 0.85
+    assert (ulp <= 1).mean() > 0.97
 
 
-@pytest.mark.parametrize("fmt", ["fp8_e4m3", "int8_per_token_head", "fp8_per_token_head"])
+@pytest.mark.parametrize("fmt", ["fp8_e4m3", "int8_per_token_head", "fp8_per_token_head", "fp8_e5m2"])
 @pytest.mark.parametrize("hq,hk,d,ps", [(8, 2, 128, 16), (4, 4, 64, 16), (32, 8, 128, 32)])
-def test_tiles_over_one_byte_pools_match_the_row_kernel(gpu, oracle, fmt, hq, hk, d, ps):
-    """The tile kernel over quantised pools against the per-row kernel over the same pools (itself
-    held to the oracle in test_kv_quant_gpu.py): same codes, same scales, probabilities rounded to
-    bf16 in the tile kernel only."""
+def test_tiles_over_one_byte_pools_match_the_oracle(gpu, oracle, fmt, hq, hk, d, ps):
+    """The tile kernel over quantised pools against the oracle's attention over the dequantised
+    values float(code) * scale (codes and scales written by the library's quantising write,
+    itself bit-exact against the oracle's quantiser), to the bar of the bf16 pools; the per-row
+    kernel over the same pools is compared as well."""
     import torch
 
     from pie_amd import ops
@@ -90,7 +91,7 @@ def test_tiles_over_one_byte_pools_match_the_row_kernel(gpu, oracle, fmt, hq, hk
     pages = b["k_pages"].shape[0]
     kp = torch.zeros((pages, ps, hk, d), dtype=torch.uint8, device=gpu)
     vp = torch.zeros_like(kp)
-    scaled = fmt != "fp8_e4m3"
+    scaled = fmt not in ("fp8_e4m3", "fp8_e5m2")
     ks = torch.ones((pages, ps, hk), dtype=torch.float32, device=gpu) if scaled else None
     vs = torch.ones((pages, ps, hk), dtype=torch.float32, device=gpu) if scaled else None
     slots = dev(np.arange(pages * ps, dtype=np.int64))
@@ -102,8 +103,18 @@ def test_tiles_over_one_byte_pools_match_the_row_kernel(gpu, oracle, fmt, hq, hk
     ref = ops.attention_rows_paged_kvq(fmt, qd, kp, vp, ks, vs, pi, rb, rl)[0]
     torch.cuda.synchronize()
     got = oracle.bf16_to_f32(o.view(torch.uint16).cpu().numpy()).astype(np.float64)
-    want = oracle.bf16_to_f32(ref.view(torch.uint16).cpu().numpy()).astype(np.float64)
-    tol = 2.0 ** -7 * np.maximum(np.abs(want), np.abs(got)) + 6e-3
-    err = np.abs(got - want)
+    # the oracle: its own quantiser on the same bf16 rows (the codes the GPU wrote, bit for bit),
+    # attention in double over float(code) * scale
+    deq = {}
+    for name in ("k_pages", "v_pages"):
+        codes, scales, dq = oracle.kv_quant_rows(b[name].reshape(pages * ps * hk, d), fmt)
+        deq[name] = dq.reshape(pages, ps, hk, d)
+        pool = (kp if name == "k_pages" else vp).cpu().numpy()
+        assert np.array_equal(pool.reshape(-1, d), codes)
+    truth, _, _ = oracle.attn_rows_f32kv(q, deq["k_pages"], deq["v_pages"], b["page_indices"], row_begin, row_len,
+                                         hq, hk, d, ps, mode=2)
+    tol = 2.0 ** -8 * np.maximum(np.abs(truth), np.abs(got)) + 1e-4
+    err = np.abs(got - truth)
     assert np.all(err <= tol), f"worst {np.max(err / tol):.2f}x tol"
-    assert np.linalg.norm(got - want) <= 4e-3 * np.linalg.norm(want)
+    want = oracle.bf16_to_f32(ref.view(torch.uint16).cpu().numpy()).astype(np.float64)
+    assert np.all(np.abs(got - want) <= 2.0 ** -7 * np.maximum(np.abs(want), np.abs(got)) + 2e-4)

@@ -409,7 +409,7 @@ def test_host_swap_pool_round_trip(gpu, oracle):
             assert d.handle(drvmod.copy_frame(direction, [0], [0])).payload.status.status == 4
 
 
-KV_FORMATS = ["fp8_e4m3", "int8_per_token_head", "fp8_per_token_head"]
+KV_FORMATS = ["fp8_e4m3", "int8_per_token_head", "fp8_per_token_head", "fp8_e5m2"]
 
 
 @pytest.mark.parametrize("kv_dtype", KV_FORMATS)
@@ -436,8 +436,11 @@ def test_generation_with_one_byte_kv_cache_matches_oracle(gpu, oracle, kw, kv_dt
     prompts = ragged_prompts(rng, cfg["vocab"], 37, 2)
     with drvmod.Driver(toml_config(**kw)) as d:
         om, _ = oracle_model_from_driver(d, cfg)
-        otoks, near, checks = teacher_forced_compare(oracle, drvmod, d, om, cfg, prompts, 8, cos_min=0.998,
-                                                     rel=0.1, tie=2.0 ** -4)
+        # (e5m2 keeps two mantissa bits: a code step is twice as coarse, 12-25 % of the element,
+        # so 1 - cosine — quadratic in the deviation — gets four times e4m3's allowance)
+        bars = dict(cos_min=0.992, rel=0.2, tie=2.0 ** -3) if kv_dtype == "fp8_e5m2" else \
+            dict(cos_min=0.998, rel=0.1, tie=2.0 ** -4)
+        otoks, near, checks = teacher_forced_compare(oracle, drvmod, d, om, cfg, prompts, 8, **bars)
         assert checks == 16 and near < 16   # (the tiny model's logits are flat: most steps are near-ties at 2^-4)
     with drvmod.Driver(toml_config(**kw)) as d:
         gtoks, _ = d.generate(prompts[0], 8, replicate=2)
@@ -522,7 +525,7 @@ def test_custom_masks_over_a_one_byte_kv_cache_match_oracle(gpu, oracle, kv):
 def test_unknown_kv_cache_dtypes_are_refused(gpu):
     from pie_amd import driver as drvmod
 
-    for bad, msg in (("fp8_e5m2", "not implemented"), ("turboquant", "invalid kv_cache_dtype")):
+    for bad, msg in (("nvfp4", "not implemented"), ("turboquant", "invalid kv_cache_dtype")):
         with pytest.raises(Exception, match=msg):
             drvmod.Driver(toml_config(kv_cache_dtype=bad))
 

@@ -9,7 +9,7 @@ from paged_cases import make_paged_batch
 
 pytestmark = pytest.mark.gpu
 
-FORMATS = ["fp8_e4m3", "int8_per_token_head", "fp8_per_token_head"]
+FORMATS = ["fp8_e4m3", "int8_per_token_head", "fp8_per_token_head", "fp8_e5m2"]
 
 
 @pytest.mark.parametrize("fmt", FORMATS)
@@ -27,7 +27,7 @@ def test_kv_write_quant_bit_exact(gpu, oracle, fmt, hk, d):
     slots[5] = -1                                              # a token without a slot
     kp = torch.full((pages, ps, hk, d), 0x55, dtype=torch.uint8, device=gpu)
     vp = torch.full((pages, ps, hk, d), 0x55, dtype=torch.uint8, device=gpu)
-    scaled = fmt != "fp8_e4m3"
+    scaled = fmt not in ("fp8_e4m3", "fp8_e5m2")
     ks = torch.full((pages, ps, hk), -7.0, dtype=torch.float32, device=gpu) if scaled else None
     vs = torch.full((pages, ps, hk), -7.0, dtype=torch.float32, device=gpu) if scaled else None
     ops.kv_write_quant(fmt, dev(k, gpu, torch.bfloat16), dev(v, gpu, torch.bfloat16), dev(slots, gpu),
@@ -120,7 +120,7 @@ def test_rope_and_quantising_write_in_one_launch_equal_the_two_kernels(gpu, orac
     sg = dev(slots, gpu)
     qn = dev(oracle.f32_to_bf16(rng.uniform(0.5, 1.5, d).astype(np.float32)), gpu, torch.bfloat16) if qk_norm else None
     kn = dev(oracle.f32_to_bf16(rng.uniform(0.5, 1.5, d).astype(np.float32)), gpu, torch.bfloat16) if qk_norm else None
-    scaled = fmt != "fp8_e4m3"
+    scaled = fmt not in ("fp8_e4m3", "fp8_e5m2")
 
     def pools():
         kp = torch.full((pages, ps, hk, d), 0x55, dtype=torch.uint8, device=gpu)

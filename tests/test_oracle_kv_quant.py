@@ -8,7 +8,7 @@ import torch
 
 from paged_cases import make_paged_batch
 
-FORMATS = ["fp8_e4m3", "int8_per_token_head", "fp8_per_token_head"]
+FORMATS = ["fp8_e4m3", "int8_per_token_head", "fp8_per_token_head", "fp8_e5m2"]
 
 
 def reference_source(value: bool):
@@ -25,10 +25,18 @@ def e4m3_qdq(x):
     return t.to(torch.float8_e4m3fn).to(torch.float32).numpy()
 
 
+def e5m2_qdq(x):
+    """Saturating round-to-nearest-even e5m2 through torch (independent of the oracle)."""
+    t = torch.from_numpy(np.clip(x, -57344.0, 57344.0).astype(np.float32))
+    return t.to(torch.float8_e5m2).to(torch.float32).numpy()
+
+
 def independent_qdq(xf, fmt):
     """expected_qdq / expected_scale of the reference test, evaluated with numpy."""
     if fmt == "fp8_e4m3":
         return e4m3_qdq(xf), None
+    if fmt == "fp8_e5m2":
+        return e5m2_qdq(xf), None
     qmax = np.float32(127.0 if fmt.startswith("int8") else 448.0)
     amax = np.abs(xf).max(axis=1)
     scale = np.where(amax > 0, amax / qmax, np.float32(1.0)).astype(np.float32)
@@ -60,6 +68,10 @@ def test_codes_equal_an_independent_evaluation(oracle, fmt):
     x = oracle.f32_to_bf16((rng.standard_normal((64, 128)) * rng.uniform(0.01, 30, (64, 1))).astype(np.float32))
     xf = oracle.bf16_to_f32(x)
     codes, scales, deq = oracle.kv_quant_rows(x, fmt)
+    if fmt == "fp8_e5m2":
+        got = torch.from_numpy(codes.copy()).view(torch.float8_e5m2).to(torch.float32).numpy()
+        assert scales is None and np.array_equal(got, e5m2_qdq(xf)) and np.array_equal(deq, got)
+        return
     if fmt == "fp8_e4m3":
         scale = np.ones(64, np.float32)
     else:
@@ -129,3 +141,26 @@ def test_attention_over_f32_pools_equals_dense_attention(oracle):
             p = np.exp(s - s.max())
             want = (p / p.sum()) @ V[:, h // (hq // hk)]
             assert np.allclose(o32[r, h], want, rtol=1e-6, atol=1e-6)
+
+
+def test_e5m2_codes_against_torch(oracle):
+    """Every e5m2 code decodes to torch's float8_e5m2 value; encoding is round-to-nearest-even
+    with saturation at 57344 on ties, subnormals, the overflow edge and random values."""
+    import ctypes as C
+
+    codes = np.arange(256, dtype=np.uint8)
+    dec = np.zeros(256, np.float32)
+    oracle.lib().orc_fp8_e5m2_decode(C.c_void_p(codes.ctypes.data), C.c_void_p(dec.ctypes.data), C.c_size_t(256))
+    want = torch.from_numpy(codes.copy()).view(torch.float8_e5m2).to(torch.float32).numpy()
+    fin = np.isfinite(want)
+    assert np.array_equal(dec[fin], want[fin]) and np.array_equal(np.isnan(dec), np.isnan(want))
+    assert np.array_equal(np.isinf(dec), np.isinf(want))
+    rng = np.random.default_rng(12)
+    x = np.concatenate([rng.standard_normal(5000) * 10.0 ** rng.integers(-6, 5, 5000),
+                        [0.0, 1.125, 1.375, -1.125, 2.0 ** -16, 2.0 ** -17, 3 * 2.0 ** -17, 57344.0, 61439.0, 1e9, -1e9,
+                         2.0 ** -14, 1.5 * 2.0 ** -16]]).astype(np.float32)
+    enc = np.zeros(x.size, np.uint8)
+    oracle.lib().orc_fp8_e5m2_encode(C.c_void_p(x.ctypes.data), C.c_void_p(enc.ctypes.data), C.c_size_t(x.size))
+    got = torch.from_numpy(enc).view(torch.float8_e5m2).to(torch.float32).numpy()
+    assert np.array_equal(got, e5m2_qdq(x))
+    assert got[-3] == -57344.0 and got[-4] == 57344.0   # saturated, never inf
