@@ -35,6 +35,7 @@ struct ModelConfig {
     // MoE (qwen3_moe)
     int num_experts = 0, top_k = 0, expert_intermediate = 0;
     bool norm_topk = true;
+    int sliding_window = 0;   // > 0: a query at position p sees keys p - W + 1 .. p only
     // synthetic random-init weights: N(0, init_std) in bf16, then quantised
     std::uint64_t seed = 0x9E3779B97F4A7C15ull;
     float init_std = 0.02f;
@@ -230,6 +231,7 @@ inline DriverConfig parse_config_text(const std::string& text) {
                 else if (k == "top_k") m.top_k = (int)to_int(v, key);
                 else if (k == "expert_intermediate") m.expert_intermediate = (int)to_int(v, key);
                 else if (k == "norm_topk") m.norm_topk = to_bool(v, key);
+                else if (k == "sliding_window") m.sliding_window = (int)to_int(v, key);
                 else if (k == "seed") m.seed = (std::uint64_t)to_int(v, key);
                 else if (k == "init_std") m.init_std = (float)to_float(v, key);
                 else if (k == "router_std") m.router_std = (float)to_float(v, key);

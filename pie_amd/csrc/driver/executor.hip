@@ -528,7 +528,7 @@ void Executor::prepare_tiles(const BatchPlan& plan) {
     n_tiles_ = 0;
     const ModelConfig& m = model_.cfg();
     int cap = pie_hip_attn_prefill_tile_rows(m.q_heads, m.kv_heads);
-    if (cap <= 0 || plan.has_user_masks || page_size_ % 16 != 0 || (m.head_dim != 64 && m.head_dim != 128)) return;
+    if (cap <= 0 || masked_ || page_size_ % 16 != 0 || (m.head_dim != 64 && m.head_dim != 128)) return;
     long long blocks = 0;
     for (int r = 0; r < plan.R; ++r) {
         const int n = plan.qo_indptr[r + 1] - plan.qo_indptr[r];
@@ -560,7 +560,8 @@ void Executor::prepare_masks(const BatchPlan& plan) {
     const int N = plan.N;
     std::vector<int32_t> indptr(static_cast<size_t>(N) + 1, 0);
     std::vector<uint32_t> bounds;
-    for (int i = 0; i < N; ++i) {
+    const bool user = static_cast<int>(plan.row_mask_runs.size()) == N;   // (absent: window only)
+    for (int i = 0; i < N && user; ++i) {
         uint64_t acc = 0;
         for (uint32_t len : plan.row_mask_runs[i]) {
             acc = std::min<uint64_t>(acc + len, 0xFFFFFFFFull);
@@ -568,6 +569,7 @@ void Executor::prepare_masks(const BatchPlan& plan) {
         }
         indptr[i + 1] = static_cast<int32_t>(bounds.size());
     }
+    if (!user) std::fill(indptr.begin(), indptr.end(), 0);
     const size_t off_bounds = align_up(4ull * (N + 1), 16);
     const size_t total = off_bounds + 4ull * std::max<size_t>(bounds.size(), 1);
     mask_in_host_.pinned = true;
@@ -583,7 +585,8 @@ void Executor::prepare_masks(const BatchPlan& plan) {
     const Inputs lay = input_layout(N, static_cast<int>(plan.sample_rows.size()));   // this forward's staging layout
     const auto* row_len = reinterpret_cast<const int32_t*>(in_dev_ + lay.off_row_len);
     PIE_KERNEL(pie_hip_attn_mask_bitmap(reinterpret_cast<const uint32_t*>(dv + off_bounds),
-                                        reinterpret_cast<const int32_t*>(dv), row_len, 0,
+                                        reinterpret_cast<const int32_t*>(dv), row_len,
+                                        std::max(0, model_.cfg().sliding_window),
                                         static_cast<uint16_t*>(mask_bitmap_.ptr), N, mask_stride_, stream_));
 }
 
@@ -780,7 +783,10 @@ void Executor::forward(const BatchPlan& plan, std::vector<uint32_t>& tokens_out,
     if (S) std::memcpy(in_host_ + in.off_sample_rows, plan.sample_rows.data(), static_cast<size_t>(S) * 4);
     std::memcpy(in_host_ + in.off_pages, plan.page_indices.data(), plan.page_indices.size() * 4);
     PIE_HIP_CHECK(hipMemcpyAsync(in_dev_, in_host_, used, hipMemcpyHostToDevice, stream_));
-    masked_ = plan.has_user_masks;
+    // a sliding window (driver/portable/src/plan.cpp:60-70: keys below p - W + 1 are hidden)
+    // matters once some context is longer than the window; such batches take the masked kernels
+    const int window = model_.cfg().sliding_window;
+    masked_ = plan.has_user_masks || (window > 0 && plan.max_kv_len > window);
     if (masked_) prepare_masks(plan);
     prepare_tiles(plan);
     const bool sampling = !plan.all_greedy && S > 0;
@@ -794,7 +800,7 @@ void Executor::forward(const BatchPlan& plan, std::vector<uint32_t>& tokens_out,
     if (t) t->h2d_us = us_since(t0);
 
     t0 = clk::now();
-    const bool use_graph = cfg_.runtime.use_graphs && plan.pure_decode && !samp_gather_in_body_;
+    const bool use_graph = cfg_.runtime.use_graphs && plan.pure_decode && !samp_gather_in_body_ && !masked_;
     if (use_graph) {
         // The split grid depends on the context bound only through 512-token buckets.
         const int bucket = (plan.max_kv_len + 511) / 512 * 512;

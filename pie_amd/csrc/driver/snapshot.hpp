@@ -310,6 +310,10 @@ inline void apply_hf_config(ModelConfig& m, const std::string& dir) {
     else if (type == "qwen3_moe") m.arch = "qwen3_moe";
     else throw std::runtime_error("snapshot: unsupported model_type '" + type + "'");
     m.hidden = static_cast<int>(c.number_or("hidden_size", 0));
+    // (Mistral-type checkpoints: "sliding_window": N or null; Qwen3 writes one next to
+    // "use_sliding_window": false, which switches it off)
+    if (m.sliding_window <= 0 && c.bool_or("use_sliding_window", true))
+        m.sliding_window = static_cast<int>(c.number_or("sliding_window", 0));
     m.layers = static_cast<int>(c.number_or("num_hidden_layers", 0));
     m.q_heads = static_cast<int>(c.number_or("num_attention_heads", 0));
     m.kv_heads = static_cast<int>(c.number_or("num_key_value_heads", m.q_heads));

@@ -629,6 +629,50 @@ def test_decode_batches_of_16_and_64_distinct_requests(gpu, oracle, kw, count):
             assert near <= checks // 2
 
 
+@pytest.mark.parametrize("kw", [dict(quant="int4b8"), dict(quant="bf16", kv_cache_dtype="int8_per_token_head"),
+                                dict(arch="qwen3", quant="int8", head_dim=128, q_heads=4, kv_heads=1)],
+                         ids=["llama3", "llama3-int8kv", "qwen3"])
+def test_sliding_window_models_match_oracle(gpu, oracle, kw):
+    """[model] sliding_window = W (Mistral-type checkpoints): a query at position p sees keys
+    p - W + 1 .. p (driver/portable/src/plan.cpp:60-70).  Prefill rows and decode steps past the
+    window against the oracle with the same window, and the window really hides the old keys
+    (the logits differ from the full-context model's)."""
+    from pie_amd import driver as drvmod
+
+    W = 24
+    cfg = full_cfg(**kw)
+    rng = np.random.default_rng(1200)
+    prompt = rng.integers(0, cfg["vocab"], 41)
+    ps, V = cfg["page_size"], cfg["vocab"]
+    bars = dict(cos_min=0.998, rel=0.1, tie=2.0 ** -4) if kw.get("kv_cache_dtype") else {}
+    with drvmod.Driver(toml_config(**kw, sliding_window=W)) as d, drvmod.Driver(toml_config(**kw)) as full:
+        om, _ = oracle_model_from_driver(d, cfg)
+        n = len(prompt)
+        npg = (n + ps - 1) // ps
+        args = dict(token_ids=prompt, position_ids=np.arange(n), kv_page_indices=np.arange(npg), kv_page_indptr=[0, npg],
+                    kv_last_page_lens=[n - (npg - 1) * ps], qo_indptr=[0, n], sampling_indices=[20, 30, n - 1],
+                    sampling_indptr=[0, 3])
+        res = d.forward(drvmod.ForwardFrame(**args))
+        glog = d.export_tensor("debug.logits", np.uint16).reshape(-1, V)[:3].copy()
+        otok, olog, _ = om.forward(**args, want_logits=True, masks=[[]] * n, window=W)
+        for i in range(3):
+            check_step(oracle, glog[i], olog[i], res.tokens[i], otok[i], **bars)
+        full.forward(drvmod.ForwardFrame(**args))
+        flog = full.export_tensor("debug.logits", np.uint16).reshape(-1, V)[:3]
+        assert np.array_equal(flog[0], glog[0])                  # position 20: inside the window
+        assert cosine(oracle.bf16_to_f32(flog[2]), oracle.bf16_to_f32(glog[2])) < 0.9999   # position 40: clipped
+        tok = int(otok[2])
+        for s in range(n, n + 4):
+            npg = s // ps + 1
+            step = dict(token_ids=[tok], position_ids=[s], kv_page_indices=np.arange(npg), kv_page_indptr=[0, npg],
+                        kv_last_page_lens=[s + 1 - (npg - 1) * ps], qo_indptr=[0, 1])
+            res = d.forward(drvmod.ForwardFrame(**step))
+            lg = d.export_tensor("debug.logits", np.uint16).reshape(-1, V)[0]
+            ot, ol, _ = om.forward(**step, want_logits=True, masks=[[]], window=W)
+            check_step(oracle, lg, ol[0], res.tokens[0], ot[0], **bars)
+            tok = int(ot[0])
+
+
 def test_start_up_warm_up_changes_no_result(gpu):
     """[runtime] warmup runs a synthetic chunk over unowned pages at start-up: with it on or off
     the same request gives the same tokens and the same logits, bit for bit."""
