@@ -353,7 +353,9 @@ int pie_hip_attn_rows_paged_masked(const uint16_t* q, const uint16_t* k_pages, c
  */
 enum {
     PIE_HIP_SAMPLER_MULTINOMIAL = 0, PIE_HIP_SAMPLER_TOP_K = 1, PIE_HIP_SAMPLER_TOP_P = 2,
-    PIE_HIP_SAMPLER_MIN_P = 3, PIE_HIP_SAMPLER_TOP_K_TOP_P = 4, PIE_HIP_SAMPLER_DIST = 6,
+    PIE_HIP_SAMPLER_MIN_P = 3, PIE_HIP_SAMPLER_TOP_K_TOP_P = 4,
+    PIE_HIP_SAMPLER_EMBEDDING = 5,   /* a slot without output (the reference's executor emits nothing for it) */
+    PIE_HIP_SAMPLER_DIST = 6,
     PIE_HIP_SAMPLER_RAW_LOGITS = 7, PIE_HIP_SAMPLER_LOGPROB = 8, PIE_HIP_SAMPLER_LOGPROBS = 9,
     PIE_HIP_SAMPLER_ENTROPY = 10
 };

@@ -134,6 +134,7 @@ struct ResponseStore {
                         logprobs_val_indptr.push_back(static_cast<uint32_t>(logprobs_values.size()));
                         break;
                     case PIE_SAMPLER_KIND_ENTROPY: entropies.push_back(samples->values[o0]); break;
+                    case PIE_SAMPLER_KIND_EMBEDDING: break;   // no output
                     default: tokens.push_back(slot_tokens[s]); break;
                 }
                 if (plan.slot_samplers[s].kind == PIE_SAMPLER_KIND_RAW_LOGITS) raw_at += vocab;

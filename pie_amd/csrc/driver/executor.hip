@@ -628,6 +628,9 @@ void Executor::prepare_samplers(const BatchPlan& plan) {
                         throw std::runtime_error("sampler: Logprob label id out of vocab");
                 break;
             case PIE_SAMPLER_KIND_ENTROPY: n = 1; break;
+            // the response has no field for it: the slot is accepted and yields nothing, as the
+            // portable executor's per-slot switch leaves it (executor.cpp:1367-1392, default arm)
+            case PIE_SAMPLER_KIND_EMBEDDING: break;
             default:
                 throw std::runtime_error("sampler: unknown type " + std::to_string(static_cast<int>(sp.kind)));
         }

@@ -503,6 +503,7 @@ __global__ __launch_bounds__(kSampBlock) void sample_kernel(SampleArgs a) {
     const float* row = a.logits + static_cast<size_t>(s) * V;
     const int kind = a.kind[s];
     if (kind == PIE_HIP_SAMPLER_RAW_LOGITS) return;   // the caller reads the f32 row itself
+    if (kind == PIE_HIP_SAMPLER_EMBEDDING) return;    // no output for this slot
     float mx;
     int amax;
     block_argmax(row, V, sh, tid, lane, wv, mx, amax);

@@ -79,6 +79,35 @@ def test_every_sampler_kind_on_one_position(gpu, oracle):
         assert res.entropies_indptr == [0, 1] and res.tokens_indptr == [0, 5]
 
 
+def test_embedding_slots_are_accepted_and_yield_nothing(gpu):
+    """Wire sampler kind 5 (Embedding) has no field in the forward response; the reference's
+    executor emits nothing for such a slot (driver/portable/src/executor/executor.cpp:1367-1392,
+    default arm) and answers the others.  Same here: the request succeeds, the slots around the
+    Embedding slot give what they give without it."""
+    from pie_amd import driver as drvmod
+
+    cfg = full_cfg(vocab=4096)
+    V = cfg["vocab"]
+    rng = np.random.default_rng(72)
+    prompt = rng.integers(0, V, 17)
+    greedy = dict(kind=K["top_p"], temperature=0.0, p=1.0)
+    with drvmod.Driver(toml_config(vocab=V)) as d:
+        args = prefill_args(prompt, cfg["page_size"])
+        last = len(prompt) - 1
+        plain = d.forward(drvmod.ForwardFrame(**args, sampling_indices=[last, last], sampling_indptr=[0, 2],
+                                              samplers=[greedy, dict(kind=K["entropy"])], sampler_indptr=[0, 2]))
+        res = d.forward(drvmod.ForwardFrame(**args, sampling_indices=[last, last, last], sampling_indptr=[0, 3],
+                                            samplers=[greedy, dict(kind=5), dict(kind=K["entropy"])],
+                                            sampler_indptr=[0, 3]))
+        assert res.num_requests == 1 and plain.num_requests == 1
+        assert res.tokens_of(0) == plain.tokens_of(0) and len(res.tokens_of(0)) == 1
+        assert res.entropies_of(0) == plain.entropies_of(0) and len(res.entropies_of(0)) == 1
+        assert not res.dists_of(0) and not res.logits_of(0) and not res.logprobs_of(0)
+        only = d.forward(drvmod.ForwardFrame(**args, sampling_indices=[last], sampling_indptr=[0, 1],
+                                             samplers=[dict(kind=5)], sampler_indptr=[0, 1]))
+        assert only.num_requests == 1 and only.tokens_of(0) == []
+
+
 def test_sampled_decode_batch_under_graphs_and_logit_masks(gpu, oracle):
     """Four contexts decode with different samplers (one constrained by a BRLE logit mask, one
     greedy); the decode body replays from its HIP graph, the samplers run after it."""
