@@ -118,13 +118,12 @@ def gemv_roofline(drv, hip, model, reps: int):
         for l in range(model["layers"]):
             for name, (N, K) in shapes.items():
                 e0, e1 = hip.event(), hip.event()
-                k.pie_hip_gemv_time_next(e0, e1)
-                st = k.pie_hip_gemv_w4a16(C.c_void_p(acts[K].data_ptr()),
-                                          C.c_void_p(drv.tensor_ptr(f"layers.{l}.{name}.data")),
-                                          C.c_void_p(drv.tensor_ptr(f"layers.{l}.{name}.scale")),
-                                          C.c_void_p(outs[N].data_ptr()), 1, N, K, G, 0, stream)
+                st = k.pie_hip_gemv_w4a16_timed(C.c_void_p(acts[K].data_ptr()),
+                                                C.c_void_p(drv.tensor_ptr(f"layers.{l}.{name}.data")),
+                                                C.c_void_p(drv.tensor_ptr(f"layers.{l}.{name}.scale")),
+                                                C.c_void_p(outs[N].data_ptr()), 1, N, K, G, 0, e0, e1, stream)
                 if st != 0:
-                    raise RuntimeError(f"pie_hip_gemv_w4a16 status {st}")
+                    raise RuntimeError(f"pie_hip_gemv_w4a16_timed status {st}")
                 if rep > 0:
                     events.append((name, e0, e1))
     hip.sync()

@@ -224,7 +224,11 @@ typedef struct PieInProcVTable {
 int pie_driver_hip_run_inproc(int argc, char** argv, int install_signal_handlers,
                               void (*ready_cb)(const char* caps_json, void* ctx),
                               void* ready_ctx, PieInProcVTable vtable);
-/* Process-global stop for every live instance (driver/portable/src/entry.cpp:500-505). */
+/* Process-global stop for every live instance (driver/portable/src/entry.cpp:500-505): may be
+ * called from any thread.  An instance registers on entry to run_inproc, before it loads its
+ * model, so a stop requested while it loads makes it return (0) right after the ready
+ * handshake without serving; a serving instance leaves its loop when the recv in progress
+ * returns (recv may report "nothing yet" by returning 0 with a null frame). */
 void pie_driver_hip_request_stop(void);
 
 /* ---- direct (no vtable thread) embedding API ------------------------------------ */
@@ -253,11 +257,22 @@ int pie_hip_driver_handle(PieHipDriver* d, const PieFrameDesc* frame, PieRespons
 int pie_hip_driver_generate(PieHipDriver* d, const uint32_t* prompt, int n_prompt, int max_new,
                             int replicate, int warmup, uint32_t* out_tokens, double* timings_us,
                             char* err, size_t err_cap);
+/* Sampler the generation harness attaches to its decode steps instead of greedy: a wire kind
+ * 0..4 (Multinomial, TopK, TopP, MinP, TopKTopP) with its fields; the seed is advanced per step
+ * and context.  Returns 0, -1 on a bad kind. */
+int pie_hip_driver_set_generate_sampler(PieHipDriver* d, int kind, float temperature, uint32_t k,
+                                        float p, uint32_t seed);
+/* Host-only: what the snapshot reader sees in a Hugging Face checkpoint directory, as JSON
+ * {"arch", shape fields, "tensors": {name: {"dtype", "shape", "bytes", "first_bytes"}}} written
+ * to out.  Returns its length, or -1 with the reader's message in err.  No GPU is touched. */
+long long pie_hip_driver_snapshot_info(const char* dir, char* out, size_t out_cap, char* err,
+                                       size_t err_cap);
 /* Copy a named tensor to host memory (test/bench hook): model weights by name, "kv.k.<l>" /
  * "kv.v.<l>" (layer l's page pool), "debug.logits" (last forward's sampled-row logits) and
  * row 0 of the last layer's intermediates of the last forward: "debug.q" (rotated queries,
  * q_heads * head_dim bf16), "debug.attn" (attention output), "debug.act" (SwiGLU output) and
- * "debug.x" (residual stream after the layer).
+ * "debug.x" (residual stream after the layer); "info.qk_rows_paired" / "info.rope_interleaved"
+ * (one int32 each: whether wqkv's q / k rows are stored pair-interleaved, and the RoPE pairing).
  * Returns the byte size, 0 if the tensor does not exist; copies min(size, cap) bytes when dst
  * is non-null. */
 size_t pie_hip_driver_export_tensor(PieHipDriver* d, const char* name, void* dst, size_t cap);

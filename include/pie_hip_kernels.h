@@ -369,10 +369,13 @@ int pie_hip_sample(const float* logits_f32, const int32_t* kind, const float* te
                    uint32_t* tokens, float* values, uint32_t* ids, void* workspace,
                    size_t workspace_bytes, int num_slots, int vocab, void* stream);
 
-/* Measurement hook: the next GEMV kernel this thread launches (any format, M <= 4) is
- * bracketed by the two HIP events (hipEvent_t), so hipEventElapsedTime(start, stop) is that
- * kernel's own duration.  No reference counterpart. */
-int pie_hip_gemv_time_next(void* start_event, void* stop_event);
+/* Measurement form of pie_hip_gemv_w4a16 (M <= 4: one kernel): that kernel is bracketed by the
+ * caller's two HIP events (hipEvent_t), so hipEventElapsedTime(start, stop) is its own duration.
+ * The events belong to this call only; the library keeps nothing.  No reference counterpart. */
+int pie_hip_gemv_w4a16_timed(const uint16_t* act_bf16, const uint32_t* packed,
+                             const uint16_t* scale_bf16, uint16_t* y_bf16, int M, int N, int K,
+                             int group_size, int beta, void* start_event, void* stop_event,
+                             void* stream);
 
 /*
  * Weight-only int8 GEMV (W8A16), per-output-channel scale:

@@ -28,7 +28,7 @@ using namespace pie_hip_driver;
 
 namespace {
 
-std::atomic<bool> g_stop{false};
+std::atomic<bool> g_stop{false};   // set by SIGINT / SIGTERM when the handlers are installed
 
 using clk = std::chrono::steady_clock;
 uint32_t us_since(clk::time_point t0) {
@@ -686,7 +686,30 @@ extern "C" int pie_hip_driver_generate(PieHipDriver* d, const uint32_t* prompt, 
     }
 }
 
-extern "C" void pie_driver_hip_request_stop(void) { g_stop.store(true, std::memory_order_release); }
+// Every instance inside pie_driver_hip_run_inproc registers its stop flag on entry, before the
+// model is loaded, so a stop requested while it loads is honoured as soon as it would start to
+// serve; request_stop reaches every live instance of this flavour
+// (driver/portable/src/entry.cpp:61-94, :483-505).
+namespace {
+std::mutex g_instances_mu;
+std::vector<std::atomic<bool>*> g_instances;
+struct InstanceStop {
+    std::atomic<bool> flag{false};
+    InstanceStop() {
+        std::lock_guard<std::mutex> lk(g_instances_mu);
+        g_instances.push_back(&flag);
+    }
+    ~InstanceStop() {
+        std::lock_guard<std::mutex> lk(g_instances_mu);
+        g_instances.erase(std::remove(g_instances.begin(), g_instances.end(), &flag), g_instances.end());
+    }
+};
+}  // namespace
+
+extern "C" void pie_driver_hip_request_stop(void) {
+    std::lock_guard<std::mutex> lk(g_instances_mu);
+    for (auto* f : g_instances) f->store(true, std::memory_order_release);
+}
 
 extern "C" int pie_driver_hip_run_inproc(int argc, char** argv, int install_signal_handlers,
                                          void (*ready_cb)(const char* caps_json, void* ctx),
@@ -710,13 +733,14 @@ extern "C" int pie_driver_hip_run_inproc(int argc, char** argv, int install_sign
             std::signal(SIGINT, [](int) { g_stop.store(true); });
             std::signal(SIGTERM, [](int) { g_stop.store(true); });
         }
-        g_stop.store(false, std::memory_order_release);
+        g_stop.store(false, std::memory_order_release);   // (signals of an earlier run)
+        InstanceStop stop;
         PieHipDriver driver(load_driver_config(config_path));
         warm_up(&driver);
         if (ready_cb) ready_cb(driver.caps.c_str(), ready_ctx);
         if (driver.cfg.runtime.verbose) std::fprintf(stderr, "[pie-driver-hip] serving on in-process channel\n");
         PieResponseFrameDesc resp;
-        while (!g_stop.load(std::memory_order_acquire)) {
+        while (!g_stop.load(std::memory_order_acquire) && !stop.flag.load(std::memory_order_acquire)) {
             const PieFrameDesc* req = nullptr;
             uint32_t req_id = 0;
             const int32_t rc = vtable.recv(vtable.ctx, &req, &req_id);

@@ -698,8 +698,8 @@ __global__ __launch_bounds__(256) void argmax_pairs_kernel(const unsigned long l
     }
 }
 
-// Optional per-thread event pair that brackets exactly the next GEMV kernel (set by
-// pie_hip_gemv_time_next); consumed by one launch.
+// Event pair that brackets the kernel of a pie_hip_gemv_w4a16_timed call (set and cleared inside
+// that call).
 thread_local hipEvent_t t_start_event = nullptr;
 thread_local hipEvent_t t_stop_event = nullptr;
 
@@ -804,11 +804,6 @@ int dispatch(GemvArgs a, int M, int rows_per_wave, int waves_per_simd, hipStream
 
 using pie_hip::GemvArgs;
 
-extern "C" int pie_hip_gemv_time_next(void* start_event, void* stop_event) {
-    pie_hip::t_start_event = static_cast<hipEvent_t>(start_event);
-    pie_hip::t_stop_event = static_cast<hipEvent_t>(stop_event);
-    return PIE_HIP_OK;
-}
 
 extern "C" int pie_hip_gemv_w4a16_tuned(const uint16_t* act_bf16, const uint32_t* packed,
                                         const uint16_t* scale_bf16, uint16_t* y_bf16, int M,
@@ -827,6 +822,21 @@ extern "C" int pie_hip_gemv_w4a16(const uint16_t* act_bf16, const uint32_t* pack
                                   int K, int group_size, int beta, void* stream) {
     return pie_hip_gemv_w4a16_tuned(act_bf16, packed, scale_bf16, y_bf16, M, N, K, group_size,
                                     beta, 0, 0, stream);
+}
+
+// The same launch bracketed by the caller's two events (measurement): the events travel with
+// this one call — nothing is remembered between calls.
+extern "C" int pie_hip_gemv_w4a16_timed(const uint16_t* act_bf16, const uint32_t* packed,
+                                        const uint16_t* scale_bf16, uint16_t* y_bf16, int M, int N,
+                                        int K, int group_size, int beta, void* start_event,
+                                        void* stop_event, void* stream) {
+    if (!start_event || !stop_event || M > 4) return PIE_HIP_ERR_INVALID;   // one kernel per call
+    pie_hip::t_start_event = static_cast<hipEvent_t>(start_event);
+    pie_hip::t_stop_event = static_cast<hipEvent_t>(stop_event);
+    const int rc = pie_hip_gemv_w4a16_tuned(act_bf16, packed, scale_bf16, y_bf16, M, N, K, group_size,
+                                            beta, 0, 0, stream);
+    pie_hip::t_start_event = pie_hip::t_stop_event = nullptr;
+    return rc;
 }
 
 extern "C" int pie_hip_gemv_w8a16(const uint16_t* act_bf16, const int8_t* w_int8,

@@ -328,6 +328,89 @@ def test_run_inproc_serve_loop(gpu, tmp_path):
     assert drvmod.lib().pie_driver_hip_run_inproc(1, argv2, 0, ready, None, vt) == -1
 
 
+def _run_inproc_thread(drvmod, cfg_path, recv, send, on_ready):
+    import ctypes as C
+    import threading
+
+    vt = drvmod.InProcVTable(drvmod.RECV_FN(recv), drvmod.SEND_FN(send), None)
+    ready = drvmod.READY_FN(on_ready)
+    argv = (C.c_char_p * 3)(b"pie-driver-hip", b"--config", str(cfg_path).encode())
+    rc = []
+    th = threading.Thread(target=lambda: rc.append(
+        drvmod.lib().pie_driver_hip_run_inproc(3, argv, 0, ready, None, vt)))
+    th.keep = (vt, ready, argv)   # the callbacks must outlive the call
+    th.start()
+    return th, rc
+
+
+def test_request_stop_from_another_thread_ends_a_waiting_serve_loop(gpu, tmp_path):
+    """pie_driver_hip_request_stop from a second thread while the loop waits in recv (a vtable
+    whose recv times out with "nothing yet"): the loop returns 0 after the recv in progress,
+    having answered what it was given before."""
+    import ctypes as C
+    import threading
+    import time
+
+    from pie_amd import driver as drvmod
+
+    cfg_path = tmp_path / "driver.toml"
+    cfg_path.write_text(toml_config())
+    frame = drvmod.ForwardFrame([5], [0], [3], [0, 1], [1], [0, 1])
+    pending, got, is_ready, polls = [frame.frame], [], threading.Event(), [0]
+
+    def recv(ctx, out_req, out_id):
+        if pending:
+            out_req[0] = C.pointer(pending.pop(0))
+            out_id[0] = 7
+            return 0
+        polls[0] += 1
+        time.sleep(0.02)          # nothing yet: a null frame with status 0
+        out_req[0] = None
+        return 0
+
+    def send(ctx, req_id, resp):
+        got.append((req_id, resp.contents.payload.forward.num_requests))
+
+    th, rc = _run_inproc_thread(drvmod, cfg_path, recv, send, lambda js, ctx: is_ready.set())
+    assert is_ready.wait(timeout=120)
+    while not got or polls[0] < 3:   # the request is answered and the loop is idling in recv
+        time.sleep(0.01)
+        assert th.is_alive()
+    drvmod.lib().pie_driver_hip_request_stop()
+    th.join(timeout=30)
+    assert not th.is_alive() and rc == [0] and got == [(7, 1)]
+
+
+def test_request_stop_during_model_load_is_not_lost(gpu, tmp_path):
+    """A stop requested while the instance is still loading its model: the instance registers
+    for stops before it loads, so it returns 0 after the ready handshake without a single recv."""
+    import threading
+    import time
+
+    from pie_amd import driver as drvmod
+
+    cfg_path = tmp_path / "driver.toml"
+    # big enough that loading takes a moment: 8 layers of a 2048-wide model
+    cfg_path.write_text(toml_config(hidden=2048, layers=8, q_heads=16, kv_heads=4, head_dim=128, intermediate=8192,
+                                    vocab=32000))
+    is_ready, recvs = threading.Event(), [0]
+
+    def recv(ctx, out_req, out_id):
+        recvs[0] += 1
+        return -1
+
+    th, rc = _run_inproc_thread(drvmod, cfg_path, recv, lambda *a: None, lambda js, ctx: is_ready.set())
+    # stops in a tight loop from the moment the thread starts: the first one that finds the
+    # instance registered arrives microseconds after its entry, long before the model is loaded
+    stop = drvmod.lib().pie_driver_hip_request_stop
+    t_end = time.time() + 120
+    while th.is_alive() and time.time() < t_end:
+        stop()
+    th.join(timeout=1)
+    assert not th.is_alive() and rc == [0]
+    assert is_ready.is_set() and recvs[0] == 0
+
+
 def test_custom_attention_masks_match_oracle(gpu, oracle):
     """Prefill and a decode step under per-token BRLE attention masks
     (build_attn_mask_f16, driver/portable/src/plan.cpp:54-94) against the oracle model."""
