@@ -37,3 +37,37 @@ def test_missing_library_is_loud(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "KERNEL_LIB_PATH", tmp_path / "nope.so")
     with pytest.raises(_lib.KernelLibraryMissing):
         _lib.kernels()
+
+
+def test_rust_bindings_name_only_exported_symbols_with_matching_arity():
+    """The (uncompiled) Rust FFI declarations under pie_amd/rust bind functions that the two
+    libraries really export, with as many parameters as the C headers declare."""
+    rs = (ROOT / "pie_amd" / "rust" / "pie-driver-hip" / "src" / "lib.rs").read_text()
+    rs = re.sub(r"//[^\n]*", "", rs)
+    decls = re.findall(r"pub fn (pie_\w+)\s*\((.*?)\)\s*(?:->[^;]+)?;", rs, flags=re.S)
+    assert len(decls) >= 15
+    headers = ""
+    for h in ("pie_hip_kernels.h", "pie_driver_abi.h"):
+        headers += re.sub(r"/\*.*?\*/", "", (ROOT / "include" / h).read_text(), flags=re.S)
+    kernels = ctypes.CDLL(str(ROOT / "pie_amd" / "libpie_hip_kernels.so"))
+    driver_path = ROOT / "pie_amd" / "libpie_driver_hip.so"
+    driver = ctypes.CDLL(str(driver_path)) if driver_path.exists() else None
+
+    def arity(params: str) -> int:
+        params = params.strip()
+        if not params or params == "void":
+            return 0
+        depth, n = 0, 1
+        for ch in params:
+            depth += ch in "(<"
+            depth -= ch in ")>"
+            n += ch == "," and depth == 0
+        return n - (1 if params.rstrip().endswith(",") else 0)
+
+    for name, params in decls:
+        lib = driver if name.startswith("pie_driver_") else kernels
+        if lib is not None:
+            assert hasattr(lib, name), name
+        m = re.search(rf"\b{name}\s*\((.*?)\)\s*;", headers, flags=re.S)
+        assert m, f"{name} is not declared in include/"
+        assert arity(params) == arity(m.group(1)), name
