@@ -563,6 +563,11 @@ int pie_hip_residual_rmsnorm(uint16_t* hidden_bf16, const uint16_t* residual_bf1
  * Reference: rope_standard_table_kernel, driver/cuda/src/kernels/rope.cu:35-53. */
 int pie_hip_rope_table(const int32_t* positions, const float* inv_freq, float* table,
                        int num_tokens, int head_dim, void* stream);
+/* The same with cos and sin multiplied by mscale (> 0): YaRN's attention factor
+ * (rope_yarn_original_bf16_kernel, driver/cuda/src/kernels/rope.cu:509-548; the frequencies of
+ * that scheme are a host-side inv_freq table like any other). */
+int pie_hip_rope_table_scaled(const int32_t* positions, const float* inv_freq, float* table,
+                              int num_tokens, int head_dim, float mscale, void* stream);
 
 /*
  * Split a packed QKV row [N, (hq + 2*hk)*d], apply optional per-head RMSNorm (both norm

@@ -207,6 +207,13 @@ def rope_inv_freq(d, theta, factor=0.0, low_freq_factor=1.0, high_freq_factor=4.
     return out
 
 
+def rope_inv_freq_yarn(d, theta, factor, beta_fast=32.0, beta_slow=1.0, original_max_pos=4096):
+    out = np.empty((d // 2,), np.float32)
+    lib().orc_rope_inv_freq_yarn(_p(out), C.c_int(d), C.c_float(theta), C.c_float(factor), C.c_float(beta_fast),
+                                 C.c_float(beta_slow), C.c_int(original_max_pos))
+    return out
+
+
 def rope_table(positions, inv_freq, d):
     pos = _c(positions, np.int32)
     f = _c(inv_freq, np.float32)

@@ -29,7 +29,7 @@ class _Model(C.Structure):
                 ("wqkv", C.POINTER(_Linear)), ("wo", C.POINTER(_Linear)),
                 ("wgu", C.POINTER(_Linear)), ("wdown", C.POINTER(_Linear)),
                 ("num_experts", C.c_int), ("top_k", C.c_int), ("expert_intermediate", C.c_int),
-                ("router", C.POINTER(C.c_void_p))]
+                ("router", C.POINTER(C.c_void_p)), ("rope_mscale", C.c_float)]
 
 
 class OracleModel:
@@ -91,6 +91,7 @@ class OracleModel:
         m.expert_intermediate = int(cfg.get("expert_intermediate", 0))
         if m.num_experts:
             m.router = parr([f"layers.{l}.router" for l in range(L)])
+        m.rope_mscale = float(cfg.get("rope_mscale", 1.0))
         self._m = m
         ps, tp = cfg["page_size"], cfg["total_pages"]
         shape = (tp, ps, cfg["kv_heads"], cfg["head_dim"])
@@ -368,6 +369,8 @@ def model_from_driver(drv, cfg: dict):
                 rms_eps=cfg.get("rms_eps", 1e-5), rope_interleaved=interleaved,
                 qk_norm=cfg["arch"] != "llama3", quant=quant, group_size=cfg.get("group_size", 128),
                 page_size=cfg["page_size"], total_pages=cfg["total_pages"])
+    ms = drv.export_tensor("info.rope_mscale", np.float32)
+    ocfg["rope_mscale"] = float(ms[0]) if ms is not None else 1.0
     if cfg["arch"] == "qwen3_moe":
         ocfg.update(num_experts=cfg["num_experts"], top_k=cfg["top_k"],
                     expert_intermediate=cfg["expert_intermediate"], intermediate=0)

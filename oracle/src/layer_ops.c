@@ -76,15 +76,43 @@ void orc_rope_inv_freq(float* inv_freq, int d, float theta, float factor, float 
     }
 }
 
-void orc_rope_table(const int32_t* positions, const float* inv_freq, float* table, int n_tokens,
-                    int d) {
+void orc_rope_table_scaled(const int32_t* positions, const float* inv_freq, float* table, int n_tokens,
+                           int d, float mscale) {
     const int half = d / 2;
     for (int n = 0; n < n_tokens; ++n)
         for (int i = 0; i < half; ++i) {
             const float ang = (float)positions[n] * inv_freq[i];
-            table[(size_t)n * d + i] = cosf(ang);
-            table[(size_t)n * d + i + half] = sinf(ang);
+            table[(size_t)n * d + i] = cosf(ang) * mscale;
+            table[(size_t)n * d + i + half] = sinf(ang) * mscale;
         }
+}
+
+void orc_rope_table(const int32_t* positions, const float* inv_freq, float* table, int n_tokens,
+                    int d) {
+    orc_rope_table_scaled(positions, inv_freq, table, n_tokens, d, 1.0f);
+}
+
+/* YaRN frequencies (launch_rope_yarn_original_bf16, driver/cuda/src/kernels/rope.cu:495-507,
+ * 552-589; transformers' _compute_yarn_parameters): pairs below low_dim keep theta^(-2i/d), pairs
+ * above high_dim are divided by the factor, a linear ramp between; low / high from the number of
+ * rotations beta_fast / beta_slow a pair makes over the original context. */
+void orc_rope_inv_freq_yarn(float* inv_freq, int d, float theta, float factor, float beta_fast,
+                            float beta_slow, int original_max_pos) {
+    const int half = d / 2;
+    const double pi = 3.14159265358979323846;
+    const double ln_theta = log((double)theta);
+    double lo = floor(d * log((double)original_max_pos / ((double)beta_fast * 2.0 * pi)) / (2.0 * ln_theta));
+    double hi = ceil(d * log((double)original_max_pos / ((double)beta_slow * 2.0 * pi)) / (2.0 * ln_theta));
+    if (lo < 0.0) lo = 0.0;
+    if (hi > (double)half - 1.0) hi = (double)half - 1.0;
+    if (hi < lo) hi = lo;
+    const double denom = hi == lo ? hi + 1e-3 - lo : hi - lo;
+    for (int i = 0; i < half; ++i) {
+        const double base = pow((double)theta, -2.0 * (double)i / (double)d);
+        double ramp = ((double)i - lo) / denom;
+        ramp = ramp < 0.0 ? 0.0 : (ramp > 1.0 ? 1.0 : ramp);
+        inv_freq[i] = (float)(base * ((1.0 - ramp) + ramp / (double)factor));
+    }
 }
 
 void orc_qkv_rope_kvwrite(const uint16_t* packed, uint16_t* q_out, uint16_t* k_pages,

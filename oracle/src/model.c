@@ -197,7 +197,7 @@ static void orc_llama_forward_impl(const OrcModel* m, uint16_t* const* k_pages, 
     }
 
     orc_embed(tokens, m->embed, x, N, H, V);
-    orc_rope_table(positions, m->inv_freq, tab, N, d);
+    orc_rope_table_scaled(positions, m->inv_freq, tab, N, d, m->rope_mscale > 0.f ? m->rope_mscale : 1.0f);
     for (int l = 0; l < m->layers; ++l) {
         orc_rmsnorm(x, NULL, m->attn_norm[l], xn, N, H, m->rms_eps);
         orc_linear(m, &m->wqkv[l], xn, qkv, N, qkv_dim, H, 0);

@@ -135,7 +135,8 @@ static void FN(rope_kvwrite)(const OrcModel* m, int l, const REAL* qkv, REAL* q_
                     b = b * inv * (REAL)orc_bf16_to_f32(nw[ib]);
                 }
                 const REAL ang = (REAL)positions[n] * (REAL)m->inv_freq[i];
-                const REAL c = (REAL)cos((double)ang), s = (REAL)sin((double)ang);
+                const REAL ms = m->rope_mscale > 0.f ? (REAL)m->rope_mscale : (REAL)1;
+                const REAL c = (REAL)cos((double)ang) * ms, s = (REAL)sin((double)ang) * ms;
                 const REAL ra = a * c - b * s, rb = b * c + a * s;
                 if (is_q) {
                     REAL* dst = q_out + ((size_t)n * hq + head) * d;

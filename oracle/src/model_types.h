@@ -31,6 +31,7 @@ typedef struct {
      * [E * 2*Ie, H] (per expert: gate rows then up rows) and [E * H, Ie]. */
     int num_experts, top_k, expert_intermediate;
     const uint16_t* const* router; /* [L] bf16 [E, H] */
+    float rope_mscale;             /* cos and sin are multiplied by it (YaRN's attention factor; 1 otherwise) */
 } OrcModel;
 
 #endif

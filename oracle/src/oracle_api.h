@@ -10,6 +10,8 @@ void orc_rmsnorm(uint16_t* x, const uint16_t* residual, const uint16_t* w, uint1
                  int hidden, float eps);
 void orc_rope_table(const int32_t* positions, const float* inv_freq, float* table, int n_tokens,
                     int d);
+void orc_rope_table_scaled(const int32_t* positions, const float* inv_freq, float* table, int n_tokens,
+                           int d, float mscale);
 void orc_qkv_rope_kvwrite(const uint16_t* packed, uint16_t* q_out, uint16_t* k_pages,
                           uint16_t* v_pages, const uint16_t* q_norm_w, const uint16_t* k_norm_w,
                           const float* table, const int64_t* kv_slots, int n_tokens, int hq, int hk,

@@ -26,6 +26,11 @@ struct ModelConfig {
     // llama3 wavelength-band RoPE scaling; factor <= 0 disables it
     float rope_factor = 0.f, rope_low_freq_factor = 1.f, rope_high_freq_factor = 4.f;
     int rope_original_max_pos = 8192;
+    // rope_scaling = "llama3" (wavelength bands, the default when rope_factor > 0) or "yarn"
+    // (ramp over the rotation dims between beta_fast and beta_slow, cos / sin times the
+    // attention factor; 0 = 0.1 ln(factor) + 1)
+    std::string rope_scaling;
+    float rope_beta_fast = 32.f, rope_beta_slow = 1.f, rope_attention_factor = 0.f;
     int rope_interleaved = -1;  // -1: half split, the pairing of Llama / Mistral / Qwen checkpoints
     bool tie_embeddings = false;
     // storage format of the decoder linears: "int4b8" | "int8" | "fp8" | "bf16"
@@ -190,6 +195,9 @@ inline void finalize_config(DriverConfig& c) {
     // (i, i + d/2) pairs for every architecture here, as the reference rotates them
     // (driver/cuda/src/kernels/rope.cu:10-21 keeps adjacent pairs for GLM only)
     if (m.rope_interleaved < 0) m.rope_interleaved = 0;
+    if (m.rope_scaling.empty()) m.rope_scaling = "llama3";
+    if (m.rope_scaling != "llama3" && m.rope_scaling != "yarn")
+        throw std::runtime_error("config: rope_scaling must be llama3 or yarn");
     const auto& b = c.batching;
     if (b.kv_page_size <= 0 || b.kv_page_size % 16 != 0)
         throw std::runtime_error("config: kv_page_size must be a positive multiple of 16");
@@ -222,6 +230,10 @@ inline DriverConfig parse_config_text(const std::string& text) {
                 else if (k == "rope_low_freq_factor") m.rope_low_freq_factor = (float)to_float(v, key);
                 else if (k == "rope_high_freq_factor") m.rope_high_freq_factor = (float)to_float(v, key);
                 else if (k == "rope_original_max_pos") m.rope_original_max_pos = (int)to_int(v, key);
+                else if (k == "rope_scaling") m.rope_scaling = v;
+                else if (k == "rope_beta_fast") m.rope_beta_fast = (float)to_float(v, key);
+                else if (k == "rope_beta_slow") m.rope_beta_slow = (float)to_float(v, key);
+                else if (k == "rope_attention_factor") m.rope_attention_factor = (float)to_float(v, key);
                 else if (k == "rope_interleaved") m.rope_interleaved = to_bool(v, key) ? 1 : 0;
                 else if (k == "tie_embeddings") m.tie_embeddings = to_bool(v, key);
                 else if (k == "quant") m.quant = v;

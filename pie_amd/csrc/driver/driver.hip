@@ -488,6 +488,11 @@ extern "C" size_t pie_hip_driver_export_tensor(PieHipDriver* d, const char* name
         if (dst && cap >= sizeof(v)) std::memcpy(dst, &v, sizeof(v));
         return sizeof(v);
     }
+    if (nm == "info.rope_mscale") {   // one float
+        const float v = rope_mscale(d->cfg.model);
+        if (dst && cap >= sizeof(v)) std::memcpy(dst, &v, sizeof(v));
+        return sizeof(v);
+    }
     if (nm.rfind("debug.", 0) == 0) {
         const uint16_t* buf = d->exec->debug_buffer(nm.substr(6));
         if (!buf) return 0;

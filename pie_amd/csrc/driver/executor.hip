@@ -364,7 +364,7 @@ void Executor::body(int N, int S, int max_kv_len) {
     const auto* pages = reinterpret_cast<const uint32_t*>(in_dev_ + in_.off_pages);
 
     PIE_KERNEL(pie_hip_embed(tokens, model_.embed, x_, N, H, m.vocab, s));
-    PIE_KERNEL(pie_hip_rope_table(positions, model_.inv_freq, rope_tab_, N, d, s));
+    PIE_KERNEL(pie_hip_rope_table_scaled(positions, model_.inv_freq, rope_tab_, N, d, rope_mscale(m), s));
     // RoPE pairing as the rotation kernels take it: adjacent pairs, half-split pairs, or
     // half-split pairs over projection rows re-ordered at load (then the fused epilogues apply)
     const int pairing = m.rope_interleaved ? PIE_HIP_ROPE_ADJACENT

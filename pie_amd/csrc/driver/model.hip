@@ -89,7 +89,22 @@ std::vector<float> rope_inv_freq(const ModelConfig& cfg) {
     for (int i = 0; i < half; ++i) {
         const double base = std::pow(static_cast<double>(cfg.rope_theta), -2.0 * i / d);
         double f = base;
-        if (cfg.rope_factor > 0.f && cfg.rope_original_max_pos > 0) {
+        if (cfg.rope_factor > 0.f && cfg.rope_original_max_pos > 0 && cfg.rope_scaling == "yarn") {
+            // YaRN: full rotations below low_dim, frequencies divided by the factor above
+            // high_dim, a linear ramp between (launch_rope_yarn_original_bf16,
+            // driver/cuda/src/kernels/rope.cu:495-507,552-589)
+            const double ln_theta = std::log(static_cast<double>(cfg.rope_theta));
+            auto corr = [&](double rot) {
+                return d * std::log(cfg.rope_original_max_pos / (rot * 2.0 * pi)) / (2.0 * ln_theta);
+            };
+            double lo = std::floor(corr(cfg.rope_beta_fast)), hi = std::ceil(corr(cfg.rope_beta_slow));
+            lo = std::max(lo, 0.0);
+            hi = std::min(hi, static_cast<double>(half) - 1.0);
+            hi = std::max(hi, lo);
+            const double denom = hi == lo ? hi + 1e-3 - lo : hi - lo;
+            const double ramp = std::min(1.0, std::max(0.0, (i - lo) / denom));
+            f = base * ((1.0 - ramp) + ramp / cfg.rope_factor);
+        } else if (cfg.rope_factor > 0.f && cfg.rope_original_max_pos > 0) {
             const double low_wl = cfg.rope_original_max_pos / static_cast<double>(cfg.rope_low_freq_factor);
             const double high_wl = cfg.rope_original_max_pos / static_cast<double>(cfg.rope_high_freq_factor);
             const double wl = 2.0 * pi / base;
@@ -106,6 +121,12 @@ std::vector<float> rope_inv_freq(const ModelConfig& cfg) {
         out[i] = static_cast<float>(f);
     }
     return out;
+}
+
+float rope_mscale(const ModelConfig& cfg) {
+    if (cfg.rope_scaling != "yarn" || !(cfg.rope_factor > 0.f)) return 1.f;
+    if (cfg.rope_attention_factor > 0.f) return cfg.rope_attention_factor;
+    return cfg.rope_factor <= 1.f ? 1.f : 0.1f * std::log(cfg.rope_factor) + 1.f;
 }
 
 Model::~Model() {

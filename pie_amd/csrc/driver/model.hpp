@@ -126,5 +126,8 @@ class Model {
 // Host-side inv_freq table (theta^(-2i/d) with optional llama3 band scaling,
 // driver/portable/src/model.cpp:1414-1448: the stored factor divides the base frequency).
 std::vector<float> rope_inv_freq(const ModelConfig& cfg);
+// What cos and sin are multiplied by: YaRN's attention factor (0.1 ln(factor) + 1 unless the
+// config states one), 1 for every other scheme.
+float rope_mscale(const ModelConfig& cfg);
 
 }  // namespace pie_hip_driver

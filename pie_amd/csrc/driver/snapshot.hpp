@@ -331,6 +331,14 @@ inline void apply_hf_config(ModelConfig& m, const std::string& dir) {
             m.rope_low_freq_factor = static_cast<float>(rs->number_or("low_freq_factor", 1.0));
             m.rope_high_freq_factor = static_cast<float>(rs->number_or("high_freq_factor", 4.0));
             m.rope_original_max_pos = static_cast<int>(rs->number_or("original_max_position_embeddings", 8192));
+        } else if (rt == "yarn") {
+            m.rope_scaling = "yarn";
+            m.rope_factor = static_cast<float>(rs->number_or("factor", 1.0));
+            m.rope_beta_fast = static_cast<float>(rs->number_or("beta_fast", 32.0));
+            m.rope_beta_slow = static_cast<float>(rs->number_or("beta_slow", 1.0));
+            m.rope_attention_factor = static_cast<float>(rs->number_or("attention_factor", 0.0));
+            m.rope_original_max_pos = static_cast<int>(rs->number_or(
+                "original_max_position_embeddings", c.number_or("max_position_embeddings", 8192)));
         } else if (!rt.empty() && rt != "default") {
             throw std::runtime_error("snapshot: unsupported rope_scaling type '" + rt + "'");
         }

@@ -95,15 +95,17 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(uint16_t* __restrict__ x,
 // frequency scaling (llama3 bands, YaRN) is a host-side table, not kernel code.
 __global__ void rope_table_kernel(const int32_t* __restrict__ positions,
                                   const float* __restrict__ inv_freq, float* __restrict__ table,
-                                  int d) {
+                                  int d, float mscale) {
     const int n = blockIdx.x, half = d / 2;
     const float pos = static_cast<float>(positions[n]);
     for (int i = threadIdx.x; i < half; i += blockDim.x) {
         const float ang = pos * inv_freq[i];
         float s, c;
         sincosf(ang, &s, &c);
-        table[static_cast<size_t>(n) * d + i] = c;
-        table[static_cast<size_t>(n) * d + i + half] = s;
+        // (YaRN's attention factor rides on cos and sin, driver/cuda/src/kernels/rope.cu:531-535;
+        // 1 otherwise, which changes no bit)
+        table[static_cast<size_t>(n) * d + i] = c * mscale;
+        table[static_cast<size_t>(n) * d + i + half] = s * mscale;
     }
 }
 
@@ -291,7 +293,17 @@ extern "C" int pie_hip_rope_table(const int32_t* positions, const float* inv_fre
         return PIE_HIP_ERR_INVALID;
     if (head_dim % 2 != 0) return PIE_HIP_ERR_UNSUPPORTED;
     hipLaunchKernelGGL(rope_table_kernel, dim3(num_tokens), dim3(64), 0,
-                       static_cast<hipStream_t>(stream), positions, inv_freq, table, head_dim);
+                       static_cast<hipStream_t>(stream), positions, inv_freq, table, head_dim, 1.0f);
+    return launch_status();
+}
+
+extern "C" int pie_hip_rope_table_scaled(const int32_t* positions, const float* inv_freq, float* table,
+                                         int num_tokens, int head_dim, float mscale, void* stream) {
+    if (!positions || !inv_freq || !table || num_tokens <= 0 || head_dim <= 0 || !(mscale > 0.f))
+        return PIE_HIP_ERR_INVALID;
+    if (head_dim % 2 != 0) return PIE_HIP_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(rope_table_kernel, dim3(num_tokens), dim3(64), 0,
+                       static_cast<hipStream_t>(stream), positions, inv_freq, table, head_dim, mscale);
     return launch_status();
 }
 

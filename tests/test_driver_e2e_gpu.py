@@ -253,10 +253,10 @@ def test_forward_failures_return_empty_response(gpu):
     with drvmod.Driver(toml_config()) as d:
         ok = dict(token_ids=[1], position_ids=[0], kv_page_indices=[0], kv_page_indptr=[0, 1],
                   kv_last_page_lens=[1], qo_indptr=[0, 1])
-        # out-of-range page id, position past the context, a sampler kind without an
-        # implementation (Embedding), attention masks that are not one per token row
+        # out-of-range page id, position past the context, a sampler kind that does not exist,
+        # attention masks that are not one per token row
         for bad in (dict(kv_page_indices=[9999]), dict(position_ids=[5]),
-                    dict(samplers=[dict(kind=5, temperature=0.8)], sampling_indices=[0],
+                    dict(samplers=[dict(kind=11, temperature=0.8)], sampling_indices=[0],
                          sampling_indptr=[0, 1], sampler_indptr=[0, 1]),
                     dict(masks=[[0, 1], [0, 1]])):
             args = dict(ok)
@@ -754,6 +754,30 @@ def test_sliding_window_models_match_oracle(gpu, oracle, kw):
             ot, ol, _ = om.forward(**step, want_logits=True, masks=[[]], window=W)
             check_step(oracle, lg, ol[0], res.tokens[0], ot[0], **bars)
             tok = int(ot[0])
+
+
+def test_yarn_scaled_model_matches_oracle(gpu, oracle):
+    """[model] rope_scaling = "yarn": the driver's frequency table equals the oracle's YaRN table,
+    cos / sin carry the attention factor 0.1 ln(factor) + 1, and generation past the original
+    context matches the oracle model (which rotates with the same table and factor)."""
+    from pie_amd import driver as drvmod
+
+    extra = 'rope_scaling = "yarn"\nrope_beta_fast = 8.0\nrope_beta_slow = 1.0\n'
+    kw = dict(arch="qwen3", quant="int8", head_dim=128, q_heads=4, kv_heads=1, rope_theta=10000.0, rope_factor=4.0)
+    cfg = full_cfg(**kw)
+    rng = np.random.default_rng(1300)
+    with drvmod.Driver(toml_config(**kw, model_extra=extra + "rope_original_max_pos = 16\n")) as d, \
+            drvmod.Driver(toml_config(**dict(kw, rope_factor=0.0))) as plain:
+        want = oracle.rope_inv_freq_yarn(128, 10000.0, 4.0, 8.0, 1.0, 16)
+        got = d.export_tensor("inv_freq", np.float32)
+        assert np.allclose(got, want, rtol=2e-6) and not np.allclose(got, plain.export_tensor("inv_freq", np.float32))
+        ms = d.export_tensor("info.rope_mscale", np.float32)[0]
+        assert abs(ms - (0.1 * np.log(4.0) + 1.0)) < 1e-6 and plain.export_tensor("info.rope_mscale", np.float32)[0] == 1.0
+        om, _ = oracle_model_from_driver(d, cfg)
+        assert om.cfg["rope_mscale"] == ms
+        prompts = ragged_prompts(rng, cfg["vocab"], 40, 2)     # contexts beyond the original 16 positions
+        _, near, checks = teacher_forced_compare(oracle, drvmod, d, om, cfg, prompts, 5)
+        assert checks == 10 and near <= 5
 
 
 def test_start_up_warm_up_changes_no_result(gpu):

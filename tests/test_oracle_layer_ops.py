@@ -170,3 +170,37 @@ def test_gemm_bf16_against_fp64(oracle):
     assert np.allclose(y2, truth, rtol=1e-6, atol=1e-6)
     assert np.allclose(y0, truth, rtol=0, atol=1e-4)
     assert np.array_equal(y0b, oracle.f32_to_bf16(y0))
+
+
+def test_yarn_frequencies_hand_worked(oracle):
+    """YaRN's frequency table (driver/cuda/src/kernels/rope.cu:495-507,552-589): with head_dim
+    128, theta 10000, an original context of 4096, beta_fast 32 and beta_slow 1 the correction
+    dims are 128 ln(4096 / (32 * 2 pi)) / (2 ln 10000) = 20.94 -> 20 and
+    128 ln(4096 / (2 pi)) / (2 ln 10000) = 45.03 -> 46: pairs up to 20 keep their frequency,
+    pairs from 46 on are divided by the factor, pair 33 sits exactly half way."""
+    d, theta, factor = 128, 10000.0, 4.0
+    f = oracle.rope_inv_freq_yarn(d, theta, factor, 32.0, 1.0, 4096).astype(np.float64)
+    base = theta ** (-2.0 * np.arange(d // 2) / d)
+    assert np.allclose(f[:21], base[:21], rtol=1e-6)
+    assert np.allclose(f[46:], base[46:] / factor, rtol=1e-6)
+    assert np.allclose(f[33], base[33] * (0.5 + 0.5 / factor), rtol=1e-6)
+    assert np.all(np.diff(f / base) <= 1e-6)                       # the ratio only falls along the ramp (f32 table)
+    assert np.all((f / base)[21:46] < 1.0) and np.all((f / base)[21:46] > 1.0 / factor)
+    # factor 1: nothing changes; a ramp that would pass the last pair is clipped to it
+    assert np.allclose(oracle.rope_inv_freq_yarn(d, theta, 1.0, 32.0, 1.0, 4096), base, rtol=1e-6)
+    g = oracle.rope_inv_freq_yarn(64, 10000.0, 8.0, 32.0, 1e-6, 4096).astype(np.float64)
+    b64 = 10000.0 ** (-2.0 * np.arange(32) / 64)
+    assert np.allclose(g[31], b64[31] / 8.0, rtol=1e-6)
+
+
+def test_scaled_rope_table_multiplies_cos_and_sin(oracle):
+    import ctypes as C
+
+    pos = np.array([0, 3, 1000], np.int32)
+    inv = oracle.rope_inv_freq(64, 10000.0)
+    plain = oracle.rope_table(pos, inv, 64)
+    out = np.zeros_like(plain)
+    oracle.lib().orc_rope_table_scaled(C.c_void_p(pos.ctypes.data), C.c_void_p(inv.ctypes.data),
+                                       C.c_void_p(out.ctypes.data), C.c_int(3), C.c_int(64), C.c_float(1.25))
+    assert np.array_equal(out, plain * np.float32(1.25))
+    assert np.allclose(out[0, :32], 1.25) and np.allclose(out[0, 32:], 0.0)
