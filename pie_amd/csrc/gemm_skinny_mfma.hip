@@ -416,31 +416,46 @@ struct WOne {
     uint16_t gs;
 };
 
-template <class F, int NG>
-__global__ __launch_bounds__(kSwWaves* kWave, NG == 1 ? 4 : 2) void skinny_wave_kernel(const SkinnyArgs a, const int kp_shift) {
+// MT row tiles of 16 per pass: a decoded weight fragment then feeds MT MFMAs, so a batch of 17
+// to 64 rows decodes the weights half as often.  The staged chunk shrinks by MT (the region and
+// the staging registers keep their size), so MT = 2 is the limit for int4 (one 128-k block).
+template <int MT>
+struct SwGeom {
+    static constexpr int chunk = kSwChunk / MT;         // k-values per staged chunk
+    static constexpr int stride = chunk / 8 + 1;        // 16-byte vectors per staged row (padded)
+    static constexpr int region = 16 * MT * stride;     // vectors per wave region
+};
+
+template <class F, int NG, int MT>
+__global__ __launch_bounds__(kSwWaves* kWave, NG == 1 && MT == 1 ? 4 : 2) void skinny_wave_kernel(const SkinnyArgs a, const int kp_shift) {
     constexpr int KPL = F::kPerLane, S = F::kSteps;
     constexpr int LK = 4 * KPL;                     // k covered by one wave-wide 16-byte load (a block)
-    constexpr int CB = kSwChunk / LK;               // blocks per chunk
+    constexpr int CHUNK = SwGeom<MT>::chunk, STRIDE = SwGeom<MT>::stride, REGION = SwGeom<MT>::region;
+    constexpr int CB = CHUNK / LK;                  // blocks per chunk
     constexpr int NS = NG * CB;                     // steps per chunk, tile-major order
     constexpr int PF = NS < 8 ? NS : 8;             // weight loads in flight per lane (deeper rings cost the occupancy that pays more)
     constexpr int CU = NS >= PF ? 1 : PF / NS;      // chunks per trip: ring slots stay compile-time
-    constexpr int SV = kSwRegion / kSwStride * (kSwChunk / 8) / kWave;   // staged vectors per lane and chunk
+    constexpr int VPR = CHUNK / 8;                  // staged vectors per row
+    constexpr int RPL = kWave / VPR;                // rows one wave-wide staging load covers
+    constexpr int SV = 16 * MT / RPL;               // staged vectors per lane and chunk
+    constexpr int ROWS = 16 * MT;                   // rows per pass
     constexpr bool kBiased = F::kBias != 0.f;
     constexpr bool kRowBias = kBiased && !F::kGroupScale;
-    static_assert((NS % PF == 0 || PF % NS == 0) && SV == 8, "ring and staging shapes");
+    static_assert(CB >= 1 && (NS % PF == 0 || PF % NS == 0) && SV == 8, "ring and staging shapes");
     extern __shared__ __align__(16) unsigned char smem[];
     const int tid = threadIdx.x, lane = tid & (kWave - 1);
     const int wv = __builtin_amdgcn_readfirstlane(tid / kWave);
     const int j = lane & 15, q = lane >> 4;
-    u32x4_t* lds_a = reinterpret_cast<u32x4_t*>(smem) + wv * kSwRegion;
+    u32x4_t* lds_a = reinterpret_cast<u32x4_t*>(smem) + wv * REGION;
     float* red = reinterpret_cast<float*>(smem);
-    constexpr int kRegionF = kSwRegion * 4;
+    constexpr int kRegionF = REGION * 4;
+    static_assert((NG + (kRowBias ? 1 : 0)) * 4 * kWave <= kRegionF, "a wave's partial sums of one row tile fit its region");
     const int KP = 1 << kp_shift;
     const int ks = wv & (KP - 1);
     const int N = a.N, K = a.K;
     const int p = a.offsets ? blockIdx.y : 0;
-    const int r0 = a.offsets ? a.offsets[p] : (a.m_split ? blockIdx.y * 16 : 0);
-    const int r1 = a.offsets ? a.offsets[p + 1] : (a.m_split ? min(a.M, r0 + 16) : a.M);
+    const int r0 = a.offsets ? a.offsets[p] : (a.m_split ? blockIdx.y * ROWS : 0);
+    const int r1 = a.offsets ? a.offsets[p + 1] : (a.m_split ? min(a.M, r0 + ROWS) : a.M);
     if (r1 <= r0) return;
 
     const int T = (N + 15) / 16;
@@ -486,19 +501,19 @@ __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 ? 4 : 2) void skinny_wave_
         return sl;
     };
 
-    // staging: a wave-wide load covers 512 bytes of each of two activation rows
-    const int srow = lane >> 5, svec = lane & 31;
+    // staging: a wave-wide load covers whole chunk rows (VPR vectors each) of RPL activation rows
+    const int srow = lane / VPR, svec = lane % VPR;
 
-    for (int mt0 = r0; mt0 < r1; mt0 += 16) {
+    for (int mt0 = r0; mt0 < r1; mt0 += ROWS) {
         // a pass of at most eight rows stages eight: the activations are re-read by every tile
         // group, so their traffic matters as much as the weights'.  Accumulator rows 8..15 then
         // repeat rows 0..7 and are never stored.
-        const bool r8 = r1 - mt0 <= 8;
+        const bool r8 = MT == 1 && r1 - mt0 <= 8;
         const int jr = r8 ? (j & 7) : j;
         int arow[SV];   // rows past the problem repeat its last row and are never stored
 #pragma unroll
         for (int u = 0; u < SV; ++u) {
-            const int row = min(mt0 + srow + 2 * u, r1 - 1);
+            const int row = min(mt0 + srow + RPL * u, r1 - 1);
             arow[u] = a.act_rows ? a.act_rows[row] : row;
         }
         u32x4_t stg[SV];
@@ -512,12 +527,16 @@ __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 ? 4 : 2) void skinny_wave_
         auto stage_store = [&]() {
 #pragma unroll
             for (int u = 0; u < SV; ++u)
-                if (u < SV / 2 || !r8) lds_a[(srow + 2 * u) * kSwStride + svec] = F::order(stg[u]);
+                if (u < SV / 2 || !r8) lds_a[(srow + RPL * u) * STRIDE + svec] = F::order(stg[u]);
         };
 
-        f32x4_t acc[NG], sxs[F::kGroupScale ? CB : 1], sxt = zero4;
+        f32x4_t acc[MT][NG], sxs[MT][F::kGroupScale ? CB : 1], sxt[MT];
 #pragma unroll
-        for (int i = 0; i < NG; ++i) acc[i] = zero4;
+        for (int t = 0; t < MT; ++t) {
+            sxt[t] = zero4;
+#pragma unroll
+            for (int i = 0; i < NG; ++i) acc[t][i] = zero4;
+        }
 
         WOne ring[PF];
 #pragma unroll
@@ -528,29 +547,35 @@ __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 ? 4 : 2) void skinny_wave_
         auto step = [&](const WOne& cur, int ng, int blk) {
             const int vbase = blk * (LK / 8) + q * S;
             const int sxi = F::kGroupScale ? blk : 0;
-            bf16x8_t ax[S];
+            f32x4_t part[MT];
 #pragma unroll
-            for (int s = 0; s < S; ++s) ax[s] = __builtin_bit_cast(bf16x8_t, lds_a[jr * kSwStride + vbase + s]);
-            f32x4_t part = zero4;
+            for (int t = 0; t < MT; ++t) part[t] = zero4;
 #pragma unroll
             for (int s = 0; s < S; ++s) {
                 const bf16x8_t bw = __builtin_bit_cast(bf16x8_t, F::decode(cur.w, s, magic));
-                if (kBiased && ng == 0) {
+#pragma unroll
+                for (int t = 0; t < MT; ++t) {
+                    const bf16x8_t ax = __builtin_bit_cast(bf16x8_t, lds_a[(t * 16 + jr) * STRIDE + vbase + s]);
+                    if (kBiased && ng == 0) {
+                        if (F::kGroupScale)
+                            sxs[t][sxi] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax, ones, s == 0 ? zero4 : sxs[t][sxi], 0, 0, 0);
+                        else
+                            sxt[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax, ones, sxt[t], 0, 0, 0);
+                    }
                     if (F::kGroupScale)
-                        sxs[sxi] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax[s], ones, s == 0 ? zero4 : sxs[sxi], 0, 0, 0);
+                        part[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax, bw, part[t], 0, 0, 0);
                     else
-                        sxt = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax[s], ones, sxt, 0, 0, 0);
+                        acc[t][ng] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax, bw, acc[t][ng], 0, 0, 0);
                 }
-                if (F::kGroupScale)
-                    part = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax[s], bw, part, 0, 0, 0);
-                else
-                    acc[ng] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax[s], bw, acc[ng], 0, 0, 0);
             }
             if (F::kGroupScale) {
-                if (ng == 0) sxs[sxi] = sxs[sxi] * F::kBias;
                 const float sc = bf16_bits_to_f32(cur.gs);
 #pragma unroll
-                for (int r = 0; r < 4; ++r) acc[ng][r] = fmaf(sc, part[r] + sxs[sxi][r], acc[ng][r]);
+                for (int t = 0; t < MT; ++t) {
+                    if (ng == 0) sxs[t][sxi] = sxs[t][sxi] * F::kBias;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) acc[t][ng][r] = fmaf(sc, part[t][r] + sxs[t][sxi][r], acc[t][ng][r]);
+                }
             }
         };
 
@@ -578,16 +603,20 @@ __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 ? 4 : 2) void skinny_wave_
             }
         }
 
-        // ---- the KP waves of a tile group meet; work item (tile i, accumulator row rr) ----
+        // ---- the KP waves of a tile group meet, one row tile at a time; work item (tile i,
+        // accumulator row rr) ----
+        const int nout = a.swiglu ? N / 2 : N;
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
         __syncthreads();
         float* mine = red + static_cast<size_t>(wv) * kRegionF;
 #pragma unroll
         for (int i = 0; i < NG; ++i)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) mine[(i * 4 + r) * kWave + lane] = acc[i][r];
+            for (int r = 0; r < 4; ++r) mine[(i * 4 + r) * kWave + lane] = acc[t][i][r];
         if (kRowBias) {
 #pragma unroll
-            for (int r = 0; r < 4; ++r) mine[(NG * 4 + r) * kWave + lane] = sxt[r];
+            for (int r = 0; r < 4; ++r) mine[(NG * 4 + r) * kWave + lane] = sxt[t][r];
         }
         __syncthreads();
         const float* grp = red + static_cast<size_t>(wv - ks) * kRegionF;
@@ -596,10 +625,9 @@ __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 ? 4 : 2) void skinny_wave_
             for (int w = 0; w < KP; ++w) v += grp[static_cast<size_t>(w) * kRegionF + (item * 4 + rr) * kWave + lane];
             return v;
         };
-        const int nout = a.swiglu ? N / 2 : N;
         for (int id = ks; id < NG * 4; id += KP) {
             const int i = id >> 2, rr = id & 3;
-            const int m = mt0 + 4 * q + rr;
+            const int m = mt0 + 16 * t + 4 * q + rr;
             const float bias = kRowBias ? F::kBias * total(NG, rr) : 0.f;
             float rs = row_scale[0];
 #pragma unroll
@@ -650,32 +678,33 @@ __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 ? 4 : 2) void skinny_wave_
                 a.y[o] = f32_to_bf16_bits(v);
             }
         }
+        }
         __syncthreads();   // the regions go back to staging
     }
 }
 
-template <class F, int NG>
+template <class F, int NG, int MT>
 int launch_wave_cfg(const SkinnyArgs& a, int problems, int kp_shift, hipStream_t stream) {
-    constexpr size_t smem = static_cast<size_t>(kSwWaves) * kSwRegion * 16;
+    constexpr size_t smem = static_cast<size_t>(kSwWaves) * SwGeom<MT>::region * 16;
     static const hipError_t attr = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(&skinny_wave_kernel<F, NG>),
+        reinterpret_cast<const void*>(&skinny_wave_kernel<F, NG, MT>),
         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
     if (attr != hipSuccess) return PIE_HIP_ERR_LAUNCH;
     const int tgroups = ((a.N + 15) / 16 + NG - 1) / NG;
     const int per_block = kSwWaves >> kp_shift;
-    const dim3 grid((tgroups + per_block - 1) / per_block, a.m_split ? (a.M + 15) / 16 : problems);
-    hipLaunchKernelGGL((skinny_wave_kernel<F, NG>), grid, dim3(kSwWaves * kWave), smem, stream, a, kp_shift);
+    const dim3 grid((tgroups + per_block - 1) / per_block, a.m_split ? (a.M + 16 * MT - 1) / (16 * MT) : problems);
+    hipLaunchKernelGGL((skinny_wave_kernel<F, NG, MT>), grid, dim3(kSwWaves * kWave), smem, stream, a, kp_shift);
     return launch_status();
 }
 
 // Tiles per wave and K split: the most tiles per wave (activation staging and the bias MFMAs
 // are paid once per chunk, whatever the tile count) that still gives the machine about eight
 // waves per CU.
-template <class F>
-int launch_wave(const SkinnyArgs& a, int problems, hipStream_t stream) {
-    constexpr int LK = 4 * F::kPerLane, CB = kSwChunk / LK;
+template <class F, int MT>
+int launch_wave_mt(const SkinnyArgs& a, int problems, hipStream_t stream) {
+    constexpr int LK = 4 * F::kPerLane, CB = SwGeom<MT>::chunk / LK;
     const int nch_all = (a.K / LK + CB - 1) / CB;
-    const long mult = a.m_split ? (a.M + 15) / 16 : problems;
+    const long mult = a.m_split ? (a.M + 16 * MT - 1) / (16 * MT) : problems;
     const long tiles = (a.N + 15) / 16;
     static const int force_ng = [] { const char* e = getenv("PIE_SKINNY_NG"); return e ? atoi(e) : 0; }();
     static const int force_kp = [] { const char* e = getenv("PIE_SKINNY_KP"); return e ? atoi(e) : -1; }();
@@ -685,7 +714,7 @@ int launch_wave(const SkinnyArgs& a, int problems, hipStream_t stream) {
     int ng = 1, kp_shift = 0;
     for (int cand = 4; cand >= 1; cand >>= 1) {
         const long groups = (tiles + cand - 1) / cand * mult;
-        const long cap = 256L * (cand == 1 ? 16 : 8);
+        const long cap = 256L * (cand == 1 && MT == 1 ? 16 : 8);
         int sh = 0;
         while (sh < 3 && (groups << (sh + 1)) <= cap && (2 << sh) <= nch_all) ++sh;
         if ((groups << sh) >= 1100 || cand == 1) {
@@ -697,10 +726,21 @@ int launch_wave(const SkinnyArgs& a, int problems, hipStream_t stream) {
     if (force_ng) ng = force_ng;
     if (force_kp >= 0) kp_shift = force_kp;
     switch (ng) {
-        case 4: return launch_wave_cfg<F, 4>(a, problems, kp_shift, stream);
-        case 2: return launch_wave_cfg<F, 2>(a, problems, kp_shift, stream);
-        default: return launch_wave_cfg<F, 1>(a, problems, kp_shift, stream);
+        case 4: return launch_wave_cfg<F, 4, MT>(a, problems, kp_shift, stream);
+        case 2: return launch_wave_cfg<F, 2, MT>(a, problems, kp_shift, stream);
+        default: return launch_wave_cfg<F, 1, MT>(a, problems, kp_shift, stream);
     }
+}
+
+template <class F>
+int launch_wave(const SkinnyArgs& a, int problems, hipStream_t stream) {
+    static const int force_mt = [] { const char* e = getenv("PIE_SKINNY_MT"); return e ? atoi(e) : 0; }();
+    // dense launches of more than 32 rows: 32-row passes (measured on the 8B shapes: a 48 / 64
+    // row decode step 4.63 / 4.88 -> 4.26 / 4.61 ms; at 17..32 rows the shorter chunks cost
+    // more than the second pass saves, 3.40 -> 3.47 ms)
+    const bool two = force_mt ? force_mt == 2 : (!a.offsets && a.M > 32);
+    if (two && a.K % SwGeom<2>::chunk == 0) return launch_wave_mt<F, 2>(a, problems, stream);
+    return launch_wave_mt<F, 1>(a, problems, stream);
 }
 
 template <class F, int KP, int CK, int NG, int PW, int WL, bool TILED>

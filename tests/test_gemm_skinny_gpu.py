@@ -183,7 +183,9 @@ def test_tile_major_repack_is_the_documented_permutation(gpu, oracle, kind, N, K
                                    # long K: seven chunks per K slice; 1536: a K slice left empty
                                    (6, 64, 14336), (32, 1040, 1536), (1, 4096, 4096), (3, 8192, 1024),
                                    # fewer rows than a tile (a router), two passes over small matrices
-                                   (21, 8, 512), (21, 768, 512), (21, 512, 512), (130, 72, 1024)])
+                                   (21, 8, 512), (21, 768, 512), (21, 512, 512), (130, 72, 1024),
+                                   # 32-row passes (more than 32 rows): whole, ragged, K split over waves
+                                   (64, 1040, 1536), (48, 4096, 2048), (33, 256, 4096)])
 def test_skinny_over_tile_major_weights_matches_oracle_and_row_major(gpu, oracle, kind, M, N, K):
     """Tile-major weights run the wave-private kernel (another split of K, so another sum order):
     same bar against the oracle as the row-major path, and within one bf16 step of that path on
@@ -204,16 +206,18 @@ def test_skinny_over_tile_major_weights_matches_oracle_and_row_major(gpu, oracle
 
 
 @pytest.mark.parametrize("kind", KINDS)
-def test_skinny_tile_major_one_hot_rows_are_exact(gpu, oracle, kind):
+@pytest.mark.parametrize("M", [16, 48])
+def test_skinny_tile_major_one_hot_rows_are_exact(gpu, oracle, kind, M):
     """One-hot activations over tile-major weights: y[m, n] is bf16(dequantised w[n, k_m]) exactly,
-    whatever K slice and chunk k_m falls in."""
+    whatever K slice and chunk k_m falls in (48 rows: the 32-row passes, the second half empty)."""
     import torch
     from pie_amd import ops
 
     rng = np.random.default_rng(341)
-    M, N, K = 16, 96, 4096
+    N, K = 96, 4096
     wd, mk = make_weight(oracle, rng, kind, N, K)
     ks = np.array([0, 1, 7, 8, 31, 127, 128, 255, 256, 511, 512, 1023, 2048, 3000, 4094, 4095])
+    ks = np.concatenate([ks, (ks * 7 + 3) % K, (ks * 13 + 130) % K])[:M]
     x = np.zeros((M, K), dtype=np.float32)
     x[np.arange(M), ks] = 1.0
     xb = oracle.f32_to_bf16(x)
