@@ -216,8 +216,8 @@ def attention_case():
     for fmt in ("fp8_per_token_head", "int8_per_token_head"):
         k8 = torch.randint(0, 120, (total, ps, hk, d), dtype=torch.uint8, device=dev)
         v8 = torch.randint(0, 120, (total, ps, hk, d), dtype=torch.uint8, device=dev)
-        ks = torch.rand(total, ps, hk, device=dev) * 0.01 + 0.001
-        vs = torch.rand(total, ps, hk, device=dev) * 0.01 + 0.001
+        ks = torch.rand(total, hk, ps, device=dev) * 0.01 + 0.001
+        vs = torch.rand(total, hk, ps, device=dev) * 0.01 + 0.001
         keep.append((k8, v8, ks, vs))
         launch[fmt] = (lambda fmt=fmt, k8=k8, v8=v8, ks=ks, vs=vs:
                        ops.attention_rows_paged_kvq(fmt, q, k8, v8, ks, vs, pi, rb, rl, max_kv_len=maxlen,

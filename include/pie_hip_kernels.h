@@ -477,7 +477,7 @@ int pie_hip_attn_rows_paged_static(const uint16_t* q, const uint16_t* k_pages,
  * KV-cache storage formats of the pool (the CUDA driver's kv_cache_dtype values,
  * driver/cuda/src/kv_cache_format.cpp:46-110).  One-byte formats keep the bf16 layout
  * [pages, page_size, hk, d] with one byte per element; the per-token-head formats add fp32 side
- * scales [pages, page_size, hk] for K and for V.  The fp4 block formats are not implemented
+ * scales [pages, hk, page_size] for K and for V (see pie_hip_kv_write_quant).  The fp4 block formats are not implemented
  * (PIE_HIP_ERR_UNSUPPORTED).
  */
 enum {
@@ -518,14 +518,17 @@ int pie_hip_attn_rows_paged_kvq_masked(int kv_format, const uint16_t* q, const v
  * slot kv_slots[t] of a one-byte pool (slot < 0: skipped).  Per-token-head formats:
  * scale = absmax / qmax (qmax 127 / 448; 1 for an all-zero row), code = x * (1/scale) rounded
  * to nearest even, clamped / saturated; PIE_HIP_KV_FP8_E4M3 / _E5M2: the saturating cast of x
- * (largest finite value 448 / 57344).
+ * (largest finite value 448 / 57344).  The fp32 scale pools are laid out
+ * [pages, kv heads, page_size] (the 16 scales an attention block reads for one page and head are
+ * contiguous; a page's scales are one run, so page copies move them like the codes): the scale of
+ * slot s and head h sits at ((s / page_size) * hk + h) * page_size + s % page_size.
  * Reference: write_kv_per_token_head_kernel and write_kv_fp8_per_tensor_kernel,
  * driver/cuda/src/kernels/kv_paged.cu:155-297.
  */
 int pie_hip_kv_write_quant(int kv_format, const uint16_t* k_rows, const uint16_t* v_rows,
                            const int64_t* kv_slots, void* k_pages, void* v_pages, float* k_scales,
                            float* v_scales, int num_tokens, int num_kv_heads, int head_dim,
-                           void* stream);
+                           int page_size, void* stream);
 /* pie_hip_qkv_rope_kvwrite and pie_hip_kv_write_quant in one launch for one-byte pools: every
  * (token, head) of the packed q|k|v rows is rotated (optional per-head q/k RMSNorm, either
  * pairing) and rounded to bf16 as by pie_hip_qkv_rope_kvwrite; q goes to q_out, the K and V
@@ -536,8 +539,8 @@ int pie_hip_qkv_rope_kvwrite_quant(int kv_format, const uint16_t* packed_qkv, ui
                                    void* k_pages, void* v_pages, float* k_scales, float* v_scales,
                                    const uint16_t* q_norm_weight, const uint16_t* k_norm_weight,
                                    const float* rope_table, const int64_t* kv_slots, int num_tokens,
-                                   int num_q_heads, int num_kv_heads, int head_dim, int interleaved,
-                                   float eps, void* stream);
+                                   int num_q_heads, int num_kv_heads, int head_dim, int page_size,
+                                   int interleaved, float eps, void* stream);
 
 /* ---- per-layer kernels of the llama-like decoder ---------------------------- */
 

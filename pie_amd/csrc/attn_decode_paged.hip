@@ -132,7 +132,8 @@ __global__ __launch_bounds__(kAttnBlock) void attn_decode_split_kernel(
             u.k[i] = __builtin_nontemporal_load(reinterpret_cast<const KV*>(k_pages + off));
             u.v[i] = __builtin_nontemporal_load(reinterpret_cast<const KV*>(v_pages + off));
             if constexpr (KVF != kKvBf16) {
-                const size_t th = (slot0 + i * TPI + grp) * hk + kvh;
+                // (a unit of tokens lies inside one page)
+                const size_t th = kv_scale_index(pid, tok0 - page * ps + i * TPI + grp, kvh, hk, ps);
                 u.ks[i] = k_scales ? k_scales[th] : 1.f;
                 u.vs[i] = v_scales ? v_scales[th] : 1.f;
             }
@@ -420,6 +421,11 @@ __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
             const size_t slot_idx = static_cast<size_t>(in_a ? pid_a : pid_b) * ps + (j - (in_a ? pa_end - ps : pa_end));
             return slot_idx * hk + kvh;
         };
+        auto row_sc = [&](int key) {   // the key's place in a scale pool
+            const int j = min(j0 + key, k_end - 1);
+            const bool in_a = j < pa_end;
+            return kv_scale_index(in_a ? pid_a : pid_b, j - (in_a ? pa_end - ps : pa_end), kvh, hk, ps);
+        };
 #pragma unroll
         for (int i = 0; i < NK; ++i)
             kreg[slot][i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(
@@ -434,7 +440,7 @@ __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
         }
         if constexpr (Q8) {
             const float* sp = lane < kMStepKeys ? k_scales : v_scales;
-            sreg[slot] = sp ? sp[row_th(lane & (kMStepKeys - 1))] : 1.f;
+            sreg[slot] = sp ? sp[row_sc(lane & (kMStepKeys - 1))] : 1.f;
         }
         if constexpr (MASKED) {   // (the second unit may lie past the context: its keys are dropped anyway)
             const uint16_t* mrow = mask_bits + static_cast<size_t>(r) * mask_stride;
@@ -472,13 +478,11 @@ __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
             } else {   // 16 elements of two adjacent keys: (bf16(a_e), bf16(b_e)) pairs
 #pragma unroll
                 for (int h = 0; h < 2; ++h) {
-                    float fa[8], fb[8];
-                    kv_decode_f32<KVF>(u32x2_t{a[2 * h], a[2 * h + 1]}, fa);
-                    kv_decode_f32<KVF>(u32x2_t{b[2 * h], b[2 * h + 1]}, fb);
+                    uint32_t ab[8];
+                    kv_decode_bf16_pairs<KVF>(u32x2_t{a[2 * h], a[2 * h + 1]}, u32x2_t{b[2 * h], b[2 * h + 1]}, ab);
 #pragma unroll
                     for (int e = 0; e < 8; ++e)
-                        *reinterpret_cast<uint32_t*>(&Vt[vt_at(dc * 16 + 8 * h + e, col)]) =
-                            kv_pack_trunc(fa[e], fb[e]);
+                        *reinterpret_cast<uint32_t*>(&Vt[vt_at(dc * 16 + 8 * h + e, col)]) = ab[e];
                 }
             }
         }
@@ -1074,7 +1078,7 @@ __global__ __launch_bounds__(256) void kv_write_quant_kernel(
     const uint16_t* __restrict__ k_src, const uint16_t* __restrict__ v_src,
     const int64_t* __restrict__ kv_slots, unsigned char* __restrict__ k_pages,
     unsigned char* __restrict__ v_pages, float* __restrict__ k_scales,
-    float* __restrict__ v_scales, int n_rows, int hk, int d, int kv_format) {
+    float* __restrict__ v_scales, int n_rows, int hk, int d, int ps, int kv_format) {
     const int lane = threadIdx.x & (kWave - 1);
     const int row = blockIdx.x * (256 / kWave) + threadIdx.x / kWave;   // (token, head)
     if (row >= n_rows) return;
@@ -1084,6 +1088,7 @@ __global__ __launch_bounds__(256) void kv_write_quant_kernel(
     const size_t src = static_cast<size_t>(row) * d;
     const size_t th = static_cast<size_t>(slot) * hk + h;
     const bool scaled = kv_format != PIE_HIP_KV_FP8_E4M3 && kv_format != PIE_HIP_KV_FP8_E5M2;
+    const size_t sc_at = scaled ? kv_scale_index_of_slot(slot, h, hk, ps) : 0;
     const float qmax = kv_format == PIE_HIP_KV_INT8_PER_TOKEN_HEAD ? 127.f : 448.f;
 #pragma unroll
     for (int which = 0; which < 2; ++which) {
@@ -1096,7 +1101,7 @@ __global__ __launch_bounds__(256) void kv_write_quant_kernel(
             amax = wave_max(amax);
             const float scale = amax > 0.f ? amax / qmax : 1.f;
             inv = 1.f / scale;
-            if (lane == 0) (which ? v_scales : k_scales)[th] = scale;
+            if (lane == 0) (which ? v_scales : k_scales)[sc_at] = scale;
         }
         for (int j = lane; j < d; j += kWave) {
             const float f = bf16_bits_to_f32(x[src + j]) * inv;
@@ -1125,7 +1130,7 @@ __global__ __launch_bounds__(64) void qkv_rope_kvwrite_quant_kernel(
     float* __restrict__ k_scales, float* __restrict__ v_scales,
     const uint16_t* __restrict__ q_norm_w, const uint16_t* __restrict__ k_norm_w,
     const float* __restrict__ rope_table, const int64_t* __restrict__ kv_slots, int hq, int hk,
-    int d, int interleaved, float eps, int kv_format) {
+    int d, int ps, int interleaved, float eps, int kv_format) {
     const int n = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
     const int half = d / 2;
     const size_t stride = static_cast<size_t>(hq + 2 * hk) * d;
@@ -1190,7 +1195,7 @@ __global__ __launch_bounds__(64) void qkv_rope_kvwrite_quant_kernel(
         amax = wave_max(amax);
         const float scale = amax > 0.f ? amax / qmax : 1.f;
         inv = 1.f / scale;
-        if (lane == 0) (is_k ? k_scales : v_scales)[th] = scale;
+        if (lane == 0) (is_k ? k_scales : v_scales)[kv_scale_index_of_slot(slot, h, hk, ps)] = scale;
     }
     auto code = [&](float x) {
         const float f = x * inv;
@@ -1222,11 +1227,11 @@ extern "C" int pie_hip_qkv_rope_kvwrite_quant(int kv_format, const uint16_t* pac
                                               float* v_scales, const uint16_t* q_norm_weight,
                                               const uint16_t* k_norm_weight, const float* rope_table,
                                               const int64_t* kv_slots, int num_tokens, int num_q_heads,
-                                              int num_kv_heads, int head_dim, int interleaved, float eps,
-                                              void* stream) {
+                                              int num_kv_heads, int head_dim, int page_size,
+                                              int interleaved, float eps, void* stream) {
     using namespace pie_hip;
     if (!packed_qkv || !q_out || !k_pages || !v_pages || !rope_table || !kv_slots || num_tokens <= 0 ||
-        num_q_heads <= 0 || num_kv_heads <= 0 || head_dim <= 0)
+        num_q_heads <= 0 || num_kv_heads <= 0 || head_dim <= 0 || page_size <= 0)
         return PIE_HIP_ERR_INVALID;
     if (!q_norm_weight != !k_norm_weight) return PIE_HIP_ERR_INVALID;
     const bool scaled = kv_format == PIE_HIP_KV_INT8_PER_TOKEN_HEAD || kv_format == PIE_HIP_KV_FP8_PER_TOKEN_HEAD;
@@ -1240,21 +1245,21 @@ extern "C" int pie_hip_qkv_rope_kvwrite_quant(int kv_format, const uint16_t* pac
     if (head_dim <= 128)
         hipLaunchKernelGGL(qkv_rope_kvwrite_quant_kernel<1>, grid, dim3(64), 0, st, packed_qkv, q_out, kp, vp,
                            k_scales, v_scales, q_norm_weight, k_norm_weight, rope_table, kv_slots,
-                           num_q_heads, num_kv_heads, head_dim, interleaved, eps, kv_format);
+                           num_q_heads, num_kv_heads, head_dim, page_size, interleaved, eps, kv_format);
     else
         hipLaunchKernelGGL(qkv_rope_kvwrite_quant_kernel<2>, grid, dim3(64), 0, st, packed_qkv, q_out, kp, vp,
                            k_scales, v_scales, q_norm_weight, k_norm_weight, rope_table, kv_slots,
-                           num_q_heads, num_kv_heads, head_dim, interleaved, eps, kv_format);
+                           num_q_heads, num_kv_heads, head_dim, page_size, interleaved, eps, kv_format);
     return launch_status();
 }
 
 extern "C" int pie_hip_kv_write_quant(int kv_format, const uint16_t* k_rows, const uint16_t* v_rows,
                                       const int64_t* kv_slots, void* k_pages, void* v_pages,
                                       float* k_scales, float* v_scales, int num_tokens,
-                                      int num_kv_heads, int head_dim, void* stream) {
+                                      int num_kv_heads, int head_dim, int page_size, void* stream) {
     using namespace pie_hip;
     if (!k_rows || !v_rows || !kv_slots || !k_pages || !v_pages || num_tokens < 0 || num_kv_heads <= 0 ||
-        head_dim <= 0)
+        head_dim <= 0 || page_size <= 0)
         return PIE_HIP_ERR_INVALID;
     const bool scaled = kv_format == PIE_HIP_KV_INT8_PER_TOKEN_HEAD || kv_format == PIE_HIP_KV_FP8_PER_TOKEN_HEAD;
     if (kv_format != PIE_HIP_KV_FP8_E4M3 && kv_format != PIE_HIP_KV_FP8_E5M2 && !scaled) return PIE_HIP_ERR_UNSUPPORTED;
@@ -1264,7 +1269,7 @@ extern "C" int pie_hip_kv_write_quant(int kv_format, const uint16_t* k_rows, con
     hipLaunchKernelGGL(kv_write_quant_kernel, dim3((rows + 3) / 4), dim3(256), 0,
                        static_cast<hipStream_t>(stream), k_rows, v_rows, kv_slots,
                        static_cast<unsigned char*>(k_pages), static_cast<unsigned char*>(v_pages), k_scales,
-                       v_scales, rows, num_kv_heads, head_dim, kv_format);
+                       v_scales, rows, num_kv_heads, head_dim, page_size, kv_format);
     return launch_status();
 }
 

@@ -138,6 +138,11 @@ __global__ __launch_bounds__(kTileThreads) void attn_prefill_tile_kernel(
             const uint32_t pid = page == page_a ? pid_a : pid_b;
             return (static_cast<size_t>(pid) * ps + (j - page * ps)) * hk + kvh;
         };
+        auto token_sc = [&](int key) {   // the key's place in a scale pool
+            const int j = min(j0 + key, kmax - 1);
+            const int page = j / ps;
+            return kv_scale_index(page == page_a ? pid_a : pid_b, j - page * ps, kvh, hk, ps);
+        };
         if constexpr (Q8) {
             int key, dc;
             piece_of(0, key, dc);
@@ -148,7 +153,7 @@ __global__ __launch_bounds__(kTileThreads) void attn_prefill_tile_kernel(
             }
             if (tid < 2 * kStepKeys) {
                 const float* sp = tid < kStepKeys ? k_scales : v_scales;
-                sreg[slot] = sp ? sp[token_head(tid % kStepKeys)] : 1.f;
+                sreg[slot] = sp ? sp[token_sc(tid % kStepKeys)] : 1.f;
             }
             return;
         }

@@ -121,6 +121,20 @@ __device__ __forceinline__ float wave_max(float v) {
 // does (driver/cuda/src/ops/attention_naive_paged.cu:56-112): float(code) * scale.
 constexpr int kKvBf16 = 0, kKvFp8 = 1, kKvInt8 = 2, kKvBf8 = 3;   // (kKvBf8: e5m2 casts, "fp8_e5m2")
 
+// Scale pools are laid out [pages, kv heads, page_size]: the scales a (page, head) block of an
+// attention launch reads are contiguous (64 bytes for 16 tokens), where [pages, page_size,
+// kv heads] spread them over one 32-byte sector per token that every head's block fetches
+// again.  A page's scales stay one contiguous run, so page copies move them like the codes.
+__device__ __forceinline__ size_t kv_scale_index(size_t page, int in_page, int head, int hk, int ps) {
+    return (page * hk + head) * ps + in_page;
+}
+__device__ __forceinline__ size_t kv_scale_index_of_slot(int64_t slot, int head, int hk, int ps) {
+    const uint64_t page = static_cast<uint64_t>(slot) < 0x80000000ull
+                              ? static_cast<uint32_t>(slot) / static_cast<uint32_t>(ps)
+                              : static_cast<uint64_t>(slot) / static_cast<uint32_t>(ps);
+    return kv_scale_index(page, static_cast<int>(static_cast<uint64_t>(slot) - page * ps), head, hk, ps);
+}
+
 template <int KVF>
 struct KvVec {
     using type = u32x4_t;
@@ -169,11 +183,52 @@ template <int KVF>
 __device__ __forceinline__ u32x4_t kv_decode_bf16(const typename KvVec<KVF>::type r) {
     if constexpr (KVF == kKvBf16) {
         return r;
+    } else if constexpr (KVF == kKvFp8 || KVF == kKvBf8) {
+        // two codes -> a bf16 pair in one instruction (scale 1: every code is exact in bf16)
+        typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+#define PIE_KV_TWO(w, hi)                                                                                       \
+    (KVF == kKvFp8 ? __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((w), 1.0f, (hi))) \
+                   : __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_bf8((w), 1.0f, (hi))))
+        return u32x4_t{PIE_KV_TWO(r.x, false), PIE_KV_TWO(r.x, true), PIE_KV_TWO(r.y, false), PIE_KV_TWO(r.y, true)};
+#undef PIE_KV_TWO
     } else {
         float f[8];
         kv_decode_f32<KVF>(r, f);
         return u32x4_t{kv_pack_trunc(f[0], f[1]), kv_pack_trunc(f[2], f[3]), kv_pack_trunc(f[4], f[5]),
                        kv_pack_trunc(f[6], f[7])};
+    }
+}
+
+// 8 stored elements of each of two rows -> the 8 pairs (bf16(a_e), bf16(b_e)), a_e in the low half
+template <int KVF>
+__device__ __forceinline__ void kv_decode_bf16_pairs(const typename KvVec<KVF>::type a,
+                                                     const typename KvVec<KVF>::type b, uint32_t* out) {
+    static_assert(KVF != kKvBf16, "one-byte formats only");
+    if constexpr (KVF == kKvFp8 || KVF == kKvBf8) {
+        typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+#pragma unroll
+        for (int w = 0; w < 2; ++w) {
+            // bytes (a0, b0, a1, b1) and (a2, b2, a3, b3) of this word, then two codes per conversion
+            const uint32_t m0 = __builtin_amdgcn_perm(b[w], a[w], 0x05010400u);
+            const uint32_t m1 = __builtin_amdgcn_perm(b[w], a[w], 0x07030602u);
+            if constexpr (KVF == kKvFp8) {
+                out[4 * w + 0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(m0, 1.0f, false));
+                out[4 * w + 1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(m0, 1.0f, true));
+                out[4 * w + 2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(m1, 1.0f, false));
+                out[4 * w + 3] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(m1, 1.0f, true));
+            } else {
+                out[4 * w + 0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_bf8(m0, 1.0f, false));
+                out[4 * w + 1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_bf8(m0, 1.0f, true));
+                out[4 * w + 2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_bf8(m1, 1.0f, false));
+                out[4 * w + 3] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_bf8(m1, 1.0f, true));
+            }
+        }
+    } else {
+        float fa[8], fb[8];
+        kv_decode_f32<KVF>(a, fa);
+        kv_decode_f32<KVF>(b, fb);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) out[e] = kv_pack_trunc(fa[e], fb[e]);
     }
 }
 

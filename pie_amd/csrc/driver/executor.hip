@@ -382,12 +382,12 @@ void Executor::body(int N, int S, int max_kv_len) {
             // rotation and quantising write in one launch; head dims past 256 take the two kernels
             const int st = pie_hip_qkv_rope_kvwrite_quant(kv_format_, qkv_, q_, k_pool_[l], v_pool_[l], ksc, vsc,
                                                           w.q_norm, w.k_norm, rope_tab_, slots, N, hq, hk, d,
-                                                          pairing, m.rms_eps, s);
+                                                          page_size_, pairing, m.rms_eps, s);
             if (st == PIE_HIP_ERR_UNSUPPORTED) {
                 PIE_KERNEL(pie_hip_qkv_rope_kvwrite(qkv_, q_, k_rows_, v_rows_, w.q_norm, w.k_norm, rope_tab_,
                                                     iota_slots_, N, hq, hk, d, pairing, m.rms_eps, s));
                 PIE_KERNEL(pie_hip_kv_write_quant(kv_format_, k_rows_, v_rows_, slots, k_pool_[l], v_pool_[l],
-                                                  ksc, vsc, N, hk, d, s));
+                                                  ksc, vsc, N, hk, d, page_size_, s));
             } else {
                 PIE_KERNEL(st);
             }

@@ -112,7 +112,7 @@ class Executor {
 
     std::vector<uint16_t*> k_pool_, v_pool_;  // per layer [pages, ps, hk, d] (bf16 or one byte per element)
     int kv_format_ = 0;                        // PIE_HIP_KV_*
-    std::vector<float*> k_scale_pool_, v_scale_pool_;   // per layer [pages, ps, hk], scaled formats
+    std::vector<float*> k_scale_pool_, v_scale_pool_;   // per layer [pages, hk, ps], scaled formats
     uint16_t *k_rows_ = nullptr, *v_rows_ = nullptr;     // this step's rotated K / V rows before quantisation
     int64_t* iota_slots_ = nullptr;                      // 0, 1, 2, ...: row t of k_rows_ is "slot" t
     unsigned char* swap_pool_ = nullptr;       // pinned: [layer][K|V][cpu_pages] pages (+ their scales)

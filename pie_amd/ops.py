@@ -822,7 +822,7 @@ def attention_prefill_tiles_kvq(fmt: str, q: torch.Tensor, k_pages: torch.Tensor
                                 kv_page_indices: torch.Tensor, row_page_begin: torch.Tensor,
                                 row_kv_len: torch.Tensor, tile_row_start: torch.Tensor,
                                 tile_num_rows: torch.Tensor, rows_per_tile: Optional[int] = None) -> torch.Tensor:
-    """`attention_prefill_tiles` over one-byte pools [pages, ps, hk, d] (+ f32 scales [pages, ps, hk])."""
+    """`attention_prefill_tiles` over one-byte pools [pages, ps, hk, d] (+ f32 scales [pages, hk, ps])."""
     _dev(q, torch.bfloat16, "q")
     for name, t in (("kv_page_indices", kv_page_indices), ("row_page_begin", row_page_begin),
                     ("row_kv_len", row_kv_len), ("tile_row_start", tile_row_start),
@@ -848,7 +848,7 @@ def kv_write_quant(fmt: str, k_rows: torch.Tensor, v_rows: torch.Tensor, kv_slot
                    k_scales: Optional[torch.Tensor] = None,
                    v_scales: Optional[torch.Tensor] = None) -> None:
     """Quantising KV write of rows [N, hk, d] bf16 into one-byte pools [pages, ps, hk, d]
-    (+ f32 scales [pages, ps, hk] for the per-token-head formats)."""
+    (+ f32 scales [pages, hk, ps] for the per-token-head formats)."""
     _dev(k_rows, torch.bfloat16, "k_rows")
     _dev(v_rows, torch.bfloat16, "v_rows")
     _dev(kv_slots, torch.int64, "kv_slots")
@@ -864,10 +864,10 @@ def kv_write_quant(fmt: str, k_rows: torch.Tensor, v_rows: torch.Tensor, kv_slot
         if sc is not None:
             _dev(sc, torch.float32, "scales")
             if sc.numel() != k_pages.numel() // d:
-                raise KernelError("scales must be [pages, ps, hk]")
+                raise KernelError("scales must be [pages, hk, ps]")
     _check(kernels().pie_hip_kv_write_quant(KV_FORMATS[fmt], _ptr(k_rows), _ptr(v_rows), _ptr(kv_slots),
                                             _ptr(k_pages), _ptr(v_pages), _ptr(k_scales), _ptr(v_scales),
-                                            N, hk, d, _stream()), "pie_hip_kv_write_quant")
+                                            N, hk, d, k_pages.shape[1], _stream()), "pie_hip_kv_write_quant")
 
 
 def qkv_rope_kvwrite_quant(fmt: str, packed: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
@@ -891,12 +891,12 @@ def qkv_rope_kvwrite_quant(fmt: str, packed: torch.Tensor, k_pages: torch.Tensor
         if sc is not None:
             _dev(sc, torch.float32, "scales")
             if sc.numel() != k_pages.numel() // d:
-                raise KernelError("scales must be [pages, ps, hk]")
+                raise KernelError("scales must be [pages, hk, ps]")
     q_out = torch.empty((N, hq, d), dtype=torch.bfloat16, device=packed.device)
     _check(kernels().pie_hip_qkv_rope_kvwrite_quant(
         KV_FORMATS[fmt], _ptr(packed), _ptr(q_out), _ptr(k_pages), _ptr(v_pages), _ptr(k_scales),
         _ptr(v_scales), _ptr(q_norm_w), _ptr(k_norm_w), _ptr(table), _ptr(kv_slots), N, hq, hk, d,
-        int(interleaved), C.c_float(eps), _stream()), "pie_hip_qkv_rope_kvwrite_quant")
+        k_pages.shape[1], int(interleaved), C.c_float(eps), _stream()), "pie_hip_qkv_rope_kvwrite_quant")
     return q_out
 
 

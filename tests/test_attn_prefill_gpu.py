@@ -92,8 +92,8 @@ def test_tiles_over_one_byte_pools_match_the_oracle(gpu, oracle, fmt, hq, hk, d,
     kp = torch.zeros((pages, ps, hk, d), dtype=torch.uint8, device=gpu)
     vp = torch.zeros_like(kp)
     scaled = fmt not in ("fp8_e4m3", "fp8_e5m2")
-    ks = torch.ones((pages, ps, hk), dtype=torch.float32, device=gpu) if scaled else None
-    vs = torch.ones((pages, ps, hk), dtype=torch.float32, device=gpu) if scaled else None
+    ks = torch.ones((pages, hk, ps), dtype=torch.float32, device=gpu) if scaled else None
+    vs = torch.ones((pages, hk, ps), dtype=torch.float32, device=gpu) if scaled else None
     slots = dev(np.arange(pages * ps, dtype=np.int64))
     ops.kv_write_quant(fmt, dev(b["k_pages"], torch.bfloat16).reshape(pages * ps, hk, d),
                        dev(b["v_pages"], torch.bfloat16).reshape(pages * ps, hk, d), slots, kp, vp, ks, vs)

@@ -28,8 +28,9 @@ def test_kv_write_quant_bit_exact(gpu, oracle, fmt, hk, d):
     kp = torch.full((pages, ps, hk, d), 0x55, dtype=torch.uint8, device=gpu)
     vp = torch.full((pages, ps, hk, d), 0x55, dtype=torch.uint8, device=gpu)
     scaled = fmt not in ("fp8_e4m3", "fp8_e5m2")
-    ks = torch.full((pages, ps, hk), -7.0, dtype=torch.float32, device=gpu) if scaled else None
-    vs = torch.full((pages, ps, hk), -7.0, dtype=torch.float32, device=gpu) if scaled else None
+    # scale pools are [pages, kv heads, page_size]
+    ks = torch.full((pages, hk, ps), -7.0, dtype=torch.float32, device=gpu) if scaled else None
+    vs = torch.full((pages, hk, ps), -7.0, dtype=torch.float32, device=gpu) if scaled else None
     ops.kv_write_quant(fmt, dev(k, gpu, torch.bfloat16), dev(v, gpu, torch.bfloat16), dev(slots, gpu),
                        kp, vp, ks, vs)
     torch.cuda.synchronize()
@@ -44,7 +45,8 @@ def test_kv_write_quant_bit_exact(gpu, oracle, fmt, hk, d):
                     want_s[slots[t]] = scales.reshape(N, hk)[t]
         assert np.array_equal(pool.cpu().numpy().reshape(pages * ps, hk, d), want)
         if scaled:
-            assert np.array_equal(sc.cpu().numpy().reshape(pages * ps, hk), want_s)
+            got_s = sc.cpu().numpy().transpose(0, 2, 1).reshape(pages * ps, hk)   # -> [slot, head]
+            assert np.array_equal(got_s, want_s)
 
 
 @pytest.mark.parametrize("fmt", FORMATS)
@@ -62,7 +64,8 @@ def test_attention_over_quantised_pool_matches_oracle(gpu, oracle, fmt, hq, hk, 
     pools = {}
     for name in ("k_pages", "v_pages"):
         codes, scales, deq = oracle.kv_quant_rows(b[name].reshape(P * ps * hk, d), fmt)
-        pools[name] = (codes.reshape(P, ps, hk, d), None if scales is None else scales.reshape(P, ps, hk),
+        pools[name] = (codes.reshape(P, ps, hk, d),
+                       None if scales is None else np.ascontiguousarray(scales.reshape(P, ps, hk).transpose(0, 2, 1)),
                        deq.reshape(P, ps, hk, d))
     begin, lens = b["page_indptr"][:-1].astype(np.int32), np.asarray(ctx, np.int32)
     sc = lambda s: None if s is None else dev(s, gpu)
@@ -125,8 +128,8 @@ def test_rope_and_quantising_write_in_one_launch_equal_the_two_kernels(gpu, orac
     def pools():
         kp = torch.full((pages, ps, hk, d), 0x55, dtype=torch.uint8, device=gpu)
         vp = torch.full((pages, ps, hk, d), 0x55, dtype=torch.uint8, device=gpu)
-        ks = torch.full((pages, ps, hk), -7.0, dtype=torch.float32, device=gpu) if scaled else None
-        vs = torch.full((pages, ps, hk), -7.0, dtype=torch.float32, device=gpu) if scaled else None
+        ks = torch.full((pages, hk, ps), -7.0, dtype=torch.float32, device=gpu) if scaled else None
+        vs = torch.full((pages, hk, ps), -7.0, dtype=torch.float32, device=gpu) if scaled else None
         return kp, vp, ks, vs
 
     a = pools()
