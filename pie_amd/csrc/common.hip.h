@@ -30,8 +30,10 @@ __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
     return __builtin_bit_cast(uint16_t, b);
 }
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-    return static_cast<uint32_t>(f32_to_bf16_bits(lo)) |
-           (static_cast<uint32_t>(f32_to_bf16_bits(hi)) << 16);
+    // one v_cvt_pk_bf16_f32 (round to nearest even, as the scalar conversion)
+    typedef __bf16 bf16x2_pk_t __attribute__((ext_vector_type(2)));
+    typedef float f32x2_pk_t __attribute__((ext_vector_type(2)));
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_pk_t{lo, hi}, bf16x2_pk_t));
 }
 
 // acc += a.lo*b.lo + a.hi*b.hi with bf16 inputs and an fp32 accumulator.

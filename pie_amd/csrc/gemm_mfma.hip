@@ -27,6 +27,8 @@
 //     per-lane scalars and the SwiGLU partner (gate_i, up_i interleaved) is the neighbour lane.
 #include "common.hip.h"
 
+#include <type_traits>
+
 namespace pie_hip {
 namespace {
 
@@ -62,6 +64,7 @@ __device__ __forceinline__ int swz(int r, int g) { return r * 8 + (g ^ ((r >> 1)
 struct GInt4 {
     static constexpr int kRawVecs = 1;
     static constexpr int kLoads = 2;   // vector-memory operations per thread per K step
+    static constexpr int kValuPerMfma = 4;   // decode instructions placed behind each MFMA of the 256-row tile
     static constexpr bool kRowScale = false, kDirect = false;
     struct Raw {
         u32x4_t v[1];
@@ -75,12 +78,10 @@ struct GInt4 {
                                                           ((k0 + half * 32) >> a.g_shift)];
         return r;
     }
-    static __device__ __forceinline__ void store(u32x4_t* tile, int row, int tid, const Raw& r) {
+    static __device__ __forceinline__ void store(u32x4_t* tile, int row, int tid, const Raw& r, uint32_t k128) {
         const int half = tid & 1;
         const float gs = bf16_bits_to_f32(r.gs);
         const float off = -136.f * gs;
-        uint32_t k128 = 0x43004300u;
-        asm volatile("" : "+v"(k128));
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
             const uint32_t v = r.v[0][s];
@@ -99,7 +100,7 @@ struct GInt4 {
     }
 };
 struct GFp8 {
-    static constexpr int kLoads = 2;
+    static constexpr int kLoads = 2, kValuPerMfma = 1;
     static constexpr bool kRowScale = true, kDirect = false;
     struct Raw {
         u32x4_t v[2];
@@ -115,7 +116,7 @@ struct GFp8 {
         const f32x2_t f = hi ? __builtin_amdgcn_cvt_pk_f32_fp8(w, true) : __builtin_amdgcn_cvt_pk_f32_fp8(w, false);
         return pack_trunc(f.x, f.y);
     }
-    static __device__ __forceinline__ void store(u32x4_t* tile, int row, int tid, const Raw& r) {
+    static __device__ __forceinline__ void store(u32x4_t* tile, int row, int tid, const Raw& r, uint32_t) {
         const int half = tid & 1;
 #pragma unroll
         for (int v = 0; v < 2; ++v)
@@ -127,7 +128,7 @@ struct GFp8 {
     }
 };
 struct GInt8 {
-    static constexpr int kLoads = 2;
+    static constexpr int kLoads = 2, kValuPerMfma = 2;
     static constexpr bool kRowScale = true, kDirect = false;
     using Raw = GFp8::Raw;
     static __device__ __forceinline__ Raw load(const GemmArgs& a, int n, int k0, int tid) {
@@ -139,7 +140,7 @@ struct GInt8 {
         const float hi = static_cast<float>((u >> (sh + 8)) & 0xFFu) - 128.f;
         return pack_trunc(lo, hi);
     }
-    static __device__ __forceinline__ void store(u32x4_t* tile, int row, int tid, const Raw& r) {
+    static __device__ __forceinline__ void store(u32x4_t* tile, int row, int tid, const Raw& r, uint32_t) {
         const int half = tid & 1;
 #pragma unroll
         for (int v = 0; v < 2; ++v)
@@ -151,11 +152,11 @@ struct GInt8 {
     }
 };
 struct GBf16 {
-    static constexpr int kLoads = 4;   // direct-to-LDS transfers per wave per K step
+    static constexpr int kLoads = 4, kValuPerMfma = 0;   // direct-to-LDS transfers per wave per K step
     static constexpr bool kRowScale = false, kDirect = true;
     struct Raw {};
     static __device__ __forceinline__ Raw load(const GemmArgs&, int, int, int) { return {}; }
-    static __device__ __forceinline__ void store(u32x4_t*, int, int, const Raw&) {}
+    static __device__ __forceinline__ void store(u32x4_t*, int, int, const Raw&, uint32_t) {}
 };
 
 // s_waitcnt with vmcnt(n) (n < 16) and lgkmcnt(0), expcnt untouched (gfx9 encoding)
@@ -219,6 +220,8 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(const GemmArgs a) {
     const int wn_glob = min(n0 + wrow, N - 1);
     auto load_w = [&](int kt) { return F::load(a, wn_glob, (kbeg + min(kt, nk - 1)) * BK, tid); };
 
+    uint32_t magic = 0x43004300u;   // (128.0, 128.0) as a bf16 pair, opaque to the compiler
+    asm volatile("" : "+v"(magic));
     f32x4_t acc[kMaxMT][4];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
@@ -235,48 +238,79 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(const GemmArgs a) {
     __builtin_amdgcn_sched_barrier(0);
     issue_direct(1);
     __builtin_amdgcn_sched_barrier(0);
-    if (!F::kDirect) F::store(lds_b, wrow, tid, rr[0]);
+    if (!F::kDirect) F::store(lds_b, wrow, tid, rr[0], magic);
 
     // The loop body is unrolled three times so that ring slots (LDS stage, register set) are
     // compile-time constants: a register rotation would have to wait for the newest load.
-    for (int kt0 = 0; kt0 < nk; kt0 += kStages) {
-#pragma unroll
-        for (int i = 0; i < kStages; ++i) {
-            const int kt = kt0 + i;
-            // Transfers of step kt are complete when at most the operations issued after them
-            // are outstanding: the previous iteration's weight loads and its 4 (8) transfers.
-            __builtin_amdgcn_sched_barrier(0);
-            if (F::kDirect) PIE_WAIT_VM_LGKM0(4 + MT);
-            else PIE_WAIT_VM_LGKM0(MT + F::kLoads);
-            __builtin_amdgcn_s_barrier();
-            __builtin_amdgcn_sched_barrier(0);
-            rr[i] = load_w(kt + kStages);   // slot i held step kt, already written to LDS
-            __builtin_amdgcn_sched_barrier(0);
-            issue_direct(kt + 2);           // into the stage step kt - 1 was read from
-            __builtin_amdgcn_sched_barrier(0);
+    // Whole triples of K steps run without a branch, so that one scheduling region holds a
+    // step's MFMAs, its operand reads and the decode of the next step's weights; the region's
+    // group barriers then spread the vector-ALU work and the LDS traffic between the MFMAs (a
+    // block is one wave per SIMD: nothing else would fill the matrix pipe's shadow).
+    auto step = [&](const int i, const int kt, auto tail) {
+        constexpr bool kTail = decltype(tail)::value;
+        // Transfers of step kt are complete when at most the operations issued after them
+        // are outstanding: the previous iteration's weight loads and its 4 (8) transfers.
+        __builtin_amdgcn_sched_barrier(0);
+        if (F::kDirect) PIE_WAIT_VM_LGKM0(4 + MT);
+        else PIE_WAIT_VM_LGKM0(MT + F::kLoads);
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        rr[i] = load_w(kt + kStages);   // slot i held step kt, already written to LDS
+        __builtin_amdgcn_sched_barrier(0);
+        issue_direct(kt + 2);           // into the stage step kt - 1 was read from
+        __builtin_amdgcn_sched_barrier(0);
 
-            if (kt < nk) {
-                const u32x4_t* A = lds_a + i * kATileVecs + (wm * 16 * MT + j) * 8;
-                const u32x4_t* B = lds_b + (F::kDirect ? i : (kt & 1)) * kTileVecs + (wn * 64 + j) * 8;
-                const int key = j >> 1;   // swizzle key of rows base16 + j
+        if (!kTail || kt < nk) {
+            const u32x4_t* A = lds_a + i * kATileVecs + (wm * 16 * MT + j) * 8;
+            const u32x4_t* B = lds_b + (F::kDirect ? i : (kt & 1)) * kTileVecs + (wn * 64 + j) * 8;
+            const int key = j >> 1;   // swizzle key of rows base16 + j
+            bf16x8_t af[BK / 32][kMaxMT], bfr[BK / 32][4];
 #pragma unroll
-                for (int ks = 0; ks < BK / 32; ++ks) {
-                    bf16x8_t af[kMaxMT], bfr[4];
-                    const int slot = (ks * 4 + q) ^ key;
+            for (int ks = 0; ks < BK / 32; ++ks) {
+                const int slot = (ks * 4 + q) ^ key;
 #pragma unroll
-                    for (int t = 0; t < MT; ++t) af[t] = __builtin_bit_cast(bf16x8_t, A[t * 16 * 8 + slot]);
+                for (int t = 0; t < MT; ++t) af[ks][t] = __builtin_bit_cast(bf16x8_t, A[t * 16 * 8 + slot]);
 #pragma unroll
-                    for (int t = 0; t < 4; ++t) bfr[t] = __builtin_bit_cast(bf16x8_t, B[t * 16 * 8 + slot]);
-#pragma unroll
-                    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-                        for (int nt = 0; nt < 4; ++nt)
-                            acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[mt], bfr[nt], acc[mt][nt], 0, 0, 0);
-                }
+                for (int t = 0; t < 4; ++t) bfr[ks][t] = __builtin_bit_cast(bf16x8_t, B[t * 16 * 8 + slot]);
             }
-            // next step's weights -> bf16 tile (the other buffer; its readers passed the barrier)
-            if (!F::kDirect) F::store(lds_b + ((kt + 1) & 1) * kTileVecs, wrow, tid, rr[(i + 1) % kStages]);
+#pragma unroll
+            for (int ks = 0; ks < BK / 32; ++ks)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                    for (int nt = 0; nt < 4; ++nt)
+                        acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[ks][mt], bfr[ks][nt], acc[mt][nt], 0, 0, 0);
         }
+        // next step's weights -> bf16 tile (the other buffer; its readers passed the barrier)
+        if (!F::kDirect) F::store(lds_b + ((kt + 1) & 1) * kTileVecs, wrow, tid, rr[(i + 1) % kStages], magic);
+        if (!kTail) {
+            // order of the region: the first K half's operand reads, then per MFMA a few vector-ALU
+            // instructions of the decode; the second half's reads ride in the first MFMAs' shadow,
+            // the decoded tile's four LDS writes in the last ones'
+            constexpr int kMfma = MT * 4;
+            __builtin_amdgcn_sched_group_barrier(0x100, MT + 4, 0);
+#pragma unroll
+            for (int u = 0; u < kMfma; ++u) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                if (u < MT + 4) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                if (!F::kDirect) __builtin_amdgcn_sched_group_barrier(0x002, F::kValuPerMfma, 0);
+            }
+#pragma unroll
+            for (int u = 0; u < kMfma; ++u) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                if (!F::kDirect) __builtin_amdgcn_sched_group_barrier(0x002, F::kValuPerMfma, 0);
+                if (!F::kDirect && u >= kMfma - 8 && (u & 1)) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+            }
+        }
+    };
+    int kt0 = 0;
+    for (; kt0 + kStages <= nk; kt0 += kStages) {
+#pragma unroll
+        for (int i = 0; i < kStages; ++i) step(i, kt0 + i, std::false_type{});
+    }
+    if (kt0 < nk) {
+#pragma unroll
+        for (int i = 0; i < kStages; ++i) step(i, kt0 + i, std::true_type{});
     }
 
     // ---- epilogue: lane holds column n for rows 4q + r of each 16 x 16 tile ----
