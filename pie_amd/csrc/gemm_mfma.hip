@@ -10,15 +10,16 @@
 // integer / e4m3 value itself, exact in bf16, with the row scale applied to the fp32 sum),
 // bf16 x bf16 products, fp32 accumulation, one rounding at the end.
 //
-// Tiling: a 128 x 128 (or, for large M, 256 x 128) output tile per block of four waves, each wave
-// a 64 x 64 (128 x 64) quadrant held as 4 x 4 (8 x 4) accumulators of v_mfma_f32_16x16x32_bf16; K
-// advances 64 at a time.
+// Tiling: a 128 x 128 output tile per block of four waves or, for large M, 256 x 128 per block of
+// eight (two per SIMD), each wave a 64 x 64 quadrant held as 4 x 4 accumulators of
+// v_mfma_f32_16x16x32_bf16; K advances 64 at a time.
 //   * activations (and bf16 weights) travel global -> LDS directly (global_load_lds_dwordx4,
 //     no registers) into a ring of three stages, issued two K steps ahead; every wave waits
 //     for its own transfers with an explicit vmcnt and the block meets at one barrier per step;
 //   * quantised weights travel through registers, three K steps ahead (a tile row is only
-//     16-32 bytes per thread), are decoded to bf16 and written to a double-buffered LDS tile one
-//     step before use;
+//     8-32 bytes per thread: two or four threads share a row, every wave stages its share), are
+//     decoded to bf16 and written to a double-buffered LDS tile one step before use; the rows of
+//     eight consecutive lanes are two apart, so one LDS write cycle touches eight bank groups;
 //   * LDS tiles are unpadded and XOR-swizzled in 16-byte granules (granule g of row r sits at
 //     g ^ ((r >> 1) & 7)) so that the 16 rows an MFMA operand read touches fall in distinct
 //     banks while a direct-to-LDS transfer still writes 1 KiB contiguous per wave;
@@ -60,31 +61,38 @@ __device__ __forceinline__ uint32_t pack_trunc(float lo, float hi) {
 __device__ __forceinline__ int swz(int r, int g) { return r * 8 + (g ^ ((r >> 1) & 7)); }
 
 // ---- quantised weight staging: global -> registers (raw) -> bf16 vectors in LDS ------------
-// Thread t holds the 32 k-values (t % 2) of tile row t / 2 of one K step.
-struct GInt4 {
-    static constexpr int kRawVecs = 1;
-    static constexpr int kLoads = 2;   // vector-memory operations per thread per K step
+// TPR threads share a tile row of one K step: part p of a row holds its k-values
+// [p * 64 / TPR, (p + 1) * 64 / TPR) — 32 per thread with four waves, 16 with eight.
+template <int TPR>
+struct GInt4T {
+    static constexpr int kWords = 8 / TPR;   // 32-bit words (8 nibbles each) per thread
+    static constexpr int kLoads = 2;         // vector-memory operations per thread per K step
     static constexpr int kValuPerMfma = 4;   // decode instructions placed behind each MFMA of the 256-row tile
     static constexpr bool kRowScale = false, kDirect = false;
     struct Raw {
-        u32x4_t v[1];
+        uint32_t v[kWords];
         uint16_t gs;
     };
-    static __device__ __forceinline__ Raw load(const GemmArgs& a, int n, int k0, int tid) {
+    static __device__ __forceinline__ Raw load(const GemmArgs& a, int n, int k0, int part) {
         Raw r;
-        const int half = tid & 1;
-        r.v[0] = *reinterpret_cast<const u32x4_t*>(a.w + (static_cast<size_t>(n) * a.K + k0 + half * 32) / 2);
-        r.gs = reinterpret_cast<const uint16_t*>(a.scale)[static_cast<size_t>(n) * (a.K >> a.g_shift) +
-                                                          ((k0 + half * 32) >> a.g_shift)];
+        const int kk = k0 + part * (64 / TPR);
+        const unsigned char* p = a.w + (static_cast<size_t>(n) * a.K + kk) / 2;
+        if constexpr (kWords == 4) {
+            const u32x4_t t = *reinterpret_cast<const u32x4_t*>(p);
+            r.v[0] = t.x; r.v[1] = t.y; r.v[2] = t.z; r.v[3] = t.w;
+        } else {
+            const u32x2_t t = *reinterpret_cast<const u32x2_t*>(p);
+            r.v[0] = t.x; r.v[1] = t.y;
+        }
+        r.gs = reinterpret_cast<const uint16_t*>(a.scale)[static_cast<size_t>(n) * (a.K >> a.g_shift) + (kk >> a.g_shift)];
         return r;
     }
-    static __device__ __forceinline__ void store(u32x4_t* tile, int row, int tid, const Raw& r, uint32_t k128) {
-        const int half = tid & 1;
+    static __device__ __forceinline__ void store(u32x4_t* tile, int row, int part, const Raw& r, uint32_t k128) {
         const float gs = bf16_bits_to_f32(r.gs);
         const float off = -136.f * gs;
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {
-            const uint32_t v = r.v[0][s];
+        for (int s = 0; s < kWords; ++s) {
+            const uint32_t v = r.v[s];
             uint32_t pr[4];   // pr[j] = (128 + nib_j, 128 + nib_{j+4}) as a bf16 pair
 #pragma unroll
             for (int j = 0; j < 4; ++j) pr[j] = and_or(v >> (4 * j), 0x000F000Fu, k128);
@@ -94,45 +102,48 @@ struct GInt4 {
                 f[j] = fmaf(bf16_lo(pr[j]), gs, off);       // exact: (nib - 8) * scale
                 f[j + 4] = fmaf(bf16_hi(pr[j]), gs, off);
             }
-            tile[swz(row, half * 4 + s)] = u32x4_t{pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]),
-                                                   pack_bf16x2(f[4], f[5]), pack_bf16x2(f[6], f[7])};
+            tile[swz(row, part * kWords + s)] = u32x4_t{pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]),
+                                                       pack_bf16x2(f[4], f[5]), pack_bf16x2(f[6], f[7])};
         }
     }
 };
-struct GFp8 {
-    static constexpr int kLoads = 2, kValuPerMfma = 1;
+template <int TPR>
+struct GFp8T {
+    static constexpr int kVecs = 4 / TPR;    // 16-byte vectors (16 codes each) per thread
+    static constexpr int kLoads = kVecs, kValuPerMfma = 1;
     static constexpr bool kRowScale = true, kDirect = false;
     struct Raw {
-        u32x4_t v[2];
+        u32x4_t v[kVecs];
     };
-    static __device__ __forceinline__ Raw load(const GemmArgs& a, int n, int k0, int tid) {
+    static __device__ __forceinline__ Raw load(const GemmArgs& a, int n, int k0, int part) {
         Raw r;
-        const unsigned char* p = a.w + static_cast<size_t>(n) * a.K + k0 + (tid & 1) * 32;
-        r.v[0] = *reinterpret_cast<const u32x4_t*>(p);
-        r.v[1] = *reinterpret_cast<const u32x4_t*>(p + 16);
+        const unsigned char* p = a.w + static_cast<size_t>(n) * a.K + k0 + part * (64 / TPR);
+#pragma unroll
+        for (int v = 0; v < kVecs; ++v) r.v[v] = *reinterpret_cast<const u32x4_t*>(p + 16 * v);
         return r;
     }
     static __device__ __forceinline__ uint32_t cv(uint32_t w, bool hi) {
         const f32x2_t f = hi ? __builtin_amdgcn_cvt_pk_f32_fp8(w, true) : __builtin_amdgcn_cvt_pk_f32_fp8(w, false);
         return pack_trunc(f.x, f.y);
     }
-    static __device__ __forceinline__ void store(u32x4_t* tile, int row, int tid, const Raw& r, uint32_t) {
-        const int half = tid & 1;
+    static __device__ __forceinline__ void store(u32x4_t* tile, int row, int part, const Raw& r, uint32_t) {
 #pragma unroll
-        for (int v = 0; v < 2; ++v)
+        for (int v = 0; v < kVecs; ++v)
 #pragma unroll
             for (int s = 0; s < 2; ++s) {
                 const uint32_t a = r.v[v][2 * s], b = r.v[v][2 * s + 1];
-                tile[swz(row, half * 4 + v * 2 + s)] = u32x4_t{cv(a, false), cv(a, true), cv(b, false), cv(b, true)};
+                tile[swz(row, part * 2 * kVecs + v * 2 + s)] = u32x4_t{cv(a, false), cv(a, true), cv(b, false), cv(b, true)};
             }
     }
 };
-struct GInt8 {
-    static constexpr int kLoads = 2, kValuPerMfma = 2;
+template <int TPR>
+struct GInt8T {
+    static constexpr int kVecs = 4 / TPR;
+    static constexpr int kLoads = kVecs, kValuPerMfma = 2;
     static constexpr bool kRowScale = true, kDirect = false;
-    using Raw = GFp8::Raw;
-    static __device__ __forceinline__ Raw load(const GemmArgs& a, int n, int k0, int tid) {
-        return GFp8::load(a, n, k0, tid);
+    using Raw = typename GFp8T<TPR>::Raw;
+    static __device__ __forceinline__ Raw load(const GemmArgs& a, int n, int k0, int part) {
+        return GFp8T<TPR>::load(a, n, k0, part);
     }
     static __device__ __forceinline__ uint32_t two(uint32_t u, int sh) {
         // signed bytes -> exact bf16 pair: (byte ^ 0x80) - 128
@@ -140,41 +151,60 @@ struct GInt8 {
         const float hi = static_cast<float>((u >> (sh + 8)) & 0xFFu) - 128.f;
         return pack_trunc(lo, hi);
     }
-    static __device__ __forceinline__ void store(u32x4_t* tile, int row, int tid, const Raw& r, uint32_t) {
-        const int half = tid & 1;
+    static __device__ __forceinline__ void store(u32x4_t* tile, int row, int part, const Raw& r, uint32_t) {
 #pragma unroll
-        for (int v = 0; v < 2; ++v)
+        for (int v = 0; v < kVecs; ++v)
 #pragma unroll
             for (int s = 0; s < 2; ++s) {
                 const uint32_t a = r.v[v][2 * s] ^ 0x80808080u, b = r.v[v][2 * s + 1] ^ 0x80808080u;
-                tile[swz(row, half * 4 + v * 2 + s)] = u32x4_t{two(a, 0), two(a, 16), two(b, 0), two(b, 16)};
+                tile[swz(row, part * 2 * kVecs + v * 2 + s)] = u32x4_t{two(a, 0), two(a, 16), two(b, 0), two(b, 16)};
             }
     }
 };
-struct GBf16 {
+// (the format tags the launchers take; the kernel picks the TPR form for its wave count)
+struct GInt4 {
+    template <int TPR> using Staged = GInt4T<TPR>;
+    static constexpr bool kDirect = false, kRowScale = false;
+};
+struct GFp8 {
+    template <int TPR> using Staged = GFp8T<TPR>;
+    static constexpr bool kDirect = false, kRowScale = true;
+};
+struct GInt8 {
+    template <int TPR> using Staged = GInt8T<TPR>;
+    static constexpr bool kDirect = false, kRowScale = true;
+};
+struct GBf16T {
     static constexpr int kLoads = 4, kValuPerMfma = 0;   // direct-to-LDS transfers per wave per K step
     static constexpr bool kRowScale = false, kDirect = true;
     struct Raw {};
     static __device__ __forceinline__ Raw load(const GemmArgs&, int, int, int) { return {}; }
     static __device__ __forceinline__ void store(u32x4_t*, int, int, const Raw&, uint32_t) {}
 };
+struct GBf16 {
+    template <int TPR> using Staged = GBf16T;
+    static constexpr bool kDirect = true, kRowScale = false;
+};
 
 // s_waitcnt with vmcnt(n) (n < 16) and lgkmcnt(0), expcnt untouched (gfx9 encoding)
 #define PIE_WAIT_VM_LGKM0(n) __builtin_amdgcn_s_waitcnt(0x0070 | (n))
 
-// MT: 16-row activation tiles per wave.  4: a 128 x 128 block tile (64 x 64 per wave); 8: a
-// 256 x 128 block tile (128 x 64 per wave) — 12 operand reads feed 32 MFMAs instead of 8 for 16,
-// which moves the kernel from LDS-bound to MFMA-bound when M is large enough to fill the
-// machine with the bigger tiles.
-template <class Base, int MT_>
-struct Shape : Base {
-    static constexpr int kMT = MT_;
+// MT: 16-row activation tiles per wave (4: 64 x 64 per wave; 2: 32 x 64 for small batches).
+// NW: waves per block, 4 (2 x 2 quadrants) or 8 (4 x 2: two waves per SIMD, so one wave's
+// barrier and operand-read waits sit in the other's MFMAs).
+template <class Base, int MT_, int NW_ = 4>
+struct Shape {
+    using Format = Base;
+    static constexpr int kMT = MT_, kNW = NW_;
 };
 
-template <class F>
-__global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(const GemmArgs a) {
-    constexpr int MT = F::kMT;
-    constexpr int BMv = 32 * MT;                 // activation rows per block
+template <class SH>
+__global__ __launch_bounds__(SH::kNW* kWave) void gemm_mfma_kernel(const GemmArgs a) {
+    constexpr int MT = SH::kMT, NW = SH::kNW;
+    constexpr int TPR = NW / 2;                  // threads that share a staged weight row
+    using F = typename SH::Format::template Staged<TPR>;
+    constexpr int BMv = 16 * MT * (NW / 2);      // activation rows per block
+    constexpr int TB = 16 / NW;                  // direct weight transfers per wave and K step
     constexpr int kATileVecs = BMv * (BK / 8);   // 16-byte vectors per activation stage
     extern __shared__ __align__(16) unsigned char smem[];
     u32x4_t* lds_a = reinterpret_cast<u32x4_t*>(smem);            // [kStages][A tile]
@@ -198,10 +228,10 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(const GemmArgs a) {
     const uint16_t* bptr[4];
 #pragma unroll
     for (int u = 0; u < (MT > 4 ? MT : 4); ++u) {
-        const int r = (u * 4 + wv) * 8 + (lane >> 3);
+        const int r = (u * NW + wv) * 8 + (lane >> 3);
         const int g = (lane & 7) ^ ((r >> 1) & 7);
         if (u < MT) aptr[u] = a.act + static_cast<size_t>(min(m0 + r, M - 1)) * K + g * 8;
-        if (u < 4)
+        if (u < TB)
             bptr[u] = reinterpret_cast<const uint16_t*>(a.w) + static_cast<size_t>(min(n0 + r, N - 1)) * K + g * 8;
     }
     auto issue_direct = [&](int kt) {
@@ -209,16 +239,22 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(const GemmArgs a) {
         const int st = kt % kStages;
         if (F::kDirect) {
 #pragma unroll
-            for (int u = 0; u < 4; ++u)
-                __builtin_amdgcn_global_load_lds(bptr[u] + k0, PIE_LDS_PTR(lds_b + st * kTileVecs + (u * 4 + wv) * 64), 16, 0, 0);
+            for (int u = 0; u < TB; ++u)
+                __builtin_amdgcn_global_load_lds(bptr[u] + k0, PIE_LDS_PTR(lds_b + st * kTileVecs + (u * NW + wv) * 64), 16, 0, 0);
         }
 #pragma unroll
         for (int u = 0; u < MT; ++u)
-            __builtin_amdgcn_global_load_lds(aptr[u] + k0, PIE_LDS_PTR(lds_a + st * kATileVecs + (u * 4 + wv) * 64), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds(aptr[u] + k0, PIE_LDS_PTR(lds_a + st * kATileVecs + (u * NW + wv) * 64), 16, 0, 0);
     };
-    const int wrow = tid >> 1;
+    // quantised weights: TPR threads per tile row, every wave stages 128 / NW rows.  Within
+    // eight consecutive lanes (one LDS write cycle) the rows are 2 apart, so that their swizzle
+    // keys differ and the eight 16-byte granules fall in eight different bank groups.
+    constexpr bool stager = true;
+    const int wpart = lane & (TPR - 1);
+    const int wrow = TPR == 2 ? wv * 32 + ((lane >> 4) & 3) * 8 + ((lane >> 3) & 1) + ((lane >> 1) & 3) * 2
+                              : wv * 16 + ((lane >> 4) & 3) * 4 + ((lane >> 2) & 1) * 2 + ((lane >> 3) & 1);
     const int wn_glob = min(n0 + wrow, N - 1);
-    auto load_w = [&](int kt) { return F::load(a, wn_glob, (kbeg + min(kt, nk - 1)) * BK, tid); };
+    auto load_w = [&](int kt) { return F::load(a, wn_glob, (kbeg + min(kt, nk - 1)) * BK, wpart); };
 
     uint32_t magic = 0x43004300u;   // (128.0, 128.0) as a bf16 pair, opaque to the compiler
     asm volatile("" : "+v"(magic));
@@ -234,11 +270,12 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(const GemmArgs a) {
     issue_direct(0);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int i = 0; i < kStages; ++i) rr[i] = load_w(i);
+    for (int i = 0; i < kStages; ++i)
+        if (stager) rr[i] = load_w(i);
     __builtin_amdgcn_sched_barrier(0);
     issue_direct(1);
     __builtin_amdgcn_sched_barrier(0);
-    if (!F::kDirect) F::store(lds_b, wrow, tid, rr[0], magic);
+    if (!F::kDirect && stager) F::store(lds_b, wrow, wpart, rr[0], magic);
 
     // The loop body is unrolled three times so that ring slots (LDS stage, register set) are
     // compile-time constants: a register rotation would have to wait for the newest load.
@@ -251,7 +288,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(const GemmArgs a) {
         // Transfers of step kt are complete when at most the operations issued after them
         // are outstanding: the previous iteration's weight loads and its 4 (8) transfers.
         __builtin_amdgcn_sched_barrier(0);
-        if (F::kDirect) PIE_WAIT_VM_LGKM0(4 + MT);
+        if (F::kDirect) PIE_WAIT_VM_LGKM0(TB + MT);
         else PIE_WAIT_VM_LGKM0(MT + F::kLoads);
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
@@ -282,7 +319,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma_kernel(const GemmArgs a) {
                         acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[ks][mt], bfr[ks][nt], acc[mt][nt], 0, 0, 0);
         }
         // next step's weights -> bf16 tile (the other buffer; its readers passed the barrier)
-        if (!F::kDirect) F::store(lds_b + ((kt + 1) & 1) * kTileVecs, wrow, tid, rr[(i + 1) % kStages], magic);
+        if (!F::kDirect) F::store(lds_b + ((kt + 1) & 1) * kTileVecs, wrow, wpart, rr[(i + 1) % kStages], magic);
         if (!kTail) {
             // order of the region: the first K half's operand reads, then per MFMA a few vector-ALU
             // instructions of the decode; the second half's reads ride in the first MFMAs' shadow,
@@ -380,35 +417,37 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* pa
     }
 }
 
-template <class F, int MT>
+template <class F, int MT, int NW = 4>
 int launch_gemm_mt(const GemmArgs& a, int splits, hipStream_t stream) {
-    constexpr int BMv = 32 * MT;
+    constexpr int BMv = 16 * MT * (NW / 2);
     constexpr size_t smem = (static_cast<size_t>(kStages) * BMv * (BK / 8) +
                              static_cast<size_t>(F::kDirect ? kStages : 2) * kTileVecs) * sizeof(u32x4_t);
     static const hipError_t attr =
-        hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_mfma_kernel<Shape<F, MT>>),
+        hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_mfma_kernel<Shape<F, MT, NW>>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
     if (attr != hipSuccess) return PIE_HIP_ERR_LAUNCH;
     const dim3 grid((a.N + BN - 1) / BN, (a.M + BMv - 1) / BMv, splits);
     if (grid.y > 65535) return PIE_HIP_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL((gemm_mfma_kernel<Shape<F, MT>>), grid, dim3(kThreads), smem, stream, a);
+    hipLaunchKernelGGL((gemm_mfma_kernel<Shape<F, MT, NW>>), grid, dim3(NW * kWave), smem, stream, a);
     return launch_status();
 }
 
-// Measured at M = 2048 (MI355X): with both operands direct-to-LDS (bf16 weights) a 256-row tile
-// takes 1.66x the time of a 128-row tile for twice the work (790-930 against 650-820 TFLOP/s);
-// with quantised weights the decode-and-store stage, not the operand reads, sets the pace and
-// the taller tile gains nothing (int4 650-710 either way, fp8 slower), so those keep 128 rows.
-// PIE_HIP_GEMM_MT=4|8 forces a shape (measurement hook).
+// Measured at M = 2048 (MI355X): the 256 x 128 tile with eight waves (64 x 64 per wave, two
+// waves per SIMD) takes 1.67x the time of the 128 x 128 tile with four for twice the work —
+// int4 805-905 against 690-755 TFLOP/s, fp8 830-960 against 690-860, bf16 1020-1170 against
+// 670-920; the same tile with four waves of 128 x 64 (one per SIMD, nothing to fill a wave's
+// barrier and operand-read waits) reached 790-930 for bf16 and nothing for the quantised
+// formats.  The taller tile is taken when its rounds of 256 blocks cost less.
+// PIE_HIP_GEMM_MT=4|8 forces the 128- / 256-row shape (measurement hook).
 template <class F>
 int launch_gemm(const GemmArgs& a, hipStream_t stream) {
     static const int forced = [] { const char* e = getenv("PIE_HIP_GEMM_MT"); return e ? atoi(e) : 0; }();
     if (a.M <= 64 && !forced) return launch_gemm_mt<F, 2>(a, 1, stream);   // 64-row block tiles
     const long long nt = (a.N + BN - 1) / BN;
     const long long t4 = nt * ((a.M + 127) / 128), t8 = nt * ((a.M + 255) / 256);
-    const double c4 = static_cast<double>((t4 + 255) / 256), c8 = 1.66 * static_cast<double>((t8 + 255) / 256);
-    const bool tall = forced ? forced == 8 : (F::kDirect && a.M > 128 && c8 < c4);
-    return tall ? launch_gemm_mt<F, 8>(a, 1, stream) : launch_gemm_mt<F, 4>(a, 1, stream);
+    const double c4 = static_cast<double>((t4 + 255) / 256), c8 = 1.67 * static_cast<double>((t8 + 255) / 256);
+    const bool tall = forced ? forced >= 8 : (a.M > 128 && c8 < c4);
+    return tall ? launch_gemm_mt<F, 4, 8>(a, 1, stream) : launch_gemm_mt<F, 4>(a, 1, stream);
 }
 
 // Few output tiles (M up to 128 rows of a decode batch): a block per (tile, K share) so that
