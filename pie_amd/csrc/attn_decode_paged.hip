@@ -532,8 +532,7 @@ __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
                 sv[4 * nt + rr] = v;
                 m_new = fmaxf(m_new, v);
             }
-        m_new = fmaxf(m_new, __shfl_xor(m_new, 16, kWave));
-        m_new = fmaxf(m_new, __shfl_xor(m_new, 32, kWave));
+        m_new = rows_max(m_new);
         const float safe = m_new == -INFINITY ? 0.f : m_new;
         const float alpha = exp2f(mx - safe);
         mx = m_new;

@@ -21,6 +21,8 @@
 // (fp32 accumulators), and the normaliser sums the unrounded values.
 #include "common.hip.h"
 
+#include <type_traits>
+
 namespace pie_hip {
 namespace {
 
@@ -43,7 +45,7 @@ __device__ __forceinline__ int vt_slot(int kappa) {
 // 16-code piece per thread and matrix; the step's per-(token, kv head) scales sit in LDS and
 // multiply the scores (K) and the probabilities (V): float(code) * scale as in the row kernels).
 template <int D, int GQA, int QT, int KVF = kKvBf16>
-__global__ __launch_bounds__(kTileThreads) void attn_prefill_tile_kernel(
+__global__ __launch_bounds__(kTileThreads, 2) void attn_prefill_tile_kernel(
     const uint16_t* __restrict__ q, const void* __restrict__ k_pages_raw,
     const void* __restrict__ v_pages_raw, const float* __restrict__ k_scales,
     const float* __restrict__ v_scales, uint16_t* __restrict__ o,
@@ -64,13 +66,20 @@ __global__ __launch_bounds__(kTileThreads) void attn_prefill_tile_kernel(
     const uint16_t* v_pages = static_cast<const uint16_t*>(v_pages_raw);
     const unsigned char* k_bytes = static_cast<const unsigned char*>(k_pages_raw);
     const unsigned char* v_bytes = static_cast<const unsigned char*>(v_pages_raw);
-    __shared__ __attribute__((aligned(16))) float s_sc[Q8 ? 2 * kStepKeys : 1];   // K | V scales of a step
+    // two LDS buffers: a step's tiles are written while the previous step's are read, one
+    // barrier per step
+    __shared__ __attribute__((aligned(16))) float s_sc_all[2][Q8 ? 2 * kStepKeys : 1];   // K | V scales of a step
 
-    __shared__ __attribute__((aligned(16))) uint16_t Ks[kStepKeys * KSTRIDE];
-    __shared__ __attribute__((aligned(16))) uint16_t Vt[D * kVtStride];
+    __shared__ __attribute__((aligned(16))) uint16_t Ks_all[2][kStepKeys * KSTRIDE];
+    __shared__ __attribute__((aligned(16))) uint16_t Vt_all[2][D * kVtStride];
     __shared__ int s_kmax;
 
-    const int tile = blockIdx.x, kvh = blockIdx.y;
+    // Causal tiles grow with their index, and a CU holds two blocks that are about one machine
+    // width (256 blocks) apart in launch order: every other machine width walks the tiles
+    // backwards, so a long tile shares its CU with a short one.
+    const int kvh = blockIdx.y;
+    const bool backwards = ((blockIdx.y * gridDim.x) >> 8) & 1;
+    const int tile = backwards ? gridDim.x - 1 - blockIdx.x : blockIdx.x;
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wv = tid / kWave;
     const int l16 = lane & 15, g = lane >> 4;
     const int s0 = tile_start[tile], n_rows = tile_rows[tile];
@@ -101,6 +110,14 @@ __global__ __launch_bounds__(kTileThreads) void attn_prefill_tile_kernel(
             qf[qt][ks] = __builtin_bit_cast(bf16x8_t, v);
         }
     }
+
+    // the shortest causal extent among this wave's rows: steps below it need no masking
+    int min_len_v = my_len[0];
+#pragma unroll
+    for (int qt = 1; qt < QT; ++qt) min_len_v = min(min_len_v, my_len[qt]);
+#pragma unroll
+    for (int sh = 1; sh < kWave; sh <<= 1) min_len_v = min(min_len_v, __shfl_xor(min_len_v, sh, kWave));
+    const int min_len = __builtin_amdgcn_readfirstlane(min_len_v);
 
     // K/V staging: thread -> (key pair kp, 16-byte piece dc) so that two adjacent keys of one
     // piece meet in one thread (their V values pack into 4-byte LDS writes)
@@ -166,7 +183,10 @@ __global__ __launch_bounds__(kTileThreads) void attn_prefill_tile_kernel(
             vreg[slot][u] = *reinterpret_cast<const u32x4_t*>(v_pages + off);
         }
     };
-    auto stage = [&](int slot) {
+    auto stage = [&](int slot) {   // register slot = LDS buffer
+        uint16_t* Ks = Ks_all[slot];
+        uint16_t* Vt = Vt_all[slot];
+        float* s_sc = s_sc_all[slot];
         if constexpr (Q8) {
             int key, dc;
             piece_of(0, key, dc);
@@ -227,10 +247,15 @@ __global__ __launch_bounds__(kTileThreads) void attn_prefill_tile_kernel(
         for (int dt = 0; dt < DT; ++dt) acc[qt][dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     }
 
+    // Step j reads buffer j % 2.  On entry its tiles are staged and the block has met; the
+    // step first stages step j + 1 from the other register slot into the other buffer (whose
+    // readers passed the last barrier), then refills that slot with step j + 3.
     auto step = [&](int slot, int j0) {
-        __syncthreads();   // the previous step's LDS reads are done
-        stage(slot);
-        __syncthreads();
+        const uint16_t* Ks = Ks_all[slot];
+        const uint16_t* Vt = Vt_all[slot];
+        const float* s_sc = s_sc_all[slot];
+        if (j0 + kStepKeys < kmax) stage(slot ^ 1);
+        if (j0 + 3 * kStepKeys < kmax) issue(slot ^ 1, j0 + 3 * kStepKeys);   // (slot ^ 1 held step j + 1)
         // (one-byte pools) the scales of this lane's keys 16nt + 4g + r
         f32x4_t ksc[2], vsc[2];
         if constexpr (Q8) {
@@ -240,8 +265,6 @@ __global__ __launch_bounds__(kTileThreads) void attn_prefill_tile_kernel(
                 vsc[nt] = *reinterpret_cast<const f32x4_t*>(&s_sc[kStepKeys + 16 * nt + 4 * g]);
             }
         }
-        if (j0 + PF * kStepKeys < kmax) issue(slot, j0 + PF * kStepKeys);
-
         // S^T = K . Q^T for both query tiles
         f32x4_t st[QT][2];
 #pragma unroll
@@ -259,54 +282,65 @@ __global__ __launch_bounds__(kTileThreads) void attn_prefill_tile_kernel(
                     st[qt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[qt][ks], st[qt][nt], 0, 0, 0);
             }
         }
-        // online softmax per query (= per lane%16); the 8 keys of this lane: 16nt + 4g + r
+        // online softmax per query (= per lane%16); the 8 keys of this lane: 16nt + 4g + r.
+        // bf16 pools keep the running maximum in raw score units and fold the softmax scale into
+        // the exponent's fma; steps wholly inside every row's causal extent skip the masking
+        // (a wave-uniform branch); exponentials are the bare v_exp_f32 (arguments <= 0).
         bf16x8_t pf_hi[QT], pf_lo[QT];
+        auto softmax = [&](auto masked_tag) {
+            constexpr bool kMask = decltype(masked_tag)::value;
 #pragma unroll
-        for (int qt = 0; qt < QT; ++qt) {
-            float s[8];
-            float m_new = mx[qt];
+            for (int qt = 0; qt < QT; ++qt) {
+                float s[8];
+                float m_new = mx[qt];
 #pragma unroll
-            for (int nt = 0; nt < 2; ++nt)
+                for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int key = j0 + 16 * nt + 4 * g + r;
-                    const float sc = Q8 ? scale_log2e * ksc[nt][r] : scale_log2e;
-                    const float v = key < my_len[qt] ? st[qt][nt][r] * sc : -INFINITY;
-                    s[4 * nt + r] = v;
-                    m_new = fmaxf(m_new, v);
+                    for (int r = 0; r < 4; ++r) {
+                        float v = st[qt][nt][r];
+                        if constexpr (Q8) v *= scale_log2e * ksc[nt][r];
+                        if constexpr (kMask) v = j0 + 16 * nt + 4 * g + r < my_len[qt] ? v : -INFINITY;
+                        s[4 * nt + r] = v;
+                        m_new = fmaxf(m_new, v);
+                    }
+                m_new = rows_max(m_new);
+                const float safe = m_new == -INFINITY ? 0.f : m_new;
+                const float c = Q8 ? 1.f : scale_log2e;   // (one-byte pools: already in the scores)
+                const float off = -safe * c;
+                const float alpha = __builtin_amdgcn_exp2f(fmaf(mx[qt], c, off));
+                mx[qt] = m_new;
+                // The weights reach the second product as hi + lo with both parts bf16 (hi by
+                // truncation, lo = bf16(p - hi)): 16 significant bits, so P . V keeps the accuracy
+                // of fp32 weights (the reference multiplies fp32 probabilities,
+                // driver/cuda/src/ops/attention_naive_paged.cu:148-317), and the normaliser sums
+                // the unrounded values, as the decode kernel does.
+                float sum = 0.f;
+                uint32_t hi[4], lo[4];
+#pragma unroll
+                for (int e = 0; e < 8; e += 2) {
+                    float p0 = __builtin_amdgcn_exp2f(fmaf(s[e], c, off));
+                    float p1 = __builtin_amdgcn_exp2f(fmaf(s[e + 1], c, off));
+                    sum += p0 + p1;
+                    if constexpr (Q8) {   // V = float(code) * scale: the scale rides on the weight
+                        p0 *= vsc[e >> 2][e & 3];
+                        p1 *= vsc[e >> 2][(e & 3) + 1];
+                    }
+                    const uint32_t u0 = __float_as_uint(p0), u1 = __float_as_uint(p1);
+                    hi[e >> 1] = __builtin_amdgcn_perm(u1, u0, 0x07060302u);
+                    lo[e >> 1] = pack_bf16x2(p0 - __uint_as_float(u0 & 0xFFFF0000u),
+                                             p1 - __uint_as_float(u1 & 0xFFFF0000u));
                 }
-            m_new = fmaxf(m_new, __shfl_xor(m_new, 16, kWave));
-            m_new = fmaxf(m_new, __shfl_xor(m_new, 32, kWave));
-            const float safe = m_new == -INFINITY ? 0.f : m_new;
-            const float alpha = exp2f(mx[qt] - safe);
-            mx[qt] = m_new;
-            // The weights reach the second product as hi + lo with both parts bf16 (hi by
-            // truncation, lo = bf16(p - hi)): 16 significant bits, so P . V keeps the accuracy of
-            // fp32 weights (the reference multiplies fp32 probabilities,
-            // driver/cuda/src/ops/attention_naive_paged.cu:148-317), and the normaliser sums the
-            // unrounded values, as the decode kernel does.
-            float sum = 0.f;
-            uint32_t hi[4], lo[4];
+                pf_hi[qt] = __builtin_bit_cast(bf16x8_t, u32x4_t{hi[0], hi[1], hi[2], hi[3]});
+                pf_lo[qt] = __builtin_bit_cast(bf16x8_t, u32x4_t{lo[0], lo[1], lo[2], lo[3]});
+                lsum[qt] = lsum[qt] * alpha + sum;
+                if (alpha != 1.0f) {
 #pragma unroll
-            for (int e = 0; e < 8; e += 2) {
-                float p0 = exp2f(s[e] - safe), p1 = exp2f(s[e + 1] - safe);
-                sum += p0 + p1;
-                if constexpr (Q8) {   // V = float(code) * scale: the scale rides on the weight
-                    p0 *= vsc[e >> 2][e & 3];
-                    p1 *= vsc[e >> 2][(e & 3) + 1];
+                    for (int dt = 0; dt < DT; ++dt) acc[qt][dt] *= alpha;
                 }
-                const uint32_t b0 = __float_as_uint(p0) & 0xFFFF0000u, b1 = __float_as_uint(p1) & 0xFFFF0000u;
-                hi[e >> 1] = (b0 >> 16) | b1;
-                lo[e >> 1] = pack_bf16x2(p0 - __uint_as_float(b0), p1 - __uint_as_float(b1));
             }
-            pf_hi[qt] = __builtin_bit_cast(bf16x8_t, u32x4_t{hi[0], hi[1], hi[2], hi[3]});
-            pf_lo[qt] = __builtin_bit_cast(bf16x8_t, u32x4_t{lo[0], lo[1], lo[2], lo[3]});
-            lsum[qt] = lsum[qt] * alpha + sum;
-            if (alpha != 1.0f) {
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt) acc[qt][dt] *= alpha;
-            }
-        }
+        };
+        if (j0 + kStepKeys <= min_len) softmax(std::false_type{});
+        else softmax(std::true_type{});
         // O^T += V^T . P^T
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
@@ -318,10 +352,14 @@ __global__ __launch_bounds__(kTileThreads) void attn_prefill_tile_kernel(
                 acc[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf_lo[qt], acc[qt][dt], 0, 0, 0);
             }
         }
+        __syncthreads();   // step j + 1 is staged, step j read
     };
 
     if (kmax > 0) issue(0, 0);
     if (kmax > kStepKeys) issue(1, kStepKeys);
+    if (kmax > 0) stage(0);
+    if (kmax > 2 * kStepKeys) issue(0, 2 * kStepKeys);
+    __syncthreads();
     for (int j0 = 0; j0 < kmax; j0 += PF * kStepKeys) {   // unrolled by PF: compile-time register slots
         step(0, j0);
         if (j0 + kStepKeys < kmax) step(1, j0 + kStepKeys);

@@ -105,6 +105,15 @@ __device__ __forceinline__ float wave_sum_multi(const float* v, int lane) {
     return __uint_as_float(r32[0]) + __uint_as_float(r32[1]);
 }
 
+// max over the four lanes l, l ^ 16, l ^ 32, l ^ 48 (one value per 16-lane row) with the row
+// swaps instead of two LDS permutes: exact, so identical to the shuffle form
+__device__ __forceinline__ float rows_max(float x) {
+    const auto r16 = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    x = fmaxf(__uint_as_float(r16[0]), __uint_as_float(r16[1]));
+    const auto r32 = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r32[0]), __uint_as_float(r32[1]));
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
