@@ -54,30 +54,35 @@ int fmt_code(Quant q) {
 // Measured cost models (MI355X, microseconds, int4 8B-class shapes at 16-128 rows).  Skinny GEMM:
 // ~5 us + the weights at ~2.8 TB/s for the first 16-row pass, each further (side-by-side) pass
 // adding 85 % of that stream; from the tile-major copy (wave-private form) ~3.8 TB/s and 52 % per
-// further pass, the pass count rounded up to a power of two.  Tiled GEMM: K in 64-wide steps of ~0.72 us with 64-row block
-// tiles (M <= 64), ~0.98 us with 128-row tiles, while the tiles fit the machine (512 resident
-// blocks).  Split-K tiled GEMM: the steps of one share (+3 of prologue) at 1.25 / 1.6 us with two
-// blocks per CU, per round of 512 blocks, plus ~15 us for the second kernel and the partials.
+// further pass, the pass count rounded up to a power of two.  Tiled GEMM (eight-wave blocks): K in
+// 64-wide steps of ~0.60 us with 64-row block tiles (M <= 64), ~0.68 us with 128-row tiles, while
+// the tiles fit the machine (512 resident blocks).  Split-K tiled GEMM: the steps of one share
+// (+3 of prologue) at 1.06 / 1.36 us with two blocks per CU, per round of 512 blocks, plus ~15 us
+// for the second kernel and the partials.
 enum class GemmPath { Skinny, Tiled, TiledSplitK };
 GemmPath pick_gemm(const Linear& w, int M, size_t ws_bytes) {
     if (w.K % 64 != 0 || M < 17) return GemmPath::Skinny;
     const int passes = (M + 15) / 16;
-    int p2 = 1;   // the wave-private form runs its passes side by side: cost steps at powers of two
-    while (p2 < passes) p2 <<= 1;
+    // the wave-private form runs its passes side by side: cost steps at powers of two; above 32
+    // rows a pass covers 32 rows and costs 1.38 of a 16-row one
+    const int wpasses = M > 32 ? (M + 31) / 32 : passes;
+    int p2 = 1;
+    while (p2 < wpasses) p2 <<= 1;
     // (past eight passes the machine is full: the cost grows in proportion)
-    const double wave_form = p2 <= 8 ? 1.0 + 0.52 * (p2 - 1) : (1.0 + 0.52 * 7) * passes / 8.0;
+    const double wave_form = (M > 32 ? 1.38 : 1.0) *
+                             (p2 <= 8 ? 1.0 + 0.52 * (p2 - 1) : (1.0 + 0.52 * 7) * wpasses / 8.0);
     const double skinny = w.data_tiled
                               ? 5.0 + static_cast<double>(w.data_bytes()) / 3.8e6 * wave_form
                               : 5.0 + static_cast<double>(w.data_bytes()) / 2.8e6 * (1.0 + 0.85 * (passes - 1));
     const int steps = w.K / 64;
     const double tiles = static_cast<double>((w.N + 127) / 128) * (M <= 64 ? 1 : (M + 127) / 128);
-    const double tiled = 2.0 + steps * (M <= 64 ? 0.72 : 0.98) * std::max(1.0, tiles / 512.0);
+    const double tiled = 2.0 + steps * (M <= 64 ? 0.60 : 0.68) * std::max(1.0, tiles / 512.0);
     double split = 1e30;
     const size_t need = M <= 128 ? pie_hip_gemm_mfma_workspace_bytes(M, w.N, w.K) : 0;
     if (need && need <= ws_bytes) {
         const int shares = static_cast<int>(need / (static_cast<size_t>(M) * w.N * sizeof(float)));
         const int per = (steps + shares - 1) / shares;
-        split = 15.0 + (per + 3) * (M <= 64 ? 1.25 : 1.6) * std::ceil(tiles * shares / 512.0);
+        split = 15.0 + (per + 3) * (M <= 64 ? 1.06 : 1.36) * std::ceil(tiles * shares / 512.0);
     }
     if (split < skinny && split < tiled) return GemmPath::TiledSplitK;
     return tiled < skinny ? GemmPath::Tiled : GemmPath::Skinny;

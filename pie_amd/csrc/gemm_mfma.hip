@@ -432,22 +432,25 @@ int launch_gemm_mt(const GemmArgs& a, int splits, hipStream_t stream) {
     return launch_status();
 }
 
-// Measured at M = 2048 (MI355X): the 256 x 128 tile with eight waves (64 x 64 per wave, two
-// waves per SIMD) takes 1.67x the time of the 128 x 128 tile with four for twice the work —
-// int4 805-905 against 690-755 TFLOP/s, fp8 830-960 against 690-860, bf16 1020-1170 against
-// 670-920; the same tile with four waves of 128 x 64 (one per SIMD, nothing to fill a wave's
-// barrier and operand-read waits) reached 790-930 for bf16 and nothing for the quantised
-// formats.  The taller tile is taken when its rounds of 256 blocks cost less.
+// Blocks are eight waves, two per SIMD, so that one wave's barrier and operand-read waits sit
+// in another's MFMAs: 256 x 128 tiles (64 x 64 per wave) or 128 x 128 (32 x 64 per wave).
+// Measured at M = 2048 (MI355X): int4 805-905 TFLOP/s against 690-755 with 128 x 128 tiles on
+// four waves, fp8 830-960 against 690-860, bf16 1020-1170 against 670-920 (the 256-row tile on
+// four waves of 128 x 64 reached 790-930 for bf16 and nothing for the quantised formats); at
+// M = 128 / 512 on the shapes that fill one round of blocks the 128-row tile went from 57-187
+// to 46-151 us with eight waves.  A 256-row tile takes 1.85x the time of a 128-row one for
+// twice the work; it is taken when its rounds of 256 blocks cost less.  Batches of up to 64
+// rows take 64 x 128 tiles (16 x 64 per wave: 38-119 us against 44-136 on four waves).
 // PIE_HIP_GEMM_MT=4|8 forces the 128- / 256-row shape (measurement hook).
 template <class F>
 int launch_gemm(const GemmArgs& a, hipStream_t stream) {
     static const int forced = [] { const char* e = getenv("PIE_HIP_GEMM_MT"); return e ? atoi(e) : 0; }();
-    if (a.M <= 64 && !forced) return launch_gemm_mt<F, 2>(a, 1, stream);   // 64-row block tiles
+    if (a.M <= 64 && !forced) return launch_gemm_mt<F, 1, 8>(a, 1, stream);   // 64-row block tiles (16 x 64 per wave)
     const long long nt = (a.N + BN - 1) / BN;
     const long long t4 = nt * ((a.M + 127) / 128), t8 = nt * ((a.M + 255) / 256);
-    const double c4 = static_cast<double>((t4 + 255) / 256), c8 = 1.67 * static_cast<double>((t8 + 255) / 256);
-    const bool tall = forced ? forced >= 8 : (a.M > 128 && c8 < c4);
-    return tall ? launch_gemm_mt<F, 4, 8>(a, 1, stream) : launch_gemm_mt<F, 4>(a, 1, stream);
+    const double c4 = static_cast<double>((t4 + 255) / 256), c8 = 1.85 * static_cast<double>((t8 + 255) / 256);
+    const bool tall = forced ? forced == 8 : (a.M > 128 && c8 < c4);
+    return tall ? launch_gemm_mt<F, 4, 8>(a, 1, stream) : launch_gemm_mt<F, 2, 8>(a, 1, stream);
 }
 
 // Few output tiles (M up to 128 rows of a decode batch): a block per (tile, K share) so that
@@ -471,7 +474,7 @@ int launch_gemm_splitk(GemmArgs a, int splits, float* ws, hipStream_t stream) {
     a.partial = ws;
     a.beta = 0;
     a.swiglu = 0;
-    const int st = a.M <= 64 ? launch_gemm_mt<F, 2>(a, splits, stream) : launch_gemm_mt<F, 4>(a, splits, stream);
+    const int st = a.M <= 64 ? launch_gemm_mt<F, 1, 8>(a, splits, stream) : launch_gemm_mt<F, 2, 8>(a, splits, stream);
     if (st != PIE_HIP_OK) return st;
     const size_t outs = static_cast<size_t>(a.M) * (swiglu ? a.N / 2 : a.N);
     hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3(static_cast<unsigned>((outs + 255) / 256)), dim3(256), 0,
