@@ -663,10 +663,11 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
 // Second stage of the lm_head form: one block per activation row reduces the per-lane
 // (value, row) pairs; the largest value wins, the lowest row among equals, NaN never
 // (argmax_bf16_kernel, driver/cuda/src/kernels/argmax.cu:36-80).
-__global__ __launch_bounds__(256) void argmax_pairs_kernel(const unsigned long long* __restrict__ part,
-                                                           int count, uint32_t* __restrict__ out) {
-    __shared__ float sv[256 / kWave];
-    __shared__ int si[256 / kWave];
+constexpr int kPairThreads = 1024;
+__global__ __launch_bounds__(kPairThreads) void argmax_pairs_kernel(const unsigned long long* __restrict__ part,
+                                                                    int count, uint32_t* __restrict__ out) {
+    __shared__ float sv[kPairThreads / kWave];
+    __shared__ int si[kPairThreads / kWave];
     const unsigned long long* row = part + static_cast<size_t>(blockIdx.x) * count;
     float bv = -INFINITY;
     int bi = 0;
@@ -676,9 +677,17 @@ __global__ __launch_bounds__(256) void argmax_pairs_kernel(const unsigned long l
             bi = i;
         }
     };
-    for (int i = threadIdx.x; i < count; i += blockDim.x) {
-        const unsigned long long e = row[i];
-        upd(__uint_as_float(static_cast<uint32_t>(e >> 32)), static_cast<int>(e & 0xFFFFFFFFull));
+    // eight loads in flight per thread (the pairs of a row are a few thousand)
+    for (int i0 = threadIdx.x; i0 < count; i0 += 8 * kPairThreads) {
+        unsigned long long e[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int i = i0 + u * kPairThreads;
+            e[u] = i < count ? row[i] : (static_cast<unsigned long long>(0xFF800000u) << 32) | 0x7FFFFFFFull;   // (-inf, no row)
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            upd(__uint_as_float(static_cast<uint32_t>(e[u] >> 32)), static_cast<int>(e[u] & 0xFFFFFFFFull));
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
@@ -693,7 +702,7 @@ __global__ __launch_bounds__(256) void argmax_pairs_kernel(const unsigned long l
     }
     __syncthreads();
     if (threadIdx.x == 0) {
-        for (int w = 1; w < 256 / kWave; ++w) upd(sv[w], si[w]);
+        for (int w = 1; w < kPairThreads / kWave; ++w) upd(sv[w], si[w]);
         out[blockIdx.x] = static_cast<uint32_t>(bi == 0x7FFFFFFF ? 0 : bi);
     }
 }
@@ -896,7 +905,7 @@ extern "C" int pie_hip_lm_head_argmax(const uint16_t* act_bf16, const uint16_t* 
     const int rc = dispatch<FmtBf16>(a, M, 4, 2, st);
     if (rc != PIE_HIP_OK) return rc;
     const int count = gemv_grid(V, false, 2) * kWavesPerBlock * 4;
-    hipLaunchKernelGGL(argmax_pairs_kernel, dim3(M), dim3(256), 0, st,
+    hipLaunchKernelGGL(argmax_pairs_kernel, dim3(M), dim3(kPairThreads), 0, st,
                        static_cast<const unsigned long long*>(workspace), count, out_tokens);
     return launch_status();
 }
