@@ -477,15 +477,20 @@ int pie_hip_attn_rows_paged_static(const uint16_t* q, const uint16_t* k_pages,
  * KV-cache storage formats of the pool (the CUDA driver's kv_cache_dtype values,
  * driver/cuda/src/kv_cache_format.cpp:46-110).  One-byte formats keep the bf16 layout
  * [pages, page_size, hk, d] with one byte per element; the per-token-head formats add fp32 side
- * scales [pages, hk, page_size] for K and for V (see pie_hip_kv_write_quant).  The fp4 block formats are not implemented
- * (PIE_HIP_ERR_UNSUPPORTED).
+ * scales [pages, hk, page_size] for K and for V (see pie_hip_kv_write_quant).  The 4-bit block format
+ * ("fp4_e2m1" / "nvfp4": the same scheme under two names) packs two e2m1 codes per byte,
+ * [pages, page_size, hk, d/2] with the even element in the low nibble, and keeps one fp32 scale
+ * per block of 16 elements, [pages, hk, page_size, d/16]; the attention entry points do not read
+ * it directly (PIE_HIP_ERR_UNSUPPORTED): as in the reference, the pages a batch reads are first
+ * expanded into a bf16 pool by pie_hip_kv_dequant_pages.
  */
 enum {
     PIE_HIP_KV_BF16 = 0,
     PIE_HIP_KV_FP8_E4M3 = 1,             /* saturating cast of the value, no scales */
     PIE_HIP_KV_INT8_PER_TOKEN_HEAD = 2,  /* scale = absmax/127, code = rint(x / scale) */
     PIE_HIP_KV_FP8_PER_TOKEN_HEAD = 3,   /* scale = absmax/448, code = e4m3(x / scale) */
-    PIE_HIP_KV_FP8_E5M2 = 4              /* saturating e5m2 cast of the value, no scales */
+    PIE_HIP_KV_FP8_E5M2 = 4,             /* saturating e5m2 cast of the value, no scales */
+    PIE_HIP_KV_FP4_BLOCK = 5             /* per 16 elements: scale = absmax/6, code = nearest e2m1 level */
 };
 
 /*
@@ -529,6 +534,21 @@ int pie_hip_kv_write_quant(int kv_format, const uint16_t* k_rows, const uint16_t
                            const int64_t* kv_slots, void* k_pages, void* v_pages, float* k_scales,
                            float* v_scales, int num_tokens, int num_kv_heads, int head_dim,
                            int page_size, void* stream);
+/* PIE_HIP_KV_FP4_BLOCK in pie_hip_kv_write_quant: per block of 16 elements scale = absmax / 6
+ * (1 for an all-zero block), code = the nearest of +-{0, .5, 1, 1.5, 2, 3, 4, 6} to x * (1/scale),
+ * the smaller magnitude on a tie, sign bit for x < 0 (write_kv_fp4_block_kernel,
+ * driver/cuda/src/kernels/kv_paged.cu:292-417); head_dim a multiple of 16.
+ *
+ * Expansion of the pages a batch reads into bf16 pools of the same geometry
+ * [pages, page_size, hk, d] (page ids unchanged; other pages are not touched): every element
+ * becomes bf16(float(code) * scale), for any of the one-byte formats and the 4-bit block format.
+ * page_ids may name a page more than once.
+ * Reference: launch_dequant_kv_cache_layer_to_bf16_active and the dequant_*_pages_active kernels,
+ * driver/cuda/src/kernels/kv_paged.cu:419-531, :698-770. */
+int pie_hip_kv_dequant_pages(int kv_format, const void* k_pages, const void* v_pages,
+                             const float* k_scales, const float* v_scales, uint16_t* k_out,
+                             uint16_t* v_out, const uint32_t* page_ids, int num_pages,
+                             int num_kv_heads, int head_dim, int page_size, void* stream);
 /* pie_hip_qkv_rope_kvwrite and pie_hip_kv_write_quant in one launch for one-byte pools: every
  * (token, head) of the packed q|k|v rows is rotated (optional per-head q/k RMSNorm, either
  * pairing) and rounded to bf16 as by pie_hip_qkv_rope_kvwrite; q goes to q_out, the K and V

@@ -335,7 +335,8 @@ def brle_allow(runs, pos: int, n_kv: int, window: int = 0) -> np.ndarray:
     return out[:n_kv]
 
 
-KV_FORMATS = {"bf16": 0, "fp8_e4m3": 1, "int8_per_token_head": 2, "fp8_per_token_head": 3, "fp8_e5m2": 4}
+KV_FORMATS = {"bf16": 0, "fp8_e4m3": 1, "int8_per_token_head": 2, "fp8_per_token_head": 3, "fp8_e5m2": 4,
+              "fp4_e2m1": 5, "nvfp4": 5}
 
 
 def kv_quant_rows(x_bf16, fmt: str):
@@ -344,6 +345,14 @@ def kv_quant_rows(x_bf16, fmt: str):
     or None for fp8_e4m3, dequantised f32 [rows, d] = float(code) * scale)."""
     x = _c(x_bf16, np.uint16)
     rows, d = x.shape
+    if KV_FORMATS[fmt] == 5:
+        # 4-bit e2m1 codes, two per byte, and one scale per block of 16 elements; the dequantised
+        # values are bf16(level * scale) as the reference's attention reads them
+        codes = np.zeros((rows, (d + 1) // 2), np.uint8)
+        scales = np.ones((rows, (d + 15) // 16), np.float32)
+        deq = np.zeros((rows, d), np.float32)
+        lib().orc_kv_quant_rows(_p(x), _p(codes), _p(scales), _p(deq), C.c_int(rows), C.c_int(d), C.c_int(5))
+        return codes, scales, deq
     codes = np.zeros((rows, d), np.uint8)
     scales = np.ones(rows, np.float32)
     deq = np.zeros((rows, d), np.float32)

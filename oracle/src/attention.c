@@ -262,6 +262,14 @@ void orc_attn_rows_f32kv(const uint16_t* q, const float* k_pages, const float* v
  *                                code = clamp(rintf(x * inv), -128, 127)
  *   fmt 3 (fp8_per_token_head):  scale = absmax/448 (1 when 0), code = e4m3_satfinite(x * inv)
  *   fmt 4 (fp8_e5m2):            code = e5m2_satfinite(x); scales untouched
+ *   fmt 5 (fp4_e2m1 / nvfp4):    per block of 16 elements scale = absmax/6 (1 when 0), code =
+ *                                the nearest of +-{0, .5, 1, 1.5, 2, 3, 4, 6} to x * (1/scale), the
+ *                                smaller magnitude on a tie, sign bit set for x < 0; two codes per
+ *                                byte, the even element in the low nibble
+ *                                (write_kv_fp4_block_kernel, kv_paged.cu:292-417).  codes is
+ *                                [rows, (d+1)/2], scales [rows, ceil(d/16)], and dequant holds
+ *                                bf16(level * scale) — the value the reference's attention reads
+ *                                after dequant_fp4_pages_active_kernel (kv_paged.cu:496-531)
  * dequant (optional, f32): float(code) * scale, as the attention kernels read it.
  */
 uint8_t orc_f32_to_fp8_e4m3(float f);
@@ -304,8 +312,56 @@ void orc_fp8_e5m2_encode(const float* src, uint8_t* dst, size_t n) {
     for (size_t i = 0; i < n; ++i) dst[i] = orc_f32_to_fp8_e5m2(src[i]);
 }
 
+float orc_fp4_e2m1_value(uint8_t code) {
+    static const float levels[8] = {0.f, 0.5f, 1.f, 1.5f, 2.f, 3.f, 4.f, 6.f};
+    const float v = levels[code & 7];
+    return (code & 8) ? -v : v;
+}
+uint8_t orc_fp4_e2m1_quant(float x) {
+    static const float levels[8] = {0.f, 0.5f, 1.f, 1.5f, 2.f, 3.f, 4.f, 6.f};
+    const float ax = fabsf(x);
+    int best = 0;
+    float best_err = fabsf(ax - levels[0]);
+    for (int i = 1; i < 8; ++i) {
+        const float err = fabsf(ax - levels[i]);
+        if (err < best_err) {
+            best_err = err;
+            best = i;
+        }
+    }
+    return (uint8_t)((x < 0.f ? 8 : 0) | best);
+}
+
+static void orc_kv_quant_rows_fp4(const uint16_t* x, uint8_t* codes, float* scales, float* dequant,
+                                  int rows, int d) {
+    const int bs = 16, nb = (d + bs - 1) / bs, pd = (d + 1) / 2;
+    for (int r = 0; r < rows; ++r) {
+        const uint16_t* src = x + (size_t)r * d;
+        uint8_t* dst = codes + (size_t)r * pd;
+        for (int j = 0; j < pd; ++j) dst[j] = 0;
+        for (int b = 0; b < nb; ++b) {
+            const int lo = b * bs, hi = lo + bs < d ? lo + bs : d;
+            float amax = 0.f;
+            for (int j = lo; j < hi; ++j) amax = fmaxf(amax, fabsf(orc_bf16_to_f32(src[j])));
+            const float scale = amax > 0.f ? amax / 6.f : 1.f;
+            const float inv = 1.f / scale;
+            if (scales) scales[(size_t)r * nb + b] = scale;
+            for (int j = lo; j < hi; ++j) {
+                const uint8_t c = orc_fp4_e2m1_quant(orc_bf16_to_f32(src[j]) * inv);
+                dst[j / 2] |= (uint8_t)(c << ((j & 1) ? 4 : 0));
+                if (dequant)
+                    dequant[(size_t)r * d + j] = orc_bf16_to_f32(orc_f32_to_bf16(orc_fp4_e2m1_value(c) * scale));
+            }
+        }
+    }
+}
+
 void orc_kv_quant_rows(const uint16_t* x, uint8_t* codes, float* scales, float* dequant, int rows,
                        int d, int fmt) {
+    if (fmt == 5) {
+        orc_kv_quant_rows_fp4(x, codes, scales, dequant, rows, d);
+        return;
+    }
     for (int r = 0; r < rows; ++r) {
         const uint16_t* src = x + (size_t)r * d;
         float scale = 1.f, inv = 1.f;

@@ -159,7 +159,7 @@ void orc_attn_rows_f32kv(const uint16_t* q, const float* k_pages, const float* v
                          const int64_t* allow_off);
 
 /* kv_format != 0: a one-byte KV-cache format (1 fp8_e4m3, 2 int8_per_token_head,
- * 3 fp8_per_token_head).  The step's rotated K / V rows are quantised per (token, head) as
+ * 3 fp8_per_token_head, 4 fp8_e5m2, 5 fp4 blocks).  The step's rotated K / V rows are quantised per (token, head) as
  * kv_paged.cu:155-297 does and the pools k_f32 / v_f32 [L][pages, ps, hk, d] hold the values the
  * attention reads back, float(code) * scale (attention_naive_paged.cu:56-112). */
 static void orc_llama_forward_impl(const OrcModel* m, uint16_t* const* k_pages, uint16_t* const* v_pages,
@@ -190,7 +190,7 @@ static void orc_llama_forward_impl(const OrcModel* m, uint16_t* const* k_pages, 
         k_rows = (uint16_t*)malloc((size_t)N * kvrow * 2);
         v_rows = (uint16_t*)malloc((size_t)N * kvrow * 2);
         codes = (uint8_t*)malloc((size_t)N * kvrow);
-        scales = (float*)malloc((size_t)N * hk * 4);
+        scales = (float*)malloc((size_t)N * hk * ((d + 15) / 16) * 4);   /* (fp4: one per 16-element block) */
         deq = (float*)malloc((size_t)N * kvrow * 4);
         iota = (int64_t*)malloc((size_t)N * 8);
         for (int i = 0; i < N; ++i) iota[i] = i;

@@ -1073,6 +1073,64 @@ __device__ __forceinline__ unsigned char f32_to_e5m2_sat(float f) {
     return static_cast<unsigned char>(__builtin_amdgcn_cvt_pk_bf8_f32(c, c, 0, false) & 0xFF);
 }
 
+// Nearest of +-{0, .5, 1, 1.5, 2, 3, 4, 6}, the smaller magnitude on a tie, sign bit for x < 0
+// (quant_fp4_e2m1, kv_paged.cu:309-323): the level index is the number of midpoints below |x|.
+__device__ __forceinline__ unsigned f32_to_e2m1(float x) {
+    const float ax = fabsf(x);
+    const unsigned mag = (ax > 0.25f) + (ax > 0.75f) + (ax > 1.25f) + (ax > 1.75f) + (ax > 2.5f) + (ax > 3.5f) +
+                         (ax > 5.f);
+    return mag | (x < 0.f ? 8u : 0u);
+}
+__device__ __forceinline__ float e2m1_to_f32(unsigned code) {
+    // magnitudes 0, .5, 1, 1.5 are code / 2; 2, 3, 4, 6 are (2 + (code & 1)) << ((code >> 1) - 2)
+    const unsigned m = code & 7u;
+    const float v = m < 4u ? 0.5f * static_cast<float>(m) : static_cast<float>((2u + (m & 1u)) << ((m >> 1) - 2u));
+    return (code & 8u) ? -v : v;
+}
+
+// One-byte / 4-bit pools -> bf16 pools for the pages a batch reads: thread = eight consecutive
+// elements of one (page, slot, kv head) row; the value is bf16(float(code) * scale)
+// (dequant_*_pages_active_kernel, kv_paged.cu:419-531).
+__global__ __launch_bounds__(256) void kv_dequant_pages_kernel(
+    const unsigned char* __restrict__ k_pages, const unsigned char* __restrict__ v_pages,
+    const float* __restrict__ k_scales, const float* __restrict__ v_scales,
+    uint16_t* __restrict__ k_out, uint16_t* __restrict__ v_out, const uint32_t* __restrict__ page_ids,
+    size_t total, int hk, int d, int ps, int kv_format) {
+    const size_t idx = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (idx >= total) return;
+    const int vecs = d / 8;                       // eight-element pieces per row
+    const int piece = static_cast<int>(idx % vecs);
+    size_t rest = idx / vecs;
+    const int h = static_cast<int>(rest % hk);
+    rest /= hk;
+    const int slot = static_cast<int>(rest % ps);
+    const size_t page = page_ids[rest / ps];
+    const size_t th = (page * ps + slot) * hk + h;
+    const size_t sc_at = kv_scale_index(page, slot, h, hk, ps);
+#pragma unroll
+    for (int which = 0; which < 2; ++which) {
+        const unsigned char* src = which ? v_pages : k_pages;
+        const float* scales = which ? v_scales : k_scales;
+        float f[8];
+        float scale = 1.f;
+        if (kv_format == PIE_HIP_KV_FP4_BLOCK) {
+            const uint32_t w = *reinterpret_cast<const uint32_t*>(src + th * (d / 2) + piece * 4);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) f[e] = e2m1_to_f32((w >> (4 * e)) & 0xFu);
+            scale = scales[sc_at * ((d + 15) / 16) + (piece >> 1)];
+        } else {
+            const u32x2_t w = *reinterpret_cast<const u32x2_t*>(src + th * d + piece * 8);
+            if (kv_format == PIE_HIP_KV_INT8_PER_TOKEN_HEAD) kv_decode_f32<kKvInt8>(w, f);
+            else if (kv_format == PIE_HIP_KV_FP8_E5M2) kv_decode_f32<kKvBf8>(w, f);
+            else kv_decode_f32<kKvFp8>(w, f);
+            if (scales) scale = scales[sc_at];
+        }
+        const u32x4_t out = {pack_bf16x2(f[0] * scale, f[1] * scale), pack_bf16x2(f[2] * scale, f[3] * scale),
+                             pack_bf16x2(f[4] * scale, f[5] * scale), pack_bf16x2(f[6] * scale, f[7] * scale)};
+        *reinterpret_cast<u32x4_t*>((which ? v_out : k_out) + th * d + piece * 8) = out;
+    }
+}
+
 __global__ __launch_bounds__(256) void kv_write_quant_kernel(
     const uint16_t* __restrict__ k_src, const uint16_t* __restrict__ v_src,
     const int64_t* __restrict__ kv_slots, unsigned char* __restrict__ k_pages,
@@ -1086,6 +1144,35 @@ __global__ __launch_bounds__(256) void kv_write_quant_kernel(
     if (slot < 0) return;
     const size_t src = static_cast<size_t>(row) * d;
     const size_t th = static_cast<size_t>(slot) * hk + h;
+    if (kv_format == PIE_HIP_KV_FP4_BLOCK) {
+        // e2m1 codes, two per byte, one fp32 scale per block of 16 elements: a lane owns two
+        // adjacent elements, eight lanes a block (write_kv_fp4_block_kernel, kv_paged.cu:325-417)
+        const int nb = (d + 15) / 16, pd = d / 2;
+        const size_t sc0 = kv_scale_index_of_slot(slot, h, hk, ps) * nb;
+#pragma unroll
+        for (int which = 0; which < 2; ++which) {
+            const uint16_t* x = which ? v_src : k_src;
+            unsigned char* dst = (which ? v_pages : k_pages) + th * pd;
+            float* sc = (which ? v_scales : k_scales) + sc0;
+            for (int base = 0; base < d; base += 2 * kWave) {
+                const int j0 = base + 2 * lane;
+                const bool in = j0 < d;
+                const float f0 = in ? bf16_bits_to_f32(x[src + j0]) : 0.f;
+                const float f1 = in ? bf16_bits_to_f32(x[src + j0 + 1]) : 0.f;
+                float amax = fmaxf(fabsf(f0), fabsf(f1));
+                amax = fmaxf(amax, __shfl_xor(amax, 1, kWave));
+                amax = fmaxf(amax, __shfl_xor(amax, 2, kWave));
+                amax = fmaxf(amax, __shfl_xor(amax, 4, kWave));
+                const float scale = amax > 0.f ? amax / 6.f : 1.f;
+                const float inv = 1.f / scale;
+                if (in) {
+                    dst[j0 >> 1] = static_cast<unsigned char>(f32_to_e2m1(f0 * inv) | (f32_to_e2m1(f1 * inv) << 4));
+                    if ((lane & 7) == 0) sc[j0 >> 4] = scale;
+                }
+            }
+        }
+        return;
+    }
     const bool scaled = kv_format != PIE_HIP_KV_FP8_E4M3 && kv_format != PIE_HIP_KV_FP8_E5M2;
     const size_t sc_at = scaled ? kv_scale_index_of_slot(slot, h, hk, ps) : 0;
     const float qmax = kv_format == PIE_HIP_KV_INT8_PER_TOKEN_HEAD ? 127.f : 448.f;
@@ -1260,15 +1347,40 @@ extern "C" int pie_hip_kv_write_quant(int kv_format, const uint16_t* k_rows, con
     if (!k_rows || !v_rows || !kv_slots || !k_pages || !v_pages || num_tokens < 0 || num_kv_heads <= 0 ||
         head_dim <= 0 || page_size <= 0)
         return PIE_HIP_ERR_INVALID;
-    const bool scaled = kv_format == PIE_HIP_KV_INT8_PER_TOKEN_HEAD || kv_format == PIE_HIP_KV_FP8_PER_TOKEN_HEAD;
+    const bool scaled = kv_format == PIE_HIP_KV_INT8_PER_TOKEN_HEAD || kv_format == PIE_HIP_KV_FP8_PER_TOKEN_HEAD ||
+                        kv_format == PIE_HIP_KV_FP4_BLOCK;
     if (kv_format != PIE_HIP_KV_FP8_E4M3 && kv_format != PIE_HIP_KV_FP8_E5M2 && !scaled) return PIE_HIP_ERR_UNSUPPORTED;
     if (scaled && (!k_scales || !v_scales)) return PIE_HIP_ERR_INVALID;
+    if (kv_format == PIE_HIP_KV_FP4_BLOCK && head_dim % 16 != 0) return PIE_HIP_ERR_UNSUPPORTED;
     if (num_tokens == 0) return PIE_HIP_OK;
     const int rows = num_tokens * num_kv_heads;
     hipLaunchKernelGGL(kv_write_quant_kernel, dim3((rows + 3) / 4), dim3(256), 0,
                        static_cast<hipStream_t>(stream), k_rows, v_rows, kv_slots,
                        static_cast<unsigned char*>(k_pages), static_cast<unsigned char*>(v_pages), k_scales,
                        v_scales, rows, num_kv_heads, head_dim, page_size, kv_format);
+    return launch_status();
+}
+
+extern "C" int pie_hip_kv_dequant_pages(int kv_format, const void* k_pages, const void* v_pages,
+                                        const float* k_scales, const float* v_scales, uint16_t* k_out,
+                                        uint16_t* v_out, const uint32_t* page_ids, int num_pages,
+                                        int num_kv_heads, int head_dim, int page_size, void* stream) {
+    using namespace pie_hip;
+    if (!k_pages || !v_pages || !k_out || !v_out || !page_ids || num_pages < 0 || num_kv_heads <= 0 ||
+        head_dim <= 0 || page_size <= 0)
+        return PIE_HIP_ERR_INVALID;
+    const bool scaled = kv_format == PIE_HIP_KV_INT8_PER_TOKEN_HEAD || kv_format == PIE_HIP_KV_FP8_PER_TOKEN_HEAD ||
+                        kv_format == PIE_HIP_KV_FP4_BLOCK;
+    if (kv_format != PIE_HIP_KV_FP8_E4M3 && kv_format != PIE_HIP_KV_FP8_E5M2 && !scaled) return PIE_HIP_ERR_UNSUPPORTED;
+    if (scaled != (k_scales != nullptr) || scaled != (v_scales != nullptr)) return PIE_HIP_ERR_INVALID;
+    if (head_dim % 8 != 0 || (kv_format == PIE_HIP_KV_FP4_BLOCK && head_dim % 16 != 0)) return PIE_HIP_ERR_UNSUPPORTED;
+    if (num_pages == 0) return PIE_HIP_OK;
+    const size_t total = static_cast<size_t>(num_pages) * page_size * num_kv_heads * (head_dim / 8);
+    if ((total + 255) / 256 > 0x7FFFFFFFull) return PIE_HIP_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(kv_dequant_pages_kernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), static_cast<const unsigned char*>(k_pages),
+                       static_cast<const unsigned char*>(v_pages), k_scales, v_scales, k_out, v_out, page_ids,
+                       total, num_kv_heads, head_dim, page_size, kv_format);
     return launch_status();
 }
 

@@ -814,7 +814,8 @@ def attention_prefill_tiles(q: torch.Tensor, k_pages: torch.Tensor, v_pages: tor
     return o
 
 
-KV_FORMATS = {"bf16": 0, "fp8_e4m3": 1, "int8_per_token_head": 2, "fp8_per_token_head": 3, "fp8_e5m2": 4}
+KV_FORMATS = {"bf16": 0, "fp8_e4m3": 1, "int8_per_token_head": 2, "fp8_per_token_head": 3, "fp8_e5m2": 4,
+              "fp4_e2m1": 5, "nvfp4": 5}
 
 
 def attention_prefill_tiles_kvq(fmt: str, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
@@ -855,19 +856,38 @@ def kv_write_quant(fmt: str, k_rows: torch.Tensor, v_rows: torch.Tensor, kv_slot
     N, hk, d = k_rows.shape
     if tuple(v_rows.shape) != (N, hk, d) or kv_slots.numel() != N:
         raise KernelError("shape mismatch")
+    fp4 = KV_FORMATS[fmt] == 5          # two codes per byte, one scale per 16 elements
+    dstore = d // 2 if fp4 else d
     for t in (k_pages, v_pages):
-        if t.element_size() != 1 or not t.is_contiguous() or t.shape[-2:] != (hk, d):
-            raise KernelError("pools must be contiguous one-byte [pages, ps, hk, d]")
-    if N and int(kv_slots.max()) >= k_pages.numel() // (hk * d):
+        if t.element_size() != 1 or not t.is_contiguous() or t.shape[-2:] != (hk, dstore):
+            raise KernelError("pools must be contiguous one-byte [pages, ps, hk, d] (d/2 for the 4-bit format)")
+    if N and int(kv_slots.max()) >= k_pages.numel() // (hk * dstore):
         raise KernelError("kv slot out of range")
     for sc in (k_scales, v_scales):
         if sc is not None:
             _dev(sc, torch.float32, "scales")
-            if sc.numel() != k_pages.numel() // d:
-                raise KernelError("scales must be [pages, hk, ps]")
+            if sc.numel() != k_pages.numel() // dstore * (d // 16 if fp4 else 1):
+                raise KernelError("scales must be [pages, hk, ps] ([pages, hk, ps, d/16] for the 4-bit format)")
     _check(kernels().pie_hip_kv_write_quant(KV_FORMATS[fmt], _ptr(k_rows), _ptr(v_rows), _ptr(kv_slots),
                                             _ptr(k_pages), _ptr(v_pages), _ptr(k_scales), _ptr(v_scales),
                                             N, hk, d, k_pages.shape[1], _stream()), "pie_hip_kv_write_quant")
+
+
+def kv_dequant_pages(fmt: str, k_pages: torch.Tensor, v_pages: torch.Tensor, k_scales: Optional[torch.Tensor],
+                     v_scales: Optional[torch.Tensor], k_out: torch.Tensor, v_out: torch.Tensor,
+                     page_ids: torch.Tensor) -> None:
+    """Expand the named pages of a one-byte / 4-bit pool into bf16 pools [pages, ps, hk, d]."""
+    _dev(k_out, torch.bfloat16, "k_out")
+    _dev(v_out, torch.bfloat16, "v_out")
+    _dev(page_ids, torch.int32, "page_ids")
+    pages, ps, hk, d = k_out.shape
+    if tuple(v_out.shape) != (pages, ps, hk, d) or k_pages.shape[0] != pages:
+        raise KernelError("shape mismatch")
+    if page_ids.numel() and int(page_ids.max()) >= pages:
+        raise KernelError("page id out of range")
+    _check(kernels().pie_hip_kv_dequant_pages(KV_FORMATS[fmt], _ptr(k_pages), _ptr(v_pages), _ptr(k_scales),
+                                              _ptr(v_scales), _ptr(k_out), _ptr(v_out), _ptr(page_ids),
+                                              page_ids.numel(), hk, d, ps, _stream()), "pie_hip_kv_dequant_pages")
 
 
 def qkv_rope_kvwrite_quant(fmt: str, packed: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,

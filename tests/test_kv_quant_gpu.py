@@ -148,3 +148,83 @@ def test_rope_and_quantising_write_in_one_launch_equal_the_two_kernels(gpu, orac
         if x is not None:
             assert torch.equal(x, y)
     assert not torch.all(a[0] == 0x55)
+
+
+@pytest.mark.parametrize("hk,d", [(8, 128), (2, 64), (4, 256), (3, 48)])
+def test_fp4_block_write_is_bit_exact_and_pages_expand_to_the_oracles_values(gpu, oracle, hk, d):
+    """The 4-bit block format: codes (two per byte), block scales and the bf16 expansion of the
+    written pages against the oracle's quantiser, bit for bit; pages the list does not name stay
+    untouched."""
+    import torch
+    from pie_amd import ops
+
+    rng = np.random.default_rng(90 + hk + d)
+    N, pages, ps = 41, 9, 16
+    nb = d // 16
+    k = oracle.f32_to_bf16((rng.standard_normal((N, hk, d)) * rng.uniform(0.05, 20, (N, hk, 1))).astype(np.float32))
+    v = oracle.f32_to_bf16(rng.standard_normal((N, hk, d)).astype(np.float32))
+    k[3] = 0                                                   # an all-zero token
+    v[7, :, 16:32] = 0                                         # an all-zero block
+    slots = rng.permutation(pages * ps)[:N].astype(np.int64)
+    slots[5] = -1                                              # a token without a slot
+    kp = torch.full((pages, ps, hk, d // 2), 0x55, dtype=torch.uint8, device=gpu)
+    vp = torch.full((pages, ps, hk, d // 2), 0x55, dtype=torch.uint8, device=gpu)
+    ks = torch.full((pages, hk, ps, nb), -7.0, dtype=torch.float32, device=gpu)
+    vs = torch.full((pages, hk, ps, nb), -7.0, dtype=torch.float32, device=gpu)
+    for name in ("fp4_e2m1", "nvfp4"):
+        ops.kv_write_quant(name, dev(k, gpu, torch.bfloat16), dev(v, gpu, torch.bfloat16), dev(slots, gpu),
+                           kp, vp, ks, vs)
+    torch.cuda.synchronize()
+    deq = {}
+    for tag, src, pool, sc in (("k", k, kp, ks), ("v", v, vp, vs)):
+        codes, scales, dq = oracle.kv_quant_rows(src.reshape(N * hk, d), "nvfp4")
+        want = np.full((pages * ps, hk, d // 2), 0x55, np.uint8)
+        want_s = np.full((pages * ps, hk, nb), -7.0, np.float32)
+        want_d = np.zeros((pages * ps, hk, d), np.float32)
+        for t in range(N):
+            if slots[t] >= 0:
+                want[slots[t]] = codes.reshape(N, hk, d // 2)[t]
+                want_s[slots[t]] = scales.reshape(N, hk, nb)[t]
+                want_d[slots[t]] = dq.reshape(N, hk, d)[t]
+        assert np.array_equal(pool.cpu().numpy().reshape(pages * ps, hk, d // 2), want)
+        got_s = sc.cpu().numpy().transpose(0, 2, 1, 3).reshape(pages * ps, hk, nb)   # -> [slot, head, block]
+        assert np.array_equal(got_s, want_s)
+        deq[tag] = want_d
+    # expansion of the pages that hold tokens (one of them named twice); the others keep their fill
+    written = np.unique(slots[slots >= 0] // ps)
+    ids = np.concatenate([written[:-1], written[:1]]).astype(np.int32)
+    ko = torch.full((pages, ps, hk, d), 3.0, dtype=torch.bfloat16, device=gpu)
+    vo = torch.full((pages, ps, hk, d), 3.0, dtype=torch.bfloat16, device=gpu)
+    ops.kv_dequant_pages("nvfp4", kp, vp, ks, vs, ko, vo, dev(ids, gpu))
+    torch.cuda.synchronize()
+    mask = np.zeros(pages * ps, bool)
+    mask[slots[slots >= 0]] = True
+    for tag, out in (("k", ko), ("v", vo)):
+        got = oracle.bf16_to_f32(out.view(torch.uint16).cpu().numpy()).reshape(pages * ps, hk, d)
+        named = np.isin(np.arange(pages * ps) // ps, ids)
+        assert np.array_equal(got[mask & named], deq[tag][mask & named])
+        assert np.all(got[~named] == 3.0)
+
+
+@pytest.mark.parametrize("fmt", FORMATS)
+def test_page_expansion_of_one_byte_pools_is_code_times_scale_rounded_to_bf16(gpu, oracle, fmt):
+    import torch
+    from pie_amd import ops
+
+    rng = np.random.default_rng(17)
+    pages, ps, hk, d = 6, 16, 4, 128
+    src = oracle.f32_to_bf16((rng.standard_normal((pages * ps * hk, d)) * 3).astype(np.float32))
+    codes, scales, dq = oracle.kv_quant_rows(src, fmt)
+    kp = dev(codes.reshape(pages, ps, hk, d), gpu)
+    sc = None if scales is None else dev(np.ascontiguousarray(scales.reshape(pages, ps, hk).transpose(0, 2, 1)), gpu)
+    ko = torch.zeros((pages, ps, hk, d), dtype=torch.bfloat16, device=gpu)
+    vo = torch.zeros_like(ko)
+    ids = dev(np.array([4, 0, 5, 2], np.int32), gpu)
+    ops.kv_dequant_pages(fmt, kp, kp, sc, sc, ko, vo, ids)
+    torch.cuda.synchronize()
+    want = oracle.f32_to_bf16(dq).reshape(pages, ps, hk, d)
+    got = ko.view(torch.uint16).cpu().numpy()
+    for pg in (4, 0, 5, 2):
+        assert np.array_equal(got[pg], want[pg])
+    assert np.all(got[1] == 0) and np.all(got[3] == 0)
+    assert np.array_equal(vo.view(torch.uint16).cpu().numpy(), got)

@@ -164,3 +164,80 @@ def test_e5m2_codes_against_torch(oracle):
     got = torch.from_numpy(enc).view(torch.float8_e5m2).to(torch.float32).numpy()
     assert np.array_equal(got, e5m2_qdq(x))
     assert got[-3] == -57344.0 and got[-4] == 57344.0   # saturated, never inf
+
+
+# ---- 4-bit block format ("fp4_e2m1" / "nvfp4": e2m1 codes, one fp32 scale per 16 elements) ----
+FP4_LEVELS = np.array([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0], np.float32)
+
+
+def fp4_independent(xf):
+    """write_kv_fp4_block_kernel restated with numpy: (codes [rows, d] unpacked, scales [rows, nb],
+    bf16-rounded level * scale)."""
+    rows, d = xf.shape
+    nb = (d + 15) // 16
+    codes = np.zeros((rows, d), np.uint8)
+    scales = np.ones((rows, nb), np.float32)
+    for b in range(nb):
+        blk = xf[:, 16 * b:16 * b + 16]
+        amax = np.abs(blk).max(axis=1)
+        sc = np.where(amax > 0, amax / np.float32(6.0), np.float32(1.0)).astype(np.float32)
+        scales[:, b] = sc
+        y = (blk * (np.float32(1.0) / sc)[:, None]).astype(np.float32)
+        err = np.abs(np.abs(y)[:, :, None] - FP4_LEVELS[None, None, :])
+        mag = np.argmin(err, axis=2)          # first minimum: the smaller magnitude on a tie
+        codes[:, 16 * b:16 * b + 16] = (mag | np.where(y < 0, 8, 0)).astype(np.uint8)
+    lev = np.where(codes & 8, -FP4_LEVELS[codes & 7], FP4_LEVELS[codes & 7])
+    sc_full = np.repeat(scales, 16, axis=1)[:, :d]
+    return codes, scales, (lev * sc_full).astype(np.float32)
+
+
+@pytest.mark.parametrize("name", ["fp4_e2m1", "nvfp4"])
+@pytest.mark.parametrize("value", [False, True])
+def test_fp4_reference_pattern_within_reference_bars(oracle, name, value):
+    """The reference test's source pattern (17 dims: a full block and a one-element block) with
+    its bars: 0.02 on the values, 1e-5 on the scales (test_kv_cache_quant.cu:128-139, :158-169)."""
+    x = oracle.f32_to_bf16(reference_source(value))
+    xf = oracle.bf16_to_f32(x)
+    codes, scales, deq = oracle.kv_quant_rows(x, name)
+    assert codes.shape == (4, 9) and scales.shape == (4, 2)
+    want_codes, want_scales, want = fp4_independent(xf)
+    # the reference test divides by the scale where the kernel multiplies by its reciprocal
+    amax = np.stack([np.abs(xf[:, :16]).max(axis=1), np.abs(xf[:, 16:]).max(axis=1)], axis=1)
+    assert np.max(np.abs(scales - amax / 6.0)) <= 1e-5
+    assert np.max(np.abs(deq - want)) <= 0.02
+    assert np.array_equal(scales, want_scales)
+
+
+def test_fp4_codes_packing_and_dequant_equal_an_independent_evaluation(oracle):
+    rng = np.random.default_rng(77)
+    x = oracle.f32_to_bf16((rng.standard_normal((64, 128)) * rng.uniform(0.01, 30, (64, 1))).astype(np.float32))
+    x[3] = 0                                           # an all-zero row: scale 1, codes 0
+    x[5, 16:32] = 0                                    # an all-zero block inside a row
+    xf = oracle.bf16_to_f32(x)
+    codes, scales, deq = oracle.kv_quant_rows(x, "nvfp4")
+    want_codes, want_scales, want = fp4_independent(xf)
+    unpacked = np.stack([codes & 0xF, codes >> 4], axis=2).reshape(64, 128)   # even element in the low nibble
+    assert np.array_equal(unpacked, want_codes)
+    assert np.array_equal(scales, want_scales)
+    assert np.all(scales[3] == 1.0) and np.all(codes[3] == 0) and scales[5, 1] == 1.0
+    # dequantised values are bf16(level * scale)
+    assert np.array_equal(deq, oracle.bf16_to_f32(oracle.f32_to_bf16(want)))
+    # every block's largest magnitude maps to level 6 and comes back within one bf16 rounding
+    top = np.abs(deq).reshape(64, 8, 16).max(axis=2)
+    ref = np.abs(xf).reshape(64, 8, 16).max(axis=2)
+    assert np.all(np.abs(top - ref) <= ref * 2.0 ** -8)
+
+
+def test_fp4_hand_worked_levels_and_ties(oracle):
+    """One block whose largest magnitude is 6 (scale exactly 1): every midpoint between two levels
+    goes to the smaller magnitude, the sign bit follows x < 0, -0 keeps code 0."""
+    vals = np.array([6.0, 0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, -0.25, -0.75, -5.0, 5.5, 0.3, -0.0, 2.51, -6.0],
+                    np.float32)
+    x = oracle.f32_to_bf16(vals.reshape(1, 16))
+    assert np.array_equal(oracle.bf16_to_f32(x).reshape(-1)[:8], vals[:8])   # all exact in bf16 except 0.3, 2.51
+    codes, scales, deq = oracle.kv_quant_rows(x, "fp4_e2m1")
+    assert scales.shape == (1, 1) and scales[0, 0] == 1.0
+    got = np.stack([codes & 0xF, codes >> 4], axis=2).reshape(-1)
+    want = [7, 0, 1, 2, 3, 4, 5, 6, 8 | 0, 8 | 1, 8 | 6, 7, 1, 0, 5, 8 | 7]
+    assert list(got) == want
+    assert list(deq.reshape(-1)[:8]) == [6.0, 0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0]
