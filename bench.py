@@ -502,7 +502,7 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--kv-cache-dtype", default="auto",
-                    choices=["auto", "bf16", "fp8_e4m3", "int8_per_token_head", "fp8_per_token_head"],
+                    choices=["auto", "bf16", "fp8_e4m3", "fp8_e5m2", "int8_per_token_head", "fp8_per_token_head", "nvfp4"],
                     help="KV-cache storage of the driver under test (the headline run keeps bf16)")
     ap.add_argument("--no-extra", action="store_true")
     ap.add_argument("--model", default="llama8b-w4a16", choices=["llama8b-w4a16", *OTHER_MODELS])

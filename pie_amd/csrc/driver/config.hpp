@@ -165,8 +165,7 @@ inline int kv_format_code(const std::string& value) {
     if (v == "int8_per_token_head") return 2;
     if (v == "fp8_per_token_head") return 3;
     if (v == "fp8_e5m2") return 4;
-    if (v == "fp4_e2m1" || v == "nvfp4")
-        throw std::runtime_error("config: kv_cache_dtype '" + value + "' is not implemented by this driver");
+    if (v == "fp4_e2m1" || v == "nvfp4") return 5;   // one scheme under two names (kv_cache_format.cpp:99-107)
     throw std::runtime_error("invalid kv_cache_dtype '" + value +
                              "'; expected one of: auto, bf16, bfloat16, fp8_e4m3, fp8_e5m2, "
                              "int8_per_token_head, fp8_per_token_head, fp4_e2m1, nvfp4");

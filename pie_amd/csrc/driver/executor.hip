@@ -259,6 +259,8 @@ Executor::~Executor() {
         if (p) (void)hipFree(p);
     for (auto* p : k_scale_pool_) (void)hipFree(p);
     for (auto* p : v_scale_pool_) (void)hipFree(p);
+    if (kv_shadow_k_) (void)hipFree(kv_shadow_k_);
+    if (kv_shadow_v_) (void)hipFree(kv_shadow_v_);
     for (Growable* g : {&mask_in_host_, &mask_in_dev_, &mask_bitmap_, &tile_in_host_, &tile_in_dev_}) g->release();
     for (Growable* g : {&samp_f32_, &samp_ws_, &samp_in_dev_, &samp_in_host_, &samp_out_dev_, &samp_out_host_})
         g->release();
@@ -272,11 +274,16 @@ Executor::~Executor() {
 // driver/cuda/src/kv_cache_format.cpp:27-49.
 size_t Executor::page_bytes() const {
     const ModelConfig& m = model_.cfg();
-    return static_cast<size_t>(page_size_) * m.kv_heads * m.head_dim * (kv_format_ == PIE_HIP_KV_BF16 ? 2 : 1);
+    const size_t elems = static_cast<size_t>(page_size_) * m.kv_heads * m.head_dim;
+    if (kv_format_ == PIE_HIP_KV_FP4_BLOCK) return elems / 2;   // two codes per byte
+    return elems * (kv_format_ == PIE_HIP_KV_BF16 ? 2 : 1);
 }
 size_t Executor::scale_page_bytes() const {
+    const ModelConfig& m = model_.cfg();
+    if (kv_format_ == PIE_HIP_KV_FP4_BLOCK)   // one scale per block of 16 elements
+        return static_cast<size_t>(page_size_) * m.kv_heads * ((m.head_dim + 15) / 16) * sizeof(float);
     const bool scaled = kv_format_ == PIE_HIP_KV_INT8_PER_TOKEN_HEAD || kv_format_ == PIE_HIP_KV_FP8_PER_TOKEN_HEAD;
-    return scaled ? static_cast<size_t>(page_size_) * model_.cfg().kv_heads * sizeof(float) : 0;
+    return scaled ? static_cast<size_t>(page_size_) * m.kv_heads * sizeof(float) : 0;
 }
 
 // Allocate the pool; on out-of-memory halve the page count down to 64 pages
@@ -298,6 +305,22 @@ void Executor::alloc_kv() {
                 k_scale_pool_.push_back(static_cast<float*>(k));
                 if (hipMalloc(&v, sbytes) != hipSuccess) { ok = false; break; }
                 v_scale_pool_.push_back(static_cast<float*>(v));
+            }
+        }
+        if (ok && kv_format_ == PIE_HIP_KV_FP4_BLOCK) {
+            // the bf16 pages the attention kernels read (k_bf16_pages / v_bf16_pages of the
+            // reference's layer view, driver/cuda/src/kernels/kv_paged.cu:698-770)
+            const ModelConfig& m = model_.cfg();
+            const size_t shadow = static_cast<size_t>(total_pages_) * page_size_ * m.kv_heads * m.head_dim * 2;
+            void *k = nullptr, *v = nullptr;
+            if (hipMalloc(&k, shadow) != hipSuccess || hipMalloc(&v, shadow) != hipSuccess) {
+                if (k) (void)hipFree(k);
+                ok = false;
+            } else {
+                kv_shadow_k_ = static_cast<uint16_t*>(k);
+                kv_shadow_v_ = static_cast<uint16_t*>(v);
+                PIE_HIP_CHECK(hipMemsetAsync(kv_shadow_k_, 0, shadow, stream_));
+                PIE_HIP_CHECK(hipMemsetAsync(kv_shadow_v_, 0, shadow, stream_));
             }
         }
         if (ok) {
@@ -422,32 +445,41 @@ void Executor::body(int N, int S, int max_kv_len) {
                                                     rope_tab_, slots, N, hq, hk, d, pairing, m.rms_eps, s));
             }
         }
-        if (kvq && n_tiles_ > 0 && !masked_) {
+        // 4-bit blocks: the pages this batch reads become bf16 in the shared pool pair, which the
+        // bf16 attention kernels then read under the same page ids
+        const bool fp4 = kv_format_ == PIE_HIP_KV_FP4_BLOCK;
+        if (fp4)
+            PIE_KERNEL(pie_hip_kv_dequant_pages(kv_format_, k_pool_[l], v_pool_[l], ksc, vsc, kv_shadow_k_,
+                                                kv_shadow_v_, pages, n_page_refs_, hk, d, page_size_, s));
+        const uint16_t* kat = fp4 ? kv_shadow_k_ : k_pool_[l];
+        const uint16_t* vat = fp4 ? kv_shadow_v_ : v_pool_[l];
+        const bool kvq_attn = kvq && !fp4;
+        if (kvq_attn && n_tiles_ > 0 && !masked_) {
             const auto* td = static_cast<const int32_t*>(tile_in_dev_.ptr);
             PIE_KERNEL(pie_hip_attn_prefill_tiles_kvq(kv_format_, q_, k_pool_[l], v_pool_[l], ksc, vsc, attn_,
                                                       pages, row_begin, row_len, td, td + n_tiles_, n_tiles_,
                                                       tile_rows_, hq, hk, d, page_size_, -1.f, s));
-        } else if (kvq && masked_) {
+        } else if (kvq_attn && masked_) {
             PIE_KERNEL(pie_hip_attn_rows_paged_kvq_masked(
                 kv_format_, q_, k_pool_[l], v_pool_[l], ksc, vsc, attn_, nullptr, pages, row_begin, row_len,
                 static_cast<const uint16_t*>(mask_bitmap_.ptr), mask_stride_, N, hq, hk, d, page_size_, -1.f,
                 max_kv_len, attn_ws_, attn_ws_bytes_, s));
-        } else if (kvq) {
+        } else if (kvq_attn) {
             PIE_KERNEL(pie_hip_attn_rows_paged_kvq(kv_format_, q_, k_pool_[l], v_pool_[l], ksc, vsc, attn_,
                                                    nullptr, pages, row_begin, row_len, N, hq, hk, d,
                                                    page_size_, -1.f, max_kv_len, attn_ws_, attn_ws_bytes_, s));
         } else if (n_tiles_ > 0) {
             const auto* td = static_cast<const int32_t*>(tile_in_dev_.ptr);
-            PIE_KERNEL(pie_hip_attn_prefill_tiles(q_, k_pool_[l], v_pool_[l], attn_, pages, row_begin,
+            PIE_KERNEL(pie_hip_attn_prefill_tiles(q_, kat, vat, attn_, pages, row_begin,
                                                   row_len, td, td + n_tiles_, n_tiles_, tile_rows_, hq,
                                                   hk, d, page_size_, -1.f, s));
         } else if (masked_) {
             PIE_KERNEL(pie_hip_attn_rows_paged_masked(
-                q_, k_pool_[l], v_pool_[l], attn_, nullptr, pages, row_begin, row_len,
+                q_, kat, vat, attn_, nullptr, pages, row_begin, row_len,
                 static_cast<const uint16_t*>(mask_bitmap_.ptr), mask_stride_, N, hq, hk, d, page_size_,
                 -1.f, max_kv_len, attn_ws_, attn_ws_bytes_, s));
         } else {
-            PIE_KERNEL(pie_hip_attn_rows_paged(q_, k_pool_[l], v_pool_[l], attn_, nullptr, pages,
+            PIE_KERNEL(pie_hip_attn_rows_paged(q_, kat, vat, attn_, nullptr, pages,
                                                row_begin, row_len, N, hq, hk, d, page_size_, -1.f,
                                                max_kv_len, attn_ws_, attn_ws_bytes_, s));
         }
@@ -808,7 +840,10 @@ void Executor::forward(const BatchPlan& plan, std::vector<uint32_t>& tokens_out,
     if (t) t->h2d_us = us_since(t0);
 
     t0 = clk::now();
-    const bool use_graph = cfg_.runtime.use_graphs && plan.pure_decode && !samp_gather_in_body_ && !masked_;
+    n_page_refs_ = static_cast<int>(plan.page_indices.size());
+    // (4-bit blocks: the page expansion's extent changes from step to step, so no graph)
+    const bool use_graph = cfg_.runtime.use_graphs && plan.pure_decode && !samp_gather_in_body_ && !masked_ &&
+                           kv_format_ != PIE_HIP_KV_FP4_BLOCK;
     if (use_graph) {
         // The split grid depends on the context bound only through 512-token buckets.
         const int bucket = (plan.max_kv_len + 511) / 512 * 512;

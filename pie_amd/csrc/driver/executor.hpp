@@ -112,7 +112,11 @@ class Executor {
 
     std::vector<uint16_t*> k_pool_, v_pool_;  // per layer [pages, ps, hk, d] (bf16 or one byte per element)
     int kv_format_ = 0;                        // PIE_HIP_KV_*
-    std::vector<float*> k_scale_pool_, v_scale_pool_;   // per layer [pages, hk, ps], scaled formats
+    std::vector<float*> k_scale_pool_, v_scale_pool_;   // per layer [pages, hk, ps] ([pages, hk, ps, d/16] for 4-bit blocks)
+    // 4-bit block format: one bf16 pool pair of the whole pool's geometry, shared by the layers;
+    // the pages a batch reads are expanded into it before each layer's attention
+    uint16_t *kv_shadow_k_ = nullptr, *kv_shadow_v_ = nullptr;
+    int n_page_refs_ = 0;                      // page list entries of the forward in flight
     uint16_t *k_rows_ = nullptr, *v_rows_ = nullptr;     // this step's rotated K / V rows before quantisation
     int64_t* iota_slots_ = nullptr;                      // 0, 1, 2, ...: row t of k_rows_ is "slot" t
     unsigned char* swap_pool_ = nullptr;       // pinned: [layer][K|V][cpu_pages] pages (+ their scales)

@@ -132,6 +132,18 @@ extern "C" {
         page_size: c_int, sm_scale: f32, max_kv_len: c_int, workspace: *mut c_void,
         workspace_bytes: usize, stream: *mut c_void,
     ) -> c_int;
+    pub fn pie_hip_kv_write_quant(
+        kv_format: c_int, k_rows: *const u16, v_rows: *const u16, kv_slots: *const i64,
+        k_pages: *mut c_void, v_pages: *mut c_void, k_scales: *mut f32, v_scales: *mut f32,
+        num_tokens: c_int, num_kv_heads: c_int, head_dim: c_int, page_size: c_int,
+        stream: *mut c_void,
+    ) -> c_int;
+    pub fn pie_hip_kv_dequant_pages(
+        kv_format: c_int, k_pages: *const c_void, v_pages: *const c_void, k_scales: *const f32,
+        v_scales: *const f32, k_out: *mut u16, v_out: *mut u16, page_ids: *const u32,
+        num_pages: c_int, num_kv_heads: c_int, head_dim: c_int, page_size: c_int,
+        stream: *mut c_void,
+    ) -> c_int;
 
     // ---- layer ops ------------------------------------------------------------------------------
     pub fn pie_hip_embed(
