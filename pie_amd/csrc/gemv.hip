@@ -36,6 +36,7 @@
 //   * a wave64 butterfly finishes the row (one shared butterfly for the 2-4 rows of a
 //     step when there is a single activation row); the lane that stores an output has
 //     prefetched the residual / row scale it needs with the unit's loads.
+#include <type_traits>
 #include <hip/hip_ext.h>
 
 #include "common.hip.h"
@@ -232,7 +233,8 @@ struct FmtFp8 : FmtF32Act, RowScale<SB> {
 template <int R>
 struct Unit {
     u32x4_t w[R];
-    uint16_t gs[R];  // group scale (int4)
+    uint16_t gs[R];  // group scale (int4), one load per row ...
+    uint16_t gsv;    // ... or one load for the unit: lane l holds (row l / gpc, group l % gpc of the chunk)
     uint16_t prev;   // y element this lane may add to (lane = r*M + m), for beta = 1
     float rs;        // row scale for that lane's row (int8 / fp8)
     float rs2;       // swiglu epilogue: row scale of the pair's second (up) row
@@ -266,11 +268,15 @@ struct GemvArgs {
     // it stored and its row; slot (m, wave * R + r) of amax_part receives the pair (value bits in
     // the high word, row in the low word), for a second small kernel to reduce
     unsigned long long* amax_part;
+    // a wave's row slice (set by launch): the first slice_r waves take slice_q + 1 rows (or row
+    // pairs), the others slice_q
+    int slice_q, slice_r;
 };
 
 // ROPE: the q|k|v epilogue (rotation + KV write); its per-lane cos / sin / slot ride with every
 // unit's loads like the residual does, so the epilogue itself issues no loads.
-template <class F, int R, int M, bool ROPE>
+// GS1: the unit's int4 group scales come with one load (see issue()).
+template <class F, int R, int M, bool ROPE, bool GS1>
 __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
     constexpr int WPP = F::WPP, XV = F::XV;
     constexpr int kChunkK = kWave * WPP;  // weights covered by one wave-wide 16 B load
@@ -293,8 +299,9 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
     // (slices fall on even rows for the swiglu epilogue, which pairs rows 2i and 2i+1)
     const bool pairs = a.swiglu || ROPE;
     const int gran = pairs ? 2 : 1;
-    const int row_begin = static_cast<int>(wg * (N / gran) / total_waves) * gran;
-    const int row_end = static_cast<int>((wg + 1) * (N / gran) / total_waves) * gran;
+    const int wgi = static_cast<int>(wg);
+    const int row_begin = (wgi * a.slice_q + min(wgi, a.slice_r)) * gran;
+    const int row_end = row_begin + (a.slice_q + (wgi < a.slice_r ? 1 : 0)) * gran;
     const int ngroups = (row_end - row_begin + R - 1) / R;
     const int nunits = ngroups * nchunks;
 
@@ -302,6 +309,12 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
     // rows past the slice re-read its last row and are dropped at the store.
     // (`live` false: a unit past the end of the slice; every lane then re-reads one 16-byte
     // piece, so the request costs a single cache line)
+    // int4 group scales: when the R rows' groups of one chunk fit a wave (gpc groups per chunk and
+    // row, R * gpc <= 64) one load fetches them all and the lanes pick theirs with a lane
+    // permute — a vector-memory instruction occupies the CU's address unit for sixteen cycles
+    // whatever it fetches, and the eight waves of a CU issue their first units at the same time
+    constexpr bool one_gs = GS1 && F::kGroupScale;
+    const int gpc_shift = one_gs ? __builtin_ctz(static_cast<unsigned>(kChunkK)) - a.g_shift : 0;
     auto issue = [&](Unit<R>& u, int g, int c, bool live) {
         const int kbase = c * kChunkK + lane * WPP;
         const bool valid = kbase < K;
@@ -314,8 +327,16 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
             const int row = live ? min(row_begin + g * R + r, row_end - 1) : row_begin;
             u.w[r] = __builtin_nontemporal_load(a.w + static_cast<size_t>(row) * row_stride_v4 +
                                                 piece);
-            if constexpr (F::kGroupScale)
+            if constexpr (F::kGroupScale && !one_gs)
                 u.gs[r] = a.gscale[static_cast<size_t>(row) * groups_per_row + gidx];
+        }
+        if constexpr (one_gs) {
+            {
+                const int lr = min(lane >> gpc_shift, R - 1);
+                const int row = live ? min(row_begin + g * R + lr, row_end - 1) : row_begin;
+                const int grp = live ? min(((c * kChunkK) >> a.g_shift) + (lane & ((1 << gpc_shift) - 1)), groups_per_row - 1) : 0;
+                u.gsv = a.gscale[static_cast<size_t>(row) * groups_per_row + grp];
+            }
         }
         // Every unit prefetches what the lane that finishes an output needs, so the
         // epilogue never stalls the pipeline (only the last chunk's values are used).
@@ -373,16 +394,35 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
         for (int jj = 0; jj < kPreJ; ++jj) {
             const int sv = tid + jj * kBlock;
             const int svc = min(sv, nv - 1);
+            // (a block-uniform test: a vector-memory instruction costs the CU's address unit
+            // sixteen cycles whatever it fetches, and eight waves issue their prologues at once)
+            const bool any = jj * kBlock < nv;
 #pragma unroll
             for (int m = 0; m < M; ++m) {
-                const u32x4_t v = *reinterpret_cast<const u32x4_t*>(a.act + static_cast<size_t>(m) * K + svc * 8);
-                xr[jj * M + m] = sv < nv ? v : u32x4_t{0u, 0u, 0u, 0u};
+                u32x4_t v = {0u, 0u, 0u, 0u};
+                if (any) v = *reinterpret_cast<const u32x4_t*>(a.act + static_cast<size_t>(m) * K + svc * 8);
+                xr[jj * M + m] = v;   // (lanes past the row hold a repeat until the masking below)
             }
-            if (a.norm_w) nw[jj] = *reinterpret_cast<const u32x4_t*>(a.norm_w + svc * 8);
+            nw[jj] = u32x4_t{0u, 0u, 0u, 0u};
+            if (a.norm_w && any) nw[jj] = *reinterpret_cast<const u32x4_t*>(a.norm_w + svc * 8);
         }
     }
+    // (the scheduling barriers keep every use of the activations behind the first weight
+    // requests: left alone, the compiler masks the vectors right after their loads and so waits
+    // for the activations before it has asked for a single weight)
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int i = 0; i < kUnits; ++i) issue_next(un[i], ug[i], uc[i]);
+    __builtin_amdgcn_sched_barrier(0);
+    if (pre) {
+#pragma unroll
+        for (int jj = 0; jj < kPreJ; ++jj) {
+            const bool in_row = tid + jj * kBlock < nv;
+#pragma unroll
+            for (int m = 0; m < M; ++m)
+                xr[jj * M + m] = in_row ? xr[jj * M + m] : u32x4_t{0u, 0u, 0u, 0u};
+        }
+    }
 
     float inv_rms[M];
 #pragma unroll
@@ -526,7 +566,11 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
             for (int r = 0; r < R; ++r) {
                 const float p = F::dot(u.w[r], xs, p0);
                 if constexpr (F::kGroupScale) {
-                    const float s = valid ? bf16_bits_to_f32(u.gs[r]) : 0.f;
+                    uint16_t gsr = u.gs[r];
+                    if constexpr (one_gs)
+                        gsr = static_cast<uint16_t>(__builtin_amdgcn_ds_bpermute(
+                            ((r << gpc_shift) + ((lane * WPP) >> a.g_shift)) * 4, static_cast<int>(u.gsv)));
+                    const float s = valid ? bf16_bits_to_f32(gsr) : 0.f;
                     acc[r][m] = fmaf(s, p, acc[r][m]);
                 } else {
                     acc[r][m] += valid ? p : 0.f;
@@ -649,6 +693,17 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
     // reduced.  Loads are issued unconditionally so the wait before each compute only covers
     // the unit it consumes.
     for (int u = 0; u < nunits; u += kUnits) {
+        // Issue priority falls with progress.  The SIMD's arbiter serves its oldest wave first,
+        // so of a CU's two blocks the one dispatched first would finish well ahead of the other
+        // and leave its wave slots idle for the last third of the launch; a wave that has
+        // fallen behind its SIMD neighbour now outranks it until it has caught up.
+        {
+            const int quarter = (u * 4) / nunits;
+            if (quarter == 0) __builtin_amdgcn_s_setprio(3);
+            else if (quarter == 1) __builtin_amdgcn_s_setprio(2);
+            else if (quarter == 2) __builtin_amdgcn_s_setprio(1);
+            else __builtin_amdgcn_s_setprio(0);
+        }
 #pragma unroll
         for (int i = 0; i < kUnits; ++i) {
             if (u + i < nunits) compute(un[i], ug[i], uc[i]);
@@ -720,24 +775,47 @@ int gemv_grid(int N, bool pairs, int waves_per_simd) {
 }
 
 template <class F, int R, int M>
-int launch(const GemvArgs& a, int waves_per_simd, hipStream_t stream) {
+int launch(const GemvArgs& a_in, int waves_per_simd, hipStream_t stream) {
     constexpr int kChunkK = kWave * F::WPP;
-    const int nchunks = (a.K + kChunkK - 1) / kChunkK;
+    const int nchunks = (a_in.K + kChunkK - 1) / kChunkK;
     const size_t smem = static_cast<size_t>(M) * nchunks * kWave * (F::XV * 16 + 4);
     if (smem > 64 * 1024) return PIE_HIP_ERR_UNSUPPORTED;
-    const int grid = gemv_grid(a.N, a.swiglu || a.rope_table, waves_per_simd);
+    const int grid = gemv_grid(a_in.N, a_in.swiglu || a_in.rope_table, waves_per_simd);
+    GemvArgs a = a_in;
+    const int units = a.N / ((a.swiglu || a.rope_table) ? 2 : 1), waves = grid * kWavesPerBlock;
+    a.slice_q = units / waves;
+    a.slice_r = units % waves;
+    // (group scales with one load per unit: the R rows' groups of a chunk fit one wave)
+    const bool gs1 = F::kGroupScale && a.g_shift >= 0 && a.g_shift <= __builtin_ctz(static_cast<unsigned>(kChunkK)) &&
+                     (R << (__builtin_ctz(static_cast<unsigned>(kChunkK)) - a.g_shift)) <= kWave;
+    auto go = [&](auto rope, auto one) {
+        constexpr bool kRope = decltype(rope)::value, kOne = decltype(one)::value;
+        if (!kRope && t_start_event && t_stop_event) {
+            hipExtLaunchKernelGGL((gemv_kernel<F, R, M, kRope, kOne>), dim3(grid), dim3(kBlock),
+                                  static_cast<uint32_t>(smem), stream, t_start_event, t_stop_event, 0, a);
+            t_start_event = t_stop_event = nullptr;
+        } else {
+            hipLaunchKernelGGL((gemv_kernel<F, R, M, kRope, kOne>), dim3(grid), dim3(kBlock), smem, stream, a);
+        }
+    };
     if (a.rope_table) {
-        if constexpr (R % 2 == 0)
-            hipLaunchKernelGGL((gemv_kernel<F, R, M, true>), dim3(grid), dim3(kBlock), smem, stream, a);
-        else
+        if constexpr (R % 2 == 0) {
+            if constexpr (F::kGroupScale) {
+                if (gs1) go(std::true_type{}, std::true_type{});
+                else go(std::true_type{}, std::false_type{});
+            } else {
+                go(std::true_type{}, std::false_type{});
+            }
+        } else {
             return PIE_HIP_ERR_INVALID;
-    } else if (t_start_event && t_stop_event) {
-        hipExtLaunchKernelGGL((gemv_kernel<F, R, M, false>), dim3(grid), dim3(kBlock),
-                              static_cast<uint32_t>(smem), stream, t_start_event, t_stop_event, 0,
-                              a);
-        t_start_event = t_stop_event = nullptr;
+        }
     } else {
-        hipLaunchKernelGGL((gemv_kernel<F, R, M, false>), dim3(grid), dim3(kBlock), smem, stream, a);
+        if constexpr (F::kGroupScale) {
+            if (gs1) go(std::false_type{}, std::true_type{});
+            else go(std::false_type{}, std::false_type{});
+        } else {
+            go(std::false_type{}, std::false_type{});
+        }
     }
     return launch_status();
 }
