@@ -271,12 +271,17 @@ struct GemvArgs {
     // a wave's row slice (set by launch): the first slice_r waves take slice_q + 1 rows (or row
     // pairs), the others slice_q
     int slice_q, slice_r;
+    int groups_per_row;   // K / G (int4), set by launch
 };
 
 // ROPE: the q|k|v epilogue (rotation + KV write); its per-lane cos / sin / slot ride with every
 // unit's loads like the residual does, so the epilogue itself issues no loads.
-// GS1: the unit's int4 group scales come with one load (see issue()).
-template <class F, int R, int M, bool ROPE, bool GS1>
+// GS1: the unit's int4 group scales come with one load (see issue()).  PJ: activation vectors
+// (8 values) a thread holds per row in the register prologue — 2 covers K <= 4096, the other
+// value 8 / M; a vector-memory instruction costs the CU's address unit sixteen cycles whatever
+// it fetches and every instruction ahead of the first weight request delays it, so short rows
+// get a prologue with no idle trips.
+template <class F, int R, int M, bool ROPE, bool GS1, int PJ>
 __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
     constexpr int WPP = F::WPP, XV = F::XV;
     constexpr int kChunkK = kWave * WPP;  // weights covered by one wave-wide 16 B load
@@ -288,7 +293,7 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
     const int nchunks = (K + kChunkK - 1) / kChunkK;
     const int vec_per_m = nchunks * XV * kWave;
     const int row_stride_v4 = K / WPP;
-    const int groups_per_row = F::kGroupScale ? K / a.G : 0;
+    const int groups_per_row = a.groups_per_row;
 
     u32x4_t* lds_x = reinterpret_cast<u32x4_t*>(smem);               // [M][nchunks][XV][64]
     float* lds_sx = reinterpret_cast<float*>(lds_x + M * vec_per_m);  // [M][nchunks][64]
@@ -385,36 +390,30 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
     // requested before the weights: memory operations return in order, so a prologue that
     // loads activations after the first weight requests starts only when those have arrived
     // from HBM.  Longer rows keep the two-pass prologue below.
-    constexpr int kPreJ = 8 / M;
+    constexpr int kPreJ = PJ > 0 ? PJ : 1;
     const int nv = K / 8, nvp = nchunks * (kChunkK / 8);   // real / padded source vectors per row
-    const bool pre = nvp <= kPreJ * kBlock;
-    u32x4_t xr[kPreJ * M], nw[kPreJ];
-    if (pre) {
+    constexpr bool pre = PJ > 0;   // (the launch picks PJ so that the row fits: nvp <= PJ * kBlock)
+    float inv_rms[M];
+#pragma unroll
+    for (int m = 0; m < M; ++m) inv_rms[m] = 1.f;
+    if constexpr (pre) {
+        u32x4_t xr[kPreJ * M], nw[kPreJ];
 #pragma unroll
         for (int jj = 0; jj < kPreJ; ++jj) {
             const int sv = tid + jj * kBlock;
             const int svc = min(sv, nv - 1);
-            // (a block-uniform test: a vector-memory instruction costs the CU's address unit
-            // sixteen cycles whatever it fetches, and eight waves issue their prologues at once)
-            const bool any = jj * kBlock < nv;
 #pragma unroll
-            for (int m = 0; m < M; ++m) {
-                u32x4_t v = {0u, 0u, 0u, 0u};
-                if (any) v = *reinterpret_cast<const u32x4_t*>(a.act + static_cast<size_t>(m) * K + svc * 8);
-                xr[jj * M + m] = v;   // (lanes past the row hold a repeat until the masking below)
-            }
-            nw[jj] = u32x4_t{0u, 0u, 0u, 0u};
-            if (a.norm_w && any) nw[jj] = *reinterpret_cast<const u32x4_t*>(a.norm_w + svc * 8);
+            for (int m = 0; m < M; ++m)   // (lanes past the row hold a repeat until the masking below)
+                xr[jj * M + m] = *reinterpret_cast<const u32x4_t*>(a.act + static_cast<size_t>(m) * K + svc * 8);
+            if (a.norm_w) nw[jj] = *reinterpret_cast<const u32x4_t*>(a.norm_w + svc * 8);
         }
-    }
-    // (the scheduling barriers keep every use of the activations behind the first weight
-    // requests: left alone, the compiler masks the vectors right after their loads and so waits
-    // for the activations before it has asked for a single weight)
-    __builtin_amdgcn_sched_barrier(0);
+        // (the scheduling barriers keep every use of the activations behind the first weight
+        // requests: left alone, the compiler masks the vectors right after their loads and so waits
+        // for the activations before it has asked for a single weight)
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int i = 0; i < kUnits; ++i) issue_next(un[i], ug[i], uc[i]);
-    __builtin_amdgcn_sched_barrier(0);
-    if (pre) {
+        for (int i = 0; i < kUnits; ++i) issue_next(un[i], ug[i], uc[i]);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int jj = 0; jj < kPreJ; ++jj) {
             const bool in_row = tid + jj * kBlock < nv;
@@ -422,12 +421,6 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
             for (int m = 0; m < M; ++m)
                 xr[jj * M + m] = in_row ? xr[jj * M + m] : u32x4_t{0u, 0u, 0u, 0u};
         }
-    }
-
-    float inv_rms[M];
-#pragma unroll
-    for (int m = 0; m < M; ++m) inv_rms[m] = 1.f;
-    if (pre) {
         // ---- activations from registers (requested before the weights) ----
         if (a.norm_w) {
             float* red = lds_sx;  // free until the sums are written below
@@ -484,6 +477,8 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
         }
         __syncthreads();
     } else {
+#pragma unroll
+    for (int i = 0; i < kUnits; ++i) issue_next(un[i], ug[i], uc[i]);
     // Optional fused RMSNorm: sum of squares of each activation row (fp32), block-reduced.
     if (a.norm_w) {
         float* red = lds_sx;  // free until the sum_x pass below
@@ -785,17 +780,32 @@ int launch(const GemvArgs& a_in, int waves_per_simd, hipStream_t stream) {
     const int units = a.N / ((a.swiglu || a.rope_table) ? 2 : 1), waves = grid * kWavesPerBlock;
     a.slice_q = units / waves;
     a.slice_r = units % waves;
+    a.groups_per_row = F::kGroupScale && a.G > 0 ? a.K / a.G : 0;
     // (group scales with one load per unit: the R rows' groups of a chunk fit one wave)
     const bool gs1 = F::kGroupScale && a.g_shift >= 0 && a.g_shift <= __builtin_ctz(static_cast<unsigned>(kChunkK)) &&
                      (R << (__builtin_ctz(static_cast<unsigned>(kChunkK)) - a.g_shift)) <= kWave;
-    auto go = [&](auto rope, auto one) {
+    constexpr int kLongJ = 8 / M;   // (the register prologue's reach: rows of up to 2048 * kLongJ values)
+    const int nvp = nchunks * (kChunkK / 8);
+    const bool short_row = nvp <= 2 * kBlock;
+    auto go_j = [&](auto rope, auto one, auto pj) {
         constexpr bool kRope = decltype(rope)::value, kOne = decltype(one)::value;
+        constexpr int kPj = decltype(pj)::value;
         if (!kRope && t_start_event && t_stop_event) {
-            hipExtLaunchKernelGGL((gemv_kernel<F, R, M, kRope, kOne>), dim3(grid), dim3(kBlock),
+            hipExtLaunchKernelGGL((gemv_kernel<F, R, M, kRope, kOne, kPj>), dim3(grid), dim3(kBlock),
                                   static_cast<uint32_t>(smem), stream, t_start_event, t_stop_event, 0, a);
             t_start_event = t_stop_event = nullptr;
         } else {
-            hipLaunchKernelGGL((gemv_kernel<F, R, M, kRope, kOne>), dim3(grid), dim3(kBlock), smem, stream, a);
+            hipLaunchKernelGGL((gemv_kernel<F, R, M, kRope, kOne, kPj>), dim3(grid), dim3(kBlock), smem, stream, a);
+        }
+    };
+    auto go = [&](auto rope, auto one) {
+        if (short_row) {
+            go_j(rope, one, std::integral_constant<int, 2>{});
+        } else if (nvp <= kLongJ * kBlock) {
+            if constexpr (kLongJ > 2) go_j(rope, one, std::integral_constant<int, kLongJ>{});
+            else go_j(rope, one, std::integral_constant<int, 0>{});
+        } else {
+            go_j(rope, one, std::integral_constant<int, 0>{});   // (the two-pass prologue through LDS)
         }
     };
     if (a.rope_table) {
