@@ -44,7 +44,7 @@
 namespace pie_hip {
 namespace {
 
-constexpr int kBlock = 256;  // 4 waves: one per SIMD of a CU
+constexpr int kBlock = 512;  // 8 waves: two per SIMD of a CU, so one block's prologue serves the whole CU
 constexpr int kWavesPerBlock = kBlock / kWave;
 constexpr int kNumCU = 256;
 constexpr int kUnits = 2;   // work units in flight per wave
@@ -277,8 +277,8 @@ struct GemvArgs {
 // ROPE: the q|k|v epilogue (rotation + KV write); its per-lane cos / sin / slot ride with every
 // unit's loads like the residual does, so the epilogue itself issues no loads.
 // GS1: the unit's int4 group scales come with one load (see issue()).  PJ: activation vectors
-// (8 values) a thread holds per row in the register prologue — 2 covers K <= 4096, the other
-// value 8 / M; a vector-memory instruction costs the CU's address unit sixteen cycles whatever
+// (8 values) a thread holds per row in the register prologue — 1 covers K <= 4096, the other
+// value min(4, 8 / M); a vector-memory instruction costs the CU's address unit sixteen cycles whatever
 // it fetches and every instruction ahead of the first weight request delays it, so short rows
 // get a prologue with no idle trips.
 template <class F, int R, int M, bool ROPE, bool GS1, int PJ>
@@ -764,7 +764,8 @@ thread_local hipEvent_t t_stop_event = nullptr;
 
 // Blocks of a launch: the machine-sized grid, but at least one row (or row pair) per wave.
 int gemv_grid(int N, bool pairs, int waves_per_simd) {
-    int grid = kNumCU * waves_per_simd;
+    int grid = kNumCU * 4 * waves_per_simd / kWavesPerBlock;
+    if (grid < 1) grid = 1;
     const int max_grid = (N / (pairs ? 2 : 1) + kWavesPerBlock - 1) / kWavesPerBlock;
     return grid > max_grid ? max_grid : grid;
 }
@@ -784,9 +785,9 @@ int launch(const GemvArgs& a_in, int waves_per_simd, hipStream_t stream) {
     // (group scales with one load per unit: the R rows' groups of a chunk fit one wave)
     const bool gs1 = F::kGroupScale && a.g_shift >= 0 && a.g_shift <= __builtin_ctz(static_cast<unsigned>(kChunkK)) &&
                      (R << (__builtin_ctz(static_cast<unsigned>(kChunkK)) - a.g_shift)) <= kWave;
-    constexpr int kLongJ = 8 / M;   // (the register prologue's reach: rows of up to 2048 * kLongJ values)
+    constexpr int kLongJ = 8 / M < 4 ? 8 / M : 4;   // (the register prologue's reach: rows of up to 4096 * kLongJ values)
     const int nvp = nchunks * (kChunkK / 8);
-    const bool short_row = nvp <= 2 * kBlock;
+    const bool short_row = nvp <= kBlock;
     auto go_j = [&](auto rope, auto one, auto pj) {
         constexpr bool kRope = decltype(rope)::value, kOne = decltype(one)::value;
         constexpr int kPj = decltype(pj)::value;
@@ -800,10 +801,9 @@ int launch(const GemvArgs& a_in, int waves_per_simd, hipStream_t stream) {
     };
     auto go = [&](auto rope, auto one) {
         if (short_row) {
-            go_j(rope, one, std::integral_constant<int, 2>{});
+            go_j(rope, one, std::integral_constant<int, 1>{});
         } else if (nvp <= kLongJ * kBlock) {
-            if constexpr (kLongJ > 2) go_j(rope, one, std::integral_constant<int, kLongJ>{});
-            else go_j(rope, one, std::integral_constant<int, 0>{});
+            go_j(rope, one, std::integral_constant<int, kLongJ>{});
         } else {
             go_j(rope, one, std::integral_constant<int, 0>{});   // (the two-pass prologue through LDS)
         }
@@ -856,7 +856,7 @@ int dispatch(GemvArgs a, int M, int rows_per_wave, int waves_per_simd, hipStream
     if (waves_per_simd > 8) return PIE_HIP_ERR_INVALID;
     if (rows_per_wave <= 0) {
         const long long per_wave =
-            a.N / (static_cast<long long>(kNumCU) * kWavesPerBlock * waves_per_simd);
+            a.N / (static_cast<long long>(kNumCU) * 4 * waves_per_simd);
         rows_per_wave = per_wave >= 4 ? 4 : (per_wave >= 3 ? 3 : (per_wave >= 2 ? 2 : 1));
     }
     if ((a.swiglu || a.rope_table) && rows_per_wave % 2 != 0) rows_per_wave = rows_per_wave == 3 ? 4 : 2;
