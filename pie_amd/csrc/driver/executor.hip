@@ -99,15 +99,20 @@ void linear_fused(const Linear& w, const uint16_t* act, const uint16_t* norm_w, 
                   size_t gemm_ws_bytes, hipStream_t s) {
     const int fmt = fmt_code(w.kind);
     const int sbf = w.scale_bf16 ? 1 : 0;
-    // Two to four rows: the GEMV pays its dot products once per row (8B shapes, 1..4 rows: gate|up
-    // 16.7 / 21.6 / 26.7 / 31.8 us, down 11.3 / 15.9 / 26.1 / 29.7), the skinny GEMM over the
-    // tile-major copy does not (19 / 12.7 us at any of them) but needs the norm as its own launch
-    // (~4.8 us).  Measured costs decide; without a tile-major copy the GEMV keeps all four.
+    // Two to four rows: the GEMV pays its dot products once per row, the skinny GEMM over the
+    // tile-major copy does not but needs the norm as its own launch (~4.8 us).  Costs fitted to
+    // the 8B shapes decide (decode steps of 2 / 3 / 4 rows over 512-token contexts: 1.91 / 2.46 /
+    // 2.79 ms with the GEMV everywhere, 2.11 / 2.19 / 2.26 ms with the skinny GEMM everywhere);
+    // without a tile-major copy the GEMV keeps all four.
     bool gemv = M <= 4;
-    if (gemv && M >= 2 && w.data_tiled) {
+    // (PIE_GEMV_MAX_ROWS = n: rows up to n take the GEMV, more the skinny GEMM, whatever the costs say)
+    static const int forced_rows = [] { const char* e = getenv("PIE_GEMV_MAX_ROWS"); return e ? atoi(e) : -1; }();
+    if (forced_rows >= 0) {
+        gemv = M <= std::min(forced_rows, 4);
+    } else if (gemv && M >= 2 && w.data_tiled) {
         const double bytes = static_cast<double>(w.data_bytes());
-        const double t_gemv = 5.0 + bytes / 5.5e6 * (1.0 + 0.5 * (M - 1));
-        const double t_skinny = 5.0 + bytes / 3.9e6 + (norm_w ? 4.8 : 0.0);
+        const double t_gemv = 3.4 + bytes / 5.5e6 * (1.0 + 0.5 * (M - 1));
+        const double t_skinny = 4.4 + bytes / 3.9e6 + (norm_w ? 4.8 : 0.0);
         gemv = t_gemv <= t_skinny;
     }
     if (!gemv) {

@@ -453,15 +453,17 @@ __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 && MT == 1 ? 4 : 2) void s
     const int KP = 1 << kp_shift;
     const int ks = wv & (KP - 1);
     const int N = a.N, K = a.K;
-    const int p = a.offsets ? blockIdx.y : 0;
-    const int r0 = a.offsets ? a.offsets[p] : (a.m_split ? blockIdx.y * ROWS : 0);
-    const int r1 = a.offsets ? a.offsets[p + 1] : (a.m_split ? min(a.M, r0 + ROWS) : a.M);
+    // (dense problems only: the grouped MoE launches run the block-shared kernel.  Every scalar
+    // instruction ahead of the first weight request delays it: four waves per SIMD walk this
+    // prologue at once)
+    const int r0 = a.m_split ? blockIdx.y * ROWS : 0;
+    const int r1 = a.m_split ? min(a.M, r0 + ROWS) : a.M;
     if (r1 <= r0) return;
 
     const int T = (N + 15) / 16;
     const int tile0 = (blockIdx.x * (kSwWaves >> kp_shift) + (wv >> kp_shift)) * NG;
-    const unsigned char* wbase = a.w + static_cast<size_t>(p) * a.w_stride;
-    const unsigned char* sbase = a.scale ? a.scale + static_cast<size_t>(p) * a.scale_stride : nullptr;
+    const unsigned char* wbase = a.w;
+    const unsigned char* sbase = a.scale;
     const uint16_t* gsbase = reinterpret_cast<const uint16_t*>(sbase);
     const int blk_shift = a.g_shift - (F::kGroupScale ? 7 : 0);
     const int nb = K / LK;
@@ -476,11 +478,15 @@ __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 && MT == 1 ? 4 : 2) void s
     const unsigned char* wt[NG];
     const uint16_t* st[NG];
     float row_scale[NG];
+    // (one 64-bit product for the wave's first tile; the others are 32-bit steps from it)
+    const int tfirst = min(tile0, T - 1);
+    const unsigned char* wt0 = wbase + static_cast<size_t>(tfirst) * nb * 1024;
+    const uint16_t* st0 = gsbase + static_cast<size_t>(tfirst) * 16 * groups;
 #pragma unroll
     for (int i = 0; i < NG; ++i) {
         const int tile = min(tile0 + i, T - 1);
-        wt[i] = wbase + static_cast<size_t>(tile) * nb * 1024;
-        st[i] = gsbase + static_cast<size_t>(tile) * 16 * groups;
+        wt[i] = wt0 + static_cast<unsigned>(tile - tfirst) * static_cast<unsigned>(nb * 1024);
+        st[i] = st0 + static_cast<unsigned>(tile - tfirst) * static_cast<unsigned>(16 * groups);
         row_scale[i] = 1.f;
         const int n = min(tile * 16 + j, N - 1);
         if (!F::kGroupScale && sbase)
@@ -513,8 +519,7 @@ __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 && MT == 1 ? 4 : 2) void s
         int arow[SV];   // rows past the problem repeat its last row and are never stored
 #pragma unroll
         for (int u = 0; u < SV; ++u) {
-            const int row = min(mt0 + srow + RPL * u, r1 - 1);
-            arow[u] = a.act_rows ? a.act_rows[row] : row;
+            arow[u] = min(mt0 + srow + RPL * u, r1 - 1);
         }
         u32x4_t stg[SV];
         auto stage_load = [&](int c) {
@@ -538,10 +543,12 @@ __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 && MT == 1 ? 4 : 2) void s
             for (int i = 0; i < NG; ++i) acc[t][i] = zero4;
         }
 
+        // (the activations first: loads return in order, so staged behind the weight ring they
+        // would reach LDS only after the last of its eight loads has come back from HBM)
         WOne ring[PF];
+        stage_load(0);
 #pragma unroll
         for (int l = 0; l < PF; ++l) ring[l] = load_w(l / NS, l % NS);
-        stage_load(0);
         stage_store();
 
         auto step = [&](const WOne& cur, int ng, int blk) {
@@ -580,6 +587,17 @@ __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 && MT == 1 ? 4 : 2) void s
         };
 
         for (int c0 = 0; c0 < nch; c0 += CU) {
+            // Issue priority falls with progress: the SIMD's arbiter serves its oldest wave
+            // first, so of the two (or four) waves that share a SIMD one would finish its K slice
+            // well ahead and then idle at the barrier below; a wave that has fallen behind
+            // outranks its neighbours until it has caught up.
+            {
+                const int quarter = (c0 * 4) / nch;
+                if (quarter == 0) __builtin_amdgcn_s_setprio(3);
+                else if (quarter == 1) __builtin_amdgcn_s_setprio(2);
+                else if (quarter == 2) __builtin_amdgcn_s_setprio(1);
+                else __builtin_amdgcn_s_setprio(0);
+            }
 #pragma unroll
             for (int cu = 0; cu < CU; ++cu) {
                 const int c = c0 + cu;
@@ -608,7 +626,9 @@ __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 && MT == 1 ? 4 : 2) void s
         const int nout = a.swiglu ? N / 2 : N;
 #pragma unroll
         for (int t = 0; t < MT; ++t) {
-        __syncthreads();
+        // (a wave's partial sums go to its own staging region, which no other wave reads before
+        // the barrier below: only the second row tile has to wait for the readers of the first)
+        if (t > 0) __syncthreads();
         float* mine = red + static_cast<size_t>(wv) * kRegionF;
 #pragma unroll
         for (int i = 0; i < NG; ++i)
@@ -795,8 +815,7 @@ int launch_skinny(SkinnyArgs a, int problems, hipStream_t stream) {
     // MoE launches stay with the block-shared form, whose eight tiles per staged chunk halve the
     // activation traffic (30B-A3B, 64 rows: 7.9 against 11.0 ms per step)
     if (a.rope_table) return launch_wave<F>(a, problems, stream);   // (entry point checked K)
-    static const bool grouped_wave = getenv("PIE_SKINNY_GROUPED_WAVE") != nullptr;
-    if (a.tiled && (!a.offsets || grouped_wave) && !old_form && a.K % kSwChunk == 0) return launch_wave<F>(a, problems, stream);
+    if (a.tiled && !a.offsets && !old_form && a.K % kSwChunk == 0) return launch_wave<F>(a, problems, stream);
     if (a.K % (8 * LK) == 0) {
         if (tiles / 8 >= 448) return launch_cfg<F, 4, CK, 8, 4, 2>(a, problems, stream);
         if (tiles / 4 >= 448) return launch_cfg<F, 4, CK, 4, 4, 2>(a, problems, stream);
