@@ -49,7 +49,7 @@ OTHER_MODELS = {
     "qwen3-30b-a3b-fp8": (dict(arch="qwen3_moe", hidden=2048, layers=48, q_heads=32, kv_heads=4,
                                head_dim=128, intermediate=0, vocab=151936, rope_theta=1000000.0,
                                quant="fp8", scale_dtype="bf16", num_experts=128, top_k=8,
-                               expert_intermediate=768, router_std=0.0221),
+                               expert_intermediate=768, router_std=0.0221, embed_std=16.0),
                           "Qwen3-30B-A3B-shaped MoE (128 experts, top-8, fp8 e4m3 experts with bf16 "
                           "row scales) greedy decode"),
 }
@@ -331,6 +331,7 @@ def other_configs_extra(drvmod):
         drv = drvmod.Driver(toml(model, page_size, pages, 2048, max(16, batch)))
         t_init = time.perf_counter() - t0
         try:
+            drv.set_generate_divergence(7919)   # distinct rows in the decode batch (distinct MoE routes)
             _, tm = drv.generate(prompt, max_new, replicate=batch, warmup=warm)
         finally:
             drv.close()
@@ -554,6 +555,8 @@ def main():
         drv.set_generate_sampler(kind, 0.8, k, p, seed=12345)
         label = (label or "Llama-3-8B-shaped W4A16 (int4b8 group 128) decode") + f", {args.sampler} sampling at T=0.8"
     torch.cuda.synchronize()
+    if args.batch > 1:
+        drv.set_generate_divergence(7919)   # distinct rows in the decode batch (distinct MoE routes)
     tokens, tm = drv.generate(prompt, max_new, replicate=args.batch, warmup=args.warmup)
     steps = tm["decode_steps"]
     assert steps == args.steps, (steps, args.steps)

@@ -262,6 +262,11 @@ int pie_hip_driver_generate(PieHipDriver* d, const uint32_t* prompt, int n_promp
  * and context.  Returns 0, -1 on a bad kind. */
 int pie_hip_driver_set_generate_sampler(PieHipDriver* d, int kind, float temperature, uint32_t k,
                                         float p, uint32_t seed);
+/* Generation harness only (no counterpart in the reference): with stride > 0 replica c of
+ * pie_hip_driver_generate feeds (its last sampled token + c * stride) % vocab into every decode
+ * step, so the rows of a decode batch differ (distinct MoE routes); 0 (default) keeps identical
+ * replicas. */
+int pie_hip_driver_set_generate_divergence(PieHipDriver* d, uint32_t stride);
 /* Host-only: what the snapshot reader sees in a Hugging Face checkpoint directory, as JSON
  * {"arch", shape fields, "tensors": {name: {"dtype", "shape", "bytes", "first_bytes"}}} written
  * to out.  Returns its length, or -1 with the reader's message in err.  No GPU is touched. */

@@ -45,6 +45,8 @@ struct ModelConfig {
     std::uint64_t seed = 0x9E3779B97F4A7C15ull;
     float init_std = 0.02f;
     float router_std = 0.f;  // MoE router rows; 0 = init_std
+    float embed_std = 0.f;   // embedding rows; 0 = init_std (a large value lets a token's own embedding
+                             // dominate the residual stream, so distinct tokens take distinct MoE routes)
     // `[model] hf_path` (portable driver's key) or `snapshot_dir` (CUDA driver's key): a Hugging
     // Face snapshot directory; its config.json then fixes the shape fields above and the weights
     // come from its safetensors files instead of the synthetic initialiser
@@ -246,6 +248,7 @@ inline DriverConfig parse_config_text(const std::string& text) {
                 else if (k == "seed") m.seed = (std::uint64_t)to_int(v, key);
                 else if (k == "init_std") m.init_std = (float)to_float(v, key);
                 else if (k == "router_std") m.router_std = (float)to_float(v, key);
+                else if (k == "embed_std") m.embed_std = (float)to_float(v, key);
                 else if (k == "hf_path" || k == "snapshot_dir") m.checkpoint_dir = v;
                 // other [model] keys (paths, dtype hints) belong to loaders this driver lacks
             } else if (sec == "batching") {

@@ -237,6 +237,7 @@ struct PieHipDriver {
     std::string last_error;
     PieSamplerDesc gen_sampler{};   // decode-step sampler of the generation harness (kind 2, T 0 = greedy)
     bool gen_sampler_set = false;
+    uint32_t gen_diverge = 0;   // generation harness: replica c starts decoding from (first token + c * this) % vocab
 
     explicit PieHipDriver(const DriverConfig& c) : cfg(c) {
         int ndev = 0;
@@ -550,6 +551,16 @@ extern "C" int pie_hip_driver_set_generate_sampler(PieHipDriver* d, int kind, fl
     return 0;
 }
 
+// Replicas of the generation harness share the prompt; with stride > 0 replica c feeds
+// (its last sampled token + c * stride) % vocab into every decode step, so the rows of a decode
+// batch differ (distinct hidden states, distinct MoE routes) even where a synthetic model's greedy
+// tokens coincide.  0: identical replicas.
+extern "C" int pie_hip_driver_set_generate_divergence(PieHipDriver* d, uint32_t stride) {
+    if (!d) return -1;
+    d->gen_diverge = stride;
+    return 0;
+}
+
 extern "C" int pie_hip_driver_generate(PieHipDriver* d, const uint32_t* prompt, int n_prompt,
                                        int max_new, int replicate, int warmup,
                                        uint32_t* out_tokens, double* timings_us, char* err,
@@ -631,6 +642,7 @@ extern "C" int pie_hip_driver_generate(PieHipDriver* d, const uint32_t* prompt, 
         auto t_decode = clk::now();
         (void)hipEventRecord(e0, d->exec->stream());
         int timed_steps = 0;
+        const uint64_t vocab = static_cast<uint64_t>(std::max(1, d->model.cfg().vocab));
         for (int s = 1; s < max_new; ++s) {
             if (s == warmup + 1 && warmup > 0) {  // restart the clocks after the warm-up steps
                 (void)hipStreamSynchronize(d->exec->stream());
@@ -643,7 +655,7 @@ extern "C" int pie_hip_driver_generate(PieHipDriver* d, const uint32_t* prompt, 
             const int np = (pos + 1 + ps - 1) / ps;
             FrameBuilder fb;
             for (int c = 0; c < replicate; ++c) {
-                fb.tokens.push_back(last[c]);
+                fb.tokens.push_back(static_cast<uint32_t>((last[c] + static_cast<uint64_t>(c) * d->gen_diverge) % vocab));
                 fb.positions.push_back(static_cast<uint32_t>(pos));
                 for (int p = 0; p < np; ++p) fb.pages.push_back(static_cast<uint32_t>(c * pages_per_ctx + p));
                 fb.last_lens.push_back(static_cast<uint32_t>(pos + 1 - (np - 1) * ps));

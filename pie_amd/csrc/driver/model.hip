@@ -277,7 +277,7 @@ void Model::init_synthetic(const ModelConfig& cfg, hipStream_t stream) {
     auto next_seed = [&]() { return seed += 0xA0761D6478BD642Full; };
 
     embed = static_cast<uint16_t*>(alloc(static_cast<size_t>(V) * H * 2, "embed"));
-    fill_normal(embed, static_cast<size_t>(V) * H, next_seed(), 0.f, cfg.init_std, stream);
+    fill_normal(embed, static_cast<size_t>(V) * H, next_seed(), 0.f, cfg.embed_std > 0.f ? cfg.embed_std : cfg.init_std, stream);
     if (cfg.tie_embeddings) {
         lm_head = embed;
         names_["lm_head"] = names_["embed"];

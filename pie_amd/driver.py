@@ -147,6 +147,8 @@ def lib() -> C.CDLL:
         l.pie_hip_driver_handle.argtypes = [C.c_void_p, C.POINTER(FrameDesc), C.POINTER(ResponseFrameDesc)]
         l.pie_hip_driver_generate.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int,
                                               C.c_int, C.c_void_p, C.c_void_p, C.c_char_p, C.c_size_t]
+        l.pie_hip_driver_set_generate_divergence.argtypes = [C.c_void_p, C.c_uint32]
+        l.pie_hip_driver_set_generate_divergence.restype = C.c_int
         l.pie_hip_driver_set_generate_sampler.argtypes = [C.c_void_p, C.c_int, C.c_float, C.c_uint32,
                                                           C.c_float, C.c_uint32]
         l.pie_hip_driver_export_tensor.restype = C.c_size_t
@@ -371,6 +373,12 @@ class Driver:
             raise RuntimeError(f"pie_hip_driver_generate: {err.value.decode()}")
         return out, dict(prefill_us=tm[0], decode_wall_us=tm[1], decode_device_us=tm[2],
                          decode_steps=int(tm[3]))
+
+    def set_generate_divergence(self, stride: int) -> None:
+        """Replica c of `generate` feeds (its last sampled token + c * stride) % vocab into every
+        decode step: the rows of a decode batch then differ (0: identical replicas)."""
+        if lib().pie_hip_driver_set_generate_divergence(self._h, stride) != 0:
+            raise RuntimeError("pie_hip_driver_set_generate_divergence failed")
 
     def set_generate_sampler(self, kind: int, temperature: float, k: int = 0, p: float = 1.0,
                              seed: int = 1):
