@@ -89,7 +89,7 @@ void orc_router_gap_rows(float* out, int n) {
     for (int i = 0; i < n; ++i) out[i] = i < ORC_ROUTER_GAP_ROWS ? g_router_row_gap[i] : 0.f;
 }
 static void orc_router_gap_note(const uint16_t* logits, int N, int E, int K) {
-    if (K >= E) return;
+    if (K < 1 || K >= E || E > 512) return;
     for (int n = 0; n < N; ++n) {
         float v[512];
         for (int j = 0; j < E; ++j) v[j] = orc_bf16_to_f32(logits[(size_t)n * E + j]);
