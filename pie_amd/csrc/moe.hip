@@ -21,17 +21,33 @@ constexpr int kMaxExperts = 512;   // the reference's MAX_EXPERTS (topk_softmax.
 constexpr int kMaxTopK = 16;       // the reference's combine unroll bound (moe_dispatch.cu:128)
 constexpr int kPerLane = kMaxExperts / kWave;
 
-// (value, index) max with ties to the lower index, across the wave.
+// (value, index) max with ties to the lower index, across the wave: four DPP steps inside a
+// 16-lane row, two row swaps across rows (no LDS permutes; the result does not depend on the
+// order of the steps).
+template <int CTRL>
+__device__ __forceinline__ void argmax_dpp_step(float& v, int& i) {
+    const float ov = __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), CTRL, 0xF, 0xF, false));
+    const int oi = __builtin_amdgcn_update_dpp(i, i, CTRL, 0xF, 0xF, false);
+    const bool take = ov > v || (ov == v && oi < i);
+    v = take ? ov : v;
+    i = take ? oi : i;
+}
+__device__ __forceinline__ void argmax_pick(float& v, int& i, float v0, int i0, float v1, int i1) {
+    const bool first = v0 > v1 || (v0 == v1 && i0 < i1);
+    v = first ? v0 : v1;
+    i = first ? i0 : i1;
+}
 __device__ __forceinline__ void wave_argmax(float& v, int& i) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-        const float ov = __shfl_xor(v, off, kWave);
-        const int oi = __shfl_xor(i, off, kWave);
-        if (ov > v || (ov == v && oi < i)) {
-            v = ov;
-            i = oi;
-        }
-    }
+    argmax_dpp_step<0xB1>(v, i);    // quad_perm [1,0,3,2]
+    argmax_dpp_step<0x4E>(v, i);    // quad_perm [2,3,0,1]
+    argmax_dpp_step<0x141>(v, i);   // row_half_mirror
+    argmax_dpp_step<0x140>(v, i);   // row_mirror: every lane holds its row's winner
+    const auto v16 = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    const auto i16 = __builtin_amdgcn_permlane16_swap(static_cast<unsigned>(i), static_cast<unsigned>(i), false, false);
+    argmax_pick(v, i, __uint_as_float(v16[0]), static_cast<int>(i16[0]), __uint_as_float(v16[1]), static_cast<int>(i16[1]));
+    const auto v32 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    const auto i32 = __builtin_amdgcn_permlane32_swap(static_cast<unsigned>(i), static_cast<unsigned>(i), false, false);
+    argmax_pick(v, i, __uint_as_float(v32[0]), static_cast<int>(i32[0]), __uint_as_float(v32[1]), static_cast<int>(i32[1]));
 }
 
 // One wave per token: softmax over the experts, top-k with exclusion, renormalise.
@@ -42,6 +58,8 @@ __global__ __launch_bounds__(256) void moe_topk_kernel(const uint16_t* __restric
     const int t = blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
     if (t >= N) return;
     const uint16_t* row = logits + static_cast<size_t>(t) * E;
+    // (entries j >= nper hold no expert: the passes below skip them)
+    const int nper = (E + kWave - 1) / kWave;
     float p[kPerLane];
     float mx = -3.4e38f;
 #pragma unroll
@@ -55,8 +73,10 @@ __global__ __launch_bounds__(256) void moe_topk_kernel(const uint16_t* __restric
 #pragma unroll
     for (int j = 0; j < kPerLane; ++j) {
         const int e = lane + kWave * j;
-        p[j] = e < E ? expf(p[j] - mx) : 0.f;
-        sum += p[j];
+        float ex = 0.f;
+        if (j < nper) ex = e < E ? expf(p[j] - mx) : 0.f;   // (a wave-uniform test)
+        p[j] = ex;
+        sum += ex;
     }
     sum = wave_sum(sum);
     const float inv_z = 1.f / sum;
@@ -69,7 +89,7 @@ __global__ __launch_bounds__(256) void moe_topk_kernel(const uint16_t* __restric
         int bi = kMaxExperts;
 #pragma unroll
         for (int j = 0; j < kPerLane; ++j)
-            if (p[j] > bv) {
+            if (j < nper && p[j] > bv) {
                 bv = p[j];
                 bi = lane + kWave * j;
             }
@@ -77,7 +97,7 @@ __global__ __launch_bounds__(256) void moe_topk_kernel(const uint16_t* __restric
         bi = min(bi, E - 1);   // only reachable with NaN logits; keeps every index in range
 #pragma unroll
         for (int j = 0; j < kPerLane; ++j)
-            if (bi == lane + kWave * j) p[j] = -1.f;   // exclude on the next pass
+            if (j < nper && bi == lane + kWave * j) p[j] = -1.f;   // exclude on the next pass
         w_sum += bv;
         if (lane == k) {
             my_w = bv;
