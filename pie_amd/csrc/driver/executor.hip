@@ -115,7 +115,14 @@ void linear_fused(const Linear& w, const uint16_t* act, const uint16_t* norm_w, 
         const double t_skinny = 4.4 + bytes / 3.9e6 + (norm_w ? 4.8 : 0.0);
         gemv = t_gemv <= t_skinny;
     }
-    if (!gemv) {
+    if (gemv) {
+        const int st = pie_hip_linear_fused(fmt, act, norm_w, eps, w.data, w.scale, sbf, w.group, y, M, w.N, w.K,
+                                            beta, swiglu, s);
+        if (st == PIE_HIP_OK) return;
+        if (st != PIE_HIP_ERR_UNSUPPORTED) PIE_KERNEL(st);
+        // (a row too long for the GEMV's staged activations: the matrix-core kernels take any K)
+    }
+    {
         const uint16_t* a = act;
         if (norm_w) {
             PIE_KERNEL(pie_hip_rmsnorm(act, norm_w, norm_tmp, M, w.K, eps, s));
@@ -142,10 +149,7 @@ void linear_fused(const Linear& w, const uint16_t* act, const uint16_t* norm_w, 
         if (st != PIE_HIP_ERR_UNSUPPORTED) PIE_KERNEL(st);
         PIE_KERNEL(pie_hip_linear_fused(fmt, a, nullptr, eps, w.data, w.scale, sbf, w.group, y, M,
                                         w.N, w.K, beta, swiglu, s));
-        return;
     }
-    PIE_KERNEL(pie_hip_linear_fused(fmt, act, norm_w, eps, w.data, w.scale, sbf, w.group, y, M,
-                                    w.N, w.K, beta, swiglu, s));
 }
 
 }  // namespace
@@ -424,13 +428,18 @@ void Executor::body(int N, int S, int max_kv_len) {
             } else {
                 PIE_KERNEL(st);
             }
-        } else if (N <= 4 && fused_rope && !w.q_norm) {
-            // decode rows of llama-type layers: rotation and KV write ride in the projection
-            PIE_KERNEL(pie_hip_qkv_rope_fused(fmt_code(w.wqkv.kind), x_, w.attn_norm, m.rms_eps,
-                                              w.wqkv.data, w.wqkv.scale, w.wqkv.scale_bf16 ? 1 : 0,
-                                              w.wqkv.group, N, H, rope_tab_, slots, q_, k_pool_[l],
-                                              v_pool_[l], hq, hk, d, pairing, s));
         } else {
+            // decode rows of llama-type layers: rotation and KV write ride in the projection
+            // (a hidden size past the GEMV's staged-activation limit takes the general route)
+            int fused_st = PIE_HIP_ERR_UNSUPPORTED;
+            if (N <= 4 && fused_rope && !w.q_norm) {
+                fused_st = pie_hip_qkv_rope_fused(fmt_code(w.wqkv.kind), x_, w.attn_norm, m.rms_eps, w.wqkv.data,
+                                                  w.wqkv.scale, w.wqkv.scale_bf16 ? 1 : 0, w.wqkv.group, N, H,
+                                                  rope_tab_, slots, q_, k_pool_[l], v_pool_[l], hq, hk, d,
+                                                  pairing, s);
+                if (fused_st != PIE_HIP_OK && fused_st != PIE_HIP_ERR_UNSUPPORTED) PIE_KERNEL(fused_st);
+            }
+            if (fused_st != PIE_HIP_OK) {
             // a decode batch of llama-type layers on the skinny GEMM: rotation and KV write ride
             // in its epilogue too (one launch less per layer)
             bool done = false;
@@ -448,6 +457,7 @@ void Executor::body(int N, int S, int max_kv_len) {
                 linear_fused(w.wqkv, x_, w.attn_norm, m.rms_eps, qkv_, N, 0, 0, xn_, gemm_ws_, gemm_ws_bytes_, s);
                 PIE_KERNEL(pie_hip_qkv_rope_kvwrite(qkv_, q_, k_pool_[l], v_pool_[l], w.q_norm, w.k_norm,
                                                     rope_tab_, slots, N, hq, hk, d, pairing, m.rms_eps, s));
+            }
             }
         }
         // 4-bit blocks: the pages this batch reads become bf16 in the shared pool pair, which the

@@ -102,6 +102,9 @@ def check_step(oracle, gpu_logit_bits, orc_logit_bits, gpu_tok, orc_tok, cos_min
     dict(quant="int4b8", page_size=32, use_graphs=False),
     dict(quant="int4b8", rope_interleaved=True),
     dict(quant="bf16", rope_interleaved=True, use_graphs=False),
+    # a down projection whose rows are past the GEMV's staged-activation limit for one-byte
+    # weights (16 384 values): single-row decode steps take the matrix-core route for it
+    dict(quant="int8", scale_dtype="bf16", intermediate=16384),
     dict(arch="qwen3_moe", quant="fp8", head_dim=128, q_heads=4, kv_heads=1, num_experts=8, top_k=2,
          expert_intermediate=256, router_std=0.2, intermediate=0),
     dict(arch="qwen3_moe", quant="int4b8", head_dim=128, q_heads=4, kv_heads=1, num_experts=16,

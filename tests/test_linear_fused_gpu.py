@@ -74,6 +74,41 @@ def test_norm_fused_equals_norm_then_linear(gpu, oracle, kind, M, N, K):
 
 
 @pytest.mark.parametrize("kind", ["int4b8", "int8", "fp8", "bf16"])
+@pytest.mark.parametrize("M,N,K", [
+    # rows of up to 4096 values: one activation vector per thread in the register prologue
+    (2, 64, 4096), (4, 40, 4096),
+    # longer rows: four vectors per thread (one or two activation rows), two with three or four
+    (1, 64, 6144), (1, 48, 14336), (2, 48, 14336), (1, 40, 4224), (1, 32, 16384), (4, 40, 8192),
+    # past the registers' reach: the two-pass prologue through LDS
+    (3, 40, 14336), (1, 32, 18432),
+])
+def test_norm_fused_over_every_activation_prologue(gpu, oracle, kind, M, N, K):
+    """The GEMV picks its activation prologue from the row length and the row count; every
+    variant stages the same bf16 values (fused norm on and off) as the norm kernel followed by
+    the plain projection."""
+    import torch
+    from pie_amd import ops
+
+    if kind in ("int8", "fp8") and K > 15360:
+        pytest.skip("one-byte weights stage their activations as f32: rows of up to 15 360 values (the driver sends longer ones to the matrix-core GEMM)")
+    rng = np.random.default_rng(130 + M + K)
+    wd, mk = make_weight(oracle, rng, kind, N, K)
+    x = oracle.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32) * 2)
+    nw = oracle.f32_to_bf16(rng.uniform(0.5, 1.5, K).astype(np.float32))
+    w = mk(gpu)
+    xg, nwg = dev(x, gpu, torch.bfloat16), dev(nw, gpu, torch.bfloat16)
+    plain = bits(ops.linear_fused(xg, w))
+    ref_plain = oracle_linear(oracle, wd, x)
+    assert close_to_oracle(oracle, plain, ref_plain)
+    assert (ulp_diff(plain, ref_plain) <= 1).mean() > 0.98
+    fused = bits(ops.linear_fused(xg, w, norm_weight=nwg, eps=1e-5))
+    unfused = bits(ops.linear_fused(ops.rmsnorm_bf16(xg, nwg, 1e-5), w))
+    d = ulp_diff(fused, unfused)
+    assert d.max() <= 1 and (d == 0).mean() > 0.97
+    assert close_to_oracle(oracle, fused, oracle_linear(oracle, wd, oracle.rmsnorm(x, nw, 1e-5)))
+
+
+@pytest.mark.parametrize("kind", ["int4b8", "int8", "fp8", "bf16"])
 @pytest.mark.parametrize("M,I,K", [(1, 256, 2048), (2, 1024, 512), (4, 152, 1024), (5, 64, 4096)])
 def test_swiglu_epilogue_equals_linear_then_swiglu(gpu, oracle, kind, M, I, K):
     import torch
