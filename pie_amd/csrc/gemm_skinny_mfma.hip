@@ -499,8 +499,12 @@ __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 && MT == 1 ? 4 : 2) void s
     const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
 
     // step `lin` of chunk c: tile lin / CB, block lin % CB of the chunk
+    // (the ring runs ahead of the arithmetic, so its last trips reach past the wave's K slice:
+    // those requests repeat the slice's own last block — a cache hit — instead of fetching the
+    // neighbour's blocks a second time)
+    const int b_last = max(b_lo, min(nb, b_lo + nch * CB) - 1);
     auto load_w = [&](int c, int lin) {
-        const int b = min(b_lo + c * CB + lin % CB, nb - 1);
+        const int b = min(b_lo + c * CB + lin % CB, b_last);
         WOne sl;
         sl.w = *reinterpret_cast<const u32x4_t*>(wt[lin / CB] + static_cast<size_t>(b) * 1024 + lane16);
         sl.gs = F::kGroupScale ? (st[lin / CB] + static_cast<size_t>(b >> blk_shift) * 16)[j] : uint16_t(0);
@@ -523,7 +527,7 @@ __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 && MT == 1 ? 4 : 2) void s
         }
         u32x4_t stg[SV];
         auto stage_load = [&](int c) {
-            const int k0 = min((b_lo + c * CB) * LK + svec * 8, K - 8);
+            const int k0 = min((b_lo + min(c, max(nch - 1, 0)) * CB) * LK + svec * 8, K - 8);   // (past the slice: its last chunk again)
 #pragma unroll
             for (int u = 0; u < SV; ++u)
                 if (u < SV / 2 || !r8)
