@@ -74,6 +74,9 @@ struct RuntimeConfig {
     // request does not pay one-time costs (measured: 58 ms cold against 47 ms for a 2048-token
     // prefill of an 8B model); writes only KV pages nobody owns yet
     bool warmup = true;
+    // time the candidate kernels of every decoder linear at start-up (2-4 and 17-128 rows, a few
+    // tens of milliseconds) and dispatch on the measurements instead of the fitted cost model
+    bool tune_linears = true;
     std::string snapshot_dir;
 };
 
@@ -266,6 +269,7 @@ inline DriverConfig parse_config_text(const std::string& text) {
                 else if (k == "use_graphs") r.use_graphs = to_bool(v, key);
                 else if (k == "tiled_weights") r.tiled_weights = to_bool(v, key);
                 else if (k == "warmup") r.warmup = to_bool(v, key);
+                else if (k == "tune_linears") r.tune_linears = to_bool(v, key);
                 else if (k == "snapshot_dir") r.snapshot_dir = v;
             }
         }

@@ -94,9 +94,12 @@ GemmPath pick_gemm(const Linear& w, int M, size_t ws_bytes) {
 // (norm as its own kernel into `norm_tmp`): the matrix-core skinny GEMM, which streams the
 // weights once per 16 rows, or the tiled matrix-core GEMM where its cost model wins; shapes those do
 // not take fall back to the GEMV path.
-void linear_fused(const Linear& w, const uint16_t* act, const uint16_t* norm_w, float eps,
+// `force`: -1 = pick (the start-up measurement when there is one, else the cost model); 0..3 = that
+// kernel whatever the costs (the tuner's own launches).  Returns false when a forced kernel does
+// not take the shape.
+bool linear_fused(const Linear& w, const uint16_t* act, const uint16_t* norm_w, float eps,
                   uint16_t* y, int M, int beta, int swiglu, uint16_t* norm_tmp, void* gemm_ws,
-                  size_t gemm_ws_bytes, hipStream_t s) {
+                  size_t gemm_ws_bytes, hipStream_t s, int force = -1) {
     const int fmt = fmt_code(w.kind);
     const int sbf = w.scale_bf16 ? 1 : 0;
     // Two to four rows: the GEMV pays its dot products once per row, the skinny GEMM over the
@@ -107,7 +110,10 @@ void linear_fused(const Linear& w, const uint16_t* act, const uint16_t* norm_w, 
     bool gemv = M <= 4;
     // (PIE_GEMV_MAX_ROWS = n: rows up to n take the GEMV, more the skinny GEMM, whatever the costs say)
     static const int forced_rows = [] { const char* e = getenv("PIE_GEMV_MAX_ROWS"); return e ? atoi(e) : -1; }();
-    if (forced_rows >= 0) {
+    const int tuned = force >= 0 ? force : (M <= 128 ? w.tuned[M] : -1);
+    if (tuned >= 0) {
+        gemv = tuned == 0 && M <= 4;
+    } else if (forced_rows >= 0) {
         gemv = M <= std::min(forced_rows, 4);
     } else if (gemv && M >= 2 && w.data_tiled) {
         const double bytes = static_cast<double>(w.data_bytes());
@@ -118,8 +124,9 @@ void linear_fused(const Linear& w, const uint16_t* act, const uint16_t* norm_w, 
     if (gemv) {
         const int st = pie_hip_linear_fused(fmt, act, norm_w, eps, w.data, w.scale, sbf, w.group, y, M, w.N, w.K,
                                             beta, swiglu, s);
-        if (st == PIE_HIP_OK) return;
+        if (st == PIE_HIP_OK) return true;
         if (st != PIE_HIP_ERR_UNSUPPORTED) PIE_KERNEL(st);
+        if (force >= 0) return false;
         // (a row too long for the GEMV's staged activations: the matrix-core kernels take any K)
     }
     {
@@ -128,7 +135,10 @@ void linear_fused(const Linear& w, const uint16_t* act, const uint16_t* norm_w, 
             PIE_KERNEL(pie_hip_rmsnorm(act, norm_w, norm_tmp, M, w.K, eps, s));
             a = norm_tmp;
         }
-        const GemmPath path = pick_gemm(w, M, gemm_ws_bytes);
+        const GemmPath path = tuned == 1   ? GemmPath::Skinny
+                              : tuned == 2 ? GemmPath::Tiled
+                              : tuned == 3 ? GemmPath::TiledSplitK
+                                           : pick_gemm(w, M, gemm_ws_bytes);
         if (path != GemmPath::Skinny) {
             // the tiled GEMM (weights dequantised to bf16 while staged), in K shares for a
             // decode batch whose output has few tiles
@@ -137,19 +147,22 @@ void linear_fused(const Linear& w, const uint16_t* act, const uint16_t* norm_w, 
                                                           w.K, beta, swiglu, gemm_ws, gemm_ws_bytes, s)
                                : pie_hip_gemm_mfma(fmt, a, w.data, w.scale, sbf, w.group, y, M, w.N, w.K,
                                                    beta, swiglu, s);
-            if (sg == PIE_HIP_OK) return;
+            if (sg == PIE_HIP_OK) return true;
             if (sg != PIE_HIP_ERR_UNSUPPORTED) PIE_KERNEL(sg);
+            if (force >= 0) return false;
         }
         const int st = w.data_tiled
                            ? pie_hip_gemm_skinny_tiled(fmt, a, w.data_tiled, w.scale_tiled ? w.scale_tiled : w.scale,
                                                        sbf, w.group, y, M, w.N, w.K, beta, swiglu, s)
                            : pie_hip_gemm_skinny(fmt, a, w.data, w.scale, sbf, w.group, y, M, w.N, w.K, beta,
                                                  swiglu, s);
-        if (st == PIE_HIP_OK) return;
+        if (st == PIE_HIP_OK) return true;
         if (st != PIE_HIP_ERR_UNSUPPORTED) PIE_KERNEL(st);
+        if (force >= 0) return false;
         PIE_KERNEL(pie_hip_linear_fused(fmt, a, nullptr, eps, w.data, w.scale, sbf, w.group, y, M,
                                         w.N, w.K, beta, swiglu, s));
     }
+    return true;
 }
 
 }  // namespace
@@ -248,6 +261,7 @@ Executor::Executor(const DriverConfig& cfg, Model& model) : cfg_(cfg), model_(mo
     PIE_HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&in_host_), in_.total, hipHostMallocDefault));
     PIE_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&in_dev_), in_.total));
     PIE_HIP_CHECK(hipHostMalloc(reinterpret_cast<void**>(&out_host_), T * 4, hipHostMallocDefault));
+    tune_linears();
 }
 
 Executor::~Executor() {
@@ -293,6 +307,93 @@ size_t Executor::scale_page_bytes() const {
         return static_cast<size_t>(page_size_) * m.kv_heads * ((m.head_dim + 15) / 16) * sizeof(float);
     const bool scaled = kv_format_ == PIE_HIP_KV_INT8_PER_TOKEN_HEAD || kv_format_ == PIE_HIP_KV_FP8_PER_TOKEN_HEAD;
     return scaled ? static_cast<size_t>(page_size_) * m.kv_heads * sizeof(float) : 0;
+}
+
+// Start-up measurement of the decoder linears' candidate kernels.  For every role (q|k|v, wo,
+// gate|up, down) and a ladder of row counts the GEMV (2-4 rows), the skinny GEMM and the tiled GEMM
+// (17-128 rows; in K shares where the workspace allows) run over the weights of successive layers
+// (so that they come from HBM, as in a forward pass) on zeroed activations; the fastest goes into
+// every layer's table for the row counts up to the next rung.
+void Executor::tune_linears() {
+    const ModelConfig& m = model_.cfg();
+    if (model_.layers.empty() || !cfg_.runtime.tune_linears || getenv("PIE_NO_TUNE")) return;
+    hipStream_t s = stream_;
+    const size_t T = static_cast<size_t>(max_tokens_);
+    const int H = m.hidden, d = m.head_dim, hq = m.q_heads, hk = m.kv_heads;
+    const int I = model_.is_moe() ? m.expert_intermediate : m.intermediate;
+    PIE_HIP_CHECK(hipMemsetAsync(x_, 0, T * H * 2, s));
+    PIE_HIP_CHECK(hipMemsetAsync(attn_, 0, T * hq * d * 2, s));
+    if (!model_.is_moe()) PIE_HIP_CHECK(hipMemsetAsync(act_, 0, T * I * 2, s));
+    struct Role {
+        Linear LayerWeights::*lin;
+        uint16_t* LayerWeights::*norm;
+        const uint16_t* act;
+        uint16_t* y;
+        int beta, swiglu;
+        double tiled_handicap_us;   // what the tiled route costs beyond the GEMM (a separate RoPE launch)
+    };
+    std::vector<Role> roles = {
+        {&LayerWeights::wqkv, &LayerWeights::attn_norm, x_, qkv_, 0, 0, 4.0},
+        {&LayerWeights::wo, nullptr, attn_, x_, 1, 0, 0.0},
+    };
+    if (!model_.is_moe()) {
+        roles.push_back({&LayerWeights::wgu, &LayerWeights::ffn_norm, x_, act_, 0, 1, 0.0});
+        roles.push_back({&LayerWeights::wdown, nullptr, act_, x_, 1, 0, 0.0});
+    }
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    PIE_HIP_CHECK(hipEventCreate(&e0));
+    PIE_HIP_CHECK(hipEventCreate(&e1));
+    const int L = static_cast<int>(model_.layers.size());
+    int rot = 0;
+    auto time_us = [&](const Role& r, int M, int force) -> double {
+        constexpr int kWarm = 1, kReps = 4;
+        for (int i = 0; i < kWarm + kReps; ++i) {
+            if (i == kWarm) PIE_HIP_CHECK(hipEventRecord(e0, s));
+            LayerWeights& lw = model_.layers[static_cast<size_t>(rot++ % L)];
+            const uint16_t* nw = r.norm ? lw.*(r.norm) : nullptr;
+            if (!linear_fused(lw.*(r.lin), r.act, nw, m.rms_eps, r.y, M, r.beta, r.swiglu, xn_, gemm_ws_,
+                              gemm_ws_bytes_, s, force))
+                return 1e30;
+        }
+        PIE_HIP_CHECK(hipEventRecord(e1, s));
+        PIE_HIP_CHECK(hipEventSynchronize(e1));
+        float ms = 0.f;
+        PIE_HIP_CHECK(hipEventElapsedTime(&ms, e0, e1));
+        return static_cast<double>(ms) * 1e3 / kReps;
+    };
+    const int ladder[] = {2, 3, 4, 17, 24, 32, 33, 40, 48, 56, 64, 65, 72, 80, 88, 96, 97, 104, 112, 120, 128};
+    for (const Role& r : roles) {
+        const Linear& l0 = model_.layers[0].*(r.lin);
+        if (!l0.data || !l0.data_tiled) continue;   // (without the tile-major copy the cost model's defaults stand)
+        int prev = 1;
+        for (int M : ladder) {
+            if (M > max_tokens_) break;
+            int best = -1;
+            double best_t = 1e30;
+            for (int cand = M <= 4 ? 0 : 1; cand <= (M <= 4 ? 1 : 3); ++cand) {
+                if (cand == 3 && (M > 128 || pie_hip_gemm_mfma_workspace_bytes(M, l0.N, l0.K) == 0 ||
+                                  pie_hip_gemm_mfma_workspace_bytes(M, l0.N, l0.K) > gemm_ws_bytes_))
+                    continue;
+                if (cand >= 2 && l0.K % 64 != 0) continue;
+                double t = time_us(r, M, cand);
+                if (cand >= 2) t += r.tiled_handicap_us;
+                if (t < best_t) {
+                    best_t = t;
+                    best = cand;
+                }
+            }
+            // rows 5..16 stay with the skinny GEMM; a rung decides for the row counts above the
+            // previous rung up to itself
+            const int lo = M <= 4 ? M : std::max(prev + 1, 17);
+            if (best >= 0)
+                for (auto& lw : model_.layers)
+                    for (int mm = lo; mm <= M; ++mm) (lw.*(r.lin)).tuned[static_cast<size_t>(mm)] = static_cast<int8_t>(best);
+            prev = M;
+        }
+    }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    PIE_HIP_CHECK(hipStreamSynchronize(s));
 }
 
 // Allocate the pool; on out-of-memory halve the page count down to 64 pages
@@ -443,8 +544,9 @@ void Executor::body(int N, int S, int max_kv_len) {
             // a decode batch of llama-type layers on the skinny GEMM: rotation and KV write ride
             // in its epilogue too (one launch less per layer)
             bool done = false;
+            const int tuned_qkv = N <= 128 ? w.wqkv.tuned[N] : -1;
             if (fused_rope && !w.q_norm && w.wqkv.data_tiled &&
-                pick_gemm(w.wqkv, N, gemm_ws_bytes_) == GemmPath::Skinny) {
+                (tuned_qkv >= 0 ? tuned_qkv <= 1 : pick_gemm(w.wqkv, N, gemm_ws_bytes_) == GemmPath::Skinny)) {
                 PIE_KERNEL(pie_hip_rmsnorm(x_, w.attn_norm, xn_, N, H, m.rms_eps, s));
                 const int st = pie_hip_qkv_rope_skinny_tiled(
                     fmt_code(w.wqkv.kind), xn_, w.wqkv.data_tiled,

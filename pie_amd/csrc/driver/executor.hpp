@@ -104,6 +104,7 @@ class Executor {
     void collect_samplers(const BatchPlan& plan, SampleOutputs& out);
     void moe_block(const LayerWeights& w, int N, hipStream_t s);
     void alloc_kv();
+    void tune_linears();
 
     DriverConfig cfg_;
     Model& model_;

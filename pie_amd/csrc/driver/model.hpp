@@ -12,6 +12,7 @@
 // three stay unquantised like the reference (driver/cuda/src/config.hpp:20-30).
 #pragma once
 
+#include <array>
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -34,6 +35,10 @@ struct Linear {
     // optional copies in the skinny GEMM's tile-major layout (pie_hip_repack_mfma_tiles)
     void* data_tiled = nullptr;
     void* scale_tiled = nullptr;   // int4 group scales; other formats keep `scale`
+    // kernel that measured fastest for M activation rows at start-up (index M, 0..128):
+    // 0 GEMV, 1 skinny GEMM, 2 tiled GEMM, 3 tiled GEMM in K shares; -1: not measured, the cost
+    // model decides
+    std::array<int8_t, 129> tuned = [] { std::array<int8_t, 129> t{}; t.fill(-1); return t; }();
     size_t data_bytes() const {
         const size_t nk = static_cast<size_t>(N) * K;
         switch (kind) {
