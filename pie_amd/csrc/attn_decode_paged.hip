@@ -315,16 +315,17 @@ __global__ __launch_bounds__(kAttnBlock) void attn_decode_split_kernel(
 //   S^T[key, query] = K . Q^T      A = K fragment from the wave's LDS region (row = key, k = d; rows
 //                                  padded to D + 8), B = the GQA query heads of the row in the
 //                                  first GQA of 16 columns (the rest are zero)
-//   O^T[d, query]  += V^T . P^T    A = V^T from the wave's LDS region, B = P from registers
+//   O^T[d, query]  += V^T . P^T    A = V^T read transposed (ds_read_b64_tr_b16) from the V rows
+//                                  in the wave's LDS region, B = P from registers
 // The query sits on the lane%16 axis of both accumulators, so max / sum / rescale are per lane
 // and cost two cross-lane steps per 32 keys instead of four per key and head.  The keys of a
 // step leave the first product in the order [4g..4g+3, 16+4g..16+4g+3] per 16-lane group g —
-// the order V^T is laid out in LDS (rows padded to 80 B: conflict-free operand reads).
+// the rows the group's two transposing reads of a V^T fragment take (V rows padded to D + 16).
 // Probabilities enter the second product as a bf16 pair (hi + lo), i.e. with 16 mantissa bits,
 // so the result keeps the accuracy of the fp32 kernel above.
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
 constexpr int kMStepKeys = 32;
-constexpr int kMVtStride = kMStepKeys + 8;
 
 template <int D, int GQA, int KVF = kKvBf16, bool MASKED = false>
 __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
@@ -345,22 +346,21 @@ __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
     constexpr int EB = Q8 ? 1 : 2;             // stored bytes per element
     constexpr int LPR = D * EB / 16;           // 16-byte pieces per stored K/V row
     constexpr int NK = kMStepKeys * LPR / kWave;   // K load instructions per step
-    constexpr int VC = 16 * LPR / kWave;       // (key pair, piece) combos per lane per step
-    constexpr int PG = LPR < 8 ? LPR : 8;      // adjacent lanes that take adjacent V pieces
     constexpr int PF = 2;                      // steps of K/V in flight per wave
-    static_assert(GQA <= 16 && VC >= 1 && NK >= 1, "shape");
+    static_assert(GQA <= 16 && NK >= 1, "shape");
     const unsigned char* k_pages = static_cast<const unsigned char*>(k_pages_raw);
     const unsigned char* v_pages = static_cast<const unsigned char*>(v_pages_raw);
     constexpr int KSTRIDE = D + 8;             // bf16 elements per K row in LDS (padded: conflict-free reads)
-    // V^T rows are 80 bytes; every 16 rows the region skips another 32 bytes, so the eight pieces
-    // (row groups) a staging write touches start in different banks
-    __shared__ __attribute__((aligned(16))) uint16_t vt_all[kAttnWaves][D * kMVtStride + D];
-    auto vt_at = [](int row, int col) { return row * kMVtStride + (row >> 4) * 16 + col; };
+    // V rows sit in LDS as they are stored (padded to D + 16: the four rows a transposing read
+    // touches start eight banks apart); the V^T operand of the second product comes out of
+    // ds_read_b64_tr_b16, which hands lane i of a 16-lane group element i of four 16-element rows
+    constexpr int VSTRIDE = D + 16;
+    __shared__ __attribute__((aligned(16))) uint16_t vs_all[kAttnWaves][kMStepKeys * VSTRIDE];
     __shared__ __attribute__((aligned(16))) uint16_t ks_all[kAttnWaves][kMStepKeys * KSTRIDE];
     __shared__ float sm_m[kAttnWaves][16];
     __shared__ float sm_l[kAttnWaves][16];
     __shared__ __attribute__((aligned(16))) float sc_all[Q8 ? kAttnWaves : 1][kWave];   // K | V scales of a step
-    static_assert(sizeof(float) * GQA * D <= sizeof(uint16_t) * D * kMVtStride, "per-wave output fits its V^T region");
+    static_assert(sizeof(float) * GQA * D <= sizeof(uint16_t) * kMStepKeys * VSTRIDE, "per-wave output fits its V region");
 
     const int kvh = blockIdx.x, split = blockIdx.y, r = blockIdx.z;
     const int tid = threadIdx.x, lane = tid & (kWave - 1);
@@ -389,22 +389,13 @@ __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
         }
     }
 
-    uint16_t* Vt = vt_all[wv];
+    uint16_t* Vs = vs_all[wv];
     uint16_t* Ks = ks_all[wv];
-    // K loads: whole rows, LPR adjacent lanes per key (kWave / LPR keys per instruction)
+    // K and V loads: whole rows, LPR adjacent lanes per key (kWave / LPR keys per instruction)
     constexpr int KPI = kWave / LPR;
-    u32x4_t kreg[PF][NK], vreg[PF][2 * VC];
+    u32x4_t kreg[PF][NK], vreg[PF][NK];
     float sreg[PF];   // one-byte pools: lane < 32 holds the K scale of key `lane`, the others V's
     uint32_t mreg[PF];   // MASKED: the visibility words of the step's two 16-token units
-    // V loads: combo c of a lane = (key pair, 16-byte piece); eight adjacent lanes take eight
-    // adjacent pieces (128 contiguous bytes of a row)
-    auto v_piece = [&](int c) { return (lane % PG) + PG * (c % (LPR / PG)); };
-    // key pairs of one instruction: (0,1,8,9,2,3,10,11) + 4c', whose V^T columns are words 0..7
-    // (8..15) of a row — with the row-group skew every lane of a staging write has its own bank
-    auto v_pair = [&](int c) {
-        const int i = lane / PG;
-        return (i & 1) + 2 * ((i >> 2) & 1) + 8 * ((i >> 1) & 1) + 4 * ((i >> 3) + (kWave / PG / 8) * (c / (LPR / PG)));
-    };
     // A 32-key step starts on a multiple of 16 and touches at most two pages (page_size % 16 == 0);
     // their ids come through scalar loads.  Keys past the split repeat its last key (finite
     // data; their probabilities are zero).
@@ -431,13 +422,9 @@ __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
             kreg[slot][i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(
                 k_pages + row_th(lane / LPR + KPI * i) * (D * EB) + (lane % LPR) * 16));
 #pragma unroll
-        for (int c = 0; c < VC; ++c) {
-            const int pair = v_pair(c), dc = v_piece(c);
-#pragma unroll
-            for (int u = 0; u < 2; ++u)
-                vreg[slot][2 * c + u] = __builtin_nontemporal_load(
-                    reinterpret_cast<const u32x4_t*>(v_pages + row_th(2 * pair + u) * (D * EB) + dc * 16));
-        }
+        for (int i = 0; i < NK; ++i)
+            vreg[slot][i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(
+                v_pages + row_th(lane / LPR + KPI * i) * (D * EB) + (lane % LPR) * 16));
         if constexpr (Q8) {
             const float* sp = lane < kMStepKeys ? k_scales : v_scales;
             sreg[slot] = sp ? sp[row_sc(lane & (kMStepKeys - 1))] : 1.f;
@@ -448,42 +435,23 @@ __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
             mreg[slot] = static_cast<uint32_t>(mrow[u0]) | (static_cast<uint32_t>(mrow[min(u0 + 1, nunits - 1)]) << 16);
         }
     };
-    // V rows -> V^T in the wave's LDS region: two adjacent keys of one piece meet in one lane and
-    // leave as 4-byte writes (slot of key kappa: 8*(kappa%16/4) + kappa%4, +4 for kappa >= 16)
+    // K and V rows into the wave's LDS regions as they are stored (one-byte codes become bf16 on
+    // the way)
     auto stage = [&](int slot) {
 #pragma unroll
         for (int i = 0; i < NK; ++i) {
-            uint16_t* dst = &Ks[(lane / LPR + KPI * i) * KSTRIDE + (lane % LPR) * (16 / EB)];
+            const int row = lane / LPR + KPI * i, piece = (lane % LPR) * (16 / EB);
+            uint16_t* kd = &Ks[row * KSTRIDE + piece];
+            uint16_t* vd = &Vs[row * VSTRIDE + piece];
             if constexpr (!Q8) {
-                *reinterpret_cast<u32x4_t*>(dst) = kreg[slot][i];
+                *reinterpret_cast<u32x4_t*>(kd) = kreg[slot][i];
+                *reinterpret_cast<u32x4_t*>(vd) = vreg[slot][i];
             } else {   // 16 codes -> 16 bf16
-                const u32x4_t w = kreg[slot][i];
-                *reinterpret_cast<u32x4_t*>(dst) = kv_decode_bf16<KVF>(u32x2_t{w.x, w.y});
-                *reinterpret_cast<u32x4_t*>(dst + 8) = kv_decode_bf16<KVF>(u32x2_t{w.z, w.w});
-            }
-        }
-#pragma unroll
-        for (int c = 0; c < VC; ++c) {
-            const int pair = v_pair(c), dc = v_piece(c);
-            const int kappa = 2 * pair;
-            const int col = kappa < 16 ? 8 * (kappa >> 2) + (kappa & 3) : 8 * ((kappa - 16) >> 2) + 4 + (kappa & 3);
-            const u32x4_t a = vreg[slot][2 * c], b = vreg[slot][2 * c + 1];
-            if constexpr (!Q8) {
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const uint32_t lo = (a[e >> 1] >> (16 * (e & 1))) & 0xFFFFu;
-                    const uint32_t hi = (b[e >> 1] >> (16 * (e & 1))) & 0xFFFFu;
-                    *reinterpret_cast<uint32_t*>(&Vt[vt_at(dc * 8 + e, col)]) = lo | (hi << 16);
-                }
-            } else {   // 16 elements of two adjacent keys: (bf16(a_e), bf16(b_e)) pairs
-#pragma unroll
-                for (int h = 0; h < 2; ++h) {
-                    uint32_t ab[8];
-                    kv_decode_bf16_pairs<KVF>(u32x2_t{a[2 * h], a[2 * h + 1]}, u32x2_t{b[2 * h], b[2 * h + 1]}, ab);
-#pragma unroll
-                    for (int e = 0; e < 8; ++e)
-                        *reinterpret_cast<uint32_t*>(&Vt[vt_at(dc * 16 + 8 * h + e, col)]) = ab[e];
-                }
+                const u32x4_t w = kreg[slot][i], x = vreg[slot][i];
+                *reinterpret_cast<u32x4_t*>(kd) = kv_decode_bf16<KVF>(u32x2_t{w.x, w.y});
+                *reinterpret_cast<u32x4_t*>(kd + 8) = kv_decode_bf16<KVF>(u32x2_t{w.z, w.w});
+                *reinterpret_cast<u32x4_t*>(vd) = kv_decode_bf16<KVF>(u32x2_t{x.x, x.y});
+                *reinterpret_cast<u32x4_t*>(vd + 8) = kv_decode_bf16<KVF>(u32x2_t{x.z, x.w});
             }
         }
         if constexpr (Q8) sc_all[wv][lane] = sreg[slot];
@@ -560,8 +528,14 @@ __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
         const bf16x8_t p_lo = __builtin_bit_cast(bf16x8_t, u32x4_t{lo[0], lo[1], lo[2], lo[3]});
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
-            const bf16x8_t vf = __builtin_bit_cast(
-                bf16x8_t, *reinterpret_cast<const u32x4_t*>(&Vt[vt_at(16 * dt + l16, 8 * g)]));
+            // V^T fragment of dimension 16 dt + l16: keys 4g..4g+3 and 16+4g..16+4g+3, the order of
+            // the probabilities above.  Lane i of the group addresses 8 bytes of row (i / 4) at
+            // column block (i % 4) and receives element i of each of the four rows.
+            const uint16_t* va = &Vs[(4 * g + (l16 >> 2)) * VSTRIDE + 16 * dt + 4 * (l16 & 3)];
+            const bf16x4_t v0 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) bf16x4_t*)(va));
+            const bf16x4_t v1 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+                (__attribute__((address_space(3))) bf16x4_t*)(va + 16 * VSTRIDE));
+            const bf16x8_t vf = __builtin_shufflevector(v0, v1, 0, 1, 2, 3, 4, 5, 6, 7);
             acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, p_hi, acc[dt], 0, 0, 0);
             acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, p_lo, acc[dt], 0, 0, 0);
         }
@@ -578,7 +552,7 @@ __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
     // this wave's result into its own LDS region (as floats), then the four waves are merged
     lsum += __shfl_xor(lsum, 16, kWave);
     lsum += __shfl_xor(lsum, 32, kWave);
-    float* so = reinterpret_cast<float*>(Vt);   // [GQA][D]
+    float* so = reinterpret_cast<float*>(Vs);   // [GQA][D]
     if (l16 < GQA) {
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
@@ -600,7 +574,7 @@ __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
 #pragma unroll
         for (int w = 0; w < kAttnWaves; ++w) {
             const float a = exp2f(sm_m[w][h] - safe);
-            ov += reinterpret_cast<const float*>(vt_all[w])[h * D + dd] * a;
+            ov += reinterpret_cast<const float*>(vs_all[w])[h * D + dd] * a;
             ls += sm_l[w][h] * a;
         }
         const int head = kvh * GQA + h;

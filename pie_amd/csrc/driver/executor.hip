@@ -88,6 +88,24 @@ GemmPath pick_gemm(const Linear& w, int M, size_t ws_bytes) {
     return tiled < skinny ? GemmPath::Tiled : GemmPath::Skinny;
 }
 
+// The fitted cost model's kernel for M rows of `w`: 0 GEMV, 1 skinny GEMM, 2 tiled GEMM, 3 tiled GEMM
+// in K shares.  Two to four rows: the GEMV pays its dot products once per row, the skinny GEMM over
+// the tile-major copy does not but needs the norm as its own launch (~4.8 us).  Costs fitted to
+// the 8B shapes decide (decode steps of 2 / 3 / 4 rows over 512-token contexts: 1.91 / 2.46 /
+// 2.79 ms with the GEMV everywhere, 2.11 / 2.19 / 2.26 ms with the skinny GEMM everywhere);
+// without a tile-major copy the GEMV keeps all four.
+int model_route(const Linear& w, int M, bool has_norm, size_t ws_bytes) {
+    if (M <= 4) {
+        if (M < 2 || !w.data_tiled) return 0;
+        const double bytes = static_cast<double>(w.data_bytes());
+        const double t_gemv = 3.4 + bytes / 5.5e6 * (1.0 + 0.5 * (M - 1));
+        const double t_skinny = 4.4 + bytes / 3.9e6 + (has_norm ? 4.8 : 0.0);
+        if (t_gemv <= t_skinny) return 0;
+    }
+    const GemmPath p = pick_gemm(w, M, ws_bytes);
+    return p == GemmPath::Skinny ? 1 : p == GemmPath::Tiled ? 2 : 3;
+}
+
 // y = epilogue(rmsnorm?(act) · W^T) by the weight's storage format — the dispatcher role of
 // gemm_act_x_w (driver/cuda/src/ops/gemm.cpp:1414-1583).  Up to four rows: the weight-streaming
 // GEMV with the norm riding in its activation staging and SwiGLU in its epilogue.  More rows
@@ -102,24 +120,17 @@ bool linear_fused(const Linear& w, const uint16_t* act, const uint16_t* norm_w, 
                   size_t gemm_ws_bytes, hipStream_t s, int force = -1) {
     const int fmt = fmt_code(w.kind);
     const int sbf = w.scale_bf16 ? 1 : 0;
-    // Two to four rows: the GEMV pays its dot products once per row, the skinny GEMM over the
-    // tile-major copy does not but needs the norm as its own launch (~4.8 us).  Costs fitted to
-    // the 8B shapes decide (decode steps of 2 / 3 / 4 rows over 512-token contexts: 1.91 / 2.46 /
-    // 2.79 ms with the GEMV everywhere, 2.11 / 2.19 / 2.26 ms with the skinny GEMM everywhere);
-    // without a tile-major copy the GEMV keeps all four.
-    bool gemv = M <= 4;
     // (PIE_GEMV_MAX_ROWS = n: rows up to n take the GEMV, more the skinny GEMM, whatever the costs say)
     static const int forced_rows = [] { const char* e = getenv("PIE_GEMV_MAX_ROWS"); return e ? atoi(e) : -1; }();
-    const int tuned = force >= 0 ? force : (M <= 128 ? w.tuned[M] : -1);
+    int tuned = force >= 0 ? force : (M <= 128 ? w.tuned[M] : -1);
+    bool gemv;
     if (tuned >= 0) {
         gemv = tuned == 0 && M <= 4;
     } else if (forced_rows >= 0) {
         gemv = M <= std::min(forced_rows, 4);
-    } else if (gemv && M >= 2 && w.data_tiled) {
-        const double bytes = static_cast<double>(w.data_bytes());
-        const double t_gemv = 3.4 + bytes / 5.5e6 * (1.0 + 0.5 * (M - 1));
-        const double t_skinny = 4.4 + bytes / 3.9e6 + (norm_w ? 4.8 : 0.0);
-        gemv = t_gemv <= t_skinny;
+    } else {
+        tuned = model_route(w, M, norm_w != nullptr, gemm_ws_bytes);
+        gemv = tuned == 0;
     }
     if (gemv) {
         const int st = pie_hip_linear_fused(fmt, act, norm_w, eps, w.data, w.scale, sbf, w.group, y, M, w.N, w.K,
@@ -138,7 +149,7 @@ bool linear_fused(const Linear& w, const uint16_t* act, const uint16_t* norm_w, 
         const GemmPath path = tuned == 1   ? GemmPath::Skinny
                               : tuned == 2 ? GemmPath::Tiled
                               : tuned == 3 ? GemmPath::TiledSplitK
-                                           : pick_gemm(w, M, gemm_ws_bytes);
+                                           : pick_gemm(w, M, gemm_ws_bytes);   // (forced row limit, GEMV refusal)
         if (path != GemmPath::Skinny) {
             // the tiled GEMM (weights dequantised to bf16 while staged), in K shares for a
             // decode batch whose output has few tiles
@@ -369,7 +380,8 @@ void Executor::tune_linears() {
         for (int M : ladder) {
             if (M > max_tokens_) break;
             int best = -1;
-            double best_t = 1e30;
+            double best_t = 1e30, model_t = 1e30;
+            const int by_model = model_route(l0, M, r.norm != nullptr, gemm_ws_bytes_);
             for (int cand = M <= 4 ? 0 : 1; cand <= (M <= 4 ? 1 : 3); ++cand) {
                 if (cand == 3 && (M > 128 || pie_hip_gemm_mfma_workspace_bytes(M, l0.N, l0.K) == 0 ||
                                   pie_hip_gemm_mfma_workspace_bytes(M, l0.N, l0.K) > gemm_ws_bytes_))
@@ -377,11 +389,16 @@ void Executor::tune_linears() {
                 if (cand >= 2 && l0.K % 64 != 0) continue;
                 double t = time_us(r, M, cand);
                 if (cand >= 2) t += r.tiled_handicap_us;
+                if (cand == by_model) model_t = t;
                 if (t < best_t) {
                     best_t = t;
                     best = cand;
                 }
             }
+            // A measurement overrides the cost model only where it is clearly faster (a tenth and
+            // half a microsecond): candidates that tie keep the model's kernel, so that timing noise
+            // does not change which kernel — and with it which rounding — a restart gets.
+            if (model_t < 1e29 && !(best_t < 0.9 * model_t && best_t + 0.5 < model_t)) best = by_model;
             // rows 5..16 stay with the skinny GEMM; a rung decides for the row counts above the
             // previous rung up to itself
             const int lo = M <= 4 ? M : std::max(prev + 1, 17);

@@ -791,14 +791,33 @@ def test_yarn_scaled_model_matches_oracle(gpu, oracle):
 
 def test_start_up_warm_up_changes_no_result(gpu):
     """[runtime] warmup runs a synthetic chunk over unowned pages at start-up: with it on or off
-    the same request gives the same tokens and the same logits, bit for bit."""
+    the same request gives the same tokens and the same logits, bit for bit (with the kernel per
+    linear fixed by the cost model: the start-up measurement may pick another, see the next test)."""
     from pie_amd import driver as drvmod
 
     rng = np.random.default_rng(98)
     prompt = rng.integers(0, 2048, 23)
     outs = []
     for warm in (True, False):
-        with drvmod.Driver(toml_config(warmup=warm)) as d:
+        with drvmod.Driver(toml_config(warmup=warm, tune_linears=False)) as d:
             toks, _ = d.generate(prompt, 6, replicate=2)
             outs.append((toks.copy(), d.export_tensor("debug.logits", np.uint16).copy()))
     assert np.array_equal(outs[0][0], outs[1][0]) and np.array_equal(outs[0][1], outs[1][1])
+
+
+def test_start_up_kernel_measurement_keeps_results_within_rounding(gpu, oracle):
+    """[runtime] tune_linears times each decoder linear's candidate kernels at start-up and may route
+    a row count to another kernel than the cost model: the kernels sum in different orders, so the
+    logits agree to bf16 rounding (cosine, worst element), not bit for bit."""
+    from pie_amd import driver as drvmod
+
+    rng = np.random.default_rng(99)
+    prompt = rng.integers(0, 2048, 19)
+    outs = []
+    for tune in (True, False):
+        with drvmod.Driver(toml_config(tune_linears=tune)) as d:
+            d.generate(prompt, 1, replicate=3)
+            outs.append(oracle.bf16_to_f32(d.export_tensor("debug.logits", np.uint16)).astype(np.float64).ravel())
+    a, b = outs
+    assert a.shape == b.shape and cosine(a, b) > 0.9995
+    assert np.max(np.abs(a - b)) <= 0.05 * np.max(np.abs(b)) + 1e-3
