@@ -498,16 +498,17 @@ __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 && MT == 1 ? 4 : 2) void s
     const bf16x8_t ones = __builtin_bit_cast(bf16x8_t, u32x4_t{0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u});
     const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
 
-    // step `lin` of chunk c: tile lin / CB, block lin % CB of the chunk
+    // step `lin` of chunk c: block lin / NG of the chunk, tile lin % NG — block-major, so the
+    // activation fragments of a block are read from LDS once and serve all NG tiles
     // (the ring runs ahead of the arithmetic, so its last trips reach past the wave's K slice:
     // those requests repeat the slice's own last block — a cache hit — instead of fetching the
     // neighbour's blocks a second time)
     const int b_last = max(b_lo, min(nb, b_lo + nch * CB) - 1);
     auto load_w = [&](int c, int lin) {
-        const int b = min(b_lo + c * CB + lin % CB, b_last);
+        const int b = min(b_lo + c * CB + lin / NG, b_last);
         WOne sl;
-        sl.w = *reinterpret_cast<const u32x4_t*>(wt[lin / CB] + static_cast<size_t>(b) * 1024 + lane16);
-        sl.gs = F::kGroupScale ? (st[lin / CB] + static_cast<size_t>(b >> blk_shift) * 16)[j] : uint16_t(0);
+        sl.w = *reinterpret_cast<const u32x4_t*>(wt[lin % NG] + static_cast<size_t>(b) * 1024 + lane16);
+        sl.gs = F::kGroupScale ? (st[lin % NG] + static_cast<size_t>(b >> blk_shift) * 16)[j] : uint16_t(0);
         return sl;
     };
 
@@ -539,7 +540,7 @@ __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 && MT == 1 ? 4 : 2) void s
                 if (u < SV / 2 || !r8) lds_a[(srow + RPL * u) * STRIDE + svec] = F::order(stg[u]);
         };
 
-        f32x4_t acc[MT][NG], sxs[MT][F::kGroupScale ? CB : 1], sxt[MT];
+        f32x4_t acc[MT][NG], sxt[MT];
 #pragma unroll
         for (int t = 0; t < MT; ++t) {
             sxt[t] = zero4;
@@ -555,38 +556,54 @@ __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 && MT == 1 ? 4 : 2) void s
         for (int l = 0; l < PF; ++l) ring[l] = load_w(l / NS, l % NS);
         stage_store();
 
+        // The fragments of the current block (read at its first tile) and, for group-scaled
+        // biased codes, bias * (the block's activation sums): the sums come from MFMAs against
+        // ones and enter every tile's product as its initial accumulator.
+        bf16x8_t ax[MT][S];
+        f32x4_t sxb[MT];
         auto step = [&](const WOne& cur, int ng, int blk) {
-            const int vbase = blk * (LK / 8) + q * S;
-            const int sxi = F::kGroupScale ? blk : 0;
+            if (ng == 0) {
+                const int vbase = blk * (LK / 8) + q * S;
+#pragma unroll
+                for (int t = 0; t < MT; ++t)
+#pragma unroll
+                    for (int s = 0; s < S; ++s)
+                        ax[t][s] = __builtin_bit_cast(bf16x8_t, lds_a[(t * 16 + jr) * STRIDE + vbase + s]);
+                if (kBiased) {
+#pragma unroll
+                    for (int t = 0; t < MT; ++t) {
+                        if (F::kGroupScale) {
+                            f32x4_t sx = zero4;
+#pragma unroll
+                            for (int s = 0; s < S; ++s) sx = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax[t][s], ones, sx, 0, 0, 0);
+                            sxb[t] = sx * F::kBias;
+                        } else {
+#pragma unroll
+                            for (int s = 0; s < S; ++s) sxt[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax[t][s], ones, sxt[t], 0, 0, 0);
+                        }
+                    }
+                }
+            }
             f32x4_t part[MT];
 #pragma unroll
-            for (int t = 0; t < MT; ++t) part[t] = zero4;
+            for (int t = 0; t < MT; ++t) part[t] = F::kGroupScale && kBiased ? sxb[t] : zero4;
 #pragma unroll
             for (int s = 0; s < S; ++s) {
                 const bf16x8_t bw = __builtin_bit_cast(bf16x8_t, F::decode(cur.w, s, magic));
 #pragma unroll
                 for (int t = 0; t < MT; ++t) {
-                    const bf16x8_t ax = __builtin_bit_cast(bf16x8_t, lds_a[(t * 16 + jr) * STRIDE + vbase + s]);
-                    if (kBiased && ng == 0) {
-                        if (F::kGroupScale)
-                            sxs[t][sxi] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax, ones, s == 0 ? zero4 : sxs[t][sxi], 0, 0, 0);
-                        else
-                            sxt[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax, ones, sxt[t], 0, 0, 0);
-                    }
                     if (F::kGroupScale)
-                        part[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax, bw, part[t], 0, 0, 0);
+                        part[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax[t][s], bw, part[t], 0, 0, 0);
                     else
-                        acc[t][ng] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax, bw, acc[t][ng], 0, 0, 0);
+                        acc[t][ng] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ax[t][s], bw, acc[t][ng], 0, 0, 0);
                 }
             }
             if (F::kGroupScale) {
                 const float sc = bf16_bits_to_f32(cur.gs);
 #pragma unroll
-                for (int t = 0; t < MT; ++t) {
-                    if (ng == 0) sxs[t][sxi] = sxs[t][sxi] * F::kBias;
+                for (int t = 0; t < MT; ++t)
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) acc[t][ng][r] = fmaf(sc, part[t][r] + sxs[t][sxi][r], acc[t][ng][r]);
-                }
+                    for (int r = 0; r < 4; ++r) acc[t][ng][r] = fmaf(sc, part[t][r], acc[t][ng][r]);
             }
         };
 
@@ -616,7 +633,7 @@ __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 && MT == 1 ? 4 : 2) void s
                     // at the loop end, which waits for every load in flight.  The scheduling
                     // barriers keep the order (left alone, the scheduler also gathers all loads
                     // of a chunk behind all of its arithmetic).
-                    step(ring[slot], lin / CB, lin % CB);   // K is whole chunks: no step is partial
+                    step(ring[slot], lin % NG, lin / NG);   // K is whole chunks: no step is partial
                     __builtin_amdgcn_sched_barrier(0);
                     ring[slot] = load_w(c + (lin + PF) / NS, (lin + PF) % NS);
                     __builtin_amdgcn_sched_barrier(0);
