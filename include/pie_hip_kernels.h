@@ -217,11 +217,14 @@ int pie_hip_moe_grouped_gemm(int format, const uint16_t* act_bf16, const int32_t
  * row-major [N, K] matrix — are stored at byte ((t * nb + b) * 64 + 16 q + j) * 16, nb =
  * row_bytes / 64, so every wave load is 1 KiB contiguous instead of 16 rows x 64 bytes (rows past
  * N are zero; dst holds ceil(N/16) * 16 * row_bytes bytes).  int4 group scales [N, groups] become
- * [tile][group][16 rows].  Built once at load; the values and their evaluation order are those of
- * the row-major entry points, bit for bit.  Role in the reference: Marlin's offline weight
- * repack (driver/cuda/third_party/marlin/marlin_wrapper.hpp:39-51).
+ * [tile][group][16 rows].  Built once at load; the values are those of the row-major entry
+ * points.  int4b8 weights take pie_hip_repack_mfma_tiles_int4, which also re-orders the eight
+ * codes of every 32-bit word (codes 2i and 2i + 1 to nibbles i and i + 4) so that the kernels'
+ * decode yields them in k order; the other formats take pie_hip_repack_mfma_tiles.  Role in the
+ * reference: Marlin's offline weight repack (driver/cuda/third_party/marlin/marlin_wrapper.hpp:39-51).
  */
 int pie_hip_repack_mfma_tiles(const void* src, void* dst, int N, size_t row_bytes, void* stream);
+int pie_hip_repack_mfma_tiles_int4(const void* src, void* dst, int N, size_t row_bytes, void* stream);
 int pie_hip_repack_scale_tiles(const uint16_t* src, uint16_t* dst, int N, int groups, void* stream);
 /* pie_hip_gemm_skinny / pie_hip_moe_grouped_gemm over weights (and int4 group scales) in that
  * layout; every other argument as there (expert strides in bytes of the tiled buffers). */

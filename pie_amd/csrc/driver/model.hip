@@ -140,7 +140,10 @@ void Model::build_tiled_copies(hipStream_t stream) {
             const size_t row_bytes = w->data_bytes() / static_cast<size_t>(w->N);
             if (row_bytes % 64 != 0) continue;
             w->data_tiled = alloc(w->data_bytes(), "");
-            if (pie_hip_repack_mfma_tiles(w->data, w->data_tiled, w->N, row_bytes, stream) != PIE_HIP_OK)
+            const int st = w->kind == Quant::Int4b8
+                               ? pie_hip_repack_mfma_tiles_int4(w->data, w->data_tiled, w->N, row_bytes, stream)
+                               : pie_hip_repack_mfma_tiles(w->data, w->data_tiled, w->N, row_bytes, stream);
+            if (st != PIE_HIP_OK)
                 throw std::runtime_error("model: weight repack failed");
             if (w->kind == Quant::Int4b8) {
                 w->scale_tiled = alloc(w->scale_bytes(), "");

@@ -245,7 +245,7 @@ __global__ __launch_bounds__(KP* kWave) void skinny_kernel(const SkinnyArgs a) {
             const int nvec = min(CK, K - min(c, nchunks - 1) * CK) / 8;
 #pragma unroll
             for (int u = 0; u < SV; ++u)
-                if (u * TPR + sv < nvec) lds_a[sm * STRIDE + u * TPR + sv] = F::order(stg[u]);
+                if (u * TPR + sv < nvec) lds_a[sm * STRIDE + u * TPR + sv] = TILED ? stg[u] : F::order(stg[u]);   // (tile-major int4 codes sit in k order)
         };
 
         constexpr int NSX = F::kGroupScale ? GC * WL : 1;
@@ -504,11 +504,20 @@ __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 && MT == 1 ? 4 : 2) void s
     // those requests repeat the slice's own last block — a cache hit — instead of fetching the
     // neighbour's blocks a second time)
     const int b_last = max(b_lo, min(nb, b_lo + nch * CB) - 1);
+    // Group scales: one load per block for all NG tiles — lane 16 i + j fetches tile i's scale of
+    // weight row j — carried in the ring slot of the block's first tile; a tile's step reads its
+    // value across the wave.  (A load per tile and step made a third of the kernel's vector-memory
+    // instructions, and those, not the bytes, are what a CU's address unit runs out of.)
+    static_assert(NG <= 4, "a wave's lanes hold the scales of NG tiles of 16 rows");
+    const uint16_t* gsp = st[0];
+#pragma unroll
+    for (int i = 1; i < NG; ++i) gsp = (lane >> 4) == i ? st[i] : gsp;
+    if ((lane >> 4) >= NG) gsp = st[NG - 1];
     auto load_w = [&](int c, int lin) {
         const int b = min(b_lo + c * CB + lin / NG, b_last);
         WOne sl;
         sl.w = *reinterpret_cast<const u32x4_t*>(wt[lin % NG] + static_cast<size_t>(b) * 1024 + lane16);
-        sl.gs = F::kGroupScale ? (st[lin % NG] + static_cast<size_t>(b >> blk_shift) * 16)[j] : uint16_t(0);
+        sl.gs = F::kGroupScale && lin % NG == 0 ? (gsp + static_cast<size_t>(b >> blk_shift) * 16)[j] : uint16_t(0);
         return sl;
     };
 
@@ -537,7 +546,7 @@ __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 && MT == 1 ? 4 : 2) void s
         auto stage_store = [&]() {
 #pragma unroll
             for (int u = 0; u < SV; ++u)
-                if (u < SV / 2 || !r8) lds_a[(srow + RPL * u) * STRIDE + svec] = F::order(stg[u]);
+                if (u < SV / 2 || !r8) lds_a[(srow + RPL * u) * STRIDE + svec] = stg[u];
         };
 
         f32x4_t acc[MT][NG], sxt[MT];
@@ -561,8 +570,10 @@ __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 && MT == 1 ? 4 : 2) void s
         // ones and enter every tile's product as its initial accumulator.
         bf16x8_t ax[MT][S];
         f32x4_t sxb[MT];
+        int gsb = 0;   // the current block's scales, tile i's in lanes 16 i .. 16 i + 15
         auto step = [&](const WOne& cur, int ng, int blk) {
             if (ng == 0) {
+                gsb = cur.gs;
                 const int vbase = blk * (LK / 8) + q * S;
 #pragma unroll
                 for (int t = 0; t < MT; ++t)
@@ -599,7 +610,8 @@ __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 && MT == 1 ? 4 : 2) void s
                 }
             }
             if (F::kGroupScale) {
-                const float sc = bf16_bits_to_f32(cur.gs);
+                const float sc = bf16_bits_to_f32(static_cast<uint16_t>(
+                    ng == 0 && NG == 1 ? gsb : __builtin_amdgcn_ds_bpermute((ng * 16 + j) * 4, gsb)));
 #pragma unroll
                 for (int t = 0; t < MT; ++t)
 #pragma unroll
@@ -851,9 +863,21 @@ int launch_skinny(SkinnyArgs a, int problems, hipStream_t stream) {
 // and K block b — byte 64 b + 16 q of row 16 t + j — move to ((t*nb + b)*64 + 16 q + j)*16, so a
 // wave's load is 1 KiB contiguous.  One thread per 16-byte block of the destination; rows past N
 // are zero.
+// int4 (`nibble_pairs`): the eight codes of a 32-bit word also change places — codes 2i and 2i + 1
+// go to nibbles i and i + 4 — so that the decode's (nibble i, nibble i + 4) pairs come out in k
+// order and the activations are staged as they are stored.
+__device__ __forceinline__ uint32_t pair_nibbles(uint32_t v) {
+    uint32_t r = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        r |= ((v >> (8 * i)) & 0xFu) << (4 * i);
+        r |= ((v >> (8 * i + 4)) & 0xFu) << (4 * i + 16);
+    }
+    return r;
+}
 __global__ __launch_bounds__(256) void repack_tiles_kernel(const u32x4_t* __restrict__ src,
                                                            u32x4_t* __restrict__ dst, int N, int nb,
-                                                           size_t total) {
+                                                           size_t total, int nibble_pairs) {
     const size_t idx = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
     if (idx >= total) return;
     const int lane = static_cast<int>(idx & 63);
@@ -863,6 +887,7 @@ __global__ __launch_bounds__(256) void repack_tiles_kernel(const u32x4_t* __rest
     const size_t n = tile * 16 + (lane & 15);
     u32x4_t v = {0u, 0u, 0u, 0u};
     if (n < static_cast<size_t>(N)) v = src[n * (static_cast<size_t>(nb) * 4) + b * 4 + (lane >> 4)];
+    if (nibble_pairs) v = u32x4_t{pair_nibbles(v.x), pair_nibbles(v.y), pair_nibbles(v.z), pair_nibbles(v.w)};
     dst[idx] = v;
 }
 // int4 group scales [N, groups] -> [tile][group][16 rows]
@@ -1035,8 +1060,8 @@ extern "C" int pie_hip_moe_grouped_gemm_tiled(int format, const uint16_t* act_bf
     return dispatch_skinny(format, a, num_experts, static_cast<hipStream_t>(stream));
 }
 
-extern "C" int pie_hip_repack_mfma_tiles(const void* src, void* dst, int N, size_t row_bytes,
-                                         void* stream) {
+namespace {
+int repack_tiles(const void* src, void* dst, int N, size_t row_bytes, void* stream, int nibble_pairs) {
     if (!src || !dst || N <= 0 || row_bytes == 0) return PIE_HIP_ERR_INVALID;
     if (row_bytes % 64 != 0) return PIE_HIP_ERR_UNSUPPORTED;
     const int nb = static_cast<int>(row_bytes / 64);
@@ -1044,8 +1069,19 @@ extern "C" int pie_hip_repack_mfma_tiles(const void* src, void* dst, int N, size
     if ((total + 255) / 256 > 0x7FFFFFFFull) return PIE_HIP_ERR_UNSUPPORTED;
     hipLaunchKernelGGL(pie_hip::repack_tiles_kernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256),
                        0, static_cast<hipStream_t>(stream), static_cast<const pie_hip::u32x4_t*>(src),
-                       static_cast<pie_hip::u32x4_t*>(dst), N, nb, total);
+                       static_cast<pie_hip::u32x4_t*>(dst), N, nb, total, nibble_pairs);
     return pie_hip::launch_status();
+}
+}  // namespace
+
+extern "C" int pie_hip_repack_mfma_tiles(const void* src, void* dst, int N, size_t row_bytes,
+                                         void* stream) {
+    return repack_tiles(src, dst, N, row_bytes, stream, 0);
+}
+
+extern "C" int pie_hip_repack_mfma_tiles_int4(const void* src, void* dst, int N, size_t row_bytes,
+                                              void* stream) {
+    return repack_tiles(src, dst, N, row_bytes, stream, 1);
 }
 
 extern "C" int pie_hip_repack_scale_tiles(const uint16_t* src, uint16_t* dst, int N, int groups,

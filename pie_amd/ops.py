@@ -392,8 +392,9 @@ def repack_mfma_tiles(w: WeightView) -> WeightView:
     flat = w.data.reshape(rows, -1).contiguous()
     row_bytes = flat.shape[1] * flat.element_size()
     dst = torch.empty(((rows + 15) // 16 * 16, flat.shape[1]), dtype=flat.dtype, device=flat.device)
-    _check(kernels().pie_hip_repack_mfma_tiles(_ptr(flat), _ptr(dst), rows, C.c_size_t(row_bytes), _stream()),
-           "pie_hip_repack_mfma_tiles")
+    # (int4: the codes of every 32-bit word are also put in the order the kernels decode them in)
+    repack = kernels().pie_hip_repack_mfma_tiles_int4 if w.kind == "int4b8" else kernels().pie_hip_repack_mfma_tiles
+    _check(repack(_ptr(flat), _ptr(dst), rows, C.c_size_t(row_bytes), _stream()), "pie_hip_repack_mfma_tiles")
     scale = w.scale
     if w.kind == "int4b8":
         sf = w.scale.reshape(rows, -1).contiguous()

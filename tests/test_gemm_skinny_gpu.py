@@ -154,7 +154,8 @@ def test_moe_grouped_gemm_matches_per_expert_oracle(gpu, oracle, kind, swiglu):
 @pytest.mark.parametrize("N,K", [(80, 1024), (100, 512), (12304, 512)])
 def test_tile_major_repack_is_the_documented_permutation(gpu, oracle, kind, N, K):
     """dst[((t*nb + b)*64 + 16q + j)*16 ..] = the 16 bytes at byte 64b + 16q of row 16t + j; rows
-    past N are zero; int4 group scales become [tile][group][16]."""
+    past N are zero; int4: codes 2i, 2i + 1 of every 32-bit word sit in nibbles i, i + 4, and the
+    group scales become [tile][group][16]."""
     import torch
     from pie_amd import ops
 
@@ -168,6 +169,13 @@ def test_tile_major_repack_is_the_documented_permutation(gpu, oracle, kind, N, K
     padded = np.zeros((tiles * 16, row_bytes), np.uint8)
     padded[:N] = src
     want = padded.reshape(tiles, 16, nb, 4, 16).transpose(0, 2, 3, 1, 4)      # [t][b][q][j][16 bytes]
+    if kind == "int4b8":
+        words = np.ascontiguousarray(want).reshape(-1).view(np.uint32)
+        paired = np.zeros_like(words)
+        for i in range(4):
+            paired |= ((words >> np.uint32(8 * i)) & np.uint32(0xF)) << np.uint32(4 * i)
+            paired |= ((words >> np.uint32(8 * i + 4)) & np.uint32(0xF)) << np.uint32(4 * i + 16)
+        want = paired.view(np.uint8)
     assert np.array_equal(t.data.view(torch.uint8).cpu().numpy().reshape(-1), want.reshape(-1))
     if kind == "int4b8":
         sc = w.scale.view(torch.uint16).cpu().numpy()
