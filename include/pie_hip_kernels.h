@@ -260,10 +260,16 @@ int pie_hip_moe_grouped_gemm_tiled(int format, const uint16_t* act_bf16, const i
  *   expert_offsets [E+1], route_token [T*top_k] (token of each sorted route),
  *   route_pos [T*top_k] (sorted position of route (t, k)).
  * num_experts <= 512, top_k <= 16 (the reference's bounds).
+ * pie_hip_moe_route_opt: renormalize = 0 leaves the chosen experts' softmax probabilities undivided
+ * (norm_topk = false: the graph form divides only under it, graph_common.cpp:279-283);
+ * pie_hip_moe_route is renormalize = 1.
  */
 int pie_hip_moe_route(const uint16_t* router_logits_bf16, int32_t* topk_idx, float* topk_weight,
                       int32_t* expert_offsets, int32_t* route_token, int32_t* route_pos,
                       int num_tokens, int num_experts, int top_k, void* stream);
+int pie_hip_moe_route_opt(const uint16_t* router_logits_bf16, int32_t* topk_idx, float* topk_weight,
+                      int32_t* expert_offsets, int32_t* route_token, int32_t* route_pos,
+                      int num_tokens, int num_experts, int top_k, int renormalize, void* stream);
 
 /*
  * MoE combine: out[t, :] = bf16( (add ? out[t, :] : 0) + sum_k topk_weight[t, k] *

@@ -302,13 +302,15 @@ def gemm_fp8(act_bf16, q, scale_inv, mode: int = 0, y_in=None, want_abs: bool = 
     return (y32, y16, ab) if want_abs else (y32, y16)
 
 
-def topk_softmax(logits_bf16, top_k: int):
-    """(idx int32 [N, k], weights f32 [N, k]) — driver/cuda/src/kernels/topk_softmax.cu:19-86."""
+def topk_softmax(logits_bf16, top_k: int, renorm: bool = True):
+    """(idx int32 [N, k], weights f32 [N, k]) — driver/cuda/src/kernels/topk_softmax.cu:19-86;
+    renorm=False leaves the chosen experts' probabilities undivided (norm_topk = false,
+    driver/portable/src/graph_common.cpp:279-283)."""
     lg = _c(logits_bf16, np.uint16)
     N, E = lg.shape
     idx = np.empty((N, top_k), np.int32)
     w = np.empty((N, top_k), np.float32)
-    lib().orc_topk_softmax(_p(lg), _p(idx), _p(w), C.c_int(N), C.c_int(E), C.c_int(top_k))
+    lib().orc_topk_softmax_opt(_p(lg), _p(idx), _p(w), C.c_int(N), C.c_int(E), C.c_int(top_k), C.c_int(1 if renorm else 0))
     return idx, w
 
 

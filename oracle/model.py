@@ -29,7 +29,7 @@ class _Model(C.Structure):
                 ("wqkv", C.POINTER(_Linear)), ("wo", C.POINTER(_Linear)),
                 ("wgu", C.POINTER(_Linear)), ("wdown", C.POINTER(_Linear)),
                 ("num_experts", C.c_int), ("top_k", C.c_int), ("expert_intermediate", C.c_int),
-                ("router", C.POINTER(C.c_void_p)), ("rope_mscale", C.c_float)]
+                ("router", C.POINTER(C.c_void_p)), ("rope_mscale", C.c_float), ("raw_topk", C.c_int)]
 
 
 class OracleModel:
@@ -92,6 +92,7 @@ class OracleModel:
         if m.num_experts:
             m.router = parr([f"layers.{l}.router" for l in range(L)])
         m.rope_mscale = float(cfg.get("rope_mscale", 1.0))
+        m.raw_topk = 0 if cfg.get("norm_topk", True) else 1
         self._m = m
         ps, tp = cfg["page_size"], cfg["total_pages"]
         shape = (tp, ps, cfg["kv_heads"], cfg["head_dim"])
@@ -373,5 +374,6 @@ def model_from_driver(drv, cfg: dict):
     ocfg["rope_mscale"] = float(ms[0]) if ms is not None else 1.0
     if cfg["arch"] == "qwen3_moe":
         ocfg.update(num_experts=cfg["num_experts"], top_k=cfg["top_k"],
-                    expert_intermediate=cfg["expert_intermediate"], intermediate=0)
+                    expert_intermediate=cfg["expert_intermediate"], intermediate=0,
+                    norm_topk="norm_topk = false" not in cfg.get("model_extra", ""))
     return OracleModel(ocfg, t), t

@@ -125,7 +125,7 @@ static void orc_moe_ffn(const OrcModel* m, int l, const uint16_t* xn, uint16_t* 
     float* wts = (float*)malloc((size_t)N * K * 4);
     uint16_t* yr = (uint16_t*)malloc((size_t)N * K * H * 2);
     orc_gemm_bf16(xn, m->router[l], NULL, lf, logits, NULL, N, E, H, 0, 0);
-    orc_topk_softmax(logits, idx, wts, N, E, K);
+    orc_topk_softmax_opt(logits, idx, wts, N, E, K, m->raw_topk ? 0 : 1);
     orc_router_gap_note(logits, N, E, K);
 #pragma omp parallel for schedule(dynamic)
     for (int r = 0; r < N * K; ++r) {

@@ -201,7 +201,7 @@ static void FN(attention)(const OrcModel* m, const REAL* q, const double* k_pool
 }
 
 /* x[t] += sum_k w_k * down_e(silu(gate_e xn) * up_e xn) over the token's top-k experts, weights
- * = softmax probabilities of the chosen experts divided by their sum; nothing rounded per route
+ * = softmax probabilities of the chosen experts divided by their sum (as they are under raw_topk); nothing rounded per route
  * (driver/portable/src/graph_common.cpp:237-345). */
 static void FN(moe_ffn)(const OrcModel* m, int l, const REAL* xn, REAL* x, int N) {
     const int H = m->hidden, E = m->num_experts, K = m->top_k, Ie = m->expert_intermediate;
@@ -264,7 +264,7 @@ static void FN(moe_ffn)(const OrcModel* m, int l, const REAL* xn, REAL* x, int N
                 act[i] = g / (1 + (REAL)exp((double)-g)) * gu[Ie + i];
             }
             FN(linear)(m, &wd, m->quant, act, y, 1, H, Ie, 0);
-            const REAL wk = wsel[k] / wsum;
+            const REAL wk = m->raw_topk ? wsel[k] : wsel[k] / wsum;
             for (int i = 0; i < H; ++i) x[(size_t)t * H + i] += wk * y[i];
         }
         free(gu); free(act); free(y);

@@ -32,6 +32,8 @@ typedef struct {
     int num_experts, top_k, expert_intermediate;
     const uint16_t* const* router; /* [L] bf16 [E, H] */
     float rope_mscale;             /* cos and sin are multiplied by it (YaRN's attention factor; 1 otherwise) */
+    int raw_topk;                  /* MoE: 1 = the chosen experts' probabilities are not divided by their sum
+                                      (norm_topk = false, driver/portable/src/graph_common.cpp:279-283) */
 } OrcModel;
 
 #endif

@@ -5,7 +5,9 @@
  * 19-86): softmax over the experts in fp32 (max, exp, sum, multiply by 1/Z), K passes of argmax
  * with exclusion where a strictly greater value wins (so the lowest index wins ties), weights
  * divided by their sum accumulated in selection order.  Same selection rule as the graph form
- * softmax -> top_k -> gather -> divide by the sum (driver/portable/src/graph_common.cpp:262-283).
+ * softmax -> top_k -> gather -> divide by the sum (driver/portable/src/graph_common.cpp:262-283),
+ * which divides only under norm_topk (:279-283): orc_topk_softmax_opt with renorm = 0 returns the
+ * chosen experts' softmax probabilities as they are.
  * The reference sums the exponentials in a strided tree; here the sum is sequential — results
  * agree to fp32 rounding.
  *
@@ -15,11 +17,17 @@
  * added onto the bf16 residual before that rounding.
  *
  * Pinned by tests/test_oracle_moe.py: against numpy float64 softmax + stable argsort on
- * separated logits, constructed ties, weights summing to one, and a float64 weighted sum.
+ * separated logits (with and without the division), constructed ties, weights summing to one,
+ * and a float64 weighted sum.
  */
 #include "oracle_api.h"
 
 void orc_topk_softmax(const uint16_t* logits, int32_t* topk_idx, float* topk_w, int N, int E, int K) {
+    orc_topk_softmax_opt(logits, topk_idx, topk_w, N, E, K, 1);
+}
+
+void orc_topk_softmax_opt(const uint16_t* logits, int32_t* topk_idx, float* topk_w, int N, int E, int K,
+                          int renorm) {
     for (int n = 0; n < N; ++n) {
         const uint16_t* row = logits + (size_t)n * E;
         float probs[512];
@@ -49,6 +57,7 @@ void orc_topk_softmax(const uint16_t* logits, int32_t* topk_idx, float* topk_w, 
             w_sum += best_v;
             probs[best_i] = -1.f;
         }
+        if (!renorm) continue;
         const float inv_w = 1.f / w_sum;
         for (int k = 0; k < K; ++k) topk_w[(size_t)n * K + k] *= inv_w;
     }

@@ -41,6 +41,8 @@ void orc_attn_rows_masked(const uint16_t* q, const uint16_t* k_pages, const uint
 void orc_brle_allow(const uint32_t* runs, size_t n_runs, int pos, int n_kv, int window,
                     uint8_t* out);
 void orc_topk_softmax(const uint16_t* logits, int32_t* topk_idx, float* topk_w, int N, int E, int K);
+void orc_topk_softmax_opt(const uint16_t* logits, int32_t* topk_idx, float* topk_w, int N, int E, int K,
+                          int renorm);
 void orc_moe_combine(const uint16_t* y_routes, const float* topk_w, uint16_t* out, int N, int K,
                      int H, int add);
 void orc_pcg32_sequence(uint64_t seed, uint64_t stream, uint32_t* out, int n);

@@ -217,12 +217,6 @@ static DriverConfig load_driver_config(const std::string& src) {
         finalize_config(c);
         if (c.runtime.snapshot_dir.empty()) c.runtime.snapshot_dir = c.model.checkpoint_dir;
     }
-    // The routing kernel always divides the top-k probabilities by their sum
-    // (driver/portable/src/graph_common.cpp:279-283 does so only under norm_topk): a model that
-    // asks for raw probabilities would get other expert weights without a word.
-    if (c.model.arch == "qwen3_moe" && !c.model.norm_topk)
-        throw std::runtime_error("config: norm_topk = false (norm_topk_prob) is not implemented: "
-                                 "router weights are always renormalised over the top-k experts");
     return c;
 }
 

@@ -488,8 +488,8 @@ void Executor::moe_block(const LayerWeights& w, int N, hipStream_t s) {
     const int sbf = w.wgu.scale_bf16 ? 1 : 0;
     PIE_KERNEL(pie_hip_rmsnorm(x_, w.ffn_norm, xn_, N, H, m.rms_eps, s));
     linear_fused(w.router, xn_, nullptr, m.rms_eps, moe_logits_, N, 0, 0, nullptr, gemm_ws_, gemm_ws_bytes_, s);
-    PIE_KERNEL(pie_hip_moe_route(moe_logits_, moe_idx_, moe_w_, moe_offsets_, moe_route_token_,
-                                 moe_route_pos_, N, E, K, s));
+    PIE_KERNEL(pie_hip_moe_route_opt(moe_logits_, moe_idx_, moe_w_, moe_offsets_, moe_route_token_,
+                                     moe_route_pos_, N, E, K, m.norm_topk ? 1 : 0, s));
     const int hint = std::max(1, std::min(N, 2 * ((N * K + E - 1) / E)));
     // experts stacked along the rows: the tile-major copy of the stack keeps expert e at the same
     // byte stride (every expert has a multiple of 16 rows)

@@ -50,10 +50,12 @@ __device__ __forceinline__ void wave_argmax(float& v, int& i) {
     argmax_pick(v, i, __uint_as_float(v32[0]), static_cast<int>(i32[0]), __uint_as_float(v32[1]), static_cast<int>(i32[1]));
 }
 
-// One wave per token: softmax over the experts, top-k with exclusion, renormalise.
+// One wave per token: softmax over the experts, top-k with exclusion, renormalise (`renorm`; without
+// it the chosen experts keep their softmax probabilities, driver/portable/src/graph_common.cpp:279-283).
 __global__ __launch_bounds__(256) void moe_topk_kernel(const uint16_t* __restrict__ logits,
                                                        int32_t* __restrict__ topk_idx,
-                                                       float* __restrict__ topk_w, int N, int E, int K) {
+                                                       float* __restrict__ topk_w, int N, int E, int K,
+                                                       int renorm) {
     const int lane = threadIdx.x & (kWave - 1);
     const int t = blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
     if (t >= N) return;
@@ -107,7 +109,7 @@ __global__ __launch_bounds__(256) void moe_topk_kernel(const uint16_t* __restric
     const float inv_w = 1.f / w_sum;
     if (lane < K) {
         topk_idx[static_cast<size_t>(t) * K + lane] = my_e;
-        topk_w[static_cast<size_t>(t) * K + lane] = my_w * inv_w;
+        topk_w[static_cast<size_t>(t) * K + lane] = renorm ? my_w * inv_w : my_w;
     }
 }
 
@@ -199,6 +201,14 @@ extern "C" int pie_hip_moe_route(const uint16_t* router_logits_bf16, int32_t* to
                                  float* topk_weight, int32_t* expert_offsets,
                                  int32_t* route_token, int32_t* route_pos, int num_tokens,
                                  int num_experts, int top_k, void* stream) {
+    return pie_hip_moe_route_opt(router_logits_bf16, topk_idx, topk_weight, expert_offsets, route_token,
+                                 route_pos, num_tokens, num_experts, top_k, 1, stream);
+}
+
+extern "C" int pie_hip_moe_route_opt(const uint16_t* router_logits_bf16, int32_t* topk_idx,
+                                     float* topk_weight, int32_t* expert_offsets,
+                                     int32_t* route_token, int32_t* route_pos, int num_tokens,
+                                     int num_experts, int top_k, int renormalize, void* stream) {
     using namespace pie_hip;
     if (!router_logits_bf16 || !topk_idx || !topk_weight || !expert_offsets || !route_token ||
         !route_pos || num_tokens <= 0)
@@ -208,7 +218,8 @@ extern "C" int pie_hip_moe_route(const uint16_t* router_logits_bf16, int32_t* to
         return PIE_HIP_ERR_UNSUPPORTED;
     hipStream_t st = static_cast<hipStream_t>(stream);
     hipLaunchKernelGGL(moe_topk_kernel, dim3((num_tokens + 3) / 4), dim3(256), 0, st,
-                       router_logits_bf16, topk_idx, topk_weight, num_tokens, num_experts, top_k);
+                       router_logits_bf16, topk_idx, topk_weight, num_tokens, num_experts, top_k,
+                       renormalize ? 1 : 0);
     hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(kRouteThreads), 0, st, topk_idx, expert_offsets,
                        route_token, route_pos, num_tokens, num_experts, top_k);
     return launch_status();

@@ -474,8 +474,9 @@ def moe_grouped_gemm(act: torch.Tensor, route_act_rows: Optional[torch.Tensor],
     return y
 
 
-def moe_route(router_logits: torch.Tensor, top_k: int):
-    """Softmax -> top-k -> renormalise per token, plus the expert-sorted route layout.
+def moe_route(router_logits: torch.Tensor, top_k: int, renormalize: bool = True):
+    """Softmax -> top-k -> renormalise per token (renormalize=False: the chosen experts keep their
+    softmax probabilities), plus the expert-sorted route layout.
     Returns (topk_idx [T,k] int32, topk_w [T,k] f32, expert_offsets [E+1] int32,
     route_token [T*k] int32, route_pos [T*k] int32)."""
     _dev(router_logits, torch.bfloat16, "router_logits")
@@ -486,8 +487,9 @@ def moe_route(router_logits: torch.Tensor, top_k: int):
     offs = torch.empty(E + 1, dtype=torch.int32, device=d)
     rtok = torch.empty(T * top_k, dtype=torch.int32, device=d)
     rpos = torch.empty(T * top_k, dtype=torch.int32, device=d)
-    _check(kernels().pie_hip_moe_route(_ptr(router_logits), _ptr(idx), _ptr(w), _ptr(offs), _ptr(rtok),
-                                       _ptr(rpos), T, E, top_k, _stream()), "pie_hip_moe_route")
+    _check(kernels().pie_hip_moe_route_opt(_ptr(router_logits), _ptr(idx), _ptr(w), _ptr(offs), _ptr(rtok),
+                                           _ptr(rpos), T, E, top_k, int(renormalize), _stream()),
+           "pie_hip_moe_route_opt")
     return idx, w, offs, rtok, rpos
 
 

@@ -622,15 +622,28 @@ def test_unknown_kv_cache_dtypes_are_refused(gpu):
             drvmod.Driver(toml_config(kv_cache_dtype=bad))
 
 
-def test_raw_router_probabilities_are_refused(gpu):
-    """norm_topk = false (config.json norm_topk_prob) asks for un-renormalised router weights,
-    which the routing kernel does not produce: start-up fails instead of computing other weights."""
+def test_raw_router_probabilities_match_oracle(gpu, oracle):
+    """norm_topk = false (config.json norm_topk_prob): the chosen experts keep their softmax
+    probabilities (driver/portable/src/graph_common.cpp:279-283 divides by their sum only under
+    norm_topk).  Teacher-forced steps against the oracle run the same way, and the setting
+    changes the logits."""
     from pie_amd import driver as drvmod
 
-    toml = toml_config(arch="qwen3_moe", quant="bf16", num_experts=4, top_k=2, expert_intermediate=64,
-                       intermediate=0).replace("top_k = 2", "top_k = 2\nnorm_topk = false")
-    with pytest.raises(Exception, match="norm_topk"):
-        drvmod.Driver(toml)
+    kw = dict(arch="qwen3_moe", quant="bf16", head_dim=64, q_heads=8, kv_heads=2, num_experts=6, top_k=3,
+              expert_intermediate=128, router_std=0.2, intermediate=0, model_extra="norm_topk = false\n")
+    cfg = full_cfg(**kw)
+    rng = np.random.default_rng(97)
+    prompts = ragged_prompts(rng, cfg["vocab"], 19, 2)
+    with drvmod.Driver(toml_config(**kw)) as d:
+        om, _ = oracle_model_from_driver(d, cfg)
+        _, _, checks = teacher_forced_compare(oracle, drvmod, d, om, cfg, prompts, 6)
+        assert checks == 12
+        d.generate(prompts[0], 1, replicate=1)
+        raw = oracle.bf16_to_f32(d.export_tensor("debug.logits", np.uint16)).astype(np.float64).ravel()
+    with drvmod.Driver(toml_config(**dict(kw, model_extra=""))) as d:
+        d.generate(prompts[0], 1, replicate=1)
+        normed = oracle.bf16_to_f32(d.export_tensor("debug.logits", np.uint16)).astype(np.float64).ravel()
+    assert raw.shape == normed.shape and not np.array_equal(raw, normed)
 
 
 @pytest.mark.parametrize("kw", [dict(quant="int4b8"), dict(arch="qwen3", quant="bf16", head_dim=128, q_heads=4,

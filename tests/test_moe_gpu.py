@@ -25,6 +25,10 @@ def test_route_matches_oracle_and_layout_is_a_counting_sort(gpu, oracle, T, E, K
     oidx, ow = oracle.topk_softmax(logits, K)
     assert np.array_equal(idx, oidx)           # integer outputs: bit-exact
     assert np.allclose(w, ow, rtol=2e-6, atol=1e-9)
+    # norm_topk = false: the same routes, the probabilities undivided
+    idx_r, w_r = (t.cpu().numpy() for t in ops.moe_route(dev(logits, gpu, torch.bfloat16), K, renormalize=False)[:2])
+    _, ow_r = oracle.topk_softmax(logits, K, renorm=False)
+    assert np.array_equal(idx_r, oidx) and np.allclose(w_r, ow_r, rtol=2e-6, atol=1e-9)
     # layout: offsets are the exclusive scan of the per-expert route counts
     counts = np.bincount(idx.reshape(-1), minlength=E)
     assert np.array_equal(offs, np.concatenate([[0], np.cumsum(counts)]))

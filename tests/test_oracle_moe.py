@@ -21,6 +21,13 @@ def test_topk_softmax_matches_float64_softmax_and_stable_argsort(oracle):
         ref_w /= ref_w.sum(axis=1, keepdims=True)
         assert np.allclose(w, ref_w, rtol=2e-6, atol=1e-9)
         assert np.allclose(w.sum(axis=1), 1.0, atol=1e-6)
+        # norm_topk = false (driver/portable/src/graph_common.cpp:279-283): the same experts, their
+        # softmax probabilities undivided
+        idx_raw, w_raw = oracle.topk_softmax(logits, K, renorm=False)
+        assert np.array_equal(idx_raw, ref_idx)
+        assert np.allclose(w_raw, np.take_along_axis(p, ref_idx, 1), rtol=2e-6, atol=1e-9)
+        if K < E:
+            assert np.all(w_raw.sum(axis=1) < 1.0)
 
 
 def test_topk_softmax_ties_go_to_the_lowest_index_and_closed_form(oracle):
