@@ -508,16 +508,22 @@ __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 && MT == 1 ? 4 : 2) void s
     // weight row j — carried in the ring slot of the block's first tile; a tile's step reads its
     // value across the wave.  (A load per tile and step made a third of the kernel's vector-memory
     // instructions, and those, not the bytes, are what a CU's address unit runs out of.)
-    static_assert(NG <= 4, "a wave's lanes hold the scales of NG tiles of 16 rows");
-    const uint16_t* gsp = st[0];
+    // (eight tiles: two such loads per block, with the slots of tiles 0 and 4)
+    constexpr int NGS = (NG + 3) / 4;
+    const uint16_t* gsp[NGS];
 #pragma unroll
-    for (int i = 1; i < NG; ++i) gsp = (lane >> 4) == i ? st[i] : gsp;
-    if ((lane >> 4) >= NG) gsp = st[NG - 1];
+    for (int h = 0; h < NGS; ++h) {
+        gsp[h] = st[min(4 * h, NG - 1)];
+#pragma unroll
+        for (int i = 1; i < 4; ++i)
+            if (4 * h + i < NG) gsp[h] = (lane >> 4) == i ? st[4 * h + i] : gsp[h];
+        if (4 * h + (lane >> 4) >= NG) gsp[h] = st[NG - 1];
+    }
     auto load_w = [&](int c, int lin) {
         const int b = min(b_lo + c * CB + lin / NG, b_last);
         WOne sl;
         sl.w = *reinterpret_cast<const u32x4_t*>(wt[lin % NG] + static_cast<size_t>(b) * 1024 + lane16);
-        sl.gs = F::kGroupScale && lin % NG == 0 ? (gsp + static_cast<size_t>(b >> blk_shift) * 16)[j] : uint16_t(0);
+        sl.gs = F::kGroupScale && lin % NG % 4 == 0 ? (gsp[lin % NG / 4] + static_cast<size_t>(b >> blk_shift) * 16)[j] : uint16_t(0);
         return sl;
     };
 
@@ -572,8 +578,8 @@ __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 && MT == 1 ? 4 : 2) void s
         f32x4_t sxb[MT];
         int gsb = 0;   // the current block's scales, tile i's in lanes 16 i .. 16 i + 15
         auto step = [&](const WOne& cur, int ng, int blk) {
+            if (ng % 4 == 0) gsb = cur.gs;
             if (ng == 0) {
-                gsb = cur.gs;
                 const int vbase = blk * (LK / 8) + q * S;
 #pragma unroll
                 for (int t = 0; t < MT; ++t)
@@ -611,7 +617,7 @@ __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 && MT == 1 ? 4 : 2) void s
             }
             if (F::kGroupScale) {
                 const float sc = bf16_bits_to_f32(static_cast<uint16_t>(
-                    ng == 0 && NG == 1 ? gsb : __builtin_amdgcn_ds_bpermute((ng * 16 + j) * 4, gsb)));
+                    ng == 0 && NG == 1 ? gsb : __builtin_amdgcn_ds_bpermute((ng % 4 * 16 + j) * 4, gsb)));
 #pragma unroll
                 for (int t = 0; t < MT; ++t)
 #pragma unroll
@@ -764,8 +770,13 @@ int launch_wave_mt(const SkinnyArgs& a, int problems, hipStream_t stream) {
     // a CU holds one block of eight waves (two with one tile per wave: fewer registers).  Take
     // the most tiles per wave whose K split still puts >= 1100 waves on the machine without
     // going past what is resident at once (a second round of blocks costs more than idle CUs).
+    // (eight tiles per wave — half the staged activation bytes per weight byte — for the 32-row
+    // passes, where the partial sums of a row tile still fit the wave's LDS region: gate|up of an 8B
+    // model at 64 rows 34.3 -> 30.4 us.  With 16-row passes the kernel needs more registers than a
+    // wave has and starts its loads 6 us late: 16.4 -> 22.6 us at 16 rows)
+    constexpr bool kEight = MT == 2 && 8 * 4 * kWave + (F::kBias != 0.f && !F::kGroupScale ? 4 * kWave : 0) <= SwGeom<MT>::region * 4;
     int ng = 1, kp_shift = 0;
-    for (int cand = 4; cand >= 1; cand >>= 1) {
+    for (int cand = kEight ? 8 : 4; cand >= 1; cand >>= 1) {
         const long groups = (tiles + cand - 1) / cand * mult;
         const long cap = 256L * (cand == 1 && MT == 1 ? 16 : 8);
         int sh = 0;
@@ -778,7 +789,10 @@ int launch_wave_mt(const SkinnyArgs& a, int problems, hipStream_t stream) {
     }
     if (force_ng) ng = force_ng;
     if (force_kp >= 0) kp_shift = force_kp;
+    if constexpr (kEight)
+        if (ng == 8) return launch_wave_cfg<F, 8, MT>(a, problems, kp_shift, stream);
     switch (ng) {
+        case 8:
         case 4: return launch_wave_cfg<F, 4, MT>(a, problems, kp_shift, stream);
         case 2: return launch_wave_cfg<F, 2, MT>(a, problems, kp_shift, stream);
         default: return launch_wave_cfg<F, 1, MT>(a, problems, kp_shift, stream);
