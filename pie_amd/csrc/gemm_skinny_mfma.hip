@@ -419,18 +419,22 @@ struct WOne {
 // MT row tiles of 16 per pass: a decoded weight fragment then feeds MT MFMAs, so a batch of 17
 // to 64 rows decodes the weights half as often.  The staged chunk shrinks by MT (the region and
 // the staging registers keep their size), so MT = 2 is the limit for int4 (one 128-k block).
-template <int MT>
+// Eight tiles per wave take the 128-k chunk with 16-row passes too: half the staging registers
+// pay for the second four accumulators and weight pointers.
+template <int MT, int NG>
 struct SwGeom {
-    static constexpr int chunk = kSwChunk / MT;         // k-values per staged chunk
+    static constexpr int chunk = kSwChunk / (MT == 1 && NG == 8 ? 2 : MT);   // k-values per staged chunk
     static constexpr int stride = chunk / 8 + 1;        // 16-byte vectors per staged row (padded)
-    static constexpr int region = 16 * MT * stride;     // vectors per wave region
+    static constexpr int staged = 16 * MT * stride;     // vectors of a staged chunk
+    static constexpr int meet = (NG + 1) * kWave;       // vectors of a row tile's partial sums (+ the row-bias sums)
+    static constexpr int region = staged > meet ? staged : meet;   // vectors per wave region
 };
 
 template <class F, int NG, int MT>
 __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 && MT == 1 ? 4 : 2) void skinny_wave_kernel(const SkinnyArgs a, const int kp_shift) {
     constexpr int KPL = F::kPerLane, S = F::kSteps;
     constexpr int LK = 4 * KPL;                     // k covered by one wave-wide 16-byte load (a block)
-    constexpr int CHUNK = SwGeom<MT>::chunk, STRIDE = SwGeom<MT>::stride, REGION = SwGeom<MT>::region;
+    constexpr int CHUNK = SwGeom<MT, NG>::chunk, STRIDE = SwGeom<MT, NG>::stride, REGION = SwGeom<MT, NG>::region;
     constexpr int CB = CHUNK / LK;                  // blocks per chunk
     constexpr int NS = NG * CB;                     // steps per chunk, tile-major order
     constexpr int PF = NS < 8 ? NS : 8;             // weight loads in flight per lane (deeper rings cost the occupancy that pays more)
@@ -441,7 +445,7 @@ __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 && MT == 1 ? 4 : 2) void s
     constexpr int ROWS = 16 * MT;                   // rows per pass
     constexpr bool kBiased = F::kBias != 0.f;
     constexpr bool kRowBias = kBiased && !F::kGroupScale;
-    static_assert(CB >= 1 && (NS % PF == 0 || PF % NS == 0) && SV == 8, "ring and staging shapes");
+    static_assert(CB >= 1 && (NS % PF == 0 || PF % NS == 0) && (SV == 8 || SV == 4), "ring and staging shapes");
     extern __shared__ __align__(16) unsigned char smem[];
     const int tid = threadIdx.x, lane = tid & (kWave - 1);
     const int wv = __builtin_amdgcn_readfirstlane(tid / kWave);
@@ -744,7 +748,7 @@ __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 && MT == 1 ? 4 : 2) void s
 
 template <class F, int NG, int MT>
 int launch_wave_cfg(const SkinnyArgs& a, int problems, int kp_shift, hipStream_t stream) {
-    constexpr size_t smem = static_cast<size_t>(kSwWaves) * SwGeom<MT>::region * 16;
+    constexpr size_t smem = static_cast<size_t>(kSwWaves) * SwGeom<MT, NG>::region * 16;
     static const hipError_t attr = hipFuncSetAttribute(
         reinterpret_cast<const void*>(&skinny_wave_kernel<F, NG, MT>),
         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
@@ -761,8 +765,7 @@ int launch_wave_cfg(const SkinnyArgs& a, int problems, int kp_shift, hipStream_t
 // waves per CU.
 template <class F, int MT>
 int launch_wave_mt(const SkinnyArgs& a, int problems, hipStream_t stream) {
-    constexpr int LK = 4 * F::kPerLane, CB = SwGeom<MT>::chunk / LK;
-    const int nch_all = (a.K / LK + CB - 1) / CB;
+    constexpr int LK = 4 * F::kPerLane;
     const long mult = a.m_split ? (a.M + 16 * MT - 1) / (16 * MT) : problems;
     const long tiles = (a.N + 15) / 16;
     static const int force_ng = [] { const char* e = getenv("PIE_SKINNY_NG"); return e ? atoi(e) : 0; }();
@@ -770,17 +773,23 @@ int launch_wave_mt(const SkinnyArgs& a, int problems, hipStream_t stream) {
     // a CU holds one block of eight waves (two with one tile per wave: fewer registers).  Take
     // the most tiles per wave whose K split still puts >= 1100 waves on the machine without
     // going past what is resident at once (a second round of blocks costs more than idle CUs).
-    // (eight tiles per wave — half the staged activation bytes per weight byte — for the 32-row
-    // passes, where the partial sums of a row tile still fit the wave's LDS region: gate|up of an 8B
-    // model at 64 rows 34.3 -> 30.4 us.  With 16-row passes the kernel needs more registers than a
-    // wave has and starts its loads 6 us late: 16.4 -> 22.6 us at 16 rows)
-    constexpr bool kEight = MT == 2 && 8 * 4 * kWave + (F::kBias != 0.f && !F::kGroupScale ? 4 * kWave : 0) <= SwGeom<MT>::region * 4;
+    // (eight tiles per wave — half the staged activation bytes per weight byte — for group-scaled
+    // int4: gate|up of an 8B model at 64 rows 34.3 -> 30.4 us.  With 16-row passes over 256-k chunks
+    // the kernel needed more registers than a wave has and started its loads 6 us late: there it
+    // takes 128-k chunks)
+    constexpr bool kEight = F::kGroupScale;
     int ng = 1, kp_shift = 0;
     for (int cand = kEight ? 8 : 4; cand >= 1; cand >>= 1) {
+        const int cb = (cand == 8 ? SwGeom<MT, 8>::chunk : SwGeom<MT, 4>::chunk) / LK;
+        const int nch_all = (a.K / LK + cb - 1) / cb;
         const long groups = (tiles + cand - 1) / cand * mult;
         const long cap = 256L * (cand == 1 && MT == 1 ? 16 : 8);
         int sh = 0;
         while (sh < 3 && (groups << (sh + 1)) <= cap && (2 << sh) <= nch_all) ++sh;
+        // (eight tiles only where four waves or fewer share a tile group: over an eighth of K the
+        // loop is too short for its prologue and the eight-wave meeting — gate|up at 16 rows 16.4 us
+        // with four tiles, 17.9 with eight; at 32 rows, two passes side by side, 25.0 against 20.4)
+        if (cand == 8 && sh > 2) continue;
         if ((groups << sh) >= 1100 || cand == 1) {
             ng = cand;
             kp_shift = sh;
@@ -806,7 +815,7 @@ int launch_wave(const SkinnyArgs& a, int problems, hipStream_t stream) {
     // row decode step 4.63 / 4.88 -> 4.26 / 4.61 ms; at 17..32 rows the shorter chunks cost
     // more than the second pass saves, 3.40 -> 3.47 ms)
     const bool two = force_mt ? force_mt == 2 : (!a.offsets && a.M > 32);
-    if (two && a.K % SwGeom<2>::chunk == 0) return launch_wave_mt<F, 2>(a, problems, stream);
+    if (two && a.K % SwGeom<2, 4>::chunk == 0) return launch_wave_mt<F, 2>(a, problems, stream);
     return launch_wave_mt<F, 1>(a, problems, stream);
 }
 

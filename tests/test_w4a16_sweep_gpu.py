@@ -39,9 +39,23 @@ def _kernels(ops, M):
     return k
 
 
+# The fused gate|up projection of the 8B model, the widest matrix a decode batch multiplies: its
+# tile count is what sends 17-32 and 33-64 rows to the eight-tiles-per-wave instantiations.
+GATE_UP = [(28672, 4096, 16), (28672, 4096, 32), (28672, 4096, 64)]   # (N, K, M)
+
+
 @pytest.mark.parametrize("M", [8, 32, 128, 2048])
 @pytest.mark.parametrize("N,K", SHAPES)
 def test_sweep_shapes_match_oracle_on_sampled_columns(gpu, oracle, N, K, M):
+    _sampled_columns(gpu, oracle, N, K, M)
+
+
+@pytest.mark.parametrize("N,K,M", GATE_UP)
+def test_gate_up_shape_matches_oracle_on_sampled_columns(gpu, oracle, N, K, M):
+    _sampled_columns(gpu, oracle, N, K, M)
+
+
+def _sampled_columns(gpu, oracle, N, K, M):
     import torch
     from pie_amd import ops
 
@@ -87,6 +101,15 @@ def test_sweep_shapes_one_hot_rows_are_exact_everywhere(gpu, oracle, N, K, M):
     """Row m of the activations is the unit vector e_k(m): y[m, n] must be bf16(q[n, k] * s[n, k/G])
     for every one of the N columns — tile indexing, operand layouts, bias removal and the K split
     of every instantiation, over the whole output."""
+    _one_hot_rows(gpu, oracle, N, K, M)
+
+
+@pytest.mark.parametrize("N,K,M", GATE_UP)
+def test_gate_up_shape_one_hot_rows_are_exact_everywhere(gpu, oracle, N, K, M):
+    _one_hot_rows(gpu, oracle, N, K, M)
+
+
+def _one_hot_rows(gpu, oracle, N, K, M):
     import torch
     from pie_amd import ops
 
