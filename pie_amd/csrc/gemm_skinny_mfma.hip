@@ -230,22 +230,31 @@ __global__ __launch_bounds__(KP* kWave) void skinny_kernel(const SkinnyArgs a) {
     const int sm = tid / TPR, sv = tid % TPR;
 
     for (int mt0 = r0; mt0 < r1; mt0 += 16) {
-        // rows past the problem repeat its last row and are never stored
+        // rows past the problem repeat its last row and are never stored.  A pass of at most four
+        // (eight) rows stages four (eight): the other rows of the MFMA operand read those again,
+        // their accumulator rows are never stored, and the staging traffic — every tile group
+        // fetches the activations again, for an expert with a handful of routes they are as many
+        // bytes as a block's weights — falls to a quarter (half).
+        const int rmask = r1 - mt0 <= 4 ? 3 : r1 - mt0 <= 8 ? 7 : 15;
+        const int jr = j & rmask;
+        const bool stager = sm <= rmask;
         const int srow = min(mt0 + sm, r1 - 1);
         const uint16_t* arow = a.act + static_cast<size_t>(a.act_rows ? a.act_rows[srow] : srow) * K;
         u32x4_t stg[SV];
         auto stage_load = [&](int c) {
             const int cc = min(c, nchunks - 1);
             const int nvec = min(CK, K - cc * CK) / 8;
+            if (stager) {
 #pragma unroll
-            for (int u = 0; u < SV; ++u)
-                stg[u] = *reinterpret_cast<const u32x4_t*>(arow + cc * CK + min(u * TPR + sv, nvec - 1) * 8);
+                for (int u = 0; u < SV; ++u)
+                    stg[u] = *reinterpret_cast<const u32x4_t*>(arow + cc * CK + min(u * TPR + sv, nvec - 1) * 8);
+            }
         };
         auto stage_store = [&](int c) {
             const int nvec = min(CK, K - min(c, nchunks - 1) * CK) / 8;
 #pragma unroll
             for (int u = 0; u < SV; ++u)
-                if (u * TPR + sv < nvec) lds_a[sm * STRIDE + u * TPR + sv] = TILED ? stg[u] : F::order(stg[u]);   // (tile-major int4 codes sit in k order)
+                if (stager && u * TPR + sv < nvec) lds_a[sm * STRIDE + u * TPR + sv] = TILED ? stg[u] : F::order(stg[u]);   // (tile-major int4 codes sit in k order)
         };
 
         constexpr int NSX = F::kGroupScale ? GC * WL : 1;
@@ -273,7 +282,7 @@ __global__ __launch_bounds__(KP* kWave) void skinny_kernel(const SkinnyArgs a) {
                 const int sxi = F::kGroupScale ? g * WL + h : 0;
                 bf16x8_t ax[S];
 #pragma unroll
-                for (int s = 0; s < S; ++s) ax[s] = __builtin_bit_cast(bf16x8_t, lds_a[j * STRIDE + vbase + s]);
+                for (int s = 0; s < S; ++s) ax[s] = __builtin_bit_cast(bf16x8_t, lds_a[jr * STRIDE + vbase + s]);
                 f32x4_t part = zero4;
 #pragma unroll
                 for (int s = 0; s < S; ++s) {
