@@ -92,14 +92,14 @@ GemmPath pick_gemm(const Linear& w, int M, size_t ws_bytes) {
 // in K shares.  Two to four rows: the GEMV pays its dot products once per row, the skinny GEMM over
 // the tile-major copy does not but needs the norm as its own launch (~4.8 us).  Costs fitted to
 // the 8B shapes decide (decode steps of 2 / 3 / 4 rows over 512-token contexts: 1.91 / 2.46 /
-// 2.79 ms with the GEMV everywhere, 2.11 / 2.19 / 2.26 ms with the skinny GEMM everywhere);
+// 2.79 ms with the GEMV everywhere, 2.01 / 2.08 / 2.14 ms with the skinny GEMM everywhere);
 // without a tile-major copy the GEMV keeps all four.
 int model_route(const Linear& w, int M, bool has_norm, size_t ws_bytes) {
     if (M <= 4) {
         if (M < 2 || !w.data_tiled) return 0;
         const double bytes = static_cast<double>(w.data_bytes());
-        const double t_gemv = 3.4 + bytes / 5.5e6 * (1.0 + 0.5 * (M - 1));
-        const double t_skinny = 4.4 + bytes / 3.9e6 + (has_norm ? 4.8 : 0.0);
+        const double t_gemv = 3.4 + bytes / 5.5e6 * (M == 2 ? 1.35 : 1.0 + 0.5 * (M - 1));   // (a second row costs the GEMV less than the third and fourth)
+        const double t_skinny = 4.4 + bytes / 4.2e6 + (has_norm ? 4.8 : 0.0);
         if (t_gemv <= t_skinny) return 0;
     }
     const GemmPath p = pick_gemm(w, M, ws_bytes);

@@ -547,8 +547,9 @@ __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 && MT == 1 ? 4 : 2) void s
         // a pass of at most eight rows stages eight: the activations are re-read by every tile
         // group, so their traffic matters as much as the weights'.  Accumulator rows 8..15 then
         // repeat rows 0..7 and are never stored.
-        const bool r8 = MT == 1 && r1 - mt0 <= 8;
-        const int jr = r8 ? (j & 7) : j;
+        // (four rows for passes of at most four: a decode batch of three or four requests)
+        const int rstage = MT == 1 ? (r1 - mt0 <= 4 ? 4 : r1 - mt0 <= 8 ? 8 : 16) : 16 * MT;
+        const int jr = MT == 1 ? (j & (rstage - 1)) : j;
         int arow[SV];   // rows past the problem repeat its last row and are never stored
 #pragma unroll
         for (int u = 0; u < SV; ++u) {
@@ -559,13 +560,13 @@ __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 && MT == 1 ? 4 : 2) void s
             const int k0 = min((b_lo + min(c, max(nch - 1, 0)) * CB) * LK + svec * 8, K - 8);   // (past the slice: its last chunk again)
 #pragma unroll
             for (int u = 0; u < SV; ++u)
-                if (u < SV / 2 || !r8)
+                if (RPL * u < rstage)
                     stg[u] = *reinterpret_cast<const u32x4_t*>(a.act + static_cast<size_t>(arow[u]) * K + k0);
         };
         auto stage_store = [&]() {
 #pragma unroll
             for (int u = 0; u < SV; ++u)
-                if (u < SV / 2 || !r8) lds_a[(srow + RPL * u) * STRIDE + svec] = stg[u];
+                if (RPL * u < rstage) lds_a[(srow + RPL * u) * STRIDE + svec] = stg[u];
         };
 
         f32x4_t acc[MT][NG], sxt[MT];
