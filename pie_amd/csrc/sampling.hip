@@ -21,10 +21,19 @@
 //   at a time in double and compares the float-rounded value, so a draw within float rounding of
 //   a boundary may land on the neighbouring token.
 //
+//   With at most sixteen slots over a wide vocabulary the row-wide passes (maximum, exponentials
+//   and their sum, normalisation and candidate statistics, the candidates' compaction) run first
+//   over up to 32 blocks per slot, four short launches; the one block per slot then starts from
+//   their results.  Partial results are combined in part order, so a call's output does not
+//   depend on how the blocks were scheduled.
+//
 //   The descending order comes from a block-wide LSD radix sort (8-bit digits, 4 passes over
 //   the non-negative float bit patterns): each wave owns a contiguous segment, ranks its 64
 //   keys per step by matching digits across the wave (8 ballots), and scatters stably, so
 //   equal keys keep ascending ids.
+#include <algorithm>
+#include <cstdlib>
+
 #include "common.hip.h"
 
 namespace pie_hip {
@@ -55,6 +64,7 @@ struct SampleArgs {
     uint32_t* id_a;
     uint32_t* id_b;
     int V;
+    int parts;                  // > 0: the front-end kernels below have run with this many parts per slot
 };
 
 // Candidate thresholds t_j = p_max * 2^(-3j), j = 1..kLevels: how many entries, and how much
@@ -258,9 +268,12 @@ __device__ void sort_desc(uint32_t* key_a, uint32_t* key_b, uint32_t* id_a, uint
 //   kExceedScaled: thr * float(total) < float(s_i), total = s_{limit-1}   (categorical draw)
 // `limit` when there is none.  Block-uniform result.
 enum { kReach = 0, kExceed = 1, kExceedScaled = 2 };
+// (from_lo, from_hi, from_base): a sub-range already known to hold the answer and the sum of
+// everything before it — the walk then starts there instead of at the whole range (kExceed only).
 template <int MODE>
 __device__ int find_first(const uint32_t* __restrict__ pbits, int limit, float thr, BlockShared& sh,
-                          int lane, int wv, double* total_out) {
+                          int lane, int wv, double* total_out, int from_lo = -1, int from_hi = 0,
+                          double from_base = 0.0) {
     // Narrow the range 16-fold per level: every wave sums one sub-range (coalesced, batched
     // loads), the first sub-range whose end satisfies the rule holds the answer; the last
     // <= 64 entries are scanned by lane.  Sums are double; only the compared value is rounded.
@@ -268,6 +281,12 @@ __device__ int find_first(const uint32_t* __restrict__ pbits, int limit, float t
     double base = 0.0;
     float x = thr;
     bool top = true;
+    if (from_lo >= 0) {
+        lo = from_lo;
+        hi = from_hi;
+        base = from_base;
+        top = false;
+    }
     while (top || hi - lo > kWave) {
         const int span = hi - lo;
         const int sub = ((span + kSampWaves * kWave - 1) / (kSampWaves * kWave)) * kWave;
@@ -496,6 +515,375 @@ __device__ float log_sum_exp(const float* row, int V, float mx, BlockShared& sh,
     return mx + static_cast<float>(log(fmax(1e-30, sum)));
 }
 
+// What the draw can touch is a head of the descending order: the first top_k entries, the
+// prefix reaching top_p, the entries above the min-p threshold, or (nothing restricting)
+// the prefix whose mass exceeds u * total.  Any set {p >= t} containing that head gives
+// the same result as the whole vocabulary, so only such a set is compacted and sorted;
+// t is the first of the levels p_max * 2^(-3j) that covers the need (exact for min-p).
+struct DrawNeed {
+    int need_count;
+    float need_mass;
+    uint32_t floor_bits;   // nonzero: the exact lower bound of the kept entries (min-p)
+    bool keep_all, wants_k, wants_p;
+    float thr_p;
+};
+__device__ __forceinline__ DrawNeed draw_need(const SampleArgs& a, int s, int kind, const SoftmaxStats& st, float u) {
+    DrawNeed d;
+    d.wants_k = kind == PIE_HIP_SAMPLER_TOP_K || kind == PIE_HIP_SAMPLER_TOP_K_TOP_P;
+    d.wants_p = kind == PIE_HIP_SAMPLER_TOP_P || kind == PIE_HIP_SAMPLER_TOP_K_TOP_P;
+    const uint32_t top_k = a.top_k[s];
+    d.thr_p = fminf(fmaxf(a.top_p[s], 0.0f), 1.0f);
+    const float thr_m = a.min_p[s] * __uint_as_float(st.max_bits);
+    d.need_count = 0;
+    d.need_mass = 0.f;
+    d.floor_bits = 0u;
+    d.keep_all = false;
+    if (d.wants_k && top_k != 0u) d.need_count = static_cast<int>(min(top_k, static_cast<uint32_t>(st.n_pos)));
+    else if (d.wants_p && d.thr_p < 1.0f) d.need_mass = d.thr_p;
+    else if (kind == PIE_HIP_SAMPLER_MIN_P && thr_m > 0.0f && thr_m <= __uint_as_float(st.max_bits))
+        d.floor_bits = __float_as_uint(thr_m);
+    else {
+        d.keep_all = true;
+        d.need_mass = u * static_cast<float>(st.total);
+    }
+    return d;
+}
+// the first level whose candidates cover the need; 1 (every positive entry) when none does
+__device__ __forceinline__ uint32_t level_floor(const DrawNeed& d, uint32_t top_bits, const uint32_t* cc, const float* cm) {
+    if (d.floor_bits) return d.floor_bits;
+    for (int j = 0; j < kLevels; ++j) {
+        const bool enough = d.need_count > 0 ? cc[j] >= static_cast<uint32_t>(d.need_count)
+                                             : cm[j] >= d.need_mass + 1e-4f;
+        if (enough && top_bits > (j + 1) * kLevelStep) return top_bits - (j + 1) * kLevelStep;
+    }
+    return 1u;
+}
+__device__ __forceinline__ bool sorts_candidates(int kind) {
+    return kind == PIE_HIP_SAMPLER_TOP_K || kind == PIE_HIP_SAMPLER_TOP_P || kind == PIE_HIP_SAMPLER_MIN_P ||
+           kind == PIE_HIP_SAMPLER_TOP_K_TOP_P;
+}
+
+// ---- front end over many blocks ----------------------------------------------------------------
+// One block per slot walks a 128 k row four times from a single CU (80-145 us).  With few slots the
+// row-wide passes — maximum, exponentials and their sum, normalisation with the candidate
+// statistics — are cut into `parts` contiguous segments, one block each, in three launches; the
+// per-part results are combined in part order (a fixed order: the same inputs give the same bits
+// every time), and sample_kernel starts from the normalised probabilities — for the kinds that
+// sort a candidate set, from the candidates too: each part compacts its own, in index order, to the
+// head of its segment of (key_b, id_b).  A slot's part records sit at the head of its id_a region,
+// which nothing else uses before sample_kernel has read them.
+constexpr int kFrontBlock = 256;
+constexpr int kFrontWaves = kFrontBlock / kWave;
+constexpr int kFrontLoads = 8;
+constexpr int kMaxParts = 32;
+struct FrontPart {
+    float mx;
+    int amax;
+    int n_pos;
+    uint32_t max_bits;
+    double sum;       // of the part's exponentials
+    double ps;        // of its normalised probabilities
+    uint32_t lc[kLevels];
+    float lm[kLevels];
+    int cnt;          // candidates this part put at the head of its segment of (key_b, id_b); -1: none made
+    uint32_t t_bits;  // the threshold they were taken at
+    uint32_t pad[2];
+};
+static_assert(sizeof(FrontPart) == 112, "part record layout");
+
+__device__ __forceinline__ FrontPart* front_parts(const SampleArgs& a, int s) {
+    return reinterpret_cast<FrontPart*>(a.id_a + static_cast<size_t>(s) * a.V);
+}
+__device__ __forceinline__ void front_segment(int V, int parts, int part, int& lo, int& hi) {
+    const int seg = ((V + parts - 1) / parts + kFrontBlock - 1) / kFrontBlock * kFrontBlock;
+    lo = min(V, part * seg);
+    hi = min(V, lo + seg);
+}
+// (max, first index) over all parts of a slot, as block_argmax orders them
+__device__ __forceinline__ void front_max(const FrontPart* fp, int parts, float& mx, int& amax) {
+    mx = fp[0].mx;
+    amax = fp[0].amax;
+    for (int b = 1; b < parts; ++b) {
+        const float ov = fp[b].mx;
+        const int oi = fp[b].amax;
+        if (ov > mx || (ov == mx && oi < amax)) {
+            mx = ov;
+            amax = oi;
+        }
+    }
+}
+
+__global__ __launch_bounds__(kFrontBlock) void sample_front_max_kernel(SampleArgs a) {
+    __shared__ float s_v[kFrontWaves];
+    __shared__ int s_i[kFrontWaves];
+    const int part = blockIdx.x, s = blockIdx.y, tid = threadIdx.x, lane = tid & (kWave - 1), wv = tid / kWave;
+    const float* row = a.logits + static_cast<size_t>(s) * a.V;
+    int lo, hi;
+    front_segment(a.V, a.parts, part, lo, hi);
+    float bv = -INFINITY;
+    int bi = 0x7FFFFFFF;
+    for (int v0 = lo + tid; v0 < hi; v0 += kFrontBlock * kFrontLoads) {
+        float x[kFrontLoads];
+#pragma unroll
+        for (int j = 0; j < kFrontLoads; ++j) {
+            const int v = v0 + j * kFrontBlock;
+            x[j] = v < hi ? row[v] : -INFINITY;
+        }
+#pragma unroll
+        for (int j = 0; j < kFrontLoads; ++j) {
+            const int v = v0 + j * kFrontBlock;
+            if (v < hi && (x[j] > bv || (bi == 0x7FFFFFFF && x[j] == bv))) {
+                bv = x[j];
+                bi = v;
+            }
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(bv, off, kWave);
+        const int oi = __shfl_xor(bi, off, kWave);
+        if (ov > bv || (ov == bv && oi < bi)) {
+            bv = ov;
+            bi = oi;
+        }
+    }
+    if (lane == 0) {
+        s_v[wv] = bv;
+        s_i[wv] = bi;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        for (int w = 1; w < kFrontWaves; ++w)
+            if (s_v[w] > bv || (s_v[w] == bv && s_i[w] < bi)) {
+                bv = s_v[w];
+                bi = s_i[w];
+            }
+        FrontPart* fp = front_parts(a, s) + part;
+        fp->mx = bv;
+        fp->amax = bi;
+    }
+}
+
+__device__ __forceinline__ double front_block_sum_f64(double v, double* sh, int lane, int wv) {
+    v = wave_sum_f64(v);
+    if (lane == 0) sh[wv] = v;
+    __syncthreads();
+    double t = 0.0;
+#pragma unroll
+    for (int w = 0; w < kFrontWaves; ++w) t += sh[w];
+    __syncthreads();
+    return t;
+}
+
+// e = expf((x - max) / T) into key_a, the part's sum of e in double
+__global__ __launch_bounds__(kFrontBlock) void sample_front_exp_kernel(SampleArgs a) {
+    __shared__ double s_d[kFrontWaves];
+    const int part = blockIdx.x, s = blockIdx.y, tid = threadIdx.x, lane = tid & (kWave - 1), wv = tid / kWave;
+    const float* row = a.logits + static_cast<size_t>(s) * a.V;
+    uint32_t* out = a.key_a + static_cast<size_t>(s) * a.V;
+    FrontPart* fp = front_parts(a, s);
+    float mx;
+    int amax;
+    front_max(fp, a.parts, mx, amax);
+    const float inv_t = 1.0f / fmaxf(a.temperature[s], 1e-5f);
+    int lo, hi;
+    front_segment(a.V, a.parts, part, lo, hi);
+    double acc = 0.0;
+    for (int v0 = lo + tid; v0 < hi; v0 += kFrontBlock * kFrontLoads) {
+        float x[kFrontLoads];
+#pragma unroll
+        for (int j = 0; j < kFrontLoads; ++j) {
+            const int v = v0 + j * kFrontBlock;
+            x[j] = v < hi ? row[v] : 0.f;
+        }
+#pragma unroll
+        for (int j = 0; j < kFrontLoads; ++j) {
+            const int v = v0 + j * kFrontBlock;
+            if (v < hi) {
+                const float e = expf((x[j] - mx) * inv_t);
+                out[v] = __float_as_uint(e);
+                acc += static_cast<double>(e);
+            }
+        }
+    }
+    const double sum = front_block_sum_f64(acc, s_d, lane, wv);
+    if (tid == 0) fp[part].sum = sum;
+}
+
+// p = e / sum in place, and the part's share of softmax_to_bits' statistics
+__global__ __launch_bounds__(kFrontBlock) void sample_front_norm_kernel(SampleArgs a) {
+    __shared__ double s_d[kFrontWaves];
+    __shared__ uint32_t s_u[kFrontWaves][2 + kLevels];
+    __shared__ float s_f[kFrontWaves][kLevels];
+    const int part = blockIdx.x, s = blockIdx.y, tid = threadIdx.x, lane = tid & (kWave - 1), wv = tid / kWave;
+    uint32_t* out = a.key_a + static_cast<size_t>(s) * a.V;
+    FrontPart* fp = front_parts(a, s);
+    double sum = 0.0;
+    for (int b = 0; b < a.parts; ++b) sum += fp[b].sum;
+    const float inv_sum = static_cast<float>(1.0 / fmax(1e-30, sum));
+    const uint32_t top_bits = __float_as_uint(inv_sum);   // p_max = expf(0) * inv_sum
+    int lo, hi;
+    front_segment(a.V, a.parts, part, lo, hi);
+    int pos = 0;
+    double ps = 0.0;
+    uint32_t mb = 0u;
+    uint32_t lc[kLevels];
+    float lm[kLevels];
+#pragma unroll
+    for (int j = 0; j < kLevels; ++j) {
+        lc[j] = 0u;
+        lm[j] = 0.f;
+    }
+    for (int v0 = lo + tid; v0 < hi; v0 += kFrontBlock * kFrontLoads) {
+        uint32_t eb[kFrontLoads];
+#pragma unroll
+        for (int j = 0; j < kFrontLoads; ++j) {
+            const int v = v0 + j * kFrontBlock;
+            eb[j] = v < hi ? out[v] : 0u;
+        }
+#pragma unroll
+        for (int j = 0; j < kFrontLoads; ++j) {
+            const int v = v0 + j * kFrontBlock;
+            if (v >= hi) continue;
+            const float p = __uint_as_float(eb[j]) * inv_sum;
+            const uint32_t bits = __float_as_uint(p);
+            out[v] = bits;
+            if (p > 0.0f) {
+                ++pos;
+                ps += static_cast<double>(p);
+                mb = max(mb, bits);
+#pragma unroll
+                for (int l = 0; l < kLevels; ++l) {
+                    const bool in = bits + (l + 1) * kLevelStep >= top_bits;
+                    lc[l] += in;
+                    lm[l] += in ? p : 0.f;
+                }
+            }
+        }
+    }
+    const double ps_all = front_block_sum_f64(ps, s_d, lane, wv);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        pos += __shfl_xor(pos, off, kWave);
+        mb = max(mb, static_cast<uint32_t>(__shfl_xor(mb, off, kWave)));
+#pragma unroll
+        for (int l = 0; l < kLevels; ++l) {
+            lc[l] += __shfl_xor(lc[l], off, kWave);
+            lm[l] += __shfl_xor(lm[l], off, kWave);
+        }
+    }
+    if (lane == 0) {
+        s_u[wv][0] = static_cast<uint32_t>(pos);
+        s_u[wv][1] = mb;
+#pragma unroll
+        for (int l = 0; l < kLevels; ++l) {
+            s_u[wv][2 + l] = lc[l];
+            s_f[wv][l] = lm[l];
+        }
+    }
+    __syncthreads();
+    if (tid == 0) {
+        FrontPart& o = fp[part];
+        int n = 0;
+        uint32_t m = 0u;
+        for (int w = 0; w < kFrontWaves; ++w) {
+            n += static_cast<int>(s_u[w][0]);
+            m = max(m, s_u[w][1]);
+        }
+        o.n_pos = n;
+        o.max_bits = m;
+        o.ps = ps_all;
+        o.cnt = -1;
+        for (int l = 0; l < kLevels; ++l) {
+            uint32_t c = 0u;
+            float f = 0.f;
+            for (int w = 0; w < kFrontWaves; ++w) {
+                c += s_u[w][2 + l];
+                f += s_f[w][l];
+            }
+            o.lc[l] = c;
+            o.lm[l] = f;
+        }
+    }
+}
+
+// The part's entries with p >= t, in index order, to (key_b, id_b)[lo ..): t is the level every
+// block of the slot derives from the combined statistics, exactly as sample_kernel would.
+__global__ __launch_bounds__(kFrontBlock) void sample_front_compact_kernel(SampleArgs a) {
+    __shared__ FrontPart s_parts[kMaxParts];
+    __shared__ int s_cnt[kFrontWaves];
+    const int part = blockIdx.x, s = blockIdx.y, tid = threadIdx.x, lane = tid & (kWave - 1), wv = tid / kWave;
+    const int kind = a.kind[s];
+    if (!sorts_candidates(kind) || a.temperature[s] <= 1e-5f) return;
+    const int V = a.V;
+    FrontPart* gp = front_parts(a, s);
+    {
+        const uint32_t* src = reinterpret_cast<const uint32_t*>(gp);
+        uint32_t* dst = reinterpret_cast<uint32_t*>(s_parts);
+        const int words = a.parts * static_cast<int>(sizeof(FrontPart) / 4);
+        for (int i = tid; i < words; i += kFrontBlock) dst[i] = src[i];
+    }
+    __syncthreads();
+    SoftmaxStats st{0, 0.0, 0u};
+    uint32_t cc[kLevels];
+    float cm[kLevels];
+#pragma unroll
+    for (int l = 0; l < kLevels; ++l) {
+        cc[l] = 0u;
+        cm[l] = 0.f;
+    }
+    for (int b = 0; b < a.parts; ++b) {
+        st.n_pos += s_parts[b].n_pos;
+        st.total += s_parts[b].ps;
+        st.max_bits = max(st.max_bits, s_parts[b].max_bits);
+#pragma unroll
+        for (int l = 0; l < kLevels; ++l) {
+            cc[l] += s_parts[b].lc[l];
+            cm[l] += s_parts[b].lm[l];
+        }
+    }
+    if (st.n_pos == 0) return;
+    const DrawNeed need = draw_need(a, s, kind, st, a.uniform[s]);
+    const uint32_t t_bits = level_floor(need, st.max_bits, cc, cm);
+    const uint32_t* kin = a.key_a + static_cast<size_t>(s) * V;
+    uint32_t* kout = a.key_b + static_cast<size_t>(s) * V;
+    uint32_t* iout = a.id_b + static_cast<size_t>(s) * V;
+    int lo, hi;
+    front_segment(V, a.parts, part, lo, hi);
+    // each wave a contiguous quarter of the segment, so that the order is the index order
+    const int sub = ((hi - lo + kFrontBlock - 1) / kFrontBlock) * kWave;
+    const int wlo = min(hi, lo + wv * sub), whi = min(hi, wlo + sub);
+    int c = 0;
+    for (int i0 = wlo; i0 < whi; i0 += kWave) {
+        const int i = i0 + lane;
+        c += __popcll(__ballot(i < whi && kin[i] >= t_bits));
+    }
+    if (lane == 0) s_cnt[wv] = c;
+    __syncthreads();
+    int base = lo, total = 0;
+#pragma unroll
+    for (int w = 0; w < kFrontWaves; ++w) {
+        if (w < wv) base += s_cnt[w];
+        total += s_cnt[w];
+    }
+    for (int i0 = wlo; i0 < whi; i0 += kWave) {
+        const int i = i0 + lane;
+        const uint32_t key = i < whi ? kin[i] : 0u;
+        const bool take = i < whi && key >= t_bits;
+        const uint64_t bm = __ballot(take);
+        if (take) {
+            const int at = base + __popcll(bm & ((1ull << lane) - 1ull));
+            kout[at] = key;
+            iout[at] = static_cast<uint32_t>(i);
+        }
+        base += __popcll(bm);
+    }
+    if (tid == 0) {
+        gp[part].cnt = total;
+        gp[part].t_bits = t_bits;
+    }
+}
+
 __global__ __launch_bounds__(kSampBlock) void sample_kernel(SampleArgs a) {
     __shared__ BlockShared sh;
     const int s = blockIdx.x, tid = threadIdx.x, lane = tid & (kWave - 1), wv = tid / kWave;
@@ -506,7 +894,41 @@ __global__ __launch_bounds__(kSampBlock) void sample_kernel(SampleArgs a) {
     if (kind == PIE_HIP_SAMPLER_EMBEDDING) return;    // no output for this slot
     float mx;
     int amax;
-    block_argmax(row, V, sh, tid, lane, wv, mx, amax);
+    const bool front = a.parts > 0;
+    SoftmaxStats fst{0, 0.0, 0u};
+    __shared__ FrontPart s_parts[kMaxParts];
+    if (front) {
+        // the part records through LDS: every thread then combines the same values in the same order
+        {
+            const uint32_t* src = reinterpret_cast<const uint32_t*>(front_parts(a, s));
+            uint32_t* dst = reinterpret_cast<uint32_t*>(s_parts);
+            const int words = a.parts * static_cast<int>(sizeof(FrontPart) / 4);
+            for (int i = tid; i < words; i += kSampBlock) dst[i] = src[i];
+        }
+        __syncthreads();
+        const FrontPart* fp = s_parts;
+        front_max(fp, a.parts, mx, amax);
+        for (int b = 0; b < a.parts; ++b) {
+            fst.n_pos += fp[b].n_pos;
+            fst.total += fp[b].ps;
+            fst.max_bits = max(fst.max_bits, fp[b].max_bits);
+        }
+        if (tid < kSampWaves * kLevels) {
+            const int w = tid / kLevels, l = tid % kLevels;
+            uint32_t c = 0u;
+            float f = 0.f;
+            if (w == 0)
+                for (int b = 0; b < a.parts; ++b) {
+                    c += fp[b].lc[l];
+                    f += fp[b].lm[l];
+                }
+            sh.lcnt[w][l] = c;
+            sh.lmass[w][l] = f;
+        }
+        __syncthreads();
+    } else {
+        block_argmax(row, V, sh, tid, lane, wv, mx, amax);
+    }
     const int o0 = a.out_indptr[s], o1 = a.out_indptr[s + 1];
 
     if (kind == PIE_HIP_SAMPLER_LOGPROB || kind == PIE_HIP_SAMPLER_LOGPROBS) {
@@ -543,7 +965,7 @@ __global__ __launch_bounds__(kSampBlock) void sample_kernel(SampleArgs a) {
     const float temperature = a.temperature[s];
 
     if (kind == PIE_HIP_SAMPLER_DIST) {
-        softmax_to_bits<false>(row, V, mx, temperature, ka, sh, tid, lane, wv);
+        if (!front) softmax_to_bits<false>(row, V, mx, temperature, ka, sh, tid, lane, wv);
         sort_desc(ka, kb, ia, ib, V, false, sh, tid, lane, wv);
         const int k = min(o1 - o0, V);
         for (int i = tid; i < k; i += kSampBlock) {
@@ -561,80 +983,103 @@ __global__ __launch_bounds__(kSampBlock) void sample_kernel(SampleArgs a) {
     const float u = a.uniform[s];
     double total;
     if (kind == PIE_HIP_SAMPLER_MULTINOMIAL) {
-        softmax_to_bits<false>(row, V, mx, temperature, ka, sh, tid, lane, wv);
-        const int tok = find_first<kExceed>(ka, V, u, sh, lane, wv, &total);
+        if (!front) softmax_to_bits<false>(row, V, mx, temperature, ka, sh, tid, lane, wv);
+        int tok = V;
+        if (front) {
+            // the walk's own rule applied to the parts' sums — the first part whose end exceeds u
+            // holds the token — then the walk inside that part only
+            const FrontPart* fp = s_parts;
+            double run = 0.0, before = 0.0;
+            int pick = -1;
+            for (int b = 0; b < a.parts; ++b) {
+                run += fp[b].ps;
+                if (pick < 0) {
+                    if (u < static_cast<float>(run)) pick = b;
+                    else before = run;
+                }
+            }
+            if (pick >= 0) {
+                int plo, phi;
+                front_segment(V, a.parts, pick, plo, phi);
+                tok = find_first<kExceed>(ka, V, u, sh, lane, wv, &total, plo, phi, before);
+            }
+        } else {
+            tok = find_first<kExceed>(ka, V, u, sh, lane, wv, &total);
+        }
         if (tid == 0) a.tokens[s] = static_cast<uint32_t>(tok < V ? tok : amax);
         return;
     }
-    const SoftmaxStats st = softmax_to_bits<true>(row, V, mx, temperature, ka, sh, tid, lane, wv);
+    const SoftmaxStats st = front ? fst : softmax_to_bits<true>(row, V, mx, temperature, ka, sh, tid, lane, wv);
     const int n_pos = st.n_pos;
     if (n_pos == 0) {
         if (tid == 0) a.tokens[s] = 0u;
         return;
     }
-    // What the draw can touch is a head of the descending order: the first top_k entries, the
-    // prefix reaching top_p, the entries above the min-p threshold, or (nothing restricting)
-    // the prefix whose mass exceeds u * total.  Any set {p >= t} containing that head gives
-    // the same result as the whole vocabulary, so only such a set is compacted and sorted;
-    // t is the first of the levels p_max * 2^(-3j) that covers the need (exact for min-p).
-    const bool wants_k = kind == PIE_HIP_SAMPLER_TOP_K || kind == PIE_HIP_SAMPLER_TOP_K_TOP_P;
-    const bool wants_p = kind == PIE_HIP_SAMPLER_TOP_P || kind == PIE_HIP_SAMPLER_TOP_K_TOP_P;
-    const uint32_t top_k = a.top_k[s];
-    const float thr_p = fminf(fmaxf(a.top_p[s], 0.0f), 1.0f);
-    const float thr_m = a.min_p[s] * __uint_as_float(st.max_bits);
-    int need_count = 0;
-    float need_mass = 0.f;
-    uint32_t floor_bits = 0u;     // nonzero: the exact lower bound of the kept entries (min-p)
-    bool keep_all = false;
-    if (wants_k && top_k != 0u) need_count = static_cast<int>(min(top_k, static_cast<uint32_t>(n_pos)));
-    else if (wants_p && thr_p < 1.0f) need_mass = thr_p;
-    else if (kind == PIE_HIP_SAMPLER_MIN_P && thr_m > 0.0f && thr_m <= __uint_as_float(st.max_bits))
-        floor_bits = __float_as_uint(thr_m);
-    else {
-        keep_all = true;
-        need_mass = u * static_cast<float>(st.total);
-    }
+    const DrawNeed need = draw_need(a, s, kind, st, u);
+    const int need_count = need.need_count;
+    const float need_mass = need.need_mass, thr_p = need.thr_p;
+    const bool keep_all = need.keep_all, wants_p = need.wants_p;
     for (int attempt = 0; attempt < 2; ++attempt) {
-        uint32_t t_bits = 1u;     // every positive entry
-        if (floor_bits) t_bits = floor_bits;
-        else if (attempt == 0) {
-            // the first level whose candidates cover the need (every thread computes the same)
-            const uint32_t top_bits = st.max_bits;
-            for (int j = 0; j < kLevels; ++j) {
-                uint32_t cc = 0u;
-                float cm = 0.f;
-#pragma unroll
-                for (int w = 0; w < kSampWaves; ++w) {
-                    cc += sh.lcnt[w][j];
-                    cm += sh.lmass[w][j];
+        uint32_t *ck = kb, *ci = ib;   // where the sorted candidates end up
+        int m;
+        if (attempt == 0 && front && s_parts[0].cnt >= 0) {
+            // the parts' candidate lists (each at the head of its segment of (key_b, id_b)) end to
+            // end into (key_a, id_a): the order compact_ge gives
+            m = 0;
+            for (int b = 0; b < a.parts; ++b) {
+                int plo, phi;
+                front_segment(V, a.parts, b, plo, phi);
+                const int cb = s_parts[b].cnt;
+                for (int i = tid; i < cb; i += kSampBlock) {
+                    ka[m + i] = kb[plo + i];
+                    ia[m + i] = ib[plo + i];
                 }
-                const bool enough = need_count > 0 ? cc >= static_cast<uint32_t>(need_count)
-                                                   : cm >= need_mass + 1e-4f;
-                if (enough && top_bits > (j + 1) * kLevelStep) {
-                    t_bits = top_bits - (j + 1) * kLevelStep;
-                    break;
-                }
+                m += cb;
             }
+            __syncthreads();
+            sort_desc(ka, kb, ia, ib, m, true, sh, tid, lane, wv);
+            ck = ka;
+            ci = ia;
+        } else {
+            uint32_t t_bits = 1u;     // every positive entry
+            if (attempt == 0) {
+                // the first level whose candidates cover the need (every thread computes the same)
+                uint32_t cc[kLevels];
+                float cm[kLevels];
+#pragma unroll
+                for (int j = 0; j < kLevels; ++j) {
+                    cc[j] = 0u;
+                    cm[j] = 0.f;
+#pragma unroll
+                    for (int w = 0; w < kSampWaves; ++w) {
+                        cc[j] += sh.lcnt[w][j];
+                        cm[j] += sh.lmass[w][j];
+                    }
+                }
+                t_bits = level_floor(need, st.max_bits, cc, cm);
+            } else if (need.floor_bits) {
+                t_bits = need.floor_bits;
+            }
+            m = compact_ge(ka, t_bits, kb, ib, V, sh, lane, wv);
+            sort_desc(kb, ka, ib, ia, m, true, sh, tid, lane, wv);   // note: overwrites ka
         }
-        const int m = compact_ge(ka, t_bits, kb, ib, V, sh, lane, wv);
         const bool whole = m == n_pos;
-        sort_desc(kb, ka, ib, ia, m, true, sh, tid, lane, wv);   // note: overwrites ka
         bool ok = true;
         uint32_t tok = 0u;
         if (keep_all) {
-            const int i = find_first<kExceed>(kb, m, need_mass, sh, lane, wv, &total);
+            const int i = find_first<kExceed>(ck, m, need_mass, sh, lane, wv, &total);
             ok = i < m || whole;
-            tok = ib[i < m ? i : m - 1];
+            tok = ci[i < m ? i : m - 1];
         } else {
             int keep = m;
             if (need_count > 0) keep = min(need_count, m);
             if (wants_p && thr_p < 1.0f) {
-                const int i = find_first<kReach>(kb, keep, thr_p, sh, lane, wv, &total);
+                const int i = find_first<kReach>(ck, keep, thr_p, sh, lane, wv, &total);
                 if (i < keep) keep = i + 1;
                 else ok = whole || need_count > 0;   // the prefix must end inside the candidates
             }
-            const int i = find_first<kExceedScaled>(kb, keep, u, sh, lane, wv, &total);
-            tok = total <= 0.0 ? ib[0] : ib[i < keep ? i : keep - 1];
+            const int i = find_first<kExceedScaled>(ck, keep, u, sh, lane, wv, &total);
+            tok = total <= 0.0 ? ci[0] : ci[i < keep ? i : keep - 1];
         }
         if (ok || attempt == 1) {
             if (tid == 0) a.tokens[s] = tok;
@@ -727,7 +1172,25 @@ extern "C" int pie_hip_sample(const float* logits_f32, const int32_t* kind, cons
     a.id_a = a.key_b + n;
     a.id_b = a.id_a + n;
     a.V = vocab;
-    hipLaunchKernelGGL(sample_kernel, dim3(num_slots), dim3(kSampBlock), 0,
-                       static_cast<hipStream_t>(stream), a);
+    // Few slots over a wide vocabulary: the row-wide passes run over many blocks first
+    // (PIE_HIP_SAMPLE_PARTS = n forces the part count, 0 the single-block path: measurement hook).
+    static const int forced_parts = [] { const char* e = getenv("PIE_HIP_SAMPLE_PARTS"); return e ? atoi(e) : -1; }();
+    int parts = 0;
+    // (measured at a 128 k vocabulary, peaked rows: 1 / 8 slots 40-60 us less per call for the kinds
+    // that sort candidates, 20-40 us less for the multinomial walk; at 64 slots the four launches
+    // cost more than one block per slot, which fills a quarter of the machine by itself)
+    if (vocab >= 16384 && num_slots <= 16) parts = std::min(kMaxParts, 256 / num_slots);
+    if (forced_parts >= 0) parts = std::min(forced_parts, kMaxParts);
+    if (parts == 1 || static_cast<size_t>(parts) * sizeof(FrontPart) > static_cast<size_t>(vocab) * 4) parts = 0;
+    a.parts = parts;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (parts > 0) {
+        const dim3 grid(parts, num_slots);
+        hipLaunchKernelGGL(sample_front_max_kernel, grid, dim3(kFrontBlock), 0, st, a);
+        hipLaunchKernelGGL(sample_front_exp_kernel, grid, dim3(kFrontBlock), 0, st, a);
+        hipLaunchKernelGGL(sample_front_norm_kernel, grid, dim3(kFrontBlock), 0, st, a);
+        hipLaunchKernelGGL(sample_front_compact_kernel, grid, dim3(kFrontBlock), 0, st, a);
+    }
+    hipLaunchKernelGGL(sample_kernel, dim3(num_slots), dim3(kSampBlock), 0, st, a);
     return launch_status();
 }

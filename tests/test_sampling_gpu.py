@@ -60,6 +60,35 @@ def test_token_samplers_match_oracle(gpu, oracle, V):
     assert near <= S // 4, near
 
 
+@pytest.mark.parametrize("V", [32000, 128256])
+def test_few_slots_take_the_many_block_front_end(gpu, oracle, V):
+    """Calls of at most sixteen slots over a wide vocabulary run the row-wide passes over many
+    blocks per slot before the one block per slot: the same slots sampled eight and one at a time
+    give the tokens the oracle gives, and the tokens of a 24-slot call (one block per slot alone)."""
+    import torch
+    from pie_amd import ops
+
+    rng = np.random.default_rng(905 + V)
+    S = 24
+    scales = rng.choice([3.0, 5.0, 8.0], size=S)
+    bits, lg = make_logits(oracle, rng, S, V, scales)
+    kinds, temp, top_k, top_p, min_p, seeds = random_slots(rng, S)
+    u = np.array([oracle.pcg32_first_uniform(int(s)) for s in seeds], np.float32)
+    f32 = ops.sample_gather_logits(dev(bits, gpu, torch.bfloat16))
+    whole = ops.sample(f32, kinds, temp, top_k, top_p, min_p, u)[0].cpu().numpy().view(np.uint32)
+    chunks = [(i, i + 8) for i in range(0, S, 8)] + [(i, i + 1) for i in range(5)]
+    for lo, hi in chunks:
+        sl = slice(lo, hi)
+        got = ops.sample(f32[sl].contiguous(), kinds[sl], temp[sl], top_k[sl], top_p[sl], min_p[sl], u[sl])[0]
+        got = got.cpu().numpy().view(np.uint32)
+        assert np.array_equal(got, whole[sl]), (lo, hi)
+        for s in range(lo, hi):
+            want, margin = oracle.sample_token(lg[s], kinds[s], float(temp[s]), int(top_k[s]),
+                                               float(top_p[s]), float(min_p[s]), u=float(u[s]))
+            if margin > TOL:
+                assert got[s - lo] == want, (s, kinds[s], temp[s], top_k[s], top_p[s], min_p[s], margin)
+
+
 def test_sorted_order_and_rows_argument(gpu, oracle):
     """Rows picked out of a larger logits matrix; top_k = 1 / tiny top_p / min_p = 1 / T = 0 all
     reduce to the first-index argmax, also with an exact tie of the maximum."""
