@@ -439,7 +439,7 @@ struct SwGeom {
     static constexpr int region = staged > meet ? staged : meet;   // vectors per wave region
 };
 
-template <class F, int NG, int MT>
+template <class F, int NG, int MT, bool GROUPED = false>
 __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 && MT == 1 ? 4 : 2) void skinny_wave_kernel(const SkinnyArgs a, const int kp_shift) {
     constexpr int KPL = F::kPerLane, S = F::kSteps;
     constexpr int LK = 4 * KPL;                     // k covered by one wave-wide 16-byte load (a block)
@@ -466,17 +466,19 @@ __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 && MT == 1 ? 4 : 2) void s
     const int KP = 1 << kp_shift;
     const int ks = wv & (KP - 1);
     const int N = a.N, K = a.K;
-    // (dense problems only: the grouped MoE launches run the block-shared kernel.  Every scalar
-    // instruction ahead of the first weight request delays it: four waves per SIMD walk this
-    // prologue at once)
-    const int r0 = a.m_split ? blockIdx.y * ROWS : 0;
-    const int r1 = a.m_split ? min(a.M, r0 + ROWS) : a.M;
+    // (GROUPED: blockIdx.y is the problem — an expert — with its rows offsets[p] .. offsets[p + 1],
+    // its weights and scales one stride further, its activation rows gathered by route.  A compile-
+    // time case: every scalar instruction ahead of the first weight request delays it, four waves
+    // per SIMD walk this prologue at once)
+    const int p = GROUPED ? blockIdx.y : 0;
+    const int r0 = GROUPED ? a.offsets[p] : (a.m_split ? blockIdx.y * ROWS : 0);
+    const int r1 = GROUPED ? a.offsets[p + 1] : (a.m_split ? min(a.M, r0 + ROWS) : a.M);
     if (r1 <= r0) return;
 
     const int T = (N + 15) / 16;
     const int tile0 = (blockIdx.x * (kSwWaves >> kp_shift) + (wv >> kp_shift)) * NG;
-    const unsigned char* wbase = a.w;
-    const unsigned char* sbase = a.scale;
+    const unsigned char* wbase = GROUPED ? a.w + static_cast<size_t>(p) * a.w_stride : a.w;
+    const unsigned char* sbase = GROUPED && a.scale ? a.scale + static_cast<size_t>(p) * a.scale_stride : a.scale;
     const uint16_t* gsbase = reinterpret_cast<const uint16_t*>(sbase);
     const int blk_shift = a.g_shift - (F::kGroupScale ? 7 : 0);
     const int nb = K / LK;
@@ -554,6 +556,7 @@ __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 && MT == 1 ? 4 : 2) void s
 #pragma unroll
         for (int u = 0; u < SV; ++u) {
             arow[u] = min(mt0 + srow + RPL * u, r1 - 1);
+            if (GROUPED && a.act_rows) arow[u] = a.act_rows[arow[u]];
         }
         u32x4_t stg[SV];
         auto stage_load = [&](int c) {
@@ -756,17 +759,17 @@ __global__ __launch_bounds__(kSwWaves* kWave, NG == 1 && MT == 1 ? 4 : 2) void s
     }
 }
 
-template <class F, int NG, int MT>
+template <class F, int NG, int MT, bool GROUPED = false>
 int launch_wave_cfg(const SkinnyArgs& a, int problems, int kp_shift, hipStream_t stream) {
     constexpr size_t smem = static_cast<size_t>(kSwWaves) * SwGeom<MT, NG>::region * 16;
     static const hipError_t attr = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(&skinny_wave_kernel<F, NG, MT>),
+        reinterpret_cast<const void*>(&skinny_wave_kernel<F, NG, MT, GROUPED>),
         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
     if (attr != hipSuccess) return PIE_HIP_ERR_LAUNCH;
     const int tgroups = ((a.N + 15) / 16 + NG - 1) / NG;
     const int per_block = kSwWaves >> kp_shift;
     const dim3 grid((tgroups + per_block - 1) / per_block, a.m_split ? (a.M + 16 * MT - 1) / (16 * MT) : problems);
-    hipLaunchKernelGGL((skinny_wave_kernel<F, NG, MT>), grid, dim3(kSwWaves * kWave), smem, stream, a, kp_shift);
+    hipLaunchKernelGGL((skinny_wave_kernel<F, NG, MT, GROUPED>), grid, dim3(kSwWaves * kWave), smem, stream, a, kp_shift);
     return launch_status();
 }
 
@@ -879,9 +882,14 @@ int launch_skinny(SkinnyArgs a, int problems, hipStream_t stream) {
     // dense tile-major launches take the wave-private form (measured, 8B decode steps of 8 / 16 /
     // 32 / 64 rows: 2.43 / 2.78 / 3.42 / 5.18 ms against 2.75 / 2.95 / 4.07 / 5.64); the grouped
     // MoE launches stay with the block-shared form, whose eight tiles per staged chunk halve the
-    // activation traffic (30B-A3B, 64 rows: 7.9 against 11.0 ms per step)
+    // activation traffic (30B-A3B, 64 rows: 7.9 against 11.0 ms per step) — except over a short K, below
     if (a.rope_table) return launch_wave<F>(a, problems, stream);   // (entry point checked K)
     if (a.tiled && !a.offsets && !old_form && a.K % kSwChunk == 0) return launch_wave<F>(a, problems, stream);
+    // grouped launches over a short K (an expert's down projection: K = 768): one tile per wave over
+    // the whole K, no waves to meet — 43.4 against 47.9 us for the 128 experts of a 30B-A3B layer;
+    // at K = 2048 (gate|up) the block-shared form keeps its lead, 74.1 against 75.8 us
+    if (a.tiled && a.offsets && !old_form && a.K <= 1024 && a.K % kSwChunk == 0)
+        return launch_wave_cfg<F, 1, 1, true>(a, problems, 0, stream);
     if (a.K % (8 * LK) == 0) {
         if (tiles / 8 >= 448) return launch_cfg<F, 4, CK, 8, 4, 2>(a, problems, stream);
         if (tiles / 4 >= 448) return launch_cfg<F, 4, CK, 4, 4, 2>(a, problems, stream);
