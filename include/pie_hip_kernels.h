@@ -36,7 +36,17 @@ extern "C" {
 #define PIE_HIP_ERR_UNSUPPORTED 2 /* shape the kernels do not cover              */
 #define PIE_HIP_ERR_LAUNCH 3      /* HIP reported an error at launch             */
 
-/* Library/ABI version: bumped on any signature change. */
+/* Library/ABI version: bumped on any change of a signature or of a memory layout an entry point
+ * reads or writes.  A caller compares the macro it was built against with what the loaded
+ * library returns and refuses to run on a mismatch (an old caller would link and compute
+ * garbage).  History:
+ *   1  first layout
+ *   2  `pairing` argument of pie_hip_qkv_rope_fused / pie_hip_qkv_rope_skinny_tiled; `page_size`
+ *      argument of pie_hip_kv_write_quant / pie_hip_qkv_rope_kvwrite_quant; KV scale pools
+ *      [pages, hk, page_size] (were [pages, page_size, hk]); int4 tile-major weights in decode
+ *      order (pie_hip_repack_mfma_tiles_int4); pie_hip_gemv_time_next removed
+ *   3  current */
+#define PIE_HIP_ABI_VERSION 3
 int pie_hip_abi_version(void);
 
 /* ---- W4A16 ("int4b8", symmetric, group-quantised) ------------------------- */

@@ -6,7 +6,7 @@ from pathlib import Path
 
 _PKG = Path(__file__).resolve().parent
 KERNEL_LIB_PATH = _PKG / "libpie_hip_kernels.so"
-ABI_VERSION = 1
+ABI_VERSION = 3   # PIE_HIP_ABI_VERSION of include/pie_hip_kernels.h this module was written against
 
 _kernels = None
 

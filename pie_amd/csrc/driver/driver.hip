@@ -21,6 +21,7 @@
 #include "executor.hpp"
 #include "model.hpp"
 #include "pie_driver_abi.h"
+#include "pie_hip_kernels.h"
 #include "planner.hpp"
 #include "snapshot.hpp"
 
@@ -234,6 +235,10 @@ struct PieHipDriver {
     uint32_t gen_diverge = 0;   // generation harness: replica c starts decoding from (first token + c * this) % vocab
 
     explicit PieHipDriver(const DriverConfig& c) : cfg(c) {
+        // the kernel library found at run time must be the one this driver was compiled against
+        if (pie_hip_abi_version() != PIE_HIP_ABI_VERSION)
+            throw std::runtime_error("libpie_hip_kernels.so has ABI version " + std::to_string(pie_hip_abi_version()) +
+                                     ", this driver was built against " + std::to_string(PIE_HIP_ABI_VERSION));
         int ndev = 0;
         if (hipGetDeviceCount(&ndev) != hipSuccess || ndev <= 0)
             throw std::runtime_error("no HIP device is visible: this driver has no CPU path");

@@ -138,7 +138,7 @@ __global__ void quant_int4b8_group_kernel(const uint16_t* __restrict__ w,
 }  // namespace
 }  // namespace pie_hip
 
-extern "C" int pie_hip_abi_version(void) { return 1; }
+extern "C" int pie_hip_abi_version(void) { return PIE_HIP_ABI_VERSION; }
 
 extern "C" int pie_hip_unpack_w4(const uint32_t* packed, int8_t* q, int out_dim, int in_dim,
                                  void* stream) {

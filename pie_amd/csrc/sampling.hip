@@ -309,10 +309,14 @@ __device__ int find_first(const uint32_t* __restrict__ pbits, int limit, float t
             *total_out = total;
             if (MODE == kExceedScaled) x = thr * static_cast<float>(total);
         }
-        int pick = -1;
-        double before = base, run = base;
+        int pick = -1, last_mass = -1;
+        double before = base, run = base, before_last = base;
 #pragma unroll
         for (int w = 0; w < kSampWaves; ++w) {
+            if (sh.f64[w] > 0.0) {
+                last_mass = w;
+                before_last = run;
+            }
             run += sh.f64[w];
             const float cum = static_cast<float>(run);
             const bool hit = MODE == kReach ? cum >= x : x < cum;
@@ -322,7 +326,13 @@ __device__ int find_first(const uint32_t* __restrict__ pbits, int limit, float t
         __syncthreads();
         if (pick < 0) {
             if (top) return limit;      // the rule is never met
-            return hi - 1;              // (re-associated sums disagreeing in the last bit)
+            // The level above found the crossing inside this range and this level's
+            // re-associated sums disagree in the last bit: the answer is the range's last entry
+            // with a positive probability (never an entry the softmax or a logit mask zeroed),
+            // so carry on inside the last sub-range that holds any mass.
+            pick = last_mass;
+            before = before_last;
+            if (pick < 0) return hi - 1;   // (a range without mass is never chosen by the level above)
         }
         base = before;
         lo = min(hi, lo + pick * sub);
@@ -338,7 +348,10 @@ __device__ int find_first(const uint32_t* __restrict__ pbits, int limit, float t
     }
     const float cum = static_cast<float>(base + incl);
     const uint64_t b = __ballot(i < hi && (MODE == kReach ? cum >= x : x < cum));
-    return b ? lo + __ffsll(static_cast<long long>(b)) - 1 : hi - 1;
+    if (b) return lo + __ffsll(static_cast<long long>(b)) - 1;
+    // same disagreement in the last 64 entries: the last one with a positive probability
+    const uint64_t pos = __ballot(i < hi && __uint_as_float(pbits[min(i, hi - 1)]) > 0.0f);
+    return pos ? lo + 63 - __clzll(static_cast<long long>(pos)) : hi - 1;
 }
 
 // p = softmax(row / T) as float bit patterns in `out`.  Also: the number of entries with p > 0,
@@ -1182,6 +1195,9 @@ extern "C" int pie_hip_sample(const float* logits_f32, const int32_t* kind, cons
     if (vocab >= 16384 && num_slots <= 16) parts = std::min(kMaxParts, 256 / num_slots);
     if (forced_parts >= 0) parts = std::min(forced_parts, kMaxParts);
     if (parts == 1 || static_cast<size_t>(parts) * sizeof(FrontPart) > static_cast<size_t>(vocab) * 4) parts = 0;
+    // a slot's part records hold doubles at byte 4 * slot * vocab of the id_a region: keep them
+    // 8-byte aligned (an odd vocabulary takes the single-block path)
+    if (vocab % 2 != 0 && num_slots > 1) parts = 0;
     a.parts = parts;
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (parts > 0) {

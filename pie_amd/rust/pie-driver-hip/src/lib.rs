@@ -18,6 +18,7 @@ use std::ffi::{c_char, c_int, c_void, CStr};
 
 /// `void (*ready_cb)(const char* caps_json, void* ctx)`: called once, after weights and the KV
 /// pool are allocated, with the capabilities JSON.
+/// The C side accepts NULL (no notification), hence `Option<ReadyCb>` in the signatures.
 pub type ReadyCb = unsafe extern "C" fn(caps_json: *const c_char, ctx: *mut c_void);
 
 /// `PieInProcVTable` (`driver/bridge/include/pie_bridge.h:437-451`), passed by value.
@@ -37,7 +38,7 @@ extern "C" {
         argc: c_int,
         argv: *mut *mut c_char,
         install_signal_handlers: c_int,
-        ready_cb: ReadyCb,
+        ready_cb: Option<ReadyCb>,
         ready_ctx: *mut c_void,
         vtable: InProcVTable,
     ) -> c_int;
@@ -46,125 +47,15 @@ extern "C" {
     pub fn pie_driver_hip_request_stop();
 }
 
-/// Status codes of the kernel library.
-pub const PIE_HIP_OK: c_int = 0;
-pub const PIE_HIP_ERR_INVALID: c_int = 1;
-pub const PIE_HIP_ERR_UNSUPPORTED: c_int = 2;
-pub const PIE_HIP_ERR_LAUNCH: c_int = 3;
+/// Raw declarations and constants of the kernel library, generated from
+/// `include/pie_hip_kernels.h` by `gen_sys.py` (every entry point, every `PIE_HIP_*` constant).
+pub mod sys;
+pub use sys::*;
 
-/// Weight storage formats (`format` arguments).
-pub const PIE_HIP_FMT_INT4B8: c_int = 0;
-pub const PIE_HIP_FMT_INT8: c_int = 1;
-pub const PIE_HIP_FMT_FP8: c_int = 2;
-pub const PIE_HIP_FMT_BF16: c_int = 3;
-
-/// KV-cache storage formats (`kv_format` arguments).
-pub const PIE_HIP_KV_BF16: c_int = 0;
-pub const PIE_HIP_KV_FP8_E4M3: c_int = 1;
-pub const PIE_HIP_KV_INT8_PER_TOKEN_HEAD: c_int = 2;
-pub const PIE_HIP_KV_FP8_PER_TOKEN_HEAD: c_int = 3;
-pub const PIE_HIP_KV_FP8_E5M2: c_int = 4;
-
-/// RoPE pairings of the rotation kernels and fused epilogues.
-pub const PIE_HIP_ROPE_HALF: c_int = 0;
-pub const PIE_HIP_ROPE_ADJACENT: c_int = 1;
-pub const PIE_HIP_ROPE_HALF_PAIRED_ROWS: c_int = 2;
-
-extern "C" {
-    pub fn pie_hip_abi_version() -> c_int;
-
-    // ---- quantised linears -------------------------------------------------------------------
-    pub fn pie_hip_linear_fused(
-        format: c_int, act_bf16: *const u16, norm_weight_bf16: *const u16, eps: f32,
-        weight: *const c_void, scale: *const c_void, scale_is_bf16: c_int, group_size: c_int,
-        y_bf16: *mut u16, m: c_int, n: c_int, k: c_int, beta: c_int, swiglu: c_int,
-        stream: *mut c_void,
-    ) -> c_int;
-    pub fn pie_hip_qkv_rope_fused(
-        format: c_int, act_bf16: *const u16, norm_weight_bf16: *const u16, eps: f32,
-        weight: *const c_void, scale: *const c_void, scale_is_bf16: c_int, group_size: c_int,
-        m: c_int, k: c_int, rope_table: *const f32, kv_slots: *const i64, q_out: *mut u16,
-        k_pages: *mut u16, v_pages: *mut u16, num_q_heads: c_int, num_kv_heads: c_int,
-        head_dim: c_int, pairing: c_int, stream: *mut c_void,
-    ) -> c_int;
-    pub fn pie_hip_gemm_skinny_tiled(
-        format: c_int, act_bf16: *const u16, weight: *const c_void, scale: *const c_void,
-        scale_is_bf16: c_int, group_size: c_int, y_bf16: *mut u16, m: c_int, n: c_int, k: c_int,
-        beta: c_int, swiglu: c_int, stream: *mut c_void,
-    ) -> c_int;
-    pub fn pie_hip_gemm_mfma(
-        format: c_int, act_bf16: *const u16, weight: *const c_void, scale: *const c_void,
-        scale_is_bf16: c_int, group_size: c_int, y_bf16: *mut u16, m: c_int, n: c_int, k: c_int,
-        beta: c_int, swiglu: c_int, stream: *mut c_void,
-    ) -> c_int;
-    pub fn pie_hip_lm_head_argmax_workspace_bytes(m: c_int, v: c_int) -> usize;
-    pub fn pie_hip_lm_head_argmax(
-        act_bf16: *const u16, norm_weight_bf16: *const u16, eps: f32, w_bf16: *const u16,
-        logits_bf16: *mut u16, out_tokens: *mut u32, m: c_int, v: c_int, h: c_int,
-        workspace: *mut c_void, workspace_bytes: usize, stream: *mut c_void,
-    ) -> c_int;
-
-    // ---- paged attention ----------------------------------------------------------------------
-    pub fn pie_hip_attn_decode_workspace_bytes(
-        num_requests: c_int, num_q_heads: c_int, num_kv_heads: c_int, head_dim: c_int,
-        max_kv_len: c_int,
-    ) -> usize;
-    pub fn pie_hip_attn_rows_paged(
-        q: *const u16, k_pages: *const u16, v_pages: *const u16, o: *mut u16, lse: *mut f32,
-        kv_page_indices: *const u32, row_page_begin: *const u32, row_kv_len: *const i32,
-        num_rows: c_int, num_q_heads: c_int, num_kv_heads: c_int, head_dim: c_int,
-        page_size: c_int, sm_scale: f32, max_kv_len: c_int, workspace: *mut c_void,
-        workspace_bytes: usize, stream: *mut c_void,
-    ) -> c_int;
-    /// The same without a workspace or any allocation (split partials in a 16 MiB device array
-    /// built into the library); larger batches return `PIE_HIP_ERR_UNSUPPORTED`.
-    pub fn pie_hip_attn_rows_paged_static(
-        q: *const u16, k_pages: *const u16, v_pages: *const u16, o: *mut u16, lse: *mut f32,
-        kv_page_indices: *const u32, row_page_begin: *const u32, row_kv_len: *const i32,
-        num_rows: c_int, num_q_heads: c_int, num_kv_heads: c_int, head_dim: c_int,
-        page_size: c_int, sm_scale: f32, max_kv_len: c_int, stream: *mut c_void,
-    ) -> c_int;
-    pub fn pie_hip_attn_rows_paged_kvq(
-        kv_format: c_int, q: *const u16, k_pages: *const c_void, v_pages: *const c_void,
-        k_scales: *const f32, v_scales: *const f32, o: *mut u16, lse: *mut f32,
-        kv_page_indices: *const u32, row_page_begin: *const u32, row_kv_len: *const i32,
-        num_rows: c_int, num_q_heads: c_int, num_kv_heads: c_int, head_dim: c_int,
-        page_size: c_int, sm_scale: f32, max_kv_len: c_int, workspace: *mut c_void,
-        workspace_bytes: usize, stream: *mut c_void,
-    ) -> c_int;
-    pub fn pie_hip_kv_write_quant(
-        kv_format: c_int, k_rows: *const u16, v_rows: *const u16, kv_slots: *const i64,
-        k_pages: *mut c_void, v_pages: *mut c_void, k_scales: *mut f32, v_scales: *mut f32,
-        num_tokens: c_int, num_kv_heads: c_int, head_dim: c_int, page_size: c_int,
-        stream: *mut c_void,
-    ) -> c_int;
-    pub fn pie_hip_kv_dequant_pages(
-        kv_format: c_int, k_pages: *const c_void, v_pages: *const c_void, k_scales: *const f32,
-        v_scales: *const f32, k_out: *mut u16, v_out: *mut u16, page_ids: *const u32,
-        num_pages: c_int, num_kv_heads: c_int, head_dim: c_int, page_size: c_int,
-        stream: *mut c_void,
-    ) -> c_int;
-
-    // ---- layer ops ------------------------------------------------------------------------------
-    pub fn pie_hip_embed(
-        token_ids: *const u32, table_bf16: *const u16, y_bf16: *mut u16, num_tokens: c_int,
-        hidden: c_int, vocab: c_int, stream: *mut c_void,
-    ) -> c_int;
-    pub fn pie_hip_rmsnorm(
-        x_bf16: *const u16, weight_bf16: *const u16, y_bf16: *mut u16, num_tokens: c_int,
-        hidden: c_int, eps: f32, stream: *mut c_void,
-    ) -> c_int;
-    pub fn pie_hip_rope_table(
-        positions: *const i32, inv_freq: *const f32, table: *mut f32, num_tokens: c_int,
-        head_dim: c_int, stream: *mut c_void,
-    ) -> c_int;
-    pub fn pie_hip_argmax(
-        logits_bf16: *const u16, out_idx: *mut u32, rows: c_int, vocab: c_int, stream: *mut c_void,
-    ) -> c_int;
-    pub fn pie_hip_copy_kv_pages(
-        pool: *mut c_void, src_pages: *const u32, dst_pages: *const u32, num_pairs: c_int,
-        page_bytes: usize, stream: *mut c_void,
-    ) -> c_int;
+/// Refuses a kernel library whose ABI version differs from the header these bindings were
+/// generated from: an older or newer library links, and then computes garbage.
+pub fn check_abi() -> Result<(), KernelError> {
+    if unsafe { pie_hip_abi_version() } == PIE_HIP_ABI_VERSION { Ok(()) } else { Err(KernelError::AbiMismatch) }
 }
 
 /// A kernel-library status as a `Result`.
@@ -182,6 +73,8 @@ pub enum KernelError {
     InvalidArgument,
     UnsupportedShape,
     Launch,
+    /// The loaded library's `pie_hip_abi_version()` is not `PIE_HIP_ABI_VERSION`.
+    AbiMismatch,
 }
 
 /// Runs the driver on the calling thread, the way the server's flavour dispatcher does for the
@@ -193,10 +86,11 @@ pub enum KernelError {
 pub unsafe fn run_inproc(
     args: &[&CStr],
     install_signal_handlers: bool,
-    ready_cb: ReadyCb,
+    ready_cb: Option<ReadyCb>,
     ready_ctx: *mut c_void,
     vtable: InProcVTable,
 ) -> Result<(), c_int> {
+    check_abi().map_err(|_| -2)?;
     let mut argv: Vec<*mut c_char> = args.iter().map(|a| a.as_ptr() as *mut c_char).collect();
     let rc = pie_driver_hip_run_inproc(
         argv.len() as c_int,

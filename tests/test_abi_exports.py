@@ -28,6 +28,49 @@ def test_kernel_library_exports_declared_symbols():
     from pie_amd._lib import ABI_VERSION
 
     assert lib.pie_hip_abi_version() == ABI_VERSION
+    # header macro, Python mirror, Rust constant and the built library agree
+    header = (ROOT / "include" / "pie_hip_kernels.h").read_text()
+    assert int(re.search(r"#define\s+PIE_HIP_ABI_VERSION\s+(\d+)", header).group(1)) == ABI_VERSION
+    rs = _rust_sources()
+    assert int(re.search(r"pub const PIE_HIP_ABI_VERSION: c_int = (\d+);", rs).group(1)) == ABI_VERSION
+
+
+def test_rust_constants_match_the_header():
+    """Every PIE_HIP_* integer macro of the kernel header exists in the Rust crate with the same
+    value (formats, KV storage kinds, RoPE pairings, sampler kinds, status codes)."""
+    header = re.sub(r"/\*.*?\*/", "", (ROOT / "include" / "pie_hip_kernels.h").read_text(), flags=re.S)
+    rs = _rust_sources()
+    macros = dict(re.findall(r"#define\s+(PIE_HIP_[A-Z0-9_]+)\s+(-?\d+)\s*$", header, flags=re.M))
+    for body in re.findall(r"enum\s*\{(.*?)\}", header, flags=re.S):
+        macros.update(re.findall(r"(PIE_HIP_[A-Z0-9_]+)\s*=\s*(-?\d+)", body))
+    consts = dict(re.findall(r"pub const (PIE_HIP_[A-Z0-9_]+): c_int = (-?\d+);", rs))
+    assert len(macros) >= 15
+    missing = sorted(set(macros) - set(consts))
+    assert not missing, f"header macros without a Rust constant: {missing}"
+    wrong = {k: (macros[k], consts[k]) for k in macros if int(macros[k]) != int(consts[k])}
+    assert not wrong, wrong
+
+
+def _rust_sources() -> str:
+    src = ROOT / "pie_amd" / "rust" / "pie-driver-hip" / "src"
+    return (src / "lib.rs").read_text() + "\n" + (src / "sys.rs").read_text()
+
+
+def test_generated_rust_declarations_are_up_to_date_and_cover_the_header():
+    """src/sys.rs is what gen_sys.py makes of the current header, and it binds every declared
+    entry point."""
+    import subprocess
+    import sys
+
+    gen = ROOT / "pie_amd" / "rust" / "pie-driver-hip" / "gen_sys.py"
+    assert subprocess.run([sys.executable, str(gen), "--check"]).returncode == 0, \
+        "include/pie_hip_kernels.h changed: run pie_amd/rust/pie-driver-hip/gen_sys.py"
+    rs = _rust_sources()
+    bound = set(re.findall(r"pub fn (pie_hip_\w+)\s*\(", rs))
+    names = set(declared(ROOT / "include" / "pie_hip_kernels.h", "pie_hip_"))
+    assert names <= bound, sorted(names - bound)
+    # the ready callback may be null on the C side
+    assert "ready_cb: Option<ReadyCb>" in rs
 
 
 def test_missing_library_is_loud(monkeypatch, tmp_path):
@@ -42,8 +85,7 @@ def test_missing_library_is_loud(monkeypatch, tmp_path):
 def test_rust_bindings_name_only_exported_symbols_with_matching_arity():
     """The (uncompiled) Rust FFI declarations under pie_amd/rust bind functions that the two
     libraries really export, with as many parameters as the C headers declare."""
-    rs = (ROOT / "pie_amd" / "rust" / "pie-driver-hip" / "src" / "lib.rs").read_text()
-    rs = re.sub(r"//[^\n]*", "", rs)
+    rs = re.sub(r"//[^\n]*", "", _rust_sources())
     decls = re.findall(r"pub fn (pie_\w+)\s*\((.*?)\)\s*(?:->[^;]+)?;", rs, flags=re.S)
     assert len(decls) >= 15
     headers = ""

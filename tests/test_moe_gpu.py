@@ -57,23 +57,27 @@ def test_combine_is_bit_exact(gpu, oracle, add):
     assert np.array_equal(got, ref)
 
 
-def test_expert_block_at_c5_expert_shape(gpu, oracle):
+def _expert_block(gpu, oracle, seed, T, E, K, tiled, H=2048, Ie=768):
     """norm'd activations -> router -> route -> grouped gate/up (+SwiGLU) -> grouped down ->
-    combine, fp8 e4m3 experts with bf16 row scales: H 2048, expert FFN 768 (32 of the 128
-    experts, top-4, to keep the CPU side small)."""
+    combine, fp8 e4m3 experts with bf16 row scales, against the oracle's per-route evaluation.
+    `tiled`: the launches a driver with tile-major weights makes (gate|up in the block-shared
+    grouped form, down in the wave-private grouped form over K = Ie), with the driver's
+    rows-per-expert hint; otherwise the row-major entry."""
     import torch
     from pie_amd import ops
 
-    rng = np.random.default_rng(520)
-    T, H, Ie, E, K = 48, 2048, 768, 32, 4
+    rng = np.random.default_rng(seed)
     x = oracle.f32_to_bf16(rng.standard_normal((T, H)).astype(np.float32))
     router = oracle.f32_to_bf16(rng.standard_normal((E, H)).astype(np.float32) * (1.0 / np.sqrt(H)))
 
     def fp8_stack(n, k):
-        w = oracle.f32_to_bf16(rng.standard_normal((E * n, k), dtype=np.float32) * 0.02)
-        q, s = oracle.quant_fp8_per_channel(w)
-        sb = oracle.f32_to_bf16(s)
-        return q, sb
+        qs, ss = [], []
+        for _ in range(E):      # expert by expert: the float copy of a whole stack is gigabytes
+            w = oracle.f32_to_bf16(rng.standard_normal((n, k), dtype=np.float32) * 0.02)
+            q, s = oracle.quant_fp8_per_channel(w)
+            qs.append(q)
+            ss.append(oracle.f32_to_bf16(s))
+        return np.concatenate(qs), np.concatenate(ss)
     gu_q, gu_s = fp8_stack(2 * Ie, H)      # canonical: per expert gate rows then up rows
     dn_q, dn_s = fp8_stack(H, Ie)
 
@@ -81,11 +85,13 @@ def test_expert_block_at_c5_expert_shape(gpu, oracle):
     logits = oracle.gemm_bf16(x, router, mode=0)[1]
     oidx, ow = oracle.topk_softmax(logits, K)
     yr = np.empty((T * K, H), np.uint16)
+    act_ref = np.empty((T * K, Ie), np.uint16)
     for r in range(T * K):
         t, e = r // K, oidx.reshape(-1)[r]
         g = oracle.gemm_fp8(x[t:t + 1], gu_q[e * 2 * Ie:(e + 1) * 2 * Ie],
                             oracle.bf16_to_f32(gu_s[e * 2 * Ie:(e + 1) * 2 * Ie]), mode=0)[1]
         a = oracle.swiglu(g)
+        act_ref[r] = a[0]
         yr[r] = oracle.gemm_fp8(a, dn_q[e * H:(e + 1) * H], oracle.bf16_to_f32(dn_s[e * H:(e + 1) * H]),
                                 mode=0)[1][0]
     ref = oracle.moe_combine(yr, ow, x)
@@ -97,14 +103,83 @@ def test_expert_block_at_c5_expert_shape(gpu, oracle):
     idx, w, offs, rtok, rpos = ops.moe_route(lg, K)
     perm = np.empty(2 * Ie, np.int64)
     perm[0::2], perm[1::2] = np.arange(Ie), np.arange(Ie) + Ie
-    gu_qi = gu_q.reshape(E, 2 * Ie, H)[:, perm]
-    gu_si = gu_s.reshape(E, 2 * Ie)[:, perm]
-    h = ops.moe_grouped_gemm(xg, rtok, offs, "fp8", dev(gu_qi, gpu), dev(gu_si, gpu, torch.bfloat16),
-                             2 * Ie, H, rows_hint=16, swiglu=True)
-    y = ops.moe_grouped_gemm(h, None, offs, "fp8", dev(dn_q.reshape(E, H, Ie), gpu),
-                             dev(dn_s.reshape(E, H), gpu, torch.bfloat16), H, Ie, rows_hint=16)
+    gu_qi = dev(np.ascontiguousarray(gu_q.reshape(E, 2 * Ie, H)[:, perm]), gpu)
+    gu_si = dev(np.ascontiguousarray(gu_s.reshape(E, 2 * Ie)[:, perm]), gpu, torch.bfloat16)
+    dn_qg = dev(dn_q.reshape(E, H, Ie), gpu)
+    dn_sg = dev(dn_s.reshape(E, H), gpu, torch.bfloat16)
+    # the executor's hint (Executor::moe_block): twice the mean routes per expert, at most T
+    hint = max(1, min(T, 2 * ((T * K + E - 1) // E))) if tiled else 16
+    if tiled:
+        # experts stacked along the rows: the tile-major copy keeps expert e at the same stride
+        gu_qi = ops.repack_mfma_tiles(ops.WeightView("fp8", gu_qi.reshape(E * 2 * Ie, H), None, 0,
+                                                     E * 2 * Ie, H)).data.reshape(E, 2 * Ie, -1)
+        dn_qg = ops.repack_mfma_tiles(ops.WeightView("fp8", dn_qg.reshape(E * H, Ie), None, 0,
+                                                     E * H, Ie)).data.reshape(E, H, -1)
+    h = ops.moe_grouped_gemm(xg, rtok, offs, "fp8", gu_qi, gu_si, 2 * Ie, H, rows_hint=hint, swiglu=True,
+                             tiled=tiled)
+    y = ops.moe_grouped_gemm(h, None, offs, "fp8", dn_qg, dn_sg, H, Ie, rows_hint=hint, tiled=tiled)
     out = bits(ops.moe_combine(y, rpos, w, xg.clone()))
     same_routes = np.array_equal(idx.cpu().numpy(), oidx)
     assert same_routes, "router near-tie flipped an expert; pick another seed"
+    # every stage against the oracle: the SwiGLU'd gate|up rows (route-sorted on the GPU) ...
+    pos = rpos.cpu().numpy()
+    hb = bits(h)[pos]
+    assert close_to_oracle(oracle, hb, act_ref, rel=2.0 ** -6)
+    assert (ulp_diff(hb, act_ref) <= 1).mean() > 0.97
+    # ... the down projection of each route ...
+    yb = bits(y)[pos]
+    assert close_to_oracle(oracle, yb, yr, rel=2.0 ** -6)
+    assert (ulp_diff(yb, yr) <= 1).mean() > 0.95
+    # ... and the combined block
     assert close_to_oracle(oracle, out, ref, rel=2.0 ** -6)
     assert (ulp_diff(out, ref) <= 1).mean() > 0.97
+    return dict(xg=xg, rtok=rtok, offs=offs, gu=(gu_qi, gu_si), dn=(dn_qg, dn_sg), hint=hint,
+                gu_q=gu_q, gu_s=gu_s, dn_q=dn_q, dn_s=dn_s, oidx=oidx, rpos=pos)
+
+
+def test_expert_block_at_c5_expert_shape(gpu, oracle):
+    """H 2048, expert FFN 768, 32 of the 128 experts, top-4, through the row-major entry."""
+    _expert_block(gpu, oracle, 520, T=48, E=32, K=4, tiled=False)
+
+
+def test_expert_block_at_c5_full_routing_through_the_tile_major_kernels(gpu, oracle):
+    """The Qwen3-30B-A3B decode batch as the driver runs it: 64 tokens, 128 experts, top-8,
+    H 2048, expert FFN 768, fp8 e4m3 with bf16 row scales, tile-major weights — gate|up through
+    the block-shared grouped kernel, down through the wave-private grouped kernel over K = 768
+    (six 128-blocks) — every stage against the oracle, then exactness of single weights."""
+    import torch
+    from pie_amd import ops
+
+    T, E, K, H, Ie = 64, 128, 8, 2048, 768
+    st = _expert_block(gpu, oracle, 521, T=T, E=E, K=K, tiled=True)
+    # one-hot activation rows reproduce single dequantised weights bit for bit (operand layouts
+    # of both grouped kernels): route r of expert e reads a row that is 1 at column c_r
+    rng = np.random.default_rng(522)
+    offs = st["offs"].cpu().numpy()
+    routes = int(offs[-1])
+    expert_of = np.repeat(np.arange(E), np.diff(offs))
+    # down: K = Ie
+    cols = rng.integers(0, Ie, routes)
+    a = np.zeros((routes, Ie), np.float32)
+    a[np.arange(routes), cols] = 1.0
+    y = bits(ops.moe_grouped_gemm(dev(oracle.f32_to_bf16(a), gpu, torch.bfloat16), None, st["offs"], "fp8",
+                                  st["dn"][0], st["dn"][1], H, Ie, rows_hint=st["hint"], tiled=True))
+    dn_q = st["dn_q"].reshape(E, H, Ie)
+    dn_s = oracle.bf16_to_f32(st["dn_s"].reshape(E, H))
+    want = oracle.f32_to_bf16(oracle.fp8_decode(dn_q[expert_of, :, cols]) * dn_s[expert_of])
+    # (compared as values: a weight code of -0 gives -0 here and +0 from an accumulator that starts at +0)
+    assert np.array_equal(oracle.bf16_to_f32(y), oracle.bf16_to_f32(want))
+    # gate|up without SwiGLU: K = H, rows gathered by route
+    cols = rng.integers(0, H, T)
+    a = np.zeros((T, H), np.float32)
+    a[np.arange(T), cols] = 1.0
+    g = bits(ops.moe_grouped_gemm(dev(oracle.f32_to_bf16(a), gpu, torch.bfloat16), st["rtok"], st["offs"],
+                                  "fp8", st["gu"][0], st["gu"][1], 2 * Ie, H, rows_hint=st["hint"],
+                                  tiled=True))
+    perm = np.empty(2 * Ie, np.int64)
+    perm[0::2], perm[1::2] = np.arange(Ie), np.arange(Ie) + Ie
+    gu_q = st["gu_q"].reshape(E, 2 * Ie, H)[:, perm]
+    gu_s = oracle.bf16_to_f32(st["gu_s"].reshape(E, 2 * Ie)[:, perm])
+    tok = st["rtok"].cpu().numpy()
+    want = oracle.f32_to_bf16(oracle.fp8_decode(gu_q[expert_of, :, cols[tok]]) * gu_s[expert_of])
+    assert np.array_equal(oracle.bf16_to_f32(g), oracle.bf16_to_f32(want))

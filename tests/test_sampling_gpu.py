@@ -168,3 +168,33 @@ def test_special_samplers_match_oracle(gpu, oracle, V):
     assert abs(values[indptr[4]] - oracle.entropy(lg[4])) < 2e-5 * max(1.0, oracle.entropy(lg[4]))
     with pytest.raises(ops.KernelError):
         ops.sample(f32[:1], ["logprob"], [1.0], [0], [1.0], [0.0], [0.0], out_counts=[1], labels=[[V]])
+
+
+@pytest.mark.parametrize("slots", [1, 3])
+def test_multinomial_draw_exactly_on_a_part_boundary(gpu, oracle, slots):
+    """The many-block front end picks the part from the parts' sums and walks inside it.  Rows
+    whose probabilities are exact binary fractions (64 equal logits, everything else masked to
+    -inf) make every cumulative sum exact, so a uniform placed exactly on the cumulative mass at
+    the end of a part must yield the first allowed token of the following part (rule: first
+    index whose running sum exceeds u) — never a masked token, never the greedy fallback."""
+    import torch
+    from pie_amd import ops
+
+    V, parts = 32768, 32
+    seg = V // parts
+    allowed = np.sort(np.concatenate([np.arange(parts) * seg + 5, np.arange(parts) * seg + seg - 3]))
+    lg = np.full((slots, V), -np.inf, np.float32)
+    lg[:, allowed] = 1.5
+    f32 = dev(lg, gpu)
+    cases = [(j, 2 * j / 64.0) for j in (1, 7, 31)] + [(None, 0.0), (None, 63.0 / 64.0), (None, 13.0 / 64.0)]
+    for j, u in cases:
+        uu = np.full(slots, u, np.float32)
+        tok = ops.sample(f32, ["multinomial"] * slots, np.ones(slots, np.float32), np.zeros(slots, np.uint32),
+                         np.ones(slots, np.float32), np.zeros(slots, np.float32), uu)[0]
+        got = tok.cpu().numpy().view(np.uint32)
+        want = allowed[int(np.floor(u * 64.0 + 1e-9))]      # cumulative (m + 1)/64 first exceeds u
+        if j is not None:
+            assert want == j * seg + 5                       # the first allowed token of part j
+        assert np.all(got == want), (u, got, want)
+        ref, _ = oracle.sample_token(lg[0], "multinomial", 1.0, 0, 1.0, 0.0, u=float(u))
+        assert ref == want
