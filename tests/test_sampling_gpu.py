@@ -198,3 +198,45 @@ def test_multinomial_draw_exactly_on_a_part_boundary(gpu, oracle, slots):
         assert np.all(got == want), (u, got, want)
         ref, _ = oracle.sample_token(lg[0], "multinomial", 1.0, 0, 1.0, 0.0, u=float(u))
         assert ref == want
+
+
+@pytest.mark.parametrize("V", [32000, 128256])
+def test_tokens_against_the_reference_build(gpu, oracle, V):
+    """The device samplers against the reference's own sample_token, compiled from its sources
+    (oracle/_ref): every draw must name the reference's token, another member of its group of
+    bit-equal probabilities (the reference's sort leaves their order open), or — for draws
+    whose deciding comparison lies within TOL of flipping — a neighbouring token; the three
+    counts are printed."""
+    import torch
+    from oracle import ref
+    from pie_amd import ops
+
+    if ref.lib() is None:
+        pytest.skip("no prebuilt oracle/_ref library on this machine")
+    rng = np.random.default_rng(930 + V)
+    S = 192 if V < 100000 else 64
+    bits, lg = make_logits(oracle, rng, S, V, rng.choice([2.0, 3.0, 5.0, 8.0], size=S))
+    kinds, temp, top_k, top_p, min_p, seeds = random_slots(rng, S)
+    u = np.array([oracle.pcg32_first_uniform(int(s)) for s in seeds], np.float32)
+    f32 = ops.sample_gather_logits(dev(bits, gpu, torch.bfloat16))
+    got = np.concatenate([ops.sample(f32[i:i + 64], kinds[i:i + 64], temp[i:i + 64], top_k[i:i + 64],
+                                     top_p[i:i + 64], min_p[i:i + 64], u[i:i + 64])[0].cpu().numpy().view(np.uint32)
+                          for i in range(0, S, 64)])
+    same = tie = near = 0
+    for s in range(S):
+        want = ref.sample_token(lg[s], kinds[s], float(temp[s]), int(top_k[s]), float(top_p[s]),
+                                float(min_p[s]), int(seeds[s]))
+        if got[s] == want:
+            same += 1
+            continue
+        pr = oracle.softmax_temperature(lg[s], float(temp[s]))
+        if pr[got[s]] == pr[want]:
+            tie += 1
+            continue
+        _, margin = oracle.sample_token(lg[s], kinds[s], float(temp[s]), int(top_k[s]), float(top_p[s]),
+                                        float(min_p[s]), u=float(u[s]))
+        assert margin <= TOL, (s, kinds[s], temp[s], top_k[s], top_p[s], min_p[s], got[s], want, margin)
+        near += 1
+    print(f"V {V}: {same} draws equal to the reference's token, {tie} on another member of a group of equal "
+          f"probabilities, {near} on a neighbour inside the decision margin, of {S}")
+    assert near <= S // 16
