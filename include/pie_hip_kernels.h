@@ -282,6 +282,37 @@ int pie_hip_moe_route_opt(const uint16_t* router_logits_bf16, int32_t* topk_idx,
                       int num_tokens, int num_experts, int top_k, int renormalize, void* stream);
 
 /*
+ * A decode batch's way into the MoE block in two launches instead of four: per token the RMSNorm
+ * of its hidden row (norm_out = what pie_hip_rmsnorm stores, bit for bit), the router logits
+ * bf16(sum_k norm_out[t, k] * router[e, k]) over the bf16 router matrix [E, hidden] (fp32 sums in
+ * this kernel's own order: they may differ from a GEMM's in the last bf16 bit), pie_hip_moe_route_opt's
+ * softmax / top-k on them, then the expert-sorted layout.  router_logits may be NULL (not stored).
+ * Each token's block reads the whole router matrix through the L2: meant for batches of up to a
+ * few hundred rows.  hidden <= 8192, a multiple of 8; expert and top-k bounds as pie_hip_moe_route.
+ * Replaces rmsnorm + router gemm + topk_softmax_bf16_kernel of the reference's MoE block
+ * (driver/cuda/src/model/kimi_forward.cpp:640-700; graph form driver/portable/src/graph_common.cpp:237-283).
+ */
+int pie_hip_moe_norm_route(const uint16_t* x_bf16, const uint16_t* norm_weight_bf16, float eps,
+                           const uint16_t* router_bf16, uint16_t* norm_out_bf16,
+                           uint16_t* router_logits_bf16, int32_t* topk_idx, float* topk_weight,
+                           int32_t* expert_offsets, int32_t* route_token, int32_t* route_pos,
+                           int num_tokens, int hidden, int num_experts, int top_k, int renormalize,
+                           void* stream);
+
+/*
+ * pie_hip_moe_combine with add = 1 followed by pie_hip_rmsnorm of the updated rows with the next
+ * layer's norm weight, in one launch and with both results bit-identical to the two:
+ * out[t, :] = bf16(out[t, :] + sum_k w[t, k] * y_routes[route_pos[t, k], :]),
+ * norm_out[t, :] = rmsnorm(out[t, :]) * norm_weight.  hidden <= 8192, a multiple of 8.
+ * Reference: token_batched_weighted_sum_add_bf16_kernel (driver/cuda/src/kernels/moe_dispatch.cu:152-196)
+ * + rmsnorm_bf16_kernel (driver/cuda/src/kernels/rmsnorm.cu:14-54).
+ */
+int pie_hip_moe_combine_norm(const uint16_t* y_routes_bf16, const int32_t* route_pos,
+                             const float* topk_weight, uint16_t* out_bf16,
+                             const uint16_t* norm_weight_bf16, float eps, uint16_t* norm_out_bf16,
+                             int num_tokens, int top_k, int hidden, void* stream);
+
+/*
  * MoE combine: out[t, :] = bf16( (add ? out[t, :] : 0) + sum_k topk_weight[t, k] *
  * y_routes[route_pos[t, k], :] ), fp32 sum in top-k order, one rounding —
  * token_batched_weighted_sum[_add]_bf16_kernel, driver/cuda/src/kernels/moe_dispatch.cu:152-196.

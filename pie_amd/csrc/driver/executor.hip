@@ -487,15 +487,29 @@ void Executor::alloc_kv() {
 // (driver/portable/src/graph_common.cpp:237-345; kernel-by-kernel form
 // driver/cuda/src/model/kimi_forward.cpp:662-714): norm, router GEMM, one routing kernel, two
 // grouped expert GEMMs that read every touched expert once, one combine onto the residual.
-void Executor::moe_block(const LayerWeights& w, int N, hipStream_t s) {
+void Executor::moe_block(const LayerWeights& w, int N, const uint16_t* next_norm, hipStream_t s) {
     const ModelConfig& m = model_.cfg();
     const int H = m.hidden, E = m.num_experts, K = m.top_k, Ie = m.expert_intermediate;
     const int fmt = fmt_code(w.wgu.kind);
     const int sbf = w.wgu.scale_bf16 ? 1 : 0;
+    // a decode batch: norm, router logits and top-k per token in one launch (every token's block
+    // reads the router matrix through the L2, which stops paying at a few hundred rows)
+    // (PIE_MOE_FUSED=0: the separate launches, for measurement)
+    static const bool fused_on = [] { const char* e = getenv("PIE_MOE_FUSED"); return !e || atoi(e) != 0; }();
+    if (!fused_on) next_norm = nullptr;
+    int routed = PIE_HIP_ERR_UNSUPPORTED;
+    if (fused_on && N <= kFusedRouteRows && w.router.kind == Quant::Bf16)
+        routed = pie_hip_moe_norm_route(x_, w.ffn_norm, m.rms_eps, static_cast<const uint16_t*>(w.router.data), xn_,
+                                        moe_logits_, moe_idx_, moe_w_, moe_offsets_, moe_route_token_,
+                                        moe_route_pos_, N, H, E, K, m.norm_topk ? 1 : 0, s);
+    if (routed == PIE_HIP_ERR_UNSUPPORTED) {
     PIE_KERNEL(pie_hip_rmsnorm(x_, w.ffn_norm, xn_, N, H, m.rms_eps, s));
     linear_fused(w.router, xn_, nullptr, m.rms_eps, moe_logits_, N, 0, 0, nullptr, gemm_ws_, gemm_ws_bytes_, s);
     PIE_KERNEL(pie_hip_moe_route_opt(moe_logits_, moe_idx_, moe_w_, moe_offsets_, moe_route_token_,
                                      moe_route_pos_, N, E, K, m.norm_topk ? 1 : 0, s));
+    } else {
+        PIE_KERNEL(routed);
+    }
     const int hint = std::max(1, std::min(N, 2 * ((N * K + E - 1) / E)));
     // experts stacked along the rows: the tile-major copy of the stack keeps expert e at the same
     // byte stride (every expert has a multiple of 16 rows)
@@ -508,10 +522,21 @@ void Executor::moe_block(const LayerWeights& w, int N, hipStream_t s) {
                        act_, 2 * Ie, H, 1, s));
     PIE_KERNEL(grouped(fmt, act_, nullptr, moe_offsets_, E, hint, wptr(w.wdown), w.wdown.data_bytes() / E,
                        sptr(w.wdown), w.wdown.scale_bytes() / E, sbf, w.wdown.group, moe_y_, H, Ie, 0, s));
-    PIE_KERNEL(pie_hip_moe_combine(moe_y_, moe_route_pos_, moe_w_, x_, N, K, H, 1, s));
+    // with the next layer's attention norm riding along when that layer takes its rows normalised
+    int combined = PIE_HIP_ERR_UNSUPPORTED;
+    if (next_norm)
+        combined = pie_hip_moe_combine_norm(moe_y_, moe_route_pos_, moe_w_, x_, next_norm, m.rms_eps, xn_, N, K, H, s);
+    if (combined == PIE_HIP_ERR_UNSUPPORTED) {
+        PIE_KERNEL(pie_hip_moe_combine(moe_y_, moe_route_pos_, moe_w_, x_, N, K, H, 1, s));
+        xn_holds_next_norm_ = false;
+    } else {
+        PIE_KERNEL(combined);
+        xn_holds_next_norm_ = true;
+    }
 }
 
 void Executor::body(int N, int S, int max_kv_len) {
+    xn_holds_next_norm_ = false;
     const Inputs in_ = input_layout(N, S);
     const ModelConfig& m = model_.cfg();
     const int H = m.hidden, d = m.head_dim, hq = m.q_heads, hk = m.kv_heads;
@@ -536,10 +561,14 @@ void Executor::body(int N, int S, int max_kv_len) {
         const bool kvq = kv_format_ != PIE_HIP_KV_BF16;
         float* ksc = kvq && !k_scale_pool_.empty() ? k_scale_pool_[l] : nullptr;
         float* vsc = kvq && !v_scale_pool_.empty() ? v_scale_pool_[l] : nullptr;
+        // (the previous layer's MoE combine may have left this layer's normalised rows in xn_)
+        const bool prenormed = xn_holds_next_norm_;
+        xn_holds_next_norm_ = false;
         if (kvq) {
             // one-byte pools: the rotated K / V rows of this step are staged as bf16 rows (row t
             // in "slot" t) and quantised into the tokens' real slots
-            linear_fused(w.wqkv, x_, w.attn_norm, m.rms_eps, qkv_, N, 0, 0, xn_, gemm_ws_, gemm_ws_bytes_, s);
+            linear_fused(w.wqkv, prenormed ? xn_ : x_, prenormed ? nullptr : w.attn_norm, m.rms_eps, qkv_, N, 0, 0, xn_,
+                         gemm_ws_, gemm_ws_bytes_, s);
             // rotation and quantising write in one launch; head dims past 256 take the two kernels
             const int st = pie_hip_qkv_rope_kvwrite_quant(kv_format_, qkv_, q_, k_pool_[l], v_pool_[l], ksc, vsc,
                                                           w.q_norm, w.k_norm, rope_tab_, slots, N, hq, hk, d,
@@ -579,7 +608,8 @@ void Executor::body(int N, int S, int max_kv_len) {
                 else if (st != PIE_HIP_ERR_UNSUPPORTED) PIE_KERNEL(st);
             }
             if (!done) {
-                linear_fused(w.wqkv, x_, w.attn_norm, m.rms_eps, qkv_, N, 0, 0, xn_, gemm_ws_, gemm_ws_bytes_, s);
+                linear_fused(w.wqkv, prenormed ? xn_ : x_, prenormed ? nullptr : w.attn_norm, m.rms_eps, qkv_, N, 0, 0,
+                             xn_, gemm_ws_, gemm_ws_bytes_, s);
                 PIE_KERNEL(pie_hip_qkv_rope_kvwrite(qkv_, q_, k_pool_[l], v_pool_[l], w.q_norm, w.k_norm,
                                                     rope_tab_, slots, N, hq, hk, d, pairing, m.rms_eps, s));
             }
@@ -625,7 +655,10 @@ void Executor::body(int N, int S, int max_kv_len) {
         }
         linear_fused(w.wo, attn_, nullptr, m.rms_eps, x_, N, 1, 0, xn_, gemm_ws_, gemm_ws_bytes_, s);
         if (model_.is_moe()) {
-            moe_block(w, N, s);
+            // the next layer's rows come normalised when that layer runs the plain projection
+            // (q/k norm: no fused RoPE epilogue) on more than the GEMV's four rows
+            const bool next_plain = l + 1 < m.layers && N > 4 && model_.layers[l + 1].q_norm != nullptr;
+            moe_block(w, N, next_plain ? model_.layers[l + 1].attn_norm : nullptr, s);
             continue;
         }
         linear_fused(w.wgu, x_, w.ffn_norm, m.rms_eps, act_, N, 0, 1, xn_, gemm_ws_, gemm_ws_bytes_, s);

@@ -102,7 +102,9 @@ class Executor {
     void prepare_samplers(const BatchPlan& plan);
     void enqueue_samplers();
     void collect_samplers(const BatchPlan& plan, SampleOutputs& out);
-    void moe_block(const LayerWeights& w, int N, hipStream_t s);
+    void moe_block(const LayerWeights& w, int N, const uint16_t* next_norm, hipStream_t s);
+    static constexpr int kFusedRouteRows = 256;   // batches up to this size take pie_hip_moe_norm_route
+    bool xn_holds_next_norm_ = false;             // (while a forward is being enqueued) xn_ = the coming layer's normalised rows
     void alloc_kv();
     void tune_linears();
 

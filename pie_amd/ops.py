@@ -510,6 +510,52 @@ def moe_combine(y_routes: torch.Tensor, route_pos: torch.Tensor, topk_w: torch.T
     return out
 
 
+def moe_combine_norm(y_routes: torch.Tensor, route_pos: torch.Tensor, topk_w: torch.Tensor,
+                     out: torch.Tensor, norm_weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """moe_combine onto `out` (in place) and the RMSNorm of the updated rows in one launch;
+    returns the normalised rows."""
+    for n, t, dt in (("y_routes", y_routes, torch.bfloat16), ("route_pos", route_pos, torch.int32),
+                     ("topk_w", topk_w, torch.float32), ("out", out, torch.bfloat16),
+                     ("norm_weight", norm_weight, torch.bfloat16)):
+        _dev(t, dt, n)
+    T, K = topk_w.shape
+    H = y_routes.shape[1]
+    if tuple(out.shape) != (T, H) or norm_weight.numel() != H:
+        raise KernelError("shape mismatch")
+    xn = torch.empty_like(out)
+    _check(kernels().pie_hip_moe_combine_norm(_ptr(y_routes), _ptr(route_pos), _ptr(topk_w), _ptr(out),
+                                              _ptr(norm_weight), C.c_float(eps), _ptr(xn), T, K, H, _stream()),
+           "pie_hip_moe_combine_norm")
+    return xn
+
+
+def moe_norm_route(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, router: torch.Tensor, top_k: int,
+                   renormalize: bool = True):
+    """RMSNorm of the rows, router logits, softmax -> top-k and the expert-sorted layout for a
+    decode batch.  Returns (xn [T,H], logits [T,E] bf16, topk_idx, topk_w, expert_offsets,
+    route_token, route_pos) as `moe_route` does."""
+    _dev(x, torch.bfloat16, "x")
+    _dev(norm_weight, torch.bfloat16, "norm_weight")
+    _dev(router, torch.bfloat16, "router")
+    T, H = x.shape
+    E = router.shape[0]
+    if router.shape[1] != H or norm_weight.numel() != H:
+        raise KernelError("shape mismatch")
+    d = x.device
+    xn = torch.empty_like(x)
+    logits = torch.empty((T, E), dtype=torch.bfloat16, device=d)
+    idx = torch.empty((T, top_k), dtype=torch.int32, device=d)
+    w = torch.empty((T, top_k), dtype=torch.float32, device=d)
+    offs = torch.empty(E + 1, dtype=torch.int32, device=d)
+    rtok = torch.empty(T * top_k, dtype=torch.int32, device=d)
+    rpos = torch.empty(T * top_k, dtype=torch.int32, device=d)
+    _check(kernels().pie_hip_moe_norm_route(_ptr(x), _ptr(norm_weight), C.c_float(eps), _ptr(router), _ptr(xn),
+                                            _ptr(logits), _ptr(idx), _ptr(w), _ptr(offs), _ptr(rtok), _ptr(rpos),
+                                            T, H, E, top_k, int(renormalize), _stream()),
+           "pie_hip_moe_norm_route")
+    return xn, logits, idx, w, offs, rtok, rpos
+
+
 def gemm_mfma(act: torch.Tensor, w: WeightView, y: Optional[torch.Tensor] = None, beta: int = 0,
               swiglu: bool = False, split_k: bool = False,
               workspace: Optional[torch.Tensor] = None) -> torch.Tensor:

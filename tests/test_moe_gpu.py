@@ -57,6 +57,59 @@ def test_combine_is_bit_exact(gpu, oracle, add):
     assert np.array_equal(got, ref)
 
 
+@pytest.mark.parametrize("T,H,E,K", [(64, 2048, 128, 8), (1, 2048, 128, 8), (5, 512, 6, 2), (200, 4096, 64, 6),
+                                     (17, 7168, 384, 8)])
+def test_norm_route_in_one_launch(gpu, oracle, T, H, E, K):
+    """pie_hip_moe_norm_route: the stored normalised rows are pie_hip_rmsnorm's bit for bit, the
+    router logits are the oracle's bf16 products up to the order of the fp32 sum, and given the
+    logits it stored the routing is the oracle's exactly, laid out as a counting sort."""
+    import torch
+    from pie_amd import ops
+
+    rng = np.random.default_rng(530 + T + E)
+    x = dev(oracle.f32_to_bf16(rng.standard_normal((T, H)).astype(np.float32) * 3.0), gpu, torch.bfloat16)
+    nw = dev(oracle.f32_to_bf16((1.0 + 0.2 * rng.standard_normal(H)).astype(np.float32)), gpu, torch.bfloat16)
+    router = oracle.f32_to_bf16(rng.standard_normal((E, H)).astype(np.float32) * (1.0 / np.sqrt(H)))
+    for renorm in (True, False):
+        xn, lg, idx, w, offs, rtok, rpos = ops.moe_norm_route(x, nw, 1e-6, dev(router, gpu, torch.bfloat16), K,
+                                                              renormalize=renorm)
+        assert np.array_equal(bits(xn), bits(ops.rmsnorm_bf16(x, nw, 1e-6)))
+        want = oracle.gemm_bf16(bits(xn), router, mode=0)[1]
+        assert (ulp_diff(bits(lg), want) <= 1).all() and (bits(lg) == want).mean() > 0.97
+        oidx, ow = oracle.topk_softmax(bits(lg), K, renorm=renorm)
+        idx, w, offs, rtok, rpos = (t.cpu().numpy() for t in (idx, w, offs, rtok, rpos))
+        assert np.array_equal(idx, oidx)
+        assert np.allclose(w, ow, rtol=2e-6, atol=1e-9)
+        counts = np.bincount(idx.reshape(-1), minlength=E)
+        assert np.array_equal(offs, np.concatenate([[0], np.cumsum(counts)]))
+        flat = idx.reshape(-1)
+        assert np.array_equal(np.sort(rpos), np.arange(T * K))
+        assert np.all(rpos >= offs[flat]) and np.all(rpos < offs[flat + 1])
+        assert np.array_equal(rtok[rpos], np.arange(T * K) // K)
+        # the same routing as the two-launch form gives on the same logits
+        ref = ops.moe_route(lg, K, renormalize=renorm)
+        assert np.array_equal(ref[0].cpu().numpy(), idx) and np.array_equal(ref[1].cpu().numpy(), w)
+
+
+@pytest.mark.parametrize("T,K,H", [(64, 8, 2048), (3, 2, 512), (130, 6, 8192)])
+def test_combine_with_the_next_norm_equals_the_two_launches(gpu, oracle, T, K, H):
+    import torch
+    from pie_amd import ops
+
+    rng = np.random.default_rng(540 + T)
+    y = dev(oracle.f32_to_bf16(rng.standard_normal((T * K, H)).astype(np.float32)), gpu, torch.bfloat16)
+    w = dev(rng.dirichlet(np.ones(K), T).astype(np.float32), gpu)
+    pos = dev(rng.permutation(T * K).astype(np.int32), gpu)
+    base = dev(oracle.f32_to_bf16(rng.standard_normal((T, H)).astype(np.float32)), gpu, torch.bfloat16)
+    nw = dev(oracle.f32_to_bf16((1.0 + 0.2 * rng.standard_normal(H)).astype(np.float32)), gpu, torch.bfloat16)
+    a = base.clone()
+    ops.moe_combine(y, pos, w, a)
+    an = ops.rmsnorm_bf16(a, nw, 1e-6)
+    b = base.clone()
+    bn = ops.moe_combine_norm(y, pos, w, b, nw, 1e-6)
+    assert np.array_equal(bits(a), bits(b)) and np.array_equal(bits(an), bits(bn))
+
+
 def _expert_block(gpu, oracle, seed, T, E, K, tiled, H=2048, Ie=768):
     """norm'd activations -> router -> route -> grouped gate/up (+SwiGLU) -> grouped down ->
     combine, fp8 e4m3 experts with bf16 row scales, against the oracle's per-route evaluation.
