@@ -78,14 +78,20 @@ def check_step(oracle, gpu_logit_bits, orc_logit_bits, gpu_tok, orc_tok, cos_min
     assert cosine(g, o) >= cos_min
     assert np.max(np.abs(g - o)) <= rel * np.max(np.abs(o)) + 1e-3
     top2 = np.sort(o)[-2:]
-    margin = tie * abs(top2[1]) + 1e-6
+    # a near-tie: the oracle's two best logits are closer than the measured noise between the two
+    # logit vectors can bridge — four times the rms deviation of this very row (the difference of
+    # two entries' deviations has sqrt(2) of it: 2.8 sigma) — and never more than `tie` of the best
+    # logit (2^-6 = two bf16 steps in the worst case), the bound that stood alone before
+    noise = 4.0 * float(np.sqrt(np.mean((g - o) ** 2)))
+    margin = min(tie * abs(top2[1]), noise) + 1e-6
     near_tie = router_tie or (top2[1] - top2[0]) <= margin
     if not near_tie:
         assert int(gpu_tok) == int(orc_tok)
     elif not router_tie:
         # a near-tie is not skipped: the token must be one of the tied candidates, i.e. a token
-        # whose oracle logit is within the margin of the oracle's best
-        assert o[int(gpu_tok)] >= top2[1] - margin
+        # whose oracle logit is within `tie` of the oracle's best (the two entries' own deviations
+        # can exceed the row's rms several times)
+        assert o[int(gpu_tok)] >= top2[1] - (tie * abs(top2[1]) + 1e-6)
     # the token the driver returns is the argmax of its own logits, first index on ties
     assert int(gpu_tok) == int(np.argmax(g))
     return int(near_tie)
@@ -127,7 +133,9 @@ def test_greedy_generation_matches_oracle(gpu, oracle, kw):
         # steps of the best; those rows are held to "one of the tied candidates" by check_step)
         # (MoE: a request also counts as near-tie once any token of its history had a router
         # margin at bf16 resolution; those steps are held to the looser bar, never skipped)
-        assert checks == 30 and (near <= 15 or cfg["num_experts"])
+        print(f"near-ties {near} of {checks}")
+        # (measured 0 - 6 of 30 on the dense models; the old 2^-6 bound alone gave about a third)
+        assert checks == 30 and (near <= checks // 4 or cfg["num_experts"])
     # free-running generation through the driver's own harness reproduces the oracle's
     # sequence (up to the first near-tie, if any)
     with drvmod.Driver(toml_config(**kw)) as d:
@@ -533,7 +541,8 @@ def test_generation_with_one_byte_kv_cache_matches_oracle(gpu, oracle, kw, kv_dt
         otoks, near, checks = teacher_forced_compare(oracle, drvmod, d, om, cfg, prompts, 8, **bars)
         # (the tiny model's logits are flat: most steps are near-ties at 2^-4, all of them at the
         # 4-bit format's 2^-2 — there every token is still held to the tied candidates)
-        assert checks == 16 and (near < 16 or kv_dtype in ("nvfp4", "fp4_e2m1"))
+        print(f"near-ties {near} of {checks} ({kv_dtype})")
+        assert checks == 16 and (near <= (12 if kv_dtype == "fp8_e5m2" else 8) or kv_dtype in ("nvfp4", "fp4_e2m1"))
     with drvmod.Driver(toml_config(**kw)) as d:
         gtoks, _ = d.generate(prompts[0], 8, replicate=2)
         if near == 0:
@@ -702,7 +711,8 @@ def test_small_decode_batches_match_oracle(gpu, oracle, kw, replicate):
     with drvmod.Driver(toml_config(**kw, total_pages=96)) as d:
         om, _ = oracle_model_from_driver(d, dict(cfg, total_pages=96))
         _, near, checks = teacher_forced_compare(oracle, drvmod, d, om, cfg, prompts, 6)
-        assert checks == 6 * replicate and near <= checks // 2
+        print(f"near-ties {near} of {checks}")
+        assert checks == 6 * replicate and near <= checks // 5
 
 
 @pytest.mark.parametrize("kw", [
@@ -730,8 +740,11 @@ def test_decode_batches_of_16_and_64_distinct_requests(gpu, oracle, kw, count):
         om, _ = oracle_model_from_driver(d, cfg)
         _, near, checks = teacher_forced_compare(oracle, drvmod, d, om, cfg, prompts, 4, **bars)
         assert checks == 4 * count
-        if not kw.get("kv_cache_dtype") and not cfg["num_experts"]:
-            assert near <= checks // 2
+        print(f"near-ties {near} of {checks}")
+        # (one-byte KV pools: the quantisation noise is the margin, most steps count as near-ties
+        # and are held to the tied candidates)
+        if not cfg["num_experts"] and not kw.get("kv_cache_dtype"):
+            assert near <= checks // 8
 
 
 @pytest.mark.parametrize("kw", [dict(quant="int4b8"), dict(quant="bf16", kv_cache_dtype="int8_per_token_head"),
@@ -802,7 +815,8 @@ def test_yarn_scaled_model_matches_oracle(gpu, oracle):
         assert om.cfg["rope_mscale"] == ms
         prompts = ragged_prompts(rng, cfg["vocab"], 40, 2)     # contexts beyond the original 16 positions
         _, near, checks = teacher_forced_compare(oracle, drvmod, d, om, cfg, prompts, 5)
-        assert checks == 10 and near <= 5
+        print(f"near-ties {near} of {checks}")
+        assert checks == 10 and near <= 4
 
 
 def test_start_up_warm_up_changes_no_result(gpu):
