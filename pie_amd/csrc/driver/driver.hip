@@ -488,6 +488,18 @@ extern "C" size_t pie_hip_driver_export_tensor(PieHipDriver* d, const char* name
         if (dst && cap >= sizeof(v)) std::memcpy(dst, &v, sizeof(v));
         return sizeof(v);
     }
+    if (nm == "info.tuned") {
+        // the kernel each decoder linear runs per row count, as the start-up measurement left it:
+        // int8 [4 linears (wqkv, wo, wgu, wdown)][129 row counts] of layer 0 (every layer holds the
+        // same), -1 = the cost model decides, 0 GEMV, 1 skinny GEMM, 2 tiled GEMM, 3 tiled GEMM in K shares
+        const auto& lw = d->model.layers.at(0);
+        const Linear* lins[4] = {&lw.wqkv, &lw.wo, &lw.wgu, &lw.wdown};
+        int8_t tab[4][129];
+        for (int i = 0; i < 4; ++i)
+            for (int m = 0; m <= 128; ++m) tab[i][m] = lins[i]->tuned[static_cast<size_t>(m)];
+        if (dst && cap >= sizeof(tab)) std::memcpy(dst, tab, sizeof(tab));
+        return sizeof(tab);
+    }
     if (nm == "info.rope_mscale") {   // one float
         const float v = rope_mscale(d->cfg.model);
         if (dst && cap >= sizeof(v)) std::memcpy(dst, &v, sizeof(v));
@@ -749,7 +761,13 @@ extern "C" int pie_driver_hip_run_inproc(int argc, char** argv, int install_sign
             std::signal(SIGINT, [](int) { g_stop.store(true); });
             std::signal(SIGTERM, [](int) { g_stop.store(true); });
         }
-        g_stop.store(false, std::memory_order_release);   // (signals of an earlier run)
+        {
+            // a signal of an earlier run is forgotten only when no instance is serving: a second
+            // instance that starts during a reload must not erase a SIGINT / SIGTERM the first
+            // has not seen yet
+            std::lock_guard<std::mutex> lk(g_instances_mu);
+            if (g_instances.empty()) g_stop.store(false, std::memory_order_release);
+        }
         InstanceStop stop;
         PieHipDriver driver(load_driver_config(config_path));
         warm_up(&driver);

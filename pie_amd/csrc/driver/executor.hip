@@ -383,8 +383,17 @@ void Executor::tune_linears() {
         const Linear& l0 = model_.layers[0].*(r.lin);
         if (!l0.data || !l0.data_tiled) continue;   // (without the tile-major copy the cost model's defaults stand)
         int prev = 1;
+        // llama-type layers send two to four decode rows of q|k|v to the GEMV with the RoPE
+        // epilogue whatever a measurement says (Executor::body): those rungs would decide nothing
+        const bool qkv_fused_rows = r.lin == &LayerWeights::wqkv && !model_.layers[0].q_norm &&
+                                    (m.rope_interleaved || model_.qk_rows_paired()) && (d & (d - 1)) == 0 &&
+                                    kv_format_ == PIE_HIP_KV_BF16;
         for (int M : ladder) {
             if (M > max_tokens_) break;
+            if (M <= 4 && qkv_fused_rows) {
+                prev = M;
+                continue;
+            }
             int best = -1;
             double best_t = 1e30, model_t = 1e30;
             const int by_model = model_route(l0, M, r.norm != nullptr, gemm_ws_bytes_);

@@ -848,6 +848,15 @@ def test_start_up_kernel_measurement_keeps_results_within_rounding(gpu, oracle):
         with drvmod.Driver(toml_config(tune_linears=tune)) as d:
             d.generate(prompt, 1, replicate=3)
             outs.append(oracle.bf16_to_f32(d.export_tensor("debug.logits", np.uint16)).astype(np.float64).ravel())
+            # the table the measurement left (what a deployment logs to know which kernels — and
+            # so which rounding — this process runs): per linear and row count, -1 = cost model
+            tab = d.export_tensor("info.tuned", np.int8).reshape(4, 129)
+            assert np.all((tab >= -1) & (tab <= 3))
+            if not tune:
+                assert np.all(tab == -1)
+            else:
+                # llama-type q|k|v rows 2..4 always take the GEMV with the RoPE epilogue: not measured
+                assert np.all(tab[0, 2:5] == -1) and np.all(tab[:, 5:17] == -1)
     a, b = outs
     assert a.shape == b.shape and cosine(a, b) > 0.9995
     assert np.max(np.abs(a - b)) <= 0.05 * np.max(np.abs(b)) + 1e-3
