@@ -77,6 +77,21 @@ def entropy(logits_f32) -> float:
     return float(h.value)
 
 
+def sample_token_from_topk(top_idx, top_probs, kind: str, temperature=1.0, top_k=0, top_p=1.0, min_p=0.0,
+                           seed=1) -> int:
+    """sample_token_from_topk (sampler.cpp:411-): the host finalize of the reference's batch
+    shortcut over a descending top-K list of softmaxed probabilities."""
+    idx = np.ascontiguousarray(np.asarray(top_idx, np.int32))
+    pr = np.ascontiguousarray(np.asarray(top_probs, np.float32))
+    tok = C.c_uint32(0)
+    rc = lib().ref_sample_token_from_topk(_p(idx), _p(pr), C.c_int(idx.size), C.c_int(REF_TYPE[kind]),
+                                          C.c_float(temperature), C.c_uint32(top_k), C.c_float(top_p),
+                                          C.c_float(min_p), C.c_uint32(seed), C.c_uint64(0), C.byref(tok))
+    if rc != 0:
+        raise RuntimeError("the reference's sample_token_from_topk threw")
+    return int(tok.value)
+
+
 def apply_brle_logit_mask(logits_f32, runs) -> np.ndarray:
     lg = np.array(logits_f32, np.float32, copy=True)
     r = _u32(runs)

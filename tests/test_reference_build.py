@@ -66,6 +66,58 @@ def test_sample_token_equals_the_reference_except_inside_groups_of_equal_probabi
         assert tie <= S // 20       # float32 logits rarely collide
 
 
+@pytest.mark.parametrize("scale", [8.0, 3.0, 1.0])
+def test_where_the_batch_shortcut_of_the_reference_departs_from_its_full_rule(oracle, ref, scale):
+    """For batches whose slots share one temperature the reference downloads the 256 most probable
+    tokens per slot and finishes on the host (executor.cpp:586-629, sample_token_from_topk); this
+    driver applies the full-vocabulary rule (sample_token) to every batch.  Both are the
+    reference's own code here: they give the same token whenever the full rule keeps at most 256
+    candidates (peaked rows: practically always), and differ only where the shortcut truncated —
+    counted and printed per logit scale."""
+    rng = np.random.default_rng(4150 + int(scale * 10))
+    V, S = 32000, 150
+    lg = oracle.bf16_to_f32(oracle.f32_to_bf16((rng.standard_normal((S, V)) * scale).astype(np.float32)))
+    kinds = ["top_k", "top_p", "min_p", "top_k_top_p"]
+    same = truncated = tie = 0
+    for s in range(S):
+        kind = kinds[s % 4]
+        T = float(rng.choice([0.6, 1.0]))
+        k = int(rng.choice([0, 5, 50, 200]))
+        p = float(rng.choice([0.8, 0.95]))
+        mp = float(rng.choice([0.02, 0.1]))
+        seed = int(rng.integers(1, 2 ** 32))
+        full = ref.sample_token(lg[s], kind, T, k, p, mp, seed)
+        ids, vals = ref.distribution(lg[s], T, 256)            # the reference's softmax + top-256, descending
+        short = ref.sample_token_from_topk(ids, vals, kind, T, k, p, mp, seed)
+        # how many candidates the full rule keeps (float running sums, as apply_top_p / apply_min_p)
+        pr = np.sort(oracle.softmax_temperature(lg[s], T))[::-1]
+        pr = pr[pr > 0]
+        keep = len(pr)
+        if kind in ("top_k", "top_k_top_p") and 0 < k < keep:
+            keep = k
+        if kind in ("top_p", "top_k_top_p") and p < 1.0:
+            cum = np.cumsum(pr[:keep], dtype=np.float32)
+            hit = np.nonzero(cum >= np.float32(p))[0]
+            keep = int(hit[0]) + 1 if len(hit) else keep
+        if kind == "min_p":
+            cut = int(np.sum(pr[:keep] >= np.float32(mp) * pr[0]))
+            keep = cut if cut > 0 else keep
+        if full == short:
+            same += 1
+        elif keep > 256:
+            truncated += 1
+        else:
+            # (the two paths sort with partial_sort / sort over different ranges: equal probabilities
+            # may come out in another order)
+            prob = oracle.softmax_temperature(lg[s], T)
+            assert prob[full] == prob[short], (s, kind, T, k, p, mp, keep, full, short)
+            tie += 1
+    print(f"logit scale {scale}: shortcut = full rule on {same} of {S} draws, {truncated} differ because the full "
+          f"rule keeps more than 256 candidates, {tie} inside a group of equal probabilities")
+    if scale >= 8.0:
+        assert truncated <= S // 10
+
+
 def test_temperature_zero_is_first_index_argmax(oracle, ref):
     rng = np.random.default_rng(4200)
     row = _rows(oracle, rng, 1, 5000)[0]
