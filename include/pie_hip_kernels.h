@@ -116,6 +116,27 @@ int pie_hip_linear_fused(int format, const uint16_t* act_bf16, const uint16_t* n
                          int swiglu, void* stream);
 
 /*
+ * The attention output projection of a decode step with the attention's split merge in its
+ * prologue: y[m, :] = bf16( (beta ? y[m, :] : 0) + o[m, :] . W^T ), where o[m, :] (K = num_q_heads *
+ * head_dim values) is the merged, normalised, bf16-rounded attention output of row m — computed
+ * from the partial results pie_hip_attn_rows_paged_partials left in attn_workspace with the
+ * operations of the separate merge launch in the same order, so y is bit-identical to
+ * pie_hip_attn_rows_paged followed by pie_hip_linear_fused.  One launch less per layer: the merge
+ * hides behind the projection's first weight requests.  num_splits / units_per_split: the plan
+ * pie_hip_attn_decode_plan gave for the same (num_rows = M, num_kv_heads, max_kv_len).  Takes one
+ * row with up to eight splits or two rows with up to four, K <= 4096, head_dim a power of two;
+ * otherwise PIE_HIP_ERR_UNSUPPORTED (then run pie_hip_attn_rows_paged and pie_hip_linear_fused).
+ * Reference: the split-KV merge of the decode attention (attention_flashinfer.hpp:17-24 plans it,
+ * the library merges) followed by the o_proj gemm of driver/cuda/src/model/llama_like.cpp:370-705.
+ */
+int pie_hip_linear_attn_merge_supported(int format, int M, int num_splits, int num_q_heads, int head_dim,
+                                        int group_size);   /* 1: taken, 0: PIE_HIP_ERR_UNSUPPORTED */
+int pie_hip_linear_attn_merge(int format, const void* attn_workspace, int num_splits, int units_per_split,
+                              const int32_t* row_kv_len, int num_q_heads, int head_dim, const void* weight,
+                              const void* scale, int scale_is_bf16, int group_size, uint16_t* y_bf16, int M,
+                              int N, int beta, void* stream);
+
+/*
  * The fused q|k|v projection of a decode step with RoPE and the KV-cache write in its epilogue:
  * rows of W are the q, k and v heads ([(hq + 2 hk) * d, K]); adjacent output pairs (2i, 2i+1)
  * of every q and k head are rotated by rope_table[m] (interleaved pairing,
@@ -496,6 +517,21 @@ int pie_hip_attn_decode_paged(const uint16_t* q, const uint16_t* k_pages, const 
  * decode batch as one row per request.  Workspace: pie_hip_attn_decode_workspace_bytes with
  * num_requests = num_rows.
  */
+/* How a decode attention launch over (num_rows, num_kv_heads, max_kv_len) splits its rows:
+ * units_per_split 16-token units per split, num_splits splits per row (1: no workspace, no merge). */
+int pie_hip_attn_decode_plan(int num_rows, int num_kv_heads, int max_kv_len, int* units_per_split,
+                             int* num_splits);
+/* pie_hip_attn_rows_paged (kv_format PIE_HIP_KV_BF16) / pie_hip_attn_rows_paged_kvq without the merge
+ * launch: the splits' partial results stay in the workspace — [rows, q heads, splits, head_dim] f32
+ * unnormalised outputs, then [rows, q heads, splits, 2] f32 (max, sum) in units of scale * log2(e);
+ * slots of splits past a row's own extent are left unwritten — for pie_hip_linear_attn_merge.
+ * PIE_HIP_ERR_INVALID when the plan has a single split (nothing to merge). */
+int pie_hip_attn_rows_paged_partials(int kv_format, const uint16_t* q, const void* k_pages, const void* v_pages,
+                                     const float* k_scales, const float* v_scales,
+                                     const uint32_t* kv_page_indices, const uint32_t* row_page_begin,
+                                     const int32_t* row_kv_len, int num_rows, int num_q_heads,
+                                     int num_kv_heads, int head_dim, int page_size, float sm_scale,
+                                     int max_kv_len, void* workspace, size_t workspace_bytes, void* stream);
 int pie_hip_attn_rows_paged(const uint16_t* q, const uint16_t* k_pages, const uint16_t* v_pages,
                             uint16_t* o, float* lse, const uint32_t* kv_page_indices,
                             const uint32_t* row_page_begin, const int32_t* row_kv_len,

@@ -33,7 +33,7 @@ namespace {
 
 constexpr int kAttnBlock = 256;
 constexpr int kAttnWaves = kAttnBlock / kWave;
-constexpr int kUnitTokens = 16;
+constexpr int kUnitTokens = kAttnUnitTokens;
 
 template <int CTRL>
 __device__ __forceinline__ float dpp_add(float v) {
@@ -48,24 +48,6 @@ __device__ __forceinline__ float token_lanes_sum(float v) {
     v = dpp_add<0x141>(v);  // row_half_mirror
     if (LPR == 16) v = dpp_add<0x140>(v);  // row_mirror
     return v;
-}
-
-// A query row's KV extent comes either from the wire arrays of a decode batch
-// (kv_page_indptr / kv_last_page_lens) or, when `row_len` is given, from explicit per-row
-// (first page-list entry, visible key count) pairs that a planner derived.
-struct RowExtent {
-    uint32_t pg_lo;
-    int kv_len;
-};
-__device__ __forceinline__ RowExtent row_extent(const uint32_t* __restrict__ page_indptr,
-                                                const uint32_t* __restrict__ last_lens,
-                                                const uint32_t* __restrict__ row_begin,
-                                                const int32_t* __restrict__ row_len, int r,
-                                                int ps) {
-    if (row_len) return {row_begin[r], row_len[r]};
-    const uint32_t lo = page_indptr[r];
-    const int npages = static_cast<int>(page_indptr[r + 1] - lo);
-    return {lo, npages > 0 ? (npages - 1) * ps + static_cast<int>(last_lens[r]) : 0};
 }
 
 template <int D, int GQA, int KVF = kKvBf16>
@@ -706,6 +688,10 @@ struct SplitPlan {
     int nsplit;
 };
 
+// pie_hip_attn_rows_paged_partials: the split launch alone, its partial results left in the
+// workspace for a consumer that merges them itself (set around the one dispatch call)
+thread_local bool t_defer_merge = false;
+
 // Same rule for the workspace query and the launch: aim for >= ~8 blocks per CU over the
 // whole batch, never less than one unit per wave and per block.
 SplitPlan plan_splits(int R, int hk, int max_kv_len) {
@@ -767,9 +753,10 @@ int launch_decode(const uint16_t* q, const void* k_pages, const void* v_pages,
                                last_lens, row_begin, row_len,
                                part_o, part_ml, nullptr, nullptr, mask_bits, mask_stride, hq, hk, ps, ps_shift,
                                plan.units_per_split, plan.nsplit, scale_log2e);
-            hipLaunchKernelGGL((attn_decode_merge_kernel<D>), dim3(R * hq), dim3(D), 0, stream, part_o,
-                               part_ml, page_indptr, last_lens, row_begin, row_len, o, lse, hq, ps,
-                               plan.units_per_split, plan.nsplit);
+            if (!t_defer_merge)
+                hipLaunchKernelGGL((attn_decode_merge_kernel<D>), dim3(R * hq), dim3(D), 0, stream, part_o,
+                                   part_ml, page_indptr, last_lens, row_begin, row_len, o, lse, hq, ps,
+                                   plan.units_per_split, plan.nsplit);
             return launch_status();
         }
     }
@@ -791,10 +778,11 @@ int launch_decode(const uint16_t* q, const void* k_pages, const void* v_pages,
                        dim3(kAttnBlock), 0, stream, q, k_pages, v_pages, k_scales, v_scales, page_indices, page_indptr,
                        last_lens, row_begin, row_len, part_o, part_ml, nullptr, nullptr, mask_bits,
                        mask_stride, hq, hk, ps, plan.units_per_split, plan.nsplit, scale_log2e);
-    hipLaunchKernelGGL((attn_decode_merge_kernel<D>), dim3(R * hq), dim3(D), 0, stream, part_o,
-                       part_ml, page_indptr, last_lens, row_begin, row_len, o, lse, hq, ps,
-                       plan.units_per_split,
-                       plan.nsplit);
+    if (!t_defer_merge)
+        hipLaunchKernelGGL((attn_decode_merge_kernel<D>), dim3(R * hq), dim3(D), 0, stream, part_o,
+                           part_ml, page_indptr, last_lens, row_begin, row_len, o, lse, hq, ps,
+                           plan.units_per_split,
+                           plan.nsplit);
     return launch_status();
 }
 
@@ -931,6 +919,37 @@ extern "C" int pie_hip_attn_rows_paged(const uint16_t* q, const uint16_t* k_page
                                   row_page_begin, row_kv_len, num_rows, num_q_heads, num_kv_heads,
                                   head_dim, page_size, sm_scale, max_kv_len, workspace,
                                   workspace_bytes, stream);
+}
+
+extern "C" int pie_hip_attn_decode_plan(int num_rows, int num_kv_heads, int max_kv_len, int* units_per_split,
+                                        int* num_splits) {
+    if (num_rows <= 0 || num_kv_heads <= 0 || max_kv_len < 0 || !units_per_split || !num_splits)
+        return PIE_HIP_ERR_INVALID;
+    const pie_hip::SplitPlan plan = pie_hip::plan_splits(num_rows, num_kv_heads, max_kv_len);
+    *units_per_split = plan.units_per_split;
+    *num_splits = plan.nsplit;
+    return PIE_HIP_OK;
+}
+
+extern "C" int pie_hip_attn_rows_paged_partials(int kv_format, const uint16_t* q, const void* k_pages,
+                                                const void* v_pages, const float* k_scales,
+                                                const float* v_scales, const uint32_t* kv_page_indices,
+                                                const uint32_t* row_page_begin, const int32_t* row_kv_len,
+                                                int num_rows, int num_q_heads, int num_kv_heads, int head_dim,
+                                                int page_size, float sm_scale, int max_kv_len, void* workspace,
+                                                size_t workspace_bytes, void* stream) {
+    if (!row_page_begin || !row_kv_len || !workspace || num_rows <= 0 || num_kv_heads <= 0)
+        return PIE_HIP_ERR_INVALID;
+    if (pie_hip::plan_splits(num_rows, num_kv_heads, max_kv_len).nsplit < 2) return PIE_HIP_ERR_INVALID;
+    // (the output pointer is only checked, never written: the partial results are the output)
+    pie_hip::t_defer_merge = true;
+    const int rc = pie_hip::attn_dispatch(q, k_pages, v_pages, static_cast<uint16_t*>(workspace), nullptr,
+                                          kv_page_indices, nullptr, nullptr, row_page_begin, row_kv_len, num_rows,
+                                          num_q_heads, num_kv_heads, head_dim, page_size, sm_scale, max_kv_len,
+                                          workspace, workspace_bytes, stream, nullptr, 0, kv_format, k_scales,
+                                          v_scales);
+    pie_hip::t_defer_merge = false;
+    return rc;
 }
 
 // ---------------------------------------------------------------------------------------------

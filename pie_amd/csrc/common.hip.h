@@ -125,6 +125,28 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
+// Decode attention splits a row's keys in units of this many tokens (the partial results of the
+// splits are merged by attn_decode_merge_kernel or by the output projection's prologue).
+constexpr int kAttnUnitTokens = 16;
+
+// A query row's KV extent comes either from the wire arrays of a decode batch
+// (kv_page_indptr / kv_last_page_lens) or, when `row_len` is given, from explicit per-row
+// (first page-list entry, visible key count) pairs that a planner derived.
+struct RowExtent {
+    uint32_t pg_lo;
+    int kv_len;
+};
+__device__ __forceinline__ RowExtent row_extent(const uint32_t* __restrict__ page_indptr,
+                                                const uint32_t* __restrict__ last_lens,
+                                                const uint32_t* __restrict__ row_begin,
+                                                const int32_t* __restrict__ row_len, int r,
+                                                int ps) {
+    if (row_len) return {row_begin[r], row_len[r]};
+    const uint32_t lo = page_indptr[r];
+    const int npages = static_cast<int>(page_indptr[r + 1] - lo);
+    return {lo, npages > 0 ? (npages - 1) * ps + static_cast<int>(last_lens[r]) : 0};
+}
+
 // KV storage of the pool (driver/cuda/src/kv_cache_format.hpp:11-17): bf16; one-byte e4m3 with
 // optional fp32 scales per (token, kv head) — "fp8_e4m3" stores casts, "fp8_per_token_head"
 // stores x / scale; int8 with such scales; one-byte e5m2 casts ("fp8_e5m2").  A lane still owns 8 elements of a row: 16 bytes of

@@ -77,6 +77,10 @@ struct RuntimeConfig {
     // time the candidate kernels of every decoder linear at start-up (2-4 and 17-128 rows, a few
     // tens of milliseconds) and dispatch on the measurements instead of the fitted cost model
     bool tune_linears = true;
+    // one or two decode rows: the attention output projection merges the attention's splits in
+    // its prologue where that is measured to pay (no separate merge launch; the attention output
+    // rows are then never stored)
+    bool attn_merge_proj = true;
     std::string snapshot_dir;
 };
 
@@ -270,6 +274,7 @@ inline DriverConfig parse_config_text(const std::string& text) {
                 else if (k == "tiled_weights") r.tiled_weights = to_bool(v, key);
                 else if (k == "warmup") r.warmup = to_bool(v, key);
                 else if (k == "tune_linears") r.tune_linears = to_bool(v, key);
+                else if (k == "attn_merge_proj") r.attn_merge_proj = to_bool(v, key);
                 else if (k == "snapshot_dir") r.snapshot_dir = v;
             }
         }

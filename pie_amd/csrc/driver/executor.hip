@@ -106,6 +106,21 @@ int model_route(const Linear& w, int M, bool has_norm, size_t ws_bytes) {
     return p == GemmPath::Skinny ? 1 : p == GemmPath::Tiled ? 2 : 3;
 }
 
+// (PIE_GEMV_MAX_ROWS = n: rows up to n take the GEMV, more the skinny GEMM, whatever the costs say)
+int forced_gemv_rows() {
+    static const int forced_rows = [] { const char* e = getenv("PIE_GEMV_MAX_ROWS"); return e ? atoi(e) : -1; }();
+    return forced_rows;
+}
+
+// Whether linear_fused sends M rows of this linear to the GEMV (its first choice, before any
+// refusal by the kernel).
+bool routes_to_gemv(const Linear& w, int M, bool has_norm, size_t ws_bytes) {
+    const int tuned = M <= 128 ? w.tuned[M] : -1;
+    if (tuned >= 0) return tuned == 0 && M <= 4;
+    if (forced_gemv_rows() >= 0) return M <= std::min(forced_gemv_rows(), 4);
+    return model_route(w, M, has_norm, ws_bytes) == 0;
+}
+
 // y = epilogue(rmsnorm?(act) · W^T) by the weight's storage format — the dispatcher role of
 // gemm_act_x_w (driver/cuda/src/ops/gemm.cpp:1414-1583).  Up to four rows: the weight-streaming
 // GEMV with the norm riding in its activation staging and SwiGLU in its epilogue.  More rows
@@ -120,8 +135,7 @@ bool linear_fused(const Linear& w, const uint16_t* act, const uint16_t* norm_w, 
                   size_t gemm_ws_bytes, hipStream_t s, int force = -1) {
     const int fmt = fmt_code(w.kind);
     const int sbf = w.scale_bf16 ? 1 : 0;
-    // (PIE_GEMV_MAX_ROWS = n: rows up to n take the GEMV, more the skinny GEMM, whatever the costs say)
-    static const int forced_rows = [] { const char* e = getenv("PIE_GEMV_MAX_ROWS"); return e ? atoi(e) : -1; }();
+    const int forced_rows = forced_gemv_rows();
     int tuned = force >= 0 ? force : (M <= 128 ? w.tuned[M] : -1);
     bool gemv;
     if (tuned >= 0) {
@@ -633,7 +647,35 @@ void Executor::body(int N, int S, int max_kv_len) {
         const uint16_t* kat = fp4 ? kv_shadow_k_ : k_pool_[l];
         const uint16_t* vat = fp4 ? kv_shadow_v_ : v_pool_[l];
         const bool kvq_attn = kvq && !fp4;
-        if (kvq_attn && n_tiles_ > 0 && !masked_) {
+        // One or two decode rows whose output projection runs the GEMV: the attention stops at its
+        // splits' partial results and the projection merges them while its first weights travel —
+        // one launch less per layer, but EVERY block of the projection reads all the partial results,
+        // so only where those are few: measured on the 1B shape (32 heads of 64, four splits, 32 KB)
+        // 0.573 -> 0.553 ms per step; on the 8B shape with eight splits (128 KB) the projection grows
+        // from 4.7 to 8.8 us, more than the merge launch it saves.  ([runtime] attn_merge_proj = false
+        // or PIE_ATTN_MERGE_PROJ=0 keeps the separate merge.)
+        bool merged_into_wo = false;
+        if (N <= 2 && n_tiles_ == 0 && !masked_ && cfg_.runtime.attn_merge_proj) {
+            static const bool merge_on = [] { const char* e = getenv("PIE_ATTN_MERGE_PROJ"); return !e || atoi(e) != 0; }();
+            int ups = 0, ns = 1;
+            if (merge_on && routes_to_gemv(w.wo, N, false, gemm_ws_bytes_) &&
+                pie_hip_attn_decode_plan(N, hk, max_kv_len, &ups, &ns) == PIE_HIP_OK && ns >= 2 &&
+                static_cast<size_t>(N) * hq * ns * d * sizeof(float) <= kMergeProjMaxBytes &&
+                pie_hip_linear_attn_merge_supported(fmt_code(w.wo.kind), N, ns, hq, d, w.wo.group)) {
+                PIE_KERNEL(pie_hip_attn_rows_paged_partials(kvq_attn ? kv_format_ : PIE_HIP_KV_BF16, q_,
+                                                            kvq_attn ? static_cast<const void*>(k_pool_[l]) : kat,
+                                                            kvq_attn ? static_cast<const void*>(v_pool_[l]) : vat,
+                                                            kvq_attn ? ksc : nullptr, kvq_attn ? vsc : nullptr, pages,
+                                                            row_begin, row_len, N, hq, hk, d, page_size_, -1.f,
+                                                            max_kv_len, attn_ws_, attn_ws_bytes_, s));
+                PIE_KERNEL(pie_hip_linear_attn_merge(fmt_code(w.wo.kind), attn_ws_, ns, ups, row_len, hq, d, w.wo.data,
+                                                     w.wo.scale, w.wo.scale_bf16 ? 1 : 0, w.wo.group, x_, N, w.wo.N, 1,
+                                                     s));
+                merged_into_wo = true;
+            }
+        }
+        if (merged_into_wo) {
+        } else if (kvq_attn && n_tiles_ > 0 && !masked_) {
             const auto* td = static_cast<const int32_t*>(tile_in_dev_.ptr);
             PIE_KERNEL(pie_hip_attn_prefill_tiles_kvq(kv_format_, q_, k_pool_[l], v_pool_[l], ksc, vsc, attn_,
                                                       pages, row_begin, row_len, td, td + n_tiles_, n_tiles_,
@@ -662,6 +704,7 @@ void Executor::body(int N, int S, int max_kv_len) {
                                                row_begin, row_len, N, hq, hk, d, page_size_, -1.f,
                                                max_kv_len, attn_ws_, attn_ws_bytes_, s));
         }
+        if (!merged_into_wo)
         linear_fused(w.wo, attn_, nullptr, m.rms_eps, x_, N, 1, 0, xn_, gemm_ws_, gemm_ws_bytes_, s);
         if (model_.is_moe()) {
             // the next layer's rows come normalised when that layer runs the plain projection

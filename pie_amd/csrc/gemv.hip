@@ -272,7 +272,65 @@ struct GemvArgs {
     // pairs), the others slice_q
     int slice_q, slice_r;
     int groups_per_row;   // K / G (int4), set by launch
+    // Output projection of a decode step with the attention's split merge in its prologue
+    // (mg_part_o != null, act unused): the activation row m is the merged, normalised and
+    // bf16-rounded attention output of row m, computed from the split kernel's partial results
+    // exactly as attn_decode_merge_kernel computes it.  K = mg_hq * mg_d.
+    const float* mg_part_o;      // [M, hq, nsplit, d] f32
+    const float* mg_part_ml;     // [M, hq, nsplit, 2] f32 (max, sum)
+    const int32_t* mg_row_len;   // visible keys per row
+    int mg_nsplit, mg_units_per_split, mg_hq, mg_d;
 };
+
+// attn_decode_merge_kernel's arithmetic for the eight output dimensions d0 .. d0 + 7 of one
+// (row, head), from values already in registers: po[s][0..7] the partial outputs and ml[s] the
+// (max, sum) pair of split s, ns the splits the row really has (<= NSP <= 8).  Same operations in
+// the same order — the weights exp2(m_s - max), the normaliser in the order of that kernel's
+// wave reduction (lanes s and s + 4 first, then + 2, then + 1), four interleaved accumulators
+// over the splits, one division — so the packed result is what that kernel stores, bit for bit.
+template <int NSP>
+__device__ __forceinline__ u32x4_t merge_splits(const f32x4_t (&po)[NSP][2], const f32x2_t (&ml)[NSP], int ns) {
+    float mx = -INFINITY;
+#pragma unroll
+    for (int s = 0; s < NSP; ++s) mx = s < ns ? fmaxf(mx, ml[s][0]) : mx;
+    const float safe = (mx == -INFINITY) ? 0.f : mx;
+    float w[8], lv[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+        w[s] = 0.f;
+        lv[s] = 0.f;
+        if (s < NSP) {
+            if (s < ns) {
+                w[s] = exp2f(ml[s][0] - safe);
+                lv[s] = ml[s][1] * w[s];
+            }
+        }
+    }
+    const float ls = ((lv[0] + lv[4]) + (lv[2] + lv[6])) + ((lv[1] + lv[5]) + (lv[3] + lv[7]));
+    float out[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        float acc0 = 0.f, acc1 = 0.f, acc2 = 0.f, acc3 = 0.f;
+        int done = 0;
+#pragma unroll
+        for (int b = 0; b + 4 <= NSP; b += 4) {
+            if (b + 4 <= ns) {
+                acc0 = fmaf(po[b][e >> 2][e & 3], w[b], acc0);
+                acc1 = fmaf(po[b + 1][e >> 2][e & 3], w[b + 1], acc1);
+                acc2 = fmaf(po[b + 2][e >> 2][e & 3], w[b + 2], acc2);
+                acc3 = fmaf(po[b + 3][e >> 2][e & 3], w[b + 3], acc3);
+                done = b + 4;
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < NSP; ++b)
+            if (b >= done && b < ns) acc0 = fmaf(po[b][e >> 2][e & 3], w[b], acc0);
+        const float ov = (acc0 + acc1) + (acc2 + acc3);
+        out[e] = ls > 0.f ? ov / ls : 0.f;
+    }
+    return u32x4_t{pack_bf16x2(out[0], out[1]), pack_bf16x2(out[2], out[3]), pack_bf16x2(out[4], out[5]),
+                   pack_bf16x2(out[6], out[7])};
+}
 
 // ROPE: the q|k|v epilogue (rotation + KV write); its per-lane cos / sin / slot ride with every
 // unit's loads like the residual does, so the epilogue itself issues no loads.
@@ -281,7 +339,8 @@ struct GemvArgs {
 // value min(4, 8 / M); a vector-memory instruction costs the CU's address unit sixteen cycles whatever
 // it fetches and every instruction ahead of the first weight request delays it, so short rows
 // get a prologue with no idle trips.
-template <class F, int R, int M, bool ROPE, bool GS1, int PJ>
+// MG: 0, or the most splits (4 or 8) of the attention-merge prologue (PJ = 1, no norm, no RoPE).
+template <class F, int R, int M, bool ROPE, bool GS1, int PJ, int MG = 0>
 __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
     constexpr int WPP = F::WPP, XV = F::XV;
     constexpr int kChunkK = kWave * WPP;  // weights covered by one wave-wide 16 B load
@@ -398,6 +457,33 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
     for (int m = 0; m < M; ++m) inv_rms[m] = 1.f;
     if constexpr (pre) {
         u32x4_t xr[kPreJ * M], nw[kPreJ];
+        constexpr int NSP = MG > 0 ? MG : 1;
+        f32x4_t mg_po[M][NSP][2];
+        f32x2_t mg_ml[M][NSP];
+        int mg_ns[M];
+        if constexpr (MG > 0) {
+            // every split slot of the row is requested, used or not (slots past the row's own
+            // splits repeat its last configured slot and never enter the arithmetic)
+            static_assert(PJ == 1 && !ROPE, "merge prologue: one vector per thread");
+            const int svc = min(tid, nv - 1);
+            const int dsh = __builtin_ctz(static_cast<unsigned>(a.mg_d));   // head_dim is a power of two here
+            const int head = (svc * 8) >> dsh, d0 = (svc * 8) & (a.mg_d - 1);
+#pragma unroll
+            for (int m = 0; m < M; ++m) {
+                const size_t rh = static_cast<size_t>(m) * a.mg_hq + head;
+#pragma unroll
+                for (int s = 0; s < NSP; ++s) {
+                    const size_t slot = rh * a.mg_nsplit + min(s, a.mg_nsplit - 1);
+                    const float* p = a.mg_part_o + (slot << dsh) + d0;
+                    mg_po[m][s][0] = *reinterpret_cast<const f32x4_t*>(p);
+                    mg_po[m][s][1] = *reinterpret_cast<const f32x4_t*>(p + 4);
+                    mg_ml[m][s] = *reinterpret_cast<const f32x2_t*>(a.mg_part_ml + slot * 2);
+                }
+                const int kv_len = a.mg_row_len[m];
+                const int nunits = (kv_len + kAttnUnitTokens - 1) / kAttnUnitTokens;
+                mg_ns[m] = min(a.mg_nsplit, (nunits + a.mg_units_per_split - 1) / a.mg_units_per_split);
+            }
+        } else {
 #pragma unroll
         for (int jj = 0; jj < kPreJ; ++jj) {
             const int sv = tid + jj * kBlock;
@@ -407,6 +493,7 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
                 xr[jj * M + m] = *reinterpret_cast<const u32x4_t*>(a.act + static_cast<size_t>(m) * K + svc * 8);
             if (a.norm_w) nw[jj] = *reinterpret_cast<const u32x4_t*>(a.norm_w + svc * 8);
         }
+        }
         // (the scheduling barriers keep every use of the activations behind the first weight
         // requests: left alone, the compiler masks the vectors right after their loads and so waits
         // for the activations before it has asked for a single weight)
@@ -414,6 +501,10 @@ __global__ __launch_bounds__(kBlock) void gemv_kernel(const GemvArgs a) {
 #pragma unroll
         for (int i = 0; i < kUnits; ++i) issue_next(un[i], ug[i], uc[i]);
         __builtin_amdgcn_sched_barrier(0);
+        if constexpr (MG > 0) {
+#pragma unroll
+            for (int m = 0; m < M; ++m) xr[m] = merge_splits<NSP>(mg_po[m], mg_ml[m], mg_ns[m]);
+        }
 #pragma unroll
         for (int jj = 0; jj < kPreJ; ++jj) {
             const bool in_row = tid + jj * kBlock < nv;
@@ -788,9 +879,22 @@ int launch(const GemvArgs& a_in, int waves_per_simd, hipStream_t stream) {
     constexpr int kLongJ = 8 / M < 4 ? 8 / M : 4;   // (the register prologue's reach: rows of up to 4096 * kLongJ values)
     const int nvp = nchunks * (kChunkK / 8);
     const bool short_row = nvp <= kBlock;
+    if (a.mg_part_o && (!short_row || a.rope_table || a.norm_w || a.mg_nsplit > 8 || M * (a.mg_nsplit <= 4 ? 4 : 8) > 8))
+        return PIE_HIP_ERR_UNSUPPORTED;
     auto go_j = [&](auto rope, auto one, auto pj) {
         constexpr bool kRope = decltype(rope)::value, kOne = decltype(one)::value;
         constexpr int kPj = decltype(pj)::value;
+        if constexpr (!kRope && kPj == 1 && M <= 2) {
+            // (the partial results sit in registers across the first weight requests: eight
+            // splits of one row, or four of two)
+            if (a.mg_part_o) {
+                if (a.mg_nsplit <= 4)
+                    hipLaunchKernelGGL((gemv_kernel<F, R, M, false, kOne, 1, 4>), dim3(grid), dim3(kBlock), smem, stream, a);
+                else if constexpr (M == 1)
+                    hipLaunchKernelGGL((gemv_kernel<F, R, M, false, kOne, 1, 8>), dim3(grid), dim3(kBlock), smem, stream, a);
+                return;
+            }
+        }
         if (!kRope && t_start_event && t_stop_event) {
             hipExtLaunchKernelGGL((gemv_kernel<F, R, M, kRope, kOne, kPj>), dim3(grid), dim3(kBlock),
                                   static_cast<uint32_t>(smem), stream, t_start_event, t_stop_event, 0, a);
@@ -844,7 +948,7 @@ int launch_m(int M, const GemvArgs& a, int wps, hipStream_t stream) {
 // rows_per_wave (R) in {1,2,3,4}; waves_per_simd in 1..8.  0 = pick.
 template <class F>
 int dispatch(GemvArgs a, int M, int rows_per_wave, int waves_per_simd, hipStream_t stream) {
-    if (!a.act || !a.w || !a.y || M <= 0 || a.N <= 0 || a.K <= 0) return PIE_HIP_ERR_INVALID;
+    if ((!a.act && !a.mg_part_o) || !a.w || !a.y || M <= 0 || a.N <= 0 || a.K <= 0) return PIE_HIP_ERR_INVALID;
     if (a.K % F::WPP != 0) return PIE_HIP_ERR_UNSUPPORTED;
     if (a.norm_w && a.K % 8 != 0) return PIE_HIP_ERR_UNSUPPORTED;
     if (a.swiglu && (a.N % 2 != 0 || a.beta)) return PIE_HIP_ERR_INVALID;
@@ -867,6 +971,7 @@ int dispatch(GemvArgs a, int M, int rows_per_wave, int waves_per_simd, hipStream
     if (per_m > 64 * 1024) return PIE_HIP_ERR_UNSUPPORTED;
     int mcap = static_cast<int>(64 * 1024 / per_m);
     if (mcap > 4) mcap = 4;
+    if (a.mg_part_o && M > mcap) return PIE_HIP_ERR_UNSUPPORTED;   // (the merge prologue indexes rows from 0)
     const uint16_t* act = a.act;
     uint16_t* y = a.y;
     const float* rope_table = a.rope_table;
@@ -1008,6 +1113,82 @@ extern "C" int pie_hip_linear_fused(int format, const uint16_t* act_bf16,
     using namespace pie_hip;
     GemvArgs a{act_bf16, static_cast<const u32x4_t*>(weight), nullptr, nullptr, y_bf16, N, K,
                group_size, beta, norm_weight_bf16, eps, swiglu ? 1 : 0};
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (format) {
+        case PIE_HIP_FMT_INT4B8:
+            if (!scale || group_size <= 0) return PIE_HIP_ERR_INVALID;
+            if (group_size % 32 != 0 || K % group_size != 0) return PIE_HIP_ERR_UNSUPPORTED;
+            a.gscale = static_cast<const uint16_t*>(scale);
+            return dispatch<FmtInt4>(a, M, 0, 0, st);
+        case PIE_HIP_FMT_INT8:
+            if (!scale) return PIE_HIP_ERR_INVALID;
+            a.rscale = scale;
+            return scale_is_bf16 ? dispatch<FmtInt8<true>>(a, M, 0, 0, st)
+                                 : dispatch<FmtInt8<false>>(a, M, 0, 0, st);
+        case PIE_HIP_FMT_FP8:
+            if (!scale) return PIE_HIP_ERR_INVALID;
+            a.rscale = scale;
+            return scale_is_bf16 ? dispatch<FmtFp8<true>>(a, M, 0, 0, st)
+                                 : dispatch<FmtFp8<false>>(a, M, 0, 0, st);
+        case PIE_HIP_FMT_BF16:
+            return dispatch<FmtBf16>(a, M, 0, 0, st);
+        default:
+            return PIE_HIP_ERR_INVALID;
+    }
+}
+
+namespace pie_hip {
+namespace {
+template <class F>
+bool merge_shape_ok(int M, int K, int num_splits) {
+    constexpr int kChunkK = kWave * F::WPP;
+    if (K % F::WPP != 0) return false;
+    const int nchunks = (K + kChunkK - 1) / kChunkK;
+    if (nchunks * (kChunkK / 8) > kBlock) return false;                                   // one vector per thread
+    if (static_cast<size_t>(M) * nchunks * kWave * (F::XV * 16 + 4) > 64 * 1024) return false;   // staged rows in LDS
+    return num_splits >= 2 && num_splits <= 8 && M * (num_splits <= 4 ? 4 : 8) <= 8;
+}
+}  // namespace
+}  // namespace pie_hip
+
+// Whether pie_hip_linear_attn_merge takes the shape (1) or answers PIE_HIP_ERR_UNSUPPORTED (0).
+extern "C" int pie_hip_linear_attn_merge_supported(int format, int M, int num_splits, int num_q_heads,
+                                                   int head_dim, int group_size) {
+    using namespace pie_hip;
+    if (M <= 0 || num_q_heads <= 0 || head_dim < 8 || (head_dim & (head_dim - 1)) != 0) return 0;
+    const int K = num_q_heads * head_dim;
+    switch (format) {
+        case PIE_HIP_FMT_INT4B8:
+            return group_size > 0 && group_size % 32 == 0 && K % group_size == 0 && merge_shape_ok<FmtInt4>(M, K, num_splits);
+        case PIE_HIP_FMT_INT8: return merge_shape_ok<FmtInt8<true>>(M, K, num_splits);
+        case PIE_HIP_FMT_FP8: return merge_shape_ok<FmtFp8<true>>(M, K, num_splits);
+        case PIE_HIP_FMT_BF16: return merge_shape_ok<FmtBf16>(M, K, num_splits);
+        default: return 0;
+    }
+}
+
+// The attention output projection of a decode step with the split merge of the attention in its
+// prologue: y (+)= merge(partials) . W^T, the merged rows bit-identical to attn_decode_merge_kernel's.
+extern "C" int pie_hip_linear_attn_merge(int format, const void* attn_workspace, int num_splits,
+                                         int units_per_split, const int32_t* row_kv_len, int num_q_heads,
+                                         int head_dim, const void* weight, const void* scale, int scale_is_bf16,
+                                         int group_size, uint16_t* y_bf16, int M, int N, int beta, void* stream) {
+    using namespace pie_hip;
+    if (!attn_workspace || !row_kv_len || num_splits < 2 || units_per_split <= 0 || num_q_heads <= 0 ||
+        head_dim <= 0 || M <= 0)
+        return PIE_HIP_ERR_INVALID;
+    if ((head_dim & (head_dim - 1)) != 0 || head_dim < 8) return PIE_HIP_ERR_UNSUPPORTED;
+    const int K = num_q_heads * head_dim;
+    GemvArgs a{nullptr, static_cast<const u32x4_t*>(weight), nullptr, nullptr, y_bf16, N, K, group_size, beta};
+    // the workspace layout of the split launch: partial outputs, then the (max, sum) pairs
+    const size_t n_part = static_cast<size_t>(M) * num_q_heads * num_splits;
+    a.mg_part_o = static_cast<const float*>(attn_workspace);
+    a.mg_part_ml = a.mg_part_o + n_part * head_dim;
+    a.mg_row_len = row_kv_len;
+    a.mg_nsplit = num_splits;
+    a.mg_units_per_split = units_per_split;
+    a.mg_hq = num_q_heads;
+    a.mg_d = head_dim;
     hipStream_t st = static_cast<hipStream_t>(stream);
     switch (format) {
         case PIE_HIP_FMT_INT4B8:

@@ -805,6 +805,58 @@ def attention_rows_paged(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
     return o
 
 
+def attn_decode_plan(rows: int, hk: int, max_kv_len: int):
+    """(units_per_split, num_splits) of a decode attention launch."""
+    ups, ns = C.c_int(0), C.c_int(0)
+    _check(kernels().pie_hip_attn_decode_plan(rows, hk, max_kv_len, C.byref(ups), C.byref(ns)),
+           "pie_hip_attn_decode_plan")
+    return ups.value, ns.value
+
+
+def attention_rows_paged_partials(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
+                                  kv_page_indices: torch.Tensor, row_page_begin: torch.Tensor,
+                                  row_kv_len: torch.Tensor, max_kv_len: int, fmt: str = "bf16",
+                                  k_scales: Optional[torch.Tensor] = None,
+                                  v_scales: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The split launch of `attention_rows_paged` (or `_kvq`) alone: returns the workspace holding
+    the splits' partial results, for `linear_attn_merge`."""
+    _dev(q, torch.bfloat16, "q")
+    for name, t in (("kv_page_indices", kv_page_indices), ("row_page_begin", row_page_begin),
+                    ("row_kv_len", row_kv_len)):
+        _dev(t, torch.int32, name)
+    rows, hq, d = q.shape
+    _, ps, hk, _ = k_pages.shape
+    need = attn_decode_workspace_bytes(rows, hq, hk, d, max_kv_len)
+    ws = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)
+    st = kernels().pie_hip_attn_rows_paged_partials(
+        KV_FORMATS[fmt], _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(k_scales), _ptr(v_scales),
+        _ptr(kv_page_indices), _ptr(row_page_begin), _ptr(row_kv_len), rows, hq, hk, d, ps, C.c_float(-1.0),
+        max_kv_len, _ptr(ws), C.c_size_t(need), _stream())
+    _check(st, "pie_hip_attn_rows_paged_partials")
+    return ws
+
+
+def linear_attn_merge(ws: torch.Tensor, num_splits: int, units_per_split: int, row_kv_len: torch.Tensor,
+                      hq: int, d: int, w: WeightView, y: Optional[torch.Tensor] = None,
+                      beta: int = 0) -> torch.Tensor:
+    """The output projection over the merged attention rows, merge included (one launch)."""
+    _dev(row_kv_len, torch.int32, "row_kv_len")
+    M = row_kv_len.numel()
+    if w.K != hq * d:
+        raise KernelError("weight K != hq * d")
+    if y is None:
+        if beta:
+            raise KernelError("beta=1 needs an existing y")
+        y = torch.empty((M, w.N), dtype=torch.bfloat16, device=ws.device)
+    _dev(y, torch.bfloat16, "y")
+    scale_is_bf16 = int(w.scale is not None and w.scale.dtype == torch.bfloat16)
+    st = kernels().pie_hip_linear_attn_merge(FMT[w.kind], _ptr(ws), num_splits, units_per_split, _ptr(row_kv_len),
+                                             hq, d, _ptr(w.data), _ptr(w.scale), scale_is_bf16, w.group_size,
+                                             _ptr(y), M, w.N, beta, _stream())
+    _check(st, "pie_hip_linear_attn_merge")
+    return y
+
+
 ATTN_STATIC_SCRATCH_BYTES = 16 << 20
 
 

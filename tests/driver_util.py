@@ -9,7 +9,7 @@ def toml_config(arch="llama3", hidden=512, layers=2, q_heads=8, kv_heads=2, head
                 rope_theta=500000.0, rope_factor=0.0, tie=False, seed=1234, use_graphs=True,
                 rms_eps=1e-5, num_experts=0, top_k=0, expert_intermediate=0, router_std=0.0,
                 cpu_pages=0, kv_cache_dtype="auto", warmup=True, rope_interleaved=None, sliding_window=0, model_extra="",
-                tune_linears=True):
+                tune_linears=True, attn_merge_proj=True):
     moe = "" if not num_experts else (f"num_experts = {num_experts}\ntop_k = {top_k}\n"
                                       f"expert_intermediate = {expert_intermediate}\n"
                                       f"router_std = {router_std}\n")
@@ -49,6 +49,7 @@ kv_cache_dtype = "{kv_cache_dtype}"
 use_graphs = {"true" if use_graphs else "false"}
 warmup = {"true" if warmup else "false"}
 tune_linears = {"true" if tune_linears else "false"}
+attn_merge_proj = {"true" if attn_merge_proj else "false"}
 verbose = true
 """
 

@@ -671,7 +671,8 @@ def test_last_layer_intermediates_match_oracle(gpu, oracle, kw):
     rng = np.random.default_rng(95)
     prompt = rng.integers(0, cfg["vocab"], 19)
     H, I, QD = cfg["hidden"], cfg["intermediate"], cfg["q_heads"] * cfg["head_dim"]
-    with drvmod.Driver(toml_config(**kw)) as d:
+    # (the attention rows are stored: no merge inside the output projection)
+    with drvmod.Driver(toml_config(**kw, attn_merge_proj=False)) as d:
         om, _ = oracle_model_from_driver(d, cfg)
         n, npg = len(prompt), (len(prompt) + ps - 1) // ps
         fr = (prompt, np.arange(n), np.arange(npg), [0, npg], [n - (npg - 1) * ps], [0, n])
@@ -693,6 +694,52 @@ def test_last_layer_intermediates_match_oracle(gpu, oracle, kw):
         assert len(got[k]) == len(cap[k]) and np.any(o != 0), k
         assert cosine(g, o) >= 0.9999, (k, cosine(g, o))
         assert np.max(np.abs(g - o)) <= 2.0 ** -5 * np.max(np.abs(o)) + 1e-3, k
+
+
+@pytest.mark.parametrize("kw", [dict(quant="int4b8"), dict(quant="int8", kv_cache_dtype="fp8_per_token_head"),
+                                dict(arch="qwen3", quant="bf16", head_dim=128, q_heads=4, kv_heads=1, rope_theta=1e6)],
+                         ids=["llama3-int4b8", "llama3-int8-fp8kv", "qwen3-bf16"])
+def test_output_projection_that_merges_the_attention_splits_changes_no_bit(gpu, kw):
+    """[runtime] attn_merge_proj: decode steps of one and of two rows give the same logits, bit for
+    bit, with the merge inside the output projection (the default) and as a launch of its own."""
+    from pie_amd import driver as drvmod
+
+    cfg = full_cfg(**kw)
+    ps = cfg["page_size"]
+    rng = np.random.default_rng(96)
+    prompts = [rng.integers(0, cfg["vocab"], n) for n in (37, 21)]
+    logits = {}
+    for merge in (True, False):
+        rows = []
+        with drvmod.Driver(toml_config(**kw, attn_merge_proj=merge, tune_linears=False)) as d:
+            V = cfg["vocab"]
+            pages, lens, toks = [], [], []
+            nxt = 0
+            for p in prompts:     # prefill one request at a time
+                n, npg = len(p), (len(p) + ps - 1) // ps
+                pg = np.arange(nxt, nxt + npg + 1)       # one spare page for the decode steps
+                nxt += npg + 1
+                t = int(d.forward(drvmod.ForwardFrame(p, np.arange(n), pg[:npg], [0, npg], [n - (npg - 1) * ps],
+                                                      [0, n])).tokens[0])
+                pages.append(pg)
+                lens.append(n)
+                toks.append(t)
+            for nreq in (1, 2):   # a decode step of one row, then of two
+                for _ in range(3):
+                    tk, pos, pgl, indptr, last = [], [], [], [0], []
+                    for r in range(nreq):
+                        n = lens[r]
+                        npg = (n + 1 + ps - 1) // ps
+                        tk.append(toks[r]); pos.append(n)
+                        pgl.extend(pages[r][:npg]); indptr.append(len(pgl)); last.append(n + 1 - (npg - 1) * ps)
+                    out = d.forward(drvmod.ForwardFrame(tk, pos, pgl, indptr, last, list(range(nreq + 1))))
+                    rows.append(d.export_tensor("debug.logits", np.uint16)[: nreq * V].copy())
+                    for r in range(nreq):
+                        toks[r] = int(out.tokens[r]); lens[r] += 1
+        logits[merge] = rows
+    assert len(logits[True]) == 6
+    for a, b in zip(logits[True], logits[False]):
+        assert np.any(a != 0) and np.array_equal(a, b)
 
 
 @pytest.mark.parametrize("kw", [dict(quant="int4b8"), dict(quant="fp8"),
