@@ -146,19 +146,21 @@ __global__ __launch_bounds__(kTileThreads, 2) void attn_prefill_tile_kernel(
     // scalar loads, so the vector-memory queue holds K/V loads only, in step order
     auto issue = [&](int slot, int j0) {
         const int ja = min(j0, kmax - 1), jb = min(j0 + kStepKeys - 1, kmax - 1);
+        // (the step's first page by one scalar division; a key is in it or in the next one — no
+        // division per lane, which was a fifth of the step's instructions)
         const int page_a = ja / ps;
+        const int pa_end = (page_a + 1) * ps;
         const uint32_t pid_a = __builtin_amdgcn_readfirstlane(page_indices[pg_lo + page_a]);
-        const uint32_t pid_b = __builtin_amdgcn_readfirstlane(page_indices[pg_lo + jb / ps]);
+        const uint32_t pid_b = __builtin_amdgcn_readfirstlane(page_indices[pg_lo + page_a + (jb >= pa_end ? 1 : 0)]);
         auto token_head = [&](int key) {
             const int j = min(j0 + key, kmax - 1);
-            const int page = j / ps;
-            const uint32_t pid = page == page_a ? pid_a : pid_b;
-            return (static_cast<size_t>(pid) * ps + (j - page * ps)) * hk + kvh;
+            const bool in_a = j < pa_end;
+            return (static_cast<size_t>(in_a ? pid_a : pid_b) * ps + (j - (in_a ? pa_end - ps : pa_end))) * hk + kvh;
         };
         auto token_sc = [&](int key) {   // the key's place in a scale pool
             const int j = min(j0 + key, kmax - 1);
-            const int page = j / ps;
-            return kv_scale_index(page == page_a ? pid_a : pid_b, j - page * ps, kvh, hk, ps);
+            const bool in_a = j < pa_end;
+            return kv_scale_index(in_a ? pid_a : pid_b, j - (in_a ? pa_end - ps : pa_end), kvh, hk, ps);
         };
         if constexpr (Q8) {
             int key, dc;
