@@ -651,8 +651,9 @@ void Executor::body(int N, int S, int max_kv_len) {
         // splits' partial results and the projection merges them while its first weights travel —
         // one launch less per layer, but EVERY block of the projection reads all the partial results,
         // so only where those are few: measured on the 1B shape (32 heads of 64, four splits, 32 KB)
-        // 0.573 -> 0.553 ms per step; on the 8B shape with eight splits (128 KB) the projection grows
-        // from 4.7 to 8.8 us, more than the merge launch it saves.  ([runtime] attn_merge_proj = false
+        // 0.578 -> 0.560 ms per step and on the 8B shape with four splits (64 KB, contexts below 512)
+        // 1.589 -> 1.553; with eight splits (128 KB) the projection grows from 4.7 to 8.8 us, more than
+        // the merge launch it saves (1.580 -> 1.601).  ([runtime] attn_merge_proj = false
         // or PIE_ATTN_MERGE_PROJ=0 keeps the separate merge.)
         bool merged_into_wo = false;
         if (N <= 2 && n_tiles_ == 0 && !masked_ && cfg_.runtime.attn_merge_proj) {

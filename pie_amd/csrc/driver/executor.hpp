@@ -104,7 +104,7 @@ class Executor {
     void collect_samplers(const BatchPlan& plan, SampleOutputs& out);
     void moe_block(const LayerWeights& w, int N, const uint16_t* next_norm, hipStream_t s);
     static constexpr int kFusedRouteRows = 256;   // batches up to this size take pie_hip_moe_norm_route
-    static constexpr size_t kMergeProjMaxBytes = 32 * 1024;   // partial results a merging output projection reads per block
+    static constexpr size_t kMergeProjMaxBytes = 64 * 1024;   // partial results a merging output projection reads per block
     bool xn_holds_next_norm_ = false;             // (while a forward is being enqueued) xn_ = the coming layer's normalised rows
     void alloc_kv();
     void tune_linears();
