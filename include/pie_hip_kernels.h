@@ -521,6 +521,13 @@ int pie_hip_attn_decode_paged(const uint16_t* q, const uint16_t* k_pages, const 
  * units_per_split 16-token units per split, num_splits splits per row (1: no workspace, no merge). */
 int pie_hip_attn_decode_plan(int num_rows, int num_kv_heads, int max_kv_len, int* units_per_split,
                              int* num_splits);
+/* Whether a decode attention launch without custom masks over pools of kv_format takes the chunked
+ * form instead of that grid of splits: as many blocks as the device holds at once, each with the same
+ * share of the batch's keys (one wave per kv head, the rows' keys in 16-token units cut into equal
+ * chunks), for one-byte pools when the grid would queue blocks behind one another.  The workspace
+ * query covers both forms; results agree to the rounding of the fp32 merge.  Informational (tests,
+ * profiles): 1 or 0. */
+int pie_hip_attn_decode_is_chunked(int kv_format, int num_rows, int num_kv_heads, int max_kv_len);
 /* pie_hip_attn_rows_paged (kv_format PIE_HIP_KV_BF16) / pie_hip_attn_rows_paged_kvq without the merge
  * launch: the splits' partial results stay in the workspace — [rows, q heads, splits, head_dim] f32
  * unnormalised outputs, then [rows, q heads, splits, 2] f32 (max, sum) in units of scale * log2(e);

@@ -25,6 +25,7 @@
 //   * a second, tiny kernel merges the splits (skipped when there is one split).
 #include <cstdio>
 #include <mutex>
+#include <type_traits>
 
 #include "common.hip.h"
 
@@ -307,10 +308,11 @@ __global__ __launch_bounds__(kAttnBlock) void attn_decode_split_kernel(
 // so the result keeps the accuracy of the fp32 kernel above.
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+typedef int i32x2_t __attribute__((ext_vector_type(2)));
 constexpr int kMStepKeys = 32;
 
-template <int D, int GQA, int KVF = kKvBf16, bool MASKED = false>
-__global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
+template <int D, int GQA, int KVF = kKvBf16, bool MASKED = false, bool CHUNKS = false, int NW = kAttnWaves>
+__global__ __launch_bounds__(NW * kWave, 2) void attn_decode_mfma_kernel(
     const uint16_t* __restrict__ q, const void* __restrict__ k_pages_raw,
     const void* __restrict__ v_pages_raw, const float* __restrict__ k_scales,
     const float* __restrict__ v_scales, const uint32_t* __restrict__ page_indices,
@@ -318,7 +320,9 @@ __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
     const uint32_t* __restrict__ row_begin, const int32_t* __restrict__ row_len,
     float* __restrict__ part_o, float* __restrict__ part_ml, uint16_t* __restrict__ o_direct,
     float* __restrict__ lse, const uint16_t* __restrict__ mask_bits, int mask_stride, int hq, int hk,
-    int ps, int ps_shift, int units_per_split, int nsplit, float scale_log2e) {
+    int ps, int ps_shift, int units_per_split, int nsplit, float scale_log2e, int num_rows) {
+    static_assert(!(CHUNKS && MASKED), "the chunked launch takes no custom masks");
+    static_assert(CHUNKS || NW == kAttnWaves, "the gridded launch has four waves per block");
     constexpr int KS = D / 32;                 // k steps of the first product
     constexpr int DT = D / 16;                 // d tiles of the second product
     // One-byte pools: the codes become bf16 (exactly) on the way into the wave's LDS regions, the
@@ -337,30 +341,43 @@ __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
     // touches start eight banks apart); the V^T operand of the second product comes out of
     // ds_read_b64_tr_b16, which hands lane i of a 16-lane group element i of four 16-element rows
     constexpr int VSTRIDE = D + 16;
-    __shared__ __attribute__((aligned(16))) uint16_t vs_all[kAttnWaves][kMStepKeys * VSTRIDE];
-    __shared__ __attribute__((aligned(16))) uint16_t ks_all[kAttnWaves][kMStepKeys * KSTRIDE];
-    __shared__ float sm_m[kAttnWaves][16];
-    __shared__ float sm_l[kAttnWaves][16];
-    __shared__ __attribute__((aligned(16))) float sc_all[Q8 ? kAttnWaves : 1][kWave];   // K | V scales of a step
-    static_assert(sizeof(float) * GQA * D <= sizeof(uint16_t) * kMStepKeys * VSTRIDE, "per-wave output fits its V region");
+    // One-byte pools: rows of D codes padded to D + 16 bytes, the upper sixteen V rows 128 bytes
+    // further (a 16-lane group's transposing read takes rows 4g.. and 16 + 4g..: without the
+    // offset the two land on the same banks); a lane's 8-byte K fragment reads and the
+    // transposing 8-byte V reads are then conflict-free per half wave.
+    constexpr int STRIDE8 = D + 16, VUPPER8 = 128;
+    constexpr int VREGION = Q8 ? (kMStepKeys * STRIDE8 + VUPPER8) / 2 : kMStepKeys * VSTRIDE;   // uint16 units
+    constexpr int KREGION = Q8 ? kMStepKeys * STRIDE8 / 2 : kMStepKeys * KSTRIDE;
+    static_assert(KREGION % 8 == 0, "a wave's V region starts on a 16-byte boundary");
+    __shared__ __attribute__((aligned(16))) uint16_t kv_all[NW][KREGION + VREGION];   // per wave: K region, V region
+    __shared__ float sm_m[CHUNKS ? 1 : NW][16];
+    __shared__ float sm_l[CHUNKS ? 1 : NW][16];
+    __shared__ __attribute__((aligned(16))) float sc_all[Q8 ? NW : 1][kWave];   // K | V scales of a step
+    static_assert(sizeof(float) * GQA * D <= sizeof(uint16_t) * VREGION, "per-wave output fits its V region");
 
-    const int kvh = blockIdx.x, split = blockIdx.y, r = blockIdx.z;
     const int tid = threadIdx.x, lane = tid & (kWave - 1);
     const int wv = __builtin_amdgcn_readfirstlane(tid / kWave);
     const int l16 = lane & 15, g = lane >> 4;
 
-    const RowExtent ext = row_extent(page_indptr, last_lens, row_begin, row_len, r, ps);
-    const uint32_t pg_lo = ext.pg_lo;
-    const int kv_len = ext.kv_len;
-    const int nunits = (kv_len + kUnitTokens - 1) / kUnitTokens;
-    const int u_begin = split * units_per_split;
-    if (u_begin >= nunits) return;
-    const int k_begin = u_begin * kUnitTokens;
-    const int k_end = min(min(u_begin + units_per_split, nunits) * kUnitTokens, kv_len);
+    // The (row, kv head, key range) in work.  One per block in the gridded launch; the chunked
+    // launch walks a table of them (below).
+    int kvh = 0, split = 0, r = 0, nunits = 0, k_begin = 0, k_end = 0;
+    uint32_t pg_lo = 0;
+    if constexpr (!CHUNKS) {
+        kvh = blockIdx.x, split = blockIdx.y, r = blockIdx.z;
+        const RowExtent ext = row_extent(page_indptr, last_lens, row_begin, row_len, r, ps);
+        pg_lo = ext.pg_lo;
+        const int kv_len = ext.kv_len;
+        nunits = (kv_len + kUnitTokens - 1) / kUnitTokens;
+        const int u_begin = split * units_per_split;
+        if (u_begin >= nunits) return;
+        k_begin = u_begin * kUnitTokens;
+        k_end = min(min(u_begin + units_per_split, nunits) * kUnitTokens, kv_len);
+    }
 
     // Q^T fragment: column l16 = query head l16 of this kv head's group (zero beyond GQA)
     bf16x8_t qf[KS];
-    {
+    auto load_q = [&]() {
         const bool valid = l16 < GQA;
         const uint16_t* qp = q + (static_cast<size_t>(r) * hq + kvh * GQA + (valid ? l16 : 0)) * D + 8 * g;
 #pragma unroll
@@ -369,10 +386,11 @@ __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
             if (!valid) v = u32x4_t{0u, 0u, 0u, 0u};
             qf[ks] = __builtin_bit_cast(bf16x8_t, v);
         }
-    }
+    };
+    if constexpr (!CHUNKS) load_q();
 
-    uint16_t* Vs = vs_all[wv];
-    uint16_t* Ks = ks_all[wv];
+    uint16_t* Ks = kv_all[wv];
+    uint16_t* Vs = Ks + KREGION;
     // K and V loads: whole rows, LPR adjacent lanes per key (kWave / LPR keys per instruction)
     constexpr int KPI = kWave / LPR;
     u32x4_t kreg[PF][NK], vreg[PF][NK];
@@ -381,7 +399,7 @@ __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
     // A 32-key step starts on a multiple of 16 and touches at most two pages (page_size % 16 == 0);
     // their ids come through scalar loads.  Keys past the split repeat its last key (finite
     // data; their probabilities are zero).
-    auto issue = [&](int slot, int j0) {
+    auto issue = [&](int slot, int j0, int kvh, uint32_t pg_lo, int k_end) {   // (the context of the keys requested, which in the chunked launch may be the next item's)
         const int ja = min(j0, k_end - 1);
         const int page_a = ps_shift >= 0 ? ja >> ps_shift : ja / ps;
         const int pa_end = (page_a + 1) * ps;
@@ -422,18 +440,18 @@ __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
     auto stage = [&](int slot) {
 #pragma unroll
         for (int i = 0; i < NK; ++i) {
-            const int row = lane / LPR + KPI * i, piece = (lane % LPR) * (16 / EB);
-            uint16_t* kd = &Ks[row * KSTRIDE + piece];
-            uint16_t* vd = &Vs[row * VSTRIDE + piece];
+            const int row = lane / LPR + KPI * i;
             if constexpr (!Q8) {
+                const int piece = (lane % LPR) * 8;
+                uint16_t* kd = &Ks[row * KSTRIDE + piece];
+                uint16_t* vd = &Vs[row * VSTRIDE + piece];
                 *reinterpret_cast<u32x4_t*>(kd) = kreg[slot][i];
                 *reinterpret_cast<u32x4_t*>(vd) = vreg[slot][i];
-            } else {   // 16 codes -> 16 bf16
-                const u32x4_t w = kreg[slot][i], x = vreg[slot][i];
-                *reinterpret_cast<u32x4_t*>(kd) = kv_decode_bf16<KVF>(u32x2_t{w.x, w.y});
-                *reinterpret_cast<u32x4_t*>(kd + 8) = kv_decode_bf16<KVF>(u32x2_t{w.z, w.w});
-                *reinterpret_cast<u32x4_t*>(vd) = kv_decode_bf16<KVF>(u32x2_t{x.x, x.y});
-                *reinterpret_cast<u32x4_t*>(vd + 8) = kv_decode_bf16<KVF>(u32x2_t{x.z, x.w});
+            } else {   // 16 codes, as stored
+                unsigned char* kb = reinterpret_cast<unsigned char*>(Ks) + row * STRIDE8 + (lane % LPR) * 16;
+                unsigned char* vb = reinterpret_cast<unsigned char*>(Vs) + row * STRIDE8 + (row >> 4) * VUPPER8 + (lane % LPR) * 16;
+                *reinterpret_cast<u32x4_t*>(kb) = kreg[slot][i];
+                *reinterpret_cast<u32x4_t*>(vb) = vreg[slot][i];
             }
         }
         if constexpr (Q8) sc_all[wv][lane] = sreg[slot];
@@ -444,18 +462,101 @@ __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
     for (int dt = 0; dt < DT; ++dt) acc[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     float mx = -INFINITY, lsum = 0.f;
 
-    constexpr int kStride = kAttnWaves * kMStepKeys;   // keys between two steps of one wave
+    // keys between two steps of one wave: the gridded launch deals a split's steps to its four
+    // waves in turn, a wave of the chunked launch walks its own kv head's keys alone
+    constexpr int kStride = CHUNKS ? kMStepKeys : kAttnWaves * kMStepKeys;
+
+    // ---- chunked launch: the table of this block's items and the cursor of the K/V requests ----
+    // An item is a (row, key range), worked on by all waves at once — wave w takes kv head w, so
+    // the block as a whole reads whole token rows of the pool.  A wave's requests run PF steps
+    // ahead of its arithmetic and cross from one item into the next, so it pays the wait for
+    // its first keys once.
+    constexpr int kMaxItems = 32;
+    constexpr int QV = CHUNKS ? (GQA * D * 2 + 1023) / 1024 : 1;   // 1 KiB pieces of a q tile
+    __shared__ int it_row[CHUNKS ? kMaxItems : 1], it_kb[CHUNKS ? kMaxItems : 1], it_ke[CHUNKS ? kMaxItems : 1],
+        it_pg[CHUNKS ? kMaxItems : 1], it_slot[CHUNKS ? kMaxItems : 1];
+    __shared__ int it_meta[CHUNKS ? 2 : 1];
+    __shared__ __attribute__((aligned(16))) unsigned char q_next[CHUNKS ? NW : 1][CHUNKS ? QV * 1024 : 16];
+    int n_items = 0, ci = 0, cj = 0, c_ke = 0;
+    uint32_t c_pg = 0;
+    auto cursor_load = [&]() {
+        if (ci < n_items) {
+            cj = __builtin_amdgcn_readfirstlane(it_kb[ci]);
+            c_ke = __builtin_amdgcn_readfirstlane(it_ke[ci]);
+            c_pg = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(it_pg[ci]));
+        }
+    };
+    auto issue_cursor = [&](int slot) {
+        if constexpr (CHUNKS) {
+            if (ci < n_items) {
+                issue(slot, cj, kvh, c_pg, c_ke);
+                cj += kStride;
+                if (cj >= c_ke) {
+                    ++ci;
+                    cursor_load();
+                }
+            }
+        }
+    };
+
     auto step = [&](int slot, int j0) {
         stage(slot);
         f32x4_t st[2] = {f32x4_t{0.f, 0.f, 0.f, 0.f}, f32x4_t{0.f, 0.f, 0.f, 0.f}};
+        // The fragments of a product are requested together, ahead of its first MFMA (left to
+        // itself the compiler requests each next to its use to save registers, and the wave
+        // then sits out one LDS round trip per fragment): all of them for one-byte pools (two
+        // registers each), KG k-steps at a time for bf16 pools (four each).
+        using KFrag = typename std::conditional<Q8, u32x2_t, u32x4_t>::type;
+        constexpr int KG = Q8 ? KS : (KS < 2 ? KS : 2);
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks)
+        for (int k0 = 0; k0 < KS; k0 += KG) {
+            KFrag kc[KG][2];
 #pragma unroll
-            for (int nt = 0; nt < 2; ++nt)
-                st[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                    __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const u32x4_t*>(
-                                                     &Ks[(16 * nt + l16) * KSTRIDE + 32 * ks + 8 * g])),
-                    qf[ks], st[nt], 0, 0, 0);
+            for (int ks = 0; ks < KG; ++ks)
+#pragma unroll
+                for (int nt = 0; nt < 2; ++nt) {
+                    if constexpr (!Q8)
+                        kc[ks][nt] = *reinterpret_cast<const u32x4_t*>(&Ks[(16 * nt + l16) * KSTRIDE + 32 * (k0 + ks) + 8 * g]);
+                    else
+                        kc[ks][nt] = *reinterpret_cast<const u32x2_t*>(
+                            reinterpret_cast<const unsigned char*>(Ks) + (16 * nt + l16) * STRIDE8 + 32 * (k0 + ks) + 8 * g);
+                }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int ks = 0; ks < KG; ++ks)
+#pragma unroll
+                for (int nt = 0; nt < 2; ++nt) {
+                    u32x4_t kf;
+                    if constexpr (!Q8) kf = kc[ks][nt];
+                    else kf = kv_decode_bf16<KVF>(kc[ks][nt]);   // 8 codes -> 8 bf16 (exact)
+                    st[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, kf), qf[k0 + ks], st[nt], 0, 0, 0);
+                }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // the first V^T fragments are requested here: they arrive while the softmax runs
+        constexpr int VG = Q8 ? DT : (DT < 4 ? DT : 4);
+        u32x4_t vc[VG];   // (one-byte pools use the first two words)
+        auto vfetch = [&](int d0) {
+#pragma unroll
+            for (int dd = 0; dd < VG; ++dd) {
+                const int dt = d0 + dd;
+                if constexpr (!Q8) {
+                    const uint16_t* va = &Vs[(4 * g + (l16 >> 2)) * VSTRIDE + 16 * dt + 4 * (l16 & 3)];
+                    const bf16x4_t v0 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) bf16x4_t*)(va));
+                    const bf16x4_t v1 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+                        (__attribute__((address_space(3))) bf16x4_t*)(va + 16 * VSTRIDE));
+                    vc[dd] = __builtin_bit_cast(u32x4_t, __builtin_shufflevector(v0, v1, 0, 1, 2, 3, 4, 5, 6, 7));
+                } else {
+                    const int rr = l16 >> 1;
+                    const int vrow = rr < 4 ? 4 * g + rr : 12 + 4 * g + rr;
+                    const unsigned char* va = reinterpret_cast<const unsigned char*>(Vs) + vrow * STRIDE8 + (vrow >> 4) * VUPPER8 +
+                                              16 * dt + 8 * (l16 & 1);
+                    const i32x2_t c = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) i32x2_t*)(va));
+                    vc[dd] = u32x4_t{static_cast<uint32_t>(c.x), static_cast<uint32_t>(c.y), 0u, 0u};
+                }
+            }
+        };
+        vfetch(0);
         // (one-byte pools) the scales of this lane's keys, before the slot is refilled
         f32x4_t ksc[2], vsc[2];
         if constexpr (Q8) {
@@ -466,7 +567,8 @@ __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
             }
         }
         const uint32_t vis = MASKED ? mreg[slot] : 0xFFFFFFFFu;   // bit 16nt + t: key t of unit nt visible
-        if (j0 + PF * kStride < k_end) issue(slot, j0 + PF * kStride);
+        if constexpr (CHUNKS) issue_cursor(slot);
+        else if (j0 + PF * kStride < k_end) issue(slot, j0 + PF * kStride, kvh, pg_lo, k_end);
 
         // online softmax of query l16 over this lane's keys 16nt + 4g + r
         float sv[8];
@@ -508,69 +610,229 @@ __global__ __launch_bounds__(kAttnBlock, 2) void attn_decode_mfma_kernel(
         }
         const bf16x8_t p_hi = __builtin_bit_cast(bf16x8_t, u32x4_t{hi[0], hi[1], hi[2], hi[3]});
         const bf16x8_t p_lo = __builtin_bit_cast(bf16x8_t, u32x4_t{lo[0], lo[1], lo[2], lo[3]});
+        // V^T fragment of dimension 16 dt + l16: keys 4g..4g+3 and 16+4g..16+4g+3, the order of
+        // the probabilities above.  bf16 pools: lane i of the group addresses 8 bytes of row
+        // (i / 4) at column block (i % 4) and receives element i of each of the four rows, twice.
+        // One-byte pools: the one-byte transposing read — lane i addresses 8 bytes of row (i / 2)
+        // at column block (i % 2) and receives byte i of each of the eight rows.
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-            // V^T fragment of dimension 16 dt + l16: keys 4g..4g+3 and 16+4g..16+4g+3, the order of
-            // the probabilities above.  Lane i of the group addresses 8 bytes of row (i / 4) at
-            // column block (i % 4) and receives element i of each of the four rows.
-            const uint16_t* va = &Vs[(4 * g + (l16 >> 2)) * VSTRIDE + 16 * dt + 4 * (l16 & 3)];
-            const bf16x4_t v0 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) bf16x4_t*)(va));
-            const bf16x4_t v1 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
-                (__attribute__((address_space(3))) bf16x4_t*)(va + 16 * VSTRIDE));
-            const bf16x8_t vf = __builtin_shufflevector(v0, v1, 0, 1, 2, 3, 4, 5, 6, 7);
-            acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, p_hi, acc[dt], 0, 0, 0);
-            acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, p_lo, acc[dt], 0, 0, 0);
+        for (int d0 = 0; d0 < DT; d0 += VG) {
+            if (d0 > 0) vfetch(d0);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int dd = 0; dd < VG; ++dd) {
+                bf16x8_t vf;
+                if constexpr (!Q8) vf = __builtin_bit_cast(bf16x8_t, vc[dd]);
+                else vf = __builtin_bit_cast(bf16x8_t, kv_decode_bf16<KVF>(u32x2_t{vc[dd].x, vc[dd].y}));
+                acc[d0 + dd] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, p_hi, acc[d0 + dd], 0, 0, 0);
+                acc[d0 + dd] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, p_lo, acc[d0 + dd], 0, 0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
         }
     };
 
-    const int first = k_begin + wv * kMStepKeys;
-    if (first < k_end) issue(0, first);
-    if (first + kStride < k_end) issue(1, first + kStride);
-    for (int j0 = first; j0 < k_end; j0 += PF * kStride) {
-        step(0, j0);
-        if (j0 + kStride < k_end) step(1, j0 + kStride);
-    }
-
     // this wave's result into its own LDS region (as floats), then the four waves are merged
-    lsum += __shfl_xor(lsum, 16, kWave);
-    lsum += __shfl_xor(lsum, 32, kWave);
-    float* so = reinterpret_cast<float*>(Vs);   // [GQA][D]
-    if (l16 < GQA) {
+    // into slot pidx0 + h * pstride of the partial results (or, with one split, into the output)
+    auto finish = [&](size_t pidx0, int pstride) {
+        lsum += __shfl_xor(lsum, 16, kWave);
+        lsum += __shfl_xor(lsum, 32, kWave);
+        if constexpr (CHUNKS) {
+            // (a wave owns its kv head: its partial result goes out as it stands)
+            if (l16 < GQA) {
+                const size_t pidx = pidx0 + static_cast<size_t>(l16) * pstride;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-            for (int rr = 0; rr < 4; ++rr) so[l16 * D + 16 * dt + 4 * g + rr] = acc[dt][rr];
-        if (g == 0) {
-            sm_m[wv][l16] = mx;
-            sm_l[wv][l16] = lsum;
-        }
-    }
-    __syncthreads();
-    for (int idx = tid; idx < GQA * D; idx += kAttnBlock) {
-        const int h = idx / D, dd = idx - h * D;
-        float m_all = sm_m[0][h];
-#pragma unroll
-        for (int w = 1; w < kAttnWaves; ++w) m_all = fmaxf(m_all, sm_m[w][h]);
-        const float safe = (m_all == -INFINITY) ? 0.f : m_all;
-        float ov = 0.f, ls = 0.f;
-#pragma unroll
-        for (int w = 0; w < kAttnWaves; ++w) {
-            const float a = exp2f(sm_m[w][h] - safe);
-            ov += reinterpret_cast<const float*>(vs_all[w])[h * D + dd] * a;
-            ls += sm_l[w][h] * a;
-        }
-        const int head = kvh * GQA + h;
-        const size_t rh = static_cast<size_t>(r) * hq + head;
-        if (o_direct) {
-            o_direct[rh * D + dd] = f32_to_bf16_bits(ls > 0.f ? ov / ls : 0.f);
-            if (lse && dd == 0)
-                lse[rh] = ls > 0.f ? (logf(ls) + m_all * 0.6931471805599453f) : -INFINITY;
-        } else {
-            part_o[(rh * nsplit + split) * D + dd] = ov;
-            if (dd == 0) {
-                part_ml[(rh * nsplit + split) * 2 + 0] = m_all;
-                part_ml[(rh * nsplit + split) * 2 + 1] = ls;
+                for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f32x4_t*>(&part_o[pidx * D + 16 * dt + 4 * g]) = acc[dt];
+                if (g == 0) {
+                    part_ml[pidx * 2 + 0] = mx;
+                    part_ml[pidx * 2 + 1] = lsum;
+                }
             }
+            return;
+        }
+        float* so = reinterpret_cast<float*>(Vs);   // [GQA][D]
+        if (l16 < GQA) {
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int rr = 0; rr < 4; ++rr) so[l16 * D + 16 * dt + 4 * g + rr] = acc[dt][rr];
+            if (g == 0) {
+                sm_m[wv][l16] = mx;
+                sm_l[wv][l16] = lsum;
+            }
+        }
+        __syncthreads();
+        for (int idx = tid; idx < GQA * D; idx += kAttnBlock) {
+            const int h = idx / D, dd = idx - h * D;
+            float m_all = sm_m[0][h];
+#pragma unroll
+            for (int w = 1; w < kAttnWaves; ++w) m_all = fmaxf(m_all, sm_m[w][h]);
+            const float safe = (m_all == -INFINITY) ? 0.f : m_all;
+            float ov = 0.f, ls = 0.f;
+#pragma unroll
+            for (int w = 0; w < kAttnWaves; ++w) {
+                const float a = exp2f(sm_m[w][h] - safe);
+                ov += reinterpret_cast<const float*>(kv_all[w] + KREGION)[h * D + dd] * a;
+                ls += sm_l[w][h] * a;
+            }
+            const int head = kvh * GQA + h;
+            const size_t rh = static_cast<size_t>(r) * hq + head;
+            if (o_direct) {
+                o_direct[rh * D + dd] = f32_to_bf16_bits(ls > 0.f ? ov / ls : 0.f);
+                if (lse && dd == 0)
+                    lse[rh] = ls > 0.f ? (logf(ls) + m_all * 0.6931471805599453f) : -INFINITY;
+            } else {
+                const size_t pidx = pidx0 + static_cast<size_t>(h) * pstride;
+                part_o[pidx * D + dd] = ov;
+                if (dd == 0) {
+                    part_ml[pidx * 2 + 0] = m_all;
+                    part_ml[pidx * 2 + 1] = ls;
+                }
+            }
+        }
+    };
+
+    if constexpr (!CHUNKS) {
+        const int first = k_begin + wv * kMStepKeys;
+        if (first < k_end) issue(0, first, kvh, pg_lo, k_end);
+        if (first + kStride < k_end) issue(1, first + kStride, kvh, pg_lo, k_end);
+        for (int j0 = first; j0 < k_end; j0 += PF * kStride) {
+            step(0, j0);
+            if (j0 + kStride < k_end) step(1, j0 + kStride);
+        }
+        finish((static_cast<size_t>(r) * hq + kvh * GQA) * nsplit + split, nsplit);
+    } else {
+        // ---- The chunked launch.  The keys of all rows, in 16-token units, form one line; block
+        // b takes units [b C, (b + 1) C) of it, C = the line's length over the grid, rounded up:
+        // every block the same number of keys, whatever the rows' lengths, no block waits for a
+        // slot, and the waves of a block (one per kv head) read the same tokens at the same
+        // time, i.e. whole rows of the pool.  A chunk cuts the rows it covers into items; the
+        // piece of row r inside chunk b goes to slot b + r of the partial results (along the
+        // line either b or r grows from one piece to the next, so the slots are distinct and a
+        // row's pieces are consecutive), which the merge kernel finds again from the same
+        // arithmetic.
+        const int R = num_rows, NB = gridDim.x, b = blockIdx.x;
+        kvh = wv;
+        int* row_pref = reinterpret_cast<int*>(&kv_all[0][0]);   // [R + 1] units before each row (set-up only: the first wave's regions are idle)
+        int* row_pg = row_pref + kAttnBlock + 4;
+        int* row_kl = row_pg + kAttnBlock;
+        static_assert(sizeof(kv_all[0]) >= sizeof(int) * (3 * kAttnBlock + 4), "set-up tables fit a wave's regions");
+        int pos = -1;
+        for (;;) {
+            if (wv == 0) {   // units per row and their prefix sums (again for every table: the regions held keys since)
+                int carry = 0;
+                for (int base = 0; base < R; base += kWave) {
+                    const int rr = base + lane;
+                    int n = 0;
+                    if (rr < R) {
+                        const RowExtent ext = row_extent(page_indptr, last_lens, row_begin, row_len, rr, ps);
+                        n = (ext.kv_len + kUnitTokens - 1) / kUnitTokens;
+                        row_pg[rr] = static_cast<int>(ext.pg_lo);
+                        row_kl[rr] = ext.kv_len;
+                    }
+                    int x = n;
+#pragma unroll
+                    for (int off = 1; off < kWave; off <<= 1) {
+                        const int y = __shfl_up(x, off, kWave);
+                        if (lane >= off) x += y;
+                    }
+                    if (rr < R) row_pref[rr + 1] = carry + x;
+                    carry += __shfl(x, kWave - 1, kWave);
+                }
+                if (lane == 0) row_pref[0] = 0;
+            }
+            __syncthreads();
+            if (tid == 0) {
+                const int total = row_pref[R];
+                const int C = (total + NB - 1) / NB;
+                if (pos < 0) pos = b * C;
+                const int chunk_end = min(total, (b + 1) * C);
+                int x = pos, n = 0;
+                while (x < chunk_end && n < kMaxItems) {
+                    int lo = 0, hi = R;   // the row of line position x: pref[lo] <= x < pref[hi]
+                    while (hi - lo > 1) {
+                        const int mid = (lo + hi) >> 1;
+                        if (row_pref[mid] <= x) lo = mid;
+                        else hi = mid;
+                    }
+                    const int u0 = x - row_pref[lo];
+                    const int take = min(row_pref[lo + 1] - x, chunk_end - x);
+                    it_row[n] = lo;
+                    it_kb[n] = u0 * kUnitTokens;
+                    it_ke[n] = min((u0 + take) * kUnitTokens, row_kl[lo]);
+                    it_pg[n] = row_pg[lo];
+                    it_slot[n] = b + lo;
+                    x += take;
+                    ++n;
+                }
+                it_meta[0] = n;
+                it_meta[1] = x < chunk_end ? x : -2;   // where the next table starts, if the chunk has more
+            }
+            __syncthreads();
+            n_items = __builtin_amdgcn_readfirstlane(it_meta[0]);
+            pos = __builtin_amdgcn_readfirstlane(it_meta[1]);
+            if (n_items == 0) break;
+
+            ci = 0;
+            cursor_load();
+            issue_cursor(0);
+            issue_cursor(1);
+            // The steps of all items in one sequence, alternating between the two slots of keys
+            // in flight; between two steps, where an item ends: its partial result goes out, the
+            // next one's q fragments come in.
+            int item = 0, j0 = 0, slot_out = 0;
+            auto begin_item = [&]() {
+                r = __builtin_amdgcn_readfirstlane(it_row[item]);
+                k_end = __builtin_amdgcn_readfirstlane(it_ke[item]);
+                slot_out = __builtin_amdgcn_readfirstlane(it_slot[item]);
+                j0 = __builtin_amdgcn_readfirstlane(it_kb[item]);
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) acc[dt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+                mx = -INFINITY, lsum = 0.f;
+                if (item == 0) {
+                    load_q();
+                } else {   // (parked in this wave's q_next during the item before)
+                    const bool valid = l16 < GQA;
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) {
+                        u32x4_t v = *reinterpret_cast<const u32x4_t*>(&q_next[wv][((valid ? l16 : 0) * D + 32 * ks + 8 * g) * 2]);
+                        if (!valid) v = u32x4_t{0u, 0u, 0u, 0u};
+                        qf[ks] = __builtin_bit_cast(bf16x8_t, v);
+                    }
+                }
+            };
+            auto one_step = [&](int slot) {   // false once the table is worked off
+                // during an item's last step the next item's q tile is fetched (whole 16-byte
+                // pieces, lane by lane) and parked in LDS
+                const bool last = j0 + kStride >= k_end;
+                const bool fetch_q = last && item + 1 < n_items;
+                u32x4_t qt[QV];
+                if (fetch_q) {
+                    const unsigned char* qsrc = reinterpret_cast<const unsigned char*>(
+                        q + (static_cast<size_t>(it_row[item + 1]) * hq + kvh * GQA) * D);
+#pragma unroll
+                    for (int i = 0; i < QV; ++i)
+                        qt[i] = *reinterpret_cast<const u32x4_t*>(qsrc + min(i * 1024 + lane * 16, GQA * D * 2 - 16));
+                }
+                step(slot, j0);
+                if (fetch_q) {
+#pragma unroll
+                    for (int i = 0; i < QV; ++i) *reinterpret_cast<u32x4_t*>(&q_next[wv][i * 1024 + lane * 16]) = qt[i];
+                }
+                j0 += kStride;
+                if (last) {
+                    finish((static_cast<size_t>(slot_out) * hk + kvh) * GQA, 1);
+                    if (++item >= n_items) return false;
+                    begin_item();
+                }
+                return true;
+            };
+            begin_item();
+            for (;;) {
+                if (!one_step(0)) break;
+                if (!one_step(1)) break;
+            }
+            if (pos < 0) break;
+            __syncthreads();   // every wave is through with the table before it is rebuilt
         }
     }
 }
@@ -683,6 +945,73 @@ __global__ void attn_decode_clear_empty_kernel(const uint32_t* __restrict__ page
     if (lse && threadIdx.x == 0) lse[rh] = -INFINITY;
 }
 
+// The merge of a chunked launch (attn_decode_mfma_kernel<..., CHUNKS = true>): one block per
+// (row, q head).  The block recomputes where its row lies on the line of 16-token units (the
+// units of the rows before it) and from that the chunks that cut it: their pieces sit in
+// consecutive slots of the partial results, the piece of chunk b in slot b + row, a slot
+// holding the row's q heads in order.
+template <int D>
+__global__ __launch_bounds__(D) void attn_decode_merge_chunks_kernel(
+    const float* __restrict__ part_o, const float* __restrict__ part_ml,
+    const uint32_t* __restrict__ page_indptr, const uint32_t* __restrict__ last_lens,
+    const uint32_t* __restrict__ row_begin, const int32_t* __restrict__ row_len,
+    uint16_t* __restrict__ o, float* __restrict__ lse, int hq, int ps, int R, int NB) {
+    __shared__ int s_red[3][D / kWave];
+    const int rh = blockIdx.x;
+    const int r = rh / hq, head = rh - r * hq;
+    const int dd = threadIdx.x, lane = dd & (kWave - 1), wv = dd / kWave;
+    int before = 0, total = 0, mine = 0;
+    for (int rr = dd; rr < R; rr += D) {
+        const int n = (row_extent(page_indptr, last_lens, row_begin, row_len, rr, ps).kv_len + kUnitTokens - 1) / kUnitTokens;
+        total += n;
+        if (rr < r) before += n;
+        if (rr == r) mine = n;
+    }
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+        before += __shfl_xor(before, off, kWave);
+        total += __shfl_xor(total, off, kWave);
+        mine += __shfl_xor(mine, off, kWave);
+    }
+    if (lane == 0) {
+        s_red[0][wv] = before;
+        s_red[1][wv] = total;
+        s_red[2][wv] = mine;
+    }
+    __syncthreads();
+    before = total = mine = 0;
+#pragma unroll
+    for (int w = 0; w < D / kWave; ++w) {
+        before += s_red[0][w];
+        total += s_red[1][w];
+        mine += s_red[2][w];
+    }
+    const size_t out = static_cast<size_t>(rh) * D + dd;
+    if (mine == 0) {
+        o[out] = 0;
+        if (lse && dd == 0) lse[rh] = -INFINITY;
+        return;
+    }
+    const int C = (total + NB - 1) / NB;
+    const int b_lo = before / C, b_hi = (before + mine - 1) / C;
+    const size_t slot0 = static_cast<size_t>(b_lo) + r;
+    const int ns = b_hi - b_lo + 1;
+    const float* ml = part_ml + (slot0 * hq + head) * 2;
+    const float* po = part_o + (slot0 * hq + head) * D + dd;
+    const size_t ml_step = static_cast<size_t>(hq) * 2, po_step = static_cast<size_t>(hq) * D;
+    float mx = -INFINITY;
+    for (int i = 0; i < ns; ++i) mx = fmaxf(mx, ml[i * ml_step]);
+    const float safe = (mx == -INFINITY) ? 0.f : mx;
+    float ov = 0.f, ls = 0.f;
+    for (int i = 0; i < ns; ++i) {
+        const float a = exp2f(ml[i * ml_step] - safe);
+        ov = fmaf(po[i * po_step], a, ov);
+        ls = fmaf(ml[i * ml_step + 1], a, ls);
+    }
+    o[out] = f32_to_bf16_bits(ls > 0.f ? ov / ls : 0.f);
+    if (lse && dd == 0) lse[rh] = ls > 0.f ? (logf(ls) + mx * 0.6931471805599453f) : -INFINITY;
+}
+
 struct SplitPlan {
     int units_per_split;
     int nsplit;
@@ -714,6 +1043,48 @@ SplitPlan plan_splits(int R, int hk, int max_kv_len) {
     return {static_cast<int>(ups), nsplit};
 }
 
+// The chunked launch (attn_decode_mfma_kernel<..., CHUNKS = true>): as many blocks as the device
+// holds at once, every block the same share of the batch's keys.  Taken for one-byte pools when
+// the gridded launch would queue blocks behind one another — its blocks then start and end at
+// different times, each waits for its first keys on its own, and a third of the wave slots sit
+// idle — and the batch fits the kernel's set-up.  Measured (MI355X, 64 rows of 512-8192 keys,
+// 8 kv heads of 128): fp8 / int8 pools 121 / 124 -> 102 us (0.55 -> 0.67 of the HBM peak), a
+// 64-row decode step of an 8B model over fp8 pools at 2048 keys 5.42 -> 5.03 ms.  bf16 pools keep
+// the gridded launch: it already reads at the rate the chunked one reaches (5.6 TB/s), and the
+// chunked launch measured slower there (186 -> 201 us, the same step 6.19 -> 6.64 ms).
+struct ChunkPlan {
+    bool use;
+    int blocks;
+    size_t slots;   // partial results: blocks + rows slots of hq heads each
+};
+int resident_attn_blocks() {
+    constexpr int kMaxDev = 64;
+    static std::mutex mu;
+    static int cached[kMaxDev] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDev) return 0;
+    std::lock_guard<std::mutex> lock(mu);
+    if (cached[dev] == 0) {
+        int cus = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) return 0;
+        cached[dev] = cus;
+    }
+    return cached[dev];   // (compute units)
+}
+ChunkPlan plan_chunks(int R, int hk, int max_kv_len, const SplitPlan& plan, bool one_byte_pool) {
+    static const int forced = [] { const char* e = getenv("PIE_HIP_ATTN_CHUNKS"); return e ? atoi(e) : -1; }();   // measurement hook
+    // a CU holds eight waves of the kernel (two per SIMD: its registers) = 8 / hk blocks of one
+    // wave per kv head
+    const int cus = resident_attn_blocks();
+    const bool shape = hk == 1 || hk == 2 || hk == 4 || hk == 8;
+    const int nb = shape ? cus * (8 / hk) : 0;
+    const long long max_units = (max_kv_len + kUnitTokens - 1) / kUnitTokens;
+    const bool fits = nb > 0 && R <= kAttnBlock && static_cast<long long>(R) * max_units < (1ll << 30);
+    const bool queues = static_cast<long long>(R) * hk * plan.nsplit > 2 * cus;   // more blocks than the gridded launch has resident
+    const bool use = fits && !t_defer_merge && (forced >= 0 ? forced != 0 : one_byte_pool && queues);
+    return {use, nb, static_cast<size_t>(nb) + static_cast<size_t>(R)};
+}
+
 template <int D, int GQA, bool MASKED, int KVF = kKvBf16>
 int launch_decode(const uint16_t* q, const void* k_pages, const void* v_pages,
                   const float* k_scales, const float* v_scales, uint16_t* o, float* lse, const uint32_t* page_indices, const uint32_t* page_indptr,
@@ -733,6 +1104,29 @@ int launch_decode(const uint16_t* q, const void* k_pages, const void* v_pages,
         const bool mfma = forced >= 0 ? forced == 0 : true;
         if (mfma) {
             const int ps_shift = (ps & (ps - 1)) == 0 ? __builtin_ctz(static_cast<unsigned>(ps)) : -1;
+            if constexpr (!MASKED) {
+                const ChunkPlan cp = plan_chunks(R, hk, max_kv_len, plan, KVF != kKvBf16);
+                if (cp.use) {
+                    const size_t n_part = cp.slots * hq;
+                    const size_t need = n_part * (D + 2) * sizeof(float);
+                    if (!workspace || workspace_bytes < need) return PIE_HIP_ERR_INVALID;
+                    float* part_o = static_cast<float*>(workspace);
+                    float* part_ml = part_o + n_part * D;
+#define PIE_CHUNK_LAUNCH(NWAVES)                                                                                       \
+    hipLaunchKernelGGL((attn_decode_mfma_kernel<D, GQA, KVF, false, true, NWAVES>), dim3(cp.blocks), dim3(NWAVES * kWave), \
+                       0, stream, q, k_pages, v_pages, k_scales, v_scales, page_indices, page_indptr, last_lens,       \
+                       row_begin, row_len, part_o, part_ml, nullptr, nullptr, nullptr, 0, hq, hk, ps, ps_shift, 0, 0,  \
+                       scale_log2e, R)
+                    if (hk == 8) PIE_CHUNK_LAUNCH(8);
+                    else if (hk == 4) PIE_CHUNK_LAUNCH(4);
+                    else if (hk == 2) PIE_CHUNK_LAUNCH(2);
+                    else PIE_CHUNK_LAUNCH(1);
+#undef PIE_CHUNK_LAUNCH
+                    hipLaunchKernelGGL((attn_decode_merge_chunks_kernel<D>), dim3(R * hq), dim3(D), 0, stream, part_o,
+                                       part_ml, page_indptr, last_lens, row_begin, row_len, o, lse, hq, ps, R, cp.blocks);
+                    return launch_status();
+                }
+            }
             if (plan.nsplit == 1) {
                 hipLaunchKernelGGL((attn_decode_clear_empty_kernel<D>), dim3(R * hq), dim3(D), 0, stream,
                                    page_indptr, last_lens, row_begin, row_len, o, lse, hq, ps);
@@ -740,7 +1134,7 @@ int launch_decode(const uint16_t* q, const void* k_pages, const void* v_pages,
                                    stream, q, k_pages, v_pages, k_scales, v_scales, page_indices, page_indptr,
                                    last_lens, row_begin, row_len,
                                    nullptr, nullptr, o, lse, mask_bits, mask_stride, hq, hk, ps, ps_shift,
-                                   plan.units_per_split, 1, scale_log2e);
+                                   plan.units_per_split, 1, scale_log2e, R);
                 return launch_status();
             }
             const size_t n_part = static_cast<size_t>(R) * hq * plan.nsplit;
@@ -752,7 +1146,7 @@ int launch_decode(const uint16_t* q, const void* k_pages, const void* v_pages,
                                stream, q, k_pages, v_pages, k_scales, v_scales, page_indices, page_indptr,
                                last_lens, row_begin, row_len,
                                part_o, part_ml, nullptr, nullptr, mask_bits, mask_stride, hq, hk, ps, ps_shift,
-                               plan.units_per_split, plan.nsplit, scale_log2e);
+                               plan.units_per_split, plan.nsplit, scale_log2e, R);
             if (!t_defer_merge)
                 hipLaunchKernelGGL((attn_decode_merge_kernel<D>), dim3(R * hq), dim3(D), 0, stream, part_o,
                                    part_ml, page_indptr, last_lens, row_begin, row_len, o, lse, hq, ps,
@@ -794,9 +1188,14 @@ extern "C" size_t pie_hip_attn_decode_workspace_bytes(int num_requests, int num_
                                                       int max_kv_len) {
     if (num_requests <= 0 || num_q_heads <= 0 || num_kv_heads <= 0 || head_dim <= 0) return 0;
     const pie_hip::SplitPlan plan = pie_hip::plan_splits(num_requests, num_kv_heads, max_kv_len);
-    if (plan.nsplit == 1) return 0;
-    return static_cast<size_t>(num_requests) * num_q_heads * plan.nsplit * (head_dim + 2) *
-           sizeof(float);
+    const size_t gridded = plan.nsplit == 1 ? 0
+                                            : static_cast<size_t>(num_requests) * num_q_heads * plan.nsplit *
+                                                  (head_dim + 2) * sizeof(float);
+    // (the chunked launch's partial results, where a launch over one-byte pools without custom
+    // masks would take it; bf16 pools and masked rows of the same shape keep the gridded launch)
+    const pie_hip::ChunkPlan cp = pie_hip::plan_chunks(num_requests, num_kv_heads, max_kv_len, plan, true);
+    const size_t chunked = cp.use ? cp.slots * num_q_heads * (head_dim + 2) * sizeof(float) : 0;
+    return gridded > chunked ? gridded : chunked;
 }
 
 namespace pie_hip {
@@ -919,6 +1318,12 @@ extern "C" int pie_hip_attn_rows_paged(const uint16_t* q, const uint16_t* k_page
                                   row_page_begin, row_kv_len, num_rows, num_q_heads, num_kv_heads,
                                   head_dim, page_size, sm_scale, max_kv_len, workspace,
                                   workspace_bytes, stream);
+}
+
+extern "C" int pie_hip_attn_decode_is_chunked(int kv_format, int num_rows, int num_kv_heads, int max_kv_len) {
+    if (num_rows <= 0 || num_kv_heads <= 0 || max_kv_len < 0) return 0;
+    const pie_hip::SplitPlan plan = pie_hip::plan_splits(num_rows, num_kv_heads, max_kv_len);
+    return pie_hip::plan_chunks(num_rows, num_kv_heads, max_kv_len, plan, kv_format != PIE_HIP_KV_BF16).use ? 1 : 0;
 }
 
 extern "C" int pie_hip_attn_decode_plan(int num_rows, int num_kv_heads, int max_kv_len, int* units_per_split,
@@ -1443,3 +1848,4 @@ extern "C" int pie_hip_attn_rows_paged_masked(const uint16_t* q, const uint16_t*
                                   head_dim, page_size, sm_scale, max_kv_len, workspace,
                                   workspace_bytes, stream, mask_bitmap, mask_stride_units);
 }
+

@@ -813,6 +813,12 @@ def attn_decode_plan(rows: int, hk: int, max_kv_len: int):
     return ups.value, ns.value
 
 
+def attn_decode_is_chunked(fmt: str, rows: int, hk: int, max_kv_len: int) -> bool:
+    """Whether a decode attention launch of this shape over pools of `fmt` takes the chunked form."""
+    code = 0 if fmt == "bf16" else KV_FORMATS[fmt]
+    return bool(kernels().pie_hip_attn_decode_is_chunked(code, rows, hk, max_kv_len))
+
+
 def attention_rows_paged_partials(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                                   kv_page_indices: torch.Tensor, row_page_begin: torch.Tensor,
                                   row_kv_len: torch.Tensor, max_kv_len: int, fmt: str = "bf16",

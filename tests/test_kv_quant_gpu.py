@@ -87,6 +87,58 @@ def test_attention_over_quantised_pool_matches_oracle(gpu, oracle, fmt, hq, hk, 
     assert np.allclose(lse_g[fin], lse64[fin], rtol=0, atol=2e-4)
 
 
+@pytest.mark.parametrize("fmt,hq,hk,d,ps,rows,longest", [
+    ("fp8_per_token_head", 32, 8, 128, 16, 40, 1600), ("int8_per_token_head", 32, 8, 128, 16, 40, 1600),
+    ("fp8_e4m3", 32, 8, 128, 16, 40, 1600), ("fp8_e5m2", 16, 4, 64, 32, 70, 1600),
+    ("int8_per_token_head", 32, 4, 128, 16, 70, 1600), ("fp8_per_token_head", 4, 2, 128, 16, 100, 2500),
+    ("int8_per_token_head", 2, 1, 64, 16, 200, 2100)])
+def test_large_ragged_batch_over_quantised_pools_takes_the_chunked_launch(gpu, oracle, fmt, hq, hk, d, ps, rows,
+                                                                          longest):
+    """Batches whose split grid would queue blocks run as equal chunks of the batch's keys, one wave
+    per kv head, pieces of a row merged from consecutive slots: empty rows, rows of one key, rows that
+    end inside a unit, rows cut by several chunks and chunks that cover many short rows."""
+    import torch
+    from pie_amd import ops
+
+    rng = np.random.default_rng(70 + hq + d + rows)
+    ctx = rng.integers(0, longest + 1, size=rows)
+    ctx[0], ctx[1], ctx[2], ctx[3], ctx[-1] = longest, 0, 1, 17, 16
+    ctx[5:15] = rng.integers(1, 20, size=10)                  # a run of short rows inside one chunk
+    ctx = [int(c) for c in ctx]
+    assert ops.attn_decode_is_chunked(fmt, rows, hk, max(ctx))
+    assert not ops.attn_decode_is_chunked("bf16", rows, hk, max(ctx))
+    b = make_paged_batch(rng, ctx, hk, d, ps, shared_prefix_tokens=2 * ps, shared_fraction=0.2,
+                         f32_to_bf16=oracle.f32_to_bf16)
+    P = b["num_pages"]
+    q = oracle.f32_to_bf16(rng.standard_normal((rows, hq, d)).astype(np.float32))
+    pools = {}
+    for name in ("k_pages", "v_pages"):
+        codes, scales, deq = oracle.kv_quant_rows(b[name].reshape(P * ps * hk, d), fmt)
+        pools[name] = (codes.reshape(P, ps, hk, d),
+                       None if scales is None else np.ascontiguousarray(scales.reshape(P, ps, hk).transpose(0, 2, 1)),
+                       deq.reshape(P, ps, hk, d))
+    begin, lens = b["page_indptr"][:-1].astype(np.int32), np.asarray(ctx, np.int32)
+    sc = lambda s: None if s is None else dev(s, gpu)
+    args = (fmt, dev(q, gpu, torch.bfloat16), dev(pools["k_pages"][0], gpu), dev(pools["v_pages"][0], gpu),
+            sc(pools["k_pages"][1]), sc(pools["v_pages"][1]), dev(b["page_indices"].view(np.int32), gpu),
+            dev(begin, gpu), dev(lens, gpu))
+    o, lse = ops.attention_rows_paged_kvq(*args, lse=True)
+    o2, _ = ops.attention_rows_paged_kvq(*args, lse=True)      # a second launch over the same workspace shape
+    torch.cuda.synchronize()
+    assert torch.equal(o.view(torch.uint16), o2.view(torch.uint16))
+    truth, _, lse64 = oracle.attn_rows_f32kv(q, pools["k_pages"][2], pools["v_pages"][2], b["page_indices"],
+                                             begin, lens, hq, hk, d, ps, mode=2)
+    got = oracle.bf16_to_f32(o.view(torch.uint16).cpu().numpy()).astype(np.float64)
+    tol = 2.0 ** -8 * np.maximum(np.abs(truth), np.abs(got)) + 1e-4
+    err = np.abs(got - truth)
+    assert np.all(err <= tol), f"worst {np.max(err / tol):.2f}x tol"
+    assert not np.any(got[1]), "a row without keys is all zeros"
+    lse_g = lse.cpu().numpy()
+    fin = np.isfinite(lse64)
+    assert np.array_equal(np.isneginf(lse_g), np.isneginf(lse64))
+    assert np.allclose(lse_g[fin], lse64[fin], rtol=0, atol=2e-4)
+
+
 def test_quantised_pool_argument_checks(gpu):
     import torch
     from pie_amd import ops
