@@ -320,7 +320,8 @@ __global__ __launch_bounds__(NW * kWave, 2) void attn_decode_mfma_kernel(
     const uint32_t* __restrict__ row_begin, const int32_t* __restrict__ row_len,
     float* __restrict__ part_o, float* __restrict__ part_ml, uint16_t* __restrict__ o_direct,
     float* __restrict__ lse, const uint16_t* __restrict__ mask_bits, int mask_stride, int hq, int hk,
-    int ps, int ps_shift, int units_per_split, int nsplit, float scale_log2e, int num_rows) {
+    int ps, int ps_shift, int units_per_split, int nsplit, float scale_log2e, int num_rows,
+    int* __restrict__ row_pieces) {
     static_assert(!(CHUNKS && MASKED), "the chunked launch takes no custom masks");
     static_assert(CHUNKS || NW == kAttnWaves, "the gridded launch has four waves per block");
     constexpr int KS = D / 32;                 // k steps of the first product
@@ -741,6 +742,15 @@ __global__ __launch_bounds__(NW * kWave, 2) void attn_decode_mfma_kernel(
                 if (lane == 0) row_pref[0] = 0;
             }
             __syncthreads();
+            if (b == 0 && pos == -1) {   // for the merge: each row's first slot and number of pieces
+                const int C = max((row_pref[R] + NB - 1) / NB, 1);
+                for (int rr = tid; rr < R; rr += NW * kWave) {
+                    const int lo = row_pref[rr], hi = row_pref[rr + 1];
+                    const int b_lo = lo / C;
+                    row_pieces[2 * rr] = b_lo + rr;
+                    row_pieces[2 * rr + 1] = hi > lo ? (hi - 1) / C - b_lo + 1 : 0;
+                }
+            }
             if (tid == 0) {
                 const int total = row_pref[R];
                 const int C = (total + NB - 1) / NB;
@@ -946,64 +956,53 @@ __global__ void attn_decode_clear_empty_kernel(const uint32_t* __restrict__ page
 }
 
 // The merge of a chunked launch (attn_decode_mfma_kernel<..., CHUNKS = true>): one block per
-// (row, q head).  The block recomputes where its row lies on the line of 16-token units (the
-// units of the rows before it) and from that the chunks that cut it: their pieces sit in
-// consecutive slots of the partial results, the piece of chunk b in slot b + row, a slot
-// holding the row's q heads in order.
+// (row, q head).  A row's pieces sit in consecutive slots of the partial results — the piece of
+// chunk b in slot b + row, a slot holding the row's q heads in order; the launch's first block
+// left each row's first slot and number of pieces in row_pieces.
 template <int D>
 __global__ __launch_bounds__(D) void attn_decode_merge_chunks_kernel(
-    const float* __restrict__ part_o, const float* __restrict__ part_ml,
-    const uint32_t* __restrict__ page_indptr, const uint32_t* __restrict__ last_lens,
-    const uint32_t* __restrict__ row_begin, const int32_t* __restrict__ row_len,
-    uint16_t* __restrict__ o, float* __restrict__ lse, int hq, int ps, int R, int NB) {
-    __shared__ int s_red[3][D / kWave];
+    const float* __restrict__ part_o, const float* __restrict__ part_ml, const int* __restrict__ row_pieces,
+    uint16_t* __restrict__ o, float* __restrict__ lse, int hq) {
     const int rh = blockIdx.x;
     const int r = rh / hq, head = rh - r * hq;
-    const int dd = threadIdx.x, lane = dd & (kWave - 1), wv = dd / kWave;
-    int before = 0, total = 0, mine = 0;
-    for (int rr = dd; rr < R; rr += D) {
-        const int n = (row_extent(page_indptr, last_lens, row_begin, row_len, rr, ps).kv_len + kUnitTokens - 1) / kUnitTokens;
-        total += n;
-        if (rr < r) before += n;
-        if (rr == r) mine = n;
-    }
-#pragma unroll
-    for (int off = 1; off < kWave; off <<= 1) {
-        before += __shfl_xor(before, off, kWave);
-        total += __shfl_xor(total, off, kWave);
-        mine += __shfl_xor(mine, off, kWave);
-    }
-    if (lane == 0) {
-        s_red[0][wv] = before;
-        s_red[1][wv] = total;
-        s_red[2][wv] = mine;
-    }
-    __syncthreads();
-    before = total = mine = 0;
-#pragma unroll
-    for (int w = 0; w < D / kWave; ++w) {
-        before += s_red[0][w];
-        total += s_red[1][w];
-        mine += s_red[2][w];
-    }
+    const int dd = threadIdx.x;
+    const size_t slot0 = static_cast<size_t>(row_pieces[2 * r]);
+    const int ns = row_pieces[2 * r + 1];
     const size_t out = static_cast<size_t>(rh) * D + dd;
-    if (mine == 0) {
+    if (ns == 0) {
         o[out] = 0;
         if (lse && dd == 0) lse[rh] = -INFINITY;
         return;
     }
-    const int C = (total + NB - 1) / NB;
-    const int b_lo = before / C, b_hi = (before + mine - 1) / C;
-    const size_t slot0 = static_cast<size_t>(b_lo) + r;
-    const int ns = b_hi - b_lo + 1;
     const float* ml = part_ml + (slot0 * hq + head) * 2;
     const float* po = part_o + (slot0 * hq + head) * D + dd;
     const size_t ml_step = static_cast<size_t>(hq) * 2, po_step = static_cast<size_t>(hq) * D;
+    // (a row is cut by few chunks: the first pieces are requested at once, ahead of the weights)
+    constexpr int kPre = 4;
+    float pre_o[kPre], pre_m[kPre], pre_l[kPre];
+#pragma unroll
+    for (int i = 0; i < kPre; ++i) {
+        const int ii = min(i, ns - 1);
+        pre_o[i] = po[ii * po_step];
+        pre_m[i] = ml[ii * ml_step];
+        pre_l[i] = ml[ii * ml_step + 1];
+    }
     float mx = -INFINITY;
-    for (int i = 0; i < ns; ++i) mx = fmaxf(mx, ml[i * ml_step]);
+#pragma unroll
+    for (int i = 0; i < kPre; ++i)
+        if (i < ns) mx = fmaxf(mx, pre_m[i]);
+    for (int i = kPre; i < ns; ++i) mx = fmaxf(mx, ml[i * ml_step]);
     const float safe = (mx == -INFINITY) ? 0.f : mx;
     float ov = 0.f, ls = 0.f;
-    for (int i = 0; i < ns; ++i) {
+#pragma unroll
+    for (int i = 0; i < kPre; ++i) {
+        if (i < ns) {
+            const float a = exp2f(pre_m[i] - safe);
+            ov = fmaf(pre_o[i], a, ov);
+            ls = fmaf(pre_l[i], a, ls);
+        }
+    }
+    for (int i = kPre; i < ns; ++i) {
         const float a = exp2f(ml[i * ml_step] - safe);
         ov = fmaf(po[i * po_step], a, ov);
         ls = fmaf(ml[i * ml_step + 1], a, ls);
@@ -1108,22 +1107,23 @@ int launch_decode(const uint16_t* q, const void* k_pages, const void* v_pages,
                 const ChunkPlan cp = plan_chunks(R, hk, max_kv_len, plan, KVF != kKvBf16);
                 if (cp.use) {
                     const size_t n_part = cp.slots * hq;
-                    const size_t need = n_part * (D + 2) * sizeof(float);
+                    const size_t need = n_part * (D + 2) * sizeof(float) + static_cast<size_t>(R) * 2 * sizeof(int);
                     if (!workspace || workspace_bytes < need) return PIE_HIP_ERR_INVALID;
                     float* part_o = static_cast<float*>(workspace);
                     float* part_ml = part_o + n_part * D;
+                    int* row_pieces = reinterpret_cast<int*>(part_ml + n_part * 2);
 #define PIE_CHUNK_LAUNCH(NWAVES)                                                                                       \
     hipLaunchKernelGGL((attn_decode_mfma_kernel<D, GQA, KVF, false, true, NWAVES>), dim3(cp.blocks), dim3(NWAVES * kWave), \
                        0, stream, q, k_pages, v_pages, k_scales, v_scales, page_indices, page_indptr, last_lens,       \
                        row_begin, row_len, part_o, part_ml, nullptr, nullptr, nullptr, 0, hq, hk, ps, ps_shift, 0, 0,  \
-                       scale_log2e, R)
+                       scale_log2e, R, row_pieces)
                     if (hk == 8) PIE_CHUNK_LAUNCH(8);
                     else if (hk == 4) PIE_CHUNK_LAUNCH(4);
                     else if (hk == 2) PIE_CHUNK_LAUNCH(2);
                     else PIE_CHUNK_LAUNCH(1);
 #undef PIE_CHUNK_LAUNCH
                     hipLaunchKernelGGL((attn_decode_merge_chunks_kernel<D>), dim3(R * hq), dim3(D), 0, stream, part_o,
-                                       part_ml, page_indptr, last_lens, row_begin, row_len, o, lse, hq, ps, R, cp.blocks);
+                                       part_ml, row_pieces, o, lse, hq);
                     return launch_status();
                 }
             }
@@ -1134,7 +1134,7 @@ int launch_decode(const uint16_t* q, const void* k_pages, const void* v_pages,
                                    stream, q, k_pages, v_pages, k_scales, v_scales, page_indices, page_indptr,
                                    last_lens, row_begin, row_len,
                                    nullptr, nullptr, o, lse, mask_bits, mask_stride, hq, hk, ps, ps_shift,
-                                   plan.units_per_split, 1, scale_log2e, R);
+                                   plan.units_per_split, 1, scale_log2e, R, nullptr);
                 return launch_status();
             }
             const size_t n_part = static_cast<size_t>(R) * hq * plan.nsplit;
@@ -1146,7 +1146,7 @@ int launch_decode(const uint16_t* q, const void* k_pages, const void* v_pages,
                                stream, q, k_pages, v_pages, k_scales, v_scales, page_indices, page_indptr,
                                last_lens, row_begin, row_len,
                                part_o, part_ml, nullptr, nullptr, mask_bits, mask_stride, hq, hk, ps, ps_shift,
-                               plan.units_per_split, plan.nsplit, scale_log2e, R);
+                               plan.units_per_split, plan.nsplit, scale_log2e, R, nullptr);
             if (!t_defer_merge)
                 hipLaunchKernelGGL((attn_decode_merge_kernel<D>), dim3(R * hq), dim3(D), 0, stream, part_o,
                                    part_ml, page_indptr, last_lens, row_begin, row_len, o, lse, hq, ps,
@@ -1194,7 +1194,9 @@ extern "C" size_t pie_hip_attn_decode_workspace_bytes(int num_requests, int num_
     // (the chunked launch's partial results, where a launch over one-byte pools without custom
     // masks would take it; bf16 pools and masked rows of the same shape keep the gridded launch)
     const pie_hip::ChunkPlan cp = pie_hip::plan_chunks(num_requests, num_kv_heads, max_kv_len, plan, true);
-    const size_t chunked = cp.use ? cp.slots * num_q_heads * (head_dim + 2) * sizeof(float) : 0;
+    const size_t chunked = cp.use ? cp.slots * num_q_heads * (head_dim + 2) * sizeof(float) +
+                                        static_cast<size_t>(num_requests) * 2 * sizeof(int)
+                                  : 0;
     return gridded > chunked ? gridded : chunked;
 }
 
