@@ -349,7 +349,10 @@ int pie_hip_moe_combine(const uint16_t* y_routes_bf16, const int32_t* route_pos,
  * (consecutive rows that share one page list, i.e. row_page_begin is equal across the tile;
  * at most rows_per_tile rows, which is pie_hip_attn_prefill_tile_rows(hq, hk) = 128 / (hq/hk)
  * or half of it — the smaller tile doubles the number of blocks for small batches); each row
- * still sees its own first row_kv_len[row] keys.  Probabilities are rounded to bf16 before they multiply V
+ * still sees its own first row_kv_len[row] keys.  Tiles may come in any order; blocks start in tile
+ * order (the kv heads of a tile side by side), so listing the tiles with the longest key extents
+ * first lets the short ones fill the slots that free up — on a causal prompt of more tiles than the
+ * device holds at once that is worth 15-30 % (4096 tokens: 355 -> 278 us).  Probabilities are rounded to bf16 before they multiply V
  * (fp32 softmax sums and accumulators), so results agree with the per-row kernel to about one
  * bf16 step rather than bit for bit.  d in {64,128}, hq/hk in {1,2,4,8}, page_size % 16 == 0.
  * Reference: the causal prefill branch of launch_attention_naive_paged_prefill,

@@ -74,12 +74,15 @@ __global__ __launch_bounds__(kTileThreads, 2) void attn_prefill_tile_kernel(
     __shared__ __attribute__((aligned(16))) uint16_t Vt_all[2][D * kVtStride];
     __shared__ int s_kmax;
 
-    // Causal tiles grow with their index, and a CU holds two blocks that are about one machine
-    // width (256 blocks) apart in launch order: every other machine width walks the tiles
-    // backwards, so a long tile shares its CU with a short one.
-    const int kvh = blockIdx.y;
-    const bool backwards = ((blockIdx.y * gridDim.x) >> 8) & 1;
-    const int tile = backwards ? gridDim.x - 1 - blockIdx.x : blockIdx.x;
+    // Blocks start in the order of their linear index: tile-major, the kv heads of a tile side by
+    // side.  A caller that lists its tiles longest first therefore gets the long causal tiles
+    // started first and the short ones handed to the slots that free up — the longest-first rule,
+    // which for a causal prompt of more tiles than slots comes within a step of an even split
+    // (measured, 32 q / 8 kv heads of 128: 3072 tokens 242 -> 169 us, 4096 tokens 355 -> 278, 8192
+    // tokens 1072 -> 934).
+    const int lin = blockIdx.y * gridDim.x + blockIdx.x;
+    const int tile = lin / hk;
+    const int kvh = lin - tile * hk;
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wv = tid / kWave;
     const int l16 = lane & 15, g = lane >> 4;
     const int s0 = tile_start[tile], n_rows = tile_rows[tile];
