@@ -1033,7 +1033,18 @@ SplitPlan plan_splits(int R, int hk, int max_kv_len) {
     // rows, down to 128 tokens so the machine fills
     const long long min_ups = rows * ((max_units + 31) / 32) >= 512 ? 32 : 2 * kAttnWaves;
     long long want_split = (want_blocks + rows - 1) / rows;
-    if (want_split < 1) want_split = 1;
+    // Batches whose 512-token blocks would not fill two rounds of the resident grid (512 blocks of
+    // four waves) take exactly one round: as many splits as put rows * splits at 512.  A second,
+    // partial round leaves most of the machine waiting for its last blocks (measured, 8B decode
+    // steps at 2048 keys, batch 4 / 8 / 16: 2.34 / 2.61 / 3.15 -> 2.29 / 2.55 / 3.08 ms; 16 rows at
+    // 1024 keys 2.84 -> 2.77; one and two rows plan as before).
+    if (rows * ((max_units + 31) / 32) < 768 && rows <= 512) {
+        const long long ns = 512 / rows;
+        long long u = (max_units + ns - 1) / ns;
+        if (u < 2 * kAttnWaves) u = 2 * kAttnWaves;   // >= 2 units per wave amortises the merge
+        if (u > max_units) u = max_units;
+        return {static_cast<int>(u), static_cast<int>((max_units + u - 1) / u)};
+    }
     long long ups = (max_units + want_split - 1) / want_split;
     if (ups < min_ups) ups = min_ups;  // >= 2 units per wave amortises the merge
     if (ups > max_units) ups = max_units;
