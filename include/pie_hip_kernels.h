@@ -602,6 +602,21 @@ int pie_hip_attn_rows_paged_kvq(int kv_format, const uint16_t* q, const void* k_
                                 int num_rows, int num_q_heads, int num_kv_heads, int head_dim,
                                 int page_size, float sm_scale, int max_kv_len, void* workspace,
                                 size_t workspace_bytes, void* stream);
+/* The same call (any kv_format, PIE_HIP_KV_BF16 with NULL scales included) for a batch whose rows
+ * the caller knows to be about equally long, e.g. a decode batch whose longest context is within an
+ * eighth of the mean: the launch then takes one round of resident blocks — for 64 rows of 8 kv
+ * heads one block per (row, kv head), nothing to merge — where rows of unknown lengths get several
+ * splits so that a long one does not run on alone.  Same results contract and workspace query;
+ * a wrong hint costs time, not correctness.  Reference: the decode branch of
+ * launch_attention_naive_paged, driver/cuda/src/ops/attention_naive_paged.cu:319-447 (one launch
+ * per batch; the split plan is this library's). */
+int pie_hip_attn_rows_paged_kvq_uniform(int kv_format, const uint16_t* q, const void* k_pages,
+                                        const void* v_pages, const float* k_scales, const float* v_scales,
+                                        uint16_t* o, float* lse, const uint32_t* kv_page_indices,
+                                        const uint32_t* row_page_begin, const int32_t* row_kv_len,
+                                        int num_rows, int num_q_heads, int num_kv_heads, int head_dim,
+                                        int page_size, float sm_scale, int max_kv_len, void* workspace,
+                                        size_t workspace_bytes, void* stream);
 /* The same over rows with custom attention masks: mask_bitmap as for
  * pie_hip_attn_rows_paged_masked (one visibility word per row and 16-token unit). */
 int pie_hip_attn_rows_paged_kvq_masked(int kv_format, const uint16_t* q, const void* k_pages,

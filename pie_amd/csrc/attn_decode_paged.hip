@@ -23,6 +23,7 @@
 //   * the next unit's K and V rows are requested before the current unit is
 //     reduced, so 2 x (K+V) = 16 KiB per wave is in flight;
 //   * a second, tiny kernel merges the splits (skipped when there is one split).
+#include <algorithm>
 #include <cstdio>
 #include <mutex>
 #include <type_traits>
@@ -1019,10 +1020,13 @@ struct SplitPlan {
 // pie_hip_attn_rows_paged_partials: the split launch alone, its partial results left in the
 // workspace for a consumer that merges them itself (set around the one dispatch call)
 thread_local bool t_defer_merge = false;
+// pie_hip_attn_rows_paged_kvq_uniform: the caller knows the rows to be about equally long (set
+// around the one dispatch call)
+thread_local bool t_uniform_rows = false;
 
 // Same rule for the workspace query and the launch: aim for >= ~8 blocks per CU over the
 // whole batch, never less than one unit per wave and per block.
-SplitPlan plan_splits(int R, int hk, int max_kv_len) {
+SplitPlan plan_splits(int R, int hk, int max_kv_len, bool uniform = false) {
     const int max_units = (max_kv_len + kUnitTokens - 1) / kUnitTokens;
     if (max_units <= 0) return {1, 1};
     const long long rows = static_cast<long long>(R) * hk;
@@ -1034,16 +1038,23 @@ SplitPlan plan_splits(int R, int hk, int max_kv_len) {
     const long long min_ups = rows * ((max_units + 31) / 32) >= 512 ? 32 : 2 * kAttnWaves;
     long long want_split = (want_blocks + rows - 1) / rows;
     // Batches whose 512-token blocks would not fill two rounds of the resident grid (512 blocks of
-    // four waves) take exactly one round: as many splits as put rows * splits at 512.  A second,
-    // partial round leaves most of the machine waiting for its last blocks (measured, 8B decode
-    // steps at 2048 keys, batch 4 / 8 / 16: 2.34 / 2.61 / 3.15 -> 2.29 / 2.55 / 3.08 ms; 16 rows at
-    // 1024 keys 2.84 -> 2.77; one and two rows plan as before).
-    if (rows * ((max_units + 31) / 32) < 768 && rows <= 512) {
+    // four waves) take exactly one round: as many splits as put rows * splits at 512 (and not
+    // under 448: a round that leaves an eighth of the slots empty is no gain).  A second, partial
+    // round leaves most of the machine waiting for its last blocks (measured, 8B decode steps at
+    // 2048 keys, batch 4 / 8 / 16: 2.34 / 2.61 / 3.15 -> 2.29 / 2.55 / 3.08 ms; 16 rows at 1024 keys
+    // 2.84 -> 2.77; one and two rows plan as before).  Rows the caller knows to be about equally
+    // long take the single round up to six rounds' worth of such blocks — then no block outlasts
+    // the others, and with one split per row there is nothing to merge (batch 64 at 2048 / 512
+    // keys 6.15 / 4.20 -> 5.74 / 3.87 ms, batch 32 at 1024 keys 3.49 -> 3.41, the MoE batch 10.19 ->
+    // 10.03); with rows of unknown lengths a long one would run on alone.
+    if (rows * ((max_units + 31) / 32) < (uniform ? 3000 : 768) && rows <= 512) {
         const long long ns = 512 / rows;
-        long long u = (max_units + ns - 1) / ns;
-        if (u < 2 * kAttnWaves) u = 2 * kAttnWaves;   // >= 2 units per wave amortises the merge
-        if (u > max_units) u = max_units;
-        return {static_cast<int>(u), static_cast<int>((max_units + u - 1) / u)};
+        if (rows * ns >= 448) {
+            long long u = (max_units + ns - 1) / ns;
+            if (u < 2 * kAttnWaves) u = 2 * kAttnWaves;   // >= 2 units per wave amortises the merge
+            if (u > max_units) u = max_units;
+            return {static_cast<int>(u), static_cast<int>((max_units + u - 1) / u)};
+        }
     }
     long long ups = (max_units + want_split - 1) / want_split;
     if (ups < min_ups) ups = min_ups;  // >= 2 units per wave amortises the merge
@@ -1102,7 +1113,7 @@ int launch_decode(const uint16_t* q, const void* k_pages, const void* v_pages,
                   int R, int hq, int hk, int ps, float sm_scale,
                   int max_kv_len, void* workspace, size_t workspace_bytes, const uint16_t* mask_bits,
                   int mask_stride, hipStream_t stream) {
-    const SplitPlan plan = plan_splits(R, hk, max_kv_len);
+    const SplitPlan plan = plan_splits(R, hk, max_kv_len, t_uniform_rows);
     const float scale_log2e = sm_scale * 1.4426950408889634f;
     {
         // The matrix-core kernel: bf16 and one-byte pools, rows with and without a custom mask.  Measured (MI355X, 8B / 30B-A3B
@@ -1199,8 +1210,11 @@ extern "C" size_t pie_hip_attn_decode_workspace_bytes(int num_requests, int num_
                                                       int max_kv_len) {
     if (num_requests <= 0 || num_q_heads <= 0 || num_kv_heads <= 0 || head_dim <= 0) return 0;
     const pie_hip::SplitPlan plan = pie_hip::plan_splits(num_requests, num_kv_heads, max_kv_len);
-    const size_t gridded = plan.nsplit == 1 ? 0
-                                            : static_cast<size_t>(num_requests) * num_q_heads * plan.nsplit *
+    // (the plan for rows of unknown lengths and the one for rows known to be equally long:
+    // whichever needs more)
+    const int most_splits = std::max(plan.nsplit, pie_hip::plan_splits(num_requests, num_kv_heads, max_kv_len, true).nsplit);
+    const size_t gridded = most_splits == 1 ? 0
+                                            : static_cast<size_t>(num_requests) * num_q_heads * most_splits *
                                                   (head_dim + 2) * sizeof(float);
     // (the chunked launch's partial results, where a launch over one-byte pools without custom
     // masks would take it; bf16 pools and masked rows of the same shape keep the gridded launch)
@@ -1448,6 +1462,24 @@ extern "C" int pie_hip_attn_rows_paged_kvq(int kv_format, const uint16_t* q, con
                                   row_page_begin, row_kv_len, num_rows, num_q_heads, num_kv_heads,
                                   head_dim, page_size, sm_scale, max_kv_len, workspace,
                                   workspace_bytes, stream, nullptr, 0, kv_format, k_scales, v_scales);
+}
+
+extern "C" int pie_hip_attn_rows_paged_kvq_uniform(int kv_format, const uint16_t* q, const void* k_pages,
+                                                   const void* v_pages, const float* k_scales,
+                                                   const float* v_scales, uint16_t* o, float* lse,
+                                                   const uint32_t* kv_page_indices,
+                                                   const uint32_t* row_page_begin,
+                                                   const int32_t* row_kv_len, int num_rows,
+                                                   int num_q_heads, int num_kv_heads, int head_dim,
+                                                   int page_size, float sm_scale, int max_kv_len,
+                                                   void* workspace, size_t workspace_bytes, void* stream) {
+    pie_hip::t_uniform_rows = true;
+    const int rc = pie_hip_attn_rows_paged_kvq(kv_format, q, k_pages, v_pages, k_scales, v_scales, o, lse,
+                                               kv_page_indices, row_page_begin, row_kv_len, num_rows, num_q_heads,
+                                               num_kv_heads, head_dim, page_size, sm_scale, max_kv_len, workspace,
+                                               workspace_bytes, stream);
+    pie_hip::t_uniform_rows = false;
+    return rc;
 }
 
 extern "C" int pie_hip_attn_rows_paged_kvq_masked(int kv_format, const uint16_t* q, const void* k_pages,

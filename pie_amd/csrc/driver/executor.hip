@@ -687,9 +687,9 @@ void Executor::body(int N, int S, int max_kv_len) {
                 static_cast<const uint16_t*>(mask_bitmap_.ptr), mask_stride_, N, hq, hk, d, page_size_, -1.f,
                 max_kv_len, attn_ws_, attn_ws_bytes_, s));
         } else if (kvq_attn) {
-            PIE_KERNEL(pie_hip_attn_rows_paged_kvq(kv_format_, q_, k_pool_[l], v_pool_[l], ksc, vsc, attn_,
-                                                   nullptr, pages, row_begin, row_len, N, hq, hk, d,
-                                                   page_size_, -1.f, max_kv_len, attn_ws_, attn_ws_bytes_, s));
+            PIE_KERNEL((uniform_rows_ ? pie_hip_attn_rows_paged_kvq_uniform : pie_hip_attn_rows_paged_kvq)(
+                kv_format_, q_, k_pool_[l], v_pool_[l], ksc, vsc, attn_, nullptr, pages, row_begin, row_len, N, hq,
+                hk, d, page_size_, -1.f, max_kv_len, attn_ws_, attn_ws_bytes_, s));
         } else if (n_tiles_ > 0) {
             const auto* td = static_cast<const int32_t*>(tile_in_dev_.ptr);
             PIE_KERNEL(pie_hip_attn_prefill_tiles(q_, kat, vat, attn_, pages, row_begin,
@@ -700,6 +700,10 @@ void Executor::body(int N, int S, int max_kv_len) {
                 q_, kat, vat, attn_, nullptr, pages, row_begin, row_len,
                 static_cast<const uint16_t*>(mask_bitmap_.ptr), mask_stride_, N, hq, hk, d, page_size_,
                 -1.f, max_kv_len, attn_ws_, attn_ws_bytes_, s));
+        } else if (uniform_rows_) {
+            PIE_KERNEL(pie_hip_attn_rows_paged_kvq_uniform(PIE_HIP_KV_BF16, q_, kat, vat, nullptr, nullptr, attn_,
+                                                           nullptr, pages, row_begin, row_len, N, hq, hk, d,
+                                                           page_size_, -1.f, max_kv_len, attn_ws_, attn_ws_bytes_, s));
         } else {
             PIE_KERNEL(pie_hip_attn_rows_paged(q_, kat, vat, attn_, nullptr, pages,
                                                row_begin, row_len, N, hq, hk, d, page_size_, -1.f,
@@ -1077,13 +1081,25 @@ void Executor::forward(const BatchPlan& plan, std::vector<uint32_t>& tokens_out,
 
     t0 = clk::now();
     n_page_refs_ = static_cast<int>(plan.page_indices.size());
+    // A decode batch whose longest context is within an eighth of the mean: the attention launch
+    // may then plan one round of equally long blocks (a graph is captured per answer).
+    uniform_rows_ = false;
+    if (plan.pure_decode && N >= 2 && !masked_) {
+        long long total = 0;
+        int longest = 0;
+        for (int i = 0; i < N; ++i) {
+            total += plan.row_kv_len[i];
+            longest = std::max(longest, plan.row_kv_len[i]);
+        }
+        uniform_rows_ = 8LL * longest * N <= 9 * total;
+    }
     // (4-bit blocks: the page expansion's extent changes from step to step, so no graph)
     const bool use_graph = cfg_.runtime.use_graphs && plan.pure_decode && !samp_gather_in_body_ && !masked_ &&
                            kv_format_ != PIE_HIP_KV_FP4_BLOCK;
     if (use_graph) {
         // The split grid depends on the context bound only through 512-token buckets.
         const int bucket = (plan.max_kv_len + 511) / 512 * 512;
-        const auto key = std::make_tuple(N, S, bucket);
+        const auto key = std::make_tuple(N, S, bucket, uniform_rows_ ? 1 : 0);
         auto it = graphs_.find(key);
         if (it == graphs_.end()) {
             hipGraph_t graph = nullptr;

@@ -186,7 +186,8 @@ class Executor {
     bool samp_gather_in_body_ = false;
     uint64_t unseeded_draws_ = 0;
 
-    std::map<std::tuple<int, int, int>, hipGraphExec_t> graphs_;
+    std::map<std::tuple<int, int, int, int>, hipGraphExec_t> graphs_;   // (rows, sampling slots, context bucket, rows equally long)
+    bool uniform_rows_ = false;   // this step's rows are about equally long (decode batches)
     int last_logit_rows_ = 0;
 };
 

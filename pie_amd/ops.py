@@ -1032,14 +1032,15 @@ def attention_rows_paged_kvq(fmt: str, q: torch.Tensor, k_pages: torch.Tensor, v
                              kv_page_indices: torch.Tensor, row_page_begin: torch.Tensor,
                              row_kv_len: torch.Tensor, lse: bool = False,
                              max_kv_len: Optional[int] = None, o: Optional[torch.Tensor] = None,
-                             workspace: Optional[torch.Tensor] = None):
-    """Per-row paged attention over a one-byte KV pool.  q [rows, hq, d] bf16.  With
-    max_kv_len, o and workspace given the call neither synchronises nor allocates (graph
-    capture); the extents are then the caller's responsibility."""
+                             workspace: Optional[torch.Tensor] = None, uniform: bool = False):
+    """Per-row paged attention over a one-byte KV pool (fmt "bf16": a bf16 pool, no scales).
+    q [rows, hq, d] bf16.  With max_kv_len, o and workspace given the call neither synchronises
+    nor allocates (graph capture); the extents are then the caller's responsibility.  uniform:
+    the rows are known to be about equally long (pie_hip_attn_rows_paged_kvq_uniform)."""
     _dev(q, torch.bfloat16, "q")
     rows, hq, d = q.shape
     ps, hk = k_pages.shape[1], k_pages.shape[2]
-    if k_pages.element_size() != 1 or v_pages.element_size() != 1:
+    if fmt != "bf16" and (k_pages.element_size() != 1 or v_pages.element_size() != 1):
         raise KernelError("one-byte pools expected")
     _dev(kv_page_indices, torch.int32, "kv_page_indices")
     _dev(row_page_begin, torch.int32, "row_page_begin")
@@ -1064,9 +1065,8 @@ def attention_rows_paged_kvq(fmt: str, q: torch.Tensor, k_pages: torch.Tensor, v
     ws = workspace if workspace is not None else torch.empty(max(need, 1), dtype=torch.uint8, device=q.device)
     if ws.numel() < need:
         raise KernelError("workspace too small")
-    _check(lib.pie_hip_attn_rows_paged_kvq(KV_FORMATS[fmt], _ptr(q), _ptr(k_pages), _ptr(v_pages),
-                                           _ptr(k_scales), _ptr(v_scales), _ptr(o), _ptr(lse_t),
-                                           _ptr(kv_page_indices), _ptr(row_page_begin), _ptr(row_kv_len),
-                                           rows, hq, hk, d, ps, C.c_float(-1.0), max_kv, _ptr(ws),
-                                           C.c_size_t(need), _stream()), "pie_hip_attn_rows_paged_kvq")
+    fn = lib.pie_hip_attn_rows_paged_kvq_uniform if uniform else lib.pie_hip_attn_rows_paged_kvq
+    _check(fn(KV_FORMATS[fmt], _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(k_scales), _ptr(v_scales), _ptr(o),
+              _ptr(lse_t), _ptr(kv_page_indices), _ptr(row_page_begin), _ptr(row_kv_len), rows, hq, hk, d, ps,
+              C.c_float(-1.0), max_kv, _ptr(ws), C.c_size_t(need), _stream()), "pie_hip_attn_rows_paged_kvq")
     return o, lse_t

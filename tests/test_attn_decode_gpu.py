@@ -213,3 +213,39 @@ def test_rows_with_custom_masks_match_oracle(gpu, oracle, hq, hk, d):
     assert (np.abs(plain - masked)[same_sign] <= 1).mean() > 0.99
     pf, mf = oracle.bf16_to_f32(plain.astype(np.uint16)), oracle.bf16_to_f32(masked.astype(np.uint16))
     assert np.all(np.abs(pf - mf) <= 2.0 ** -7 * np.maximum(np.abs(pf), np.abs(mf)) + 2e-4)
+
+
+@pytest.mark.parametrize("ctx_kind", ["equal", "ragged"])
+@pytest.mark.parametrize("rows,hq,hk,d", [(64, 32, 8, 128), (32, 16, 8, 64), (64, 32, 4, 128)])
+def test_rows_declared_equally_long_take_one_round_and_match_the_oracle(gpu, oracle, rows, hq, hk, d, ctx_kind):
+    """pie_hip_attn_rows_paged_kvq_uniform: a batch of about equal contexts plans one round of blocks
+    (64 rows x 8 kv heads: one block per row and head, no merge); the hint only changes the plan, so a
+    ragged batch given it by mistake, empty row included, still comes out right."""
+    import torch
+
+    from pie_amd import ops
+
+    ps = 16
+    rng = np.random.default_rng(rows + hq + d)
+    ctx = [int(c) for c in (rng.integers(600, 641, size=rows) if ctx_kind == "equal"
+                            else rng.integers(0, 1300, size=rows))]
+    if ctx_kind == "ragged":
+        ctx[0], ctx[1] = 1290, 0
+    b = make_paged_batch(rng, ctx, hk, d, ps, f32_to_bf16=oracle.f32_to_bf16)
+    q = oracle.f32_to_bf16(rng.standard_normal((rows, hq, d)).astype(np.float32))
+
+    def dev(a, dt=None):
+        t = torch.from_numpy(np.ascontiguousarray(a)).to(gpu)
+        return t.view(dt) if dt is not None else t
+
+    begin, lens = b["page_indptr"][:-1].astype(np.int32), np.asarray(ctx, np.int32)
+    args = ("bf16", dev(q, torch.bfloat16), dev(b["k_pages"], torch.bfloat16), dev(b["v_pages"], torch.bfloat16),
+            None, None, dev(b["page_indices"].view(np.int32)), dev(begin), dev(lens))
+    o, lse = ops.attention_rows_paged_kvq(*args, lse=True, uniform=True)
+    o_plain, _ = ops.attention_rows_paged_kvq(*args, lse=True)
+    torch.cuda.synchronize()
+    check(oracle, o.view(torch.uint16).cpu().numpy(), lse.cpu().numpy(), q, b, hq, hk, d, ps)
+    # the two plans differ by the rounding of the split merge only
+    a0 = oracle.bf16_to_f32(o.view(torch.uint16).cpu().numpy())
+    a1 = oracle.bf16_to_f32(o_plain.view(torch.uint16).cpu().numpy())
+    assert np.all(np.abs(a0 - a1) <= 2.0 ** -7 * np.maximum(np.abs(a0), np.abs(a1)) + 1e-4)
