@@ -372,7 +372,19 @@ __global__ __launch_bounds__(NW * kWave, 2) void attn_decode_mfma_kernel(
         const int kv_len = ext.kv_len;
         nunits = (kv_len + kUnitTokens - 1) / kUnitTokens;
         const int u_begin = split * units_per_split;
-        if (u_begin >= nunits) return;
+        if (u_begin >= nunits) {
+            // (one split per row: a row without keys gets its zeros and its -inf here, no launch
+            // of its own for that)
+            if (o_direct && nunits == 0) {
+                for (int idx = tid; idx < GQA * D; idx += kAttnBlock) {
+                    const int h = idx / D, dd = idx - h * D;
+                    const size_t rh = static_cast<size_t>(r) * hq + kvh * GQA + h;
+                    o_direct[rh * D + dd] = 0;
+                    if (lse && dd == 0) lse[rh] = -INFINITY;
+                }
+            }
+            return;
+        }
         k_begin = u_begin * kUnitTokens;
         k_end = min(min(u_begin + units_per_split, nunits) * kUnitTokens, kv_len);
     }
@@ -1150,8 +1162,6 @@ int launch_decode(const uint16_t* q, const void* k_pages, const void* v_pages,
                 }
             }
             if (plan.nsplit == 1) {
-                hipLaunchKernelGGL((attn_decode_clear_empty_kernel<D>), dim3(R * hq), dim3(D), 0, stream,
-                                   page_indptr, last_lens, row_begin, row_len, o, lse, hq, ps);
                 hipLaunchKernelGGL((attn_decode_mfma_kernel<D, GQA, KVF, MASKED>), dim3(hk, 1, R), dim3(kAttnBlock), 0,
                                    stream, q, k_pages, v_pages, k_scales, v_scales, page_indices, page_indptr,
                                    last_lens, row_begin, row_len,
