@@ -1036,6 +1036,22 @@ thread_local bool t_defer_merge = false;
 // around the one dispatch call)
 thread_local bool t_uniform_rows = false;
 
+// Compute units of the current device (256 on an MI355X; that figure when no device answers).
+int resident_attn_blocks() {
+    constexpr int kMaxDev = 64;
+    static std::mutex mu;
+    static int cached[kMaxDev] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDev) return 0;
+    std::lock_guard<std::mutex> lock(mu);
+    if (cached[dev] == 0) {
+        int cus = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) return 0;
+        cached[dev] = cus;
+    }
+    return cached[dev];
+}
+
 // Same rule for the workspace query and the launch: aim for >= ~8 blocks per CU over the
 // whole batch, never less than one unit per wave and per block.
 SplitPlan plan_splits(int R, int hk, int max_kv_len, bool uniform = false) {
@@ -1059,9 +1075,11 @@ SplitPlan plan_splits(int R, int hk, int max_kv_len, bool uniform = false) {
     // the others, and with one split per row there is nothing to merge (batch 64 at 2048 / 512
     // keys 6.15 / 4.20 -> 5.74 / 3.87 ms, batch 32 at 1024 keys 3.49 -> 3.41, the MoE batch 10.19 ->
     // 10.03); with rows of unknown lengths a long one would run on alone.
-    if (rows * ((max_units + 31) / 32) < (uniform ? 3000 : 768) && rows <= 512) {
-        const long long ns = 512 / rows;
-        if (rows * ns >= 448) {
+    const int cus = resident_attn_blocks();
+    const long long slots = 2LL * (cus > 0 ? cus : 256);   // resident blocks: two of four waves per CU
+    if (rows * ((max_units + 31) / 32) < (uniform ? 6 * slots : slots + slots / 2) && rows <= slots) {
+        const long long ns = slots / rows;
+        if (rows * ns >= slots - slots / 8) {
             long long u = (max_units + ns - 1) / ns;
             if (u < 2 * kAttnWaves) u = 2 * kAttnWaves;   // >= 2 units per wave amortises the merge
             if (u > max_units) u = max_units;
@@ -1090,20 +1108,6 @@ struct ChunkPlan {
     int blocks;
     size_t slots;   // partial results: blocks + rows slots of hq heads each
 };
-int resident_attn_blocks() {
-    constexpr int kMaxDev = 64;
-    static std::mutex mu;
-    static int cached[kMaxDev] = {};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDev) return 0;
-    std::lock_guard<std::mutex> lock(mu);
-    if (cached[dev] == 0) {
-        int cus = 0;
-        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) return 0;
-        cached[dev] = cus;
-    }
-    return cached[dev];   // (compute units)
-}
 ChunkPlan plan_chunks(int R, int hk, int max_kv_len, const SplitPlan& plan, bool one_byte_pool) {
     static const int forced = [] { const char* e = getenv("PIE_HIP_ATTN_CHUNKS"); return e ? atoi(e) : -1; }();   // measurement hook
     // a CU holds eight waves of the kernel (two per SIMD: its registers) = 8 / hk blocks of one
