@@ -324,7 +324,7 @@ __global__ __launch_bounds__(NW * kWave, 2) void attn_decode_mfma_kernel(
     int ps, int ps_shift, int units_per_split, int nsplit, float scale_log2e, int num_rows,
     int* __restrict__ row_pieces) {
     static_assert(!(CHUNKS && MASKED), "the chunked launch takes no custom masks");
-    static_assert(CHUNKS || NW == kAttnWaves, "the gridded launch has four waves per block");
+    static_assert(CHUNKS || NW == kAttnWaves || NW == 2 * kAttnWaves, "the gridded launch has four or eight waves per block");
     constexpr int KS = D / 32;                 // k steps of the first product
     constexpr int DT = D / 16;                 // d tiles of the second product
     // One-byte pools: the codes become bf16 (exactly) on the way into the wave's LDS regions, the
@@ -376,7 +376,7 @@ __global__ __launch_bounds__(NW * kWave, 2) void attn_decode_mfma_kernel(
             // (one split per row: a row without keys gets its zeros and its -inf here, no launch
             // of its own for that)
             if (o_direct && nunits == 0) {
-                for (int idx = tid; idx < GQA * D; idx += kAttnBlock) {
+                for (int idx = tid; idx < GQA * D; idx += NW * kWave) {
                     const int h = idx / D, dd = idx - h * D;
                     const size_t rh = static_cast<size_t>(r) * hq + kvh * GQA + h;
                     o_direct[rh * D + dd] = 0;
@@ -477,8 +477,8 @@ __global__ __launch_bounds__(NW * kWave, 2) void attn_decode_mfma_kernel(
     float mx = -INFINITY, lsum = 0.f;
 
     // keys between two steps of one wave: the gridded launch deals a split's steps to its four
-    // waves in turn, a wave of the chunked launch walks its own kv head's keys alone
-    constexpr int kStride = CHUNKS ? kMStepKeys : kAttnWaves * kMStepKeys;
+    // (or eight) waves in turn, a wave of the chunked launch walks its own kv head's keys alone
+    constexpr int kStride = CHUNKS ? kMStepKeys : NW * kMStepKeys;
 
     // ---- chunked launch: the table of this block's items and the cursor of the K/V requests ----
     // An item is a (row, key range), worked on by all waves at once — wave w takes kv head w, so
@@ -675,15 +675,15 @@ __global__ __launch_bounds__(NW * kWave, 2) void attn_decode_mfma_kernel(
             }
         }
         __syncthreads();
-        for (int idx = tid; idx < GQA * D; idx += kAttnBlock) {
+        for (int idx = tid; idx < GQA * D; idx += NW * kWave) {
             const int h = idx / D, dd = idx - h * D;
             float m_all = sm_m[0][h];
 #pragma unroll
-            for (int w = 1; w < kAttnWaves; ++w) m_all = fmaxf(m_all, sm_m[w][h]);
+            for (int w = 1; w < NW; ++w) m_all = fmaxf(m_all, sm_m[w][h]);
             const float safe = (m_all == -INFINITY) ? 0.f : m_all;
             float ov = 0.f, ls = 0.f;
 #pragma unroll
-            for (int w = 0; w < kAttnWaves; ++w) {
+            for (int w = 0; w < NW; ++w) {
                 const float a = exp2f(sm_m[w][h] - safe);
                 ov += reinterpret_cast<const float*>(kv_all[w] + KREGION)[h * D + dd] * a;
                 ls += sm_l[w][h] * a;
@@ -1027,6 +1027,7 @@ __global__ __launch_bounds__(D) void attn_decode_merge_chunks_kernel(
 struct SplitPlan {
     int units_per_split;
     int nsplit;
+    int waves = kAttnWaves;   // per block of the gridded launch (eight: whole rows by blocks of twice the width)
 };
 
 // pie_hip_attn_rows_paged_partials: the split launch alone, its partial results left in the
@@ -1077,6 +1078,11 @@ SplitPlan plan_splits(int R, int hk, int max_kv_len, bool uniform = false) {
     // 10.03); with rows of unknown lengths a long one would run on alone.
     const int cus = resident_attn_blocks();
     const long long slots = 2LL * (cus > 0 ? cus : 256);   // resident blocks: two of four waves per CU
+    // Equally long rows that fill half of those slots (32 rows of 8 kv heads, 64 rows of 4): one
+    // block of eight waves per (row, kv head) — the same waves in flight as two splits of four
+    // waves each, and nothing to merge.
+    if (uniform && 2 * rows <= slots && 2 * rows >= slots - slots / 8 && rows * ((max_units + 31) / 32) < 6 * slots)
+        return {max_units, 1, 2 * kAttnWaves};
     if (rows * ((max_units + 31) / 32) < (uniform ? 6 * slots : slots + slots / 2) && rows <= slots) {
         const long long ns = slots / rows;
         if (rows * ns >= slots - slots / 8) {
@@ -1162,6 +1168,15 @@ int launch_decode(const uint16_t* q, const void* k_pages, const void* v_pages,
 #undef PIE_CHUNK_LAUNCH
                     hipLaunchKernelGGL((attn_decode_merge_chunks_kernel<D>), dim3(R * hq), dim3(D), 0, stream, part_o,
                                        part_ml, row_pieces, o, lse, hq);
+                    return launch_status();
+                }
+            }
+            if constexpr (!MASKED) {
+                if (plan.nsplit == 1 && plan.waves == 2 * kAttnWaves) {
+                    hipLaunchKernelGGL((attn_decode_mfma_kernel<D, GQA, KVF, false, false, 2 * kAttnWaves>), dim3(hk, 1, R),
+                                       dim3(2 * kAttnBlock), 0, stream, q, k_pages, v_pages, k_scales, v_scales,
+                                       page_indices, page_indptr, last_lens, row_begin, row_len, nullptr, nullptr, o, lse,
+                                       nullptr, 0, hq, hk, ps, ps_shift, plan.units_per_split, 1, scale_log2e, R, nullptr);
                     return launch_status();
                 }
             }
