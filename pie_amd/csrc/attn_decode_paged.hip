@@ -1085,7 +1085,13 @@ SplitPlan plan_splits(int R, int hk, int max_kv_len, bool uniform = false) {
         return {max_units, 1, 2 * kAttnWaves};
     if (rows * ((max_units + 31) / 32) < (uniform ? 6 * slots : slots + slots / 2) && rows <= slots) {
         const long long ns = slots / rows;
-        if (rows * ns >= slots - slots / 8) {
+        // (equally long rows that fill more than half the slots: one split per row also where an
+        // eighth or more of the slots stays empty, as long as the empty share times the rows'
+        // length stays under what the second round and the merge of a split plan cost — 48 rows
+        // of 8 kv heads at 512 / 2048 keys 3.85 / 5.33 -> 3.60 / 5.22 ms, 36 rows at 512 keys
+        // 3.76 -> 3.51, at 2048 keys the splits stay: 4.72 against 5.02)
+        const bool short_enough = uniform && ns == 1 && max_units * (slots - rows) <= 40 * slots;
+        if (rows * ns >= slots - slots / 8 || short_enough) {
             long long u = (max_units + ns - 1) / ns;
             if (u < 2 * kAttnWaves) u = 2 * kAttnWaves;   // >= 2 units per wave amortises the merge
             if (u > max_units) u = max_units;
