@@ -1078,11 +1078,17 @@ SplitPlan plan_splits(int R, int hk, int max_kv_len, bool uniform = false) {
     // 10.03); with rows of unknown lengths a long one would run on alone.
     const int cus = resident_attn_blocks();
     const long long slots = 2LL * (cus > 0 ? cus : 256);   // resident blocks: two of four waves per CU
-    // Equally long rows that fill half of those slots (32 rows of 8 kv heads, 64 rows of 4): one
-    // block of eight waves per (row, kv head) — the same waves in flight as two splits of four
-    // waves each, and nothing to merge.
-    if (uniform && 2 * rows <= slots && 2 * rows >= slots - slots / 8 && rows * ((max_units + 31) / 32) < 6 * slots)
-        return {max_units, 1, 2 * kAttnWaves};
+    // Equally long rows that fill at most half of those slots: one block of eight waves per (row,
+    // kv head) with nothing to merge, when its waves walk at most a few steps (of 32 keys) more than
+    // the waves of a plan that splits every row over the empty slots would.  Rows that fill half
+    // the slots (32 rows of 8 kv heads, 64 rows of 4) always do: eight waves are then the same waves
+    // in flight as two splits of four.  Fewer than 128 blocks leave most of the chip without key
+    // requests in flight, and the longer walk costs more there.
+    if (uniform && 2 * rows <= slots && rows >= 32 && rows * ((max_units + 31) / 32) < 6 * slots) {
+        const long long ns = slots / rows;
+        const long long steps_one = (max_units + 15) / 16, steps_split = (max_units + 8 * ns - 1) / (8 * ns);
+        if (steps_one - steps_split <= (rows >= 128 ? 3 : 1)) return {max_units, 1, 2 * kAttnWaves};
+    }
     if (rows * ((max_units + 31) / 32) < (uniform ? 6 * slots : slots + slots / 2) && rows <= slots) {
         const long long ns = slots / rows;
         // (equally long rows that fill more than half the slots: one split per row also where an

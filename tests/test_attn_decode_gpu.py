@@ -216,10 +216,11 @@ def test_rows_with_custom_masks_match_oracle(gpu, oracle, hq, hk, d):
 
 
 @pytest.mark.parametrize("ctx_kind", ["equal", "ragged"])
-@pytest.mark.parametrize("rows,hq,hk,d", [(64, 32, 8, 128), (32, 16, 8, 64), (64, 32, 4, 128)])
+@pytest.mark.parametrize("rows,hq,hk,d", [(64, 32, 8, 128), (32, 16, 8, 64), (64, 32, 4, 128), (16, 32, 8, 128), (24, 16, 8, 128)])
 def test_rows_declared_equally_long_take_one_round_and_match_the_oracle(gpu, oracle, rows, hq, hk, d, ctx_kind):
     """pie_hip_attn_rows_paged_kvq_uniform: a batch of about equal contexts plans one round of blocks
-    (64 rows x 8 kv heads: one block per row and head, no merge); the hint only changes the plan, so a
+    (64 rows x 8 kv heads: one block per row and head, no merge; 16 or 24 rows: one block of eight waves
+    per row and head); the hint only changes the plan, so a
     ragged batch given it by mistake, empty row included, still comes out right."""
     import torch
 
