@@ -139,6 +139,51 @@ def test_large_ragged_batch_over_quantised_pools_takes_the_chunked_launch(gpu, o
     assert np.allclose(lse_g[fin], lse64[fin], rtol=0, atol=2e-4)
 
 
+@pytest.mark.parametrize("fmt,hq,hk,d,rows,ctx_lo,ctx_hi", [
+    ("fp8_per_token_head", 32, 8, 128, 16, 580, 640), ("int8_per_token_head", 32, 4, 128, 64, 900, 1000),
+    ("fp8_e5m2", 16, 8, 64, 24, 300, 330), ("int8_per_token_head", 32, 8, 128, 40, 480, 512)])
+def test_rows_declared_equally_long_over_quantised_pools(gpu, oracle, fmt, hq, hk, d, rows, ctx_lo, ctx_hi):
+    """The equal-length hint over one-byte pools: one block of eight waves per (row, kv head) for 16, 24
+    and 64 x 4 rows, one four-wave block per pair for 40 rows — no split, nothing merged — against the
+    oracle over the dequantised pools and against the launch without the hint."""
+    import torch
+    from pie_amd import ops
+
+    ps = 16
+    rng = np.random.default_rng(33 + rows + d)
+    ctx = [int(c) for c in rng.integers(ctx_lo, ctx_hi + 1, size=rows)]
+    ctx[1] = 0
+    b = make_paged_batch(rng, ctx, hk, d, ps, f32_to_bf16=oracle.f32_to_bf16)
+    P = b["num_pages"]
+    q = oracle.f32_to_bf16(rng.standard_normal((rows, hq, d)).astype(np.float32))
+    pools = {}
+    for name in ("k_pages", "v_pages"):
+        codes, scales, deq = oracle.kv_quant_rows(b[name].reshape(P * ps * hk, d), fmt)
+        pools[name] = (codes.reshape(P, ps, hk, d),
+                       None if scales is None else np.ascontiguousarray(scales.reshape(P, ps, hk).transpose(0, 2, 1)),
+                       deq.reshape(P, ps, hk, d))
+    begin, lens = b["page_indptr"][:-1].astype(np.int32), np.asarray(ctx, np.int32)
+    sc = lambda s: None if s is None else dev(s, gpu)
+    args = (fmt, dev(q, gpu, torch.bfloat16), dev(pools["k_pages"][0], gpu), dev(pools["v_pages"][0], gpu),
+            sc(pools["k_pages"][1]), sc(pools["v_pages"][1]), dev(b["page_indices"].view(np.int32), gpu),
+            dev(begin, gpu), dev(lens, gpu))
+    o, lse = ops.attention_rows_paged_kvq(*args, lse=True, uniform=True)
+    o_plain, _ = ops.attention_rows_paged_kvq(*args, lse=True)
+    torch.cuda.synchronize()
+    truth, _, lse64 = oracle.attn_rows_f32kv(q, pools["k_pages"][2], pools["v_pages"][2], b["page_indices"],
+                                             begin, lens, hq, hk, d, ps, mode=2)
+    got = oracle.bf16_to_f32(o.view(torch.uint16).cpu().numpy()).astype(np.float64)
+    tol = 2.0 ** -8 * np.maximum(np.abs(truth), np.abs(got)) + 1e-4
+    assert np.all(np.abs(got - truth) <= tol)
+    assert not np.any(got[1]), "a row without keys is all zeros"
+    lse_g = lse.cpu().numpy()
+    fin = np.isfinite(lse64)
+    assert np.array_equal(np.isneginf(lse_g), np.isneginf(lse64))
+    assert np.allclose(lse_g[fin], lse64[fin], rtol=0, atol=2e-4)
+    plain = oracle.bf16_to_f32(o_plain.view(torch.uint16).cpu().numpy()).astype(np.float64)
+    assert np.all(np.abs(got - plain) <= 2.0 ** -7 * np.maximum(np.abs(got), np.abs(plain)) + 1e-4)
+
+
 def test_chunk_that_covers_more_rows_than_its_item_table_holds(gpu, oracle):
     """240 rows of a few keys next to 16 long ones: the chunks inside the run of short rows cover 40
     of them, more than one table of items, so a block builds its table twice."""
